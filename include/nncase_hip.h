@@ -1,0 +1,246 @@
+/*
+ * nncase_hip.h -- C ABI of libnncase_hip.so, the MI355X (gfx950) kernel
+ * library behind nncase's `hip` execution target.
+ *
+ * Conventions, copied from nncase's own pure-C surface
+ * (src/Native/include/nncase/api.h:43-110, src/Native/src/api.cpp:25-49):
+ *   - every function returns int: 0 on success, a negative value on failure
+ *     (-errno for argument / resource errors, -(0x1000 + hipError_t) for HIP
+ *     runtime errors, -nncase_errc for datatype/shape mismatches);
+ *   - every pointer argument is null-checked (-EINVAL);
+ *   - objects handed out are owned by the caller until the matching
+ *     *_destroy / *_free call;
+ *   - one context per host thread, no internal locking (the reference runtime
+ *     is single threaded: src/Native/src/runtime/interpreter.cpp).
+ * Kernels are enqueued on the context's HIP stream and the call returns at
+ * once; nncase_hip_stream_sync blocks until the stream has drained.
+ *
+ * Tensors on this boundary are dense, activations are NHWC (channels
+ * contiguous) unless a function says otherwise; weights are handed over in
+ * nncase's OIHW order on the HOST and re-laid-out once by the *_prepack calls.
+ * Data-type arguments use nncase's typecodes
+ * (src/Native/include/nncase/runtime/typecodes.def).
+ */
+#ifndef NNCASE_HIP_H
+#define NNCASE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NNCASE_HIP_API __attribute__((visibility("default")))
+
+/* nncase typecodes used on this boundary (typecodes.def). */
+enum {
+    NNCASE_HIP_DT_I8 = 0x02,
+    NNCASE_HIP_DT_I16 = 0x03,
+    NNCASE_HIP_DT_I32 = 0x04,
+    NNCASE_HIP_DT_U8 = 0x06,
+    NNCASE_HIP_DT_F16 = 0x0A,
+    NNCASE_HIP_DT_F32 = 0x0B
+};
+
+/* Error values beyond errno; returned negated.  The first block mirrors
+ * nncase_errc (src/Native/include/nncase/runtime/error.h:21-37).            */
+enum {
+    NNCASE_HIP_ERR_DATATYPE_MISMATCH = 0x05,
+    NNCASE_HIP_ERR_SHAPE_MISMATCH = 0x06,
+    NNCASE_HIP_ERR_INVALID_MEMORY_LOCATION = 0x07,
+    NNCASE_HIP_ERR_HIP_BASE = 0x1000 /* -(0x1000 + hipError_t) */
+};
+
+/* Mirrors quant_param_t (src/Native/include/nncase/runtime/simple_types.h:157-165). */
+typedef struct nncase_hip_quant_param {
+    int32_t zero_point;
+    float scale;
+} nncase_hip_quant_param_t;
+
+typedef struct nncase_hip_ctx nncase_hip_ctx_t;         /* device + stream      */
+typedef struct nncase_hip_weights nncase_hip_weights_t; /* pre-packed constants */
+
+/* ---- library / context ------------------------------------------------- */
+
+/* Library version, major << 16 | minor. */
+NNCASE_HIP_API int nncase_hip_version(void);
+
+/* Creates a context on HIP device `device` with a stream of its own.  Fails
+ * with -ENODEV when the device is not a gfx950 part.  Counterpart of
+ * nncase_interp_create (api.h:77). */
+NNCASE_HIP_API int nncase_hip_ctx_create(int device, nncase_hip_ctx_t **ctx);
+NNCASE_HIP_API int nncase_hip_ctx_destroy(nncase_hip_ctx_t *ctx);
+
+/* The hipStream_t the context enqueues on (so a caller can record events on
+ * it), and a way to make the context use a caller-owned stream instead. */
+NNCASE_HIP_API int nncase_hip_ctx_get_stream(nncase_hip_ctx_t *ctx, void **hip_stream);
+NNCASE_HIP_API int nncase_hip_ctx_set_stream(nncase_hip_ctx_t *ctx, void *hip_stream);
+
+/* Text of the last error recorded on this context ("" when none); the
+ * pointer stays valid until the next failing call on the context. */
+NNCASE_HIP_API const char *nncase_hip_last_error_string(nncase_hip_ctx_t *ctx);
+
+/* Device properties the benchmark reports: compute units, clock in kHz. */
+NNCASE_HIP_API int nncase_hip_device_info(nncase_hip_ctx_t *ctx, int *compute_units,
+                                          int *clock_khz, size_t *hbm_bytes);
+
+/* ---- device memory (counterpart of nncase_buffer_allocator_alloc /
+ *      nncase_host_buffer_map, api.h:59-67; here the memory is HBM) -------- */
+NNCASE_HIP_API int nncase_hip_malloc(nncase_hip_ctx_t *ctx, size_t bytes, void **dptr);
+NNCASE_HIP_API int nncase_hip_free(nncase_hip_ctx_t *ctx, void *dptr);
+NNCASE_HIP_API int nncase_hip_memcpy_h2d(nncase_hip_ctx_t *ctx, void *dst_dev, const void *src_host, size_t bytes);
+NNCASE_HIP_API int nncase_hip_memcpy_d2h(nncase_hip_ctx_t *ctx, void *dst_host, const void *src_dev, size_t bytes);
+NNCASE_HIP_API int nncase_hip_memset(nncase_hip_ctx_t *ctx, void *dptr, int byte, size_t bytes);
+NNCASE_HIP_API int nncase_hip_stream_sync(nncase_hip_ctx_t *ctx);
+
+/* ---- quantize / dequantize --------------------------------------------- */
+
+/* q = sat_T((int32) rne(x / scale + (float)zero_point)), T in {u8, i8, i16}.
+ * Replaces kernels::stackvm::quantize
+ * (src/Native/src/kernels/stackvm/tensor_ops.cpp:681-695 ->
+ *  reference/quantize.cpp:29-43, optimized/quantize.cpp:58-68).
+ * in_dtype is f32 or f16; `count` elements, contiguous. */
+NNCASE_HIP_API int nncase_hip_quantize(nncase_hip_ctx_t *ctx, const void *in_dev, int in_dtype, void *out_dev,
+                                       int out_dtype, size_t count, nncase_hip_quant_param_t qp);
+
+/* y = ((float)q - (float)zero_point) * scale, q in {u8, i8, i16, i32},
+ * out_dtype f32 or f16 (f16: the f32 value rounded to nearest even).
+ * Replaces kernels::stackvm::dequantize
+ * (tensor_ops.cpp:268-283 -> reference/dequantize.cpp:29-39). */
+NNCASE_HIP_API int nncase_hip_dequantize(nncase_hip_ctx_t *ctx, const void *in_dev, int in_dtype, void *out_dev,
+                                         int out_dtype, size_t count, nncase_hip_quant_param_t qp);
+
+/* ---- u8/u8 convolution and matmul --------------------------------------
+ *
+ * acc[p, oc] = bias[oc] + sum_{ky,kx,ic} (x - zx) * (w - zw)          (int32)
+ * out_dtype I32 : acc
+ * out_dtype F32 : clamp((float)acc * (sx * sw), lo, hi)
+ * out_dtype U8  : sat_u8(rne(clamp((float)acc * (sx*sw), lo, hi) / sy + (float)zy))
+ * Padding taps contribute nothing.  This is the integer-exact form of what
+ * nncase imports a quantized conv as -- Dequantize -> Conv2D(fused_clamp) ->
+ * Quantize (src/Nncase.Importer/Onnx/QLinearConv.cs:61-75,
+ * src/Nncase.Importer/TFLite/Conv2D.cs:39-98) -- and replaces
+ * kernels::stackvm::conv2d (tensor_ops.cpp:181-220 ->
+ * reference/convolution.cpp:26-105) on that sub-graph.  groups == 1 runs on
+ * int8 MFMA, groups == in_channels == out_channels runs the depthwise
+ * streaming kernel, other group counts run one MFMA launch per group.
+ */
+typedef struct nncase_hip_conv2d_desc {
+    int32_t in_channels, out_channels;
+    int32_t kernel_h, kernel_w;
+    int32_t groups;
+    nncase_hip_quant_param_t w_qp; /* per-tensor weight quantisation */
+} nncase_hip_conv2d_desc_t;
+
+/* Re-lays-out HOST weights (OIHW u8) and bias (int32[out_channels], may be
+ * NULL = zeros) into the MFMA operand order, re-biases them to s8, computes
+ * the per-output-channel sums used for zero-point correction and uploads the
+ * result.  Done once per constant, like nncase's .rdata constants. */
+NNCASE_HIP_API int nncase_hip_qconv2d_prepack(nncase_hip_ctx_t *ctx, const nncase_hip_conv2d_desc_t *desc,
+                                              const uint8_t *weights_oihw_host, const int32_t *bias_host,
+                                              nncase_hip_weights_t **weights);
+NNCASE_HIP_API int nncase_hip_weights_destroy(nncase_hip_ctx_t *ctx, nncase_hip_weights_t *weights);
+
+typedef struct nncase_hip_conv2d_args {
+    int32_t batch, in_h, in_w;           /* input is [batch, in_h, in_w, in_channels] u8   */
+    int32_t stride_h, stride_w;
+    int32_t dilation_h, dilation_w;
+    int32_t pad_h_before, pad_h_after;   /* paddings_t order of tensor_ops.cpp:192-199     */
+    int32_t pad_w_before, pad_w_after;
+    nncase_hip_quant_param_t x_qp;       /* input quantisation                             */
+    nncase_hip_quant_param_t y_qp;       /* output quantisation (U8 output only)           */
+    float clamp_min, clamp_max;          /* fused_clamp of Conv2D, applied in the fp32 domain */
+    int32_t out_dtype;                   /* NNCASE_HIP_DT_U8 / _I32 / _F32                 */
+} nncase_hip_conv2d_args_t;
+
+/* Output is [batch, out_h, out_w, out_channels] with
+ * out = (in + pad_before + pad_after - ((k-1)*dilation+1) + stride) / stride
+ * (src/Native/include/nncase/kernels/kernel_utils.h:86-93). */
+NNCASE_HIP_API int nncase_hip_qconv2d(nncase_hip_ctx_t *ctx, const uint8_t *x_dev, const nncase_hip_weights_t *weights,
+                                      void *y_dev, const nncase_hip_conv2d_args_t *args);
+
+/* MatMul A[M,K] (u8, device) x B[K,N] (u8, row-major, HOST, pre-packed) with
+ * the same three output forms; replaces kernels::stackvm::mat_mul
+ * (tensor_ops.cpp:553-565 -> reference/matmul.cpp:28-48) on the
+ * Dequantize -> MatMul (-> Quantize) sub-graph of
+ * src/Nncase.Importer/Onnx/QLinearMatmul.cs:25-28. */
+NNCASE_HIP_API int nncase_hip_qmatmul_prepack(nncase_hip_ctx_t *ctx, const uint8_t *b_host, int32_t k, int32_t n,
+                                              nncase_hip_quant_param_t b_qp, const int32_t *bias_host,
+                                              nncase_hip_weights_t **weights);
+
+typedef struct nncase_hip_matmul_args {
+    int32_t m;
+    nncase_hip_quant_param_t a_qp;
+    nncase_hip_quant_param_t y_qp;
+    float clamp_min, clamp_max;
+    int32_t out_dtype;
+} nncase_hip_matmul_args_t;
+
+NNCASE_HIP_API int nncase_hip_qmatmul(nncase_hip_ctx_t *ctx, const uint8_t *a_dev, const nncase_hip_weights_t *weights,
+                                      void *y_dev, const nncase_hip_matmul_args_t *args);
+
+/* ---- u8 glue that keeps a quantized graph resident --------------------- */
+
+/* out = Q(clamp(DQ(a) + DQ(b))), elementwise on `count` bytes (binary add,
+ * src/Native/src/kernels/stackvm/reference/binary.cpp, between the
+ * dequantize / quantize formulas above). */
+NNCASE_HIP_API int nncase_hip_qadd(nncase_hip_ctx_t *ctx, const uint8_t *a_dev, nncase_hip_quant_param_t a_qp,
+                                   const uint8_t *b_dev, nncase_hip_quant_param_t b_qp, uint8_t *out_dev,
+                                   nncase_hip_quant_param_t y_qp, float clamp_min, float clamp_max, size_t count);
+
+/* out[n, c] = Q(mean_{h,w} DQ(x[n, h, w, c])): the sequential float window sum
+ * of reduce_window2d mean (reference/reduce_window.cpp:36-109,133-135) over
+ * the whole image. */
+NNCASE_HIP_API int nncase_hip_qglobal_avgpool(nncase_hip_ctx_t *ctx, const uint8_t *x_dev, uint8_t *out_dev,
+                                              int32_t batch, int32_t h, int32_t w, int32_t channels,
+                                              nncase_hip_quant_param_t x_qp, nncase_hip_quant_param_t y_qp);
+
+/* ---- pack / unpack ------------------------------------------------------
+ * pack: every listed axis a (extent D) becomes an outer axis of extent
+ * ceil(D / lanes) in place and its lane index is appended as a trailing axis
+ * of extent `lanes`, in the order the axes are listed; elements past D are
+ * zero.  unpack is the inverse with a crop.  A dimension permutation with
+ * padding; elem_size in {1, 2, 4}.  (No counterpart in this reference tree.)
+ */
+NNCASE_HIP_API int nncase_hip_pack(nncase_hip_ctx_t *ctx, const void *in_dev, void *out_dev, int32_t elem_size,
+                                   int32_t rank, const int32_t *shape, int32_t n_axes, const int32_t *axes,
+                                   const int32_t *lanes);
+NNCASE_HIP_API int nncase_hip_unpack(nncase_hip_ctx_t *ctx, const void *in_dev, void *out_dev, int32_t elem_size,
+                                     int32_t rank, const int32_t *unpacked_shape, int32_t n_axes,
+                                     const int32_t *axes, const int32_t *lanes);
+
+/* NCHW <-> NHWC relayout of a dense tensor (the Transpose nncase inserts
+ * around NHWC imports, src/Nncase.Importer/TFLite/Conv2D.cs:28-29,67). */
+NNCASE_HIP_API int nncase_hip_nchw_to_nhwc(nncase_hip_ctx_t *ctx, const void *in_dev, void *out_dev,
+                                           int32_t elem_size, int32_t n, int32_t c, int32_t h, int32_t w);
+NNCASE_HIP_API int nncase_hip_nhwc_to_nchw(nncase_hip_ctx_t *ctx, const void *in_dev, void *out_dev,
+                                           int32_t elem_size, int32_t n, int32_t c, int32_t h, int32_t w);
+
+/* ---- paged-attention decode ---------------------------------------------
+ * One query token per sequence against a block-paged fp16 KV cache:
+ *   out[b, h, :] = softmax(scale * q[b, h, :] . K[b, kvh, 0..ctx_b)) . V[b, kvh, ...]
+ * with kvh = h / (num_q_heads / num_kv_heads), fp32 scores and accumulation.
+ *   q            [batch, num_q_heads, head_dim]                 f16
+ *   k/v cache    [num_blocks, num_kv_heads, block_size, head_dim] f16
+ *   block_table  [batch, max_blocks_per_seq] int32 (physical block ids)
+ *   ctx_lens     [batch] int32
+ *   out          [batch, num_q_heads, head_dim]                 f16 or f32
+ * (No counterpart in this reference tree.)
+ */
+typedef struct nncase_hip_paged_attn_args {
+    int32_t batch, num_q_heads, num_kv_heads, head_dim;
+    int32_t block_size, max_blocks_per_seq, num_blocks;
+    float scale;
+    int32_t out_dtype; /* NNCASE_HIP_DT_F16 or _F32 */
+} nncase_hip_paged_attn_args_t;
+
+NNCASE_HIP_API int nncase_hip_paged_attention_decode(nncase_hip_ctx_t *ctx, const void *q_dev, const void *k_cache_dev,
+                                                     const void *v_cache_dev, const int32_t *block_table_dev,
+                                                     const int32_t *ctx_lens_dev, void *out_dev,
+                                                     const nncase_hip_paged_attn_args_t *args);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NNCASE_HIP_H */

@@ -1,0 +1,121 @@
+// Context, device memory and stream entry points of libnncase_hip.so.
+#include "common.hpp"
+
+#include <new>
+
+using namespace nnhip;
+
+extern "C" int nncase_hip_version(void) { return (0 << 16) | 1; }
+
+extern "C" int nncase_hip_ctx_create(int device, nncase_hip_ctx_t **out) {
+    if (!out) return -EINVAL;
+    *out = nullptr;
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count <= 0) return -ENODEV;
+    if (device < 0 || device >= count) return -ENODEV;
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, device) != hipSuccess) return -ENODEV;
+    // The kernels are built for gfx950 only; any other part cannot run them.
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) return -ENODEV;
+    if (hipSetDevice(device) != hipSuccess) return -ENODEV;
+    nncase_hip_ctx *ctx = new (std::nothrow) nncase_hip_ctx();
+    if (!ctx) return -ENOMEM;
+    ctx->device = device;
+    ctx->compute_units = prop.multiProcessorCount;
+    ctx->clock_khz = prop.clockRate;
+    ctx->hbm_bytes = prop.totalGlobalMem;
+    e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
+    if (e != hipSuccess) {
+        delete ctx;
+        return -(NNCASE_HIP_ERR_HIP_BASE + (int)e);
+    }
+    ctx->owns_stream = true;
+    *out = ctx;
+    return 0;
+}
+
+extern "C" int nncase_hip_ctx_destroy(nncase_hip_ctx_t *ctx) {
+    NNHIP_CHECK_CTX(ctx);
+    if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+    if (ctx->owns_stream && ctx->stream) (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+    return 0;
+}
+
+extern "C" int nncase_hip_ctx_get_stream(nncase_hip_ctx_t *ctx, void **hip_stream) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, hip_stream, -EINVAL, "get_stream: null out pointer");
+    *hip_stream = (void *)ctx->stream;
+    return 0;
+}
+
+extern "C" int nncase_hip_ctx_set_stream(nncase_hip_ctx_t *ctx, void *hip_stream) {
+    NNHIP_CHECK_CTX(ctx);
+    if (ctx->stream) NNHIP_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    if (ctx->owns_stream && ctx->stream) NNHIP_HIP(ctx, hipStreamDestroy(ctx->stream));
+    ctx->stream = (hipStream_t)hip_stream;
+    ctx->owns_stream = false;
+    return 0;
+}
+
+extern "C" const char *nncase_hip_last_error_string(nncase_hip_ctx_t *ctx) { return ctx ? ctx->last_error : ""; }
+
+extern "C" int nncase_hip_device_info(nncase_hip_ctx_t *ctx, int *compute_units, int *clock_khz, size_t *hbm_bytes) {
+    NNHIP_CHECK_CTX(ctx);
+    if (compute_units) *compute_units = ctx->compute_units;
+    if (clock_khz) *clock_khz = ctx->clock_khz;
+    if (hbm_bytes) *hbm_bytes = ctx->hbm_bytes;
+    return 0;
+}
+
+extern "C" int nncase_hip_malloc(nncase_hip_ctx_t *ctx, size_t bytes, void **dptr) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, dptr, -EINVAL, "malloc: null out pointer");
+    *dptr = nullptr;
+    if (bytes == 0) bytes = 1;
+    hipError_t e = hipMalloc(dptr, bytes);
+    if (e == hipErrorOutOfMemory) return fail(ctx, -ENOMEM, "malloc: out of device memory (%zu bytes)", bytes);
+    NNHIP_HIP(ctx, e);
+    return 0;
+}
+
+extern "C" int nncase_hip_free(nncase_hip_ctx_t *ctx, void *dptr) {
+    NNHIP_CHECK_CTX(ctx);
+    if (!dptr) return 0;
+    NNHIP_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    NNHIP_HIP(ctx, hipFree(dptr));
+    return 0;
+}
+
+extern "C" int nncase_hip_memcpy_h2d(nncase_hip_ctx_t *ctx, void *dst_dev, const void *src_host, size_t bytes) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, (dst_dev && src_host) || bytes == 0, -EINVAL, "memcpy_h2d: null pointer");
+    if (!bytes) return 0;
+    NNHIP_HIP(ctx, hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, ctx->stream));
+    NNHIP_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    return 0;
+}
+
+extern "C" int nncase_hip_memcpy_d2h(nncase_hip_ctx_t *ctx, void *dst_host, const void *src_dev, size_t bytes) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, (dst_host && src_dev) || bytes == 0, -EINVAL, "memcpy_d2h: null pointer");
+    if (!bytes) return 0;
+    NNHIP_HIP(ctx, hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    NNHIP_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    return 0;
+}
+
+extern "C" int nncase_hip_memset(nncase_hip_ctx_t *ctx, void *dptr, int byte, size_t bytes) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, dptr || bytes == 0, -EINVAL, "memset: null pointer");
+    if (!bytes) return 0;
+    NNHIP_HIP(ctx, hipMemsetAsync(dptr, byte, bytes, ctx->stream));
+    return 0;
+}
+
+extern "C" int nncase_hip_stream_sync(nncase_hip_ctx_t *ctx) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    return 0;
+}

@@ -1,0 +1,232 @@
+// Pure data-movement kernels: pack / unpack (lane-blocked layouts) and the
+// NCHW <-> NHWC relayout.  All are permutations with optional zero padding,
+// bound by HBM bandwidth; each thread produces one output element so writes
+// are always coalesced, and the NCHW/NHWC transposes go through an LDS tile so
+// reads are coalesced as well.
+#include "common.hpp"
+
+#include <type_traits>
+
+namespace nnhip {
+
+constexpr int kMaxRank = 8;
+constexpr int kLayoutThreads = 256;
+
+struct PackDesc {
+    int out_rank;                 // rank of the tensor being written
+    uint32_t out_dims[2 * kMaxRank];
+    // pack: output dim k adds coord * mul[k] to input axis axis[k]
+    // unpack: output dim d reads packed outer dim d and, if lanes[d] > 1, lane dim lane_dim[d]
+    int axis[2 * kMaxRank];
+    uint32_t mul[2 * kMaxRank];
+    uint32_t in_dims[2 * kMaxRank];
+    uint64_t in_strides[2 * kMaxRank];
+    uint32_t lanes[kMaxRank];
+    int lane_dim[kMaxRank];
+    int in_rank;
+    uint64_t total;
+};
+
+template <typename T> __global__ __launch_bounds__(kLayoutThreads) void pack_kernel(const T *in, T *out, const PackDesc d) {
+    const uint64_t gid = (uint64_t)blockIdx.x * kLayoutThreads + threadIdx.x;
+    if (gid >= d.total) return;
+    uint32_t coord[kMaxRank];
+#pragma unroll
+    for (int i = 0; i < kMaxRank; i++) coord[i] = 0;
+    uint64_t rem = gid;
+    for (int k = d.out_rank - 1; k >= 0; k--) {
+        const uint32_t c = (uint32_t)(rem % d.out_dims[k]);
+        rem /= d.out_dims[k];
+        coord[d.axis[k]] += c * d.mul[k];
+    }
+    bool ok = true;
+    uint64_t off = 0;
+    for (int i = 0; i < d.in_rank; i++) {
+        ok = ok && coord[i] < d.in_dims[i];
+        off += (uint64_t)coord[i] * d.in_strides[i];
+    }
+    out[gid] = ok ? in[off] : (T)0;
+}
+
+template <typename T> __global__ __launch_bounds__(kLayoutThreads) void unpack_kernel(const T *in, T *out, const PackDesc d) {
+    const uint64_t gid = (uint64_t)blockIdx.x * kLayoutThreads + threadIdx.x;
+    if (gid >= d.total) return;
+    uint64_t rem = gid, off = 0;
+    for (int k = d.out_rank - 1; k >= 0; k--) {
+        const uint32_t c = (uint32_t)(rem % d.out_dims[k]);
+        rem /= d.out_dims[k];
+        const uint32_t l = d.lanes[k];
+        off += (uint64_t)(c / l) * d.in_strides[k];
+        if (l > 1) off += (uint64_t)(c % l) * d.in_strides[d.lane_dim[k]];
+    }
+    out[gid] = in[off];
+}
+
+// [batch][rows][cols] -> [batch][cols][rows] through a 32x32 LDS tile.
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_kernel(const T *__restrict__ in, T *__restrict__ out, int rows, int cols) {
+    __shared__ T tile[32][33];
+    const size_t boff = (size_t)blockIdx.z * rows * cols;
+    const int c0 = blockIdx.x * 32, r0 = blockIdx.y * 32;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5; // 32 x 8
+#pragma unroll
+    for (int i = 0; i < 32; i += 8) {
+        const int r = r0 + ty + i, c = c0 + tx;
+        if (r < rows && c < cols) tile[ty + i][tx] = in[boff + (size_t)r * cols + c];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 32; i += 8) {
+        const int c = c0 + ty + i, r = r0 + tx;
+        if (r < rows && c < cols) out[boff + (size_t)c * rows + r] = tile[tx][ty + i];
+    }
+}
+
+template <typename T> static int launch_transpose(nncase_hip_ctx *ctx, const void *in, void *out, int batch, int rows, int cols) {
+    const dim3 grid(ceil_div(cols, 32), ceil_div(rows, 32), batch);
+    hipLaunchKernelGGL(transpose_kernel<T>, grid, dim3(256), 0, ctx->stream, (const T *)in, (T *)out, rows, cols);
+    NNHIP_LAUNCH_CHECK(ctx, "transpose_kernel");
+    return 0;
+}
+
+static int transpose(nncase_hip_ctx *ctx, const void *in, void *out, int es, int batch, int rows, int cols) {
+    NNHIP_REQUIRE(ctx, in && out, -EINVAL, "transpose: null buffer");
+    NNHIP_REQUIRE(ctx, batch > 0 && rows > 0 && cols > 0, -EINVAL, "transpose: non-positive shape");
+    NNHIP_REQUIRE(ctx, batch <= 65535 && ceil_div(rows, 32) <= 65535, -EINVAL, "transpose: grid too large");
+    switch (es) {
+    case 1: return launch_transpose<uint8_t>(ctx, in, out, batch, rows, cols);
+    case 2: return launch_transpose<uint16_t>(ctx, in, out, batch, rows, cols);
+    case 4: return launch_transpose<uint32_t>(ctx, in, out, batch, rows, cols);
+    default: return fail(ctx, -NNCASE_HIP_ERR_DATATYPE_MISMATCH, "transpose: element size %d", es);
+    }
+}
+
+static int build_common(nncase_hip_ctx *ctx, int rank, const int32_t *shape, int n_axes, const int32_t *axes,
+                        const int32_t *lanes, int (&norm_axes)[kMaxRank]) {
+    NNHIP_REQUIRE(ctx, shape && (n_axes == 0 || (axes && lanes)), -EINVAL, "pack: null argument");
+    NNHIP_REQUIRE(ctx, rank > 0 && rank <= kMaxRank && n_axes >= 0 && n_axes <= rank, -EINVAL, "pack: rank %d / %d axes",
+                  rank, n_axes);
+    for (int i = 0; i < rank; i++) NNHIP_REQUIRE(ctx, shape[i] > 0, -EINVAL, "pack: non-positive extent");
+    for (int i = 0; i < n_axes; i++) {
+        int ax = axes[i] < 0 ? axes[i] + rank : axes[i];
+        NNHIP_REQUIRE(ctx, ax >= 0 && ax < rank && lanes[i] > 0, -EINVAL, "pack: bad axis/lanes");
+        for (int j = 0; j < i; j++) NNHIP_REQUIRE(ctx, norm_axes[j] != ax, -EINVAL, "pack: repeated axis");
+        norm_axes[i] = ax;
+    }
+    return 0;
+}
+
+template <typename K> static int launch_by_size(nncase_hip_ctx *ctx, int es, K &&k) {
+    switch (es) {
+    case 1: return k((uint8_t *)nullptr);
+    case 2: return k((uint16_t *)nullptr);
+    case 4: return k((uint32_t *)nullptr);
+    default: return fail(ctx, -NNCASE_HIP_ERR_DATATYPE_MISMATCH, "pack: element size %d", es);
+    }
+}
+
+} // namespace nnhip
+
+using namespace nnhip;
+
+extern "C" int nncase_hip_pack(nncase_hip_ctx_t *ctx, const void *in_dev, void *out_dev, int32_t elem_size, int32_t rank,
+                               const int32_t *shape, int32_t n_axes, const int32_t *axes, const int32_t *lanes) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, in_dev && out_dev, -EINVAL, "pack: null buffer");
+    int nax[kMaxRank];
+    int rc = build_common(ctx, rank, shape, n_axes, axes, lanes, nax);
+    if (rc) return rc;
+    PackDesc d;
+    memset(&d, 0, sizeof(d));
+    d.in_rank = rank;
+    d.out_rank = rank + n_axes;
+    uint64_t stride = 1;
+    for (int i = rank - 1; i >= 0; i--) {
+        d.in_dims[i] = (uint32_t)shape[i];
+        d.in_strides[i] = stride;
+        stride *= (uint64_t)shape[i];
+    }
+    d.total = 1;
+    for (int i = 0; i < rank; i++) {
+        uint32_t l = 1;
+        for (int j = 0; j < n_axes; j++)
+            if (nax[j] == i) l = (uint32_t)lanes[j];
+        d.out_dims[i] = ((uint32_t)shape[i] + l - 1) / l;
+        d.axis[i] = i;
+        d.mul[i] = l;
+        d.total *= d.out_dims[i];
+    }
+    for (int j = 0; j < n_axes; j++) {
+        d.out_dims[rank + j] = (uint32_t)lanes[j];
+        d.axis[rank + j] = nax[j];
+        d.mul[rank + j] = 1;
+        d.total *= (uint64_t)lanes[j];
+    }
+    NNHIP_REQUIRE(ctx, d.total < ((uint64_t)1 << 40), -EINVAL, "pack: tensor too large");
+    const uint64_t blocks = (d.total + kLayoutThreads - 1) / kLayoutThreads;
+    NNHIP_REQUIRE(ctx, blocks < ((uint64_t)1 << 31), -EINVAL, "pack: tensor too large");
+    return launch_by_size(ctx, elem_size, [&](auto *tag) -> int {
+        typedef typename std::remove_pointer<decltype(tag)>::type T;
+        hipLaunchKernelGGL(pack_kernel<T>, dim3((unsigned)blocks), dim3(kLayoutThreads), 0, ctx->stream, (const T *)in_dev,
+                           (T *)out_dev, d);
+        NNHIP_LAUNCH_CHECK(ctx, "pack_kernel");
+        return 0;
+    });
+}
+
+extern "C" int nncase_hip_unpack(nncase_hip_ctx_t *ctx, const void *in_dev, void *out_dev, int32_t elem_size, int32_t rank,
+                                 const int32_t *unpacked_shape, int32_t n_axes, const int32_t *axes, const int32_t *lanes) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, in_dev && out_dev, -EINVAL, "unpack: null buffer");
+    int nax[kMaxRank];
+    int rc = build_common(ctx, rank, unpacked_shape, n_axes, axes, lanes, nax);
+    if (rc) return rc;
+    PackDesc d;
+    memset(&d, 0, sizeof(d));
+    d.out_rank = rank;
+    d.in_rank = rank + n_axes;
+    // packed (input) dims and strides
+    for (int i = 0; i < rank; i++) {
+        uint32_t l = 1;
+        d.lane_dim[i] = 0;
+        for (int j = 0; j < n_axes; j++)
+            if (nax[j] == i) {
+                l = (uint32_t)lanes[j];
+                d.lane_dim[i] = rank + j;
+            }
+        d.lanes[i] = l;
+        d.in_dims[i] = ((uint32_t)unpacked_shape[i] + l - 1) / l;
+        d.out_dims[i] = (uint32_t)unpacked_shape[i];
+    }
+    for (int j = 0; j < n_axes; j++) d.in_dims[rank + j] = (uint32_t)lanes[j];
+    uint64_t stride = 1;
+    for (int i = d.in_rank - 1; i >= 0; i--) {
+        d.in_strides[i] = stride;
+        stride *= d.in_dims[i];
+    }
+    d.total = 1;
+    for (int i = 0; i < rank; i++) d.total *= d.out_dims[i];
+    const uint64_t blocks = (d.total + kLayoutThreads - 1) / kLayoutThreads;
+    NNHIP_REQUIRE(ctx, blocks < ((uint64_t)1 << 31), -EINVAL, "unpack: tensor too large");
+    return launch_by_size(ctx, elem_size, [&](auto *tag) -> int {
+        typedef typename std::remove_pointer<decltype(tag)>::type T;
+        hipLaunchKernelGGL(unpack_kernel<T>, dim3((unsigned)blocks), dim3(kLayoutThreads), 0, ctx->stream,
+                           (const T *)in_dev, (T *)out_dev, d);
+        NNHIP_LAUNCH_CHECK(ctx, "unpack_kernel");
+        return 0;
+    });
+}
+
+extern "C" int nncase_hip_nchw_to_nhwc(nncase_hip_ctx_t *ctx, const void *in_dev, void *out_dev, int32_t elem_size, int32_t n,
+                                       int32_t c, int32_t h, int32_t w) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, h > 0 && w > 0 && (int64_t)h * w < ((int64_t)1 << 31), -EINVAL, "nchw_to_nhwc: bad shape");
+    return transpose(ctx, in_dev, out_dev, elem_size, n, c, h * w); // [n][c][hw] -> [n][hw][c]
+}
+
+extern "C" int nncase_hip_nhwc_to_nchw(nncase_hip_ctx_t *ctx, const void *in_dev, void *out_dev, int32_t elem_size, int32_t n,
+                                       int32_t c, int32_t h, int32_t w) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, h > 0 && w > 0 && (int64_t)h * w < ((int64_t)1 << 31), -EINVAL, "nhwc_to_nchw: bad shape");
+    return transpose(ctx, in_dev, out_dev, elem_size, n, h * w, c); // [n][hw][c] -> [n][c][hw]
+}

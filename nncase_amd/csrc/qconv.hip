@@ -1,0 +1,140 @@
+// Entry points of the u8/u8 convolution and matmul: argument checks, shape
+// inference and dispatch to the MFMA implicit-GEMM kernel or the depthwise
+// streaming kernel.
+#include "qconv.hpp"
+
+#include <cmath>
+#include <new>
+#include <vector>
+
+namespace nnhip {
+int prepack_igemm(nncase_hip_ctx *ctx, nncase_hip_weights *w, const uint8_t *w_oihw, const int32_t *bias);
+int prepack_depthwise(nncase_hip_ctx *ctx, nncase_hip_weights *w, const uint8_t *w_oihw, const int32_t *bias);
+} // namespace nnhip
+
+using namespace nnhip;
+
+static void free_weights(nncase_hip_weights *w) {
+    if (!w) return;
+    if (w->d_packed) (void)hipFree(w->d_packed);
+    if (w->d_wsum) (void)hipFree(w->d_wsum);
+    if (w->d_bias) (void)hipFree(w->d_bias);
+    delete w;
+}
+
+extern "C" int nncase_hip_qconv2d_prepack(nncase_hip_ctx_t *ctx, const nncase_hip_conv2d_desc_t *desc,
+                                          const uint8_t *weights_oihw_host, const int32_t *bias_host,
+                                          nncase_hip_weights_t **weights) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, desc && weights_oihw_host && weights, -EINVAL, "qconv2d_prepack: null argument");
+    *weights = nullptr;
+    NNHIP_REQUIRE(ctx, desc->in_channels > 0 && desc->out_channels > 0 && desc->kernel_h > 0 && desc->kernel_w > 0,
+                  -EINVAL, "qconv2d_prepack: non-positive dimension");
+    NNHIP_REQUIRE(ctx, desc->groups > 0 && desc->in_channels % desc->groups == 0 &&
+                           desc->out_channels % desc->groups == 0,
+                  -NNCASE_HIP_ERR_SHAPE_MISMATCH, "qconv2d_prepack: groups=%d does not divide channels %d/%d",
+                  desc->groups, desc->in_channels, desc->out_channels);
+    NNHIP_REQUIRE(ctx, desc->w_qp.zero_point >= 0 && desc->w_qp.zero_point <= 255, -EINVAL,
+                  "qconv2d_prepack: weight zero point %d outside u8", desc->w_qp.zero_point);
+    nncase_hip_weights *w = new (std::nothrow) nncase_hip_weights();
+    NNHIP_REQUIRE(ctx, w, -ENOMEM, "qconv2d_prepack: out of host memory");
+    w->in_channels = desc->in_channels;
+    w->out_channels = desc->out_channels;
+    w->kernel_h = desc->kernel_h;
+    w->kernel_w = desc->kernel_w;
+    w->groups = desc->groups;
+    w->g_ic = desc->in_channels / desc->groups;
+    w->g_oc = desc->out_channels / desc->groups;
+    w->zw = desc->w_qp.zero_point;
+    w->sw = desc->w_qp.scale;
+    const bool depthwise = desc->groups > 1 && w->g_ic == 1 && w->g_oc == 1;
+    w->kind = depthwise ? nncase_hip_weights::kDepthwise : nncase_hip_weights::kIgemm;
+    NNHIP_HIP(ctx, hipSetDevice(ctx->device));
+    const int rc = depthwise ? prepack_depthwise(ctx, w, weights_oihw_host, bias_host)
+                             : prepack_igemm(ctx, w, weights_oihw_host, bias_host);
+    if (rc) {
+        free_weights(w);
+        return rc;
+    }
+    *weights = w;
+    return 0;
+}
+
+extern "C" int nncase_hip_weights_destroy(nncase_hip_ctx_t *ctx, nncase_hip_weights_t *weights) {
+    NNHIP_CHECK_CTX(ctx);
+    if (!weights) return 0;
+    NNHIP_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    free_weights(weights);
+    return 0;
+}
+
+static int check_out_dtype(nncase_hip_ctx *ctx, int dt, nncase_hip_quant_param_t y_qp, const char *who) {
+    NNHIP_REQUIRE(ctx, dt == NNCASE_HIP_DT_U8 || dt == NNCASE_HIP_DT_I32 || dt == NNCASE_HIP_DT_F32,
+                  -NNCASE_HIP_ERR_DATATYPE_MISMATCH, "%s: unsupported output type 0x%x", who, dt);
+    if (dt == NNCASE_HIP_DT_U8) {
+        NNHIP_REQUIRE(ctx, y_qp.scale > 0.f && std::isfinite(y_qp.scale), -EINVAL, "%s: output scale must be positive", who);
+        NNHIP_REQUIRE(ctx, y_qp.zero_point >= 0 && y_qp.zero_point <= 255, -EINVAL, "%s: output zero point %d outside u8",
+                      who, y_qp.zero_point);
+    }
+    return 0;
+}
+
+extern "C" int nncase_hip_qconv2d(nncase_hip_ctx_t *ctx, const uint8_t *x_dev, const nncase_hip_weights_t *w, void *y_dev,
+                                  const nncase_hip_conv2d_args_t *a) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, x_dev && w && y_dev && a, -EINVAL, "qconv2d: null argument");
+    NNHIP_REQUIRE(ctx, a->batch > 0 && a->in_h > 0 && a->in_w > 0, -EINVAL, "qconv2d: non-positive input shape");
+    NNHIP_REQUIRE(ctx, a->stride_h > 0 && a->stride_w > 0 && a->dilation_h > 0 && a->dilation_w > 0, -EINVAL,
+                  "qconv2d: stride and dilation must be positive");
+    NNHIP_REQUIRE(ctx, a->pad_h_before >= 0 && a->pad_h_after >= 0 && a->pad_w_before >= 0 && a->pad_w_after >= 0, -EINVAL,
+                  "qconv2d: negative padding");
+    NNHIP_REQUIRE(ctx, a->x_qp.zero_point >= 0 && a->x_qp.zero_point <= 255, -EINVAL,
+                  "qconv2d: input zero point %d outside u8", a->x_qp.zero_point);
+    int rc = check_out_dtype(ctx, a->out_dtype, a->y_qp, "qconv2d");
+    if (rc) return rc;
+    const int out_h = windowed_output_size(a->in_h, w->kernel_h, a->stride_h, a->dilation_h, a->pad_h_before, a->pad_h_after);
+    const int out_w = windowed_output_size(a->in_w, w->kernel_w, a->stride_w, a->dilation_w, a->pad_w_before, a->pad_w_after);
+    NNHIP_REQUIRE(ctx, out_h > 0 && out_w > 0, -NNCASE_HIP_ERR_SHAPE_MISMATCH, "qconv2d: window larger than padded input");
+    if (w->kind == nncase_hip_weights::kDepthwise) return launch_qconv_depthwise(ctx, x_dev, w, y_dev, a, out_h, out_w);
+    return launch_qconv_igemm(ctx, x_dev, w, y_dev, a, out_h, out_w);
+}
+
+extern "C" int nncase_hip_qmatmul_prepack(nncase_hip_ctx_t *ctx, const uint8_t *b_host, int32_t k, int32_t n,
+                                          nncase_hip_quant_param_t b_qp, const int32_t *bias_host,
+                                          nncase_hip_weights_t **weights) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, b_host && weights, -EINVAL, "qmatmul_prepack: null argument");
+    NNHIP_REQUIRE(ctx, k > 0 && n > 0, -EINVAL, "qmatmul_prepack: non-positive dimension");
+    // B[K,N] row-major is a 1x1 convolution's OIHW weight [N,K,1,1] transposed.
+    std::vector<uint8_t> bt((size_t)k * n);
+    for (int kk = 0; kk < k; kk++)
+        for (int j = 0; j < n; j++) bt[(size_t)j * k + kk] = b_host[(size_t)kk * n + j];
+    nncase_hip_conv2d_desc_t d;
+    d.in_channels = k;
+    d.out_channels = n;
+    d.kernel_h = d.kernel_w = 1;
+    d.groups = 1;
+    d.w_qp = b_qp;
+    return nncase_hip_qconv2d_prepack(ctx, &d, bt.data(), bias_host, weights);
+}
+
+extern "C" int nncase_hip_qmatmul(nncase_hip_ctx_t *ctx, const uint8_t *a_dev, const nncase_hip_weights_t *w, void *y_dev,
+                                  const nncase_hip_matmul_args_t *m) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, a_dev && w && y_dev && m, -EINVAL, "qmatmul: null argument");
+    NNHIP_REQUIRE(ctx, m->m > 0, -EINVAL, "qmatmul: non-positive row count");
+    NNHIP_REQUIRE(ctx, w->kind == nncase_hip_weights::kIgemm && w->kernel_h == 1 && w->kernel_w == 1 && w->groups == 1,
+                  -NNCASE_HIP_ERR_SHAPE_MISMATCH, "qmatmul: weights were not packed by qmatmul_prepack");
+    nncase_hip_conv2d_args_t c;
+    memset(&c, 0, sizeof(c));
+    c.batch = 1;
+    c.in_h = m->m;
+    c.in_w = 1;
+    c.stride_h = c.stride_w = c.dilation_h = c.dilation_w = 1;
+    c.x_qp = m->a_qp;
+    c.y_qp = m->y_qp;
+    c.clamp_min = m->clamp_min;
+    c.clamp_max = m->clamp_max;
+    c.out_dtype = m->out_dtype;
+    return nncase_hip_qconv2d(ctx, a_dev, w, y_dev, &c);
+}

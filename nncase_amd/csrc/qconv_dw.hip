@@ -1,0 +1,321 @@
+// Depthwise u8/u8 convolution (groups == channels), NHWC.  Bandwidth-bound:
+// 2 bytes of HBM traffic per output for 9 multiply-adds, so no matrix cores;
+// the work is laid out so that every global access is a dword holding 4
+// adjacent channels of one pixel and adjacent lanes hold adjacent channels.
+//
+//   acc[c] = bias[c] + sum_t (x_t[c] - zx) * (w_t[c] - zw)
+//          = sum_t x_t[c] * w''_t[c] + (bias[c] - zx * sum_t w''_t[c]),   w'' = w - zw
+// where a padding tap is read as x = zx (contributes nothing).  w'' and its
+// tap sum are pack-time constants.  The requantisation epilogue is the same
+// fp32 sequence as the dense kernel's.
+//
+// dw3x3_kernel: a thread owns 4 channels x 4 output columns and walks down a
+// strip of output rows keeping the last three input rows unpacked in
+// registers, so each input byte is loaded from memory once per strip (plus a
+// two-row halo) and unpacked once.
+// dw_generic_kernel: any kernel size / stride / dilation / channel count.
+#include "qconv.hpp"
+
+#include <algorithm>
+#include <vector>
+
+namespace nnhip {
+
+constexpr int kDwThreads = 256;
+constexpr int kDwCols = 4;  // output columns per thread
+constexpr int kDwRows = 8;  // output rows per thread (3x3 kernel)
+
+struct DwArgs {
+    const uint8_t *x;
+    void *y;
+    const int16_t *w; // [taps][channels], w - zw
+    const int32_t *wsum;
+    const int32_t *bias;
+    int batch, in_h, in_w, channels, out_h, out_w;
+    int kh, kw, stride_h, stride_w, dil_h, dil_w, pad_h, pad_w;
+    int zx;
+    uint32_t zx_splat;
+    int cq;          // channel vectors per pixel
+    int strips;      // column strips per row
+    int row_chunks;  // row chunks per image (3x3 kernel)
+    FastDiv d_cq, d_strips, d_rows, d_ow, d_oh;
+    long long total; // threads of useful work
+    Epilogue ep;
+};
+
+__device__ __forceinline__ uint32_t dw_finish_u8(int32_t v, const Epilogue &ep) {
+    const float f = clamp_ref((float)v * ep.mult, ep.lo, ep.hi);
+    return requant_u8(f, ep.sy, ep.zy);
+}
+
+__device__ __forceinline__ void dw_store4(const DwArgs &a, size_t pix, int c0, const int32_t (&v)[4]) {
+    const size_t o = pix * a.channels + c0;
+    if (a.ep.out_mode == kOutU8) {
+        uint32_t q = 0;
+#pragma unroll
+        for (int c = 0; c < 4; c++) q |= dw_finish_u8(v[c], a.ep) << (8 * c);
+        *reinterpret_cast<uint32_t *>(reinterpret_cast<uint8_t *>(a.y) + o) = q;
+    } else if (a.ep.out_mode == kOutI32) {
+        *reinterpret_cast<int4 *>(reinterpret_cast<int32_t *>(a.y) + o) = int4{v[0], v[1], v[2], v[3]};
+    } else {
+        float4 f;
+        f.x = clamp_ref((float)v[0] * a.ep.mult, a.ep.lo, a.ep.hi);
+        f.y = clamp_ref((float)v[1] * a.ep.mult, a.ep.lo, a.ep.hi);
+        f.z = clamp_ref((float)v[2] * a.ep.mult, a.ep.lo, a.ep.hi);
+        f.w = clamp_ref((float)v[3] * a.ep.mult, a.ep.lo, a.ep.hi);
+        *reinterpret_cast<float4 *>(reinterpret_cast<float *>(a.y) + o) = f;
+    }
+}
+
+template <int S> __global__ __launch_bounds__(kDwThreads) void dw3x3_kernel(const DwArgs a) {
+    constexpr int NCOL = (kDwCols - 1) * S + 3;
+    const long long gid = (long long)blockIdx.x * kDwThreads + threadIdx.x;
+    if (gid >= a.total) return;
+    // gid -> (image, row chunk, strip, channel quad), channel quad fastest
+    uint32_t t = (uint32_t)gid;
+    uint32_t q = fastdiv(t, a.d_cq);
+    const int cq = (int)(t - q * a.d_cq.div);
+    t = q;
+    q = fastdiv(t, a.d_strips);
+    const int strip = (int)(t - q * a.d_strips.div);
+    t = q;
+    q = fastdiv(t, a.d_rows);
+    const int rchunk = (int)(t - q * a.d_rows.div);
+    const int img = (int)q;
+
+    const int c0 = cq * 4;
+    const int ox0 = strip * kDwCols;
+    const int oy0 = rchunk * kDwRows;
+    const int ix0 = ox0 * S - a.pad_w;
+    const int iy_first = oy0 * S - a.pad_h;
+
+    int32_t w[9][4], ct[4];
+#pragma unroll
+    for (int tap = 0; tap < 9; tap++) {
+        const uint2 raw = *reinterpret_cast<const uint2 *>(a.w + (size_t)tap * a.channels + c0);
+        w[tap][0] = (int16_t)(raw.x & 0xffff);
+        w[tap][1] = (int16_t)(raw.x >> 16);
+        w[tap][2] = (int16_t)(raw.y & 0xffff);
+        w[tap][3] = (int16_t)(raw.y >> 16);
+    }
+    {
+        const int4 b = *reinterpret_cast<const int4 *>(a.bias + c0);
+        const int4 s = *reinterpret_cast<const int4 *>(a.wsum + c0);
+        ct[0] = b.x - a.zx * s.x;
+        ct[1] = b.y - a.zx * s.y;
+        ct[2] = b.z - a.zx * s.z;
+        ct[3] = b.w - a.zx * s.w;
+    }
+
+    const uint8_t *ximg = a.x + (size_t)img * a.in_h * a.in_w * a.channels + c0;
+    int32_t rows[3][NCOL][4]; // three most recent input rows, unpacked
+    auto load_row = [&](int buf, int iy) {
+        const bool row_ok = (unsigned)iy < (unsigned)a.in_h;
+#pragma unroll
+        for (int col = 0; col < NCOL; col++) {
+            const int ix = ix0 + col;
+            uint32_t d = a.zx_splat;
+            if (row_ok && (unsigned)ix < (unsigned)a.in_w)
+                d = *reinterpret_cast<const uint32_t *>(ximg + ((size_t)iy * a.in_w + ix) * a.channels);
+            rows[buf][col][0] = d & 0xff;
+            rows[buf][col][1] = (d >> 8) & 0xff;
+            rows[buf][col][2] = (d >> 16) & 0xff;
+            rows[buf][col][3] = d >> 24;
+        }
+    };
+
+    // Output row t (relative) reads input rows t*S + {0,1,2} (relative), kept in
+    // buffer (row index mod 3).  The loop is unrolled by 3 so every buffer index
+    // is a compile-time constant.
+    load_row(0, iy_first + 0);
+    load_row(1, iy_first + 1);
+    load_row(2, iy_first + 2);
+    for (int t0 = 0; t0 < kDwRows; t0 += 3) {
+#pragma unroll
+        for (int ph = 0; ph < 3; ph++) {
+            const int tt = t0 + ph;
+            const int oy = oy0 + tt;
+            if (tt < kDwRows && oy < a.out_h) {
+                if (tt > 0) {
+#pragma unroll
+                    for (int nr = 0; nr < S; nr++) {
+                        // rows (tt-1)*S + 3 + nr, tt % 3 == ph
+                        const int rel_c = ((ph + 2) % 3) * S + 3 + nr; // same residue mod 3 as the real index
+                        load_row(rel_c % 3, iy_first + (tt - 1) * S + 3 + nr);
+                    }
+                }
+                int32_t acc[kDwCols][4];
+#pragma unroll
+                for (int o = 0; o < kDwCols; o++)
+#pragma unroll
+                    for (int c = 0; c < 4; c++) acc[o][c] = ct[c];
+#pragma unroll
+                for (int ky = 0; ky < 3; ky++) {
+                    const int buf = (ph * S + ky) % 3;
+#pragma unroll
+                    for (int kx = 0; kx < 3; kx++)
+#pragma unroll
+                        for (int o = 0; o < kDwCols; o++)
+#pragma unroll
+                            for (int c = 0; c < 4; c++)
+                                acc[o][c] += __mul24(rows[buf][o * S + kx][c], w[ky * 3 + kx][c]);
+                }
+#pragma unroll
+                for (int o = 0; o < kDwCols; o++) {
+                    if (ox0 + o < a.out_w) {
+                        const size_t pix = ((size_t)img * a.out_h + oy) * a.out_w + ox0 + o;
+                        dw_store4(a, pix, c0, acc[o]);
+                    }
+                }
+            }
+        }
+    }
+}
+
+// One thread per (pixel, VEC channels); every tap is fetched from memory.
+template <int VEC> __global__ __launch_bounds__(kDwThreads) void dw_generic_kernel(const DwArgs a) {
+    const long long gid = (long long)blockIdx.x * kDwThreads + threadIdx.x;
+    if (gid >= a.total) return;
+    uint32_t t = (uint32_t)gid;
+    uint32_t q = fastdiv(t, a.d_cq);
+    const int c0 = (int)(t - q * a.d_cq.div) * VEC;
+    t = q;
+    q = fastdiv(t, a.d_ow);
+    const int ox = (int)(t - q * a.d_ow.div);
+    t = q;
+    q = fastdiv(t, a.d_oh);
+    const int oy = (int)(t - q * a.d_oh.div);
+    const int img = (int)q;
+
+    int32_t acc[VEC];
+#pragma unroll
+    for (int c = 0; c < VEC; c++) acc[c] = a.bias[c0 + c] - a.zx * a.wsum[c0 + c];
+    const uint8_t *ximg = a.x + (size_t)img * a.in_h * a.in_w * a.channels + c0;
+    for (int ky = 0; ky < a.kh; ky++) {
+        const int iy = oy * a.stride_h - a.pad_h + ky * a.dil_h;
+        for (int kx = 0; kx < a.kw; kx++) {
+            const int ix = ox * a.stride_w - a.pad_w + kx * a.dil_w;
+            const bool ok = (unsigned)iy < (unsigned)a.in_h && (unsigned)ix < (unsigned)a.in_w;
+            const int16_t *wt = a.w + (size_t)(ky * a.kw + kx) * a.channels + c0;
+            if (VEC == 4) {
+                uint32_t d = a.zx_splat;
+                if (ok) d = *reinterpret_cast<const uint32_t *>(ximg + ((size_t)iy * a.in_w + ix) * a.channels);
+#pragma unroll
+                for (int c = 0; c < VEC; c++) acc[c] += __mul24((int)((d >> (8 * c)) & 0xff), (int)wt[c]);
+            } else {
+                int xv = a.zx;
+                if (ok) xv = ximg[((size_t)iy * a.in_w + ix) * a.channels];
+                acc[0] += __mul24(xv, (int)wt[0]);
+            }
+        }
+    }
+    const size_t pix = ((size_t)img * a.out_h + oy) * a.out_w + ox;
+    if (VEC == 4) {
+        int32_t v[4];
+#pragma unroll
+        for (int c = 0; c < 4; c++) v[c] = acc[c < VEC ? c : 0];
+        dw_store4(a, pix, c0, v);
+    } else {
+        const size_t o = pix * a.channels + c0;
+        if (a.ep.out_mode == kOutU8) reinterpret_cast<uint8_t *>(a.y)[o] = (uint8_t)dw_finish_u8(acc[0], a.ep);
+        else if (a.ep.out_mode == kOutI32) reinterpret_cast<int32_t *>(a.y)[o] = acc[0];
+        else reinterpret_cast<float *>(a.y)[o] = clamp_ref((float)acc[0] * a.ep.mult, a.ep.lo, a.ep.hi);
+    }
+}
+
+int prepack_depthwise(nncase_hip_ctx *ctx, nncase_hip_weights *w, const uint8_t *w_oihw, const int32_t *bias) {
+    const int taps = w->kernel_h * w->kernel_w, ch = w->out_channels;
+    w->k = taps;
+    std::vector<int16_t> packed((size_t)taps * ch);
+    std::vector<int32_t> wsum(ch, 0), hb(ch, 0);
+    if (bias) std::copy(bias, bias + ch, hb.begin());
+    for (int c = 0; c < ch; c++)
+        for (int t = 0; t < taps; t++) {
+            const int v = (int)w_oihw[(size_t)c * taps + t] - w->zw; // OIHW with I == 1
+            packed[(size_t)t * ch + c] = (int16_t)v;
+            wsum[c] += v;
+        }
+    w->packed_bytes = packed.size() * sizeof(int16_t);
+    NNHIP_HIP(ctx, hipMalloc(&w->d_packed, w->packed_bytes));
+    NNHIP_HIP(ctx, hipMalloc((void **)&w->d_wsum, sizeof(int32_t) * ch));
+    NNHIP_HIP(ctx, hipMalloc((void **)&w->d_bias, sizeof(int32_t) * ch));
+    NNHIP_HIP(ctx, hipMemcpy(w->d_packed, packed.data(), w->packed_bytes, hipMemcpyHostToDevice));
+    NNHIP_HIP(ctx, hipMemcpy(w->d_wsum, wsum.data(), sizeof(int32_t) * ch, hipMemcpyHostToDevice));
+    NNHIP_HIP(ctx, hipMemcpy(w->d_bias, hb.data(), sizeof(int32_t) * ch, hipMemcpyHostToDevice));
+    return 0;
+}
+
+int launch_qconv_depthwise(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_hip_weights *w, void *y,
+                           const nncase_hip_conv2d_args_t *c, int out_h, int out_w) {
+    const int ch = w->out_channels;
+    const int64_t in_elems = (int64_t)c->batch * c->in_h * c->in_w * ch;
+    const int64_t out_elems = (int64_t)c->batch * out_h * out_w * ch;
+    NNHIP_REQUIRE(ctx, out_elems > 0, -EINVAL, "qconv2d(depthwise): empty output");
+    NNHIP_REQUIRE(ctx, in_elems < ((int64_t)1 << 40) && out_elems < ((int64_t)1 << 40), -EINVAL,
+                  "qconv2d(depthwise): tensor too large");
+    NNHIP_REQUIRE(ctx, w->kernel_h * w->kernel_w <= 258, -EINVAL, "qconv2d(depthwise): window too large");
+
+    DwArgs a;
+    memset(&a, 0, sizeof(a));
+    a.x = x;
+    a.y = y;
+    a.w = reinterpret_cast<const int16_t *>(w->d_packed);
+    a.wsum = w->d_wsum;
+    a.bias = w->d_bias;
+    a.batch = c->batch;
+    a.in_h = c->in_h;
+    a.in_w = c->in_w;
+    a.channels = ch;
+    a.out_h = out_h;
+    a.out_w = out_w;
+    a.kh = w->kernel_h;
+    a.kw = w->kernel_w;
+    a.stride_h = c->stride_h;
+    a.stride_w = c->stride_w;
+    a.dil_h = c->dilation_h;
+    a.dil_w = c->dilation_w;
+    a.pad_h = c->pad_h_before;
+    a.pad_w = c->pad_w_before;
+    a.zx = c->x_qp.zero_point;
+    a.zx_splat = (uint32_t)(c->x_qp.zero_point & 0xff) * 0x01010101u;
+    a.ep.mult = c->x_qp.scale * w->sw;
+    a.ep.lo = c->clamp_min;
+    a.ep.hi = c->clamp_max;
+    a.ep.sy = c->y_qp.scale;
+    a.ep.zy = (float)c->y_qp.zero_point;
+    a.ep.out_mode = c->out_dtype == NNCASE_HIP_DT_U8 ? kOutU8 : (c->out_dtype == NNCASE_HIP_DT_I32 ? kOutI32 : kOutF32);
+
+    const bool vec4 = (ch % 4 == 0) && ((reinterpret_cast<uintptr_t>(x) & 3u) == 0) &&
+                      ((reinterpret_cast<uintptr_t>(y) & 15u) == 0);
+    const bool k3 = vec4 && w->kernel_h == 3 && w->kernel_w == 3 && c->dilation_h == 1 && c->dilation_w == 1 &&
+                    c->stride_h == c->stride_w && (c->stride_h == 1 || c->stride_h == 2);
+    if (k3) {
+        a.cq = ch / 4;
+        a.strips = ceil_div(out_w, kDwCols);
+        a.row_chunks = ceil_div(out_h, kDwRows);
+        a.d_cq = make_fastdiv((uint32_t)a.cq);
+        a.d_strips = make_fastdiv((uint32_t)a.strips);
+        a.d_rows = make_fastdiv((uint32_t)a.row_chunks);
+        a.total = (long long)c->batch * a.row_chunks * a.strips * a.cq;
+        NNHIP_REQUIRE(ctx, a.total < ((long long)1 << 31), -EINVAL, "qconv2d(depthwise): too many work items");
+        const int grid = (int)((a.total + kDwThreads - 1) / kDwThreads);
+        if (c->stride_h == 1) hipLaunchKernelGGL(dw3x3_kernel<1>, dim3(grid), dim3(kDwThreads), 0, ctx->stream, a);
+        else hipLaunchKernelGGL(dw3x3_kernel<2>, dim3(grid), dim3(kDwThreads), 0, ctx->stream, a);
+        NNHIP_LAUNCH_CHECK(ctx, "dw3x3_kernel");
+        return 0;
+    }
+    const int vec = vec4 ? 4 : 1;
+    a.cq = ch / vec;
+    a.d_cq = make_fastdiv((uint32_t)a.cq);
+    a.d_ow = make_fastdiv((uint32_t)out_w);
+    a.d_oh = make_fastdiv((uint32_t)out_h);
+    a.total = (long long)c->batch * out_h * out_w * a.cq;
+    NNHIP_REQUIRE(ctx, a.total < ((long long)1 << 31), -EINVAL, "qconv2d(depthwise): too many work items");
+    const int grid = (int)((a.total + kDwThreads - 1) / kDwThreads);
+    if (vec == 4) hipLaunchKernelGGL(dw_generic_kernel<4>, dim3(grid), dim3(kDwThreads), 0, ctx->stream, a);
+    else hipLaunchKernelGGL(dw_generic_kernel<1>, dim3(grid), dim3(kDwThreads), 0, ctx->stream, a);
+    NNHIP_LAUNCH_CHECK(ctx, "dw_generic_kernel");
+    return 0;
+}
+
+} // namespace nnhip

@@ -1,0 +1,183 @@
+// Host side of the implicit-GEMM convolution: weight pre-packing into MFMA
+// operand order, the tiling plan, and the launch dispatch.
+#include "qconv_igemm.hpp"
+
+#include <algorithm>
+#include <vector>
+
+namespace nnhip {
+
+static const int kAllowedTiles[] = {1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 12, 14, 16};
+
+static int round_tiles(int t, int max_tiles) {
+    for (int v : kAllowedTiles)
+        if (v >= t && v <= max_tiles) return v;
+    return max_tiles;
+}
+
+// Chooses the channel-chunk width T (in 16-channel tiles), the number of
+// chunks and the LDS staging depth for a reduction of `ksteps` k-steps.
+// max_tiles bounds T (the byte-gather loader is only built for T <= 4).
+static void plan_igemm(int g_oc, int ksteps, int max_tiles, int *tiles, int *nchunks, int *kc_steps) {
+    const int tt = ceil_div(g_oc, 16);
+    const int cap = std::min(max_tiles, tt);
+    int t0, kc;
+    if (ksteps * cap <= kLdsFrags) {
+        t0 = cap;
+        kc = ksteps;
+    } else if (ksteps <= 12) {
+        t0 = std::min(cap, kLdsFrags / ksteps);
+        kc = ksteps;
+    } else {
+        t0 = std::min(cap, 4);
+        kc = 12;
+    }
+    int nc = ceil_div(tt, t0);
+    const int t = round_tiles(ceil_div(tt, nc), max_tiles);
+    while (t * kc > kLdsFrags && kc > 1) kc--; // rounding T up may overshoot the LDS budget
+    nc = ceil_div(tt, t);
+    *tiles = t;
+    *nchunks = nc;
+    *kc_steps = kc;
+}
+
+// Packs one group's weights into MFMA operand order.
+//   w_at(oc, k) -> u8 weight of output channel oc (within the group) at
+//   reduction index k = (ky * kw + kx) * g_ic + ic.
+// Fragment (chunk, ks, nt): byte (kg * 16 + i) * 16 + b holds the weight of
+//   channel chunk*16T + (i / 4) * 4T + nt * 4 + (i % 4) at k = ks*64 + kg*16 + b,
+// re-biased to s8, or 0 outside the real channel / reduction range.
+template <typename WAt>
+static void pack_group(uint8_t *dst, int32_t *wsum, int g_oc, int k, int ksteps, int tiles, int nchunks, WAt w_at) {
+    for (int oc = 0; oc < g_oc; oc++) {
+        int32_t s = 0;
+        for (int kk = 0; kk < k; kk++) s += (int32_t)(int8_t)(w_at(oc, kk) ^ 0x80);
+        wsum[oc] = s;
+    }
+    for (int chunk = 0; chunk < nchunks; chunk++)
+        for (int ks = 0; ks < ksteps; ks++)
+            for (int nt = 0; nt < tiles; nt++) {
+                uint8_t *frag = dst + (((size_t)chunk * ksteps + ks) * tiles + nt) * 1024;
+                for (int kg = 0; kg < 4; kg++)
+                    for (int i = 0; i < 16; i++) {
+                        const int oc = chunk * 16 * tiles + (i / 4) * 4 * tiles + nt * 4 + (i % 4);
+                        for (int b = 0; b < 16; b++) {
+                            const int kk = ks * 64 + kg * 16 + b;
+                            uint8_t v = 0;
+                            if (oc < g_oc && kk < k) v = (uint8_t)(w_at(oc, kk) ^ 0x80);
+                            frag[(kg * 16 + i) * 16 + b] = v;
+                        }
+                    }
+            }
+}
+
+int prepack_igemm(nncase_hip_ctx *ctx, nncase_hip_weights *w, const uint8_t *w_oihw, const int32_t *bias) {
+    const int taps = w->kernel_h * w->kernel_w;
+    NNHIP_REQUIRE(ctx, (int64_t)taps * w->g_ic < 65536, -EINVAL,
+                  "qconv2d_prepack: reduction length %lld would overflow the int32 accumulator",
+                  (long long)taps * w->g_ic);
+    w->k = taps * w->g_ic;
+    w->ksteps = ceil_div(w->k, 64);
+    const int max_tiles = (w->g_ic % 4 == 0) ? 16 : 4;
+    plan_igemm(w->g_oc, w->ksteps, max_tiles, &w->tiles, &w->nchunks, &w->kc_steps);
+    const size_t group_bytes = (size_t)w->nchunks * w->ksteps * w->tiles * 1024;
+    w->packed_bytes = group_bytes * w->groups;
+    std::vector<uint8_t> packed(w->packed_bytes);
+    std::vector<int32_t> wsum(w->out_channels), hb(w->out_channels, 0);
+    if (bias) std::copy(bias, bias + w->out_channels, hb.begin());
+    const int g_ic = w->g_ic, kh = w->kernel_h, kw = w->kernel_w;
+    for (int g = 0; g < w->groups; g++) {
+        const uint8_t *wg = w_oihw + (size_t)g * w->g_oc * g_ic * kh * kw;
+        auto w_at = [&](int oc, int kk) -> uint8_t {
+            const int tap = kk / g_ic, ic = kk % g_ic;
+            return wg[((size_t)oc * g_ic + ic) * kh * kw + tap]; // OIHW: tap = ky * kw + kx
+        };
+        pack_group(packed.data() + g * group_bytes, wsum.data() + (size_t)g * w->g_oc, w->g_oc, w->k, w->ksteps, w->tiles,
+                   w->nchunks, w_at);
+    }
+    NNHIP_HIP(ctx, hipMalloc(&w->d_packed, w->packed_bytes));
+    NNHIP_HIP(ctx, hipMalloc((void **)&w->d_wsum, sizeof(int32_t) * w->out_channels));
+    NNHIP_HIP(ctx, hipMalloc((void **)&w->d_bias, sizeof(int32_t) * w->out_channels));
+    NNHIP_HIP(ctx, hipMemcpy(w->d_packed, packed.data(), w->packed_bytes, hipMemcpyHostToDevice));
+    NNHIP_HIP(ctx, hipMemcpy(w->d_wsum, wsum.data(), sizeof(int32_t) * w->out_channels, hipMemcpyHostToDevice));
+    NNHIP_HIP(ctx, hipMemcpy(w->d_bias, hb.data(), sizeof(int32_t) * w->out_channels, hipMemcpyHostToDevice));
+    return 0;
+}
+
+int launch_qconv_igemm(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_hip_weights *w, void *y,
+                       const nncase_hip_conv2d_args_t *c, int out_h, int out_w) {
+    const int64_t m64 = (int64_t)c->batch * out_h * out_w;
+    const int64_t in_bytes = (int64_t)c->batch * c->in_h * c->in_w * w->in_channels;
+    const int out_es = c->out_dtype == NNCASE_HIP_DT_U8 ? 1 : 4;
+    NNHIP_REQUIRE(ctx, m64 > 0 && m64 < ((int64_t)1 << 30), -EINVAL, "qconv2d: %lld output pixels unsupported",
+                  (long long)m64);
+    NNHIP_REQUIRE(ctx, in_bytes < ((int64_t)1 << 31), -EINVAL, "qconv2d: input of %lld bytes exceeds 2 GiB",
+                  (long long)in_bytes);
+    NNHIP_REQUIRE(ctx, m64 * w->out_channels * out_es < ((int64_t)1 << 40), -EINVAL, "qconv2d: output too large");
+    NNHIP_REQUIRE(ctx, (reinterpret_cast<uintptr_t>(x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(y) & 15u) == 0,
+                  -NNCASE_HIP_ERR_INVALID_MEMORY_LOCATION, "qconv2d: activation buffers must be 16-byte aligned");
+
+    IgemmArgs a;
+    memset(&a, 0, sizeof(a));
+    a.x = x;
+    a.y = y;
+    a.m = (int)m64;
+    a.n = w->g_oc;
+    a.k = w->k;
+    a.ksteps = w->ksteps;
+    a.kc_steps = w->kc_steps;
+    a.ldx = w->in_channels;
+    a.ldy = w->out_channels;
+    a.g_ic = w->g_ic;
+    a.in_h = c->in_h;
+    a.in_w = c->in_w;
+    a.kw = w->kernel_w;
+    a.stride_h = c->stride_h;
+    a.stride_w = c->stride_w;
+    a.dil_h = c->dilation_h;
+    a.dil_w = c->dilation_w;
+    a.pad_h = c->pad_h_before;
+    a.pad_w = c->pad_w_before;
+    a.d_ohow = make_fastdiv((uint32_t)(out_h * out_w));
+    a.d_ow = make_fastdiv((uint32_t)out_w);
+    a.d_kw = make_fastdiv((uint32_t)w->kernel_w);
+    a.d_gic = make_fastdiv((uint32_t)w->g_ic);
+    a.zxp = c->x_qp.zero_point - 128;
+    a.zwp = w->zw - 128;
+    a.zx_splat = (uint32_t)(c->x_qp.zero_point & 0xff) * 0x01010101u;
+    a.ep.mult = c->x_qp.scale * w->sw;
+    a.ep.lo = c->clamp_min;
+    a.ep.hi = c->clamp_max;
+    a.ep.sy = c->y_qp.scale;
+    a.ep.zy = (float)c->y_qp.zero_point;
+    a.ep.out_mode = c->out_dtype == NNCASE_HIP_DT_U8 ? kOutU8 : (c->out_dtype == NNCASE_HIP_DT_I32 ? kOutI32 : kOutF32);
+
+    const bool pointwise = w->kernel_h == 1 && w->kernel_w == 1 && c->stride_h == 1 && c->stride_w == 1 &&
+                           c->pad_h_before == 0 && c->pad_w_before == 0 && out_h == c->in_h && out_w == c->in_w;
+    int mode;
+    if (w->g_ic % 16 == 0) mode = pointwise ? kRows16 : kVec16;
+    else if (w->g_ic % 8 == 0) mode = kVec8;
+    else if (w->g_ic % 4 == 0) mode = kVec4;
+    else mode = kBytes;
+
+    const size_t group_bytes = (size_t)w->nchunks * w->ksteps * w->tiles * 1024;
+    for (int g = 0; g < w->groups; g++) {
+        a.wpk = reinterpret_cast<const uint8_t *>(w->d_packed) + g * group_bytes;
+        a.wsum = w->d_wsum + (size_t)g * w->g_oc;
+        a.bias = w->d_bias + (size_t)g * w->g_oc;
+        a.x_coff = g * w->g_ic;
+        a.y_coff = g * w->g_oc;
+        int rc;
+        switch (mode) {
+        case kRows16: rc = launch_igemm_rows16(ctx, a, w->tiles, w->nchunks); break;
+        case kVec16: rc = launch_igemm_vec16(ctx, a, w->tiles, w->nchunks); break;
+        case kVec8: rc = launch_igemm_vec8(ctx, a, w->tiles, w->nchunks); break;
+        case kVec4: rc = launch_igemm_vec4(ctx, a, w->tiles, w->nchunks); break;
+        default: rc = launch_igemm_bytes(ctx, a, w->tiles, w->nchunks); break;
+        }
+        if (rc) return rc;
+    }
+    return 0;
+}
+
+} // namespace nnhip

@@ -1,0 +1,376 @@
+// u8/u8 convolution and matmul as an implicit GEMM on the gfx950 int8 matrix
+// cores (v_mfma_i32_16x16x64_i8), int32 accumulation, zero points folded in as
+// sums, fp32 requantisation fused in the epilogue.
+//
+// Orientation.  The MFMA "A" operand (rows) is a 16-channel slice of the
+// pre-packed weights, the "B" operand (columns) is a group of 16 output
+// pixels, so after the multiply every lane owns 4 consecutive output channels
+// of ONE pixel per tile and, because the weight rows were permuted at pack
+// time, 4*T consecutive channels over the T tiles of its chunk: the epilogue
+// writes NHWC bytes with dword / dwordx4 stores and no cross-lane traffic.
+//
+// Zero points.  u8 values are re-biased to s8 with x' = x ^ 0x80 (= x - 128):
+//   sum (x - zx)(w - zw) = sum x'w' - zw' * sum_k x' - zx' * sum_k w' + K zx' zw'
+// with zx' = zx - 128, zw' = zw - 128.  sum_k w' is a pack-time constant;
+// sum_k x' (per pixel) comes from one extra MFMA per k-step against an
+// all-ones weight fragment held in registers, which leaves the sum in every
+// lane that needs it.  Padding taps are loaded as x = zx (they contribute
+// nothing); k positions past the end of the reduction load as x' = 0 and hit
+// zero weights.
+//
+// Data movement.  A block owns one chunk of output channels: it copies that
+// chunk's weight fragments into LDS once and then walks pixel tiles with a
+// grid stride, streaming activations global -> registers (each activation
+// fragment feeds all T tiles) while the previous fragment is being multiplied.
+//
+// The activation loader is a template parameter (one translation unit per
+// mode so the instantiations compile in parallel):
+//   kRows16  1x1 / stride 1 / no padding, channels % 16 == 0: a pixel's
+//            reduction row is contiguous, one 16-byte load per lane and k-step
+//   kVec16/8/4  any window; channels % VW == 0, so a VW-byte piece of the
+//            reduction never straddles two taps
+//   kBytes   anything else (e.g. 3 input channels): byte gathers
+#pragma once
+
+#include "qconv.hpp"
+
+namespace nnhip {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kThreads = 256;
+constexpr int kWaves = 4;
+constexpr int kLdsFrags = 48; // weight fragments (1 KiB each) resident in LDS per block
+
+enum LoadMode { kRows16 = 0, kVec16 = 1, kVec8 = 2, kVec4 = 3, kBytes = 4 };
+
+struct IgemmArgs {
+    const uint8_t *x;
+    void *y;
+    const uint8_t *wpk;    // fragments of this group: [nchunks][ksteps][T][1024]
+    const int32_t *wsum;   // [n] of this group
+    const int32_t *bias;   // [n] of this group
+    int m;                 // output pixels
+    int n;                 // output channels of this group
+    int k;                 // reduction length
+    int ksteps, kc_steps;  // total k-steps, k-steps per LDS stage
+    int ldx, x_coff;       // input pixel stride / channel offset of the group (bytes)
+    int ldy, y_coff;       // output pixel stride / channel offset (elements)
+    int g_ic;
+    int in_h, in_w;
+    int kw, stride_h, stride_w, dil_h, dil_w, pad_h, pad_w;
+    FastDiv d_ohow, d_ow, d_kw, d_gic;
+    int zxp, zwp;          // zx - 128, zw - 128
+    uint32_t zx_splat;     // zx in all four bytes
+    int num_mtiles;
+    Epilogue ep;
+};
+
+struct PixInfo {
+    int base; // kRows16: pixel index; other modes: pixel index of the image origin; < 0: no such pixel
+    int iy0, ix0;
+};
+
+template <int MODE> __device__ __forceinline__ PixInfo pix_info(const IgemmArgs &a, int p) {
+    PixInfo pi;
+    pi.iy0 = pi.ix0 = 0;
+    if (p >= a.m) {
+        pi.base = -1;
+        return pi;
+    }
+    if (MODE == kRows16) {
+        pi.base = p;
+        return pi;
+    }
+    const uint32_t img = fastdiv((uint32_t)p, a.d_ohow);
+    const uint32_t rem = (uint32_t)p - img * a.d_ohow.div;
+    const uint32_t oy = fastdiv(rem, a.d_ow);
+    const uint32_t ox = rem - oy * a.d_ow.div;
+    pi.base = (int)img * a.in_h * a.in_w;
+    pi.iy0 = (int)oy * a.stride_h - a.pad_h;
+    pi.ix0 = (int)ox * a.stride_w - a.pad_w;
+    return pi;
+}
+
+// Byte offset of input element (tap of reduction index kk) for pixel pi, or -1
+// when the tap falls into the padding.
+__device__ __forceinline__ int tap_offset(const IgemmArgs &a, const PixInfo &pi, int kk) {
+    const uint32_t tap = fastdiv((uint32_t)kk, a.d_gic);
+    const int c = kk - (int)tap * a.g_ic;
+    const uint32_t ky = fastdiv(tap, a.d_kw);
+    const int kx = (int)tap - (int)ky * a.kw;
+    const int iy = pi.iy0 + (int)ky * a.dil_h;
+    const int ix = pi.ix0 + kx * a.dil_w;
+    if ((unsigned)iy >= (unsigned)a.in_h || (unsigned)ix >= (unsigned)a.in_w) return -1;
+    return (int)((uint32_t)(pi.base + iy * a.in_w + ix) * (uint32_t)a.ldx + a.x_coff + c);
+}
+
+// 16 bytes of the activation operand for k in [kc*16, kc*16+16) of pixel `pi`,
+// already re-biased to s8.
+template <int MODE> __device__ __forceinline__ v4i load_act(const IgemmArgs &a, const PixInfo &pi, int kc) {
+    uint32_t w[4] = {0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u}; // x' = 0
+    if (pi.base >= 0) {
+        if (MODE == kRows16) {
+            if (kc * 16 < a.k) {
+                const u32x4 v = *reinterpret_cast<const u32x4 *>(
+                    a.x + (size_t)((uint32_t)pi.base * (uint32_t)a.ldx + a.x_coff + kc * 16));
+                w[0] = v[0], w[1] = v[1], w[2] = v[2], w[3] = v[3];
+            }
+        } else if (MODE == kBytes) {
+#pragma unroll
+            for (int b = 0; b < 16; b++) {
+                const int kk = kc * 16 + b;
+                if (kk < a.k) {
+                    const int off = tap_offset(a, pi, kk);
+                    const uint32_t byte = off >= 0 ? (uint32_t)a.x[(size_t)(uint32_t)off] : (a.zx_splat & 0xffu);
+                    w[b >> 2] = (w[b >> 2] & ~(0xffu << (8 * (b & 3)))) | (byte << (8 * (b & 3)));
+                }
+            }
+        } else {
+            constexpr int VW = MODE == kVec16 ? 16 : (MODE == kVec8 ? 8 : 4);
+#pragma unroll
+            for (int piece = 0; piece < 16 / VW; piece++) {
+                const int kk = kc * 16 + piece * VW;
+                if (kk < a.k) {
+                    const int off = tap_offset(a, pi, kk);
+                    if (VW == 16) {
+                        u32x4 v = {a.zx_splat, a.zx_splat, a.zx_splat, a.zx_splat};
+                        if (off >= 0) v = *reinterpret_cast<const u32x4 *>(a.x + (size_t)(uint32_t)off);
+                        w[0] = v[0], w[1] = v[1], w[2] = v[2], w[3] = v[3];
+                    } else if (VW == 8) {
+                        u32x2 v = {a.zx_splat, a.zx_splat};
+                        if (off >= 0) v = *reinterpret_cast<const u32x2 *>(a.x + (size_t)(uint32_t)off);
+                        w[piece * 2] = v[0], w[piece * 2 + 1] = v[1];
+                    } else {
+                        uint32_t v = a.zx_splat;
+                        if (off >= 0) v = *reinterpret_cast<const uint32_t *>(a.x + (size_t)(uint32_t)off);
+                        w[piece] = v;
+                    }
+                }
+            }
+        }
+    }
+    return v4i{(int)(w[0] ^ 0x80808080u), (int)(w[1] ^ 0x80808080u), (int)(w[2] ^ 0x80808080u),
+               (int)(w[3] ^ 0x80808080u)};
+}
+
+template <int T, int RG, int MODE>
+__global__ __launch_bounds__(kThreads, 2) void qconv_igemm_kernel(const IgemmArgs a) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    int32_t *cterm = reinterpret_cast<int32_t *>(smem); // [T * 16]
+    uint8_t *wlds = smem + T * 16 * sizeof(int32_t);    // [kc_steps][T][1024]
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int j = lane & 15;  // pixel within a group of 16
+    const int gq = lane >> 4; // k-quarter on the load side, channel quarter on the store side
+    const int chunk = blockIdx.y;
+    const int ch_base = chunk * (T * 16);
+    const uint8_t *wsrc = a.wpk + (size_t)chunk * a.ksteps * T * 1024;
+    const int nkc = (a.ksteps + a.kc_steps - 1) / a.kc_steps;
+
+    // Per-channel constant of the zero-point identity, in the lane order the
+    // epilogue reads it: position gq' * 4T + nt * 4 + r <-> channel ch_base + same.
+    for (int i = threadIdx.x; i < T * 16; i += kThreads) {
+        const int ch = ch_base + i;
+        int32_t c = 0;
+        if (ch < a.n) c = a.bias[ch] - a.zxp * a.wsum[ch] + a.k * a.zxp * a.zwp;
+        cterm[i] = c;
+    }
+    auto stage_weights = [&](int kci) {
+        const int s0 = kci * a.kc_steps;
+        const int steps = min(a.kc_steps, a.ksteps - s0);
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(wsrc + (size_t)s0 * T * 1024);
+        u32x4 *dst = reinterpret_cast<u32x4 *>(wlds);
+        for (int i = threadIdx.x; i < steps * T * 64; i += kThreads) dst[i] = src[i];
+    };
+    if (nkc == 1) stage_weights(0);
+    __syncthreads();
+
+    const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
+    constexpr int pix_per_block = kWaves * RG * 16;
+
+    PixInfo pcur[RG], pnxt[RG];
+    v4i fcur[RG], fnxt[RG];
+#pragma unroll
+    for (int rg = 0; rg < RG; rg++) {
+        pnxt[rg].base = -1;
+        pnxt[rg].iy0 = pnxt[rg].ix0 = 0;
+        fnxt[rg] = v4i{0, 0, 0, 0};
+    }
+    int mt = blockIdx.x;
+    if (mt < a.num_mtiles) {
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) {
+            pcur[rg] = pix_info<MODE>(a, mt * pix_per_block + (wave * RG + rg) * 16 + j);
+            fcur[rg] = load_act<MODE>(a, pcur[rg], gq);
+        }
+    }
+    for (; mt < a.num_mtiles; mt += gridDim.x) {
+        v4i acc[RG][T];
+        v4i rs[RG];
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) {
+            rs[rg] = v4i{0, 0, 0, 0};
+#pragma unroll
+            for (int nt = 0; nt < T; nt++) acc[rg][nt] = v4i{0, 0, 0, 0};
+        }
+        const int mt_next = mt + gridDim.x;
+        for (int kci = 0; kci < nkc; kci++) {
+            if (nkc > 1) {
+                __syncthreads(); // previous stage fully consumed
+                stage_weights(kci);
+                __syncthreads();
+            }
+            const int s0 = kci * a.kc_steps;
+            const int s1 = min(a.ksteps, s0 + a.kc_steps);
+            for (int ks = s0; ks < s1; ks++) {
+                // issue the loads of the next fragment before multiplying this one
+                if (ks + 1 < a.ksteps) {
+#pragma unroll
+                    for (int rg = 0; rg < RG; rg++) fnxt[rg] = load_act<MODE>(a, pcur[rg], (ks + 1) * 4 + gq);
+                } else if (mt_next < a.num_mtiles) {
+#pragma unroll
+                    for (int rg = 0; rg < RG; rg++) {
+                        pnxt[rg] = pix_info<MODE>(a, mt_next * pix_per_block + (wave * RG + rg) * 16 + j);
+                        fnxt[rg] = load_act<MODE>(a, pnxt[rg], gq);
+                    }
+                }
+#pragma unroll
+                for (int rg = 0; rg < RG; rg++)
+                    rs[rg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, fcur[rg], rs[rg], 0, 0, 0);
+                const uint8_t *wstep = wlds + (size_t)(ks - s0) * T * 1024 + lane * 16;
+#pragma unroll
+                for (int nt = 0; nt < T; nt++) {
+                    const v4i wf = *reinterpret_cast<const v4i *>(wstep + nt * 1024);
+#pragma unroll
+                    for (int rg = 0; rg < RG; rg++)
+                        acc[rg][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf, fcur[rg], acc[rg][nt], 0, 0, 0);
+                }
+#pragma unroll
+                for (int rg = 0; rg < RG; rg++) fcur[rg] = fnxt[rg];
+            }
+        }
+
+        // ---- epilogue: zero-point correction, requantisation, NHWC store ----
+        const int ch0 = ch_base + gq * (4 * T); // first of this lane's 4T channels
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) {
+            const int p = mt * pix_per_block + (wave * RG + rg) * 16 + j;
+            if (p < a.m && ch0 < a.n) {
+                const int32_t rsz = a.zwp * rs[rg][0];
+                const size_t obase = (size_t)p * a.ldy + a.y_coff + ch0;
+                if (a.ep.out_mode == kOutU8) {
+                    uint8_t *yo = reinterpret_cast<uint8_t *>(a.y) + obase;
+                    uint32_t packed[T];
+#pragma unroll
+                    for (int nt = 0; nt < T; nt++) {
+                        const v4i ct = *reinterpret_cast<const v4i *>(cterm + gq * (4 * T) + nt * 4);
+                        uint32_t q = 0;
+#pragma unroll
+                        for (int r = 0; r < 4; r++) {
+                            const int32_t v = acc[rg][nt][r] + ct[r] - rsz;
+                            const float f = clamp_ref((float)v * a.ep.mult, a.ep.lo, a.ep.hi);
+                            q |= requant_u8(f, a.ep.sy, a.ep.zy) << (8 * r);
+                        }
+                        packed[nt] = q;
+                    }
+                    if (((a.ldy | a.y_coff) & 3) == 0 && ch0 + 4 * T <= a.n) {
+#pragma unroll
+                        for (int nt = 0; nt < T; nt += 4) {
+                            if (nt + 4 <= T) {
+                                *reinterpret_cast<u32x4_a4 *>(yo + nt * 4) =
+                                    u32x4_a4{packed[nt], packed[nt + 1 < T ? nt + 1 : nt], packed[nt + 2 < T ? nt + 2 : nt],
+                                             packed[nt + 3 < T ? nt + 3 : nt]};
+                            } else {
+#pragma unroll
+                                for (int e = nt; e < T; e++) *reinterpret_cast<uint32_t *>(yo + e * 4) = packed[e];
+                            }
+                        }
+                    } else {
+#pragma unroll
+                        for (int nt = 0; nt < T; nt++)
+#pragma unroll
+                            for (int r = 0; r < 4; r++)
+                                if (ch0 + nt * 4 + r < a.n) yo[nt * 4 + r] = (uint8_t)(packed[nt] >> (8 * r));
+                    }
+                } else {
+                    // int32 accumulators or clamped fp32, one dword per channel
+                    uint32_t *yo = reinterpret_cast<uint32_t *>(a.y) + obase;
+#pragma unroll
+                    for (int nt = 0; nt < T; nt++) {
+                        const v4i ct = *reinterpret_cast<const v4i *>(cterm + gq * (4 * T) + nt * 4);
+                        uint32_t o[4];
+#pragma unroll
+                        for (int r = 0; r < 4; r++) {
+                            const int32_t v = acc[rg][nt][r] + ct[r] - rsz;
+                            if (a.ep.out_mode == kOutI32) o[r] = (uint32_t)v;
+                            else o[r] = __float_as_uint(clamp_ref((float)v * a.ep.mult, a.ep.lo, a.ep.hi));
+                        }
+                        if (ch0 + nt * 4 + 4 <= a.n) {
+                            *reinterpret_cast<u32x4_a4 *>(yo + nt * 4) = u32x4_a4{o[0], o[1], o[2], o[3]};
+                        } else {
+#pragma unroll
+                            for (int r = 0; r < 4; r++)
+                                if (ch0 + nt * 4 + r < a.n) yo[nt * 4 + r] = o[r];
+                        }
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) pcur[rg] = pnxt[rg];
+    }
+}
+
+template <int T, int MODE> int launch_t(nncase_hip_ctx *ctx, const IgemmArgs &a, int nchunks) {
+    constexpr int RG = (T <= 8) ? 4 : 2;
+    IgemmArgs args = a;
+    constexpr int pix_per_block = kWaves * RG * 16;
+    args.num_mtiles = ceil_div(a.m, pix_per_block);
+    int gx = args.num_mtiles < ctx->compute_units * 2 ? args.num_mtiles : ctx->compute_units * 2;
+    // Blocks are dealt to the 8 XCDs round-robin by linear id; with a multiple of 8
+    // columns the blocks that share a pixel tile (same x, different chunk) land on
+    // one XCD and find the activations in its L2.
+    if (nchunks > 1) gx = ceil_div(gx, 8) * 8;
+    const size_t lds = (size_t)T * 16 * sizeof(int32_t) + (size_t)a.kc_steps * T * 1024;
+    hipLaunchKernelGGL((qconv_igemm_kernel<T, RG, MODE>), dim3(gx, nchunks, 1), dim3(kThreads), lds, ctx->stream, args);
+    NNHIP_LAUNCH_CHECK(ctx, "qconv_igemm_kernel");
+    return 0;
+}
+
+template <int MODE> int launch_mode(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks) {
+    switch (tiles) {
+    case 1: return launch_t<1, MODE>(ctx, a, nchunks);
+    case 2: return launch_t<2, MODE>(ctx, a, nchunks);
+    case 3: return launch_t<3, MODE>(ctx, a, nchunks);
+    case 4: return launch_t<4, MODE>(ctx, a, nchunks);
+    default: break;
+    }
+    if constexpr (MODE != kBytes) {
+        switch (tiles) {
+        case 5: return launch_t<5, MODE>(ctx, a, nchunks);
+        case 6: return launch_t<6, MODE>(ctx, a, nchunks);
+        case 7: return launch_t<7, MODE>(ctx, a, nchunks);
+        case 8: return launch_t<8, MODE>(ctx, a, nchunks);
+        case 9: return launch_t<9, MODE>(ctx, a, nchunks);
+        case 10: return launch_t<10, MODE>(ctx, a, nchunks);
+        case 12: return launch_t<12, MODE>(ctx, a, nchunks);
+        case 14: return launch_t<14, MODE>(ctx, a, nchunks);
+        case 16: return launch_t<16, MODE>(ctx, a, nchunks);
+        default: break;
+        }
+    }
+    return fail(ctx, -EINVAL, "igemm: no kernel for %d tiles (load mode %d)", tiles, MODE);
+}
+
+int launch_igemm_rows16(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks);
+int launch_igemm_vec16(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks);
+int launch_igemm_vec8(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks);
+int launch_igemm_vec4(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks);
+int launch_igemm_bytes(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks);
+
+} // namespace nnhip

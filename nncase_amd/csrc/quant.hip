@@ -1,0 +1,280 @@
+// Quantize / Dequantize streaming kernels and the u8 elementwise glue
+// (residual add, global average pool).  All HBM-bound: every thread moves
+// 4 elements per step with one vector load and one vector store, the grid is
+// a few waves per SIMD deep and walks the tensor with a grid stride so the
+// loads of several steps are in flight together.
+//
+// Arithmetic contracts (each fp32 step is a single IEEE operation; the file
+// is compiled with -ffp-contract=off):
+//   quantize    q = sat_T((int32) rne(x / scale + bias))          reference/quantize.cpp:36-43
+//   dequantize  y = ((float) q - bias) * scale                    reference/dequantize.cpp:36-39
+#include "common.hpp"
+
+#include <hip/hip_fp16.h>
+
+namespace nnhip {
+
+constexpr int kEwThreads = 256;
+constexpr int kEwVec = 4;
+constexpr int kEwUnroll = 4;
+
+template <typename T> struct Vec4;
+template <> struct Vec4<float> { typedef float4 type; };
+template <> struct Vec4<int32_t> { typedef int4 type; };
+template <> struct Vec4<__half> { typedef uint2 type; };
+template <> struct Vec4<int16_t> { typedef uint2 type; };
+template <> struct Vec4<uint8_t> { typedef uint32_t type; };
+template <> struct Vec4<int8_t> { typedef uint32_t type; };
+
+template <typename T> __device__ __forceinline__ void load4(const T *p, T (&v)[4]) {
+    typename Vec4<T>::type raw = *reinterpret_cast<const typename Vec4<T>::type *>(p);
+    __builtin_memcpy(v, &raw, sizeof(raw));
+}
+template <typename T> __device__ __forceinline__ void store4(T *p, const T (&v)[4]) {
+    typename Vec4<T>::type raw;
+    __builtin_memcpy(&raw, v, sizeof(raw));
+    *reinterpret_cast<typename Vec4<T>::type *>(p) = raw;
+}
+
+template <typename T> __device__ __forceinline__ float to_f32(T v) { return (float)v; }
+template <> __device__ __forceinline__ float to_f32<__half>(__half v) { return __half2float(v); }
+
+template <typename TQ> struct QLimits;
+template <> struct QLimits<uint8_t> { static constexpr float lo = 0.f, hi = 255.f; };
+template <> struct QLimits<int8_t> { static constexpr float lo = -128.f, hi = 127.f; };
+template <> struct QLimits<int16_t> { static constexpr float lo = -32768.f, hi = 32767.f; };
+
+// rne(v) then saturate.  The clamp is done on the float before rounding: the
+// limits are integers, so clamp and round-half-even commute, and values
+// beyond the int32 range saturate instead of wrapping.
+template <typename TQ> __device__ __forceinline__ TQ quantize_one(float x, float scale, float bias) {
+    float v = x / scale + bias;
+    v = fminf(fmaxf(v, QLimits<TQ>::lo), QLimits<TQ>::hi); // NaN -> lo
+    return (TQ)(int32_t)rintf(v);
+}
+
+template <typename TIn, typename TQ>
+__global__ __launch_bounds__(kEwThreads) void quantize_kernel(const TIn *__restrict__ in, TQ *__restrict__ out,
+                                                              size_t count, float scale, float bias, int vec_ok) {
+    const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t nthreads = (size_t)gridDim.x * blockDim.x;
+    const size_t nvec = vec_ok ? count / kEwVec : 0;
+    size_t i = tid;
+    for (; i + (kEwUnroll - 1) * nthreads < nvec; i += kEwUnroll * nthreads) {
+        TIn v[kEwUnroll][4];
+#pragma unroll
+        for (int u = 0; u < kEwUnroll; u++) load4(in + (i + u * nthreads) * kEwVec, v[u]);
+#pragma unroll
+        for (int u = 0; u < kEwUnroll; u++) {
+            TQ q[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) q[e] = quantize_one<TQ>(to_f32(v[u][e]), scale, bias);
+            store4(out + (i + u * nthreads) * kEwVec, q);
+        }
+    }
+    for (; i < nvec; i += nthreads) {
+        TIn v[4];
+        TQ q[4];
+        load4(in + i * kEwVec, v);
+#pragma unroll
+        for (int e = 0; e < 4; e++) q[e] = quantize_one<TQ>(to_f32(v[e]), scale, bias);
+        store4(out + i * kEwVec, q);
+    }
+    for (size_t j = nvec * kEwVec + tid; j < count; j += nthreads) out[j] = quantize_one<TQ>(to_f32(in[j]), scale, bias);
+}
+
+template <typename TOut> __device__ __forceinline__ TOut from_f32(float v);
+template <> __device__ __forceinline__ float from_f32<float>(float v) { return v; }
+template <> __device__ __forceinline__ __half from_f32<__half>(float v) { return __float2half_rn(v); }
+
+template <typename TQ, typename TOut>
+__global__ __launch_bounds__(kEwThreads) void dequantize_kernel(const TQ *__restrict__ in, TOut *__restrict__ out,
+                                                                size_t count, float scale, float bias, int vec_ok) {
+    const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t nthreads = (size_t)gridDim.x * blockDim.x;
+    const size_t nvec = vec_ok ? count / kEwVec : 0;
+    size_t i = tid;
+    for (; i + (kEwUnroll - 1) * nthreads < nvec; i += kEwUnroll * nthreads) {
+        TQ v[kEwUnroll][4];
+#pragma unroll
+        for (int u = 0; u < kEwUnroll; u++) load4(in + (i + u * nthreads) * kEwVec, v[u]);
+#pragma unroll
+        for (int u = 0; u < kEwUnroll; u++) {
+            TOut y[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) y[e] = from_f32<TOut>(((float)v[u][e] - bias) * scale);
+            store4(out + (i + u * nthreads) * kEwVec, y);
+        }
+    }
+    for (; i < nvec; i += nthreads) {
+        TQ v[4];
+        TOut y[4];
+        load4(in + i * kEwVec, v);
+#pragma unroll
+        for (int e = 0; e < 4; e++) y[e] = from_f32<TOut>(((float)v[e] - bias) * scale);
+        store4(out + i * kEwVec, y);
+    }
+    for (size_t j = nvec * kEwVec + tid; j < count; j += nthreads) out[j] = from_f32<TOut>(((float)in[j] - bias) * scale);
+}
+
+// out = Q(clamp(DQ(a) + DQ(b))) on bytes.
+__global__ __launch_bounds__(kEwThreads) void qadd_kernel(const uint8_t *__restrict__ a, const uint8_t *__restrict__ b,
+                                                          uint8_t *__restrict__ out, size_t count, float za, float sa,
+                                                          float zb, float sb, float zy, float sy, float lo, float hi,
+                                                          int vec_ok) {
+    const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t nthreads = (size_t)gridDim.x * blockDim.x;
+    auto one = [&](uint8_t qa, uint8_t qb) -> uint8_t {
+        const float fa = ((float)qa - za) * sa;
+        const float fb = ((float)qb - zb) * sb;
+        float s = fa + fb;
+        s = fmaxf(fminf(s, hi), lo);
+        float t = s / sy + zy;
+        t = fminf(fmaxf(t, 0.f), 255.f);
+        return (uint8_t)(int32_t)rintf(t);
+    };
+    // 16 bytes per thread per step
+    const size_t nvec = vec_ok ? count / 16 : 0;
+    for (size_t i = tid; i < nvec; i += nthreads) {
+        const uint4 va = *reinterpret_cast<const uint4 *>(a + i * 16);
+        const uint4 vb = *reinterpret_cast<const uint4 *>(b + i * 16);
+        uint8_t ba[16], bb[16], bo[16];
+        __builtin_memcpy(ba, &va, 16);
+        __builtin_memcpy(bb, &vb, 16);
+#pragma unroll
+        for (int e = 0; e < 16; e++) bo[e] = one(ba[e], bb[e]);
+        uint4 vo;
+        __builtin_memcpy(&vo, bo, 16);
+        *reinterpret_cast<uint4 *>(out + i * 16) = vo;
+    }
+    for (size_t j = nvec * 16 + tid; j < count; j += nthreads) out[j] = one(a[j], b[j]);
+}
+
+// Global average pool over NHWC u8.  One thread per (image, channel): the sum
+// runs over the pixels in (y, x) order with a float accumulator, exactly the
+// order of the reference's window loop, so the result is bit-identical.
+// Adjacent threads read adjacent channels, so every load is coalesced.
+__global__ __launch_bounds__(kEwThreads) void qglobal_avgpool_kernel(const uint8_t *__restrict__ x,
+                                                                     uint8_t *__restrict__ out, int batch, int hw,
+                                                                     int channels, float zx, float sx, float zy,
+                                                                     float sy) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= batch * channels) return;
+    const int n = idx / channels, c = idx - n * channels;
+    const uint8_t *p = x + (size_t)n * hw * channels + c;
+    float value = 0.f;
+    for (int i = 0; i < hw; i++) value = value + ((float)p[(size_t)i * channels] - zx) * sx;
+    const float mean = value / (float)hw;
+    float t = mean / sy + zy;
+    t = fminf(fmaxf(t, 0.f), 255.f);
+    out[idx] = (uint8_t)(int32_t)rintf(t);
+}
+
+inline int ew_grid(const nncase_hip_ctx *ctx, size_t work_items) {
+    size_t blocks = (work_items + kEwThreads - 1) / kEwThreads;
+    const size_t cap = (size_t)ctx->compute_units * 16; // 16 blocks of 4 waves per CU
+    if (blocks > cap) blocks = cap;
+    if (blocks == 0) blocks = 1;
+    return (int)blocks;
+}
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+template <typename TIn, typename TQ>
+int launch_quantize(nncase_hip_ctx *ctx, const void *in, void *out, size_t count, float scale, float bias) {
+    const int vec_ok = aligned16(in) && aligned16(out);
+    const int grid = ew_grid(ctx, (count + kEwVec - 1) / kEwVec);
+    hipLaunchKernelGGL((quantize_kernel<TIn, TQ>), dim3(grid), dim3(kEwThreads), 0, ctx->stream, (const TIn *)in,
+                       (TQ *)out, count, scale, bias, vec_ok);
+    NNHIP_LAUNCH_CHECK(ctx, "quantize_kernel");
+    return 0;
+}
+
+template <typename TQ, typename TOut>
+int launch_dequantize(nncase_hip_ctx *ctx, const void *in, void *out, size_t count, float scale, float bias) {
+    const int vec_ok = aligned16(in) && aligned16(out);
+    const int grid = ew_grid(ctx, (count + kEwVec - 1) / kEwVec);
+    hipLaunchKernelGGL((dequantize_kernel<TQ, TOut>), dim3(grid), dim3(kEwThreads), 0, ctx->stream, (const TQ *)in,
+                       (TOut *)out, count, scale, bias, vec_ok);
+    NNHIP_LAUNCH_CHECK(ctx, "dequantize_kernel");
+    return 0;
+}
+
+} // namespace nnhip
+
+using namespace nnhip;
+
+extern "C" int nncase_hip_quantize(nncase_hip_ctx_t *ctx, const void *in_dev, int in_dtype, void *out_dev,
+                                   int out_dtype, size_t count, nncase_hip_quant_param_t qp) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, (in_dev && out_dev) || count == 0, -EINVAL, "quantize: null buffer");
+    NNHIP_REQUIRE(ctx, qp.scale != 0.f, -EINVAL, "quantize: scale is zero");
+    if (count == 0) return 0;
+    const float bias = (float)qp.zero_point;
+#define NNHIP_Q_CASE(IN_DT, TIn, OUT_DT, TQ)                                                                           \
+    if (in_dtype == IN_DT && out_dtype == OUT_DT)                                                                      \
+    return launch_quantize<TIn, TQ>(ctx, in_dev, out_dev, count, qp.scale, bias)
+    NNHIP_Q_CASE(NNCASE_HIP_DT_F32, float, NNCASE_HIP_DT_U8, uint8_t);
+    NNHIP_Q_CASE(NNCASE_HIP_DT_F32, float, NNCASE_HIP_DT_I8, int8_t);
+    NNHIP_Q_CASE(NNCASE_HIP_DT_F32, float, NNCASE_HIP_DT_I16, int16_t);
+    NNHIP_Q_CASE(NNCASE_HIP_DT_F16, __half, NNCASE_HIP_DT_U8, uint8_t);
+    NNHIP_Q_CASE(NNCASE_HIP_DT_F16, __half, NNCASE_HIP_DT_I8, int8_t);
+    NNHIP_Q_CASE(NNCASE_HIP_DT_F16, __half, NNCASE_HIP_DT_I16, int16_t);
+#undef NNHIP_Q_CASE
+    return fail(ctx, -NNCASE_HIP_ERR_DATATYPE_MISMATCH, "quantize: unsupported types in=0x%x out=0x%x", in_dtype,
+                out_dtype);
+}
+
+extern "C" int nncase_hip_dequantize(nncase_hip_ctx_t *ctx, const void *in_dev, int in_dtype, void *out_dev,
+                                     int out_dtype, size_t count, nncase_hip_quant_param_t qp) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, (in_dev && out_dev) || count == 0, -EINVAL, "dequantize: null buffer");
+    if (count == 0) return 0;
+    const float bias = (float)qp.zero_point;
+#define NNHIP_DQ_CASE(IN_DT, TQ, OUT_DT, TOut)                                                                         \
+    if (in_dtype == IN_DT && out_dtype == OUT_DT)                                                                      \
+    return launch_dequantize<TQ, TOut>(ctx, in_dev, out_dev, count, qp.scale, bias)
+    NNHIP_DQ_CASE(NNCASE_HIP_DT_U8, uint8_t, NNCASE_HIP_DT_F32, float);
+    NNHIP_DQ_CASE(NNCASE_HIP_DT_I8, int8_t, NNCASE_HIP_DT_F32, float);
+    NNHIP_DQ_CASE(NNCASE_HIP_DT_I16, int16_t, NNCASE_HIP_DT_F32, float);
+    NNHIP_DQ_CASE(NNCASE_HIP_DT_I32, int32_t, NNCASE_HIP_DT_F32, float);
+    NNHIP_DQ_CASE(NNCASE_HIP_DT_U8, uint8_t, NNCASE_HIP_DT_F16, __half);
+    NNHIP_DQ_CASE(NNCASE_HIP_DT_I8, int8_t, NNCASE_HIP_DT_F16, __half);
+    NNHIP_DQ_CASE(NNCASE_HIP_DT_I16, int16_t, NNCASE_HIP_DT_F16, __half);
+    NNHIP_DQ_CASE(NNCASE_HIP_DT_I32, int32_t, NNCASE_HIP_DT_F16, __half);
+#undef NNHIP_DQ_CASE
+    return fail(ctx, -NNCASE_HIP_ERR_DATATYPE_MISMATCH, "dequantize: unsupported types in=0x%x out=0x%x", in_dtype,
+                out_dtype);
+}
+
+extern "C" int nncase_hip_qadd(nncase_hip_ctx_t *ctx, const uint8_t *a_dev, nncase_hip_quant_param_t a_qp,
+                               const uint8_t *b_dev, nncase_hip_quant_param_t b_qp, uint8_t *out_dev,
+                               nncase_hip_quant_param_t y_qp, float clamp_min, float clamp_max, size_t count) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, (a_dev && b_dev && out_dev) || count == 0, -EINVAL, "qadd: null buffer");
+    NNHIP_REQUIRE(ctx, y_qp.scale != 0.f, -EINVAL, "qadd: output scale is zero");
+    if (count == 0) return 0;
+    const int vec_ok = aligned16(a_dev) && aligned16(b_dev) && aligned16(out_dev);
+    const int grid = ew_grid(ctx, (count + 15) / 16);
+    hipLaunchKernelGGL(qadd_kernel, dim3(grid), dim3(kEwThreads), 0, ctx->stream, a_dev, b_dev, out_dev, count,
+                       (float)a_qp.zero_point, a_qp.scale, (float)b_qp.zero_point, b_qp.scale, (float)y_qp.zero_point,
+                       y_qp.scale, clamp_min, clamp_max, vec_ok);
+    NNHIP_LAUNCH_CHECK(ctx, "qadd_kernel");
+    return 0;
+}
+
+extern "C" int nncase_hip_qglobal_avgpool(nncase_hip_ctx_t *ctx, const uint8_t *x_dev, uint8_t *out_dev, int32_t batch,
+                                          int32_t h, int32_t w, int32_t channels, nncase_hip_quant_param_t x_qp,
+                                          nncase_hip_quant_param_t y_qp) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, x_dev && out_dev, -EINVAL, "qglobal_avgpool: null buffer");
+    NNHIP_REQUIRE(ctx, batch > 0 && h > 0 && w > 0 && channels > 0, -EINVAL, "qglobal_avgpool: bad shape");
+    NNHIP_REQUIRE(ctx, (int64_t)batch * channels < (int64_t)1 << 31, -EINVAL, "qglobal_avgpool: too large");
+    NNHIP_REQUIRE(ctx, y_qp.scale != 0.f, -EINVAL, "qglobal_avgpool: output scale is zero");
+    const int total = batch * channels;
+    hipLaunchKernelGGL(qglobal_avgpool_kernel, dim3((total + kEwThreads - 1) / kEwThreads), dim3(kEwThreads), 0,
+                       ctx->stream, x_dev, out_dev, batch, h * w, channels, (float)x_qp.zero_point, x_qp.scale,
+                       (float)y_qp.zero_point, y_qp.scale);
+    NNHIP_LAUNCH_CHECK(ctx, "qglobal_avgpool_kernel");
+    return 0;
+}

@@ -1,0 +1,204 @@
+"""Host-side mirror of the reference's kernel interface for the operators the `hip`
+target owns: same names, argument order and meaning as `kernels::stackvm::*`
+(src/Native/include/nncase/kernels/stackvm/tensor_ops.h, tensor_ops.cpp:181-220,268-283,
+553-565,681-695), operating on host arrays the way the reference's kernels operate on
+host tensors.  Every call stages its operands into HBM, runs the HIP kernel through the
+C ABI and copies the result back -- what the native `hip` runtime module does at an
+EXTCALL boundary.  Tensors are NCHW / OIHW here, as in the reference; the library works on
+NHWC internally and the relayout runs on the device.
+
+Quantised operators take the quantisation parameters the reference's importer attaches as
+Dequantize / Quantize nodes around the float op (QLinearConv.cs:61-75).
+"""
+from __future__ import annotations
+
+from typing import Optional, Sequence, Tuple
+
+import numpy as np
+
+from . import runtime as rt
+from .runtime import Context, QuantParam, qp
+
+_default_ctx: Optional[Context] = None
+
+
+def default_context() -> Context:
+    global _default_ctx
+    if _default_ctx is None:
+        _default_ctx = Context(0)
+    return _default_ctx
+
+
+def _ctx(ctx):
+    return ctx or default_context()
+
+
+def quantize(input: np.ndarray, quant_param: QuantParam, out_dtype=np.uint8, ctx: Context = None) -> np.ndarray:
+    """kernels::stackvm::quantize(out_type, input, quant_param)."""
+    c = _ctx(ctx)
+    x = np.asarray(input, order="C")
+    if x.dtype not in (np.float32, np.float16):
+        raise rt.HipError(-rt.ERR_DATATYPE_MISMATCH, "quantize", f"input dtype {x.dtype}")
+    out_dtype = np.dtype(out_dtype)
+    if x.size == 0:
+        return np.empty(x.shape, out_dtype)
+    src, dst = c.to_device(x), c.alloc(x.size * out_dtype.itemsize)
+    c.quantize(src, rt.NP_TO_DT[x.dtype], dst, rt.NP_TO_DT.get(out_dtype, 0xFF), x.size, quant_param)
+    return dst.download(x.shape, out_dtype)
+
+
+def dequantize(input: np.ndarray, quant_param: QuantParam, out_dtype=np.float32, ctx: Context = None) -> np.ndarray:
+    """kernels::stackvm::dequantize(out_type, input, quant_param)."""
+    c = _ctx(ctx)
+    q = np.asarray(input, order="C")
+    out_dtype = np.dtype(out_dtype)
+    if q.dtype not in rt.NP_TO_DT:
+        raise rt.HipError(-rt.ERR_DATATYPE_MISMATCH, "dequantize", f"input dtype {q.dtype}")
+    if q.size == 0:
+        return np.empty(q.shape, out_dtype)
+    src, dst = c.to_device(q), c.alloc(q.size * out_dtype.itemsize)
+    c.dequantize(src, rt.NP_TO_DT[q.dtype], dst, rt.NP_TO_DT.get(out_dtype, 0xFF), q.size, quant_param)
+    return dst.download(q.shape, out_dtype)
+
+
+def _out_dt(out_dtype) -> int:
+    return rt.NP_TO_DT[np.dtype(out_dtype)]
+
+
+def conv2d(input: np.ndarray, weights: np.ndarray, bias: Optional[np.ndarray], stride: Sequence[int],
+           padding: Sequence[Sequence[int]], dilation: Sequence[int], groups: int, fused_clamp: Tuple[float, float],
+           input_qp: QuantParam, weights_qp: QuantParam, output_qp: Optional[QuantParam] = None, out_dtype=np.uint8,
+           ctx: Context = None) -> np.ndarray:
+    """kernels::stackvm::conv2d(pad_mode=constant, input, weights, bias, stride, padding, dilation,
+    groups, fused_clamp) on u8 NCHW input / u8 OIHW weights / int32 bias.
+
+    out_dtype uint8 -> requantised with output_qp; int32 -> accumulators; float32 -> clamped
+    acc * (sx * sw).  Returns NCHW.
+    """
+    c = _ctx(ctx)
+    x = np.ascontiguousarray(input, np.uint8)
+    w = np.ascontiguousarray(weights, np.uint8)
+    n, ch, h, wd = x.shape
+    oc, gic, kh, kw = w.shape
+    if gic * groups != ch:
+        raise rt.HipError(-rt.ERR_SHAPE_MISMATCH, "conv2d", f"weights expect {gic * groups} input channels, input has {ch}")
+    (ph0, ph1), (pw0, pw1) = padding
+    oh = rt.windowed_output_size(h, kh, stride[0], dilation[0], ph0, ph1)
+    ow = rt.windowed_output_size(wd, kw, stride[1], dilation[1], pw0, pw1)
+    wts = c.prepack_conv2d(w, bias, weights_qp, groups)
+    x_nchw = c.to_device(x)
+    x_nhwc = c.alloc(x.size)
+    c.nchw_to_nhwc(x_nchw, x_nhwc, 1, n, ch, h, wd)
+    out_dtype = np.dtype(out_dtype)
+    es = out_dtype.itemsize
+    y_nhwc = c.alloc(max(1, n * oh * ow * oc * es))
+    y_nchw = c.alloc(max(1, n * oh * ow * oc * es))
+    args = rt.Conv2dArgs(n, h, wd, stride[0], stride[1], dilation[0], dilation[1], ph0, ph1, pw0, pw1, input_qp,
+                         output_qp or qp(0, 1.0), fused_clamp[0], fused_clamp[1], _out_dt(out_dtype))
+    c.qconv2d(x_nhwc, wts, y_nhwc, args)
+    c.nhwc_to_nchw(y_nhwc, y_nchw, es, n, oc, oh, ow)
+    out = y_nchw.download((n, oc, oh, ow), out_dtype)
+    wts.destroy()
+    return out
+
+
+def mat_mul(lhs: np.ndarray, rhs: np.ndarray, lhs_qp: QuantParam, rhs_qp: QuantParam,
+            output_qp: Optional[QuantParam] = None, out_dtype=np.float32, bias: Optional[np.ndarray] = None,
+            fused_clamp: Tuple[float, float] = (-rt.FLT_MAX, rt.FLT_MAX), ctx: Context = None) -> np.ndarray:
+    """kernels::stackvm::mat_mul(lhs, rhs) on u8 operands: lhs [..., M, K] (batch dims are
+    flattened into rows), rhs [K, N] constant."""
+    c = _ctx(ctx)
+    a = np.ascontiguousarray(lhs, np.uint8)
+    b = np.ascontiguousarray(rhs, np.uint8)
+    if b.ndim != 2 or a.ndim < 1 or a.shape[-1] != b.shape[0]:
+        raise rt.HipError(-rt.ERR_SHAPE_MISMATCH, "mat_mul", f"{a.shape} x {b.shape}")
+    k, n = b.shape
+    lead = a.shape[:-1]
+    m = int(np.prod(lead)) if lead else 1
+    out_dtype = np.dtype(out_dtype)
+    wts = c.prepack_matmul(b, bias, rhs_qp)
+    da = c.to_device(a)
+    dy = c.alloc(max(1, m * n * out_dtype.itemsize))
+    args = rt.MatmulArgs(m, lhs_qp, output_qp or qp(0, 1.0), fused_clamp[0], fused_clamp[1], _out_dt(out_dtype))
+    c.qmatmul(da, wts, dy, args)
+    out = dy.download(tuple(lead) + (n,), out_dtype)
+    wts.destroy()
+    return out
+
+
+def binary_add(lhs: np.ndarray, rhs: np.ndarray, lhs_qp: QuantParam, rhs_qp: QuantParam, output_qp: QuantParam,
+               fused_clamp: Tuple[float, float] = (-rt.FLT_MAX, rt.FLT_MAX), ctx: Context = None) -> np.ndarray:
+    """Quantize(Dequantize(lhs) + Dequantize(rhs)) on equal-shape u8 tensors."""
+    c = _ctx(ctx)
+    a, b = np.ascontiguousarray(lhs, np.uint8), np.ascontiguousarray(rhs, np.uint8)
+    if a.shape != b.shape:
+        raise rt.HipError(-rt.ERR_SHAPE_MISMATCH, "binary_add", f"{a.shape} vs {b.shape}")
+    da, db, dy = c.to_device(a), c.to_device(b), c.alloc(a.size)
+    c.qadd(da, lhs_qp, db, rhs_qp, dy, output_qp, a.size, fused_clamp)
+    return dy.download(a.shape, np.uint8)
+
+
+def global_average_pool(input: np.ndarray, input_qp: QuantParam, output_qp: QuantParam, ctx: Context = None) -> np.ndarray:
+    """reduce_window2d(mean) over the whole image of a u8 NCHW tensor -> u8 [N, C, 1, 1]."""
+    c = _ctx(ctx)
+    x = np.ascontiguousarray(input, np.uint8)
+    n, ch, h, w = x.shape
+    d_nchw, d_nhwc, dy = c.to_device(x), c.alloc(x.size), c.alloc(n * ch)
+    c.nchw_to_nhwc(d_nchw, d_nhwc, 1, n, ch, h, w)
+    c.qglobal_avgpool(d_nhwc, dy, n, h, w, ch, input_qp, output_qp)
+    return dy.download((n, ch, 1, 1), np.uint8)
+
+
+def pack(input: np.ndarray, axes: Sequence[int], lanes: Sequence[int], ctx: Context = None) -> np.ndarray:
+    c = _ctx(ctx)
+    x = np.ascontiguousarray(input)
+    nd = x.ndim
+    ax = [a % nd for a in axes]
+    out_shape = [(-(-x.shape[d] // lanes[ax.index(d)])) if d in ax else x.shape[d] for d in range(nd)] + list(lanes)
+    src, dst = c.to_device(x), c.alloc(int(np.prod(out_shape)) * x.itemsize)
+    c.pack(src, dst, x.itemsize, list(x.shape), list(axes), list(lanes))
+    return dst.download(tuple(out_shape), x.dtype)
+
+
+def unpack(input: np.ndarray, axes: Sequence[int], lanes: Sequence[int], unpacked_shape: Sequence[int],
+           ctx: Context = None) -> np.ndarray:
+    c = _ctx(ctx)
+    y = np.ascontiguousarray(input)
+    src, dst = c.to_device(y), c.alloc(int(np.prod(unpacked_shape)) * y.itemsize)
+    c.unpack(src, dst, y.itemsize, list(unpacked_shape), list(axes), list(lanes))
+    return dst.download(tuple(unpacked_shape), y.dtype)
+
+
+def transpose_nchw_to_nhwc(input: np.ndarray, ctx: Context = None) -> np.ndarray:
+    c = _ctx(ctx)
+    x = np.ascontiguousarray(input)
+    n, ch, h, w = x.shape
+    src, dst = c.to_device(x), c.alloc(x.nbytes)
+    c.nchw_to_nhwc(src, dst, x.itemsize, n, ch, h, w)
+    return dst.download((n, h, w, ch), x.dtype)
+
+
+def transpose_nhwc_to_nchw(input: np.ndarray, ctx: Context = None) -> np.ndarray:
+    c = _ctx(ctx)
+    x = np.ascontiguousarray(input)
+    n, h, w, ch = x.shape
+    src, dst = c.to_device(x), c.alloc(x.nbytes)
+    c.nhwc_to_nchw(src, dst, x.itemsize, n, ch, h, w)
+    return dst.download((n, ch, h, w), x.dtype)
+
+
+def paged_attention_decode(q: np.ndarray, k_cache: np.ndarray, v_cache: np.ndarray, block_table: np.ndarray,
+                           ctx_lens: np.ndarray, scale: float, out_dtype=np.float32, ctx: Context = None) -> np.ndarray:
+    """q [B, Hq, D] f16; caches [blocks, Hkv, block, D] f16; block_table [B, max_blocks] i32; ctx_lens [B] i32."""
+    c = _ctx(ctx)
+    qh = np.ascontiguousarray(q, np.float16)
+    kc, vc = np.ascontiguousarray(k_cache, np.float16), np.ascontiguousarray(v_cache, np.float16)
+    bt, cl = np.ascontiguousarray(block_table, np.int32), np.ascontiguousarray(ctx_lens, np.int32)
+    bsz, hq, d = qh.shape
+    nb, hkv, blk, _ = kc.shape
+    out_dtype = np.dtype(out_dtype)
+    dq, dk, dv, dbt, dcl = (c.to_device(t) for t in (qh, kc, vc, bt, cl))
+    dout = c.alloc(bsz * hq * d * out_dtype.itemsize)
+    args = rt.PagedAttnArgs(bsz, hq, hkv, d, blk, bt.shape[1], nb, float(scale), rt.NP_TO_DT[out_dtype])
+    c.paged_attention_decode(dq, dk, dv, dbt, dcl, dout, args)
+    return dout.download((bsz, hq, d), out_dtype)

@@ -1,0 +1,306 @@
+"""ctypes binding of libnncase_hip.so -- the same C ABI a C# `[DllImport("nncase_hip")]`
+or the native `hip` runtime module would bind (include/nncase_hip.h).
+
+There is no CPU fallback: if the library has not been built, or no gfx950 device is
+present, creating a Context raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import errno
+import os
+from typing import Optional, Sequence, Tuple
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libnncase_hip.so")
+
+# nncase typecodes (src/Native/include/nncase/runtime/typecodes.def)
+DT_I8, DT_I16, DT_I32, DT_U8, DT_F16, DT_F32 = 0x02, 0x03, 0x04, 0x06, 0x0A, 0x0B
+NP_TO_DT = {np.dtype(np.int8): DT_I8, np.dtype(np.int16): DT_I16, np.dtype(np.int32): DT_I32,
+            np.dtype(np.uint8): DT_U8, np.dtype(np.float16): DT_F16, np.dtype(np.float32): DT_F32}
+DT_TO_NP = {v: k for k, v in NP_TO_DT.items()}
+FLT_MAX = float(np.finfo(np.float32).max)
+
+ERR_DATATYPE_MISMATCH, ERR_SHAPE_MISMATCH, ERR_INVALID_MEMORY_LOCATION, ERR_HIP_BASE = 0x05, 0x06, 0x07, 0x1000
+
+
+class QuantParam(C.Structure):
+    """quant_param_t (src/Native/include/nncase/runtime/simple_types.h:157-165)."""
+    _fields_ = [("zero_point", C.c_int32), ("scale", C.c_float)]
+
+    def __repr__(self):
+        return f"QuantParam(zero_point={self.zero_point}, scale={self.scale!r})"
+
+
+class Conv2dDesc(C.Structure):
+    _fields_ = [("in_channels", C.c_int32), ("out_channels", C.c_int32), ("kernel_h", C.c_int32),
+                ("kernel_w", C.c_int32), ("groups", C.c_int32), ("w_qp", QuantParam)]
+
+
+class Conv2dArgs(C.Structure):
+    _fields_ = [("batch", C.c_int32), ("in_h", C.c_int32), ("in_w", C.c_int32),
+                ("stride_h", C.c_int32), ("stride_w", C.c_int32),
+                ("dilation_h", C.c_int32), ("dilation_w", C.c_int32),
+                ("pad_h_before", C.c_int32), ("pad_h_after", C.c_int32),
+                ("pad_w_before", C.c_int32), ("pad_w_after", C.c_int32),
+                ("x_qp", QuantParam), ("y_qp", QuantParam),
+                ("clamp_min", C.c_float), ("clamp_max", C.c_float), ("out_dtype", C.c_int32)]
+
+
+class MatmulArgs(C.Structure):
+    _fields_ = [("m", C.c_int32), ("a_qp", QuantParam), ("y_qp", QuantParam),
+                ("clamp_min", C.c_float), ("clamp_max", C.c_float), ("out_dtype", C.c_int32)]
+
+
+class PagedAttnArgs(C.Structure):
+    _fields_ = [("batch", C.c_int32), ("num_q_heads", C.c_int32), ("num_kv_heads", C.c_int32),
+                ("head_dim", C.c_int32), ("block_size", C.c_int32), ("max_blocks_per_seq", C.c_int32),
+                ("num_blocks", C.c_int32), ("scale", C.c_float), ("out_dtype", C.c_int32)]
+
+
+# name -> (restype, argtypes); every symbol include/nncase_hip.h declares
+_VP, _I, _SZ = C.c_void_p, C.c_int, C.c_size_t
+_I32P = C.POINTER(C.c_int32)
+SYMBOLS = {
+    "nncase_hip_version": (_I, []),
+    "nncase_hip_ctx_create": (_I, [_I, C.POINTER(_VP)]),
+    "nncase_hip_ctx_destroy": (_I, [_VP]),
+    "nncase_hip_ctx_get_stream": (_I, [_VP, C.POINTER(_VP)]),
+    "nncase_hip_ctx_set_stream": (_I, [_VP, _VP]),
+    "nncase_hip_last_error_string": (C.c_char_p, [_VP]),
+    "nncase_hip_device_info": (_I, [_VP, C.POINTER(_I), C.POINTER(_I), C.POINTER(_SZ)]),
+    "nncase_hip_malloc": (_I, [_VP, _SZ, C.POINTER(_VP)]),
+    "nncase_hip_free": (_I, [_VP, _VP]),
+    "nncase_hip_memcpy_h2d": (_I, [_VP, _VP, _VP, _SZ]),
+    "nncase_hip_memcpy_d2h": (_I, [_VP, _VP, _VP, _SZ]),
+    "nncase_hip_memset": (_I, [_VP, _VP, _I, _SZ]),
+    "nncase_hip_stream_sync": (_I, [_VP]),
+    "nncase_hip_quantize": (_I, [_VP, _VP, _I, _VP, _I, _SZ, QuantParam]),
+    "nncase_hip_dequantize": (_I, [_VP, _VP, _I, _VP, _I, _SZ, QuantParam]),
+    "nncase_hip_qconv2d_prepack": (_I, [_VP, C.POINTER(Conv2dDesc), _VP, _VP, C.POINTER(_VP)]),
+    "nncase_hip_weights_destroy": (_I, [_VP, _VP]),
+    "nncase_hip_qconv2d": (_I, [_VP, _VP, _VP, _VP, C.POINTER(Conv2dArgs)]),
+    "nncase_hip_qmatmul_prepack": (_I, [_VP, _VP, C.c_int32, C.c_int32, QuantParam, _VP, C.POINTER(_VP)]),
+    "nncase_hip_qmatmul": (_I, [_VP, _VP, _VP, _VP, C.POINTER(MatmulArgs)]),
+    "nncase_hip_qadd": (_I, [_VP, _VP, QuantParam, _VP, QuantParam, _VP, QuantParam, C.c_float, C.c_float, _SZ]),
+    "nncase_hip_qglobal_avgpool": (_I, [_VP, _VP, _VP, C.c_int32, C.c_int32, C.c_int32, C.c_int32, QuantParam,
+                                        QuantParam]),
+    "nncase_hip_pack": (_I, [_VP, _VP, _VP, C.c_int32, C.c_int32, _I32P, C.c_int32, _I32P, _I32P]),
+    "nncase_hip_unpack": (_I, [_VP, _VP, _VP, C.c_int32, C.c_int32, _I32P, C.c_int32, _I32P, _I32P]),
+    "nncase_hip_nchw_to_nhwc": (_I, [_VP, _VP, _VP, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
+    "nncase_hip_nhwc_to_nchw": (_I, [_VP, _VP, _VP, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
+    "nncase_hip_paged_attention_decode": (_I, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, C.POINTER(PagedAttnArgs)]),
+}
+
+_lib: Optional[C.CDLL] = None
+
+
+def load_library() -> C.CDLL:
+    """Loads the built library; raises if it has not been built (no fallback)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(f"{LIB_PATH} is missing: build it with `python -m nncase_amd.build` "
+                               "(there is no CPU fallback for the hip target)")
+        lib = C.CDLL(LIB_PATH)
+        for name, (res, args) in SYMBOLS.items():
+            fn = getattr(lib, name)  # AttributeError if the export is missing
+            fn.restype, fn.argtypes = res, args
+        _lib = lib
+    return _lib
+
+
+class HipError(RuntimeError):
+    """Mirrors the C# interop's `InvalidOperationException("Status code: N")`
+    (src/Nncase.Simulator/Runtime/Interop/ErrorCode.cs:25-31)."""
+
+    def __init__(self, code: int, where: str, detail: str = ""):
+        self.code = code
+        name = errno.errorcode.get(-code, "") if -code < ERR_HIP_BASE else f"hipError {-code - ERR_HIP_BASE}"
+        super().__init__(f"{where}: status code {code} {name} {detail}".strip())
+
+
+def qp(zero_point: int, scale: float) -> QuantParam:
+    return QuantParam(int(zero_point), float(np.float32(scale)))
+
+
+class DeviceBuffer:
+    """An HBM allocation owned through the context (nncase_hip_malloc / _free)."""
+
+    def __init__(self, ctx: "Context", nbytes: int):
+        self.ctx, self.nbytes = ctx, int(nbytes)
+        p = C.c_void_p()
+        ctx._check(ctx.lib.nncase_hip_malloc(ctx.handle, max(1, self.nbytes), C.byref(p)), "malloc")
+        self.ptr = p.value
+
+    def upload(self, arr: np.ndarray) -> "DeviceBuffer":
+        arr = np.ascontiguousarray(arr)
+        assert arr.nbytes <= self.nbytes
+        self.ctx._check(self.ctx.lib.nncase_hip_memcpy_h2d(self.ctx.handle, self.ptr, arr.ctypes.data, arr.nbytes), "h2d")
+        return self
+
+    def download(self, shape, dtype) -> np.ndarray:
+        out = np.empty(shape, dtype)
+        assert out.nbytes <= self.nbytes
+        self.ctx._check(self.ctx.lib.nncase_hip_memcpy_d2h(self.ctx.handle, out.ctypes.data, self.ptr, out.nbytes), "d2h")
+        return out
+
+    def fill(self, byte: int) -> "DeviceBuffer":
+        self.ctx._check(self.ctx.lib.nncase_hip_memset(self.ctx.handle, self.ptr, byte, self.nbytes), "memset")
+        return self
+
+    def free(self):
+        if self.ptr:
+            self.ctx.lib.nncase_hip_free(self.ctx.handle, self.ptr)
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class Weights:
+    """Pre-packed constants of one conv / matmul (nncase_hip_weights_t)."""
+
+    def __init__(self, ctx: "Context", handle, out_channels: int, kernel: Tuple[int, int], in_channels: int, groups: int):
+        self.ctx, self.handle = ctx, handle
+        self.out_channels, self.kernel, self.in_channels, self.groups = out_channels, kernel, in_channels, groups
+
+    def destroy(self):
+        if self.handle:
+            self.ctx.lib.nncase_hip_weights_destroy(self.ctx.handle, self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass
+
+
+def windowed_output_size(size, filt, stride, dilation, before, after) -> int:
+    """src/Native/include/nncase/kernels/kernel_utils.h:86-93."""
+    eff = (filt - 1) * dilation + 1
+    return (size + before + after - eff + stride) // stride
+
+
+class Context:
+    """One device + stream (nncase_hip_ctx_t)."""
+
+    def __init__(self, device: int = 0):
+        self.lib = load_library()
+        h = C.c_void_p()
+        rc = self.lib.nncase_hip_ctx_create(device, C.byref(h))
+        if rc != 0:
+            raise HipError(rc, "nncase_hip_ctx_create", "(no gfx950 device?)")
+        self.handle = h.value
+        cu, khz, mem = C.c_int(), C.c_int(), C.c_size_t()
+        self.lib.nncase_hip_device_info(self.handle, C.byref(cu), C.byref(khz), C.byref(mem))
+        self.compute_units, self.clock_khz, self.hbm_bytes = cu.value, khz.value, mem.value
+
+    # -- plumbing ---------------------------------------------------------------------
+    def _check(self, rc: int, where: str):
+        if rc != 0:
+            msg = self.lib.nncase_hip_last_error_string(self.handle)
+            raise HipError(rc, where, msg.decode() if msg else "")
+
+    def close(self):
+        if getattr(self, "handle", None):
+            self.lib.nncase_hip_ctx_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    @property
+    def stream(self) -> int:
+        s = C.c_void_p()
+        self._check(self.lib.nncase_hip_ctx_get_stream(self.handle, C.byref(s)), "get_stream")
+        return s.value or 0
+
+    def set_stream(self, hip_stream: int):
+        self._check(self.lib.nncase_hip_ctx_set_stream(self.handle, C.c_void_p(hip_stream)), "set_stream")
+
+    def sync(self):
+        self._check(self.lib.nncase_hip_stream_sync(self.handle), "stream_sync")
+
+    def alloc(self, nbytes: int) -> DeviceBuffer:
+        return DeviceBuffer(self, nbytes)
+
+    def to_device(self, arr: np.ndarray) -> DeviceBuffer:
+        arr = np.ascontiguousarray(arr)
+        return DeviceBuffer(self, arr.nbytes).upload(arr)
+
+    # -- operators (raw device pointers) ----------------------------------------------
+    def quantize(self, src: DeviceBuffer, in_dtype: int, dst: DeviceBuffer, out_dtype: int, count: int, q: QuantParam):
+        self._check(self.lib.nncase_hip_quantize(self.handle, src.ptr, in_dtype, dst.ptr, out_dtype, count, q), "quantize")
+
+    def dequantize(self, src: DeviceBuffer, in_dtype: int, dst: DeviceBuffer, out_dtype: int, count: int, q: QuantParam):
+        self._check(self.lib.nncase_hip_dequantize(self.handle, src.ptr, in_dtype, dst.ptr, out_dtype, count, q),
+                    "dequantize")
+
+    def prepack_conv2d(self, weights_oihw: np.ndarray, bias: Optional[np.ndarray], w_qp: QuantParam, groups: int = 1) -> Weights:
+        w = np.ascontiguousarray(weights_oihw, np.uint8)
+        oc, gic, kh, kw = w.shape
+        desc = Conv2dDesc(gic * groups, oc, kh, kw, groups, w_qp)
+        b = None if bias is None else np.ascontiguousarray(bias, np.int32)
+        if b is not None:
+            assert b.shape == (oc,)
+        h = C.c_void_p()
+        self._check(self.lib.nncase_hip_qconv2d_prepack(self.handle, C.byref(desc), w.ctypes.data,
+                                                        None if b is None else b.ctypes.data, C.byref(h)), "qconv2d_prepack")
+        return Weights(self, h.value, oc, (kh, kw), gic * groups, groups)
+
+    def qconv2d(self, x: DeviceBuffer, w: Weights, y: DeviceBuffer, args: Conv2dArgs):
+        self._check(self.lib.nncase_hip_qconv2d(self.handle, x.ptr, w.handle, y.ptr, C.byref(args)), "qconv2d")
+
+    def prepack_matmul(self, b_kn: np.ndarray, bias: Optional[np.ndarray], b_qp: QuantParam) -> Weights:
+        b = np.ascontiguousarray(b_kn, np.uint8)
+        k, n = b.shape
+        bi = None if bias is None else np.ascontiguousarray(bias, np.int32)
+        h = C.c_void_p()
+        self._check(self.lib.nncase_hip_qmatmul_prepack(self.handle, b.ctypes.data, k, n, b_qp,
+                                                        None if bi is None else bi.ctypes.data, C.byref(h)), "qmatmul_prepack")
+        return Weights(self, h.value, n, (1, 1), k, 1)
+
+    def qmatmul(self, a: DeviceBuffer, w: Weights, y: DeviceBuffer, args: MatmulArgs):
+        self._check(self.lib.nncase_hip_qmatmul(self.handle, a.ptr, w.handle, y.ptr, C.byref(args)), "qmatmul")
+
+    def qadd(self, a: DeviceBuffer, a_qp, b: DeviceBuffer, b_qp, out: DeviceBuffer, y_qp, count: int,
+             clamp=(-FLT_MAX, FLT_MAX)):
+        self._check(self.lib.nncase_hip_qadd(self.handle, a.ptr, a_qp, b.ptr, b_qp, out.ptr, y_qp, clamp[0], clamp[1], count),
+                    "qadd")
+
+    def qglobal_avgpool(self, x: DeviceBuffer, out: DeviceBuffer, batch, h, w, channels, x_qp, y_qp):
+        self._check(self.lib.nncase_hip_qglobal_avgpool(self.handle, x.ptr, out.ptr, batch, h, w, channels, x_qp, y_qp),
+                    "qglobal_avgpool")
+
+    def pack(self, src: DeviceBuffer, dst: DeviceBuffer, elem_size: int, shape: Sequence[int], axes: Sequence[int],
+             lanes: Sequence[int]):
+        sh, ax, ln = (C.c_int32 * len(shape))(*shape), (C.c_int32 * max(1, len(axes)))(*axes), (C.c_int32 * max(1, len(lanes)))(*lanes)
+        self._check(self.lib.nncase_hip_pack(self.handle, src.ptr, dst.ptr, elem_size, len(shape), sh, len(axes), ax, ln), "pack")
+
+    def unpack(self, src: DeviceBuffer, dst: DeviceBuffer, elem_size: int, unpacked_shape: Sequence[int],
+               axes: Sequence[int], lanes: Sequence[int]):
+        sh = (C.c_int32 * len(unpacked_shape))(*unpacked_shape)
+        ax, ln = (C.c_int32 * max(1, len(axes)))(*axes), (C.c_int32 * max(1, len(lanes)))(*lanes)
+        self._check(self.lib.nncase_hip_unpack(self.handle, src.ptr, dst.ptr, elem_size, len(unpacked_shape), sh, len(axes),
+                                               ax, ln), "unpack")
+
+    def nchw_to_nhwc(self, src: DeviceBuffer, dst: DeviceBuffer, elem_size, n, c, h, w):
+        self._check(self.lib.nncase_hip_nchw_to_nhwc(self.handle, src.ptr, dst.ptr, elem_size, n, c, h, w), "nchw_to_nhwc")
+
+    def nhwc_to_nchw(self, src: DeviceBuffer, dst: DeviceBuffer, elem_size, n, c, h, w):
+        self._check(self.lib.nncase_hip_nhwc_to_nchw(self.handle, src.ptr, dst.ptr, elem_size, n, c, h, w), "nhwc_to_nchw")
+
+    def paged_attention_decode(self, q: DeviceBuffer, k_cache: DeviceBuffer, v_cache: DeviceBuffer,
+                               block_table: DeviceBuffer, ctx_lens: DeviceBuffer, out: DeviceBuffer, args: PagedAttnArgs):
+        self._check(self.lib.nncase_hip_paged_attention_decode(self.handle, q.ptr, k_cache.ptr, v_cache.ptr, block_table.ptr,
+                                                               ctx_lens.ptr, out.ptr, C.byref(args)), "paged_attention_decode")
