@@ -1,0 +1,250 @@
+"""GPU parity: u8/u8 conv2d (dense, grouped, depthwise) and matmul through the C ABI vs
+the CPU oracle.  int32 accumulators, clamped fp32 values and requantised u8 bytes are all
+compared bit-exactly: the fp32 epilogue is the same sequence of single IEEE operations on
+both sides."""
+import itertools
+import zlib
+
+import numpy as np
+import pytest
+
+from nncase_amd import kernels as K
+from nncase_amd import quant
+from nncase_amd import runtime as rt
+from nncase_amd.runtime import qp
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+f32 = np.float32
+FULL = (-rt.FLT_MAX, rt.FLT_MAX)
+
+
+def same_padding(size, k, stride, dilation):
+    """TF 'SAME' padding as nncase's importer computes it (Util.GetPaddings)."""
+    out = -(-size // stride)
+    eff = (k - 1) * dilation + 1
+    total = max((out - 1) * stride + eff - size, 0)
+    return (total // 2, total - total // 2)
+
+
+def run_case(ctx, n, c, h, w, oc, kh, kw, stride, pad, dil, groups, seed, zx=7, zw=131, clamp=None, modes=("u8", "i32", "f32")):
+    rng = np.random.default_rng(seed)
+    x = rng.integers(0, 256, (n, c, h, w), dtype=np.uint8)
+    wt = rng.integers(0, 256, (oc, c // groups, kh, kw), dtype=np.uint8)
+    bias = rng.integers(-3000, 3000, oc).astype(np.int32)
+    sx, sw = f32(0.0235), f32(0.0041)
+    common = dict(stride=stride, padding=pad, dilation=dil, groups=groups)
+    # the real-valued output decides the clamp and the output quantisation, so that the
+    # requantiser sees values spread over (and beyond) the u8 range whatever the shape is
+    real = O.qconv2d(x, wt, bias, zx, sx, zw, sw, out_mode=O.OUT_F32, **common)
+    if clamp is not FULL:
+        lo, hi = np.percentile(real, [10, 90]).astype(f32)
+        clamp = (float(lo), float(hi)) if hi > lo else FULL
+    span = float(real.max() - real.min()) or 1.0
+    sy = f32(span * 0.7 / 255)
+    zy_free = int(np.rint(-40 - real.min() / sy))  # puts the smallest value 40 codes below 0
+    zy = int(np.clip(zy_free, 0, 255))
+    if "i32" in modes:
+        got = K.conv2d(x, wt, bias, stride, pad, dil, groups, FULL, qp(zx, sx), qp(zw, sw), None, np.int32, ctx=ctx)
+        want = O.qconv2d(x, wt, bias, zx, sx, zw, sw, out_mode=O.OUT_I32, **common)
+        assert got.shape == want.shape
+        assert np.array_equal(got, want), f"int32 accumulators differ in {(got != want).sum()} of {got.size}"
+    if "f32" in modes:
+        got = K.conv2d(x, wt, bias, stride, pad, dil, groups, clamp, qp(zx, sx), qp(zw, sw), None, np.float32, ctx=ctx)
+        want = O.qconv2d(x, wt, bias, zx, sx, zw, sw, fused_clamp=clamp, out_mode=O.OUT_F32, **common)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    if "u8" in modes:
+        for cl in (clamp, FULL):
+            got = K.conv2d(x, wt, bias, stride, pad, dil, groups, cl, qp(zx, sx), qp(zw, sw), qp(zy, sy), np.uint8, ctx=ctx)
+            want = O.qconv2d(x, wt, bias, zx, sx, zw, sw, zy, sy, fused_clamp=cl, out_mode=O.OUT_U8, **common)
+            assert np.array_equal(got, want), f"u8 outputs differ in {(got != want).sum()} of {got.size}"
+        if len(np.unique(real)) > 64 and zy == zy_free:
+            assert len(np.unique(want)) > 8  # the case really exercises the requantiser
+
+
+# ---- reference grids ----------------------------------------------------------------------------
+# tests/importer/tflite_/basic/test_depthwise_conv2d.py: n {1,3}, C {1,16}, HxW {1x1, 33x65}, k {1,3,5},
+# stride {[1,1],[1,3]}, padding {SAME, VALID}
+DW_GRID = [(n, c, hw, k, s, p) for n, c, hw, k, s, p in itertools.product(
+    (1, 3), (1, 16), ((1, 1), (33, 65)), (1, 3, 5), ((1, 1), (1, 3)), ("SAME", "VALID"))
+    if not (p == "VALID" and hw == (1, 1) and k > 1)]
+
+
+@pytest.mark.parametrize("n,c,hw,k,stride,padding", DW_GRID)
+def test_depthwise_reference_grid(hip_ctx, n, c, hw, k, stride, padding):
+    h, w = hw
+    pad = (same_padding(h, k, stride[0], 1), same_padding(w, k, stride[1], 1)) if padding == "SAME" else ((0, 0), (0, 0))
+    run_case(hip_ctx, n, c, h, w, c, k, k, stride, pad, (1, 1), c, seed=zlib.crc32(repr((n, c, hw, k, stride, padding)).encode()))
+
+
+# tests/importer/tflite_/basic/test_conv2d.py: same plus stride [5,5] and dilation [2,2]
+CONV_GRID = [(n, c, hw, k, s, d, p) for n, c, hw, k, s, d, p in itertools.product(
+    (1, 3), (1, 16), ((1, 1), (33, 65)), (1, 3, 5), ((1, 1), (1, 3), (5, 5)), ((1, 1), (2, 2)), ("SAME", "VALID"))
+    if not (p == "VALID" and hw == (1, 1) and k > 1) and not (d == (2, 2) and s != (1, 1))]
+
+
+@pytest.mark.parametrize("n,c,hw,k,stride,dil,padding", CONV_GRID)
+def test_conv2d_reference_grid(hip_ctx, n, c, hw, k, stride, dil, padding):
+    h, w = hw
+    pad = (same_padding(h, k, stride[0], dil[0]), same_padding(w, k, stride[1], dil[1])) if padding == "SAME" else ((0, 0), (0, 0))
+    eff = (k - 1) * dil[0] + 1
+    if padding == "VALID" and (eff > h or eff > w):
+        pytest.skip("window larger than the image")
+    run_case(hip_ctx, n, c, h, w, 8, k, k, stride, pad, dil, 1, seed=zlib.crc32(repr((n, c, hw, k, stride, dil, padding)).encode()),
+             modes=("u8", "i32"))
+
+
+# tests/kernels/test_conv2d.json + tests/importer/onnx_/basic/test_conv.py
+@pytest.mark.parametrize("case", [
+    (1, 4, 5, 5, 8, 3, (1, 1), ((1, 1), (1, 1)), (1, 1), 1),
+    (1, 4, 16, 16, 8, 1, (2, 2), ((1, 1), (1, 1)), (1, 1), 1),
+    (1, 4, 16, 16, 8, 3, (2, 2), ((1, 1), (1, 1)), (2, 2), 1),
+    (1, 3, 16, 16, 5, 3, (2, 2), ((0, 1), (0, 1)), (2, 2), 1),   # SAME_UPPER-like
+    (1, 3, 16, 16, 5, 3, (2, 2), ((1, 0), (1, 0)), (1, 1), 1),   # SAME_LOWER-like
+    (2, 6, 9, 7, 4, 3, (5, 5), ((0, 2), (1, 0)), (1, 1), 2),     # grouped, asymmetric padding
+    (1, 32, 10, 10, 48, 3, (1, 1), ((1, 1), (1, 1)), (1, 1), 4), # grouped with 8 channels per group
+    (1, 16, 6, 6, 32, 3, (1, 1), ((1, 1), (1, 1)), (1, 1), 16),  # depthwise with multiplier 2
+])
+def test_conv2d_kernel_grid(hip_ctx, case):
+    n, c, h, w, oc, k, stride, pad, dil, groups = case
+    run_case(hip_ctx, n, c, h, w, oc, k, k, stride, pad, dil, groups, seed=sum(case[:6]))
+
+
+# ---- shapes of the benchmark configurations ------------------------------------------------------
+# every distinct (Cin, Cout) pointwise layer of MobileNetV2 on a small image, plus stem / depthwise / FC shapes
+MBV2_PW = [(32, 16), (16, 96), (96, 24), (24, 144), (144, 24), (144, 32), (32, 192), (192, 32), (192, 64), (64, 384),
+           (384, 64), (384, 96), (96, 576), (576, 96), (576, 160), (160, 960), (960, 160), (960, 320), (320, 1280)]
+
+
+@pytest.mark.parametrize("cin,cout", MBV2_PW)
+def test_mobilenet_pointwise_shapes(hip_ctx, cin, cout):
+    # 2 x 13 x 11 = 286 pixels: not a multiple of the pixel tile, exercises the ragged last tile
+    run_case(hip_ctx, 2, cin, 13, 11, cout, 1, 1, (1, 1), ((0, 0), (0, 0)), (1, 1), 1, seed=cin * 7 + cout, modes=("u8", "i32"))
+
+
+def test_mobilenet_stem_fc_and_depthwise_shapes(hip_ctx):
+    run_case(hip_ctx, 2, 3, 32, 32, 32, 3, 3, (2, 2), ((0, 1), (0, 1)), (1, 1), 1, seed=1)           # stem 3x3 s2, 3 channels
+    run_case(hip_ctx, 4, 1280, 1, 1, 1000, 1, 1, (1, 1), ((0, 0), (0, 0)), (1, 1), 1, seed=2, clamp=FULL)  # FC as 1x1
+    for c, s, hw in ((32, 1, 28), (96, 2, 28), (144, 1, 14), (192, 2, 14), (576, 1, 7), (960, 1, 7)):
+        pad = ((1, 1), (1, 1)) if s == 1 else ((0, 1), (0, 1))
+        run_case(hip_ctx, 2, c, hw, hw, c, 3, 3, (s, s), pad, (1, 1), c, seed=c + s)
+
+
+def test_large_reduction_stages_weights_through_lds_in_chunks(hip_ctx):
+    # 3x3 over 256 channels: K = 2304 (36 k-steps) -> weights staged in several LDS chunks
+    run_case(hip_ctx, 1, 256, 10, 10, 64, 3, 3, (1, 1), ((1, 1), (1, 1)), (1, 1), 1, seed=3, modes=("u8", "i32"))
+    run_case(hip_ctx, 1, 128, 12, 12, 256, 3, 3, (2, 2), ((1, 1), (1, 1)), (1, 1), 1, seed=4, modes=("u8",))
+
+
+def test_extreme_values_and_zero_points(hip_ctx):
+    for zx, zw in ((0, 0), (255, 255), (0, 255), (128, 128), (1, 254)):
+        for fill_x, fill_w in ((0, 0), (255, 255), (255, 0), (0, 255)):
+            x = np.full((1, 64, 4, 4), fill_x, np.uint8)
+            w = np.full((16, 64, 3, 3), fill_w, np.uint8)
+            args = ((1, 1), ((1, 1), (1, 1)), (1, 1), 1, FULL, qp(zx, 1.0), qp(zw, 1.0), None, np.int32)
+            got = K.conv2d(x, w, None, *args, ctx=hip_ctx)
+            want = O.qconv2d(x, w, None, zx, 1.0, zw, 1.0, stride=(1, 1), padding=((1, 1), (1, 1)), out_mode=O.OUT_I32)
+            assert np.array_equal(got, want)
+
+
+def test_config2_conv_block(hip_ctx):
+    """BASELINE config 2 at batch 1: 1x1 64->144, 3x3 depthwise, 1x1 144->64 on 56x56, ReLU6, per-tensor PTQ."""
+    rng = np.random.default_rng(1)
+    xf = rng.random((1, 64, 56, 56), dtype=f32)
+    zx, sx = quant.get_quant_param((xf.min(), xf.max()))
+    x = O.quantize(xf, sx, zx)
+
+    def kaiming(shape):
+        fan_in = shape[1] * shape[2] * shape[3]
+        return (rng.standard_normal(shape) * np.sqrt(2.0 / fan_in)).astype(f32)
+
+    stages = [(kaiming((144, 64, 1, 1)), 1, ((0, 0), (0, 0))), (kaiming((144, 1, 3, 3)), 144, ((1, 1), (1, 1))),
+              (kaiming((64, 144, 1, 1)), 1, ((0, 0), (0, 0)))]
+    cur, cur_qp = x, (zx, sx)
+    for wf, groups, pad in stages:
+        wq, zw, sw = quant.quantize_weights(wf)
+        bq = np.rint(rng.standard_normal(wf.shape[0]) * 0.01 / (cur_qp[1] * sw)).astype(np.int32)
+        yq = quant.get_quant_param((0.0, 6.0))
+        want = O.qconv2d(cur, wq, bq, cur_qp[0], cur_qp[1], zw, sw, yq[0], yq[1], padding=pad, groups=groups, fused_clamp=(0.0, 6.0))
+        got = K.conv2d(cur, wq, bq, (1, 1), pad, (1, 1), groups, (0.0, 6.0), qp(*cur_qp), qp(zw, sw), qp(*yq), np.uint8, ctx=hip_ctx)
+        assert np.array_equal(got, want)
+        chain = O.qconv2d_float_chain(cur, wq, bq, cur_qp[0], cur_qp[1], zw, sw, yq[0], yq[1], padding=pad, groups=groups,
+                                      fused_clamp=(0.0, 6.0))
+        d = np.abs(got.astype(np.int32) - chain.astype(np.int32))
+        assert d.max() <= 1 and O.cosine(got, chain) > 0.999  # the reference's own bar is cosine >= 0.98 with PTQ
+        cur, cur_qp = got, yq
+
+
+# ---- matmul --------------------------------------------------------------------------------------
+def test_config1_matmul(hip_ctx):
+    """BASELINE config 1: A[512,1024] u8 (0.02, 128) x B[1024,1024] u8 per-tensor asymmetric -> fp32."""
+    rng = np.random.default_rng(0)
+    a = rng.integers(0, 256, (512, 1024), dtype=np.uint8)
+    bq, zb, sb = quant.quantize_weights((rng.standard_normal((1024, 1024)) * 0.05).astype(f32))
+    acc = K.mat_mul(a, bq, qp(128, 0.02), qp(zb, sb), None, np.int32, ctx=hip_ctx)
+    assert np.array_equal(acc, O.qmatmul(a, bq, None, 128, 0.02, zb, sb, out_mode=O.OUT_I32))
+    out = K.mat_mul(a, bq, qp(128, 0.02), qp(zb, sb), None, np.float32, ctx=hip_ctx)
+    want = O.qmatmul(a, bq, None, 128, 0.02, zb, sb, out_mode=O.OUT_F32)
+    assert np.array_equal(out.view(np.uint32), want.view(np.uint32))
+    # against what the CPU target computes (float matmul of dequantised operands): north-star tolerance 1e-3 relative
+    ref = O.matmul_f32(O.dequantize(a[:64], 0.02, 128), O.dequantize(bq, sb, zb))
+    np.testing.assert_allclose(out[:64], ref, rtol=1e-3, atol=1e-3 * np.abs(ref).max())
+
+
+@pytest.mark.parametrize("m,k,n", [(1, 6, 3), (6, 6, 1), (7, 70, 13), (130, 257, 100), (33, 64, 1000), (3, 1, 5)])
+def test_matmul_shapes(hip_ctx, m, k, n):
+    rng = np.random.default_rng(m * 100 + n)
+    a = rng.integers(0, 256, (m, k), dtype=np.uint8)
+    b = rng.integers(0, 256, (k, n), dtype=np.uint8)
+    bias = rng.integers(-500, 500, n).astype(np.int32)
+    got = K.mat_mul(a, b, qp(9, 0.02), qp(200, 0.003), None, np.int32, bias=bias, ctx=hip_ctx)
+    assert np.array_equal(got, O.qmatmul(a, b, bias, 9, 0.02, 200, 0.003))
+    gotq = K.mat_mul(a, b, qp(9, 0.02), qp(200, 0.003), qp(128, 0.5), np.uint8, bias=bias, ctx=hip_ctx)
+    assert np.array_equal(gotq, O.qmatmul(a, b, bias, 9, 0.02, 200, 0.003, 128, 0.5, out_mode=O.OUT_U8))
+
+
+def test_matmul_batched_lhs_is_flattened(hip_ctx):
+    # the reference broadcasts rank<=4 batches of lhs against a constant rhs: rows are independent
+    rng = np.random.default_rng(77)
+    a = rng.integers(0, 256, (2, 3, 6, 6), dtype=np.uint8)
+    b = rng.integers(0, 256, (6, 3), dtype=np.uint8)
+    got = K.mat_mul(a, b, qp(1, 1.0), qp(2, 1.0), None, np.int32, ctx=hip_ctx)
+    want = (a.astype(np.int64) - 1) @ (b.astype(np.int64) - 2)
+    assert got.shape == (2, 3, 6, 3) and np.array_equal(got, want)
+
+
+def test_linearity_at_full_size(hip_ctx):
+    """Size-independent check at a BASELINE-sized layer (56x56x24 -> 144, batch 32): with zero
+    points 0, acc(x1 + x2) == acc(x1) + acc(x2), and acc(x, w = 1) is the per-pixel channel sum."""
+    rng = np.random.default_rng(5)
+    n, c, hw, oc = 32, 24, 56, 144
+    x1 = rng.integers(0, 128, (n, c, hw, hw), dtype=np.uint8)
+    x2 = rng.integers(0, 128, (n, c, hw, hw), dtype=np.uint8)
+    w = rng.integers(0, 256, (oc, c, 1, 1), dtype=np.uint8)
+    args = ((1, 1), ((0, 0), (0, 0)), (1, 1), 1, FULL, qp(0, 1.0), qp(0, 1.0), None, np.int32)
+    a1 = K.conv2d(x1, w, None, *args, ctx=hip_ctx)
+    a2 = K.conv2d(x2, w, None, *args, ctx=hip_ctx)
+    a12 = K.conv2d(x1 + x2, w, None, *args, ctx=hip_ctx)
+    assert np.array_equal(a12, a1 + a2)
+    ones = K.conv2d(x1, np.ones_like(w), None, *args, ctx=hip_ctx)
+    assert np.array_equal(ones[:, 0], x1.astype(np.int32).sum(1)) and np.array_equal(ones[:, 0], ones[:, oc - 1])
+
+
+def test_error_paths(hip_ctx):
+    x = np.zeros((1, 8, 4, 4), np.uint8)
+    w = np.zeros((4, 8, 3, 3), np.uint8)
+    with pytest.raises(rt.HipError) as e:   # window larger than the padded input
+        K.conv2d(x[:, :, :2, :2], w, None, (1, 1), ((0, 0), (0, 0)), (1, 1), 1, FULL, qp(0, 1), qp(0, 1), None, np.int32, ctx=hip_ctx)
+    assert e.value.code == -rt.ERR_SHAPE_MISMATCH
+    with pytest.raises(rt.HipError) as e:   # channel mismatch
+        K.conv2d(x, np.zeros((4, 6, 3, 3), np.uint8), None, (1, 1), ((0, 0), (0, 0)), (1, 1), 1, FULL, qp(0, 1), qp(0, 1), None, np.int32, ctx=hip_ctx)
+    assert e.value.code == -rt.ERR_SHAPE_MISMATCH
+    with pytest.raises(rt.HipError) as e:   # groups do not divide channels
+        hip_ctx.prepack_conv2d(np.zeros((4, 3, 1, 1), np.uint8), None, qp(0, 1), groups=3)
+    assert e.value.code == -rt.ERR_SHAPE_MISMATCH
+    with pytest.raises(rt.HipError) as e:   # output scale must be positive for u8 output
+        K.conv2d(x, w, None, (1, 1), ((1, 1), (1, 1)), (1, 1), 1, FULL, qp(0, 1), qp(0, 1), qp(0, 0.0), np.uint8, ctx=hip_ctx)
+    assert e.value.code == -22
+    with pytest.raises(rt.HipError) as e:   # zero point outside u8
+        K.conv2d(x, w, None, (1, 1), ((1, 1), (1, 1)), (1, 1), 1, FULL, qp(300, 1), qp(0, 1), None, np.int32, ctx=hip_ctx)
+    assert e.value.code == -22

@@ -1,0 +1,45 @@
+"""GPU parity: pack / unpack and NCHW<->NHWC relayout (pure permutations, bit-exact)."""
+import numpy as np
+import pytest
+
+from nncase_amd import kernels as K
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("shape,axes,lanes,dtype", [
+    ((2, 64, 3, 5), [1], [32], np.uint8),          # NCHW -> NC/32 HW 32
+    ((2, 5, 3, 7), [1], [4], np.uint8),            # ragged: 5 channels into lanes of 4
+    ((6, 10), [1, 0], [4, 2], np.float32),         # two axes, lanes appended in the listed order
+    ((1024, 144), [0, 1], [16, 64], np.uint8),     # [K, N] -> weight-tile style blocking
+    ((3, 1, 17), [2], [8], np.float16),
+    ((7,), [0], [16], np.int32),
+    ((2, 3, 4, 5, 6), [-1, 1], [4, 2], np.uint8),
+])
+def test_pack_unpack(hip_ctx, shape, axes, lanes, dtype):
+    rng = np.random.default_rng(len(shape) + shape[0])
+    x = rng.integers(1, 120, shape).astype(dtype)
+    y = K.pack(x, axes, lanes, ctx=hip_ctx)
+    want = O.pack(x, axes, lanes)
+    assert y.shape == want.shape and np.array_equal(y.view(np.uint8), want.view(np.uint8))
+    back = K.unpack(y, axes, lanes, shape, ctx=hip_ctx)
+    assert np.array_equal(back.view(np.uint8), x.view(np.uint8))
+
+
+def test_pack_roundtrip_full_size(hip_ctx):
+    # round trip at a BASELINE size (batch-32 conv-block activation), ragged lanes
+    x = (np.arange(32 * 144 * 56 * 56, dtype=np.uint32) * 2654435761 >> 11).astype(np.uint8).reshape(32, 144, 56, 56)
+    y = K.pack(x, [1], [64], ctx=hip_ctx)
+    assert y.shape == (32, 3, 56, 56, 64) and (y[:, 2, :, :, 16:] == 0).all()
+    assert np.array_equal(K.unpack(y, [1], [64], x.shape, ctx=hip_ctx), x)
+
+
+@pytest.mark.parametrize("shape", [(1, 3, 224, 224), (2, 144, 7, 5), (3, 1, 1, 1), (1, 33, 65, 2)])
+@pytest.mark.parametrize("dtype", [np.uint8, np.float16, np.float32])
+def test_nchw_nhwc(hip_ctx, shape, dtype):
+    rng = np.random.default_rng(shape[1])
+    x = rng.integers(0, 200, shape).astype(dtype)
+    y = K.transpose_nchw_to_nhwc(x, ctx=hip_ctx)
+    assert np.array_equal(y, x.transpose(0, 2, 3, 1))
+    assert np.array_equal(K.transpose_nhwc_to_nchw(y, ctx=hip_ctx), x)
