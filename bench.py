@@ -1,0 +1,193 @@
+#!/usr/bin/env python3
+"""Headline benchmark: images/s of the u8/u8 MobileNetV2 (width 1.0, 224x224, random-init
+weights, per-tensor PTQ calibrated on 32 seeded images) at batch 64 on one MI355X, running as
+a resident `hip` function (one HIP-graph replay per step) with the input already in HBM.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 64]
+
+Prints ONE JSON line.  Besides the contract fields it carries
+  roofline     -- the kernel with the largest share of device time: algorithmic bytes per
+                  launch / mean launch duration (HIP events on the stream the kernels run on)
+                  against the 8 TB/s HBM peak
+  cpu_baseline -- the same graph executed the way nncase's CPU target executes it
+                  (Dequantize -> float Conv2D -> Quantize with the loop-for-loop restatement of
+                  its kernels), one thread, on a bounded number of batch-1 images.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
+INT8_PEAK_TOPS = 5000.0    # dense int8 MFMA
+
+
+def algorithmic_bytes(qg, batch):
+    """Per operator of the recorded function: bytes an ideal implementation must move
+    (read every input once, write every output once, read the constants once)."""
+    out = []
+    for n in qg.nodes:
+        c, h, w = n.out_shape
+        o = batch * c * h * w
+        if n.op == "input":
+            out.append(o * 4 + o)
+        elif n.op == "conv":
+            sc, sh, sw = qg.nodes[n.inputs[0]].out_shape
+            out.append(batch * sc * sh * sw + o + n.weights.size + 4 * n.bias.size)
+        elif n.op == "add":
+            out.append(3 * o)
+        elif n.op == "gap":
+            sc, sh, sw = qg.nodes[n.inputs[0]].out_shape
+            out.append(batch * sc * sh * sw + o)
+    last = qg.nodes[-1]
+    o = batch * int(np.prod(last.out_shape))
+    out.append(o + 4 * o)  # final dequantize
+    return out
+
+
+def conv_macs(qg, batch):
+    out = []
+    for n in qg.nodes:
+        if n.op == "conv":
+            oc, gic, kh, kw = n.weights.shape
+            out.append(batch * oc * n.out_shape[1] * n.out_shape[2] * gic * kh * kw)
+        else:
+            out.append(0)
+    out.append(0)
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--batch", type=int, default=64)
+    ap.add_argument("--cpu-images", type=int, default=8, help="batch-1 images timed on the CPU baseline (0 = skip)")
+    ap.add_argument("--profile-iters", type=int, default=10)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (the workload is one GPU's share at its real shape); "
+                 "--gpus N with N > 1 is not supported")
+
+    from nncase_amd import netbuilder as nb
+    from nncase_amd.runtime import Context
+
+    ctx = Context(0)  # raises if libnncase_hip.so is missing or there is no gfx950 device
+    graph = nb.mobilenet_v2(seed=2)
+    calib = np.random.default_rng(3).random((32, 224, 224, 3), dtype=np.float32)
+    qg = nb.quantize_graph(graph, calib)
+    x = np.random.default_rng(4).random((args.batch, 224, 224, 3), dtype=np.float32)
+
+    model = nb.HipModel(ctx, qg, args.batch, capture_graph=True)
+    model.set_input(x)  # resident in HBM before the timed region
+    for _ in range(args.warmup):
+        model.invoke()
+    ctx.sync()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        model.invoke()
+    ctx.sync()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+    images_per_s = args.batch / (dt / args.steps)
+
+    # ---- per-kernel device time (HIP events on the context's stream) --------------------------
+    op_ms = model.fn.profile(args.profile_iters)
+    names = [model.fn.op_kernel(i) for i in range(len(model.fn))]
+    abytes = algorithmic_bytes(qg, args.batch)
+    macs = conv_macs(qg, args.batch)
+    groups = {}
+    for name, ms, b, m in zip(names, op_ms, abytes, macs):
+        g = groups.setdefault(name, {"ms": 0.0, "bytes": 0, "macs": 0, "launches": 0})
+        g["ms"] += ms
+        g["bytes"] += b
+        g["macs"] += m
+        g["launches"] += 1
+    dom_name, dom = max(groups.items(), key=lambda kv: kv[1]["ms"])
+    dom_gbs = dom["bytes"] / (dom["ms"] * 1e-3) / 1e9
+
+    def klass(name):
+        return "dense" if name.startswith("qconv_igemm") else ("depthwise" if name.startswith("dw") else "elementwise")
+
+    classes = {}
+    for name, g in groups.items():
+        c = classes.setdefault(klass(name), {"ms": 0.0, "bytes": 0, "macs": 0})
+        for k in ("ms", "bytes", "macs"):
+            c[k] += g[k]
+    class_report = {k: {"ms": round(v["ms"], 4), "hbm_GBps": round(v["bytes"] / (v["ms"] * 1e-3) / 1e9, 1),
+                        "hbm_frac": round(v["bytes"] / (v["ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                        "int8_TOPS": round(2 * v["macs"] / (v["ms"] * 1e-3) / 1e12, 2),
+                        "mfma_frac": round(2 * v["macs"] / (v["ms"] * 1e-3) / 1e12 / INT8_PEAK_TOPS, 5)}
+                    for k, v in classes.items()}
+
+    # ---- batch-1 latency (same graph, HIP-graph replay) -----------------------------------------
+    m1 = nb.HipModel(ctx, qg, 1, capture_graph=True)
+    m1.set_input(x[:1])
+    for _ in range(20):
+        m1.invoke()
+    ctx.sync()
+    t1 = time.perf_counter()
+    for _ in range(200):
+        m1.invoke()
+    ctx.sync()
+    b1_ms = (time.perf_counter() - t1) / 200 * 1e3
+
+    # ---- CPU baseline: the CPU target's float chain, 1 thread, bounded sample -------------------
+    cpu = None
+    if args.cpu_images > 0:
+        from oracle import netref
+        t2 = time.perf_counter()
+        for i in range(args.cpu_images):
+            netref.run_float_chain(qg, x[i % args.batch:i % args.batch + 1])
+        cpu_dt = time.perf_counter() - t2
+        cpu = {"value": round(args.cpu_images / cpu_dt, 4), "unit": "images/s", "cores": 1, "kind": "port",
+               "host_cores": os.cpu_count(),
+               "sample": f"{args.cpu_images} batch-1 images of the same MobileNetV2 graph, every conv as Dequantize -> float "
+                         "Conv2D(fused_clamp) -> Quantize with the restated nncase CPU-target loops, -O2, 1 thread"}
+
+    total_macs = sum(macs)
+    line = {
+        "metric": "images/sec u8/u8 MobileNetV2 b64",
+        "value": round(images_per_s, 1),
+        "unit": "images/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "u8",
+        "data": "synthetic",
+        "config": {"workload": f"MobileNetV2 w1.0 224x224 u8/u8 per-tensor PTQ (32 calibration images), batch {args.batch}, "
+                               "NHWC f32 input resident in HBM -> quantize -> 52 convs + 10 adds + pool + FC -> dequantize",
+                   "batch": args.batch, "ops_per_step": len(model.fn), "execution": "resident hip function, HIP-graph replay"},
+        "roofline": {"bound": "hbm", "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(dom_gbs / HBM_PEAK_GBS, 4), "traffic": None, "kernel": dom_name,
+                     "launches_per_step": dom["launches"], "avg_launch_us": round(dom["ms"] / dom["launches"] * 1e3, 2),
+                     "algorithmic_bytes_per_launch": int(dom["bytes"] / dom["launches"]),
+                     "share_of_device_time": round(dom["ms"] / sum(op_ms), 4)},
+        "cpu_baseline": cpu,
+        "int8_TOPS_whole_net": round(2 * total_macs / (ms_per_step * 1e-3) / 1e12, 2),
+        "hbm_GBps_whole_net": round(sum(abytes) / (ms_per_step * 1e-3) / 1e9, 1),
+        "sum_of_kernel_ms": round(sum(op_ms), 4),
+        "kernel_classes": class_report,
+        "kernels": {k: {"ms": round(v["ms"], 4), "launches": v["launches"],
+                        "hbm_GBps": round(v["bytes"] / (v["ms"] * 1e-3) / 1e9, 1)} for k, v in sorted(groups.items())},
+        "batch1": {"ms_per_image": round(b1_ms, 4), "images_per_s": round(1e3 / b1_ms, 1)},
+        "device": {"compute_units": ctx.compute_units, "clock_mhz": ctx.clock_khz / 1000.0},
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -240,6 +240,59 @@ NNCASE_HIP_API int nncase_hip_paged_attention_decode(nncase_hip_ctx_t *ctx, cons
                                                      const int32_t *ctx_lens_dev, void *out_dev,
                                                      const nncase_hip_paged_attn_args_t *args);
 
+/* ---- resident functions --------------------------------------------------
+ * A function is the `hip` module's counterpart of a runtime_function
+ * (src/Native/include/nncase/runtime/runtime_function.h:55-63): an ordered
+ * list of the operators above with their device operands bound, built once
+ * when the module is loaded and invoked many times.  invoke() enqueues every
+ * operator on the context's stream in order and returns; after
+ * nncase_hip_function_capture() the same sequence is replayed as one HIP
+ * graph launch (the operands must stay where they were when captured).
+ * Operand buffers and weights stay owned by the caller and must outlive the
+ * function.
+ */
+typedef struct nncase_hip_function nncase_hip_function_t;
+
+NNCASE_HIP_API int nncase_hip_function_create(nncase_hip_ctx_t *ctx, nncase_hip_function_t **fn);
+NNCASE_HIP_API int nncase_hip_function_destroy(nncase_hip_function_t *fn);
+NNCASE_HIP_API int nncase_hip_function_add_quantize(nncase_hip_function_t *fn, const void *in_dev, int in_dtype,
+                                                    void *out_dev, int out_dtype, size_t count,
+                                                    nncase_hip_quant_param_t qp);
+NNCASE_HIP_API int nncase_hip_function_add_dequantize(nncase_hip_function_t *fn, const void *in_dev, int in_dtype,
+                                                      void *out_dev, int out_dtype, size_t count,
+                                                      nncase_hip_quant_param_t qp);
+NNCASE_HIP_API int nncase_hip_function_add_qconv2d(nncase_hip_function_t *fn, const uint8_t *x_dev,
+                                                   const nncase_hip_weights_t *weights, void *y_dev,
+                                                   const nncase_hip_conv2d_args_t *args);
+NNCASE_HIP_API int nncase_hip_function_add_qadd(nncase_hip_function_t *fn, const uint8_t *a_dev,
+                                                nncase_hip_quant_param_t a_qp, const uint8_t *b_dev,
+                                                nncase_hip_quant_param_t b_qp, uint8_t *out_dev,
+                                                nncase_hip_quant_param_t y_qp, float clamp_min, float clamp_max,
+                                                size_t count);
+NNCASE_HIP_API int nncase_hip_function_add_qglobal_avgpool(nncase_hip_function_t *fn, const uint8_t *x_dev,
+                                                           uint8_t *out_dev, int32_t batch, int32_t h, int32_t w,
+                                                           int32_t channels, nncase_hip_quant_param_t x_qp,
+                                                           nncase_hip_quant_param_t y_qp);
+/* Number of operators recorded so far. */
+NNCASE_HIP_API int nncase_hip_function_size(nncase_hip_function_t *fn, int32_t *count);
+/* Enqueues the whole function (graph replay if captured). */
+NNCASE_HIP_API int nncase_hip_function_invoke(nncase_hip_function_t *fn);
+/* Enqueues operator `index` alone (per-operator timing and debugging). */
+NNCASE_HIP_API int nncase_hip_function_invoke_one(nncase_hip_function_t *fn, int32_t index);
+/* Captures the operator sequence into a HIP graph used by later invokes. */
+NNCASE_HIP_API int nncase_hip_function_capture(nncase_hip_function_t *fn);
+/* Per-operator device time: every operator is enqueued `iterations` times
+ * back to back between two HIP events recorded on the context's stream and
+ * the mean duration in milliseconds is written to avg_ms[index] (the array
+ * holds nncase_hip_function_size entries).  Blocks until done.  The HIP
+ * counterpart of the reference's per-op profiler
+ * (src/Native/include/nncase/runtime/stackvm/op_profile.h:41-76). */
+NNCASE_HIP_API int nncase_hip_function_profile(nncase_hip_function_t *fn, int32_t iterations, float *avg_ms);
+/* Name of the kernel operator `index` launches, e.g.
+ * "qconv_igemm<T=9,RG=2,rows16>"; NUL-terminated, truncated to `capacity`. */
+NNCASE_HIP_API int nncase_hip_function_op_kernel(nncase_hip_function_t *fn, int32_t index, char *name,
+                                                 size_t capacity);
+
 #ifdef __cplusplus
 }
 #endif

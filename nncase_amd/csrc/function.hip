@@ -1,0 +1,230 @@
+// Resident functions: an ordered operator list bound to device operands,
+// replayable eagerly or as one HIP graph.
+#include "qconv.hpp"
+
+#include <new>
+#include <vector>
+
+namespace {
+
+struct Op {
+    enum Kind { kQuantize, kDequantize, kConv, kAdd, kPool } kind;
+    const void *in0 = nullptr, *in1 = nullptr;
+    void *out = nullptr;
+    const nncase_hip_weights_t *weights = nullptr;
+    nncase_hip_conv2d_args_t conv{};
+    nncase_hip_quant_param_t qp0{}, qp1{}, qp2{};
+    int dt_in = 0, dt_out = 0;
+    size_t count = 0;
+    float lo = 0.f, hi = 0.f;
+    int32_t batch = 0, h = 0, w = 0, channels = 0;
+};
+
+} // namespace
+
+struct nncase_hip_function {
+    nncase_hip_ctx *ctx = nullptr;
+    std::vector<Op> ops;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+};
+
+using namespace nnhip;
+
+static int run_op(nncase_hip_function *fn, const Op &op) {
+    nncase_hip_ctx *ctx = fn->ctx;
+    switch (op.kind) {
+    case Op::kQuantize:
+        return nncase_hip_quantize(ctx, op.in0, op.dt_in, op.out, op.dt_out, op.count, op.qp0);
+    case Op::kDequantize:
+        return nncase_hip_dequantize(ctx, op.in0, op.dt_in, op.out, op.dt_out, op.count, op.qp0);
+    case Op::kConv:
+        return nncase_hip_qconv2d(ctx, (const uint8_t *)op.in0, op.weights, op.out, &op.conv);
+    case Op::kAdd:
+        return nncase_hip_qadd(ctx, (const uint8_t *)op.in0, op.qp0, (const uint8_t *)op.in1, op.qp1, (uint8_t *)op.out,
+                               op.qp2, op.lo, op.hi, op.count);
+    case Op::kPool:
+        return nncase_hip_qglobal_avgpool(ctx, (const uint8_t *)op.in0, (uint8_t *)op.out, op.batch, op.h, op.w,
+                                          op.channels, op.qp0, op.qp1);
+    }
+    return -EINVAL;
+}
+
+static void drop_graph(nncase_hip_function *fn) {
+    if (fn->exec) (void)hipGraphExecDestroy(fn->exec);
+    if (fn->graph) (void)hipGraphDestroy(fn->graph);
+    fn->exec = nullptr;
+    fn->graph = nullptr;
+}
+
+static int push(nncase_hip_function *fn, const Op &op) {
+    drop_graph(fn); // a captured graph no longer matches the list
+    fn->ops.push_back(op);
+    return 0;
+}
+
+extern "C" int nncase_hip_function_create(nncase_hip_ctx_t *ctx, nncase_hip_function_t **out) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, out, -EINVAL, "function_create: null out pointer");
+    nncase_hip_function *fn = new (std::nothrow) nncase_hip_function();
+    NNHIP_REQUIRE(ctx, fn, -ENOMEM, "function_create: out of host memory");
+    fn->ctx = ctx;
+    *out = fn;
+    return 0;
+}
+
+extern "C" int nncase_hip_function_destroy(nncase_hip_function_t *fn) {
+    if (!fn) return -EINVAL;
+    (void)hipStreamSynchronize(fn->ctx->stream);
+    drop_graph(fn);
+    delete fn;
+    return 0;
+}
+
+extern "C" int nncase_hip_function_add_quantize(nncase_hip_function_t *fn, const void *in_dev, int in_dtype, void *out_dev,
+                                                int out_dtype, size_t count, nncase_hip_quant_param_t qp) {
+    if (!fn) return -EINVAL;
+    NNHIP_REQUIRE(fn->ctx, in_dev && out_dev, -EINVAL, "function_add_quantize: null buffer");
+    Op op;
+    op.kind = Op::kQuantize;
+    op.in0 = in_dev, op.out = out_dev, op.dt_in = in_dtype, op.dt_out = out_dtype, op.count = count, op.qp0 = qp;
+    return push(fn, op);
+}
+
+extern "C" int nncase_hip_function_add_dequantize(nncase_hip_function_t *fn, const void *in_dev, int in_dtype, void *out_dev,
+                                                  int out_dtype, size_t count, nncase_hip_quant_param_t qp) {
+    if (!fn) return -EINVAL;
+    NNHIP_REQUIRE(fn->ctx, in_dev && out_dev, -EINVAL, "function_add_dequantize: null buffer");
+    Op op;
+    op.kind = Op::kDequantize;
+    op.in0 = in_dev, op.out = out_dev, op.dt_in = in_dtype, op.dt_out = out_dtype, op.count = count, op.qp0 = qp;
+    return push(fn, op);
+}
+
+extern "C" int nncase_hip_function_add_qconv2d(nncase_hip_function_t *fn, const uint8_t *x_dev,
+                                               const nncase_hip_weights_t *weights, void *y_dev,
+                                               const nncase_hip_conv2d_args_t *args) {
+    if (!fn) return -EINVAL;
+    NNHIP_REQUIRE(fn->ctx, x_dev && weights && y_dev && args, -EINVAL, "function_add_qconv2d: null argument");
+    Op op;
+    op.kind = Op::kConv;
+    op.in0 = x_dev, op.out = y_dev, op.weights = weights, op.conv = *args;
+    return push(fn, op);
+}
+
+extern "C" int nncase_hip_function_add_qadd(nncase_hip_function_t *fn, const uint8_t *a_dev, nncase_hip_quant_param_t a_qp,
+                                            const uint8_t *b_dev, nncase_hip_quant_param_t b_qp, uint8_t *out_dev,
+                                            nncase_hip_quant_param_t y_qp, float clamp_min, float clamp_max, size_t count) {
+    if (!fn) return -EINVAL;
+    NNHIP_REQUIRE(fn->ctx, a_dev && b_dev && out_dev, -EINVAL, "function_add_qadd: null buffer");
+    Op op;
+    op.kind = Op::kAdd;
+    op.in0 = a_dev, op.in1 = b_dev, op.out = out_dev, op.qp0 = a_qp, op.qp1 = b_qp, op.qp2 = y_qp;
+    op.lo = clamp_min, op.hi = clamp_max, op.count = count;
+    return push(fn, op);
+}
+
+extern "C" int nncase_hip_function_add_qglobal_avgpool(nncase_hip_function_t *fn, const uint8_t *x_dev, uint8_t *out_dev,
+                                                       int32_t batch, int32_t h, int32_t w, int32_t channels,
+                                                       nncase_hip_quant_param_t x_qp, nncase_hip_quant_param_t y_qp) {
+    if (!fn) return -EINVAL;
+    NNHIP_REQUIRE(fn->ctx, x_dev && out_dev, -EINVAL, "function_add_qglobal_avgpool: null buffer");
+    Op op;
+    op.kind = Op::kPool;
+    op.in0 = x_dev, op.out = out_dev, op.batch = batch, op.h = h, op.w = w, op.channels = channels;
+    op.qp0 = x_qp, op.qp1 = y_qp;
+    return push(fn, op);
+}
+
+extern "C" int nncase_hip_function_size(nncase_hip_function_t *fn, int32_t *count) {
+    if (!fn || !count) return -EINVAL;
+    *count = (int32_t)fn->ops.size();
+    return 0;
+}
+
+extern "C" int nncase_hip_function_invoke_one(nncase_hip_function_t *fn, int32_t index) {
+    if (!fn) return -EINVAL;
+    NNHIP_REQUIRE(fn->ctx, index >= 0 && (size_t)index < fn->ops.size(), -EINVAL, "function_invoke_one: index %d of %zu",
+                  index, fn->ops.size());
+    return run_op(fn, fn->ops[index]);
+}
+
+extern "C" int nncase_hip_function_invoke(nncase_hip_function_t *fn) {
+    if (!fn) return -EINVAL;
+    if (fn->exec) {
+        NNHIP_HIP(fn->ctx, hipGraphLaunch(fn->exec, fn->ctx->stream));
+        return 0;
+    }
+    for (const Op &op : fn->ops) {
+        const int rc = run_op(fn, op);
+        if (rc) return rc;
+    }
+    return 0;
+}
+
+extern "C" int nncase_hip_function_capture(nncase_hip_function_t *fn) {
+    if (!fn) return -EINVAL;
+    nncase_hip_ctx *ctx = fn->ctx;
+    drop_graph(fn);
+    NNHIP_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    NNHIP_HIP(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+    int rc = 0;
+    for (const Op &op : fn->ops) {
+        rc = run_op(fn, op);
+        if (rc) break;
+    }
+    hipGraph_t graph = nullptr;
+    const hipError_t e = hipStreamEndCapture(ctx->stream, &graph);
+    if (rc) {
+        if (graph) (void)hipGraphDestroy(graph);
+        return rc;
+    }
+    NNHIP_HIP(ctx, e);
+    fn->graph = graph;
+    const hipError_t ie = hipGraphInstantiate(&fn->exec, fn->graph, nullptr, nullptr, 0);
+    if (ie != hipSuccess) {
+        drop_graph(fn);
+        return hip_fail(ctx, ie, "hipGraphInstantiate");
+    }
+    return 0;
+}
+
+extern "C" int nncase_hip_function_op_kernel(nncase_hip_function_t *fn, int32_t index, char *name, size_t capacity) {
+    if (!fn || !name || capacity == 0) return -EINVAL;
+    NNHIP_REQUIRE(fn->ctx, index >= 0 && (size_t)index < fn->ops.size(), -EINVAL, "function_op_kernel: index %d of %zu", index,
+                  fn->ops.size());
+    const Op &op = fn->ops[index];
+    switch (op.kind) {
+    case Op::kQuantize: snprintf(name, capacity, "quantize"); break;
+    case Op::kDequantize: snprintf(name, capacity, "dequantize"); break;
+    case Op::kConv: describe_conv_kernel(op.weights, &op.conv, name, capacity); break;
+    case Op::kAdd: snprintf(name, capacity, "qadd"); break;
+    case Op::kPool: snprintf(name, capacity, "qglobal_avgpool"); break;
+    }
+    return 0;
+}
+
+extern "C" int nncase_hip_function_profile(nncase_hip_function_t *fn, int32_t iterations, float *avg_ms) {
+    if (!fn || !avg_ms) return -EINVAL;
+    nncase_hip_ctx *ctx = fn->ctx;
+    NNHIP_REQUIRE(ctx, iterations > 0, -EINVAL, "function_profile: iterations must be positive");
+    hipEvent_t e0, e1;
+    NNHIP_HIP(ctx, hipEventCreate(&e0));
+    NNHIP_HIP(ctx, hipEventCreate(&e1));
+    int rc = 0;
+    for (size_t i = 0; i < fn->ops.size() && rc == 0; i++) {
+        rc = run_op(fn, fn->ops[i]); // warm
+        if (rc) break;
+        hipError_t e = hipEventRecord(e0, ctx->stream);
+        for (int it = 0; it < iterations && rc == 0; it++) rc = run_op(fn, fn->ops[i]);
+        if (e == hipSuccess) e = hipEventRecord(e1, ctx->stream);
+        if (e == hipSuccess) e = hipEventSynchronize(e1);
+        float ms = 0.f;
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+        if (e != hipSuccess && rc == 0) rc = hip_fail(ctx, e, "function_profile");
+        avg_ms[i] = ms / (float)iterations;
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    return rc;
+}

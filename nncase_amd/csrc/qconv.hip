@@ -14,6 +14,18 @@ int prepack_depthwise(nncase_hip_ctx *ctx, nncase_hip_weights *w, const uint8_t 
 
 using namespace nnhip;
 
+void nnhip::describe_conv_kernel(const nncase_hip_weights *w, const nncase_hip_conv2d_args_t *a, char *buf, size_t cap) {
+    if (w->kind == nncase_hip_weights::kDepthwise) {
+        if (depthwise_uses_3x3(w, a)) snprintf(buf, cap, "dw3x3<S=%d>", a->stride_h);
+        else snprintf(buf, cap, "dw_generic<VEC=%d>", w->out_channels % 4 == 0 ? 4 : 1);
+        return;
+    }
+    static const char *modes[] = {"rows16", "vec16", "vec8", "vec4", "bytes"};
+    const int out_h = windowed_output_size(a->in_h, w->kernel_h, a->stride_h, a->dilation_h, a->pad_h_before, a->pad_h_after);
+    const int out_w = windowed_output_size(a->in_w, w->kernel_w, a->stride_w, a->dilation_w, a->pad_w_before, a->pad_w_after);
+    snprintf(buf, cap, "qconv_igemm<T=%d,RG=%d,%s>", w->tiles, w->tiles <= 8 ? 4 : 2, modes[igemm_load_mode(w, a, out_h, out_w)]);
+}
+
 static void free_weights(nncase_hip_weights *w) {
     if (!w) return;
     if (w->d_packed) (void)hipFree(w->d_packed);

@@ -40,6 +40,11 @@ int launch_qconv_igemm(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_hip_w
 int launch_qconv_depthwise(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_hip_weights *w, void *y,
                            const nncase_hip_conv2d_args_t *a, int out_h, int out_w);
 
+// Writes the name of the kernel a conv with these weights / arguments launches.
+void describe_conv_kernel(const nncase_hip_weights *w, const nncase_hip_conv2d_args_t *a, char *buf, size_t cap);
+int igemm_load_mode(const nncase_hip_weights *w, const nncase_hip_conv2d_args_t *c, int out_h, int out_w);
+bool depthwise_uses_3x3(const nncase_hip_weights *w, const nncase_hip_conv2d_args_t *c);
+
 // Bit-exact requantisation of one fp32 value: sat_u8(rne(y / sy + zy)).
 // The saturation is applied to the float (its limits are integers, so it
 // commutes with round-half-even); the division is IEEE correctly rounded.

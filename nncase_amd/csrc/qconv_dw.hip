@@ -245,6 +245,11 @@ int prepack_depthwise(nncase_hip_ctx *ctx, nncase_hip_weights *w, const uint8_t 
     return 0;
 }
 
+bool depthwise_uses_3x3(const nncase_hip_weights *w, const nncase_hip_conv2d_args_t *c) {
+    return w->out_channels % 4 == 0 && w->kernel_h == 3 && w->kernel_w == 3 && c->dilation_h == 1 && c->dilation_w == 1 &&
+           c->stride_h == c->stride_w && (c->stride_h == 1 || c->stride_h == 2);
+}
+
 int launch_qconv_depthwise(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_hip_weights *w, void *y,
                            const nncase_hip_conv2d_args_t *c, int out_h, int out_w) {
     const int ch = w->out_channels;
@@ -287,8 +292,7 @@ int launch_qconv_depthwise(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_h
 
     const bool vec4 = (ch % 4 == 0) && ((reinterpret_cast<uintptr_t>(x) & 3u) == 0) &&
                       ((reinterpret_cast<uintptr_t>(y) & 15u) == 0);
-    const bool k3 = vec4 && w->kernel_h == 3 && w->kernel_w == 3 && c->dilation_h == 1 && c->dilation_w == 1 &&
-                    c->stride_h == c->stride_w && (c->stride_h == 1 || c->stride_h == 2);
+    const bool k3 = vec4 && depthwise_uses_3x3(w, c);
     if (k3) {
         a.cq = ch / 4;
         a.strips = ceil_div(out_w, kDwCols);

@@ -104,6 +104,15 @@ int prepack_igemm(nncase_hip_ctx *ctx, nncase_hip_weights *w, const uint8_t *w_o
     return 0;
 }
 
+int igemm_load_mode(const nncase_hip_weights *w, const nncase_hip_conv2d_args_t *c, int out_h, int out_w) {
+    const bool pointwise = w->kernel_h == 1 && w->kernel_w == 1 && c->stride_h == 1 && c->stride_w == 1 &&
+                           c->pad_h_before == 0 && c->pad_w_before == 0 && out_h == c->in_h && out_w == c->in_w;
+    if (w->g_ic % 16 == 0) return pointwise ? kRows16 : kVec16;
+    if (w->g_ic % 8 == 0) return kVec8;
+    if (w->g_ic % 4 == 0) return kVec4;
+    return kBytes;
+}
+
 int launch_qconv_igemm(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_hip_weights *w, void *y,
                        const nncase_hip_conv2d_args_t *c, int out_h, int out_w) {
     const int64_t m64 = (int64_t)c->batch * out_h * out_w;
@@ -152,13 +161,7 @@ int launch_qconv_igemm(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_hip_w
     a.ep.zy = (float)c->y_qp.zero_point;
     a.ep.out_mode = c->out_dtype == NNCASE_HIP_DT_U8 ? kOutU8 : (c->out_dtype == NNCASE_HIP_DT_I32 ? kOutI32 : kOutF32);
 
-    const bool pointwise = w->kernel_h == 1 && w->kernel_w == 1 && c->stride_h == 1 && c->stride_w == 1 &&
-                           c->pad_h_before == 0 && c->pad_w_before == 0 && out_h == c->in_h && out_w == c->in_w;
-    int mode;
-    if (w->g_ic % 16 == 0) mode = pointwise ? kRows16 : kVec16;
-    else if (w->g_ic % 8 == 0) mode = kVec8;
-    else if (w->g_ic % 4 == 0) mode = kVec4;
-    else mode = kBytes;
+    const int mode = igemm_load_mode(w, c, out_h, out_w);
 
     const size_t group_bytes = (size_t)w->nchunks * w->ksteps * w->tiles * 1024;
     for (int g = 0; g < w->groups; g++) {

@@ -92,6 +92,21 @@ SYMBOLS = {
     "nncase_hip_nchw_to_nhwc": (_I, [_VP, _VP, _VP, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
     "nncase_hip_nhwc_to_nchw": (_I, [_VP, _VP, _VP, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
     "nncase_hip_paged_attention_decode": (_I, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, C.POINTER(PagedAttnArgs)]),
+    "nncase_hip_function_create": (_I, [_VP, C.POINTER(_VP)]),
+    "nncase_hip_function_destroy": (_I, [_VP]),
+    "nncase_hip_function_add_quantize": (_I, [_VP, _VP, _I, _VP, _I, _SZ, QuantParam]),
+    "nncase_hip_function_add_dequantize": (_I, [_VP, _VP, _I, _VP, _I, _SZ, QuantParam]),
+    "nncase_hip_function_add_qconv2d": (_I, [_VP, _VP, _VP, _VP, C.POINTER(Conv2dArgs)]),
+    "nncase_hip_function_add_qadd": (_I, [_VP, _VP, QuantParam, _VP, QuantParam, _VP, QuantParam, C.c_float, C.c_float,
+                                          _SZ]),
+    "nncase_hip_function_add_qglobal_avgpool": (_I, [_VP, _VP, _VP, C.c_int32, C.c_int32, C.c_int32, C.c_int32,
+                                                     QuantParam, QuantParam]),
+    "nncase_hip_function_size": (_I, [_VP, C.POINTER(C.c_int32)]),
+    "nncase_hip_function_invoke": (_I, [_VP]),
+    "nncase_hip_function_invoke_one": (_I, [_VP, C.c_int32]),
+    "nncase_hip_function_capture": (_I, [_VP]),
+    "nncase_hip_function_profile": (_I, [_VP, C.c_int32, C.POINTER(C.c_float)]),
+    "nncase_hip_function_op_kernel": (_I, [_VP, C.c_int32, C.c_char_p, _SZ]),
 }
 
 _lib: Optional[C.CDLL] = None
@@ -304,3 +319,79 @@ class Context:
                                block_table: DeviceBuffer, ctx_lens: DeviceBuffer, out: DeviceBuffer, args: PagedAttnArgs):
         self._check(self.lib.nncase_hip_paged_attention_decode(self.handle, q.ptr, k_cache.ptr, v_cache.ptr, block_table.ptr,
                                                                ctx_lens.ptr, out.ptr, C.byref(args)), "paged_attention_decode")
+
+
+class Function:
+    """Resident operator list (nncase_hip_function_t): the `hip` module's runtime_function."""
+
+    def __init__(self, ctx: Context):
+        self.ctx = ctx
+        h = C.c_void_p()
+        ctx._check(ctx.lib.nncase_hip_function_create(ctx.handle, C.byref(h)), "function_create")
+        self.handle = h.value
+        self._keep = []  # operands must outlive the function
+
+    def _ck(self, rc, where):
+        self.ctx._check(rc, where)
+
+    def add_quantize(self, src, in_dtype, dst, out_dtype, count, q):
+        self._keep += [src, dst]
+        self._ck(self.ctx.lib.nncase_hip_function_add_quantize(self.handle, src.ptr, in_dtype, dst.ptr, out_dtype, count, q),
+                 "function_add_quantize")
+
+    def add_dequantize(self, src, in_dtype, dst, out_dtype, count, q):
+        self._keep += [src, dst]
+        self._ck(self.ctx.lib.nncase_hip_function_add_dequantize(self.handle, src.ptr, in_dtype, dst.ptr, out_dtype, count, q),
+                 "function_add_dequantize")
+
+    def add_qconv2d(self, x, w: Weights, y, args: Conv2dArgs):
+        self._keep += [x, w, y]
+        self._ck(self.ctx.lib.nncase_hip_function_add_qconv2d(self.handle, x.ptr, w.handle, y.ptr, C.byref(args)),
+                 "function_add_qconv2d")
+
+    def add_qadd(self, a, a_qp, b, b_qp, out, y_qp, count, clamp=(-FLT_MAX, FLT_MAX)):
+        self._keep += [a, b, out]
+        self._ck(self.ctx.lib.nncase_hip_function_add_qadd(self.handle, a.ptr, a_qp, b.ptr, b_qp, out.ptr, y_qp, clamp[0],
+                                                          clamp[1], count), "function_add_qadd")
+
+    def add_qglobal_avgpool(self, x, out, batch, h, w, channels, x_qp, y_qp):
+        self._keep += [x, out]
+        self._ck(self.ctx.lib.nncase_hip_function_add_qglobal_avgpool(self.handle, x.ptr, out.ptr, batch, h, w, channels,
+                                                                     x_qp, y_qp), "function_add_qglobal_avgpool")
+
+    def __len__(self):
+        n = C.c_int32()
+        self._ck(self.ctx.lib.nncase_hip_function_size(self.handle, C.byref(n)), "function_size")
+        return n.value
+
+    def invoke(self):
+        self._ck(self.ctx.lib.nncase_hip_function_invoke(self.handle), "function_invoke")
+
+    def invoke_one(self, index: int):
+        self._ck(self.ctx.lib.nncase_hip_function_invoke_one(self.handle, index), "function_invoke_one")
+
+    def capture(self):
+        self._ck(self.ctx.lib.nncase_hip_function_capture(self.handle), "function_capture")
+
+    def profile(self, iterations: int = 10):
+        """Mean device milliseconds per operator (HIP events on the context's stream)."""
+        n = len(self)
+        out = (C.c_float * n)()
+        self._ck(self.ctx.lib.nncase_hip_function_profile(self.handle, iterations, out), "function_profile")
+        return [float(v) for v in out]
+
+    def op_kernel(self, index: int) -> str:
+        buf = C.create_string_buffer(96)
+        self._ck(self.ctx.lib.nncase_hip_function_op_kernel(self.handle, index, buf, 96), "function_op_kernel")
+        return buf.value.decode()
+
+    def destroy(self):
+        if self.handle:
+            self.ctx.lib.nncase_hip_function_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass

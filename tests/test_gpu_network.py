@@ -1,0 +1,79 @@
+"""GPU parity of whole quantised graphs run as a resident `hip` function (eager and as a HIP
+graph) against the CPU oracle executing the same graph node by node: every intermediate u8
+tensor and the dequantised output must be bit-identical.  The float chain the CPU target
+really executes is cross-checked layer by layer (same inputs) to the <= 1 LSB bar."""
+import numpy as np
+import pytest
+
+from nncase_amd import netbuilder as nb
+from oracle import netref
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+f32 = np.float32
+
+
+def check_model(hip_ctx, qg, x, capture):
+    model = nb.HipModel(hip_ctx, qg, x.shape[0], capture_graph=capture)
+    y = model.run(x)
+    want, outs = netref.run_integer(qg, x, keep_all=True)
+    for i, ref in enumerate(outs):
+        got = model.tensor(i)
+        assert np.array_equal(got, ref), f"node {i} ({qg.nodes[i].name}): {(got != ref).sum()} of {ref.size} bytes differ"
+    assert np.array_equal(y.view(np.uint32), want.view(np.uint32))
+    return model, y, outs
+
+
+def test_conv_block_config2(hip_ctx):
+    g = nb.conv_block(seed=1)
+    rng = np.random.default_rng(1)
+    calib = rng.random((32, 56, 56, 64), dtype=f32)
+    qg = nb.quantize_graph(g, calib)
+    assert qg.macs_per_image == {"dense": 2 * 28901376, "depthwise": 4064256}
+    x = rng.random((2, 56, 56, 64), dtype=f32)
+    check_model(hip_ctx, qg, x, capture=False)
+    model, y, outs = check_model(hip_ctx, qg, x, capture=True)
+    # HIP-graph replays interleaved with eager work keep giving the same bytes
+    for _ in range(3):
+        model.set_input(x)
+        model.invoke()
+        hip_ctx.sync()
+        assert np.array_equal(model.output().view(np.uint32), y.view(np.uint32))
+        model.fn.invoke_one(1)
+        hip_ctx.sync()
+
+
+def test_mobilenetv2_config3(hip_ctx):
+    g = nb.mobilenet_v2(seed=2)
+    rng = np.random.default_rng(3)
+    calib = rng.random((32, 224, 224, 3), dtype=f32)
+    qg = nb.quantize_graph(g, calib)
+    assert qg.macs_per_image == {"dense": 280057856, "depthwise": 20716416}
+    x = rng.random((2, 224, 224, 3), dtype=f32)
+    model, y, outs = check_model(hip_ctx, qg, x, capture=True)
+    # the reference's own acceptance bar for a PTQ model: cosine >= 0.98 against the float model
+    fl = nb.float_forward(g, x)[-1]
+    assert O.cosine(y, fl) > 0.98
+    # layer-by-layer cross-check against the CPU target's float chain on identical inputs
+    for i, n in enumerate(qg.nodes):
+        if n.op != "conv" or i % 5:
+            continue
+        src = qg.nodes[n.inputs[0]]
+        chain = O.qconv2d_float_chain(outs[n.inputs[0]][:1], n.weights, n.bias, src.out_qp[0], src.out_qp[1], n.w_qp[0], n.w_qp[1],
+                                      n.out_qp[0], n.out_qp[1], n.stride, n.padding, (1, 1), n.groups, n.clamp)
+        d = np.abs(chain.astype(np.int32) - outs[i][:1].astype(np.int32))
+        assert d.max() <= 1, f"{n.name}: float chain differs by {d.max()} LSB"
+    # batch independence: image 0 alone gives the same logits (size-independent property)
+    m1 = nb.HipModel(hip_ctx, qg, 1, capture_graph=False)
+    assert np.array_equal(m1.run(x[:1]).view(np.uint32), y[:1].view(np.uint32))
+
+
+def test_profile_and_kernel_names(hip_ctx):
+    g = nb.conv_block(seed=1)
+    rng = np.random.default_rng(1)
+    qg = nb.quantize_graph(g, rng.random((4, 56, 56, 64), dtype=f32))
+    model = nb.HipModel(hip_ctx, qg, 2, capture_graph=False)
+    names = [model.fn.op_kernel(i) for i in range(len(model.fn))]
+    assert names == ["quantize", "qconv_igemm<T=9,RG=2,rows16>", "dw3x3<S=1>", "qconv_igemm<T=4,RG=4,rows16>", "dequantize"]
+    ms = model.fn.profile(3)
+    assert len(ms) == 5 and all(0 < t < 50 for t in ms)
