@@ -73,6 +73,10 @@ def main():
     ap.add_argument("--batch", type=int, default=64)
     ap.add_argument("--cpu-images", type=int, default=8, help="batch-1 images timed on the CPU baseline (0 = skip)")
     ap.add_argument("--profile-iters", type=int, default=10)
+    ap.add_argument("--batch1-steps", type=int, default=200, help="timed batch-1 invocations (0 = skip the batch-1 figure)")
+    ap.add_argument("--no-graph", action="store_true",
+                    help="enqueue the operators one by one instead of replaying the HIP graph (used under rocprofv3 "
+                         "--kernel-trace, whose tracer crashes inside hipGraphLaunch on this image)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (the workload is one GPU's share at its real shape); "
@@ -87,7 +91,7 @@ def main():
     qg = nb.quantize_graph(graph, calib)
     x = np.random.default_rng(4).random((args.batch, 224, 224, 3), dtype=np.float32)
 
-    model = nb.HipModel(ctx, qg, args.batch, capture_graph=True)
+    model = nb.HipModel(ctx, qg, args.batch, capture_graph=not args.no_graph)
     model.set_input(x)  # resident in HBM before the timed region
     for _ in range(args.warmup):
         model.invoke()
@@ -130,16 +134,19 @@ def main():
                     for k, v in classes.items()}
 
     # ---- batch-1 latency (same graph, HIP-graph replay) -----------------------------------------
-    m1 = nb.HipModel(ctx, qg, 1, capture_graph=True)
-    m1.set_input(x[:1])
-    for _ in range(20):
-        m1.invoke()
-    ctx.sync()
-    t1 = time.perf_counter()
-    for _ in range(200):
-        m1.invoke()
-    ctx.sync()
-    b1_ms = (time.perf_counter() - t1) / 200 * 1e3
+    b1 = None
+    if args.batch1_steps > 0:
+        m1 = nb.HipModel(ctx, qg, 1, capture_graph=not args.no_graph)
+        m1.set_input(x[:1])
+        for _ in range(20):
+            m1.invoke()
+        ctx.sync()
+        t1 = time.perf_counter()
+        for _ in range(args.batch1_steps):
+            m1.invoke()
+        ctx.sync()
+        b1_ms = (time.perf_counter() - t1) / args.batch1_steps * 1e3
+        b1 = {"ms_per_image": round(b1_ms, 4), "images_per_s": round(1e3 / b1_ms, 1)}
 
     # ---- CPU baseline: the CPU target's float chain, 1 thread, bounded sample -------------------
     cpu = None
@@ -170,7 +177,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": f"MobileNetV2 w1.0 224x224 u8/u8 per-tensor PTQ (32 calibration images), batch {args.batch}, "
                                "NHWC f32 input resident in HBM -> quantize -> 52 convs + 10 adds + pool + FC -> dequantize",
-                   "batch": args.batch, "ops_per_step": len(model.fn), "execution": "resident hip function, HIP-graph replay"},
+                   "batch": args.batch, "ops_per_step": len(model.fn), "execution": "resident hip function, " + ("eager launches" if args.no_graph else "HIP-graph replay")},
         "roofline": {"bound": "hbm", "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(dom_gbs / HBM_PEAK_GBS, 4), "traffic": None, "kernel": dom_name,
                      "launches_per_step": dom["launches"], "avg_launch_us": round(dom["ms"] / dom["launches"] * 1e3, 2),
@@ -183,7 +190,7 @@ def main():
         "kernel_classes": class_report,
         "kernels": {k: {"ms": round(v["ms"], 4), "launches": v["launches"],
                         "hbm_GBps": round(v["bytes"] / (v["ms"] * 1e-3) / 1e9, 1)} for k, v in sorted(groups.items())},
-        "batch1": {"ms_per_image": round(b1_ms, 4), "images_per_s": round(1e3 / b1_ms, 1)},
+        "batch1": b1,
         "device": {"compute_units": ctx.compute_units, "clock_mhz": ctx.clock_khz / 1000.0},
     }
     print(json.dumps(line))

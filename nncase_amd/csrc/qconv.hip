@@ -26,6 +26,52 @@ void nnhip::describe_conv_kernel(const nncase_hip_weights *w, const nncase_hip_c
     snprintf(buf, cap, "qconv_igemm<T=%d,RG=%d,%s>", w->tiles, w->tiles <= 8 ? 4 : 2, modes[igemm_load_mode(w, a, out_h, out_w)]);
 }
 
+float nnhip::reciprocal_rn(float b) {
+    float best = (float)(1.0 / (double)b);
+    // the product of two floats is exact in double, so |1 - b * r| ranks the candidates exactly
+    double err = std::fabs(1.0 - (double)b * (double)best);
+    const float cand[2] = {std::nextafterf(best, INFINITY), std::nextafterf(best, -INFINITY)};
+    for (float c : cand) {
+        const double e = std::fabs(1.0 - (double)b * (double)c);
+        if (e < err) {
+            err = e;
+            best = c;
+        }
+    }
+    return best;
+}
+
+int nnhip::make_epilogue(nncase_hip_ctx *ctx, Epilogue *ep, float sx, float sw, nncase_hip_quant_param_t y_qp, float clamp_min,
+                         float clamp_max, int out_dtype, const char *who) {
+    ep->mult = sx * sw;
+    ep->lo = clamp_min;
+    ep->hi = clamp_max;
+    ep->sy = y_qp.scale;
+    ep->zy = (float)y_qp.zero_point;
+    ep->rsy = 1.f;
+    ep->qlo = 0.f;
+    ep->qhi = 255.f;
+    ep->out_mode = out_dtype == NNCASE_HIP_DT_U8 ? kOutU8 : (out_dtype == NNCASE_HIP_DT_I32 ? kOutI32 : kOutF32);
+    NNHIP_REQUIRE(ctx, !(clamp_min > clamp_max), -EINVAL, "%s: fused clamp minimum above maximum", who);
+    if (ep->out_mode != kOutU8) return 0;
+    // Range in which q0 = f * rsy and the residual f - sy * q0 stay normal for every f whose
+    // requantised value is not already pinned to an end of [0, 255].
+    NNHIP_REQUIRE(ctx, ep->sy >= 0x1p-64f && ep->sy <= 0x1p64f, -ERANGE, "%s: output scale %g outside [2^-64, 2^64]", who,
+                  (double)ep->sy);
+    NNHIP_REQUIRE(ctx, std::isfinite(ep->mult) && std::fabs(ep->mult) <= 0x1p64f &&
+                           std::fabs((double)ep->mult) / (double)ep->sy <= 0x1p64,
+                  -ERANGE, "%s: input scale * weight scale = %g outside the supported range", who, (double)ep->mult);
+    ep->rsy = reciprocal_rn(ep->sy);
+    // g(v) = RN(RN(v / sy) + zy), evaluated with the same single fp32 operations as the device
+    volatile float glo = clamp_min / ep->sy;
+    glo = glo + ep->zy;
+    volatile float ghi = clamp_max / ep->sy;
+    ghi = ghi + ep->zy;
+    ep->qlo = std::fmin(std::fmax((float)glo, 0.f), 255.f);
+    ep->qhi = std::fmin(std::fmax((float)ghi, 0.f), 255.f);
+    return 0;
+}
+
 static void free_weights(nncase_hip_weights *w) {
     if (!w) return;
     if (w->d_packed) (void)hipFree(w->d_packed);

@@ -28,12 +28,31 @@ namespace nnhip {
 // Output forms of the conv / matmul epilogue.
 enum OutMode { kOutU8 = 0, kOutI32 = 1, kOutF32 = 2 };
 
+// Parameters of the fused epilogue  acc -> fp32 -> clamp -> requantise.
+//   f = (float)acc * mult
+//   F32 output: clamp(f, lo, hi)
+//   U8  output: sat_u8(rne(clamp(f, lo, hi) / sy + zy))
+// g(v) = RN(RN(v / sy) + zy) is monotone non-decreasing, so it commutes with the
+// clamp and the two clamps fold into one on g(f):
+//   clamp(g(clamp(f, lo, hi)), 0, 255) = clamp(g(f), qlo, qhi),
+//   qlo = clamp(g(lo), 0, 255), qhi = clamp(g(hi), 0, 255)      (computed on the host)
 struct Epilogue {
-    float mult;   // sx * sw
-    float lo, hi; // fused clamp on the fp32 value
-    float sy, zy; // output quantisation
+    float mult;     // sx * sw
+    float lo, hi;   // fused clamp on the fp32 value (F32 output)
+    float sy, rsy;  // output scale and its correctly rounded reciprocal
+    float zy;
+    float qlo, qhi; // clamp on the requantised value before rounding to an integer
     int out_mode;
 };
+
+// Fills an Epilogue; returns 0 or a negative error for scales outside the range in
+// which the division-free requantisation is exact.
+int make_epilogue(nncase_hip_ctx *ctx, Epilogue *ep, float sx, float sw, nncase_hip_quant_param_t y_qp, float clamp_min,
+                  float clamp_max, int out_dtype, const char *who);
+
+// RN(1 / b) for a finite positive b, exactly (the double quotient is corrected by
+// comparing exact residuals of the neighbouring floats).
+float reciprocal_rn(float b);
 
 int launch_qconv_igemm(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_hip_weights *w, void *y,
                        const nncase_hip_conv2d_args_t *a, int out_h, int out_w);
@@ -45,13 +64,31 @@ void describe_conv_kernel(const nncase_hip_weights *w, const nncase_hip_conv2d_a
 int igemm_load_mode(const nncase_hip_weights *w, const nncase_hip_conv2d_args_t *c, int out_h, int out_w);
 bool depthwise_uses_3x3(const nncase_hip_weights *w, const nncase_hip_conv2d_args_t *c);
 
-// Bit-exact requantisation of one fp32 value: sat_u8(rne(y / sy + zy)).
-// The saturation is applied to the float (its limits are integers, so it
-// commutes with round-half-even); the division is IEEE correctly rounded.
-__device__ __forceinline__ uint32_t requant_u8(float y, float sy, float zy) {
-    float t = y / sy + zy;
-    t = __builtin_fminf(__builtin_fmaxf(t, 0.f), 255.f);
-    return (uint32_t)(int32_t)__builtin_rintf(t);
+// Correctly rounded a / b from b and rb = RN(1 / b): one multiply and two fused
+// multiply-adds (Markstein's correction step: the residual a - b*q0 is exact in an
+// FMA and q0 + residual * rb rounds to the correctly rounded quotient).  Valid while
+// neither the quotient nor the residual leaves the normal range; make_epilogue
+// guarantees that for every value whose rounding can matter.
+__device__ __forceinline__ float div_rn(float a, float b, float rb) {
+    const float q0 = a * rb;
+    const float e = __builtin_fmaf(-b, q0, a);
+    return __builtin_fmaf(e, rb, q0);
+}
+
+// sat_u8(rne(f / sy + zy)) of an fp32 value, returned in the LOW BYTE of the result
+// (the other bytes are not zero).  Adding 1.5 * 2^23 makes the fp32 adder perform the
+// round-half-even to an integer and leaves that integer in the low mantissa bits.
+__device__ __forceinline__ uint32_t requant_u8_lowbyte(float f, const Epilogue &ep) {
+    float u = div_rn(f, ep.sy, ep.rsy) + ep.zy;
+    u = __builtin_amdgcn_fmed3f(u, ep.qlo, ep.qhi);
+    return __float_as_uint(u + 12582912.0f);
+}
+
+// Packs the low bytes of four dwords into one dword (3 byte-permutes).
+__device__ __forceinline__ uint32_t pack_low_bytes(uint32_t b0, uint32_t b1, uint32_t b2, uint32_t b3) {
+    const uint32_t lo = __builtin_amdgcn_perm(b1, b0, 0x0c0c0400u); // [b0.0, b1.0, 0, 0]
+    const uint32_t hi = __builtin_amdgcn_perm(b3, b2, 0x04000c0cu); // [0, 0, b2.0, b3.0]
+    return lo | hi;
 }
 
 __device__ __forceinline__ float clamp_ref(float v, float lo, float hi) {

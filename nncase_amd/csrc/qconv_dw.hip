@@ -43,18 +43,13 @@ struct DwArgs {
     Epilogue ep;
 };
 
-__device__ __forceinline__ uint32_t dw_finish_u8(int32_t v, const Epilogue &ep) {
-    const float f = clamp_ref((float)v * ep.mult, ep.lo, ep.hi);
-    return requant_u8(f, ep.sy, ep.zy);
-}
-
 __device__ __forceinline__ void dw_store4(const DwArgs &a, size_t pix, int c0, const int32_t (&v)[4]) {
     const size_t o = pix * a.channels + c0;
     if (a.ep.out_mode == kOutU8) {
-        uint32_t q = 0;
+        uint32_t b[4];
 #pragma unroll
-        for (int c = 0; c < 4; c++) q |= dw_finish_u8(v[c], a.ep) << (8 * c);
-        *reinterpret_cast<uint32_t *>(reinterpret_cast<uint8_t *>(a.y) + o) = q;
+        for (int c = 0; c < 4; c++) b[c] = requant_u8_lowbyte((float)v[c] * a.ep.mult, a.ep);
+        *reinterpret_cast<uint32_t *>(reinterpret_cast<uint8_t *>(a.y) + o) = pack_low_bytes(b[0], b[1], b[2], b[3]);
     } else if (a.ep.out_mode == kOutI32) {
         *reinterpret_cast<int4 *>(reinterpret_cast<int32_t *>(a.y) + o) = int4{v[0], v[1], v[2], v[3]};
     } else {
@@ -217,7 +212,8 @@ template <int VEC> __global__ __launch_bounds__(kDwThreads) void dw_generic_kern
         dw_store4(a, pix, c0, v);
     } else {
         const size_t o = pix * a.channels + c0;
-        if (a.ep.out_mode == kOutU8) reinterpret_cast<uint8_t *>(a.y)[o] = (uint8_t)dw_finish_u8(acc[0], a.ep);
+        if (a.ep.out_mode == kOutU8)
+            reinterpret_cast<uint8_t *>(a.y)[o] = (uint8_t)requant_u8_lowbyte((float)acc[0] * a.ep.mult, a.ep);
         else if (a.ep.out_mode == kOutI32) reinterpret_cast<int32_t *>(a.y)[o] = acc[0];
         else reinterpret_cast<float *>(a.y)[o] = clamp_ref((float)acc[0] * a.ep.mult, a.ep.lo, a.ep.hi);
     }
@@ -283,12 +279,10 @@ int launch_qconv_depthwise(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_h
     a.pad_w = c->pad_w_before;
     a.zx = c->x_qp.zero_point;
     a.zx_splat = (uint32_t)(c->x_qp.zero_point & 0xff) * 0x01010101u;
-    a.ep.mult = c->x_qp.scale * w->sw;
-    a.ep.lo = c->clamp_min;
-    a.ep.hi = c->clamp_max;
-    a.ep.sy = c->y_qp.scale;
-    a.ep.zy = (float)c->y_qp.zero_point;
-    a.ep.out_mode = c->out_dtype == NNCASE_HIP_DT_U8 ? kOutU8 : (c->out_dtype == NNCASE_HIP_DT_I32 ? kOutI32 : kOutF32);
+    {
+        const int rc = make_epilogue(ctx, &a.ep, c->x_qp.scale, w->sw, c->y_qp, c->clamp_min, c->clamp_max, c->out_dtype, "qconv2d");
+        if (rc) return rc;
+    }
 
     const bool vec4 = (ch % 4 == 0) && ((reinterpret_cast<uintptr_t>(x) & 3u) == 0) &&
                       ((reinterpret_cast<uintptr_t>(y) & 15u) == 0);

@@ -154,12 +154,10 @@ int launch_qconv_igemm(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_hip_w
     a.zxp = c->x_qp.zero_point - 128;
     a.zwp = w->zw - 128;
     a.zx_splat = (uint32_t)(c->x_qp.zero_point & 0xff) * 0x01010101u;
-    a.ep.mult = c->x_qp.scale * w->sw;
-    a.ep.lo = c->clamp_min;
-    a.ep.hi = c->clamp_max;
-    a.ep.sy = c->y_qp.scale;
-    a.ep.zy = (float)c->y_qp.zero_point;
-    a.ep.out_mode = c->out_dtype == NNCASE_HIP_DT_U8 ? kOutU8 : (c->out_dtype == NNCASE_HIP_DT_I32 ? kOutI32 : kOutF32);
+    {
+        const int rc = make_epilogue(ctx, &a.ep, c->x_qp.scale, w->sw, c->y_qp, c->clamp_min, c->clamp_max, c->out_dtype, "qconv2d");
+        if (rc) return rc;
+    }
 
     const int mode = igemm_load_mode(w, c, out_h, out_w);
 

@@ -269,14 +269,13 @@ __global__ __launch_bounds__(kThreads, 2) void qconv_igemm_kernel(const IgemmArg
 #pragma unroll
                     for (int nt = 0; nt < T; nt++) {
                         const v4i ct = *reinterpret_cast<const v4i *>(cterm + gq * (4 * T) + nt * 4);
-                        uint32_t q = 0;
+                        uint32_t b[4];
 #pragma unroll
                         for (int r = 0; r < 4; r++) {
                             const int32_t v = acc[rg][nt][r] + ct[r] - rsz;
-                            const float f = clamp_ref((float)v * a.ep.mult, a.ep.lo, a.ep.hi);
-                            q |= requant_u8(f, a.ep.sy, a.ep.zy) << (8 * r);
+                            b[r] = requant_u8_lowbyte((float)v * a.ep.mult, a.ep);
                         }
-                        packed[nt] = q;
+                        packed[nt] = pack_low_bytes(b[0], b[1], b[2], b[3]);
                     }
                     if (((a.ldy | a.y_coff) & 3) == 0 && ch0 + 4 * T <= a.n) {
 #pragma unroll

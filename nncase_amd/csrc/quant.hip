@@ -8,9 +8,11 @@
 // is compiled with -ffp-contract=off):
 //   quantize    q = sat_T((int32) rne(x / scale + bias))          reference/quantize.cpp:36-43
 //   dequantize  y = ((float) q - bias) * scale                    reference/dequantize.cpp:36-39
-#include "common.hpp"
+#include "qconv.hpp"
 
 #include <hip/hip_fp16.h>
+
+#include <cmath>
 
 namespace nnhip {
 
@@ -117,37 +119,35 @@ __global__ __launch_bounds__(kEwThreads) void dequantize_kernel(const TQ *__rest
     for (size_t j = nvec * kEwVec + tid; j < count; j += nthreads) out[j] = from_f32<TOut>(((float)in[j] - bias) * scale);
 }
 
-// out = Q(clamp(DQ(a) + DQ(b))) on bytes.
+// out = Q(clamp(DQ(a) + DQ(b))) on bytes; the clamp and the u8 saturation are folded into
+// one clamp on the requantised value, the division is the exact FMA form (see qconv.hpp).
 __global__ __launch_bounds__(kEwThreads) void qadd_kernel(const uint8_t *__restrict__ a, const uint8_t *__restrict__ b,
                                                           uint8_t *__restrict__ out, size_t count, float za, float sa,
-                                                          float zb, float sb, float zy, float sy, float lo, float hi,
-                                                          int vec_ok) {
+                                                          float zb, float sb, const Epilogue ep, int vec_ok) {
     const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t nthreads = (size_t)gridDim.x * blockDim.x;
-    auto one = [&](uint8_t qa, uint8_t qb) -> uint8_t {
+    auto one = [&](uint32_t qa, uint32_t qb) -> uint32_t {
         const float fa = ((float)qa - za) * sa;
         const float fb = ((float)qb - zb) * sb;
-        float s = fa + fb;
-        s = fmaxf(fminf(s, hi), lo);
-        float t = s / sy + zy;
-        t = fminf(fmaxf(t, 0.f), 255.f);
-        return (uint8_t)(int32_t)rintf(t);
+        return requant_u8_lowbyte(fa + fb, ep);
     };
     // 16 bytes per thread per step
     const size_t nvec = vec_ok ? count / 16 : 0;
     for (size_t i = tid; i < nvec; i += nthreads) {
         const uint4 va = *reinterpret_cast<const uint4 *>(a + i * 16);
         const uint4 vb = *reinterpret_cast<const uint4 *>(b + i * 16);
-        uint8_t ba[16], bb[16], bo[16];
-        __builtin_memcpy(ba, &va, 16);
-        __builtin_memcpy(bb, &vb, 16);
+        const uint32_t wa[4] = {va.x, va.y, va.z, va.w}, wb[4] = {vb.x, vb.y, vb.z, vb.w};
+        uint32_t wo[4];
 #pragma unroll
-        for (int e = 0; e < 16; e++) bo[e] = one(ba[e], bb[e]);
-        uint4 vo;
-        __builtin_memcpy(&vo, bo, 16);
-        *reinterpret_cast<uint4 *>(out + i * 16) = vo;
+        for (int d = 0; d < 4; d++) {
+            uint32_t r[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) r[e] = one((wa[d] >> (8 * e)) & 0xffu, (wb[d] >> (8 * e)) & 0xffu);
+            wo[d] = pack_low_bytes(r[0], r[1], r[2], r[3]);
+        }
+        *reinterpret_cast<uint4 *>(out + i * 16) = uint4{wo[0], wo[1], wo[2], wo[3]};
     }
-    for (size_t j = nvec * 16 + tid; j < count; j += nthreads) out[j] = one(a[j], b[j]);
+    for (size_t j = nvec * 16 + tid; j < count; j += nthreads) out[j] = (uint8_t)one(a[j], b[j]);
 }
 
 // Global average pool over NHWC u8.  One thread per (image, channel): the sum
@@ -252,13 +252,18 @@ extern "C" int nncase_hip_qadd(nncase_hip_ctx_t *ctx, const uint8_t *a_dev, nnca
                                nncase_hip_quant_param_t y_qp, float clamp_min, float clamp_max, size_t count) {
     NNHIP_CHECK_CTX(ctx);
     NNHIP_REQUIRE(ctx, (a_dev && b_dev && out_dev) || count == 0, -EINVAL, "qadd: null buffer");
-    NNHIP_REQUIRE(ctx, y_qp.scale != 0.f, -EINVAL, "qadd: output scale is zero");
     if (count == 0) return 0;
+    NNHIP_REQUIRE(ctx, std::isfinite(a_qp.scale) && std::isfinite(b_qp.scale) && std::fabs(a_qp.scale) <= 0x1p20f &&
+                           std::fabs(b_qp.scale) <= 0x1p20f,
+                  -ERANGE, "qadd: input scale outside the supported range");
+    Epilogue ep;
+    // the sum's magnitude is bounded by 255 * (|sa| + |sb|); mult is unused here
+    const int rc = make_epilogue(ctx, &ep, 1.f, 1.f, y_qp, clamp_min, clamp_max, NNCASE_HIP_DT_U8, "qadd");
+    if (rc) return rc;
     const int vec_ok = aligned16(a_dev) && aligned16(b_dev) && aligned16(out_dev);
     const int grid = ew_grid(ctx, (count + 15) / 16);
     hipLaunchKernelGGL(qadd_kernel, dim3(grid), dim3(kEwThreads), 0, ctx->stream, a_dev, b_dev, out_dev, count,
-                       (float)a_qp.zero_point, a_qp.scale, (float)b_qp.zero_point, b_qp.scale, (float)y_qp.zero_point,
-                       y_qp.scale, clamp_min, clamp_max, vec_ok);
+                       (float)a_qp.zero_point, a_qp.scale, (float)b_qp.zero_point, b_qp.scale, ep, vec_ok);
     NNHIP_LAUNCH_CHECK(ctx, "qadd_kernel");
     return 0;
 }

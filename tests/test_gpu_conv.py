@@ -248,3 +248,37 @@ def test_error_paths(hip_ctx):
     with pytest.raises(rt.HipError) as e:   # zero point outside u8
         K.conv2d(x, w, None, (1, 1), ((1, 1), (1, 1)), (1, 1), 1, FULL, qp(300, 1), qp(0, 1), None, np.int32, ctx=hip_ctx)
     assert e.value.code == -22
+
+
+def test_requantisation_is_exact_for_many_scales(hip_ctx):
+    """The device replaces y / sy by a multiply and two FMAs with a pre-rounded reciprocal; the
+    bytes must still equal the oracle's true fp32 division for every accumulator, including
+    scales that are powers of two (exact .5 ties), have an all-ones mantissa, or are tiny/huge."""
+    rng = np.random.default_rng(2024)
+    x = rng.integers(0, 256, (1, 64, 64, 64), dtype=np.uint8)      # 4096 pixels
+    w = rng.integers(0, 256, (64, 64, 1, 1), dtype=np.uint8)       # 262144 accumulators per case
+    bias = rng.integers(-20000, 20000, 64).astype(np.int32)
+    acc = O.qconv2d(x, w, bias, 3, 1.0, 128, 1.0, out_mode=O.OUT_I32)
+    span = float(acc.max() - acc.min())
+    special = [np.float32(2.0 ** -7), np.float32(0.5), np.nextafter(np.float32(1.0), np.float32(0)),
+               np.nextafter(np.float32(0.03125), np.float32(0)), np.float32(1.0) + np.float32(2.0 ** -23)]
+    for i in range(48):
+        sx = f32(10.0 ** rng.uniform(-3, 0))
+        sw = f32(10.0 ** rng.uniform(-4, -1))
+        m = float(sx) * float(sw)
+        sy = special[i] if i < len(special) else f32(span * m / 255 * 10.0 ** rng.uniform(-1.0, 0.5))
+        if i < len(special):  # choose sx * sw so that the u8 range is covered for the special scales too
+            sx, sw = f32(float(sy) * 255 / span), f32(1.0)
+        zy = int(rng.integers(0, 256))
+        clamp = FULL if i % 3 else (0.0, float(sy) * 200)
+        got = K.conv2d(x, w, bias, (1, 1), ((0, 0), (0, 0)), (1, 1), 1, clamp, qp(3, sx), qp(128, sw), qp(zy, sy), np.uint8, ctx=hip_ctx)
+        want = O.qconv2d(x, w, bias, 3, sx, 128, sw, zy, sy, fused_clamp=clamp)
+        assert np.array_equal(got, want), f"case {i}: sx={sx} sw={sw} sy={sy} zy={zy}: {(got != want).sum()} bytes differ"
+    # extreme but supported scales, and the documented rejection beyond them
+    for sy in (f32(2.0 ** -60), f32(2.0 ** 60)):
+        got = K.conv2d(x, w, bias, (1, 1), ((0, 0), (0, 0)), (1, 1), 1, FULL, qp(3, 1.0), qp(128, float(sy) / 100), qp(7, sy), np.uint8, ctx=hip_ctx)
+        want = O.qconv2d(x, w, bias, 3, 1.0, 128, float(sy) / 100, 7, sy)
+        assert np.array_equal(got, want)
+    with pytest.raises(rt.HipError) as e:
+        K.conv2d(x, w, bias, (1, 1), ((0, 0), (0, 0)), (1, 1), 1, FULL, qp(3, 1.0), qp(128, 1.0), qp(7, 2.0 ** -70), np.uint8, ctx=hip_ctx)
+    assert e.value.code == -34  # ERANGE
