@@ -131,6 +131,9 @@ typedef struct nncase_hip_conv2d_desc {
     int32_t kernel_h, kernel_w;
     int32_t groups;
     nncase_hip_quant_param_t w_qp; /* per-tensor weight quantisation */
+    /* batch * out_h * out_w the weights will be run with (shapes are static in a
+     * kmodel); used only to pick a tiling that fills the device. 0 = unknown. */
+    int64_t expected_pixels;
 } nncase_hip_conv2d_desc_t;
 
 /* Re-lays-out HOST weights (OIHW u8) and bias (int32[out_channels], may be
@@ -167,7 +170,7 @@ NNCASE_HIP_API int nncase_hip_qconv2d(nncase_hip_ctx_t *ctx, const uint8_t *x_de
  * src/Nncase.Importer/Onnx/QLinearMatmul.cs:25-28. */
 NNCASE_HIP_API int nncase_hip_qmatmul_prepack(nncase_hip_ctx_t *ctx, const uint8_t *b_host, int32_t k, int32_t n,
                                               nncase_hip_quant_param_t b_qp, const int32_t *bias_host,
-                                              nncase_hip_weights_t **weights);
+                                              int64_t expected_rows, nncase_hip_weights_t **weights);
 
 typedef struct nncase_hip_matmul_args {
     int32_t m;

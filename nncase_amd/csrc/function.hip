@@ -197,7 +197,7 @@ extern "C" int nncase_hip_function_op_kernel(nncase_hip_function_t *fn, int32_t 
     switch (op.kind) {
     case Op::kQuantize: snprintf(name, capacity, "quantize"); break;
     case Op::kDequantize: snprintf(name, capacity, "dequantize"); break;
-    case Op::kConv: describe_conv_kernel(op.weights, &op.conv, name, capacity); break;
+    case Op::kConv: describe_conv_kernel(fn->ctx, op.weights, &op.conv, name, capacity); break;
     case Op::kAdd: snprintf(name, capacity, "qadd"); break;
     case Op::kPool: snprintf(name, capacity, "qglobal_avgpool"); break;
     }

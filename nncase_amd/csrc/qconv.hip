@@ -3,6 +3,7 @@
 // streaming kernel.
 #include "qconv.hpp"
 
+#include <algorithm>
 #include <cmath>
 #include <new>
 #include <vector>
@@ -14,16 +15,23 @@ int prepack_depthwise(nncase_hip_ctx *ctx, nncase_hip_weights *w, const uint8_t 
 
 using namespace nnhip;
 
-void nnhip::describe_conv_kernel(const nncase_hip_weights *w, const nncase_hip_conv2d_args_t *a, char *buf, size_t cap) {
+void nnhip::describe_conv_kernel(const nncase_hip_ctx *ctx, const nncase_hip_weights *w, const nncase_hip_conv2d_args_t *a,
+                                 char *buf, size_t cap) {
     if (w->kind == nncase_hip_weights::kDepthwise) {
         if (depthwise_uses_3x3(w, a)) snprintf(buf, cap, "dw3x3<S=%d>", a->stride_h);
         else snprintf(buf, cap, "dw_generic<VEC=%d>", w->out_channels % 4 == 0 ? 4 : 1);
         return;
     }
+    if (w->d_smallc && a->dilation_h == 1 && a->dilation_w == 1) {
+        snprintf(buf, cap, "qconv_smallc<C=%d>", w->in_channels);
+        return;
+    }
     static const char *modes[] = {"rows16", "vec16", "vec8", "vec4", "bytes"};
     const int out_h = windowed_output_size(a->in_h, w->kernel_h, a->stride_h, a->dilation_h, a->pad_h_before, a->pad_h_after);
     const int out_w = windowed_output_size(a->in_w, w->kernel_w, a->stride_w, a->dilation_w, a->pad_w_before, a->pad_w_after);
-    snprintf(buf, cap, "qconv_igemm<T=%d,RG=%d,%s>", w->tiles, w->tiles <= 8 ? 4 : 2, modes[igemm_load_mode(w, a, out_h, out_w)]);
+    const long long m = (long long)a->batch * out_h * out_w;
+    snprintf(buf, cap, "qconv_igemm<T=%d,RG=%d,%s>", w->tiles, igemm_pixel_groups(ctx, w, (int)std::min<long long>(m, 1 << 30)),
+             modes[igemm_load_mode(w, a, out_h, out_w)]);
 }
 
 float nnhip::reciprocal_rn(float b) {
@@ -77,6 +85,7 @@ static void free_weights(nncase_hip_weights *w) {
     if (w->d_packed) (void)hipFree(w->d_packed);
     if (w->d_wsum) (void)hipFree(w->d_wsum);
     if (w->d_bias) (void)hipFree(w->d_bias);
+    if (w->d_smallc) (void)hipFree(w->d_smallc);
     delete w;
 }
 
@@ -105,11 +114,13 @@ extern "C" int nncase_hip_qconv2d_prepack(nncase_hip_ctx_t *ctx, const nncase_hi
     w->g_oc = desc->out_channels / desc->groups;
     w->zw = desc->w_qp.zero_point;
     w->sw = desc->w_qp.scale;
+    w->pixels_hint = desc->expected_pixels > 0 ? desc->expected_pixels : 0;
     const bool depthwise = desc->groups > 1 && w->g_ic == 1 && w->g_oc == 1;
     w->kind = depthwise ? nncase_hip_weights::kDepthwise : nncase_hip_weights::kIgemm;
     NNHIP_HIP(ctx, hipSetDevice(ctx->device));
-    const int rc = depthwise ? prepack_depthwise(ctx, w, weights_oihw_host, bias_host)
-                             : prepack_igemm(ctx, w, weights_oihw_host, bias_host);
+    int rc = depthwise ? prepack_depthwise(ctx, w, weights_oihw_host, bias_host)
+                       : prepack_igemm(ctx, w, weights_oihw_host, bias_host);
+    if (rc == 0 && !depthwise && smallc_supported(w)) rc = prepack_smallc(ctx, w, weights_oihw_host);
     if (rc) {
         free_weights(w);
         return rc;
@@ -154,11 +165,12 @@ extern "C" int nncase_hip_qconv2d(nncase_hip_ctx_t *ctx, const uint8_t *x_dev, c
     const int out_w = windowed_output_size(a->in_w, w->kernel_w, a->stride_w, a->dilation_w, a->pad_w_before, a->pad_w_after);
     NNHIP_REQUIRE(ctx, out_h > 0 && out_w > 0, -NNCASE_HIP_ERR_SHAPE_MISMATCH, "qconv2d: window larger than padded input");
     if (w->kind == nncase_hip_weights::kDepthwise) return launch_qconv_depthwise(ctx, x_dev, w, y_dev, a, out_h, out_w);
+    if (w->d_smallc && a->dilation_h == 1 && a->dilation_w == 1) return launch_qconv_smallc(ctx, x_dev, w, y_dev, a, out_h, out_w);
     return launch_qconv_igemm(ctx, x_dev, w, y_dev, a, out_h, out_w);
 }
 
 extern "C" int nncase_hip_qmatmul_prepack(nncase_hip_ctx_t *ctx, const uint8_t *b_host, int32_t k, int32_t n,
-                                          nncase_hip_quant_param_t b_qp, const int32_t *bias_host,
+                                          nncase_hip_quant_param_t b_qp, const int32_t *bias_host, int64_t expected_rows,
                                           nncase_hip_weights_t **weights) {
     NNHIP_CHECK_CTX(ctx);
     NNHIP_REQUIRE(ctx, b_host && weights, -EINVAL, "qmatmul_prepack: null argument");
@@ -173,6 +185,7 @@ extern "C" int nncase_hip_qmatmul_prepack(nncase_hip_ctx_t *ctx, const uint8_t *
     d.kernel_h = d.kernel_w = 1;
     d.groups = 1;
     d.w_qp = b_qp;
+    d.expected_pixels = expected_rows;
     return nncase_hip_qconv2d_prepack(ctx, &d, bt.data(), bias_host, weights);
 }
 

@@ -13,6 +13,7 @@ struct nncase_hip_weights {
     int tiles = 0;          // 16-channel MFMA tiles per channel chunk (T)
     int nchunks = 0;        // channel chunks per group
     int kc_steps = 0;       // k-steps staged in LDS at a time
+    int64_t pixels_hint = 0; // output pixels per call the tiling was planned for (0 = unknown)
     int32_t zw = 0;
     float sw = 1.f;
     // igemm: [groups][nchunks][ksteps][tiles] fragments of 1024 bytes (s8, MFMA operand order)
@@ -21,6 +22,9 @@ struct nncase_hip_weights {
     int32_t *d_wsum = nullptr; // igemm: sum_k (w ^ 0x80 as s8) per out channel; depthwise: sum_t (w - zw)
     int32_t *d_bias = nullptr; // [out_channels]
     size_t packed_bytes = 0;
+    // few-input-channel 3x3 convolutions also carry a [oc][k] s8 layout for the per-pixel dot-product kernel
+    void *d_smallc = nullptr;
+    size_t smallc_bytes = 0;
 };
 
 namespace nnhip {
@@ -56,11 +60,17 @@ float reciprocal_rn(float b);
 
 int launch_qconv_igemm(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_hip_weights *w, void *y,
                        const nncase_hip_conv2d_args_t *a, int out_h, int out_w);
+int launch_qconv_smallc(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_hip_weights *w, void *y,
+                        const nncase_hip_conv2d_args_t *a, int out_h, int out_w);
+bool smallc_supported(const nncase_hip_weights *w);
+int prepack_smallc(nncase_hip_ctx *ctx, nncase_hip_weights *w, const uint8_t *w_oihw);
 int launch_qconv_depthwise(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_hip_weights *w, void *y,
                            const nncase_hip_conv2d_args_t *a, int out_h, int out_w);
 
 // Writes the name of the kernel a conv with these weights / arguments launches.
-void describe_conv_kernel(const nncase_hip_weights *w, const nncase_hip_conv2d_args_t *a, char *buf, size_t cap);
+void describe_conv_kernel(const nncase_hip_ctx *ctx, const nncase_hip_weights *w, const nncase_hip_conv2d_args_t *a, char *buf,
+                          size_t cap);
+int igemm_pixel_groups(const nncase_hip_ctx *ctx, const nncase_hip_weights *w, int m);
 int igemm_load_mode(const nncase_hip_weights *w, const nncase_hip_conv2d_args_t *c, int out_h, int out_w);
 bool depthwise_uses_3x3(const nncase_hip_weights *w, const nncase_hip_conv2d_args_t *c);
 

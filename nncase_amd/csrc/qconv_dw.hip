@@ -23,7 +23,7 @@ namespace nnhip {
 
 constexpr int kDwThreads = 256;
 constexpr int kDwCols = 4;  // output columns per thread
-constexpr int kDwRows = 8;  // output rows per thread (3x3 kernel)
+constexpr int kDwMaxRows = 8; // most output rows one thread walks down (3x3 kernel)
 
 struct DwArgs {
     const uint8_t *x;
@@ -38,13 +38,14 @@ struct DwArgs {
     int cq;          // channel vectors per pixel
     int strips;      // column strips per row
     int row_chunks;  // row chunks per image (3x3 kernel)
+    int rows;        // output rows per thread (3x3 kernel)
     FastDiv d_cq, d_strips, d_rows, d_ow, d_oh;
     long long total; // threads of useful work
     Epilogue ep;
 };
 
-__device__ __forceinline__ void dw_store4(const DwArgs &a, size_t pix, int c0, const int32_t (&v)[4]) {
-    const size_t o = pix * a.channels + c0;
+// Stores 4 adjacent channels of one output pixel; `o` is the element offset of the first.
+__device__ __forceinline__ void dw_store4(const DwArgs &a, uint32_t o, const int32_t (&v)[4]) {
     if (a.ep.out_mode == kOutU8) {
         uint32_t b[4];
 #pragma unroll
@@ -62,12 +63,14 @@ __device__ __forceinline__ void dw_store4(const DwArgs &a, size_t pix, int c0, c
     }
 }
 
+// All offsets are 32-bit element offsets from the (uniform) tensor bases, advanced by
+// additions only; the host checks that both tensors stay below 2^31 elements.
 template <int S> __global__ __launch_bounds__(kDwThreads) void dw3x3_kernel(const DwArgs a) {
     constexpr int NCOL = (kDwCols - 1) * S + 3;
-    const long long gid = (long long)blockIdx.x * kDwThreads + threadIdx.x;
-    if (gid >= a.total) return;
+    const uint32_t gid = blockIdx.x * kDwThreads + threadIdx.x;
+    if (gid >= (uint32_t)a.total) return;
     // gid -> (image, row chunk, strip, channel quad), channel quad fastest
-    uint32_t t = (uint32_t)gid;
+    uint32_t t = gid;
     uint32_t q = fastdiv(t, a.d_cq);
     const int cq = (int)(t - q * a.d_cq.div);
     t = q;
@@ -80,14 +83,14 @@ template <int S> __global__ __launch_bounds__(kDwThreads) void dw3x3_kernel(cons
 
     const int c0 = cq * 4;
     const int ox0 = strip * kDwCols;
-    const int oy0 = rchunk * kDwRows;
+    const int oy0 = rchunk * a.rows;
     const int ix0 = ox0 * S - a.pad_w;
     const int iy_first = oy0 * S - a.pad_h;
 
     int32_t w[9][4], ct[4];
 #pragma unroll
     for (int tap = 0; tap < 9; tap++) {
-        const uint2 raw = *reinterpret_cast<const uint2 *>(a.w + (size_t)tap * a.channels + c0);
+        const uint2 raw = *reinterpret_cast<const uint2 *>(a.w + (uint32_t)(tap * a.channels + c0));
         w[tap][0] = (int16_t)(raw.x & 0xffff);
         w[tap][1] = (int16_t)(raw.x >> 16);
         w[tap][2] = (int16_t)(raw.y & 0xffff);
@@ -102,41 +105,53 @@ template <int S> __global__ __launch_bounds__(kDwThreads) void dw3x3_kernel(cons
         ct[3] = b.w - a.zx * s.w;
     }
 
-    const uint8_t *ximg = a.x + (size_t)img * a.in_h * a.in_w * a.channels + c0;
+    const uint32_t in_row = (uint32_t)(a.in_w * a.channels); // elements per input row
+    // offset of (img, row 0, column ix0, channel c0); may "underflow" for ix0 < 0, the sum with
+    // a valid column is in range again (all arithmetic is modulo 2^32)
+    const uint32_t in_base = (uint32_t)img * (uint32_t)a.in_h * in_row + (uint32_t)(ix0 * a.channels + c0);
+    bool col_ok[NCOL];
+#pragma unroll
+    for (int col = 0; col < NCOL; col++) col_ok[col] = (unsigned)(ix0 + col) < (unsigned)a.in_w;
+
     int32_t rows[3][NCOL][4]; // three most recent input rows, unpacked
-    auto load_row = [&](int buf, int iy) {
-        const bool row_ok = (unsigned)iy < (unsigned)a.in_h;
+    int next_iy = iy_first;   // rows are consumed strictly in order
+    uint32_t next_off = in_base + (uint32_t)iy_first * in_row;
+    auto load_row = [&](int buf) {
+        const bool row_ok = (unsigned)next_iy < (unsigned)a.in_h;
 #pragma unroll
         for (int col = 0; col < NCOL; col++) {
-            const int ix = ix0 + col;
             uint32_t d = a.zx_splat;
-            if (row_ok && (unsigned)ix < (unsigned)a.in_w)
-                d = *reinterpret_cast<const uint32_t *>(ximg + ((size_t)iy * a.in_w + ix) * a.channels);
+            if (row_ok && col_ok[col])
+                d = *reinterpret_cast<const uint32_t *>(a.x + (next_off + (uint32_t)(col * a.channels)));
             rows[buf][col][0] = d & 0xff;
             rows[buf][col][1] = (d >> 8) & 0xff;
             rows[buf][col][2] = (d >> 16) & 0xff;
             rows[buf][col][3] = d >> 24;
         }
+        next_iy++;
+        next_off += in_row;
     };
+
+    const uint32_t out_row = (uint32_t)(a.out_w * a.channels);
+    uint32_t out_off = ((uint32_t)img * (uint32_t)a.out_h + (uint32_t)oy0) * out_row + (uint32_t)(ox0 * a.channels + c0);
 
     // Output row t (relative) reads input rows t*S + {0,1,2} (relative), kept in
     // buffer (row index mod 3).  The loop is unrolled by 3 so every buffer index
     // is a compile-time constant.
-    load_row(0, iy_first + 0);
-    load_row(1, iy_first + 1);
-    load_row(2, iy_first + 2);
-    for (int t0 = 0; t0 < kDwRows; t0 += 3) {
+    load_row(0);
+    load_row(1);
+    load_row(2);
+    for (int t0 = 0; t0 < a.rows; t0 += 3) {
 #pragma unroll
         for (int ph = 0; ph < 3; ph++) {
             const int tt = t0 + ph;
             const int oy = oy0 + tt;
-            if (tt < kDwRows && oy < a.out_h) {
+            if (tt < a.rows && oy < a.out_h) {
                 if (tt > 0) {
 #pragma unroll
                     for (int nr = 0; nr < S; nr++) {
-                        // rows (tt-1)*S + 3 + nr, tt % 3 == ph
-                        const int rel_c = ((ph + 2) % 3) * S + 3 + nr; // same residue mod 3 as the real index
-                        load_row(rel_c % 3, iy_first + (tt - 1) * S + 3 + nr);
+                        // input row (tt-1)*S + 3 + nr; tt % 3 == ph fixes its residue mod 3
+                        load_row((((ph + 2) % 3) * S + 3 + nr) % 3);
                     }
                 }
                 int32_t acc[kDwCols][4];
@@ -156,12 +171,9 @@ template <int S> __global__ __launch_bounds__(kDwThreads) void dw3x3_kernel(cons
                                 acc[o][c] += __mul24(rows[buf][o * S + kx][c], w[ky * 3 + kx][c]);
                 }
 #pragma unroll
-                for (int o = 0; o < kDwCols; o++) {
-                    if (ox0 + o < a.out_w) {
-                        const size_t pix = ((size_t)img * a.out_h + oy) * a.out_w + ox0 + o;
-                        dw_store4(a, pix, c0, acc[o]);
-                    }
-                }
+                for (int o = 0; o < kDwCols; o++)
+                    if (ox0 + o < a.out_w) dw_store4(a, out_off + (uint32_t)(o * a.channels), acc[o]);
+                out_off += out_row;
             }
         }
     }
@@ -204,14 +216,13 @@ template <int VEC> __global__ __launch_bounds__(kDwThreads) void dw_generic_kern
             }
         }
     }
-    const size_t pix = ((size_t)img * a.out_h + oy) * a.out_w + ox;
+    const uint32_t o = (((uint32_t)img * a.out_h + oy) * a.out_w + ox) * a.channels + c0;
     if (VEC == 4) {
         int32_t v[4];
 #pragma unroll
         for (int c = 0; c < 4; c++) v[c] = acc[c < VEC ? c : 0];
-        dw_store4(a, pix, c0, v);
+        dw_store4(a, o, v);
     } else {
-        const size_t o = pix * a.channels + c0;
         if (a.ep.out_mode == kOutU8)
             reinterpret_cast<uint8_t *>(a.y)[o] = (uint8_t)requant_u8_lowbyte((float)acc[0] * a.ep.mult, a.ep);
         else if (a.ep.out_mode == kOutI32) reinterpret_cast<int32_t *>(a.y)[o] = acc[0];
@@ -252,8 +263,8 @@ int launch_qconv_depthwise(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_h
     const int64_t in_elems = (int64_t)c->batch * c->in_h * c->in_w * ch;
     const int64_t out_elems = (int64_t)c->batch * out_h * out_w * ch;
     NNHIP_REQUIRE(ctx, out_elems > 0, -EINVAL, "qconv2d(depthwise): empty output");
-    NNHIP_REQUIRE(ctx, in_elems < ((int64_t)1 << 40) && out_elems < ((int64_t)1 << 40), -EINVAL,
-                  "qconv2d(depthwise): tensor too large");
+    NNHIP_REQUIRE(ctx, in_elems < ((int64_t)1 << 31) && out_elems < ((int64_t)1 << 31), -EINVAL,
+                  "qconv2d(depthwise): tensors of 2^31 elements or more are not supported");
     NNHIP_REQUIRE(ctx, w->kernel_h * w->kernel_w <= 258, -EINVAL, "qconv2d(depthwise): window too large");
 
     DwArgs a;
@@ -290,7 +301,12 @@ int launch_qconv_depthwise(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_h
     if (k3) {
         a.cq = ch / 4;
         a.strips = ceil_div(out_w, kDwCols);
-        a.row_chunks = ceil_div(out_h, kDwRows);
+        // Long row strips amortise the two-row halo; short ones keep enough threads in flight
+        // (at least two waves per SIMD) when the image is small.
+        a.rows = kDwMaxRows;
+        const long long want_threads = (long long)ctx->compute_units * 4 * 64 * 2;
+        while (a.rows > 1 && (long long)c->batch * ceil_div(out_h, a.rows) * a.strips * a.cq < want_threads) a.rows /= 2;
+        a.row_chunks = ceil_div(out_h, a.rows);
         a.d_cq = make_fastdiv((uint32_t)a.cq);
         a.d_strips = make_fastdiv((uint32_t)a.strips);
         a.d_rows = make_fastdiv((uint32_t)a.row_chunks);

@@ -7,38 +7,41 @@
 
 namespace nnhip {
 
-static const int kAllowedTiles[] = {1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 12, 14, 16};
+static const int kAllowedTiles[] = {1, 2, 3, 4, 5, 6, 8, 9, 10, 12, 16};
 
-static int round_tiles(int t, int max_tiles) {
+static int round_tiles(int t) {
     for (int v : kAllowedTiles)
-        if (v >= t && v <= max_tiles) return v;
-    return max_tiles;
+        if (v >= t) return v;
+    return 16;
 }
 
-// Chooses the channel-chunk width T (in 16-channel tiles), the number of
-// chunks and the LDS staging depth for a reduction of `ksteps` k-steps.
+// Chooses the channel-chunk width T (in 16-channel tiles), the number of chunks and the
+// LDS staging depth for a reduction of `ksteps` k-steps.  Wide chunks reuse every
+// activation fragment for more output channels; narrow ones give more blocks.  With a
+// pixel-count hint the widest chunk that still yields about two blocks per compute unit
+// (at the smallest pixel tile) is taken; without one, the widest that fits the LDS budget.
 // max_tiles bounds T (the byte-gather loader is only built for T <= 4).
-static void plan_igemm(int g_oc, int ksteps, int max_tiles, int *tiles, int *nchunks, int *kc_steps) {
+static void plan_igemm(int g_oc, int ksteps, int max_tiles, int64_t pixels_hint, int compute_units, int *tiles, int *nchunks,
+                       int *kc_steps) {
     const int tt = ceil_div(g_oc, 16);
-    const int cap = std::min(max_tiles, tt);
-    int t0, kc;
-    if (ksteps * cap <= kLdsFrags) {
-        t0 = cap;
-        kc = ksteps;
-    } else if (ksteps <= 12) {
-        t0 = std::min(cap, kLdsFrags / ksteps);
-        kc = ksteps;
-    } else {
-        t0 = std::min(cap, 4);
-        kc = 12;
+    const long long target = 2LL * compute_units;
+    int best_t = 1, best_kc = std::min(ksteps, kLdsFrags);
+    for (int nc = 1; nc <= tt; nc++) {
+        if (ceil_div(tt, nc) > 16) continue; // more tiles than the widest kernel
+        const int t = round_tiles(ceil_div(tt, nc));
+        if (t > max_tiles) continue;
+        int kc;
+        if (ksteps * t <= kLdsFrags) kc = ksteps;              // whole reduction resident
+        else if (ksteps > 12 && t <= 4) kc = kLdsFrags / t;     // long reduction: staged in pieces
+        else continue;
+        best_t = t;
+        best_kc = kc;
+        if (pixels_hint <= 0 || t == 1) break;
+        if ((long long)ceil_div((int)std::min<int64_t>(pixels_hint, 1 << 30), kWaves * 16) * ceil_div(tt, t) >= target) break;
     }
-    int nc = ceil_div(tt, t0);
-    const int t = round_tiles(ceil_div(tt, nc), max_tiles);
-    while (t * kc > kLdsFrags && kc > 1) kc--; // rounding T up may overshoot the LDS budget
-    nc = ceil_div(tt, t);
-    *tiles = t;
-    *nchunks = nc;
-    *kc_steps = kc;
+    *tiles = best_t;
+    *nchunks = ceil_div(tt, best_t);
+    *kc_steps = best_kc;
 }
 
 // Packs one group's weights into MFMA operand order.
@@ -79,7 +82,7 @@ int prepack_igemm(nncase_hip_ctx *ctx, nncase_hip_weights *w, const uint8_t *w_o
     w->k = taps * w->g_ic;
     w->ksteps = ceil_div(w->k, 64);
     const int max_tiles = (w->g_ic % 4 == 0) ? 16 : 4;
-    plan_igemm(w->g_oc, w->ksteps, max_tiles, &w->tiles, &w->nchunks, &w->kc_steps);
+    plan_igemm(w->g_oc, w->ksteps, max_tiles, w->pixels_hint, ctx->compute_units, &w->tiles, &w->nchunks, &w->kc_steps);
     const size_t group_bytes = (size_t)w->nchunks * w->ksteps * w->tiles * 1024;
     w->packed_bytes = group_bytes * w->groups;
     std::vector<uint8_t> packed(w->packed_bytes);
@@ -102,6 +105,10 @@ int prepack_igemm(nncase_hip_ctx *ctx, nncase_hip_weights *w, const uint8_t *w_o
     NNHIP_HIP(ctx, hipMemcpy(w->d_wsum, wsum.data(), sizeof(int32_t) * w->out_channels, hipMemcpyHostToDevice));
     NNHIP_HIP(ctx, hipMemcpy(w->d_bias, hb.data(), sizeof(int32_t) * w->out_channels, hipMemcpyHostToDevice));
     return 0;
+}
+
+int igemm_pixel_groups(const nncase_hip_ctx *ctx, const nncase_hip_weights *w, int m) {
+    return choose_rg(ctx, w->tiles, w->nchunks, m);
 }
 
 int igemm_load_mode(const nncase_hip_weights *w, const nncase_hip_conv2d_args_t *c, int out_h, int out_w) {
@@ -168,13 +175,14 @@ int launch_qconv_igemm(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_hip_w
         a.bias = w->d_bias + (size_t)g * w->g_oc;
         a.x_coff = g * w->g_ic;
         a.y_coff = g * w->g_oc;
+        const int rg = choose_rg(ctx, w->tiles, w->nchunks, a.m);
         int rc;
         switch (mode) {
-        case kRows16: rc = launch_igemm_rows16(ctx, a, w->tiles, w->nchunks); break;
-        case kVec16: rc = launch_igemm_vec16(ctx, a, w->tiles, w->nchunks); break;
-        case kVec8: rc = launch_igemm_vec8(ctx, a, w->tiles, w->nchunks); break;
-        case kVec4: rc = launch_igemm_vec4(ctx, a, w->tiles, w->nchunks); break;
-        default: rc = launch_igemm_bytes(ctx, a, w->tiles, w->nchunks); break;
+        case kRows16: rc = launch_igemm_rows16(ctx, a, w->tiles, w->nchunks, rg); break;
+        case kVec16: rc = launch_igemm_vec16(ctx, a, w->tiles, w->nchunks, rg); break;
+        case kVec8: rc = launch_igemm_vec8(ctx, a, w->tiles, w->nchunks, rg); break;
+        case kVec4: rc = launch_igemm_vec4(ctx, a, w->tiles, w->nchunks, rg); break;
+        default: rc = launch_igemm_bytes(ctx, a, w->tiles, w->nchunks, rg); break;
         }
         if (rc) return rc;
     }

@@ -325,8 +325,16 @@ __global__ __launch_bounds__(kThreads, 2) void qconv_igemm_kernel(const IgemmArg
     }
 }
 
-template <int T, int MODE> int launch_t(nncase_hip_ctx *ctx, const IgemmArgs &a, int nchunks) {
-    constexpr int RG = (T <= 8) ? 4 : 2;
+// Pixel groups per wave (RG) for a chunk width of T tiles: the widest that still gives
+// every compute unit a couple of blocks.  RG = 4 is only built for T <= 8 (register budget).
+inline int choose_rg(const nncase_hip_ctx *ctx, int tiles, int nchunks, int m) {
+    const long long target = 2LL * ctx->compute_units;
+    for (int rg = tiles <= 8 ? 4 : 2; rg > 1; rg /= 2)
+        if ((long long)ceil_div(m, kWaves * rg * 16) * nchunks >= target) return rg;
+    return 1;
+}
+
+template <int T, int RG, int MODE> int launch_trg(nncase_hip_ctx *ctx, const IgemmArgs &a, int nchunks) {
     IgemmArgs args = a;
     constexpr int pix_per_block = kWaves * RG * 16;
     args.num_mtiles = ceil_div(a.m, pix_per_block);
@@ -341,35 +349,42 @@ template <int T, int MODE> int launch_t(nncase_hip_ctx *ctx, const IgemmArgs &a,
     return 0;
 }
 
-template <int MODE> int launch_mode(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks) {
+template <int T, int MODE> int launch_t(nncase_hip_ctx *ctx, const IgemmArgs &a, int nchunks, int rg) {
+    if (rg == 1) return launch_trg<T, 1, MODE>(ctx, a, nchunks);
+    if (rg == 2) return launch_trg<T, 2, MODE>(ctx, a, nchunks);
+    if constexpr (T <= 8) {
+        if (rg == 4) return launch_trg<T, 4, MODE>(ctx, a, nchunks);
+    }
+    return fail(ctx, -EINVAL, "igemm: no kernel for %d tiles x %d pixel groups", T, rg);
+}
+
+template <int MODE> int launch_mode(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks, int rg) {
     switch (tiles) {
-    case 1: return launch_t<1, MODE>(ctx, a, nchunks);
-    case 2: return launch_t<2, MODE>(ctx, a, nchunks);
-    case 3: return launch_t<3, MODE>(ctx, a, nchunks);
-    case 4: return launch_t<4, MODE>(ctx, a, nchunks);
+    case 1: return launch_t<1, MODE>(ctx, a, nchunks, rg);
+    case 2: return launch_t<2, MODE>(ctx, a, nchunks, rg);
+    case 3: return launch_t<3, MODE>(ctx, a, nchunks, rg);
+    case 4: return launch_t<4, MODE>(ctx, a, nchunks, rg);
     default: break;
     }
     if constexpr (MODE != kBytes) {
         switch (tiles) {
-        case 5: return launch_t<5, MODE>(ctx, a, nchunks);
-        case 6: return launch_t<6, MODE>(ctx, a, nchunks);
-        case 7: return launch_t<7, MODE>(ctx, a, nchunks);
-        case 8: return launch_t<8, MODE>(ctx, a, nchunks);
-        case 9: return launch_t<9, MODE>(ctx, a, nchunks);
-        case 10: return launch_t<10, MODE>(ctx, a, nchunks);
-        case 12: return launch_t<12, MODE>(ctx, a, nchunks);
-        case 14: return launch_t<14, MODE>(ctx, a, nchunks);
-        case 16: return launch_t<16, MODE>(ctx, a, nchunks);
+        case 5: return launch_t<5, MODE>(ctx, a, nchunks, rg);
+        case 6: return launch_t<6, MODE>(ctx, a, nchunks, rg);
+        case 8: return launch_t<8, MODE>(ctx, a, nchunks, rg);
+        case 9: return launch_t<9, MODE>(ctx, a, nchunks, rg);
+        case 10: return launch_t<10, MODE>(ctx, a, nchunks, rg);
+        case 12: return launch_t<12, MODE>(ctx, a, nchunks, rg);
+        case 16: return launch_t<16, MODE>(ctx, a, nchunks, rg);
         default: break;
         }
     }
     return fail(ctx, -EINVAL, "igemm: no kernel for %d tiles (load mode %d)", tiles, MODE);
 }
 
-int launch_igemm_rows16(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks);
-int launch_igemm_vec16(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks);
-int launch_igemm_vec8(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks);
-int launch_igemm_vec4(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks);
-int launch_igemm_bytes(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks);
+int launch_igemm_rows16(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks, int rg);
+int launch_igemm_vec16(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks, int rg);
+int launch_igemm_vec8(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks, int rg);
+int launch_igemm_vec4(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks, int rg);
+int launch_igemm_bytes(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks, int rg);
 
 } // namespace nnhip

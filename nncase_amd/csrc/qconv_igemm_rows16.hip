@@ -2,7 +2,7 @@
 #include "qconv_igemm.hpp"
 
 namespace nnhip {
-int launch_igemm_rows16(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks) {
-    return launch_mode<kRows16>(ctx, a, tiles, nchunks);
+int launch_igemm_rows16(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks, int rg) {
+    return launch_mode<kRows16>(ctx, a, tiles, nchunks, rg);
 }
 } // namespace nnhip

@@ -85,7 +85,7 @@ def conv2d(input: np.ndarray, weights: np.ndarray, bias: Optional[np.ndarray], s
     (ph0, ph1), (pw0, pw1) = padding
     oh = rt.windowed_output_size(h, kh, stride[0], dilation[0], ph0, ph1)
     ow = rt.windowed_output_size(wd, kw, stride[1], dilation[1], pw0, pw1)
-    wts = c.prepack_conv2d(w, bias, weights_qp, groups)
+    wts = c.prepack_conv2d(w, bias, weights_qp, groups, expected_pixels=n * oh * ow)
     x_nchw = c.to_device(x)
     x_nhwc = c.alloc(x.size)
     c.nchw_to_nhwc(x_nchw, x_nhwc, 1, n, ch, h, wd)
@@ -116,7 +116,7 @@ def mat_mul(lhs: np.ndarray, rhs: np.ndarray, lhs_qp: QuantParam, rhs_qp: QuantP
     lead = a.shape[:-1]
     m = int(np.prod(lead)) if lead else 1
     out_dtype = np.dtype(out_dtype)
-    wts = c.prepack_matmul(b, bias, rhs_qp)
+    wts = c.prepack_matmul(b, bias, rhs_qp, expected_rows=m)
     da = c.to_device(a)
     dy = c.alloc(max(1, m * n * out_dtype.itemsize))
     args = rt.MatmulArgs(m, lhs_qp, output_qp or qp(0, 1.0), fused_clamp[0], fused_clamp[1], _out_dt(out_dtype))

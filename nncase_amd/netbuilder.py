@@ -247,7 +247,7 @@ class HipModel:
                 self.fn.add_quantize(self.input_f32, rt.DT_F32, buf, rt.DT_U8, self.in_count, qp(*n.out_qp))
             elif n.op == "conv":
                 src = qg.nodes[n.inputs[0]]
-                wt = ctx.prepack_conv2d(n.weights, n.bias, qp(*n.w_qp), n.groups)
+                wt = ctx.prepack_conv2d(n.weights, n.bias, qp(*n.w_qp), n.groups, expected_pixels=batch * hh * ww)
                 self.weights[-1] = wt
                 (ph0, ph1), (pw0, pw1) = n.padding
                 args = rt.Conv2dArgs(batch, src.out_shape[1], src.out_shape[2], n.stride[0], n.stride[1], 1, 1, ph0, ph1, pw0,

