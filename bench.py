@@ -120,7 +120,7 @@ def main():
     dom_gbs = dom["bytes"] / (dom["ms"] * 1e-3) / 1e9
 
     def klass(name):
-        return "dense" if name.startswith("qconv_igemm") else ("depthwise" if name.startswith("dw") else "elementwise")
+        return "dense" if name.startswith("qconv_") else ("depthwise" if name.startswith("dw") else "elementwise")
 
     classes = {}
     for name, g in groups.items():

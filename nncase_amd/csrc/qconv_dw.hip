@@ -63,8 +63,24 @@ __device__ __forceinline__ void dw_store4(const DwArgs &a, uint32_t o, const int
     }
 }
 
+// acc + x.i16[H] * w.i16[H] (v_mad_i32_i16 with op_sel picking the 16-bit halves): the
+// multiply-add reads both 16-bit halves of a register directly, so activations are kept
+// as two zero-extended bytes per register and weights as the int16 pairs they are stored as.
+__device__ __forceinline__ int32_t mad16_lo(uint32_t x, uint32_t w, int32_t acc) {
+    int32_t d;
+    asm("v_mad_i32_i16 %0, %1, %2, %3" : "=v"(d) : "v"(x), "v"(w), "v"(acc));
+    return d;
+}
+__device__ __forceinline__ int32_t mad16_hi(uint32_t x, uint32_t w, int32_t acc) {
+    int32_t d;
+    asm("v_mad_i32_i16 %0, %1, %2, %3 op_sel:[1,1,0,0]" : "=v"(d) : "v"(x), "v"(w), "v"(acc));
+    return d;
+}
+
 // All offsets are 32-bit element offsets from the (uniform) tensor bases, advanced by
 // additions only; the host checks that both tensors stay below 2^31 elements.
+// The loads of the rows the NEXT output row needs are issued before the current row is
+// computed, so a whole row of arithmetic covers their latency.
 template <int S> __global__ __launch_bounds__(kDwThreads) void dw3x3_kernel(const DwArgs a) {
     constexpr int NCOL = (kDwCols - 1) * S + 3;
     const uint32_t gid = blockIdx.x * kDwThreads + threadIdx.x;
@@ -87,14 +103,13 @@ template <int S> __global__ __launch_bounds__(kDwThreads) void dw3x3_kernel(cons
     const int ix0 = ox0 * S - a.pad_w;
     const int iy_first = oy0 * S - a.pad_h;
 
-    int32_t w[9][4], ct[4];
+    uint32_t w01[9], w23[9]; // (w - zw) of channels (0,1) and (2,3) as int16 pairs, per tap
+    int32_t ct[4];
 #pragma unroll
     for (int tap = 0; tap < 9; tap++) {
         const uint2 raw = *reinterpret_cast<const uint2 *>(a.w + (uint32_t)(tap * a.channels + c0));
-        w[tap][0] = (int16_t)(raw.x & 0xffff);
-        w[tap][1] = (int16_t)(raw.x >> 16);
-        w[tap][2] = (int16_t)(raw.y & 0xffff);
-        w[tap][3] = (int16_t)(raw.y >> 16);
+        w01[tap] = raw.x;
+        w23[tap] = raw.y;
     }
     {
         const int4 b = *reinterpret_cast<const int4 *>(a.bias + c0);
@@ -106,30 +121,37 @@ template <int S> __global__ __launch_bounds__(kDwThreads) void dw3x3_kernel(cons
     }
 
     const uint32_t in_row = (uint32_t)(a.in_w * a.channels); // elements per input row
-    // offset of (img, row 0, column ix0, channel c0); may "underflow" for ix0 < 0, the sum with
-    // a valid column is in range again (all arithmetic is modulo 2^32)
-    const uint32_t in_base = (uint32_t)img * (uint32_t)a.in_h * in_row + (uint32_t)(ix0 * a.channels + c0);
+    const uint32_t in_base = (uint32_t)img * (uint32_t)a.in_h * in_row + (uint32_t)c0; // (img, row 0, column 0, c0)
+    // Loads are unconditional: a tap outside the image reads the nearest pixel inside it
+    // (always a valid address) and the value is replaced by the zero point afterwards, so
+    // the border handling costs one select per load and no divergent branches.
     bool col_ok[NCOL];
+    uint32_t col_off[NCOL];
 #pragma unroll
-    for (int col = 0; col < NCOL; col++) col_ok[col] = (unsigned)(ix0 + col) < (unsigned)a.in_w;
+    for (int col = 0; col < NCOL; col++) {
+        const int ix = ix0 + col;
+        col_ok[col] = (unsigned)ix < (unsigned)a.in_w;
+        col_off[col] = (uint32_t)(min(max(ix, 0), a.in_w - 1) * a.channels);
+    }
 
-    int32_t rows[3][NCOL][4]; // three most recent input rows, unpacked
-    int next_iy = iy_first;   // rows are consumed strictly in order
-    uint32_t next_off = in_base + (uint32_t)iy_first * in_row;
-    auto load_row = [&](int buf) {
+    uint32_t r01[3][NCOL], r23[3][NCOL]; // three most recent input rows, two channels per register
+    int next_iy = iy_first;             // rows are fetched strictly in order
+    auto fetch_row = [&](uint32_t (&raw)[NCOL]) {
         const bool row_ok = (unsigned)next_iy < (unsigned)a.in_h;
+        const uint32_t row_off = in_base + (uint32_t)min(max(next_iy, 0), a.in_h - 1) * in_row;
 #pragma unroll
         for (int col = 0; col < NCOL; col++) {
-            uint32_t d = a.zx_splat;
-            if (row_ok && col_ok[col])
-                d = *reinterpret_cast<const uint32_t *>(a.x + (next_off + (uint32_t)(col * a.channels)));
-            rows[buf][col][0] = d & 0xff;
-            rows[buf][col][1] = (d >> 8) & 0xff;
-            rows[buf][col][2] = (d >> 16) & 0xff;
-            rows[buf][col][3] = d >> 24;
+            const uint32_t v = *reinterpret_cast<const uint32_t *>(a.x + (row_off + col_off[col]));
+            raw[col] = (row_ok && col_ok[col]) ? v : a.zx_splat;
         }
         next_iy++;
-        next_off += in_row;
+    };
+    auto unpack_row = [&](int buf, const uint32_t (&raw)[NCOL]) {
+#pragma unroll
+        for (int col = 0; col < NCOL; col++) {
+            r01[buf][col] = __builtin_amdgcn_perm(0u, raw[col], 0x0c010c00u); // [b0, 0, b1, 0]
+            r23[buf][col] = __builtin_amdgcn_perm(0u, raw[col], 0x0c030c02u); // [b2, 0, b3, 0]
+        }
     };
 
     const uint32_t out_row = (uint32_t)(a.out_w * a.channels);
@@ -138,21 +160,33 @@ template <int S> __global__ __launch_bounds__(kDwThreads) void dw3x3_kernel(cons
     // Output row t (relative) reads input rows t*S + {0,1,2} (relative), kept in
     // buffer (row index mod 3).  The loop is unrolled by 3 so every buffer index
     // is a compile-time constant.
-    load_row(0);
-    load_row(1);
-    load_row(2);
-    for (int t0 = 0; t0 < a.rows; t0 += 3) {
+    uint32_t pre[S][NCOL]; // rows fetched ahead for the next output row
+    {
+        uint32_t raw[NCOL];
+#pragma unroll
+        for (int b = 0; b < 3; b++) {
+            fetch_row(raw);
+            unpack_row(b, raw);
+        }
+    }
+    const int nrows = min(a.rows, a.out_h - oy0); // >= 1
+    if (nrows > 1) {
+#pragma unroll
+        for (int nr = 0; nr < S; nr++) fetch_row(pre[nr]);
+    }
+    for (int t0 = 0; t0 < nrows; t0 += 3) {
 #pragma unroll
         for (int ph = 0; ph < 3; ph++) {
             const int tt = t0 + ph;
-            const int oy = oy0 + tt;
-            if (tt < a.rows && oy < a.out_h) {
+            if (tt < nrows) {
                 if (tt > 0) {
+                    // input rows (tt-1)*S + 3 + nr; tt % 3 == ph fixes their residue mod 3
 #pragma unroll
-                    for (int nr = 0; nr < S; nr++) {
-                        // input row (tt-1)*S + 3 + nr; tt % 3 == ph fixes its residue mod 3
-                        load_row((((ph + 2) % 3) * S + 3 + nr) % 3);
-                    }
+                    for (int nr = 0; nr < S; nr++) unpack_row((((ph + 2) % 3) * S + 3 + nr) % 3, pre[nr]);
+                }
+                if (tt + 1 < nrows) {
+#pragma unroll
+                    for (int nr = 0; nr < S; nr++) fetch_row(pre[nr]);
                 }
                 int32_t acc[kDwCols][4];
 #pragma unroll
@@ -165,10 +199,13 @@ template <int S> __global__ __launch_bounds__(kDwThreads) void dw3x3_kernel(cons
 #pragma unroll
                     for (int kx = 0; kx < 3; kx++)
 #pragma unroll
-                        for (int o = 0; o < kDwCols; o++)
-#pragma unroll
-                            for (int c = 0; c < 4; c++)
-                                acc[o][c] += __mul24(rows[buf][o * S + kx][c], w[ky * 3 + kx][c]);
+                        for (int o = 0; o < kDwCols; o++) {
+                            const int col = o * S + kx, tap = ky * 3 + kx;
+                            acc[o][0] = mad16_lo(r01[buf][col], w01[tap], acc[o][0]);
+                            acc[o][1] = mad16_hi(r01[buf][col], w01[tap], acc[o][1]);
+                            acc[o][2] = mad16_lo(r23[buf][col], w23[tap], acc[o][2]);
+                            acc[o][3] = mad16_hi(r23[buf][col], w23[tap], acc[o][3]);
+                        }
                 }
 #pragma unroll
                 for (int o = 0; o < kDwCols; o++)
@@ -301,11 +338,31 @@ int launch_qconv_depthwise(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_h
     if (k3) {
         a.cq = ch / 4;
         a.strips = ceil_div(out_w, kDwCols);
-        // Long row strips amortise the two-row halo; short ones keep enough threads in flight
-        // (at least two waves per SIMD) when the image is small.
-        a.rows = kDwMaxRows;
-        const long long want_threads = (long long)ctx->compute_units * 4 * 64 * 2;
-        while (a.rows > 1 && (long long)c->batch * ceil_div(out_h, a.rows) * a.strips * a.cq < want_threads) a.rows /= 2;
+        // Rows per thread.  Long strips amortise the two-row halo and the per-thread set-up;
+        // short ones give more waves.  While every SIMD gets at least a few waves, the waves are
+        // dealt out in whole numbers, so the length that minimises (waves per SIMD, rounded up)
+        // x (work per wave) wins; smaller problems are latency-bound and take the shortest
+        // strips that still leave two waves per SIMD.
+        {
+            const long long simds = (long long)ctx->compute_units * 4;
+            auto waves_for = [&](int rows) {
+                return ((long long)c->batch * ceil_div(out_h, rows) * a.strips * a.cq + 63) / 64;
+            };
+            if (waves_for(kDwMaxRows) >= 3 * simds) {
+                long long best_cost = -1;
+                for (int rows = 2; rows <= kDwMaxRows; rows++) {
+                    const long long per_simd = (waves_for(rows) + simds - 1) / simds;
+                    const long long cost = per_simd * (rows * 340 + 100);
+                    if (best_cost < 0 || cost < best_cost) {
+                        best_cost = cost;
+                        a.rows = rows;
+                    }
+                }
+            } else {
+                a.rows = kDwMaxRows;
+                while (a.rows > 1 && waves_for(a.rows) < 2 * simds) a.rows /= 2;
+            }
+        }
         a.row_chunks = ceil_div(out_h, a.rows);
         a.d_cq = make_fastdiv((uint32_t)a.cq);
         a.d_strips = make_fastdiv((uint32_t)a.strips);

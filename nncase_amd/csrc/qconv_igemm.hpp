@@ -261,7 +261,7 @@ __global__ __launch_bounds__(kThreads, 2) void qconv_igemm_kernel(const IgemmArg
         for (int rg = 0; rg < RG; rg++) {
             const int p = mt * pix_per_block + (wave * RG + rg) * 16 + j;
             if (p < a.m && ch0 < a.n) {
-                const int32_t rsz = a.zwp * rs[rg][0];
+                const int32_t nrsz = -a.zwp * rs[rg][0];
                 const size_t obase = (size_t)p * a.ldy + a.y_coff + ch0;
                 if (a.ep.out_mode == kOutU8) {
                     uint8_t *yo = reinterpret_cast<uint8_t *>(a.y) + obase;
@@ -272,7 +272,7 @@ __global__ __launch_bounds__(kThreads, 2) void qconv_igemm_kernel(const IgemmArg
                         uint32_t b[4];
 #pragma unroll
                         for (int r = 0; r < 4; r++) {
-                            const int32_t v = acc[rg][nt][r] + ct[r] - rsz;
+                            const int32_t v = acc[rg][nt][r] + ct[r] + nrsz;
                             b[r] = requant_u8_lowbyte((float)v * a.ep.mult, a.ep);
                         }
                         packed[nt] = pack_low_bytes(b[0], b[1], b[2], b[3]);
@@ -305,7 +305,7 @@ __global__ __launch_bounds__(kThreads, 2) void qconv_igemm_kernel(const IgemmArg
                         uint32_t o[4];
 #pragma unroll
                         for (int r = 0; r < 4; r++) {
-                            const int32_t v = acc[rg][nt][r] + ct[r] - rsz;
+                            const int32_t v = acc[rg][nt][r] + ct[r] + nrsz;
                             if (a.ep.out_mode == kOutI32) o[r] = (uint32_t)v;
                             else o[r] = __float_as_uint(clamp_ref((float)v * a.ep.mult, a.ep.lo, a.ep.hi));
                         }
