@@ -101,6 +101,14 @@ __device__ __forceinline__ uint32_t pack_low_bytes(uint32_t b0, uint32_t b1, uin
     return lo | hi;
 }
 
+// a + b + c in one instruction (the compiler otherwise re-associates the zero-point
+// correction into a subtract and an add).
+__device__ __forceinline__ int32_t add3(int32_t a, int32_t b, int32_t c) {
+    int32_t d;
+    asm("v_add3_u32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "v"(c));
+    return d;
+}
+
 __device__ __forceinline__ float clamp_ref(float v, float lo, float hi) {
     return __builtin_fmaxf(__builtin_fminf(v, hi), lo);
 }

@@ -136,21 +136,21 @@ template <int S> __global__ __launch_bounds__(kDwThreads) void dw3x3_kernel(cons
 
     uint32_t r01[3][NCOL], r23[3][NCOL]; // three most recent input rows, two channels per register
     int next_iy = iy_first;             // rows are fetched strictly in order
-    auto fetch_row = [&](uint32_t (&raw)[NCOL]) {
-        const bool row_ok = (unsigned)next_iy < (unsigned)a.in_h;
+    // fetch_row only issues the loads (nothing depends on their data); unpack_row, called one
+    // output row later, applies the border replacement and splits the bytes.
+    auto fetch_row = [&](uint32_t (&raw)[NCOL], bool &row_ok) {
+        row_ok = (unsigned)next_iy < (unsigned)a.in_h;
         const uint32_t row_off = in_base + (uint32_t)min(max(next_iy, 0), a.in_h - 1) * in_row;
 #pragma unroll
-        for (int col = 0; col < NCOL; col++) {
-            const uint32_t v = *reinterpret_cast<const uint32_t *>(a.x + (row_off + col_off[col]));
-            raw[col] = (row_ok && col_ok[col]) ? v : a.zx_splat;
-        }
+        for (int col = 0; col < NCOL; col++) raw[col] = *reinterpret_cast<const uint32_t *>(a.x + (row_off + col_off[col]));
         next_iy++;
     };
-    auto unpack_row = [&](int buf, const uint32_t (&raw)[NCOL]) {
+    auto unpack_row = [&](int buf, const uint32_t (&raw)[NCOL], bool row_ok) {
 #pragma unroll
         for (int col = 0; col < NCOL; col++) {
-            r01[buf][col] = __builtin_amdgcn_perm(0u, raw[col], 0x0c010c00u); // [b0, 0, b1, 0]
-            r23[buf][col] = __builtin_amdgcn_perm(0u, raw[col], 0x0c030c02u); // [b2, 0, b3, 0]
+            const uint32_t d = (row_ok && col_ok[col]) ? raw[col] : a.zx_splat;
+            r01[buf][col] = __builtin_amdgcn_perm(0u, d, 0x0c010c00u); // [b0, 0, b1, 0]
+            r23[buf][col] = __builtin_amdgcn_perm(0u, d, 0x0c030c02u); // [b2, 0, b3, 0]
         }
     };
 
@@ -161,18 +161,19 @@ template <int S> __global__ __launch_bounds__(kDwThreads) void dw3x3_kernel(cons
     // buffer (row index mod 3).  The loop is unrolled by 3 so every buffer index
     // is a compile-time constant.
     uint32_t pre[S][NCOL]; // rows fetched ahead for the next output row
+    bool pre_ok[S];
     {
-        uint32_t raw[NCOL];
+        uint32_t raw[3][NCOL];
+        bool ok[3];
 #pragma unroll
-        for (int b = 0; b < 3; b++) {
-            fetch_row(raw);
-            unpack_row(b, raw);
-        }
+        for (int b = 0; b < 3; b++) fetch_row(raw[b], ok[b]);
+#pragma unroll
+        for (int b = 0; b < 3; b++) unpack_row(b, raw[b], ok[b]);
     }
     const int nrows = min(a.rows, a.out_h - oy0); // >= 1
     if (nrows > 1) {
 #pragma unroll
-        for (int nr = 0; nr < S; nr++) fetch_row(pre[nr]);
+        for (int nr = 0; nr < S; nr++) fetch_row(pre[nr], pre_ok[nr]);
     }
     for (int t0 = 0; t0 < nrows; t0 += 3) {
 #pragma unroll
@@ -182,11 +183,11 @@ template <int S> __global__ __launch_bounds__(kDwThreads) void dw3x3_kernel(cons
                 if (tt > 0) {
                     // input rows (tt-1)*S + 3 + nr; tt % 3 == ph fixes their residue mod 3
 #pragma unroll
-                    for (int nr = 0; nr < S; nr++) unpack_row((((ph + 2) % 3) * S + 3 + nr) % 3, pre[nr]);
+                    for (int nr = 0; nr < S; nr++) unpack_row((((ph + 2) % 3) * S + 3 + nr) % 3, pre[nr], pre_ok[nr]);
                 }
                 if (tt + 1 < nrows) {
 #pragma unroll
-                    for (int nr = 0; nr < S; nr++) fetch_row(pre[nr]);
+                    for (int nr = 0; nr < S; nr++) fetch_row(pre[nr], pre_ok[nr]);
                 }
                 int32_t acc[kDwCols][4];
 #pragma unroll

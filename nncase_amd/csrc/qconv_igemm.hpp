@@ -34,6 +34,9 @@
 
 #include "qconv.hpp"
 
+#include <algorithm>
+#include <cstdlib>
+
 namespace nnhip {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
@@ -95,66 +98,104 @@ template <int MODE> __device__ __forceinline__ PixInfo pix_info(const IgemmArgs 
     return pi;
 }
 
-// Byte offset of input element (tap of reduction index kk) for pixel pi, or -1
-// when the tap falls into the padding.
-__device__ __forceinline__ int tap_offset(const IgemmArgs &a, const PixInfo &pi, int kk) {
+// Location of the input element that reduction index kk of pixel `pi` reads.  The returned
+// offset is always inside the tensor (coordinates are clamped); `inside` tells whether the
+// tap really lies in the image or in the padding.
+__device__ __forceinline__ uint32_t tap_offset(const IgemmArgs &a, const PixInfo &pi, int kk, bool *inside) {
     const uint32_t tap = fastdiv((uint32_t)kk, a.d_gic);
     const int c = kk - (int)tap * a.g_ic;
     const uint32_t ky = fastdiv(tap, a.d_kw);
     const int kx = (int)tap - (int)ky * a.kw;
     const int iy = pi.iy0 + (int)ky * a.dil_h;
     const int ix = pi.ix0 + kx * a.dil_w;
-    if ((unsigned)iy >= (unsigned)a.in_h || (unsigned)ix >= (unsigned)a.in_w) return -1;
-    return (int)((uint32_t)(pi.base + iy * a.in_w + ix) * (uint32_t)a.ldx + a.x_coff + c);
+    *inside = (unsigned)iy < (unsigned)a.in_h && (unsigned)ix < (unsigned)a.in_w;
+    const int cy = min(max(iy, 0), a.in_h - 1), cx = min(max(ix, 0), a.in_w - 1);
+    return (uint32_t)(pi.base + cy * a.in_w + cx) * (uint32_t)a.ldx + a.x_coff + c;
 }
 
-// 16 bytes of the activation operand for k in [kc*16, kc*16+16) of pixel `pi`,
-// already re-biased to s8.
-template <int MODE> __device__ __forceinline__ v4i load_act(const IgemmArgs &a, const PixInfo &pi, int kc) {
-    uint32_t w[4] = {0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u}; // x' = 0
-    if (pi.base >= 0) {
-        if (MODE == kRows16) {
-            if (kc * 16 < a.k) {
-                const u32x4 v = *reinterpret_cast<const u32x4 *>(
-                    a.x + (size_t)((uint32_t)pi.base * (uint32_t)a.ldx + a.x_coff + kc * 16));
-                w[0] = v[0], w[1] = v[1], w[2] = v[2], w[3] = v[3];
-            }
-        } else if (MODE == kBytes) {
+// A 16-byte slice of the activation operand in flight.  The load is issued
+// unconditionally from an address that is always valid; what the slice should have
+// contained where the load does not apply (padding taps: the zero point; reduction
+// indices past K or pixels past M: x' = 0) is kept in `fill` / `take` and applied only
+// when the slice is consumed, so nothing depends on the loaded data until then and the
+// load stays in flight across the multiply of the previous slice.
+struct ActFrag {
+    u32x4 raw;     // loaded bytes
+    u32x4 fill;    // replacement per dword
+    uint32_t take; // bit d set: dword d comes from raw
+};
+
+__device__ __forceinline__ v4i finish_act(const ActFrag &f) {
+    u32x4 r;
+    r[0] = (f.take & 1u) ? f.raw[0] : f.fill[0];
+    r[1] = (f.take & 2u) ? f.raw[1] : f.fill[1];
+    r[2] = (f.take & 4u) ? f.raw[2] : f.fill[2];
+    r[3] = (f.take & 8u) ? f.raw[3] : f.fill[3];
+    r ^= 0x80808080u;
+    return __builtin_bit_cast(v4i, r);
+}
+
+template <int MODE> __device__ __forceinline__ ActFrag load_act(const IgemmArgs &a, const PixInfo &pi, int kc) {
+    const u32x4 zero_s8 = {0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u}; // x' = 0
+    ActFrag f;
+    f.take = 0;
+    f.raw = zero_s8;
+    f.fill = zero_s8;
+    const bool pix_ok = pi.base >= 0;
+    PixInfo sp = pi; // any valid pixel for the address
+    if (!pix_ok) sp.base = 0, sp.iy0 = 0, sp.ix0 = 0;
+    if (MODE == kRows16) {
+        const bool in_k = kc * 16 < a.k;
+        const int kcc = in_k ? kc : 0;
+        f.raw = *reinterpret_cast<const u32x4 *>(a.x + (size_t)((uint32_t)sp.base * (uint32_t)a.ldx + a.x_coff + kcc * 16));
+        f.take = (pix_ok && in_k) ? 0xfu : 0u;
+    } else if (MODE == kBytes) {
+        // byte gathers: assembled immediately (this loader does not overlap with the multiply)
+        uint32_t w0 = 0x80808080u, w1 = 0x80808080u, w2 = 0x80808080u, w3 = 0x80808080u;
+        if (pix_ok) {
 #pragma unroll
             for (int b = 0; b < 16; b++) {
                 const int kk = kc * 16 + b;
                 if (kk < a.k) {
-                    const int off = tap_offset(a, pi, kk);
-                    const uint32_t byte = off >= 0 ? (uint32_t)a.x[(size_t)(uint32_t)off] : (a.zx_splat & 0xffu);
-                    w[b >> 2] = (w[b >> 2] & ~(0xffu << (8 * (b & 3)))) | (byte << (8 * (b & 3)));
-                }
-            }
-        } else {
-            constexpr int VW = MODE == kVec16 ? 16 : (MODE == kVec8 ? 8 : 4);
-#pragma unroll
-            for (int piece = 0; piece < 16 / VW; piece++) {
-                const int kk = kc * 16 + piece * VW;
-                if (kk < a.k) {
-                    const int off = tap_offset(a, pi, kk);
-                    if (VW == 16) {
-                        u32x4 v = {a.zx_splat, a.zx_splat, a.zx_splat, a.zx_splat};
-                        if (off >= 0) v = *reinterpret_cast<const u32x4 *>(a.x + (size_t)(uint32_t)off);
-                        w[0] = v[0], w[1] = v[1], w[2] = v[2], w[3] = v[3];
-                    } else if (VW == 8) {
-                        u32x2 v = {a.zx_splat, a.zx_splat};
-                        if (off >= 0) v = *reinterpret_cast<const u32x2 *>(a.x + (size_t)(uint32_t)off);
-                        w[piece * 2] = v[0], w[piece * 2 + 1] = v[1];
-                    } else {
-                        uint32_t v = a.zx_splat;
-                        if (off >= 0) v = *reinterpret_cast<const uint32_t *>(a.x + (size_t)(uint32_t)off);
-                        w[piece] = v;
-                    }
+                    bool inside;
+                    const uint32_t off = tap_offset(a, pi, kk, &inside);
+                    const uint32_t byte = inside ? (uint32_t)a.x[(size_t)off] : (a.zx_splat & 0xffu);
+                    const uint32_t clr = ~(0xffu << (8 * (b & 3))), ins = byte << (8 * (b & 3));
+                    if ((b >> 2) == 0) w0 = (w0 & clr) | ins;
+                    if ((b >> 2) == 1) w1 = (w1 & clr) | ins;
+                    if ((b >> 2) == 2) w2 = (w2 & clr) | ins;
+                    if ((b >> 2) == 3) w3 = (w3 & clr) | ins;
                 }
             }
         }
+        f.fill = u32x4{w0, w1, w2, w3};
+    } else {
+        constexpr int VW = MODE == kVec16 ? 16 : (MODE == kVec8 ? 8 : 4);
+#pragma unroll
+        for (int piece = 0; piece < 16 / VW; piece++) {
+            const int kk = kc * 16 + piece * VW;
+            const bool in_k = kk < a.k;
+            bool inside;
+            const uint32_t off = tap_offset(a, sp, in_k ? kk : 0, &inside);
+            const bool ok = pix_ok && in_k && inside;
+            const uint32_t fill = (pix_ok && in_k) ? a.zx_splat : 0x80808080u; // padding tap : outside the problem
+            if (VW == 16) {
+                f.raw = *reinterpret_cast<const u32x4 *>(a.x + (size_t)off);
+                f.fill = u32x4{fill, fill, fill, fill};
+                f.take = ok ? 0xfu : 0u;
+            } else if (VW == 8) {
+                const u32x2 v = *reinterpret_cast<const u32x2 *>(a.x + (size_t)off);
+                f.raw[piece * 2] = v[0], f.raw[piece * 2 + 1] = v[1];
+                f.fill[piece * 2] = fill, f.fill[piece * 2 + 1] = fill;
+                f.take |= ok ? (3u << (piece * 2)) : 0u;
+            } else {
+                f.raw[piece] = *reinterpret_cast<const uint32_t *>(a.x + (size_t)off);
+                f.fill[piece] = fill;
+                f.take |= ok ? (1u << piece) : 0u;
+            }
+        }
     }
-    return v4i{(int)(w[0] ^ 0x80808080u), (int)(w[1] ^ 0x80808080u), (int)(w[2] ^ 0x80808080u),
-               (int)(w[3] ^ 0x80808080u)};
+    return f;
 }
 
 template <int T, int RG, int MODE>
@@ -194,12 +235,13 @@ __global__ __launch_bounds__(kThreads, 2) void qconv_igemm_kernel(const IgemmArg
     constexpr int pix_per_block = kWaves * RG * 16;
 
     PixInfo pcur[RG], pnxt[RG];
-    v4i fcur[RG], fnxt[RG];
+    ActFrag fcur[RG], fnxt[RG];
 #pragma unroll
     for (int rg = 0; rg < RG; rg++) {
         pnxt[rg].base = -1;
         pnxt[rg].iy0 = pnxt[rg].ix0 = 0;
-        fnxt[rg] = v4i{0, 0, 0, 0};
+        fnxt[rg].raw = fnxt[rg].fill = u32x4{0, 0, 0, 0};
+        fnxt[rg].take = 0;
     }
     int mt = blockIdx.x;
     if (mt < a.num_mtiles) {
@@ -239,16 +281,19 @@ __global__ __launch_bounds__(kThreads, 2) void qconv_igemm_kernel(const IgemmArg
                         fnxt[rg] = load_act<MODE>(a, pnxt[rg], gq);
                     }
                 }
+                v4i xf[RG]; // the slice loaded one step ago, now needed
+#pragma unroll
+                for (int rg = 0; rg < RG; rg++) xf[rg] = finish_act(fcur[rg]);
 #pragma unroll
                 for (int rg = 0; rg < RG; rg++)
-                    rs[rg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, fcur[rg], rs[rg], 0, 0, 0);
+                    rs[rg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, xf[rg], rs[rg], 0, 0, 0);
                 const uint8_t *wstep = wlds + (size_t)(ks - s0) * T * 1024 + lane * 16;
 #pragma unroll
                 for (int nt = 0; nt < T; nt++) {
                     const v4i wf = *reinterpret_cast<const v4i *>(wstep + nt * 1024);
 #pragma unroll
                     for (int rg = 0; rg < RG; rg++)
-                        acc[rg][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf, fcur[rg], acc[rg][nt], 0, 0, 0);
+                        acc[rg][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf, xf[rg], acc[rg][nt], 0, 0, 0);
                 }
 #pragma unroll
                 for (int rg = 0; rg < RG; rg++) fcur[rg] = fnxt[rg];
@@ -272,7 +317,7 @@ __global__ __launch_bounds__(kThreads, 2) void qconv_igemm_kernel(const IgemmArg
                         uint32_t b[4];
 #pragma unroll
                         for (int r = 0; r < 4; r++) {
-                            const int32_t v = acc[rg][nt][r] + ct[r] + nrsz;
+                            const int32_t v = add3(acc[rg][nt][r], ct[r], nrsz);
                             b[r] = requant_u8_lowbyte((float)v * a.ep.mult, a.ep);
                         }
                         packed[nt] = pack_low_bytes(b[0], b[1], b[2], b[3]);
@@ -305,7 +350,7 @@ __global__ __launch_bounds__(kThreads, 2) void qconv_igemm_kernel(const IgemmArg
                         uint32_t o[4];
 #pragma unroll
                         for (int r = 0; r < 4; r++) {
-                            const int32_t v = acc[rg][nt][r] + ct[r] + nrsz;
+                            const int32_t v = add3(acc[rg][nt][r], ct[r], nrsz);
                             if (a.ep.out_mode == kOutI32) o[r] = (uint32_t)v;
                             else o[r] = __float_as_uint(clamp_ref((float)v * a.ep.mult, a.ep.lo, a.ep.hi));
                         }
@@ -329,7 +374,8 @@ __global__ __launch_bounds__(kThreads, 2) void qconv_igemm_kernel(const IgemmArg
 // every compute unit a couple of blocks.  RG = 4 is only built for T <= 8 (register budget).
 inline int choose_rg(const nncase_hip_ctx *ctx, int tiles, int nchunks, int m) {
     const long long target = 2LL * ctx->compute_units;
-    for (int rg = tiles <= 8 ? 4 : 2; rg > 1; rg /= 2)
+    static const int max_rg = getenv("NNHIP_MAX_RG") ? atoi(getenv("NNHIP_MAX_RG")) : 4;
+    for (int rg = std::min(max_rg, tiles <= 8 ? 4 : 2); rg > 1; rg /= 2)
         if ((long long)ceil_div(m, kWaves * rg * 16) * nchunks >= target) return rg;
     return 1;
 }
