@@ -155,6 +155,14 @@ typedef struct nncase_hip_conv2d_args {
     nncase_hip_quant_param_t y_qp;       /* output quantisation (U8 output only)           */
     float clamp_min, clamp_max;          /* fused_clamp of Conv2D, applied in the fp32 domain */
     int32_t out_dtype;                   /* NNCASE_HIP_DT_U8 / _I32 / _F32                 */
+    /* Optional fused residual add (U8 output, dense kernels only).  With residual_dev set
+     * the call computes what nncase_hip_qconv2d followed by nncase_hip_qadd would:
+     *   y = Q_sum(clamp(DQ_y(conv result requantised with y_qp) + DQ_res(residual)))
+     * without writing the convolution's own u8 tensor.  residual_dev has the output's shape. */
+    const uint8_t *residual_dev;
+    nncase_hip_quant_param_t residual_qp;
+    nncase_hip_quant_param_t sum_qp;
+    float sum_clamp_min, sum_clamp_max;
 } nncase_hip_conv2d_args_t;
 
 /* Output is [batch, out_h, out_w, out_channels] with

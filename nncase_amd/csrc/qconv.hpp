@@ -49,8 +49,18 @@ struct Epilogue {
     int out_mode;
 };
 
+// Second requantisation stage of a fused residual add:
+//   s = ((float)q - zy) * sy + ((float)r - zr) * sr;   out = sat_u8(rne(clamp(s) / sum.sy + sum.zy))
+struct ResidualEpilogue {
+    const uint8_t *res; // nullptr: no residual
+    float zy, sy;       // dequantisation of the convolution's own u8 result
+    float zr, sr;       // dequantisation of the residual
+    Epilogue sum;       // requantisation of the sum (mult unused)
+};
+
 // Fills an Epilogue; returns 0 or a negative error for scales outside the range in
 // which the division-free requantisation is exact.
+int make_residual_epilogue(nncase_hip_ctx *ctx, ResidualEpilogue *rep, const nncase_hip_conv2d_args_t *c);
 int make_epilogue(nncase_hip_ctx *ctx, Epilogue *ep, float sx, float sw, nncase_hip_quant_param_t y_qp, float clamp_min,
                   float clamp_max, int out_dtype, const char *who);
 
@@ -99,6 +109,13 @@ __device__ __forceinline__ uint32_t pack_low_bytes(uint32_t b0, uint32_t b1, uin
     const uint32_t lo = __builtin_amdgcn_perm(b1, b0, 0x0c0c0400u); // [b0.0, b1.0, 0, 0]
     const uint32_t hi = __builtin_amdgcn_perm(b3, b2, 0x04000c0cu); // [0, 0, b2.0, b3.0]
     return lo | hi;
+}
+
+// Byte e of `res` added to the u8 code in the low byte of `q`; result in the low byte.
+__device__ __forceinline__ uint32_t residual_lowbyte(uint32_t q, uint32_t res, int e, const ResidualEpilogue &r) {
+    const float fa = ((float)(q & 0xffu) - r.zy) * r.sy;
+    const float fb = ((float)((res >> (8 * e)) & 0xffu) - r.zr) * r.sr;
+    return requant_u8_lowbyte(fa + fb, r.sum);
 }
 
 // a + b + c in one instruction (the compiler otherwise re-associates the zero-point

@@ -70,6 +70,7 @@ struct IgemmArgs {
     uint32_t zx_splat;     // zx in all four bytes
     int num_mtiles;
     Epilogue ep;
+    ResidualEpilogue rep;
 };
 
 struct PixInfo {
@@ -321,6 +322,25 @@ __global__ __launch_bounds__(kThreads, 2) void qconv_igemm_kernel(const IgemmArg
                             b[r] = requant_u8_lowbyte((float)v * a.ep.mult, a.ep);
                         }
                         packed[nt] = pack_low_bytes(b[0], b[1], b[2], b[3]);
+                    }
+                    if (a.rep.res) { // fused residual add on the requantised bytes
+                        const uint8_t *ro = a.rep.res + obase;
+                        const bool whole = ((a.ldy | a.y_coff) & 3) == 0 && ch0 + 4 * T <= a.n;
+#pragma unroll
+                        for (int nt = 0; nt < T; nt++) {
+                            uint32_t rv = 0;
+                            if (whole) {
+                                rv = *reinterpret_cast<const uint32_t *>(ro + nt * 4);
+                            } else {
+#pragma unroll
+                                for (int r = 0; r < 4; r++)
+                                    if (ch0 + nt * 4 + r < a.n) rv |= (uint32_t)ro[nt * 4 + r] << (8 * r);
+                            }
+                            uint32_t b[4];
+#pragma unroll
+                            for (int r = 0; r < 4; r++) b[r] = residual_lowbyte(packed[nt] >> (8 * r), rv, r, a.rep);
+                            packed[nt] = pack_low_bytes(b[0], b[1], b[2], b[3]);
+                        }
                     }
                     if (((a.ldy | a.y_coff) & 3) == 0 && ch0 + 4 * T <= a.n) {
 #pragma unroll

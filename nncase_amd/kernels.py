@@ -68,7 +68,8 @@ def _out_dt(out_dtype) -> int:
 def conv2d(input: np.ndarray, weights: np.ndarray, bias: Optional[np.ndarray], stride: Sequence[int],
            padding: Sequence[Sequence[int]], dilation: Sequence[int], groups: int, fused_clamp: Tuple[float, float],
            input_qp: QuantParam, weights_qp: QuantParam, output_qp: Optional[QuantParam] = None, out_dtype=np.uint8,
-           ctx: Context = None) -> np.ndarray:
+           ctx: Context = None, residual: Optional[np.ndarray] = None, residual_qp: Optional[QuantParam] = None,
+           sum_qp: Optional[QuantParam] = None, sum_clamp: Tuple[float, float] = (-rt.FLT_MAX, rt.FLT_MAX)) -> np.ndarray:
     """kernels::stackvm::conv2d(pad_mode=constant, input, weights, bias, stride, padding, dilation,
     groups, fused_clamp) on u8 NCHW input / u8 OIHW weights / int32 bias.
 
@@ -95,6 +96,14 @@ def conv2d(input: np.ndarray, weights: np.ndarray, bias: Optional[np.ndarray], s
     y_nchw = c.alloc(max(1, n * oh * ow * oc * es))
     args = rt.Conv2dArgs(n, h, wd, stride[0], stride[1], dilation[0], dilation[1], ph0, ph1, pw0, pw1, input_qp,
                          output_qp or qp(0, 1.0), fused_clamp[0], fused_clamp[1], _out_dt(out_dtype))
+    if residual is not None:  # fused Quantize(Dequantize(conv) + Dequantize(residual)), residual given as NCHW u8
+        r = np.ascontiguousarray(residual, np.uint8)
+        if r.shape != (n, oc, oh, ow):
+            raise rt.HipError(-rt.ERR_SHAPE_MISMATCH, "conv2d", f"residual shape {r.shape} != output shape {(n, oc, oh, ow)}")
+        r_nchw, r_nhwc = c.to_device(r), c.alloc(r.size)
+        c.nchw_to_nhwc(r_nchw, r_nhwc, 1, n, oc, oh, ow)
+        args.residual_dev, args.residual_qp, args.sum_qp = r_nhwc.ptr, residual_qp, sum_qp
+        args.sum_clamp_min, args.sum_clamp_max = sum_clamp
     c.qconv2d(x_nhwc, wts, y_nhwc, args)
     c.nhwc_to_nchw(y_nhwc, y_nchw, es, n, oc, oh, ow)
     out = y_nchw.download((n, oc, oh, ow), out_dtype)

@@ -228,18 +228,38 @@ class HipModel:
     """A QuantGraph resident on the device: packed weights, one HBM buffer per tensor, and the
     operator list recorded in a `hip` function.  run() = upload input, invoke, download output."""
 
-    def __init__(self, ctx: Context, qg: QuantGraph, batch: int, capture_graph: bool = True):
+    def __init__(self, ctx: Context, qg: QuantGraph, batch: int, capture_graph: bool = True, fuse_residual: bool = True):
         self.ctx, self.qg, self.batch = ctx, qg, batch
         h, w, c = qg.input_shape
         self.in_count = batch * h * w * c
         self.input_f32 = ctx.alloc(self.in_count * 4)
         self.fn = Function(ctx)
-        self.buffers: List[rt.DeviceBuffer] = []
+        self.buffers: List[Optional[rt.DeviceBuffer]] = []
         self.weights: List[Optional[rt.Weights]] = []
         self.op_names: List[str] = []
         self.op_nodes: List[int] = []
+        # A residual add whose second operand is a dense conv consumed by nothing else is folded into
+        # that conv's epilogue (the conv's own u8 tensor is then never written).
+        consumers = [0] * len(qg.nodes)
+        for n in qg.nodes:
+            for j in n.inputs:
+                consumers[j] += 1
+        self.fused_into: Dict[int, int] = {}   # conv node -> add node
+        if fuse_residual:
+            for i, n in enumerate(qg.nodes):
+                if n.op == "add":
+                    a, b = n.inputs
+                    nb_ = qg.nodes[b]
+                    dense = nb_.op == "conv" and not (nb_.groups > 1 and nb_.weights.shape[1] == 1) and nb_.weights.shape[1] * nb_.groups > 4
+                    if dense and consumers[b] == 1 and b == i - 1 and a < b:
+                        self.fused_into[b] = i
         for i, n in enumerate(qg.nodes):
             cc, hh, ww = n.out_shape
+            fused_add = self.fused_into.get(i)
+            if n.op == "add" and i in self.fused_into.values():
+                self.buffers.append(self.buffers[i - 1])  # written by the fused conv
+                self.weights.append(None)
+                continue
             buf = ctx.alloc(batch * cc * hh * ww)
             self.buffers.append(buf)
             self.weights.append(None)
@@ -252,6 +272,14 @@ class HipModel:
                 (ph0, ph1), (pw0, pw1) = n.padding
                 args = rt.Conv2dArgs(batch, src.out_shape[1], src.out_shape[2], n.stride[0], n.stride[1], 1, 1, ph0, ph1, pw0,
                                      pw1, qp(*src.out_qp), qp(*n.out_qp), n.clamp[0], n.clamp[1], rt.DT_U8)
+                if fused_add is not None:
+                    add = qg.nodes[fused_add]
+                    res_node = add.inputs[0]
+                    args.residual_dev = self.buffers[res_node].ptr
+                    args.residual_qp = qp(*qg.nodes[res_node].out_qp)
+                    args.sum_qp = qp(*add.out_qp)
+                    args.sum_clamp_min, args.sum_clamp_max = FULL_CLAMP
+                    self.fn._keep.append(self.buffers[res_node])
                 self.fn.add_qconv2d(self.buffers[n.inputs[0]], wt, buf, args)
             elif n.op == "add":
                 a, b = (qg.nodes[j] for j in n.inputs)
@@ -263,8 +291,8 @@ class HipModel:
                                             src.out_shape[0], qp(*src.out_qp), qp(*n.out_qp))
             else:
                 raise ValueError(n.op)
-            self.op_names.append(f"{n.op}:{n.name}")
-            self.op_nodes.append(i)
+            self.op_names.append(f"{n.op}:{n.name}" + ("+add" if fused_add is not None else ""))
+            self.op_nodes.append(i if fused_add is None else fused_add)
         last = qg.nodes[-1]
         self.out_shape = (batch,) + tuple(last.out_shape)
         self.out_count = int(np.prod(self.out_shape))
@@ -289,8 +317,14 @@ class HipModel:
         y = self.output_f32.download((self.batch, h, w, c), f32)
         return np.ascontiguousarray(y.transpose(0, 3, 1, 2))
 
+    def materialized(self, node: int) -> bool:
+        """False for a conv whose output only exists inside a fused residual add."""
+        return node not in self.fused_into
+
     def tensor(self, node: int) -> np.ndarray:
         """u8 output of a node as NCHW (for layer-by-layer parity checks)."""
+        if not self.materialized(node):
+            raise ValueError(f"node {node} is fused into node {self.fused_into[node]} and never written")
         c, h, w = self.qg.nodes[node].out_shape
         y = self.buffers[node].download((self.batch, h, w, c), np.uint8)
         return np.ascontiguousarray(y.transpose(0, 3, 1, 2))

@@ -46,7 +46,9 @@ class Conv2dArgs(C.Structure):
                 ("pad_h_before", C.c_int32), ("pad_h_after", C.c_int32),
                 ("pad_w_before", C.c_int32), ("pad_w_after", C.c_int32),
                 ("x_qp", QuantParam), ("y_qp", QuantParam),
-                ("clamp_min", C.c_float), ("clamp_max", C.c_float), ("out_dtype", C.c_int32)]
+                ("clamp_min", C.c_float), ("clamp_max", C.c_float), ("out_dtype", C.c_int32),
+                ("residual_dev", C.c_void_p), ("residual_qp", QuantParam), ("sum_qp", QuantParam),
+                ("sum_clamp_min", C.c_float), ("sum_clamp_max", C.c_float)]
 
 
 class MatmulArgs(C.Structure):

@@ -282,3 +282,24 @@ def test_requantisation_is_exact_for_many_scales(hip_ctx):
     with pytest.raises(rt.HipError) as e:
         K.conv2d(x, w, bias, (1, 1), ((0, 0), (0, 0)), (1, 1), 1, FULL, qp(3, 1.0), qp(128, 1.0), qp(7, 2.0 ** -70), np.uint8, ctx=hip_ctx)
     assert e.value.code == -34  # ERANGE
+
+
+@pytest.mark.parametrize("cin,cout,hw,k", [(144, 24, 13, 1), (960, 160, 7, 1), (32, 40, 9, 3), (24, 30, 5, 1)])
+def test_fused_residual_equals_conv_then_add(hip_ctx, cin, cout, hw, k):
+    """conv with a fused residual == the same conv followed by the separate add, bit for bit (oracle: conv then qadd)."""
+    rng = np.random.default_rng(cin + cout)
+    x = rng.integers(0, 256, (2, cin, hw, hw), dtype=np.uint8)
+    w = rng.integers(0, 256, (cout, cin, k, k), dtype=np.uint8)
+    bias = rng.integers(-3000, 3000, cout).astype(np.int32)
+    res = rng.integers(0, 256, (2, cout, hw, hw), dtype=np.uint8)
+    pad = ((k // 2, k // 2), (k // 2, k // 2))
+    sx, sw = f32(0.0235), f32(0.0041)
+    real = O.qconv2d(x, w, bias, 7, sx, 131, sw, padding=pad, out_mode=O.OUT_F32)
+    sy = f32((real.max() - real.min()) / 255)
+    zy = int(np.clip(np.rint(-real.min() / sy), 0, 255))
+    conv = O.qconv2d(x, w, bias, 7, sx, 131, sw, zy, sy, padding=pad)
+    want = O.qadd(conv, res, zy, sy, 99, 0.031, 101, float(sy) * 1.3)
+    got = K.conv2d(x, w, bias, (1, 1), pad, (1, 1), 1, FULL, qp(7, sx), qp(131, sw), qp(zy, sy), np.uint8, ctx=hip_ctx,
+                   residual=res, residual_qp=qp(99, 0.031), sum_qp=qp(101, float(sy) * 1.3))
+    assert np.array_equal(got, want)
+    assert len(np.unique(want)) > 16

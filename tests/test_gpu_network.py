@@ -13,11 +13,13 @@ pytestmark = pytest.mark.gpu
 f32 = np.float32
 
 
-def check_model(hip_ctx, qg, x, capture):
-    model = nb.HipModel(hip_ctx, qg, x.shape[0], capture_graph=capture)
+def check_model(hip_ctx, qg, x, capture, fuse_residual=True):
+    model = nb.HipModel(hip_ctx, qg, x.shape[0], capture_graph=capture, fuse_residual=fuse_residual)
     y = model.run(x)
     want, outs = netref.run_integer(qg, x, keep_all=True)
     for i, ref in enumerate(outs):
+        if not model.materialized(i):
+            continue
         got = model.tensor(i)
         assert np.array_equal(got, ref), f"node {i} ({qg.nodes[i].name}): {(got != ref).sum()} of {ref.size} bytes differ"
     assert np.array_equal(y.view(np.uint32), want.view(np.uint32))
@@ -50,7 +52,10 @@ def test_mobilenetv2_config3(hip_ctx):
     qg = nb.quantize_graph(g, calib)
     assert qg.macs_per_image == {"dense": 280057856, "depthwise": 20716416}
     x = rng.random((2, 224, 224, 3), dtype=f32)
+    plain, _, _ = check_model(hip_ctx, qg, x, capture=False, fuse_residual=False)   # every tensor, add as its own kernel
+    assert len(plain.fused_into) == 0 and len(plain.fn) == 66
     model, y, outs = check_model(hip_ctx, qg, x, capture=True)
+    assert len(model.fused_into) == 10 and len(model.fn) == 56                        # residual adds folded into the convs
     # the reference's own acceptance bar for a PTQ model: cosine >= 0.98 against the float model
     fl = nb.float_forward(g, x)[-1]
     assert O.cosine(y, fl) > 0.98
