@@ -65,8 +65,92 @@ def conv_macs(qg, batch):
     return out
 
 
+def time_calls(ctx, fn, warmup, steps):
+    """Mean device milliseconds of fn() over `steps` back-to-back calls (wall clock, synchronised both sides)."""
+    for _ in range(warmup):
+        fn()
+    ctx.sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    ctx.sync()
+    return (time.perf_counter() - t0) / steps * 1e3
+
+
+def side_workload(args):
+    """The other BASELINE configurations' kernels at their real shapes (one JSON line each):
+    --workload matmul            config 1: A[512,1024] u8 x B[1024,1024] u8 -> f32
+    --workload conv_block        config 2: 1x1 64->144, dw 3x3, 1x1 144->64 on 56x56, batch 32
+    --workload paged_attention   config 5: batch 32, 14 q / 2 kv heads, d 64, block 16, ctx U[512,4096], fp16
+    """
+    from nncase_amd import netbuilder as nb
+    from nncase_amd import quant
+    from nncase_amd import runtime as rt
+    from nncase_amd.runtime import Context, qp
+
+    ctx = Context(0)
+    base = {"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "data": "synthetic"}
+    if args.workload == "matmul":
+        rng = np.random.default_rng(0)
+        a = rng.integers(0, 256, (512, 1024), dtype=np.uint8)
+        bq, zb, sb = quant.quantize_weights((rng.standard_normal((1024, 1024)) * 0.05).astype(np.float32))
+        w = ctx.prepack_matmul(bq, None, qp(zb, sb), expected_rows=512)
+        da, dy = ctx.to_device(a), ctx.alloc(512 * 1024 * 4)
+        margs = rt.MatmulArgs(512, qp(128, 0.02), qp(0, 1.0), -rt.FLT_MAX, rt.FLT_MAX, rt.DT_F32)
+        ms = time_calls(ctx, lambda: ctx.qmatmul(da, w, dy, margs), args.warmup, args.steps)
+        ops, nbytes = 2 * 512 * 1024 * 1024, 524288 + 1048576 + 2097152
+        line = dict(base, metric="int8 TOPS u8/u8 MatMul 512x1024x1024 -> f32", value=round(ops / (ms * 1e-3) / 1e12, 2), unit="TOPS",
+                    ms_per_step=round(ms, 5), dtype="u8", config={"workload": "config 1: A[512,1024] u8 x B[1024,1024] u8, f32 out"},
+                    roofline={"bound": "mfma", "achieved": round(ops / (ms * 1e-3) / 1e12, 2), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+                              "frac": round(ops / (ms * 1e-3) / 1e12 / INT8_PEAK_TOPS, 5), "traffic": None,
+                              "hbm_GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                              "note": "1.07 G int8-op and 3.67 MB: both roofline floors are < 0.5 us, the launch is latency-bound"})
+    elif args.workload == "conv_block":
+        batch = 32
+        rng = np.random.default_rng(1)
+        qg = nb.quantize_graph(nb.conv_block(seed=1), rng.random((32, 56, 56, 64), dtype=np.float32))
+        model = nb.HipModel(ctx, qg, batch, capture_graph=True)
+        model.set_input(rng.random((batch, 56, 56, 64), dtype=np.float32))
+        ms = time_calls(ctx, model.invoke, args.warmup, args.steps)
+        op_ms = model.fn.profile(10)
+        nbytes = sum(algorithmic_bytes(qg, batch))
+        line = dict(base, metric="images/sec u8/u8 conv block b32", value=round(batch / (ms * 1e-3), 1), unit="images/s",
+                    ms_per_step=round(ms, 5), dtype="u8",
+                    config={"workload": "config 2: f32 in -> quantize -> 1x1 64->144, dw 3x3, 1x1 144->64 (ReLU6) on 56x56 -> dequantize, batch 32"},
+                    roofline={"bound": "hbm", "achieved": round(nbytes / (sum(op_ms) * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                              "frac": round(nbytes / (sum(op_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None},
+                    kernels={model.fn.op_kernel(i): round(t * 1e3, 2) for i, t in enumerate(op_ms)})
+    elif args.workload == "paged_attention":
+        rng = np.random.default_rng(5)
+        bsz, hq, hkv, d, blk = 32, 14, 2, 64, 16
+        lens = rng.integers(512, 4097, bsz).astype(np.int32)
+        max_blocks = 4096 // blk
+        nblocks = bsz * max_blocks
+        q = rng.standard_normal((bsz, hq, d)).astype(np.float16)
+        kc = rng.standard_normal((nblocks, hkv, blk, d)).astype(np.float16)
+        vc = rng.standard_normal((nblocks, hkv, blk, d)).astype(np.float16)
+        bt = rng.permutation(nblocks).reshape(bsz, max_blocks).astype(np.int32)
+        dq, dk, dv, dbt, dcl = (ctx.to_device(t) for t in (q, kc, vc, bt, lens))
+        dout = ctx.alloc(bsz * hq * d * 2)
+        pargs = rt.PagedAttnArgs(bsz, hq, hkv, d, blk, max_blocks, nblocks, 0.125, rt.DT_F16)
+        ms = time_calls(ctx, lambda: ctx.paged_attention_decode(dq, dk, dv, dbt, dcl, dout, pargs), args.warmup, args.steps)
+        kv_bytes = int(lens.sum()) * hkv * d * 2 * 2
+        line = dict(base, metric="sequence-layers/sec paged-attention decode b32", value=round(bsz / (ms * 1e-3), 1), unit="sequence-layers/s",
+                    ms_per_step=round(ms, 5), dtype="f16",
+                    config={"workload": "config 5 attention layer: batch 32, 14 q / 2 kv heads, head_dim 64, block 16, ctx U[512,4096], "
+                                        f"{int(lens.sum())} cached tokens, fp16 KV"},
+                    roofline={"bound": "hbm", "achieved": round(kv_bytes / (ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                              "frac": round(kv_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
+                              "algorithmic_bytes_per_launch": kv_bytes})
+    else:
+        sys.exit(f"unknown workload {args.workload}")
+    print(json.dumps(line))
+
+
 def main():
     ap = argparse.ArgumentParser()
+    ap.add_argument("--workload", default="mobilenetv2", help="mobilenetv2 (headline, default) | matmul | conv_block | paged_attention")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
@@ -77,15 +161,29 @@ def main():
     ap.add_argument("--no-graph", action="store_true",
                     help="enqueue the operators one by one instead of replaying the HIP graph (used under rocprofv3 "
                          "--kernel-trace, whose tracer crashes inside hipGraphLaunch on this image)")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="first launch a plain 256 MiB -> 256 MiB copy kernel three times, so that a rocprofv3 --pmc run of "
+                         "this command can scale FETCH_SIZE / WRITE_SIZE by what they read for a copy of known size")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (the workload is one GPU's share at its real shape); "
                  "--gpus N with N > 1 is not supported")
+    if args.workload != "mobilenetv2":
+        return side_workload(args)
 
     from nncase_amd import netbuilder as nb
     from nncase_amd.runtime import Context
 
     ctx = Context(0)  # raises if libnncase_hip.so is missing or there is no gfx950 device
+    if args.copy_probe:
+        n = 64 << 20  # dwords
+        src, dst = ctx.alloc(n * 4), ctx.alloc(n * 4)
+        src.fill(1)
+        dst.fill(0)
+        for _ in range(3):
+            ctx.pack(src, dst, 4, [n], [], [])  # no packed axes: pack_kernel<unsigned int> is an element-wise copy
+        ctx.sync()
+        del src, dst
     graph = nb.mobilenet_v2(seed=2)
     calib = np.random.default_rng(3).random((32, 224, 224, 3), dtype=np.float32)
     qg = nb.quantize_graph(graph, calib)

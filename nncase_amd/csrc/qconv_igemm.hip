@@ -3,7 +3,6 @@
 #include "qconv_igemm.hpp"
 
 #include <algorithm>
-#include <cstdlib>
 #include <vector>
 
 namespace nnhip {
@@ -82,8 +81,7 @@ int prepack_igemm(nncase_hip_ctx *ctx, nncase_hip_weights *w, const uint8_t *w_o
                   (long long)taps * w->g_ic);
     w->k = taps * w->g_ic;
     w->ksteps = ceil_div(w->k, 64);
-    int max_tiles = (w->g_ic % 4 == 0) ? 16 : 4;
-    if (getenv("NNHIP_MAX_T")) max_tiles = std::min(max_tiles, atoi(getenv("NNHIP_MAX_T")));
+    const int max_tiles = (w->g_ic % 4 == 0) ? 16 : 4;
     plan_igemm(w->g_oc, w->ksteps, max_tiles, w->pixels_hint, ctx->compute_units, &w->tiles, &w->nchunks, &w->kc_steps);
     const size_t group_bytes = (size_t)w->nchunks * w->ksteps * w->tiles * 1024;
     w->packed_bytes = group_bytes * w->groups;

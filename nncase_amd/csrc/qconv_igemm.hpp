@@ -34,9 +34,6 @@
 
 #include "qconv.hpp"
 
-#include <algorithm>
-#include <cstdlib>
-
 namespace nnhip {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
@@ -390,12 +387,15 @@ __global__ __launch_bounds__(kThreads, 2) void qconv_igemm_kernel(const IgemmArg
     }
 }
 
-// Pixel groups per wave (RG) for a chunk width of T tiles: the widest that still gives
-// every compute unit a couple of blocks.  RG = 4 is only built for T <= 8 (register budget).
+// Pixel groups per wave (RG) for a chunk width of T tiles.  The kernels are bound by the
+// VALU work of the epilogue, and a dependent VALU instruction issues only every ~8 cycles
+// from one wave, so what matters is having >= 4 waves per SIMD: RG is capped so that the
+// kernel stays within 128 VGPRs, and lowered further while the grid would not give every
+// compute unit a couple of blocks.
 inline int choose_rg(const nncase_hip_ctx *ctx, int tiles, int nchunks, int m) {
     const long long target = 2LL * ctx->compute_units;
-    static const int max_rg = getenv("NNHIP_MAX_RG") ? atoi(getenv("NNHIP_MAX_RG")) : 4;
-    for (int rg = std::min(max_rg, tiles <= 8 ? 4 : 2); rg > 1; rg /= 2)
+    const int cap = tiles == 1 ? 4 : (tiles <= 6 ? 2 : 1);
+    for (int rg = cap; rg > 1; rg /= 2)
         if ((long long)ceil_div(m, kWaves * rg * 16) * nchunks >= target) return rg;
     return 1;
 }
