@@ -129,7 +129,7 @@ def side_workload(args):
         nblocks = bsz * max_blocks
         q = rng.standard_normal((bsz, hq, d)).astype(np.float16)
         kc = rng.standard_normal((nblocks, hkv, blk, d)).astype(np.float16)
-        vc = rng.standard_normal((nblocks, hkv, blk, d)).astype(np.float16)
+        vc = rng.standard_normal((nblocks, hkv, d, blk)).astype(np.float16)  # V is cached d-major
         bt = rng.permutation(nblocks).reshape(bsz, max_blocks).astype(np.int32)
         dq, dk, dv, dbt, dcl = (ctx.to_device(t) for t in (q, kc, vc, bt, lens))
         dout = ctx.alloc(bsz * hq * d * 2)

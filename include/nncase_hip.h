@@ -233,11 +233,16 @@ NNCASE_HIP_API int nncase_hip_nhwc_to_nchw(nncase_hip_ctx_t *ctx, const void *in
  *   out[b, h, :] = softmax(scale * q[b, h, :] . K[b, kvh, 0..ctx_b)) . V[b, kvh, ...]
  * with kvh = h / (num_q_heads / num_kv_heads), fp32 scores and accumulation.
  *   q            [batch, num_q_heads, head_dim]                 f16
- *   k/v cache    [num_blocks, num_kv_heads, block_size, head_dim] f16
+ *   k cache      [num_blocks, num_kv_heads, block_size, head_dim] f16
+ *   v cache      [num_blocks, num_kv_heads, head_dim, block_size] f16 (d-major:
+ *                a lane's matrix-core operand, 4 consecutive tokens of one d,
+ *                is then one 8-byte load)
  *   block_table  [batch, max_blocks_per_seq] int32 (physical block ids)
  *   ctx_lens     [batch] int32
  *   out          [batch, num_q_heads, head_dim]                 f16 or f32
- * (No counterpart in this reference tree.)
+ * head_dim 64 or 128; block_size a multiple of 16; at most 16 query heads per
+ * kv head; scale may have either sign.  Slots of a block past the context
+ * length may hold anything.  (No counterpart in this reference tree.)
  */
 typedef struct nncase_hip_paged_attn_args {
     int32_t batch, num_q_heads, num_kv_heads, head_dim;

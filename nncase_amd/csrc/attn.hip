@@ -1,185 +1,231 @@
 // Paged-attention decode: one query token per sequence against a block-paged
 // fp16 KV cache.  HBM-bound (every cached K and V element is read once per
-// step, ~7 flop per byte), so the kernel is organised around the KV stream:
+// step, ~7 flop per byte), so the kernel is organised around the KV stream and
+// keeps the arithmetic on the matrix cores:
 //
-//   grid = (splits, kv heads, sequences).  A block owns one kv head of one
-//   sequence and a contiguous range of `kSplitTokens` cached tokens, and
-//   serves ALL query heads that share the kv head, so K and V cross the memory
-//   system once however many query heads there are (GQA).
-//   A wave reads a run of tokens as one contiguous, fully coalesced segment
-//   (each lane 32 bytes = 16 fp16 of one token), i.e. physical KV blocks are
-//   consumed whole in the order the block table lists them.
-//   Pass 1 writes scaled logits to LDS, the block takes the max and the
-//   exponentials there, pass 2 accumulates P.V in fp32 registers; partial
-//   (max, sum, unnormalised output) triples go to a workspace and a second
-//   kernel merges the splits.
+//   grid = (sequences x kv heads, splits).  A block owns one kv head of one
+//   sequence and a contiguous range of cached tokens, and serves ALL query
+//   heads that share the kv head, so K and V cross the memory system once
+//   however many query heads there are (GQA).  Each of its four waves owns a
+//   contiguous run of 16-token tiles and issues the loads of ALL its K and V
+//   tiles before any arithmetic (8 KiB of K + 8 KiB of V in flight per wave).
+//
+//   Logits: S^T[token, head] = K[token, :] . Q^T[:, head] with K rows as the
+//   MFMA A operand (one 16-byte load per lane straight from the cache) and the
+//   query heads, padded to 16, as B.  The accumulator layout of S^T (lane =
+//   head, 4 consecutive tokens per lane) IS the A-operand layout of the 16x16x16
+//   product P.V, so probabilities never move between lanes.  V is cached
+//   d-major ([block][kv head][d][token]) so that a lane's B operand (4
+//   consecutive tokens of one d) is one 8-byte load.  P is split into two fp16
+//   terms (p = hi + lo), which keeps the P.V product at fp32-level accuracy.
+//
+//   Every wave keeps its own (max, sum, unnormalised output); the block merges
+//   its four waves through LDS and writes one partial per split.  The block
+//   that finishes last for a (sequence, kv head) - found with one atomic
+//   counter per pair, which it resets for the next call - merges the splits
+//   and writes the output, so there is a single launch per call.
 #include "common.hpp"
 
 #include <hip/hip_fp16.h>
 
 namespace nnhip {
 
-typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t au32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t au32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kAttnThreads = 256;
 constexpr int kAttnWaves = 4;
-constexpr int kSplitTokens = 512;
-constexpr int kMaxGroup = 8; // query heads per kv head
+constexpr int kAttnHeads = 16; // query heads per kv head, padded to the MFMA tile
+constexpr float kLog2e = 1.4426950408889634f;
+
+constexpr int kAttnMaxSplits = 128; // (max, sum) of 16 heads x 128 splits fit the 16 KiB LDS buffer at merge time
 
 struct AttnArgs {
     const uint16_t *q, *k_cache, *v_cache;
     const int32_t *block_table, *ctx_lens;
-    float *part_o; // [batch][q heads][splits][D]
-    float *part_ml; // [batch][q heads][splits][2]
+    float *part_o;  // [batch][q heads][splits][D], unnormalised, relative to the split's max
+    float *part_ml; // [batch][q heads][splits][2]: max of (logit * scale * log2 e), sum of 2^(. - max)
+    uint32_t *done; // [batch][kv heads] blocks finished; zero between calls
     void *out;
-    int batch, hq, hkv, group, d, block_size, max_blocks, num_blocks, splits;
-    float scale;
+    int batch, hq, hkv, group, d, block_size, max_blocks, num_blocks, splits, split_tokens;
+    FastDiv d_block;
+    float scale_log2e;
     int out_f16;
 };
 
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
-    return v;
+__device__ __forceinline__ void coherent_store(float *p, float v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
-    return v;
+__device__ __forceinline__ float coherent_load(const float *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// D = head_dim (64 or 128).  LPT lanes share one token (16 fp16 each).
-template <int D> __global__ __launch_bounds__(kAttnThreads) void paged_attn_split_kernel(const AttnArgs a) {
-    constexpr int LPT = D / 16;   // lanes per token
-    constexpr int TPW = 64 / LPT; // tokens per wave step
-    __shared__ float sc[kMaxGroup][kSplitTokens]; // logits, then probabilities
-    __shared__ float red[kAttnWaves][kMaxGroup][D];
-    __shared__ float hmax[kMaxGroup], hsum[kMaxGroup];
+// NT = 16-token tiles per wave (even).
+template <int D, int NT> __global__ __launch_bounds__(kAttnThreads, 2) void paged_attn_kernel(const AttnArgs a) {
+    constexpr int KS = D / 32; // 32-deep steps of the logit product
+    constexpr int DT = D / 16; // 16-wide column tiles of the output
+    constexpr int WAVE_TOKENS = NT * 16;
+    constexpr int SPLIT = kAttnWaves * WAVE_TOKENS;
+    __shared__ float red[kAttnWaves][kAttnHeads][D];
+    __shared__ float smax[kAttnWaves][kAttnHeads], ssum[kAttnWaves][kAttnHeads];
+    __shared__ uint32_t s_last;
 
-    const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+    // kv head fastest, then sequence, then split: consecutive workgroups go to different XCDs, so
+    // every XCD gets the same mix of early (always present) and late (long contexts only) splits
+    const int kvh = blockIdx.x % a.hkv, b = blockIdx.x / a.hkv, split = blockIdx.y;
     const int ctx = min(a.ctx_lens[b], a.max_blocks * a.block_size);
-    const int tok0 = split * kSplitTokens;
-    if (tok0 >= ctx) return; // uniform for the block
-    const int ntok = min(kSplitTokens, ctx - tok0);
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int lt = lane / LPT;  // token within the wave step
-    const int dq = lane % LPT;  // which 16-element slice of the head
+    const int tok0 = split * SPLIT;
     const int G = a.group;
-
-    // this lane's slice of every query head of the group
-    half2_t qv[kMaxGroup][8];
-#pragma unroll
-    for (int h = 0; h < kMaxGroup; h++) {
-        if (h < G) {
-            const uint4 *src =
-                reinterpret_cast<const uint4 *>(a.q + ((size_t)b * a.hq + kvh * G + h) * D + dq * 16);
-            const uint4 lo = src[0], hi = src[1];
-            __builtin_memcpy(&qv[h][0], &lo, 16);
-            __builtin_memcpy(&qv[h][4], &hi, 16);
-        } else {
-#pragma unroll
-            for (int i = 0; i < 8; i++) qv[h][i] = half2_t{0, 0};
-        }
+    if (ctx <= 0) { // empty context: zeros, written by the first block of the pair
+        if (split == 0)
+            for (int idx = threadIdx.x; idx < G * D; idx += kAttnThreads) {
+                const size_t oi = ((size_t)b * a.hq + kvh * G) * D + idx;
+                if (a.out_f16) reinterpret_cast<__half *>(a.out)[oi] = __float2half_rn(0.f);
+                else reinterpret_cast<float *>(a.out)[oi] = 0.f;
+            }
+        return;
     }
+    if (tok0 >= ctx) return; // uniform for the block
+    const int ns = (ctx + SPLIT - 1) / SPLIT; // blocks of this (sequence, kv head) that get here
+    const int lane = threadIdx.x & 63;
+    // the wave index as a scalar, so that everything derived from it (tile positions, block-table
+    // lookups, cache base addresses) stays on the scalar unit
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int j = lane & 15, g = lane >> 4;
+    const int wave_tok0 = tok0 + wave * WAVE_TOKENS;
+    const int last_tile_tok = ((ctx - 1) >> 4) << 4;
     const int32_t *table = a.block_table + (size_t)b * a.max_blocks;
-    const int steps = (ntok + TPW - 1) / TPW;
 
-    // ---- pass 1: logits ----------------------------------------------------
-    for (int st = wave; st < steps; st += kAttnWaves) {
-        const int tl = st * TPW + lt; // token within the split
-        float s[kMaxGroup];
+    float m_w = -INFINITY, l_w = 0.f;
+    f32x4 o[DT];
 #pragma unroll
-        for (int h = 0; h < kMaxGroup; h++) s[h] = 0.f;
-        if (tl < ntok) {
-            const int tok = tok0 + tl;
+    for (int dt = 0; dt < DT; dt++) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    if (wave_tok0 < ctx) { // uniform for the wave
+        // ---- issue every load of this wave ----------------------------------------------
+        // A tile past the end of the context re-reads the last valid tile (always mapped
+        // memory); its logits are masked and its V operand is zeroed below.
+        // All block-table entries first (scalar loads), then every K and V load back to back: a
+        // lookup between two tiles' loads would wait for the earlier tile's data as well.
+        au32x4 kf[NT][KS];
+        au32x2 vf[NT][DT];
+        int pbs[NT], inb[NT];
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            const int tt = min(wave_tok0 + t * 16, last_tile_tok);
+            const uint32_t lb = fastdiv((uint32_t)tt, a.d_block);
+            inb[t] = tt - (int)lb * a.block_size;
+            pbs[t] = table[lb];
+        }
+        const uint32_t koff = (uint32_t)(j * D + g * 8) * 2u;            // bytes, the same for every tile
+        const uint32_t voff = (uint32_t)(j * a.block_size + g * 4) * 2u;
+        const size_t vstep = (size_t)a.block_size * 32;                  // 16 rows of d
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
             // a block id outside the cache would fault; read block 0 instead (undefined result, no fault)
-            const int pb = min(max(table[tok / a.block_size], 0), a.num_blocks - 1);
-            const uint16_t *kp =
-                a.k_cache + (((size_t)pb * a.hkv + kvh) * a.block_size + tok % a.block_size) * D + dq * 16;
-            const uint4 lo = reinterpret_cast<const uint4 *>(kp)[0], hi = reinterpret_cast<const uint4 *>(kp)[1];
-            half2_t kv[8];
-            __builtin_memcpy(&kv[0], &lo, 16);
-            __builtin_memcpy(&kv[4], &hi, 16);
+            const int pb = min(max(pbs[t], 0), a.num_blocks - 1);
+            const size_t head_base = ((size_t)pb * a.hkv + kvh) * (size_t)a.block_size * D;
+            const char *kb = reinterpret_cast<const char *>(a.k_cache) + (head_base + (size_t)inb[t] * D) * 2;
 #pragma unroll
-            for (int h = 0; h < kMaxGroup; h++)
-                if (h < G) {
+            for (int ks = 0; ks < KS; ks++) kf[t][ks] = *reinterpret_cast<const au32x4 *>(kb + ks * 64 + koff);
+            const char *vb = reinterpret_cast<const char *>(a.v_cache) + (head_base + (size_t)inb[t]) * 2;
 #pragma unroll
-                    for (int i = 0; i < 8; i++) s[h] = __builtin_amdgcn_fdot2(qv[h][i], kv[i], s[h], false);
-                }
+            for (int dt = 0; dt < DT; dt++) vf[t][dt] = *reinterpret_cast<const au32x2 *>(vb + dt * vstep + voff);
         }
+        // query heads of the group as the B operand (columns past the group are zero)
+        f16x8 qf[KS];
+        {
+            const uint16_t *qp = a.q + ((size_t)b * a.hq + kvh * G + min(j, G - 1)) * D + g * 8;
 #pragma unroll
-        for (int h = 0; h < kMaxGroup; h++)
-            if (h < G) {
-                float v = s[h];
-#pragma unroll
-                for (int o = 1; o < LPT; o <<= 1) v += __shfl_xor(v, o);
-                if (dq == 0) sc[h][st * TPW + lt] = (tl < ntok) ? v * a.scale : -INFINITY;
+            for (int ks = 0; ks < KS; ks++) {
+                au32x4 raw = *reinterpret_cast<const au32x4 *>(qp + ks * 32);
+                if (j >= G) raw = au32x4{0u, 0u, 0u, 0u};
+                __builtin_memcpy(&qf[ks], &raw, 16);
             }
+        }
+
+        // keep every load above the arithmetic (the scheduler would otherwise sink the V loads
+        // below the logit products to save registers, exposing a second memory round trip)
+        __builtin_amdgcn_sched_barrier(0);
+
+        // ---- logits, scaled to base-2 exponents -------------------------------------------
+        float s[NT][4];
+        float m_lane = -INFINITY;
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) {
+                f16x8 kk;
+                __builtin_memcpy(&kk, &kf[t][ks], 16);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(kk, qf[ks], acc, 0, 0, 0);
+            }
+            const int left = ctx - (wave_tok0 + t * 16 + g * 4); // valid tokens among this lane's four
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const float v = acc[r] * a.scale_log2e;
+                s[t][r] = r < left ? v : -INFINITY;
+                m_lane = fmaxf(m_lane, s[t][r]);
+            }
+        }
+        m_w = fmaxf(m_lane, __shfl_xor(m_lane, 16));
+        m_w = fmaxf(m_w, __shfl_xor(m_w, 32)); // finite: the wave's first token is valid for every head
+
+        // ---- probabilities and P.V, two token tiles per 16x16x32 product ----------------------
+        float l_lane = 0.f;
+#pragma unroll
+        for (int t = 0; t < NT; t += 2) {
+            f16x8 ph, pl;
+            uint32_t keep[2][2];
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                const int left = ctx - (wave_tok0 + (t + u) * 16 + g * 4);
+                keep[u][0] = (left > 0 ? 0x0000ffffu : 0u) | (left > 1 ? 0xffff0000u : 0u);
+                keep[u][1] = (left > 2 ? 0x0000ffffu : 0u) | (left > 3 ? 0xffff0000u : 0u);
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const float p = __builtin_amdgcn_exp2f(s[t + u][r] - m_w);
+                    l_lane += p;
+                    const _Float16 hi = (_Float16)p;
+                    ph[u * 4 + r] = hi;
+                    pl[u * 4 + r] = (_Float16)(p - (float)hi);
+                }
+            }
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++) {
+                // k slot (g, e): token 4g + e of tile t for e < 4, of tile t+1 otherwise - the same in both operands
+                const au32x4 raw = au32x4{vf[t][dt].x & keep[0][0], vf[t][dt].y & keep[0][1],
+                                          vf[t + 1][dt].x & keep[1][0], vf[t + 1][dt].y & keep[1][1]};
+                f16x8 vv;
+                __builtin_memcpy(&vv, &raw, 16);
+                o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ph, vv, o[dt], 0, 0, 0);
+                o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pl, vv, o[dt], 0, 0, 0);
+            }
+        }
+        l_w = l_lane + __shfl_xor(l_lane, 16);
+        l_w += __shfl_xor(l_w, 32);
+    }
+
+    // ---- merge the four waves ----------------------------------------------------------------
+    if (g == 0) {
+        smax[wave][j] = m_w;
+        ssum[wave][j] = l_w;
     }
     __syncthreads();
-
-    // ---- softmax statistics over the split ---------------------------------
-    const int padded = steps * TPW;
-    for (int h = wave; h < G; h += kAttnWaves) {
-        float m = -INFINITY;
-        for (int i = lane; i < padded; i += 64) m = fmaxf(m, sc[h][i]);
-        m = wave_max(m);
-        float l = 0.f;
-        for (int i = lane; i < padded; i += 64) {
-            const float p = __expf(sc[h][i] - m);
-            sc[h][i] = p;
-            l += p;
-        }
-        l = wave_sum(l);
-        if (lane == 0) {
-            hmax[h] = m;
-            hsum[h] = l;
-        }
+    // o[dt][r] belongs to head 4g + r, column dt*16 + j
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const int h = g * 4 + r;
+        float m = smax[0][h];
+#pragma unroll
+        for (int w = 1; w < kAttnWaves; w++) m = fmaxf(m, smax[w][h]);
+        const float f = __builtin_amdgcn_exp2f(smax[wave][h] - m); // 0 for a wave without tokens
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++) red[wave][h][dt * 16 + j] = o[dt][r] * f;
     }
-    __syncthreads();
-
-    // ---- pass 2: P.V ----------------------------------------------------------
-    float o[kMaxGroup][16];
-#pragma unroll
-    for (int h = 0; h < kMaxGroup; h++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) o[h][i] = 0.f;
-    for (int st = wave; st < steps; st += kAttnWaves) {
-        const int tl = st * TPW + lt;
-        if (tl < ntok) {
-            const int tok = tok0 + tl;
-            const int pb = min(max(table[tok / a.block_size], 0), a.num_blocks - 1);
-            const uint16_t *vp =
-                a.v_cache + (((size_t)pb * a.hkv + kvh) * a.block_size + tok % a.block_size) * D + dq * 16;
-            const uint4 lo = reinterpret_cast<const uint4 *>(vp)[0], hi = reinterpret_cast<const uint4 *>(vp)[1];
-            _Float16 vv[16];
-            __builtin_memcpy(&vv[0], &lo, 16);
-            __builtin_memcpy(&vv[8], &hi, 16);
-#pragma unroll
-            for (int h = 0; h < kMaxGroup; h++)
-                if (h < G) {
-                    const float p = sc[h][tl];
-#pragma unroll
-                    for (int i = 0; i < 16; i++) o[h][i] += p * (float)vv[i];
-                }
-        }
-    }
-    // sum over the lanes that hold different tokens of the same slice, then over waves
-#pragma unroll
-    for (int h = 0; h < kMaxGroup; h++)
-        if (h < G) {
-#pragma unroll
-            for (int i = 0; i < 16; i++) {
-                float v = o[h][i];
-#pragma unroll
-                for (int off = LPT; off < 64; off <<= 1) v += __shfl_xor(v, off);
-                o[h][i] = v;
-            }
-            if (lt == 0) {
-#pragma unroll
-                for (int i = 0; i < 16; i++) red[wave][h][dq * 16 + i] = o[h][i];
-            }
-        }
     __syncthreads();
     for (int idx = threadIdx.x; idx < G * D; idx += kAttnThreads) {
         const int h = idx / D, e = idx % D;
@@ -187,44 +233,75 @@ template <int D> __global__ __launch_bounds__(kAttnThreads) void paged_attn_spli
 #pragma unroll
         for (int w = 0; w < kAttnWaves; w++) v += red[w][h][e];
         const size_t row = ((size_t)b * a.hq + kvh * G + h) * a.splits + split;
-        a.part_o[row * D + e] = v;
+        coherent_store(a.part_o + row * D + e, v);
         if (e == 0) {
-            a.part_ml[row * 2 + 0] = hmax[h];
-            a.part_ml[row * 2 + 1] = hsum[h];
+            float m = smax[0][h];
+#pragma unroll
+            for (int w = 1; w < kAttnWaves; w++) m = fmaxf(m, smax[w][h]);
+            float l = 0.f;
+#pragma unroll
+            for (int w = 0; w < kAttnWaves; w++) l += ssum[w][h] * __builtin_amdgcn_exp2f(smax[w][h] - m);
+            coherent_store(a.part_ml + row * 2 + 0, m);
+            coherent_store(a.part_ml + row * 2 + 1, l);
         }
     }
+
+    // ---- the last block of the (sequence, kv head) to finish merges the splits -------------------
+    // The partials are written and read with device-scope accesses, which go through to the
+    // memory side instead of staying in the L2 of the XCD that issued them; waiting for this
+    // thread's stores and then for the block makes them globally visible before the count.
+    // (A device-scope fence would do the same by writing back and invalidating the whole L2,
+    // once per block - an order of magnitude slower here.)
+    uint32_t *done = a.done + (size_t)b * a.hkv + kvh;
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (ns > 1) {
+        if (threadIdx.x == 0)
+            s_last = __hip_atomic_fetch_add(done, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (uint32_t)(ns - 1);
+        __syncthreads();
+        if (!s_last) return;
+    }
+    // (max, sum) of every (head, split) into LDS with one round trip, then each thread merges one
+    // output element, eight splits' partials in flight at a time.
+    float *wm = &red[0][0][0], *wl = wm + kAttnHeads * kAttnMaxSplits; // `red` is free again
+    for (int idx = threadIdx.x; idx < G * ns; idx += kAttnThreads) {
+        const int h = idx / ns, sp = idx - h * ns;
+        const size_t row = ((size_t)b * a.hq + kvh * G + h) * a.splits + sp;
+        wm[idx] = coherent_load(a.part_ml + row * 2);
+        wl[idx] = coherent_load(a.part_ml + row * 2 + 1);
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < G * D; idx += kAttnThreads) {
+        const int h = idx / D, e = idx % D;
+        const float *po = a.part_o + ((size_t)b * a.hq + kvh * G + h) * a.splits * D + e;
+        float m = -INFINITY;
+        for (int sp = 0; sp < ns; sp++) m = fmaxf(m, wm[h * ns + sp]);
+        float num = 0.f, den = 0.f;
+        for (int sp0 = 0; sp0 < ns; sp0 += 8) {
+            float v[8];
+#pragma unroll
+            for (int k = 0; k < 8; k++) v[k] = coherent_load(po + (size_t)min(sp0 + k, ns - 1) * D);
+#pragma unroll
+            for (int k = 0; k < 8; k++)
+                if (sp0 + k < ns) {
+                    const float w = __builtin_amdgcn_exp2f(wm[h * ns + sp0 + k] - m);
+                    num += w * v[k];
+                    den += w * wl[h * ns + sp0 + k];
+                }
+        }
+        const float r = num / den;
+        const size_t oi = ((size_t)b * a.hq + kvh * G + h) * D + e;
+        if (a.out_f16) reinterpret_cast<__half *>(a.out)[oi] = __float2half_rn(r);
+        else reinterpret_cast<float *>(a.out)[oi] = r;
+    }
+    if (ns > 1 && threadIdx.x == 0) // ready for the next call on this stream
+        __hip_atomic_store(done, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Merges the per-split partials of one (sequence, query head).
-__global__ void paged_attn_merge_kernel(const AttnArgs a) {
-    const int h = blockIdx.x, b = blockIdx.y, e = threadIdx.x; // blockDim.x == D
-    const int ctx = min(a.ctx_lens[b], a.max_blocks * a.block_size);
-    const int ns = (ctx + kSplitTokens - 1) / kSplitTokens;
-    const size_t row0 = ((size_t)b * a.hq + h) * a.splits;
-    float m = -INFINITY;
-    for (int s = 0; s < ns; s++) m = fmaxf(m, a.part_ml[(row0 + s) * 2]);
-    float num = 0.f, den = 0.f;
-    for (int s = 0; s < ns; s++) {
-        const float w = __expf(a.part_ml[(row0 + s) * 2] - m);
-        num += w * a.part_o[(row0 + s) * a.d + e];
-        den += w * a.part_ml[(row0 + s) * 2 + 1];
-    }
-    const float r = ns > 0 ? num / den : 0.f;
-    const size_t oi = ((size_t)b * a.hq + h) * a.d + e;
-    if (a.out_f16) reinterpret_cast<__half *>(a.out)[oi] = __float2half_rn(r);
-    else reinterpret_cast<float *>(a.out)[oi] = r;
-}
 
 } // namespace nnhip
 
 using namespace nnhip;
-
-struct AttnWorkspace {
-    void *ptr = nullptr;
-    size_t bytes = 0;
-};
-// One workspace per device, grown on demand and kept until the process ends.
-static AttnWorkspace g_attn_ws[16];
 
 extern "C" int nncase_hip_paged_attention_decode(nncase_hip_ctx_t *ctx, const void *q_dev, const void *k_cache_dev,
                                                  const void *v_cache_dev, const int32_t *block_table_dev,
@@ -238,16 +315,16 @@ extern "C" int nncase_hip_paged_attention_decode(nncase_hip_ctx_t *ctx, const vo
                   -EINVAL, "paged_attention_decode: non-positive dimension");
     NNHIP_REQUIRE(ctx, p->head_dim == 64 || p->head_dim == 128, -NNCASE_HIP_ERR_SHAPE_MISMATCH,
                   "paged_attention_decode: head_dim %d (64 or 128 supported)", p->head_dim);
-    NNHIP_REQUIRE(ctx, p->num_q_heads % p->num_kv_heads == 0 && p->num_q_heads / p->num_kv_heads <= kMaxGroup,
+    NNHIP_REQUIRE(ctx, p->num_q_heads % p->num_kv_heads == 0 && p->num_q_heads / p->num_kv_heads <= kAttnHeads,
                   -NNCASE_HIP_ERR_SHAPE_MISMATCH, "paged_attention_decode: %d query heads per kv head unsupported (max %d)",
-                  p->num_q_heads / p->num_kv_heads, kMaxGroup);
-    const int tpw = 64 / (p->head_dim / 16);
-    NNHIP_REQUIRE(ctx, p->block_size > 0 && p->block_size % tpw == 0, -NNCASE_HIP_ERR_SHAPE_MISMATCH,
-                  "paged_attention_decode: block_size %d must be a multiple of %d", p->block_size, tpw);
+                  p->num_q_heads / p->num_kv_heads, kAttnHeads);
+    NNHIP_REQUIRE(ctx, p->block_size > 0 && p->block_size % 16 == 0, -NNCASE_HIP_ERR_SHAPE_MISMATCH,
+                  "paged_attention_decode: block_size %d must be a multiple of 16", p->block_size);
+    NNHIP_REQUIRE(ctx, (int64_t)p->max_blocks_per_seq * p->block_size < (int64_t(1) << 31), -EINVAL,
+                  "paged_attention_decode: context capacity exceeds 2^31 tokens");
     NNHIP_REQUIRE(ctx, p->out_dtype == NNCASE_HIP_DT_F16 || p->out_dtype == NNCASE_HIP_DT_F32,
                   -NNCASE_HIP_ERR_DATATYPE_MISMATCH, "paged_attention_decode: output type 0x%x", p->out_dtype);
-    NNHIP_REQUIRE(ctx, p->batch <= 65535 && p->num_kv_heads <= 65535, -EINVAL, "paged_attention_decode: grid too large");
-    NNHIP_REQUIRE(ctx, ctx->device >= 0 && ctx->device < 16, -EINVAL, "paged_attention_decode: device index");
+    NNHIP_REQUIRE(ctx, (int64_t)p->batch * p->num_kv_heads < (int64_t(1) << 31), -EINVAL, "paged_attention_decode: grid too large");
 
     AttnArgs a;
     memset(&a, 0, sizeof(a));
@@ -266,29 +343,59 @@ extern "C" int nncase_hip_paged_attention_decode(nncase_hip_ctx_t *ctx, const vo
     a.max_blocks = p->max_blocks_per_seq;
     a.num_blocks = p->num_blocks;
     const int64_t max_tokens = (int64_t)p->max_blocks_per_seq * p->block_size;
-    a.splits = (int)((max_tokens + kSplitTokens - 1) / kSplitTokens);
-    a.scale = p->scale;
+    // Tiles per wave: the largest run that still leaves about three blocks per compute unit when
+    // every sequence is at full length (the kernel cannot know the real lengths on the host).
+    const int nt_max = 512 / p->head_dim; // 8 KiB of K per wave
+    auto splits_at = [&](int tiles) { return (max_tokens + kAttnWaves * tiles * 16 - 1) / (kAttnWaves * tiles * 16); };
+    int nt = 2;
+    while (nt < nt_max && (splits_at(nt) > kAttnMaxSplits ||
+                           (int64_t)p->batch * p->num_kv_heads * splits_at(nt * 2) >= (int64_t)3 * ctx->compute_units))
+        nt *= 2;
+    a.split_tokens = kAttnWaves * nt * 16;
+    a.splits = (int)((max_tokens + a.split_tokens - 1) / a.split_tokens);
+    NNHIP_REQUIRE(ctx, a.splits <= kAttnMaxSplits, -EINVAL,
+                  "paged_attention_decode: context capacity of %lld tokens exceeds %d (head_dim %d)", (long long)max_tokens,
+                  kAttnMaxSplits * a.split_tokens, p->head_dim);
+    a.d_block = make_fastdiv((uint32_t)p->block_size);
+    a.scale_log2e = p->scale * kLog2e;
     a.out_f16 = p->out_dtype == NNCASE_HIP_DT_F16;
 
     const size_t rows = (size_t)a.batch * a.hq * a.splits;
     const size_t need = rows * (a.d + 2) * sizeof(float);
-    AttnWorkspace &ws = g_attn_ws[ctx->device];
-    if (ws.bytes < need) {
+    if (ctx->attn_ws_bytes < need) {
         NNHIP_HIP(ctx, hipStreamSynchronize(ctx->stream));
-        if (ws.ptr) NNHIP_HIP(ctx, hipFree(ws.ptr));
-        ws.ptr = nullptr;
-        ws.bytes = 0;
-        NNHIP_HIP(ctx, hipMalloc(&ws.ptr, need));
-        ws.bytes = need;
+        if (ctx->attn_ws) NNHIP_HIP(ctx, hipFree(ctx->attn_ws));
+        ctx->attn_ws = nullptr;
+        ctx->attn_ws_bytes = 0;
+        NNHIP_HIP(ctx, hipMalloc(&ctx->attn_ws, need));
+        ctx->attn_ws_bytes = need;
     }
-    a.part_o = reinterpret_cast<float *>(ws.ptr);
+    const size_t counters = (size_t)a.batch * a.hkv * sizeof(uint32_t);
+    if (ctx->attn_done_bytes < counters) {
+        NNHIP_HIP(ctx, hipStreamSynchronize(ctx->stream));
+        if (ctx->attn_done) NNHIP_HIP(ctx, hipFree(ctx->attn_done));
+        ctx->attn_done = nullptr;
+        ctx->attn_done_bytes = 0;
+        const size_t cap = (counters + 4095) / 4096 * 4096;
+        NNHIP_HIP(ctx, hipMalloc(&ctx->attn_done, cap));
+        ctx->attn_done_bytes = cap;
+        // zero before the first launch; every launch leaves the counters it used at zero again
+        NNHIP_HIP(ctx, hipMemsetAsync(ctx->attn_done, 0, cap, ctx->stream));
+    }
+    a.done = reinterpret_cast<uint32_t *>(ctx->attn_done);
+    a.part_o = reinterpret_cast<float *>(ctx->attn_ws);
     a.part_ml = a.part_o + rows * a.d;
 
-    const dim3 grid(a.splits, a.hkv, a.batch);
-    if (a.d == 64) hipLaunchKernelGGL(paged_attn_split_kernel<64>, grid, dim3(kAttnThreads), 0, ctx->stream, a);
-    else hipLaunchKernelGGL(paged_attn_split_kernel<128>, grid, dim3(kAttnThreads), 0, ctx->stream, a);
-    NNHIP_LAUNCH_CHECK(ctx, "paged_attn_split_kernel");
-    hipLaunchKernelGGL(paged_attn_merge_kernel, dim3(a.hq, a.batch), dim3(a.d), 0, ctx->stream, a);
-    NNHIP_LAUNCH_CHECK(ctx, "paged_attn_merge_kernel");
+    const dim3 grid(a.hkv * a.batch, a.splits);
+    const dim3 block(kAttnThreads);
+    if (a.d == 64) {
+        if (nt == 8) hipLaunchKernelGGL((paged_attn_kernel<64, 8>), grid, block, 0, ctx->stream, a);
+        else if (nt == 4) hipLaunchKernelGGL((paged_attn_kernel<64, 4>), grid, block, 0, ctx->stream, a);
+        else hipLaunchKernelGGL((paged_attn_kernel<64, 2>), grid, block, 0, ctx->stream, a);
+    } else {
+        if (nt == 4) hipLaunchKernelGGL((paged_attn_kernel<128, 4>), grid, block, 0, ctx->stream, a);
+        else hipLaunchKernelGGL((paged_attn_kernel<128, 2>), grid, block, 0, ctx->stream, a);
+    }
+    NNHIP_LAUNCH_CHECK(ctx, "paged_attn_kernel");
     return 0;
 }

@@ -19,6 +19,12 @@ struct nncase_hip_ctx {
     int compute_units = 0;
     int clock_khz = 0;
     size_t hbm_bytes = 0;
+    // paged-attention partials and completion counters: grown on demand, owned by the context
+    // (calls on one context are ordered on its stream, so they can share it)
+    void *attn_ws = nullptr;
+    size_t attn_ws_bytes = 0;
+    void *attn_done = nullptr; // counters live apart from the partials: they must stay zero between calls
+    size_t attn_done_bytes = 0;
     char last_error[512] = {0};
 };
 

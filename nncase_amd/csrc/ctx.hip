@@ -38,6 +38,8 @@ extern "C" int nncase_hip_ctx_create(int device, nncase_hip_ctx_t **out) {
 extern "C" int nncase_hip_ctx_destroy(nncase_hip_ctx_t *ctx) {
     NNHIP_CHECK_CTX(ctx);
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+    if (ctx->attn_ws) (void)hipFree(ctx->attn_ws);
+    if (ctx->attn_done) (void)hipFree(ctx->attn_done);
     if (ctx->owns_stream && ctx->stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
     return 0;

@@ -77,11 +77,18 @@ __device__ __forceinline__ int32_t mad16_hi(uint32_t x, uint32_t w, int32_t acc)
     return d;
 }
 
+// A conditional between two named objects is an lvalue in C++, which the compiler may turn
+// into a load through a selected address (private memory); taking the operands by value
+// keeps the choice a register select.
+__device__ __forceinline__ uint32_t select_u32(bool c, uint32_t yes, uint32_t no) { return c ? yes : no; }
+
 // All offsets are 32-bit element offsets from the (uniform) tensor bases, advanced by
 // additions only; the host checks that both tensors stay below 2^31 elements.
 // The loads of the rows the NEXT output row needs are issued before the current row is
 // computed, so a whole row of arithmetic covers their latency.
-template <int S> __global__ __launch_bounds__(kDwThreads) void dw3x3_kernel(const DwArgs a) {
+// The stride-2 kernel holds nine input columns per row; asking for three blocks per CU keeps it
+// at 3 waves per SIMD (without the bound the allocator takes 176 VGPRs and drops to 2).
+template <int S> __global__ __launch_bounds__(kDwThreads, (S == 2 ? 3 : 1)) void dw3x3_kernel(const DwArgs a) {
     constexpr int NCOL = (kDwCols - 1) * S + 3;
     const uint32_t gid = blockIdx.x * kDwThreads + threadIdx.x;
     if (gid >= (uint32_t)a.total) return;
@@ -97,6 +104,7 @@ template <int S> __global__ __launch_bounds__(kDwThreads) void dw3x3_kernel(cons
     const int rchunk = (int)(t - q * a.d_rows.div);
     const int img = (int)q;
 
+    const uint32_t zx_splat = a.zx_splat;
     const int c0 = cq * 4;
     const int ox0 = strip * kDwCols;
     const int oy0 = rchunk * a.rows;
@@ -148,7 +156,7 @@ template <int S> __global__ __launch_bounds__(kDwThreads) void dw3x3_kernel(cons
     auto unpack_row = [&](int buf, const uint32_t (&raw)[NCOL], bool row_ok) {
 #pragma unroll
         for (int col = 0; col < NCOL; col++) {
-            const uint32_t d = (row_ok && col_ok[col]) ? raw[col] : a.zx_splat;
+            const uint32_t d = select_u32(row_ok && col_ok[col], raw[col], zx_splat);
             r01[buf][col] = __builtin_amdgcn_perm(0u, d, 0x0c010c00u); // [b0, 0, b1, 0]
             r23[buf][col] = __builtin_amdgcn_perm(0u, d, 0x0c030c02u); // [b2, 0, b3, 0]
         }

@@ -196,15 +196,23 @@ def transpose_nhwc_to_nchw(input: np.ndarray, ctx: Context = None) -> np.ndarray
     return dst.download((n, ch, h, w), x.dtype)
 
 
+def v_cache_from_token_major(v_cache: np.ndarray) -> np.ndarray:
+    """[blocks, Hkv, block, D] -> the d-major [blocks, Hkv, D, block] layout the decode kernel reads."""
+    return np.ascontiguousarray(np.asarray(v_cache).transpose(0, 1, 3, 2))
+
+
 def paged_attention_decode(q: np.ndarray, k_cache: np.ndarray, v_cache: np.ndarray, block_table: np.ndarray,
                            ctx_lens: np.ndarray, scale: float, out_dtype=np.float32, ctx: Context = None) -> np.ndarray:
-    """q [B, Hq, D] f16; caches [blocks, Hkv, block, D] f16; block_table [B, max_blocks] i32; ctx_lens [B] i32."""
+    """q [B, Hq, D] f16; K cache [blocks, Hkv, block, D] f16; V cache [blocks, Hkv, D, block] f16 (d-major, see
+    v_cache_from_token_major); block_table [B, max_blocks] i32; ctx_lens [B] i32."""
     c = _ctx(ctx)
     qh = np.ascontiguousarray(q, np.float16)
     kc, vc = np.ascontiguousarray(k_cache, np.float16), np.ascontiguousarray(v_cache, np.float16)
     bt, cl = np.ascontiguousarray(block_table, np.int32), np.ascontiguousarray(ctx_lens, np.int32)
     bsz, hq, d = qh.shape
     nb, hkv, blk, _ = kc.shape
+    if vc.shape != (nb, hkv, d, blk):
+        raise ValueError(f"v_cache shape {vc.shape}: expected the d-major layout {(nb, hkv, d, blk)}")
     out_dtype = np.dtype(out_dtype)
     dq, dk, dv, dbt, dcl = (c.to_device(t) for t in (qh, kc, vc, bt, cl))
     dout = c.alloc(bsz * hq * d * out_dtype.itemsize)

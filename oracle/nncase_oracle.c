@@ -598,10 +598,11 @@ ORACLE_API int attn_paged_decode_f64(const uint16_t *q, const uint16_t *k_cache,
             }
             for (int32_t t = 0; t < len; t++) {
                 const int32_t pb = block_table[(size_t)b * max_blocks + t / block];
-                const uint16_t *vr =
-                    v_cache + (((size_t)pb * hkv + kvh) * block + t % block) * d;
+                /* V is cached d-major: [block][kv head][d][token in block] */
+                const uint16_t *vr = v_cache + ((size_t)pb * hkv + kvh) * d * block + t % block;
                 const double p = logit[t] / den;
-                for (int32_t e = 0; e < d; e++) o[e] += p * (double)ref_f16_to_f32(vr[e]);
+                for (int32_t e = 0; e < d; e++)
+                    o[e] += p * (double)ref_f16_to_f32(vr[(size_t)e * block]);
             }
         }
         free(logit);

@@ -260,13 +260,13 @@ def qconv2d_float_chain(x, w, bias, zx, sx, zw, sw, zy, sy, stride=(1, 1), paddi
 
 # ---------------------------------------------------------------- no reference counterpart
 def paged_attention_decode(q_bits, k_cache_bits, v_cache_bits, block_table, ctx_lens, scale):
-    """float64 brute force.  q [B,Hq,D] f16 bits; caches [blocks,Hkv,block,D] f16 bits."""
+    """float64 brute force.  q [B,Hq,D] f16 bits; K cache [blocks,Hkv,block,D], V cache [blocks,Hkv,D,block] f16 bits."""
     q = _c(q_bits, np.uint16)
     kc, vc = _c(k_cache_bits, np.uint16), _c(v_cache_bits, np.uint16)
     bt, cl = _c(block_table, np.int32), _c(ctx_lens, np.int32)
     bsz, hq, d = q.shape
     nb, hkv, blk, d2 = kc.shape
-    assert d == d2 and vc.shape == kc.shape
+    assert d == d2 and vc.shape == (nb, hkv, d, blk)
     out = np.empty((bsz, hq, d), np.float64)
     rc = lib().attn_paged_decode_f64(_p(q), _p(kc), _p(vc), _p(bt), _p(cl), _p(out), _i(bsz), _i(hq), _i(hkv), _i(d),
                                      _i(blk), _i(bt.shape[1]), _i(nb), C.c_double(scale))

@@ -23,8 +23,11 @@ def make_case(rng, bsz, hq, hkv, d, blk, max_ctx, ctx_lens=None):
 
 
 def check(hip_ctx, q, kc, vc, bt, cl, scale, out_dtype=np.float32):
-    got = K.paged_attention_decode(q, kc, vc, bt, cl, scale, out_dtype, ctx=hip_ctx).astype(np.float64)
-    want = O.paged_attention_decode(q.view(np.uint16), kc.view(np.uint16), vc.view(np.uint16), bt, cl, scale)
+    """vc is token-major [blocks, Hkv, block, D] (easy to index in the expectations); the kernel and
+    the oracle both take the d-major cache layout."""
+    vt = K.v_cache_from_token_major(vc)
+    got = K.paged_attention_decode(q, kc, vt, bt, cl, scale, out_dtype, ctx=hip_ctx).astype(np.float64)
+    want = O.paged_attention_decode(q.view(np.uint16), kc.view(np.uint16), vt.view(np.uint16), bt, cl, scale)
     tol = RTOL * np.abs(want).max(axis=-1, keepdims=True) + (1e-3 if out_dtype == np.float16 else 1e-6)
     assert (np.abs(got - want) <= tol).all(), f"max err {np.abs(got - want).max()}"
     return got
@@ -36,6 +39,9 @@ def check(hip_ctx, q, kc, vc, bt, cl, scale, out_dtype=np.float32):
     (2, 8, 1, 64, 32, 1100),     # MQA, 8 query heads on one kv head, block 32, three splits
     (2, 8, 2, 128, 16, 600),     # head_dim 128
     (1, 2, 2, 64, 64, 64),
+    (2, 16, 1, 64, 48, 500),     # 16 query heads on one kv head; block size not a power of two
+    (2, 32, 2, 128, 16, 300),    # 16 per kv head at head_dim 128
+    (3, 1, 1, 128, 32, 257),     # a single head
 ])
 def test_random_cases(hip_ctx, bsz, hq, hkv, d, blk, max_ctx):
     rng = np.random.default_rng(bsz * 1000 + hq)
@@ -60,7 +66,7 @@ def test_closed_forms(hip_ctx):
     base = check(hip_ctx, q, kc, vc, bt, cl, 0.125)
     # uniform keys -> plain mean of the cached values
     ku = np.ones_like(kc)
-    got = K.paged_attention_decode(q, ku, vc, bt, cl, 0.125, ctx=hip_ctx)
+    got = K.paged_attention_decode(q, ku, K.v_cache_from_token_major(vc), bt, cl, 0.125, ctx=hip_ctx)
     for b in range(2):
         toks = [(bt[b, t // 16], t % 16) for t in range(cl[b])]
         for kvh in range(2):
@@ -69,10 +75,29 @@ def test_closed_forms(hip_ctx):
     # relabelling physical blocks leaves the output bit-identical
     perm = rng.permutation(kc.shape[0])
     inv = np.argsort(perm).astype(np.int32)
-    again = K.paged_attention_decode(q, kc[perm], vc[perm], inv[bt], cl, 0.125, ctx=hip_ctx)
+    again = K.paged_attention_decode(q, kc[perm], K.v_cache_from_token_major(vc[perm]), inv[bt], cl, 0.125, ctx=hip_ctx)
     assert np.array_equal(again.astype(np.float64), base)
-    # large logits do not overflow the softmax
+    # large logits do not overflow the softmax; a negative scale is honoured
     check(hip_ctx, (q * 30).astype(np.float16), kc, vc, bt, cl, 1.0)
+    check(hip_ctx, q, kc, vc, bt, cl, -0.125)
+
+
+def test_slots_past_the_context_are_ignored(hip_ctx):
+    """Cache slots of the last block beyond ctx_len (and blocks the table lists past it) may hold
+    anything, NaN and Inf included, without touching the result."""
+    rng = np.random.default_rng(13)
+    lens = [5, 16, 37, 600]
+    q, kc, vc, bt, cl = make_case(rng, len(lens), 14, 2, 64, 16, 640, lens)
+    base = check(hip_ctx, q, kc, vc, bt, cl, 0.125)
+    kc2, vc2 = kc.copy(), vc.copy()
+    poison = np.array([np.nan, np.inf, -np.inf, 65504.0], np.float16)
+    for b, n in enumerate(lens):
+        for t in range(n, bt.shape[1] * 16):
+            kc2[bt[b, t // 16], :, t % 16, :] = poison[t % 4]
+            vc2[bt[b, t // 16], :, t % 16, :] = poison[(t + 1) % 4]
+    vt2 = K.v_cache_from_token_major(vc2)
+    again = K.paged_attention_decode(q, kc2, vt2, bt, cl, 0.125, ctx=hip_ctx).astype(np.float64)
+    assert np.array_equal(again, base)
 
 
 def test_config5_shape(hip_ctx):
@@ -82,14 +107,43 @@ def test_config5_shape(hip_ctx):
     check(hip_ctx, q, kc, vc, bt, cl, 0.125, np.float16)
 
 
+def test_long_runs_per_wave(hip_ctx):
+    """Enough sequences that the kernel takes its longest per-wave runs (8 tiles of 16 tokens at head_dim 64,
+    4 at head_dim 128), with ragged lengths around the split boundaries."""
+    rng = np.random.default_rng(17)
+    lens = np.concatenate([[1, 511, 512, 513, 1023, 1025, 2048], rng.integers(1, 2049, 89)])
+    q, kc, vc, bt, cl = make_case(rng, len(lens), 8, 4, 64, 16, 2048, lens)
+    check(hip_ctx, q, kc, vc, bt, cl, 0.125)
+    lens = np.concatenate([[1, 255, 256, 257, 1024], rng.integers(1, 1025, 91)])
+    q, kc, vc, bt, cl = make_case(rng, len(lens), 8, 8, 128, 16, 1024, lens)
+    check(hip_ctx, q, kc, vc, bt, cl, 0.09)
+
+
+def test_repeated_calls_reuse_the_workspace(hip_ctx):
+    """The completion counters return to zero after every call: different shapes back to back."""
+    rng = np.random.default_rng(19)
+    for bsz, hq, hkv, d, max_ctx in [(4, 14, 2, 64, 2000), (2, 8, 8, 128, 700), (4, 14, 2, 64, 2000), (1, 4, 1, 64, 90)]:
+        case = make_case(rng, bsz, hq, hkv, d, 16, max_ctx)
+        check(hip_ctx, *case, 0.125)
+        check(hip_ctx, *case, 0.125)
+
+
 def test_error_paths(hip_ctx):
     from nncase_amd import runtime as rt
     rng = np.random.default_rng(1)
     q, kc, vc, bt, cl = make_case(rng, 1, 3, 2, 64, 16, 32)   # 3 query heads on 2 kv heads
     with pytest.raises(rt.HipError) as e:
-        K.paged_attention_decode(q, kc, vc, bt, cl, 0.125, ctx=hip_ctx)
+        K.paged_attention_decode(q, kc, K.v_cache_from_token_major(vc), bt, cl, 0.125, ctx=hip_ctx)
     assert e.value.code == -rt.ERR_SHAPE_MISMATCH
     q, kc, vc, bt, cl = make_case(rng, 1, 2, 2, 32, 16, 32)   # unsupported head_dim
     with pytest.raises(rt.HipError) as e:
-        K.paged_attention_decode(q, kc, vc, bt, cl, 0.125, ctx=hip_ctx)
+        K.paged_attention_decode(q, kc, K.v_cache_from_token_major(vc), bt, cl, 0.125, ctx=hip_ctx)
+    assert e.value.code == -rt.ERR_SHAPE_MISMATCH
+    q, kc, vc, bt, cl = make_case(rng, 1, 2, 2, 64, 8, 32)    # block size not a multiple of 16
+    with pytest.raises(rt.HipError) as e:
+        K.paged_attention_decode(q, kc, K.v_cache_from_token_major(vc), bt, cl, 0.125, ctx=hip_ctx)
+    assert e.value.code == -rt.ERR_SHAPE_MISMATCH
+    q, kc, vc, bt, cl = make_case(rng, 1, 17, 1, 64, 16, 32)  # 17 query heads on one kv head
+    with pytest.raises(rt.HipError) as e:
+        K.paged_attention_decode(q, kc, K.v_cache_from_token_major(vc), bt, cl, 0.125, ctx=hip_ctx)
     assert e.value.code == -rt.ERR_SHAPE_MISMATCH

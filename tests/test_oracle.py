@@ -345,7 +345,9 @@ def test_paged_attention_closed_forms():
     vc = rng.standard_normal((nb, hkv, blk, d)).astype(np.float16)
     bt = np.stack([rng.permutation(nb)[:4] for _ in range(bsz)]).astype(np.int32)
     cl = np.array([1, 17, 64], np.int32)
-    out = O.paged_attention_decode(q.view(np.uint16), kc.view(np.uint16), vc.view(np.uint16), bt, cl, 0.125)
+    def dmajor(v):  # the V cache is d-major: [blocks, Hkv, D, block]
+        return np.ascontiguousarray(v.transpose(0, 1, 3, 2)).view(np.uint16)
+    out = O.paged_attention_decode(q.view(np.uint16), kc.view(np.uint16), dmajor(vc), bt, cl, 0.125)
     # ctx == 1 -> the V row of the first cached token, kv head = h // 2
     for h in range(hq):
         assert np.array_equal(out[0, h], vc[bt[0, 0], h // 2, 0].astype(np.float64))
@@ -361,13 +363,13 @@ def test_paged_attention_closed_forms():
             np.testing.assert_allclose(out[b, h], p_ @ V, rtol=1e-12, atol=1e-12)
     # uniform K -> mean of V
     kc2 = np.ones_like(kc)
-    out2 = O.paged_attention_decode(q.view(np.uint16), kc2.view(np.uint16), vc.view(np.uint16), bt, cl, 0.125)
+    out2 = O.paged_attention_decode(q.view(np.uint16), kc2.view(np.uint16), dmajor(vc), bt, cl, 0.125)
     toks = [(bt[1, t // blk], t % blk) for t in range(17)]
     np.testing.assert_allclose(out2[1, 3], np.mean([vc[p, 1, o].astype(np.float64) for p, o in toks], axis=0), rtol=1e-12, atol=1e-12)
     # relabelling physical blocks (cache permuted together with the table) changes nothing
     perm = rng.permutation(nb)
     inv = np.argsort(perm)
-    out3 = O.paged_attention_decode(q.view(np.uint16), kc[perm].view(np.uint16), vc[perm].view(np.uint16), inv[bt].astype(np.int32), cl, 0.125)
+    out3 = O.paged_attention_decode(q.view(np.uint16), kc[perm].view(np.uint16), dmajor(vc[perm]), inv[bt].astype(np.int32), cl, 0.125)
     assert np.array_equal(out, out3)
 
 
