@@ -30,18 +30,48 @@ HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 INT8_PEAK_TOPS = 5000.0    # dense int8 MFMA
 
 
-def algorithmic_bytes(qg, batch):
+# Bytes that crossed the L2 <-> fabric boundary per launch (average over the launches of a kernel in
+# one step) at the headline workload, from two rocprofv3 --pmc runs of this script (FETCH_SIZE, then
+# WRITE_SIZE, each scaled by what the same counter reads for the 256 MiB copy that --copy-probe
+# launches: x1.9997 and x1.0000).  Counters cannot be read from inside a timed run, so the figures
+# are recorded here and reported only for the configuration they were measured on.
+MEASURED_TRAFFIC_B64 = {
+    "dequantize": 354803,
+    "dw3x3<S=1>": 19398340,
+    "dw3x3<S=2>": 41830103,
+    "qconv_igemm<T=1,RG=1,rows16>": 6041031,
+    "qconv_igemm<T=1,RG=4,rows16>": 38694361,
+    "qconv_igemm<T=12,RG=1,rows16>": 10391442,
+    "qconv_igemm<T=2,RG=1,rows16>": 10279565,
+    "qconv_igemm<T=2,RG=2,rows16>": 31506435,
+    "qconv_igemm<T=5,RG=1,rows16>": 5171008,
+    "qconv_igemm<T=6,RG=1,rows16>": 8668773,
+    "qconv_igemm<T=6,RG=2,rows16>": 90218140,
+    "qconv_igemm<T=8,RG=1,rows16>": 6011810,
+    "qconv_igemm<T=9,RG=1,vec8>": 33995909,
+    "qconv_smallc<C=3>": 38855552,
+    "qglobal_avgpool": 4122090,
+    "quantize": 48214802,
+}
+
+
+def algorithmic_bytes(qg, batch, fused_into):
     """Per operator of the recorded function: bytes an ideal implementation must move
-    (read every input once, write every output once, read the constants once)."""
+    (read every input once, write every output once, read the constants once).
+    fused_into maps a conv node to the residual add folded into its epilogue: that add is
+    no operator of its own, and its conv reads the residual tensor as well."""
     out = []
-    for n in qg.nodes:
+    fused_adds = set(fused_into.values())
+    for i, n in enumerate(qg.nodes):
+        if i in fused_adds:
+            continue
         c, h, w = n.out_shape
         o = batch * c * h * w
         if n.op == "input":
             out.append(o * 4 + o)
         elif n.op == "conv":
             sc, sh, sw = qg.nodes[n.inputs[0]].out_shape
-            out.append(batch * sc * sh * sw + o + n.weights.size + 4 * n.bias.size)
+            out.append(batch * sc * sh * sw + o + n.weights.size + 4 * n.bias.size + (o if i in fused_into else 0))
         elif n.op == "add":
             out.append(3 * o)
         elif n.op == "gap":
@@ -53,9 +83,12 @@ def algorithmic_bytes(qg, batch):
     return out
 
 
-def conv_macs(qg, batch):
+def conv_macs(qg, batch, fused_into):
     out = []
-    for n in qg.nodes:
+    fused_adds = set(fused_into.values())
+    for i, n in enumerate(qg.nodes):
+        if i in fused_adds:
+            continue
         if n.op == "conv":
             oc, gic, kh, kw = n.weights.shape
             out.append(batch * oc * n.out_shape[1] * n.out_shape[2] * gic * kh * kw)
@@ -114,7 +147,7 @@ def side_workload(args):
         model.set_input(rng.random((batch, 56, 56, 64), dtype=np.float32))
         ms = time_calls(ctx, model.invoke, args.warmup, args.steps)
         op_ms = model.fn.profile(10)
-        nbytes = sum(algorithmic_bytes(qg, batch))
+        nbytes = sum(algorithmic_bytes(qg, batch, model.fused_into))
         line = dict(base, metric="images/sec u8/u8 conv block b32", value=round(batch / (ms * 1e-3), 1), unit="images/s",
                     ms_per_step=round(ms, 5), dtype="u8",
                     config={"workload": "config 2: f32 in -> quantize -> 1x1 64->144, dw 3x3, 1x1 144->64 (ReLU6) on 56x56 -> dequantize, batch 32"},
@@ -205,8 +238,9 @@ def main():
     # ---- per-kernel device time (HIP events on the context's stream) --------------------------
     op_ms = model.fn.profile(args.profile_iters)
     names = [model.fn.op_kernel(i) for i in range(len(model.fn))]
-    abytes = algorithmic_bytes(qg, args.batch)
-    macs = conv_macs(qg, args.batch)
+    abytes = algorithmic_bytes(qg, args.batch, model.fused_into)
+    macs = conv_macs(qg, args.batch, model.fused_into)
+    assert len(abytes) == len(macs) == len(names) == len(op_ms)
     groups = {}
     for name, ms, b, m in zip(names, op_ms, abytes, macs):
         g = groups.setdefault(name, {"ms": 0.0, "bytes": 0, "macs": 0, "launches": 0})
@@ -277,7 +311,8 @@ def main():
                                "NHWC f32 input resident in HBM -> quantize -> 52 convs + 10 adds + pool + FC -> dequantize",
                    "batch": args.batch, "ops_per_step": len(model.fn), "execution": "resident hip function, " + ("eager launches" if args.no_graph else "HIP-graph replay")},
         "roofline": {"bound": "hbm", "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(dom_gbs / HBM_PEAK_GBS, 4), "traffic": None, "kernel": dom_name,
+                     "frac": round(dom_gbs / HBM_PEAK_GBS, 4),
+                     "traffic": MEASURED_TRAFFIC_B64.get(dom_name) if args.batch == 64 else None, "kernel": dom_name,
                      "launches_per_step": dom["launches"], "avg_launch_us": round(dom["ms"] / dom["launches"] * 1e3, 2),
                      "algorithmic_bytes_per_launch": int(dom["bytes"] / dom["launches"]),
                      "share_of_device_time": round(dom["ms"] / sum(op_ms), 4)},

@@ -41,7 +41,7 @@ constexpr int kAttnWaves = 4;
 constexpr int kAttnHeads = 16; // query heads per kv head, padded to the MFMA tile
 constexpr float kLog2e = 1.4426950408889634f;
 
-constexpr int kAttnMaxSplits = 128; // (max, sum) of 16 heads x 128 splits fit the 16 KiB LDS buffer at merge time
+constexpr int kAttnMaxSplits = 1024; // splits of one sequence (bounds the merge loop and the workspace)
 
 struct AttnArgs {
     const uint16_t *q, *k_cache, *v_cache;
@@ -76,9 +76,28 @@ template <int D, int NT> __global__ __launch_bounds__(kAttnThreads, 2) void page
     // kv head fastest, then sequence, then split: consecutive workgroups go to different XCDs, so
     // every XCD gets the same mix of early (always present) and late (long contexts only) splits
     const int kvh = blockIdx.x % a.hkv, b = blockIdx.x / a.hkv, split = blockIdx.y;
-    const int ctx = min(a.ctx_lens[b], a.max_blocks * a.block_size);
     const int tok0 = split * SPLIT;
     const int G = a.group;
+    const int lane = threadIdx.x & 63;
+    // the wave index as a scalar, so that everything derived from it (tile positions, block-table
+    // lookups, cache base addresses) stays on the scalar unit
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int j = lane & 15, g = lane >> 4;
+    const int wave_tok0 = tok0 + wave * WAVE_TOKENS;
+    // The block-table entries of this wave's tiles do not depend on the context length, so they
+    // are fetched together with it (one scalar-memory round trip instead of two).  A tile past
+    // the end of the context may get any entry of the table; its block id is clamped into the
+    // cache, its logits are masked and its V operand is zeroed.
+    const int32_t *table = a.block_table + (size_t)b * a.max_blocks;
+    int pbs[NT], inb[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        const int tt = wave_tok0 + t * 16;
+        const uint32_t lb = fastdiv((uint32_t)tt, a.d_block);
+        inb[t] = tt - (int)lb * a.block_size;
+        pbs[t] = table[min((int)lb, a.max_blocks - 1)];
+    }
+    const int ctx = min(a.ctx_lens[b], a.max_blocks * a.block_size);
     if (ctx <= 0) { // empty context: zeros, written by the first block of the pair
         if (split == 0)
             for (int idx = threadIdx.x; idx < G * D; idx += kAttnThreads) {
@@ -90,14 +109,6 @@ template <int D, int NT> __global__ __launch_bounds__(kAttnThreads, 2) void page
     }
     if (tok0 >= ctx) return; // uniform for the block
     const int ns = (ctx + SPLIT - 1) / SPLIT; // blocks of this (sequence, kv head) that get here
-    const int lane = threadIdx.x & 63;
-    // the wave index as a scalar, so that everything derived from it (tile positions, block-table
-    // lookups, cache base addresses) stays on the scalar unit
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int j = lane & 15, g = lane >> 4;
-    const int wave_tok0 = tok0 + wave * WAVE_TOKENS;
-    const int last_tile_tok = ((ctx - 1) >> 4) << 4;
-    const int32_t *table = a.block_table + (size_t)b * a.max_blocks;
 
     float m_w = -INFINITY, l_w = 0.f;
     f32x4 o[DT];
@@ -106,20 +117,10 @@ template <int D, int NT> __global__ __launch_bounds__(kAttnThreads, 2) void page
 
     if (wave_tok0 < ctx) { // uniform for the wave
         // ---- issue every load of this wave ----------------------------------------------
-        // A tile past the end of the context re-reads the last valid tile (always mapped
-        // memory); its logits are masked and its V operand is zeroed below.
-        // All block-table entries first (scalar loads), then every K and V load back to back: a
-        // lookup between two tiles' loads would wait for the earlier tile's data as well.
+        // Every K and V load back to back (the block-table entries are already here: a lookup
+        // between two tiles' loads would wait for the earlier tile's data as well).
         au32x4 kf[NT][KS];
         au32x2 vf[NT][DT];
-        int pbs[NT], inb[NT];
-#pragma unroll
-        for (int t = 0; t < NT; t++) {
-            const int tt = min(wave_tok0 + t * 16, last_tile_tok);
-            const uint32_t lb = fastdiv((uint32_t)tt, a.d_block);
-            inb[t] = tt - (int)lb * a.block_size;
-            pbs[t] = table[lb];
-        }
         const uint32_t koff = (uint32_t)(j * D + g * 8) * 2u;            // bytes, the same for every tile
         const uint32_t voff = (uint32_t)(j * a.block_size + g * 4) * 2u;
         const size_t vstep = (size_t)a.block_size * 32;                  // 16 rows of d
@@ -232,19 +233,27 @@ template <int D, int NT> __global__ __launch_bounds__(kAttnThreads, 2) void page
         float v = 0.f;
 #pragma unroll
         for (int w = 0; w < kAttnWaves; w++) v += red[w][h][e];
-        const size_t row = ((size_t)b * a.hq + kvh * G + h) * a.splits + split;
-        coherent_store(a.part_o + row * D + e, v);
-        if (e == 0) {
-            float m = smax[0][h];
+        float m = smax[0][h];
 #pragma unroll
-            for (int w = 1; w < kAttnWaves; w++) m = fmaxf(m, smax[w][h]);
-            float l = 0.f;
+        for (int w = 1; w < kAttnWaves; w++) m = fmaxf(m, smax[w][h]);
+        float l = 0.f;
 #pragma unroll
-            for (int w = 0; w < kAttnWaves; w++) l += ssum[w][h] * __builtin_amdgcn_exp2f(smax[w][h] - m);
-            coherent_store(a.part_ml + row * 2 + 0, m);
-            coherent_store(a.part_ml + row * 2 + 1, l);
+        for (int w = 0; w < kAttnWaves; w++) l += ssum[w][h] * __builtin_amdgcn_exp2f(smax[w][h] - m);
+        if (ns == 1) { // the whole context was in this block
+            const float r = v / l;
+            const size_t oi = ((size_t)b * a.hq + kvh * G + h) * D + e;
+            if (a.out_f16) reinterpret_cast<__half *>(a.out)[oi] = __float2half_rn(r);
+            else reinterpret_cast<float *>(a.out)[oi] = r;
+        } else {
+            const size_t row = ((size_t)b * a.hq + kvh * G + h) * a.splits + split;
+            coherent_store(a.part_o + row * D + e, v);
+            if (e == 0) {
+                coherent_store(a.part_ml + row * 2 + 0, m);
+                coherent_store(a.part_ml + row * 2 + 1, l);
+            }
         }
     }
+    if (ns == 1) return;
 
     // ---- the last block of the (sequence, kv head) to finish merges the splits -------------------
     // The partials are written and read with device-scope accesses, which go through to the
@@ -255,46 +264,47 @@ template <int D, int NT> __global__ __launch_bounds__(kAttnThreads, 2) void page
     uint32_t *done = a.done + (size_t)b * a.hkv + kvh;
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
-    if (ns > 1) {
-        if (threadIdx.x == 0)
-            s_last = __hip_atomic_fetch_add(done, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (uint32_t)(ns - 1);
-        __syncthreads();
-        if (!s_last) return;
-    }
-    // (max, sum) of every (head, split) into LDS with one round trip, then each thread merges one
-    // output element, eight splits' partials in flight at a time.
-    float *wm = &red[0][0][0], *wl = wm + kAttnHeads * kAttnMaxSplits; // `red` is free again
-    for (int idx = threadIdx.x; idx < G * ns; idx += kAttnThreads) {
-        const int h = idx / ns, sp = idx - h * ns;
-        const size_t row = ((size_t)b * a.hq + kvh * G + h) * a.splits + sp;
-        wm[idx] = coherent_load(a.part_ml + row * 2);
-        wl[idx] = coherent_load(a.part_ml + row * 2 + 1);
-    }
+    if (threadIdx.x == 0)
+        s_last = __hip_atomic_fetch_add(done, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (uint32_t)(ns - 1);
     __syncthreads();
+    if (!s_last) return;
+    // Each thread merges one output element: the (max, sum, value) triples of eight splits are
+    // requested together (one memory round trip per eight splits), and groups of eight are
+    // combined with a running maximum.
     for (int idx = threadIdx.x; idx < G * D; idx += kAttnThreads) {
         const int h = idx / D, e = idx % D;
-        const float *po = a.part_o + ((size_t)b * a.hq + kvh * G + h) * a.splits * D + e;
-        float m = -INFINITY;
-        for (int sp = 0; sp < ns; sp++) m = fmaxf(m, wm[h * ns + sp]);
-        float num = 0.f, den = 0.f;
+        const size_t row0 = ((size_t)b * a.hq + kvh * G + h) * a.splits;
+        float m = -INFINITY, num = 0.f, den = 0.f;
         for (int sp0 = 0; sp0 < ns; sp0 += 8) {
-            float v[8];
+            float pm[8], pl[8], pv[8];
 #pragma unroll
-            for (int k = 0; k < 8; k++) v[k] = coherent_load(po + (size_t)min(sp0 + k, ns - 1) * D);
+            for (int k = 0; k < 8; k++) {
+                const size_t row = row0 + min(sp0 + k, ns - 1);
+                pm[k] = coherent_load(a.part_ml + row * 2);
+                pl[k] = coherent_load(a.part_ml + row * 2 + 1);
+                pv[k] = coherent_load(a.part_o + row * D + e);
+            }
+            float mc = m;
+#pragma unroll
+            for (int k = 0; k < 8; k++) mc = fmaxf(mc, pm[k]); // a repeated last split does not change the max
+            const float f = __builtin_amdgcn_exp2f(m - mc);      // 0 on the first group (m = -inf)
+            num *= f;
+            den *= f;
 #pragma unroll
             for (int k = 0; k < 8; k++)
                 if (sp0 + k < ns) {
-                    const float w = __builtin_amdgcn_exp2f(wm[h * ns + sp0 + k] - m);
-                    num += w * v[k];
-                    den += w * wl[h * ns + sp0 + k];
+                    const float w = __builtin_amdgcn_exp2f(pm[k] - mc);
+                    num += w * pv[k];
+                    den += w * pl[k];
                 }
+            m = mc;
         }
         const float r = num / den;
         const size_t oi = ((size_t)b * a.hq + kvh * G + h) * D + e;
         if (a.out_f16) reinterpret_cast<__half *>(a.out)[oi] = __float2half_rn(r);
         else reinterpret_cast<float *>(a.out)[oi] = r;
     }
-    if (ns > 1 && threadIdx.x == 0) // ready for the next call on this stream
+    if (threadIdx.x == 0) // ready for the next call on this stream
         __hip_atomic_store(done, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 

@@ -90,7 +90,13 @@ __device__ __forceinline__ uint32_t select_u32(bool c, uint32_t yes, uint32_t no
 // at 3 waves per SIMD (without the bound the allocator takes 176 VGPRs and drops to 2).
 template <int S> __global__ __launch_bounds__(kDwThreads, (S == 2 ? 3 : 1)) void dw3x3_kernel(const DwArgs a) {
     constexpr int NCOL = (kDwCols - 1) * S + 3;
-    const uint32_t gid = blockIdx.x * kDwThreads + threadIdx.x;
+    // Workgroups are dealt to the 8 XCDs round-robin, each XCD with an L2 of its own.  Renumber them
+    // so that every XCD works on one contiguous run of the tensor: vertically adjacent row chunks,
+    // which share two input rows, then meet in the same L2 instead of being fetched once per XCD.
+    const uint32_t nblk = gridDim.x, per = nblk >> 3, rem = nblk & 7u;
+    const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3;
+    const uint32_t blk = xcd * per + min(xcd, rem) + slot;
+    const uint32_t gid = blk * kDwThreads + threadIdx.x;
     if (gid >= (uint32_t)a.total) return;
     // gid -> (image, row chunk, strip, channel quad), channel quad fastest
     uint32_t t = gid;
