@@ -279,6 +279,13 @@ def main():
         ctx.sync()
         b1_ms = (time.perf_counter() - t1) / args.batch1_steps * 1e3
         b1 = {"ms_per_image": round(b1_ms, 4), "images_per_s": round(1e3 / b1_ms, 1)}
+        # the batched run must give image 0 the very logits it gets alone (integer arithmetic: bit-exact);
+        # the batch-1 graph is the one the GPU tests follow tensor by tensor against the CPU oracle
+        model.invoke()
+        ctx.sync()
+        if not np.array_equal(model.output()[:1].view(np.uint32), m1.output().view(np.uint32)):
+            sys.exit("bench.py: batch-%d logits of image 0 differ from its batch-1 logits" % args.batch)
+        b1["batch_consistent"] = True
 
     # ---- CPU baseline: the CPU target's float chain, 1 thread, bounded sample -------------------
     cpu = None

@@ -185,10 +185,6 @@ template <int S> __global__ __launch_bounds__(kDwThreads, (S == 2 ? 3 : 1)) void
         for (int b = 0; b < 3; b++) unpack_row(b, raw[b], ok[b]);
     }
     const int nrows = min(a.rows, a.out_h - oy0); // >= 1
-    if (nrows > 1) {
-#pragma unroll
-        for (int nr = 0; nr < S; nr++) fetch_row(pre[nr], pre_ok[nr]);
-    }
     for (int t0 = 0; t0 < nrows; t0 += 3) {
 #pragma unroll
         for (int ph = 0; ph < 3; ph++) {

@@ -130,6 +130,21 @@ def test_mobilenet_stem_fc_and_depthwise_shapes(hip_ctx):
         run_case(hip_ctx, 2, c, hw, hw, c, 3, 3, (s, s), pad, (1, 1), c, seed=c + s)
 
 
+# Large launches make the depthwise kernel walk strips of several output rows per thread (the strip
+# length grows with the number of waves per SIMD); small shapes only ever take one-row strips.  On a
+# 256-CU device these shapes give strips of 7, 8, 7, 2, 4, 2, 4 (MobileNetV2's depthwise layers at batch
+# 64), then 5, and 8 / 4 / 2 with a ragged last strip, for stride 1 and 2.
+DW_LARGE = [(64, 32, 112, 1), (64, 96, 112, 2), (64, 144, 56, 1), (64, 144, 56, 2), (64, 192, 28, 1), (64, 384, 14, 1),
+            (64, 576, 14, 1), (64, 960, 7, 1), (48, 144, 75, 1), (32, 96, 75, 1), (64, 144, 30, 1), (32, 96, 37, 1),
+            (64, 96, 75, 2), (96, 144, 37, 2)]
+
+
+@pytest.mark.parametrize("n,c,hw,s", DW_LARGE)
+def test_depthwise_multi_row_strips_at_full_batch(hip_ctx, n, c, hw, s):
+    pad = ((1, 1), (1, 1)) if s == 1 else ((0, 1), (0, 1))
+    run_case(hip_ctx, n, c, hw, hw, c, 3, 3, (s, s), pad, (1, 1), c, seed=n + c + hw + s, modes=("u8", "i32"))
+
+
 def test_large_reduction_stages_weights_through_lds_in_chunks(hip_ctx):
     # 3x3 over 256 channels: K = 2304 (36 k-steps) -> weights staged in several LDS chunks
     run_case(hip_ctx, 1, 256, 10, 10, 64, 3, 3, (1, 1), ((1, 1), (1, 1)), (1, 1), 1, seed=3, modes=("u8", "i32"))

@@ -73,6 +73,35 @@ def test_mobilenetv2_config3(hip_ctx):
     assert np.array_equal(m1.run(x[:1]).view(np.uint32), y[:1].view(np.uint32))
 
 
+def test_mobilenetv2_batch64_equals_small_batches(hip_ctx):
+    """The headline configuration (batch 64) picks other tilings and strip lengths than the small batches
+    the oracle can follow: every tensor of the batch-64 run must equal, image by image, what a batch-4 run
+    of the same images gives (integer arithmetic: bit-exact), and image 0 must equal the oracle's logits."""
+    g = nb.mobilenet_v2(seed=2)
+    rng = np.random.default_rng(3)
+    qg = nb.quantize_graph(g, rng.random((32, 224, 224, 3), dtype=f32))
+    x = np.random.default_rng(4).random((64, 224, 224, 3), dtype=f32)
+    for fuse in (False, True):
+        big = nb.HipModel(hip_ctx, qg, 64, capture_graph=True, fuse_residual=fuse)
+        y = big.run(x)
+        smalls = []
+        for lo in (0, 60):
+            small = nb.HipModel(hip_ctx, qg, 4, capture_graph=False, fuse_residual=fuse)
+            ys = small.run(x[lo:lo + 4])
+            assert np.array_equal(ys.view(np.uint32), y[lo:lo + 4].view(np.uint32))
+            smalls.append((lo, small))
+        for i in range(len(qg.nodes)):
+            if not big.materialized(i):
+                continue
+            whole = big.tensor(i)
+            for lo, small in smalls:
+                a, b = whole[lo:lo + 4], small.tensor(i)
+                assert np.array_equal(a, b), f"node {i} ({qg.nodes[i].name}), images {lo}..{lo + 3}: {(a != b).sum()} bytes differ"
+    want = netref.run_integer(qg, x[:1])
+    want = want[0] if isinstance(want, tuple) else want
+    assert np.array_equal(y[:1].view(np.uint32), np.asarray(want).view(np.uint32))
+
+
 def test_profile_and_kernel_names(hip_ctx):
     g = nb.conv_block(seed=1)
     rng = np.random.default_rng(1)
