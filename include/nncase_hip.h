@@ -207,6 +207,50 @@ NNCASE_HIP_API int nncase_hip_qglobal_avgpool(nncase_hip_ctx_t *ctx, const uint8
                                               int32_t batch, int32_t h, int32_t w, int32_t channels,
                                               nncase_hip_quant_param_t x_qp, nncase_hip_quant_param_t y_qp);
 
+/* u8 -> u8 operators between Dequantize and Quantize as 256-entry byte tables:
+ * table[v] = Q_y(f(DQ_x(v))), evaluated on the host with the CPU kernels' fp32
+ * operations (dequantize.cpp:36-39, quantize.cpp:36-43).
+ *   NNCASE_HIP_LUT_REQUANT  f(x) = x: the Quantize(Dequantize(.)) pair a graph
+ *                           holds where tensors of different quant params meet
+ *   NNCASE_HIP_LUT_SWISH    f(x) = x / (1 + exp(-x)), unary swish
+ *                           (src/Native/src/kernels/stackvm/reference/activation.cpp:36)
+ * nncase_hip_make_unary_lut is host-only; nncase_hip_lut_u8 applies a table to
+ * `count` bytes on the device. */
+#define NNCASE_HIP_LUT_REQUANT 0
+#define NNCASE_HIP_LUT_SWISH 1
+NNCASE_HIP_API int nncase_hip_make_unary_lut(int32_t kind, nncase_hip_quant_param_t x_qp, nncase_hip_quant_param_t y_qp,
+                                             uint8_t *lut256_host);
+NNCASE_HIP_API int nncase_hip_lut_u8(nncase_hip_ctx_t *ctx, const uint8_t *in_dev, uint8_t *out_dev, size_t count,
+                                     const uint8_t *lut256_host);
+
+/* Concat along the channel axis of NHWC u8 tensors (kernels::stackvm::concat,
+ * src/Native/src/kernels/stackvm/tensor_ops.cpp, on the innermost axis) with
+ * every input requantised to the output's quant params, i.e. the
+ * Dequantize -> Concat -> Quantize sub-graph of a u8/u8 model:
+ *   out[p, off_i + c] = Q_out(DQ_i(in_i[p, c])),  off_i = channels_0 + .. + channels_{i-1}. */
+#define NNCASE_HIP_MAX_CONCAT 8
+NNCASE_HIP_API int nncase_hip_qconcat_channels(nncase_hip_ctx_t *ctx, int32_t n_inputs, const uint8_t *const *in_dev,
+                                               const int32_t *channels, const nncase_hip_quant_param_t *in_qps,
+                                               uint8_t *out_dev, nncase_hip_quant_param_t out_qp, int64_t pixels);
+
+/* resize_image(nearest_neighbor) on an NHWC tensor of 1/2/4-byte elements
+ * (kernels::stackvm::resize_image, tensor_ops.cpp:888-932;
+ * reference/resize_image.cpp:91-139).  Mode values are the reference's
+ * image_resize_transformation_mode_t / image_resize_nearest_mode_t
+ * (src/Native/include/nncase/runtime/stackvm/opcode.h:330-343). */
+#define NNCASE_HIP_RESIZE_HALF_PIXEL 0
+#define NNCASE_HIP_RESIZE_PYTORCH_HALF_PIXEL 1
+#define NNCASE_HIP_RESIZE_ALIGN_CORNERS 2
+#define NNCASE_HIP_RESIZE_ASYMMETRIC 3
+#define NNCASE_HIP_RESIZE_TFCROP_AND_RESIZE 4
+#define NNCASE_HIP_NEAREST_ROUND_PREFER_FLOOR 0
+#define NNCASE_HIP_NEAREST_ROUND_PREFER_CEIL 1
+#define NNCASE_HIP_NEAREST_FLOOR 2
+#define NNCASE_HIP_NEAREST_CEIL 3
+NNCASE_HIP_API int nncase_hip_resize_nearest(nncase_hip_ctx_t *ctx, const void *in_dev, void *out_dev, int32_t elem_size,
+                                             int32_t batch, int32_t in_h, int32_t in_w, int32_t channels, int32_t out_h,
+                                             int32_t out_w, int32_t transformation_mode, int32_t nearest_mode);
+
 /* ---- pack / unpack ------------------------------------------------------
  * pack: every listed axis a (extent D) becomes an outer axis of extent
  * ceil(D / lanes) in place and its lane index is appended as a trailing axis
@@ -289,6 +333,16 @@ NNCASE_HIP_API int nncase_hip_function_add_qglobal_avgpool(nncase_hip_function_t
                                                            uint8_t *out_dev, int32_t batch, int32_t h, int32_t w,
                                                            int32_t channels, nncase_hip_quant_param_t x_qp,
                                                            nncase_hip_quant_param_t y_qp);
+NNCASE_HIP_API int nncase_hip_function_add_lut_u8(nncase_hip_function_t *fn, const uint8_t *in_dev, uint8_t *out_dev,
+                                                  size_t count, const uint8_t *lut256_host);
+NNCASE_HIP_API int nncase_hip_function_add_qconcat_channels(nncase_hip_function_t *fn, int32_t n_inputs,
+                                                            const uint8_t *const *in_dev, const int32_t *channels,
+                                                            const nncase_hip_quant_param_t *in_qps, uint8_t *out_dev,
+                                                            nncase_hip_quant_param_t out_qp, int64_t pixels);
+NNCASE_HIP_API int nncase_hip_function_add_resize_nearest(nncase_hip_function_t *fn, const void *in_dev, void *out_dev,
+                                                          int32_t elem_size, int32_t batch, int32_t in_h, int32_t in_w,
+                                                          int32_t channels, int32_t out_h, int32_t out_w,
+                                                          int32_t transformation_mode, int32_t nearest_mode);
 /* Number of operators recorded so far. */
 NNCASE_HIP_API int nncase_hip_function_size(nncase_hip_function_t *fn, int32_t *count);
 /* Enqueues the whole function (graph replay if captured). */

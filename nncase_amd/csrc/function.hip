@@ -8,7 +8,7 @@
 namespace {
 
 struct Op {
-    enum Kind { kQuantize, kDequantize, kConv, kAdd, kPool } kind;
+    enum Kind { kQuantize, kDequantize, kConv, kAdd, kPool, kLut, kConcat, kResize } kind;
     const void *in0 = nullptr, *in1 = nullptr;
     void *out = nullptr;
     const nncase_hip_weights_t *weights = nullptr;
@@ -18,6 +18,14 @@ struct Op {
     size_t count = 0;
     float lo = 0.f, hi = 0.f;
     int32_t batch = 0, h = 0, w = 0, channels = 0;
+    // byte table / concat / resize
+    uint8_t lut[256] = {0};
+    int32_t n_inputs = 0;
+    const uint8_t *cat_in[NNCASE_HIP_MAX_CONCAT] = {nullptr};
+    int32_t cat_channels[NNCASE_HIP_MAX_CONCAT] = {0};
+    nncase_hip_quant_param_t cat_qp[NNCASE_HIP_MAX_CONCAT] = {};
+    int64_t pixels = 0;
+    int32_t elem_size = 0, out_h = 0, out_w = 0, tmode = 0, nmode = 0;
 };
 
 } // namespace
@@ -46,6 +54,14 @@ static int run_op(nncase_hip_function *fn, const Op &op) {
     case Op::kPool:
         return nncase_hip_qglobal_avgpool(ctx, (const uint8_t *)op.in0, (uint8_t *)op.out, op.batch, op.h, op.w,
                                           op.channels, op.qp0, op.qp1);
+    case Op::kLut:
+        return nncase_hip_lut_u8(ctx, (const uint8_t *)op.in0, (uint8_t *)op.out, op.count, op.lut);
+    case Op::kConcat:
+        return nncase_hip_qconcat_channels(ctx, op.n_inputs, op.cat_in, op.cat_channels, op.cat_qp, (uint8_t *)op.out,
+                                           op.qp0, op.pixels);
+    case Op::kResize:
+        return nncase_hip_resize_nearest(ctx, op.in0, op.out, op.elem_size, op.batch, op.h, op.w, op.channels, op.out_h,
+                                         op.out_w, op.tmode, op.nmode);
     }
     return -EINVAL;
 }
@@ -136,6 +152,44 @@ extern "C" int nncase_hip_function_add_qglobal_avgpool(nncase_hip_function_t *fn
     return push(fn, op);
 }
 
+extern "C" int nncase_hip_function_add_lut_u8(nncase_hip_function_t *fn, const uint8_t *in_dev, uint8_t *out_dev,
+                                              size_t count, const uint8_t *lut256_host) {
+    if (!fn) return -EINVAL;
+    NNHIP_REQUIRE(fn->ctx, in_dev && out_dev && lut256_host, -EINVAL, "function_add_lut_u8: null argument");
+    Op op;
+    op.kind = Op::kLut;
+    op.in0 = in_dev, op.out = out_dev, op.count = count;
+    memcpy(op.lut, lut256_host, 256);
+    return push(fn, op);
+}
+
+extern "C" int nncase_hip_function_add_qconcat_channels(nncase_hip_function_t *fn, int32_t n_inputs,
+                                                        const uint8_t *const *in_dev, const int32_t *channels,
+                                                        const nncase_hip_quant_param_t *in_qps, uint8_t *out_dev,
+                                                        nncase_hip_quant_param_t out_qp, int64_t pixels) {
+    if (!fn) return -EINVAL;
+    NNHIP_REQUIRE(fn->ctx, n_inputs > 0 && n_inputs <= NNCASE_HIP_MAX_CONCAT && in_dev && channels && in_qps && out_dev,
+                  -EINVAL, "function_add_qconcat_channels: bad argument (1..%d inputs)", NNCASE_HIP_MAX_CONCAT);
+    Op op;
+    op.kind = Op::kConcat;
+    op.n_inputs = n_inputs, op.out = out_dev, op.qp0 = out_qp, op.pixels = pixels;
+    for (int i = 0; i < n_inputs; i++) op.cat_in[i] = in_dev[i], op.cat_channels[i] = channels[i], op.cat_qp[i] = in_qps[i];
+    return push(fn, op);
+}
+
+extern "C" int nncase_hip_function_add_resize_nearest(nncase_hip_function_t *fn, const void *in_dev, void *out_dev,
+                                                      int32_t elem_size, int32_t batch, int32_t in_h, int32_t in_w,
+                                                      int32_t channels, int32_t out_h, int32_t out_w,
+                                                      int32_t transformation_mode, int32_t nearest_mode) {
+    if (!fn) return -EINVAL;
+    NNHIP_REQUIRE(fn->ctx, in_dev && out_dev, -EINVAL, "function_add_resize_nearest: null buffer");
+    Op op;
+    op.kind = Op::kResize;
+    op.in0 = in_dev, op.out = out_dev, op.elem_size = elem_size, op.batch = batch, op.h = in_h, op.w = in_w;
+    op.channels = channels, op.out_h = out_h, op.out_w = out_w, op.tmode = transformation_mode, op.nmode = nearest_mode;
+    return push(fn, op);
+}
+
 extern "C" int nncase_hip_function_size(nncase_hip_function_t *fn, int32_t *count) {
     if (!fn || !count) return -EINVAL;
     *count = (int32_t)fn->ops.size();
@@ -200,6 +254,9 @@ extern "C" int nncase_hip_function_op_kernel(nncase_hip_function_t *fn, int32_t 
     case Op::kConv: describe_conv_kernel(fn->ctx, op.weights, &op.conv, name, capacity); break;
     case Op::kAdd: snprintf(name, capacity, "qadd"); break;
     case Op::kPool: snprintf(name, capacity, "qglobal_avgpool"); break;
+    case Op::kLut: snprintf(name, capacity, "lut_u8"); break;
+    case Op::kConcat: snprintf(name, capacity, "qconcat<%d>", op.n_inputs); break;
+    case Op::kResize: snprintf(name, capacity, "resize_nearest"); break;
     }
     return 0;
 }

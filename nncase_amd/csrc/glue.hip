@@ -1,0 +1,242 @@
+// u8 glue operators that keep a quantized graph resident on the device between the
+// convolutions: byte-table unary operators (requantisation, swish), channel concat with
+// requantisation to a common scale, nearest-neighbour resize.  All are bound by HBM
+// bandwidth; the arithmetic that decides a byte is done once per table entry on the host
+// (256 evaluations with the same fp32 operations the CPU kernels use), so the device only
+// moves bytes and the result is bit-exact by construction.
+#include "common.hpp"
+
+#include <cmath>
+
+namespace nnhip {
+
+constexpr int kGlueThreads = 256;
+
+struct ByteTable {
+    uint32_t w[64]; // 256 entries, little-endian packed
+};
+
+__device__ __forceinline__ uint32_t lut4(const uint8_t *t, uint32_t v) {
+    return (uint32_t)t[v & 0xffu] | ((uint32_t)t[(v >> 8) & 0xffu] << 8) | ((uint32_t)t[(v >> 16) & 0xffu] << 16) |
+           ((uint32_t)t[v >> 24] << 24);
+}
+
+__device__ __forceinline__ void stage_table(uint8_t *t, const ByteTable &lut) {
+    if (threadIdx.x < 64) reinterpret_cast<uint32_t *>(t)[threadIdx.x] = lut.w[threadIdx.x];
+    __syncthreads();
+}
+
+// out[i] = table[in[i]], 16 bytes per thread per step.
+__global__ __launch_bounds__(kGlueThreads) void lut_u8_kernel(const uint8_t *__restrict__ in, uint8_t *__restrict__ out,
+                                                             size_t count, const ByteTable lut, int vec_ok) {
+    __shared__ __align__(16) uint8_t t[256];
+    stage_table(t, lut);
+    const size_t tid = (size_t)blockIdx.x * kGlueThreads + threadIdx.x;
+    const size_t nthreads = (size_t)gridDim.x * kGlueThreads;
+    const size_t nvec = vec_ok ? count / 16 : 0;
+    for (size_t i = tid; i < nvec; i += nthreads) {
+        const uint4 v = *reinterpret_cast<const uint4 *>(in + i * 16);
+        *reinterpret_cast<uint4 *>(out + i * 16) = uint4{lut4(t, v.x), lut4(t, v.y), lut4(t, v.z), lut4(t, v.w)};
+    }
+    for (size_t j = nvec * 16 + tid; j < count; j += nthreads) out[j] = t[in[j]];
+}
+
+// One input of a channel concat: out[p, c_off + c] = table[in[p, c]] for c < c_in.
+// VEC = bytes per thread (4 when every channel count and offset is a multiple of 4).
+template <int VEC>
+__global__ __launch_bounds__(kGlueThreads) void concat_lut_kernel(const uint8_t *__restrict__ in, uint8_t *__restrict__ out,
+                                                                 uint32_t total, FastDiv d_cv, uint32_t c_in,
+                                                                 uint32_t c_out, uint32_t c_off, const ByteTable lut) {
+    __shared__ __align__(16) uint8_t t[256];
+    stage_table(t, lut);
+    const uint32_t gid = blockIdx.x * kGlueThreads + threadIdx.x;
+    if (gid >= total) return;
+    const uint32_t p = fastdiv(gid, d_cv);
+    const uint32_t c = (gid - p * d_cv.div) * VEC;
+    const size_t src = (size_t)p * c_in + c, dst = (size_t)p * c_out + c_off + c;
+    if (VEC == 4) *reinterpret_cast<uint32_t *>(out + dst) = lut4(t, *reinterpret_cast<const uint32_t *>(in + src));
+    else out[dst] = t[in[src]];
+}
+
+// Coordinate of an output index in the input (get_coordinate_from_resized,
+// src/Native/include/nncase/kernels/stackvm/resize_image.h:30-66) and the rounding to a pixel
+// (get_nearest_pixel_from_origin, :68-92): the same single fp32 operations in the same order.
+__device__ __forceinline__ float resize_coordinate(int mode, float x_resized, float x_scale, float length_resized,
+                                                   float length_original) {
+    switch (mode) {
+    case 3: return x_resized * x_scale;
+    case 1: return length_resized > 1 ? (x_resized + 0.5f) * x_scale - 0.5f : 0.0f;
+    case 2: return length_resized == 1 ? 0.f : x_resized * (length_original - 1) / (length_resized - 1);
+    case 4: return 0.f; // tfcrop_and_resize: the nearest kernel passes roi (0, 0), which maps every index to 0
+    default: return ((x_resized + 0.5f) * x_scale) - 0.5f;
+    }
+}
+
+__device__ __forceinline__ int resize_nearest_pixel(int mode, float x, int length) {
+    float r;
+    switch (mode) {
+    case 1: r = roundf(x); break;
+    case 2: r = floorf(x); break;
+    case 3: r = ceilf(x); break;
+    default: r = (x == truncf(x) + 0.5f) ? floorf(x) : roundf(x); break; // halves prefer the floor
+    }
+    // the reference clamps after the conversion to int64; clamping the float first gives the same index
+    r = fminf(fmaxf(r, 0.f), (float)(length - 1));
+    return (int)r;
+}
+
+struct ResizeArgs {
+    const uint8_t *in;
+    uint8_t *out;
+    int in_h, in_w, out_h, out_w;
+    uint32_t row_vecs; // vectors per pixel (channels * element size / VEC)
+    FastDiv d_vecs, d_ow, d_oh;
+    uint32_t total;
+    float h_scale, w_scale;
+    int tmode, nmode;
+};
+
+// NHWC: every output pixel copies the channel vector of its source pixel.
+template <typename V> __global__ __launch_bounds__(kGlueThreads) void resize_nearest_kernel(const ResizeArgs a) {
+    const uint32_t gid = blockIdx.x * kGlueThreads + threadIdx.x;
+    if (gid >= a.total) return;
+    uint32_t q = fastdiv(gid, a.d_vecs);
+    const uint32_t v = gid - q * a.d_vecs.div;
+    uint32_t t = q;
+    q = fastdiv(t, a.d_ow);
+    const int ox = (int)(t - q * a.d_ow.div);
+    t = q;
+    q = fastdiv(t, a.d_oh);
+    const int oy = (int)(t - q * a.d_oh.div);
+    const uint32_t n = q;
+    const int iy = resize_nearest_pixel(a.nmode, resize_coordinate(a.tmode, (float)oy, a.h_scale, (float)a.out_h, (float)a.in_h), a.in_h);
+    const int ix = resize_nearest_pixel(a.nmode, resize_coordinate(a.tmode, (float)ox, a.w_scale, (float)a.out_w, (float)a.in_w), a.in_w);
+    const size_t src = (((size_t)n * a.in_h + iy) * a.in_w + ix) * a.row_vecs + v;
+    reinterpret_cast<V *>(a.out)[gid] = reinterpret_cast<const V *>(a.in)[src];
+}
+
+inline ByteTable pack_table(const uint8_t *lut) {
+    ByteTable t;
+    memcpy(t.w, lut, 256);
+    return t;
+}
+
+} // namespace nnhip
+
+using namespace nnhip;
+
+extern "C" int nncase_hip_make_unary_lut(int32_t kind, nncase_hip_quant_param_t x_qp, nncase_hip_quant_param_t y_qp,
+                                         uint8_t *lut) {
+    if (!lut || (kind != NNCASE_HIP_LUT_REQUANT && kind != NNCASE_HIP_LUT_SWISH)) return -EINVAL;
+    if (!(y_qp.scale != 0.f)) return -EINVAL;
+    for (int v = 0; v < 256; v++) {
+        const float x = ((float)v - (float)x_qp.zero_point) * x_qp.scale;
+        float f = x;
+        if (kind == NNCASE_HIP_LUT_SWISH) f = x / (1 + expf(-x));
+        const float t = f / y_qp.scale + (float)y_qp.zero_point;
+        float r = nearbyintf(t); // round half to even (default rounding mode)
+        if (!(r >= 0.f)) r = 0.f; // also NaN
+        if (r > 255.f) r = 255.f;
+        lut[v] = (uint8_t)r;
+    }
+    return 0;
+}
+
+extern "C" int nncase_hip_lut_u8(nncase_hip_ctx_t *ctx, const uint8_t *in_dev, uint8_t *out_dev, size_t count,
+                                 const uint8_t *lut_host) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, lut_host, -EINVAL, "lut_u8: null table");
+    if (count == 0) return 0;
+    NNHIP_REQUIRE(ctx, in_dev && out_dev, -EINVAL, "lut_u8: null buffer");
+    const int vec_ok = ((reinterpret_cast<uintptr_t>(in_dev) | reinterpret_cast<uintptr_t>(out_dev)) & 15u) == 0;
+    const size_t vecs = (count + 15) / 16;
+    const size_t want = (vecs + kGlueThreads - 1) / kGlueThreads;
+    const size_t cap = (size_t)ctx->compute_units * 16;
+    const int grid = (int)(want < cap ? (want ? want : 1) : cap);
+    hipLaunchKernelGGL(lut_u8_kernel, dim3(grid), dim3(kGlueThreads), 0, ctx->stream, in_dev, out_dev, count,
+                       pack_table(lut_host), vec_ok);
+    NNHIP_LAUNCH_CHECK(ctx, "lut_u8_kernel");
+    return 0;
+}
+
+extern "C" int nncase_hip_qconcat_channels(nncase_hip_ctx_t *ctx, int32_t n_inputs, const uint8_t *const *in_dev,
+                                           const int32_t *channels, const nncase_hip_quant_param_t *in_qps,
+                                           uint8_t *out_dev, nncase_hip_quant_param_t out_qp, int64_t pixels) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, n_inputs > 0 && n_inputs <= NNCASE_HIP_MAX_CONCAT && in_dev && channels && in_qps && out_dev, -EINVAL,
+                  "qconcat_channels: bad argument (1..%d inputs)", NNCASE_HIP_MAX_CONCAT);
+    NNHIP_REQUIRE(ctx, pixels >= 0, -EINVAL, "qconcat_channels: negative pixel count");
+    NNHIP_REQUIRE(ctx, out_qp.scale != 0.f, -EINVAL, "qconcat_channels: output scale is zero");
+    int64_t c_out = 0;
+    bool vec = (reinterpret_cast<uintptr_t>(out_dev) & 3u) == 0;
+    for (int i = 0; i < n_inputs; i++) {
+        NNHIP_REQUIRE(ctx, channels[i] > 0 && in_dev[i], -EINVAL, "qconcat_channels: input %d is empty or null", i);
+        vec = vec && channels[i] % 4 == 0 && (reinterpret_cast<uintptr_t>(in_dev[i]) & 3u) == 0;
+        c_out += channels[i];
+    }
+    if (pixels == 0) return 0;
+    uint32_t c_off = 0;
+    for (int i = 0; i < n_inputs; i++) {
+        uint8_t lut[256];
+        const int rc = nncase_hip_make_unary_lut(NNCASE_HIP_LUT_REQUANT, in_qps[i], out_qp, lut);
+        NNHIP_REQUIRE(ctx, rc == 0, rc, "qconcat_channels: cannot build the requantisation table of input %d", i);
+        const int v = vec ? 4 : 1;
+        const int64_t total = pixels * (channels[i] / v);
+        NNHIP_REQUIRE(ctx, total < ((int64_t)1 << 31), -EINVAL, "qconcat_channels: input %d too large", i);
+        const FastDiv d_cv = make_fastdiv((uint32_t)(channels[i] / v));
+        const dim3 grid((unsigned)((total + kGlueThreads - 1) / kGlueThreads));
+        if (vec)
+            hipLaunchKernelGGL(concat_lut_kernel<4>, grid, dim3(kGlueThreads), 0, ctx->stream, in_dev[i], out_dev, (uint32_t)total,
+                               d_cv, (uint32_t)channels[i], (uint32_t)c_out, c_off, pack_table(lut));
+        else
+            hipLaunchKernelGGL(concat_lut_kernel<1>, grid, dim3(kGlueThreads), 0, ctx->stream, in_dev[i], out_dev, (uint32_t)total,
+                               d_cv, (uint32_t)channels[i], (uint32_t)c_out, c_off, pack_table(lut));
+        NNHIP_LAUNCH_CHECK(ctx, "concat_lut_kernel");
+        c_off += (uint32_t)channels[i];
+    }
+    return 0;
+}
+
+extern "C" int nncase_hip_resize_nearest(nncase_hip_ctx_t *ctx, const void *in_dev, void *out_dev, int32_t elem_size,
+                                         int32_t batch, int32_t in_h, int32_t in_w, int32_t channels, int32_t out_h,
+                                         int32_t out_w, int32_t transformation_mode, int32_t nearest_mode) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, in_dev && out_dev, -EINVAL, "resize_nearest: null buffer");
+    NNHIP_REQUIRE(ctx, elem_size == 1 || elem_size == 2 || elem_size == 4, -NNCASE_HIP_ERR_DATATYPE_MISMATCH,
+                  "resize_nearest: element size %d", elem_size);
+    NNHIP_REQUIRE(ctx, batch > 0 && in_h > 0 && in_w > 0 && channels > 0 && out_h > 0 && out_w > 0, -EINVAL,
+                  "resize_nearest: non-positive dimension");
+    NNHIP_REQUIRE(ctx, transformation_mode >= 0 && transformation_mode <= 4 && nearest_mode >= 0 && nearest_mode <= 3, -EINVAL,
+                  "resize_nearest: unknown mode (%d, %d)", transformation_mode, nearest_mode);
+    NNHIP_REQUIRE(ctx, in_h < (1 << 24) && in_w < (1 << 24) && out_h < (1 << 24) && out_w < (1 << 24), -EINVAL,
+                  "resize_nearest: extent beyond 2^24 (indices are computed in fp32, as in the CPU kernel)");
+    const int64_t row_bytes = (int64_t)channels * elem_size;
+    const uintptr_t addr = reinterpret_cast<uintptr_t>(in_dev) | reinterpret_cast<uintptr_t>(out_dev);
+    int vec = 1;
+    if (row_bytes % 16 == 0 && (addr & 15u) == 0) vec = 16;
+    else if (row_bytes % 4 == 0 && (addr & 3u) == 0) vec = 4;
+    ResizeArgs a;
+    a.in = (const uint8_t *)in_dev;
+    a.out = (uint8_t *)out_dev;
+    a.in_h = in_h, a.in_w = in_w, a.out_h = out_h, a.out_w = out_w;
+    a.row_vecs = (uint32_t)(row_bytes / vec);
+    const int64_t total = (int64_t)batch * out_h * out_w * a.row_vecs;
+    NNHIP_REQUIRE(ctx, total < ((int64_t)1 << 31), -EINVAL, "resize_nearest: too many work items");
+    a.total = (uint32_t)total;
+    a.d_vecs = make_fastdiv(a.row_vecs);
+    a.d_ow = make_fastdiv((uint32_t)out_w);
+    a.d_oh = make_fastdiv((uint32_t)out_h);
+    // get_resize_scales, src/Native/include/nncase/kernels/kernel_utils.h:224-233
+    const bool align = transformation_mode == 2;
+    a.h_scale = (float)in_h / out_h;
+    a.w_scale = (float)in_w / out_w;
+    if (align && out_h > 1) a.h_scale = (float)(in_h - 1) / (out_h - 1);
+    if (align && out_w > 1) a.w_scale = (float)(in_w - 1) / (out_w - 1);
+    a.tmode = transformation_mode, a.nmode = nearest_mode;
+    const dim3 grid((unsigned)((total + kGlueThreads - 1) / kGlueThreads));
+    if (vec == 16) hipLaunchKernelGGL(resize_nearest_kernel<uint4>, grid, dim3(kGlueThreads), 0, ctx->stream, a);
+    else if (vec == 4) hipLaunchKernelGGL(resize_nearest_kernel<uint32_t>, grid, dim3(kGlueThreads), 0, ctx->stream, a);
+    else hipLaunchKernelGGL(resize_nearest_kernel<uint8_t>, grid, dim3(kGlueThreads), 0, ctx->stream, a);
+    NNHIP_LAUNCH_CHECK(ctx, "resize_nearest_kernel");
+    return 0;
+}

@@ -158,6 +158,59 @@ def global_average_pool(input: np.ndarray, input_qp: QuantParam, output_qp: Quan
     return dy.download((n, ch, 1, 1), np.uint8)
 
 
+def _to_nhwc_dev(c, x: np.ndarray):
+    n, ch, h, w = x.shape
+    d_nchw, d_nhwc = c.to_device(x), c.alloc(max(1, x.nbytes))
+    c.nchw_to_nhwc(d_nchw, d_nhwc, x.itemsize, n, ch, h, w)
+    return d_nhwc
+
+
+def _from_nhwc_dev(c, d_nhwc, shape_nchw, dtype) -> np.ndarray:
+    n, ch, h, w = shape_nchw
+    dtype = np.dtype(dtype)
+    d_nchw = c.alloc(max(1, int(np.prod(shape_nchw)) * dtype.itemsize))
+    c.nhwc_to_nchw(d_nhwc, d_nchw, dtype.itemsize, n, ch, h, w)
+    return d_nchw.download(tuple(shape_nchw), dtype)
+
+
+def unary_u8(kind: int, input: np.ndarray, input_qp: QuantParam, output_qp: QuantParam, ctx: Context = None) -> np.ndarray:
+    """Quantize(unary(Dequantize(x))) on u8 data of any shape as one byte-table pass;
+    kind = runtime.LUT_REQUANT (identity) or runtime.LUT_SWISH (kernels::stackvm::unary swish)."""
+    c = _ctx(ctx)
+    x = np.ascontiguousarray(input, np.uint8)
+    lut = rt.make_unary_lut(kind, input_qp, output_qp)
+    src, dst = c.to_device(x), c.alloc(max(1, x.size))
+    c.lut_u8(src, dst, x.size, lut)
+    return dst.download(x.shape, np.uint8)
+
+
+def concat(inputs: Sequence[np.ndarray], input_qps: Sequence[QuantParam], output_qp: QuantParam, ctx: Context = None) -> np.ndarray:
+    """kernels::stackvm::concat on axis 1 of u8 NCHW tensors, every input requantised to output_qp."""
+    c = _ctx(ctx)
+    xs = [np.ascontiguousarray(x, np.uint8) for x in inputs]
+    n, _, h, w = xs[0].shape
+    for x in xs:
+        if x.ndim != 4 or (x.shape[0], x.shape[2], x.shape[3]) != (n, h, w):
+            raise rt.HipError(-rt.ERR_SHAPE_MISMATCH, "concat", f"{[x.shape for x in xs]}")
+    chans = [x.shape[1] for x in xs]
+    devs = [_to_nhwc_dev(c, x) for x in xs]
+    out = c.alloc(max(1, n * h * w * sum(chans)))
+    c.qconcat_channels(devs, chans, list(input_qps), out, output_qp, n * h * w)
+    return _from_nhwc_dev(c, out, (n, sum(chans), h, w), np.uint8)
+
+
+def resize_image_nearest(input: np.ndarray, out_h: int, out_w: int, transformation_mode: int = rt.RESIZE_HALF_PIXEL,
+                         nearest_mode: int = rt.NEAREST_ROUND_PREFER_FLOOR, ctx: Context = None) -> np.ndarray:
+    """kernels::stackvm::resize_image(nearest_neighbor) on an NCHW tensor with 1/2/4-byte elements."""
+    c = _ctx(ctx)
+    x = np.ascontiguousarray(input)
+    n, ch, h, w = x.shape
+    src = _to_nhwc_dev(c, x)
+    dst = c.alloc(max(1, n * ch * out_h * out_w * x.itemsize))
+    c.resize_nearest(src, dst, x.itemsize, n, h, w, ch, out_h, out_w, transformation_mode, nearest_mode)
+    return _from_nhwc_dev(c, dst, (n, ch, out_h, out_w), x.dtype)
+
+
 def pack(input: np.ndarray, axes: Sequence[int], lanes: Sequence[int], ctx: Context = None) -> np.ndarray:
     c = _ctx(ctx)
     x = np.ascontiguousarray(input)

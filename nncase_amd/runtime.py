@@ -89,6 +89,15 @@ SYMBOLS = {
     "nncase_hip_qadd": (_I, [_VP, _VP, QuantParam, _VP, QuantParam, _VP, QuantParam, C.c_float, C.c_float, _SZ]),
     "nncase_hip_qglobal_avgpool": (_I, [_VP, _VP, _VP, C.c_int32, C.c_int32, C.c_int32, C.c_int32, QuantParam,
                                         QuantParam]),
+    "nncase_hip_make_unary_lut": (_I, [C.c_int32, QuantParam, QuantParam, _VP]),
+    "nncase_hip_lut_u8": (_I, [_VP, _VP, _VP, _SZ, _VP]),
+    "nncase_hip_qconcat_channels": (_I, [_VP, C.c_int32, C.POINTER(_VP), _I32P, C.POINTER(QuantParam), _VP, QuantParam,
+                                         C.c_int64]),
+    "nncase_hip_resize_nearest": (_I, [_VP, _VP, _VP] + [C.c_int32] * 9),
+    "nncase_hip_function_add_lut_u8": (_I, [_VP, _VP, _VP, _SZ, _VP]),
+    "nncase_hip_function_add_qconcat_channels": (_I, [_VP, C.c_int32, C.POINTER(_VP), _I32P, C.POINTER(QuantParam), _VP,
+                                                      QuantParam, C.c_int64]),
+    "nncase_hip_function_add_resize_nearest": (_I, [_VP, _VP, _VP] + [C.c_int32] * 9),
     "nncase_hip_pack": (_I, [_VP, _VP, _VP, C.c_int32, C.c_int32, _I32P, C.c_int32, _I32P, _I32P]),
     "nncase_hip_unpack": (_I, [_VP, _VP, _VP, C.c_int32, C.c_int32, _I32P, C.c_int32, _I32P, _I32P]),
     "nncase_hip_nchw_to_nhwc": (_I, [_VP, _VP, _VP, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
@@ -141,6 +150,28 @@ class HipError(RuntimeError):
 
 def qp(zero_point: int, scale: float) -> QuantParam:
     return QuantParam(int(zero_point), float(np.float32(scale)))
+
+
+LUT_REQUANT, LUT_SWISH = 0, 1
+RESIZE_HALF_PIXEL, RESIZE_PYTORCH_HALF_PIXEL, RESIZE_ALIGN_CORNERS, RESIZE_ASYMMETRIC, RESIZE_TFCROP_AND_RESIZE = range(5)
+NEAREST_ROUND_PREFER_FLOOR, NEAREST_ROUND_PREFER_CEIL, NEAREST_FLOOR, NEAREST_CEIL = range(4)
+
+
+def make_unary_lut(kind: int, x_qp: "QuantParam", y_qp: "QuantParam") -> np.ndarray:
+    """Host-side 256-entry table lut[v] = Q_y(f(DQ_x(v))) built by the library (same libm as the CPU kernels)."""
+    lut = np.empty(256, np.uint8)
+    rc = load_library().nncase_hip_make_unary_lut(kind, x_qp, y_qp, lut.ctypes.data)
+    if rc != 0:
+        raise HipError(rc, "make_unary_lut", "invalid kind or zero output scale")
+    return lut
+
+
+def _concat_args(inputs, channels, in_qps):
+    n = len(inputs)
+    ptrs = (_VP * n)(*[b.ptr for b in inputs])
+    ch = (C.c_int32 * n)(*channels)
+    qps = (QuantParam * n)(*in_qps)
+    return n, ptrs, ch, qps
 
 
 class DeviceBuffer:
@@ -301,6 +332,22 @@ class Context:
         self._check(self.lib.nncase_hip_qglobal_avgpool(self.handle, x.ptr, out.ptr, batch, h, w, channels, x_qp, y_qp),
                     "qglobal_avgpool")
 
+    def lut_u8(self, src: DeviceBuffer, dst: DeviceBuffer, count: int, lut: np.ndarray):
+        t = np.ascontiguousarray(lut, np.uint8)
+        assert t.size == 256
+        self._check(self.lib.nncase_hip_lut_u8(self.handle, src.ptr, dst.ptr, count, t.ctypes.data), "lut_u8")
+
+    def qconcat_channels(self, inputs: Sequence[DeviceBuffer], channels: Sequence[int], in_qps, out: DeviceBuffer, out_qp,
+                         pixels: int):
+        n, ptrs, ch, qps = _concat_args(inputs, channels, in_qps)
+        self._check(self.lib.nncase_hip_qconcat_channels(self.handle, n, ptrs, ch, qps, out.ptr, out_qp, pixels),
+                    "qconcat_channels")
+
+    def resize_nearest(self, src: DeviceBuffer, dst: DeviceBuffer, elem_size, batch, in_h, in_w, channels, out_h, out_w,
+                       transformation_mode=0, nearest_mode=0):
+        self._check(self.lib.nncase_hip_resize_nearest(self.handle, src.ptr, dst.ptr, elem_size, batch, in_h, in_w, channels,
+                                                       out_h, out_w, transformation_mode, nearest_mode), "resize_nearest")
+
     def pack(self, src: DeviceBuffer, dst: DeviceBuffer, elem_size: int, shape: Sequence[int], axes: Sequence[int],
              lanes: Sequence[int]):
         sh, ax, ln = (C.c_int32 * len(shape))(*shape), (C.c_int32 * max(1, len(axes)))(*axes), (C.c_int32 * max(1, len(lanes)))(*lanes)
@@ -362,6 +409,26 @@ class Function:
         self._keep += [x, out]
         self._ck(self.ctx.lib.nncase_hip_function_add_qglobal_avgpool(self.handle, x.ptr, out.ptr, batch, h, w, channels,
                                                                      x_qp, y_qp), "function_add_qglobal_avgpool")
+
+    def add_lut_u8(self, src, dst, count, lut):
+        self._keep += [src, dst]
+        t = np.ascontiguousarray(lut, np.uint8)
+        assert t.size == 256
+        self._ck(self.ctx.lib.nncase_hip_function_add_lut_u8(self.handle, src.ptr, dst.ptr, count, t.ctypes.data),
+                 "function_add_lut_u8")
+
+    def add_qconcat_channels(self, inputs, channels, in_qps, out, out_qp, pixels):
+        self._keep += list(inputs) + [out]
+        n, ptrs, ch, qps = _concat_args(inputs, channels, in_qps)
+        self._ck(self.ctx.lib.nncase_hip_function_add_qconcat_channels(self.handle, n, ptrs, ch, qps, out.ptr, out_qp, pixels),
+                 "function_add_qconcat_channels")
+
+    def add_resize_nearest(self, src, dst, elem_size, batch, in_h, in_w, channels, out_h, out_w, transformation_mode=0,
+                           nearest_mode=0):
+        self._keep += [src, dst]
+        self._ck(self.ctx.lib.nncase_hip_function_add_resize_nearest(self.handle, src.ptr, dst.ptr, elem_size, batch, in_h,
+                                                                     in_w, channels, out_h, out_w, transformation_mode,
+                                                                     nearest_mode), "function_add_resize_nearest")
 
     def __len__(self):
         n = C.c_int32()

@@ -548,6 +548,92 @@ ORACLE_API void q_global_avgpool_u8(const uint8_t *x, uint8_t *out, int32_t n,
         }
 }
 
+/* Byte tables for u8 -> u8 operators that sit between Dequantize and Quantize
+ * (the form a unary op takes in a u8/u8 graph): lut[v] = Q(f(DQ(v))).
+ * kind 0: identity (a pure requantisation, what Concat inserts when its
+ *         inputs carry different quant params);
+ * kind 1: swish / SiLU, x / (1 + exp(-x))
+ *         (src/Native/src/kernels/stackvm/reference/activation.cpp:36).       */
+ORACLE_API void q_unary_lut_u8(int32_t kind, int32_t zx, float sx, int32_t zy, float sy,
+                               uint8_t *lut) {
+    for (int v = 0; v < 256; v++) {
+        float x = ((float)v - (float)zx) * sx;
+        float f = x;
+        if (kind == 1) f = x / (1 + expf(-x));
+        float t = f / sy + (float)zy;
+        lut[v] = (uint8_t)clampi_ref(rne_sat_i32(t), 0, 255);
+    }
+}
+
+/* Nearest-neighbour resize of an NCHW tensor of `es`-byte elements
+ * (src/Native/src/kernels/stackvm/reference/resize_image.cpp:91-139; the
+ * coordinate and rounding functions of
+ * src/Native/include/nncase/kernels/stackvm/resize_image.h:30-92, scales from
+ * src/Native/include/nncase/kernels/kernel_utils.h:224-233).
+ * transformation_mode: 0 half_pixel, 1 pytorch_half_pixel, 2 align_corners,
+ * 3 asymmetric, 4 tfcrop_and_resize (the kernel passes roi 0, 0);
+ * nearest_mode: 0 round_prefer_floor, 1 round_prefer_ceil, 2 floor, 3 ceil.   */
+static float resize_coordinate(int32_t mode, float x_resized, float x_scale,
+                               float length_resized, float length_original) {
+    switch (mode) {
+    case 3: return x_resized * x_scale;
+    case 1: return length_resized > 1 ? (x_resized + 0.5f) * x_scale - 0.5f : 0.0f;
+    case 2:
+        return length_resized == 1 ? 0 : x_resized * (length_original - 1) / (length_resized - 1);
+    case 4: {
+        const float roi_start = 0, roi_end = 0;
+        double orig = length_resized > 1
+                          ? roi_start * (length_original - 1) +
+                                (x_resized * (roi_end - roi_start) * (length_original - 1)) /
+                                    (length_resized - 1)
+                          : 0.5 * (roi_start + roi_end) * (length_original - 1);
+        return (float)orig;
+    }
+    default: return ((x_resized + 0.5f) * x_scale) - 0.5f;
+    }
+}
+
+static int64_t resize_nearest_pixel(int32_t mode, float x_original) {
+    switch (mode) {
+    case 1: return (int64_t)roundf(x_original);
+    case 2: return (int64_t)floorf(x_original);
+    case 3: return (int64_t)ceilf(x_original);
+    default:
+        if (x_original == (int64_t)x_original + 0.5f) return (int64_t)floorf(x_original);
+        return (int64_t)roundf(x_original);
+    }
+}
+
+ORACLE_API void ref_resize_nearest(const uint8_t *in, uint8_t *out, int32_t es, int32_t n,
+                                   int32_t c, int32_t h, int32_t w, int32_t out_h,
+                                   int32_t out_w, int32_t transformation_mode,
+                                   int32_t nearest_mode) {
+    const int align_corners = transformation_mode == 2;
+    float height_scale = (float)h / out_h;
+    float width_scale = (float)w / out_w;
+    if (align_corners && out_h > 1) height_scale = (float)(h - 1) / (out_h - 1);
+    if (align_corners && out_w > 1) width_scale = (float)(w - 1) / (out_w - 1);
+    for (int32_t b = 0; b < n; b++)
+        for (int32_t oc = 0; oc < c; oc++)
+            for (int32_t oy = 0; oy < out_h; oy++) {
+                float iy = resize_coordinate(transformation_mode, (float)oy, height_scale,
+                                             (float)out_h, (float)h);
+                int64_t in_y = resize_nearest_pixel(nearest_mode, iy);
+                if (in_y < 0) in_y = 0;
+                if (in_y >= h) in_y = h - 1;
+                for (int32_t ox = 0; ox < out_w; ox++) {
+                    float ix = resize_coordinate(transformation_mode, (float)ox, width_scale,
+                                                 (float)out_w, (float)w);
+                    int64_t in_x = resize_nearest_pixel(nearest_mode, ix);
+                    if (in_x < 0) in_x = 0;
+                    if (in_x >= w) in_x = w - 1;
+                    const uint8_t *src = in + ((((size_t)b * c + oc) * h + in_y) * w + in_x) * es;
+                    uint8_t *dst = out + ((((size_t)b * c + oc) * out_h + oy) * out_w + ox) * es;
+                    for (int32_t k = 0; k < es; k++) dst[k] = src[k];
+                }
+            }
+}
+
 /* ------------------------------------------------------------------------ */
 /* (3) definitions with no reference counterpart                            */
 /* ------------------------------------------------------------------------ */

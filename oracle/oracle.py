@@ -259,6 +259,37 @@ def qconv2d_float_chain(x, w, bias, zx, sx, zw, sw, zy, sy, stride=(1, 1), paddi
 
 
 # ---------------------------------------------------------------- no reference counterpart
+LUT_REQUANT, LUT_SWISH = 0, 1
+
+
+def unary_lut(kind, zx, sx, zy, sy) -> np.ndarray:
+    """256-entry table lut[v] = Q(f(DQ(v))); kind LUT_REQUANT (identity) or LUT_SWISH."""
+    lut = np.empty(256, np.uint8)
+    lib().q_unary_lut_u8(_i(kind), _i(zx), _f(sx), _i(zy), _f(sy), _p(lut))
+    return lut
+
+
+def qconcat(xs, qps, out_qp, axis=1) -> np.ndarray:
+    """Concat of u8 tensors carrying different quant params: every input is requantised to
+    out_qp (Q(DQ(x)), the Quantize/Dequantize pair the graph holds around Concat), then joined."""
+    parts = [unary_lut(LUT_REQUANT, z, s, out_qp[0], out_qp[1])[np.asarray(x, np.uint8)] for x, (z, s) in zip(xs, qps)]
+    return np.concatenate(parts, axis=axis)
+
+
+HALF_PIXEL, PYTORCH_HALF_PIXEL, ALIGN_CORNERS, ASYMMETRIC, TFCROP_AND_RESIZE = range(5)
+ROUND_PREFER_FLOOR, ROUND_PREFER_CEIL, FLOOR, CEIL = range(4)
+
+
+def resize_nearest(x: np.ndarray, out_h: int, out_w: int, transformation_mode=HALF_PIXEL, nearest_mode=ROUND_PREFER_FLOOR):
+    """resize_image(nearest_neighbor) on an NCHW tensor of any 1/2/4-byte dtype."""
+    x = np.ascontiguousarray(x)
+    n, c, h, w = x.shape
+    out = np.empty((n, c, out_h, out_w), x.dtype)
+    lib().ref_resize_nearest(_p(x), _p(out), _i(x.dtype.itemsize), _i(n), _i(c), _i(h), _i(w), _i(out_h), _i(out_w),
+                             _i(transformation_mode), _i(nearest_mode))
+    return out
+
+
 def paged_attention_decode(q_bits, k_cache_bits, v_cache_bits, block_table, ctx_lens, scale):
     """float64 brute force.  q [B,Hq,D] f16 bits; K cache [blocks,Hkv,block,D], V cache [blocks,Hkv,D,block] f16 bits."""
     q = _c(q_bits, np.uint16)

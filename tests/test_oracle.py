@@ -389,3 +389,53 @@ def test_pack_unpack_definition():
     assert y3.shape == (3, 3, 4, 2)
     assert y3[2, 1, 3, 1] == x3[2 * 2 + 1, 1 * 4 + 3] and y3[0, 2, 2, 0] == 0
     assert np.array_equal(O.unpack(y3, [1, 0], [4, 2], x3.shape), x3)
+
+
+# ----------------------------------------------------------------------------- u8 glue: byte tables, concat, resize
+def test_unary_tables():
+    v = np.arange(256, dtype=np.uint8)
+    # the requantisation table is the composition of the (separately pinned) dequantize and quantize
+    for zx, sx, zy, sy in [(128, 0.05, 3, 0.023), (7, 0.0235, 131, 0.0041), (0, 0.1, 0, 0.1), (255, 1.0, 0, 0.5)]:
+        lut = O.unary_lut(O.LUT_REQUANT, zx, sx, zy, sy)
+        assert np.array_equal(lut, O.quantize(O.dequantize(v, sx, zx), sy, zy, O.U8))
+    assert np.array_equal(O.unary_lut(O.LUT_REQUANT, 9, 0.25, 9, 0.25), v)            # same params: identity
+    # swish: zero maps to the zero point, the table follows the float64 function to <= 1 code and agrees
+    # with it almost everywhere, saturates at both ends, and is monotone right of the function's minimum
+    zx, sx, zy, sy = 100, 0.08, 12, 0.05
+    lut = O.unary_lut(O.LUT_SWISH, zx, sx, zy, sy).astype(np.int64)
+    x = (v.astype(np.float64) - zx) * np.float64(np.float32(sx))
+    want = np.clip(np.rint(x / (1 + np.exp(-x)) / np.float64(np.float32(sy)) + zy), 0, 255)
+    assert lut[zx] == zy and np.abs(lut - want).max() <= 1 and (lut == want).sum() >= 250
+    assert lut[-1] == 255 and (np.diff(lut[zx:]) >= 0).all()
+    assert lut.min() == zy + round(-0.27846 / 0.05)                                    # min of swish = -0.27846
+    parts = O.qconcat([np.full((1, 2, 1, 1), 10, np.uint8), np.full((1, 3, 1, 1), 20, np.uint8)], [(0, 0.5), (10, 0.25)], (1, 0.5))
+    assert parts.shape == (1, 5, 1, 1) and parts.ravel().tolist() == [11, 11, 6, 6, 6]
+
+
+def test_resize_nearest_known_answers():
+    """Outputs printed in the ONNX operator documentation of Resize (the operator the reference's
+    kernel test compares with through onnxruntime, tests/kernels/test_resize_image.cpp)."""
+    a = np.arange(1, 17, dtype=np.float32).reshape(1, 1, 4, 4)
+    pat = lambda cols: np.array([[a[0, 0, r, c] for c in cols] for r in cols], np.float32).reshape(1, 1, 8, 8)
+    # resize_upsample_sizes_nearest_ceil_half_pixel
+    assert np.array_equal(O.resize_nearest(a, 8, 8, O.HALF_PIXEL, O.CEIL), pat([0, 1, 1, 2, 2, 3, 3, 3]))
+    # resize_upsample_sizes_nearest_floor_align_corners
+    assert np.array_equal(O.resize_nearest(a, 8, 8, O.ALIGN_CORNERS, O.FLOOR), pat([0, 0, 0, 1, 1, 2, 2, 3]))
+    # resize_upsample_sizes_nearest_round_prefer_ceil_asymmetric
+    assert np.array_equal(O.resize_nearest(a, 8, 8, O.ASYMMETRIC, O.ROUND_PREFER_CEIL), pat([0, 1, 1, 2, 2, 3, 3, 3]))
+    # resize_downsample_scales_nearest: [[1,2,3,4],[5,6,7,8]] scaled by 0.6 -> [[1, 3]]
+    b = np.arange(1, 9, dtype=np.float32).reshape(1, 1, 2, 4)
+    assert O.resize_nearest(b, 1, 2).ravel().tolist() == [1, 3]
+    # resize_upsample_scales_nearest: scales (2, 3) repeat every pixel
+    c = np.array([[1, 2], [3, 4]], np.uint8).reshape(1, 1, 2, 2)
+    assert np.array_equal(O.resize_nearest(c, 4, 6), c.repeat(2, axis=2).repeat(3, axis=3))
+    # integer factors in the other modes; identity; element sizes 2 and 4
+    rng = np.random.default_rng(41)
+    x = rng.integers(0, 255, (2, 3, 5, 7), dtype=np.uint8)
+    assert np.array_equal(O.resize_nearest(x, 10, 14, O.ASYMMETRIC, O.FLOOR), x.repeat(2, axis=2).repeat(2, axis=3))
+    assert np.array_equal(O.resize_nearest(x, 5, 7, O.PYTORCH_HALF_PIXEL), x)
+    assert np.array_equal(O.resize_nearest(x[:, :, ::1, :6], 5, 3, O.ASYMMETRIC, O.FLOOR), x[:, :, :, 0:6:2])
+    assert (O.resize_nearest(x, 4, 4, O.TFCROP_AND_RESIZE) == x[:, :, :1, :1]).all()      # roi (0, 0): every index 0
+    for dt in (np.uint16, np.float32):
+        y = rng.integers(0, 60000, (1, 2, 3, 3)).astype(dt)
+        assert np.array_equal(O.resize_nearest(y, 6, 6, O.ASYMMETRIC, O.FLOOR), y.repeat(2, axis=2).repeat(2, axis=3))
