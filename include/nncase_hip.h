@@ -46,6 +46,9 @@ enum {
 /* Error values beyond errno; returned negated.  The first block mirrors
  * nncase_errc (src/Native/include/nncase/runtime/error.h:21-37).            */
 enum {
+    NNCASE_HIP_ERR_INVALID_MODEL_IDENTIFIER = 0x01,
+    NNCASE_HIP_ERR_INVALID_MODEL_VERSION = 0x03,
+    NNCASE_HIP_ERR_RUNTIME_NOT_FOUND = 0x04,
     NNCASE_HIP_ERR_DATATYPE_MISMATCH = 0x05,
     NNCASE_HIP_ERR_SHAPE_MISMATCH = 0x06,
     NNCASE_HIP_ERR_INVALID_MEMORY_LOCATION = 0x07,
@@ -362,6 +365,30 @@ NNCASE_HIP_API int nncase_hip_function_profile(nncase_hip_function_t *fn, int32_
  * "qconv_igemm<T=9,RG=2,rows16>"; NUL-terminated, truncated to `capacity`. */
 NNCASE_HIP_API int nncase_hip_function_op_kernel(nncase_hip_function_t *fn, int32_t index, char *name,
                                                  size_t capacity);
+
+/* ---- kmodel v7 files with a "hip" entry module -------------------------------
+ * Loads a kmodel (container of src/Native/include/nncase/runtime/model.h:38-74,
+ * validated like interpreter::initialize_model, src/Native/src/runtime/
+ * interpreter.cpp:95-102) whose entry function lives in a module of kind
+ * "hip": uploads and pre-packs the module's .rdata constants, allocates one
+ * device buffer per tensor and records the function's operator list into a
+ * resident function (residual adds are folded into the dense convolution that
+ * feeds them).  This is what the hip runtime module's initialize_before_functions
+ * / runtime_function::initialize_core do
+ * (src/Native/include/nncase/runtime/runtime_module.h, runtime_function.h:55-63).
+ * The file image may be released after the call. */
+typedef struct nncase_hip_kmodel nncase_hip_kmodel_t;
+NNCASE_HIP_API int nncase_hip_kmodel_load(nncase_hip_ctx_t *ctx, const void *data, size_t size, nncase_hip_kmodel_t **kmodel);
+NNCASE_HIP_API int nncase_hip_kmodel_destroy(nncase_hip_kmodel_t *kmodel);
+/* The entry function (owned by the kmodel): invoke / capture / profile it with nncase_hip_function_*. */
+NNCASE_HIP_API int nncase_hip_kmodel_function(nncase_hip_kmodel_t *kmodel, nncase_hip_function_t **fn);
+/* Device buffer, typecode and NHWC extents of the entry function's input / output
+ * (interpreter::input_tensor / output_tensor) or of tensor `which` >= 0; the pointer is
+ * NULL for a tensor that only exists inside a fused operator. */
+#define NNCASE_HIP_KMODEL_INPUT (-1)
+#define NNCASE_HIP_KMODEL_OUTPUT (-2)
+NNCASE_HIP_API int nncase_hip_kmodel_tensor(nncase_hip_kmodel_t *kmodel, int32_t which, void **dev_ptr, int32_t *dtype,
+                                            int32_t *dims4);
 
 #ifdef __cplusplus
 }

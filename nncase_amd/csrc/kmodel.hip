@@ -1,0 +1,407 @@
+// Native loader for kmodel v7 files whose entry function lives in a module of kind "hip".
+//
+// Container (all little-endian; src/Native/include/nncase/runtime/model.h:38-74, reader order of
+// src/Native/src/runtime/interpreter.cpp:40-91 and runtime_module.cpp:124-180):
+//   model_header, then per module: module_header, functions (function_header, parameter and
+//   return type signatures, function sections), module sections; every `size` field covers its
+//   header and body, so modules / functions / sections are skipped by size.
+// The hip module keeps its operator list in the module section ".text" (the function header's
+// entrypoint / text_size select the function's slice, as for the stackvm module) and its
+// constants in ".rdata".  Loading uploads and pre-packs the constants, allocates one device
+// buffer per tensor and records the operators into a resident function, which is what the
+// module's runtime_function::invoke_core would run (src/Native/include/nncase/runtime/
+// runtime_function.h:55-63).
+#include "common.hpp"
+
+#include <memory>
+#include <new>
+#include <string>
+#include <vector>
+
+namespace {
+
+#pragma pack(push, 1)
+struct model_header {
+    uint32_t identifier, version, flags, alignment, modules, entry_module, entry_function, reserved0;
+};
+struct module_header {
+    char kind[16];
+    uint32_t version, sections, functions, reserved0;
+    uint64_t size;
+};
+struct function_header {
+    uint32_t parameters, sections;
+    uint64_t entrypoint, text_size, size;
+};
+struct section_header {
+    char name[16];
+    uint32_t flags, reserved0;
+    uint64_t size, body_start, body_size, memory_size;
+};
+struct hipf_header {
+    char magic[4];
+    uint32_t version, n_tensors, n_ops, input_tensor, output_tensor, reserved[2];
+};
+struct hipf_tensor {
+    uint32_t dtype, rank, dims[4];
+    int32_t zero_point;
+    float scale;
+};
+struct hipf_op {
+    uint32_t opcode, n_inputs;
+    int32_t inputs[8];
+    int32_t output;
+    uint32_t reserved;
+    uint64_t rdata0, rdata1;
+    int32_t p[16];
+    float f[4];
+};
+#pragma pack(pop)
+static_assert(sizeof(model_header) == 32 && sizeof(module_header) == 40 && sizeof(function_header) == 32 &&
+                  sizeof(section_header) == 56,
+              "kmodel v7 header sizes");
+static_assert(sizeof(hipf_header) == 32 && sizeof(hipf_tensor) == 32 && sizeof(hipf_op) == 144, "hip text record sizes");
+
+constexpr uint32_t kModelIdentifier = 0x4B4D444C; // 'KMDL'
+constexpr uint32_t kModelVersion = 7;
+constexpr uint64_t kNoRdata = ~uint64_t(0);
+enum { kOpQuantize, kOpDequantize, kOpConv2d, kOpAdd, kOpGlobalAvgPool, kOpLut, kOpConcat, kOpResizeNearest, kOpMaxPool };
+
+struct Span {
+    const uint8_t *p = nullptr;
+    size_t n = 0;
+};
+
+size_t dtype_size(uint32_t dt) {
+    switch (dt) {
+    case NNCASE_HIP_DT_U8:
+    case NNCASE_HIP_DT_I8: return 1;
+    case NNCASE_HIP_DT_I16:
+    case NNCASE_HIP_DT_F16: return 2;
+    case NNCASE_HIP_DT_I32:
+    case NNCASE_HIP_DT_F32: return 4;
+    default: return 0;
+    }
+}
+
+} // namespace
+
+struct nncase_hip_kmodel {
+    nncase_hip_ctx *ctx = nullptr;
+    std::vector<hipf_tensor> tensors;
+    std::vector<void *> buffers;      // one device buffer per tensor (aliases share an entry's value)
+    std::vector<char> owns;           // whether buffers[i] is freed with the model
+    std::vector<nncase_hip_weights_t *> weights;
+    nncase_hip_function_t *fn = nullptr;
+    uint32_t input_tensor = 0, output_tensor = 0;
+};
+
+using namespace nnhip;
+
+extern "C" int nncase_hip_kmodel_destroy(nncase_hip_kmodel_t *m) {
+    if (!m) return -EINVAL;
+    if (m->fn) (void)nncase_hip_function_destroy(m->fn); // synchronises the stream first
+    for (auto *w : m->weights)
+        if (w) (void)nncase_hip_weights_destroy(m->ctx, w);
+    for (size_t i = 0; i < m->buffers.size(); i++)
+        if (m->owns[i] && m->buffers[i]) (void)hipFree(m->buffers[i]);
+    delete m;
+    return 0;
+}
+
+// Finds section `name` among `count` section records starting at `pos`; bodies are addressed by
+// absolute position in the file.
+static bool find_section(const uint8_t *file, size_t size, size_t pos, uint32_t count, const char *name, Span *out) {
+    for (uint32_t i = 0; i < count; i++) {
+        if (pos + sizeof(section_header) > size) return false;
+        section_header h;
+        memcpy(&h, file + pos, sizeof(h));
+        if (h.size < sizeof(h) || h.size > size - pos) return false;
+        if (strncmp(h.name, name, 16) == 0) {
+            if (h.body_start > size || h.body_size > size - h.body_start) return false;
+            out->p = file + h.body_start;
+            out->n = (size_t)h.body_size;
+            return true;
+        }
+        pos += (size_t)h.size;
+    }
+    return false;
+}
+
+extern "C" int nncase_hip_kmodel_load(nncase_hip_ctx_t *ctx, const void *data, size_t size, nncase_hip_kmodel_t **out) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, data && out, -EINVAL, "kmodel_load: null argument");
+    *out = nullptr;
+    const uint8_t *file = static_cast<const uint8_t *>(data);
+    NNHIP_REQUIRE(ctx, size >= sizeof(model_header), -EINVAL, "kmodel_load: file shorter than a model header");
+    model_header mh;
+    memcpy(&mh, file, sizeof(mh));
+    // the two checks of interpreter::initialize_model (src/Native/src/runtime/interpreter.cpp:95-102)
+    NNHIP_REQUIRE(ctx, mh.identifier == kModelIdentifier, -NNCASE_HIP_ERR_INVALID_MODEL_IDENTIFIER,
+                  "kmodel_load: invalid model identifier 0x%08x", mh.identifier);
+    NNHIP_REQUIRE(ctx, mh.version == kModelVersion, -NNCASE_HIP_ERR_INVALID_MODEL_VERSION,
+                  "kmodel_load: model version %u (this runtime reads version %u)", mh.version, kModelVersion);
+    NNHIP_REQUIRE(ctx, mh.entry_module != 0xFFFFFFFFu && mh.entry_module < mh.modules, -EINVAL,
+                  "kmodel_load: model has no entry function");
+
+    // ---- walk to the entry module ------------------------------------------------------------
+    size_t pos = sizeof(model_header);
+    module_header modh{};
+    for (uint32_t i = 0;; i++) {
+        NNHIP_REQUIRE(ctx, pos + sizeof(module_header) <= size, -EINVAL, "kmodel_load: truncated module header");
+        memcpy(&modh, file + pos, sizeof(modh));
+        NNHIP_REQUIRE(ctx, modh.size >= sizeof(modh) && modh.size <= size - pos, -EINVAL, "kmodel_load: bad module size");
+        if (i == mh.entry_module) break;
+        pos += (size_t)modh.size;
+    }
+    NNHIP_REQUIRE(ctx, strncmp(modh.kind, "hip", 16) == 0, -NNCASE_HIP_ERR_RUNTIME_NOT_FOUND,
+                  "kmodel_load: entry module kind \"%.16s\" is not \"hip\"", modh.kind);
+    NNHIP_REQUIRE(ctx, mh.entry_function < modh.functions, -EINVAL, "kmodel_load: entry function index out of range");
+    const size_t module_end = pos + (size_t)modh.size;
+    size_t fpos = pos + sizeof(module_header);
+    function_header fh{};
+    for (uint32_t i = 0; i < modh.functions; i++) { // skip_functions, runtime_module.cpp:112-117
+        NNHIP_REQUIRE(ctx, fpos + sizeof(function_header) <= module_end, -EINVAL, "kmodel_load: truncated function header");
+        function_header h;
+        memcpy(&h, file + fpos, sizeof(h));
+        NNHIP_REQUIRE(ctx, h.size >= sizeof(h) && h.size <= module_end - fpos, -EINVAL, "kmodel_load: bad function size");
+        if (i == mh.entry_function) fh = h;
+        fpos += (size_t)h.size;
+    }
+    Span text_all, rdata;
+    NNHIP_REQUIRE(ctx, find_section(file, size, fpos, modh.sections, ".text", &text_all), -EINVAL,
+                  "kmodel_load: hip module has no .text section");
+    if (!find_section(file, size, fpos, modh.sections, ".rdata", &rdata)) rdata = Span{};
+    NNHIP_REQUIRE(ctx, fh.entrypoint <= text_all.n && fh.text_size <= text_all.n - fh.entrypoint, -EINVAL,
+                  "kmodel_load: function text outside the .text section");
+    const uint8_t *text = text_all.p + fh.entrypoint;
+    const size_t text_size = (size_t)fh.text_size;
+
+    // ---- function text --------------------------------------------------------------------------
+    NNHIP_REQUIRE(ctx, text_size >= sizeof(hipf_header), -EINVAL, "kmodel_load: function text too short");
+    hipf_header th;
+    memcpy(&th, text, sizeof(th));
+    NNHIP_REQUIRE(ctx, memcmp(th.magic, "HIPF", 4) == 0 && th.version == 1, -EINVAL, "kmodel_load: not a hip function text");
+    NNHIP_REQUIRE(ctx, th.n_tensors <= (1u << 20) && th.n_ops <= (1u << 20), -EINVAL, "kmodel_load: implausible counts");
+    const size_t need = sizeof(hipf_header) + (size_t)th.n_tensors * sizeof(hipf_tensor) + (size_t)th.n_ops * sizeof(hipf_op);
+    NNHIP_REQUIRE(ctx, need <= text_size, -EINVAL, "kmodel_load: function text truncated");
+    NNHIP_REQUIRE(ctx, th.input_tensor < th.n_tensors && th.output_tensor < th.n_tensors, -EINVAL,
+                  "kmodel_load: input / output tensor index out of range");
+
+    std::unique_ptr<nncase_hip_kmodel, int (*)(nncase_hip_kmodel *)> m(new (std::nothrow) nncase_hip_kmodel(),
+                                                                      nncase_hip_kmodel_destroy);
+    NNHIP_REQUIRE(ctx, m, -ENOMEM, "kmodel_load: out of host memory");
+    m->ctx = ctx;
+    m->input_tensor = th.input_tensor, m->output_tensor = th.output_tensor;
+    m->tensors.resize(th.n_tensors);
+    memcpy(m->tensors.data(), text + sizeof(hipf_header), (size_t)th.n_tensors * sizeof(hipf_tensor));
+    std::vector<hipf_op> ops(th.n_ops);
+    memcpy(ops.data(), text + sizeof(hipf_header) + (size_t)th.n_tensors * sizeof(hipf_tensor), (size_t)th.n_ops * sizeof(hipf_op));
+
+    auto elems = [&](uint32_t t) {
+        const hipf_tensor &x = m->tensors[t];
+        return (size_t)x.dims[0] * x.dims[1] * x.dims[2] * x.dims[3];
+    };
+    auto tqp = [&](uint32_t t) { return nncase_hip_quant_param_t{m->tensors[t].zero_point, m->tensors[t].scale}; };
+    for (uint32_t t = 0; t < th.n_tensors; t++) {
+        const hipf_tensor &x = m->tensors[t];
+        NNHIP_REQUIRE(ctx, x.rank == 4 && dtype_size(x.dtype) != 0, -NNCASE_HIP_ERR_DATATYPE_MISMATCH,
+                      "kmodel_load: tensor %u has rank %u / dtype 0x%x", t, x.rank, x.dtype);
+        NNHIP_REQUIRE(ctx, x.dims[0] && x.dims[1] && x.dims[2] && x.dims[3] && elems(t) < (size_t(1) << 40), -EINVAL,
+                      "kmodel_load: tensor %u has an empty or implausible shape", t);
+    }
+
+    // ---- which adds fold into the dense conv right before them -------------------------------
+    std::vector<int> consumers(th.n_tensors, 0), producer(th.n_tensors, -1);
+    for (uint32_t k = 0; k < th.n_ops; k++) {
+        const hipf_op &o = ops[k];
+        NNHIP_REQUIRE(ctx, o.n_inputs >= 1 && o.n_inputs <= 8 && o.output >= 0 && (uint32_t)o.output < th.n_tensors, -EINVAL,
+                      "kmodel_load: operator %u has bad operand counts", k);
+        for (uint32_t i = 0; i < o.n_inputs; i++) {
+            NNHIP_REQUIRE(ctx, o.inputs[i] >= 0 && (uint32_t)o.inputs[i] < th.n_tensors, -EINVAL,
+                          "kmodel_load: operator %u reads tensor %d", k, o.inputs[i]);
+            NNHIP_REQUIRE(ctx, (uint32_t)o.inputs[i] == th.input_tensor || producer[o.inputs[i]] >= 0, -EINVAL,
+                          "kmodel_load: operator %u reads tensor %d before it is written", k, o.inputs[i]);
+            consumers[o.inputs[i]]++;
+        }
+        NNHIP_REQUIRE(ctx, producer[o.output] < 0 && (uint32_t)o.output != th.input_tensor, -EINVAL,
+                      "kmodel_load: tensor %d is written twice", o.output);
+        producer[o.output] = (int)k;
+    }
+    std::vector<int> fused_add(th.n_ops, -1); // conv op -> add op folded into it
+    std::vector<char> skipped(th.n_ops, 0);
+    for (uint32_t k = 1; k < th.n_ops; k++) {
+        const hipf_op &add = ops[k], &conv = ops[k - 1];
+        if (add.opcode != kOpAdd || add.n_inputs != 2 || conv.opcode != kOpConv2d) continue;
+        const bool depthwise = conv.p[4] > 1 && conv.p[1] == 1;
+        const bool dense = !depthwise && (int64_t)conv.p[1] * conv.p[4] > 4;
+        if (dense && add.inputs[1] == conv.output && consumers[conv.output] == 1 && add.inputs[0] != conv.output &&
+            (uint32_t)conv.output != th.output_tensor) {
+            fused_add[k - 1] = (int)k;
+            skipped[k] = 1;
+        }
+    }
+
+    // ---- device buffers ---------------------------------------------------------------------------
+    m->buffers.assign(th.n_tensors, nullptr);
+    m->owns.assign(th.n_tensors, 0);
+    for (uint32_t k = 0; k < th.n_ops; k++)
+        if (fused_add[k] >= 0) m->owns[ops[k].output] = 2; // never materialised
+    for (uint32_t t = 0; t < th.n_tensors; t++) {
+        if (m->owns[t] == 2) {
+            m->owns[t] = 0;
+            continue;
+        }
+        NNHIP_HIP(ctx, hipMalloc(&m->buffers[t], elems(t) * dtype_size(m->tensors[t].dtype)));
+        m->owns[t] = 1;
+    }
+
+    // ---- operators ----------------------------------------------------------------------------------
+    NNHIP_REQUIRE(ctx, nncase_hip_function_create(ctx, &m->fn) == 0, -ENOMEM, "kmodel_load: cannot create the function");
+    auto rd = [&](uint64_t off, size_t bytes) -> const uint8_t * {
+        if (off == kNoRdata || off > rdata.n || bytes > rdata.n - off) return nullptr;
+        return rdata.p + off;
+    };
+    for (uint32_t k = 0; k < th.n_ops; k++) {
+        if (skipped[k]) continue;
+        const hipf_op &o = ops[k];
+        const uint32_t in0 = (uint32_t)o.inputs[0], dst = (uint32_t)o.output;
+        const hipf_tensor &ti = m->tensors[in0], &to = m->tensors[dst];
+        int rc = -EINVAL;
+        switch (o.opcode) {
+        case kOpQuantize:
+            NNHIP_REQUIRE(ctx, elems(in0) == elems(dst), -NNCASE_HIP_ERR_SHAPE_MISMATCH, "kmodel_load: op %u shapes differ", k);
+            rc = nncase_hip_function_add_quantize(m->fn, m->buffers[in0], (int)ti.dtype, m->buffers[dst], (int)to.dtype, elems(dst),
+                                                  tqp(dst));
+            break;
+        case kOpDequantize:
+            NNHIP_REQUIRE(ctx, elems(in0) == elems(dst), -NNCASE_HIP_ERR_SHAPE_MISMATCH, "kmodel_load: op %u shapes differ", k);
+            rc = nncase_hip_function_add_dequantize(m->fn, m->buffers[in0], (int)ti.dtype, m->buffers[dst], (int)to.dtype,
+                                                    elems(dst), tqp(in0));
+            break;
+        case kOpConv2d: {
+            const int oc = o.p[0], gic = o.p[1], kh = o.p[2], kw = o.p[3], groups = o.p[4];
+            NNHIP_REQUIRE(ctx, oc > 0 && gic > 0 && kh > 0 && kw > 0 && groups > 0, -EINVAL, "kmodel_load: op %u conv shape", k);
+            NNHIP_REQUIRE(ctx, ti.dtype == NNCASE_HIP_DT_U8 && to.dtype == NNCASE_HIP_DT_U8, -NNCASE_HIP_ERR_DATATYPE_MISMATCH,
+                          "kmodel_load: op %u conv on non-u8 tensors", k);
+            NNHIP_REQUIRE(ctx, (uint32_t)(gic * groups) == ti.dims[3] && (uint32_t)oc == to.dims[3] && ti.dims[0] == to.dims[0],
+                          -NNCASE_HIP_ERR_SHAPE_MISMATCH, "kmodel_load: op %u conv channels / batch do not match its tensors", k);
+            const size_t wbytes = (size_t)oc * gic * kh * kw;
+            const uint8_t *w = rd(o.rdata0, wbytes);
+            NNHIP_REQUIRE(ctx, w, -EINVAL, "kmodel_load: op %u weights outside .rdata", k);
+            const uint8_t *b = nullptr;
+            if (o.rdata1 != kNoRdata) {
+                b = rd(o.rdata1, (size_t)oc * 4);
+                NNHIP_REQUIRE(ctx, b && (o.rdata1 & 3) == 0, -EINVAL, "kmodel_load: op %u bias outside .rdata or misaligned", k);
+            }
+            nncase_hip_conv2d_desc_t desc{};
+            desc.in_channels = gic * groups, desc.out_channels = oc, desc.kernel_h = kh, desc.kernel_w = kw, desc.groups = groups;
+            desc.w_qp = nncase_hip_quant_param_t{o.p[13], o.f[2]};
+            desc.expected_pixels = (int64_t)to.dims[0] * to.dims[1] * to.dims[2];
+            nncase_hip_weights_t *wt = nullptr;
+            rc = nncase_hip_qconv2d_prepack(ctx, &desc, w, reinterpret_cast<const int32_t *>(b), &wt);
+            if (rc) return rc;
+            m->weights.push_back(wt);
+            nncase_hip_conv2d_args_t a{};
+            a.batch = (int)ti.dims[0], a.in_h = (int)ti.dims[1], a.in_w = (int)ti.dims[2];
+            a.stride_h = o.p[5], a.stride_w = o.p[6], a.dilation_h = o.p[7], a.dilation_w = o.p[8];
+            a.pad_h_before = o.p[9], a.pad_h_after = o.p[10], a.pad_w_before = o.p[11], a.pad_w_after = o.p[12];
+            a.x_qp = tqp(in0), a.y_qp = tqp(dst);
+            a.clamp_min = o.f[0], a.clamp_max = o.f[1];
+            a.out_dtype = NNCASE_HIP_DT_U8;
+            NNHIP_REQUIRE(ctx, windowed_output_size(a.in_h, kh, a.stride_h, a.dilation_h, a.pad_h_before, a.pad_h_after) == (int)to.dims[1] &&
+                                   windowed_output_size(a.in_w, kw, a.stride_w, a.dilation_w, a.pad_w_before, a.pad_w_after) == (int)to.dims[2],
+                          -NNCASE_HIP_ERR_SHAPE_MISMATCH, "kmodel_load: op %u conv output extent does not match its tensor", k);
+            void *y = m->buffers[dst];
+            if (fused_add[k] >= 0) {
+                const hipf_op &add = ops[fused_add[k]];
+                const uint32_t res = (uint32_t)add.inputs[0], sum = (uint32_t)add.output;
+                NNHIP_REQUIRE(ctx, elems(res) == elems(dst) && elems(sum) == elems(dst), -NNCASE_HIP_ERR_SHAPE_MISMATCH,
+                              "kmodel_load: op %d add shapes differ", fused_add[k]);
+                a.residual_dev = static_cast<const uint8_t *>(m->buffers[res]);
+                a.residual_qp = tqp(res), a.sum_qp = tqp(sum);
+                a.sum_clamp_min = add.f[0], a.sum_clamp_max = add.f[1];
+                y = m->buffers[sum];
+            }
+            rc = nncase_hip_function_add_qconv2d(m->fn, static_cast<const uint8_t *>(m->buffers[in0]), wt, y, &a);
+            break;
+        }
+        case kOpAdd: {
+            NNHIP_REQUIRE(ctx, o.n_inputs == 2, -EINVAL, "kmodel_load: op %u add needs two inputs", k);
+            const uint32_t in1 = (uint32_t)o.inputs[1];
+            NNHIP_REQUIRE(ctx, elems(in0) == elems(dst) && elems(in1) == elems(dst), -NNCASE_HIP_ERR_SHAPE_MISMATCH,
+                          "kmodel_load: op %u add shapes differ", k);
+            rc = nncase_hip_function_add_qadd(m->fn, static_cast<const uint8_t *>(m->buffers[in0]), tqp(in0),
+                                              static_cast<const uint8_t *>(m->buffers[in1]), tqp(in1),
+                                              static_cast<uint8_t *>(m->buffers[dst]), tqp(dst), o.f[0], o.f[1], elems(dst));
+            break;
+        }
+        case kOpGlobalAvgPool:
+            NNHIP_REQUIRE(ctx, to.dims[0] == ti.dims[0] && to.dims[3] == ti.dims[3] && to.dims[1] == 1 && to.dims[2] == 1,
+                          -NNCASE_HIP_ERR_SHAPE_MISMATCH, "kmodel_load: op %u pool shapes", k);
+            rc = nncase_hip_function_add_qglobal_avgpool(m->fn, static_cast<const uint8_t *>(m->buffers[in0]),
+                                                         static_cast<uint8_t *>(m->buffers[dst]), (int)ti.dims[0], (int)ti.dims[1],
+                                                         (int)ti.dims[2], (int)ti.dims[3], tqp(in0), tqp(dst));
+            break;
+        case kOpLut: {
+            const uint8_t *lut = rd(o.rdata0, 256);
+            NNHIP_REQUIRE(ctx, lut, -EINVAL, "kmodel_load: op %u table outside .rdata", k);
+            NNHIP_REQUIRE(ctx, elems(in0) == elems(dst), -NNCASE_HIP_ERR_SHAPE_MISMATCH, "kmodel_load: op %u shapes differ", k);
+            rc = nncase_hip_function_add_lut_u8(m->fn, static_cast<const uint8_t *>(m->buffers[in0]),
+                                                static_cast<uint8_t *>(m->buffers[dst]), elems(dst), lut);
+            break;
+        }
+        case kOpConcat: {
+            const uint8_t *ins[8];
+            int32_t ch[8];
+            nncase_hip_quant_param_t qps[8];
+            uint32_t total = 0;
+            for (uint32_t i = 0; i < o.n_inputs; i++) {
+                const hipf_tensor &x = m->tensors[o.inputs[i]];
+                NNHIP_REQUIRE(ctx, x.dims[0] == to.dims[0] && x.dims[1] == to.dims[1] && x.dims[2] == to.dims[2],
+                              -NNCASE_HIP_ERR_SHAPE_MISMATCH, "kmodel_load: op %u concat input %u extent", k, i);
+                ins[i] = static_cast<const uint8_t *>(m->buffers[o.inputs[i]]);
+                ch[i] = (int32_t)x.dims[3];
+                qps[i] = tqp((uint32_t)o.inputs[i]);
+                total += x.dims[3];
+            }
+            NNHIP_REQUIRE(ctx, total == to.dims[3], -NNCASE_HIP_ERR_SHAPE_MISMATCH, "kmodel_load: op %u concat channels", k);
+            rc = nncase_hip_function_add_qconcat_channels(m->fn, (int32_t)o.n_inputs, ins, ch, qps, static_cast<uint8_t *>(m->buffers[dst]),
+                                                          tqp(dst), (int64_t)to.dims[0] * to.dims[1] * to.dims[2]);
+            break;
+        }
+        case kOpResizeNearest:
+            NNHIP_REQUIRE(ctx, ti.dtype == to.dtype && ti.dims[0] == to.dims[0] && ti.dims[3] == to.dims[3],
+                          -NNCASE_HIP_ERR_SHAPE_MISMATCH, "kmodel_load: op %u resize tensors", k);
+            rc = nncase_hip_function_add_resize_nearest(m->fn, m->buffers[in0], m->buffers[dst], (int)dtype_size(ti.dtype),
+                                                        (int)ti.dims[0], (int)ti.dims[1], (int)ti.dims[2], (int)ti.dims[3],
+                                                        (int)to.dims[1], (int)to.dims[2], o.p[0], o.p[1]);
+            break;
+        default:
+            return fail(ctx, -NNCASE_HIP_ERR_RUNTIME_NOT_FOUND, "kmodel_load: operator %u has unknown opcode %u", k, o.opcode);
+        }
+        if (rc) return rc;
+    }
+    *out = m.release();
+    return 0;
+}
+
+extern "C" int nncase_hip_kmodel_function(nncase_hip_kmodel_t *m, nncase_hip_function_t **fn) {
+    if (!m || !fn) return -EINVAL;
+    *fn = m->fn;
+    return 0;
+}
+
+extern "C" int nncase_hip_kmodel_tensor(nncase_hip_kmodel_t *m, int32_t which, void **dev_ptr, int32_t *dtype, int32_t *dims4) {
+    if (!m) return -EINVAL;
+    uint32_t t;
+    if (which == NNCASE_HIP_KMODEL_INPUT) t = m->input_tensor;
+    else if (which == NNCASE_HIP_KMODEL_OUTPUT) t = m->output_tensor;
+    else if (which >= 0 && (size_t)which < m->tensors.size()) t = (uint32_t)which;
+    else return fail(m->ctx, -EINVAL, "kmodel_tensor: index %d out of range", which);
+    if (dev_ptr) *dev_ptr = m->buffers[t]; // null for a tensor that only exists inside a fused operator
+    if (dtype) *dtype = (int32_t)m->tensors[t].dtype;
+    if (dims4)
+        for (int i = 0; i < 4; i++) dims4[i] = (int32_t)m->tensors[t].dims[i];
+    return 0;
+}

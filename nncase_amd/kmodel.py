@@ -1,0 +1,369 @@
+"""kmodel v7 container (reader / writer) and the section format of the `hip` module.
+
+Container layout, all little-endian (src/Native/include/nncase/runtime/model.h:38-74 ==
+src/Nncase.CodeGen/CodeGen/KModelTypes.cs; writer order src/Nncase.CodeGen/CodeGen/LinkedModel.cs:28-172;
+reader src/Native/src/runtime/interpreter.cpp:40-91, runtime_module.cpp:124-180):
+
+    model_header   32 B  {u32 identifier 'KMDL' (bytes "LDMK"), version 7, flags, alignment, modules,
+                          entry_module, entry_function, reserved0}
+    per module:
+      module_header 40 B {char kind[16]; u32 version, sections, functions, reserved0; u64 size}
+      per function:
+        function_header 32 B {u32 parameters, sections; u64 entrypoint, text_size, size}
+        parameter type signatures, return type signature (type_serializer.cpp:24-97)
+        function sections
+      module sections
+    section_header 56 B  {char name[16]; u32 flags, reserved0; u64 size, body_start, body_size, memory_size}
+
+Every `size` includes its own header and the padding to 8 bytes that follows the body; `body_start`
+is the absolute stream position of the body after aligning to the section's alignment.
+
+The `hip` module (kind "hip", version 1) holds one function whose `.text` is a flat operator list over
+numbered NHWC tensors (HIPF format below) and a module section `.rdata` with the constants (u8 OIHW
+weights, int32 biases, byte tables).  libnncase_hip.so loads such a module natively
+(nncase_hip_kmodel_load); this file is the compiler-side writer and a generic reader.
+
+HIPF (function text), 8-byte aligned records:
+    header 32 B : "HIPF", u32 version=1, n_tensors, n_ops, input_tensor, output_tensor, reserved[2]
+    tensor 32 B : u32 dtype (typecode), rank, dims[4] (N, H, W, C), i32 zero_point, f32 scale
+    op    144 B : u32 opcode, n_inputs; i32 inputs[8]; i32 output; u32 reserved;
+                  u64 rdata0, rdata1 (offsets into .rdata, ~0 = none); i32 p[16]; f32 f[4]
+"""
+from __future__ import annotations
+
+import struct
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+
+MODEL_IDENTIFIER = 0x4B4D444C      # 'KMDL' as a C++ multi-character constant -> bytes 4C 44 4D 4B
+MODEL_VERSION = 7
+MODEL_HAS_NO_ENTRY = 0xFFFFFFFF
+MIN_ALIGNMENT = 8
+
+MODEL_HEADER = struct.Struct("<8I")
+MODULE_HEADER = struct.Struct("<16s4IQ")
+FUNCTION_HEADER = struct.Struct("<2I3Q")
+SECTION_HEADER = struct.Struct("<16s2I4Q")
+
+# typecodes (src/Native/include/nncase/runtime/typecodes.def)
+DT = {"bool": 0x00, "i8": 0x02, "i16": 0x03, "i32": 0x04, "i64": 0x05, "u8": 0x06, "u16": 0x07, "u32": 0x08, "u64": 0x09,
+      "f16": 0x0A, "f32": 0x0B, "f64": 0x0C, "bf16": 0x0D}
+DT_NAME = {v: k for k, v in DT.items()}
+SIG_INVALID, SIG_ANY, SIG_TENSOR, SIG_TUPLE, SIG_CALLABLE, SIG_END = 0, 1, 2, 3, 4, 0xFF
+DIM_UNKNOWN, DIM_FIXED = 0, 1
+
+
+# ------------------------------------------------------------------------------------------------ type signatures
+@dataclass(frozen=True)
+class TensorType:
+    dtype: str
+    shape: Optional[Tuple[Optional[int], ...]]      # None = scalar; a None entry = unknown dimension
+
+
+@dataclass(frozen=True)
+class TupleType:
+    fields: Tuple[object, ...]
+
+
+def encode_type(t) -> bytes:
+    if isinstance(t, TensorType):
+        out = bytes([SIG_TENSOR, DT[t.dtype]])
+        if t.shape is None:
+            return out + b"\x00"
+        out += b"\x01"
+        for d in t.shape:
+            out += bytes([DIM_UNKNOWN]) if d is None else bytes([DIM_FIXED]) + struct.pack("<I", d)
+        return out + bytes([SIG_END])
+    if isinstance(t, TupleType):
+        return bytes([SIG_TUPLE]) + b"".join(encode_type(f) for f in t.fields) + bytes([SIG_END])
+    raise TypeError(f"unsupported type {t!r}")
+
+
+def decode_type(buf: bytes, pos: int):
+    tok = buf[pos]
+    pos += 1
+    if tok == SIG_TENSOR:
+        dtype = DT_NAME[buf[pos]]
+        scalar = buf[pos + 1] == 0
+        pos += 2
+        if scalar:
+            return TensorType(dtype, None), pos
+        dims: List[Optional[int]] = []
+        while buf[pos] != SIG_END:
+            kind = buf[pos]
+            pos += 1
+            if kind == DIM_FIXED:
+                dims.append(struct.unpack_from("<I", buf, pos)[0])
+                pos += 4
+            elif kind == DIM_UNKNOWN:
+                dims.append(None)
+            else:
+                raise ValueError(f"invalid dim token {kind}")
+        return TensorType(dtype, tuple(dims)), pos + 1
+    if tok == SIG_TUPLE:
+        fields = []
+        while buf[pos] != SIG_END:
+            f, pos = decode_type(buf, pos)
+            fields.append(f)
+        return TupleType(tuple(fields)), pos + 1
+    raise ValueError(f"unsupported type signature token {tok}")
+
+
+# ------------------------------------------------------------------------------------------------ container
+@dataclass
+class Section:
+    name: str
+    body: bytes
+    flags: int = 0
+    alignment: int = 8
+    memory_size: Optional[int] = None
+    body_start: int = 0          # filled by the reader / writer
+
+
+@dataclass
+class Function:
+    parameter_types: List[object]
+    return_type: object
+    entrypoint: int = 0
+    text_size: int = 0
+    sections: List[Section] = field(default_factory=list)
+
+
+@dataclass
+class Module:
+    kind: str
+    version: int
+    functions: List[Function] = field(default_factory=list)
+    sections: List[Section] = field(default_factory=list)
+
+    def section(self, name: str) -> Section:
+        for s in self.sections:
+            if s.name == name:
+                return s
+        raise KeyError(name)
+
+
+@dataclass
+class KModel:
+    modules: List[Module]
+    entry_module: int = MODEL_HAS_NO_ENTRY
+    entry_function: int = MODEL_HAS_NO_ENTRY
+    alignment: int = MIN_ALIGNMENT
+
+    # ---- writer -------------------------------------------------------------------------------------
+    def serialize(self) -> bytes:
+        out = bytearray()
+
+        def align(a: int):
+            out.extend(b"\0" * ((-len(out)) % a))
+            return len(out)
+
+        def name16(s: str) -> bytes:
+            b = s.encode("utf-8")
+            if not 1 <= len(b) <= 16:
+                raise ValueError(f"invalid name {s!r}")
+            return b.ljust(16, b"\0")
+
+        def write_section(s: Section):
+            head = len(out)
+            out.extend(b"\0" * SECTION_HEADER.size)
+            s.body_start = align(s.alignment)
+            out.extend(s.body)
+            end = align(MIN_ALIGNMENT)
+            mem = len(s.body) if s.memory_size is None else s.memory_size
+            SECTION_HEADER.pack_into(out, head, name16(s.name), s.flags, 0, end - head, s.body_start, len(s.body), mem)
+
+        alignment = MIN_ALIGNMENT
+        for m in self.modules:
+            for s in m.sections:
+                alignment = int(np.lcm(alignment, s.alignment))
+        out.extend(MODEL_HEADER.pack(MODEL_IDENTIFIER, MODEL_VERSION, 0, alignment, len(self.modules), self.entry_module,
+                                     self.entry_function, 0))
+        for m in self.modules:
+            mhead = len(out)
+            out.extend(b"\0" * MODULE_HEADER.size)
+            for f in m.functions:
+                fhead = len(out)
+                out.extend(b"\0" * FUNCTION_HEADER.size)
+                for t in f.parameter_types:
+                    out.extend(encode_type(t))
+                out.extend(encode_type(f.return_type))
+                for s in f.sections:
+                    write_section(s)
+                end = align(MIN_ALIGNMENT)
+                FUNCTION_HEADER.pack_into(out, fhead, len(f.parameter_types), len(f.sections), f.entrypoint, f.text_size, end - fhead)
+            for s in m.sections:
+                write_section(s)
+            end = align(MIN_ALIGNMENT)
+            MODULE_HEADER.pack_into(out, mhead, name16(m.kind), m.version, len(m.sections), len(m.functions), 0, end - mhead)
+        return bytes(out)
+
+    # ---- reader -------------------------------------------------------------------------------------
+    @staticmethod
+    def parse(buf: bytes) -> "KModel":
+        ident, version, _flags, alignment, n_modules, entry_module, entry_function, _ = MODEL_HEADER.unpack_from(buf, 0)
+        if ident != MODEL_IDENTIFIER:
+            raise ValueError("invalid model identifier")       # nncase_errc::invalid_model_indentifier
+        if version != MODEL_VERSION:
+            raise ValueError(f"invalid model version {version}")  # nncase_errc::invalid_model_version
+
+        def read_section(pos: int):
+            name, flags, _r, size, body_start, body_size, memory_size = SECTION_HEADER.unpack_from(buf, pos)
+            s = Section(name.rstrip(b"\0").decode(), bytes(buf[body_start:body_start + body_size]), flags, 8, memory_size, body_start)
+            return s, pos + size
+
+        modules = []
+        pos = MODEL_HEADER.size
+        for _ in range(n_modules):
+            kind, mver, n_sections, n_functions, _r, msize = MODULE_HEADER.unpack_from(buf, pos)
+            m = Module(kind.rstrip(b"\0").decode(), mver)
+            p = pos + MODULE_HEADER.size
+            for _f in range(n_functions):
+                n_params, n_fsec, entrypoint, text_size, fsize = FUNCTION_HEADER.unpack_from(buf, p)
+                q = p + FUNCTION_HEADER.size
+                params = []
+                for _p in range(n_params):
+                    t, q = decode_type(buf, q)
+                    params.append(t)
+                ret, q = decode_type(buf, q)
+                fn = Function(params, ret, entrypoint, text_size)
+                for _s in range(n_fsec):
+                    s, q = read_section(q)
+                    fn.sections.append(s)
+                m.functions.append(fn)
+                p += fsize
+            for _s in range(n_sections):
+                s, p = read_section(p)
+                m.sections.append(s)
+            modules.append(m)
+            pos += msize
+        return KModel(modules, entry_module, entry_function, alignment)
+
+
+# ------------------------------------------------------------------------------------------------ hip module
+HIP_MODULE_KIND = "hip"
+HIP_MODULE_VERSION = 1
+HIPF_MAGIC = b"HIPF"
+HIPF_VERSION = 1
+HIPF_HEADER = struct.Struct("<4s7I")
+HIPF_TENSOR = struct.Struct("<6Iif")
+HIPF_OP = struct.Struct("<2I8iiI2Q16i4f")
+NO_RDATA = 0xFFFFFFFFFFFFFFFF
+OP_QUANTIZE, OP_DEQUANTIZE, OP_CONV2D, OP_ADD, OP_GLOBAL_AVGPOOL, OP_LUT, OP_CONCAT, OP_RESIZE_NEAREST, OP_MAXPOOL = range(9)
+OP_NAMES = ["quantize", "dequantize", "conv2d", "add", "global_avgpool", "lut", "concat", "resize_nearest", "maxpool"]
+assert HIPF_HEADER.size == 32 and HIPF_TENSOR.size == 32 and HIPF_OP.size == 144
+
+
+@dataclass
+class HipTensor:
+    dtype: str
+    dims: Tuple[int, int, int, int]     # N, H, W, C
+    zero_point: int = 0
+    scale: float = 1.0
+
+
+@dataclass
+class HipOp:
+    opcode: int
+    inputs: Tuple[int, ...]
+    output: int
+    rdata0: int = NO_RDATA
+    rdata1: int = NO_RDATA
+    p: Tuple[int, ...] = ()
+    f: Tuple[float, ...] = ()
+
+
+class RData:
+    """Constant pool: 64-byte aligned blobs."""
+
+    def __init__(self):
+        self.buf = bytearray()
+
+    def add(self, arr: np.ndarray) -> int:
+        self.buf.extend(b"\0" * ((-len(self.buf)) % 64))
+        off = len(self.buf)
+        self.buf.extend(np.ascontiguousarray(arr).tobytes())
+        return off
+
+
+def encode_hip_text(tensors: Sequence[HipTensor], ops: Sequence[HipOp], input_tensor: int, output_tensor: int) -> bytes:
+    out = bytearray(HIPF_HEADER.pack(HIPF_MAGIC, HIPF_VERSION, len(tensors), len(ops), input_tensor, output_tensor, 0, 0))
+    for t in tensors:
+        out.extend(HIPF_TENSOR.pack(DT[t.dtype], 4, *t.dims, int(t.zero_point), float(np.float32(t.scale))))
+    for o in ops:
+        ins = tuple(o.inputs) + (-1,) * (8 - len(o.inputs))
+        p = tuple(int(v) for v in o.p) + (0,) * (16 - len(o.p))
+        f = tuple(float(np.float32(v)) for v in o.f) + (0.0,) * (4 - len(o.f))
+        out.extend(HIPF_OP.pack(o.opcode, len(o.inputs), *ins, o.output, 0, o.rdata0, o.rdata1, *p, *f))
+    return bytes(out)
+
+
+def decode_hip_text(text: bytes):
+    magic, version, n_tensors, n_ops, input_tensor, output_tensor, _, _ = HIPF_HEADER.unpack_from(text, 0)
+    if magic != HIPF_MAGIC or version != HIPF_VERSION:
+        raise ValueError("not a hip function text")
+    pos = HIPF_HEADER.size
+    tensors, ops = [], []
+    for _ in range(n_tensors):
+        dt, _rank, n, h, w, c, zp, sc = HIPF_TENSOR.unpack_from(text, pos)
+        tensors.append(HipTensor(DT_NAME[dt], (n, h, w, c), zp, sc))
+        pos += HIPF_TENSOR.size
+    for _ in range(n_ops):
+        v = HIPF_OP.unpack_from(text, pos)
+        opcode, n_in = v[0], v[1]
+        ops.append(HipOp(opcode, tuple(v[2:2 + n_in]), v[10], v[12], v[13], tuple(v[14:30]), tuple(v[30:34])))
+        pos += HIPF_OP.size
+    return tensors, ops, input_tensor, output_tensor
+
+
+def compile_quant_graph(qg, batch: int) -> bytes:
+    """Emits a one-module kmodel (kind "hip") for a netbuilder.QuantGraph at a fixed batch:
+    f32 NHWC input -> quantize -> the graph's u8 operators -> dequantize -> f32 output."""
+    rdata = RData()
+    tensors: List[HipTensor] = []
+    ops: List[HipOp] = []
+    c0, h0, w0 = qg.nodes[0].out_shape
+    tensors.append(HipTensor("f32", (batch, h0, w0, c0)))
+    node_tensor: Dict[int, int] = {}
+    for i, n in enumerate(qg.nodes):
+        c, h, w = n.out_shape
+        tensors.append(HipTensor("u8", (batch, h, w, c), int(n.out_qp[0]), float(n.out_qp[1])))
+        tid = len(tensors) - 1
+        node_tensor[i] = tid
+        ins = tuple(node_tensor[j] for j in n.inputs)
+        if n.op == "input":
+            ops.append(HipOp(OP_QUANTIZE, (0,), tid))
+        elif n.op == "conv":
+            oc, gic, kh, kw = n.weights.shape
+            w_off = rdata.add(n.weights.astype(np.uint8))
+            b_off = NO_RDATA if n.bias is None else rdata.add(n.bias.astype(np.int32))
+            (ph0, ph1), (pw0, pw1) = n.padding
+            ops.append(HipOp(OP_CONV2D, ins, tid, w_off, b_off,
+                             (oc, gic, kh, kw, n.groups, n.stride[0], n.stride[1], 1, 1, ph0, ph1, pw0, pw1, int(n.w_qp[0])),
+                             (n.clamp[0], n.clamp[1], float(n.w_qp[1]))))
+        elif n.op == "add":
+            clamp = getattr(n, "clamp", None) or (-3.4028234663852886e38, 3.4028234663852886e38)
+            ops.append(HipOp(OP_ADD, ins, tid, f=(clamp[0], clamp[1])))
+        elif n.op == "gap":
+            ops.append(HipOp(OP_GLOBAL_AVGPOOL, ins, tid))
+        elif n.op == "lut":
+            ops.append(HipOp(OP_LUT, ins, tid, rdata.add(np.asarray(n.lut, np.uint8))))
+        elif n.op == "concat":
+            ops.append(HipOp(OP_CONCAT, ins, tid))
+        elif n.op == "resize":
+            ops.append(HipOp(OP_RESIZE_NEAREST, ins, tid, p=(n.resize_modes[0], n.resize_modes[1])))
+        elif n.op == "maxpool":
+            ops.append(HipOp(OP_MAXPOOL, ins, tid, p=(n.pool[0], n.pool[1], n.pool[2])))
+        else:
+            raise ValueError(f"cannot serialise operator {n.op!r}")
+    last = qg.nodes[-1]
+    c, h, w = last.out_shape
+    tensors.append(HipTensor("f32", (batch, h, w, c)))
+    ops.append(HipOp(OP_DEQUANTIZE, (node_tensor[len(qg.nodes) - 1],), len(tensors) - 1))
+    text = encode_hip_text(tensors, ops, 0, len(tensors) - 1)
+    fn = Function([TensorType("f32", tensors[0].dims)], TensorType("f32", tensors[-1].dims), 0, len(text))
+    mod = Module(HIP_MODULE_KIND, HIP_MODULE_VERSION, [fn],
+                 [Section(".text", text), Section(".rdata", bytes(rdata.buf), alignment=64)])
+    return KModel([mod], entry_module=0, entry_function=0).serialize()

@@ -24,6 +24,7 @@ DT_TO_NP = {v: k for k, v in NP_TO_DT.items()}
 FLT_MAX = float(np.finfo(np.float32).max)
 
 ERR_DATATYPE_MISMATCH, ERR_SHAPE_MISMATCH, ERR_INVALID_MEMORY_LOCATION, ERR_HIP_BASE = 0x05, 0x06, 0x07, 0x1000
+ERR_INVALID_MODEL_IDENTIFIER, ERR_INVALID_MODEL_VERSION, ERR_RUNTIME_NOT_FOUND = 0x01, 0x03, 0x04
 
 
 class QuantParam(C.Structure):
@@ -98,6 +99,10 @@ SYMBOLS = {
     "nncase_hip_function_add_qconcat_channels": (_I, [_VP, C.c_int32, C.POINTER(_VP), _I32P, C.POINTER(QuantParam), _VP,
                                                       QuantParam, C.c_int64]),
     "nncase_hip_function_add_resize_nearest": (_I, [_VP, _VP, _VP] + [C.c_int32] * 9),
+    "nncase_hip_kmodel_load": (_I, [_VP, _VP, _SZ, C.POINTER(_VP)]),
+    "nncase_hip_kmodel_destroy": (_I, [_VP]),
+    "nncase_hip_kmodel_function": (_I, [_VP, C.POINTER(_VP)]),
+    "nncase_hip_kmodel_tensor": (_I, [_VP, C.c_int32, C.POINTER(_VP), _I32P, _I32P]),
     "nncase_hip_pack": (_I, [_VP, _VP, _VP, C.c_int32, C.c_int32, _I32P, C.c_int32, _I32P, _I32P]),
     "nncase_hip_unpack": (_I, [_VP, _VP, _VP, C.c_int32, C.c_int32, _I32P, C.c_int32, _I32P, _I32P]),
     "nncase_hip_nchw_to_nhwc": (_I, [_VP, _VP, _VP, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
@@ -459,6 +464,71 @@ class Function:
     def destroy(self):
         if self.handle:
             self.ctx.lib.nncase_hip_function_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass
+
+
+class _Borrowed:
+    """A device address owned by someone else (a loaded kmodel's tensor)."""
+
+    def __init__(self, ctx, ptr, nbytes):
+        self.ctx, self.ptr, self.nbytes = ctx, ptr, nbytes
+
+    upload = DeviceBuffer.upload
+    download = DeviceBuffer.download
+
+
+class _BorrowedFunction(Function):
+    def __init__(self, ctx, handle):  # no create: the kmodel owns the handle
+        self.ctx, self.handle, self._keep = ctx, handle, []
+
+    def destroy(self):
+        self.handle = None
+
+
+class LoadedKModel:
+    """A kmodel with a `hip` entry module, loaded by the native loader: the counterpart of
+    Interpreter.load_model / set_input_tensor / run / get_output_tensor
+    (src/Nncase.Simulator/Runtime/Interop/RTInterpreter.cs) for this target."""
+    INPUT, OUTPUT = -1, -2
+    _NP = {DT_F32: np.float32, DT_U8: np.uint8, DT_F16: np.float16, DT_I32: np.int32, DT_I8: np.int8, DT_I16: np.int16}
+
+    def __init__(self, ctx: Context, data: bytes):
+        self.ctx = ctx
+        h = C.c_void_p()
+        buf = (C.c_char * len(data)).from_buffer_copy(data)
+        ctx._check(ctx.lib.nncase_hip_kmodel_load(ctx.handle, C.cast(buf, C.c_void_p), len(data), C.byref(h)), "kmodel_load")
+        self.handle = h.value
+        f = C.c_void_p()
+        ctx._check(ctx.lib.nncase_hip_kmodel_function(self.handle, C.byref(f)), "kmodel_function")
+        self.fn = _BorrowedFunction(ctx, f.value)
+        self.input, self.input_shape, self.input_dtype = self.tensor(self.INPUT)
+        self.output, self.output_shape, self.output_dtype = self.tensor(self.OUTPUT)
+
+    def tensor(self, which: int):
+        p, dt, dims = C.c_void_p(), C.c_int32(), (C.c_int32 * 4)()
+        self.ctx._check(self.ctx.lib.nncase_hip_kmodel_tensor(self.handle, which, C.byref(p), C.byref(dt), dims), "kmodel_tensor")
+        shape, dtype = tuple(dims), np.dtype(self._NP[dt.value])
+        buf = None if not p.value else _Borrowed(self.ctx, p.value, int(np.prod(shape)) * dtype.itemsize)
+        return buf, shape, dtype
+
+    def run(self, x: np.ndarray) -> np.ndarray:
+        x = np.ascontiguousarray(x, self.input_dtype)
+        if x.shape != self.input_shape:
+            raise HipError(-ERR_SHAPE_MISMATCH, "kmodel run", f"input {x.shape}, model expects {self.input_shape}")
+        self.input.upload(x)
+        self.fn.invoke()
+        self.ctx.sync()
+        return self.output.download(self.output_shape, self.output_dtype)
+
+    def destroy(self):
+        if self.handle:
+            self.ctx.lib.nncase_hip_kmodel_destroy(self.handle)
             self.handle = None
 
     def __del__(self):

@@ -1,0 +1,102 @@
+"""GPU: kmodel files written by nncase_amd.kmodel and loaded by the native loader give the oracle's
+bytes; malformed files are refused with the reference's error codes."""
+import json
+import os
+import struct
+
+import numpy as np
+import pytest
+
+from nncase_amd import kmodel as km
+from nncase_amd import netbuilder as nb
+from nncase_amd import runtime as rt
+from oracle import netref
+
+pytestmark = pytest.mark.gpu
+f32 = np.float32
+GOLD = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_vectors.json")))
+
+
+def run_and_check(hip_ctx, qg, x):
+    data = km.compile_quant_graph(qg, x.shape[0])
+    model = rt.LoadedKModel(hip_ctx, data)
+    assert model.input_shape == x.shape and model.input_dtype == np.float32
+    y = model.run(x)
+    want, outs = netref.run_integer(qg, x, keep_all=True)
+    want_nhwc = np.ascontiguousarray(np.asarray(want).transpose(0, 2, 3, 1)) if np.asarray(want).ndim == 4 else want
+    assert np.array_equal(y.reshape(want_nhwc.shape).view(np.uint32), want_nhwc.view(np.uint32))
+    # every tensor the loader materialised holds the oracle's bytes (tensor i + 1 is node i)
+    fused = 0
+    for i, ref in enumerate(outs):
+        buf, shape, dtype = model.tensor(i + 1)
+        if buf is None:
+            fused += 1
+            continue
+        got = buf.download(shape, dtype).transpose(0, 3, 1, 2)
+        assert np.array_equal(got, ref), f"node {i} ({qg.nodes[i].name})"
+    return model, y, fused
+
+
+def test_conv_block_kmodel(hip_ctx):
+    rng = np.random.default_rng(1)
+    qg = nb.quantize_graph(nb.conv_block(seed=1), rng.random((8, 56, 56, 64), dtype=f32))
+    x = rng.random((2, 56, 56, 64), dtype=f32)
+    model, y, fused = run_and_check(hip_ctx, qg, x)
+    assert fused == 0 and len(model.fn) == 5
+    model.fn.capture()                                   # the loaded function replays as a HIP graph
+    for _ in range(2):
+        assert np.array_equal(model.run(x).view(np.uint32), y.view(np.uint32))
+    with pytest.raises(rt.HipError) as e:
+        model.run(x[:1])
+    assert e.value.code == -rt.ERR_SHAPE_MISMATCH
+
+
+def test_mobilenetv2_kmodel(hip_ctx):
+    rng = np.random.default_rng(3)
+    qg = nb.quantize_graph(nb.mobilenet_v2(seed=2), rng.random((8, 224, 224, 3), dtype=f32))
+    x = rng.random((2, 224, 224, 3), dtype=f32)
+    model, y, fused = run_and_check(hip_ctx, qg, x)
+    assert fused == 10 and len(model.fn) == 56           # the ten residual adds are folded by the loader
+    ref = nb.HipModel(hip_ctx, qg, 2, capture_graph=False)
+    assert np.array_equal(ref.run(x).view(np.uint32).ravel(), y.view(np.uint32).ravel())
+
+
+def test_malformed_files_are_refused(hip_ctx):
+    rng = np.random.default_rng(1)
+    qg = nb.quantize_graph(nb.conv_block(seed=1), rng.random((2, 56, 56, 64), dtype=f32))
+    good = km.compile_quant_graph(qg, 1)
+
+    def code(data):
+        with pytest.raises(rt.HipError) as e:
+            rt.LoadedKModel(hip_ctx, data)
+        return e.value.code
+
+    assert code(b"KMDL" + good[4:]) == -rt.ERR_INVALID_MODEL_IDENTIFIER
+    shipped_v5 = bytes.fromhex(GOLD["K14_kmodel_header_of_shipped_model"]["hex"])
+    assert code(shipped_v5 + good[32:]) == -rt.ERR_INVALID_MODEL_VERSION
+    assert code(good[:4] + struct.pack("<I", 6) + good[8:]) == -rt.ERR_INVALID_MODEL_VERSION
+    other = km.KModel.parse(good)
+    other.modules[0].kind = "stackvm"
+    assert code(other.serialize()) == -rt.ERR_RUNTIME_NOT_FOUND      # no runtime for that module kind here
+    import errno
+    assert code(good[:20]) == -errno.EINVAL
+    assert code(good[:len(good) // 2]) == -errno.EINVAL               # truncated inside the module
+    no_entry = km.KModel.parse(good)
+    no_entry.entry_module = km.MODEL_HAS_NO_ENTRY
+    assert code(no_entry.serialize()) == -errno.EINVAL
+    # an operator that reads a tensor nobody wrote, and weights pointing outside .rdata
+    m = km.KModel.parse(good)
+    tensors, ops, tin, tout = km.decode_hip_text(m.modules[0].section(".text").body)
+    bad_ops = list(ops)
+    bad_ops[1] = km.HipOp(ops[1].opcode, (3,), ops[1].output, ops[1].rdata0, ops[1].rdata1, ops[1].p, ops[1].f)
+    for text in (km.encode_hip_text(tensors, bad_ops, tin, tout),
+                 km.encode_hip_text(tensors, [ops[0], km.HipOp(ops[1].opcode, ops[1].inputs, ops[1].output, 1 << 40, ops[1].rdata1, ops[1].p, ops[1].f)] + list(ops[2:]), tin, tout)):
+        mm = km.KModel.parse(good)
+        mm.modules[0].sections[0].body = text
+        mm.modules[0].functions[0].text_size = len(text)
+        assert code(mm.serialize()) == -errno.EINVAL
+    unknown = [ops[0], km.HipOp(77, ops[1].inputs, ops[1].output)] + list(ops[2:])
+    mm = km.KModel.parse(good)
+    mm.modules[0].sections[0].body = km.encode_hip_text(tensors, unknown, tin, tout)
+    assert code(mm.serialize()) == -rt.ERR_RUNTIME_NOT_FOUND
+    rt.LoadedKModel(hip_ctx, good).destroy()                          # and the untouched file still loads
