@@ -254,6 +254,16 @@ NNCASE_HIP_API int nncase_hip_resize_nearest(nncase_hip_ctx_t *ctx, const void *
                                              int32_t batch, int32_t in_h, int32_t in_w, int32_t channels, int32_t out_h,
                                              int32_t out_w, int32_t transformation_mode, int32_t nearest_mode);
 
+/* reduce_window2d(max) between Dequantize and Quantize on NHWC u8
+ * (kernels::stackvm::reduce_window2d, src/Native/src/kernels/stackvm/reference/reduce_window.cpp:35-109):
+ *   out = Q_y(max over the window of DQ_x(x)), and, as in the reference's loop (:88-91), the value
+ * 0 takes part once for every window position that lies in the padding.  Dilation 1. */
+NNCASE_HIP_API int nncase_hip_qmaxpool2d(nncase_hip_ctx_t *ctx, const uint8_t *x_dev, uint8_t *out_dev, int32_t batch,
+                                         int32_t in_h, int32_t in_w, int32_t channels, int32_t kernel_h, int32_t kernel_w,
+                                         int32_t stride_h, int32_t stride_w, int32_t pad_h_before, int32_t pad_h_after,
+                                         int32_t pad_w_before, int32_t pad_w_after, nncase_hip_quant_param_t x_qp,
+                                         nncase_hip_quant_param_t y_qp);
+
 /* ---- pack / unpack ------------------------------------------------------
  * pack: every listed axis a (extent D) becomes an outer axis of extent
  * ceil(D / lanes) in place and its lane index is appended as a trailing axis
@@ -346,6 +356,17 @@ NNCASE_HIP_API int nncase_hip_function_add_resize_nearest(nncase_hip_function_t 
                                                           int32_t elem_size, int32_t batch, int32_t in_h, int32_t in_w,
                                                           int32_t channels, int32_t out_h, int32_t out_w,
                                                           int32_t transformation_mode, int32_t nearest_mode);
+NNCASE_HIP_API int nncase_hip_function_add_qmaxpool2d(nncase_hip_function_t *fn, const uint8_t *x_dev, uint8_t *out_dev,
+                                                      int32_t batch, int32_t in_h, int32_t in_w, int32_t channels,
+                                                      int32_t kernel_h, int32_t kernel_w, int32_t stride_h, int32_t stride_w,
+                                                      int32_t pad_h_before, int32_t pad_h_after, int32_t pad_w_before,
+                                                      int32_t pad_w_after, nncase_hip_quant_param_t x_qp,
+                                                      nncase_hip_quant_param_t y_qp);
+/* pack with the arguments of nncase_hip_pack (rank <= 8); used e.g. to pad the channels of an RGB
+ * tensor to 4 before its convolution. */
+NNCASE_HIP_API int nncase_hip_function_add_pack(nncase_hip_function_t *fn, const void *in_dev, void *out_dev,
+                                                int32_t elem_size, int32_t rank, const int32_t *shape, int32_t n_axes,
+                                                const int32_t *axes, const int32_t *lanes);
 /* Number of operators recorded so far. */
 NNCASE_HIP_API int nncase_hip_function_size(nncase_hip_function_t *fn, int32_t *count);
 /* Enqueues the whole function (graph replay if captured). */
@@ -386,7 +407,7 @@ NNCASE_HIP_API int nncase_hip_kmodel_function(nncase_hip_kmodel_t *kmodel, nncas
  * (interpreter::input_tensor / output_tensor) or of tensor `which` >= 0; the pointer is
  * NULL for a tensor that only exists inside a fused operator. */
 #define NNCASE_HIP_KMODEL_INPUT (-1)
-#define NNCASE_HIP_KMODEL_OUTPUT (-2)
+#define NNCASE_HIP_KMODEL_OUTPUT (-2) /* output k of a function with several outputs: NNCASE_HIP_KMODEL_OUTPUT - k */
 NNCASE_HIP_API int nncase_hip_kmodel_tensor(nncase_hip_kmodel_t *kmodel, int32_t which, void **dev_ptr, int32_t *dtype,
                                             int32_t *dims4);
 

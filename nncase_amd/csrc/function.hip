@@ -8,7 +8,7 @@
 namespace {
 
 struct Op {
-    enum Kind { kQuantize, kDequantize, kConv, kAdd, kPool, kLut, kConcat, kResize } kind;
+    enum Kind { kQuantize, kDequantize, kConv, kAdd, kPool, kLut, kConcat, kResize, kMaxPool, kPack } kind;
     const void *in0 = nullptr, *in1 = nullptr;
     void *out = nullptr;
     const nncase_hip_weights_t *weights = nullptr;
@@ -26,6 +26,8 @@ struct Op {
     nncase_hip_quant_param_t cat_qp[NNCASE_HIP_MAX_CONCAT] = {};
     int64_t pixels = 0;
     int32_t elem_size = 0, out_h = 0, out_w = 0, tmode = 0, nmode = 0;
+    int32_t pool[8] = {0}; // kernel h, w, stride h, w, pad h before / after, w before / after
+    int32_t rank = 0, n_axes = 0, shape[8] = {0}, axes[8] = {0}, lanes[8] = {0};
 };
 
 } // namespace
@@ -59,6 +61,12 @@ static int run_op(nncase_hip_function *fn, const Op &op) {
     case Op::kConcat:
         return nncase_hip_qconcat_channels(ctx, op.n_inputs, op.cat_in, op.cat_channels, op.cat_qp, (uint8_t *)op.out,
                                            op.qp0, op.pixels);
+    case Op::kMaxPool:
+        return nncase_hip_qmaxpool2d(ctx, (const uint8_t *)op.in0, (uint8_t *)op.out, op.batch, op.h, op.w, op.channels,
+                                     op.pool[0], op.pool[1], op.pool[2], op.pool[3], op.pool[4], op.pool[5], op.pool[6],
+                                     op.pool[7], op.qp0, op.qp1);
+    case Op::kPack:
+        return nncase_hip_pack(ctx, op.in0, op.out, op.elem_size, op.rank, op.shape, op.n_axes, op.axes, op.lanes);
     case Op::kResize:
         return nncase_hip_resize_nearest(ctx, op.in0, op.out, op.elem_size, op.batch, op.h, op.w, op.channels, op.out_h,
                                          op.out_w, op.tmode, op.nmode);
@@ -190,6 +198,38 @@ extern "C" int nncase_hip_function_add_resize_nearest(nncase_hip_function_t *fn,
     return push(fn, op);
 }
 
+extern "C" int nncase_hip_function_add_qmaxpool2d(nncase_hip_function_t *fn, const uint8_t *x_dev, uint8_t *out_dev,
+                                                  int32_t batch, int32_t in_h, int32_t in_w, int32_t channels,
+                                                  int32_t kernel_h, int32_t kernel_w, int32_t stride_h, int32_t stride_w,
+                                                  int32_t pad_h_before, int32_t pad_h_after, int32_t pad_w_before,
+                                                  int32_t pad_w_after, nncase_hip_quant_param_t x_qp,
+                                                  nncase_hip_quant_param_t y_qp) {
+    if (!fn) return -EINVAL;
+    NNHIP_REQUIRE(fn->ctx, x_dev && out_dev, -EINVAL, "function_add_qmaxpool2d: null buffer");
+    Op op;
+    op.kind = Op::kMaxPool;
+    op.in0 = x_dev, op.out = out_dev, op.batch = batch, op.h = in_h, op.w = in_w, op.channels = channels;
+    const int32_t v[8] = {kernel_h, kernel_w, stride_h, stride_w, pad_h_before, pad_h_after, pad_w_before, pad_w_after};
+    memcpy(op.pool, v, sizeof(v));
+    op.qp0 = x_qp, op.qp1 = y_qp;
+    return push(fn, op);
+}
+
+extern "C" int nncase_hip_function_add_pack(nncase_hip_function_t *fn, const void *in_dev, void *out_dev, int32_t elem_size,
+                                            int32_t rank, const int32_t *shape, int32_t n_axes, const int32_t *axes,
+                                            const int32_t *lanes) {
+    if (!fn) return -EINVAL;
+    NNHIP_REQUIRE(fn->ctx, in_dev && out_dev && shape && rank > 0 && rank <= 8 && n_axes >= 0 && n_axes <= 8 &&
+                               (n_axes == 0 || (axes && lanes)),
+                  -EINVAL, "function_add_pack: bad argument");
+    Op op;
+    op.kind = Op::kPack;
+    op.in0 = in_dev, op.out = out_dev, op.elem_size = elem_size, op.rank = rank, op.n_axes = n_axes;
+    for (int i = 0; i < rank; i++) op.shape[i] = shape[i];
+    for (int i = 0; i < n_axes; i++) op.axes[i] = axes[i], op.lanes[i] = lanes[i];
+    return push(fn, op);
+}
+
 extern "C" int nncase_hip_function_size(nncase_hip_function_t *fn, int32_t *count) {
     if (!fn || !count) return -EINVAL;
     *count = (int32_t)fn->ops.size();
@@ -257,6 +297,8 @@ extern "C" int nncase_hip_function_op_kernel(nncase_hip_function_t *fn, int32_t 
     case Op::kLut: snprintf(name, capacity, "lut_u8"); break;
     case Op::kConcat: snprintf(name, capacity, "qconcat<%d>", op.n_inputs); break;
     case Op::kResize: snprintf(name, capacity, "resize_nearest"); break;
+    case Op::kMaxPool: snprintf(name, capacity, "qmaxpool<%dx%d>", op.pool[0], op.pool[1]); break;
+    case Op::kPack: snprintf(name, capacity, "pack"); break;
     }
     return 0;
 }

@@ -115,6 +115,67 @@ template <typename V> __global__ __launch_bounds__(kGlueThreads) void resize_nea
     reinterpret_cast<V *>(a.out)[gid] = reinterpret_cast<const V *>(a.in)[src];
 }
 
+struct PoolArgs {
+    const uint8_t *in;
+    uint8_t *out;
+    int in_h, in_w, out_h, out_w, kh, kw, stride_h, stride_w, pad_h, pad_w;
+    uint32_t cvecs; // channel vectors per pixel
+    FastDiv d_cvecs, d_ow, d_oh;
+    uint32_t total;
+    uint32_t zero_code; // Q(0.0) with the output's quant params, replicated in the four bytes
+};
+
+__device__ __forceinline__ uint32_t max_u8x4(uint32_t a, uint32_t b) {
+    // bytewise unsigned max of two packed dwords (v_pk_max_u8 does not exist; compare bytes)
+    uint32_t r = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t x = (a >> (8 * i)) & 0xffu, y = (b >> (8 * i)) & 0xffu;
+        r |= (x > y ? x : y) << (8 * i);
+    }
+    return r;
+}
+
+// reduce_window2d(max) on NHWC u8, then a byte table (the requantisation to the output's quant
+// params; the maximum commutes with the increasing maps Dequantize and Quantize, so it is taken
+// on the codes).  The reference folds the value 0 into the result once per window position that
+// lies in the padding (src/Native/src/kernels/stackvm/reference/reduce_window.cpp:88-91), so a
+// window that overlaps the border yields max(values, 0): here max(table[m], Q(0)).
+template <int VEC> __global__ __launch_bounds__(kGlueThreads) void maxpool_u8_kernel(const PoolArgs a, const ByteTable lut) {
+    __shared__ __align__(16) uint8_t t[256];
+    stage_table(t, lut);
+    const uint32_t gid = blockIdx.x * kGlueThreads + threadIdx.x;
+    if (gid >= a.total) return;
+    uint32_t q = fastdiv(gid, a.d_cvecs);
+    const uint32_t v = gid - q * a.d_cvecs.div;
+    uint32_t r = q;
+    q = fastdiv(r, a.d_ow);
+    const int ox = (int)(r - q * a.d_ow.div);
+    r = q;
+    q = fastdiv(r, a.d_oh);
+    const int oy = (int)(r - q * a.d_oh.div);
+    const uint32_t n = q;
+    const int y0 = max(oy * a.stride_h - a.pad_h, 0), y1 = min(oy * a.stride_h - a.pad_h + a.kh, a.in_h);
+    const int x0 = max(ox * a.stride_w - a.pad_w, 0), x1 = min(ox * a.stride_w - a.pad_w + a.kw, a.in_w);
+    uint32_t m = 0;
+    for (int y = y0; y < y1; y++)
+        for (int x = x0; x < x1; x++) {
+            const size_t src = (((size_t)n * a.in_h + y) * a.in_w + x) * a.cvecs + v;
+            if (VEC == 4) m = max_u8x4(m, reinterpret_cast<const uint32_t *>(a.in)[src]);
+            else m = max(m, (uint32_t)a.in[src]);
+        }
+    const bool padded = (y1 - y0) * (x1 - x0) < a.kh * a.kw;
+    if (VEC == 4) {
+        uint32_t o = lut4(t, m);
+        if (padded) o = max_u8x4(o, a.zero_code);
+        reinterpret_cast<uint32_t *>(a.out)[gid] = o;
+    } else {
+        uint32_t o = t[m];
+        if (padded) o = max(o, a.zero_code & 0xffu);
+        a.out[gid] = (uint8_t)o;
+    }
+}
+
 inline ByteTable pack_table(const uint8_t *lut) {
     ByteTable t;
     memcpy(t.w, lut, 256);
@@ -238,5 +299,45 @@ extern "C" int nncase_hip_resize_nearest(nncase_hip_ctx_t *ctx, const void *in_d
     else if (vec == 4) hipLaunchKernelGGL(resize_nearest_kernel<uint32_t>, grid, dim3(kGlueThreads), 0, ctx->stream, a);
     else hipLaunchKernelGGL(resize_nearest_kernel<uint8_t>, grid, dim3(kGlueThreads), 0, ctx->stream, a);
     NNHIP_LAUNCH_CHECK(ctx, "resize_nearest_kernel");
+    return 0;
+}
+
+extern "C" int nncase_hip_qmaxpool2d(nncase_hip_ctx_t *ctx, const uint8_t *x_dev, uint8_t *out_dev, int32_t batch, int32_t in_h,
+                                     int32_t in_w, int32_t channels, int32_t kernel_h, int32_t kernel_w, int32_t stride_h,
+                                     int32_t stride_w, int32_t pad_h_before, int32_t pad_h_after, int32_t pad_w_before,
+                                     int32_t pad_w_after, nncase_hip_quant_param_t x_qp, nncase_hip_quant_param_t y_qp) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, x_dev && out_dev, -EINVAL, "qmaxpool2d: null buffer");
+    NNHIP_REQUIRE(ctx, batch > 0 && in_h > 0 && in_w > 0 && channels > 0 && kernel_h > 0 && kernel_w > 0 && stride_h > 0 &&
+                           stride_w > 0 && pad_h_before >= 0 && pad_h_after >= 0 && pad_w_before >= 0 && pad_w_after >= 0,
+                  -EINVAL, "qmaxpool2d: bad shape");
+    // every window must contain at least one pixel of the image
+    NNHIP_REQUIRE(ctx, pad_h_before < kernel_h && pad_h_after < kernel_h && pad_w_before < kernel_w && pad_w_after < kernel_w,
+                  -EINVAL, "qmaxpool2d: padding not smaller than the window");
+    const int out_h = windowed_output_size(in_h, kernel_h, stride_h, 1, pad_h_before, pad_h_after);
+    const int out_w = windowed_output_size(in_w, kernel_w, stride_w, 1, pad_w_before, pad_w_after);
+    NNHIP_REQUIRE(ctx, out_h > 0 && out_w > 0, -NNCASE_HIP_ERR_SHAPE_MISMATCH, "qmaxpool2d: empty output");
+    uint8_t lut[256];
+    const int rc = nncase_hip_make_unary_lut(NNCASE_HIP_LUT_REQUANT, x_qp, y_qp, lut);
+    NNHIP_REQUIRE(ctx, rc == 0, rc, "qmaxpool2d: cannot build the requantisation table (zero output scale?)");
+    const bool vec = channels % 4 == 0 && ((reinterpret_cast<uintptr_t>(x_dev) | reinterpret_cast<uintptr_t>(out_dev)) & 3u) == 0;
+    PoolArgs a;
+    a.in = x_dev, a.out = out_dev;
+    a.in_h = in_h, a.in_w = in_w, a.out_h = out_h, a.out_w = out_w, a.kh = kernel_h, a.kw = kernel_w;
+    a.stride_h = stride_h, a.stride_w = stride_w, a.pad_h = pad_h_before, a.pad_w = pad_w_before;
+    a.cvecs = (uint32_t)(vec ? channels / 4 : channels);
+    const int64_t total = (int64_t)batch * out_h * out_w * a.cvecs;
+    NNHIP_REQUIRE(ctx, total < ((int64_t)1 << 31), -EINVAL, "qmaxpool2d: too many work items");
+    a.total = (uint32_t)total;
+    a.d_cvecs = make_fastdiv(a.cvecs), a.d_ow = make_fastdiv((uint32_t)out_w), a.d_oh = make_fastdiv((uint32_t)out_h);
+    {
+        float r = nearbyintf(0.f / y_qp.scale + (float)y_qp.zero_point);
+        r = r < 0.f ? 0.f : (r > 255.f ? 255.f : r);
+        a.zero_code = (uint32_t)r * 0x01010101u;
+    }
+    const dim3 grid((unsigned)((total + kGlueThreads - 1) / kGlueThreads));
+    if (vec) hipLaunchKernelGGL(maxpool_u8_kernel<4>, grid, dim3(kGlueThreads), 0, ctx->stream, a, pack_table(lut));
+    else hipLaunchKernelGGL(maxpool_u8_kernel<1>, grid, dim3(kGlueThreads), 0, ctx->stream, a, pack_table(lut));
+    NNHIP_LAUNCH_CHECK(ctx, "maxpool_u8_kernel");
     return 0;
 }

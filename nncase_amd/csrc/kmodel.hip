@@ -40,7 +40,7 @@ struct section_header {
 };
 struct hipf_header {
     char magic[4];
-    uint32_t version, n_tensors, n_ops, input_tensor, output_tensor, reserved[2];
+    uint32_t version, n_tensors, n_ops, input_tensor, output_tensor, n_outputs, reserved;
 };
 struct hipf_tensor {
     uint32_t dtype, rank, dims[4];
@@ -65,7 +65,8 @@ static_assert(sizeof(hipf_header) == 32 && sizeof(hipf_tensor) == 32 && sizeof(h
 constexpr uint32_t kModelIdentifier = 0x4B4D444C; // 'KMDL'
 constexpr uint32_t kModelVersion = 7;
 constexpr uint64_t kNoRdata = ~uint64_t(0);
-enum { kOpQuantize, kOpDequantize, kOpConv2d, kOpAdd, kOpGlobalAvgPool, kOpLut, kOpConcat, kOpResizeNearest, kOpMaxPool };
+enum { kOpQuantize, kOpDequantize, kOpConv2d, kOpAdd, kOpGlobalAvgPool, kOpLut, kOpConcat, kOpResizeNearest, kOpMaxPool,
+       kOpPadChannels };
 
 struct Span {
     const uint8_t *p = nullptr;
@@ -93,7 +94,7 @@ struct nncase_hip_kmodel {
     std::vector<char> owns;           // whether buffers[i] is freed with the model
     std::vector<nncase_hip_weights_t *> weights;
     nncase_hip_function_t *fn = nullptr;
-    uint32_t input_tensor = 0, output_tensor = 0;
+    uint32_t input_tensor = 0, output_tensor = 0, n_outputs = 1; // outputs are consecutive tensors
 };
 
 using namespace nnhip;
@@ -185,14 +186,16 @@ extern "C" int nncase_hip_kmodel_load(nncase_hip_ctx_t *ctx, const void *data, s
     NNHIP_REQUIRE(ctx, th.n_tensors <= (1u << 20) && th.n_ops <= (1u << 20), -EINVAL, "kmodel_load: implausible counts");
     const size_t need = sizeof(hipf_header) + (size_t)th.n_tensors * sizeof(hipf_tensor) + (size_t)th.n_ops * sizeof(hipf_op);
     NNHIP_REQUIRE(ctx, need <= text_size, -EINVAL, "kmodel_load: function text truncated");
-    NNHIP_REQUIRE(ctx, th.input_tensor < th.n_tensors && th.output_tensor < th.n_tensors, -EINVAL,
-                  "kmodel_load: input / output tensor index out of range");
+    const uint32_t n_outputs = th.n_outputs ? th.n_outputs : 1;
+    NNHIP_REQUIRE(ctx, th.input_tensor < th.n_tensors && th.output_tensor < th.n_tensors &&
+                           n_outputs <= th.n_tensors - th.output_tensor,
+                  -EINVAL, "kmodel_load: input / output tensor index out of range");
 
     std::unique_ptr<nncase_hip_kmodel, int (*)(nncase_hip_kmodel *)> m(new (std::nothrow) nncase_hip_kmodel(),
                                                                       nncase_hip_kmodel_destroy);
     NNHIP_REQUIRE(ctx, m, -ENOMEM, "kmodel_load: out of host memory");
     m->ctx = ctx;
-    m->input_tensor = th.input_tensor, m->output_tensor = th.output_tensor;
+    m->input_tensor = th.input_tensor, m->output_tensor = th.output_tensor, m->n_outputs = n_outputs;
     m->tensors.resize(th.n_tensors);
     memcpy(m->tensors.data(), text + sizeof(hipf_header), (size_t)th.n_tensors * sizeof(hipf_tensor));
     std::vector<hipf_op> ops(th.n_ops);
@@ -236,7 +239,7 @@ extern "C" int nncase_hip_kmodel_load(nncase_hip_ctx_t *ctx, const void *data, s
         const bool depthwise = conv.p[4] > 1 && conv.p[1] == 1;
         const bool dense = !depthwise && (int64_t)conv.p[1] * conv.p[4] > 4;
         if (dense && add.inputs[1] == conv.output && consumers[conv.output] == 1 && add.inputs[0] != conv.output &&
-            (uint32_t)conv.output != th.output_tensor) {
+            !((uint32_t)conv.output >= th.output_tensor && (uint32_t)conv.output < th.output_tensor + n_outputs)) {
             fused_add[k - 1] = (int)k;
             skipped[k] = 1;
         }
@@ -377,6 +380,26 @@ extern "C" int nncase_hip_kmodel_load(nncase_hip_ctx_t *ctx, const void *data, s
                                                         (int)ti.dims[0], (int)ti.dims[1], (int)ti.dims[2], (int)ti.dims[3],
                                                         (int)to.dims[1], (int)to.dims[2], o.p[0], o.p[1]);
             break;
+        case kOpMaxPool:
+            NNHIP_REQUIRE(ctx, ti.dims[0] == to.dims[0] && ti.dims[3] == to.dims[3] && o.p[0] > 0 && o.p[1] > 0 && o.p[2] >= 0 &&
+                                   windowed_output_size((int)ti.dims[1], o.p[0], o.p[1], 1, o.p[2], o.p[2]) == (int)to.dims[1] &&
+                                   windowed_output_size((int)ti.dims[2], o.p[0], o.p[1], 1, o.p[2], o.p[2]) == (int)to.dims[2],
+                          -NNCASE_HIP_ERR_SHAPE_MISMATCH, "kmodel_load: op %u pool tensors", k);
+            rc = nncase_hip_function_add_qmaxpool2d(m->fn, static_cast<const uint8_t *>(m->buffers[in0]),
+                                                    static_cast<uint8_t *>(m->buffers[dst]), (int)ti.dims[0], (int)ti.dims[1],
+                                                    (int)ti.dims[2], (int)ti.dims[3], o.p[0], o.p[0], o.p[1], o.p[1], o.p[2], o.p[2],
+                                                    o.p[2], o.p[2], tqp(in0), tqp(dst));
+            break;
+        case kOpPadChannels: {
+            NNHIP_REQUIRE(ctx, ti.dtype == to.dtype && ti.dims[0] == to.dims[0] && ti.dims[1] == to.dims[1] &&
+                                   ti.dims[2] == to.dims[2] && ti.dims[3] <= to.dims[3],
+                          -NNCASE_HIP_ERR_SHAPE_MISMATCH, "kmodel_load: op %u channel padding tensors", k);
+            const int32_t shape[4] = {(int32_t)ti.dims[0], (int32_t)ti.dims[1], (int32_t)ti.dims[2], (int32_t)ti.dims[3]};
+            const int32_t axis = 3, lanes = (int32_t)to.dims[3];
+            rc = nncase_hip_function_add_pack(m->fn, m->buffers[in0], m->buffers[dst], (int)dtype_size(ti.dtype), 4, shape, 1, &axis,
+                                              &lanes);
+            break;
+        }
         default:
             return fail(ctx, -NNCASE_HIP_ERR_RUNTIME_NOT_FOUND, "kmodel_load: operator %u has unknown opcode %u", k, o.opcode);
         }
@@ -396,7 +419,8 @@ extern "C" int nncase_hip_kmodel_tensor(nncase_hip_kmodel_t *m, int32_t which, v
     if (!m) return -EINVAL;
     uint32_t t;
     if (which == NNCASE_HIP_KMODEL_INPUT) t = m->input_tensor;
-    else if (which == NNCASE_HIP_KMODEL_OUTPUT) t = m->output_tensor;
+    else if (which <= NNCASE_HIP_KMODEL_OUTPUT && (uint32_t)(NNCASE_HIP_KMODEL_OUTPUT - which) < m->n_outputs)
+        t = m->output_tensor + (uint32_t)(NNCASE_HIP_KMODEL_OUTPUT - which);
     else if (which >= 0 && (size_t)which < m->tensors.size()) t = (uint32_t)which;
     else return fail(m->ctx, -EINVAL, "kmodel_tensor: index %d out of range", which);
     if (dev_ptr) *dev_ptr = m->buffers[t]; // null for a tensor that only exists inside a fused operator

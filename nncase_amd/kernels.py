@@ -211,6 +211,21 @@ def resize_image_nearest(input: np.ndarray, out_h: int, out_w: int, transformati
     return _from_nhwc_dev(c, dst, (n, ch, out_h, out_w), x.dtype)
 
 
+def max_pool2d(input: np.ndarray, kernel: Sequence[int], stride: Sequence[int], padding: Sequence[Sequence[int]],
+               input_qp: QuantParam, output_qp: QuantParam, ctx: Context = None) -> np.ndarray:
+    """reduce_window2d(max) on a u8 NCHW tensor between Dequantize(input_qp) and Quantize(output_qp)."""
+    c = _ctx(ctx)
+    x = np.ascontiguousarray(input, np.uint8)
+    n, ch, h, w = x.shape
+    (ph0, ph1), (pw0, pw1) = padding
+    oh = rt.windowed_output_size(h, kernel[0], stride[0], 1, ph0, ph1)
+    ow = rt.windowed_output_size(w, kernel[1], stride[1], 1, pw0, pw1)
+    src = _to_nhwc_dev(c, x)
+    dst = c.alloc(max(1, n * ch * oh * ow))
+    c.qmaxpool2d(src, dst, n, h, w, ch, kernel, stride, padding, input_qp, output_qp)
+    return _from_nhwc_dev(c, dst, (n, ch, oh, ow), np.uint8)
+
+
 def pack(input: np.ndarray, axes: Sequence[int], lanes: Sequence[int], ctx: Context = None) -> np.ndarray:
     c = _ctx(ctx)
     x = np.ascontiguousarray(input)

@@ -24,7 +24,8 @@ weights, int32 biases, byte tables).  libnncase_hip.so loads such a module nativ
 (nncase_hip_kmodel_load); this file is the compiler-side writer and a generic reader.
 
 HIPF (function text), 8-byte aligned records:
-    header 32 B : "HIPF", u32 version=1, n_tensors, n_ops, input_tensor, output_tensor, reserved[2]
+    header 32 B : "HIPF", u32 version=1, n_tensors, n_ops, input_tensor, output_tensor, n_outputs, reserved
+                  (the outputs are tensors output_tensor .. output_tensor + n_outputs - 1; n_outputs 0 reads as 1)
     tensor 32 B : u32 dtype (typecode), rank, dims[4] (N, H, W, C), i32 zero_point, f32 scale
     op    144 B : u32 opcode, n_inputs; i32 inputs[8]; i32 output; u32 reserved;
                   u64 rdata0, rdata1 (offsets into .rdata, ~0 = none); i32 p[16]; f32 f[4]
@@ -251,8 +252,10 @@ HIPF_HEADER = struct.Struct("<4s7I")
 HIPF_TENSOR = struct.Struct("<6Iif")
 HIPF_OP = struct.Struct("<2I8iiI2Q16i4f")
 NO_RDATA = 0xFFFFFFFFFFFFFFFF
-OP_QUANTIZE, OP_DEQUANTIZE, OP_CONV2D, OP_ADD, OP_GLOBAL_AVGPOOL, OP_LUT, OP_CONCAT, OP_RESIZE_NEAREST, OP_MAXPOOL = range(9)
-OP_NAMES = ["quantize", "dequantize", "conv2d", "add", "global_avgpool", "lut", "concat", "resize_nearest", "maxpool"]
+(OP_QUANTIZE, OP_DEQUANTIZE, OP_CONV2D, OP_ADD, OP_GLOBAL_AVGPOOL, OP_LUT, OP_CONCAT, OP_RESIZE_NEAREST, OP_MAXPOOL,
+ OP_PAD_CHANNELS) = range(10)
+OP_NAMES = ["quantize", "dequantize", "conv2d", "add", "global_avgpool", "lut", "concat", "resize_nearest", "maxpool",
+            "pad_channels"]
 assert HIPF_HEADER.size == 32 and HIPF_TENSOR.size == 32 and HIPF_OP.size == 144
 
 
@@ -288,8 +291,10 @@ class RData:
         return off
 
 
-def encode_hip_text(tensors: Sequence[HipTensor], ops: Sequence[HipOp], input_tensor: int, output_tensor: int) -> bytes:
-    out = bytearray(HIPF_HEADER.pack(HIPF_MAGIC, HIPF_VERSION, len(tensors), len(ops), input_tensor, output_tensor, 0, 0))
+def encode_hip_text(tensors: Sequence[HipTensor], ops: Sequence[HipOp], input_tensor: int, output_tensor: int,
+                    n_outputs: int = 1) -> bytes:
+    out = bytearray(HIPF_HEADER.pack(HIPF_MAGIC, HIPF_VERSION, len(tensors), len(ops), input_tensor, output_tensor,
+                                     0 if n_outputs == 1 else n_outputs, 0))
     for t in tensors:
         out.extend(HIPF_TENSOR.pack(DT[t.dtype], 4, *t.dims, int(t.zero_point), float(np.float32(t.scale))))
     for o in ops:
@@ -301,7 +306,7 @@ def encode_hip_text(tensors: Sequence[HipTensor], ops: Sequence[HipOp], input_te
 
 
 def decode_hip_text(text: bytes):
-    magic, version, n_tensors, n_ops, input_tensor, output_tensor, _, _ = HIPF_HEADER.unpack_from(text, 0)
+    magic, version, n_tensors, n_ops, input_tensor, output_tensor, _n_outputs, _ = HIPF_HEADER.unpack_from(text, 0)
     if magic != HIPF_MAGIC or version != HIPF_VERSION:
         raise ValueError("not a hip function text")
     pos = HIPF_HEADER.size
@@ -356,14 +361,20 @@ def compile_quant_graph(qg, batch: int) -> bytes:
             ops.append(HipOp(OP_RESIZE_NEAREST, ins, tid, p=(n.resize_modes[0], n.resize_modes[1])))
         elif n.op == "maxpool":
             ops.append(HipOp(OP_MAXPOOL, ins, tid, p=(n.pool[0], n.pool[1], n.pool[2])))
+        elif n.op == "padc":
+            ops.append(HipOp(OP_PAD_CHANNELS, ins, tid))
         else:
             raise ValueError(f"cannot serialise operator {n.op!r}")
-    last = qg.nodes[-1]
-    c, h, w = last.out_shape
-    tensors.append(HipTensor("f32", (batch, h, w, c)))
-    ops.append(HipOp(OP_DEQUANTIZE, (node_tensor[len(qg.nodes) - 1],), len(tensors) - 1))
-    text = encode_hip_text(tensors, ops, 0, len(tensors) - 1)
-    fn = Function([TensorType("f32", tensors[0].dims)], TensorType("f32", tensors[-1].dims), 0, len(text))
+    first_out = len(tensors)
+    out_types = []
+    for j in qg.output_nodes:
+        c, h, w = qg.nodes[j].out_shape
+        tensors.append(HipTensor("f32", (batch, h, w, c)))
+        ops.append(HipOp(OP_DEQUANTIZE, (node_tensor[j],), len(tensors) - 1))
+        out_types.append(TensorType("f32", tensors[-1].dims))
+    text = encode_hip_text(tensors, ops, 0, first_out, len(out_types))
+    ret = out_types[0] if len(out_types) == 1 else TupleType(tuple(out_types))
+    fn = Function([TensorType("f32", tensors[0].dims)], ret, 0, len(text))
     mod = Module(HIP_MODULE_KIND, HIP_MODULE_VERSION, [fn],
                  [Section(".text", text), Section(".rdata", bytes(rdata.buf), alignment=64)])
     return KModel([mod], entry_module=0, entry_function=0).serialize()

@@ -32,7 +32,7 @@ FULL_CLAMP = (-rt.FLT_MAX, rt.FLT_MAX)
 # --------------------------------------------------------------------------------------------- float graph
 @dataclass
 class Node:
-    op: str                      # "input" | "conv" | "add" | "gap"
+    op: str                      # "input" | "conv" | "add" | "gap" | "swish" | "concat" | "resize" | "maxpool"
     inputs: Tuple[int, ...] = ()
     name: str = ""
     # conv
@@ -42,12 +42,16 @@ class Node:
     padding: Tuple[Tuple[int, int], Tuple[int, int]] = ((0, 0), (0, 0))
     groups: int = 1
     clamp: Tuple[float, float] = FULL_CLAMP
+    # resize: output = input extent * scale (nearest, asymmetric coordinates, floor); maxpool: (kernel, stride, pad)
+    scale: int = 2
+    pool: Tuple[int, int, int] = (5, 1, 2)
 
 
 @dataclass
 class FloatGraph:
     nodes: List[Node] = field(default_factory=list)
     input_shape: Tuple[int, int, int] = (224, 224, 3)  # H, W, C (NHWC at the boundary)
+    outputs: Optional[List[int]] = None                 # node ids returned (default: the last node)
 
     def add(self, node: Node) -> int:
         self.nodes.append(node)
@@ -115,6 +119,68 @@ def conv_block(seed: int = 1) -> FloatGraph:
     return g
 
 
+def yolov5s(seed: int = 4, input_hw: int = 640, num_outputs: int = 255) -> FloatGraph:
+    """YOLOv5s-style CSP backbone + PAN neck + detect head (v6 layer table, width 0.5, depth 0.33),
+    random Kaiming weights, BN folded, SiLU after every Conv block, three detect convolutions."""
+    rng = np.random.default_rng(seed)
+    g = FloatGraph(input_shape=(input_hw, input_hw, 3))
+    x = g.add(Node("input", name="input"))
+    counter = [0]
+
+    def conv(src, cin, cout, k, s, pad=None):
+        i = counter[0]
+        counter[0] += 1
+        y = _conv_bn(rng, g, src, cin, cout, k, s, 1, False, f"conv{i}")
+        if pad is not None:
+            g.nodes[y].padding = ((pad, pad), (pad, pad))
+        return g.add(Node("swish", (y,), f"conv{i}.silu"))
+
+    def c3(src, c1, c2, n, shortcut=True):
+        c_ = c2 // 2
+        a = conv(src, c1, c_, 1, 1)
+        for _ in range(n):
+            y = conv(conv(a, c_, c_, 1, 1), c_, c_, 3, 1)
+            a = g.add(Node("add", (a, y), f"bottleneck{counter[0]}.add")) if shortcut else y
+        b = conv(src, c1, c_, 1, 1)
+        return conv(g.add(Node("concat", (a, b), f"c3_{counter[0]}.cat")), 2 * c_, c2, 1, 1)
+
+    def sppf(src, c1, c2):
+        c_ = c1 // 2
+        x1 = conv(src, c1, c_, 1, 1)
+        y1 = g.add(Node("maxpool", (x1,), "sppf.mp1"))
+        y2 = g.add(Node("maxpool", (y1,), "sppf.mp2"))
+        y3 = g.add(Node("maxpool", (y2,), "sppf.mp3"))
+        return conv(g.add(Node("concat", (x1, y1, y2, y3), "sppf.cat")), 4 * c_, c2, 1, 1)
+
+    x = conv(x, 3, 32, 6, 2, pad=2)
+    x = conv(x, 32, 64, 3, 2)
+    x = c3(x, 64, 64, 1)
+    x = conv(x, 64, 128, 3, 2)
+    p3 = c3(x, 128, 128, 2)
+    x = conv(p3, 128, 256, 3, 2)
+    p4 = c3(x, 256, 256, 3)
+    x = conv(p4, 256, 512, 3, 2)
+    x = c3(x, 512, 512, 1)
+    x = sppf(x, 512, 512)
+    n10 = conv(x, 512, 256, 1, 1)
+    x = g.add(Node("resize", (n10,), "up1"))
+    x = c3(g.add(Node("concat", (x, p4), "cat_p4")), 512, 256, 1, False)
+    n14 = conv(x, 256, 128, 1, 1)
+    x = g.add(Node("resize", (n14,), "up2"))
+    o3 = c3(g.add(Node("concat", (x, p3), "cat_p3")), 256, 128, 1, False)
+    x = conv(o3, 128, 128, 3, 2)
+    o4 = c3(g.add(Node("concat", (x, n14), "cat_n14")), 256, 256, 1, False)
+    x = conv(o4, 256, 256, 3, 2)
+    o5 = c3(g.add(Node("concat", (x, n10), "cat_n10")), 512, 512, 1, False)
+    heads = []
+    for name, src, c in (("detect_p3", o3, 128), ("detect_p4", o4, 256), ("detect_p5", o5, 512)):
+        w = (rng.standard_normal((num_outputs, c, 1, 1)) * np.sqrt(1.0 / c)).astype(f32)
+        b = (rng.standard_normal(num_outputs) * 0.1).astype(f32)
+        heads.append(g.add(Node("conv", (src,), name, w, b)))
+    g.outputs = heads
+    return g
+
+
 # --------------------------------------------------------------------------------------------- host float pass
 def _conv_float(x: np.ndarray, n: Node) -> np.ndarray:
     """NCHW float conv via im2col + matmul (calibration only)."""
@@ -154,6 +220,17 @@ def float_forward(g: FloatGraph, x_nhwc: np.ndarray) -> List[np.ndarray]:
             y = outs[n.inputs[0]] + outs[n.inputs[1]]
         elif n.op == "gap":
             y = outs[n.inputs[0]].mean(axis=(2, 3), keepdims=True).astype(f32)
+        elif n.op == "swish":
+            v = outs[n.inputs[0]]
+            y = (v / (1 + np.exp(-v))).astype(f32)
+        elif n.op == "concat":
+            y = np.concatenate([outs[j] for j in n.inputs], axis=1)
+        elif n.op == "resize":
+            y = outs[n.inputs[0]].repeat(n.scale, axis=2).repeat(n.scale, axis=3)
+        elif n.op == "maxpool":
+            k, st, p = n.pool
+            v = np.pad(outs[n.inputs[0]], ((0, 0), (0, 0), (p, p), (p, p)), constant_values=0.0)  # the reference folds 0 in for padding
+            y = np.lib.stride_tricks.sliding_window_view(v, (k, k), axis=(2, 3))[:, :, ::st, ::st].max(axis=(-1, -2)).astype(f32)
         else:
             raise ValueError(n.op)
         outs.append(y)
@@ -175,13 +252,21 @@ class QNode:
     padding: Tuple[Tuple[int, int], Tuple[int, int]] = ((0, 0), (0, 0))
     groups: int = 1
     clamp: Tuple[float, float] = FULL_CLAMP
+    lut: Optional[np.ndarray] = None         # "lut": 256-entry byte table Q(f(DQ(.)))
+    resize_modes: Tuple[int, int] = (rt.RESIZE_ASYMMETRIC, rt.NEAREST_FLOOR)   # "resize"
+    pool: Tuple[int, int, int] = (5, 1, 2)   # "maxpool": kernel, stride, pad
 
 
 @dataclass
 class QuantGraph:
-    """u8/u8 graph: float32 NHWC input -> Quantize -> u8 nodes -> Dequantize -> float32 output."""
+    """u8/u8 graph: float32 NHWC input -> Quantize -> u8 nodes -> Dequantize -> float32 output(s)."""
     nodes: List[QNode]
     input_shape: Tuple[int, int, int]
+    outputs: Optional[List[int]] = None      # node ids that are dequantised and returned (default: the last node)
+
+    @property
+    def output_nodes(self) -> List[int]:
+        return list(self.outputs) if self.outputs else [len(self.nodes) - 1]
 
     @property
     def macs_per_image(self) -> Dict[str, int]:
@@ -219,8 +304,40 @@ def quantize_graph(g: FloatGraph, calib_nhwc: np.ndarray, calib_batch: int = 8) 
             qn.weights, qn.w_qp = wq, (zw, sw)
             qn.bias = np.clip(np.rint(n.bias / bscale), -2 ** 31, 2 ** 31 - 1).astype(np.int32)
             qn.stride, qn.padding, qn.groups, qn.clamp = n.stride, n.padding, n.groups, n.clamp
+        elif n.op == "swish":
+            # Dequantize -> swish -> Quantize of a u8 tensor is a byte table; the library evaluates it
+            # with the CPU kernels' fp32 operations
+            qn.op = "lut"
+            src_qp = qnodes[n.inputs[0]].out_qp
+            qn.lut = rt.make_unary_lut(rt.LUT_SWISH, qp(*src_qp), qp(zp, sc))
+        elif n.op == "maxpool":
+            qn.pool = n.pool
+        elif n.op == "resize":
+            assert shapes[i][1] == shapes[n.inputs[0]][1] * n.scale
         qnodes.append(qn)
-    return QuantGraph(qnodes, g.input_shape)
+    return pad_small_channel_convs(QuantGraph(qnodes, g.input_shape, g.outputs))
+
+
+def pad_small_channel_convs(qg: QuantGraph) -> QuantGraph:
+    """A dense conv over fewer than 4 input channels whose window is not 3x3 (YOLOv5's 6x6 RGB stem)
+    would gather single bytes.  Pad its input to 4 channels ("padc": zero-filled 4th channel) and its
+    weights with the weight zero point, which contributes (w - zw) = 0 whatever the padded byte is:
+    the integer result is unchanged and the conv reads whole dwords."""
+    nodes: List[QNode] = []
+    remap: Dict[int, int] = {}
+    for i, n in enumerate(qg.nodes):
+        n = QNode(**{**n.__dict__, "inputs": tuple(remap[j] for j in n.inputs)})
+        if n.op == "conv" and n.groups == 1 and n.weights.shape[1] < 4 and n.weights.shape[2:] != (3, 3):
+            src = nodes[n.inputs[0]]
+            c, h, w = src.out_shape
+            nodes.append(QNode("padc", (n.inputs[0],), n.name + ".pad4", src.out_qp, (4, h, w)))
+            wpad = np.full((n.weights.shape[0], 4) + n.weights.shape[2:], n.w_qp[0], np.uint8)
+            wpad[:, :c] = n.weights
+            n.weights, n.inputs = wpad, (len(nodes) - 1,)
+        nodes.append(n)
+        remap[i] = len(nodes) - 1
+    outs = None if qg.outputs is None else [remap[j] for j in qg.outputs]
+    return QuantGraph(nodes, qg.input_shape, outs)
 
 
 # --------------------------------------------------------------------------------------------- device binding
@@ -251,7 +368,7 @@ class HipModel:
                     a, b = n.inputs
                     nb_ = qg.nodes[b]
                     dense = nb_.op == "conv" and not (nb_.groups > 1 and nb_.weights.shape[1] == 1) and nb_.weights.shape[1] * nb_.groups > 4
-                    if dense and consumers[b] == 1 and b == i - 1 and a < b:
+                    if dense and consumers[b] == 1 and b == i - 1 and a < b and b not in qg.output_nodes:
                         self.fused_into[b] = i
         for i, n in enumerate(qg.nodes):
             cc, hh, ww = n.out_shape
@@ -285,6 +402,24 @@ class HipModel:
                 a, b = (qg.nodes[j] for j in n.inputs)
                 self.fn.add_qadd(self.buffers[n.inputs[0]], qp(*a.out_qp), self.buffers[n.inputs[1]], qp(*b.out_qp), buf,
                                  qp(*n.out_qp), batch * cc * hh * ww)
+            elif n.op == "lut":
+                self.fn.add_lut_u8(self.buffers[n.inputs[0]], buf, batch * cc * hh * ww, n.lut)
+            elif n.op == "concat":
+                srcs = [qg.nodes[j] for j in n.inputs]
+                self.fn.add_qconcat_channels([self.buffers[j] for j in n.inputs], [s_.out_shape[0] for s_ in srcs],
+                                             [qp(*s_.out_qp) for s_ in srcs], buf, qp(*n.out_qp), batch * hh * ww)
+            elif n.op == "resize":
+                src = qg.nodes[n.inputs[0]]
+                self.fn.add_resize_nearest(self.buffers[n.inputs[0]], buf, 1, batch, src.out_shape[1], src.out_shape[2], cc, hh, ww,
+                                           n.resize_modes[0], n.resize_modes[1])
+            elif n.op == "maxpool":
+                src = qg.nodes[n.inputs[0]]
+                k, st, p = n.pool
+                self.fn.add_qmaxpool2d(self.buffers[n.inputs[0]], buf, batch, src.out_shape[1], src.out_shape[2], cc, (k, k), (st, st),
+                                       ((p, p), (p, p)), qp(*src.out_qp), qp(*n.out_qp))
+            elif n.op == "padc":
+                src = qg.nodes[n.inputs[0]]
+                self.fn.add_pack(self.buffers[n.inputs[0]], buf, 1, [batch, hh, ww, src.out_shape[0]], [3], [cc])
             elif n.op == "gap":
                 src = qg.nodes[n.inputs[0]]
                 self.fn.add_qglobal_avgpool(self.buffers[n.inputs[0]], buf, batch, src.out_shape[1], src.out_shape[2],
@@ -293,13 +428,19 @@ class HipModel:
                 raise ValueError(n.op)
             self.op_names.append(f"{n.op}:{n.name}" + ("+add" if fused_add is not None else ""))
             self.op_nodes.append(i if fused_add is None else fused_add)
-        last = qg.nodes[-1]
+        self.outputs_f32: List[rt.DeviceBuffer] = []
+        for j in qg.output_nodes:
+            node = qg.nodes[j]
+            count = batch * int(np.prod(node.out_shape))
+            out = ctx.alloc(count * 4)
+            self.fn.add_dequantize(self.buffers[j], rt.DT_U8, out, rt.DT_F32, count, qp(*node.out_qp))
+            self.outputs_f32.append(out)
+            self.op_names.append("dequantize:" + node.name)
+            self.op_nodes.append(j)
+        self.output_f32 = self.outputs_f32[0]
+        last = qg.nodes[qg.output_nodes[0]]
         self.out_shape = (batch,) + tuple(last.out_shape)
         self.out_count = int(np.prod(self.out_shape))
-        self.output_f32 = ctx.alloc(self.out_count * 4)
-        self.fn.add_dequantize(self.buffers[-1], rt.DT_U8, self.output_f32, rt.DT_F32, self.out_count, qp(*last.out_qp))
-        self.op_names.append("dequantize:output")
-        self.op_nodes.append(len(qg.nodes) - 1)
         if capture_graph:
             self.fn.capture()
 
@@ -311,11 +452,14 @@ class HipModel:
     def invoke(self):
         self.fn.invoke()
 
-    def output(self) -> np.ndarray:
-        """Dequantised float32 output, NCHW-shaped [batch, C, H, W] (H = W = 1 for classifiers)."""
-        c, h, w = self.qg.nodes[-1].out_shape
-        y = self.output_f32.download((self.batch, h, w, c), f32)
+    def output(self, index: int = 0) -> np.ndarray:
+        """Dequantised float32 output `index`, NCHW-shaped [batch, C, H, W] (H = W = 1 for classifiers)."""
+        c, h, w = self.qg.nodes[self.qg.output_nodes[index]].out_shape
+        y = self.outputs_f32[index].download((self.batch, h, w, c), f32)
         return np.ascontiguousarray(y.transpose(0, 3, 1, 2))
+
+    def all_outputs(self) -> List[np.ndarray]:
+        return [self.output(i) for i in range(len(self.outputs_f32))]
 
     def materialized(self, node: int) -> bool:
         """False for a conv whose output only exists inside a fused residual add."""

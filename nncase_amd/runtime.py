@@ -99,6 +99,9 @@ SYMBOLS = {
     "nncase_hip_function_add_qconcat_channels": (_I, [_VP, C.c_int32, C.POINTER(_VP), _I32P, C.POINTER(QuantParam), _VP,
                                                       QuantParam, C.c_int64]),
     "nncase_hip_function_add_resize_nearest": (_I, [_VP, _VP, _VP] + [C.c_int32] * 9),
+    "nncase_hip_qmaxpool2d": (_I, [_VP, _VP, _VP] + [C.c_int32] * 12 + [QuantParam, QuantParam]),
+    "nncase_hip_function_add_qmaxpool2d": (_I, [_VP, _VP, _VP] + [C.c_int32] * 12 + [QuantParam, QuantParam]),
+    "nncase_hip_function_add_pack": (_I, [_VP, _VP, _VP, C.c_int32, C.c_int32, _I32P, C.c_int32, _I32P, _I32P]),
     "nncase_hip_kmodel_load": (_I, [_VP, _VP, _SZ, C.POINTER(_VP)]),
     "nncase_hip_kmodel_destroy": (_I, [_VP]),
     "nncase_hip_kmodel_function": (_I, [_VP, C.POINTER(_VP)]),
@@ -348,6 +351,11 @@ class Context:
         self._check(self.lib.nncase_hip_qconcat_channels(self.handle, n, ptrs, ch, qps, out.ptr, out_qp, pixels),
                     "qconcat_channels")
 
+    def qmaxpool2d(self, x: DeviceBuffer, out: DeviceBuffer, batch, h, w, channels, kernel, stride, padding, x_qp, y_qp):
+        (ph0, ph1), (pw0, pw1) = padding
+        self._check(self.lib.nncase_hip_qmaxpool2d(self.handle, x.ptr, out.ptr, batch, h, w, channels, kernel[0], kernel[1],
+                                                   stride[0], stride[1], ph0, ph1, pw0, pw1, x_qp, y_qp), "qmaxpool2d")
+
     def resize_nearest(self, src: DeviceBuffer, dst: DeviceBuffer, elem_size, batch, in_h, in_w, channels, out_h, out_w,
                        transformation_mode=0, nearest_mode=0):
         self._check(self.lib.nncase_hip_resize_nearest(self.handle, src.ptr, dst.ptr, elem_size, batch, in_h, in_w, channels,
@@ -427,6 +435,19 @@ class Function:
         n, ptrs, ch, qps = _concat_args(inputs, channels, in_qps)
         self._ck(self.ctx.lib.nncase_hip_function_add_qconcat_channels(self.handle, n, ptrs, ch, qps, out.ptr, out_qp, pixels),
                  "function_add_qconcat_channels")
+
+    def add_qmaxpool2d(self, x, out, batch, h, w, channels, kernel, stride, padding, x_qp, y_qp):
+        self._keep += [x, out]
+        (ph0, ph1), (pw0, pw1) = padding
+        self._ck(self.ctx.lib.nncase_hip_function_add_qmaxpool2d(self.handle, x.ptr, out.ptr, batch, h, w, channels, kernel[0],
+                                                                 kernel[1], stride[0], stride[1], ph0, ph1, pw0, pw1, x_qp, y_qp),
+                 "function_add_qmaxpool2d")
+
+    def add_pack(self, src, dst, elem_size, shape, axes, lanes):
+        self._keep += [src, dst]
+        sh, ax, ln = (C.c_int32 * len(shape))(*shape), (C.c_int32 * max(1, len(axes)))(*axes), (C.c_int32 * max(1, len(lanes)))(*lanes)
+        self._ck(self.ctx.lib.nncase_hip_function_add_pack(self.handle, src.ptr, dst.ptr, elem_size, len(shape), sh, len(axes), ax, ln),
+                 "function_add_pack")
 
     def add_resize_nearest(self, src, dst, elem_size, batch, in_h, in_w, channels, out_h, out_w, transformation_mode=0,
                            nearest_mode=0):
@@ -509,6 +530,12 @@ class LoadedKModel:
         self.fn = _BorrowedFunction(ctx, f.value)
         self.input, self.input_shape, self.input_dtype = self.tensor(self.INPUT)
         self.output, self.output_shape, self.output_dtype = self.tensor(self.OUTPUT)
+        self.outputs = [(self.output, self.output_shape, self.output_dtype)]
+        while True:  # further outputs of a function that returns a tuple
+            try:
+                self.outputs.append(self.tensor(self.OUTPUT - len(self.outputs)))
+            except HipError:
+                break
 
     def tensor(self, which: int):
         p, dt, dims = C.c_void_p(), C.c_int32(), (C.c_int32 * 4)()
@@ -524,7 +551,8 @@ class LoadedKModel:
         self.input.upload(x)
         self.fn.invoke()
         self.ctx.sync()
-        return self.output.download(self.output_shape, self.output_dtype)
+        ys = [b.download(shape, dt) for b, shape, dt in self.outputs]
+        return ys[0] if len(ys) == 1 else ys
 
     def destroy(self):
         if self.handle:

@@ -1,6 +1,9 @@
 """Runs a quantised graph (nncase_amd.netbuilder.QuantGraph, used here as plain data) through
 the CPU oracle.  TEST INFRASTRUCTURE ONLY.
 
+Byte-table, concat, resize, max-pool and channel-padding nodes are byte-exact in both runs (the CPU
+target evaluates them between Dequantize and Quantize with the same fp32 formulas the tables hold).
+
 run_integer(): node by node with the integer-exact operator definitions -- the values the
                HIP path must reproduce bit for bit.
 run_float_chain(): what nncase's CPU target executes for the same model, every quantised conv
@@ -42,11 +45,26 @@ def run_integer(qg, x_nhwc: np.ndarray, keep_all: bool = False):
             src = qg.nodes[n.inputs[0]]
             y = O.qglobal_avgpool(outs[n.inputs[0]], src.out_qp[0], src.out_qp[1], n.out_qp[0], n.out_qp[1])
             y = y.reshape(y.shape[0], y.shape[1], 1, 1)
+        elif n.op == "lut":
+            src = qg.nodes[n.inputs[0]]
+            y = O.unary_lut(O.LUT_SWISH, src.out_qp[0], src.out_qp[1], n.out_qp[0], n.out_qp[1])[outs[n.inputs[0]]]
+        elif n.op == "concat":
+            y = O.qconcat([outs[j] for j in n.inputs], [qg.nodes[j].out_qp for j in n.inputs], n.out_qp)
+        elif n.op == "resize":
+            c, h, w = n.out_shape
+            y = O.resize_nearest(outs[n.inputs[0]], h, w, n.resize_modes[0], n.resize_modes[1])
+        elif n.op == "maxpool":
+            src = qg.nodes[n.inputs[0]]
+            k, st, p = n.pool
+            y = O.qmaxpool(outs[n.inputs[0]], (k, k), (st, st), ((p, p), (p, p)), src.out_qp[0], src.out_qp[1], n.out_qp[0], n.out_qp[1])
+        elif n.op == "padc":
+            v = outs[n.inputs[0]]
+            y = np.pad(v, ((0, 0), (0, n.out_shape[0] - v.shape[1]), (0, 0), (0, 0)))
         else:
             raise ValueError(n.op)
         outs.append(y)
-    last = qg.nodes[-1]
-    final = O.dequantize(outs[-1], last.out_qp[1], last.out_qp[0])
+    finals = [O.dequantize(outs[j], qg.nodes[j].out_qp[1], qg.nodes[j].out_qp[0]) for j in qg.output_nodes]
+    final = finals[0] if len(finals) == 1 else finals
     return (final, outs) if keep_all else (final, None)
 
 
@@ -70,9 +88,24 @@ def run_float_chain(qg, x_nhwc: np.ndarray, keep_all: bool = False):
             xf = O.dequantize(outs[n.inputs[0]], src.out_qp[1], src.out_qp[0])
             m = O.reduce_window2d_mean_f32(xf, xf.shape[2:], (1, 1))
             y = O.quantize(m, n.out_qp[1], n.out_qp[0], O.U8)
+        elif n.op == "lut":
+            src = qg.nodes[n.inputs[0]]
+            y = O.unary_lut(O.LUT_SWISH, src.out_qp[0], src.out_qp[1], n.out_qp[0], n.out_qp[1])[outs[n.inputs[0]]]
+        elif n.op == "concat":
+            y = O.qconcat([outs[j] for j in n.inputs], [qg.nodes[j].out_qp for j in n.inputs], n.out_qp)
+        elif n.op == "resize":
+            c, h, w = n.out_shape
+            y = O.resize_nearest(outs[n.inputs[0]], h, w, n.resize_modes[0], n.resize_modes[1])
+        elif n.op == "maxpool":
+            src = qg.nodes[n.inputs[0]]
+            k, st, p = n.pool
+            y = O.qmaxpool(outs[n.inputs[0]], (k, k), (st, st), ((p, p), (p, p)), src.out_qp[0], src.out_qp[1], n.out_qp[0], n.out_qp[1])
+        elif n.op == "padc":
+            v = outs[n.inputs[0]]
+            y = np.pad(v, ((0, 0), (0, n.out_shape[0] - v.shape[1]), (0, 0), (0, 0)))
         else:
             raise ValueError(n.op)
         outs.append(y)
-    last = qg.nodes[-1]
-    final = O.dequantize(outs[-1], last.out_qp[1], last.out_qp[0])
+    finals = [O.dequantize(outs[j], qg.nodes[j].out_qp[1], qg.nodes[j].out_qp[0]) for j in qg.output_nodes]
+    final = finals[0] if len(finals) == 1 else finals
     return (final, outs) if keep_all else (final, None)

@@ -52,6 +52,7 @@
  * Build:  gcc -O2 -fno-fast-math -ffp-contract=off -fPIC -shared \
  *             -o oracle/libnncase_oracle.so oracle/nncase_oracle.c -lm
  */
+#include <float.h>
 #include <math.h>
 #include <stddef.h>
 #include <stdint.h>
@@ -632,6 +633,40 @@ ORACLE_API void ref_resize_nearest(const uint8_t *in, uint8_t *out, int32_t es, 
                     for (int32_t k = 0; k < es; k++) dst[k] = src[k];
                 }
             }
+}
+
+/* Max pooling of a u8 NCHW tensor between Dequantize and Quantize:
+ * the window loop of reduce_window2d with binary_op = max, init = lowest,
+ * window_op = identity (src/Native/src/kernels/stackvm/reference/reduce_window.cpp:35-109):
+ * only in-bounds positions are read, then the value 0 is folded in once per
+ * position that lies in the padding (:88-91).                                 */
+ORACLE_API void q_maxpool_u8(const uint8_t *x, uint8_t *out, int32_t n, int32_t c, int32_t h,
+                             int32_t w, int32_t kh, int32_t kw, int32_t sh, int32_t sw,
+                             int32_t ph0, int32_t ph1, int32_t pw0, int32_t pw1, int32_t zx,
+                             float sx, int32_t zy, float sy) {
+    const int32_t out_h = oracle_windowed_output_size(h, kh, sh, 1, ph0, ph1);
+    const int32_t out_w = oracle_windowed_output_size(w, kw, sw, 1, pw0, pw1);
+    for (int32_t b = 0; b < n; b++)
+        for (int32_t ch = 0; ch < c; ch++)
+            for (int32_t oy = 0; oy < out_h; oy++)
+                for (int32_t ox = 0; ox < out_w; ox++) {
+                    const int32_t y0 = oy * sh - ph0, x0 = ox * sw - pw0;
+                    const int32_t fy0 = y0 < 0 ? -y0 : 0, fy1 = (h - y0) < kh ? (h - y0) : kh;
+                    const int32_t fx0 = x0 < 0 ? -x0 : 0, fx1 = (w - x0) < kw ? (w - x0) : kw;
+                    float value = -FLT_MAX;
+                    int32_t count = 0;
+                    for (int32_t ky = fy0; ky < fy1; ky++)
+                        for (int32_t kx = fx0; kx < fx1; kx++) {
+                            const uint8_t q = x[(((size_t)b * c + ch) * h + (y0 + ky)) * w + (x0 + kx)];
+                            const float v = ((float)q - (float)zx) * sx;
+                            value = value > v ? value : v;
+                            count++;
+                        }
+                    for (int32_t i = 0; i < kh * kw - count; i++) value = value > 0.0f ? value : 0.0f;
+                    float t = value / sy + (float)zy;
+                    out[(((size_t)b * c + ch) * out_h + oy) * out_w + ox] =
+                        (uint8_t)clampi_ref(rne_sat_i32(t), 0, 255);
+                }
 }
 
 /* ------------------------------------------------------------------------ */

@@ -290,6 +290,19 @@ def resize_nearest(x: np.ndarray, out_h: int, out_w: int, transformation_mode=HA
     return out
 
 
+def qmaxpool(x, kernel, stride, padding, zx, sx, zy, sy) -> np.ndarray:
+    """reduce_window2d(max) on u8 NCHW between Dequantize(zx, sx) and Quantize(zy, sy)."""
+    x = _c(x, np.uint8)
+    n, c, h, w = x.shape
+    (ph0, ph1), (pw0, pw1) = padding
+    oh = windowed_output_size(h, kernel[0], stride[0], 1, ph0, ph1)
+    ow = windowed_output_size(w, kernel[1], stride[1], 1, pw0, pw1)
+    out = np.empty((n, c, oh, ow), np.uint8)
+    lib().q_maxpool_u8(_p(x), _p(out), _i(n), _i(c), _i(h), _i(w), _i(kernel[0]), _i(kernel[1]), _i(stride[0]), _i(stride[1]),
+                       _i(ph0), _i(ph1), _i(pw0), _i(pw1), _i(zx), _f(sx), _i(zy), _f(sy))
+    return out
+
+
 def paged_attention_decode(q_bits, k_cache_bits, v_cache_bits, block_table, ctx_lens, scale):
     """float64 brute force.  q [B,Hq,D] f16 bits; K cache [blocks,Hkv,block,D], V cache [blocks,Hkv,D,block] f16 bits."""
     q = _c(q_bits, np.uint16)

@@ -123,3 +123,27 @@ def test_error_paths(hip_ctx):
         rt.make_unary_lut(5, qp(0, 1.0), qp(0, 1.0))
     with pytest.raises(rt.HipError):
         rt.make_unary_lut(rt.LUT_SWISH, qp(0, 1.0), qp(0, 0.0))      # zero output scale
+
+
+@pytest.mark.parametrize("k,s,p", [(5, 1, 2), (3, 2, 1), (2, 2, 0), (3, 1, 0), (5, 1, (2, 1)), (9, 1, 4), (13, 1, 6)])
+@pytest.mark.parametrize("c", [16, 3])
+def test_maxpool_between_dequantize_and_quantize(hip_ctx, k, s, p, c):
+    rng = np.random.default_rng(k * 10 + s + c)
+    pad = ((p, p), (p, p)) if isinstance(p, int) else ((p[0], p[1]), (p[1], p[0]))
+    x = rng.integers(0, 256, (2, c, 17, 13), dtype=np.uint8)
+    for (zx, sx, zy, sy) in [(90, 0.05, 90, 0.05), (120, 0.04, 7, 0.031), (0, 0.1, 30, 0.12), (255, 0.02, 200, 0.02)]:
+        got = K.max_pool2d(x, (k, k), (s, s), pad, qp(zx, sx), qp(zy, sy), ctx=hip_ctx)
+        want = O.qmaxpool(x, (k, k), (s, s), pad, zx, sx, zy, sy)
+        assert got.shape == want.shape and np.array_equal(got, want)
+
+
+def test_maxpool_sppf_shape(hip_ctx):
+    """Config-4 SPPF pooling: 5x5, stride 1, pad 2 on [16, 256, 20, 20]; the float path agrees."""
+    rng = np.random.default_rng(2)
+    x = rng.integers(0, 256, (16, 256, 20, 20), dtype=np.uint8)
+    zx, sx = 13, 0.047
+    got = K.max_pool2d(x, (5, 5), (1, 1), ((2, 2), (2, 2)), qp(zx, sx), qp(zx, sx), ctx=hip_ctx)
+    assert np.array_equal(got, O.qmaxpool(x, (5, 5), (1, 1), ((2, 2), (2, 2)), zx, sx, zx, sx))
+    xp = np.pad(np.maximum(x, 0), ((0, 0), (0, 0), (2, 2), (2, 2)), constant_values=zx)   # 0.0 is the code zx
+    win = np.lib.stride_tricks.sliding_window_view(xp, (5, 5), axis=(2, 3)).max(axis=(-1, -2))
+    assert np.array_equal(got, win)

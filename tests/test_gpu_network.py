@@ -102,6 +102,61 @@ def test_mobilenetv2_batch64_equals_small_batches(hip_ctx):
     assert np.array_equal(y[:1].view(np.uint32), np.asarray(want).view(np.uint32))
 
 
+def test_yolov5s_config4(hip_ctx):
+    """YOLOv5s-style backbone + neck + head at a reduced input (128 x 128, batch 2): every u8 tensor and the
+    three dequantised head outputs equal the oracle's; the same graph through a kmodel file gives the same bytes."""
+    from nncase_amd import kmodel as km
+    from nncase_amd import runtime as rt
+    g = nb.yolov5s(seed=4, input_hw=128)
+    rng = np.random.default_rng(6)
+    qg = nb.quantize_graph(g, rng.random((4, 128, 128, 3), dtype=f32))
+    ops = [n.op for n in qg.nodes]
+    assert ops.count("conv") == 60 and ops.count("lut") == 57 and ops.count("concat") == 13 and ops.count("maxpool") == 3
+    assert ops.count("resize") == 2 and ops.count("add") == 7 and ops.count("padc") == 1 and len(qg.output_nodes) == 3
+    x = rng.random((2, 128, 128, 3), dtype=f32)
+    wants, outs = netref.run_integer(qg, x, keep_all=True)
+    for capture in (False, True):
+        model = nb.HipModel(hip_ctx, qg, 2, capture_graph=capture)
+        model.run(x)
+        for i, ref in enumerate(outs):
+            got = model.tensor(i)
+            assert np.array_equal(got, ref), f"node {i} ({qg.nodes[i].name}, {qg.nodes[i].op}): {(got != ref).sum()} of {ref.size} bytes differ"
+        for got, want in zip(model.all_outputs(), wants):
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    # the zero-padded 4th stem channel changes nothing: the stem conv equals the 3-channel convolution
+    stem = next(i for i, n in enumerate(qg.nodes) if n.op == "conv")
+    n, src = qg.nodes[stem], qg.nodes[0]
+    plain = O.qconv2d(outs[0], n.weights[:, :3], n.bias, src.out_qp[0], src.out_qp[1], n.w_qp[0], n.w_qp[1], n.out_qp[0], n.out_qp[1],
+                      n.stride, n.padding, (1, 1), 1, n.clamp, O.OUT_U8)
+    assert np.array_equal(plain, outs[stem])
+    # float model vs quantised model: the reference's acceptance bar
+    fl = nb.float_forward(g, x)
+    for want, j in zip(wants, g.outputs):
+        assert O.cosine(want, fl[j]) > 0.98
+    loaded = rt.LoadedKModel(hip_ctx, km.compile_quant_graph(qg, 2))
+    ys = loaded.run(x)
+    assert len(ys) == 3
+    for y, want in zip(ys, wants):
+        assert np.array_equal(y.transpose(0, 3, 1, 2).view(np.uint32), want.view(np.uint32))
+
+
+def test_yolov5s_batch_consistency_at_larger_size(hip_ctx):
+    """Size-independent property at a size the oracle does not follow: 320 x 320 at batch 8 equals the same
+    images at batch 1, tensor by tensor."""
+    g = nb.yolov5s(seed=4, input_hw=320)
+    rng = np.random.default_rng(7)
+    qg = nb.quantize_graph(g, rng.random((2, 320, 320, 3), dtype=f32))
+    x = rng.random((8, 320, 320, 3), dtype=f32)
+    big = nb.HipModel(hip_ctx, qg, 8, capture_graph=True)
+    big.run(x)
+    for img in (0, 7):
+        one = nb.HipModel(hip_ctx, qg, 1, capture_graph=False)
+        one.run(x[img:img + 1])
+        for i in range(len(qg.nodes)):
+            a, b = big.tensor(i)[img:img + 1], one.tensor(i)
+            assert np.array_equal(a, b), f"node {i} ({qg.nodes[i].name}), image {img}: {(a != b).sum()} bytes differ"
+
+
 def test_profile_and_kernel_names(hip_ctx):
     g = nb.conv_block(seed=1)
     rng = np.random.default_rng(1)

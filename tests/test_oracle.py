@@ -439,3 +439,20 @@ def test_resize_nearest_known_answers():
     for dt in (np.uint16, np.float32):
         y = rng.integers(0, 60000, (1, 2, 3, 3)).astype(dt)
         assert np.array_equal(O.resize_nearest(y, 6, 6, O.ASYMMETRIC, O.FLOOR), y.repeat(2, axis=2).repeat(2, axis=3))
+
+
+def test_maxpool_restatement():
+    rng = np.random.default_rng(43)
+    x = rng.integers(0, 256, (2, 3, 9, 7), dtype=np.uint8)
+    zx, sx, zy, sy = 100, 0.05, 20, 0.07
+    xf = O.dequantize(x, sx, zx)
+    for k, s, p in ((3, 1, 1), (5, 1, 2), (2, 2, 0), (3, 2, 1)):
+        got = O.qmaxpool(x, (k, k), (s, s), ((p, p), (p, p)), zx, sx, zy, sy)
+        # float definition: pad with 0.0 (the value the reference folds in for padded positions), window max, quantize
+        xp = np.pad(xf, ((0, 0), (0, 0), (p, p), (p, p)), constant_values=0.0)
+        win = np.lib.stride_tricks.sliding_window_view(xp, (k, k), axis=(2, 3))[:, :, ::s, ::s].max(axis=(-1, -2))
+        assert np.array_equal(got, O.quantize(win.astype(np.float32), sy, zy, O.U8))
+    # all-negative window at the border: the padding's 0 wins; in the interior it does not
+    neg = np.full((1, 1, 4, 4), 10, np.uint8)
+    out = O.qmaxpool(neg, (3, 3), (1, 1), ((1, 1), (1, 1)), 50, 0.1, 50, 0.1)
+    assert out[0, 0, 0, 0] == 50 and out[0, 0, 1, 1] == 10 and out[0, 0, 3, 2] == 50
