@@ -154,6 +154,41 @@ def side_workload(args):
                     roofline={"bound": "hbm", "achieved": round(nbytes / (sum(op_ms) * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                               "frac": round(nbytes / (sum(op_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None},
                     kernels={model.fn.op_kernel(i): round(t * 1e3, 2) for i, t in enumerate(op_ms)})
+    elif args.workload == "yolov5s":
+        batch, hw = 16, 640
+        rng = np.random.default_rng(7)
+        g = nb.yolov5s(seed=4, input_hw=hw)
+        qg = nb.quantize_graph(g, rng.random((2, hw, hw, 3), dtype=np.float32), calib_batch=1)
+        model = nb.HipModel(ctx, qg, batch, capture_graph=True)
+        x = rng.random((batch, hw, hw, 3), dtype=np.float32)
+        model.set_input(x)
+        ms = time_calls(ctx, model.invoke, args.warmup, args.steps)
+        op_ms = model.fn.profile(5)
+        names = [model.fn.op_kernel(i) for i in range(len(model.fn))]
+        macs = sum(qg.macs_per_image.values()) * batch
+        groups = {}
+        for nme, t in zip(names, op_ms):
+            key = nme.split("<")[0]
+            groups[key] = groups.get(key, 0.0) + t
+        conv_ms = sum(t for nme, t in zip(names, op_ms) if nme.startswith("qconv"))
+        # batch consistency: image 0 alone gives the same three head tensors
+        one = nb.HipModel(ctx, qg, 1, capture_graph=False)
+        one.run(x[:1])
+        model.invoke()
+        ctx.sync()
+        for a, b in zip(model.all_outputs(), one.all_outputs()):
+            if not np.array_equal(a[:1].view(np.uint32), b.view(np.uint32)):
+                sys.exit("bench.py: batch-16 head outputs of image 0 differ from its batch-1 outputs")
+        line = dict(base, metric="images/sec u8/u8 YOLOv5s 640x640 b16", value=round(batch / (ms * 1e-3), 1), unit="images/s",
+                    ms_per_step=round(ms, 4), dtype="u8",
+                    config={"workload": "config 4: YOLOv5s-style backbone + neck + head, 640x640, u8/u8 per-tensor PTQ (2 calibration "
+                                        "images), batch 16, SiLU as byte tables, " + str(len(model.fn)) + " operators, HIP-graph replay",
+                            "batch_consistent": True},
+                    roofline={"bound": "mfma", "achieved": round(2 * macs / (conv_ms * 1e-3) / 1e12, 1), "peak": INT8_PEAK_TOPS,
+                              "unit": "TOP/s", "frac": round(2 * macs / (conv_ms * 1e-3) / 1e12 / INT8_PEAK_TOPS, 4), "traffic": None,
+                              "note": "all convolutions together: int8 op count / summed conv kernel time"},
+                    sum_of_kernel_ms=round(sum(op_ms), 4),
+                    kernel_groups_ms={k: round(v, 4) for k, v in sorted(groups.items(), key=lambda kv: -kv[1])})
     elif args.workload == "paged_attention":
         rng = np.random.default_rng(5)
         bsz, hq, hkv, d, blk = 32, 14, 2, 64, 16
@@ -183,7 +218,7 @@ def side_workload(args):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--workload", default="mobilenetv2", help="mobilenetv2 (headline, default) | matmul | conv_block | paged_attention")
+    ap.add_argument("--workload", default="mobilenetv2", help="mobilenetv2 (headline, default) | matmul | conv_block | yolov5s | paged_attention")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)

@@ -166,6 +166,13 @@ typedef struct nncase_hip_conv2d_args {
     nncase_hip_quant_param_t residual_qp;
     nncase_hip_quant_param_t sum_qp;
     float sum_clamp_min, sum_clamp_max;
+    /* Optional fused unary operator (U8 output, dense kernels only): a 256-entry HOST table
+     * (nncase_hip_make_unary_lut) applied to the requantised byte,
+     *   y = post_lut[Q_y(conv)]   = Quantize(unary(Dequantize(conv result))) of the u8/u8 graph,
+     * before the residual add if there is one; post_lut_qp is the quant param of the table's
+     * output (used to dequantise it for the residual add).  The table is copied by the call. */
+    const uint8_t *post_lut_host;
+    nncase_hip_quant_param_t post_lut_qp;
 } nncase_hip_conv2d_args_t;
 
 /* Output is [batch, out_h, out_w, out_channels] with

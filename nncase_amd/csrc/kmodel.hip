@@ -231,16 +231,33 @@ extern "C" int nncase_hip_kmodel_load(nncase_hip_ctx_t *ctx, const void *data, s
                       "kmodel_load: tensor %d is written twice", o.output);
         producer[o.output] = (int)k;
     }
-    std::vector<int> fused_add(th.n_ops, -1); // conv op -> add op folded into it
+    // conv -> byte table -> residual add chains collapse into the dense conv's epilogue
+    std::vector<int> fused_add(th.n_ops, -1), fused_lut(th.n_ops, -1); // conv op -> add / table op folded into it
     std::vector<char> skipped(th.n_ops, 0);
+    auto is_output = [&](int32_t t) { return (uint32_t)t >= th.output_tensor && (uint32_t)t < th.output_tensor + n_outputs; };
+    auto dense_conv = [&](const hipf_op &c) {
+        const bool depthwise = c.p[4] > 1 && c.p[1] == 1;
+        return c.opcode == kOpConv2d && !depthwise && (int64_t)c.p[1] * c.p[4] > 4 && consumers[c.output] == 1 && !is_output(c.output);
+    };
     for (uint32_t k = 1; k < th.n_ops; k++) {
-        const hipf_op &add = ops[k], &conv = ops[k - 1];
-        if (add.opcode != kOpAdd || add.n_inputs != 2 || conv.opcode != kOpConv2d) continue;
-        const bool depthwise = conv.p[4] > 1 && conv.p[1] == 1;
-        const bool dense = !depthwise && (int64_t)conv.p[1] * conv.p[4] > 4;
-        if (dense && add.inputs[1] == conv.output && consumers[conv.output] == 1 && add.inputs[0] != conv.output &&
-            !((uint32_t)conv.output >= th.output_tensor && (uint32_t)conv.output < th.output_tensor + n_outputs)) {
-            fused_add[k - 1] = (int)k;
+        const hipf_op &lut = ops[k], &conv = ops[k - 1];
+        if (lut.opcode == kOpLut && lut.n_inputs == 1 && lut.inputs[0] == conv.output && dense_conv(conv)) {
+            fused_lut[k - 1] = (int)k;
+            skipped[k] = 1;
+        }
+    }
+    for (uint32_t k = 1; k < th.n_ops; k++) {
+        const hipf_op &add = ops[k];
+        if (add.opcode != kOpAdd || add.n_inputs != 2) continue;
+        // the producer of the second operand: a dense conv, or a table already folded into one
+        uint32_t c = k - 1;
+        if (skipped[c] && ops[c].opcode == kOpLut && c >= 1 && fused_lut[c - 1] == (int)c) c--;
+        const hipf_op &conv = ops[c];
+        const int32_t produced = fused_lut[c] >= 0 ? ops[fused_lut[c]].output : conv.output;
+        const bool ok_conv = fused_lut[c] >= 0 ? true : dense_conv(conv);
+        if (conv.opcode == kOpConv2d && ok_conv && add.inputs[1] == produced && consumers[produced] == 1 && !is_output(produced) &&
+            add.inputs[0] != produced && (fused_lut[c] >= 0 ? (uint32_t)fused_lut[c] == k - 1 : c == k - 1)) {
+            fused_add[c] = (int)k;
             skipped[k] = 1;
         }
     }
@@ -248,8 +265,10 @@ extern "C" int nncase_hip_kmodel_load(nncase_hip_ctx_t *ctx, const void *data, s
     // ---- device buffers ---------------------------------------------------------------------------
     m->buffers.assign(th.n_tensors, nullptr);
     m->owns.assign(th.n_tensors, 0);
-    for (uint32_t k = 0; k < th.n_ops; k++)
-        if (fused_add[k] >= 0) m->owns[ops[k].output] = 2; // never materialised
+    for (uint32_t k = 0; k < th.n_ops; k++) { // tensors that only exist inside a fused operator
+        if (fused_add[k] >= 0 || fused_lut[k] >= 0) m->owns[ops[k].output] = 2;
+        if (fused_add[k] >= 0 && fused_lut[k] >= 0) m->owns[ops[fused_lut[k]].output] = 2;
+    }
     for (uint32_t t = 0; t < th.n_tensors; t++) {
         if (m->owns[t] == 2) {
             m->owns[t] = 0;
@@ -316,6 +335,16 @@ extern "C" int nncase_hip_kmodel_load(nncase_hip_ctx_t *ctx, const void *data, s
                                    windowed_output_size(a.in_w, kw, a.stride_w, a.dilation_w, a.pad_w_before, a.pad_w_after) == (int)to.dims[2],
                           -NNCASE_HIP_ERR_SHAPE_MISMATCH, "kmodel_load: op %u conv output extent does not match its tensor", k);
             void *y = m->buffers[dst];
+            if (fused_lut[k] >= 0) {
+                const hipf_op &lut = ops[fused_lut[k]];
+                const uint8_t *table = rd(lut.rdata0, 256);
+                NNHIP_REQUIRE(ctx, table, -EINVAL, "kmodel_load: op %d table outside .rdata", fused_lut[k]);
+                NNHIP_REQUIRE(ctx, elems((uint32_t)lut.output) == elems(dst), -NNCASE_HIP_ERR_SHAPE_MISMATCH,
+                              "kmodel_load: op %d shapes differ", fused_lut[k]);
+                a.post_lut_host = table; // copied when the operator is recorded
+                a.post_lut_qp = tqp((uint32_t)lut.output);
+                y = m->buffers[lut.output];
+            }
             if (fused_add[k] >= 0) {
                 const hipf_op &add = ops[fused_add[k]];
                 const uint32_t res = (uint32_t)add.inputs[0], sum = (uint32_t)add.output;

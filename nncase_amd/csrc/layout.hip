@@ -48,6 +48,17 @@ template <typename T> __global__ __launch_bounds__(kLayoutThreads) void pack_ker
     out[gid] = ok ? in[off] : (T)0;
 }
 
+// out[row] = the `c` (<= 4) bytes of row `row`, zero-extended to a dword.
+__global__ __launch_bounds__(kLayoutThreads) void pad_bytes_to_dword_kernel(const uint8_t *__restrict__ in,
+                                                                          uint32_t *__restrict__ out, uint32_t rows, int c) {
+    const uint32_t r = blockIdx.x * kLayoutThreads + threadIdx.x;
+    if (r >= rows) return;
+    const uint8_t *p = in + (size_t)r * c;
+    uint32_t v = 0;
+    for (int i = 0; i < c; i++) v |= (uint32_t)p[i] << (8 * i);
+    out[r] = v;
+}
+
 template <typename T> __global__ __launch_bounds__(kLayoutThreads) void unpack_kernel(const T *in, T *out, const PackDesc d) {
     const uint64_t gid = (uint64_t)blockIdx.x * kLayoutThreads + threadIdx.x;
     if (gid >= d.total) return;
@@ -136,6 +147,20 @@ extern "C" int nncase_hip_pack(nncase_hip_ctx_t *ctx, const void *in_dev, void *
     int nax[kMaxRank];
     int rc = build_common(ctx, rank, shape, n_axes, axes, lanes, nax);
     if (rc) return rc;
+    // Padding the innermost axis of bytes to one 4-byte lane block (RGB -> RGBX in front of a conv):
+    // one thread per pixel, a dword store.
+    if (elem_size == 1 && n_axes == 1 && nax[0] == rank - 1 && lanes[0] == 4 && shape[rank - 1] <= 4 &&
+        (reinterpret_cast<uintptr_t>(out_dev) & 3u) == 0) {
+        uint64_t rows = 1;
+        for (int i = 0; i < rank - 1; i++) rows *= (uint64_t)shape[i];
+        NNHIP_REQUIRE(ctx, rows < ((uint64_t)1 << 31), -EINVAL, "pack: tensor too large");
+        if (rows == 0) return 0;
+        hipLaunchKernelGGL(pad_bytes_to_dword_kernel, dim3((unsigned)((rows + kLayoutThreads - 1) / kLayoutThreads)),
+                           dim3(kLayoutThreads), 0, ctx->stream, (const uint8_t *)in_dev, (uint32_t *)out_dev, (uint32_t)rows,
+                           (int)shape[rank - 1]);
+        NNHIP_LAUNCH_CHECK(ctx, "pad_bytes_to_dword_kernel");
+        return 0;
+    }
     PackDesc d;
     memset(&d, 0, sizeof(d));
     d.in_rank = rank;

@@ -22,7 +22,7 @@ void nnhip::describe_conv_kernel(const nncase_hip_ctx *ctx, const nncase_hip_wei
         else snprintf(buf, cap, "dw_generic<VEC=%d>", w->out_channels % 4 == 0 ? 4 : 1);
         return;
     }
-    if (w->d_smallc && a->dilation_h == 1 && a->dilation_w == 1 && !a->residual_dev) {
+    if (w->d_smallc && a->dilation_h == 1 && a->dilation_w == 1 && !a->residual_dev && !a->post_lut_host) {
         snprintf(buf, cap, "qconv_smallc<C=%d>", w->in_channels);
         return;
     }
@@ -30,7 +30,7 @@ void nnhip::describe_conv_kernel(const nncase_hip_ctx *ctx, const nncase_hip_wei
     const int out_h = windowed_output_size(a->in_h, w->kernel_h, a->stride_h, a->dilation_h, a->pad_h_before, a->pad_h_after);
     const int out_w = windowed_output_size(a->in_w, w->kernel_w, a->stride_w, a->dilation_w, a->pad_w_before, a->pad_w_after);
     const long long m = (long long)a->batch * out_h * out_w;
-    snprintf(buf, cap, "qconv_igemm%s<T=%d,RG=%d,%s>", a->residual_dev ? "+add" : "", w->tiles, igemm_pixel_groups(ctx, w, (int)std::min<long long>(m, 1 << 30)),
+    snprintf(buf, cap, "qconv_igemm%s%s<T=%d,RG=%d,%s>", a->post_lut_host ? "+lut" : "", a->residual_dev ? "+add" : "", w->tiles, igemm_pixel_groups(ctx, w, (int)std::min<long long>(m, 1 << 30)),
              modes[igemm_load_mode(w, a, out_h, out_w)]);
 }
 
@@ -91,8 +91,10 @@ int nnhip::make_residual_epilogue(nncase_hip_ctx *ctx, ResidualEpilogue *rep, co
     NNHIP_REQUIRE(ctx, std::isfinite(c->y_qp.scale) && std::isfinite(c->residual_qp.scale) &&
                            std::fabs(c->y_qp.scale) <= 0x1p20f && std::fabs(c->residual_qp.scale) <= 0x1p20f,
                   -ERANGE, "qconv2d: residual input scale outside the supported range");
-    rep->zy = (float)c->y_qp.zero_point;
-    rep->sy = c->y_qp.scale;
+    // the residual stage dequantises what the first stage produced: the table's output if there is one
+    const nncase_hip_quant_param_t own = c->post_lut_host ? c->post_lut_qp : c->y_qp;
+    rep->zy = (float)own.zero_point;
+    rep->sy = own.scale;
     rep->zr = (float)c->residual_qp.zero_point;
     rep->sr = c->residual_qp.scale;
     return make_epilogue(ctx, &rep->sum, 1.f, 1.f, c->sum_qp, c->sum_clamp_min, c->sum_clamp_max, NNCASE_HIP_DT_U8,
@@ -183,11 +185,15 @@ extern "C" int nncase_hip_qconv2d(nncase_hip_ctx_t *ctx, const uint8_t *x_dev, c
     const int out_h = windowed_output_size(a->in_h, w->kernel_h, a->stride_h, a->dilation_h, a->pad_h_before, a->pad_h_after);
     const int out_w = windowed_output_size(a->in_w, w->kernel_w, a->stride_w, a->dilation_w, a->pad_w_before, a->pad_w_after);
     NNHIP_REQUIRE(ctx, out_h > 0 && out_w > 0, -NNCASE_HIP_ERR_SHAPE_MISMATCH, "qconv2d: window larger than padded input");
-    if (a->residual_dev) {
-        rc = check_out_dtype(ctx, NNCASE_HIP_DT_U8, a->sum_qp, "qconv2d(residual)");
-        if (rc) return rc;
+    if (a->residual_dev || a->post_lut_host) {
+        if (a->residual_dev) {
+            rc = check_out_dtype(ctx, NNCASE_HIP_DT_U8, a->sum_qp, "qconv2d(residual)");
+            if (rc) return rc;
+        }
+        NNHIP_REQUIRE(ctx, a->out_dtype == NNCASE_HIP_DT_U8, -NNCASE_HIP_ERR_DATATYPE_MISMATCH,
+                      "qconv2d: a fused table or residual needs u8 output");
         NNHIP_REQUIRE(ctx, w->kind == nncase_hip_weights::kIgemm, -EINVAL,
-                      "qconv2d: a fused residual is only supported by the dense (MFMA) kernels");
+                      "qconv2d: a fused table or residual is only supported by the dense (MFMA) kernels");
         return launch_qconv_igemm(ctx, x_dev, w, y_dev, a, out_h, out_w);
     }
     if (w->kind == nncase_hip_weights::kDepthwise) return launch_qconv_depthwise(ctx, x_dev, w, y_dev, a, out_h, out_w);

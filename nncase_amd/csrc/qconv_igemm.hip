@@ -170,6 +170,10 @@ int launch_qconv_igemm(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_hip_w
         const int rc = make_residual_epilogue(ctx, &a.rep, c);
         if (rc) return rc;
     }
+    if (c->post_lut_host) {
+        a.use_lut = 1;
+        memcpy(a.lut, c->post_lut_host, 256);
+    }
     const int mode = igemm_load_mode(w, c, out_h, out_w);
 
     const size_t group_bytes = (size_t)w->nchunks * w->ksteps * w->tiles * 1024;

@@ -68,6 +68,8 @@ struct IgemmArgs {
     int num_mtiles;
     Epilogue ep;
     ResidualEpilogue rep;
+    int use_lut;           // apply `lut` to the requantised byte (before the residual add)
+    uint32_t lut[64];
 };
 
 struct PixInfo {
@@ -200,7 +202,8 @@ template <int T, int RG, int MODE>
 __global__ __launch_bounds__(kThreads, 2) void qconv_igemm_kernel(const IgemmArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     int32_t *cterm = reinterpret_cast<int32_t *>(smem); // [T * 16]
-    uint8_t *wlds = smem + T * 16 * sizeof(int32_t);    // [kc_steps][T][1024]
+    uint8_t *lutl = smem + T * 16 * sizeof(int32_t);    // [256] byte table of the fused unary operator
+    uint8_t *wlds = lutl + 256;                         // [kc_steps][T][1024]
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -219,6 +222,7 @@ __global__ __launch_bounds__(kThreads, 2) void qconv_igemm_kernel(const IgemmArg
         if (ch < a.n) c = a.bias[ch] - a.zxp * a.wsum[ch] + a.k * a.zxp * a.zwp;
         cterm[i] = c;
     }
+    if (a.use_lut && threadIdx.x < 64) reinterpret_cast<uint32_t *>(lutl)[threadIdx.x] = a.lut[threadIdx.x];
     auto stage_weights = [&](int kci) {
         const int s0 = kci * a.kc_steps;
         const int steps = min(a.kc_steps, a.ksteps - s0);
@@ -320,6 +324,14 @@ __global__ __launch_bounds__(kThreads, 2) void qconv_igemm_kernel(const IgemmArg
                         }
                         packed[nt] = pack_low_bytes(b[0], b[1], b[2], b[3]);
                     }
+                    if (a.use_lut) { // fused unary operator: one LDS byte read per output
+#pragma unroll
+                        for (int nt = 0; nt < T; nt++) {
+                            const uint32_t v = packed[nt];
+                            packed[nt] = (uint32_t)lutl[v & 0xffu] | ((uint32_t)lutl[(v >> 8) & 0xffu] << 8) |
+                                         ((uint32_t)lutl[(v >> 16) & 0xffu] << 16) | ((uint32_t)lutl[v >> 24] << 24);
+                        }
+                    }
                     if (a.rep.res) { // fused residual add on the requantised bytes
                         const uint8_t *ro = a.rep.res + obase;
                         const bool whole = ((a.ldy | a.y_coff) & 3) == 0 && ch0 + 4 * T <= a.n;
@@ -409,7 +421,7 @@ template <int T, int RG, int MODE> int launch_trg(nncase_hip_ctx *ctx, const Ige
     // columns the blocks that share a pixel tile (same x, different chunk) land on
     // one XCD and find the activations in its L2.
     if (nchunks > 1) gx = ceil_div(gx, 8) * 8;
-    const size_t lds = (size_t)T * 16 * sizeof(int32_t) + (size_t)a.kc_steps * T * 1024;
+    const size_t lds = (size_t)T * 16 * sizeof(int32_t) + 256 + (size_t)a.kc_steps * T * 1024;
     hipLaunchKernelGGL((qconv_igemm_kernel<T, RG, MODE>), dim3(gx, nchunks, 1), dim3(kThreads), lds, ctx->stream, args);
     NNHIP_LAUNCH_CHECK(ctx, "qconv_igemm_kernel");
     return 0;

@@ -361,20 +361,39 @@ class HipModel:
         for n in qg.nodes:
             for j in n.inputs:
                 consumers[j] += 1
+        # A byte-table node (swish) whose only producer is a dense conv consumed by nothing else is applied in
+        # that conv's epilogue; a residual add can then still be folded behind it.  Tensors that only exist
+        # inside a fused operator are never written (materialized() is False for them).
+        def dense_conv(j):
+            nj = qg.nodes[j]
+            return (nj.op == "conv" and not (nj.groups > 1 and nj.weights.shape[1] == 1) and nj.weights.shape[1] * nj.groups > 4
+                    and consumers[j] == 1 and j not in qg.output_nodes)
+        self.fused_lut: Dict[int, int] = {}    # conv node -> lut node
         self.fused_into: Dict[int, int] = {}   # conv node -> add node
         if fuse_residual:
             for i, n in enumerate(qg.nodes):
+                if n.op == "lut" and n.inputs[0] == i - 1 and dense_conv(i - 1):
+                    self.fused_lut[i - 1] = i
+            lut_owner = {v: k for k, v in self.fused_lut.items()}
+            for i, n in enumerate(qg.nodes):
                 if n.op == "add":
                     a, b = n.inputs
-                    nb_ = qg.nodes[b]
-                    dense = nb_.op == "conv" and not (nb_.groups > 1 and nb_.weights.shape[1] == 1) and nb_.weights.shape[1] * nb_.groups > 4
-                    if dense and consumers[b] == 1 and b == i - 1 and a < b and b not in qg.output_nodes:
-                        self.fused_into[b] = i
+                    conv = lut_owner.get(b, b)                      # the conv that produces operand b
+                    last = self.fused_lut.get(conv, conv)           # ... and the last node fused into it so far
+                    if last == b == i - 1 and a < conv and consumers[b] == 1 and b not in qg.output_nodes and \
+                            (b in lut_owner or dense_conv(b)):
+                        self.fused_into[conv] = i
+        self.never_written = set(self.fused_into.keys()) | set(self.fused_lut.keys())
+        for conv, add in self.fused_into.items():
+            if conv in self.fused_lut:
+                self.never_written.add(self.fused_lut[conv])
+        skip_nodes = set(self.fused_into.values()) | set(self.fused_lut.values())
         for i, n in enumerate(qg.nodes):
             cc, hh, ww = n.out_shape
             fused_add = self.fused_into.get(i)
-            if n.op == "add" and i in self.fused_into.values():
-                self.buffers.append(self.buffers[i - 1])  # written by the fused conv
+            fused_lut = self.fused_lut.get(i)
+            if i in skip_nodes:
+                self.buffers.append(self.buffers[i - 1])  # written by the conv it is fused into
                 self.weights.append(None)
                 continue
             buf = ctx.alloc(batch * cc * hh * ww)
@@ -389,6 +408,8 @@ class HipModel:
                 (ph0, ph1), (pw0, pw1) = n.padding
                 args = rt.Conv2dArgs(batch, src.out_shape[1], src.out_shape[2], n.stride[0], n.stride[1], 1, 1, ph0, ph1, pw0,
                                      pw1, qp(*src.out_qp), qp(*n.out_qp), n.clamp[0], n.clamp[1], rt.DT_U8)
+                if fused_lut is not None:
+                    args.set_post_lut(qg.nodes[fused_lut].lut, qp(*qg.nodes[fused_lut].out_qp))
                 if fused_add is not None:
                     add = qg.nodes[fused_add]
                     res_node = add.inputs[0]
@@ -426,8 +447,8 @@ class HipModel:
                                             src.out_shape[0], qp(*src.out_qp), qp(*n.out_qp))
             else:
                 raise ValueError(n.op)
-            self.op_names.append(f"{n.op}:{n.name}" + ("+add" if fused_add is not None else ""))
-            self.op_nodes.append(i if fused_add is None else fused_add)
+            self.op_names.append(f"{n.op}:{n.name}" + ("+lut" if fused_lut is not None else "") + ("+add" if fused_add is not None else ""))
+            self.op_nodes.append(fused_add if fused_add is not None else (fused_lut if fused_lut is not None else i))
         self.outputs_f32: List[rt.DeviceBuffer] = []
         for j in qg.output_nodes:
             node = qg.nodes[j]
@@ -462,13 +483,13 @@ class HipModel:
         return [self.output(i) for i in range(len(self.outputs_f32))]
 
     def materialized(self, node: int) -> bool:
-        """False for a conv whose output only exists inside a fused residual add."""
-        return node not in self.fused_into
+        """False for a tensor that only exists inside a fused operator (conv + table + residual add)."""
+        return node not in self.never_written
 
     def tensor(self, node: int) -> np.ndarray:
         """u8 output of a node as NCHW (for layer-by-layer parity checks)."""
         if not self.materialized(node):
-            raise ValueError(f"node {node} is fused into node {self.fused_into[node]} and never written")
+            raise ValueError(f"node {node} only exists inside a fused operator and is never written")
         c, h, w = self.qg.nodes[node].out_shape
         y = self.buffers[node].download((self.batch, h, w, c), np.uint8)
         return np.ascontiguousarray(y.transpose(0, 3, 1, 2))

@@ -8,6 +8,7 @@ from __future__ import annotations
 
 import ctypes as C
 import errno
+import weakref
 import os
 from typing import Optional, Sequence, Tuple
 
@@ -49,7 +50,16 @@ class Conv2dArgs(C.Structure):
                 ("x_qp", QuantParam), ("y_qp", QuantParam),
                 ("clamp_min", C.c_float), ("clamp_max", C.c_float), ("out_dtype", C.c_int32),
                 ("residual_dev", C.c_void_p), ("residual_qp", QuantParam), ("sum_qp", QuantParam),
-                ("sum_clamp_min", C.c_float), ("sum_clamp_max", C.c_float)]
+                ("sum_clamp_min", C.c_float), ("sum_clamp_max", C.c_float),
+                ("post_lut_host", C.c_void_p), ("post_lut_qp", QuantParam)]
+
+    def set_post_lut(self, lut: np.ndarray, lut_qp: "QuantParam"):
+        """Fuses a 256-entry byte table (make_unary_lut) behind the requantisation; the table is copied
+        by the call that consumes these arguments, the array only has to live until then."""
+        self._lut = np.ascontiguousarray(lut, np.uint8)
+        assert self._lut.size == 256
+        self.post_lut_host = self._lut.ctypes.data
+        self.post_lut_qp = lut_qp
 
 
 class MatmulArgs(C.Structure):
@@ -209,7 +219,8 @@ class DeviceBuffer:
 
     def free(self):
         if self.ptr:
-            self.ctx.lib.nncase_hip_free(self.ctx.handle, self.ptr)
+            if self.ctx.handle:
+                self.ctx.lib.nncase_hip_free(self.ctx.handle, self.ptr)
             self.ptr = None
 
     def __del__(self):
@@ -228,7 +239,8 @@ class Weights:
 
     def destroy(self):
         if self.handle:
-            self.ctx.lib.nncase_hip_weights_destroy(self.ctx.handle, self.handle)
+            if self.ctx.handle:
+                self.ctx.lib.nncase_hip_weights_destroy(self.ctx.handle, self.handle)
             self.handle = None
 
     def __del__(self):
@@ -264,8 +276,16 @@ class Context:
             msg = self.lib.nncase_hip_last_error_string(self.handle)
             raise HipError(rc, where, msg.decode() if msg else "")
 
+    def _adopt(self, child):
+        """Functions and loaded kmodels hold a pointer to the native context: they are destroyed with it."""
+        if not hasattr(self, "_children"):
+            self._children = weakref.WeakSet()
+        self._children.add(child)
+
     def close(self):
         if getattr(self, "handle", None):
+            for child in list(getattr(self, "_children", ())):
+                child.destroy()
             self.lib.nncase_hip_ctx_destroy(self.handle)
             self.handle = None
 
@@ -394,6 +414,7 @@ class Function:
         ctx._check(ctx.lib.nncase_hip_function_create(ctx.handle, C.byref(h)), "function_create")
         self.handle = h.value
         self._keep = []  # operands must outlive the function
+        ctx._adopt(self)
 
     def _ck(self, rc, where):
         self.ctx._check(rc, where)
@@ -484,7 +505,8 @@ class Function:
 
     def destroy(self):
         if self.handle:
-            self.ctx.lib.nncase_hip_function_destroy(self.handle)
+            if self.ctx.handle:  # a function of a closed context went with it
+                self.ctx.lib.nncase_hip_function_destroy(self.handle)
             self.handle = None
 
     def __del__(self):
@@ -525,6 +547,7 @@ class LoadedKModel:
         buf = (C.c_char * len(data)).from_buffer_copy(data)
         ctx._check(ctx.lib.nncase_hip_kmodel_load(ctx.handle, C.cast(buf, C.c_void_p), len(data), C.byref(h)), "kmodel_load")
         self.handle = h.value
+        ctx._adopt(self)
         f = C.c_void_p()
         ctx._check(ctx.lib.nncase_hip_kmodel_function(self.handle, C.byref(f)), "kmodel_function")
         self.fn = _BorrowedFunction(ctx, f.value)
@@ -556,7 +579,8 @@ class LoadedKModel:
 
     def destroy(self):
         if self.handle:
-            self.ctx.lib.nncase_hip_kmodel_destroy(self.handle)
+            if self.ctx.handle:
+                self.ctx.lib.nncase_hip_kmodel_destroy(self.handle)
             self.handle = None
 
     def __del__(self):

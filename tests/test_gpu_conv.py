@@ -318,3 +318,32 @@ def test_fused_residual_equals_conv_then_add(hip_ctx, cin, cout, hw, k):
                    residual=res, residual_qp=qp(99, 0.031), sum_qp=qp(101, float(sy) * 1.3))
     assert np.array_equal(got, want)
     assert len(np.unique(want)) > 16
+
+
+@pytest.mark.parametrize("cin,cout,hw,k,with_residual", [(64, 32, 12, 1, False), (32, 32, 9, 3, True), (128, 255, 5, 1, False),
+                                                         (4, 32, 20, 6, False), (256, 128, 7, 3, True)])
+def test_fused_table_equals_conv_then_table(hip_ctx, cin, cout, hw, k, with_residual):
+    """conv with a fused swish table (and a residual add behind it) == conv, then the table, then the add."""
+    rng = np.random.default_rng(cin + cout + k)
+    x = rng.integers(0, 256, (2, cin, hw, hw), dtype=np.uint8)
+    w = rng.integers(0, 256, (cout, cin, k, k), dtype=np.uint8)
+    bias = rng.integers(-2000, 2000, cout).astype(np.int32)
+    pad = ((k // 2, k // 2), (k // 2, k // 2)) if k != 6 else ((2, 2), (2, 2))
+    stride = (2, 2) if k == 6 else (1, 1)
+    zx, sx, zw, sw = 9, f32(0.031), 127, f32(0.004)
+    real = O.qconv2d(x, w, bias, zx, sx, zw, sw, stride=stride, padding=pad, out_mode=O.OUT_F32)
+    sy = f32((real.max() - real.min()) / 255)
+    zy = int(np.clip(np.rint(-real.min() / sy), 0, 255))
+    y = O.qconv2d(x, w, bias, zx, sx, zw, sw, zy, sy, stride=stride, padding=pad, out_mode=O.OUT_U8)
+    lz, ls = 18, f32(sy * 0.9)
+    lut = O.unary_lut(O.LUT_SWISH, zy, sy, lz, ls)
+    want = lut[y]
+    kw = {}
+    if with_residual:
+        r = rng.integers(0, 256, y.shape, dtype=np.uint8)
+        rq, sq = (77, f32(0.02)), (40, f32(ls * 1.3))
+        want = O.qadd(want, r, lz, ls, rq[0], rq[1], sq[0], sq[1])
+        kw = dict(residual=r, residual_qp=qp(*rq), sum_qp=qp(*sq))
+    got = K.conv2d(x, w, bias, stride, pad, (1, 1), 1, FULL, qp(zx, sx), qp(zw, sw), qp(zy, sy), np.uint8, ctx=hip_ctx,
+                   post_lut=rt.make_unary_lut(rt.LUT_SWISH, qp(zy, sy), qp(lz, ls)), post_lut_qp=qp(lz, ls), **kw)
+    assert np.array_equal(got, want), f"{(got != want).sum()} of {want.size} bytes differ"

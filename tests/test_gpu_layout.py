@@ -16,6 +16,9 @@ pytestmark = pytest.mark.gpu
     ((3, 1, 17), [2], [8], np.float16),
     ((7,), [0], [16], np.int32),
     ((2, 3, 4, 5, 6), [-1, 1], [4, 2], np.uint8),
+    ((2, 9, 11, 3), [3], [4], np.uint8),           # RGB -> RGBX: the dword fast path
+    ((5, 7, 1), [2], [4], np.uint8),
+    ((4, 6, 4), [-1], [4], np.uint8),              # already 4 wide
 ])
 def test_pack_unpack(hip_ctx, shape, axes, lanes, dtype):
     rng = np.random.default_rng(len(shape) + shape[0])
