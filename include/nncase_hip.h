@@ -147,6 +147,14 @@ NNCASE_HIP_API int nncase_hip_qconv2d_prepack(nncase_hip_ctx_t *ctx, const nncas
                                               const uint8_t *weights_oihw_host, const int32_t *bias_host,
                                               nncase_hip_weights_t **weights);
 NNCASE_HIP_API int nncase_hip_weights_destroy(nncase_hip_ctx_t *ctx, nncase_hip_weights_t *weights);
+/* Attaches a fused unary operator to pre-packed dense (non-depthwise) weights:
+ * a 256-entry host table (nncase_hip_make_unary_lut) that every u8-output call applies to the
+ * requantised byte,  y = table[Q_y(conv)]  = Quantize(unary(Dequantize(conv result))) of the
+ * u8/u8 graph, before the residual add if the call has one; table_qp is the quant param of the
+ * table's output (the residual stage dequantises with it).  The activation that follows a
+ * convolution is as static as its weights, so it is uploaded once with them.  NULL detaches. */
+NNCASE_HIP_API int nncase_hip_weights_set_post_lut(nncase_hip_ctx_t *ctx, nncase_hip_weights_t *weights,
+                                                   const uint8_t *lut256_host, nncase_hip_quant_param_t table_qp);
 
 typedef struct nncase_hip_conv2d_args {
     int32_t batch, in_h, in_w;           /* input is [batch, in_h, in_w, in_channels] u8   */
@@ -166,13 +174,6 @@ typedef struct nncase_hip_conv2d_args {
     nncase_hip_quant_param_t residual_qp;
     nncase_hip_quant_param_t sum_qp;
     float sum_clamp_min, sum_clamp_max;
-    /* Optional fused unary operator (U8 output, dense kernels only): a 256-entry HOST table
-     * (nncase_hip_make_unary_lut) applied to the requantised byte,
-     *   y = post_lut[Q_y(conv)]   = Quantize(unary(Dequantize(conv result))) of the u8/u8 graph,
-     * before the residual add if there is one; post_lut_qp is the quant param of the table's
-     * output (used to dequantise it for the residual add).  The table is copied by the call. */
-    const uint8_t *post_lut_host;
-    nncase_hip_quant_param_t post_lut_qp;
 } nncase_hip_conv2d_args_t;
 
 /* Output is [batch, out_h, out_w, out_channels] with

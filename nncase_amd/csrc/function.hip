@@ -48,11 +48,8 @@ static int run_op(nncase_hip_function *fn, const Op &op) {
         return nncase_hip_quantize(ctx, op.in0, op.dt_in, op.out, op.dt_out, op.count, op.qp0);
     case Op::kDequantize:
         return nncase_hip_dequantize(ctx, op.in0, op.dt_in, op.out, op.dt_out, op.count, op.qp0);
-    case Op::kConv: {
-        nncase_hip_conv2d_args_t c = op.conv;
-        if (c.post_lut_host) c.post_lut_host = op.lut; // the op owns a copy of the table
-        return nncase_hip_qconv2d(ctx, (const uint8_t *)op.in0, op.weights, op.out, &c);
-    }
+    case Op::kConv:
+        return nncase_hip_qconv2d(ctx, (const uint8_t *)op.in0, op.weights, op.out, &op.conv);
     case Op::kAdd:
         return nncase_hip_qadd(ctx, (const uint8_t *)op.in0, op.qp0, (const uint8_t *)op.in1, op.qp1, (uint8_t *)op.out,
                                op.qp2, op.lo, op.hi, op.count);
@@ -136,7 +133,6 @@ extern "C" int nncase_hip_function_add_qconv2d(nncase_hip_function_t *fn, const 
     Op op;
     op.kind = Op::kConv;
     op.in0 = x_dev, op.out = y_dev, op.weights = weights, op.conv = *args;
-    if (args->post_lut_host) memcpy(op.lut, args->post_lut_host, 256);
     return push(fn, op);
 }
 
@@ -295,7 +291,7 @@ extern "C" int nncase_hip_function_op_kernel(nncase_hip_function_t *fn, int32_t 
     switch (op.kind) {
     case Op::kQuantize: snprintf(name, capacity, "quantize"); break;
     case Op::kDequantize: snprintf(name, capacity, "dequantize"); break;
-    case Op::kConv: describe_conv_kernel(fn->ctx, op.weights, &op.conv, name, capacity); break; // reads only the pointer's presence
+    case Op::kConv: describe_conv_kernel(fn->ctx, op.weights, &op.conv, name, capacity); break;
     case Op::kAdd: snprintf(name, capacity, "qadd"); break;
     case Op::kPool: snprintf(name, capacity, "qglobal_avgpool"); break;
     case Op::kLut: snprintf(name, capacity, "lut_u8"); break;

@@ -341,8 +341,8 @@ extern "C" int nncase_hip_kmodel_load(nncase_hip_ctx_t *ctx, const void *data, s
                 NNHIP_REQUIRE(ctx, table, -EINVAL, "kmodel_load: op %d table outside .rdata", fused_lut[k]);
                 NNHIP_REQUIRE(ctx, elems((uint32_t)lut.output) == elems(dst), -NNCASE_HIP_ERR_SHAPE_MISMATCH,
                               "kmodel_load: op %d shapes differ", fused_lut[k]);
-                a.post_lut_host = table; // copied when the operator is recorded
-                a.post_lut_qp = tqp((uint32_t)lut.output);
+                rc = nncase_hip_weights_set_post_lut(ctx, wt, table, tqp((uint32_t)lut.output));
+                if (rc) return rc;
                 y = m->buffers[lut.output];
             }
             if (fused_add[k] >= 0) {

@@ -22,7 +22,7 @@ void nnhip::describe_conv_kernel(const nncase_hip_ctx *ctx, const nncase_hip_wei
         else snprintf(buf, cap, "dw_generic<VEC=%d>", w->out_channels % 4 == 0 ? 4 : 1);
         return;
     }
-    if (w->d_smallc && a->dilation_h == 1 && a->dilation_w == 1 && !a->residual_dev && !a->post_lut_host) {
+    if (w->d_smallc && a->dilation_h == 1 && a->dilation_w == 1 && !a->residual_dev) {
         snprintf(buf, cap, "qconv_smallc<C=%d>", w->in_channels);
         return;
     }
@@ -30,8 +30,12 @@ void nnhip::describe_conv_kernel(const nncase_hip_ctx *ctx, const nncase_hip_wei
     const int out_h = windowed_output_size(a->in_h, w->kernel_h, a->stride_h, a->dilation_h, a->pad_h_before, a->pad_h_after);
     const int out_w = windowed_output_size(a->in_w, w->kernel_w, a->stride_w, a->dilation_w, a->pad_w_before, a->pad_w_after);
     const long long m = (long long)a->batch * out_h * out_w;
-    snprintf(buf, cap, "qconv_igemm%s%s<T=%d,RG=%d,%s>", a->post_lut_host ? "+lut" : "", a->residual_dev ? "+add" : "", w->tiles, igemm_pixel_groups(ctx, w, (int)std::min<long long>(m, 1 << 30)),
-             modes[igemm_load_mode(w, a, out_h, out_w)]);
+    const int mode = igemm_load_mode(w, a, out_h, out_w);
+    const int mi = (int)std::min<long long>(m, 1 << 30);
+    const bool stream = igemm_streams_weights(w, mode);
+    snprintf(buf, cap, "qconv_igemm%s%s%s<T=%d,RG=%d,%s>", stream ? "_stream" : "", w->d_post_lut ? "+lut" : "",
+             a->residual_dev ? "+add" : "", w->tiles, stream ? stream_pixel_groups(ctx, w, mi) : igemm_pixel_groups(ctx, w, mi),
+             modes[mode]);
 }
 
 float nnhip::reciprocal_rn(float b) {
@@ -80,7 +84,8 @@ int nnhip::make_epilogue(nncase_hip_ctx *ctx, Epilogue *ep, float sx, float sw, 
     return 0;
 }
 
-int nnhip::make_residual_epilogue(nncase_hip_ctx *ctx, ResidualEpilogue *rep, const nncase_hip_conv2d_args_t *c) {
+int nnhip::make_residual_epilogue(nncase_hip_ctx *ctx, ResidualEpilogue *rep, const nncase_hip_conv2d_args_t *c,
+                                  const nncase_hip_weights *w) {
     memset(rep, 0, sizeof(*rep));
     rep->res = c->residual_dev;
     if (!c->residual_dev) return 0;
@@ -92,7 +97,7 @@ int nnhip::make_residual_epilogue(nncase_hip_ctx *ctx, ResidualEpilogue *rep, co
                            std::fabs(c->y_qp.scale) <= 0x1p20f && std::fabs(c->residual_qp.scale) <= 0x1p20f,
                   -ERANGE, "qconv2d: residual input scale outside the supported range");
     // the residual stage dequantises what the first stage produced: the table's output if there is one
-    const nncase_hip_quant_param_t own = c->post_lut_host ? c->post_lut_qp : c->y_qp;
+    const nncase_hip_quant_param_t own = (w && w->d_post_lut) ? w->post_lut_qp : c->y_qp;
     rep->zy = (float)own.zero_point;
     rep->sy = own.scale;
     rep->zr = (float)c->residual_qp.zero_point;
@@ -107,6 +112,7 @@ static void free_weights(nncase_hip_weights *w) {
     if (w->d_wsum) (void)hipFree(w->d_wsum);
     if (w->d_bias) (void)hipFree(w->d_bias);
     if (w->d_smallc) (void)hipFree(w->d_smallc);
+    if (w->d_post_lut) (void)hipFree(w->d_post_lut);
     delete w;
 }
 
@@ -158,6 +164,24 @@ extern "C" int nncase_hip_weights_destroy(nncase_hip_ctx_t *ctx, nncase_hip_weig
     return 0;
 }
 
+extern "C" int nncase_hip_weights_set_post_lut(nncase_hip_ctx_t *ctx, nncase_hip_weights_t *w, const uint8_t *lut256_host,
+                                               nncase_hip_quant_param_t table_qp) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, w, -EINVAL, "weights_set_post_lut: null weights");
+    NNHIP_HIP(ctx, hipStreamSynchronize(ctx->stream)); // earlier launches may still read the old table
+    if (!lut256_host) {
+        if (w->d_post_lut) (void)hipFree(w->d_post_lut);
+        w->d_post_lut = nullptr;
+        return 0;
+    }
+    NNHIP_REQUIRE(ctx, w->kind == nncase_hip_weights::kIgemm, -EINVAL,
+                  "weights_set_post_lut: a fused table is only supported by the dense (MFMA) kernels");
+    if (!w->d_post_lut) NNHIP_HIP(ctx, hipMalloc((void **)&w->d_post_lut, 256));
+    NNHIP_HIP(ctx, hipMemcpy(w->d_post_lut, lut256_host, 256, hipMemcpyHostToDevice));
+    w->post_lut_qp = table_qp;
+    return 0;
+}
+
 static int check_out_dtype(nncase_hip_ctx *ctx, int dt, nncase_hip_quant_param_t y_qp, const char *who) {
     NNHIP_REQUIRE(ctx, dt == NNCASE_HIP_DT_U8 || dt == NNCASE_HIP_DT_I32 || dt == NNCASE_HIP_DT_F32,
                   -NNCASE_HIP_ERR_DATATYPE_MISMATCH, "%s: unsupported output type 0x%x", who, dt);
@@ -185,13 +209,13 @@ extern "C" int nncase_hip_qconv2d(nncase_hip_ctx_t *ctx, const uint8_t *x_dev, c
     const int out_h = windowed_output_size(a->in_h, w->kernel_h, a->stride_h, a->dilation_h, a->pad_h_before, a->pad_h_after);
     const int out_w = windowed_output_size(a->in_w, w->kernel_w, a->stride_w, a->dilation_w, a->pad_w_before, a->pad_w_after);
     NNHIP_REQUIRE(ctx, out_h > 0 && out_w > 0, -NNCASE_HIP_ERR_SHAPE_MISMATCH, "qconv2d: window larger than padded input");
-    if (a->residual_dev || a->post_lut_host) {
+    if (a->residual_dev || w->d_post_lut) {
         if (a->residual_dev) {
             rc = check_out_dtype(ctx, NNCASE_HIP_DT_U8, a->sum_qp, "qconv2d(residual)");
             if (rc) return rc;
+            NNHIP_REQUIRE(ctx, a->out_dtype == NNCASE_HIP_DT_U8, -NNCASE_HIP_ERR_DATATYPE_MISMATCH,
+                          "qconv2d: a fused residual needs u8 output");
         }
-        NNHIP_REQUIRE(ctx, a->out_dtype == NNCASE_HIP_DT_U8, -NNCASE_HIP_ERR_DATATYPE_MISMATCH,
-                      "qconv2d: a fused table or residual needs u8 output");
         NNHIP_REQUIRE(ctx, w->kind == nncase_hip_weights::kIgemm, -EINVAL,
                       "qconv2d: a fused table or residual is only supported by the dense (MFMA) kernels");
         return launch_qconv_igemm(ctx, x_dev, w, y_dev, a, out_h, out_w);

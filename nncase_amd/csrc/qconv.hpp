@@ -19,6 +19,8 @@ struct nncase_hip_weights {
     // igemm: [groups][nchunks][ksteps][tiles] fragments of 1024 bytes (s8, MFMA operand order)
     // depthwise: [kernel_h * kernel_w][channels] int16 (w - zw)
     void *d_packed = nullptr;
+    uint32_t *d_post_lut = nullptr; // optional fused unary operator: 256-entry byte table (dense kernels)
+    nncase_hip_quant_param_t post_lut_qp{0, 1.f};
     int32_t *d_wsum = nullptr; // igemm: sum_k (w ^ 0x80 as s8) per out channel; depthwise: sum_t (w - zw)
     int32_t *d_bias = nullptr; // [out_channels]
     size_t packed_bytes = 0;
@@ -60,7 +62,8 @@ struct ResidualEpilogue {
 
 // Fills an Epilogue; returns 0 or a negative error for scales outside the range in
 // which the division-free requantisation is exact.
-int make_residual_epilogue(nncase_hip_ctx *ctx, ResidualEpilogue *rep, const nncase_hip_conv2d_args_t *c);
+int make_residual_epilogue(nncase_hip_ctx *ctx, ResidualEpilogue *rep, const nncase_hip_conv2d_args_t *c,
+                           const nncase_hip_weights *w);
 int make_epilogue(nncase_hip_ctx *ctx, Epilogue *ep, float sx, float sw, nncase_hip_quant_param_t y_qp, float clamp_min,
                   float clamp_max, int out_dtype, const char *who);
 
@@ -81,6 +84,8 @@ int launch_qconv_depthwise(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_h
 void describe_conv_kernel(const nncase_hip_ctx *ctx, const nncase_hip_weights *w, const nncase_hip_conv2d_args_t *a, char *buf,
                           size_t cap);
 int igemm_pixel_groups(const nncase_hip_ctx *ctx, const nncase_hip_weights *w, int m);
+bool igemm_streams_weights(const nncase_hip_weights *w, int mode);
+int stream_pixel_groups(const nncase_hip_ctx *ctx, const nncase_hip_weights *w, int m);
 int igemm_load_mode(const nncase_hip_weights *w, const nncase_hip_conv2d_args_t *c, int out_h, int out_w);
 bool depthwise_uses_3x3(const nncase_hip_weights *w, const nncase_hip_conv2d_args_t *c);
 

@@ -111,6 +111,16 @@ int igemm_pixel_groups(const nncase_hip_ctx *ctx, const nncase_hip_weights *w, i
     return choose_rg(ctx, w->tiles, w->nchunks, m);
 }
 
+// Weights that do not fit the LDS budget at once are streamed through it (16-byte loaders only).
+bool igemm_streams_weights(const nncase_hip_weights *w, int mode) {
+    return w->kc_steps < w->ksteps && w->tiles <= 4 && (mode == kRows16 || mode == kVec16);
+}
+
+// Two pixel groups per wave halve the LDS traffic per multiply; taken when that still leaves a block per CU.
+int stream_pixel_groups(const nncase_hip_ctx *ctx, const nncase_hip_weights *w, int m) {
+    return (long long)ceil_div(m, kWaves * 2 * 16) * w->nchunks >= ctx->compute_units ? 2 : 1;
+}
+
 int igemm_load_mode(const nncase_hip_weights *w, const nncase_hip_conv2d_args_t *c, int out_h, int out_w) {
     const bool pointwise = w->kernel_h == 1 && w->kernel_w == 1 && c->stride_h == 1 && c->stride_w == 1 &&
                            c->pad_h_before == 0 && c->pad_w_before == 0 && out_h == c->in_h && out_w == c->in_w;
@@ -167,13 +177,10 @@ int launch_qconv_igemm(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_hip_w
     }
 
     {
-        const int rc = make_residual_epilogue(ctx, &a.rep, c);
+        const int rc = make_residual_epilogue(ctx, &a.rep, c, w);
         if (rc) return rc;
     }
-    if (c->post_lut_host) {
-        a.use_lut = 1;
-        memcpy(a.lut, c->post_lut_host, 256);
-    }
+    a.lut = c->out_dtype == NNCASE_HIP_DT_U8 ? w->d_post_lut : nullptr;
     const int mode = igemm_load_mode(w, c, out_h, out_w);
 
     const size_t group_bytes = (size_t)w->nchunks * w->ksteps * w->tiles * 1024;
@@ -183,8 +190,15 @@ int launch_qconv_igemm(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_hip_w
         a.bias = w->d_bias + (size_t)g * w->g_oc;
         a.x_coff = g * w->g_ic;
         a.y_coff = g * w->g_oc;
-        const int rg = choose_rg(ctx, w->tiles, w->nchunks, a.m);
         int rc;
+        if (igemm_streams_weights(w, mode)) {
+            const int rg = stream_pixel_groups(ctx, w, a.m);
+            rc = mode == kRows16 ? launch_igemm_stream_rows16(ctx, a, w->tiles, w->nchunks, rg)
+                                 : launch_igemm_stream_vec16(ctx, a, w->tiles, w->nchunks, rg);
+            if (rc) return rc;
+            continue;
+        }
+        const int rg = choose_rg(ctx, w->tiles, w->nchunks, a.m);
         switch (mode) {
         case kRows16: rc = launch_igemm_rows16(ctx, a, w->tiles, w->nchunks, rg); break;
         case kVec16: rc = launch_igemm_vec16(ctx, a, w->tiles, w->nchunks, rg); break;

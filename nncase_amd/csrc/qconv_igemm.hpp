@@ -68,8 +68,7 @@ struct IgemmArgs {
     int num_mtiles;
     Epilogue ep;
     ResidualEpilogue rep;
-    int use_lut;           // apply `lut` to the requantised byte (before the residual add)
-    uint32_t lut[64];
+    const uint32_t *lut;   // 256-entry byte table applied to the requantised byte (before the residual add), or null
 };
 
 struct PixInfo {
@@ -198,6 +197,99 @@ template <int MODE> __device__ __forceinline__ ActFrag load_act(const IgemmArgs 
     return f;
 }
 
+// Epilogue of one 16-pixel x 16T-channel tile of a wave: zero-point correction, requantisation
+// (optionally a byte table and a residual add behind it), NHWC store.  Lane (j, gq) holds pixel p
+// and the 4T consecutive channels from ch0 on; rowsum is the pixel's sum of x' over the reduction.
+template <int T>
+__device__ __forceinline__ void igemm_store_tile(const IgemmArgs &a, const v4i (&acc)[T], int32_t rowsum, int p, int ch0, int gq,
+                                                 const int32_t *cterm, const uint8_t *lutl) {
+    if (!(p < a.m && ch0 < a.n)) return;
+    const int32_t nrsz = -a.zwp * rowsum;
+    const size_t obase = (size_t)p * a.ldy + a.y_coff + ch0;
+    if (a.ep.out_mode == kOutU8) {
+        uint8_t *yo = reinterpret_cast<uint8_t *>(a.y) + obase;
+        uint32_t packed[T];
+#pragma unroll
+        for (int nt = 0; nt < T; nt++) {
+            const v4i ct = *reinterpret_cast<const v4i *>(cterm + gq * (4 * T) + nt * 4);
+            uint32_t b[4];
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int32_t v = add3(acc[nt][r], ct[r], nrsz);
+                b[r] = requant_u8_lowbyte((float)v * a.ep.mult, a.ep);
+            }
+            packed[nt] = pack_low_bytes(b[0], b[1], b[2], b[3]);
+        }
+        if (a.lut) { // fused unary operator: one LDS byte read per output
+#pragma unroll
+            for (int nt = 0; nt < T; nt++) {
+                const uint32_t v = packed[nt];
+                packed[nt] = (uint32_t)lutl[v & 0xffu] | ((uint32_t)lutl[(v >> 8) & 0xffu] << 8) |
+                             ((uint32_t)lutl[(v >> 16) & 0xffu] << 16) | ((uint32_t)lutl[v >> 24] << 24);
+            }
+        }
+        if (a.rep.res) { // fused residual add on the requantised bytes
+            const uint8_t *ro = a.rep.res + obase;
+            const bool whole = ((a.ldy | a.y_coff) & 3) == 0 && ch0 + 4 * T <= a.n;
+#pragma unroll
+            for (int nt = 0; nt < T; nt++) {
+                uint32_t rv = 0;
+                if (whole) {
+                    rv = *reinterpret_cast<const uint32_t *>(ro + nt * 4);
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        if (ch0 + nt * 4 + r < a.n) rv |= (uint32_t)ro[nt * 4 + r] << (8 * r);
+                }
+                uint32_t b[4];
+#pragma unroll
+                for (int r = 0; r < 4; r++) b[r] = residual_lowbyte(packed[nt] >> (8 * r), rv, r, a.rep);
+                packed[nt] = pack_low_bytes(b[0], b[1], b[2], b[3]);
+            }
+        }
+        if (((a.ldy | a.y_coff) & 3) == 0 && ch0 + 4 * T <= a.n) {
+#pragma unroll
+            for (int nt = 0; nt < T; nt += 4) {
+                if (nt + 4 <= T) {
+                    *reinterpret_cast<u32x4_a4 *>(yo + nt * 4) =
+                        u32x4_a4{packed[nt], packed[nt + 1 < T ? nt + 1 : nt], packed[nt + 2 < T ? nt + 2 : nt],
+                                 packed[nt + 3 < T ? nt + 3 : nt]};
+                } else {
+#pragma unroll
+                    for (int e = nt; e < T; e++) *reinterpret_cast<uint32_t *>(yo + e * 4) = packed[e];
+                }
+            }
+        } else {
+#pragma unroll
+            for (int nt = 0; nt < T; nt++)
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    if (ch0 + nt * 4 + r < a.n) yo[nt * 4 + r] = (uint8_t)(packed[nt] >> (8 * r));
+        }
+    } else {
+        // int32 accumulators or clamped fp32, one dword per channel
+        uint32_t *yo = reinterpret_cast<uint32_t *>(a.y) + obase;
+#pragma unroll
+        for (int nt = 0; nt < T; nt++) {
+            const v4i ct = *reinterpret_cast<const v4i *>(cterm + gq * (4 * T) + nt * 4);
+            uint32_t o[4];
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int32_t v = add3(acc[nt][r], ct[r], nrsz);
+                if (a.ep.out_mode == kOutI32) o[r] = (uint32_t)v;
+                else o[r] = __float_as_uint(clamp_ref((float)v * a.ep.mult, a.ep.lo, a.ep.hi));
+            }
+            if (ch0 + nt * 4 + 4 <= a.n) {
+                *reinterpret_cast<u32x4_a4 *>(yo + nt * 4) = u32x4_a4{o[0], o[1], o[2], o[3]};
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    if (ch0 + nt * 4 + r < a.n) yo[nt * 4 + r] = o[r];
+            }
+        }
+    }
+}
+
 template <int T, int RG, int MODE>
 __global__ __launch_bounds__(kThreads, 2) void qconv_igemm_kernel(const IgemmArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -222,7 +314,7 @@ __global__ __launch_bounds__(kThreads, 2) void qconv_igemm_kernel(const IgemmArg
         if (ch < a.n) c = a.bias[ch] - a.zxp * a.wsum[ch] + a.k * a.zxp * a.zwp;
         cterm[i] = c;
     }
-    if (a.use_lut && threadIdx.x < 64) reinterpret_cast<uint32_t *>(lutl)[threadIdx.x] = a.lut[threadIdx.x];
+    if (a.lut && threadIdx.x < 64) reinterpret_cast<uint32_t *>(lutl)[threadIdx.x] = a.lut[threadIdx.x];
     auto stage_weights = [&](int kci) {
         const int s0 = kci * a.kc_steps;
         const int steps = min(a.kc_steps, a.ksteps - s0);
@@ -305,99 +397,186 @@ __global__ __launch_bounds__(kThreads, 2) void qconv_igemm_kernel(const IgemmArg
         // ---- epilogue: zero-point correction, requantisation, NHWC store ----
         const int ch0 = ch_base + gq * (4 * T); // first of this lane's 4T channels
 #pragma unroll
-        for (int rg = 0; rg < RG; rg++) {
-            const int p = mt * pix_per_block + (wave * RG + rg) * 16 + j;
-            if (p < a.m && ch0 < a.n) {
-                const int32_t nrsz = -a.zwp * rs[rg][0];
-                const size_t obase = (size_t)p * a.ldy + a.y_coff + ch0;
-                if (a.ep.out_mode == kOutU8) {
-                    uint8_t *yo = reinterpret_cast<uint8_t *>(a.y) + obase;
-                    uint32_t packed[T];
-#pragma unroll
-                    for (int nt = 0; nt < T; nt++) {
-                        const v4i ct = *reinterpret_cast<const v4i *>(cterm + gq * (4 * T) + nt * 4);
-                        uint32_t b[4];
-#pragma unroll
-                        for (int r = 0; r < 4; r++) {
-                            const int32_t v = add3(acc[rg][nt][r], ct[r], nrsz);
-                            b[r] = requant_u8_lowbyte((float)v * a.ep.mult, a.ep);
-                        }
-                        packed[nt] = pack_low_bytes(b[0], b[1], b[2], b[3]);
-                    }
-                    if (a.use_lut) { // fused unary operator: one LDS byte read per output
-#pragma unroll
-                        for (int nt = 0; nt < T; nt++) {
-                            const uint32_t v = packed[nt];
-                            packed[nt] = (uint32_t)lutl[v & 0xffu] | ((uint32_t)lutl[(v >> 8) & 0xffu] << 8) |
-                                         ((uint32_t)lutl[(v >> 16) & 0xffu] << 16) | ((uint32_t)lutl[v >> 24] << 24);
-                        }
-                    }
-                    if (a.rep.res) { // fused residual add on the requantised bytes
-                        const uint8_t *ro = a.rep.res + obase;
-                        const bool whole = ((a.ldy | a.y_coff) & 3) == 0 && ch0 + 4 * T <= a.n;
-#pragma unroll
-                        for (int nt = 0; nt < T; nt++) {
-                            uint32_t rv = 0;
-                            if (whole) {
-                                rv = *reinterpret_cast<const uint32_t *>(ro + nt * 4);
-                            } else {
-#pragma unroll
-                                for (int r = 0; r < 4; r++)
-                                    if (ch0 + nt * 4 + r < a.n) rv |= (uint32_t)ro[nt * 4 + r] << (8 * r);
-                            }
-                            uint32_t b[4];
-#pragma unroll
-                            for (int r = 0; r < 4; r++) b[r] = residual_lowbyte(packed[nt] >> (8 * r), rv, r, a.rep);
-                            packed[nt] = pack_low_bytes(b[0], b[1], b[2], b[3]);
-                        }
-                    }
-                    if (((a.ldy | a.y_coff) & 3) == 0 && ch0 + 4 * T <= a.n) {
-#pragma unroll
-                        for (int nt = 0; nt < T; nt += 4) {
-                            if (nt + 4 <= T) {
-                                *reinterpret_cast<u32x4_a4 *>(yo + nt * 4) =
-                                    u32x4_a4{packed[nt], packed[nt + 1 < T ? nt + 1 : nt], packed[nt + 2 < T ? nt + 2 : nt],
-                                             packed[nt + 3 < T ? nt + 3 : nt]};
-                            } else {
-#pragma unroll
-                                for (int e = nt; e < T; e++) *reinterpret_cast<uint32_t *>(yo + e * 4) = packed[e];
-                            }
-                        }
-                    } else {
-#pragma unroll
-                        for (int nt = 0; nt < T; nt++)
-#pragma unroll
-                            for (int r = 0; r < 4; r++)
-                                if (ch0 + nt * 4 + r < a.n) yo[nt * 4 + r] = (uint8_t)(packed[nt] >> (8 * r));
-                    }
-                } else {
-                    // int32 accumulators or clamped fp32, one dword per channel
-                    uint32_t *yo = reinterpret_cast<uint32_t *>(a.y) + obase;
-#pragma unroll
-                    for (int nt = 0; nt < T; nt++) {
-                        const v4i ct = *reinterpret_cast<const v4i *>(cterm + gq * (4 * T) + nt * 4);
-                        uint32_t o[4];
-#pragma unroll
-                        for (int r = 0; r < 4; r++) {
-                            const int32_t v = add3(acc[rg][nt][r], ct[r], nrsz);
-                            if (a.ep.out_mode == kOutI32) o[r] = (uint32_t)v;
-                            else o[r] = __float_as_uint(clamp_ref((float)v * a.ep.mult, a.ep.lo, a.ep.hi));
-                        }
-                        if (ch0 + nt * 4 + 4 <= a.n) {
-                            *reinterpret_cast<u32x4_a4 *>(yo + nt * 4) = u32x4_a4{o[0], o[1], o[2], o[3]};
-                        } else {
-#pragma unroll
-                            for (int r = 0; r < 4; r++)
-                                if (ch0 + nt * 4 + r < a.n) yo[nt * 4 + r] = o[r];
-                        }
-                    }
-                }
-            }
-        }
+        for (int rg = 0; rg < RG; rg++)
+            igemm_store_tile<T>(a, acc[rg], rs[rg][0], mt * pix_per_block + (wave * RG + rg) * 16 + j, ch0, gq, cterm, lutl);
 #pragma unroll
         for (int rg = 0; rg < RG; rg++) pcur[rg] = pnxt[rg];
     }
 }
+
+// ---- long reductions: weights streamed through LDS -----------------------------------------------
+// When the weights of a channel chunk do not fit the LDS budget (3x3 and larger windows over many
+// channels), they are streamed: every k-step's T fragments go global -> registers -> a three-slot LDS
+// ring, one barrier per k-step, and both the weights and the activation slices are requested three
+// k-steps before they are multiplied.  With one or two blocks per compute unit there are too few
+// waves to hide memory latency by switching waves, so the latency has to be covered inside the wave;
+// a one-step prefetch exposes a full memory round trip per k-step on such layers.
+struct ActSlice { // vec16 / rows16: one 16-byte load per k-step, one fill value
+    u32x4 raw;
+    uint32_t fill;
+    uint32_t take; // 0 or ~0
+};
+
+template <int MODE> __device__ __forceinline__ ActSlice load_slice(const IgemmArgs &a, const PixInfo &pi, int kc) {
+    static_assert(MODE == kRows16 || MODE == kVec16, "one 16-byte piece per slice");
+    ActSlice f;
+    const bool pix_ok = pi.base >= 0;
+    PixInfo sp = pi;
+    if (!pix_ok) sp.base = 0, sp.iy0 = 0, sp.ix0 = 0;
+    const bool in_k = kc * 16 < a.k;
+    if (MODE == kRows16) {
+        f.raw = *reinterpret_cast<const u32x4 *>(a.x + (size_t)((uint32_t)sp.base * (uint32_t)a.ldx + a.x_coff + (in_k ? kc : 0) * 16));
+        f.fill = 0x80808080u;
+        f.take = (pix_ok && in_k) ? ~0u : 0u;
+    } else {
+        bool inside;
+        const uint32_t off = tap_offset(a, sp, in_k ? kc * 16 : 0, &inside);
+        f.raw = *reinterpret_cast<const u32x4 *>(a.x + (size_t)off);
+        f.fill = (pix_ok && in_k) ? a.zx_splat : 0x80808080u; // padding tap : outside the problem
+        f.take = (pix_ok && in_k && inside) ? ~0u : 0u;
+    }
+    return f;
+}
+
+__device__ __forceinline__ v4i finish_slice(const ActSlice &f) {
+    u32x4 r;
+#pragma unroll
+    for (int d = 0; d < 4; d++) r[d] = ((f.raw[d] & f.take) | (f.fill & ~f.take)) ^ 0x80808080u;
+    return __builtin_bit_cast(v4i, r);
+}
+
+template <int T, int RG, int MODE>
+__global__ __launch_bounds__(kThreads, 2) void qconv_igemm_stream_kernel(const IgemmArgs a) {
+    // three ring slots: the one being multiplied, the one being written, and one in between
+    constexpr int WV = T * 64;                             // 16-byte vectors of weights per k-step
+    constexpr int NW = (WV + kThreads - 1) / kThreads;     // ... per thread
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    int32_t *cterm = reinterpret_cast<int32_t *>(smem);   // [T * 16]
+    uint8_t *lutl = smem + T * 16 * sizeof(int32_t);      // [256]
+    uint8_t *wring = lutl + 256;                           // [NSLOT][T][1024]
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int j = lane & 15, gq = lane >> 4;
+    const int chunk = blockIdx.y;
+    const int ch_base = chunk * (T * 16);
+    const u32x4 *wsrc = reinterpret_cast<const u32x4 *>(a.wpk + (size_t)chunk * a.ksteps * T * 1024);
+    const int KS = a.ksteps;
+
+    for (int i = threadIdx.x; i < T * 16; i += kThreads) {
+        const int ch = ch_base + i;
+        cterm[i] = ch < a.n ? a.bias[ch] - a.zxp * a.wsum[ch] + a.k * a.zxp * a.zwp : 0;
+    }
+    if (a.lut && threadIdx.x < 64) reinterpret_cast<uint32_t *>(lutl)[threadIdx.x] = a.lut[threadIdx.x];
+
+    const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
+    constexpr int pix_per_block = kWaves * RG * 16;
+    auto load_w = [&](u32x4 (&dst)[NW], int ks) {
+#pragma unroll
+        for (int i = 0; i < NW; i++) {
+            const int v = threadIdx.x + i * kThreads;
+            if (v < WV) dst[i] = wsrc[(size_t)ks * WV + v];
+        }
+    };
+    auto store_w = [&](const u32x4 (&src)[NW], int slot) {
+        u32x4 *dst = reinterpret_cast<u32x4 *>(wring + (size_t)slot * T * 1024);
+#pragma unroll
+        for (int i = 0; i < NW; i++) {
+            const int v = threadIdx.x + i * kThreads;
+            if (v < WV) dst[v] = src[i];
+        }
+    };
+
+    for (int mt = blockIdx.x; mt < a.num_mtiles; mt += gridDim.x) {
+        PixInfo pix[RG];
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) pix[rg] = pix_info<MODE>(a, mt * pix_per_block + (wave * RG + rg) * 16 + j);
+        v4i acc[RG][T], rs[RG];
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) {
+            rs[rg] = v4i{0, 0, 0, 0};
+#pragma unroll
+            for (int nt = 0; nt < T; nt++) acc[rg][nt] = v4i{0, 0, 0, 0};
+        }
+        // ---- fill the pipeline: weights of k-steps 0..2, activation slices of k-steps 0..2 ----
+        u32x4 wreg[2][NW];
+        ActSlice af[3][RG];
+        {
+            u32x4 w0[NW];
+            load_w(w0, 0);
+            if (1 < KS) load_w(wreg[1], 1);
+            if (2 < KS) load_w(wreg[0], 2);
+#pragma unroll
+            for (int d = 0; d < 3; d++)
+#pragma unroll
+                for (int rg = 0; rg < RG; rg++) af[d][rg] = load_slice<MODE>(a, pix[rg], (d < KS ? d : 0) * 4 + gq);
+            __syncthreads(); // the previous pixel tile no longer reads the ring (and cterm is written)
+            store_w(w0, 0);
+            __syncthreads();
+        }
+        for (int s0 = 0; s0 < KS; s0 += 6) {
+#pragma unroll
+            for (int u = 0; u < 6; u++) {
+                const int s = s0 + u;
+                if (s < KS) { // uniform for the block
+                    v4i xf[RG];
+#pragma unroll
+                    for (int rg = 0; rg < RG; rg++) xf[rg] = finish_slice(af[u % 3][rg]);
+                    if (s + 3 < KS) {
+#pragma unroll
+                        for (int rg = 0; rg < RG; rg++) af[u % 3][rg] = load_slice<MODE>(a, pix[rg], (s + 3) * 4 + gq);
+                    }
+                    if (s + 1 < KS) store_w(wreg[(u + 1) % 2], (u + 1) % 3);
+                    if (s + 3 < KS) load_w(wreg[(u + 1) % 2], s + 3);
+#pragma unroll
+                    for (int rg = 0; rg < RG; rg++)
+                        rs[rg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, xf[rg], rs[rg], 0, 0, 0);
+                    const uint8_t *wstep = wring + (size_t)(u % 3) * T * 1024 + lane * 16;
+#pragma unroll
+                    for (int nt = 0; nt < T; nt++) {
+                        const v4i wf = *reinterpret_cast<const v4i *>(wstep + nt * 1024);
+#pragma unroll
+                        for (int rg = 0; rg < RG; rg++)
+                            acc[rg][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf, xf[rg], acc[rg][nt], 0, 0, 0);
+                    }
+                    __syncthreads();
+                }
+            }
+        }
+        const int ch0 = ch_base + gq * (4 * T);
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++)
+            igemm_store_tile<T>(a, acc[rg], rs[rg][0], mt * pix_per_block + (wave * RG + rg) * 16 + j, ch0, gq, cterm, lutl);
+    }
+}
+
+template <int T, int RG, int MODE> int launch_stream_trg(nncase_hip_ctx *ctx, const IgemmArgs &a, int nchunks) {
+    IgemmArgs args = a;
+    constexpr int pix_per_block = kWaves * RG * 16;
+    args.num_mtiles = ceil_div(a.m, pix_per_block);
+    int gx = args.num_mtiles < ctx->compute_units * 4 ? args.num_mtiles : ctx->compute_units * 4;
+    if (nchunks > 1) gx = ceil_div(gx, 8) * 8; // chunks of one pixel tile on one XCD
+    const size_t lds = (size_t)T * 16 * sizeof(int32_t) + 256 + (size_t)3 * T * 1024;
+    hipLaunchKernelGGL((qconv_igemm_stream_kernel<T, RG, MODE>), dim3(gx, nchunks, 1), dim3(kThreads), lds, ctx->stream, args);
+    NNHIP_LAUNCH_CHECK(ctx, "qconv_igemm_stream_kernel");
+    return 0;
+}
+
+template <int MODE> int launch_stream_mode(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks, int rg) {
+#define NNHIP_STREAM_CASE(TT)                                                                                          \
+    case TT: return rg >= 2 ? launch_stream_trg<TT, 2, MODE>(ctx, a, nchunks) : launch_stream_trg<TT, 1, MODE>(ctx, a, nchunks);
+    switch (tiles) {
+        NNHIP_STREAM_CASE(1)
+        NNHIP_STREAM_CASE(2)
+        NNHIP_STREAM_CASE(3)
+        NNHIP_STREAM_CASE(4)
+    default: return fail(ctx, -EINVAL, "qconv2d: no streaming kernel for %d channel tiles", tiles);
+    }
+#undef NNHIP_STREAM_CASE
+}
+
+int launch_igemm_stream_rows16(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks, int rg);
+int launch_igemm_stream_vec16(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks, int rg);
 
 // Pixel groups per wave (RG) for a chunk width of T tiles.  The kernels are bound by the
 // VALU work of the epilogue, and a dependent VALU instruction issues only every ~8 cycles

@@ -97,8 +97,8 @@ def conv2d(input: np.ndarray, weights: np.ndarray, bias: Optional[np.ndarray], s
     y_nchw = c.alloc(max(1, n * oh * ow * oc * es))
     args = rt.Conv2dArgs(n, h, wd, stride[0], stride[1], dilation[0], dilation[1], ph0, ph1, pw0, pw1, input_qp,
                          output_qp or qp(0, 1.0), fused_clamp[0], fused_clamp[1], _out_dt(out_dtype))
-    if post_lut is not None:  # fused Quantize(unary(Dequantize(conv))) as a byte table
-        args.set_post_lut(post_lut, post_lut_qp)
+    if post_lut is not None:  # fused Quantize(unary(Dequantize(conv))) as a byte table attached to the weights
+        wts.set_post_lut(post_lut, post_lut_qp)
     if residual is not None:  # fused Quantize(Dequantize(conv) + Dequantize(residual)), residual given as NCHW u8
         r = np.ascontiguousarray(residual, np.uint8)
         if r.shape != (n, oc, oh, ow):

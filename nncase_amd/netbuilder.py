@@ -409,7 +409,7 @@ class HipModel:
                 args = rt.Conv2dArgs(batch, src.out_shape[1], src.out_shape[2], n.stride[0], n.stride[1], 1, 1, ph0, ph1, pw0,
                                      pw1, qp(*src.out_qp), qp(*n.out_qp), n.clamp[0], n.clamp[1], rt.DT_U8)
                 if fused_lut is not None:
-                    args.set_post_lut(qg.nodes[fused_lut].lut, qp(*qg.nodes[fused_lut].out_qp))
+                    wt.set_post_lut(qg.nodes[fused_lut].lut, qp(*qg.nodes[fused_lut].out_qp))
                 if fused_add is not None:
                     add = qg.nodes[fused_add]
                     res_node = add.inputs[0]

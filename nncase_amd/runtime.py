@@ -50,16 +50,7 @@ class Conv2dArgs(C.Structure):
                 ("x_qp", QuantParam), ("y_qp", QuantParam),
                 ("clamp_min", C.c_float), ("clamp_max", C.c_float), ("out_dtype", C.c_int32),
                 ("residual_dev", C.c_void_p), ("residual_qp", QuantParam), ("sum_qp", QuantParam),
-                ("sum_clamp_min", C.c_float), ("sum_clamp_max", C.c_float),
-                ("post_lut_host", C.c_void_p), ("post_lut_qp", QuantParam)]
-
-    def set_post_lut(self, lut: np.ndarray, lut_qp: "QuantParam"):
-        """Fuses a 256-entry byte table (make_unary_lut) behind the requantisation; the table is copied
-        by the call that consumes these arguments, the array only has to live until then."""
-        self._lut = np.ascontiguousarray(lut, np.uint8)
-        assert self._lut.size == 256
-        self.post_lut_host = self._lut.ctypes.data
-        self.post_lut_qp = lut_qp
+                ("sum_clamp_min", C.c_float), ("sum_clamp_max", C.c_float)]
 
 
 class MatmulArgs(C.Structure):
@@ -94,6 +85,7 @@ SYMBOLS = {
     "nncase_hip_dequantize": (_I, [_VP, _VP, _I, _VP, _I, _SZ, QuantParam]),
     "nncase_hip_qconv2d_prepack": (_I, [_VP, C.POINTER(Conv2dDesc), _VP, _VP, C.POINTER(_VP)]),
     "nncase_hip_weights_destroy": (_I, [_VP, _VP]),
+    "nncase_hip_weights_set_post_lut": (_I, [_VP, _VP, _VP, QuantParam]),
     "nncase_hip_qconv2d": (_I, [_VP, _VP, _VP, _VP, C.POINTER(Conv2dArgs)]),
     "nncase_hip_qmatmul_prepack": (_I, [_VP, _VP, C.c_int32, C.c_int32, QuantParam, _VP, C.c_int64, C.POINTER(_VP)]),
     "nncase_hip_qmatmul": (_I, [_VP, _VP, _VP, _VP, C.POINTER(MatmulArgs)]),
@@ -236,6 +228,17 @@ class Weights:
     def __init__(self, ctx: "Context", handle, out_channels: int, kernel: Tuple[int, int], in_channels: int, groups: int):
         self.ctx, self.handle = ctx, handle
         self.out_channels, self.kernel, self.in_channels, self.groups = out_channels, kernel, in_channels, groups
+
+    def set_post_lut(self, lut: Optional[np.ndarray], lut_qp: "QuantParam" = None):
+        """Attaches a fused 256-entry byte table (make_unary_lut) applied behind the requantisation of every
+        u8-output call with these weights; None detaches it."""
+        if lut is None:
+            self.ctx._check(self.ctx.lib.nncase_hip_weights_set_post_lut(self.ctx.handle, self.handle, None, qp(0, 1.0)), "weights_set_post_lut")
+            return self
+        t = np.ascontiguousarray(lut, np.uint8)
+        assert t.size == 256
+        self.ctx._check(self.ctx.lib.nncase_hip_weights_set_post_lut(self.ctx.handle, self.handle, t.ctypes.data, lut_qp), "weights_set_post_lut")
+        return self
 
     def destroy(self):
         if self.handle:
