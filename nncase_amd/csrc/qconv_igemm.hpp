@@ -197,6 +197,10 @@ template <int MODE> __device__ __forceinline__ ActFrag load_act(const IgemmArgs 
     return f;
 }
 
+struct __attribute__((packed, aligned(1))) U32Unaligned {
+    uint32_t v;
+};
+
 // Epilogue of one 16-pixel x 16T-channel tile of a wave: zero-point correction, requantisation
 // (optionally a byte table and a residual add behind it), NHWC store.  Lane (j, gq) holds pixel p
 // and the 4T consecutive channels from ch0 on; rowsum is the pixel's sum of x' over the reduction.
@@ -259,6 +263,11 @@ __device__ __forceinline__ void igemm_store_tile(const IgemmArgs &a, const v4i (
                     for (int e = nt; e < T; e++) *reinterpret_cast<uint32_t *>(yo + e * 4) = packed[e];
                 }
             }
+        } else if (ch0 + 4 * T <= a.n) {
+            // a channel count that is no multiple of 4 (255-channel detection heads): pixel rows start at
+            // any byte, the lane's 4T bytes still go out as dwords (the memory system takes unaligned dwords)
+#pragma unroll
+            for (int nt = 0; nt < T; nt++) reinterpret_cast<U32Unaligned *>(yo + nt * 4)->v = packed[nt];
         } else {
 #pragma unroll
             for (int nt = 0; nt < T; nt++)
