@@ -189,6 +189,44 @@ def side_workload(args):
                               "note": "all convolutions together: int8 op count / summed conv kernel time"},
                     sum_of_kernel_ms=round(sum(op_ms), 4),
                     kernel_groups_ms={k: round(v, 4) for k, v in sorted(groups.items(), key=lambda kv: -kv[1])})
+    elif args.workload == "llm_decode":
+        from nncase_amd import llm
+        cfg = llm.DecoderConfig()
+        batch, max_ctx = 32, 4096
+        rng = np.random.default_rng(5)
+        weights = llm.random_weights(cfg, seed=5)
+        lens = rng.integers(512, max_ctx + 1, batch).astype(np.int32)
+        max_blocks = (max_ctx + args.steps + args.warmup + 64) // cfg.block_size + 1
+        nblocks = batch * max_blocks
+        bt = rng.permutation(nblocks).reshape(batch, max_blocks).astype(np.int32)
+        # one random cache image, uploaded once per layer (every layer has its own device copy)
+        kc = rng.standard_normal((nblocks, cfg.kv_heads, cfg.block_size, cfg.head_dim), dtype=np.float32).astype(np.float16)
+        vc = rng.standard_normal((nblocks, cfg.kv_heads, cfg.head_dim, cfg.block_size), dtype=np.float32).astype(np.float16)
+        dec = llm.HipDecoder(ctx, cfg, weights, batch, max_blocks, bt, lens, [kc] * cfg.layers, [vc] * cfg.layers,
+                             capture_graph=True, feedback=True)
+        dec.set_tokens(rng.integers(0, cfg.vocab, batch).astype(np.int32))
+        ms = time_calls(ctx, dec.step, args.warmup, args.steps)
+        toks = dec.result()
+        assert toks.min() >= 0 and toks.max() < cfg.vocab
+        steps_done = args.warmup + args.steps
+        mean_ctx = float(lens.mean()) + steps_done / 2
+        kv_bytes = int(mean_ctx * batch * cfg.kv_heads * cfg.head_dim * 2 * 2 * cfg.layers)
+        w_bytes = dec.weight_bytes()
+        op_ms = dec.fn.profile(3)
+        groups = {}
+        for i, t in enumerate(op_ms):
+            k_ = dec.fn.op_kernel(i)
+            groups[k_] = groups.get(k_, 0.0) + t
+        line = dict(base, metric="tokens/sec LLM decode step b32 (Qwen2-0.5B shape, W8A16, fp16 paged KV)", value=round(batch / (ms * 1e-3), 1),
+                    unit="tokens/s", ms_per_step=round(ms, 4), dtype="f16",
+                    config={"workload": "config 5: 24 layers, hidden 896, 14 q / 2 kv heads, head_dim 64, MLP 4864, vocab 151936, W8A16 per-output-channel "
+                                        "weights, fp16 paged KV (block 16), batch 32, ctx U[512,4096], greedy arg-max fed back on the device, "
+                                        f"{len(dec.fn)} operators, one HIP-graph replay per step"},
+                    roofline={"bound": "hbm", "achieved": round((kv_bytes + w_bytes) / (ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                              "frac": round((kv_bytes + w_bytes) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
+                              "algorithmic_bytes_per_step": kv_bytes + w_bytes, "weight_bytes": w_bytes, "kv_bytes": kv_bytes},
+                    sum_of_kernel_ms=round(sum(op_ms), 4),
+                    kernel_groups_ms={k_: round(v, 4) for k_, v in sorted(groups.items(), key=lambda kv: -kv[1])})
     elif args.workload == "paged_attention":
         rng = np.random.default_rng(5)
         bsz, hq, hkv, d, blk = 32, 14, 2, 64, 16
@@ -218,7 +256,7 @@ def side_workload(args):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--workload", default="mobilenetv2", help="mobilenetv2 (headline, default) | matmul | conv_block | yolov5s | paged_attention")
+    ap.add_argument("--workload", default="mobilenetv2", help="mobilenetv2 (headline, default) | matmul | conv_block | yolov5s | paged_attention | llm_decode")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)

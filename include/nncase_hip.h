@@ -314,12 +314,52 @@ typedef struct nncase_hip_paged_attn_args {
     int32_t block_size, max_blocks_per_seq, num_blocks;
     float scale;
     int32_t out_dtype; /* NNCASE_HIP_DT_F16 or _F32 */
+    /* added to every ctx_lens[b] (a decode step attends to the token it has just appended, before the
+     * lengths are advanced at the end of the step: 1; otherwise 0) */
+    int32_t ctx_len_offset;
 } nncase_hip_paged_attn_args_t;
 
 NNCASE_HIP_API int nncase_hip_paged_attention_decode(nncase_hip_ctx_t *ctx, const void *q_dev, const void *k_cache_dev,
                                                      const void *v_cache_dev, const int32_t *block_table_dev,
                                                      const int32_t *ctx_lens_dev, void *out_dev,
                                                      const nncase_hip_paged_attn_args_t *args);
+
+/* ---- the rest of an LLM decode step (fp16 activations, W8A16 weights) --------
+ * No counterpart in this reference tree (its LLM path lives in another branch); the
+ * arithmetic is defined here and checked against float64 restatements.
+ *
+ * W8A16 linear layer: out[m, n] = scale[n] * sum_k a[m, k] * w[n, k] (+ bias[n]), a fp16,
+ * w int8 with one fp32 scale per output channel, fp32 accumulation.  k a multiple of 64,
+ * n a multiple of 16, 1..64 token rows per call.
+ *   NNCASE_HIP_GEMM_PLAIN   out is [m, n]
+ *   NNCASE_HIP_GEMM_SWIGLU  the matrix holds the gate projection in rows [0, n/2) and the up
+ *                           projection in rows [n/2, n): out[m, j] = silu(gate_j) * up_j, [m, n/2]
+ * residual_dev (fp16, shape of out, may be NULL) is added to the result; out is fp16 or fp32. */
+#define NNCASE_HIP_GEMM_PLAIN 0
+#define NNCASE_HIP_GEMM_SWIGLU 1
+typedef struct nncase_hip_w8a16 nncase_hip_w8a16_t;
+NNCASE_HIP_API int nncase_hip_w8a16_prepack(nncase_hip_ctx_t *ctx, const int8_t *w_nk_host, const float *scale_host,
+                                            const float *bias_host, int32_t k, int32_t n, nncase_hip_w8a16_t **weights);
+NNCASE_HIP_API int nncase_hip_w8a16_destroy(nncase_hip_ctx_t *ctx, nncase_hip_w8a16_t *weights);
+NNCASE_HIP_API int nncase_hip_w8a16_gemm(nncase_hip_ctx_t *ctx, const void *a_dev, const nncase_hip_w8a16_t *weights,
+                                         void *out_dev, int32_t m, int32_t mode, const void *residual_dev, int32_t out_dtype);
+/* out[r, :] = x[r, :] * rsqrt(mean(x[r, :]^2) + eps) * weight, fp16 in / out, fp32 arithmetic. */
+NNCASE_HIP_API int nncase_hip_rmsnorm_f16(nncase_hip_ctx_t *ctx, const void *x_dev, const void *weight_dev, void *out_dev,
+                                          int32_t rows, int32_t hidden, float eps);
+/* qkv [batch, (Hq + 2 Hkv) * d] fp16 (q heads, k heads, v heads) of one new token per sequence:
+ * rotary embedding (rotate-half pairing, angle pos * theta^(-2i/d), pos = ctx_lens[b]) of q and k;
+ * q goes to q_out [batch, Hq, d], the rotated k and v are appended at position ctx_lens[b] of the
+ * paged cache (layouts of nncase_hip_paged_attention_decode).  ctx_lens is NOT advanced. */
+NNCASE_HIP_API int nncase_hip_rope_kv_append(nncase_hip_ctx_t *ctx, const void *qkv_dev, void *q_out_dev, void *k_cache_dev,
+                                             void *v_cache_dev, const int32_t *block_table_dev, const int32_t *ctx_lens_dev,
+                                             const nncase_hip_paged_attn_args_t *geometry, float rope_theta);
+/* out[r] = index of the largest element of row r (the lowest index among equals). */
+NNCASE_HIP_API int nncase_hip_argmax_f32(nncase_hip_ctx_t *ctx, const float *x_dev, int32_t *out_dev, int32_t rows, int32_t cols);
+/* out[r, :] = table[ids[r], :] (fp16 rows). */
+NNCASE_HIP_API int nncase_hip_embedding_f16(nncase_hip_ctx_t *ctx, const void *table_dev, const int32_t *ids_dev, void *out_dev,
+                                            int32_t rows, int32_t hidden, int32_t vocab);
+/* x[i] += delta (advances the context lengths after a decode step). */
+NNCASE_HIP_API int nncase_hip_add_i32(nncase_hip_ctx_t *ctx, int32_t *x_dev, int32_t count, int32_t delta);
 
 /* ---- resident functions --------------------------------------------------
  * A function is the `hip` module's counterpart of a runtime_function
@@ -375,6 +415,26 @@ NNCASE_HIP_API int nncase_hip_function_add_qmaxpool2d(nncase_hip_function_t *fn,
 NNCASE_HIP_API int nncase_hip_function_add_pack(nncase_hip_function_t *fn, const void *in_dev, void *out_dev,
                                                 int32_t elem_size, int32_t rank, const int32_t *shape, int32_t n_axes,
                                                 const int32_t *axes, const int32_t *lanes);
+/* The decode-step operators above, recorded with the same arguments (paged attention included), so a
+ * whole decode step replays as one HIP graph. */
+NNCASE_HIP_API int nncase_hip_function_add_w8a16_gemm(nncase_hip_function_t *fn, const void *a_dev, const nncase_hip_w8a16_t *weights,
+                                                      void *out_dev, int32_t m, int32_t mode, const void *residual_dev,
+                                                      int32_t out_dtype);
+NNCASE_HIP_API int nncase_hip_function_add_rmsnorm_f16(nncase_hip_function_t *fn, const void *x_dev, const void *weight_dev,
+                                                       void *out_dev, int32_t rows, int32_t hidden, float eps);
+NNCASE_HIP_API int nncase_hip_function_add_rope_kv_append(nncase_hip_function_t *fn, const void *qkv_dev, void *q_out_dev,
+                                                          void *k_cache_dev, void *v_cache_dev, const int32_t *block_table_dev,
+                                                          const int32_t *ctx_lens_dev,
+                                                          const nncase_hip_paged_attn_args_t *geometry, float rope_theta);
+NNCASE_HIP_API int nncase_hip_function_add_paged_attention_decode(nncase_hip_function_t *fn, const void *q_dev,
+                                                                  const void *k_cache_dev, const void *v_cache_dev,
+                                                                  const int32_t *block_table_dev, const int32_t *ctx_lens_dev,
+                                                                  void *out_dev, const nncase_hip_paged_attn_args_t *args);
+NNCASE_HIP_API int nncase_hip_function_add_argmax_f32(nncase_hip_function_t *fn, const float *x_dev, int32_t *out_dev,
+                                                      int32_t rows, int32_t cols);
+NNCASE_HIP_API int nncase_hip_function_add_embedding_f16(nncase_hip_function_t *fn, const void *table_dev, const int32_t *ids_dev,
+                                                         void *out_dev, int32_t rows, int32_t hidden, int32_t vocab);
+NNCASE_HIP_API int nncase_hip_function_add_add_i32(nncase_hip_function_t *fn, int32_t *x_dev, int32_t count, int32_t delta);
 /* Number of operators recorded so far. */
 NNCASE_HIP_API int nncase_hip_function_size(nncase_hip_function_t *fn, int32_t *count);
 /* Enqueues the whole function (graph replay if captured). */

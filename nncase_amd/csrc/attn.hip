@@ -50,7 +50,7 @@ struct AttnArgs {
     float *part_ml; // [batch][q heads][splits][2]: max of (logit * scale * log2 e), sum of 2^(. - max)
     uint32_t *done; // [batch][kv heads] blocks finished; zero between calls
     void *out;
-    int batch, hq, hkv, group, d, block_size, max_blocks, num_blocks, splits, split_tokens;
+    int batch, hq, hkv, group, d, block_size, max_blocks, num_blocks, splits, split_tokens, len_offset;
     FastDiv d_block;
     float scale_log2e;
     int out_f16;
@@ -97,7 +97,7 @@ template <int D, int NT> __global__ __launch_bounds__(kAttnThreads, 2) void page
         inb[t] = tt - (int)lb * a.block_size;
         pbs[t] = table[min((int)lb, a.max_blocks - 1)];
     }
-    const int ctx = min(a.ctx_lens[b], a.max_blocks * a.block_size);
+    const int ctx = min(a.ctx_lens[b] + a.len_offset, a.max_blocks * a.block_size);
     if (ctx <= 0) { // empty context: zeros, written by the first block of the pair
         if (split == 0)
             for (int idx = threadIdx.x; idx < G * D; idx += kAttnThreads) {
@@ -352,6 +352,7 @@ extern "C" int nncase_hip_paged_attention_decode(nncase_hip_ctx_t *ctx, const vo
     a.block_size = p->block_size;
     a.max_blocks = p->max_blocks_per_seq;
     a.num_blocks = p->num_blocks;
+    a.len_offset = p->ctx_len_offset;
     const int64_t max_tokens = (int64_t)p->max_blocks_per_seq * p->block_size;
     // Tiles per wave: the largest run that still leaves about three blocks per compute unit when
     // every sequence is at full length (the kernel cannot know the real lengths on the host).

@@ -8,7 +8,8 @@
 namespace {
 
 struct Op {
-    enum Kind { kQuantize, kDequantize, kConv, kAdd, kPool, kLut, kConcat, kResize, kMaxPool, kPack } kind;
+    enum Kind { kQuantize, kDequantize, kConv, kAdd, kPool, kLut, kConcat, kResize, kMaxPool, kPack,
+                kGemm, kRmsNorm, kRope, kAttn, kArgmax, kEmbed, kAddI32 } kind;
     const void *in0 = nullptr, *in1 = nullptr;
     void *out = nullptr;
     const nncase_hip_weights_t *weights = nullptr;
@@ -28,6 +29,13 @@ struct Op {
     int32_t elem_size = 0, out_h = 0, out_w = 0, tmode = 0, nmode = 0;
     int32_t pool[8] = {0}; // kernel h, w, stride h, w, pad h before / after, w before / after
     int32_t rank = 0, n_axes = 0, shape[8] = {0}, axes[8] = {0}, lanes[8] = {0};
+    // decode-step operators
+    const nncase_hip_w8a16_t *w8 = nullptr;
+    const void *in2 = nullptr, *in3 = nullptr, *in4 = nullptr; // further operands (caches, tables)
+    void *out2 = nullptr, *out3 = nullptr;
+    nncase_hip_paged_attn_args_t attn{};
+    int32_t mode = 0, delta = 0;
+    float eps = 0.f;
 };
 
 } // namespace
@@ -67,6 +75,22 @@ static int run_op(nncase_hip_function *fn, const Op &op) {
                                      op.pool[7], op.qp0, op.qp1);
     case Op::kPack:
         return nncase_hip_pack(ctx, op.in0, op.out, op.elem_size, op.rank, op.shape, op.n_axes, op.axes, op.lanes);
+    case Op::kGemm:
+        return nncase_hip_w8a16_gemm(ctx, op.in0, op.w8, op.out, op.batch, op.mode, op.in1, op.dt_out);
+    case Op::kRmsNorm:
+        return nncase_hip_rmsnorm_f16(ctx, op.in0, op.in1, op.out, op.batch, op.channels, op.eps);
+    case Op::kRope:
+        return nncase_hip_rope_kv_append(ctx, op.in0, op.out, op.out2, op.out3, (const int32_t *)op.in2, (const int32_t *)op.in3,
+                                         &op.attn, op.eps);
+    case Op::kAttn:
+        return nncase_hip_paged_attention_decode(ctx, op.in0, op.in1, op.in2, (const int32_t *)op.in3, (const int32_t *)op.in4,
+                                                 op.out, &op.attn);
+    case Op::kArgmax:
+        return nncase_hip_argmax_f32(ctx, (const float *)op.in0, (int32_t *)op.out, op.batch, op.channels);
+    case Op::kEmbed:
+        return nncase_hip_embedding_f16(ctx, op.in0, (const int32_t *)op.in1, op.out, op.batch, op.channels, op.w);
+    case Op::kAddI32:
+        return nncase_hip_add_i32(ctx, (int32_t *)op.out, op.batch, op.delta);
     case Op::kResize:
         return nncase_hip_resize_nearest(ctx, op.in0, op.out, op.elem_size, op.batch, op.h, op.w, op.channels, op.out_h,
                                          op.out_w, op.tmode, op.nmode);
@@ -230,6 +254,84 @@ extern "C" int nncase_hip_function_add_pack(nncase_hip_function_t *fn, const voi
     return push(fn, op);
 }
 
+extern "C" int nncase_hip_function_add_w8a16_gemm(nncase_hip_function_t *fn, const void *a_dev, const nncase_hip_w8a16_t *weights,
+                                                  void *out_dev, int32_t m, int32_t mode, const void *residual_dev,
+                                                  int32_t out_dtype) {
+    if (!fn) return -EINVAL;
+    NNHIP_REQUIRE(fn->ctx, a_dev && weights && out_dev, -EINVAL, "function_add_w8a16_gemm: null argument");
+    Op op;
+    op.kind = Op::kGemm;
+    op.in0 = a_dev, op.w8 = weights, op.out = out_dev, op.batch = m, op.mode = mode, op.in1 = residual_dev, op.dt_out = out_dtype;
+    return push(fn, op);
+}
+
+extern "C" int nncase_hip_function_add_rmsnorm_f16(nncase_hip_function_t *fn, const void *x_dev, const void *weight_dev,
+                                                   void *out_dev, int32_t rows, int32_t hidden, float eps) {
+    if (!fn) return -EINVAL;
+    NNHIP_REQUIRE(fn->ctx, x_dev && weight_dev && out_dev, -EINVAL, "function_add_rmsnorm_f16: null argument");
+    Op op;
+    op.kind = Op::kRmsNorm;
+    op.in0 = x_dev, op.in1 = weight_dev, op.out = out_dev, op.batch = rows, op.channels = hidden, op.eps = eps;
+    return push(fn, op);
+}
+
+extern "C" int nncase_hip_function_add_rope_kv_append(nncase_hip_function_t *fn, const void *qkv_dev, void *q_out_dev,
+                                                      void *k_cache_dev, void *v_cache_dev, const int32_t *block_table_dev,
+                                                      const int32_t *ctx_lens_dev, const nncase_hip_paged_attn_args_t *geometry,
+                                                      float rope_theta) {
+    if (!fn) return -EINVAL;
+    NNHIP_REQUIRE(fn->ctx, qkv_dev && q_out_dev && k_cache_dev && v_cache_dev && block_table_dev && ctx_lens_dev && geometry, -EINVAL,
+                  "function_add_rope_kv_append: null argument");
+    Op op;
+    op.kind = Op::kRope;
+    op.in0 = qkv_dev, op.out = q_out_dev, op.out2 = k_cache_dev, op.out3 = v_cache_dev, op.in2 = block_table_dev, op.in3 = ctx_lens_dev;
+    op.attn = *geometry, op.eps = rope_theta;
+    return push(fn, op);
+}
+
+extern "C" int nncase_hip_function_add_paged_attention_decode(nncase_hip_function_t *fn, const void *q_dev, const void *k_cache_dev,
+                                                              const void *v_cache_dev, const int32_t *block_table_dev,
+                                                              const int32_t *ctx_lens_dev, void *out_dev,
+                                                              const nncase_hip_paged_attn_args_t *args) {
+    if (!fn) return -EINVAL;
+    NNHIP_REQUIRE(fn->ctx, q_dev && k_cache_dev && v_cache_dev && block_table_dev && ctx_lens_dev && out_dev && args, -EINVAL,
+                  "function_add_paged_attention_decode: null argument");
+    Op op;
+    op.kind = Op::kAttn;
+    op.in0 = q_dev, op.in1 = k_cache_dev, op.in2 = v_cache_dev, op.in3 = block_table_dev, op.in4 = ctx_lens_dev, op.out = out_dev;
+    op.attn = *args;
+    return push(fn, op);
+}
+
+extern "C" int nncase_hip_function_add_argmax_f32(nncase_hip_function_t *fn, const float *x_dev, int32_t *out_dev, int32_t rows,
+                                                  int32_t cols) {
+    if (!fn) return -EINVAL;
+    NNHIP_REQUIRE(fn->ctx, x_dev && out_dev, -EINVAL, "function_add_argmax_f32: null argument");
+    Op op;
+    op.kind = Op::kArgmax;
+    op.in0 = x_dev, op.out = out_dev, op.batch = rows, op.channels = cols;
+    return push(fn, op);
+}
+
+extern "C" int nncase_hip_function_add_embedding_f16(nncase_hip_function_t *fn, const void *table_dev, const int32_t *ids_dev,
+                                                     void *out_dev, int32_t rows, int32_t hidden, int32_t vocab) {
+    if (!fn) return -EINVAL;
+    NNHIP_REQUIRE(fn->ctx, table_dev && ids_dev && out_dev, -EINVAL, "function_add_embedding_f16: null argument");
+    Op op;
+    op.kind = Op::kEmbed;
+    op.in0 = table_dev, op.in1 = ids_dev, op.out = out_dev, op.batch = rows, op.channels = hidden, op.w = vocab;
+    return push(fn, op);
+}
+
+extern "C" int nncase_hip_function_add_add_i32(nncase_hip_function_t *fn, int32_t *x_dev, int32_t count, int32_t delta) {
+    if (!fn) return -EINVAL;
+    NNHIP_REQUIRE(fn->ctx, x_dev, -EINVAL, "function_add_add_i32: null argument");
+    Op op;
+    op.kind = Op::kAddI32;
+    op.out = x_dev, op.batch = count, op.delta = delta;
+    return push(fn, op);
+}
+
 extern "C" int nncase_hip_function_size(nncase_hip_function_t *fn, int32_t *count) {
     if (!fn || !count) return -EINVAL;
     *count = (int32_t)fn->ops.size();
@@ -299,6 +401,13 @@ extern "C" int nncase_hip_function_op_kernel(nncase_hip_function_t *fn, int32_t 
     case Op::kResize: snprintf(name, capacity, "resize_nearest"); break;
     case Op::kMaxPool: snprintf(name, capacity, "qmaxpool<%dx%d>", op.pool[0], op.pool[1]); break;
     case Op::kPack: snprintf(name, capacity, "pack"); break;
+    case Op::kGemm: snprintf(name, capacity, op.mode == NNCASE_HIP_GEMM_SWIGLU ? "w8a16_gemm+swiglu" : (op.in1 ? "w8a16_gemm+residual" : "w8a16_gemm")); break;
+    case Op::kRmsNorm: snprintf(name, capacity, "rmsnorm_f16"); break;
+    case Op::kRope: snprintf(name, capacity, "rope_kv_append"); break;
+    case Op::kAttn: snprintf(name, capacity, "paged_attention_decode"); break;
+    case Op::kArgmax: snprintf(name, capacity, "argmax_f32"); break;
+    case Op::kEmbed: snprintf(name, capacity, "embedding_f16"); break;
+    case Op::kAddI32: snprintf(name, capacity, "add_i32"); break;
     }
     return 0;
 }

@@ -1,0 +1,447 @@
+// The rest of an LLM decode step around paged attention (fp16 activations, W8A16 weights):
+// RMSNorm, the small-M weight-streaming GEMM, rotary embedding + KV append into the block-paged
+// cache, arg-max, embedding gather and the per-step advance of the context lengths.
+//
+// A decode step multiplies a handful of token rows (M = batch, <= 64) with every weight matrix, so
+// each int8 weight byte is read from HBM exactly once and the step is bound by that stream
+// (~0.5 GB for a Qwen2-0.5B-shaped model).  The GEMM is organised around it: weights are
+// pre-packed so that a wave's load of one k-step is a contiguous 1 KiB fragment (16 bytes per
+// lane), converted int8 -> fp16 in registers (exactly: (w ^ 0x80) | 0x6400 is the fp16 1024 + w + 128)
+// and fed to v_mfma_f32_16x16x32_f16 as the A operand (16 output channels), the token rows being
+// the B operand; a lane ends up with 4 consecutive output channels of one token.  The four waves
+// of a block split the reduction and combine through LDS.  Per-output-channel scales, bias, the
+// residual add and the SwiGLU gate are applied in the epilogue.
+#include "common.hpp"
+
+#include <hip/hip_fp16.h>
+
+#include <cmath>
+#include <new>
+#include <vector>
+
+namespace nnhip {
+
+typedef _Float16 h16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 h16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4v __attribute__((ext_vector_type(4)));
+typedef uint32_t lu32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kLlmThreads = 256;
+constexpr int kMaxRows = 64; // token rows per GEMM call (4 MFMA column tiles)
+
+} // namespace nnhip
+
+// Pre-packed W8A16 matrix: out[m, n] = scale[n] * sum_k a[m, k] * w[n, k] (+ bias[n]).
+struct nncase_hip_w8a16 {
+    int k = 0, n = 0;      // reduction length (multiple of 64), output channels (multiple of 16)
+    int ntiles = 0, ksteps = 0;
+    void *d_packed = nullptr; // [ntiles][ksteps][64 lanes][16 B]: lane (i = l % 16, kg = l / 16) holds
+                              // w[tile * 16 + i][ks * 64 + kg * 16 .. + 15]
+    float *d_scale = nullptr; // [n]
+    float *d_bias = nullptr;  // [n] or null
+};
+
+namespace nnhip {
+
+struct GemmArgs {
+    const uint16_t *a; // [m][k] fp16
+    const lu32x4 *w;
+    const float *scale, *bias;
+    const uint16_t *residual; // [m][n_out] fp16 or null
+    void *out;                // [m][n_out] fp16 or fp32
+    int m, k, n_out, ksteps, mode, out_f32;
+    int up_tile_offset; // SwiGLU: tile t of the gate pairs with tile t + up_tile_offset of the up projection
+};
+
+// 8 int8 weights (two dwords' low / high halves handled by the caller) -> 8 fp16, exact.
+__device__ __forceinline__ h16x8 w8_to_f16(uint32_t lo, uint32_t hi) {
+    const uint32_t x0 = lo ^ 0x80808080u, x1 = hi ^ 0x80808080u;
+    uint32_t h[4];
+    h[0] = __builtin_amdgcn_perm(0x64646464u, x0, 0x07010700u); // [b0, 0x64, b1, 0x64] -> halves 1024 + b0, 1024 + b1
+    h[1] = __builtin_amdgcn_perm(0x64646464u, x0, 0x07030702u);
+    h[2] = __builtin_amdgcn_perm(0x64646464u, x1, 0x07010700u);
+    h[3] = __builtin_amdgcn_perm(0x64646464u, x1, 0x07030702u);
+    h16x8 v;
+    __builtin_memcpy(&v, h, 16);
+    return v - (_Float16)1152.0f; // 1024 + (w + 128) - 1152 = w, exact in fp16
+}
+
+// Epilogue of 4 consecutive output channels of one token: SwiGLU gate, residual, conversion, store.
+template <int G> __device__ __forceinline__ void store_gemm_row(const GemmArgs &a, const float (&v)[G][4], size_t o) {
+    float y[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        if (G == 2) y[r] = v[0][r] / (1.f + __expf(-v[0][r])) * v[G - 1][r]; // silu(gate) * up
+        else y[r] = v[0][r];
+        if (a.residual) y[r] += __half2float(reinterpret_cast<const __half *>(a.residual)[o + r]);
+    }
+    if (a.out_f32) {
+        *reinterpret_cast<float4 *>(reinterpret_cast<float *>(a.out) + o) = float4{y[0], y[1], y[2], y[3]};
+    } else {
+        __half h[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) h[r] = __float2half_rn(y[r]);
+        uint2 pk;
+        __builtin_memcpy(&pk, h, 8);
+        *reinterpret_cast<uint2 *>(reinterpret_cast<__half *>(a.out) + o) = pk;
+    }
+}
+
+// MT = 16-token column tiles (m <= 16 * MT); G = matrices multiplied at once (2: SwiGLU gate and up).
+// grid.x = output tiles of 16 channels.  The eight waves of a block split the reduction; a wave
+// requests the weights and token slices of four k-steps before it multiplies any of them, so a
+// whole share of a short reduction (896 / 8 waves = 2 k-steps) is a single memory round trip.
+constexpr int kGemmWaves = 8;
+constexpr int kGemmThreads = kGemmWaves * 64;
+constexpr int kGemmBatch = 4;
+
+// SPLIT: the block's waves share one output tile and split its reduction (few tiles, long reductions);
+// otherwise every wave owns a tile of its own and the whole reduction (many tiles: the vocabulary head).
+template <int MT, int G, bool SPLIT> __global__ __launch_bounds__(kGemmThreads) void w8a16_gemm_kernel(const GemmArgs a) {
+    __shared__ float red[SPLIT ? kGemmWaves : 1][G][MT][64][4];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int i16 = lane & 15, kg = lane >> 4;
+    const int per = SPLIT ? (a.ksteps + kGemmWaves - 1) / kGemmWaves : a.ksteps;
+    const int ks0 = SPLIT ? wave * per : 0, ks1 = min(a.ksteps, ks0 + per);
+    const int out_tile = SPLIT ? (int)blockIdx.x : (int)blockIdx.x * kGemmWaves + wave;
+    if (out_tile >= a.up_tile_offset) return; // SPLIT: never; otherwise the last block's spare waves (uniform per wave)
+    f32x4v acc[G][MT];
+#pragma unroll
+    for (int g = 0; g < G; g++)
+#pragma unroll
+        for (int t = 0; t < MT; t++) acc[g][t] = f32x4v{0.f, 0.f, 0.f, 0.f};
+
+    const int tile[2] = {out_tile, out_tile + a.up_tile_offset};
+    // token rows of this lane (clamped: rows past m read row m - 1 and are never stored)
+    const uint16_t *arow[MT];
+#pragma unroll
+    for (int t = 0; t < MT; t++) arow[t] = a.a + (size_t)min(t * 16 + i16, a.m - 1) * a.k + kg * 16;
+
+    for (int kb = ks0; kb < ks1; kb += kGemmBatch) {
+        lu32x4 wv[kGemmBatch][G];
+        lu32x4 av[kGemmBatch][MT][2];
+#pragma unroll
+        for (int u = 0; u < kGemmBatch; u++) {
+            const int ks = min(kb + u, ks1 - 1); // steps past the share re-read the last one and are not multiplied
+#pragma unroll
+            for (int g = 0; g < G; g++) wv[u][g] = a.w[((size_t)tile[g] * a.ksteps + ks) * 64 + lane];
+#pragma unroll
+            for (int t = 0; t < MT; t++) {
+                av[u][t][0] = *reinterpret_cast<const lu32x4 *>(arow[t] + ks * 64);
+                av[u][t][1] = *reinterpret_cast<const lu32x4 *>(arow[t] + ks * 64 + 8);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kGemmBatch; u++) {
+            if (kb + u < ks1) { // uniform for the wave
+#pragma unroll
+                for (int g = 0; g < G; g++) {
+                    const h16x8 w0 = w8_to_f16(wv[u][g][0], wv[u][g][1]), w1 = w8_to_f16(wv[u][g][2], wv[u][g][3]);
+#pragma unroll
+                    for (int t = 0; t < MT; t++) {
+                        h16x8 x0, x1;
+                        __builtin_memcpy(&x0, &av[u][t][0], 16);
+                        __builtin_memcpy(&x1, &av[u][t][1], 16);
+                        acc[g][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w0, x0, acc[g][t], 0, 0, 0);
+                        acc[g][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w1, x1, acc[g][t], 0, 0, 0);
+                    }
+                }
+            }
+        }
+    }
+    // ---- combine the waves' partial sums ------------------------------------------------------------
+    if (SPLIT) {
+#pragma unroll
+        for (int g = 0; g < G; g++)
+#pragma unroll
+            for (int t = 0; t < MT; t++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) red[wave][g][t][lane][r] = acc[g][t][r];
+        __syncthreads();
+        if (wave >= MT) return; // wave w finishes token tile w
+    }
+    // lane (i16 = token within the tile, kg): channels tile * 16 + kg * 4 + r
+#pragma unroll
+    for (int tt = 0; tt < (SPLIT ? 1 : MT); tt++) {
+        const int t = SPLIT ? wave : tt;
+        const int m = t * 16 + i16;
+        float v[G][4];
+#pragma unroll
+        for (int g = 0; g < G; g++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                float s = 0.f;
+                if (SPLIT) {
+#pragma unroll
+                    for (int w = 0; w < kGemmWaves; w++) s += red[w][g][t][lane][r]; // fixed order: deterministic
+                } else {
+                    s = acc[g][tt][r];
+                }
+                const int ch = tile[g] * 16 + kg * 4 + r;
+                s *= a.scale[ch];
+                if (a.bias) s += a.bias[ch];
+                v[g][r] = s;
+            }
+        if (m >= a.m) continue;
+        store_gemm_row<G>(a, v, (size_t)m * a.n_out + out_tile * 16 + kg * 4);
+    }
+}
+
+// out[r, :] = x[r, :] * rsqrt(mean(x[r, :]^2) + eps) * weight, fp32 arithmetic; one wave per row.
+__global__ __launch_bounds__(kLlmThreads) void rmsnorm_f16_kernel(const __half *__restrict__ x, const __half *__restrict__ w,
+                                                                 __half *__restrict__ out, int rows, int hidden, float eps) {
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (row >= rows) return;
+    const __half *xr = x + (size_t)row * hidden;
+    float ss = 0.f;
+    for (int i = lane; i < hidden; i += 64) {
+        const float v = __half2float(xr[i]);
+        ss += v * v;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+    const float r = 1.0f / sqrtf(ss / (float)hidden + eps);
+    for (int i = lane; i < hidden; i += 64)
+        out[(size_t)row * hidden + i] = __float2half_rn(__half2float(xr[i]) * r * __half2float(w[i]));
+}
+
+struct RopeArgs {
+    const __half *qkv; // [batch][(hq + 2 * hkv) * d]: q heads, then k heads, then v heads
+    __half *q_out;     // [batch][hq][d]
+    __half *k_cache;   // [blocks][hkv][block][d]
+    __half *v_cache;   // [blocks][hkv][d][block]
+    const int32_t *block_table, *ctx_lens; // the new token of sequence b goes to position ctx_lens[b]
+    int batch, hq, hkv, d, block_size, max_blocks, num_blocks;
+    float theta;
+};
+
+// Rotary embedding (rotate-half pairing: element i with i + d/2, angle pos * theta^(-2i/d)) of the q
+// and k heads of the new token, and the append of the rotated k and of v at position ctx_lens[b]
+// of the paged cache.  One thread per (sequence, head, pair).
+__global__ __launch_bounds__(kLlmThreads) void rope_append_kernel(const RopeArgs a) {
+    const int half = a.d / 2;
+    const int heads = a.hq + 2 * a.hkv;
+    const int gid = blockIdx.x * kLlmThreads + threadIdx.x;
+    if (gid >= a.batch * heads * half) return;
+    const int i = gid % half, h = (gid / half) % heads, b = gid / (half * heads);
+    const __half *src = a.qkv + ((size_t)b * heads + h) * a.d;
+    const float x0 = __half2float(src[i]), x1 = __half2float(src[i + half]);
+    const int pos = a.ctx_lens[b];
+    const int lb = pos / a.block_size, in_block = pos - lb * a.block_size;
+    const bool fits = lb < a.max_blocks;
+    const int pb = fits ? min(max(a.block_table[(size_t)b * a.max_blocks + lb], 0), a.num_blocks - 1) : 0;
+    if (h < a.hq + a.hkv) {
+        const float inv = powf(a.theta, -2.0f * (float)i / (float)a.d);
+        const float ang = (float)pos * inv;
+        const float c = cosf(ang), s = sinf(ang);
+        const __half y0 = __float2half_rn(x0 * c - x1 * s), y1 = __float2half_rn(x1 * c + x0 * s);
+        if (h < a.hq) {
+            __half *dst = a.q_out + ((size_t)b * a.hq + h) * a.d;
+            dst[i] = y0, dst[i + half] = y1;
+        } else if (fits) {
+            __half *dst = a.k_cache + ((((size_t)pb * a.hkv + (h - a.hq)) * a.block_size) + in_block) * a.d;
+            dst[i] = y0, dst[i + half] = y1;
+        }
+    } else if (fits) {
+        __half *dst = a.v_cache + ((size_t)pb * a.hkv + (h - a.hq - a.hkv)) * a.d * a.block_size + in_block;
+        dst[(size_t)i * a.block_size] = __float2half_rn(x0);
+        dst[(size_t)(i + half) * a.block_size] = __float2half_rn(x1);
+    }
+}
+
+// Index of the largest element of every row (the lowest index among equals); one block of 1024
+// threads per row, 16-byte loads, so that a 152 K-entry vocabulary row is a few dozen independent
+// loads per thread.
+constexpr int kArgmaxThreads = 1024;
+__device__ __forceinline__ void argmax_take(float v, int i, float &best, int &bi) {
+    if (v > best || (v == best && i < bi)) best = v, bi = i;
+}
+__global__ __launch_bounds__(kArgmaxThreads) void argmax_f32_kernel(const float *__restrict__ x, int32_t *__restrict__ out, int cols) {
+    __shared__ float sv[kArgmaxThreads];
+    __shared__ int si[kArgmaxThreads];
+    const float *row = x + (size_t)blockIdx.x * cols;
+    float best = -INFINITY;
+    int bi = 0x7fffffff;
+    // rows start 16-byte aligned when cols is a multiple of 4 (x itself is aligned by the allocator)
+    const int nvec = ((cols & 3) == 0 && (reinterpret_cast<uintptr_t>(x) & 15u) == 0) ? cols / 4 : 0;
+    for (int i = threadIdx.x; i < nvec; i += kArgmaxThreads) {
+        const float4 v = reinterpret_cast<const float4 *>(row)[i];
+        argmax_take(v.x, 4 * i, best, bi);
+        argmax_take(v.y, 4 * i + 1, best, bi);
+        argmax_take(v.z, 4 * i + 2, best, bi);
+        argmax_take(v.w, 4 * i + 3, best, bi);
+    }
+    for (int i = nvec * 4 + threadIdx.x; i < cols; i += kArgmaxThreads) argmax_take(row[i], i, best, bi);
+    sv[threadIdx.x] = best, si[threadIdx.x] = bi;
+    __syncthreads();
+    for (int s = kArgmaxThreads / 2; s > 0; s >>= 1) {
+        if (threadIdx.x < s) argmax_take(sv[threadIdx.x + s], si[threadIdx.x + s], sv[threadIdx.x], si[threadIdx.x]);
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) out[blockIdx.x] = si[0] == 0x7fffffff ? 0 : si[0];
+}
+
+__global__ __launch_bounds__(kLlmThreads) void embed_f16_kernel(const __half *__restrict__ table, const int32_t *__restrict__ ids,
+                                                               __half *__restrict__ out, int rows, int hidden, int vocab) {
+    const int gid = blockIdx.x * kLlmThreads + threadIdx.x;
+    if (gid >= rows * hidden) return;
+    const int r = gid / hidden, c = gid - r * hidden;
+    const int id = min(max(ids[r], 0), vocab - 1);
+    out[gid] = table[(size_t)id * hidden + c];
+}
+
+__global__ void add_i32_kernel(int32_t *x, int n, int32_t delta) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) x[i] += delta;
+}
+
+} // namespace nnhip
+
+using namespace nnhip;
+
+extern "C" int nncase_hip_w8a16_destroy(nncase_hip_ctx_t *ctx, nncase_hip_w8a16_t *w) {
+    NNHIP_CHECK_CTX(ctx);
+    if (!w) return 0;
+    NNHIP_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    if (w->d_packed) (void)hipFree(w->d_packed);
+    if (w->d_scale) (void)hipFree(w->d_scale);
+    if (w->d_bias) (void)hipFree(w->d_bias);
+    delete w;
+    return 0;
+}
+
+extern "C" int nncase_hip_w8a16_prepack(nncase_hip_ctx_t *ctx, const int8_t *w_host, const float *scale_host,
+                                        const float *bias_host, int32_t k, int32_t n, nncase_hip_w8a16_t **out) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, w_host && scale_host && out, -EINVAL, "w8a16_prepack: null argument");
+    *out = nullptr;
+    NNHIP_REQUIRE(ctx, k > 0 && n > 0 && k % 64 == 0 && n % 16 == 0, -NNCASE_HIP_ERR_SHAPE_MISMATCH,
+                  "w8a16_prepack: k = %d must be a multiple of 64 and n = %d a multiple of 16", k, n);
+    nncase_hip_w8a16 *w = new (std::nothrow) nncase_hip_w8a16();
+    NNHIP_REQUIRE(ctx, w, -ENOMEM, "w8a16_prepack: out of host memory");
+    w->k = k, w->n = n, w->ntiles = n / 16, w->ksteps = k / 64;
+    const size_t bytes = (size_t)n * k;
+    std::vector<int8_t> packed(bytes);
+    for (int t = 0; t < w->ntiles; t++)
+        for (int ks = 0; ks < w->ksteps; ks++)
+            for (int l = 0; l < 64; l++) {
+                const int i = l & 15, kg = l >> 4;
+                memcpy(&packed[(((size_t)t * w->ksteps + ks) * 64 + l) * 16], w_host + (size_t)(t * 16 + i) * k + ks * 64 + kg * 16, 16);
+            }
+    auto cleanup = [&](int rc) {
+        (void)nncase_hip_w8a16_destroy(ctx, w);
+        return rc;
+    };
+    if (hipMalloc(&w->d_packed, bytes) != hipSuccess || hipMalloc((void **)&w->d_scale, sizeof(float) * n) != hipSuccess)
+        return cleanup(fail(ctx, -ENOMEM, "w8a16_prepack: out of device memory"));
+    if (bias_host && hipMalloc((void **)&w->d_bias, sizeof(float) * n) != hipSuccess)
+        return cleanup(fail(ctx, -ENOMEM, "w8a16_prepack: out of device memory"));
+    if (hipMemcpy(w->d_packed, packed.data(), bytes, hipMemcpyHostToDevice) != hipSuccess ||
+        hipMemcpy(w->d_scale, scale_host, sizeof(float) * n, hipMemcpyHostToDevice) != hipSuccess ||
+        (bias_host && hipMemcpy(w->d_bias, bias_host, sizeof(float) * n, hipMemcpyHostToDevice) != hipSuccess))
+        return cleanup(fail(ctx, -EIO, "w8a16_prepack: upload failed"));
+    *out = w;
+    return 0;
+}
+
+extern "C" int nncase_hip_w8a16_gemm(nncase_hip_ctx_t *ctx, const void *a_dev, const nncase_hip_w8a16_t *w, void *out_dev,
+                                     int32_t m, int32_t mode, const void *residual_dev, int32_t out_dtype) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, a_dev && w && out_dev, -EINVAL, "w8a16_gemm: null argument");
+    NNHIP_REQUIRE(ctx, m > 0 && m <= kMaxRows, -NNCASE_HIP_ERR_SHAPE_MISMATCH, "w8a16_gemm: %d token rows (1..%d supported)", m, kMaxRows);
+    NNHIP_REQUIRE(ctx, mode == NNCASE_HIP_GEMM_PLAIN || mode == NNCASE_HIP_GEMM_SWIGLU, -EINVAL, "w8a16_gemm: unknown mode %d", mode);
+    NNHIP_REQUIRE(ctx, out_dtype == NNCASE_HIP_DT_F16 || out_dtype == NNCASE_HIP_DT_F32, -NNCASE_HIP_ERR_DATATYPE_MISMATCH,
+                  "w8a16_gemm: output type 0x%x", out_dtype);
+    NNHIP_REQUIRE(ctx, mode != NNCASE_HIP_GEMM_SWIGLU || w->ntiles % 2 == 0, -NNCASE_HIP_ERR_SHAPE_MISMATCH,
+                  "w8a16_gemm: SwiGLU needs gate and up halves of equal size");
+    NNHIP_REQUIRE(ctx, ((reinterpret_cast<uintptr_t>(a_dev) | reinterpret_cast<uintptr_t>(out_dev)) & 15u) == 0,
+                  -NNCASE_HIP_ERR_INVALID_MEMORY_LOCATION, "w8a16_gemm: buffers must be 16-byte aligned");
+    GemmArgs a;
+    memset(&a, 0, sizeof(a));
+    a.a = (const uint16_t *)a_dev;
+    a.w = (const lu32x4 *)w->d_packed;
+    a.scale = w->d_scale, a.bias = w->d_bias;
+    a.residual = (const uint16_t *)residual_dev;
+    a.out = out_dev;
+    a.m = m, a.k = w->k, a.ksteps = w->ksteps, a.mode = mode, a.out_f32 = out_dtype == NNCASE_HIP_DT_F32;
+    const int out_tiles = mode == NNCASE_HIP_GEMM_SWIGLU ? w->ntiles / 2 : w->ntiles;
+    a.up_tile_offset = out_tiles;
+    a.n_out = out_tiles * 16;
+    // few output tiles: the block's waves split the reduction of one tile; many: a tile per wave
+    const bool split = out_tiles < 4 * ctx->compute_units;
+    const dim3 grid(split ? out_tiles : (out_tiles + kGemmWaves - 1) / kGemmWaves), block(kGemmThreads);
+    const int mt = (m + 15) / 16;
+    const bool glu = mode == NNCASE_HIP_GEMM_SWIGLU;
+#define NNHIP_GEMM_LAUNCH(MTV)                                                                                                 \
+    do {                                                                                                                       \
+        if (glu && split) hipLaunchKernelGGL((w8a16_gemm_kernel<MTV, 2, true>), grid, block, 0, ctx->stream, a);              \
+        else if (glu) hipLaunchKernelGGL((w8a16_gemm_kernel<MTV, 2, false>), grid, block, 0, ctx->stream, a);                 \
+        else if (split) hipLaunchKernelGGL((w8a16_gemm_kernel<MTV, 1, true>), grid, block, 0, ctx->stream, a);                \
+        else hipLaunchKernelGGL((w8a16_gemm_kernel<MTV, 1, false>), grid, block, 0, ctx->stream, a);                          \
+    } while (0)
+    if (mt == 1) NNHIP_GEMM_LAUNCH(1);
+    else if (mt == 2) NNHIP_GEMM_LAUNCH(2);
+    else NNHIP_GEMM_LAUNCH(4);
+#undef NNHIP_GEMM_LAUNCH
+    NNHIP_LAUNCH_CHECK(ctx, "w8a16_gemm_kernel");
+    return 0;
+}
+
+extern "C" int nncase_hip_rmsnorm_f16(nncase_hip_ctx_t *ctx, const void *x_dev, const void *weight_dev, void *out_dev, int32_t rows,
+                                      int32_t hidden, float eps) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, x_dev && weight_dev && out_dev && rows > 0 && hidden > 0, -EINVAL, "rmsnorm_f16: bad argument");
+    hipLaunchKernelGGL(rmsnorm_f16_kernel, dim3((rows + 3) / 4), dim3(kLlmThreads), 0, ctx->stream, (const __half *)x_dev,
+                       (const __half *)weight_dev, (__half *)out_dev, rows, hidden, eps);
+    NNHIP_LAUNCH_CHECK(ctx, "rmsnorm_f16_kernel");
+    return 0;
+}
+
+extern "C" int nncase_hip_rope_kv_append(nncase_hip_ctx_t *ctx, const void *qkv_dev, void *q_out_dev, void *k_cache_dev,
+                                         void *v_cache_dev, const int32_t *block_table_dev, const int32_t *ctx_lens_dev,
+                                         const nncase_hip_paged_attn_args_t *p, float rope_theta) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, qkv_dev && q_out_dev && k_cache_dev && v_cache_dev && block_table_dev && ctx_lens_dev && p, -EINVAL,
+                  "rope_kv_append: null argument");
+    NNHIP_REQUIRE(ctx, p->batch > 0 && p->num_q_heads > 0 && p->num_kv_heads > 0 && p->head_dim > 0 && p->head_dim % 2 == 0 &&
+                           p->block_size > 0 && p->max_blocks_per_seq > 0 && p->num_blocks > 0 && rope_theta > 0.f,
+                  -EINVAL, "rope_kv_append: bad geometry");
+    RopeArgs a;
+    a.qkv = (const __half *)qkv_dev, a.q_out = (__half *)q_out_dev, a.k_cache = (__half *)k_cache_dev, a.v_cache = (__half *)v_cache_dev;
+    a.block_table = block_table_dev, a.ctx_lens = ctx_lens_dev;
+    a.batch = p->batch, a.hq = p->num_q_heads, a.hkv = p->num_kv_heads, a.d = p->head_dim, a.block_size = p->block_size;
+    a.max_blocks = p->max_blocks_per_seq, a.num_blocks = p->num_blocks, a.theta = rope_theta;
+    const int64_t total = (int64_t)a.batch * (a.hq + 2 * a.hkv) * (a.d / 2);
+    NNHIP_REQUIRE(ctx, total < ((int64_t)1 << 31), -EINVAL, "rope_kv_append: too large");
+    hipLaunchKernelGGL(rope_append_kernel, dim3((unsigned)((total + kLlmThreads - 1) / kLlmThreads)), dim3(kLlmThreads), 0, ctx->stream, a);
+    NNHIP_LAUNCH_CHECK(ctx, "rope_append_kernel");
+    return 0;
+}
+
+extern "C" int nncase_hip_argmax_f32(nncase_hip_ctx_t *ctx, const float *x_dev, int32_t *out_dev, int32_t rows, int32_t cols) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, x_dev && out_dev && rows > 0 && cols > 0, -EINVAL, "argmax_f32: bad argument");
+    hipLaunchKernelGGL(argmax_f32_kernel, dim3(rows), dim3(kArgmaxThreads), 0, ctx->stream, x_dev, out_dev, cols);
+    NNHIP_LAUNCH_CHECK(ctx, "argmax_f32_kernel");
+    return 0;
+}
+
+extern "C" int nncase_hip_embedding_f16(nncase_hip_ctx_t *ctx, const void *table_dev, const int32_t *ids_dev, void *out_dev,
+                                        int32_t rows, int32_t hidden, int32_t vocab) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, table_dev && ids_dev && out_dev && rows > 0 && hidden > 0 && vocab > 0, -EINVAL, "embedding_f16: bad argument");
+    const int64_t total = (int64_t)rows * hidden;
+    NNHIP_REQUIRE(ctx, total < ((int64_t)1 << 31), -EINVAL, "embedding_f16: too large");
+    hipLaunchKernelGGL(embed_f16_kernel, dim3((unsigned)((total + kLlmThreads - 1) / kLlmThreads)), dim3(kLlmThreads), 0, ctx->stream,
+                       (const __half *)table_dev, ids_dev, (__half *)out_dev, rows, hidden, vocab);
+    NNHIP_LAUNCH_CHECK(ctx, "embed_f16_kernel");
+    return 0;
+}
+
+extern "C" int nncase_hip_add_i32(nncase_hip_ctx_t *ctx, int32_t *x_dev, int32_t count, int32_t delta) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, x_dev && count > 0, -EINVAL, "add_i32: bad argument");
+    hipLaunchKernelGGL(add_i32_kernel, dim3((count + 255) / 256), dim3(256), 0, ctx->stream, x_dev, count, delta);
+    NNHIP_LAUNCH_CHECK(ctx, "add_i32_kernel");
+    return 0;
+}

@@ -1,0 +1,149 @@
+"""A Qwen2-shaped decoder for the decode step of the LLM benchmark configuration: random-init W8A16
+weights (int8 per output channel, fp16 activations), RMSNorm, rotary embedding, a block-paged fp16
+KV cache and greedy sampling, recorded once as a resident `hip` function (one HIP-graph replay per
+generated token for the whole batch).
+
+Per layer:  h = x + O(attn(rope(QKV(rmsnorm(x)))));  x' = h + Down(silu(Gate(n)) * Up(n)), n = rmsnorm(h)
+Last:       logits = LMHead(rmsnorm(x));  next token = argmax(logits)
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, List, Optional
+
+import numpy as np
+
+from . import runtime as rt
+from .runtime import Context, Function
+
+
+@dataclass
+class DecoderConfig:
+    layers: int = 24
+    hidden: int = 896
+    q_heads: int = 14
+    kv_heads: int = 2
+    head_dim: int = 64
+    mlp: int = 4864
+    vocab: int = 151936
+    rms_eps: float = 1e-6
+    rope_theta: float = 1e6
+    block_size: int = 16
+
+
+def quantize_rows(w: np.ndarray):
+    """Per-output-channel symmetric int8: w[n, :] ~ scale[n] * q[n, :], q in [-127, 127]."""
+    amax = np.maximum(np.abs(w).max(axis=1), 1e-8)
+    scale = (amax / 127.0).astype(np.float32)
+    q = np.clip(np.rint(w / scale[:, None]), -127, 127).astype(np.int8)
+    return q, scale
+
+
+def random_weights(cfg: DecoderConfig, seed: int = 5) -> Dict[str, object]:
+    """Host-side weights of the whole model (numpy), shared by the device model and the float64 reference."""
+    rng = np.random.default_rng(seed)
+    qd = cfg.q_heads * cfg.head_dim
+    kvd = cfg.kv_heads * cfg.head_dim
+
+    def lin(n, k, std):
+        return quantize_rows((rng.standard_normal((n, k), dtype=np.float32) * std))
+
+    layers = []
+    for _ in range(cfg.layers):
+        layers.append({
+            "ln1": (1.0 + 0.1 * rng.standard_normal(cfg.hidden)).astype(np.float16),
+            "qkv": lin(qd + 2 * kvd, cfg.hidden, cfg.hidden ** -0.5),
+            "qkv_bias": (rng.standard_normal(qd + 2 * kvd) * 0.1).astype(np.float32),
+            "o": lin(cfg.hidden, qd, qd ** -0.5 * 0.5),
+            "ln2": (1.0 + 0.1 * rng.standard_normal(cfg.hidden)).astype(np.float16),
+            "gate_up": lin(2 * cfg.mlp, cfg.hidden, cfg.hidden ** -0.5),
+            "down": lin(cfg.hidden, cfg.mlp, cfg.mlp ** -0.5 * 0.5),
+        })
+    emb = (rng.standard_normal((cfg.vocab, cfg.hidden), dtype=np.float32) * 0.5).astype(np.float16)
+    return {"layers": layers, "embedding": emb, "ln_f": (1.0 + 0.1 * rng.standard_normal(cfg.hidden)).astype(np.float16),
+            "lm_head": lin(cfg.vocab, cfg.hidden, cfg.hidden ** -0.5)}
+
+
+class HipDecoder:
+    """The decode step resident on the device.  The KV cache is pre-filled by the caller (`k_cache`, `v_cache`
+    numpy arrays in the paged layouts) for the given context lengths; step() appends one token per sequence."""
+
+    def __init__(self, ctx: Context, cfg: DecoderConfig, weights: Dict[str, object], batch: int, max_blocks_per_seq: int,
+                 block_table: np.ndarray, ctx_lens: np.ndarray, k_caches: List[np.ndarray], v_caches: List[np.ndarray],
+                 capture_graph: bool = True, feedback: bool = False):
+        self.ctx, self.cfg, self.batch = ctx, cfg, batch
+        c = cfg
+        qd, kvd = c.q_heads * c.head_dim, c.kv_heads * c.head_dim
+        num_blocks = k_caches[0].shape[0]
+        f16 = 2
+        self.tokens = ctx.alloc(batch * 4)
+        self.next_tokens = ctx.alloc(batch * 4)
+        self.block_table = ctx.to_device(np.ascontiguousarray(block_table, np.int32))
+        self.ctx_lens = ctx.to_device(np.ascontiguousarray(ctx_lens, np.int32))
+        self.x = [ctx.alloc(batch * c.hidden * f16), ctx.alloc(batch * c.hidden * f16)]
+        self.norm = ctx.alloc(batch * c.hidden * f16)
+        self.qkv = ctx.alloc(batch * (qd + 2 * kvd) * f16)
+        self.q = ctx.alloc(batch * qd * f16)
+        self.att = ctx.alloc(batch * qd * f16)
+        self.act = ctx.alloc(batch * c.mlp * f16)
+        self.logits = ctx.alloc(batch * c.vocab * 4)
+        self.embedding = ctx.to_device(weights["embedding"])
+        self.ln_f = ctx.to_device(weights["ln_f"])
+        self.lm_head = ctx.prepack_w8a16(*weights["lm_head"])
+        self.geometry = rt.PagedAttnArgs(batch, c.q_heads, c.kv_heads, c.head_dim, c.block_size, max_blocks_per_seq, num_blocks,
+                                         float(c.head_dim ** -0.5), rt.DT_F16)
+        self.attn_args = rt.PagedAttnArgs(batch, c.q_heads, c.kv_heads, c.head_dim, c.block_size, max_blocks_per_seq, num_blocks,
+                                          float(c.head_dim ** -0.5), rt.DT_F16, 1)
+        self.layers = []
+        fn = Function(ctx)
+        fn.add_embedding_f16(self.embedding, self.tokens, self.x[0], batch, c.hidden, c.vocab)
+        for li, lw in enumerate(weights["layers"]):
+            L = {"ln1": ctx.to_device(lw["ln1"]), "ln2": ctx.to_device(lw["ln2"]),
+                 "qkv": ctx.prepack_w8a16(lw["qkv"][0], lw["qkv"][1], lw["qkv_bias"]), "o": ctx.prepack_w8a16(*lw["o"]),
+                 "gate_up": ctx.prepack_w8a16(*lw["gate_up"]), "down": ctx.prepack_w8a16(*lw["down"]),
+                 "k": ctx.to_device(np.ascontiguousarray(k_caches[li], np.float16)),
+                 "v": ctx.to_device(np.ascontiguousarray(v_caches[li], np.float16))}
+            self.layers.append(L)
+            x, h = self.x[0], self.x[1]
+            fn.add_rmsnorm_f16(x, L["ln1"], self.norm, batch, c.hidden, c.rms_eps)
+            fn.add_w8a16_gemm(self.norm, L["qkv"], self.qkv, batch)
+            fn.add_rope_kv_append(self.qkv, self.q, L["k"], L["v"], self.block_table, self.ctx_lens, self.geometry, c.rope_theta)
+            # the appended token takes part in its own attention (lengths + 1); the lengths themselves advance
+            # once, at the end of the step
+            fn.add_paged_attention_decode(self.q, L["k"], L["v"], self.block_table, self.ctx_lens, self.att, self.attn_args)
+            fn.add_w8a16_gemm(self.att, L["o"], h, batch, residual=x)
+            fn.add_rmsnorm_f16(h, L["ln2"], self.norm, batch, c.hidden, c.rms_eps)
+            fn.add_w8a16_gemm(self.norm, L["gate_up"], self.act, batch, mode=rt.GEMM_SWIGLU)
+            fn.add_w8a16_gemm(self.act, L["down"], x, batch, residual=h)
+        fn.add_rmsnorm_f16(self.x[0], self.ln_f, self.norm, batch, c.hidden, c.rms_eps)
+        fn.add_w8a16_gemm(self.norm, self.lm_head, self.logits, batch, out_dtype=rt.DT_F32)
+        # feedback: the arg-max lands in the token buffer the next step's embedding reads (greedy generation
+        # without a host round trip); otherwise the caller feeds every step's tokens
+        self.feedback = feedback
+        fn.add_argmax_f32(self.logits, self.tokens if feedback else self.next_tokens, batch, c.vocab)
+        fn.add_add_i32(self.ctx_lens, batch, 1)   # the step is complete: the caches hold one more token
+        self.fn = fn
+        # warm-up (sizes the attention workspace before capture) on a scratch copy of the state it changes:
+        # the caches get the token appended again by the first real step, the lengths are restored
+        self.tokens.upload(np.zeros(batch, np.int32))
+        fn.invoke()
+        ctx.sync()
+        self.ctx_lens.upload(np.ascontiguousarray(ctx_lens, np.int32))
+        if capture_graph:
+            fn.capture()
+
+    def set_tokens(self, ids: np.ndarray):
+        self.tokens.upload(np.ascontiguousarray(ids, np.int32))
+
+    def step(self):
+        """One decode step for the whole batch (asynchronous)."""
+        self.fn.invoke()
+
+    def result(self) -> np.ndarray:
+        return (self.tokens if self.feedback else self.next_tokens).download((self.batch,), np.int32)
+
+    def weight_bytes(self) -> int:
+        c = self.cfg
+        qd, kvd = c.q_heads * c.head_dim, c.kv_heads * c.head_dim
+        per_layer = (qd + 2 * kvd) * c.hidden + c.hidden * qd + 2 * c.mlp * c.hidden + c.hidden * c.mlp
+        return c.layers * per_layer + c.vocab * c.hidden

@@ -61,7 +61,7 @@ class MatmulArgs(C.Structure):
 class PagedAttnArgs(C.Structure):
     _fields_ = [("batch", C.c_int32), ("num_q_heads", C.c_int32), ("num_kv_heads", C.c_int32),
                 ("head_dim", C.c_int32), ("block_size", C.c_int32), ("max_blocks_per_seq", C.c_int32),
-                ("num_blocks", C.c_int32), ("scale", C.c_float), ("out_dtype", C.c_int32)]
+                ("num_blocks", C.c_int32), ("scale", C.c_float), ("out_dtype", C.c_int32), ("ctx_len_offset", C.c_int32)]
 
 
 # name -> (restype, argtypes); every symbol include/nncase_hip.h declares
@@ -104,6 +104,21 @@ SYMBOLS = {
     "nncase_hip_qmaxpool2d": (_I, [_VP, _VP, _VP] + [C.c_int32] * 12 + [QuantParam, QuantParam]),
     "nncase_hip_function_add_qmaxpool2d": (_I, [_VP, _VP, _VP] + [C.c_int32] * 12 + [QuantParam, QuantParam]),
     "nncase_hip_function_add_pack": (_I, [_VP, _VP, _VP, C.c_int32, C.c_int32, _I32P, C.c_int32, _I32P, _I32P]),
+    "nncase_hip_w8a16_prepack": (_I, [_VP, _VP, _VP, _VP, C.c_int32, C.c_int32, C.POINTER(_VP)]),
+    "nncase_hip_w8a16_destroy": (_I, [_VP, _VP]),
+    "nncase_hip_w8a16_gemm": (_I, [_VP, _VP, _VP, _VP, C.c_int32, C.c_int32, _VP, C.c_int32]),
+    "nncase_hip_rmsnorm_f16": (_I, [_VP, _VP, _VP, _VP, C.c_int32, C.c_int32, C.c_float]),
+    "nncase_hip_rope_kv_append": (_I, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, C.POINTER(PagedAttnArgs), C.c_float]),
+    "nncase_hip_argmax_f32": (_I, [_VP, _VP, _VP, C.c_int32, C.c_int32]),
+    "nncase_hip_embedding_f16": (_I, [_VP, _VP, _VP, _VP, C.c_int32, C.c_int32, C.c_int32]),
+    "nncase_hip_add_i32": (_I, [_VP, _VP, C.c_int32, C.c_int32]),
+    "nncase_hip_function_add_w8a16_gemm": (_I, [_VP, _VP, _VP, _VP, C.c_int32, C.c_int32, _VP, C.c_int32]),
+    "nncase_hip_function_add_rmsnorm_f16": (_I, [_VP, _VP, _VP, _VP, C.c_int32, C.c_int32, C.c_float]),
+    "nncase_hip_function_add_rope_kv_append": (_I, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, C.POINTER(PagedAttnArgs), C.c_float]),
+    "nncase_hip_function_add_paged_attention_decode": (_I, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, C.POINTER(PagedAttnArgs)]),
+    "nncase_hip_function_add_argmax_f32": (_I, [_VP, _VP, _VP, C.c_int32, C.c_int32]),
+    "nncase_hip_function_add_embedding_f16": (_I, [_VP, _VP, _VP, _VP, C.c_int32, C.c_int32, C.c_int32]),
+    "nncase_hip_function_add_add_i32": (_I, [_VP, _VP, C.c_int32, C.c_int32]),
     "nncase_hip_kmodel_load": (_I, [_VP, _VP, _SZ, C.POINTER(_VP)]),
     "nncase_hip_kmodel_destroy": (_I, [_VP]),
     "nncase_hip_kmodel_function": (_I, [_VP, C.POINTER(_VP)]),
@@ -162,6 +177,7 @@ def qp(zero_point: int, scale: float) -> QuantParam:
     return QuantParam(int(zero_point), float(np.float32(scale)))
 
 
+GEMM_PLAIN, GEMM_SWIGLU = 0, 1
 LUT_REQUANT, LUT_SWISH = 0, 1
 RESIZE_HALF_PIXEL, RESIZE_PYTORCH_HALF_PIXEL, RESIZE_ALIGN_CORNERS, RESIZE_ASYMMETRIC, RESIZE_TFCROP_AND_RESIZE = range(5)
 NEAREST_ROUND_PREFER_FLOOR, NEAREST_ROUND_PREFER_CEIL, NEAREST_FLOOR, NEAREST_CEIL = range(4)
@@ -402,6 +418,31 @@ class Context:
     def nhwc_to_nchw(self, src: DeviceBuffer, dst: DeviceBuffer, elem_size, n, c, h, w):
         self._check(self.lib.nncase_hip_nhwc_to_nchw(self.handle, src.ptr, dst.ptr, elem_size, n, c, h, w), "nhwc_to_nchw")
 
+    # -- decode-step operators ---------------------------------------------------------------
+    def prepack_w8a16(self, w_nk: np.ndarray, scale: np.ndarray, bias: Optional[np.ndarray] = None) -> "W8A16":
+        return W8A16(self, w_nk, scale, bias)
+
+    def w8a16_gemm(self, a: DeviceBuffer, w: "W8A16", out: DeviceBuffer, m: int, mode: int = GEMM_PLAIN,
+                   residual: Optional[DeviceBuffer] = None, out_dtype: int = DT_F16):
+        self._check(self.lib.nncase_hip_w8a16_gemm(self.handle, a.ptr, w.handle, out.ptr, m, mode,
+                                                   residual.ptr if residual is not None else None, out_dtype), "w8a16_gemm")
+
+    def rmsnorm_f16(self, x: DeviceBuffer, weight: DeviceBuffer, out: DeviceBuffer, rows: int, hidden: int, eps: float):
+        self._check(self.lib.nncase_hip_rmsnorm_f16(self.handle, x.ptr, weight.ptr, out.ptr, rows, hidden, eps), "rmsnorm_f16")
+
+    def rope_kv_append(self, qkv, q_out, k_cache, v_cache, block_table, ctx_lens, geometry: PagedAttnArgs, theta: float):
+        self._check(self.lib.nncase_hip_rope_kv_append(self.handle, qkv.ptr, q_out.ptr, k_cache.ptr, v_cache.ptr, block_table.ptr,
+                                                       ctx_lens.ptr, C.byref(geometry), theta), "rope_kv_append")
+
+    def argmax_f32(self, x: DeviceBuffer, out: DeviceBuffer, rows: int, cols: int):
+        self._check(self.lib.nncase_hip_argmax_f32(self.handle, x.ptr, out.ptr, rows, cols), "argmax_f32")
+
+    def embedding_f16(self, table: DeviceBuffer, ids: DeviceBuffer, out: DeviceBuffer, rows: int, hidden: int, vocab: int):
+        self._check(self.lib.nncase_hip_embedding_f16(self.handle, table.ptr, ids.ptr, out.ptr, rows, hidden, vocab), "embedding_f16")
+
+    def add_i32(self, x: DeviceBuffer, count: int, delta: int):
+        self._check(self.lib.nncase_hip_add_i32(self.handle, x.ptr, count, delta), "add_i32")
+
     def paged_attention_decode(self, q: DeviceBuffer, k_cache: DeviceBuffer, v_cache: DeviceBuffer,
                                block_table: DeviceBuffer, ctx_lens: DeviceBuffer, out: DeviceBuffer, args: PagedAttnArgs):
         self._check(self.lib.nncase_hip_paged_attention_decode(self.handle, q.ptr, k_cache.ptr, v_cache.ptr, block_table.ptr,
@@ -473,6 +514,42 @@ class Function:
         self._ck(self.ctx.lib.nncase_hip_function_add_pack(self.handle, src.ptr, dst.ptr, elem_size, len(shape), sh, len(axes), ax, ln),
                  "function_add_pack")
 
+    def add_w8a16_gemm(self, a, w, out, m, mode=GEMM_PLAIN, residual=None, out_dtype=DT_F16):
+        self._keep += [a, w, out] + ([residual] if residual is not None else [])
+        self._ck(self.ctx.lib.nncase_hip_function_add_w8a16_gemm(self.handle, a.ptr, w.handle, out.ptr, m, mode,
+                                                                 residual.ptr if residual is not None else None, out_dtype),
+                 "function_add_w8a16_gemm")
+
+    def add_rmsnorm_f16(self, x, weight, out, rows, hidden, eps):
+        self._keep += [x, weight, out]
+        self._ck(self.ctx.lib.nncase_hip_function_add_rmsnorm_f16(self.handle, x.ptr, weight.ptr, out.ptr, rows, hidden, eps),
+                 "function_add_rmsnorm_f16")
+
+    def add_rope_kv_append(self, qkv, q_out, k_cache, v_cache, block_table, ctx_lens, geometry, theta):
+        self._keep += [qkv, q_out, k_cache, v_cache, block_table, ctx_lens]
+        self._ck(self.ctx.lib.nncase_hip_function_add_rope_kv_append(self.handle, qkv.ptr, q_out.ptr, k_cache.ptr, v_cache.ptr,
+                                                                     block_table.ptr, ctx_lens.ptr, C.byref(geometry), theta),
+                 "function_add_rope_kv_append")
+
+    def add_paged_attention_decode(self, q, k_cache, v_cache, block_table, ctx_lens, out, args):
+        self._keep += [q, k_cache, v_cache, block_table, ctx_lens, out]
+        self._ck(self.ctx.lib.nncase_hip_function_add_paged_attention_decode(self.handle, q.ptr, k_cache.ptr, v_cache.ptr,
+                                                                             block_table.ptr, ctx_lens.ptr, out.ptr, C.byref(args)),
+                 "function_add_paged_attention_decode")
+
+    def add_argmax_f32(self, x, out, rows, cols):
+        self._keep += [x, out]
+        self._ck(self.ctx.lib.nncase_hip_function_add_argmax_f32(self.handle, x.ptr, out.ptr, rows, cols), "function_add_argmax_f32")
+
+    def add_embedding_f16(self, table, ids, out, rows, hidden, vocab):
+        self._keep += [table, ids, out]
+        self._ck(self.ctx.lib.nncase_hip_function_add_embedding_f16(self.handle, table.ptr, ids.ptr, out.ptr, rows, hidden, vocab),
+                 "function_add_embedding_f16")
+
+    def add_add_i32(self, x, count, delta):
+        self._keep += [x]
+        self._ck(self.ctx.lib.nncase_hip_function_add_add_i32(self.handle, x.ptr, count, delta), "function_add_add_i32")
+
     def add_resize_nearest(self, src, dst, elem_size, batch, in_h, in_w, channels, out_h, out_w, transformation_mode=0,
                            nearest_mode=0):
         self._keep += [src, dst]
@@ -510,6 +587,33 @@ class Function:
         if self.handle:
             if self.ctx.handle:  # a function of a closed context went with it
                 self.ctx.lib.nncase_hip_function_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass
+
+
+class W8A16:
+    """Pre-packed int8 weight matrix [n, k] with per-output-channel fp32 scales (nncase_hip_w8a16_t)."""
+
+    def __init__(self, ctx: Context, w_nk: np.ndarray, scale: np.ndarray, bias: Optional[np.ndarray] = None):
+        w = np.ascontiguousarray(w_nk, np.int8)
+        sc = np.ascontiguousarray(scale, np.float32)
+        b = None if bias is None else np.ascontiguousarray(bias, np.float32)
+        self.ctx, self.n, self.k = ctx, w.shape[0], w.shape[1]
+        assert sc.shape == (self.n,) and (b is None or b.shape == (self.n,))
+        h = C.c_void_p()
+        ctx._check(ctx.lib.nncase_hip_w8a16_prepack(ctx.handle, w.ctypes.data, sc.ctypes.data, None if b is None else b.ctypes.data,
+                                                    self.k, self.n, C.byref(h)), "w8a16_prepack")
+        self.handle = h.value
+
+    def destroy(self):
+        if self.handle:
+            if self.ctx.handle:
+                self.ctx.lib.nncase_hip_w8a16_destroy(self.ctx.handle, self.handle)
             self.handle = None
 
     def __del__(self):

@@ -48,4 +48,4 @@ def test_struct_layouts_match_the_header():
     assert C.sizeof(rt.Conv2dDesc) == 5 * 4 + 8 + 4 + 8  # 4 bytes of padding before the int64
     assert C.sizeof(rt.Conv2dArgs) == 11 * 4 + 8 + 8 + 3 * 4 + 8 + 8 + 8 + 2 * 4
     assert C.sizeof(rt.MatmulArgs) == 4 + 8 + 8 + 3 * 4
-    assert C.sizeof(rt.PagedAttnArgs) == 9 * 4
+    assert C.sizeof(rt.PagedAttnArgs) == 10 * 4

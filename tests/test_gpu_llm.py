@@ -1,0 +1,172 @@
+"""GPU parity of the decode-step operators and of a whole decode step against float64 restatements.
+The reference tree has no counterpart (parity unpinned by the reference); tolerance 1e-3 relative to the
+largest magnitude of each output row, as for attention."""
+import numpy as np
+import pytest
+
+from nncase_amd import llm
+from nncase_amd import runtime as rt
+from oracle import llm_ref as R
+
+pytestmark = pytest.mark.gpu
+RTOL = 1e-3
+
+
+def close(got, want, rtol=RTOL, atol=1e-3):
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    tol = rtol * np.abs(want).max(axis=-1, keepdims=True) + atol
+    assert (np.abs(got - want) <= tol).all(), f"max err {np.abs(got - want).max()} (max |want| {np.abs(want).max()})"
+
+
+@pytest.mark.parametrize("m,k,n", [(1, 64, 16), (32, 896, 1152), (7, 128, 48), (33, 192, 64), (64, 4864, 896), (16, 896, 2048)])
+@pytest.mark.parametrize("out32", [False, True])
+def test_w8a16_gemm(hip_ctx, m, k, n, out32):
+    rng = np.random.default_rng(m + k + n)
+    a = rng.standard_normal((m, k)).astype(np.float16)
+    q = rng.integers(-127, 128, (n, k), dtype=np.int8)
+    q[0, :] = -128 if k > 64 else q[0, :]                       # the full int8 range
+    scale = rng.uniform(0.001, 0.01, n).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    res = rng.standard_normal((m, n)).astype(np.float16)
+    w = hip_ctx.prepack_w8a16(q, scale, bias)
+    da, dres = hip_ctx.to_device(a), hip_ctx.to_device(res)
+    dt = np.float32 if out32 else np.float16
+    out = hip_ctx.alloc(m * n * np.dtype(dt).itemsize)
+    hip_ctx.w8a16_gemm(da, w, out, m, out_dtype=rt.DT_F32 if out32 else rt.DT_F16)
+    close(out.download((m, n), dt), R.w8a16_linear(a, q, scale, bias))
+    hip_ctx.w8a16_gemm(da, w, out, m, residual=dres, out_dtype=rt.DT_F32 if out32 else rt.DT_F16)
+    close(out.download((m, n), dt), R.w8a16_linear(a, q, scale, bias) + res.astype(np.float64))
+    # exact case: small integers survive fp16 and the fp32 accumulator exactly
+    ai = rng.integers(-4, 5, (m, k)).astype(np.float16)
+    w1 = hip_ctx.prepack_w8a16(q, np.ones(n, np.float32))
+    o32 = hip_ctx.alloc(m * n * 4)
+    hip_ctx.w8a16_gemm(hip_ctx.to_device(ai), w1, o32, m, out_dtype=rt.DT_F32)
+    assert np.array_equal(o32.download((m, n), np.float32), (ai.astype(np.int64) @ q.astype(np.int64).T).astype(np.float32))
+
+
+def test_w8a16_swiglu(hip_ctx):
+    rng = np.random.default_rng(3)
+    m, k, mlp = 32, 896, 4864
+    a = rng.standard_normal((m, k)).astype(np.float16)
+    q = rng.integers(-127, 128, (2 * mlp, k), dtype=np.int8)
+    scale = rng.uniform(0.0005, 0.002, 2 * mlp).astype(np.float32)
+    w = hip_ctx.prepack_w8a16(q, scale)
+    out = hip_ctx.alloc(m * mlp * 2)
+    hip_ctx.w8a16_gemm(hip_ctx.to_device(a), w, out, m, mode=rt.GEMM_SWIGLU)
+    gu = R.w8a16_linear(a, q, scale)
+    close(out.download((m, mlp), np.float16), R.silu(gu[:, :mlp]) * gu[:, mlp:])
+
+
+def test_w8a16_error_paths(hip_ctx):
+    q = np.zeros((16, 64), np.int8)
+    with pytest.raises(rt.HipError) as e:
+        hip_ctx.prepack_w8a16(np.zeros((16, 48), np.int8), np.ones(16, np.float32))       # k not a multiple of 64
+    assert e.value.code == -rt.ERR_SHAPE_MISMATCH
+    with pytest.raises(rt.HipError):
+        hip_ctx.prepack_w8a16(np.zeros((10, 64), np.int8), np.ones(10, np.float32))       # n not a multiple of 16
+    w = hip_ctx.prepack_w8a16(q, np.ones(16, np.float32))
+    buf = hip_ctx.alloc(65 * 64 * 2)
+    with pytest.raises(rt.HipError):
+        hip_ctx.w8a16_gemm(buf, w, buf, 65)                                                 # more than 64 token rows
+
+
+@pytest.mark.parametrize("rows,hidden", [(1, 64), (32, 896), (5, 1000), (64, 4864)])
+def test_rmsnorm(hip_ctx, rows, hidden):
+    rng = np.random.default_rng(rows + hidden)
+    x = (rng.standard_normal((rows, hidden)) * 3).astype(np.float16)
+    w = (1 + 0.1 * rng.standard_normal(hidden)).astype(np.float16)
+    out = hip_ctx.alloc(rows * hidden * 2)
+    hip_ctx.rmsnorm_f16(hip_ctx.to_device(x), hip_ctx.to_device(w), out, rows, hidden, 1e-6)
+    close(out.download((rows, hidden), np.float16), R.rmsnorm(x, w, 1e-6))
+
+
+def test_rope_and_kv_append(hip_ctx):
+    rng = np.random.default_rng(9)
+    B, hq, hkv, d, blk, max_blocks = 5, 14, 2, 64, 16, 8
+    nb = B * max_blocks + 2
+    lens = np.array([0, 1, 15, 16, 100], np.int32)
+    bt = rng.permutation(nb)[:B * max_blocks].reshape(B, max_blocks).astype(np.int32)
+    qkv = rng.standard_normal((B, (hq + 2 * hkv) * d)).astype(np.float16)
+    kc = rng.standard_normal((nb, hkv, blk, d)).astype(np.float16)
+    vc = rng.standard_normal((nb, hkv, d, blk)).astype(np.float16)
+    dk, dv = hip_ctx.to_device(kc), hip_ctx.to_device(vc)
+    dq = hip_ctx.alloc(B * hq * d * 2)
+    geo = rt.PagedAttnArgs(B, hq, hkv, d, blk, max_blocks, nb, 0.125, rt.DT_F16)
+    hip_ctx.rope_kv_append(hip_ctx.to_device(qkv), dq, dk, dv, hip_ctx.to_device(bt), hip_ctx.to_device(lens), geo, 1e6)
+    q = dq.download((B, hq, d), np.float16)
+    k2, v2 = dk.download(kc.shape, np.float16), dv.download(vc.shape, np.float16)
+    want_k, want_v = kc.copy(), vc.copy()
+    for b in range(B):
+        heads = qkv[b].reshape(hq + 2 * hkv, d)
+        close(q[b], R.rope(heads[:hq], int(lens[b]), 1e6), atol=2e-3)
+        pb, off = bt[b, lens[b] // blk], lens[b] % blk
+        close(k2[pb, :, off, :], R.rope(heads[hq:hq + hkv], int(lens[b]), 1e6), atol=2e-3)
+        assert np.array_equal(v2[pb, :, :, off], heads[hq + hkv:])        # v is copied, not rotated
+        want_k[pb, :, off, :] = k2[pb, :, off, :]
+        want_v[pb, :, :, off] = v2[pb, :, :, off]
+    assert np.array_equal(k2, want_k) and np.array_equal(v2, want_v)       # nothing else in the caches moved
+    assert np.array_equal(q[0], qkv[0].reshape(-1, d)[:hq])                # position 0: rotation by zero
+
+
+def test_argmax_embedding_and_counter(hip_ctx):
+    rng = np.random.default_rng(4)
+    x = rng.standard_normal((7, 151936)).astype(np.float32)
+    x[2, 777] = x[2, 5] = 50.0                                   # a tie: the lower index wins
+    x[3, :] = -np.inf
+    out = hip_ctx.alloc(7 * 4)
+    hip_ctx.argmax_f32(hip_ctx.to_device(x), out, 7, x.shape[1])
+    got = out.download((7,), np.int32)
+    want = x.argmax(axis=1)
+    assert np.array_equal(got, want) and got[2] == 5 and got[3] == 0
+    table = rng.standard_normal((1000, 96)).astype(np.float16)
+    ids = np.array([0, 999, 5, 5, 123], np.int32)
+    o = hip_ctx.alloc(5 * 96 * 2)
+    hip_ctx.embedding_f16(hip_ctx.to_device(table), hip_ctx.to_device(ids), o, 5, 96, 1000)
+    assert np.array_equal(o.download((5, 96), np.float16), table[ids])
+    c = hip_ctx.to_device(np.arange(10, dtype=np.int32))
+    hip_ctx.add_i32(c, 10, 3)
+    hip_ctx.add_i32(c, 10, -1)
+    assert np.array_equal(c.download((10,), np.int32), np.arange(10) + 2)
+
+
+def make_state(cfg, rng, batch, max_ctx):
+    max_blocks = -(-(max_ctx + 8) // cfg.block_size)
+    nb = batch * max_blocks + 1
+    lens = rng.integers(max_ctx // 2, max_ctx + 1, batch).astype(np.int32)
+    bt = rng.permutation(nb)[:batch * max_blocks].reshape(batch, max_blocks).astype(np.int32)
+    kcs = [rng.standard_normal((nb, cfg.kv_heads, cfg.block_size, cfg.head_dim)).astype(np.float16) for _ in range(cfg.layers)]
+    vcs = [rng.standard_normal((nb, cfg.kv_heads, cfg.head_dim, cfg.block_size)).astype(np.float16) for _ in range(cfg.layers)]
+    return max_blocks, lens, bt, kcs, vcs
+
+
+@pytest.mark.parametrize("capture", [False, True])
+def test_decode_steps_small_model(hip_ctx, capture):
+    """Three greedy steps of a 3-layer model (Qwen2 head geometry, reduced widths) against the float64 step:
+    logits to 1e-3, the same tokens whenever the float64 top-2 margin exceeds the tolerance, and the caches
+    the steps leave behind."""
+    cfg = llm.DecoderConfig(layers=3, hidden=256, q_heads=4, kv_heads=2, head_dim=64, mlp=512, vocab=2048)
+    rng = np.random.default_rng(12)
+    weights = llm.random_weights(cfg, seed=3)
+    batch = 6
+    max_blocks, lens, bt, kcs, vcs = make_state(cfg, rng, batch, 90)
+    dec = llm.HipDecoder(hip_ctx, cfg, weights, batch, max_blocks, bt, lens, kcs, vcs, capture_graph=capture)
+    ref_k, ref_v = [k.copy() for k in kcs], [v.copy() for v in vcs]
+    ref_lens = lens.copy()
+    tokens = rng.integers(0, cfg.vocab, batch).astype(np.int32)
+    for step in range(3):
+        dec.set_tokens(tokens)
+        dec.step()
+        hip_ctx.sync()
+        got = dec.result()
+        logits = dec.logits.download((batch, cfg.vocab), np.float32)
+        want_tok, want_logits = R.decode_step(cfg, weights, tokens, bt, ref_lens, ref_k, ref_v)
+        close(logits, want_logits, rtol=2e-3, atol=2e-3)
+        top2 = np.sort(want_logits, axis=1)[:, -2:]
+        sure = (top2[:, 1] - top2[:, 0]) > 4e-3 * np.abs(want_logits).max(axis=1)
+        assert sure.any() and np.array_equal(got[sure], want_tok[sure])
+        ref_lens += 1
+        assert np.array_equal(dec.ctx_lens.download((batch,), np.int32), ref_lens)
+        tokens = want_tok
+    for li in range(cfg.layers):   # the appended K / V rows
+        close(dec.layers[li]["k"].download(kcs[li].shape, np.float16).reshape(-1, cfg.head_dim), ref_k[li].reshape(-1, cfg.head_dim), atol=4e-3)
+        close(dec.layers[li]["v"].download(vcs[li].shape, np.float16).reshape(-1, cfg.block_size), ref_v[li].reshape(-1, cfg.block_size), atol=4e-3)
