@@ -261,6 +261,9 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--batch", type=int, default=64)
+    ap.add_argument("--lanes", type=int, default=1,
+                    help="independent chains the batch is split into and replayed concurrently (1 = one chain of "
+                         "full-batch launches); results are bit-identical for every value")
     ap.add_argument("--cpu-images", type=int, default=8, help="batch-1 images timed on the CPU baseline (0 = skip)")
     ap.add_argument("--profile-iters", type=int, default=10)
     ap.add_argument("--batch1-steps", type=int, default=200, help="timed batch-1 invocations (0 = skip the batch-1 figure)")
@@ -295,7 +298,7 @@ def main():
     qg = nb.quantize_graph(graph, calib)
     x = np.random.default_rng(4).random((args.batch, 224, 224, 3), dtype=np.float32)
 
-    model = nb.HipModel(ctx, qg, args.batch, capture_graph=not args.no_graph)
+    model = nb.HipModel(ctx, qg, args.batch, capture_graph=not args.no_graph, lanes=args.lanes)
     model.set_input(x)  # resident in HBM before the timed region
     for _ in range(args.warmup):
         model.invoke()
@@ -311,8 +314,10 @@ def main():
     # ---- per-kernel device time (HIP events on the context's stream) --------------------------
     op_ms = model.fn.profile(args.profile_iters)
     names = [model.fn.op_kernel(i) for i in range(len(model.fn))]
-    abytes = algorithmic_bytes(qg, args.batch, model.fused_into)
-    macs = conv_macs(qg, args.batch, model.fused_into)
+    # every lane launches the whole operator list on its batch/lanes images (and reads the weights itself)
+    lane_batch = args.batch // args.lanes
+    abytes = algorithmic_bytes(qg, lane_batch, model.fused_into) * args.lanes
+    macs = conv_macs(qg, lane_batch, model.fused_into) * args.lanes
     assert len(abytes) == len(macs) == len(names) == len(op_ms)
     groups = {}
     for name, ms, b, m in zip(names, op_ms, abytes, macs):
@@ -389,10 +394,13 @@ def main():
         "data": "synthetic",
         "config": {"workload": f"MobileNetV2 w1.0 224x224 u8/u8 per-tensor PTQ (32 calibration images), batch {args.batch}, "
                                "NHWC f32 input resident in HBM -> quantize -> 52 convs + 10 adds + pool + FC -> dequantize",
-                   "batch": args.batch, "ops_per_step": len(model.fn), "execution": "resident hip function, " + ("eager launches" if args.no_graph else "HIP-graph replay")},
+                   "batch": args.batch, "lanes": args.lanes, "ops_per_step": len(model.fn),
+                   "execution": "resident hip function, " + ("eager launches" if args.no_graph else "HIP-graph replay") +
+                                (f", {args.lanes} concurrent chains of {lane_batch} images" if args.lanes > 1 and not args.no_graph else "")},
         "roofline": {"bound": "hbm", "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(dom_gbs / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC_B64.get(dom_name) if args.batch == 64 else None, "kernel": dom_name,
+                     "traffic": MEASURED_TRAFFIC_B64.get(dom_name) if (args.batch, args.lanes) == (64, 1) else None, "kernel": dom_name,
+                     "images_per_launch": lane_batch,
                      "launches_per_step": dom["launches"], "avg_launch_us": round(dom["ms"] / dom["launches"] * 1e3, 2),
                      "algorithmic_bytes_per_launch": int(dom["bytes"] / dom["launches"]),
                      "share_of_device_time": round(dom["ms"] / sum(op_ms), 4)},

@@ -435,6 +435,13 @@ NNCASE_HIP_API int nncase_hip_function_add_argmax_f32(nncase_hip_function_t *fn,
 NNCASE_HIP_API int nncase_hip_function_add_embedding_f16(nncase_hip_function_t *fn, const void *table_dev, const int32_t *ids_dev,
                                                          void *out_dev, int32_t rows, int32_t hidden, int32_t vocab);
 NNCASE_HIP_API int nncase_hip_function_add_add_i32(nncase_hip_function_t *fn, int32_t *x_dev, int32_t count, int32_t delta);
+/* Operators recorded after this call belong to independent chain `lane` (default 0).  Operators of one
+ * lane run in the order recorded; different lanes must not touch each other's tensors.  A captured function
+ * runs its lanes concurrently (e.g. the two halves of a batch, whose small layers cannot fill the device
+ * alone); eager invocation runs all operators in the order recorded.  Paged attention and other operators
+ * that use the context's scratch memory must stay in one lane. */
+#define NNCASE_HIP_MAX_LANES 8
+NNCASE_HIP_API int nncase_hip_function_set_lane(nncase_hip_function_t *fn, int32_t lane);
 /* Number of operators recorded so far. */
 NNCASE_HIP_API int nncase_hip_function_size(nncase_hip_function_t *fn, int32_t *count);
 /* Enqueues the whole function (graph replay if captured). */

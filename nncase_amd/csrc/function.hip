@@ -36,6 +36,7 @@ struct Op {
     nncase_hip_paged_attn_args_t attn{};
     int32_t mode = 0, delta = 0;
     float eps = 0.f;
+    int lane = 0; // independent operator chain this operator belongs to
 };
 
 } // namespace
@@ -43,6 +44,7 @@ struct Op {
 struct nncase_hip_function {
     nncase_hip_ctx *ctx = nullptr;
     std::vector<Op> ops;
+    int cur_lane = 0, nlanes = 1;
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
 };
@@ -108,6 +110,16 @@ static void drop_graph(nncase_hip_function *fn) {
 static int push(nncase_hip_function *fn, const Op &op) {
     drop_graph(fn); // a captured graph no longer matches the list
     fn->ops.push_back(op);
+    fn->ops.back().lane = fn->cur_lane;
+    return 0;
+}
+
+extern "C" int nncase_hip_function_set_lane(nncase_hip_function_t *fn, int32_t lane) {
+    if (!fn) return -EINVAL;
+    NNHIP_REQUIRE(fn->ctx, lane >= 0 && lane < NNCASE_HIP_MAX_LANES, -EINVAL, "function_set_lane: lane %d (0..%d)", lane,
+                  NNCASE_HIP_MAX_LANES - 1);
+    fn->cur_lane = lane;
+    if (lane + 1 > fn->nlanes) fn->nlanes = lane + 1;
     return 0;
 }
 
@@ -363,14 +375,63 @@ extern "C" int nncase_hip_function_capture(nncase_hip_function_t *fn) {
     nncase_hip_ctx *ctx = fn->ctx;
     drop_graph(fn);
     NNHIP_HIP(ctx, hipStreamSynchronize(ctx->stream));
-    NNHIP_HIP(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
-    int rc = 0;
+    // Paged attention keeps its split partials and counters in one per-context scratch area: two lanes that
+    // both run it would overlap on that area, so all attention operators must sit on one lane.
+    int attn_lane = -1;
     for (const Op &op : fn->ops) {
-        rc = run_op(fn, op);
-        if (rc) break;
+        if (op.kind != Op::kAttn) continue;
+        NNHIP_REQUIRE(ctx, attn_lane < 0 || attn_lane == op.lane, -EINVAL,
+                      "function_capture: paged attention on lanes %d and %d (its scratch area is per context)", attn_lane, op.lane);
+        attn_lane = op.lane;
+    }
+    // Operators of different lanes are recorded on streams of their own, forked from and joined back into
+    // the context's stream, so the graph holds one independent chain per lane and the device overlaps them.
+    hipStream_t main_stream = ctx->stream;
+    hipStream_t side[NNCASE_HIP_MAX_LANES] = {nullptr};
+    hipEvent_t fork = nullptr, join[NNCASE_HIP_MAX_LANES] = {nullptr};
+    int rc = 0;
+    hipError_t se = hipSuccess;
+    for (int l = 1; l < fn->nlanes && se == hipSuccess; l++) {
+        se = hipStreamCreateWithFlags(&side[l], hipStreamNonBlocking);
+        if (se == hipSuccess) se = hipEventCreateWithFlags(&join[l], hipEventDisableTiming);
+    }
+    if (se == hipSuccess && fn->nlanes > 1) se = hipEventCreateWithFlags(&fork, hipEventDisableTiming);
+    auto release = [&]() {
+        for (int l = 1; l < NNCASE_HIP_MAX_LANES; l++) {
+            if (join[l]) (void)hipEventDestroy(join[l]);
+            if (side[l]) (void)hipStreamDestroy(side[l]);
+        }
+        if (fork) (void)hipEventDestroy(fork);
+    };
+    if (se != hipSuccess) {
+        release();
+        return hip_fail(ctx, se, "function_capture: lane streams");
+    }
+    se = hipStreamBeginCapture(main_stream, hipStreamCaptureModeThreadLocal);
+    if (se != hipSuccess) {
+        release();
+        return hip_fail(ctx, se, "hipStreamBeginCapture");
+    }
+    if (fn->nlanes > 1) {
+        se = hipEventRecord(fork, main_stream);
+        for (int l = 1; l < fn->nlanes && se == hipSuccess; l++) se = hipStreamWaitEvent(side[l], fork, 0);
+    }
+    if (se == hipSuccess) {
+        for (const Op &op : fn->ops) {
+            ctx->stream = op.lane == 0 ? main_stream : side[op.lane];
+            rc = run_op(fn, op);
+            if (rc) break;
+        }
+        ctx->stream = main_stream;
+        for (int l = 1; l < fn->nlanes && se == hipSuccess; l++) {
+            se = hipEventRecord(join[l], side[l]);
+            if (se == hipSuccess) se = hipStreamWaitEvent(main_stream, join[l], 0);
+        }
     }
     hipGraph_t graph = nullptr;
-    const hipError_t e = hipStreamEndCapture(ctx->stream, &graph);
+    const hipError_t e = hipStreamEndCapture(main_stream, &graph);
+    release();
+    if (se != hipSuccess && !rc) rc = hip_fail(ctx, se, "function_capture: fork / join");
     if (rc) {
         if (graph) (void)hipGraphDestroy(graph);
         return rc;

@@ -343,13 +343,23 @@ def pad_small_channel_convs(qg: QuantGraph) -> QuantGraph:
 # --------------------------------------------------------------------------------------------- device binding
 class HipModel:
     """A QuantGraph resident on the device: packed weights, one HBM buffer per tensor, and the
-    operator list recorded in a `hip` function.  run() = upload input, invoke, download output."""
+    operator list recorded in a `hip` function.  run() = upload input, invoke, download output.
 
-    def __init__(self, ctx: Context, qg: QuantGraph, batch: int, capture_graph: bool = True, fuse_residual: bool = True):
-        self.ctx, self.qg, self.batch = ctx, qg, batch
+    lanes > 1 splits the batch into that many equal image ranges and records the whole operator list once per
+    range, each on its own lane of the function: a captured function then replays the lanes on concurrent
+    streams, so one lane's launch gaps and tail waves are filled by the other's kernels.  Every tensor keeps
+    its full-batch NHWC buffer (a lane works on its image range of it) and the lanes share the packed weights,
+    so results are bit-identical to lanes == 1."""
+
+    def __init__(self, ctx: Context, qg: QuantGraph, batch: int, capture_graph: bool = True, fuse_residual: bool = True,
+                 lanes: int = 1):
+        if lanes < 1 or lanes > rt.MAX_LANES or batch % lanes:
+            raise ValueError(f"lanes={lanes} must be in 1..{rt.MAX_LANES} and divide the batch ({batch})")
+        self.ctx, self.qg, self.batch, self.lanes = ctx, qg, batch, lanes
+        bl = batch // lanes                      # images per lane
         h, w, c = qg.input_shape
         self.in_count = batch * h * w * c
-        self.input_f32 = ctx.alloc(self.in_count * 4)
+        self.input_f32 = ctx.alloc(lanes * self._lane_stride(self.in_count // lanes * 4))
         self.fn = Function(ctx)
         self.buffers: List[Optional[rt.DeviceBuffer]] = []
         self.weights: List[Optional[rt.Weights]] = []
@@ -388,76 +398,26 @@ class HipModel:
             if conv in self.fused_lut:
                 self.never_written.add(self.fused_lut[conv])
         skip_nodes = set(self.fused_into.values()) | set(self.fused_lut.values())
+        # buffers and packed weights once, shared by the lanes
         for i, n in enumerate(qg.nodes):
             cc, hh, ww = n.out_shape
-            fused_add = self.fused_into.get(i)
-            fused_lut = self.fused_lut.get(i)
+            self.weights.append(None)
             if i in skip_nodes:
                 self.buffers.append(self.buffers[i - 1])  # written by the conv it is fused into
-                self.weights.append(None)
                 continue
-            buf = ctx.alloc(batch * cc * hh * ww)
-            self.buffers.append(buf)
-            self.weights.append(None)
-            if n.op == "input":
-                self.fn.add_quantize(self.input_f32, rt.DT_F32, buf, rt.DT_U8, self.in_count, qp(*n.out_qp))
-            elif n.op == "conv":
-                src = qg.nodes[n.inputs[0]]
-                wt = ctx.prepack_conv2d(n.weights, n.bias, qp(*n.w_qp), n.groups, expected_pixels=batch * hh * ww)
-                self.weights[-1] = wt
-                (ph0, ph1), (pw0, pw1) = n.padding
-                args = rt.Conv2dArgs(batch, src.out_shape[1], src.out_shape[2], n.stride[0], n.stride[1], 1, 1, ph0, ph1, pw0,
-                                     pw1, qp(*src.out_qp), qp(*n.out_qp), n.clamp[0], n.clamp[1], rt.DT_U8)
+            self.buffers.append(ctx.alloc(lanes * self._lane_stride(bl * cc * hh * ww)))
+            if n.op == "conv":
+                wt = ctx.prepack_conv2d(n.weights, n.bias, qp(*n.w_qp), n.groups, expected_pixels=bl * hh * ww)
+                fused_lut = self.fused_lut.get(i)
                 if fused_lut is not None:
                     wt.set_post_lut(qg.nodes[fused_lut].lut, qp(*qg.nodes[fused_lut].out_qp))
-                if fused_add is not None:
-                    add = qg.nodes[fused_add]
-                    res_node = add.inputs[0]
-                    args.residual_dev = self.buffers[res_node].ptr
-                    args.residual_qp = qp(*qg.nodes[res_node].out_qp)
-                    args.sum_qp = qp(*add.out_qp)
-                    args.sum_clamp_min, args.sum_clamp_max = FULL_CLAMP
-                    self.fn._keep.append(self.buffers[res_node])
-                self.fn.add_qconv2d(self.buffers[n.inputs[0]], wt, buf, args)
-            elif n.op == "add":
-                a, b = (qg.nodes[j] for j in n.inputs)
-                self.fn.add_qadd(self.buffers[n.inputs[0]], qp(*a.out_qp), self.buffers[n.inputs[1]], qp(*b.out_qp), buf,
-                                 qp(*n.out_qp), batch * cc * hh * ww)
-            elif n.op == "lut":
-                self.fn.add_lut_u8(self.buffers[n.inputs[0]], buf, batch * cc * hh * ww, n.lut)
-            elif n.op == "concat":
-                srcs = [qg.nodes[j] for j in n.inputs]
-                self.fn.add_qconcat_channels([self.buffers[j] for j in n.inputs], [s_.out_shape[0] for s_ in srcs],
-                                             [qp(*s_.out_qp) for s_ in srcs], buf, qp(*n.out_qp), batch * hh * ww)
-            elif n.op == "resize":
-                src = qg.nodes[n.inputs[0]]
-                self.fn.add_resize_nearest(self.buffers[n.inputs[0]], buf, 1, batch, src.out_shape[1], src.out_shape[2], cc, hh, ww,
-                                           n.resize_modes[0], n.resize_modes[1])
-            elif n.op == "maxpool":
-                src = qg.nodes[n.inputs[0]]
-                k, st, p = n.pool
-                self.fn.add_qmaxpool2d(self.buffers[n.inputs[0]], buf, batch, src.out_shape[1], src.out_shape[2], cc, (k, k), (st, st),
-                                       ((p, p), (p, p)), qp(*src.out_qp), qp(*n.out_qp))
-            elif n.op == "padc":
-                src = qg.nodes[n.inputs[0]]
-                self.fn.add_pack(self.buffers[n.inputs[0]], buf, 1, [batch, hh, ww, src.out_shape[0]], [3], [cc])
-            elif n.op == "gap":
-                src = qg.nodes[n.inputs[0]]
-                self.fn.add_qglobal_avgpool(self.buffers[n.inputs[0]], buf, batch, src.out_shape[1], src.out_shape[2],
-                                            src.out_shape[0], qp(*src.out_qp), qp(*n.out_qp))
-            else:
-                raise ValueError(n.op)
-            self.op_names.append(f"{n.op}:{n.name}" + ("+lut" if fused_lut is not None else "") + ("+add" if fused_add is not None else ""))
-            self.op_nodes.append(fused_add if fused_add is not None else (fused_lut if fused_lut is not None else i))
-        self.outputs_f32: List[rt.DeviceBuffer] = []
-        for j in qg.output_nodes:
-            node = qg.nodes[j]
-            count = batch * int(np.prod(node.out_shape))
-            out = ctx.alloc(count * 4)
-            self.fn.add_dequantize(self.buffers[j], rt.DT_U8, out, rt.DT_F32, count, qp(*node.out_qp))
-            self.outputs_f32.append(out)
-            self.op_names.append("dequantize:" + node.name)
-            self.op_nodes.append(j)
+                self.weights[-1] = wt
+        self.outputs_f32: List[rt.DeviceBuffer] = [ctx.alloc(lanes * self._lane_stride(bl * int(np.prod(qg.nodes[j].out_shape)) * 4))
+                                                    for j in qg.output_nodes]
+        for lane in range(lanes):
+            self.fn.set_lane(lane)
+            self._record_lane(lane, bl, skip_nodes)
+        self.fn.set_lane(0)
         self.output_f32 = self.outputs_f32[0]
         last = qg.nodes[qg.output_nodes[0]]
         self.out_shape = (batch,) + tuple(last.out_shape)
@@ -465,10 +425,102 @@ class HipModel:
         if capture_graph:
             self.fn.capture()
 
+    def _record_lane(self, lane: int, bl: int, skip_nodes):
+        """Record the operator list for images [lane*bl, (lane+1)*bl) on the function's current lane."""
+        qg = self.qg
+
+        def B(j):                                  # this lane's image range of node j's u8 tensor
+            per = bl * int(np.prod(qg.nodes[j].out_shape))
+            return self.buffers[j].view(lane * self._lane_stride(per), per)
+
+        h, w, c = qg.input_shape
+        in_per = bl * h * w * c
+        for i, n in enumerate(qg.nodes):
+            if i in skip_nodes:
+                continue
+            cc, hh, ww = n.out_shape
+            fused_add = self.fused_into.get(i)
+            fused_lut = self.fused_lut.get(i)
+            buf = B(i)
+            if n.op == "input":
+                self.fn.add_quantize(self.input_f32.view(lane * self._lane_stride(in_per * 4), in_per * 4), rt.DT_F32, buf, rt.DT_U8, in_per, qp(*n.out_qp))
+            elif n.op == "conv":
+                src = qg.nodes[n.inputs[0]]
+                (ph0, ph1), (pw0, pw1) = n.padding
+                args = rt.Conv2dArgs(bl, src.out_shape[1], src.out_shape[2], n.stride[0], n.stride[1], 1, 1, ph0, ph1, pw0,
+                                     pw1, qp(*src.out_qp), qp(*n.out_qp), n.clamp[0], n.clamp[1], rt.DT_U8)
+                if fused_add is not None:
+                    add = qg.nodes[fused_add]
+                    res_node = add.inputs[0]
+                    res = B(res_node)
+                    args.residual_dev = res.ptr
+                    args.residual_qp = qp(*qg.nodes[res_node].out_qp)
+                    args.sum_qp = qp(*add.out_qp)
+                    args.sum_clamp_min, args.sum_clamp_max = FULL_CLAMP
+                    self.fn._keep.append(res)
+                self.fn.add_qconv2d(B(n.inputs[0]), self.weights[i], buf, args)
+            elif n.op == "add":
+                a, b = (qg.nodes[j] for j in n.inputs)
+                self.fn.add_qadd(B(n.inputs[0]), qp(*a.out_qp), B(n.inputs[1]), qp(*b.out_qp), buf,
+                                 qp(*n.out_qp), bl * cc * hh * ww)
+            elif n.op == "lut":
+                self.fn.add_lut_u8(B(n.inputs[0]), buf, bl * cc * hh * ww, n.lut)
+            elif n.op == "concat":
+                srcs = [qg.nodes[j] for j in n.inputs]
+                self.fn.add_qconcat_channels([B(j) for j in n.inputs], [s_.out_shape[0] for s_ in srcs],
+                                             [qp(*s_.out_qp) for s_ in srcs], buf, qp(*n.out_qp), bl * hh * ww)
+            elif n.op == "resize":
+                src = qg.nodes[n.inputs[0]]
+                self.fn.add_resize_nearest(B(n.inputs[0]), buf, 1, bl, src.out_shape[1], src.out_shape[2], cc, hh, ww,
+                                           n.resize_modes[0], n.resize_modes[1])
+            elif n.op == "maxpool":
+                src = qg.nodes[n.inputs[0]]
+                k, st, p = n.pool
+                self.fn.add_qmaxpool2d(B(n.inputs[0]), buf, bl, src.out_shape[1], src.out_shape[2], cc, (k, k), (st, st),
+                                       ((p, p), (p, p)), qp(*src.out_qp), qp(*n.out_qp))
+            elif n.op == "padc":
+                src = qg.nodes[n.inputs[0]]
+                self.fn.add_pack(B(n.inputs[0]), buf, 1, [bl, hh, ww, src.out_shape[0]], [3], [cc])
+            elif n.op == "gap":
+                src = qg.nodes[n.inputs[0]]
+                self.fn.add_qglobal_avgpool(B(n.inputs[0]), buf, bl, src.out_shape[1], src.out_shape[2],
+                                            src.out_shape[0], qp(*src.out_qp), qp(*n.out_qp))
+            else:
+                raise ValueError(n.op)
+            if lane == 0:
+                self.op_names.append(f"{n.op}:{n.name}" + ("+lut" if fused_lut is not None else "") + ("+add" if fused_add is not None else ""))
+                self.op_nodes.append(fused_add if fused_add is not None else (fused_lut if fused_lut is not None else i))
+        for k, j in enumerate(qg.output_nodes):
+            node = qg.nodes[j]
+            count = bl * int(np.prod(node.out_shape))
+            self.fn.add_dequantize(B(j), rt.DT_U8, self.outputs_f32[k].view(lane * self._lane_stride(count * 4), count * 4), rt.DT_F32, count, qp(*node.out_qp))
+            if lane == 0:
+                self.op_names.append("dequantize:" + node.name)
+                self.op_nodes.append(j)
+
     def set_input(self, x_nhwc: np.ndarray):
         x = np.ascontiguousarray(x_nhwc, f32)
         assert x.size == self.in_count, f"expected {self.in_count} input elements, got {x.size}"
-        self.input_f32.upload(x)
+        per = self.in_count // self.lanes * 4
+        if self._lane_stride(per) == per:
+            self.input_f32.upload(x)
+        else:
+            for lane, part in enumerate(np.split(x.reshape(-1), self.lanes)):
+                self.input_f32.view(lane * self._lane_stride(per), per).upload(part)
+
+    def _lane_stride(self, nbytes: int) -> int:
+        """Byte distance between the lanes' image ranges of a tensor: the range itself when there is one lane
+        or its size keeps every lane 256-byte aligned (the tensor is then one contiguous NHWC array), else the
+        size rounded up (the kernels want 16-byte aligned operands)."""
+        return nbytes if self.lanes == 1 or nbytes % 256 == 0 else (nbytes + 255) // 256 * 256
+
+    def _download(self, buf, shape, dtype) -> np.ndarray:
+        per_shape = (shape[0] // self.lanes,) + tuple(shape[1:])
+        per = int(np.prod(per_shape)) * np.dtype(dtype).itemsize
+        stride = self._lane_stride(per)
+        if stride == per:
+            return buf.download(shape, dtype)
+        return np.concatenate([buf.view(lane * stride, per).download(per_shape, dtype) for lane in range(self.lanes)])
 
     def invoke(self):
         self.fn.invoke()
@@ -476,7 +528,7 @@ class HipModel:
     def output(self, index: int = 0) -> np.ndarray:
         """Dequantised float32 output `index`, NCHW-shaped [batch, C, H, W] (H = W = 1 for classifiers)."""
         c, h, w = self.qg.nodes[self.qg.output_nodes[index]].out_shape
-        y = self.outputs_f32[index].download((self.batch, h, w, c), f32)
+        y = self._download(self.outputs_f32[index], (self.batch, h, w, c), f32)
         return np.ascontiguousarray(y.transpose(0, 3, 1, 2))
 
     def all_outputs(self) -> List[np.ndarray]:
@@ -491,7 +543,7 @@ class HipModel:
         if not self.materialized(node):
             raise ValueError(f"node {node} only exists inside a fused operator and is never written")
         c, h, w = self.qg.nodes[node].out_shape
-        y = self.buffers[node].download((self.batch, h, w, c), np.uint8)
+        y = self._download(self.buffers[node], (self.batch, h, w, c), np.uint8)
         return np.ascontiguousarray(y.transpose(0, 3, 1, 2))
 
     def run(self, x_nhwc: np.ndarray) -> np.ndarray:

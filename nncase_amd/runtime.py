@@ -119,6 +119,7 @@ SYMBOLS = {
     "nncase_hip_function_add_argmax_f32": (_I, [_VP, _VP, _VP, C.c_int32, C.c_int32]),
     "nncase_hip_function_add_embedding_f16": (_I, [_VP, _VP, _VP, _VP, C.c_int32, C.c_int32, C.c_int32]),
     "nncase_hip_function_add_add_i32": (_I, [_VP, _VP, C.c_int32, C.c_int32]),
+    "nncase_hip_function_set_lane": (_I, [_VP, C.c_int32]),
     "nncase_hip_kmodel_load": (_I, [_VP, _VP, _SZ, C.POINTER(_VP)]),
     "nncase_hip_kmodel_destroy": (_I, [_VP]),
     "nncase_hip_kmodel_function": (_I, [_VP, C.POINTER(_VP)]),
@@ -178,6 +179,7 @@ def qp(zero_point: int, scale: float) -> QuantParam:
 
 
 GEMM_PLAIN, GEMM_SWIGLU = 0, 1
+MAX_LANES = 8  # NNCASE_HIP_MAX_LANES
 LUT_REQUANT, LUT_SWISH = 0, 1
 RESIZE_HALF_PIXEL, RESIZE_PYTORCH_HALF_PIXEL, RESIZE_ALIGN_CORNERS, RESIZE_ASYMMETRIC, RESIZE_TFCROP_AND_RESIZE = range(5)
 NEAREST_ROUND_PREFER_FLOOR, NEAREST_ROUND_PREFER_CEIL, NEAREST_FLOOR, NEAREST_CEIL = range(4)
@@ -231,11 +233,29 @@ class DeviceBuffer:
                 self.ctx.lib.nncase_hip_free(self.ctx.handle, self.ptr)
             self.ptr = None
 
+    def view(self, offset: int, nbytes: int) -> "DeviceView":
+        return DeviceView(self, offset, nbytes)
+
     def __del__(self):
         try:
             self.free()
         except Exception:
             pass
+
+
+class DeviceView:
+    """A byte range of a DeviceBuffer (keeps the allocation alive; owns nothing)."""
+
+    def __init__(self, base: DeviceBuffer, offset: int, nbytes: int):
+        assert 0 <= offset and offset + nbytes <= base.nbytes
+        self.base, self.ctx, self.nbytes = base, base.ctx, int(nbytes)
+        self.ptr = base.ptr + int(offset)
+
+    def view(self, offset: int, nbytes: int) -> "DeviceView":
+        assert 0 <= offset and offset + nbytes <= self.nbytes
+        return DeviceView(self.base, self.ptr - self.base.ptr + offset, nbytes)
+
+    upload, download, fill = DeviceBuffer.upload, DeviceBuffer.download, DeviceBuffer.fill
 
 
 class Weights:
@@ -556,6 +576,10 @@ class Function:
         self._ck(self.ctx.lib.nncase_hip_function_add_resize_nearest(self.handle, src.ptr, dst.ptr, elem_size, batch, in_h,
                                                                      in_w, channels, out_h, out_w, transformation_mode,
                                                                      nearest_mode), "function_add_resize_nearest")
+
+    def set_lane(self, lane: int):
+        """Operators added from now on form independent chain `lane`; a captured function overlaps its lanes."""
+        self._ck(self.ctx.lib.nncase_hip_function_set_lane(self.handle, lane), "function_set_lane")
 
     def __len__(self):
         n = C.c_int32()

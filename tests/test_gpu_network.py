@@ -174,3 +174,58 @@ def test_profile_and_kernel_names(hip_ctx):
     assert all(n.startswith("qconv_igemm<T=") and n.endswith(",rows16>") for n in (names[1], names[3]))
     ms = model.fn.profile(3)
     assert len(ms) == 5 and all(0 < t < 50 for t in ms)
+
+
+@pytest.mark.parametrize("lanes,capture", [(2, True), (4, True), (2, False)])
+def test_lanes_split_the_batch_bit_exact(hip_ctx, lanes, capture):
+    """A function recorded as `lanes` independent chains over image ranges (replayed on concurrent streams
+    when captured) writes the same bytes into every tensor as the single-chain function, replay after replay."""
+    g = nb.mobilenet_v2(seed=2)
+    rng = np.random.default_rng(3)
+    qg = nb.quantize_graph(g, rng.random((32, 224, 224, 3), dtype=f32))
+    x = np.random.default_rng(4).random((16, 224, 224, 3), dtype=f32)
+    one = nb.HipModel(hip_ctx, qg, 16, capture_graph=False)
+    y1 = one.run(x)
+    many = nb.HipModel(hip_ctx, qg, 16, capture_graph=capture, lanes=lanes)
+    assert len(many.fn) == lanes * len(one.fn) and len(many.op_names) == len(one.op_names)
+    y = many.run(x)
+    assert np.array_equal(y.view(np.uint32), y1.view(np.uint32))
+    for i in range(len(qg.nodes)):
+        if one.materialized(i):
+            a, b = one.tensor(i), many.tensor(i)
+            assert np.array_equal(a, b), f"node {i} ({qg.nodes[i].name}): {(a != b).sum()} bytes differ"
+    x2 = np.random.default_rng(5).random((16, 224, 224, 3), dtype=f32)
+    y2 = one.run(x2)
+    for r in range(3):                      # replays with eager work and other inputs in between
+        assert np.array_equal(many.run(x2).view(np.uint32), y2.view(np.uint32)), f"replay {r}"
+        one.fn.invoke_one(1)
+        hip_ctx.sync()
+        assert np.array_equal(many.run(x).view(np.uint32), y1.view(np.uint32)), f"replay {r}"
+
+
+def test_lanes_yolov5s_outputs(hip_ctx):
+    g = nb.yolov5s(seed=5, input_hw=160)
+    rng = np.random.default_rng(6)
+    qg = nb.quantize_graph(g, rng.random((8, 160, 160, 3), dtype=f32))
+    x = rng.random((4, 160, 160, 3), dtype=f32)
+    one = nb.HipModel(hip_ctx, qg, 4, capture_graph=False)
+    one.run(x)
+    two = nb.HipModel(hip_ctx, qg, 4, capture_graph=True, lanes=2)
+    two.run(x)
+    for a, b in zip(one.all_outputs(), two.all_outputs()):
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
+def test_lanes_argument_checks(hip_ctx):
+    g = nb.conv_block(seed=1)
+    qg = nb.quantize_graph(g, np.random.default_rng(1).random((4, 56, 56, 64), dtype=f32))
+    with pytest.raises(ValueError):
+        nb.HipModel(hip_ctx, qg, 3, lanes=2)
+    with pytest.raises(ValueError):
+        nb.HipModel(hip_ctx, qg, 18, lanes=9)
+    from nncase_amd.runtime import Function, HipError
+    fn = Function(hip_ctx)
+    with pytest.raises(HipError):
+        fn.set_lane(8)
+    with pytest.raises(HipError):
+        fn.set_lane(-1)
