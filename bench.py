@@ -55,47 +55,35 @@ MEASURED_TRAFFIC_B64 = {
 }
 
 
-def algorithmic_bytes(qg, batch, fused_into):
-    """Per operator of the recorded function: bytes an ideal implementation must move
-    (read every input once, write every output once, read the constants once).
-    fused_into maps a conv node to the residual add folded into its epilogue: that add is
-    no operator of its own, and its conv reads the residual tensor as well."""
-    out = []
-    fused_adds = set(fused_into.values())
-    for i, n in enumerate(qg.nodes):
-        if i in fused_adds:
+def op_accounting(qg, batch, model):
+    """Per operator of the recorded function (one lane): the bytes an ideal implementation must move
+    (read every tensor that enters the operator once, write its result once, read the constants once)
+    and its multiply-adds.  An operator may cover several graph nodes (a conv with a table and a residual
+    add in its epilogue; a whole expand -> depthwise -> project block): tensors between those nodes never
+    reach HBM and do not count."""
+    size = lambda j: batch * int(np.prod(qg.nodes[j].out_shape))
+    nbytes, macs = [], []
+    for name, members in zip(model.op_names, model.op_members):
+        if name.startswith("dequantize"):
+            o = size(model.op_nodes[len(nbytes)])
+            nbytes.append(o + 4 * o)
+            macs.append(0)
             continue
-        c, h, w = n.out_shape
-        o = batch * c * h * w
-        if n.op == "input":
-            out.append(o * 4 + o)
-        elif n.op == "conv":
-            sc, sh, sw = qg.nodes[n.inputs[0]].out_shape
-            out.append(batch * sc * sh * sw + o + n.weights.size + 4 * n.bias.size + (o if i in fused_into else 0))
-        elif n.op == "add":
-            out.append(3 * o)
-        elif n.op == "gap":
-            sc, sh, sw = qg.nodes[n.inputs[0]].out_shape
-            out.append(batch * sc * sh * sw + o)
-    last = qg.nodes[-1]
-    o = batch * int(np.prod(last.out_shape))
-    out.append(o + 4 * o)  # final dequantize
-    return out
-
-
-def conv_macs(qg, batch, fused_into):
-    out = []
-    fused_adds = set(fused_into.values())
-    for i, n in enumerate(qg.nodes):
-        if i in fused_adds:
-            continue
-        if n.op == "conv":
-            oc, gic, kh, kw = n.weights.shape
-            out.append(batch * oc * n.out_shape[1] * n.out_shape[2] * gic * kh * kw)
-        else:
-            out.append(0)
-    out.append(0)
-    return out
+        inside = set(members)
+        external = {j for m in members for j in qg.nodes[m].inputs if j not in inside}
+        b = sum(size(j) for j in external) + size(members[-1])
+        m = 0
+        for j in members:
+            n = qg.nodes[j]
+            if n.op == "input":
+                b += 4 * size(j)
+            elif n.op == "conv":
+                oc, gic, kh, kw = n.weights.shape
+                b += n.weights.size + 4 * n.bias.size
+                m += batch * oc * n.out_shape[1] * n.out_shape[2] * gic * kh * kw
+        nbytes.append(b)
+        macs.append(m)
+    return nbytes, macs
 
 
 def time_calls(ctx, fn, warmup, steps):
@@ -147,7 +135,7 @@ def side_workload(args):
         model.set_input(rng.random((batch, 56, 56, 64), dtype=np.float32))
         ms = time_calls(ctx, model.invoke, args.warmup, args.steps)
         op_ms = model.fn.profile(10)
-        nbytes = sum(algorithmic_bytes(qg, batch, model.fused_into))
+        nbytes = sum(op_accounting(qg, batch, model)[0])
         line = dict(base, metric="images/sec u8/u8 conv block b32", value=round(batch / (ms * 1e-3), 1), unit="images/s",
                     ms_per_step=round(ms, 5), dtype="u8",
                     config={"workload": "config 2: f32 in -> quantize -> 1x1 64->144, dw 3x3, 1x1 144->64 (ReLU6) on 56x56 -> dequantize, batch 32"},
@@ -316,8 +304,7 @@ def main():
     names = [model.fn.op_kernel(i) for i in range(len(model.fn))]
     # every lane launches the whole operator list on its batch/lanes images (and reads the weights itself)
     lane_batch = args.batch // args.lanes
-    abytes = algorithmic_bytes(qg, lane_batch, model.fused_into) * args.lanes
-    macs = conv_macs(qg, lane_batch, model.fused_into) * args.lanes
+    abytes, macs = (v * args.lanes for v in op_accounting(qg, lane_batch, model))
     assert len(abytes) == len(macs) == len(names) == len(op_ms)
     groups = {}
     for name, ms, b, m in zip(names, op_ms, abytes, macs):
@@ -330,6 +317,8 @@ def main():
     dom_gbs = dom["bytes"] / (dom["ms"] * 1e-3) / 1e9
 
     def klass(name):
+        if name.startswith("qblock"):
+            return "fused_block"
         return "dense" if name.startswith("qconv_") else ("depthwise" if name.startswith("dw") else "elementwise")
 
     classes = {}

@@ -182,6 +182,60 @@ typedef struct nncase_hip_conv2d_args {
 NNCASE_HIP_API int nncase_hip_qconv2d(nncase_hip_ctx_t *ctx, const uint8_t *x_dev, const nncase_hip_weights_t *weights,
                                       void *y_dev, const nncase_hip_conv2d_args_t *args);
 
+/* ---- fused inverted-residual block ------------------------------------------
+ * 1x1 convolution (in -> mid channels), 3x3 depthwise convolution on the mid
+ * channels (stride 1 or 2), 1x1 convolution (mid -> out channels), optionally
+ * + the block's input: what the reference keeps as one Fusion function
+ * (src/Nncase.Core/IR/Fusion.cs:13) of three Conv2D calls
+ * (src/Native/src/kernels/stackvm/reference/convolution.cpp:26-143) and a
+ * Binary add.  One kernel computes all of it per output tile: the two mid
+ * tensors (the largest of the block) live in LDS only and never reach HBM.
+ * The result is bit-identical to nncase_hip_qconv2d called three times (the
+ * last with the input as fused residual) with the same quant params: every
+ * stage requantises to u8 exactly as the separate operators do.
+ */
+typedef struct nncase_hip_qblock_weights nncase_hip_qblock_t;
+
+typedef struct nncase_hip_qblock_desc {
+    int32_t in_channels, mid_channels, out_channels;
+    nncase_hip_quant_param_t expand_w_qp, dw_w_qp, project_w_qp; /* per-tensor weight quantisation of the stages */
+} nncase_hip_qblock_desc_t;
+
+/* 1 if the fused kernel is built for these channel counts (in_channels % 4 == 0 and <= 192,
+ * mid_channels % 4 == 0, out_channels <= 320), else 0: the caller then runs the three convolutions. */
+NNCASE_HIP_API int nncase_hip_qblock_supported(const nncase_hip_qblock_desc_t *desc);
+/* HOST weights, OIHW u8: expand [mid, in, 1, 1], depthwise [mid, 1, 3, 3], project [out, mid, 1, 1];
+ * int32 biases (NULL = zeros) in the accumulator scale of their stage. */
+NNCASE_HIP_API int nncase_hip_qblock_prepack(nncase_hip_ctx_t *ctx, const nncase_hip_qblock_desc_t *desc,
+                                             const uint8_t *w_expand_host, const int32_t *bias_expand_host,
+                                             const uint8_t *w_dw_host, const int32_t *bias_dw_host,
+                                             const uint8_t *w_project_host, const int32_t *bias_project_host,
+                                             nncase_hip_qblock_t **block);
+NNCASE_HIP_API int nncase_hip_qblock_destroy(nncase_hip_ctx_t *ctx, nncase_hip_qblock_t *block);
+
+typedef struct nncase_hip_qblock_args {
+    int32_t batch, in_h, in_w;           /* input is [batch, in_h, in_w, in_channels] u8            */
+    int32_t stride;                      /* of the depthwise stage, both axes: 1 or 2               */
+    int32_t pad_h_before, pad_h_after;   /* of the depthwise stage, each 0 or 1                     */
+    int32_t pad_w_before, pad_w_after;
+    nncase_hip_quant_param_t x_qp;       /* block input                                             */
+    nncase_hip_quant_param_t expand_qp;  /* output of the 1x1 expansion                             */
+    nncase_hip_quant_param_t dw_qp;      /* output of the depthwise stage                           */
+    nncase_hip_quant_param_t y_qp;       /* output of the 1x1 projection                            */
+    float expand_clamp_min, expand_clamp_max; /* fused_clamp of each stage, fp32 domain             */
+    float dw_clamp_min, dw_clamp_max;
+    float clamp_min, clamp_max;
+    /* add_input != 0: y = Q_sum(clamp(DQ_y(projection) + DQ_x(x))), the residual connection
+     * (needs stride 1 and out_channels == in_channels). */
+    int32_t add_input;
+    nncase_hip_quant_param_t sum_qp;
+    float sum_clamp_min, sum_clamp_max;
+} nncase_hip_qblock_args_t;
+
+/* Output is [batch, out_h, out_w, out_channels] u8 with out = (in + pad_before + pad_after - 3 + stride) / stride. */
+NNCASE_HIP_API int nncase_hip_qblock(nncase_hip_ctx_t *ctx, const uint8_t *x_dev, const nncase_hip_qblock_t *block,
+                                     uint8_t *y_dev, const nncase_hip_qblock_args_t *args);
+
 /* MatMul A[M,K] (u8, device) x B[K,N] (u8, row-major, HOST, pre-packed) with
  * the same three output forms; replaces kernels::stackvm::mat_mul
  * (tensor_ops.cpp:553-565 -> reference/matmul.cpp:28-48) on the
@@ -385,6 +439,9 @@ NNCASE_HIP_API int nncase_hip_function_add_dequantize(nncase_hip_function_t *fn,
 NNCASE_HIP_API int nncase_hip_function_add_qconv2d(nncase_hip_function_t *fn, const uint8_t *x_dev,
                                                    const nncase_hip_weights_t *weights, void *y_dev,
                                                    const nncase_hip_conv2d_args_t *args);
+NNCASE_HIP_API int nncase_hip_function_add_qblock(nncase_hip_function_t *fn, const uint8_t *x_dev,
+                                                  const nncase_hip_qblock_t *block, uint8_t *y_dev,
+                                                  const nncase_hip_qblock_args_t *args);
 NNCASE_HIP_API int nncase_hip_function_add_qadd(nncase_hip_function_t *fn, const uint8_t *a_dev,
                                                 nncase_hip_quant_param_t a_qp, const uint8_t *b_dev,
                                                 nncase_hip_quant_param_t b_qp, uint8_t *out_dev,

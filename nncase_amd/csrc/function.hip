@@ -9,7 +9,7 @@ namespace {
 
 struct Op {
     enum Kind { kQuantize, kDequantize, kConv, kAdd, kPool, kLut, kConcat, kResize, kMaxPool, kPack,
-                kGemm, kRmsNorm, kRope, kAttn, kArgmax, kEmbed, kAddI32 } kind;
+                kGemm, kRmsNorm, kRope, kAttn, kArgmax, kEmbed, kAddI32, kBlock } kind;
     const void *in0 = nullptr, *in1 = nullptr;
     void *out = nullptr;
     const nncase_hip_weights_t *weights = nullptr;
@@ -36,6 +36,8 @@ struct Op {
     nncase_hip_paged_attn_args_t attn{};
     int32_t mode = 0, delta = 0;
     float eps = 0.f;
+    const nncase_hip_qblock_t *block = nullptr;
+    nncase_hip_qblock_args_t blk{};
     int lane = 0; // independent operator chain this operator belongs to
 };
 
@@ -60,6 +62,8 @@ static int run_op(nncase_hip_function *fn, const Op &op) {
         return nncase_hip_dequantize(ctx, op.in0, op.dt_in, op.out, op.dt_out, op.count, op.qp0);
     case Op::kConv:
         return nncase_hip_qconv2d(ctx, (const uint8_t *)op.in0, op.weights, op.out, &op.conv);
+    case Op::kBlock:
+        return nncase_hip_qblock(ctx, (const uint8_t *)op.in0, op.block, (uint8_t *)op.out, &op.blk);
     case Op::kAdd:
         return nncase_hip_qadd(ctx, (const uint8_t *)op.in0, op.qp0, (const uint8_t *)op.in1, op.qp1, (uint8_t *)op.out,
                                op.qp2, op.lo, op.hi, op.count);
@@ -169,6 +173,16 @@ extern "C" int nncase_hip_function_add_qconv2d(nncase_hip_function_t *fn, const 
     Op op;
     op.kind = Op::kConv;
     op.in0 = x_dev, op.out = y_dev, op.weights = weights, op.conv = *args;
+    return push(fn, op);
+}
+
+extern "C" int nncase_hip_function_add_qblock(nncase_hip_function_t *fn, const uint8_t *x_dev, const nncase_hip_qblock_t *block,
+                                              uint8_t *y_dev, const nncase_hip_qblock_args_t *args) {
+    if (!fn) return -EINVAL;
+    NNHIP_REQUIRE(fn->ctx, x_dev && block && y_dev && args, -EINVAL, "function_add_qblock: null argument");
+    Op op;
+    op.kind = Op::kBlock;
+    op.in0 = x_dev, op.out = y_dev, op.block = block, op.blk = *args;
     return push(fn, op);
 }
 
@@ -455,6 +469,7 @@ extern "C" int nncase_hip_function_op_kernel(nncase_hip_function_t *fn, int32_t 
     case Op::kQuantize: snprintf(name, capacity, "quantize"); break;
     case Op::kDequantize: snprintf(name, capacity, "dequantize"); break;
     case Op::kConv: describe_conv_kernel(fn->ctx, op.weights, &op.conv, name, capacity); break;
+    case Op::kBlock: nncase_hip_qblock_describe(op.block, &op.blk, name, capacity); break;
     case Op::kAdd: snprintf(name, capacity, "qadd"); break;
     case Op::kPool: snprintf(name, capacity, "qglobal_avgpool"); break;
     case Op::kLut: snprintf(name, capacity, "lut_u8"); break;

@@ -1,0 +1,500 @@
+// Fused inverted-residual block: 1x1 expansion -> 3x3 depthwise -> 1x1 projection (+ input),
+// u8/u8, NHWC, one kernel.  The two expanded tensors are the largest of the block (6x the
+// input) and, run as three operators, are each written to and read back from HBM; here a
+// workgroup owns a 7x7 tile of OUTPUT pixels of one image and keeps everything between the
+// block's input and output in LDS:
+//
+//   input tile   the in-image part of the (6S+3)^2 input pixels the tile needs, as s8
+//   per chunk of 48 or 64 expanded channels (weights of the next chunk are prefetched
+//   global -> registers while this one is computed, then committed to the other LDS buffer):
+//     E  expansion on the matrix cores for every in-image pixel of the halo, requantised to
+//        u8 into the expansion tile (positions outside the image keep the zero point the
+//        tile was initialised with: they are the depthwise stage's padding)
+//     D  depthwise 3x3 from the expansion tile (16-bit multiply-adds, 4 channels per lane),
+//        requantised to u8 and stored as s8 in the depthwise tile
+//     P  projection: the depthwise tile is one k-step of the matrix-core reduction over the
+//        expanded channels, accumulated in registers across the chunks
+//   epilogue of P: zero points, requantisation, optional residual add, NHWC store.
+//
+// Every stage uses the arithmetic of the stand-alone kernels (same zero-point identity, same
+// fp32 requantisation sequence), so the output bytes equal those of three separate operators.
+// Tiles need a one-pixel halo of the expansion around them (recomputed per tile: 81 pixels
+// for 49 at stride 1, 225 input pixels for 49 outputs at stride 2).
+#include "qconv_igemm.hpp"
+
+#include <algorithm>
+#include <new>
+#include <vector>
+
+struct nncase_hip_qblock_weights {
+    int cin = 0, mid = 0, cout = 0;
+    int ke = 0;      // k-steps of the expansion (ceil(cin / 64))
+    int et = 0;      // 16-channel tiles per chunk of expanded channels (3 or 4)
+    int tpt = 0;     // 16-channel tiles of the projection's output held by every wave
+    int nchunks = 0, chunk_bytes = 0;
+    int off_p = 0, off_wd = 0, off_bd = 0, off_sd = 0, off_be = 0, off_se = 0; // byte offsets inside a chunk
+    int32_t zw_e = 0, zw_d = 0, zw_p = 0;
+    float sw_e = 1.f, sw_d = 1.f, sw_p = 1.f;
+    void *d_blob = nullptr;      // [nchunks][chunk_bytes]
+    int32_t *d_wsum_p = nullptr; // [cout]
+    int32_t *d_bias_p = nullptr; // [cout]
+};
+
+namespace nnhip {
+
+constexpr int kBlkThreads = 256;
+constexpr int kBlkTile = 7;  // output tile edge (divides every MobileNet resolution from 112 down to 7)
+constexpr int kBlkRowB = 80; // bytes per pixel of the two mid tiles: 64 channels + 16 so that rows spread over the banks
+
+struct BlockArgs {
+    const uint8_t *x;
+    const uint8_t *blob;
+    int chunk_bytes, nchunks;
+    int cin, mid, ke;
+    int xs; // bytes per pixel of the input tile (ke * 64 + 16)
+    int in_h, in_w, out_h, out_w, pad_h, pad_w, tiles_y, tiles_x;
+    int zxp_e, zwp_e, kzz_e; // expansion: zx - 128, zw - 128, cin * zxp * zwp
+    int zx_d;                // zero point of the expansion's output
+    uint32_t zmid_splat;
+    Epilogue ep_e, ep_d;
+    int off_p, off_wd, off_bd, off_sd, off_be, off_se;
+    int lds_xin, lds_et, lds_dt, lds_w;
+    IgemmArgs p; // projection stage: y, m, n, k, ldy, zxp, zwp, wsum, bias, ep, rep
+};
+
+template <int S, int TPT, int ET>
+__global__ __launch_bounds__(kBlkThreads) void qblock_kernel(const BlockArgs a) {
+    constexpr int HH = (kBlkTile - 1) * S + 3; // halo edge in input pixels
+    constexpr int HP = HH * HH;
+    constexpr int TP = kBlkTile * kBlkTile;
+    constexpr int CE = ET * 16, QUADS = ET * 4, PSTEP = kBlkThreads / QUADS;
+    constexpr int NS = (3 * ET * 1024 + TPT * 1024 + 9 * CE * 2 + 16 * CE + 4095) / 4096; // 16-byte vectors staged per thread
+
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    int32_t *cterm_p = reinterpret_cast<int32_t *>(smem); // [TPT * 16]
+    uint8_t *xin = smem + a.lds_xin;                     // [groups * 16][xs] s8
+    uint8_t *etile = smem + a.lds_et;                    // [HP][kBlkRowB] u8
+    uint8_t *dtile = smem + a.lds_dt;                    // [64][kBlkRowB] s8
+    uint8_t *wbuf = smem + a.lds_w;                      // [2][chunk_bytes]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int j = lane & 15, gq = lane >> 4;
+
+    uint32_t b = blockIdx.x;
+    const int tx = (int)(b % (uint32_t)a.tiles_x);
+    b /= (uint32_t)a.tiles_x;
+    const int ty = (int)(b % (uint32_t)a.tiles_y);
+    const int img = (int)(b / (uint32_t)a.tiles_y);
+    const int oy0 = ty * kBlkTile, ox0 = tx * kBlkTile;
+    const int iy0 = oy0 * S - a.pad_h, ix0 = ox0 * S - a.pad_w; // halo origin in input coordinates
+    // the part of the halo that lies inside the image
+    const int cy0 = max(iy0, 0), cy1 = min(iy0 + HH, a.in_h);
+    const int cx0 = max(ix0, 0), cx1 = min(ix0 + HH, a.in_w);
+    const int CW = max(cx1 - cx0, 1);
+    const int cnt = max(cy1 - cy0, 0) * max(cx1 - cx0, 0);
+    const int offy = cy0 - iy0, offx = cx0 - ix0;
+    const uint32_t rcw = 65536u / (uint32_t)CW + 1u; // idx / CW = (idx * rcw) >> 16 for idx < 256
+    const int ngroups = (cnt + 15) >> 4;
+
+    // ---- one-time fills ---------------------------------------------------------------------------
+    {
+        const u32x4 z = {a.zmid_splat, a.zmid_splat, a.zmid_splat, a.zmid_splat};
+        for (int i = tid; i < HP * (kBlkRowB / 16); i += kBlkThreads) reinterpret_cast<u32x4 *>(etile)[i] = z;
+        const u32x4 zero = {0, 0, 0, 0};
+        for (int i = tid; i < 64 * (kBlkRowB / 16); i += kBlkThreads) reinterpret_cast<u32x4 *>(dtile)[i] = zero;
+        for (int i = tid; i < TPT * 16; i += kBlkThreads) {
+            int32_t c = 0;
+            if (i < a.p.n) c = a.p.bias[i] - a.p.zxp * a.p.wsum[i] + a.p.k * a.p.zxp * a.p.zwp;
+            cterm_p[i] = c;
+        }
+        // input tile: 16 lanes copy one pixel's channels a dword each, re-biased to s8, zero past the channels
+        const int ps = tid >> 4, dl = tid & 15;
+        for (int idx = ps; idx < ngroups * 16; idx += kBlkThreads / 16) {
+            const int cy = (int)(((uint32_t)idx * rcw) >> 16), cx = idx - cy * CW;
+            const bool pix = idx < cnt;
+            const uint32_t src = (uint32_t)((img * a.in_h + cy0 + (pix ? cy : 0)) * a.in_w + cx0 + (pix ? cx : 0)) * (uint32_t)a.cin;
+            for (int s = 0; s < a.ke; s++) {
+                const int d = s * 16 + dl;
+                uint32_t v = 0;
+                if (pix && d * 4 < a.cin) v = *reinterpret_cast<const uint32_t *>(a.x + src + d * 4) ^ 0x80808080u;
+                *reinterpret_cast<uint32_t *>(xin + idx * a.xs + d * 4) = v;
+            }
+        }
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(a.blob);
+        for (int i = tid; i < a.chunk_bytes / 16; i += kBlkThreads) reinterpret_cast<u32x4 *>(wbuf)[i] = src[i];
+    }
+    __syncthreads();
+
+    const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
+    v4i accp[TPT];
+    v4i rsp = {0, 0, 0, 0};
+#pragma unroll
+    for (int nt = 0; nt < TPT; nt++) accp[nt] = v4i{0, 0, 0, 0};
+
+    const int nvec = a.chunk_bytes / 16;
+    for (int c = 0; c < a.nchunks; c++) {
+        const uint8_t *wb = wbuf + (c & 1) * a.chunk_bytes;
+        u32x4 stage[NS];
+        if (c + 1 < a.nchunks) {
+            const u32x4 *src = reinterpret_cast<const u32x4 *>(a.blob + (size_t)(c + 1) * a.chunk_bytes);
+#pragma unroll
+            for (int i = 0; i < NS; i++) {
+                const int v = i * kBlkThreads + tid;
+                stage[i] = src[v < nvec ? v : 0];
+            }
+        }
+
+        // ---- E: expansion of every in-image halo pixel, 16 pixels x 16 channels per unit -------------
+        for (int u = wave; u < ngroups * ET; u += kWaves) {
+            const int g = u / ET, nt = u - g * ET;
+            const int idx = g * 16 + j;
+            const uint8_t *xrow = xin + idx * a.xs + gq * 16;
+            const uint8_t *wfr = wb + nt * 1024 + lane * 16;
+            v4i acc = {0, 0, 0, 0}, rs = {0, 0, 0, 0};
+            for (int ks = 0; ks < a.ke; ks++) {
+                const v4i xf = *reinterpret_cast<const v4i *>(xrow + ks * 64);
+                const v4i wf = *reinterpret_cast<const v4i *>(wfr + ks * ET * 1024);
+                rs = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, xf, rs, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf, xf, acc, 0, 0, 0);
+            }
+            if (idx < cnt) {
+                const int cy = (int)(((uint32_t)idx * rcw) >> 16), cx = idx - cy * CW;
+                const int pos = (cy + offy) * HH + cx + offx;
+                const int cl = gq * (4 * ET) + nt * 4; // first of the lane's 4 channels within the chunk
+                const v4i be = *reinterpret_cast<const v4i *>(wb + a.off_be + cl * 4);
+                const v4i se = *reinterpret_cast<const v4i *>(wb + a.off_se + cl * 4);
+                const int32_t nrsz = a.kzz_e - a.zwp_e * rs[0];
+                uint32_t q[4];
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int32_t v = add3(acc[r], be[r] - a.zxp_e * se[r], nrsz);
+                    q[r] = requant_u8_lowbyte((float)v * a.ep_e.mult, a.ep_e);
+                }
+                *reinterpret_cast<uint32_t *>(etile + pos * kBlkRowB + cl) = pack_low_bytes(q[0], q[1], q[2], q[3]);
+            }
+        }
+        __syncthreads();
+
+        // ---- D: depthwise 3x3 on the expansion tile, 4 channels x 1 pixel per item ------------------------
+        if (tid < PSTEP * QUADS) {
+            const int qd = tid % QUADS, p0 = tid / QUADS;
+            uint32_t w01[9], w23[9];
+#pragma unroll
+            for (int t = 0; t < 9; t++) {
+                const u32x2 raw = *reinterpret_cast<const u32x2 *>(wb + a.off_wd + (t * CE + qd * 4) * 2);
+                w01[t] = raw[0];
+                w23[t] = raw[1];
+            }
+            const v4i bd = *reinterpret_cast<const v4i *>(wb + a.off_bd + qd * 16);
+            const v4i sd = *reinterpret_cast<const v4i *>(wb + a.off_sd + qd * 16);
+            int32_t ct[4];
+#pragma unroll
+            for (int r = 0; r < 4; r++) ct[r] = bd[r] - a.zx_d * sd[r];
+            const bool chv = c * CE + qd * 4 < a.mid;
+            for (int p = p0; p < TP; p += PSTEP) {
+                const int py = p / kBlkTile, px = p - py * kBlkTile;
+                const uint8_t *base = etile + ((py * S) * HH + px * S) * kBlkRowB + qd * 4;
+                int32_t acc[4] = {ct[0], ct[1], ct[2], ct[3]};
+#pragma unroll
+                for (int ky = 0; ky < 3; ky++)
+#pragma unroll
+                    for (int kx = 0; kx < 3; kx++) {
+                        const uint32_t d = *reinterpret_cast<const uint32_t *>(base + (ky * HH + kx) * kBlkRowB);
+                        const uint32_t x01 = __builtin_amdgcn_perm(0u, d, 0x0c010c00u);
+                        const uint32_t x23 = __builtin_amdgcn_perm(0u, d, 0x0c030c02u);
+                        const int t = ky * 3 + kx;
+                        acc[0] = mad16_lo(x01, w01[t], acc[0]);
+                        acc[1] = mad16_hi(x01, w01[t], acc[1]);
+                        acc[2] = mad16_lo(x23, w23[t], acc[2]);
+                        acc[3] = mad16_hi(x23, w23[t], acc[3]);
+                    }
+                uint32_t q[4];
+#pragma unroll
+                for (int r = 0; r < 4; r++) q[r] = requant_u8_lowbyte((float)acc[r] * a.ep_d.mult, a.ep_d);
+                const uint32_t packed = pack_low_bytes(q[0], q[1], q[2], q[3]) ^ 0x80808080u; // kept as s8
+                *reinterpret_cast<uint32_t *>(dtile + p * kBlkRowB + qd * 4) = chv ? packed : 0u;
+            }
+        }
+        __syncthreads();
+
+        // ---- P: this chunk is one k-step of the projection ----------------------------------------------------
+        {
+            const v4i xf = *reinterpret_cast<const v4i *>(dtile + (wave * 16 + j) * kBlkRowB + gq * 16);
+            rsp = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, xf, rsp, 0, 0, 0);
+            const uint8_t *wfr = wb + a.off_p + lane * 16;
+#pragma unroll
+            for (int nt = 0; nt < TPT; nt++) {
+                const v4i wf = *reinterpret_cast<const v4i *>(wfr + nt * 1024);
+                accp[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf, xf, accp[nt], 0, 0, 0);
+            }
+        }
+        if (c + 1 < a.nchunks) {
+            u32x4 *dst = reinterpret_cast<u32x4 *>(wbuf + ((c + 1) & 1) * a.chunk_bytes);
+#pragma unroll
+            for (int i = 0; i < NS; i++) {
+                const int v = i * kBlkThreads + tid;
+                if (v < nvec) dst[v] = stage[i];
+            }
+        }
+        __syncthreads();
+    }
+
+    // ---- epilogue of the projection ------------------------------------------------------------------------
+    const int pl = wave * 16 + j;
+    const int py = pl / kBlkTile, px = pl - py * kBlkTile;
+    const int oy = oy0 + py, ox = ox0 + px;
+    const bool valid = pl < TP && oy < a.out_h && ox < a.out_w;
+    const int pg = valid ? (img * a.out_h + oy) * a.out_w + ox : a.p.m;
+    igemm_store_tile<TPT>(a.p, accp, rsp[0], pg, gq * (4 * TPT), gq, cterm_p, nullptr);
+}
+
+template <int S, int TPT, int ET> static int launch_block_inst(nncase_hip_ctx *ctx, const BlockArgs &a, int blocks, size_t lds) {
+    if (lds > 48 * 1024) {
+        NNHIP_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(&qblock_kernel<S, TPT, ET>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    }
+    hipLaunchKernelGGL((qblock_kernel<S, TPT, ET>), dim3(blocks), dim3(kBlkThreads), lds, ctx->stream, a);
+    NNHIP_LAUNCH_CHECK(ctx, "qblock_kernel");
+    return 0;
+}
+
+template <int S, int TPT> static int launch_block_et(nncase_hip_ctx *ctx, const BlockArgs &a, int et, int blocks, size_t lds) {
+    return et == 3 ? launch_block_inst<S, TPT, 3>(ctx, a, blocks, lds) : launch_block_inst<S, TPT, 4>(ctx, a, blocks, lds);
+}
+
+template <int S> static int launch_block_s(nncase_hip_ctx *ctx, const BlockArgs &a, int tpt, int et, int blocks, size_t lds) {
+    switch (tpt) {
+    case 2: return launch_block_et<S, 2>(ctx, a, et, blocks, lds);
+    case 4: return launch_block_et<S, 4>(ctx, a, et, blocks, lds);
+    case 6: return launch_block_et<S, 6>(ctx, a, et, blocks, lds);
+    case 10: return launch_block_et<S, 10>(ctx, a, et, blocks, lds);
+    default: return launch_block_et<S, 20>(ctx, a, et, blocks, lds);
+    }
+}
+
+static int block_tiles(int cout) {
+    const int t = ceil_div(cout, 16);
+    for (int v : {2, 4, 6, 10, 20})
+        if (v >= t) return v;
+    return 0;
+}
+
+} // namespace nnhip
+
+using namespace nnhip;
+
+extern "C" int nncase_hip_qblock_supported(const nncase_hip_qblock_desc_t *d) {
+    if (!d) return 0;
+    return d->in_channels > 0 && d->in_channels % 4 == 0 && d->in_channels <= 192 && d->mid_channels > 0 &&
+                   d->mid_channels % 4 == 0 && d->mid_channels < 65536 && d->out_channels > 0 && block_tiles(d->out_channels) > 0
+               ? 1
+               : 0;
+}
+
+void nncase_hip_qblock_describe(const nncase_hip_qblock_t *b, const nncase_hip_qblock_args_t *a, char *buf, size_t cap) {
+    snprintf(buf, cap, "qblock%s<S=%d,P=%d,E=%d>", a->add_input ? "+add" : "", a->stride, b->tpt, b->et);
+}
+
+static void free_block(nncase_hip_qblock_t *b) {
+    if (!b) return;
+    if (b->d_blob) (void)hipFree(b->d_blob);
+    if (b->d_wsum_p) (void)hipFree(b->d_wsum_p);
+    if (b->d_bias_p) (void)hipFree(b->d_bias_p);
+    delete b;
+}
+
+extern "C" int nncase_hip_qblock_prepack(nncase_hip_ctx_t *ctx, const nncase_hip_qblock_desc_t *desc, const uint8_t *w_expand,
+                                         const int32_t *bias_expand, const uint8_t *w_dw, const int32_t *bias_dw,
+                                         const uint8_t *w_project, const int32_t *bias_project, nncase_hip_qblock_t **block) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, desc && w_expand && w_dw && w_project && block, -EINVAL, "qblock_prepack: null argument");
+    *block = nullptr;
+    NNHIP_REQUIRE(ctx, nncase_hip_qblock_supported(desc), -NNCASE_HIP_ERR_SHAPE_MISMATCH,
+                  "qblock_prepack: channels %d -> %d -> %d are outside what the fused kernel is built for", desc->in_channels,
+                  desc->mid_channels, desc->out_channels);
+    for (const nncase_hip_quant_param_t *q : {&desc->expand_w_qp, &desc->dw_w_qp, &desc->project_w_qp})
+        NNHIP_REQUIRE(ctx, q->zero_point >= 0 && q->zero_point <= 255, -EINVAL, "qblock_prepack: weight zero point %d outside u8",
+                      q->zero_point);
+    nncase_hip_qblock_t *b = new (std::nothrow) nncase_hip_qblock_t();
+    NNHIP_REQUIRE(ctx, b, -ENOMEM, "qblock_prepack: out of host memory");
+    const int cin = b->cin = desc->in_channels, mid = b->mid = desc->mid_channels, cout = b->cout = desc->out_channels;
+    b->zw_e = desc->expand_w_qp.zero_point, b->sw_e = desc->expand_w_qp.scale;
+    b->zw_d = desc->dw_w_qp.zero_point, b->sw_d = desc->dw_w_qp.scale;
+    b->zw_p = desc->project_w_qp.zero_point, b->sw_p = desc->project_w_qp.scale;
+    b->ke = ceil_div(cin, 64);
+    // 48-channel chunks when they divide the expanded channels and 64-channel ones do not (96, 144)
+    b->et = (mid % 64 != 0 && mid % 48 == 0) ? 3 : 4;
+    const int ce = b->et * 16;
+    b->tpt = block_tiles(cout);
+    b->nchunks = ceil_div(mid, ce);
+    b->off_p = b->ke * b->et * 1024;
+    b->off_wd = b->off_p + b->tpt * 1024;
+    b->off_bd = b->off_wd + 9 * ce * 2;
+    b->off_sd = b->off_bd + ce * 4;
+    b->off_be = b->off_sd + ce * 4;
+    b->off_se = b->off_be + ce * 4;
+    b->chunk_bytes = b->off_se + ce * 4;
+
+    std::vector<uint8_t> blob((size_t)b->nchunks * b->chunk_bytes, 0);
+    // expansion: [chunk][ks][tile] fragments, chunk = 16 * et channels
+    {
+        std::vector<uint8_t> frags((size_t)b->nchunks * b->ke * b->et * 1024);
+        std::vector<int32_t> wsum(mid);
+        pack_group(frags.data(), wsum.data(), mid, cin, b->ke, b->et, b->nchunks,
+                   [&](int oc, int kk) -> uint8_t { return w_expand[(size_t)oc * cin + kk]; });
+        for (int c = 0; c < b->nchunks; c++) {
+            uint8_t *dst = blob.data() + (size_t)c * b->chunk_bytes;
+            memcpy(dst, frags.data() + (size_t)c * b->ke * b->et * 1024, (size_t)b->ke * b->et * 1024);
+            int32_t *be = reinterpret_cast<int32_t *>(dst + b->off_be), *se = reinterpret_cast<int32_t *>(dst + b->off_se);
+            for (int i = 0; i < ce; i++) {
+                const int ch = c * ce + i;
+                be[i] = (ch < mid && bias_expand) ? bias_expand[ch] : 0;
+                se[i] = ch < mid ? wsum[ch] : 0;
+            }
+        }
+    }
+    // projection: chunk c of the expanded channels is k-step c, channels past the chunk's width are zero weights
+    std::vector<int32_t> wsum_p(cout), bias_p(cout, 0);
+    {
+        std::vector<uint8_t> frags((size_t)b->nchunks * b->tpt * 1024);
+        pack_group(frags.data(), wsum_p.data(), cout, b->nchunks * 64, b->nchunks, b->tpt, 1, [&](int oc, int kk) -> uint8_t {
+            const int ks = kk / 64, pos = kk % 64, ch = ks * ce + pos;
+            return (pos < ce && ch < mid) ? w_project[(size_t)oc * mid + ch] : (uint8_t)0x80;
+        });
+        for (int c = 0; c < b->nchunks; c++)
+            memcpy(blob.data() + (size_t)c * b->chunk_bytes + b->off_p, frags.data() + (size_t)c * b->tpt * 1024, (size_t)b->tpt * 1024);
+        if (bias_project) std::copy(bias_project, bias_project + cout, bias_p.begin());
+    }
+    // depthwise: (w - zw) as int16 [tap][channel of the chunk], bias and tap sum per channel
+    for (int c = 0; c < b->nchunks; c++) {
+        uint8_t *dst = blob.data() + (size_t)c * b->chunk_bytes;
+        int16_t *wd = reinterpret_cast<int16_t *>(dst + b->off_wd);
+        int32_t *bd = reinterpret_cast<int32_t *>(dst + b->off_bd), *sd = reinterpret_cast<int32_t *>(dst + b->off_sd);
+        for (int i = 0; i < ce; i++) {
+            const int ch = c * ce + i;
+            int32_t s = 0;
+            for (int t = 0; t < 9; t++) {
+                const int v = ch < mid ? (int)w_dw[(size_t)ch * 9 + t] - b->zw_d : 0;
+                wd[t * ce + i] = (int16_t)v;
+                s += v;
+            }
+            bd[i] = (ch < mid && bias_dw) ? bias_dw[ch] : 0;
+            sd[i] = s;
+        }
+    }
+    hipError_t e = hipSetDevice(ctx->device);
+    if (e == hipSuccess) e = hipMalloc(&b->d_blob, blob.size());
+    if (e == hipSuccess) e = hipMalloc((void **)&b->d_wsum_p, sizeof(int32_t) * cout);
+    if (e == hipSuccess) e = hipMalloc((void **)&b->d_bias_p, sizeof(int32_t) * cout);
+    if (e == hipSuccess) e = hipMemcpy(b->d_blob, blob.data(), blob.size(), hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMemcpy(b->d_wsum_p, wsum_p.data(), sizeof(int32_t) * cout, hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMemcpy(b->d_bias_p, bias_p.data(), sizeof(int32_t) * cout, hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+        free_block(b);
+        return hip_fail(ctx, e, "qblock_prepack");
+    }
+    *block = b;
+    return 0;
+}
+
+extern "C" int nncase_hip_qblock_destroy(nncase_hip_ctx_t *ctx, nncase_hip_qblock_t *block) {
+    NNHIP_CHECK_CTX(ctx);
+    if (!block) return 0;
+    NNHIP_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    free_block(block);
+    return 0;
+}
+
+extern "C" int nncase_hip_qblock(nncase_hip_ctx_t *ctx, const uint8_t *x_dev, const nncase_hip_qblock_t *blk, uint8_t *y_dev,
+                                 const nncase_hip_qblock_args_t *g) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, x_dev && blk && y_dev && g, -EINVAL, "qblock: null argument");
+    NNHIP_REQUIRE(ctx, g->batch > 0 && g->in_h > 0 && g->in_w > 0, -EINVAL, "qblock: non-positive input shape");
+    NNHIP_REQUIRE(ctx, g->stride == 1 || g->stride == 2, -EINVAL, "qblock: depthwise stride %d (1 or 2)", g->stride);
+    for (int pad : {g->pad_h_before, g->pad_h_after, g->pad_w_before, g->pad_w_after})
+        NNHIP_REQUIRE(ctx, pad == 0 || pad == 1, -EINVAL, "qblock: depthwise padding %d (0 or 1)", pad);
+    for (const nncase_hip_quant_param_t *q : {&g->x_qp, &g->expand_qp, &g->dw_qp})
+        NNHIP_REQUIRE(ctx, q->zero_point >= 0 && q->zero_point <= 255, -EINVAL, "qblock: zero point %d outside u8", q->zero_point);
+    const int out_h = windowed_output_size(g->in_h, 3, g->stride, 1, g->pad_h_before, g->pad_h_after);
+    const int out_w = windowed_output_size(g->in_w, 3, g->stride, 1, g->pad_w_before, g->pad_w_after);
+    NNHIP_REQUIRE(ctx, out_h > 0 && out_w > 0, -NNCASE_HIP_ERR_SHAPE_MISMATCH, "qblock: window larger than padded input");
+    NNHIP_REQUIRE(ctx, !g->add_input || (g->stride == 1 && blk->cin == blk->cout && out_h == g->in_h && out_w == g->in_w),
+                  -NNCASE_HIP_ERR_SHAPE_MISMATCH, "qblock: the residual needs an output of the input's shape");
+    const int64_t m64 = (int64_t)g->batch * out_h * out_w;
+    NNHIP_REQUIRE(ctx, m64 < ((int64_t)1 << 30) && (int64_t)g->batch * g->in_h * g->in_w * blk->cin < ((int64_t)1 << 31) &&
+                           m64 * blk->cout < ((int64_t)1 << 31),
+                  -EINVAL, "qblock: tensors of 2^31 bytes or more are not supported");
+    NNHIP_REQUIRE(ctx, (reinterpret_cast<uintptr_t>(x_dev) & 15u) == 0 && (reinterpret_cast<uintptr_t>(y_dev) & 15u) == 0,
+                  -NNCASE_HIP_ERR_INVALID_MEMORY_LOCATION, "qblock: activation buffers must be 16-byte aligned");
+
+    BlockArgs a;
+    memset(&a, 0, sizeof(a));
+    a.x = x_dev;
+    a.blob = reinterpret_cast<const uint8_t *>(blk->d_blob);
+    a.chunk_bytes = blk->chunk_bytes;
+    a.nchunks = blk->nchunks;
+    a.cin = blk->cin;
+    a.mid = blk->mid;
+    a.ke = blk->ke;
+    a.xs = blk->ke * 64 + 16;
+    a.in_h = g->in_h, a.in_w = g->in_w, a.out_h = out_h, a.out_w = out_w;
+    a.pad_h = g->pad_h_before, a.pad_w = g->pad_w_before;
+    a.tiles_y = ceil_div(out_h, kBlkTile), a.tiles_x = ceil_div(out_w, kBlkTile);
+    a.zxp_e = g->x_qp.zero_point - 128;
+    a.zwp_e = blk->zw_e - 128;
+    a.kzz_e = blk->cin * a.zxp_e * a.zwp_e;
+    a.zx_d = g->expand_qp.zero_point;
+    a.zmid_splat = (uint32_t)(g->expand_qp.zero_point & 0xff) * 0x01010101u;
+    int rc = make_epilogue(ctx, &a.ep_e, g->x_qp.scale, blk->sw_e, g->expand_qp, g->expand_clamp_min, g->expand_clamp_max,
+                           NNCASE_HIP_DT_U8, "qblock(expand)");
+    if (rc) return rc;
+    rc = make_epilogue(ctx, &a.ep_d, g->expand_qp.scale, blk->sw_d, g->dw_qp, g->dw_clamp_min, g->dw_clamp_max, NNCASE_HIP_DT_U8,
+                       "qblock(depthwise)");
+    if (rc) return rc;
+    a.off_p = blk->off_p, a.off_wd = blk->off_wd, a.off_bd = blk->off_bd, a.off_sd = blk->off_sd, a.off_be = blk->off_be,
+    a.off_se = blk->off_se;
+    a.p.y = y_dev;
+    a.p.m = (int)m64;
+    a.p.n = blk->cout;
+    a.p.k = blk->mid;
+    a.p.ldy = blk->cout;
+    a.p.zxp = g->dw_qp.zero_point - 128;
+    a.p.zwp = blk->zw_p - 128;
+    a.p.wsum = blk->d_wsum_p;
+    a.p.bias = blk->d_bias_p;
+    rc = make_epilogue(ctx, &a.p.ep, g->dw_qp.scale, blk->sw_p, g->y_qp, g->clamp_min, g->clamp_max, NNCASE_HIP_DT_U8, "qblock(project)");
+    if (rc) return rc;
+    {
+        nncase_hip_conv2d_args_t c;
+        memset(&c, 0, sizeof(c));
+        c.out_dtype = NNCASE_HIP_DT_U8;
+        c.y_qp = g->y_qp;
+        if (g->add_input) {
+            NNHIP_REQUIRE(ctx, g->sum_qp.scale > 0.f && std::isfinite(g->sum_qp.scale) && g->sum_qp.zero_point >= 0 &&
+                                   g->sum_qp.zero_point <= 255,
+                          -EINVAL, "qblock: quant param of the sum outside u8 / positive scale");
+            c.residual_dev = x_dev;
+            c.residual_qp = g->x_qp;
+            c.sum_qp = g->sum_qp;
+            c.sum_clamp_min = g->sum_clamp_min;
+            c.sum_clamp_max = g->sum_clamp_max;
+        }
+        rc = make_residual_epilogue(ctx, &a.p.rep, &c, nullptr);
+        if (rc) return rc;
+    }
+    const int hh = (kBlkTile - 1) * g->stride + 3, hp = hh * hh;
+    const int cterm_bytes = blk->tpt * 16 * 4;
+    a.lds_xin = cterm_bytes;
+    a.lds_et = a.lds_xin + ceil_div(hp, 16) * 16 * a.xs;
+    a.lds_dt = a.lds_et + hp * kBlkRowB;
+    a.lds_w = a.lds_dt + 64 * kBlkRowB;
+    const size_t lds = (size_t)a.lds_w + 2 * (size_t)blk->chunk_bytes;
+    NNHIP_REQUIRE(ctx, lds <= 160 * 1024, -EINVAL, "qblock: %zu bytes of LDS needed", lds);
+    const int64_t blocks = (int64_t)g->batch * a.tiles_y * a.tiles_x;
+    NNHIP_REQUIRE(ctx, blocks < ((int64_t)1 << 31), -EINVAL, "qblock: too many tiles");
+    NNHIP_HIP(ctx, hipSetDevice(ctx->device));
+    return g->stride == 1 ? launch_block_s<1>(ctx, a, blk->tpt, blk->et, (int)blocks, lds)
+                          : launch_block_s<2>(ctx, a, blk->tpt, blk->et, (int)blocks, lds);
+}

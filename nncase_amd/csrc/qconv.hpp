@@ -87,6 +87,10 @@ int igemm_pixel_groups(const nncase_hip_ctx *ctx, const nncase_hip_weights *w, i
 bool igemm_streams_weights(const nncase_hip_weights *w, int mode);
 int stream_pixel_groups(const nncase_hip_ctx *ctx, const nncase_hip_weights *w, int m);
 int igemm_load_mode(const nncase_hip_weights *w, const nncase_hip_conv2d_args_t *c, int out_h, int out_w);
+} // namespace nnhip
+// Writes the name of the kernel a fused block launches.
+void nncase_hip_qblock_describe(const nncase_hip_qblock_t *b, const nncase_hip_qblock_args_t *a, char *buf, size_t cap);
+namespace nnhip {
 bool depthwise_uses_3x3(const nncase_hip_weights *w, const nncase_hip_conv2d_args_t *c);
 
 // Correctly rounded a / b from b and rb = RN(1 / b): one multiply and two fused
@@ -128,6 +132,20 @@ __device__ __forceinline__ uint32_t residual_lowbyte(uint32_t q, uint32_t res, i
 __device__ __forceinline__ int32_t add3(int32_t a, int32_t b, int32_t c) {
     int32_t d;
     asm("v_add3_u32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "v"(c));
+    return d;
+}
+
+// acc + x.i16[H] * w.i16[H] (v_mad_i32_i16 with op_sel picking the 16-bit halves): the
+// multiply-add reads both 16-bit halves of a register directly, so activations are kept
+// as two zero-extended bytes per register and weights as the int16 pairs they are stored as.
+__device__ __forceinline__ int32_t mad16_lo(uint32_t x, uint32_t w, int32_t acc) {
+    int32_t d;
+    asm("v_mad_i32_i16 %0, %1, %2, %3" : "=v"(d) : "v"(x), "v"(w), "v"(acc));
+    return d;
+}
+__device__ __forceinline__ int32_t mad16_hi(uint32_t x, uint32_t w, int32_t acc) {
+    int32_t d;
+    asm("v_mad_i32_i16 %0, %1, %2, %3 op_sel:[1,1,0,0]" : "=v"(d) : "v"(x), "v"(w), "v"(acc));
     return d;
 }
 

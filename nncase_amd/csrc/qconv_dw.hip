@@ -63,20 +63,6 @@ __device__ __forceinline__ void dw_store4(const DwArgs &a, uint32_t o, const int
     }
 }
 
-// acc + x.i16[H] * w.i16[H] (v_mad_i32_i16 with op_sel picking the 16-bit halves): the
-// multiply-add reads both 16-bit halves of a register directly, so activations are kept
-// as two zero-extended bytes per register and weights as the int16 pairs they are stored as.
-__device__ __forceinline__ int32_t mad16_lo(uint32_t x, uint32_t w, int32_t acc) {
-    int32_t d;
-    asm("v_mad_i32_i16 %0, %1, %2, %3" : "=v"(d) : "v"(x), "v"(w), "v"(acc));
-    return d;
-}
-__device__ __forceinline__ int32_t mad16_hi(uint32_t x, uint32_t w, int32_t acc) {
-    int32_t d;
-    asm("v_mad_i32_i16 %0, %1, %2, %3 op_sel:[1,1,0,0]" : "=v"(d) : "v"(x), "v"(w), "v"(acc));
-    return d;
-}
-
 // A conditional between two named objects is an lvalue in C++, which the compiler may turn
 // into a load through a selected address (private memory); taking the operands by value
 // keeps the choice a register select.

@@ -71,6 +71,36 @@ struct IgemmArgs {
     const uint32_t *lut;   // 256-entry byte table applied to the requantised byte (before the residual add), or null
 };
 
+// Packs one group's weights into MFMA operand order.
+//   w_at(oc, k) -> u8 weight of output channel oc (within the group) at
+//   reduction index k = (ky * kw + kx) * g_ic + ic.
+// Fragment (chunk, ks, nt): byte (kg * 16 + i) * 16 + b holds the weight of
+//   channel chunk*16T + (i / 4) * 4T + nt * 4 + (i % 4) at k = ks*64 + kg*16 + b,
+// re-biased to s8, or 0 outside the real channel / reduction range.
+template <typename WAt>
+inline void pack_group(uint8_t *dst, int32_t *wsum, int g_oc, int k, int ksteps, int tiles, int nchunks, WAt w_at) {
+    for (int oc = 0; oc < g_oc; oc++) {
+        int32_t s = 0;
+        for (int kk = 0; kk < k; kk++) s += (int32_t)(int8_t)(w_at(oc, kk) ^ 0x80);
+        wsum[oc] = s;
+    }
+    for (int chunk = 0; chunk < nchunks; chunk++)
+        for (int ks = 0; ks < ksteps; ks++)
+            for (int nt = 0; nt < tiles; nt++) {
+                uint8_t *frag = dst + (((size_t)chunk * ksteps + ks) * tiles + nt) * 1024;
+                for (int kg = 0; kg < 4; kg++)
+                    for (int i = 0; i < 16; i++) {
+                        const int oc = chunk * 16 * tiles + (i / 4) * 4 * tiles + nt * 4 + (i % 4);
+                        for (int b = 0; b < 16; b++) {
+                            const int kk = ks * 64 + kg * 16 + b;
+                            uint8_t v = 0;
+                            if (oc < g_oc && kk < k) v = (uint8_t)(w_at(oc, kk) ^ 0x80);
+                            frag[(kg * 16 + i) * 16 + b] = v;
+                        }
+                    }
+            }
+}
+
 struct PixInfo {
     int base; // kRows16: pixel index; other modes: pixel index of the image origin; < 0: no such pixel
     int iy0, ix0;

@@ -352,7 +352,7 @@ class HipModel:
     so results are bit-identical to lanes == 1."""
 
     def __init__(self, ctx: Context, qg: QuantGraph, batch: int, capture_graph: bool = True, fuse_residual: bool = True,
-                 lanes: int = 1):
+                 lanes: int = 1, fuse_blocks: bool = False):
         if lanes < 1 or lanes > rt.MAX_LANES or batch % lanes:
             raise ValueError(f"lanes={lanes} must be in 1..{rt.MAX_LANES} and divide the batch ({batch})")
         self.ctx, self.qg, self.batch, self.lanes = ctx, qg, batch, lanes
@@ -365,6 +365,7 @@ class HipModel:
         self.weights: List[Optional[rt.Weights]] = []
         self.op_names: List[str] = []
         self.op_nodes: List[int] = []
+        self.op_members: List[List[int]] = []   # graph nodes every recorded operator computes (per lane-0 operator)
         # A residual add whose second operand is a dense conv consumed by nothing else is folded into
         # that conv's epilogue (the conv's own u8 tensor is then never written).
         consumers = [0] * len(qg.nodes)
@@ -397,16 +398,53 @@ class HipModel:
         for conv, add in self.fused_into.items():
             if conv in self.fused_lut:
                 self.never_written.add(self.fused_lut[conv])
-        skip_nodes = set(self.fused_into.values()) | set(self.fused_lut.values())
+        fused_tail = set(self.fused_into.values()) | set(self.fused_lut.values())   # nodes computed in a conv's epilogue
+        skip_nodes = set(fused_tail)
+        # Inverted-residual blocks (1x1 conv -> 3x3 depthwise -> 1x1 conv, each consumed only by the next, optionally
+        # + the block's input) run as one fused operator: the two expanded tensors then never reach HBM.
+        self.blocks: Dict[int, Tuple[int, int, Optional[int]]] = {}   # expansion node -> (depthwise, projection, add or None)
+        if fuse_blocks and fuse_residual:
+            def pointwise(n):
+                return (n.op == "conv" and n.groups == 1 and n.weights.shape[2:] == (1, 1) and tuple(n.stride) == (1, 1)
+                        and tuple(map(tuple, n.padding)) == ((0, 0), (0, 0)))
+
+            def depthwise3(n):
+                return (n.op == "conv" and n.groups == n.weights.shape[0] and n.weights.shape[1:] == (1, 3, 3)
+                        and tuple(n.stride) in ((1, 1), (2, 2)) and all(p in (0, 1) for pp in n.padding for p in pp))
+            for i in range(len(qg.nodes) - 2):
+                e, d, pr = qg.nodes[i], qg.nodes[i + 1], qg.nodes[i + 2]
+                if not (pointwise(e) and depthwise3(d) and pointwise(pr)):
+                    continue
+                if tuple(d.inputs) != (i,) or tuple(pr.inputs) != (i + 1,) or consumers[i] != 1 or consumers[i + 1] != 1:
+                    continue
+                if {i, i + 1} & set(qg.output_nodes) or {i, i + 1, i + 2} & set(self.fused_lut):
+                    continue
+                addn = self.fused_into.get(i + 2)
+                if addn is not None and (qg.nodes[addn].inputs[0] != e.inputs[0] or tuple(d.stride) != (1, 1)):
+                    continue
+                if not ctx.qblock_supported(e.weights.shape[1], e.weights.shape[0], pr.weights.shape[0]):
+                    continue
+                self.blocks[i] = (i + 1, i + 2, addn)
+        for e, (d, pr, addn) in self.blocks.items():
+            self.never_written |= {e, d}
+            skip_nodes |= {d, pr}
+        block_members = {m for e, (d, pr, _) in self.blocks.items() for m in (e, d, pr)}
         # buffers and packed weights once, shared by the lanes
         for i, n in enumerate(qg.nodes):
             cc, hh, ww = n.out_shape
             self.weights.append(None)
-            if i in skip_nodes:
-                self.buffers.append(self.buffers[i - 1])  # written by the conv it is fused into
+            if i in fused_tail:
+                self.buffers.append(self.buffers[i - 1])  # written by the operator it is fused into
                 continue
-            self.buffers.append(ctx.alloc(lanes * self._lane_stride(bl * cc * hh * ww)))
-            if n.op == "conv":
+            if i in self.blocks or i - 1 in self.blocks:
+                self.buffers.append(ctx.alloc(16))        # the expanded tensors of a fused block live in LDS only
+            else:
+                self.buffers.append(ctx.alloc(lanes * self._lane_stride(bl * cc * hh * ww)))
+            if i in self.blocks:
+                d, pr = qg.nodes[i + 1], qg.nodes[i + 2]
+                self.weights[-1] = ctx.prepack_qblock(n.weights, n.bias, qp(*n.w_qp), d.weights, d.bias, qp(*d.w_qp),
+                                                      pr.weights, pr.bias, qp(*pr.w_qp))
+            elif n.op == "conv" and i not in block_members:
                 wt = ctx.prepack_conv2d(n.weights, n.bias, qp(*n.w_qp), n.groups, expected_pixels=bl * hh * ww)
                 fused_lut = self.fused_lut.get(i)
                 if fused_lut is not None:
@@ -441,6 +479,27 @@ class HipModel:
             cc, hh, ww = n.out_shape
             fused_add = self.fused_into.get(i)
             fused_lut = self.fused_lut.get(i)
+            members = [i] + ([fused_lut] if fused_lut is not None else []) + ([fused_add] if fused_add is not None else [])
+            if i in self.blocks:
+                dn, pn, addn = self.blocks[i]
+                d, pr, src = qg.nodes[dn], qg.nodes[pn], qg.nodes[n.inputs[0]]
+                a = rt.QBlockArgs()
+                a.batch, a.in_h, a.in_w, a.stride = bl, src.out_shape[1], src.out_shape[2], d.stride[0]
+                (a.pad_h_before, a.pad_h_after), (a.pad_w_before, a.pad_w_after) = d.padding
+                a.x_qp, a.expand_qp, a.dw_qp, a.y_qp = qp(*src.out_qp), qp(*n.out_qp), qp(*d.out_qp), qp(*pr.out_qp)
+                a.expand_clamp_min, a.expand_clamp_max = n.clamp
+                a.dw_clamp_min, a.dw_clamp_max = d.clamp
+                a.clamp_min, a.clamp_max = pr.clamp
+                a.add_input = int(addn is not None)
+                if addn is not None:
+                    a.sum_qp = qp(*qg.nodes[addn].out_qp)
+                    a.sum_clamp_min, a.sum_clamp_max = FULL_CLAMP
+                self.fn.add_qblock(B(n.inputs[0]), self.weights[i], B(pn), a)
+                if lane == 0:
+                    self.op_names.append(f"block:{n.name}" + ("+add" if addn is not None else ""))
+                    self.op_nodes.append(addn if addn is not None else pn)
+                    self.op_members.append([i, dn, pn] + ([addn] if addn is not None else []))
+                continue
             buf = B(i)
             if n.op == "input":
                 self.fn.add_quantize(self.input_f32.view(lane * self._lane_stride(in_per * 4), in_per * 4), rt.DT_F32, buf, rt.DT_U8, in_per, qp(*n.out_qp))
@@ -490,6 +549,7 @@ class HipModel:
             if lane == 0:
                 self.op_names.append(f"{n.op}:{n.name}" + ("+lut" if fused_lut is not None else "") + ("+add" if fused_add is not None else ""))
                 self.op_nodes.append(fused_add if fused_add is not None else (fused_lut if fused_lut is not None else i))
+                self.op_members.append(members)
         for k, j in enumerate(qg.output_nodes):
             node = qg.nodes[j]
             count = bl * int(np.prod(node.out_shape))
@@ -497,6 +557,7 @@ class HipModel:
             if lane == 0:
                 self.op_names.append("dequantize:" + node.name)
                 self.op_nodes.append(j)
+                self.op_members.append([])
 
     def set_input(self, x_nhwc: np.ndarray):
         x = np.ascontiguousarray(x_nhwc, f32)

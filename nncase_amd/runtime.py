@@ -53,6 +53,21 @@ class Conv2dArgs(C.Structure):
                 ("sum_clamp_min", C.c_float), ("sum_clamp_max", C.c_float)]
 
 
+class QBlockDesc(C.Structure):
+    _fields_ = [("in_channels", C.c_int32), ("mid_channels", C.c_int32), ("out_channels", C.c_int32),
+                ("expand_w_qp", QuantParam), ("dw_w_qp", QuantParam), ("project_w_qp", QuantParam)]
+
+
+class QBlockArgs(C.Structure):
+    _fields_ = [("batch", C.c_int32), ("in_h", C.c_int32), ("in_w", C.c_int32), ("stride", C.c_int32),
+                ("pad_h_before", C.c_int32), ("pad_h_after", C.c_int32), ("pad_w_before", C.c_int32), ("pad_w_after", C.c_int32),
+                ("x_qp", QuantParam), ("expand_qp", QuantParam), ("dw_qp", QuantParam), ("y_qp", QuantParam),
+                ("expand_clamp_min", C.c_float), ("expand_clamp_max", C.c_float),
+                ("dw_clamp_min", C.c_float), ("dw_clamp_max", C.c_float),
+                ("clamp_min", C.c_float), ("clamp_max", C.c_float),
+                ("add_input", C.c_int32), ("sum_qp", QuantParam), ("sum_clamp_min", C.c_float), ("sum_clamp_max", C.c_float)]
+
+
 class MatmulArgs(C.Structure):
     _fields_ = [("m", C.c_int32), ("a_qp", QuantParam), ("y_qp", QuantParam),
                 ("clamp_min", C.c_float), ("clamp_max", C.c_float), ("out_dtype", C.c_int32)]
@@ -87,6 +102,11 @@ SYMBOLS = {
     "nncase_hip_weights_destroy": (_I, [_VP, _VP]),
     "nncase_hip_weights_set_post_lut": (_I, [_VP, _VP, _VP, QuantParam]),
     "nncase_hip_qconv2d": (_I, [_VP, _VP, _VP, _VP, C.POINTER(Conv2dArgs)]),
+    "nncase_hip_qblock_supported": (_I, [C.POINTER(QBlockDesc)]),
+    "nncase_hip_qblock_prepack": (_I, [_VP, C.POINTER(QBlockDesc), _VP, _VP, _VP, _VP, _VP, _VP, C.POINTER(_VP)]),
+    "nncase_hip_qblock_destroy": (_I, [_VP, _VP]),
+    "nncase_hip_qblock": (_I, [_VP, _VP, _VP, _VP, C.POINTER(QBlockArgs)]),
+    "nncase_hip_function_add_qblock": (_I, [_VP, _VP, _VP, _VP, C.POINTER(QBlockArgs)]),
     "nncase_hip_qmatmul_prepack": (_I, [_VP, _VP, C.c_int32, C.c_int32, QuantParam, _VP, C.c_int64, C.POINTER(_VP)]),
     "nncase_hip_qmatmul": (_I, [_VP, _VP, _VP, _VP, C.POINTER(MatmulArgs)]),
     "nncase_hip_qadd": (_I, [_VP, _VP, QuantParam, _VP, QuantParam, _VP, QuantParam, C.c_float, C.c_float, _SZ]),
@@ -289,6 +309,25 @@ class Weights:
             pass
 
 
+class QBlock:
+    """Pre-packed constants of a fused expand -> depthwise -> project block (nncase_hip_qblock_t)."""
+
+    def __init__(self, ctx: "Context", handle, channels: Tuple[int, int, int]):
+        self.ctx, self.handle, self.channels = ctx, handle, channels
+
+    def destroy(self):
+        if self.handle:
+            if self.ctx.handle:
+                self.ctx.lib.nncase_hip_qblock_destroy(self.ctx.handle, self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass
+
+
 def windowed_output_size(size, filt, stride, dilation, before, after) -> int:
     """src/Native/include/nncase/kernels/kernel_utils.h:86-93."""
     eff = (filt - 1) * dilation + 1
@@ -376,6 +415,29 @@ class Context:
 
     def qconv2d(self, x: DeviceBuffer, w: Weights, y: DeviceBuffer, args: Conv2dArgs):
         self._check(self.lib.nncase_hip_qconv2d(self.handle, x.ptr, w.handle, y.ptr, C.byref(args)), "qconv2d")
+
+    def qblock_supported(self, cin: int, mid: int, cout: int) -> bool:
+        d = QBlockDesc(cin, mid, cout, qp(0, 1.0), qp(0, 1.0), qp(0, 1.0))
+        return bool(self.lib.nncase_hip_qblock_supported(C.byref(d)))
+
+    def prepack_qblock(self, w_expand, b_expand, qp_expand, w_dw, b_dw, qp_dw, w_project, b_project, qp_project) -> QBlock:
+        """OIHW u8 weights [mid, in, 1, 1], [mid, 1, 3, 3], [out, mid, 1, 1] and int32 biases (or None)."""
+        we, wd, wp = (np.ascontiguousarray(w, np.uint8) for w in (w_expand, w_dw, w_project))
+        mid, cin = we.shape[:2]
+        cout = wp.shape[0]
+        assert we.shape == (mid, cin, 1, 1) and wd.shape == (mid, 1, 3, 3) and wp.shape == (cout, mid, 1, 1)
+        bs = [None if b is None else np.ascontiguousarray(b, np.int32) for b in (b_expand, b_dw, b_project)]
+        for b, n in zip(bs, (mid, mid, cout)):
+            assert b is None or b.shape == (n,)
+        bp = [None if b is None else b.ctypes.data for b in bs]
+        desc = QBlockDesc(cin, mid, cout, qp_expand, qp_dw, qp_project)
+        h = C.c_void_p()
+        self._check(self.lib.nncase_hip_qblock_prepack(self.handle, C.byref(desc), we.ctypes.data, bp[0], wd.ctypes.data, bp[1],
+                                                       wp.ctypes.data, bp[2], C.byref(h)), "qblock_prepack")
+        return QBlock(self, h.value, (cin, mid, cout))
+
+    def qblock(self, x, blk: QBlock, y, args: QBlockArgs):
+        self._check(self.lib.nncase_hip_qblock(self.handle, x.ptr, blk.handle, y.ptr, C.byref(args)), "qblock")
 
     def prepack_matmul(self, b_kn: np.ndarray, bias: Optional[np.ndarray], b_qp: QuantParam, expected_rows: int = 0) -> Weights:
         b = np.ascontiguousarray(b_kn, np.uint8)
@@ -497,6 +559,11 @@ class Function:
         self._keep += [x, w, y]
         self._ck(self.ctx.lib.nncase_hip_function_add_qconv2d(self.handle, x.ptr, w.handle, y.ptr, C.byref(args)),
                  "function_add_qconv2d")
+
+    def add_qblock(self, x, blk: QBlock, y, args: QBlockArgs):
+        self._keep += [x, blk, y]
+        self._ck(self.ctx.lib.nncase_hip_function_add_qblock(self.handle, x.ptr, blk.handle, y.ptr, C.byref(args)),
+                 "function_add_qblock")
 
     def add_qadd(self, a, a_qp, b, b_qp, out, y_qp, count, clamp=(-FLT_MAX, FLT_MAX)):
         self._keep += [a, b, out]

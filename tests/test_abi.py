@@ -48,4 +48,5 @@ def test_struct_layouts_match_the_header():
     assert C.sizeof(rt.Conv2dDesc) == 5 * 4 + 8 + 4 + 8  # 4 bytes of padding before the int64
     assert C.sizeof(rt.Conv2dArgs) == 11 * 4 + 8 + 8 + 3 * 4 + 8 + 8 + 8 + 2 * 4
     assert C.sizeof(rt.MatmulArgs) == 4 + 8 + 8 + 3 * 4
+    assert C.sizeof(rt.QBlockDesc) == 3 * 4 + 3 * 8 and C.sizeof(rt.QBlockArgs) == 8 * 4 + 4 * 8 + 6 * 4 + 4 + 8 + 2 * 4
     assert C.sizeof(rt.PagedAttnArgs) == 10 * 4

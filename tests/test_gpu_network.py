@@ -13,8 +13,8 @@ pytestmark = pytest.mark.gpu
 f32 = np.float32
 
 
-def check_model(hip_ctx, qg, x, capture, fuse_residual=True):
-    model = nb.HipModel(hip_ctx, qg, x.shape[0], capture_graph=capture, fuse_residual=fuse_residual)
+def check_model(hip_ctx, qg, x, capture, fuse_residual=True, fuse_blocks=True):
+    model = nb.HipModel(hip_ctx, qg, x.shape[0], capture_graph=capture, fuse_residual=fuse_residual, fuse_blocks=fuse_blocks)
     y = model.run(x)
     want, outs = netref.run_integer(qg, x, keep_all=True)
     for i, ref in enumerate(outs):
@@ -54,8 +54,10 @@ def test_mobilenetv2_config3(hip_ctx):
     x = rng.random((2, 224, 224, 3), dtype=f32)
     plain, _, _ = check_model(hip_ctx, qg, x, capture=False, fuse_residual=False)   # every tensor, add as its own kernel
     assert len(plain.fused_into) == 0 and len(plain.fn) == 66
-    model, y, outs = check_model(hip_ctx, qg, x, capture=True)
+    model, y, outs = check_model(hip_ctx, qg, x, capture=True, fuse_blocks=False)
     assert len(model.fused_into) == 10 and len(model.fn) == 56                        # residual adds folded into the convs
+    model, y, outs = check_model(hip_ctx, qg, x, capture=True)
+    assert len(model.blocks) == 16 and len(model.fn) == 24                            # ... and whole blocks into one operator
     # the reference's own acceptance bar for a PTQ model: cosine >= 0.98 against the float model
     fl = nb.float_forward(g, x)[-1]
     assert O.cosine(y, fl) > 0.98
@@ -174,6 +176,9 @@ def test_profile_and_kernel_names(hip_ctx):
     assert all(n.startswith("qconv_igemm<T=") and n.endswith(",rows16>") for n in (names[1], names[3]))
     ms = model.fn.profile(3)
     assert len(ms) == 5 and all(0 < t < 50 for t in ms)
+    fused = nb.HipModel(hip_ctx, qg, 2, capture_graph=False, fuse_blocks=True)
+    assert [fused.fn.op_kernel(i) for i in range(len(fused.fn))] == ["quantize", "qblock<S=1,P=4,E=3>", "dequantize"]
+    assert fused.op_members == [[0], [1, 2, 3], []]
 
 
 @pytest.mark.parametrize("lanes,capture", [(2, True), (4, True), (2, False)])
@@ -229,3 +234,28 @@ def test_lanes_argument_checks(hip_ctx):
         fn.set_lane(8)
     with pytest.raises(HipError):
         fn.set_lane(-1)
+
+
+def test_mobilenetv2_fused_blocks_match_separate_operators(hip_ctx):
+    """All 16 expand -> depthwise -> project blocks as single fused operators: every tensor that still reaches
+    HBM equals the one the operator-per-convolution function writes, and the oracle's logits for image 0."""
+    g = nb.mobilenet_v2(seed=2)
+    rng = np.random.default_rng(3)
+    qg = nb.quantize_graph(g, rng.random((32, 224, 224, 3), dtype=f32))
+    x = np.random.default_rng(4).random((8, 224, 224, 3), dtype=f32)
+    plain = nb.HipModel(hip_ctx, qg, 8, capture_graph=False)
+    y0 = plain.run(x)
+    for capture, lanes in ((False, 1), (True, 1), (True, 2)):
+        fused = nb.HipModel(hip_ctx, qg, 8, capture_graph=capture, lanes=lanes, fuse_blocks=True)
+        assert len(fused.blocks) == 16 and len(fused.fn) == lanes * (len(plain.fn) - 32)
+        y = fused.run(x)
+        assert np.array_equal(y.view(np.uint32), y0.view(np.uint32))
+        for i in range(len(qg.nodes)):
+            if fused.materialized(i):
+                a, b = plain.tensor(i), fused.tensor(i)
+                assert np.array_equal(a, b), f"node {i} ({qg.nodes[i].name}): {(a != b).sum()} bytes differ"
+        for e, (d, _, _) in fused.blocks.items():
+            assert not fused.materialized(e) and not fused.materialized(d)
+    want = netref.run_integer(qg, x[:1])
+    want = want[0] if isinstance(want, tuple) else want
+    assert np.array_equal(y0[:1].view(np.uint32), np.asarray(want).view(np.uint32))
