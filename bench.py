@@ -31,59 +31,68 @@ INT8_PEAK_TOPS = 5000.0    # dense int8 MFMA
 
 
 # Bytes that crossed the L2 <-> fabric boundary per launch (average over the launches of a kernel in
-# one step) at the headline workload, from two rocprofv3 --pmc runs of this script (FETCH_SIZE, then
-# WRITE_SIZE, each scaled by what the same counter reads for the 256 MiB copy that --copy-probe
-# launches: x1.9997 and x1.0000).  Counters cannot be read from inside a timed run, so the figures
+# one step) at the headline workload with whole-batch launches (--lanes 1), from two rocprofv3 --pmc runs
+# of this script (FETCH_SIZE, then WRITE_SIZE, each scaled by what the same counter reads for the 256 MiB
+# copy that --copy-probe launches: x1.9996 and x1.0000).  Counters cannot be read from inside a timed run, so the figures
 # are recorded here and reported only for the configuration they were measured on.
 MEASURED_TRAFFIC_B64 = {
-    "dequantize": 354803,
-    "dw3x3<S=1>": 19398340,
-    "dw3x3<S=2>": 41830103,
-    "qconv_igemm<T=1,RG=1,rows16>": 6041031,
-    "qconv_igemm<T=1,RG=4,rows16>": 38694361,
-    "qconv_igemm<T=12,RG=1,rows16>": 10391442,
-    "qconv_igemm<T=2,RG=1,rows16>": 10279565,
-    "qconv_igemm<T=2,RG=2,rows16>": 31506435,
-    "qconv_igemm<T=5,RG=1,rows16>": 5171008,
-    "qconv_igemm<T=6,RG=1,rows16>": 8668773,
-    "qconv_igemm<T=6,RG=2,rows16>": 90218140,
-    "qconv_igemm<T=8,RG=1,rows16>": 6011810,
-    "qconv_igemm<T=9,RG=1,vec8>": 33995909,
-    "qconv_smallc<C=3>": 38855552,
-    "qglobal_avgpool": 4122090,
-    "quantize": 48214802,
+    "dequantize": 354798,
+    "dw3x3<S=1>": 27522691,
+    "dw3x3<S=2>": 48854305,
+    "qblock+add<S=1,P=2>": 4926577,
+    "qblock+add<S=1,P=4>": 2721834,
+    "qblock+add<S=1,P=6>": 4578727,
+    "qblock<S=1,P=6>": 3270288,
+    "qblock<S=2,P=4>": 3331646,
+    "qconv_igemm+add<T=1,RG=1,rows16>": 5324965,
+    "qconv_igemm+add<T=2,RG=2,rows16>": 38719725,
+    "qconv_igemm<T=1,RG=1,rows16>": 6754731,
+    "qconv_igemm<T=1,RG=4,rows16>": 38690311,
+    "qconv_igemm<T=12,RG=1,rows16>": 9243161,
+    "qconv_igemm<T=2,RG=1,rows16>": 8973024,
+    "qconv_igemm<T=2,RG=2,rows16>": 24238335,
+    "qconv_igemm<T=5,RG=1,rows16>": 5183656,
+    "qconv_igemm<T=6,RG=1,rows16>": 8669379,
+    "qconv_igemm<T=6,RG=2,rows16>": 90223962,
+    "qconv_igemm<T=9,RG=1,vec8>": 33999476,
+    "qconv_smallc<C=3>": 38859992,
+    "qglobal_avgpool": 4121905,
+    "quantize": 48219051,
 }
 
 
 def op_accounting(qg, batch, model):
-    """Per operator of the recorded function (one lane): the bytes an ideal implementation must move
-    (read every tensor that enters the operator once, write its result once, read the constants once)
-    and its multiply-adds.  An operator may cover several graph nodes (a conv with a table and a residual
-    add in its epilogue; a whole expand -> depthwise -> project block): tensors between those nodes never
-    reach HBM and do not count."""
+    """Per operator of the recorded function (one lane): (bytes, floor_bytes, macs).
+    bytes is the algorithmic traffic of the graph nodes the operator computes, each counted as the
+    operator of its own the reference runs: every node reads its inputs once, writes its output once and
+    reads its constants once (a convolution with a table and a residual add in its epilogue, or a whole
+    expand -> depthwise -> project block, is several such nodes).  floor_bytes is what the fused operator
+    itself cannot avoid: the tensors that enter it, its result, its constants."""
     size = lambda j: batch * int(np.prod(qg.nodes[j].out_shape))
-    nbytes, macs = [], []
-    for name, members in zip(model.op_names, model.op_members):
+    nbytes, floors, macs = [], [], []
+    for k, (name, members) in enumerate(zip(model.op_names, model.op_members)):
         if name.startswith("dequantize"):
-            o = size(model.op_nodes[len(nbytes)])
+            o = size(model.op_nodes[k])
             nbytes.append(o + 4 * o)
+            floors.append(o + 4 * o)
             macs.append(0)
             continue
         inside = set(members)
         external = {j for m in members for j in qg.nodes[m].inputs if j not in inside}
-        b = sum(size(j) for j in external) + size(members[-1])
-        m = 0
+        consts = b = m = 0
         for j in members:
             n = qg.nodes[j]
+            b += sum(size(i) for i in n.inputs) + size(j)
             if n.op == "input":
-                b += 4 * size(j)
+                consts += 4 * size(j)            # the float32 tensor the quantize operator reads
             elif n.op == "conv":
                 oc, gic, kh, kw = n.weights.shape
-                b += n.weights.size + 4 * n.bias.size
+                consts += n.weights.size + 4 * n.bias.size
                 m += batch * oc * n.out_shape[1] * n.out_shape[2] * gic * kh * kw
-        nbytes.append(b)
+        nbytes.append(b + consts)
+        floors.append(sum(size(j) for j in external) + size(members[-1]) + consts)
         macs.append(m)
-    return nbytes, macs
+    return nbytes, floors, macs
 
 
 def time_calls(ctx, fn, warmup, steps):
@@ -249,12 +258,14 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--batch", type=int, default=64)
-    ap.add_argument("--lanes", type=int, default=1,
+    ap.add_argument("--lanes", type=int, default=2,
                     help="independent chains the batch is split into and replayed concurrently (1 = one chain of "
                          "full-batch launches); results are bit-identical for every value")
     ap.add_argument("--cpu-images", type=int, default=8, help="batch-1 images timed on the CPU baseline (0 = skip)")
     ap.add_argument("--profile-iters", type=int, default=10)
     ap.add_argument("--batch1-steps", type=int, default=200, help="timed batch-1 invocations (0 = skip the batch-1 figure)")
+    ap.add_argument("--no-fuse-blocks", action="store_true",
+                    help="run every expand -> depthwise -> project block as three operators")
     ap.add_argument("--no-graph", action="store_true",
                     help="enqueue the operators one by one instead of replaying the HIP graph (used under rocprofv3 "
                          "--kernel-trace, whose tracer crashes inside hipGraphLaunch on this image)")
@@ -286,7 +297,7 @@ def main():
     qg = nb.quantize_graph(graph, calib)
     x = np.random.default_rng(4).random((args.batch, 224, 224, 3), dtype=np.float32)
 
-    model = nb.HipModel(ctx, qg, args.batch, capture_graph=not args.no_graph, lanes=args.lanes)
+    model = nb.HipModel(ctx, qg, args.batch, capture_graph=not args.no_graph, lanes=args.lanes, fuse_blocks=not args.no_fuse_blocks)
     model.set_input(x)  # resident in HBM before the timed region
     for _ in range(args.warmup):
         model.invoke()
@@ -300,17 +311,28 @@ def main():
     images_per_s = args.batch / (dt / args.steps)
 
     # ---- per-kernel device time (HIP events on the context's stream) --------------------------
-    op_ms = model.fn.profile(args.profile_iters)
-    names = [model.fn.op_kernel(i) for i in range(len(model.fn))]
+    # Kernels of concurrently replayed chains overlap and have no duration of their own, so the per-kernel figures
+    # are taken on the one-chain recording of the same operators (every launch then covers the whole batch).
+    kmodel = model if args.lanes == 1 else nb.HipModel(ctx, qg, args.batch, capture_graph=False, lanes=1,
+                                                        fuse_blocks=not args.no_fuse_blocks)
+    if kmodel is not model:
+        kmodel.set_input(x)
+        kmodel.invoke()
+        ctx.sync()
+        if not np.array_equal(kmodel.output().view(np.uint32), model.output().view(np.uint32)):
+            sys.exit("bench.py: the one-chain and the %d-chain function disagree" % args.lanes)
+    op_ms = kmodel.fn.profile(args.profile_iters)
+    names = [kmodel.fn.op_kernel(i) for i in range(len(kmodel.fn))]
     # every lane launches the whole operator list on its batch/lanes images (and reads the weights itself)
     lane_batch = args.batch // args.lanes
-    abytes, macs = (v * args.lanes for v in op_accounting(qg, lane_batch, model))
+    abytes, fbytes, macs = op_accounting(qg, args.batch, kmodel)
     assert len(abytes) == len(macs) == len(names) == len(op_ms)
     groups = {}
-    for name, ms, b, m in zip(names, op_ms, abytes, macs):
-        g = groups.setdefault(name, {"ms": 0.0, "bytes": 0, "macs": 0, "launches": 0})
+    for name, ms, b, fb, m in zip(names, op_ms, abytes, fbytes, macs):
+        g = groups.setdefault(name, {"ms": 0.0, "bytes": 0, "floor": 0, "macs": 0, "launches": 0})
         g["ms"] += ms
         g["bytes"] += b
+        g["floor"] += fb
         g["macs"] += m
         g["launches"] += 1
     dom_name, dom = max(groups.items(), key=lambda kv: kv[1]["ms"])
@@ -382,16 +404,18 @@ def main():
         "dtype": "u8",
         "data": "synthetic",
         "config": {"workload": f"MobileNetV2 w1.0 224x224 u8/u8 per-tensor PTQ (32 calibration images), batch {args.batch}, "
-                               "NHWC f32 input resident in HBM -> quantize -> 52 convs + 10 adds + pool + FC -> dequantize",
+                               "NHWC f32 input resident in HBM -> quantize -> 52 convs + 10 adds + pool + FC -> dequantize" +
+                               (f"; {len(model.blocks)} expand/depthwise/project blocks fused into one kernel each" if model.blocks else ""),
                    "batch": args.batch, "lanes": args.lanes, "ops_per_step": len(model.fn),
                    "execution": "resident hip function, " + ("eager launches" if args.no_graph else "HIP-graph replay") +
                                 (f", {args.lanes} concurrent chains of {lane_batch} images" if args.lanes > 1 and not args.no_graph else "")},
         "roofline": {"bound": "hbm", "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(dom_gbs / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC_B64.get(dom_name) if (args.batch, args.lanes) == (64, 1) else None, "kernel": dom_name,
-                     "images_per_launch": lane_batch,
+                     "traffic": MEASURED_TRAFFIC_B64.get(dom_name) if args.batch == 64 and not args.no_fuse_blocks else None,
+                     "kernel": dom_name, "images_per_launch": args.batch,
                      "launches_per_step": dom["launches"], "avg_launch_us": round(dom["ms"] / dom["launches"] * 1e3, 2),
                      "algorithmic_bytes_per_launch": int(dom["bytes"] / dom["launches"]),
+                     "fused_floor_bytes_per_launch": int(dom["floor"] / dom["launches"]),
                      "share_of_device_time": round(dom["ms"] / sum(op_ms), 4)},
         "cpu_baseline": cpu,
         "int8_TOPS_whole_net": round(2 * total_macs / (ms_per_step * 1e-3) / 1e12, 2),
@@ -400,6 +424,7 @@ def main():
         "kernel_classes": class_report,
         "kernels": {k: {"ms": round(v["ms"], 4), "launches": v["launches"],
                         "hbm_GBps": round(v["bytes"] / (v["ms"] * 1e-3) / 1e9, 1)} for k, v in sorted(groups.items())},
+        "operators": [{"kernel": n, "us": round(t * 1e3, 2)} for n, t in zip(names, op_ms)],
         "batch1": b1,
         "device": {"compute_units": ctx.compute_units, "clock_mhz": ctx.clock_khz / 1000.0},
     }

@@ -1,25 +1,32 @@
 // Fused inverted-residual block: 1x1 expansion -> 3x3 depthwise -> 1x1 projection (+ input),
 // u8/u8, NHWC, one kernel.  The two expanded tensors are the largest of the block (6x the
 // input) and, run as three operators, are each written to and read back from HBM; here a
-// workgroup owns a 7x7 tile of OUTPUT pixels of one image and keeps everything between the
-// block's input and output in LDS:
+// workgroup (8 waves) owns a 7x7 tile of OUTPUT pixels of one image and keeps everything
+// between the block's input and output in LDS:
 //
 //   input tile   the in-image part of the (6S+3)^2 input pixels the tile needs, as s8
-//   per chunk of 48 or 64 expanded channels (weights of the next chunk are prefetched
-//   global -> registers while this one is computed, then committed to the other LDS buffer):
+//   per chunk of 64 expanded channels:
 //     E  expansion on the matrix cores for every in-image pixel of the halo, requantised to
-//        u8 into the expansion tile (positions outside the image keep the zero point the
-//        tile was initialised with: they are the depthwise stage's padding)
-//     D  depthwise 3x3 from the expansion tile (16-bit multiply-adds, 4 channels per lane),
-//        requantised to u8 and stored as s8 in the depthwise tile
+//        u8 (kept as s8) into the expansion tile; positions outside the image keep the zero
+//        point the tile was initialised with: they are the depthwise stage's padding
+//     D  depthwise 3x3 on the matrix cores as well: the reduction index is (tap, channel) and
+//        the weight operand is zero off its own channel; requantised into the depthwise tile
 //     P  projection: the depthwise tile is one k-step of the matrix-core reduction over the
 //        expanded channels, accumulated in registers across the chunks
 //   epilogue of P: zero points, requantisation, optional residual add, NHWC store.
 //
+// The stages are software-pipelined over the chunks: between two barriers a workgroup runs
+// E of chunk r, D of chunk r - 1 and P of chunk r - 2 on double-buffered tiles, and the
+// constants of the next step are prefetched global -> registers and committed to the other
+// half of a double-buffered LDS area at the end of the step.
+//
 // Every stage uses the arithmetic of the stand-alone kernels (same zero-point identity, same
 // fp32 requantisation sequence), so the output bytes equal those of three separate operators.
 // Tiles need a one-pixel halo of the expansion around them (recomputed per tile: 81 pixels
-// for 49 at stride 1, 225 input pixels for 49 outputs at stride 2).
+// for 49 at stride 1, 225 input pixels for 49 outputs at stride 2).  What bounds the kernel is
+// the requantisation arithmetic on the vector ALU (two u8 tensors are requantised that never
+// leave the compute unit), not memory: it pays on mid-sized feature maps, where the separate
+// operators are latency-bound launches.
 #include "qconv_igemm.hpp"
 
 #include <algorithm>
@@ -29,7 +36,7 @@
 struct nncase_hip_qblock_weights {
     int cin = 0, mid = 0, cout = 0;
     int ke = 0;      // k-steps of the expansion (ceil(cin / 64))
-    int et = 0;      // 16-channel tiles per chunk of expanded channels (3 or 4)
+    int et = 0;      // 16-channel tiles per chunk of expanded channels
     int tpt = 0;     // 16-channel tiles of the projection's output held by every wave
     int nchunks = 0, chunk_bytes = 0;
     int off_p = 0, off_wd = 0, off_bd = 0, off_sd = 0, off_be = 0, off_se = 0; // byte offsets inside a chunk
@@ -42,7 +49,8 @@ struct nncase_hip_qblock_weights {
 
 namespace nnhip {
 
-constexpr int kBlkThreads = 256;
+constexpr int kBlkWaves = 8;
+constexpr int kBlkThreads = kBlkWaves * 64;
 constexpr int kBlkTile = 7;  // output tile edge (divides every MobileNet resolution from 112 down to 7)
 constexpr int kBlkRowB = 80; // bytes per pixel of the two mid tiles: 64 channels + 16 so that rows spread over the banks
 
@@ -54,33 +62,48 @@ struct BlockArgs {
     int xs; // bytes per pixel of the input tile (ke * 64 + 16)
     int in_h, in_w, out_h, out_w, pad_h, pad_w, tiles_y, tiles_x;
     int zxp_e, zwp_e, kzz_e; // expansion: zx - 128, zw - 128, cin * zxp * zwp
-    int zx_d;                // zero point of the expansion's output
-    uint32_t zmid_splat;
+    int zxp_d, zwp_d, kzz_d; // depthwise: zx - 128, zw - 128, 9 * zxp * zwp
+    uint32_t zmid_splat;     // zero point of the expansion's output as s8, in all four bytes
     Epilogue ep_e, ep_d;
     int off_p, off_wd, off_bd, off_sd, off_be, off_se;
-    int lds_xin, lds_et, lds_dt, lds_w;
+    int lds_pix, lds_xin, lds_et, lds_dt, lds_w;
     IgemmArgs p; // projection stage: y, m, n, k, ldy, zxp, zwp, wsum, bias, ep, rep
 };
 
-template <int S, int TPT, int ET>
+// What the expansion needs to know about one in-image halo pixel: where its row of the expansion tile
+// starts and the zero-point term of its sum of inputs.
+struct HaloPix {
+    int32_t tile_off; // byte offset of the pixel's row in the expansion tile
+    int32_t nrsz;     // cin * zx' * zw' - zw' * sum_k x'
+};
+
+template <int S, int TPT>
 __global__ __launch_bounds__(kBlkThreads) void qblock_kernel(const BlockArgs a) {
+    constexpr int ET = 4;                      // 16-channel tiles per chunk of expanded channels
     constexpr int HH = (kBlkTile - 1) * S + 3; // halo edge in input pixels
     constexpr int HP = HH * HH;
     constexpr int TP = kBlkTile * kBlkTile;
-    constexpr int CE = ET * 16, QUADS = ET * 4, PSTEP = kBlkThreads / QUADS;
-    constexpr int NS = (3 * ET * 1024 + TPT * 1024 + 9 * CE * 2 + 16 * CE + 4095) / 4096; // 16-byte vectors staged per thread
+    constexpr int CE = ET * 16;
+    constexpr int NG = (HP + 15) / 16;                        // pixel groups of the halo at most
+    constexpr int MAXU = (NG + 1) / 2;                        // expansion units (16 pixels x 16 channels) per wave at most
+    constexpr int NS = (3 * ET * 1024 + TPT * 1024 + 9 * CE + 16 * CE + 16 * kBlkThreads - 1) / (16 * kBlkThreads); // vectors staged per thread
+    constexpr int TPW = TPT / 2; // projection tiles per wave: waves w and w + 4 share a pixel group
+    static_assert(TPT % 2 == 0 && kBlkWaves == 8, "two waves per pixel group, four channel tiles per chunk");
 
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    int32_t *cterm_p = reinterpret_cast<int32_t *>(smem); // [TPT * 16]
-    uint8_t *xin = smem + a.lds_xin;                     // [groups * 16][xs] s8
-    uint8_t *etile = smem + a.lds_et;                    // [HP][kBlkRowB] u8
-    uint8_t *dtile = smem + a.lds_dt;                    // [64][kBlkRowB] s8
-    uint8_t *wbuf = smem + a.lds_w;                      // [2][chunk_bytes]
+    int32_t *cterm_p = reinterpret_cast<int32_t *>(smem);             // [TPT * 16]
+    HaloPix *hpix = reinterpret_cast<HaloPix *>(smem + a.lds_pix);   // [groups * 16]
+    uint8_t *xin = smem + a.lds_xin;                                 // [groups * 16][xs] s8
+    uint8_t *etile = smem + a.lds_et;                                // [2][HP][kBlkRowB] s8
+    uint8_t *dtile = smem + a.lds_dt;                                // [2][64][kBlkRowB] s8
+    uint8_t *wbuf = smem + a.lds_w;                                  // [2][chunk_bytes]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int j = lane & 15, gq = lane >> 4;
+    // Every stage gives a wave one 16-channel tile (wave & 3) of half of the pixel groups (wave >> 2).
+    const int wtile = wave & 3, whalf = wave >> 2;
 
     uint32_t b = blockIdx.x;
     const int tx = (int)(b % (uint32_t)a.tiles_x);
@@ -97,48 +120,137 @@ __global__ __launch_bounds__(kBlkThreads) void qblock_kernel(const BlockArgs a) 
     const int offy = cy0 - iy0, offx = cx0 - ix0;
     const uint32_t rcw = 65536u / (uint32_t)CW + 1u; // idx / CW = (idx * rcw) >> 16 for idx < 256
     const int ngroups = (cnt + 15) >> 4;
+    const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
 
     // ---- one-time fills ---------------------------------------------------------------------------
+    // Every global load of the set-up (input tile, constants, first chunk of weights) is issued before
+    // anything waits for one of them: a dependent load -> store pair per loop trip would expose a full
+    // memory round trip each time.
+    const int nvec = a.chunk_bytes / 16;
     {
-        const u32x4 z = {a.zmid_splat, a.zmid_splat, a.zmid_splat, a.zmid_splat};
-        for (int i = tid; i < HP * (kBlkRowB / 16); i += kBlkThreads) reinterpret_cast<u32x4 *>(etile)[i] = z;
-        const u32x4 zero = {0, 0, 0, 0};
-        for (int i = tid; i < 64 * (kBlkRowB / 16); i += kBlkThreads) reinterpret_cast<u32x4 *>(dtile)[i] = zero;
-        for (int i = tid; i < TPT * 16; i += kBlkThreads) {
-            int32_t c = 0;
-            if (i < a.p.n) c = a.p.bias[i] - a.p.zxp * a.p.wsum[i] + a.p.k * a.p.zxp * a.p.zwp;
-            cterm_p[i] = c;
-        }
-        // input tile: 16 lanes copy one pixel's channels a dword each, re-biased to s8, zero past the channels
+        constexpr int NPI = (NG * 16 + kBlkThreads / 16 - 1) / (kBlkThreads / 16); // pixels per thread
         const int ps = tid >> 4, dl = tid & 15;
-        for (int idx = ps; idx < ngroups * 16; idx += kBlkThreads / 16) {
+        uint32_t xv[NPI][3];
+#pragma unroll
+        for (int it = 0; it < NPI; it++) {
+            const int idx = ps + it * (kBlkThreads / 16);
             const int cy = (int)(((uint32_t)idx * rcw) >> 16), cx = idx - cy * CW;
             const bool pix = idx < cnt;
             const uint32_t src = (uint32_t)((img * a.in_h + cy0 + (pix ? cy : 0)) * a.in_w + cx0 + (pix ? cx : 0)) * (uint32_t)a.cin;
-            for (int s = 0; s < a.ke; s++) {
+#pragma unroll
+            for (int s = 0; s < 3; s++) {
                 const int d = s * 16 + dl;
-                uint32_t v = 0;
-                if (pix && d * 4 < a.cin) v = *reinterpret_cast<const uint32_t *>(a.x + src + d * 4) ^ 0x80808080u;
-                *reinterpret_cast<uint32_t *>(xin + idx * a.xs + d * 4) = v;
+                xv[it][s] = 0x80808080u;
+                if (s < a.ke && pix && d * 4 < a.cin) xv[it][s] = *reinterpret_cast<const uint32_t *>(a.x + src + d * 4);
             }
         }
-        const u32x4 *src = reinterpret_cast<const u32x4 *>(a.blob);
-        for (int i = tid; i < a.chunk_bytes / 16; i += kBlkThreads) reinterpret_cast<u32x4 *>(wbuf)[i] = src[i];
+        u32x4 w0[NS];
+        {
+            const u32x4 *src = reinterpret_cast<const u32x4 *>(a.blob);
+#pragma unroll
+            for (int i = 0; i < NS; i++) {
+                const int v = i * kBlkThreads + tid;
+                w0[i] = src[v < nvec ? v : 0];
+            }
+        }
+        int32_t cb = 0, cs = 0;
+        if (tid < a.p.n) cb = a.p.bias[tid], cs = a.p.wsum[tid];
+
+        const u32x4 z = {a.zmid_splat, a.zmid_splat, a.zmid_splat, a.zmid_splat};
+        for (int i = tid; i < 2 * HP * (kBlkRowB / 16); i += kBlkThreads) reinterpret_cast<u32x4 *>(etile)[i] = z;
+        const u32x4 zero = {0, 0, 0, 0};
+        for (int i = tid; i < 2 * 64 * (kBlkRowB / 16); i += kBlkThreads) reinterpret_cast<u32x4 *>(dtile)[i] = zero;
+
+        if (tid < TPT * 16) cterm_p[tid] = tid < a.p.n ? cb - a.p.zxp * cs + a.p.k * a.p.zxp * a.p.zwp : 0;
+        // input tile: 16 lanes hold one pixel's channels a dword each; re-biased to s8, zero past the channels
+#pragma unroll
+        for (int it = 0; it < NPI; it++) {
+            const int idx = ps + it * (kBlkThreads / 16);
+            if (idx < ngroups * 16) {
+#pragma unroll
+                for (int s = 0; s < 3; s++)
+                    if (s < a.ke) *reinterpret_cast<uint32_t *>(xin + idx * a.xs + (s * 16 + dl) * 4) = xv[it][s] ^ 0x80808080u;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < NS; i++) {
+            const int v = i * kBlkThreads + tid;
+            if (v < nvec) reinterpret_cast<u32x4 *>(wbuf)[v] = w0[i];
+        }
+    }
+    __syncthreads();
+    // per halo pixel: row offset in the expansion tile and the zero-point term of its input sum
+    for (int g = wave; g < ngroups; g += kBlkWaves) {
+        const int idx = g * 16 + j;
+        v4i rs = {0, 0, 0, 0};
+        for (int ks = 0; ks < a.ke; ks++) {
+            const v4i xf = *reinterpret_cast<const v4i *>(xin + idx * a.xs + ks * 64 + gq * 16);
+            rs = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, xf, rs, 0, 0, 0);
+        }
+        if (gq == 0) {
+            const int cy = (int)(((uint32_t)idx * rcw) >> 16), cx = idx - cy * CW;
+            HaloPix hp;
+            hp.tile_off = idx < cnt ? ((cy + offy) * HH + cx + offx) * kBlkRowB : -1;
+            hp.nrsz = a.kzz_e - a.zwp_e * rs[0];
+            hpix[idx] = hp;
+        }
     }
     __syncthreads();
 
-    const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
-    v4i accp[TPT];
+    // ---- what stays the same for every chunk -------------------------------------------------------------------
+    // E: the wave's units are pixel groups whalf, whalf + 2, ... of channel tile wtile
+    HaloPix ehp[MAXU];
+#pragma unroll
+    for (int k = 0; k < MAXU; k++) {
+        const int g = whalf + 2 * k;
+        ehp[k] = hpix[min(g, NG - 1) * 16 + j];
+        if (g >= ngroups) ehp[k].tile_off = -1;
+    }
+    const uint8_t *exrow = xin + (whalf * 16 + j) * a.xs + gq * 16; // + k * 32 * xs + ks * 64
+    const int ecl = gq * (4 * ET) + wtile * 4;                        // the lane's 4 channels within the chunk
+    // D: pixel groups whalf and whalf + 2 of channel tile wtile; the lane's tap in k-step ks is ks * 4 + gq
+    int dxoff[2], dtap[3];
+    bool dpv[2];
+#pragma unroll
+    for (int k = 0; k < 2; k++) {
+        const int pp = (whalf + 2 * k) * 16 + j;
+        dpv[k] = pp < TP;
+        const int p = min(pp, TP - 1);
+        const int py = p / kBlkTile, px = p - py * kBlkTile;
+        dxoff[k] = ((py * S) * HH + px * S) * kBlkRowB + wtile * 16;
+    }
+#pragma unroll
+    for (int ks = 0; ks < 3; ks++) {
+        const int t = ks * 4 + gq;
+        const int tt = t < 9 ? t : 0;
+        const int ky = tt / 3, kx = tt - ky * 3;
+        dtap[ks] = (ky * HH + kx) * kBlkRowB;
+    }
+    // byte j of the 16-byte k-chunk belongs to channel j of the tile: a mask for the weight, a one for the window sum
+    u32x4 dmask, done;
+#pragma unroll
+    for (int d = 0; d < 4; d++) {
+        dmask[d] = (j >> 2) == d ? 0xffu << (8 * (j & 3)) : 0u;
+        done[d] = dmask[d] & 0x01010101u;
+    }
+    const v4i done_f = __builtin_bit_cast(v4i, done);
+    const v4i done_last = gq == 0 ? done_f : v4i{0, 0, 0, 0}; // k-step 2 only holds tap 8
+    const int dcl = wtile * 16 + gq * 4; // the lane's 4 channels within the chunk
+
+    v4i accp[TPW];
     v4i rsp = {0, 0, 0, 0};
 #pragma unroll
-    for (int nt = 0; nt < TPT; nt++) accp[nt] = v4i{0, 0, 0, 0};
+    for (int nt = 0; nt < TPW; nt++) accp[nt] = v4i{0, 0, 0, 0};
 
-    const int nvec = a.chunk_bytes / 16;
-    for (int c = 0; c < a.nchunks; c++) {
-        const uint8_t *wb = wbuf + (c & 1) * a.chunk_bytes;
+    // Record r of the constants holds the expansion weights of chunk r, the depthwise weights of chunk r - 1 and
+    // the projection weights of chunk r - 2: phase r runs E(r), D(r - 1) and P(r - 2) between two barriers, on
+    // double-buffered tiles, so the three stages of different chunks overlap inside the workgroup.
+    const int nrec = a.nchunks + 2;
+    for (int r = 0; r < nrec; r++) {
+        const uint8_t *wb = wbuf + (r & 1) * a.chunk_bytes;
         u32x4 stage[NS];
-        if (c + 1 < a.nchunks) {
-            const u32x4 *src = reinterpret_cast<const u32x4 *>(a.blob + (size_t)(c + 1) * a.chunk_bytes);
+        if (r + 1 < nrec) {
+            const u32x4 *src = reinterpret_cast<const u32x4 *>(a.blob + (size_t)(r + 1) * a.chunk_bytes);
 #pragma unroll
             for (int i = 0; i < NS; i++) {
                 const int v = i * kBlkThreads + tid;
@@ -146,92 +258,99 @@ __global__ __launch_bounds__(kBlkThreads) void qblock_kernel(const BlockArgs a) 
             }
         }
 
-        // ---- E: expansion of every in-image halo pixel, 16 pixels x 16 channels per unit -------------
-        for (int u = wave; u < ngroups * ET; u += kWaves) {
-            const int g = u / ET, nt = u - g * ET;
-            const int idx = g * 16 + j;
-            const uint8_t *xrow = xin + idx * a.xs + gq * 16;
-            const uint8_t *wfr = wb + nt * 1024 + lane * 16;
-            v4i acc = {0, 0, 0, 0}, rs = {0, 0, 0, 0};
-            for (int ks = 0; ks < a.ke; ks++) {
-                const v4i xf = *reinterpret_cast<const v4i *>(xrow + ks * 64);
-                const v4i wf = *reinterpret_cast<const v4i *>(wfr + ks * ET * 1024);
-                rs = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, xf, rs, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf, xf, acc, 0, 0, 0);
-            }
-            if (idx < cnt) {
-                const int cy = (int)(((uint32_t)idx * rcw) >> 16), cx = idx - cy * CW;
-                const int pos = (cy + offy) * HH + cx + offx;
-                const int cl = gq * (4 * ET) + nt * 4; // first of the lane's 4 channels within the chunk
-                const v4i be = *reinterpret_cast<const v4i *>(wb + a.off_be + cl * 4);
-                const v4i se = *reinterpret_cast<const v4i *>(wb + a.off_se + cl * 4);
-                const int32_t nrsz = a.kzz_e - a.zwp_e * rs[0];
-                uint32_t q[4];
-#pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    const int32_t v = add3(acc[r], be[r] - a.zxp_e * se[r], nrsz);
-                    q[r] = requant_u8_lowbyte((float)v * a.ep_e.mult, a.ep_e);
-                }
-                *reinterpret_cast<uint32_t *>(etile + pos * kBlkRowB + cl) = pack_low_bytes(q[0], q[1], q[2], q[3]);
-            }
-        }
-        __syncthreads();
-
-        // ---- D: depthwise 3x3 on the expansion tile, 4 channels x 1 pixel per item ------------------------
-        if (tid < PSTEP * QUADS) {
-            const int qd = tid % QUADS, p0 = tid / QUADS;
-            uint32_t w01[9], w23[9];
-#pragma unroll
-            for (int t = 0; t < 9; t++) {
-                const u32x2 raw = *reinterpret_cast<const u32x2 *>(wb + a.off_wd + (t * CE + qd * 4) * 2);
-                w01[t] = raw[0];
-                w23[t] = raw[1];
-            }
-            const v4i bd = *reinterpret_cast<const v4i *>(wb + a.off_bd + qd * 16);
-            const v4i sd = *reinterpret_cast<const v4i *>(wb + a.off_sd + qd * 16);
-            int32_t ct[4];
-#pragma unroll
-            for (int r = 0; r < 4; r++) ct[r] = bd[r] - a.zx_d * sd[r];
-            const bool chv = c * CE + qd * 4 < a.mid;
-            for (int p = p0; p < TP; p += PSTEP) {
-                const int py = p / kBlkTile, px = p - py * kBlkTile;
-                const uint8_t *base = etile + ((py * S) * HH + px * S) * kBlkRowB + qd * 4;
-                int32_t acc[4] = {ct[0], ct[1], ct[2], ct[3]};
-#pragma unroll
-                for (int ky = 0; ky < 3; ky++)
-#pragma unroll
-                    for (int kx = 0; kx < 3; kx++) {
-                        const uint32_t d = *reinterpret_cast<const uint32_t *>(base + (ky * HH + kx) * kBlkRowB);
-                        const uint32_t x01 = __builtin_amdgcn_perm(0u, d, 0x0c010c00u);
-                        const uint32_t x23 = __builtin_amdgcn_perm(0u, d, 0x0c030c02u);
-                        const int t = ky * 3 + kx;
-                        acc[0] = mad16_lo(x01, w01[t], acc[0]);
-                        acc[1] = mad16_hi(x01, w01[t], acc[1]);
-                        acc[2] = mad16_lo(x23, w23[t], acc[2]);
-                        acc[3] = mad16_hi(x23, w23[t], acc[3]);
-                    }
-                uint32_t q[4];
-#pragma unroll
-                for (int r = 0; r < 4; r++) q[r] = requant_u8_lowbyte((float)acc[r] * a.ep_d.mult, a.ep_d);
-                const uint32_t packed = pack_low_bytes(q[0], q[1], q[2], q[3]) ^ 0x80808080u; // kept as s8
-                *reinterpret_cast<uint32_t *>(dtile + p * kBlkRowB + qd * 4) = chv ? packed : 0u;
-            }
-        }
-        __syncthreads();
-
-        // ---- P: this chunk is one k-step of the projection ----------------------------------------------------
-        {
-            const v4i xf = *reinterpret_cast<const v4i *>(dtile + (wave * 16 + j) * kBlkRowB + gq * 16);
+        // ---- P(r - 2): one k-step of the projection ----------------------------------------------------------
+        if (r >= 2) {
+            const v4i xf = *reinterpret_cast<const v4i *>(dtile + (r & 1) * (64 * kBlkRowB) + (wtile * 16 + j) * kBlkRowB + gq * 16);
             rsp = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, xf, rsp, 0, 0, 0);
-            const uint8_t *wfr = wb + a.off_p + lane * 16;
+            const uint8_t *wfr = wb + a.off_p + whalf * (TPW * 1024) + lane * 16;
 #pragma unroll
-            for (int nt = 0; nt < TPT; nt++) {
+            for (int nt = 0; nt < TPW; nt++) {
                 const v4i wf = *reinterpret_cast<const v4i *>(wfr + nt * 1024);
                 accp[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf, xf, accp[nt], 0, 0, 0);
             }
         }
-        if (c + 1 < a.nchunks) {
-            u32x4 *dst = reinterpret_cast<u32x4 *>(wbuf + ((c + 1) & 1) * a.chunk_bytes);
+
+        // ---- E(r): expansion of the in-image halo pixels, 16 pixels x 16 channels per unit ---------------------
+        if (r < a.nchunks) {
+            uint8_t *et = etile + (r & 1) * (HP * kBlkRowB);
+            v4i wf[3];
+#pragma unroll
+            for (int ks = 0; ks < 3; ks++)
+                if (ks < a.ke) wf[ks] = *reinterpret_cast<const v4i *>(wb + (ks * ET + wtile) * 1024 + lane * 16);
+            const v4i be = *reinterpret_cast<const v4i *>(wb + a.off_be + ecl * 4);
+            const v4i se = *reinterpret_cast<const v4i *>(wb + a.off_se + ecl * 4);
+            int32_t cst[4];
+#pragma unroll
+            for (int r4 = 0; r4 < 4; r4++) cst[r4] = be[r4] - a.zxp_e * se[r4];
+#pragma unroll
+            for (int k = 0; k < MAXU; k++) {
+                if (whalf + 2 * k < ngroups) {
+                    v4i acc = {0, 0, 0, 0};
+#pragma unroll
+                    for (int ks = 0; ks < 3; ks++)
+                        if (ks < a.ke) {
+                            const v4i xf = *reinterpret_cast<const v4i *>(exrow + k * 32 * a.xs + ks * 64);
+                            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[ks], xf, acc, 0, 0, 0);
+                        }
+                    uint32_t q[4];
+                    const HaloPix hpk = hpix[(whalf + 2 * k) * 16 + j];
+#pragma unroll
+                    for (int r4 = 0; r4 < 4; r4++) {
+                        const int32_t v = add3(acc[r4], cst[r4], hpk.nrsz);
+                        q[r4] = requant_u8_lowbyte((float)v * a.ep_e.mult, a.ep_e);
+                    }
+                    if (hpk.tile_off >= 0)
+                        *reinterpret_cast<uint32_t *>(et + hpk.tile_off + ecl) = pack_low_bytes(q[0], q[1], q[2], q[3]) ^ 0x80808080u;
+                }
+            }
+        }
+
+        // ---- D(r - 1): depthwise 3x3 on the matrix cores: 16 pixels x 16 channels per unit --------------------------
+        // The reduction index is (tap, channel): a 16-byte k-chunk of the pixel operand is one tap's 16 channels
+        // (one LDS read), and the weight operand carries w' = w - 128 of channel i at byte i of the chunk and
+        // zeros elsewhere, so row i of the product only sees its own channel.  A second product against ones in
+        // the same places gives the window sum of x', which the weight zero point multiplies:
+        //   sum (x - zx)(w - zw) = sum x'w' - zw' * sum x' - zx' * sum w' + 9 zx' zw'.
+        if (r >= 1 && r <= a.nchunks) {
+            const uint8_t *et = etile + ((r - 1) & 1) * (HP * kBlkRowB);
+            uint8_t *dt = dtile + ((r - 1) & 1) * (64 * kBlkRowB);
+            v4i wfr[3];
+#pragma unroll
+            for (int ks = 0; ks < 3; ks++) {
+                const int t = ks * 4 + gq;
+                const uint32_t wbyte = t < 9 ? (uint32_t)wb[a.off_wd + t * CE + wtile * 16 + j] : 0u;
+                const uint32_t splat = wbyte * 0x01010101u;
+                wfr[ks] = __builtin_bit_cast(v4i, u32x4{dmask[0] & splat, dmask[1] & splat, dmask[2] & splat, dmask[3] & splat});
+            }
+            const v4i bd = *reinterpret_cast<const v4i *>(wb + a.off_bd + dcl * 4);
+            const v4i sd = *reinterpret_cast<const v4i *>(wb + a.off_sd + dcl * 4);
+            int32_t ct[4];
+#pragma unroll
+            for (int r4 = 0; r4 < 4; r4++) ct[r4] = bd[r4] - a.zxp_d * sd[r4] + a.kzz_d;
+            const bool chv = (r - 1) * CE + dcl < a.mid;
+#pragma unroll
+            for (int k = 0; k < 2; k++) {
+                const uint8_t *xb = et + dxoff[k];
+                v4i aw = {0, 0, 0, 0}, a1 = {0, 0, 0, 0};
+#pragma unroll
+                for (int ks = 0; ks < 3; ks++) {
+                    const v4i xf = *reinterpret_cast<const v4i *>(xb + dtap[ks]);
+                    aw = __builtin_amdgcn_mfma_i32_16x16x64_i8(wfr[ks], xf, aw, 0, 0, 0);
+                    a1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(ks == 2 ? done_last : done_f, xf, a1, 0, 0, 0);
+                }
+                uint32_t q[4];
+#pragma unroll
+                for (int r4 = 0; r4 < 4; r4++) {
+                    const int32_t v = aw[r4] - a.zwp_d * a1[r4] + ct[r4];
+                    q[r4] = requant_u8_lowbyte((float)v * a.ep_d.mult, a.ep_d);
+                }
+                const uint32_t packed = pack_low_bytes(q[0], q[1], q[2], q[3]) ^ 0x80808080u; // kept as s8
+                if (dpv[k]) *reinterpret_cast<uint32_t *>(dt + ((whalf + 2 * k) * 16 + j) * kBlkRowB + dcl) = chv ? packed : 0u;
+            }
+        }
+
+        if (r + 1 < nrec) {
+            u32x4 *dst = reinterpret_cast<u32x4 *>(wbuf + ((r + 1) & 1) * a.chunk_bytes);
 #pragma unroll
             for (int i = 0; i < NS; i++) {
                 const int v = i * kBlkThreads + tid;
@@ -241,36 +360,37 @@ __global__ __launch_bounds__(kBlkThreads) void qblock_kernel(const BlockArgs a) 
         __syncthreads();
     }
 
-    // ---- epilogue of the projection ------------------------------------------------------------------------
-    const int pl = wave * 16 + j;
+    // ---- epilogue of the projection: pixel group wtile, the wave's TPW tiles are 4 * TPW consecutive channels per lane ----
+    const int pl = wtile * 16 + j;
     const int py = pl / kBlkTile, px = pl - py * kBlkTile;
     const int oy = oy0 + py, ox = ox0 + px;
     const bool valid = pl < TP && oy < a.out_h && ox < a.out_w;
     const int pg = valid ? (img * a.out_h + oy) * a.out_w + ox : a.p.m;
-    igemm_store_tile<TPT>(a.p, accp, rsp[0], pg, gq * (4 * TPT), gq, cterm_p, nullptr);
+    const int ch0 = gq * (4 * TPT) + whalf * (4 * TPW);
+    // igemm_store_tile reads its constants at cterm + gq * 4 * TPW + nt * 4; they sit at cterm_p + ch0 + nt * 4
+    igemm_store_tile<TPW>(a.p, accp, rsp[0], pg, ch0, gq, cterm_p + ch0 - gq * (4 * TPW), nullptr);
 }
 
-template <int S, int TPT, int ET> static int launch_block_inst(nncase_hip_ctx *ctx, const BlockArgs &a, int blocks, size_t lds) {
-    if (lds > 48 * 1024) {
-        NNHIP_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(&qblock_kernel<S, TPT, ET>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+template <int S, int TPT> static int launch_block_inst(nncase_hip_ctx *ctx, const BlockArgs &a, int blocks, size_t lds) {
+    // the dynamic LDS limit of a kernel is raised once per device (the attribute call is slow next to a launch)
+    static int raised_on_device = -1;
+    if (lds > 48 * 1024 && raised_on_device != ctx->device) {
+        NNHIP_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(&qblock_kernel<S, TPT>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        raised_on_device = ctx->device;
     }
-    hipLaunchKernelGGL((qblock_kernel<S, TPT, ET>), dim3(blocks), dim3(kBlkThreads), lds, ctx->stream, a);
+    hipLaunchKernelGGL((qblock_kernel<S, TPT>), dim3(blocks), dim3(kBlkThreads), lds, ctx->stream, a);
     NNHIP_LAUNCH_CHECK(ctx, "qblock_kernel");
     return 0;
 }
 
-template <int S, int TPT> static int launch_block_et(nncase_hip_ctx *ctx, const BlockArgs &a, int et, int blocks, size_t lds) {
-    return et == 3 ? launch_block_inst<S, TPT, 3>(ctx, a, blocks, lds) : launch_block_inst<S, TPT, 4>(ctx, a, blocks, lds);
-}
-
-template <int S> static int launch_block_s(nncase_hip_ctx *ctx, const BlockArgs &a, int tpt, int et, int blocks, size_t lds) {
+template <int S> static int launch_block_s(nncase_hip_ctx *ctx, const BlockArgs &a, int tpt, int blocks, size_t lds) {
     switch (tpt) {
-    case 2: return launch_block_et<S, 2>(ctx, a, et, blocks, lds);
-    case 4: return launch_block_et<S, 4>(ctx, a, et, blocks, lds);
-    case 6: return launch_block_et<S, 6>(ctx, a, et, blocks, lds);
-    case 10: return launch_block_et<S, 10>(ctx, a, et, blocks, lds);
-    default: return launch_block_et<S, 20>(ctx, a, et, blocks, lds);
+    case 2: return launch_block_inst<S, 2>(ctx, a, blocks, lds);
+    case 4: return launch_block_inst<S, 4>(ctx, a, blocks, lds);
+    case 6: return launch_block_inst<S, 6>(ctx, a, blocks, lds);
+    case 10: return launch_block_inst<S, 10>(ctx, a, blocks, lds);
+    default: return launch_block_inst<S, 20>(ctx, a, blocks, lds);
     }
 }
 
@@ -294,7 +414,7 @@ extern "C" int nncase_hip_qblock_supported(const nncase_hip_qblock_desc_t *d) {
 }
 
 void nncase_hip_qblock_describe(const nncase_hip_qblock_t *b, const nncase_hip_qblock_args_t *a, char *buf, size_t cap) {
-    snprintf(buf, cap, "qblock%s<S=%d,P=%d,E=%d>", a->add_input ? "+add" : "", a->stride, b->tpt, b->et);
+    snprintf(buf, cap, "qblock%s<S=%d,P=%d>", a->add_input ? "+add" : "", a->stride, b->tpt);
 }
 
 static void free_block(nncase_hip_qblock_t *b) {
@@ -324,20 +444,20 @@ extern "C" int nncase_hip_qblock_prepack(nncase_hip_ctx_t *ctx, const nncase_hip
     b->zw_d = desc->dw_w_qp.zero_point, b->sw_d = desc->dw_w_qp.scale;
     b->zw_p = desc->project_w_qp.zero_point, b->sw_p = desc->project_w_qp.scale;
     b->ke = ceil_div(cin, 64);
-    // 48-channel chunks when they divide the expanded channels and 64-channel ones do not (96, 144)
-    b->et = (mid % 64 != 0 && mid % 48 == 0) ? 3 : 4;
+    b->et = 4;
     const int ce = b->et * 16;
     b->tpt = block_tiles(cout);
     b->nchunks = ceil_div(mid, ce);
     b->off_p = b->ke * b->et * 1024;
     b->off_wd = b->off_p + b->tpt * 1024;
-    b->off_bd = b->off_wd + 9 * ce * 2;
+    b->off_bd = b->off_wd + 9 * ce;
     b->off_sd = b->off_bd + ce * 4;
     b->off_be = b->off_sd + ce * 4;
     b->off_se = b->off_be + ce * 4;
     b->chunk_bytes = b->off_se + ce * 4;
 
-    std::vector<uint8_t> blob((size_t)b->nchunks * b->chunk_bytes, 0);
+    // record r: expansion part of chunk r, depthwise part of chunk r - 1, projection part of chunk r - 2
+    std::vector<uint8_t> blob((size_t)(b->nchunks + 2) * b->chunk_bytes, 0);
     // expansion: [chunk][ks][tile] fragments, chunk = 16 * et channels
     {
         std::vector<uint8_t> frags((size_t)b->nchunks * b->ke * b->et * 1024);
@@ -364,21 +484,21 @@ extern "C" int nncase_hip_qblock_prepack(nncase_hip_ctx_t *ctx, const nncase_hip
             return (pos < ce && ch < mid) ? w_project[(size_t)oc * mid + ch] : (uint8_t)0x80;
         });
         for (int c = 0; c < b->nchunks; c++)
-            memcpy(blob.data() + (size_t)c * b->chunk_bytes + b->off_p, frags.data() + (size_t)c * b->tpt * 1024, (size_t)b->tpt * 1024);
+            memcpy(blob.data() + (size_t)(c + 2) * b->chunk_bytes + b->off_p, frags.data() + (size_t)c * b->tpt * 1024, (size_t)b->tpt * 1024);
         if (bias_project) std::copy(bias_project, bias_project + cout, bias_p.begin());
     }
-    // depthwise: (w - zw) as int16 [tap][channel of the chunk], bias and tap sum per channel
+    // depthwise: w - 128 as s8 [tap][channel of the chunk], bias and tap sum of (w - 128) per channel
     for (int c = 0; c < b->nchunks; c++) {
-        uint8_t *dst = blob.data() + (size_t)c * b->chunk_bytes;
-        int16_t *wd = reinterpret_cast<int16_t *>(dst + b->off_wd);
+        uint8_t *dst = blob.data() + (size_t)(c + 1) * b->chunk_bytes;
+        uint8_t *wd = dst + b->off_wd;
         int32_t *bd = reinterpret_cast<int32_t *>(dst + b->off_bd), *sd = reinterpret_cast<int32_t *>(dst + b->off_sd);
         for (int i = 0; i < ce; i++) {
             const int ch = c * ce + i;
             int32_t s = 0;
             for (int t = 0; t < 9; t++) {
-                const int v = ch < mid ? (int)w_dw[(size_t)ch * 9 + t] - b->zw_d : 0;
-                wd[t * ce + i] = (int16_t)v;
-                s += v;
+                const uint8_t v = ch < mid ? (uint8_t)(w_dw[(size_t)ch * 9 + t] ^ 0x80) : (uint8_t)0;
+                wd[t * ce + i] = v;
+                s += (int32_t)(int8_t)v;
             }
             bd[i] = (ch < mid && bias_dw) ? bias_dw[ch] : 0;
             sd[i] = s;
@@ -445,8 +565,10 @@ extern "C" int nncase_hip_qblock(nncase_hip_ctx_t *ctx, const uint8_t *x_dev, co
     a.zxp_e = g->x_qp.zero_point - 128;
     a.zwp_e = blk->zw_e - 128;
     a.kzz_e = blk->cin * a.zxp_e * a.zwp_e;
-    a.zx_d = g->expand_qp.zero_point;
-    a.zmid_splat = (uint32_t)(g->expand_qp.zero_point & 0xff) * 0x01010101u;
+    a.zxp_d = g->expand_qp.zero_point - 128;
+    a.zwp_d = blk->zw_d - 128;
+    a.kzz_d = 9 * a.zxp_d * a.zwp_d;
+    a.zmid_splat = (uint32_t)((g->expand_qp.zero_point ^ 0x80) & 0xff) * 0x01010101u;
     int rc = make_epilogue(ctx, &a.ep_e, g->x_qp.scale, blk->sw_e, g->expand_qp, g->expand_clamp_min, g->expand_clamp_max,
                            NNCASE_HIP_DT_U8, "qblock(expand)");
     if (rc) return rc;
@@ -486,15 +608,15 @@ extern "C" int nncase_hip_qblock(nncase_hip_ctx_t *ctx, const uint8_t *x_dev, co
     }
     const int hh = (kBlkTile - 1) * g->stride + 3, hp = hh * hh;
     const int cterm_bytes = blk->tpt * 16 * 4;
-    a.lds_xin = cterm_bytes;
+    a.lds_pix = cterm_bytes;
+    a.lds_xin = a.lds_pix + ceil_div(hp, 16) * 16 * (int)sizeof(HaloPix);
     a.lds_et = a.lds_xin + ceil_div(hp, 16) * 16 * a.xs;
-    a.lds_dt = a.lds_et + hp * kBlkRowB;
-    a.lds_w = a.lds_dt + 64 * kBlkRowB;
+    a.lds_dt = a.lds_et + 2 * hp * kBlkRowB;
+    a.lds_w = a.lds_dt + 2 * 64 * kBlkRowB;
     const size_t lds = (size_t)a.lds_w + 2 * (size_t)blk->chunk_bytes;
     NNHIP_REQUIRE(ctx, lds <= 160 * 1024, -EINVAL, "qblock: %zu bytes of LDS needed", lds);
     const int64_t blocks = (int64_t)g->batch * a.tiles_y * a.tiles_x;
     NNHIP_REQUIRE(ctx, blocks < ((int64_t)1 << 31), -EINVAL, "qblock: too many tiles");
     NNHIP_HIP(ctx, hipSetDevice(ctx->device));
-    return g->stride == 1 ? launch_block_s<1>(ctx, a, blk->tpt, blk->et, (int)blocks, lds)
-                          : launch_block_s<2>(ctx, a, blk->tpt, blk->et, (int)blocks, lds);
+    return g->stride == 1 ? launch_block_s<1>(ctx, a, blk->tpt, (int)blocks, lds) : launch_block_s<2>(ctx, a, blk->tpt, (int)blocks, lds);
 }

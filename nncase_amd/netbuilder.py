@@ -352,7 +352,7 @@ class HipModel:
     so results are bit-identical to lanes == 1."""
 
     def __init__(self, ctx: Context, qg: QuantGraph, batch: int, capture_graph: bool = True, fuse_residual: bool = True,
-                 lanes: int = 1, fuse_blocks: bool = False):
+                 lanes: int = 1, fuse_blocks=True):
         if lanes < 1 or lanes > rt.MAX_LANES or batch % lanes:
             raise ValueError(f"lanes={lanes} must be in 1..{rt.MAX_LANES} and divide the batch ({batch})")
         self.ctx, self.qg, self.batch, self.lanes = ctx, qg, batch, lanes
@@ -423,6 +423,11 @@ class HipModel:
                 if addn is not None and (qg.nodes[addn].inputs[0] != e.inputs[0] or tuple(d.stride) != (1, 1)):
                     continue
                 if not ctx.qblock_supported(e.weights.shape[1], e.weights.shape[0], pr.weights.shape[0]):
+                    continue
+                # Where it pays: mid-sized feature maps.  On large maps the three operators are bandwidth-bound
+                # kernels of their own that already run near the epilogue's arithmetic cost, on 7x7 maps a
+                # workgroup per image leaves most of the device idle.
+                if fuse_blocks != "all" and not (d.out_shape[1] * d.out_shape[2] >= 196 and e.out_shape[1] * e.out_shape[2] <= 784):
                     continue
                 self.blocks[i] = (i + 1, i + 2, addn)
         for e, (d, pr, addn) in self.blocks.items():

@@ -13,7 +13,7 @@ pytestmark = pytest.mark.gpu
 f32 = np.float32
 
 
-def check_model(hip_ctx, qg, x, capture, fuse_residual=True, fuse_blocks=True):
+def check_model(hip_ctx, qg, x, capture, fuse_residual=True, fuse_blocks="all"):
     model = nb.HipModel(hip_ctx, qg, x.shape[0], capture_graph=capture, fuse_residual=fuse_residual, fuse_blocks=fuse_blocks)
     y = model.run(x)
     want, outs = netref.run_integer(qg, x, keep_all=True)
@@ -176,8 +176,8 @@ def test_profile_and_kernel_names(hip_ctx):
     assert all(n.startswith("qconv_igemm<T=") and n.endswith(",rows16>") for n in (names[1], names[3]))
     ms = model.fn.profile(3)
     assert len(ms) == 5 and all(0 < t < 50 for t in ms)
-    fused = nb.HipModel(hip_ctx, qg, 2, capture_graph=False, fuse_blocks=True)
-    assert [fused.fn.op_kernel(i) for i in range(len(fused.fn))] == ["quantize", "qblock<S=1,P=4,E=3>", "dequantize"]
+    fused = nb.HipModel(hip_ctx, qg, 2, capture_graph=False, fuse_blocks="all")
+    assert [fused.fn.op_kernel(i) for i in range(len(fused.fn))] == ["quantize", "qblock<S=1,P=4>", "dequantize"]
     assert fused.op_members == [[0], [1, 2, 3], []]
 
 
@@ -243,10 +243,10 @@ def test_mobilenetv2_fused_blocks_match_separate_operators(hip_ctx):
     rng = np.random.default_rng(3)
     qg = nb.quantize_graph(g, rng.random((32, 224, 224, 3), dtype=f32))
     x = np.random.default_rng(4).random((8, 224, 224, 3), dtype=f32)
-    plain = nb.HipModel(hip_ctx, qg, 8, capture_graph=False)
+    plain = nb.HipModel(hip_ctx, qg, 8, capture_graph=False, fuse_blocks=False)
     y0 = plain.run(x)
     for capture, lanes in ((False, 1), (True, 1), (True, 2)):
-        fused = nb.HipModel(hip_ctx, qg, 8, capture_graph=capture, lanes=lanes, fuse_blocks=True)
+        fused = nb.HipModel(hip_ctx, qg, 8, capture_graph=capture, lanes=lanes, fuse_blocks="all")
         assert len(fused.blocks) == 16 and len(fused.fn) == lanes * (len(plain.fn) - 32)
         y = fused.run(x)
         assert np.array_equal(y.view(np.uint32), y0.view(np.uint32))
