@@ -294,11 +294,10 @@ __global__ __launch_bounds__(kBlkThreads) void qblock_kernel(const BlockArgs a) 
                         }
                     uint32_t q[4];
                     const HaloPix hpk = hpix[(whalf + 2 * k) * 16 + j];
+                    int32_t v4[4];
 #pragma unroll
-                    for (int r4 = 0; r4 < 4; r4++) {
-                        const int32_t v = add3(acc[r4], cst[r4], hpk.nrsz);
-                        q[r4] = requant_u8_lowbyte((float)v * a.ep_e.mult, a.ep_e);
-                    }
+                    for (int r4 = 0; r4 < 4; r4++) v4[r4] = add3(acc[r4], cst[r4], hpk.nrsz);
+                    requant4_u8_lowbyte(v4, a.ep_e, q);
                     if (hpk.tile_off >= 0)
                         *reinterpret_cast<uint32_t *>(et + hpk.tile_off + ecl) = pack_low_bytes(q[0], q[1], q[2], q[3]) ^ 0x80808080u;
                 }
@@ -339,11 +338,10 @@ __global__ __launch_bounds__(kBlkThreads) void qblock_kernel(const BlockArgs a) 
                     a1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(ks == 2 ? done_last : done_f, xf, a1, 0, 0, 0);
                 }
                 uint32_t q[4];
+                int32_t v4[4];
 #pragma unroll
-                for (int r4 = 0; r4 < 4; r4++) {
-                    const int32_t v = aw[r4] - a.zwp_d * a1[r4] + ct[r4];
-                    q[r4] = requant_u8_lowbyte((float)v * a.ep_d.mult, a.ep_d);
-                }
+                for (int r4 = 0; r4 < 4; r4++) v4[r4] = aw[r4] - a.zwp_d * a1[r4] + ct[r4];
+                requant4_u8_lowbyte(v4, a.ep_d, q);
                 const uint32_t packed = pack_low_bytes(q[0], q[1], q[2], q[3]) ^ 0x80808080u; // kept as s8
                 if (dpv[k]) *reinterpret_cast<uint32_t *>(dt + ((whalf + 2 * k) * 16 + j) * kBlkRowB + dcl) = chv ? packed : 0u;
             }

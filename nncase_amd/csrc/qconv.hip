@@ -5,7 +5,9 @@
 
 #include <algorithm>
 #include <cmath>
+#include <mutex>
 #include <new>
+#include <utility>
 #include <vector>
 
 namespace nnhip {
@@ -53,6 +55,88 @@ float nnhip::reciprocal_rn(float b) {
     return best;
 }
 
+namespace {
+
+// Host emulation of the device's two requantisation forms (same single IEEE operations).
+inline int requant_ref(int32_t v, const nnhip::Epilogue &ep) {
+    volatile float f = (float)v * ep.mult;
+    volatile float t = f / ep.sy; // what div_rn returns: the correctly rounded quotient
+    volatile float u = t + ep.zy;
+    float c = std::fmin(std::fmax((float)u, ep.qlo), ep.qhi);
+    return (int)std::nearbyintf(c);
+}
+inline int requant_fma(int32_t v, float c1, float c2, const nnhip::Epilogue &ep) {
+    const float u = std::fmaf((float)v, c1, c2);
+    float c = std::fmin(std::fmax(u, ep.qlo), ep.qhi);
+    return (int)std::nearbyintf(c);
+}
+
+// Both forms are monotone non-decreasing step functions of the accumulator, so they are equal everywhere iff
+// they agree at both ends of the int32 range and on both sides of every step of the reference form.
+void find_fast_requant(nnhip::Epilogue *ep) {
+    ep->fast = 0;
+    ep->c1 = ep->c2 = 0.f;
+    if (!(ep->mult > 0.f) || !(ep->sy > 0.f)) return;
+    const int32_t vmin = INT32_MIN + 1, vmax = INT32_MAX;
+    const int rmin = requant_ref(vmin, *ep), rmax = requant_ref(vmax, *ep);
+    // steps[k - rmin - 1] = smallest accumulator whose code is >= k
+    std::vector<int32_t> steps;
+    steps.reserve(256);
+    int32_t lo = vmin;
+    for (int k = rmin + 1; k <= rmax; k++) {
+        int64_t a = lo, b = vmax; // requant_ref(a) < k <= requant_ref(b)
+        while (b - a > 1) {
+            const int64_t m = a + (b - a) / 2;
+            if (requant_ref((int32_t)m, *ep) >= k) b = m;
+            else a = m;
+        }
+        steps.push_back((int32_t)b);
+        lo = (int32_t)a;
+    }
+    auto matches = [&](float c1, float c2) {
+        if (requant_fma(vmin, c1, c2, *ep) != rmin || requant_fma(vmax, c1, c2, *ep) != rmax) return false;
+        for (size_t i = 0; i < steps.size(); i++) {
+            const int k = rmin + 1 + (int)i;
+            // several codes can share one step when the accumulator scale is coarse
+            if (requant_fma(steps[i], c1, c2, *ep) != requant_ref(steps[i], *ep)) return false;
+            if (requant_fma(steps[i] - 1, c1, c2, *ep) != requant_ref(steps[i] - 1, *ep)) return false;
+            (void)k;
+        }
+        return true;
+    };
+    const float c1_0 = (float)((double)ep->mult / (double)ep->sy);
+    if (!std::isfinite(c1_0) || c1_0 <= 0.f) return;
+    // nominal constants first, then small perturbations of both (the reference's own rounding noise decides a
+    // few steps that sit almost exactly on an integer accumulator)
+    for (int ring = 0; ring <= 24; ring++)
+        for (int i = -ring; i <= ring; i++)
+            for (int j = -ring; j <= ring; j++) {
+                if (std::max(std::abs(i), std::abs(j)) != ring) continue;
+                float c1 = c1_0;
+                for (int s = 0; s < std::abs(i); s++) c1 = std::nextafterf(c1, i > 0 ? INFINITY : 0.f);
+                const float c2 = ep->zy + (float)j * 0x1p-18f;
+                if (matches(c1, c2)) {
+                    ep->c1 = c1;
+                    ep->c2 = c2;
+                    ep->fast = 1;
+                    return;
+                }
+            }
+}
+
+struct EpilogueKey {
+    float mult, sy, zy, lo, hi;
+    bool operator==(const EpilogueKey &o) const { return memcmp(this, &o, sizeof(*this)) == 0; }
+};
+// The search costs a few hundred thousand float operations; the same layer is set up again on every eager call.
+struct EpilogueCache {
+    std::mutex mu;
+    std::vector<std::pair<EpilogueKey, nnhip::Epilogue>> entries;
+};
+EpilogueCache g_epilogues;
+
+} // namespace
+
 int nnhip::make_epilogue(nncase_hip_ctx *ctx, Epilogue *ep, float sx, float sw, nncase_hip_quant_param_t y_qp, float clamp_min,
                          float clamp_max, int out_dtype, const char *who) {
     ep->mult = sx * sw;
@@ -63,6 +147,8 @@ int nnhip::make_epilogue(nncase_hip_ctx *ctx, Epilogue *ep, float sx, float sw, 
     ep->rsy = 1.f;
     ep->qlo = 0.f;
     ep->qhi = 255.f;
+    ep->c1 = ep->c2 = 0.f;
+    ep->fast = 0;
     ep->out_mode = out_dtype == NNCASE_HIP_DT_U8 ? kOutU8 : (out_dtype == NNCASE_HIP_DT_I32 ? kOutI32 : kOutF32);
     NNHIP_REQUIRE(ctx, !(clamp_min > clamp_max), -EINVAL, "%s: fused clamp minimum above maximum", who);
     if (ep->out_mode != kOutU8) return 0;
@@ -81,6 +167,18 @@ int nnhip::make_epilogue(nncase_hip_ctx *ctx, Epilogue *ep, float sx, float sw, 
     ghi = ghi + ep->zy;
     ep->qlo = std::fmin(std::fmax((float)glo, 0.f), 255.f);
     ep->qhi = std::fmin(std::fmax((float)ghi, 0.f), 255.f);
+    {
+        const EpilogueKey key{ep->mult, ep->sy, ep->zy, ep->lo, ep->hi};
+        std::lock_guard<std::mutex> lock(g_epilogues.mu);
+        for (const auto &e : g_epilogues.entries)
+            if (e.first == key) {
+                ep->c1 = e.second.c1, ep->c2 = e.second.c2, ep->fast = e.second.fast;
+                return 0;
+            }
+        find_fast_requant(ep);
+        if (g_epilogues.entries.size() >= 4096) g_epilogues.entries.clear();
+        g_epilogues.entries.emplace_back(key, *ep);
+    }
     return 0;
 }
 

@@ -49,6 +49,13 @@ struct Epilogue {
     float zy;
     float qlo, qhi; // clamp on the requantised value before rounding to an integer
     int out_mode;
+    // One-instruction form of the same map (U8 output): the requantised code is a monotone step function of
+    // the int32 accumulator, and the host looks for constants with which
+    //   RN(fma((float)acc, c1, c2))
+    // steps at exactly the same accumulators as the three-rounding sequence above (make_epilogue checks
+    // every step of the staircase, so the bytes are identical); fast == 0 when no such pair was found.
+    float c1, c2;
+    int fast;
 };
 
 // Second requantisation stage of a fused residual add:
@@ -111,6 +118,22 @@ __device__ __forceinline__ uint32_t requant_u8_lowbyte(float f, const Epilogue &
     float u = div_rn(f, ep.sy, ep.rsy) + ep.zy;
     u = __builtin_amdgcn_fmed3f(u, ep.qlo, ep.qhi);
     return __float_as_uint(u + 12582912.0f);
+}
+
+// The requantised codes of four int32 accumulators (low bytes), by the one-instruction form when the host
+// has proved it equal to the three-rounding sequence for this layer.
+__device__ __forceinline__ void requant4_u8_lowbyte(const int32_t (&v)[4], const Epilogue &ep, uint32_t (&q)[4]) {
+    if (ep.fast) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            float u = __builtin_fmaf((float)v[r], ep.c1, ep.c2);
+            u = __builtin_amdgcn_fmed3f(u, ep.qlo, ep.qhi);
+            q[r] = __float_as_uint(u + 12582912.0f);
+        }
+    } else {
+#pragma unroll
+        for (int r = 0; r < 4; r++) q[r] = requant_u8_lowbyte((float)v[r] * ep.mult, ep);
+    }
 }
 
 // Packs the low bytes of four dwords into one dword (3 byte-permutes).

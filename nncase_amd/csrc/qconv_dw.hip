@@ -48,8 +48,7 @@ struct DwArgs {
 __device__ __forceinline__ void dw_store4(const DwArgs &a, uint32_t o, const int32_t (&v)[4]) {
     if (a.ep.out_mode == kOutU8) {
         uint32_t b[4];
-#pragma unroll
-        for (int c = 0; c < 4; c++) b[c] = requant_u8_lowbyte((float)v[c] * a.ep.mult, a.ep);
+        requant4_u8_lowbyte(v, a.ep, b);
         *reinterpret_cast<uint32_t *>(reinterpret_cast<uint8_t *>(a.y) + o) = pack_low_bytes(b[0], b[1], b[2], b[3]);
     } else if (a.ep.out_mode == kOutI32) {
         *reinterpret_cast<int4 *>(reinterpret_cast<int32_t *>(a.y) + o) = int4{v[0], v[1], v[2], v[3]};

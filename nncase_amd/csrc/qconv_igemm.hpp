@@ -247,11 +247,10 @@ __device__ __forceinline__ void igemm_store_tile(const IgemmArgs &a, const v4i (
         for (int nt = 0; nt < T; nt++) {
             const v4i ct = *reinterpret_cast<const v4i *>(cterm + gq * (4 * T) + nt * 4);
             uint32_t b[4];
+            int32_t v[4];
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const int32_t v = add3(acc[nt][r], ct[r], nrsz);
-                b[r] = requant_u8_lowbyte((float)v * a.ep.mult, a.ep);
-            }
+            for (int r = 0; r < 4; r++) v[r] = add3(acc[nt][r], ct[r], nrsz);
+            requant4_u8_lowbyte(v, a.ep, b);
             packed[nt] = pack_low_bytes(b[0], b[1], b[2], b[3]);
         }
         if (a.lut) { // fused unary operator: one LDS byte read per output
@@ -634,7 +633,9 @@ template <int T, int RG, int MODE> int launch_trg(nncase_hip_ctx *ctx, const Ige
     IgemmArgs args = a;
     constexpr int pix_per_block = kWaves * RG * 16;
     args.num_mtiles = ceil_div(a.m, pix_per_block);
-    int gx = args.num_mtiles < ctx->compute_units * 2 ? args.num_mtiles : ctx->compute_units * 2;
+    // persistent blocks: four per compute unit (a block's chain of load -> multiply -> store per pixel tile is
+    // latency-bound, so more chains in flight beat longer ones)
+    int gx = args.num_mtiles < ctx->compute_units * 4 ? args.num_mtiles : ctx->compute_units * 4;
     // Blocks are dealt to the 8 XCDs round-robin by linear id; with a multiple of 8
     // columns the blocks that share a pixel tile (same x, different chunk) land on
     // one XCD and find the activations in its L2.
