@@ -182,6 +182,20 @@ typedef struct nncase_hip_conv2d_args {
 NNCASE_HIP_API int nncase_hip_qconv2d(nncase_hip_ctx_t *ctx, const uint8_t *x_dev, const nncase_hip_weights_t *weights,
                                       void *y_dev, const nncase_hip_conv2d_args_t *args);
 
+/* Host-only view of the u8 requantisation  q = sat_u8(rne(clamp((float)acc * (sx * sw), lo, hi) / sy + zy))
+ * (quantize.cpp:36-43 applied to Conv2D's clamped fp32 value, convolution.cpp:99-101) that the u8 epilogues run.
+ * It is a monotone step function of the accumulator; where constants exist for which
+ * RN(fma((float)acc, c1, c2)) steps at exactly the same accumulators, the kernels use that one
+ * instruction instead of the three-rounding sequence.  nncase_hip_requant_plan returns 1 and the
+ * constants if the search (every step of the staircase is compared) found a pair, else 0;
+ * nncase_hip_requant_host evaluates the form the kernels would pick (form_used: 1 = fma form,
+ * 0 = exact sequence) on host accumulators, so that callers and tests can compare it with their
+ * own arithmetic.  Neither needs a device. */
+NNCASE_HIP_API int nncase_hip_requant_plan(float sx, float sw, nncase_hip_quant_param_t y_qp, float clamp_min, float clamp_max,
+                                           float *c1, float *c2);
+NNCASE_HIP_API int nncase_hip_requant_host(float sx, float sw, nncase_hip_quant_param_t y_qp, float clamp_min, float clamp_max,
+                                           const int32_t *acc_host, size_t count, uint8_t *out_host, int32_t *form_used);
+
 /* ---- fused inverted-residual block ------------------------------------------
  * 1x1 convolution (in -> mid channels), 3x3 depthwise convolution on the mid
  * channels (stride 1 or 2), 1x1 convolution (mid -> out channels), optionally

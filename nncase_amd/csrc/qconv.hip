@@ -214,6 +214,28 @@ static void free_weights(nncase_hip_weights *w) {
     delete w;
 }
 
+extern "C" int nncase_hip_requant_plan(float sx, float sw, nncase_hip_quant_param_t y_qp, float clamp_min, float clamp_max, float *c1,
+                                       float *c2) {
+    Epilogue ep;
+    const int rc = make_epilogue(nullptr, &ep, sx, sw, y_qp, clamp_min, clamp_max, NNCASE_HIP_DT_U8, "requant_plan");
+    if (rc) return rc;
+    if (c1) *c1 = ep.c1;
+    if (c2) *c2 = ep.c2;
+    return ep.fast;
+}
+
+extern "C" int nncase_hip_requant_host(float sx, float sw, nncase_hip_quant_param_t y_qp, float clamp_min, float clamp_max,
+                                       const int32_t *acc_host, size_t count, uint8_t *out_host, int32_t *form_used) {
+    if (!acc_host || !out_host) return -EINVAL;
+    Epilogue ep;
+    const int rc = make_epilogue(nullptr, &ep, sx, sw, y_qp, clamp_min, clamp_max, NNCASE_HIP_DT_U8, "requant_host");
+    if (rc) return rc;
+    if (form_used) *form_used = ep.fast;
+    for (size_t i = 0; i < count; i++)
+        out_host[i] = (uint8_t)(ep.fast ? requant_fma(acc_host[i], ep.c1, ep.c2, ep) : requant_ref(acc_host[i], ep));
+    return 0;
+}
+
 extern "C" int nncase_hip_qconv2d_prepack(nncase_hip_ctx_t *ctx, const nncase_hip_conv2d_desc_t *desc,
                                           const uint8_t *weights_oihw_host, const int32_t *bias_host,
                                           nncase_hip_weights_t **weights) {

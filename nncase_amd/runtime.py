@@ -102,6 +102,8 @@ SYMBOLS = {
     "nncase_hip_weights_destroy": (_I, [_VP, _VP]),
     "nncase_hip_weights_set_post_lut": (_I, [_VP, _VP, _VP, QuantParam]),
     "nncase_hip_qconv2d": (_I, [_VP, _VP, _VP, _VP, C.POINTER(Conv2dArgs)]),
+    "nncase_hip_requant_plan": (_I, [C.c_float, C.c_float, QuantParam, C.c_float, C.c_float, C.POINTER(C.c_float), C.POINTER(C.c_float)]),
+    "nncase_hip_requant_host": (_I, [C.c_float, C.c_float, QuantParam, C.c_float, C.c_float, _VP, _SZ, _VP, _I32P]),
     "nncase_hip_qblock_supported": (_I, [C.POINTER(QBlockDesc)]),
     "nncase_hip_qblock_prepack": (_I, [_VP, C.POINTER(QBlockDesc), _VP, _VP, _VP, _VP, _VP, _VP, C.POINTER(_VP)]),
     "nncase_hip_qblock_destroy": (_I, [_VP, _VP]),
@@ -212,6 +214,28 @@ def make_unary_lut(kind: int, x_qp: "QuantParam", y_qp: "QuantParam") -> np.ndar
     if rc != 0:
         raise HipError(rc, "make_unary_lut", "invalid kind or zero output scale")
     return lut
+
+
+def requant_plan(sx, sw, y_qp: "QuantParam", clamp=(-FLT_MAX, FLT_MAX)):
+    """(found, c1, c2): the one-FMA form of the u8 requantisation the kernels would use for this layer, if the
+    library's host-side search proved one equal to the three-rounding sequence (host-only, no device needed)."""
+    c1, c2 = C.c_float(), C.c_float()
+    rc = load_library().nncase_hip_requant_plan(float(sx), float(sw), y_qp, clamp[0], clamp[1], C.byref(c1), C.byref(c2))
+    if rc < 0:
+        raise HipError(rc, "requant_plan", "scales outside the supported range")
+    return bool(rc), c1.value, c2.value
+
+
+def requant_host(acc: np.ndarray, sx, sw, y_qp: "QuantParam", clamp=(-FLT_MAX, FLT_MAX)):
+    """(bytes, form): the requantised codes of int32 accumulators by the form the kernels pick (1 = FMA form)."""
+    acc = np.ascontiguousarray(acc, np.int32)
+    out = np.empty(acc.shape, np.uint8)
+    form = C.c_int32()
+    rc = load_library().nncase_hip_requant_host(float(sx), float(sw), y_qp, clamp[0], clamp[1], acc.ctypes.data, acc.size,
+                                                out.ctypes.data, C.byref(form))
+    if rc != 0:
+        raise HipError(rc, "requant_host", "scales outside the supported range")
+    return out, form.value
 
 
 def _concat_args(inputs, channels, in_qps):
