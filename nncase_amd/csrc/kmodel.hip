@@ -93,6 +93,7 @@ struct nncase_hip_kmodel {
     std::vector<void *> buffers;      // one device buffer per tensor (aliases share an entry's value)
     std::vector<char> owns;           // whether buffers[i] is freed with the model
     std::vector<nncase_hip_weights_t *> weights;
+    std::vector<nncase_hip_qblock_t *> blocks;
     nncase_hip_function_t *fn = nullptr;
     uint32_t input_tensor = 0, output_tensor = 0, n_outputs = 1; // outputs are consecutive tensors
 };
@@ -104,6 +105,8 @@ extern "C" int nncase_hip_kmodel_destroy(nncase_hip_kmodel_t *m) {
     if (m->fn) (void)nncase_hip_function_destroy(m->fn); // synchronises the stream first
     for (auto *w : m->weights)
         if (w) (void)nncase_hip_weights_destroy(m->ctx, w);
+    for (auto *b : m->blocks)
+        if (b) (void)nncase_hip_qblock_destroy(m->ctx, b);
     for (size_t i = 0; i < m->buffers.size(); i++)
         if (m->owns[i] && m->buffers[i]) (void)hipFree(m->buffers[i]);
     delete m;
@@ -262,12 +265,40 @@ extern "C" int nncase_hip_kmodel_load(nncase_hip_ctx_t *ctx, const void *data, s
         }
     }
 
+    // 1x1 conv -> depthwise 3x3 -> 1x1 conv (+ the block's input), each consumed only by the next, on mid-sized
+    // maps: one fused operator whose two expanded tensors never reach HBM (see nncase_hip_qblock)
+    std::vector<char> block_head(th.n_ops, 0);
+    auto pointwise = [&](const hipf_op &c) {
+        return c.opcode == kOpConv2d && c.n_inputs == 1 && c.p[2] == 1 && c.p[3] == 1 && c.p[4] == 1 && c.p[5] == 1 && c.p[6] == 1 &&
+               c.p[7] == 1 && c.p[8] == 1 && c.p[9] == 0 && c.p[10] == 0 && c.p[11] == 0 && c.p[12] == 0;
+    };
+    for (uint32_t k = 0; k + 2 < th.n_ops; k++) {
+        const hipf_op &e = ops[k], &d = ops[k + 1], &pr = ops[k + 2];
+        if (!pointwise(e) || !pointwise(pr) || d.opcode != kOpConv2d || d.n_inputs != 1) continue;
+        const bool dw3 = d.p[1] == 1 && d.p[4] == d.p[0] && d.p[2] == 3 && d.p[3] == 3 && d.p[5] == d.p[6] && (d.p[5] == 1 || d.p[5] == 2) &&
+                         d.p[7] == 1 && d.p[8] == 1 && (unsigned)d.p[9] <= 1 && (unsigned)d.p[10] <= 1 && (unsigned)d.p[11] <= 1 &&
+                         (unsigned)d.p[12] <= 1;
+        if (!dw3 || d.inputs[0] != e.output || pr.inputs[0] != d.output) continue;
+        if (consumers[e.output] != 1 || consumers[d.output] != 1 || is_output(e.output) || is_output(d.output)) continue;
+        if (fused_lut[k] >= 0 || fused_lut[k + 1] >= 0 || fused_lut[k + 2] >= 0 || fused_add[k] >= 0 || fused_add[k + 1] >= 0) continue;
+        if (fused_add[k + 2] >= 0 && (ops[fused_add[k + 2]].inputs[0] != e.inputs[0] || d.p[5] != 1)) continue;
+        nncase_hip_qblock_desc_t bd{};
+        bd.in_channels = e.p[1], bd.mid_channels = e.p[0], bd.out_channels = pr.p[0];
+        if (d.p[0] != e.p[0] || pr.p[1] != e.p[0] || !nncase_hip_qblock_supported(&bd)) continue;
+        const hipf_tensor &te = m->tensors[e.output], &td = m->tensors[d.output];
+        if (!((uint64_t)td.dims[1] * td.dims[2] >= 196 && (uint64_t)te.dims[1] * te.dims[2] <= 784)) continue; // where it pays
+        block_head[k] = 1;
+        skipped[k + 1] = skipped[k + 2] = 1;
+        k += 2;
+    }
+
     // ---- device buffers ---------------------------------------------------------------------------
     m->buffers.assign(th.n_tensors, nullptr);
     m->owns.assign(th.n_tensors, 0);
     for (uint32_t k = 0; k < th.n_ops; k++) { // tensors that only exist inside a fused operator
         if (fused_add[k] >= 0 || fused_lut[k] >= 0) m->owns[ops[k].output] = 2;
         if (fused_add[k] >= 0 && fused_lut[k] >= 0) m->owns[ops[fused_lut[k]].output] = 2;
+        if (block_head[k]) m->owns[ops[k].output] = m->owns[ops[k + 1].output] = 2;
     }
     for (uint32_t t = 0; t < th.n_tensors; t++) {
         if (m->owns[t] == 2) {
@@ -290,6 +321,60 @@ extern "C" int nncase_hip_kmodel_load(nncase_hip_ctx_t *ctx, const void *data, s
         const uint32_t in0 = (uint32_t)o.inputs[0], dst = (uint32_t)o.output;
         const hipf_tensor &ti = m->tensors[in0], &to = m->tensors[dst];
         int rc = -EINVAL;
+        if (block_head[k]) {
+            const hipf_op &d = ops[k + 1], &pr = ops[k + 2];
+            const uint32_t te = (uint32_t)o.output, td = (uint32_t)d.output, tp = (uint32_t)pr.output;
+            const int cin = o.p[1], mid = o.p[0], cout = pr.p[0];
+            NNHIP_REQUIRE(ctx, ti.dtype == NNCASE_HIP_DT_U8 && m->tensors[tp].dtype == NNCASE_HIP_DT_U8 && (uint32_t)cin == ti.dims[3] &&
+                                   (uint32_t)cout == m->tensors[tp].dims[3] && ti.dims[0] == m->tensors[tp].dims[0],
+                          -NNCASE_HIP_ERR_SHAPE_MISMATCH, "kmodel_load: op %u block channels / batch do not match its tensors", k);
+            const uint8_t *wgt[3] = {rd(o.rdata0, (size_t)mid * cin), rd(d.rdata0, (size_t)mid * 9), rd(pr.rdata0, (size_t)cout * mid)};
+            const int32_t *bia[3] = {nullptr, nullptr, nullptr};
+            const hipf_op *stage[3] = {&o, &d, &pr};
+            for (int i = 0; i < 3; i++) {
+                NNHIP_REQUIRE(ctx, wgt[i], -EINVAL, "kmodel_load: op %u weights outside .rdata", k + i);
+                if (stage[i]->rdata1 != kNoRdata) {
+                    const uint8_t *b = rd(stage[i]->rdata1, (size_t)stage[i]->p[0] * 4);
+                    NNHIP_REQUIRE(ctx, b && (stage[i]->rdata1 & 3) == 0, -EINVAL, "kmodel_load: op %u bias outside .rdata or misaligned", k + i);
+                    bia[i] = reinterpret_cast<const int32_t *>(b);
+                }
+            }
+            nncase_hip_qblock_desc_t bd{};
+            bd.in_channels = cin, bd.mid_channels = mid, bd.out_channels = cout;
+            bd.expand_w_qp = nncase_hip_quant_param_t{o.p[13], o.f[2]};
+            bd.dw_w_qp = nncase_hip_quant_param_t{d.p[13], d.f[2]};
+            bd.project_w_qp = nncase_hip_quant_param_t{pr.p[13], pr.f[2]};
+            nncase_hip_qblock_t *blk = nullptr;
+            rc = nncase_hip_qblock_prepack(ctx, &bd, wgt[0], bia[0], wgt[1], bia[1], wgt[2], bia[2], &blk);
+            if (rc) return rc;
+            m->blocks.push_back(blk);
+            nncase_hip_qblock_args_t a{};
+            a.batch = (int)ti.dims[0], a.in_h = (int)ti.dims[1], a.in_w = (int)ti.dims[2], a.stride = d.p[5];
+            a.pad_h_before = d.p[9], a.pad_h_after = d.p[10], a.pad_w_before = d.p[11], a.pad_w_after = d.p[12];
+            a.x_qp = tqp(in0), a.expand_qp = tqp(te), a.dw_qp = tqp(td), a.y_qp = tqp(tp);
+            a.expand_clamp_min = o.f[0], a.expand_clamp_max = o.f[1];
+            a.dw_clamp_min = d.f[0], a.dw_clamp_max = d.f[1];
+            a.clamp_min = pr.f[0], a.clamp_max = pr.f[1];
+            NNHIP_REQUIRE(ctx, m->tensors[te].dims[1] == ti.dims[1] && m->tensors[te].dims[2] == ti.dims[2] &&
+                                   windowed_output_size(a.in_h, 3, a.stride, 1, a.pad_h_before, a.pad_h_after) == (int)m->tensors[tp].dims[1] &&
+                                   windowed_output_size(a.in_w, 3, a.stride, 1, a.pad_w_before, a.pad_w_after) == (int)m->tensors[tp].dims[2] &&
+                                   m->tensors[td].dims[1] == m->tensors[tp].dims[1] && m->tensors[td].dims[2] == m->tensors[tp].dims[2],
+                          -NNCASE_HIP_ERR_SHAPE_MISMATCH, "kmodel_load: op %u block extents do not match its tensors", k);
+            void *y = m->buffers[tp];
+            if (fused_add[k + 2] >= 0) {
+                const hipf_op &add = ops[fused_add[k + 2]];
+                const uint32_t sum = (uint32_t)add.output;
+                NNHIP_REQUIRE(ctx, elems(sum) == elems(tp) && elems(in0) == elems(tp), -NNCASE_HIP_ERR_SHAPE_MISMATCH,
+                              "kmodel_load: op %d add shapes differ", fused_add[k + 2]);
+                a.add_input = 1;
+                a.sum_qp = tqp(sum);
+                a.sum_clamp_min = add.f[0], a.sum_clamp_max = add.f[1];
+                y = m->buffers[sum];
+            }
+            rc = nncase_hip_function_add_qblock(m->fn, static_cast<const uint8_t *>(m->buffers[in0]), blk, static_cast<uint8_t *>(y), &a);
+            if (rc) return rc;
+            continue;
+        }
         switch (o.opcode) {
         case kOpQuantize:
             NNHIP_REQUIRE(ctx, elems(in0) == elems(dst), -NNCASE_HIP_ERR_SHAPE_MISMATCH, "kmodel_load: op %u shapes differ", k);

@@ -56,7 +56,7 @@ def test_mobilenetv2_kmodel(hip_ctx):
     qg = nb.quantize_graph(nb.mobilenet_v2(seed=2), rng.random((8, 224, 224, 3), dtype=f32))
     x = rng.random((2, 224, 224, 3), dtype=f32)
     model, y, fused = run_and_check(hip_ctx, qg, x)
-    assert fused == 10 and len(model.fn) == 56           # the ten residual adds are folded by the loader
+    assert fused == 28 and len(model.fn) == 38           # ten residual adds and nine whole blocks are folded by the loader
     ref = nb.HipModel(hip_ctx, qg, 2, capture_graph=False)
     assert np.array_equal(ref.run(x).view(np.uint32).ravel(), y.view(np.uint32).ravel())
 
