@@ -156,12 +156,16 @@ def side_workload(args):
         rng = np.random.default_rng(7)
         g = nb.yolov5s(seed=4, input_hw=hw)
         qg = nb.quantize_graph(g, rng.random((2, hw, hw, 3), dtype=np.float32), calib_batch=1)
-        model = nb.HipModel(ctx, qg, batch, capture_graph=True)
+        model = nb.HipModel(ctx, qg, batch, capture_graph=True, lanes=args.lanes)
         x = rng.random((batch, hw, hw, 3), dtype=np.float32)
         model.set_input(x)
         ms = time_calls(ctx, model.invoke, args.warmup, args.steps)
-        op_ms = model.fn.profile(5)
-        names = [model.fn.op_kernel(i) for i in range(len(model.fn))]
+        # per-kernel figures on the one-chain recording (kernels of concurrent chains have no duration of their own)
+        kmodel = model if args.lanes == 1 else nb.HipModel(ctx, qg, batch, capture_graph=False)
+        if kmodel is not model:
+            kmodel.set_input(x)
+        op_ms = kmodel.fn.profile(5)
+        names = [kmodel.fn.op_kernel(i) for i in range(len(kmodel.fn))]
         macs = sum(qg.macs_per_image.values()) * batch
         groups = {}
         for nme, t in zip(names, op_ms):
@@ -179,7 +183,8 @@ def side_workload(args):
         line = dict(base, metric="images/sec u8/u8 YOLOv5s 640x640 b16", value=round(batch / (ms * 1e-3), 1), unit="images/s",
                     ms_per_step=round(ms, 4), dtype="u8",
                     config={"workload": "config 4: YOLOv5s-style backbone + neck + head, 640x640, u8/u8 per-tensor PTQ (2 calibration "
-                                        "images), batch 16, SiLU as byte tables, " + str(len(model.fn)) + " operators, HIP-graph replay",
+                                        "images), batch 16, SiLU as byte tables, " + str(len(kmodel.fn)) + " operators, HIP-graph replay" +
+                                        (f" as {args.lanes} concurrent chains of {batch // args.lanes} images" if args.lanes > 1 else ""),
                             "batch_consistent": True},
                     roofline={"bound": "mfma", "achieved": round(2 * macs / (conv_ms * 1e-3) / 1e12, 1), "peak": INT8_PEAK_TOPS,
                               "unit": "TOP/s", "frac": round(2 * macs / (conv_ms * 1e-3) / 1e12 / INT8_PEAK_TOPS, 4), "traffic": None,
