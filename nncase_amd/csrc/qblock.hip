@@ -1,7 +1,7 @@
 // Fused inverted-residual block: 1x1 expansion -> 3x3 depthwise -> 1x1 projection (+ input),
 // u8/u8, NHWC, one kernel.  The two expanded tensors are the largest of the block (6x the
 // input) and, run as three operators, are each written to and read back from HBM; here a
-// workgroup (8 waves) owns a 7x7 tile of OUTPUT pixels of one image and keeps everything
+// workgroup (8 or 16 waves) owns a 7x7 tile of OUTPUT pixels of one image and keeps everything
 // between the block's input and output in LDS:
 //
 //   input tile   the in-image part of the (6S+3)^2 input pixels the tile needs, as s8
@@ -17,8 +17,8 @@
 //
 // The stages are software-pipelined over the chunks: between two barriers a workgroup runs
 // E of chunk r, D of chunk r - 1 and P of chunk r - 2 on double-buffered tiles, and the
-// constants of the next step are prefetched global -> registers and committed to the other
-// half of a double-buffered LDS area at the end of the step.
+// constants travel global -> registers -> the other half of a double-buffered LDS area two
+// steps ahead of their use (one step is shorter than a memory round trip).
 //
 // Every stage uses the arithmetic of the stand-alone kernels (same zero-point identity, same
 // fp32 requantisation sequence), so the output bytes equal those of three separate operators.
@@ -49,8 +49,6 @@ struct nncase_hip_qblock_weights {
 
 namespace nnhip {
 
-constexpr int kBlkWaves = 8;
-constexpr int kBlkThreads = kBlkWaves * 64;
 constexpr int kBlkTile = 7;  // output tile edge (divides every MobileNet resolution from 112 down to 7)
 constexpr int kBlkRowB = 80; // bytes per pixel of the two mid tiles: 64 channels + 16 so that rows spread over the banks
 
@@ -77,18 +75,24 @@ struct HaloPix {
     int32_t nrsz;     // cin * zx' * zw' - zw' * sum_k x'
 };
 
-template <int S, int TPT>
-__global__ __launch_bounds__(kBlkThreads) void qblock_kernel(const BlockArgs a) {
+// NW = waves per workgroup: 8, or 16 for launches of few workgroups (one per compute unit or less), where the
+// stages are chains of LDS and matrix-core round trips and more, shorter chains per SIMD hide them better.
+template <int S, int TPT, int NW>
+__global__ __launch_bounds__(NW * 64) void qblock_kernel(const BlockArgs a) {
+    constexpr int kBlkWaves = NW, kBlkThreads = NW * 64;
+    constexpr int NQ = NW / 4; // waves per channel tile = pixel-group phases
     constexpr int ET = 4;                      // 16-channel tiles per chunk of expanded channels
     constexpr int HH = (kBlkTile - 1) * S + 3; // halo edge in input pixels
     constexpr int HP = HH * HH;
     constexpr int TP = kBlkTile * kBlkTile;
     constexpr int CE = ET * 16;
     constexpr int NG = (HP + 15) / 16;                        // pixel groups of the halo at most
-    constexpr int MAXU = (NG + 1) / 2;                        // expansion units (16 pixels x 16 channels) per wave at most
+    constexpr int MAXU = (NG + NQ - 1) / NQ;                  // expansion units (16 pixels x 16 channels) per wave at most
+    constexpr int DU = 4 / NQ;                                // depthwise units per wave
     constexpr int NS = (3 * ET * 1024 + TPT * 1024 + 9 * CE + 16 * CE + 16 * kBlkThreads - 1) / (16 * kBlkThreads); // vectors staged per thread
-    constexpr int TPW = TPT / 2; // projection tiles per wave: waves w and w + 4 share a pixel group
-    static_assert(TPT % 2 == 0 && kBlkWaves == 8, "two waves per pixel group, four channel tiles per chunk");
+    constexpr int NSPLIT = (NW == 16 && TPT % 4 == 0) ? 4 : 2; // waves that share a projection pixel group
+    constexpr int TPW = TPT / NSPLIT;                          // projection tiles per wave
+    static_assert(TPT % 2 == 0 && (NW == 8 || NW == 16), "four channel tiles per chunk, 2 or 4 waves per tile");
 
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     int32_t *cterm_p = reinterpret_cast<int32_t *>(smem);             // [TPT * 16]
@@ -103,7 +107,7 @@ __global__ __launch_bounds__(kBlkThreads) void qblock_kernel(const BlockArgs a) 
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int j = lane & 15, gq = lane >> 4;
     // Every stage gives a wave one 16-channel tile (wave & 3) of half of the pixel groups (wave >> 2).
-    const int wtile = wave & 3, whalf = wave >> 2;
+    const int wtile = wave & 3, whalf = wave >> 2; // whalf: 0 .. NQ - 1
 
     uint32_t b = blockIdx.x;
     const int tx = (int)(b % (uint32_t)a.tiles_x);
@@ -198,22 +202,22 @@ __global__ __launch_bounds__(kBlkThreads) void qblock_kernel(const BlockArgs a) 
     __syncthreads();
 
     // ---- what stays the same for every chunk -------------------------------------------------------------------
-    // E: the wave's units are pixel groups whalf, whalf + 2, ... of channel tile wtile
+    // E: the wave's units are pixel groups whalf, whalf + NQ, ... of channel tile wtile
     HaloPix ehp[MAXU];
 #pragma unroll
     for (int k = 0; k < MAXU; k++) {
-        const int g = whalf + 2 * k;
+        const int g = whalf + NQ * k;
         ehp[k] = hpix[min(g, NG - 1) * 16 + j];
         if (g >= ngroups) ehp[k].tile_off = -1;
     }
     const uint8_t *exrow = xin + (whalf * 16 + j) * a.xs + gq * 16; // + k * 32 * xs + ks * 64
     const int ecl = gq * (4 * ET) + wtile * 4;                        // the lane's 4 channels within the chunk
-    // D: pixel groups whalf and whalf + 2 of channel tile wtile; the lane's tap in k-step ks is ks * 4 + gq
-    int dxoff[2], dtap[3];
-    bool dpv[2];
+    // D: pixel groups whalf (+ NQ ...) of channel tile wtile; the lane's tap in k-step ks is ks * 4 + gq
+    int dxoff[DU], dtap[3];
+    bool dpv[DU];
 #pragma unroll
-    for (int k = 0; k < 2; k++) {
-        const int pp = (whalf + 2 * k) * 16 + j;
+    for (int k = 0; k < DU; k++) {
+        const int pp = (whalf + NQ * k) * 16 + j;
         dpv[k] = pp < TP;
         const int p = min(pp, TP - 1);
         const int py = p / kBlkTile, px = p - py * kBlkTile;
@@ -245,21 +249,38 @@ __global__ __launch_bounds__(kBlkThreads) void qblock_kernel(const BlockArgs a) 
     // Record r of the constants holds the expansion weights of chunk r, the depthwise weights of chunk r - 1 and
     // the projection weights of chunk r - 2: phase r runs E(r), D(r - 1) and P(r - 2) between two barriers, on
     // double-buffered tiles, so the three stages of different chunks overlap inside the workgroup.
+    // The constants travel global -> registers -> LDS two phases ahead of their use (one phase is shorter than a
+    // memory round trip): record r + 1 is committed to the other half of the LDS area at the end of phase r from
+    // the register set it was loaded into at the end of phase r - 2, and that set is reloaded with record r + 3.
+    // The loads are unconditional (a record index past the end re-reads the last one) so that the number of
+    // younger loads in flight is a compile-time constant and waiting for one set does not drain the other.
     const int nrec = a.nchunks + 2;
-    for (int r = 0; r < nrec; r++) {
-        const uint8_t *wb = wbuf + (r & 1) * a.chunk_bytes;
-        u32x4 stage[NS];
-        if (r + 1 < nrec) {
-            const u32x4 *src = reinterpret_cast<const u32x4 *>(a.blob + (size_t)(r + 1) * a.chunk_bytes);
+    u32x4 stage_a[NS], stage_b[NS];
+    auto issue = [&](int rec, u32x4 (&st)[NS]) {
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(a.blob + (size_t)min(rec, nrec - 1) * a.chunk_bytes);
+#pragma unroll
+        for (int i = 0; i < NS; i++) {
+            const int v = i * kBlkThreads + tid;
+            st[i] = src[v < nvec ? v : 0];
+        }
+    };
+    auto commit = [&](int rec, const u32x4 (&st)[NS]) {
+        if (rec < nrec) {
+            u32x4 *dst = reinterpret_cast<u32x4 *>(wbuf + (rec & 1) * a.chunk_bytes);
 #pragma unroll
             for (int i = 0; i < NS; i++) {
                 const int v = i * kBlkThreads + tid;
-                stage[i] = src[v < nvec ? v : 0];
+                if (v < nvec) dst[v] = st[i];
             }
         }
+    };
+    issue(1, stage_a);
+    issue(2, stage_b);
+    auto phase = [&](int r) {
+        const uint8_t *wb = wbuf + (r & 1) * a.chunk_bytes;
 
         // ---- P(r - 2): one k-step of the projection ----------------------------------------------------------
-        if (r >= 2) {
+        if (r >= 2 && whalf < NSPLIT) {
             const v4i xf = *reinterpret_cast<const v4i *>(dtile + (r & 1) * (64 * kBlkRowB) + (wtile * 16 + j) * kBlkRowB + gq * 16);
             rsp = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, xf, rsp, 0, 0, 0);
             const uint8_t *wfr = wb + a.off_p + whalf * (TPW * 1024) + lane * 16;
@@ -284,16 +305,16 @@ __global__ __launch_bounds__(kBlkThreads) void qblock_kernel(const BlockArgs a) 
             for (int r4 = 0; r4 < 4; r4++) cst[r4] = be[r4] - a.zxp_e * se[r4];
 #pragma unroll
             for (int k = 0; k < MAXU; k++) {
-                if (whalf + 2 * k < ngroups) {
+                if (whalf + NQ * k < ngroups) {
                     v4i acc = {0, 0, 0, 0};
 #pragma unroll
                     for (int ks = 0; ks < 3; ks++)
                         if (ks < a.ke) {
-                            const v4i xf = *reinterpret_cast<const v4i *>(exrow + k * 32 * a.xs + ks * 64);
+                            const v4i xf = *reinterpret_cast<const v4i *>(exrow + k * (NQ * 16) * a.xs + ks * 64);
                             acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[ks], xf, acc, 0, 0, 0);
                         }
                     uint32_t q[4];
-                    const HaloPix hpk = hpix[(whalf + 2 * k) * 16 + j];
+                    const HaloPix hpk = hpix[(whalf + NQ * k) * 16 + j];
                     int32_t v4[4];
 #pragma unroll
                     for (int r4 = 0; r4 < 4; r4++) v4[r4] = add3(acc[r4], cst[r4], hpk.nrsz);
@@ -328,7 +349,7 @@ __global__ __launch_bounds__(kBlkThreads) void qblock_kernel(const BlockArgs a) 
             for (int r4 = 0; r4 < 4; r4++) ct[r4] = bd[r4] - a.zxp_d * sd[r4] + a.kzz_d;
             const bool chv = (r - 1) * CE + dcl < a.mid;
 #pragma unroll
-            for (int k = 0; k < 2; k++) {
+            for (int k = 0; k < DU; k++) {
                 const uint8_t *xb = et + dxoff[k];
                 v4i aw = {0, 0, 0, 0}, a1 = {0, 0, 0, 0};
 #pragma unroll
@@ -343,19 +364,22 @@ __global__ __launch_bounds__(kBlkThreads) void qblock_kernel(const BlockArgs a) 
                 for (int r4 = 0; r4 < 4; r4++) v4[r4] = aw[r4] - a.zwp_d * a1[r4] + ct[r4];
                 requant4_u8_lowbyte(v4, a.ep_d, q);
                 const uint32_t packed = pack_low_bytes(q[0], q[1], q[2], q[3]) ^ 0x80808080u; // kept as s8
-                if (dpv[k]) *reinterpret_cast<uint32_t *>(dt + ((whalf + 2 * k) * 16 + j) * kBlkRowB + dcl) = chv ? packed : 0u;
+                if (dpv[k]) *reinterpret_cast<uint32_t *>(dt + ((whalf + NQ * k) * 16 + j) * kBlkRowB + dcl) = chv ? packed : 0u;
             }
         }
 
-        if (r + 1 < nrec) {
-            u32x4 *dst = reinterpret_cast<u32x4 *>(wbuf + ((r + 1) & 1) * a.chunk_bytes);
-#pragma unroll
-            for (int i = 0; i < NS; i++) {
-                const int v = i * kBlkThreads + tid;
-                if (v < nvec) dst[v] = stage[i];
-            }
-        }
+    };
+    for (int r = 0; r < nrec; r += 2) {
+        phase(r);
+        commit(r + 1, stage_a);
+        issue(r + 3, stage_a);
         __syncthreads();
+        if (r + 1 < nrec) {
+            phase(r + 1);
+            commit(r + 2, stage_b);
+            issue(r + 4, stage_b);
+            __syncthreads();
+        }
     }
 
     // ---- epilogue of the projection: pixel group wtile, the wave's TPW tiles are 4 * TPW consecutive channels per lane ----
@@ -366,29 +390,34 @@ __global__ __launch_bounds__(kBlkThreads) void qblock_kernel(const BlockArgs a) 
     const int pg = valid ? (img * a.out_h + oy) * a.out_w + ox : a.p.m;
     const int ch0 = gq * (4 * TPT) + whalf * (4 * TPW);
     // igemm_store_tile reads its constants at cterm + gq * 4 * TPW + nt * 4; they sit at cterm_p + ch0 + nt * 4
-    igemm_store_tile<TPW>(a.p, accp, rsp[0], pg, ch0, gq, cterm_p + ch0 - gq * (4 * TPW), nullptr);
+    if (whalf < NSPLIT) igemm_store_tile<TPW>(a.p, accp, rsp[0], pg, ch0, gq, cterm_p + ch0 - gq * (4 * TPW), nullptr);
 }
 
-template <int S, int TPT> static int launch_block_inst(nncase_hip_ctx *ctx, const BlockArgs &a, int blocks, size_t lds) {
+template <int S, int TPT, int NW> static int launch_block_inst(nncase_hip_ctx *ctx, const BlockArgs &a, int blocks, size_t lds) {
     // the dynamic LDS limit of a kernel is raised once per device (the attribute call is slow next to a launch)
     static int raised_on_device = -1;
     if (lds > 48 * 1024 && raised_on_device != ctx->device) {
-        NNHIP_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(&qblock_kernel<S, TPT>),
+        NNHIP_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(&qblock_kernel<S, TPT, NW>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
         raised_on_device = ctx->device;
     }
-    hipLaunchKernelGGL((qblock_kernel<S, TPT>), dim3(blocks), dim3(kBlkThreads), lds, ctx->stream, a);
+    hipLaunchKernelGGL((qblock_kernel<S, TPT, NW>), dim3(blocks), dim3(NW * 64), lds, ctx->stream, a);
     NNHIP_LAUNCH_CHECK(ctx, "qblock_kernel");
     return 0;
 }
 
+// 16 waves when the launch has at most two workgroups per compute unit (and the projection is narrow enough for
+// the register budget of 16 waves), else 8.
+static bool block_wide(const nncase_hip_ctx *ctx, int tpt, long long blocks) { return tpt <= 6 && blocks <= 2LL * ctx->compute_units; }
+
 template <int S> static int launch_block_s(nncase_hip_ctx *ctx, const BlockArgs &a, int tpt, int blocks, size_t lds) {
+    const bool wide = block_wide(ctx, tpt, blocks);
     switch (tpt) {
-    case 2: return launch_block_inst<S, 2>(ctx, a, blocks, lds);
-    case 4: return launch_block_inst<S, 4>(ctx, a, blocks, lds);
-    case 6: return launch_block_inst<S, 6>(ctx, a, blocks, lds);
-    case 10: return launch_block_inst<S, 10>(ctx, a, blocks, lds);
-    default: return launch_block_inst<S, 20>(ctx, a, blocks, lds);
+    case 2: return wide ? launch_block_inst<S, 2, 16>(ctx, a, blocks, lds) : launch_block_inst<S, 2, 8>(ctx, a, blocks, lds);
+    case 4: return wide ? launch_block_inst<S, 4, 16>(ctx, a, blocks, lds) : launch_block_inst<S, 4, 8>(ctx, a, blocks, lds);
+    case 6: return wide ? launch_block_inst<S, 6, 16>(ctx, a, blocks, lds) : launch_block_inst<S, 6, 8>(ctx, a, blocks, lds);
+    case 10: return launch_block_inst<S, 10, 8>(ctx, a, blocks, lds);
+    default: return launch_block_inst<S, 20, 8>(ctx, a, blocks, lds);
     }
 }
 
