@@ -286,7 +286,9 @@ extern "C" int nncase_hip_kmodel_load(nncase_hip_ctx_t *ctx, const void *data, s
         bd.in_channels = e.p[1], bd.mid_channels = e.p[0], bd.out_channels = pr.p[0];
         if (d.p[0] != e.p[0] || pr.p[1] != e.p[0] || !nncase_hip_qblock_supported(&bd)) continue;
         const hipf_tensor &te = m->tensors[e.output], &td = m->tensors[d.output];
-        if (!((uint64_t)td.dims[1] * td.dims[2] >= 196 && (uint64_t)te.dims[1] * te.dims[2] <= 784)) continue; // where it pays
+        const uint64_t tiles7 = (uint64_t)((td.dims[1] + 6) / 7) * ((td.dims[2] + 6) / 7);
+        // where it pays: mid-sized maps, at least 64 workgroups
+        if (!((uint64_t)td.dims[1] * td.dims[2] >= 196 && (uint64_t)te.dims[1] * te.dims[2] <= 784 && td.dims[0] * tiles7 >= 64)) continue;
         block_head[k] = 1;
         skipped[k + 1] = skipped[k + 2] = 1;
         k += 2;

@@ -424,10 +424,13 @@ class HipModel:
                     continue
                 if not ctx.qblock_supported(e.weights.shape[1], e.weights.shape[0], pr.weights.shape[0]):
                     continue
-                # Where it pays: mid-sized feature maps.  On large maps the three operators are bandwidth-bound
-                # kernels of their own that already run near the epilogue's arithmetic cost, on 7x7 maps a
-                # workgroup per image leaves most of the device idle.
-                if fuse_blocks != "all" and not (d.out_shape[1] * d.out_shape[2] >= 196 and e.out_shape[1] * e.out_shape[2] <= 784):
+                # Where it pays: mid-sized feature maps at batches that give the fused kernel at least 64 workgroups.
+                # On large maps the three operators are bandwidth-bound kernels of their own that already run near
+                # the epilogue's arithmetic cost, on 7x7 maps (and at small batches) a workgroup per tile leaves most
+                # of the device idle and the three latency-bound launches are quicker.
+                tiles = -(-d.out_shape[1] // 7) * -(-d.out_shape[2] // 7)        # 7x7 output tiles per image
+                if fuse_blocks != "all" and not (d.out_shape[1] * d.out_shape[2] >= 196 and e.out_shape[1] * e.out_shape[2] <= 784
+                                                 and (batch // lanes) * tiles >= 64):
                     continue
                 self.blocks[i] = (i + 1, i + 2, addn)
         for e, (d, pr, addn) in self.blocks.items():

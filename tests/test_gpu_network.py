@@ -189,9 +189,9 @@ def test_lanes_split_the_batch_bit_exact(hip_ctx, lanes, capture):
     rng = np.random.default_rng(3)
     qg = nb.quantize_graph(g, rng.random((32, 224, 224, 3), dtype=f32))
     x = np.random.default_rng(4).random((16, 224, 224, 3), dtype=f32)
-    one = nb.HipModel(hip_ctx, qg, 16, capture_graph=False)
+    one = nb.HipModel(hip_ctx, qg, 16, capture_graph=False, fuse_blocks="all")
     y1 = one.run(x)
-    many = nb.HipModel(hip_ctx, qg, 16, capture_graph=capture, lanes=lanes)
+    many = nb.HipModel(hip_ctx, qg, 16, capture_graph=capture, lanes=lanes, fuse_blocks="all")
     assert len(many.fn) == lanes * len(one.fn) and len(many.op_names) == len(one.op_names)
     y = many.run(x)
     assert np.array_equal(y.view(np.uint32), y1.view(np.uint32))
