@@ -313,14 +313,12 @@ __global__ __launch_bounds__(NW * 64) void qblock_kernel(const BlockArgs a) {
                             const v4i xf = *reinterpret_cast<const v4i *>(exrow + k * (NQ * 16) * a.xs + ks * 64);
                             acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[ks], xf, acc, 0, 0, 0);
                         }
-                    uint32_t q[4];
                     const HaloPix hpk = hpix[(whalf + NQ * k) * 16 + j];
                     int32_t v4[4];
 #pragma unroll
                     for (int r4 = 0; r4 < 4; r4++) v4[r4] = add3(acc[r4], cst[r4], hpk.nrsz);
-                    requant4_u8_lowbyte(v4, a.ep_e, q);
-                    if (hpk.tile_off >= 0)
-                        *reinterpret_cast<uint32_t *>(et + hpk.tile_off + ecl) = pack_low_bytes(q[0], q[1], q[2], q[3]) ^ 0x80808080u;
+                    const uint32_t q = requant4_u8_packed(v4, a.ep_e);
+                    if (hpk.tile_off >= 0) *reinterpret_cast<uint32_t *>(et + hpk.tile_off + ecl) = q ^ 0x80808080u;
                 }
             }
         }
@@ -358,12 +356,10 @@ __global__ __launch_bounds__(NW * 64) void qblock_kernel(const BlockArgs a) {
                     aw = __builtin_amdgcn_mfma_i32_16x16x64_i8(wfr[ks], xf, aw, 0, 0, 0);
                     a1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(ks == 2 ? done_last : done_f, xf, a1, 0, 0, 0);
                 }
-                uint32_t q[4];
                 int32_t v4[4];
 #pragma unroll
                 for (int r4 = 0; r4 < 4; r4++) v4[r4] = aw[r4] - a.zwp_d * a1[r4] + ct[r4];
-                requant4_u8_lowbyte(v4, a.ep_d, q);
-                const uint32_t packed = pack_low_bytes(q[0], q[1], q[2], q[3]) ^ 0x80808080u; // kept as s8
+                const uint32_t packed = requant4_u8_packed(v4, a.ep_d) ^ 0x80808080u; // kept as s8
                 if (dpv[k]) *reinterpret_cast<uint32_t *>(dt + ((whalf + NQ * k) * 16 + j) * kBlkRowB + dcl) = chv ? packed : 0u;
             }
         }

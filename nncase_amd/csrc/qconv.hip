@@ -149,6 +149,7 @@ int nnhip::make_epilogue(nncase_hip_ctx *ctx, Epilogue *ep, float sx, float sw, 
     ep->qhi = 255.f;
     ep->c1 = ep->c2 = 0.f;
     ep->fast = 0;
+    ep->full = 1;
     ep->out_mode = out_dtype == NNCASE_HIP_DT_U8 ? kOutU8 : (out_dtype == NNCASE_HIP_DT_I32 ? kOutI32 : kOutF32);
     NNHIP_REQUIRE(ctx, !(clamp_min > clamp_max), -EINVAL, "%s: fused clamp minimum above maximum", who);
     if (ep->out_mode != kOutU8) return 0;
@@ -167,6 +168,7 @@ int nnhip::make_epilogue(nncase_hip_ctx *ctx, Epilogue *ep, float sx, float sw, 
     ghi = ghi + ep->zy;
     ep->qlo = std::fmin(std::fmax((float)glo, 0.f), 255.f);
     ep->qhi = std::fmin(std::fmax((float)ghi, 0.f), 255.f);
+    ep->full = std::nearbyintf(ep->qlo) == 0.f && std::nearbyintf(ep->qhi) == 255.f;
     {
         const EpilogueKey key{ep->mult, ep->sy, ep->zy, ep->lo, ep->hi};
         std::lock_guard<std::mutex> lock(g_epilogues.mu);

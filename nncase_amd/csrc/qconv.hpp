@@ -56,6 +56,7 @@ struct Epilogue {
     // every step of the staircase, so the bytes are identical); fast == 0 when no such pair was found.
     float c1, c2;
     int fast;
+    int full; // rne(qlo) == 0 and rne(qhi) == 255: the saturating conversion to u8 is the whole clamp
 };
 
 // Second requantisation stage of a fused residual add:
@@ -120,20 +121,32 @@ __device__ __forceinline__ uint32_t requant_u8_lowbyte(float f, const Epilogue &
     return __float_as_uint(u + 12582912.0f);
 }
 
-// The requantised codes of four int32 accumulators (low bytes), by the one-instruction form when the host
-// has proved it equal to the three-rounding sequence for this layer.
-__device__ __forceinline__ void requant4_u8_lowbyte(const int32_t (&v)[4], const Epilogue &ep, uint32_t (&q)[4]) {
+// The requantised codes of four int32 accumulators, packed as bytes 0..3 of a dword: the one-instruction form
+// when the host has proved it equal to the three-rounding sequence for this layer.  v_cvt_pk_u8_f32 rounds to
+// the nearest integer (ties to even), saturates to [0, 255] and inserts the byte, so conversion, clamp and
+// packing are one instruction per code; rounding is monotone, so a clamp to [qlo, qhi] before it is needed
+// only when it is tighter than the saturation.
+__device__ __forceinline__ uint32_t requant4_u8_packed(const int32_t (&v)[4], const Epilogue &ep) {
+    uint32_t d = 0;
     if (ep.fast) {
+        if (ep.full) {
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-            float u = __builtin_fmaf((float)v[r], ep.c1, ep.c2);
-            u = __builtin_amdgcn_fmed3f(u, ep.qlo, ep.qhi);
-            q[r] = __float_as_uint(u + 12582912.0f);
+            for (int r = 0; r < 4; r++) d = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_fmaf((float)v[r], ep.c1, ep.c2), r, d);
+        } else {
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const float u = __builtin_fmaf((float)v[r], ep.c1, ep.c2);
+                d = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_amdgcn_fmed3f(u, ep.qlo, ep.qhi), r, d);
+            }
         }
     } else {
 #pragma unroll
-        for (int r = 0; r < 4; r++) q[r] = requant_u8_lowbyte((float)v[r] * ep.mult, ep);
+        for (int r = 0; r < 4; r++) {
+            const float u = div_rn((float)v[r] * ep.mult, ep.sy, ep.rsy) + ep.zy;
+            d = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_amdgcn_fmed3f(u, ep.qlo, ep.qhi), r, d);
+        }
     }
+    return d;
 }
 
 // Packs the low bytes of four dwords into one dword (3 byte-permutes).
@@ -143,11 +156,17 @@ __device__ __forceinline__ uint32_t pack_low_bytes(uint32_t b0, uint32_t b1, uin
     return lo | hi;
 }
 
-// Byte e of `res` added to the u8 code in the low byte of `q`; result in the low byte.
-__device__ __forceinline__ uint32_t residual_lowbyte(uint32_t q, uint32_t res, int e, const ResidualEpilogue &r) {
-    const float fa = ((float)(q & 0xffu) - r.zy) * r.sy;
-    const float fb = ((float)((res >> (8 * e)) & 0xffu) - r.zr) * r.sr;
-    return requant_u8_lowbyte(fa + fb, r.sum);
+// The four u8 codes of `q` plus the four of `res`, each pair dequantised, added and requantised; packed.
+__device__ __forceinline__ uint32_t residual4_packed(uint32_t q, uint32_t res, const ResidualEpilogue &r) {
+    uint32_t d = 0;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        const float fa = ((float)((q >> (8 * e)) & 0xffu) - r.zy) * r.sy;
+        const float fb = ((float)((res >> (8 * e)) & 0xffu) - r.zr) * r.sr;
+        const float u = div_rn(fa + fb, r.sum.sy, r.sum.rsy) + r.sum.zy;
+        d = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_amdgcn_fmed3f(u, r.sum.qlo, r.sum.qhi), e, d);
+    }
+    return d;
 }
 
 // a + b + c in one instruction (the compiler otherwise re-associates the zero-point

@@ -47,9 +47,7 @@ struct DwArgs {
 // Stores 4 adjacent channels of one output pixel; `o` is the element offset of the first.
 __device__ __forceinline__ void dw_store4(const DwArgs &a, uint32_t o, const int32_t (&v)[4]) {
     if (a.ep.out_mode == kOutU8) {
-        uint32_t b[4];
-        requant4_u8_lowbyte(v, a.ep, b);
-        *reinterpret_cast<uint32_t *>(reinterpret_cast<uint8_t *>(a.y) + o) = pack_low_bytes(b[0], b[1], b[2], b[3]);
+        *reinterpret_cast<uint32_t *>(reinterpret_cast<uint8_t *>(a.y) + o) = requant4_u8_packed(v, a.ep);
     } else if (a.ep.out_mode == kOutI32) {
         *reinterpret_cast<int4 *>(reinterpret_cast<int32_t *>(a.y) + o) = int4{v[0], v[1], v[2], v[3]};
     } else {

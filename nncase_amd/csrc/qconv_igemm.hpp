@@ -106,6 +106,16 @@ struct PixInfo {
     int iy0, ix0;
 };
 
+// One of two pixel records by value: a conditional expression over the named records would be an lvalue
+// and could be placed in memory.
+__device__ __forceinline__ PixInfo select_pix(bool first, PixInfo a, PixInfo b) {
+    PixInfo r;
+    r.base = first ? a.base : b.base;
+    r.iy0 = first ? a.iy0 : b.iy0;
+    r.ix0 = first ? a.ix0 : b.ix0;
+    return r;
+}
+
 template <int MODE> __device__ __forceinline__ PixInfo pix_info(const IgemmArgs &a, int p) {
     PixInfo pi;
     pi.iy0 = pi.ix0 = 0;
@@ -246,12 +256,10 @@ __device__ __forceinline__ void igemm_store_tile(const IgemmArgs &a, const v4i (
 #pragma unroll
         for (int nt = 0; nt < T; nt++) {
             const v4i ct = *reinterpret_cast<const v4i *>(cterm + gq * (4 * T) + nt * 4);
-            uint32_t b[4];
             int32_t v[4];
 #pragma unroll
             for (int r = 0; r < 4; r++) v[r] = add3(acc[nt][r], ct[r], nrsz);
-            requant4_u8_lowbyte(v, a.ep, b);
-            packed[nt] = pack_low_bytes(b[0], b[1], b[2], b[3]);
+            packed[nt] = requant4_u8_packed(v, a.ep);
         }
         if (a.lut) { // fused unary operator: one LDS byte read per output
 #pragma unroll
@@ -274,10 +282,7 @@ __device__ __forceinline__ void igemm_store_tile(const IgemmArgs &a, const v4i (
                     for (int r = 0; r < 4; r++)
                         if (ch0 + nt * 4 + r < a.n) rv |= (uint32_t)ro[nt * 4 + r] << (8 * r);
                 }
-                uint32_t b[4];
-#pragma unroll
-                for (int r = 0; r < 4; r++) b[r] = residual_lowbyte(packed[nt] >> (8 * r), rv, r, a.rep);
-                packed[nt] = pack_low_bytes(b[0], b[1], b[2], b[3]);
+                packed[nt] = residual4_packed(packed[nt], rv, a.rep);
             }
         }
         if (((a.ldy | a.y_coff) & 3) == 0 && ch0 + 4 * T <= a.n) {
@@ -402,16 +407,20 @@ __global__ __launch_bounds__(kThreads, 2) void qconv_igemm_kernel(const IgemmArg
             const int s0 = kci * a.kc_steps;
             const int s1 = min(a.ksteps, s0 + a.kc_steps);
             for (int ks = s0; ks < s1; ks++) {
-                // issue the loads of the next fragment before multiplying this one
-                if (ks + 1 < a.ksteps) {
+                // Issue the loads of the next fragment before multiplying this one: the next k-step of this pixel
+                // tile, or the first of the next tile.  The loads are issued on every trip (after the last tile
+                // they re-read a valid address and the data is dropped): loads complete in order, and only a
+                // compile-time count of younger loads lets the wait below spare the ones just issued.
+                {
+                    const bool same_tile = ks + 1 < a.ksteps;
+                    if (!same_tile) {
+                        const int mtn = mt_next < a.num_mtiles ? mt_next : mt;
 #pragma unroll
-                    for (int rg = 0; rg < RG; rg++) fnxt[rg] = load_act<MODE>(a, pcur[rg], (ks + 1) * 4 + gq);
-                } else if (mt_next < a.num_mtiles) {
-#pragma unroll
-                    for (int rg = 0; rg < RG; rg++) {
-                        pnxt[rg] = pix_info<MODE>(a, mt_next * pix_per_block + (wave * RG + rg) * 16 + j);
-                        fnxt[rg] = load_act<MODE>(a, pnxt[rg], gq);
+                        for (int rg = 0; rg < RG; rg++) pnxt[rg] = pix_info<MODE>(a, mtn * pix_per_block + (wave * RG + rg) * 16 + j);
                     }
+                    const int kc_next = same_tile ? (ks + 1) * 4 + gq : gq;
+#pragma unroll
+                    for (int rg = 0; rg < RG; rg++) fnxt[rg] = load_act<MODE>(a, select_pix(same_tile, pcur[rg], pnxt[rg]), kc_next);
                 }
                 v4i xf[RG]; // the slice loaded one step ago, now needed
 #pragma unroll
@@ -647,9 +656,12 @@ template <int T, int RG, int MODE> int launch_trg(nncase_hip_ctx *ctx, const Ige
 }
 
 template <int T, int MODE> int launch_t(nncase_hip_ctx *ctx, const IgemmArgs &a, int nchunks, int rg) {
+    // only the combinations choose_rg can return are built: the others would need more registers than a wave has
     if (rg == 1) return launch_trg<T, 1, MODE>(ctx, a, nchunks);
-    if (rg == 2) return launch_trg<T, 2, MODE>(ctx, a, nchunks);
-    if constexpr (T <= 8) {
+    if constexpr (T <= 6) {
+        if (rg == 2) return launch_trg<T, 2, MODE>(ctx, a, nchunks);
+    }
+    if constexpr (T == 1) {
         if (rg == 4) return launch_trg<T, 4, MODE>(ctx, a, nchunks);
     }
     return fail(ctx, -EINVAL, "igemm: no kernel for %d tiles x %d pixel groups", T, rg);

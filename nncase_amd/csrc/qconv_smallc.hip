@@ -134,10 +134,8 @@ template <int C, int KW, int KH> __global__ __launch_bounds__(kScThreads) void q
             uint32_t q[4];
 #pragma unroll
             for (int d = 0; d < 4; d++) {
-                uint32_t b[4];
                 const int32_t v4[4] = {acc[d * 4], acc[d * 4 + 1], acc[d * 4 + 2], acc[d * 4 + 3]};
-                requant4_u8_lowbyte(v4, a.ep, b);
-                q[d] = pack_low_bytes(b[0], b[1], b[2], b[3]);
+                q[d] = requant4_u8_packed(v4, a.ep);
             }
             uint8_t *yo = reinterpret_cast<uint8_t *>(a.y) + obase + ocb;
             if (nvalid == 16 && (a.oc & 15) == 0) {

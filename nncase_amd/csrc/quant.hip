@@ -126,11 +126,13 @@ __global__ __launch_bounds__(kEwThreads) void qadd_kernel(const uint8_t *__restr
                                                           float zb, float sb, const Epilogue ep, int vec_ok) {
     const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t nthreads = (size_t)gridDim.x * blockDim.x;
-    auto one = [&](uint32_t qa, uint32_t qb) -> uint32_t {
+    // the requantised sum before rounding to a byte
+    auto value = [&](uint32_t qa, uint32_t qb) -> float {
         const float fa = ((float)qa - za) * sa;
         const float fb = ((float)qb - zb) * sb;
-        return requant_u8_lowbyte(fa + fb, ep);
+        return __builtin_amdgcn_fmed3f(div_rn(fa + fb, ep.sy, ep.rsy) + ep.zy, ep.qlo, ep.qhi);
     };
+    auto one = [&](uint32_t qa, uint32_t qb) -> uint32_t { return __builtin_amdgcn_cvt_pk_u8_f32(value(qa, qb), 0, 0u); };
     // 16 bytes per thread per step
     const size_t nvec = vec_ok ? count / 16 : 0;
     for (size_t i = tid; i < nvec; i += nthreads) {
@@ -140,10 +142,10 @@ __global__ __launch_bounds__(kEwThreads) void qadd_kernel(const uint8_t *__restr
         uint32_t wo[4];
 #pragma unroll
         for (int d = 0; d < 4; d++) {
-            uint32_t r[4];
+            uint32_t w = 0;
 #pragma unroll
-            for (int e = 0; e < 4; e++) r[e] = one((wa[d] >> (8 * e)) & 0xffu, (wb[d] >> (8 * e)) & 0xffu);
-            wo[d] = pack_low_bytes(r[0], r[1], r[2], r[3]);
+            for (int e = 0; e < 4; e++) w = __builtin_amdgcn_cvt_pk_u8_f32(value((wa[d] >> (8 * e)) & 0xffu, (wb[d] >> (8 * e)) & 0xffu), e, w);
+            wo[d] = w;
         }
         *reinterpret_cast<uint4 *>(out + i * 16) = uint4{wo[0], wo[1], wo[2], wo[3]};
     }
