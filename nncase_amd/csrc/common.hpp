@@ -114,9 +114,10 @@ inline FastDiv make_fastdiv(uint32_t d) {
 
 __device__ __forceinline__ uint32_t fastdiv(uint32_t n, const FastDiv &f) {
     // exact for n < 2^31 (Granlund-Montgomery / Hacker's Delight 10-9 form)
-    if (f.div == 1) return n;
+    // (a select, not a branch, for the divisor 1: callers count on straight-line code around their loads)
     const uint32_t t = __umulhi(n, f.mul);
-    return (t + ((n - t) >> 1)) >> (f.shift - 1);
+    const uint32_t q = (t + ((n - t) >> 1)) >> ((f.shift - 1) & 31u);
+    return f.div == 1 ? n : q;
 }
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }

@@ -13,6 +13,9 @@ struct nncase_hip_weights {
     int tiles = 0;          // 16-channel MFMA tiles per channel chunk (T)
     int nchunks = 0;        // channel chunks per group
     int kc_steps = 0;       // k-steps staged in LDS at a time
+    // igemm, reductions of at most 32: the spare half of the only k-step holds -(zw - 128) against a second copy
+    // of the activations, which makes the weight zero point's share of the product part of the multiplication
+    int fold = 0;
     int64_t pixels_hint = 0; // output pixels per call the tiling was planned for (0 = unknown)
     int32_t zw = 0;
     float sw = 1.f;
@@ -135,14 +138,20 @@ __device__ __forceinline__ uint32_t requant4_u8_packed(const int32_t (&v)[4], co
         } else {
 #pragma unroll
             for (int r = 0; r < 4; r++) {
-                const float u = __builtin_fmaf((float)v[r], ep.c1, ep.c2);
+                int32_t vr = v[r]; // hidden from the optimiser for the reason given below
+                asm volatile("" : "+v"(vr));
+                const float u = __builtin_fmaf((float)vr, ep.c1, ep.c2);
                 d = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_amdgcn_fmed3f(u, ep.qlo, ep.qhi), r, d);
             }
         }
     } else {
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-            const float u = div_rn((float)v[r] * ep.mult, ep.sy, ep.rsy) + ep.zy;
+            // (the value is hidden from the optimiser here: sharing its conversion with the branches above, it
+            // converts every accumulator of a tile ahead of the branch and keeps them all in registers)
+            int32_t vr = v[r];
+            asm volatile("" : "+v"(vr));
+            const float u = div_rn((float)vr * ep.mult, ep.sy, ep.rsy) + ep.zy;
             d = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_amdgcn_fmed3f(u, ep.qlo, ep.qhi), r, d);
         }
     }

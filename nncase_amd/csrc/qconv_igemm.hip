@@ -53,6 +53,8 @@ int prepack_igemm(nncase_hip_ctx *ctx, nncase_hip_weights *w, const uint8_t *w_o
     w->ksteps = ceil_div(w->k, 64);
     const int max_tiles = (w->g_ic % 4 == 0) ? 16 : 4;
     plan_igemm(w->g_oc, w->ksteps, max_tiles, w->pixels_hint, ctx->compute_units, &w->tiles, &w->nchunks, &w->kc_steps);
+    // -(zw - 128) has to be an s8 value
+    w->fold = w->ksteps == 1 && w->k <= 32 && w->zw >= 1;
     const size_t group_bytes = (size_t)w->nchunks * w->ksteps * w->tiles * 1024;
     w->packed_bytes = group_bytes * w->groups;
     std::vector<uint8_t> packed(w->packed_bytes);
@@ -66,7 +68,7 @@ int prepack_igemm(nncase_hip_ctx *ctx, nncase_hip_weights *w, const uint8_t *w_o
             return wg[((size_t)oc * g_ic + ic) * kh * kw + tap]; // OIHW: tap = ky * kw + kx
         };
         pack_group(packed.data() + g * group_bytes, wsum.data() + (size_t)g * w->g_oc, w->g_oc, w->k, w->ksteps, w->tiles,
-                   w->nchunks, w_at);
+                   w->nchunks, w_at, w->fold != 0, 128 - w->zw);
     }
     NNHIP_HIP(ctx, hipMalloc(&w->d_packed, w->packed_bytes));
     NNHIP_HIP(ctx, hipMalloc((void **)&w->d_wsum, sizeof(int32_t) * w->out_channels));
@@ -124,6 +126,8 @@ int launch_qconv_igemm(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_hip_w
     a.kc_steps = w->kc_steps;
     a.ldx = w->in_channels;
     a.ldy = w->out_channels;
+    // the store offsets of one pixel tile (at most 512 pixels of 4-byte channels) are 31-bit byte offsets
+    NNHIP_REQUIRE(ctx, w->out_channels < (1 << 20), -EINVAL, "qconv2d: %d output channels are not supported", w->out_channels);
     a.g_ic = w->g_ic;
     a.in_h = c->in_h;
     a.in_w = c->in_w;
@@ -140,6 +144,8 @@ int launch_qconv_igemm(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_hip_w
     a.d_gic = make_fastdiv((uint32_t)w->g_ic);
     a.zxp = c->x_qp.zero_point - 128;
     a.zwp = w->zw - 128;
+    a.zwp_rows = w->fold ? 0 : a.zwp;
+    a.kc_mask = w->fold ? 1 : -1;
     a.zx_splat = (uint32_t)(c->x_qp.zero_point & 0xff) * 0x01010101u;
     {
         const int rc = make_epilogue(ctx, &a.ep, c->x_qp.scale, w->sw, c->y_qp, c->clamp_min, c->clamp_max, c->out_dtype, "qconv2d");

@@ -64,6 +64,8 @@ struct IgemmArgs {
     int kw, stride_h, stride_w, dil_h, dil_w, pad_h, pad_w;
     FastDiv d_ohow, d_ow, d_kw, d_gic;
     int zxp, zwp;          // zx - 128, zw - 128
+    int zwp_rows;          // zwp where the kernel still owes -zwp * (sum of x') per pixel, 0 where the weights carry it
+    int kc_mask;           // applied to the index of the 16-byte slice a lane loads: 1 with such weights, else all ones
     uint32_t zx_splat;     // zx in all four bytes
     int num_mtiles;
     Epilogue ep;
@@ -76,9 +78,11 @@ struct IgemmArgs {
 //   reduction index k = (ky * kw + kx) * g_ic + ic.
 // Fragment (chunk, ks, nt): byte (kg * 16 + i) * 16 + b holds the weight of
 //   channel chunk*16T + (i / 4) * 4T + nt * 4 + (i % 4) at k = ks*64 + kg*16 + b,
-// re-biased to s8, or 0 outside the real channel / reduction range.
+// re-biased to s8, or 0 outside the real channel / reduction range.  With fold (k <= 32, one k-step) the slots
+// 32 + kk, kk < k, hold the s8 value fold_value instead: the kernel feeds them a second copy of the activations.
 template <typename WAt>
-inline void pack_group(uint8_t *dst, int32_t *wsum, int g_oc, int k, int ksteps, int tiles, int nchunks, WAt w_at) {
+inline void pack_group(uint8_t *dst, int32_t *wsum, int g_oc, int k, int ksteps, int tiles, int nchunks, WAt w_at, bool fold = false,
+                       int fold_value = 0) {
     for (int oc = 0; oc < g_oc; oc++) {
         int32_t s = 0;
         for (int kk = 0; kk < k; kk++) s += (int32_t)(int8_t)(w_at(oc, kk) ^ 0x80);
@@ -95,6 +99,7 @@ inline void pack_group(uint8_t *dst, int32_t *wsum, int g_oc, int k, int ksteps,
                             const int kk = ks * 64 + kg * 16 + b;
                             uint8_t v = 0;
                             if (oc < g_oc && kk < k) v = (uint8_t)(w_at(oc, kk) ^ 0x80);
+                            if (fold && kk >= 32 && kk - 32 < k) v = (uint8_t)(int8_t)fold_value;
                             frag[(kg * 16 + i) * 16 + b] = v;
                         }
                     }
@@ -244,21 +249,26 @@ struct __attribute__((packed, aligned(1))) U32Unaligned {
 // Epilogue of one 16-pixel x 16T-channel tile of a wave: zero-point correction, requantisation
 // (optionally a byte table and a residual add behind it), NHWC store.  Lane (j, gq) holds pixel p
 // and the 4T consecutive channels from ch0 on; rowsum is the pixel's sum of x' over the reduction.
-template <int T>
+// OWED says what acc still lacks: kOwesAll, the channel constant (read at cterm) and -zwp * rowsum; kOwesRows, only
+// -zwp_rows * rowsum; kOwesNothing.
+enum { kOwesAll = 0, kOwesRows = 1, kOwesNothing = 2 };
+template <int T, int OWED = kOwesAll>
 __device__ __forceinline__ void igemm_store_tile(const IgemmArgs &a, const v4i (&acc)[T], int32_t rowsum, int p, int ch0, int gq,
                                                  const int32_t *cterm, const uint8_t *lutl) {
     if (!(p < a.m && ch0 < a.n)) return;
-    const int32_t nrsz = -a.zwp * rowsum;
+    const int32_t nrsz = OWED == kOwesAll ? -a.zwp * rowsum : (OWED == kOwesRows ? -a.zwp_rows * rowsum : 0);
     const size_t obase = (size_t)p * a.ldy + a.y_coff + ch0;
     if (a.ep.out_mode == kOutU8) {
         uint8_t *yo = reinterpret_cast<uint8_t *>(a.y) + obase;
         uint32_t packed[T];
 #pragma unroll
         for (int nt = 0; nt < T; nt++) {
-            const v4i ct = *reinterpret_cast<const v4i *>(cterm + gq * (4 * T) + nt * 4);
+            v4i ct = {0, 0, 0, 0};
+            if (OWED == kOwesAll) ct = *reinterpret_cast<const v4i *>(cterm + gq * (4 * T) + nt * 4);
             int32_t v[4];
 #pragma unroll
-            for (int r = 0; r < 4; r++) v[r] = add3(acc[nt][r], ct[r], nrsz);
+            for (int r = 0; r < 4; r++)
+                v[r] = OWED == kOwesAll ? add3(acc[nt][r], ct[r], nrsz) : (OWED == kOwesRows ? acc[nt][r] + nrsz : acc[nt][r]);
             packed[nt] = requant4_u8_packed(v, a.ep);
         }
         if (a.lut) { // fused unary operator: one LDS byte read per output
@@ -314,11 +324,13 @@ __device__ __forceinline__ void igemm_store_tile(const IgemmArgs &a, const v4i (
         uint32_t *yo = reinterpret_cast<uint32_t *>(a.y) + obase;
 #pragma unroll
         for (int nt = 0; nt < T; nt++) {
-            const v4i ct = *reinterpret_cast<const v4i *>(cterm + gq * (4 * T) + nt * 4);
+            v4i ct = {0, 0, 0, 0};
+            if (OWED == kOwesAll) ct = *reinterpret_cast<const v4i *>(cterm + gq * (4 * T) + nt * 4);
             uint32_t o[4];
 #pragma unroll
             for (int r = 0; r < 4; r++) {
-                const int32_t v = add3(acc[nt][r], ct[r], nrsz);
+                const int32_t v =
+                    OWED == kOwesAll ? add3(acc[nt][r], ct[r], nrsz) : (OWED == kOwesRows ? acc[nt][r] + nrsz : acc[nt][r]);
                 if (a.ep.out_mode == kOutI32) o[r] = (uint32_t)v;
                 else o[r] = __float_as_uint(clamp_ref((float)v * a.ep.mult, a.ep.lo, a.ep.hi));
             }
@@ -333,8 +345,10 @@ __device__ __forceinline__ void igemm_store_tile(const IgemmArgs &a, const v4i (
     }
 }
 
+// Blocks per compute unit the register allocation has to leave room for: four (at most 128 registers) for the
+// shapes that fit comfortably, so that the scheduler does not trade the occupancy away for longer live ranges.
 template <int T, int RG, int MODE>
-__global__ __launch_bounds__(kThreads, 2) void qconv_igemm_kernel(const IgemmArgs a) {
+__global__ void __launch_bounds__(kThreads, ((RG == 1 && T <= 12) || MODE == kRows16) ? 4 : 2) qconv_igemm_kernel(const IgemmArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     int32_t *cterm = reinterpret_cast<int32_t *>(smem); // [T * 16]
     uint8_t *lutl = smem + T * 16 * sizeof(int32_t);    // [256] byte table of the fused unary operator
@@ -385,19 +399,27 @@ __global__ __launch_bounds__(kThreads, 2) void qconv_igemm_kernel(const IgemmArg
 #pragma unroll
         for (int rg = 0; rg < RG; rg++) {
             pcur[rg] = pix_info<MODE>(a, mt * pix_per_block + (wave * RG + rg) * 16 + j);
-            fcur[rg] = load_act<MODE>(a, pcur[rg], gq);
+            fcur[rg] = load_act<MODE>(a, pcur[rg], gq & a.kc_mask);
         }
     }
+#pragma clang loop unroll(disable)
     for (; mt < a.num_mtiles; mt += gridDim.x) {
+        // The sums start from the per-channel constant of the zero-point identity, read from LDS for every tile
+        // (the offset is hidden from the optimiser: kept in registers across tiles the constants would cost 4T of them).
         v4i acc[RG][T];
         v4i rs[RG];
+        int ct_off = gq * (4 * T);
+        asm volatile("" : "+v"(ct_off));
 #pragma unroll
-        for (int rg = 0; rg < RG; rg++) {
-            rs[rg] = v4i{0, 0, 0, 0};
+        for (int nt = 0; nt < T; nt++) {
+            const v4i ct = *reinterpret_cast<const v4i *>(cterm + ct_off + nt * 4);
 #pragma unroll
-            for (int nt = 0; nt < T; nt++) acc[rg][nt] = v4i{0, 0, 0, 0};
+            for (int rg = 0; rg < RG; rg++) acc[rg][nt] = ct;
         }
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) rs[rg] = v4i{0, 0, 0, 0};
         const int mt_next = mt + gridDim.x;
+#pragma clang loop unroll(disable)
         for (int kci = 0; kci < nkc; kci++) {
             if (nkc > 1) {
                 __syncthreads(); // previous stage fully consumed
@@ -406,6 +428,7 @@ __global__ __launch_bounds__(kThreads, 2) void qconv_igemm_kernel(const IgemmArg
             }
             const int s0 = kci * a.kc_steps;
             const int s1 = min(a.ksteps, s0 + a.kc_steps);
+#pragma clang loop unroll(disable)
             for (int ks = s0; ks < s1; ks++) {
                 // Issue the loads of the next fragment before multiplying this one: the next k-step of this pixel
                 // tile, or the first of the next tile.  The loads are issued on every trip (after the last tile
@@ -418,16 +441,18 @@ __global__ __launch_bounds__(kThreads, 2) void qconv_igemm_kernel(const IgemmArg
 #pragma unroll
                         for (int rg = 0; rg < RG; rg++) pnxt[rg] = pix_info<MODE>(a, mtn * pix_per_block + (wave * RG + rg) * 16 + j);
                     }
-                    const int kc_next = same_tile ? (ks + 1) * 4 + gq : gq;
+                    const int kc_next = (same_tile ? (ks + 1) * 4 + gq : gq) & a.kc_mask;
 #pragma unroll
                     for (int rg = 0; rg < RG; rg++) fnxt[rg] = load_act<MODE>(a, select_pix(same_tile, pcur[rg], pnxt[rg]), kc_next);
                 }
                 v4i xf[RG]; // the slice loaded one step ago, now needed
 #pragma unroll
                 for (int rg = 0; rg < RG; rg++) xf[rg] = finish_act(fcur[rg]);
+                { // sum of x' per pixel (not needed where the weights carry the term it is for; a branch here costs more)
 #pragma unroll
-                for (int rg = 0; rg < RG; rg++)
-                    rs[rg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, xf[rg], rs[rg], 0, 0, 0);
+                    for (int rg = 0; rg < RG; rg++)
+                        rs[rg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, xf[rg], rs[rg], 0, 0, 0);
+                }
                 const uint8_t *wstep = wlds + (size_t)(ks - s0) * T * 1024 + lane * 16;
 #pragma unroll
                 for (int nt = 0; nt < T; nt++) {
@@ -441,11 +466,18 @@ __global__ __launch_bounds__(kThreads, 2) void qconv_igemm_kernel(const IgemmArg
             }
         }
 
-        // ---- epilogue: zero-point correction, requantisation, NHWC store ----
+        // ---- epilogue: the rest of the zero-point correction, requantisation, NHWC store ----
+        // (written out for both cases: one epilogue behind a conditional correction would keep two copies of the sums)
         const int ch0 = ch_base + gq * (4 * T); // first of this lane's 4T channels
+        if (a.zwp_rows != 0) {
 #pragma unroll
-        for (int rg = 0; rg < RG; rg++)
-            igemm_store_tile<T>(a, acc[rg], rs[rg][0], mt * pix_per_block + (wave * RG + rg) * 16 + j, ch0, gq, cterm, lutl);
+            for (int rg = 0; rg < RG; rg++)
+                igemm_store_tile<T, kOwesRows>(a, acc[rg], rs[rg][0], mt * pix_per_block + (wave * RG + rg) * 16 + j, ch0, gq, cterm, lutl);
+        } else {
+#pragma unroll
+            for (int rg = 0; rg < RG; rg++)
+                igemm_store_tile<T, kOwesNothing>(a, acc[rg], 0, mt * pix_per_block + (wave * RG + rg) * 16 + j, ch0, gq, cterm, lutl);
+        }
 #pragma unroll
         for (int rg = 0; rg < RG; rg++) pcur[rg] = pnxt[rg];
     }

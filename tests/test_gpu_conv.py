@@ -162,6 +162,22 @@ def test_extreme_values_and_zero_points(hip_ctx):
             assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("zw", [0, 1, 2, 127, 128, 129, 254, 255])
+@pytest.mark.parametrize("cin,k,pad", [(16, 1, 0), (24, 1, 0), (32, 1, 0), (3, 3, 1), (8, 2, 0), (33, 1, 0), (48, 1, 0)])
+def test_short_reductions_for_every_weight_zero_point(hip_ctx, zw, cin, k, pad):
+    """Reductions of at most 32 carry the weight zero point's term inside the multiplication (except zw = 0, whose
+    negative is no s8 value); just above 32 they do not.  Random and saturated operands, padding included."""
+    run_case(hip_ctx, 2, cin, 9, 11, 40, k, k, (1, 1), ((pad, pad), (pad, pad)), (1, 1), 1, seed=zw * 7 + cin, zx=zw ^ 0x5a, zw=zw,
+             modes=("u8", "i32"))
+    for fill_x, fill_w in ((255, 255), (255, 0), (0, 255)):
+        x = np.full((1, cin, 5, 5), fill_x, np.uint8)
+        w = np.full((20, cin, k, k), fill_w, np.uint8)
+        args = ((1, 1), ((pad, pad), (pad, pad)), (1, 1), 1, FULL, qp(3, 1.0), qp(zw, 1.0), None, np.int32)
+        got = K.conv2d(x, w, None, *args, ctx=hip_ctx)
+        want = O.qconv2d(x, w, None, 3, 1.0, zw, 1.0, stride=(1, 1), padding=((pad, pad), (pad, pad)), out_mode=O.OUT_I32)
+        assert np.array_equal(got, want)
+
+
 def test_config2_conv_block(hip_ctx):
     """BASELINE config 2 at batch 1: 1x1 64->144, 3x3 depthwise, 1x1 144->64 on 56x56, ReLU6, per-tensor PTQ."""
     rng = np.random.default_rng(1)
