@@ -37,27 +37,27 @@ INT8_PEAK_TOPS = 5000.0    # dense int8 MFMA
 # are recorded here and reported only for the configuration they were measured on.
 MEASURED_TRAFFIC_B64 = {
     "dequantize": 354798,
-    "dw3x3<S=1>": 27720128,
-    "dw3x3<S=2>": 48868351,
-    "qblock+add<S=1,P=2>": 4925425,
-    "qblock+add<S=1,P=4>": 2714966,
-    "qblock+add<S=1,P=6>": 4561322,
-    "qblock<S=1,P=6>": 3254931,
-    "qblock<S=2,P=4>": 3328574,
-    "qconv_igemm+add<T=1,RG=1,rows16>": 5327013,
-    "qconv_igemm+add<T=2,RG=2,rows16>": 39152800,
-    "qconv_igemm<T=1,RG=1,rows16>": 6756181,
-    "qconv_igemm<T=1,RG=4,rows16>": 38703365,
-    "qconv_igemm<T=12,RG=1,rows16>": 9261590,
-    "qconv_igemm<T=2,RG=1,rows16>": 8967905,
-    "qconv_igemm<T=2,RG=2,rows16>": 24258555,
-    "qconv_igemm<T=5,RG=1,rows16>": 5191633,
-    "qconv_igemm<T=6,RG=1,rows16>": 8703165,
-    "qconv_igemm<T=6,RG=2,rows16>": 90245847,
-    "qconv_igemm<T=9,RG=1,vec8>": 34022000,
-    "qconv_smallc<C=3>": 38853721,
+    "dw3x3<S=1>": 27893537,
+    "dw3x3<S=2>": 48887398,
+    "qblock+add<S=1,P=2>": 4947885,
+    "qblock+add<S=1,P=4>": 2672009,
+    "qblock+add<S=1,P=6>": 4553132,
+    "qblock<S=1,P=6>": 3246740,
+    "qblock<S=2,P=4>": 3349051,
+    "qconv_igemm+add<T=1,RG=1,rows16>": 5325989,
+    "qconv_igemm+add<T=2,RG=2,rows16>": 40227168,
+    "qconv_igemm<T=1,RG=1,rows16>": 6751830,
+    "qconv_igemm<T=1,RG=4,rows16>": 38742270,
+    "qconv_igemm<T=12,RG=1,rows16>": 9312780,
+    "qconv_igemm<T=2,RG=1,rows16>": 8987358,
+    "qconv_igemm<T=2,RG=2,rows16>": 24278775,
+    "qconv_igemm<T=5,RG=1,rows16>": 5195728,
+    "qconv_igemm<T=6,RG=1,rows16>": 8725689,
+    "qconv_igemm<T=6,RG=2,rows16>": 90258260,
+    "qconv_igemm<T=9,RG=1,vec8>": 34055978,
+    "qconv_smallc<C=3>": 38872277,
     "qglobal_avgpool": 4121905,
-    "quantize": 48218539,
+    "quantize": 48219691,
 }
 
 

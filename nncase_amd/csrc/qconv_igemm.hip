@@ -126,8 +126,6 @@ int launch_qconv_igemm(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_hip_w
     a.kc_steps = w->kc_steps;
     a.ldx = w->in_channels;
     a.ldy = w->out_channels;
-    // the store offsets of one pixel tile (at most 512 pixels of 4-byte channels) are 31-bit byte offsets
-    NNHIP_REQUIRE(ctx, w->out_channels < (1 << 20), -EINVAL, "qconv2d: %d output channels are not supported", w->out_channels);
     a.g_ic = w->g_ic;
     a.in_h = c->in_h;
     a.in_w = c->in_w;
