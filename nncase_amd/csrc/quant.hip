@@ -172,6 +172,40 @@ __global__ __launch_bounds__(kEwThreads) void qglobal_avgpool_kernel(const uint8
     out[idx] = (uint8_t)(int32_t)rintf(t);
 }
 
+// The same for 4 adjacent channels per thread (dword loads), the loads of 64 pixels (a whole 7x7 map) issued before
+// their values are added: with one or two waves per SIMD the kernel is a chain of memory round trips, and this
+// leaves one per 64 pixels.  Each channel's additions keep their order.
+__global__ __launch_bounds__(kEwThreads) void qglobal_avgpool4_kernel(const uint8_t *__restrict__ x, uint8_t *__restrict__ out,
+                                                                      int batch, int hw, int channels, float zx, float sx,
+                                                                      float zy, float sy) {
+    const int cq = channels >> 2;
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= batch * cq) return;
+    const int n = idx / cq, c = (idx - n * cq) * 4;
+    const uint8_t *p = x + (size_t)n * hw * channels + c;
+    float value[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int i0 = 0; i0 < hw; i0 += 64) {
+        uint32_t d[64];
+#pragma unroll
+        for (int k = 0; k < 64; k++) d[k] = *reinterpret_cast<const uint32_t *>(p + (size_t)min(i0 + k, hw - 1) * channels);
+#pragma unroll
+        for (int k = 0; k < 64; k++)
+            if (i0 + k < hw) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) value[e] = value[e] + ((float)((d[k] >> (8 * e)) & 0xffu) - zx) * sx;
+            }
+    }
+    uint32_t q = 0;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        const float mean = value[e] / (float)hw;
+        float t = mean / sy + zy;
+        t = fminf(fmaxf(t, 0.f), 255.f);
+        q |= (uint32_t)(int32_t)rintf(t) << (8 * e);
+    }
+    *reinterpret_cast<uint32_t *>(out + (size_t)n * channels + c) = q;
+}
+
 inline int ew_grid(const nncase_hip_ctx *ctx, size_t work_items) {
     size_t blocks = (work_items + kEwThreads - 1) / kEwThreads;
     const size_t cap = (size_t)ctx->compute_units * 16; // 16 blocks of 4 waves per CU
@@ -278,6 +312,14 @@ extern "C" int nncase_hip_qglobal_avgpool(nncase_hip_ctx_t *ctx, const uint8_t *
     NNHIP_REQUIRE(ctx, batch > 0 && h > 0 && w > 0 && channels > 0, -EINVAL, "qglobal_avgpool: bad shape");
     NNHIP_REQUIRE(ctx, (int64_t)batch * channels < (int64_t)1 << 31, -EINVAL, "qglobal_avgpool: too large");
     NNHIP_REQUIRE(ctx, y_qp.scale != 0.f, -EINVAL, "qglobal_avgpool: output scale is zero");
+    if (channels % 4 == 0 && (reinterpret_cast<uintptr_t>(x_dev) & 3u) == 0 && (reinterpret_cast<uintptr_t>(out_dev) & 3u) == 0) {
+        const int total4 = batch * (channels / 4);
+        hipLaunchKernelGGL(qglobal_avgpool4_kernel, dim3((total4 + kEwThreads - 1) / kEwThreads), dim3(kEwThreads), 0, ctx->stream,
+                           x_dev, out_dev, batch, h * w, channels, (float)x_qp.zero_point, x_qp.scale, (float)y_qp.zero_point,
+                           y_qp.scale);
+        NNHIP_LAUNCH_CHECK(ctx, "qglobal_avgpool4_kernel");
+        return 0;
+    }
     const int total = batch * channels;
     hipLaunchKernelGGL(qglobal_avgpool_kernel, dim3((total + kEwThreads - 1) / kEwThreads), dim3(kEwThreads), 0,
                        ctx->stream, x_dev, out_dev, batch, h * w, channels, (float)x_qp.zero_point, x_qp.scale,

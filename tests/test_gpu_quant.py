@@ -132,7 +132,7 @@ def test_qadd(hip_ctx, count):
     assert np.array_equal(got, O.qadd(a, b, 3, 0.02, 128, 0.011, 0, 0.02, (0.0, 6.0)))
 
 
-@pytest.mark.parametrize("shape", [(1, 5, 7, 7), (3, 1280, 7, 7), (2, 17, 3, 5)])
+@pytest.mark.parametrize("shape", [(1, 5, 7, 7), (3, 1280, 7, 7), (2, 17, 3, 5), (2, 8, 1, 1), (5, 64, 4, 4), (2, 12, 9, 5), (64, 1280, 7, 7)])
 def test_qglobal_avgpool(hip_ctx, shape):
     rng = np.random.default_rng(shape[1])
     x = rng.integers(0, 256, shape, dtype=np.uint8)
