@@ -377,7 +377,18 @@ __global__ void __launch_bounds__(kThreads, ((RG == 1 && T <= 12) || MODE == kRo
         const int steps = min(a.kc_steps, a.ksteps - s0);
         const u32x4 *src = reinterpret_cast<const u32x4 *>(wsrc + (size_t)s0 * T * 1024);
         u32x4 *dst = reinterpret_cast<u32x4 *>(wlds);
-        for (int i = threadIdx.x; i < steps * T * 64; i += kThreads) dst[i] = src[i];
+        // four loads in flight per thread before the first is stored: a block with few pixel tiles spends a good
+        // part of its life here, one memory round trip per trip of this loop
+        const int n = steps * T * 64;
+        for (int i = threadIdx.x; i < n; i += 4 * kThreads) {
+            u32x4 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+                if (i + u * kThreads < n) v[u] = src[i + u * kThreads];
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+                if (i + u * kThreads < n) dst[i + u * kThreads] = v[u];
+        }
     };
     if (nkc == 1) stage_weights(0);
     __syncthreads();
