@@ -363,24 +363,17 @@ __global__ void __launch_bounds__(kThreads, ((RG == 1 && T <= 12) || MODE == kRo
     const uint8_t *wsrc = a.wpk + (size_t)chunk * a.ksteps * T * 1024;
     const int nkc = (a.ksteps + a.kc_steps - 1) / a.kc_steps;
 
-    // Per-channel constant of the zero-point identity, in the lane order the
-    // epilogue reads it: position gq' * 4T + nt * 4 + r <-> channel ch_base + same.
-    for (int i = threadIdx.x; i < T * 16; i += kThreads) {
-        const int ch = ch_base + i;
-        int32_t c = 0;
-        if (ch < a.n) c = a.bias[ch] - a.zxp * a.wsum[ch] + a.k * a.zxp * a.zwp;
-        cterm[i] = c;
-    }
-    if (a.lut && threadIdx.x < 64) reinterpret_cast<uint32_t *>(lutl)[threadIdx.x] = a.lut[threadIdx.x];
-    auto stage_weights = [&](int kci) {
+    // ---- set-up: every load it needs is issued before the first is used, in the order of use (constants, table,
+    // weights, first activation slices): a block with one or two pixel tiles is a chain of memory round trips,
+    // and this makes the set-up one of them ----
+    auto stage_weights = [&](int kci, int first) {
         const int s0 = kci * a.kc_steps;
         const int steps = min(a.kc_steps, a.ksteps - s0);
         const u32x4 *src = reinterpret_cast<const u32x4 *>(wsrc + (size_t)s0 * T * 1024);
         u32x4 *dst = reinterpret_cast<u32x4 *>(wlds);
-        // four loads in flight per thread before the first is stored: a block with few pixel tiles spends a good
-        // part of its life here, one memory round trip per trip of this loop
+        // four loads in flight per thread before the first is stored
         const int n = steps * T * 64;
-        for (int i = threadIdx.x; i < n; i += 4 * kThreads) {
+        for (int i = first + threadIdx.x; i < n; i += 4 * kThreads) {
             u32x4 v[4];
 #pragma unroll
             for (int u = 0; u < 4; u++)
@@ -390,8 +383,20 @@ __global__ void __launch_bounds__(kThreads, ((RG == 1 && T <= 12) || MODE == kRo
                 if (i + u * kThreads < n) dst[i + u * kThreads] = v[u];
         }
     };
-    if (nkc == 1) stage_weights(0);
-    __syncthreads();
+    // per-channel constant of the zero-point identity, in the lane order the epilogue reads it:
+    // position gq' * 4T + nt * 4 + r <-> channel ch_base + same (T * 16 <= kThreads: one per thread)
+    static_assert(T * 16 <= kThreads, "one constant per thread");
+    int32_t c_bias = 0, c_wsum = 0;
+    const bool c_mine = (int)threadIdx.x < T * 16, c_real = c_mine && ch_base + (int)threadIdx.x < a.n;
+    if (c_real) c_bias = a.bias[ch_base + threadIdx.x], c_wsum = a.wsum[ch_base + threadIdx.x];
+    uint32_t lut_word = 0;
+    const bool lut_mine = a.lut && threadIdx.x < 64;
+    if (lut_mine) lut_word = a.lut[threadIdx.x];
+    u32x4 w_first[4];
+    const int n_first = nkc == 1 ? a.ksteps * T * 64 : 0; // the first 4 * kThreads fragments' vectors of a resident chunk
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+        if ((int)threadIdx.x + u * kThreads < n_first) w_first[u] = reinterpret_cast<const u32x4 *>(wsrc)[threadIdx.x + u * kThreads];
 
     const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
     constexpr int pix_per_block = kWaves * RG * 16;
@@ -413,6 +418,14 @@ __global__ void __launch_bounds__(kThreads, ((RG == 1 && T <= 12) || MODE == kRo
             fcur[rg] = load_act<MODE>(a, pcur[rg], gq & a.kc_mask);
         }
     }
+    if (c_mine) cterm[threadIdx.x] = c_real ? c_bias - a.zxp * c_wsum + a.k * a.zxp * a.zwp : 0;
+    if (lut_mine) reinterpret_cast<uint32_t *>(lutl)[threadIdx.x] = lut_word;
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+        if ((int)threadIdx.x + u * kThreads < n_first) reinterpret_cast<u32x4 *>(wlds)[threadIdx.x + u * kThreads] = w_first[u];
+    if (nkc == 1) stage_weights(0, 4 * kThreads);
+    __syncthreads();
+
 #pragma clang loop unroll(disable)
     for (; mt < a.num_mtiles; mt += gridDim.x) {
         // The sums start from the per-channel constant of the zero-point identity, read from LDS for every tile
@@ -434,7 +447,7 @@ __global__ void __launch_bounds__(kThreads, ((RG == 1 && T <= 12) || MODE == kRo
         for (int kci = 0; kci < nkc; kci++) {
             if (nkc > 1) {
                 __syncthreads(); // previous stage fully consumed
-                stage_weights(kci);
+                stage_weights(kci, 0);
                 __syncthreads();
             }
             const int s0 = kci * a.kc_steps;
