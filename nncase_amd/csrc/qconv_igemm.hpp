@@ -443,6 +443,39 @@ __global__ void __launch_bounds__(kThreads, ((RG == 1 && T <= 12) || MODE == kRo
 #pragma unroll
         for (int rg = 0; rg < RG; rg++) rs[rg] = v4i{0, 0, 0, 0};
         const int mt_next = mt + gridDim.x;
+        // One pixel tile per block and a long reduction (the 7x7 layers, the classifier): the block is a chain of
+        // k-steps, each as long as a memory round trip if only one slice is in flight.  Three register sets then
+        // take the slices in turn (no copies between them: a copy would wait for the loads it copies).
+        bool deep = false;
+        constexpr bool kDeepBuilt = RG == 1 && T <= 6 && MODE == kRows16; // (wider chunks and the gathering loaders have no registers to spare)
+        if constexpr (kDeepBuilt) deep = nkc == 1 && a.ksteps >= 4 && a.num_mtiles <= (int)gridDim.x;
+        if (deep) {
+            if constexpr (kDeepBuilt) {
+                ActFrag f1 = load_act<MODE>(a, pcur[0], (4 + gq) & a.kc_mask), f2 = load_act<MODE>(a, pcur[0], (8 + gq) & a.kc_mask);
+                int ks = 0;
+                auto step = [&](ActFrag &f) __attribute__((always_inline)) {
+                    const v4i xf = finish_act(f);
+                    const int nk = ks + 3 < a.ksteps ? ks + 3 : 0; // past the end: a valid slice, dropped
+                    f = load_act<MODE>(a, pcur[0], (nk * 4 + gq) & a.kc_mask);
+                    rs[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, xf, rs[0], 0, 0, 0);
+                    const uint8_t *wstep = wlds + (size_t)ks * T * 1024 + lane * 16;
+#pragma unroll
+                    for (int nt = 0; nt < T; nt++) {
+                        const v4i wf = *reinterpret_cast<const v4i *>(wstep + nt * 1024);
+                        acc[0][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf, xf, acc[0][nt], 0, 0, 0);
+                    }
+                    ks++;
+                };
+                for (;;) {
+                    step(fcur[0]);
+                    if (ks >= a.ksteps) break;
+                    step(f1);
+                    if (ks >= a.ksteps) break;
+                    step(f2);
+                    if (ks >= a.ksteps) break;
+                }
+            }
+        } else
 #pragma clang loop unroll(disable)
         for (int kci = 0; kci < nkc; kci++) {
             if (nkc > 1) {
