@@ -178,6 +178,32 @@ def test_short_reductions_for_every_weight_zero_point(hip_ctx, zw, cin, k, pad):
         assert np.array_equal(got, want)
 
 
+def _random_conv_cases(count, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    while len(cases) < count:
+        k = int(rng.choice([1, 1, 1, 3, 2, 5]))
+        cin = int(rng.choice([1, 3, 4, 8, 12, 16, 24, 32, 40, 48, 64, 80, 96, 144, 160, 320, 384, 576, 960]))
+        if k > 1 and cin > 96:
+            continue
+        cout = int(rng.choice([4, 8, 16, 20, 24, 32, 40, 64, 96, 100, 144, 160, 255, 320]))
+        n = int(rng.integers(1, 4))
+        h, w = int(rng.integers(k, 15)), int(rng.integers(k, 15))
+        stride = int(rng.choice([1, 1, 2]))
+        pad = int(rng.integers(0, (k + 1) // 2 + 1)) if k > 1 else 0
+        cases.append((n, cin, h, w, cout, k, stride, pad, int(rng.integers(0, 256)), int(rng.integers(0, 256))))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_conv_cases(48, 20251))
+def test_random_dense_shapes_and_zero_points(hip_ctx, case):
+    """Shapes drawn at random across the loaders (row, 16/8/4-byte vectors, bytes), the single-tile and persistent
+    forms, short and long reductions, and every pairing of zero points."""
+    n, cin, h, w, cout, k, stride, pad, zx, zw = case
+    run_case(hip_ctx, n, cin, h, w, cout, k, k, (stride, stride), ((pad, pad), (pad, pad)), (1, 1), 1,
+             seed=n + cin * 3 + cout * 5 + h * 7 + w * 11, zx=zx, zw=zw, modes=("u8", "i32"))
+
+
 def test_config2_conv_block(hip_ctx):
     """BASELINE config 2 at batch 1: 1x1 64->144, 3x3 depthwise, 1x1 144->64 on 56x56, ReLU6, per-tensor PTQ."""
     rng = np.random.default_rng(1)
