@@ -411,6 +411,11 @@ NNCASE_HIP_API int nncase_hip_w8a16_prepack(nncase_hip_ctx_t *ctx, const int8_t 
 NNCASE_HIP_API int nncase_hip_w8a16_destroy(nncase_hip_ctx_t *ctx, nncase_hip_w8a16_t *weights);
 NNCASE_HIP_API int nncase_hip_w8a16_gemm(nncase_hip_ctx_t *ctx, const void *a_dev, const nncase_hip_w8a16_t *weights,
                                          void *out_dev, int32_t m, int32_t mode, const void *residual_dev, int32_t out_dtype);
+/* The same product on rmsnorm(x) (below) without the normalised rows passing through memory: bit for bit what
+ * nncase_hip_rmsnorm_f16 followed by nncase_hip_w8a16_gemm writes.  ln_weight_dev: [k] fp16, 16-byte aligned. */
+NNCASE_HIP_API int nncase_hip_rmsnorm_w8a16_gemm(nncase_hip_ctx_t *ctx, const void *x_dev, const void *ln_weight_dev, float eps,
+                                                 const nncase_hip_w8a16_t *weights, void *out_dev, int32_t m, int32_t mode,
+                                                 const void *residual_dev, int32_t out_dtype);
 /* out[r, :] = x[r, :] * rsqrt(mean(x[r, :]^2) + eps) * weight, fp16 in / out, fp32 arithmetic. */
 NNCASE_HIP_API int nncase_hip_rmsnorm_f16(nncase_hip_ctx_t *ctx, const void *x_dev, const void *weight_dev, void *out_dev,
                                           int32_t rows, int32_t hidden, float eps);
@@ -491,6 +496,10 @@ NNCASE_HIP_API int nncase_hip_function_add_pack(nncase_hip_function_t *fn, const
 NNCASE_HIP_API int nncase_hip_function_add_w8a16_gemm(nncase_hip_function_t *fn, const void *a_dev, const nncase_hip_w8a16_t *weights,
                                                       void *out_dev, int32_t m, int32_t mode, const void *residual_dev,
                                                       int32_t out_dtype);
+NNCASE_HIP_API int nncase_hip_function_add_rmsnorm_w8a16_gemm(nncase_hip_function_t *fn, const void *x_dev,
+                                                              const void *ln_weight_dev, float eps,
+                                                              const nncase_hip_w8a16_t *weights, void *out_dev, int32_t m,
+                                                              int32_t mode, const void *residual_dev, int32_t out_dtype);
 NNCASE_HIP_API int nncase_hip_function_add_rmsnorm_f16(nncase_hip_function_t *fn, const void *x_dev, const void *weight_dev,
                                                        void *out_dev, int32_t rows, int32_t hidden, float eps);
 NNCASE_HIP_API int nncase_hip_function_add_rope_kv_append(nncase_hip_function_t *fn, const void *qkv_dev, void *q_out_dev,

@@ -82,6 +82,7 @@ static int run_op(nncase_hip_function *fn, const Op &op) {
     case Op::kPack:
         return nncase_hip_pack(ctx, op.in0, op.out, op.elem_size, op.rank, op.shape, op.n_axes, op.axes, op.lanes);
     case Op::kGemm:
+        if (op.in2) return nncase_hip_rmsnorm_w8a16_gemm(ctx, op.in0, op.in2, op.eps, op.w8, op.out, op.batch, op.mode, op.in1, op.dt_out);
         return nncase_hip_w8a16_gemm(ctx, op.in0, op.w8, op.out, op.batch, op.mode, op.in1, op.dt_out);
     case Op::kRmsNorm:
         return nncase_hip_rmsnorm_f16(ctx, op.in0, op.in1, op.out, op.batch, op.channels, op.eps);
@@ -291,6 +292,18 @@ extern "C" int nncase_hip_function_add_w8a16_gemm(nncase_hip_function_t *fn, con
     return push(fn, op);
 }
 
+extern "C" int nncase_hip_function_add_rmsnorm_w8a16_gemm(nncase_hip_function_t *fn, const void *x_dev, const void *ln_weight_dev,
+                                                          float eps, const nncase_hip_w8a16_t *weights, void *out_dev, int32_t m,
+                                                          int32_t mode, const void *residual_dev, int32_t out_dtype) {
+    if (!fn) return -EINVAL;
+    NNHIP_REQUIRE(fn->ctx, x_dev && ln_weight_dev && weights && out_dev, -EINVAL, "function_add_rmsnorm_w8a16_gemm: null argument");
+    Op op;
+    op.kind = Op::kGemm;
+    op.in0 = x_dev, op.in2 = ln_weight_dev, op.eps = eps, op.w8 = weights, op.out = out_dev, op.batch = m, op.mode = mode;
+    op.in1 = residual_dev, op.dt_out = out_dtype;
+    return push(fn, op);
+}
+
 extern "C" int nncase_hip_function_add_rmsnorm_f16(nncase_hip_function_t *fn, const void *x_dev, const void *weight_dev,
                                                    void *out_dev, int32_t rows, int32_t hidden, float eps) {
     if (!fn) return -EINVAL;
@@ -477,7 +490,10 @@ extern "C" int nncase_hip_function_op_kernel(nncase_hip_function_t *fn, int32_t 
     case Op::kResize: snprintf(name, capacity, "resize_nearest"); break;
     case Op::kMaxPool: snprintf(name, capacity, "qmaxpool<%dx%d>", op.pool[0], op.pool[1]); break;
     case Op::kPack: snprintf(name, capacity, "pack"); break;
-    case Op::kGemm: snprintf(name, capacity, op.mode == NNCASE_HIP_GEMM_SWIGLU ? "w8a16_gemm+swiglu" : (op.in1 ? "w8a16_gemm+residual" : "w8a16_gemm")); break;
+    case Op::kGemm:
+        snprintf(name, capacity, "%sw8a16_gemm%s", op.in2 ? "rmsnorm+" : "",
+                 op.mode == NNCASE_HIP_GEMM_SWIGLU ? "+swiglu" : (op.in1 ? "+residual" : ""));
+        break;
     case Op::kRmsNorm: snprintf(name, capacity, "rmsnorm_f16"); break;
     case Op::kRope: snprintf(name, capacity, "rope_kv_append"); break;
     case Op::kAttn: snprintf(name, capacity, "paged_attention_decode"); break;

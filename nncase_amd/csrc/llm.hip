@@ -51,7 +51,64 @@ struct GemmArgs {
     void *out;                // [m][n_out] fp16 or fp32
     int m, k, n_out, ksteps, mode, out_f32;
     int up_tile_offset; // SwiGLU: tile t of the gate pairs with tile t + up_tile_offset of the up projection
+    // RMS normalisation of the token rows in front of the product (null: none): the block computes every row's
+    // 1 / sqrt(mean(x^2) + eps) the way rmsnorm_f16_kernel does, and a token slice becomes
+    // fp16(x * r * weight) as it is loaded, so the result is what the two kernels give one after the other
+    const uint16_t *ln_w; // [k] fp16
+    float ln_eps;
 };
+
+// 1 / sqrt(mean(x^2) + eps) of a row, the way every kernel here forms it.  A lane owns the 8 consecutive elements
+// 8 * lane .. 8 * lane + 7 of every 512-element piece of the row (one 16-byte load per piece); it adds their squares
+// in index order, piece after piece, and a butterfly adds the 64 lanes.  The order is part of the definition: the
+// product kernel that normalises its own rows must arrive at the same bits as rmsnorm_f16_kernel.
+__device__ __forceinline__ void add_squares8(const lu32x4 &v, float &ss) {
+    __half h[8];
+    __builtin_memcpy(h, &v, 16);
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        const float f = __half2float(h[e]);
+        ss += f * f;
+    }
+}
+__device__ __forceinline__ float rstd_from_sum(float ss, int hidden, float eps) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+    return 1.0f / sqrtf(ss / (float)hidden + eps);
+}
+// R rows at once (row r0 + i * stride for i < R, those below `rows`): the loads of one piece of all of them are in
+// flight together.  hidden is a multiple of 8 and the rows are 16-byte aligned.
+template <int R>
+__device__ __forceinline__ void rms_rstd_rows(const __half *x, int hidden, int rows, int r0, int stride, int lane, float eps,
+                                              float (&out)[R]) {
+    float ss[R];
+#pragma unroll
+    for (int i = 0; i < R; i++) ss[i] = 0.f;
+    for (int e0 = lane * 8; e0 < ((hidden + 511) & ~511); e0 += 512) {
+        lu32x4 v[R];
+#pragma unroll
+        for (int i = 0; i < R; i++) {
+            const int r = r0 + i * stride;
+            v[i] = lu32x4{0, 0, 0, 0}; // (+0 squares leave a sum as it is)
+            if (r < rows && e0 < hidden) v[i] = *reinterpret_cast<const lu32x4 *>(x + (size_t)r * hidden + e0);
+        }
+#pragma unroll
+        for (int i = 0; i < R; i++) add_squares8(v[i], ss[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < R; i++) out[i] = rstd_from_sum(ss[i], hidden, eps);
+}
+// any row length and alignment: the same order with one element per load
+__device__ __forceinline__ float rms_rstd_scalar(const __half *xr, int hidden, float eps, int lane) {
+    float ss = 0.f;
+    for (int e0 = lane * 8; e0 < ((hidden + 511) & ~511); e0 += 512)
+        for (int e = 0; e < 8; e++)
+            if (e0 + e < hidden) {
+                const float f = __half2float(xr[e0 + e]);
+                ss += f * f;
+            }
+    return rstd_from_sum(ss, hidden, eps);
+}
 
 // 8 int8 weights (two dwords' low / high halves handled by the caller) -> 8 fp16, exact.
 __device__ __forceinline__ h16x8 w8_to_f16(uint32_t lo, uint32_t hi) {
@@ -99,8 +156,20 @@ constexpr int kGemmBatch = 4;
 // otherwise every wave owns a tile of its own and the whole reduction (many tiles: the vocabulary head).
 template <int MT, int G, bool SPLIT> __global__ __launch_bounds__(kGemmThreads) void w8a16_gemm_kernel(const GemmArgs a) {
     __shared__ float red[SPLIT ? kGemmWaves : 1][G][MT][64][4];
+    __shared__ float rstd[MT * 16];
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int i16 = lane & 15, kg = lane >> 4;
+    if (a.ln_w) { // (uniform; before any wave leaves the block)
+        constexpr int R = MT * 16 / kGemmWaves; // rows per wave
+        float rs[R];
+        rms_rstd_rows<R>(reinterpret_cast<const __half *>(a.a), a.k, a.m, wave, kGemmWaves, lane, a.ln_eps, rs);
+        if (lane == 0) {
+#pragma unroll
+            for (int i = 0; i < R; i++)
+                if (wave + i * kGemmWaves < a.m) rstd[wave + i * kGemmWaves] = rs[i];
+        }
+        __syncthreads();
+    }
     const int per = SPLIT ? (a.ksteps + kGemmWaves - 1) / kGemmWaves : a.ksteps;
     const int ks0 = SPLIT ? wave * per : 0, ks1 = min(a.ksteps, ks0 + per);
     const int out_tile = SPLIT ? (int)blockIdx.x : (int)blockIdx.x * kGemmWaves + wave;
@@ -114,12 +183,17 @@ template <int MT, int G, bool SPLIT> __global__ __launch_bounds__(kGemmThreads) 
     const int tile[2] = {out_tile, out_tile + a.up_tile_offset};
     // token rows of this lane (clamped: rows past m read row m - 1 and are never stored)
     const uint16_t *arow[MT];
+    float rrow[MT];
 #pragma unroll
-    for (int t = 0; t < MT; t++) arow[t] = a.a + (size_t)min(t * 16 + i16, a.m - 1) * a.k + kg * 16;
+    for (int t = 0; t < MT; t++) {
+        arow[t] = a.a + (size_t)min(t * 16 + i16, a.m - 1) * a.k + kg * 16;
+        rrow[t] = a.ln_w ? rstd[min(t * 16 + i16, a.m - 1)] : 1.f;
+    }
 
     for (int kb = ks0; kb < ks1; kb += kGemmBatch) {
         lu32x4 wv[kGemmBatch][G];
         lu32x4 av[kGemmBatch][MT][2];
+        lu32x4 lw[kGemmBatch][2]; // the normalisation weights of the lane's 16 reduction indices
 #pragma unroll
         for (int u = 0; u < kGemmBatch; u++) {
             const int ks = min(kb + u, ks1 - 1); // steps past the share re-read the last one and are not multiplied
@@ -130,6 +204,30 @@ template <int MT, int G, bool SPLIT> __global__ __launch_bounds__(kGemmThreads) 
                 av[u][t][0] = *reinterpret_cast<const lu32x4 *>(arow[t] + ks * 64);
                 av[u][t][1] = *reinterpret_cast<const lu32x4 *>(arow[t] + ks * 64 + 8);
             }
+            if (a.ln_w) {
+                lw[u][0] = *reinterpret_cast<const lu32x4 *>(a.ln_w + ks * 64 + kg * 16);
+                lw[u][1] = *reinterpret_cast<const lu32x4 *>(a.ln_w + ks * 64 + kg * 16 + 8);
+            }
+        }
+        if (a.ln_w) {
+#pragma unroll
+            for (int u = 0; u < kGemmBatch; u++)
+#pragma unroll
+                for (int t = 0; t < MT; t++)
+#pragma unroll
+                    for (int hlf = 0; hlf < 2; hlf++) {
+                        __half xh[8], wh[8];
+                        __builtin_memcpy(xh, &av[u][t][hlf], 16);
+                        __builtin_memcpy(wh, &lw[u][hlf], 16);
+#pragma unroll
+                        for (int e = 0; e < 8; e++) {
+                            // the fp32 product is rounded before it is converted, as in rmsnorm_f16_kernel (see there)
+                            float pr = __half2float(xh[e]) * rrow[t] * __half2float(wh[e]);
+                            asm volatile("" : "+v"(pr));
+                            xh[e] = __float2half_rn(pr);
+                        }
+                        __builtin_memcpy(&av[u][t][hlf], xh, 16);
+                    }
         }
 #pragma unroll
         for (int u = 0; u < kGemmBatch; u++) {
@@ -193,16 +291,22 @@ __global__ __launch_bounds__(kLlmThreads) void rmsnorm_f16_kernel(const __half *
     const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
     if (row >= rows) return;
     const __half *xr = x + (size_t)row * hidden;
-    float ss = 0.f;
-    for (int i = lane; i < hidden; i += 64) {
-        const float v = __half2float(xr[i]);
-        ss += v * v;
+    float r;
+    if ((hidden & 7) == 0 && (reinterpret_cast<uintptr_t>(x) & 15u) == 0) {
+        float rs[1];
+        rms_rstd_rows<1>(x, hidden, rows, row, 1, lane, eps, rs);
+        r = rs[0];
+    } else {
+        r = rms_rstd_scalar(xr, hidden, eps, lane);
     }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
-    const float r = 1.0f / sqrtf(ss / (float)hidden + eps);
-    for (int i = lane; i < hidden; i += 64)
-        out[(size_t)row * hidden + i] = __float2half_rn(__half2float(xr[i]) * r * __half2float(w[i]));
+    for (int i = lane; i < hidden; i += 64) {
+        // The fp32 product is rounded before it is converted to fp16.  Left to itself the compiler turns multiply and
+        // conversion into one mixed-precision instruction (a single rounding) in some copies of this loop's body
+        // and not in others, so the same input could round either way depending on where it sits in the row.
+        float pr = __half2float(xr[i]) * r * __half2float(w[i]);
+        asm volatile("" : "+v"(pr));
+        out[(size_t)row * hidden + i] = __float2half_rn(pr);
+    }
 }
 
 struct RopeArgs {
@@ -344,10 +448,12 @@ extern "C" int nncase_hip_w8a16_prepack(nncase_hip_ctx_t *ctx, const int8_t *w_h
     return 0;
 }
 
-extern "C" int nncase_hip_w8a16_gemm(nncase_hip_ctx_t *ctx, const void *a_dev, const nncase_hip_w8a16_t *w, void *out_dev,
-                                     int32_t m, int32_t mode, const void *residual_dev, int32_t out_dtype) {
+static int launch_w8a16_gemm(nncase_hip_ctx_t *ctx, const void *a_dev, const nncase_hip_w8a16_t *w, void *out_dev, int32_t m,
+                             int32_t mode, const void *residual_dev, int32_t out_dtype, const void *ln_weight_dev, float ln_eps) {
     NNHIP_CHECK_CTX(ctx);
     NNHIP_REQUIRE(ctx, a_dev && w && out_dev, -EINVAL, "w8a16_gemm: null argument");
+    NNHIP_REQUIRE(ctx, (reinterpret_cast<uintptr_t>(ln_weight_dev) & 15u) == 0, -NNCASE_HIP_ERR_INVALID_MEMORY_LOCATION,
+                  "w8a16_gemm: normalisation weights must be 16-byte aligned");
     NNHIP_REQUIRE(ctx, m > 0 && m <= kMaxRows, -NNCASE_HIP_ERR_SHAPE_MISMATCH, "w8a16_gemm: %d token rows (1..%d supported)", m, kMaxRows);
     NNHIP_REQUIRE(ctx, mode == NNCASE_HIP_GEMM_PLAIN || mode == NNCASE_HIP_GEMM_SWIGLU, -EINVAL, "w8a16_gemm: unknown mode %d", mode);
     NNHIP_REQUIRE(ctx, out_dtype == NNCASE_HIP_DT_F16 || out_dtype == NNCASE_HIP_DT_F32, -NNCASE_HIP_ERR_DATATYPE_MISMATCH,
@@ -362,6 +468,8 @@ extern "C" int nncase_hip_w8a16_gemm(nncase_hip_ctx_t *ctx, const void *a_dev, c
     a.w = (const lu32x4 *)w->d_packed;
     a.scale = w->d_scale, a.bias = w->d_bias;
     a.residual = (const uint16_t *)residual_dev;
+    a.ln_w = (const uint16_t *)ln_weight_dev;
+    a.ln_eps = ln_eps;
     a.out = out_dev;
     a.m = m, a.k = w->k, a.ksteps = w->ksteps, a.mode = mode, a.out_f32 = out_dtype == NNCASE_HIP_DT_F32;
     const int out_tiles = mode == NNCASE_HIP_GEMM_SWIGLU ? w->ntiles / 2 : w->ntiles;
@@ -385,6 +493,19 @@ extern "C" int nncase_hip_w8a16_gemm(nncase_hip_ctx_t *ctx, const void *a_dev, c
 #undef NNHIP_GEMM_LAUNCH
     NNHIP_LAUNCH_CHECK(ctx, "w8a16_gemm_kernel");
     return 0;
+}
+
+extern "C" int nncase_hip_w8a16_gemm(nncase_hip_ctx_t *ctx, const void *a_dev, const nncase_hip_w8a16_t *w, void *out_dev,
+                                     int32_t m, int32_t mode, const void *residual_dev, int32_t out_dtype) {
+    return launch_w8a16_gemm(ctx, a_dev, w, out_dev, m, mode, residual_dev, out_dtype, nullptr, 0.f);
+}
+
+extern "C" int nncase_hip_rmsnorm_w8a16_gemm(nncase_hip_ctx_t *ctx, const void *x_dev, const void *ln_weight_dev, float eps,
+                                             const nncase_hip_w8a16_t *w, void *out_dev, int32_t m, int32_t mode,
+                                             const void *residual_dev, int32_t out_dtype) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, ln_weight_dev, -EINVAL, "rmsnorm_w8a16_gemm: null normalisation weights");
+    return launch_w8a16_gemm(ctx, x_dev, w, out_dev, m, mode, residual_dev, out_dtype, ln_weight_dev, eps);
 }
 
 extern "C" int nncase_hip_rmsnorm_f16(nncase_hip_ctx_t *ctx, const void *x_dev, const void *weight_dev, void *out_dev, int32_t rows,

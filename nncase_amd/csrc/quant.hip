@@ -87,7 +87,13 @@ __global__ __launch_bounds__(kEwThreads) void quantize_kernel(const TIn *__restr
 
 template <typename TOut> __device__ __forceinline__ TOut from_f32(float v);
 template <> __device__ __forceinline__ float from_f32<float>(float v) { return v; }
-template <> __device__ __forceinline__ __half from_f32<__half>(float v) { return __float2half_rn(v); }
+// (the fp32 value is hidden from the optimiser first: where it sees the multiply that produced it, it may merge
+// multiply and conversion into one mixed-precision instruction that rounds once, and does so in some copies of a
+// loop body and not in others; the result is defined as the fp16 nearest to the rounded fp32 product)
+template <> __device__ __forceinline__ __half from_f32<__half>(float v) {
+    asm volatile("" : "+v"(v));
+    return __float2half_rn(v);
+}
 
 template <typename TQ, typename TOut>
 __global__ __launch_bounds__(kEwThreads) void dequantize_kernel(const TQ *__restrict__ in, TOut *__restrict__ out,

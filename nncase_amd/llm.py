@@ -70,7 +70,7 @@ class HipDecoder:
 
     def __init__(self, ctx: Context, cfg: DecoderConfig, weights: Dict[str, object], batch: int, max_blocks_per_seq: int,
                  block_table: np.ndarray, ctx_lens: np.ndarray, k_caches: List[np.ndarray], v_caches: List[np.ndarray],
-                 capture_graph: bool = True, feedback: bool = False):
+                 capture_graph: bool = True, feedback: bool = False, fuse_norm: bool = True):
         self.ctx, self.cfg, self.batch = ctx, cfg, batch
         c = cfg
         qd, kvd = c.q_heads * c.head_dim, c.kv_heads * c.head_dim
@@ -105,18 +105,28 @@ class HipDecoder:
                  "v": ctx.to_device(np.ascontiguousarray(v_caches[li], np.float16))}
             self.layers.append(L)
             x, h = self.x[0], self.x[1]
-            fn.add_rmsnorm_f16(x, L["ln1"], self.norm, batch, c.hidden, c.rms_eps)
-            fn.add_w8a16_gemm(self.norm, L["qkv"], self.qkv, batch)
+            # the three normalisations run inside the products that consume them (fuse_norm), or as operators of their own
+            if fuse_norm:
+                fn.add_rmsnorm_w8a16_gemm(x, L["ln1"], c.rms_eps, L["qkv"], self.qkv, batch)
+            else:
+                fn.add_rmsnorm_f16(x, L["ln1"], self.norm, batch, c.hidden, c.rms_eps)
+                fn.add_w8a16_gemm(self.norm, L["qkv"], self.qkv, batch)
             fn.add_rope_kv_append(self.qkv, self.q, L["k"], L["v"], self.block_table, self.ctx_lens, self.geometry, c.rope_theta)
             # the appended token takes part in its own attention (lengths + 1); the lengths themselves advance
             # once, at the end of the step
             fn.add_paged_attention_decode(self.q, L["k"], L["v"], self.block_table, self.ctx_lens, self.att, self.attn_args)
             fn.add_w8a16_gemm(self.att, L["o"], h, batch, residual=x)
-            fn.add_rmsnorm_f16(h, L["ln2"], self.norm, batch, c.hidden, c.rms_eps)
-            fn.add_w8a16_gemm(self.norm, L["gate_up"], self.act, batch, mode=rt.GEMM_SWIGLU)
+            if fuse_norm:
+                fn.add_rmsnorm_w8a16_gemm(h, L["ln2"], c.rms_eps, L["gate_up"], self.act, batch, mode=rt.GEMM_SWIGLU)
+            else:
+                fn.add_rmsnorm_f16(h, L["ln2"], self.norm, batch, c.hidden, c.rms_eps)
+                fn.add_w8a16_gemm(self.norm, L["gate_up"], self.act, batch, mode=rt.GEMM_SWIGLU)
             fn.add_w8a16_gemm(self.act, L["down"], x, batch, residual=h)
-        fn.add_rmsnorm_f16(self.x[0], self.ln_f, self.norm, batch, c.hidden, c.rms_eps)
-        fn.add_w8a16_gemm(self.norm, self.lm_head, self.logits, batch, out_dtype=rt.DT_F32)
+        if fuse_norm:
+            fn.add_rmsnorm_w8a16_gemm(self.x[0], self.ln_f, c.rms_eps, self.lm_head, self.logits, batch, out_dtype=rt.DT_F32)
+        else:
+            fn.add_rmsnorm_f16(self.x[0], self.ln_f, self.norm, batch, c.hidden, c.rms_eps)
+            fn.add_w8a16_gemm(self.norm, self.lm_head, self.logits, batch, out_dtype=rt.DT_F32)
         # feedback: the arg-max lands in the token buffer the next step's embedding reads (greedy generation
         # without a host round trip); otherwise the caller feeds every step's tokens
         self.feedback = feedback

@@ -135,6 +135,8 @@ SYMBOLS = {
     "nncase_hip_embedding_f16": (_I, [_VP, _VP, _VP, _VP, C.c_int32, C.c_int32, C.c_int32]),
     "nncase_hip_add_i32": (_I, [_VP, _VP, C.c_int32, C.c_int32]),
     "nncase_hip_function_add_w8a16_gemm": (_I, [_VP, _VP, _VP, _VP, C.c_int32, C.c_int32, _VP, C.c_int32]),
+    "nncase_hip_rmsnorm_w8a16_gemm": (_I, [_VP, _VP, _VP, C.c_float, _VP, _VP, C.c_int32, C.c_int32, _VP, C.c_int32]),
+    "nncase_hip_function_add_rmsnorm_w8a16_gemm": (_I, [_VP, _VP, _VP, C.c_float, _VP, _VP, C.c_int32, C.c_int32, _VP, C.c_int32]),
     "nncase_hip_function_add_rmsnorm_f16": (_I, [_VP, _VP, _VP, _VP, C.c_int32, C.c_int32, C.c_float]),
     "nncase_hip_function_add_rope_kv_append": (_I, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, C.POINTER(PagedAttnArgs), C.c_float]),
     "nncase_hip_function_add_paged_attention_decode": (_I, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, C.POINTER(PagedAttnArgs)]),
@@ -533,6 +535,13 @@ class Context:
         self._check(self.lib.nncase_hip_w8a16_gemm(self.handle, a.ptr, w.handle, out.ptr, m, mode,
                                                    residual.ptr if residual is not None else None, out_dtype), "w8a16_gemm")
 
+    def rmsnorm_w8a16_gemm(self, x: DeviceBuffer, ln_weight: DeviceBuffer, eps: float, w: "W8A16", out: DeviceBuffer, m: int,
+                           mode: int = GEMM_PLAIN, residual: Optional[DeviceBuffer] = None, out_dtype: int = DT_F16):
+        """w8a16_gemm(rmsnorm_f16(x)) in one launch, bit for bit the two operators' result."""
+        self._check(self.lib.nncase_hip_rmsnorm_w8a16_gemm(self.handle, x.ptr, ln_weight.ptr, eps, w.handle, out.ptr, m, mode,
+                                                           residual.ptr if residual is not None else None, out_dtype),
+                    "rmsnorm_w8a16_gemm")
+
     def rmsnorm_f16(self, x: DeviceBuffer, weight: DeviceBuffer, out: DeviceBuffer, rows: int, hidden: int, eps: float):
         self._check(self.lib.nncase_hip_rmsnorm_f16(self.handle, x.ptr, weight.ptr, out.ptr, rows, hidden, eps), "rmsnorm_f16")
 
@@ -630,6 +639,12 @@ class Function:
         self._ck(self.ctx.lib.nncase_hip_function_add_w8a16_gemm(self.handle, a.ptr, w.handle, out.ptr, m, mode,
                                                                  residual.ptr if residual is not None else None, out_dtype),
                  "function_add_w8a16_gemm")
+
+    def add_rmsnorm_w8a16_gemm(self, x, ln_weight, eps, w, out, m, mode=GEMM_PLAIN, residual=None, out_dtype=DT_F16):
+        self._keep += [x, ln_weight, w, out] + ([residual] if residual is not None else [])
+        self._ck(self.ctx.lib.nncase_hip_function_add_rmsnorm_w8a16_gemm(self.handle, x.ptr, ln_weight.ptr, eps, w.handle, out.ptr, m,
+                                                                         mode, residual.ptr if residual is not None else None,
+                                                                         out_dtype), "function_add_rmsnorm_w8a16_gemm")
 
     def add_rmsnorm_f16(self, x, weight, out, rows, hidden, eps):
         self._keep += [x, weight, out]

@@ -57,6 +57,58 @@ def test_w8a16_swiglu(hip_ctx):
     close(out.download((m, mlp), np.float16), R.silu(gu[:, :mlp]) * gu[:, mlp:])
 
 
+@pytest.mark.parametrize("m,k,n,mode", [(1, 64, 16, "plain"), (32, 896, 1152, "plain"), (7, 128, 48, "residual"), (33, 192, 64, "plain"),
+                                        (32, 896, 9728, "swiglu"), (64, 896, 2048, "f32"), (32, 896, 151936 // 16 * 16, "f32")])
+def test_rmsnorm_fused_into_gemm_equals_the_two_operators(hip_ctx, m, k, n, mode):
+    """The product that normalises its own rows writes, bit for bit, what rmsnorm_f16 followed by w8a16_gemm writes:
+    split and per-wave reductions, SwiGLU, residual, fp32 output, the vocabulary head."""
+    rng = np.random.default_rng(m * 3 + k + n)
+    x = (rng.standard_normal((m, k)) * rng.uniform(0.1, 4.0, (m, 1))).astype(np.float16)
+    lnw = (1.0 + 0.2 * rng.standard_normal(k)).astype(np.float16)
+    q = rng.integers(-127, 128, (n, k), dtype=np.int8)
+    scale = rng.uniform(0.001, 0.01, n).astype(np.float32)
+    w = hip_ctx.prepack_w8a16(q, scale, rng.standard_normal(n).astype(np.float32))
+    gemm_mode = rt.GEMM_SWIGLU if mode == "swiglu" else rt.GEMM_PLAIN
+    n_out = n // 2 if mode == "swiglu" else n
+    dt, code = (np.float32, rt.DT_F32) if mode == "f32" else (np.float16, rt.DT_F16)
+    res = hip_ctx.to_device(rng.standard_normal((m, n_out)).astype(np.float16)) if mode == "residual" else None
+    dx, dln = hip_ctx.to_device(x), hip_ctx.to_device(lnw)
+    norm = hip_ctx.alloc(m * k * 2)
+    two, one = hip_ctx.alloc(m * n_out * np.dtype(dt).itemsize), hip_ctx.alloc(m * n_out * np.dtype(dt).itemsize)
+    hip_ctx.rmsnorm_f16(dx, dln, norm, m, k, 1e-6)
+    hip_ctx.w8a16_gemm(norm, w, two, m, mode=gemm_mode, residual=res, out_dtype=code)
+    hip_ctx.rmsnorm_w8a16_gemm(dx, dln, 1e-6, w, one, m, mode=gemm_mode, residual=res, out_dtype=code)
+    a, b = two.download((m, n_out), dt), one.download((m, n_out), dt)
+    assert np.array_equal(a.view(np.uint32 if mode == "f32" else np.uint16), b.view(np.uint32 if mode == "f32" else np.uint16))
+    assert np.isfinite(a.astype(np.float64)).all() and np.abs(a.astype(np.float64)).max() > 0
+
+
+def test_decoder_with_fused_normalisation_equals_separate_operators(hip_ctx):
+    cfg = llm.DecoderConfig(layers=2, hidden=256, q_heads=4, kv_heads=2, head_dim=64, mlp=512, vocab=2048)
+    rng = np.random.default_rng(5)
+    weights = llm.random_weights(cfg, seed=4)
+    batch = 5
+    max_blocks, lens, bt, kcs, vcs = make_state(cfg, rng, batch, 70)
+    tokens = rng.integers(0, cfg.vocab, batch).astype(np.int32)
+    outs = []
+    for fuse in (True, False):
+        dec = llm.HipDecoder(hip_ctx, cfg, weights, batch, max_blocks, bt, lens.copy(), [k.copy() for k in kcs], [v.copy() for v in vcs],
+                             capture_graph=True, fuse_norm=fuse)
+        assert len(dec.fn) == (3 + cfg.layers * 6 + 1 if fuse else 3 + cfg.layers * 8 + 2)
+        tk = tokens
+        logs = []
+        for _ in range(2):
+            dec.set_tokens(tk)
+            dec.step()
+            hip_ctx.sync()
+            tk = dec.result()
+            logs.append(dec.logits.download((batch, cfg.vocab), np.float32))
+        outs.append((tk, logs))
+    assert np.array_equal(outs[0][0], outs[1][0])
+    for a, b in zip(outs[0][1], outs[1][1]):
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
 def test_w8a16_error_paths(hip_ctx):
     q = np.zeros((16, 64), np.int8)
     with pytest.raises(rt.HipError) as e:

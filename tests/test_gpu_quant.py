@@ -82,6 +82,21 @@ def test_dequantize(hip_ctx, count):
         assert np.array_equal(got16.view(np.uint16), O.f32_to_f16_bits(want))
 
 
+@pytest.mark.parametrize("count", [1, 2, 3, 4, 5, 7, 16, 1027])
+def test_dequantize_to_fp16_rounds_the_fp32_product(hip_ctx, count):
+    """(q - zp) * scale lands exactly half way between two fp16 values after its fp32 rounding while the exact product
+    does not: the fp16 result is the nearest-even of the rounded fp32 value, in the vector body of the kernel and in
+    its scalar tail alike (a fused multiply-convert would round the exact product and give the neighbour)."""
+    scale = np.float32(0.026969021186232567)
+    codes = np.array([-172, -86, -43, 43, 86, 172], np.int16)
+    q = np.resize(codes, count).astype(np.int16)
+    want = O.dequantize(q, float(scale), 0)
+    got16 = K.dequantize(q, qp(0, float(scale)), np.float16, ctx=hip_ctx)
+    assert np.array_equal(got16.view(np.uint16), O.f32_to_f16_bits(want))
+    exact = np.float16(q.astype(np.float64) * np.float64(scale))
+    assert (exact.view(np.uint16) != O.f32_to_f16_bits(want)).all()  # the case really separates the two roundings
+
+
 def test_quantize_dequantize_roundtrip_full_size(hip_ctx):
     # size-independent property at a BASELINE size: Q(DQ(q)) == q for every code
     n = 32 * 64 * 56 * 56
