@@ -202,14 +202,8 @@ __global__ __launch_bounds__(NW * 64) void qblock_kernel(const BlockArgs a) {
     __syncthreads();
 
     // ---- what stays the same for every chunk -------------------------------------------------------------------
-    // E: the wave's units are pixel groups whalf, whalf + NQ, ... of channel tile wtile
-    HaloPix ehp[MAXU];
-#pragma unroll
-    for (int k = 0; k < MAXU; k++) {
-        const int g = whalf + NQ * k;
-        ehp[k] = hpix[min(g, NG - 1) * 16 + j];
-        if (g >= ngroups) ehp[k].tile_off = -1;
-    }
+    // E: the wave's units are pixel groups whalf, whalf + NQ, ... of channel tile wtile (their halo records are read
+    // from LDS where they are used)
     const uint8_t *exrow = xin + (whalf * 16 + j) * a.xs + gq * 16; // + k * 32 * xs + ks * 64
     const int ecl = gq * (4 * ET) + wtile * 4;                        // the lane's 4 channels within the chunk
     // D: pixel groups whalf (+ NQ ...) of channel tile wtile; the lane's tap in k-step ks is ks * 4 + gq
