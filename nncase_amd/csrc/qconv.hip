@@ -28,7 +28,7 @@ void nnhip::describe_conv_kernel(const nncase_hip_ctx *ctx, const nncase_hip_wei
         snprintf(buf, cap, "qconv_smallc<C=%d>", w->in_channels);
         return;
     }
-    static const char *modes[] = {"rows16", "vec16", "vec8", "vec4", "bytes"};
+    static const char *modes[] = {"rows16", "vec16", "vec8", "vec4", "bytes", "rows8"};
     const int out_h = windowed_output_size(a->in_h, w->kernel_h, a->stride_h, a->dilation_h, a->pad_h_before, a->pad_h_after);
     const int out_w = windowed_output_size(a->in_w, w->kernel_w, a->stride_w, a->dilation_w, a->pad_w_before, a->pad_w_after);
     const long long m = (long long)a->batch * out_h * out_w;

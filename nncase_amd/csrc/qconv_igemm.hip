@@ -97,7 +97,8 @@ int igemm_load_mode(const nncase_hip_weights *w, const nncase_hip_conv2d_args_t 
     const bool pointwise = w->kernel_h == 1 && w->kernel_w == 1 && c->stride_h == 1 && c->stride_w == 1 &&
                            c->pad_h_before == 0 && c->pad_w_before == 0 && out_h == c->in_h && out_w == c->in_w;
     if (w->g_ic % 16 == 0) return pointwise ? kRows16 : kVec16;
-    if (w->g_ic % 8 == 0) return kVec8;
+    // (the row loader reads 16 bytes at a time: the tensor has to hold that many)
+    if (w->g_ic % 8 == 0) return pointwise && (int64_t)c->batch * c->in_h * c->in_w * w->in_channels >= 16 ? kRows8 : kVec8;
     if (w->g_ic % 4 == 0) return kVec4;
     return kBytes;
 }
@@ -125,6 +126,7 @@ int launch_qconv_igemm(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_hip_w
     a.ksteps = w->ksteps;
     a.kc_steps = w->kc_steps;
     a.ldx = w->in_channels;
+    a.x_bytes = (size_t)c->batch * c->in_h * c->in_w * w->in_channels;
     a.ldy = w->out_channels;
     a.g_ic = w->g_ic;
     a.in_h = c->in_h;
@@ -177,6 +179,7 @@ int launch_qconv_igemm(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_hip_w
         case kRows16: rc = launch_igemm_rows16(ctx, a, w->tiles, w->nchunks, rg); break;
         case kVec16: rc = launch_igemm_vec16(ctx, a, w->tiles, w->nchunks, rg); break;
         case kVec8: rc = launch_igemm_vec8(ctx, a, w->tiles, w->nchunks, rg); break;
+        case kRows8: rc = launch_igemm_rows8(ctx, a, w->tiles, w->nchunks, rg); break;
         case kVec4: rc = launch_igemm_vec4(ctx, a, w->tiles, w->nchunks, rg); break;
         default: rc = launch_igemm_bytes(ctx, a, w->tiles, w->nchunks, rg); break;
         }

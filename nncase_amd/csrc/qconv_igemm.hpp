@@ -27,6 +27,7 @@
 // mode so the instantiations compile in parallel):
 //   kRows16  1x1 / stride 1 / no padding, channels % 16 == 0: a pixel's
 //            reduction row is contiguous, one 16-byte load per lane and k-step
+//   kRows8   the same for channels % 8 == 0: the last load of a row is half used
 //   kVec16/8/4  any window; channels % VW == 0, so a VW-byte piece of the
 //            reduction never straddles two taps
 //   kBytes   anything else (e.g. 3 input channels): byte gathers
@@ -45,7 +46,8 @@ constexpr int kThreads = 256;
 constexpr int kWaves = 4;
 constexpr int kLdsFrags = 48; // weight fragments (1 KiB each) resident in LDS per block
 
-enum LoadMode { kRows16 = 0, kVec16 = 1, kVec8 = 2, kVec4 = 3, kBytes = 4 };
+enum LoadMode { kRows16 = 0, kVec16 = 1, kVec8 = 2, kVec4 = 3, kBytes = 4, kRows8 = 5 };
+constexpr bool loads_rows(int mode) { return mode == kRows16 || mode == kRows8; }
 
 struct IgemmArgs {
     const uint8_t *x;
@@ -58,6 +60,7 @@ struct IgemmArgs {
     int k;                 // reduction length
     int ksteps, kc_steps;  // total k-steps, k-steps per LDS stage
     int ldx, x_coff;       // input pixel stride / channel offset of the group (bytes)
+    size_t x_bytes;        // size of the input tensor
     int ldy, y_coff;       // output pixel stride / channel offset (elements)
     int g_ic;
     int in_h, in_w;
@@ -128,7 +131,7 @@ template <int MODE> __device__ __forceinline__ PixInfo pix_info(const IgemmArgs 
         pi.base = -1;
         return pi;
     }
-    if (MODE == kRows16) {
+    if (loads_rows(MODE)) {
         pi.base = p;
         return pi;
     }
@@ -188,11 +191,22 @@ template <int MODE> __device__ __forceinline__ ActFrag load_act(const IgemmArgs 
     const bool pix_ok = pi.base >= 0;
     PixInfo sp = pi; // any valid pixel for the address
     if (!pix_ok) sp.base = 0, sp.iy0 = 0, sp.ix0 = 0;
-    if (MODE == kRows16) {
+    if (loads_rows(MODE)) {
         const bool in_k = kc * 16 < a.k;
         const int kcc = in_k ? kc : 0;
-        f.raw = *reinterpret_cast<const u32x4 *>(a.x + (size_t)((uint32_t)sp.base * (uint32_t)a.ldx + a.x_coff + kcc * 16));
-        f.take = (pix_ok && in_k) ? 0xfu : 0u;
+        const uint32_t off = (uint32_t)sp.base * (uint32_t)a.ldx + a.x_coff + kcc * 16;
+        if (MODE == kRows16) {
+            f.raw = *reinterpret_cast<const u32x4 *>(a.x + (size_t)off);
+            f.take = (pix_ok && in_k) ? 0xfu : 0u;
+        } else {
+            // The last slice of a pixel ends 8 bytes past its channels,
+            // in the next pixel (those two dwords are replaced) or, for the tensor's last pixel, past the tensor:
+            // that one slice is read 8 bytes lower and moved up, so that nothing outside the tensor is touched.
+            const bool over = (size_t)off + 16 > a.x_bytes;
+            const u32x4 v = *reinterpret_cast<const u32x4 *>(a.x + (size_t)(over ? off - 8 : off));
+            f.raw = u32x4{over ? v[2] : v[0], over ? v[3] : v[1], v[2], v[3]};
+            f.take = (pix_ok && in_k) ? (a.k - kcc * 16 >= 16 ? 0xfu : 0x3u) : 0u;
+        }
     } else if (MODE == kBytes) {
         // byte gathers: assembled immediately (this loader does not overlap with the multiply)
         uint32_t w0 = 0x80808080u, w1 = 0x80808080u, w2 = 0x80808080u, w3 = 0x80808080u;
@@ -348,7 +362,7 @@ __device__ __forceinline__ void igemm_store_tile(const IgemmArgs &a, const v4i (
 // Blocks per compute unit the register allocation has to leave room for: four (at most 128 registers) for the
 // shapes that fit comfortably, so that the scheduler does not trade the occupancy away for longer live ranges.
 template <int T, int RG, int MODE>
-__global__ void __launch_bounds__(kThreads, ((RG == 1 && T <= 12) || MODE == kRows16) ? 4 : 2) qconv_igemm_kernel(const IgemmArgs a) {
+__global__ void __launch_bounds__(kThreads, ((RG == 1 && T <= 12) || loads_rows(MODE)) ? 4 : 2) qconv_igemm_kernel(const IgemmArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     int32_t *cterm = reinterpret_cast<int32_t *>(smem); // [T * 16]
     uint8_t *lutl = smem + T * 16 * sizeof(int32_t);    // [256] byte table of the fused unary operator
@@ -782,6 +796,7 @@ template <int MODE> int launch_mode(nncase_hip_ctx *ctx, const IgemmArgs &a, int
 int launch_igemm_rows16(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks, int rg);
 int launch_igemm_vec16(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks, int rg);
 int launch_igemm_vec8(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks, int rg);
+int launch_igemm_rows8(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks, int rg);
 int launch_igemm_vec4(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks, int rg);
 int launch_igemm_bytes(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks, int rg);
 

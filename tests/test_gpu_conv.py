@@ -178,6 +178,16 @@ def test_short_reductions_for_every_weight_zero_point(hip_ctx, zw, cin, k, pad):
         assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("cin,groups", [(8, 1), (24, 1), (40, 1), (56, 1), (72, 1), (136, 1), (200, 1), (600, 1), (16, 2), (48, 2), (120, 3)])
+@pytest.mark.parametrize("n,h,w", [(1, 1, 1), (1, 1, 2), (1, 1, 3), (2, 7, 9), (3, 16, 16)])
+def test_pointwise_rows_with_half_used_last_load(hip_ctx, cin, groups, n, h, w):
+    """1x1 layers whose channels per group are a multiple of 8 but not of 16 read rows in 16-byte pieces of which the
+    last is half used; the tensor's last pixel (and a tensor smaller than one piece) must not be read past its end.
+    Short reductions carry the weight zero point's term inside the multiplication here as well."""
+    run_case(hip_ctx, n, cin, h, w, 24 * groups, 1, 1, (1, 1), ((0, 0), (0, 0)), (1, 1), groups,
+             seed=cin * 13 + n * 5 + h + w, zx=(cin * 3 + h) & 255, zw=(cin * 7 + w) & 255, modes=("u8", "i32"))
+
+
 def _random_conv_cases(count, seed):
     rng = np.random.default_rng(seed)
     cases = []
