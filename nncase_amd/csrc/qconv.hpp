@@ -16,6 +16,7 @@ struct nncase_hip_weights {
     // igemm, reductions of at most 32: the spare half of the only k-step holds -(zw - 128) against a second copy
     // of the activations, which makes the weight zero point's share of the product part of the multiplication
     int fold = 0;
+    long long dw_const_bound = 0; // depthwise: max over channels of |bias| + 255 |sum(w - zw)|
     int64_t pixels_hint = 0; // output pixels per call the tiling was planned for (0 = unknown)
     int32_t zw = 0;
     float sw = 1.f;
@@ -152,6 +153,28 @@ __device__ __forceinline__ uint32_t requant4_u8_packed(const int32_t (&v)[4], co
             int32_t vr = v[r];
             asm volatile("" : "+v"(vr));
             const float u = div_rn((float)vr * ep.mult, ep.sy, ep.rsy) + ep.zy;
+            d = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_amdgcn_fmed3f(u, ep.qlo, ep.qhi), r, d);
+        }
+    }
+    return d;
+}
+
+// The same for accumulators already held in fp32 (exact integers).
+__device__ __forceinline__ uint32_t requant4_u8_packed(const float (&v)[4], const Epilogue &ep) {
+    uint32_t d = 0;
+    if (ep.fast) {
+        if (ep.full) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) d = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_fmaf(v[r], ep.c1, ep.c2), r, d);
+        } else {
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                d = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_amdgcn_fmed3f(__builtin_fmaf(v[r], ep.c1, ep.c2), ep.qlo, ep.qhi), r, d);
+        }
+    } else {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const float u = div_rn(v[r] * ep.mult, ep.sy, ep.rsy) + ep.zy;
             d = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_amdgcn_fmed3f(u, ep.qlo, ep.qhi), r, d);
         }
     }

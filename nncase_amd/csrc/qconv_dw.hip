@@ -45,6 +45,9 @@ struct DwArgs {
 };
 
 // Stores 4 adjacent channels of one output pixel; `o` is the element offset of the first.
+__device__ __forceinline__ void dw_store4(const DwArgs &a, uint32_t o, const float (&v)[4]) {
+    *reinterpret_cast<uint32_t *>(reinterpret_cast<uint8_t *>(a.y) + o) = requant4_u8_packed(v, a.ep);
+}
 __device__ __forceinline__ void dw_store4(const DwArgs &a, uint32_t o, const int32_t (&v)[4]) {
     if (a.ep.out_mode == kOutU8) {
         *reinterpret_cast<uint32_t *>(reinterpret_cast<uint8_t *>(a.y) + o) = requant4_u8_packed(v, a.ep);
@@ -71,7 +74,14 @@ __device__ __forceinline__ uint32_t select_u32(bool c, uint32_t yes, uint32_t no
 // computed, so a whole row of arithmetic covers their latency.
 // The stride-2 kernel holds nine input columns per row; asking for three blocks per CU keeps it
 // at 3 waves per SIMD (without the bound the allocator takes 176 VGPRs and drops to 2).
-template <int S> __global__ __launch_bounds__(kDwThreads, (S == 2 ? 3 : 1)) void dw3x3_kernel(const DwArgs a) {
+//
+// FP: the sums are kept in fp32.  The host picks this form for u8 outputs when every partial sum, the
+// per-channel constant included, stays below 2^24 in magnitude: all of them are then integers that fp32 holds
+// exactly, the result is the integer form's bit for bit, and the multiply-adds run at the full rate of the
+// vector unit (v_fma_f32) instead of the integer multiplier's lower one; the accumulators need no conversion
+// before they are requantised either.
+template <int S, bool FP> __global__ __launch_bounds__(kDwThreads, (S == 2 && !FP ? 3 : 1)) void dw3x3_kernel(const DwArgs a) {
+    using acc_t = typename std::conditional<FP, float, int32_t>::type;
     constexpr int NCOL = (kDwCols - 1) * S + 3;
     // Workgroups are dealt to the 8 XCDs round-robin, each XCD with an L2 of its own.  Renumber them
     // so that every XCD works on one contiguous run of the tensor: vertically adjacent row chunks,
@@ -101,20 +111,28 @@ template <int S> __global__ __launch_bounds__(kDwThreads, (S == 2 ? 3 : 1)) void
     const int iy_first = oy0 * S - a.pad_h;
 
     uint32_t w01[9], w23[9]; // (w - zw) of channels (0,1) and (2,3) as int16 pairs, per tap
-    int32_t ct[4];
+    float wf[9][4];          // FP: the same as floats
+    acc_t ct[4];
 #pragma unroll
     for (int tap = 0; tap < 9; tap++) {
         const uint2 raw = *reinterpret_cast<const uint2 *>(a.w + (uint32_t)(tap * a.channels + c0));
-        w01[tap] = raw.x;
-        w23[tap] = raw.y;
+        if constexpr (FP) {
+            wf[tap][0] = (float)(int16_t)(raw.x & 0xffffu);
+            wf[tap][1] = (float)((int32_t)raw.x >> 16);
+            wf[tap][2] = (float)(int16_t)(raw.y & 0xffffu);
+            wf[tap][3] = (float)((int32_t)raw.y >> 16);
+        } else {
+            w01[tap] = raw.x;
+            w23[tap] = raw.y;
+        }
     }
     {
         const int4 b = *reinterpret_cast<const int4 *>(a.bias + c0);
         const int4 s = *reinterpret_cast<const int4 *>(a.wsum + c0);
-        ct[0] = b.x - a.zx * s.x;
-        ct[1] = b.y - a.zx * s.y;
-        ct[2] = b.z - a.zx * s.z;
-        ct[3] = b.w - a.zx * s.w;
+        ct[0] = (acc_t)(b.x - a.zx * s.x);
+        ct[1] = (acc_t)(b.y - a.zx * s.y);
+        ct[2] = (acc_t)(b.z - a.zx * s.z);
+        ct[3] = (acc_t)(b.w - a.zx * s.w);
     }
 
     const uint32_t in_row = (uint32_t)(a.in_w * a.channels); // elements per input row
@@ -132,6 +150,7 @@ template <int S> __global__ __launch_bounds__(kDwThreads, (S == 2 ? 3 : 1)) void
     }
 
     uint32_t r01[3][NCOL], r23[3][NCOL]; // three most recent input rows, two channels per register
+    float rf[3][NCOL][4];                // FP: one channel per register
     int next_iy = iy_first;             // rows are fetched strictly in order
     // fetch_row only issues the loads (nothing depends on their data); unpack_row, called one
     // output row later, applies the border replacement and splits the bytes.
@@ -146,8 +165,13 @@ template <int S> __global__ __launch_bounds__(kDwThreads, (S == 2 ? 3 : 1)) void
 #pragma unroll
         for (int col = 0; col < NCOL; col++) {
             const uint32_t d = select_u32(row_ok && col_ok[col], raw[col], zx_splat);
-            r01[buf][col] = __builtin_amdgcn_perm(0u, d, 0x0c010c00u); // [b0, 0, b1, 0]
-            r23[buf][col] = __builtin_amdgcn_perm(0u, d, 0x0c030c02u); // [b2, 0, b3, 0]
+            if constexpr (FP) {
+#pragma unroll
+                for (int c = 0; c < 4; c++) rf[buf][col][c] = (float)((d >> (8 * c)) & 0xffu); // v_cvt_f32_ubyte<c>
+            } else {
+                r01[buf][col] = __builtin_amdgcn_perm(0u, d, 0x0c010c00u); // [b0, 0, b1, 0]
+                r23[buf][col] = __builtin_amdgcn_perm(0u, d, 0x0c030c02u); // [b2, 0, b3, 0]
+            }
         }
     };
 
@@ -182,7 +206,7 @@ template <int S> __global__ __launch_bounds__(kDwThreads, (S == 2 ? 3 : 1)) void
 #pragma unroll
                     for (int nr = 0; nr < S; nr++) fetch_row(pre[nr], pre_ok[nr]);
                 }
-                int32_t acc[kDwCols][4];
+                acc_t acc[kDwCols][4];
 #pragma unroll
                 for (int o = 0; o < kDwCols; o++)
 #pragma unroll
@@ -195,10 +219,15 @@ template <int S> __global__ __launch_bounds__(kDwThreads, (S == 2 ? 3 : 1)) void
 #pragma unroll
                         for (int o = 0; o < kDwCols; o++) {
                             const int col = o * S + kx, tap = ky * 3 + kx;
-                            acc[o][0] = mad16_lo(r01[buf][col], w01[tap], acc[o][0]);
-                            acc[o][1] = mad16_hi(r01[buf][col], w01[tap], acc[o][1]);
-                            acc[o][2] = mad16_lo(r23[buf][col], w23[tap], acc[o][2]);
-                            acc[o][3] = mad16_hi(r23[buf][col], w23[tap], acc[o][3]);
+                            if constexpr (FP) {
+#pragma unroll
+                                for (int c = 0; c < 4; c++) acc[o][c] = __builtin_fmaf(rf[buf][col][c], wf[tap][c], acc[o][c]);
+                            } else {
+                                acc[o][0] = mad16_lo(r01[buf][col], w01[tap], acc[o][0]);
+                                acc[o][1] = mad16_hi(r01[buf][col], w01[tap], acc[o][1]);
+                                acc[o][2] = mad16_lo(r23[buf][col], w23[tap], acc[o][2]);
+                                acc[o][3] = mad16_hi(r23[buf][col], w23[tap], acc[o][3]);
+                            }
                         }
                 }
 #pragma unroll
@@ -273,6 +302,9 @@ int prepack_depthwise(nncase_hip_ctx *ctx, nncase_hip_weights *w, const uint8_t 
             packed[(size_t)t * ch + c] = (int16_t)v;
             wsum[c] += v;
         }
+    w->dw_const_bound = 0;
+    for (int c = 0; c < ch; c++)
+        w->dw_const_bound = std::max<long long>(w->dw_const_bound, std::llabs((long long)hb[c]) + 255ll * std::llabs((long long)wsum[c]));
     w->packed_bytes = packed.size() * sizeof(int16_t);
     NNHIP_HIP(ctx, hipMalloc(&w->d_packed, w->packed_bytes));
     NNHIP_HIP(ctx, hipMalloc((void **)&w->d_wsum, sizeof(int32_t) * ch));
@@ -364,8 +396,16 @@ int launch_qconv_depthwise(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_h
         a.total = (long long)c->batch * a.row_chunks * a.strips * a.cq;
         NNHIP_REQUIRE(ctx, a.total < ((long long)1 << 31), -EINVAL, "qconv2d(depthwise): too many work items");
         const int grid = (int)((a.total + kDwThreads - 1) / kDwThreads);
-        if (c->stride_h == 1) hipLaunchKernelGGL(dw3x3_kernel<1>, dim3(grid), dim3(kDwThreads), 0, ctx->stream, a);
-        else hipLaunchKernelGGL(dw3x3_kernel<2>, dim3(grid), dim3(kDwThreads), 0, ctx->stream, a);
+        // Every partial sum is an integer of magnitude at most |bias - zx * sum(w')| + 9 * 255 * 255.
+        const bool fp = a.ep.out_mode == kOutU8 && w->dw_const_bound + 9 * 255 * 255 <= (1 << 24);
+        if (c->stride_h == 1) {
+            if (fp) hipLaunchKernelGGL((dw3x3_kernel<1, true>), dim3(grid), dim3(kDwThreads), 0, ctx->stream, a);
+            else hipLaunchKernelGGL((dw3x3_kernel<1, false>), dim3(grid), dim3(kDwThreads), 0, ctx->stream, a);
+        } else {
+            // (stride 2 holds nine input columns per row: as floats they leave room for two waves per SIMD only,
+            // and the largest stride-2 layer of MobileNetV2 runs 15 % slower that way)
+            hipLaunchKernelGGL((dw3x3_kernel<2, false>), dim3(grid), dim3(kDwThreads), 0, ctx->stream, a);
+        }
         NNHIP_LAUNCH_CHECK(ctx, "dw3x3_kernel");
         return 0;
     }

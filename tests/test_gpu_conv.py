@@ -27,11 +27,12 @@ def same_padding(size, k, stride, dilation):
     return (total // 2, total - total // 2)
 
 
-def run_case(ctx, n, c, h, w, oc, kh, kw, stride, pad, dil, groups, seed, zx=7, zw=131, clamp=None, modes=("u8", "i32", "f32")):
+def run_case(ctx, n, c, h, w, oc, kh, kw, stride, pad, dil, groups, seed, zx=7, zw=131, clamp=None, modes=("u8", "i32", "f32"),
+             bias_of=None):
     rng = np.random.default_rng(seed)
     x = rng.integers(0, 256, (n, c, h, w), dtype=np.uint8)
     wt = rng.integers(0, 256, (oc, c // groups, kh, kw), dtype=np.uint8)
-    bias = rng.integers(-3000, 3000, oc).astype(np.int32)
+    bias = rng.integers(-3000, 3000, oc).astype(np.int32) if bias_of is None else bias_of(wt).astype(np.int32)
     sx, sw = f32(0.0235), f32(0.0041)
     common = dict(stride=stride, padding=pad, dilation=dil, groups=groups)
     # the real-valued output decides the clamp and the output quantisation, so that the
@@ -186,6 +187,24 @@ def test_pointwise_rows_with_half_used_last_load(hip_ctx, cin, groups, n, h, w):
     Short reductions carry the weight zero point's term inside the multiplication here as well."""
     run_case(hip_ctx, n, cin, h, w, 24 * groups, 1, 1, (1, 1), ((0, 0), (0, 0)), (1, 1), groups,
              seed=cin * 13 + n * 5 + h + w, zx=(cin * 3 + h) & 255, zw=(cin * 7 + w) & 255, modes=("u8", "i32"))
+
+
+@pytest.mark.parametrize("edge", [0, 1, -1, 2000, 10 ** 9])
+@pytest.mark.parametrize("stride", [1, 2])
+@pytest.mark.parametrize("sign", [1, -1])
+@pytest.mark.parametrize("zx,zw", [(0, 0), (255, 255), (255, 0), (7, 131)])
+def test_depthwise_3x3_sums_at_the_edge_of_exact_fp32(hip_ctx, edge, stride, sign, zx, zw):
+    """The stride-1 3x3 kernel keeps its sums in fp32 while |bias - zx * sum(w - zw)| + 9 * 255 * 255 cannot exceed
+    2^24, and in int32 beyond: biases that put every channel exactly at that limit (edge 0), just below and above it,
+    and far above it (where the conversion of the int32 sum to fp32 rounds, as the reference's does)."""
+    limit = (1 << 24) - 9 * 255 * 255
+
+    def bias_of(wt):
+        wsum = (wt.astype(np.int64) - zw).reshape(wt.shape[0], -1).sum(axis=1)
+        return sign * (limit - 255 * np.abs(wsum) + edge)
+
+    run_case(hip_ctx, 2, 24, 13, 10, 24, 3, 3, (stride, stride), ((1, 1), (1, 1)), (1, 1), 24, seed=edge % 1000 + zx + zw + stride + sign,
+             zx=zx, zw=zw, modes=("u8", "i32"), bias_of=bias_of)
 
 
 def _random_conv_cases(count, seed):
