@@ -44,10 +44,12 @@ struct DwArgs {
     Epilogue ep;
 };
 
+// A conditional between two named objects is an lvalue in C++, which the compiler may turn
+// into a load through a selected address (private memory); taking the operands by value
+// keeps the choice a register select.
+__device__ __forceinline__ uint32_t select_u32(bool c, uint32_t yes, uint32_t no) { return c ? yes : no; }
+
 // Stores 4 adjacent channels of one output pixel; `o` is the element offset of the first.
-__device__ __forceinline__ void dw_store4(const DwArgs &a, uint32_t o, const float (&v)[4]) {
-    *reinterpret_cast<uint32_t *>(reinterpret_cast<uint8_t *>(a.y) + o) = requant4_u8_packed(v, a.ep);
-}
 __device__ __forceinline__ void dw_store4(const DwArgs &a, uint32_t o, const int32_t (&v)[4]) {
     if (a.ep.out_mode == kOutU8) {
         *reinterpret_cast<uint32_t *>(reinterpret_cast<uint8_t *>(a.y) + o) = requant4_u8_packed(v, a.ep);
@@ -63,10 +65,45 @@ __device__ __forceinline__ void dw_store4(const DwArgs &a, uint32_t o, const int
     }
 }
 
-// A conditional between two named objects is an lvalue in C++, which the compiler may turn
-// into a load through a selected address (private memory); taking the operands by value
-// keeps the choice a register select.
-__device__ __forceinline__ uint32_t select_u32(bool c, uint32_t yes, uint32_t no) { return c ? yes : no; }
+// Stores one output row of a thread: kDwCols pixels of 4 adjacent channels each; `o` is the element offset of the
+// first.  u8 rows are stored without predicates (a predicated memory instruction sits behind a branch, and
+// operations behind branches cannot be counted by the waits of the rows that follow): a pixel outside the image
+// is replaced by the first pixel of the thread's first row, address and value, which always exists, is written
+// by this thread alone and so is merely written again.  `safe_off` / `safe_val` carry that pixel; `first` is
+// uniform.
+template <typename T>
+__device__ __forceinline__ void dw_store_row(const DwArgs &a, uint32_t o, const T (&v)[kDwCols][4], const bool (&col_stored)[kDwCols],
+                                             bool row_stored, bool first, uint32_t &safe_off, uint32_t &safe_val) {
+    if (std::is_same<T, float>::value || a.ep.out_mode == kOutU8) { // (fp32 sums are used for u8 outputs only)
+        uint32_t q[kDwCols];
+#pragma unroll
+        for (int c = 0; c < kDwCols; c++) q[c] = requant4_u8_packed(v[c], a.ep);
+        safe_off = first ? o : safe_off;
+        safe_val = first ? q[0] : safe_val;
+#pragma unroll
+        for (int c = 0; c < kDwCols; c++) {
+            const bool sel = row_stored && col_stored[c];
+            const uint32_t off = select_u32(sel, o + (uint32_t)(c * a.channels), safe_off);
+            *reinterpret_cast<uint32_t *>(reinterpret_cast<uint8_t *>(a.y) + off) = select_u32(sel, q[c], safe_val);
+        }
+    } else if (a.ep.out_mode == kOutI32) {
+#pragma unroll
+        for (int c = 0; c < kDwCols; c++)
+            if (row_stored && col_stored[c])
+                *reinterpret_cast<int4 *>(reinterpret_cast<int32_t *>(a.y) + o + (uint32_t)(c * a.channels)) =
+                    int4{(int32_t)v[c][0], (int32_t)v[c][1], (int32_t)v[c][2], (int32_t)v[c][3]};
+    } else {
+#pragma unroll
+        for (int c = 0; c < kDwCols; c++) {
+            float4 f;
+            f.x = clamp_ref((float)v[c][0] * a.ep.mult, a.ep.lo, a.ep.hi);
+            f.y = clamp_ref((float)v[c][1] * a.ep.mult, a.ep.lo, a.ep.hi);
+            f.z = clamp_ref((float)v[c][2] * a.ep.mult, a.ep.lo, a.ep.hi);
+            f.w = clamp_ref((float)v[c][3] * a.ep.mult, a.ep.lo, a.ep.hi);
+            if (row_stored && col_stored[c]) *reinterpret_cast<float4 *>(reinterpret_cast<float *>(a.y) + o + (uint32_t)(c * a.channels)) = f;
+        }
+    }
+}
 
 // All offsets are 32-bit element offsets from the (uniform) tensor bases, advanced by
 // additions only; the host checks that both tensors stay below 2^31 elements.
@@ -181,31 +218,51 @@ template <int S, bool FP> __global__ __launch_bounds__(kDwThreads, (S == 2 && !F
     // Output row t (relative) reads input rows t*S + {0,1,2} (relative), kept in
     // buffer (row index mod 3).  The loop is unrolled by 3 so every buffer index
     // is a compile-time constant.
-    uint32_t pre[S][NCOL]; // rows fetched ahead for the next output row
-    bool pre_ok[S];
+    //
+    // Memory operations complete in order and the wait before a row is unpacked is a count of younger
+    // operations that may still be in flight: only operations issued on every path can be counted.  So the
+    // loop issues the same loads and stores for every thread: all threads walk a.rows rows (rows below the
+    // image are computed from clamped input rows and not stored), the loads are never predicated (addresses
+    // are clamped into the image), and the predicate of a store guards the store instruction alone, after
+    // all of its row has been requantised.  The wait for a row's loads then leaves the previous row's stores
+    // in flight instead of waiting for their acknowledgement, which used to cost a memory round trip per row.
+    //
+    // Stride 1 fetches two output rows ahead (a row of arithmetic is shorter than a trip to memory); the rows
+    // in flight rotate through three register sets so that, like the row buffers, they are named by the phase.
+    constexpr int DEPTH = S == 1 ? 2 : 1;
+    constexpr int NPRE = DEPTH == 2 ? 3 : 1;
+    uint32_t pre[NPRE][S][NCOL]; // rows fetched ahead
+    bool pre_ok[NPRE][S];
     {
-        uint32_t raw[3][NCOL];
-        bool ok[3];
+        uint32_t raw[3 - S][NCOL];
+        bool ok[3 - S];
 #pragma unroll
-        for (int b = 0; b < 3; b++) fetch_row(raw[b], ok[b]);
+        for (int b = 0; b < 3 - S; b++) fetch_row(raw[b], ok[b]);
 #pragma unroll
-        for (int b = 0; b < 3; b++) unpack_row(b, raw[b], ok[b]);
+        for (int d = 0; d < DEPTH; d++)
+#pragma unroll
+            for (int nr = 0; nr < S; nr++) fetch_row(pre[d][nr], pre_ok[d][nr]);
+#pragma unroll
+        for (int b = 0; b < 3 - S; b++) unpack_row(b, raw[b], ok[b]);
     }
-    const int nrows = min(a.rows, a.out_h - oy0); // >= 1
+    const int nrows = a.rows;              // uniform
+    const int rows_here = a.out_h - oy0;   // rows of this thread that exist (>= 1)
+    uint32_t safe_off = 0, safe_val = 0;
+    bool col_stored[kDwCols];
+#pragma unroll
+    for (int o = 0; o < kDwCols; o++) col_stored[o] = ox0 + o < a.out_w;
     for (int t0 = 0; t0 < nrows; t0 += 3) {
 #pragma unroll
         for (int ph = 0; ph < 3; ph++) {
             const int tt = t0 + ph;
             if (tt < nrows) {
-                if (tt > 0) {
-                    // input rows (tt-1)*S + 3 + nr; tt % 3 == ph fixes their residue mod 3
+                // input rows tt*S + 3 - S + nr; tt % 3 == ph fixes their residue mod 3
 #pragma unroll
-                    for (int nr = 0; nr < S; nr++) unpack_row((((ph + 2) % 3) * S + 3 + nr) % 3, pre[nr], pre_ok[nr]);
-                }
-                if (tt + 1 < nrows) {
+                for (int nr = 0; nr < S; nr++) unpack_row((ph * S + 3 - S + nr) % 3, pre[DEPTH == 2 ? ph : 0][nr], pre_ok[DEPTH == 2 ? ph : 0][nr]);
+                // (also issued by the last rows, which need nothing more: a load that only some paths issue
+                // could not be counted either, and its address is clamped into the image like any other)
 #pragma unroll
-                    for (int nr = 0; nr < S; nr++) fetch_row(pre[nr], pre_ok[nr]);
-                }
+                for (int nr = 0; nr < S; nr++) fetch_row(pre[DEPTH == 2 ? (ph + 2) % 3 : 0][nr], pre_ok[DEPTH == 2 ? (ph + 2) % 3 : 0][nr]);
                 acc_t acc[kDwCols][4];
 #pragma unroll
                 for (int o = 0; o < kDwCols; o++)
@@ -230,16 +287,13 @@ template <int S, bool FP> __global__ __launch_bounds__(kDwThreads, (S == 2 && !F
                             }
                         }
                 }
-#pragma unroll
-                for (int o = 0; o < kDwCols; o++)
-                    if (ox0 + o < a.out_w) dw_store4(a, out_off + (uint32_t)(o * a.channels), acc[o]);
+                dw_store_row(a, out_off, acc, col_stored, tt < rows_here, tt == 0, safe_off, safe_val);
                 out_off += out_row;
             }
         }
     }
 }
 
-// One thread per (pixel, VEC channels); every tap is fetched from memory.
 template <int VEC> __global__ __launch_bounds__(kDwThreads) void dw_generic_kernel(const DwArgs a) {
     const long long gid = (long long)blockIdx.x * kDwThreads + threadIdx.x;
     if (gid >= a.total) return;
