@@ -181,6 +181,16 @@ __device__ __forceinline__ uint32_t requant4_u8_packed(const float (&v)[4], cons
     return d;
 }
 
+// The one-instruction-per-code form alone, for kernels that are instantiated separately for layers whose
+// epilogue has fast != 0 and full != 0: no branch on the epilogue's flags is left in the instruction stream,
+// so the conversions of a row can be scheduled among its stores and the loads of the rows that follow.
+template <typename T> __device__ __forceinline__ uint32_t requant4_u8_packed_direct(const T (&v)[4], const Epilogue &ep) {
+    uint32_t d = 0;
+#pragma unroll
+    for (int r = 0; r < 4; r++) d = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_fmaf((float)v[r], ep.c1, ep.c2), r, d);
+    return d;
+}
+
 // Packs the low bytes of four dwords into one dword (3 byte-permutes).
 __device__ __forceinline__ uint32_t pack_low_bytes(uint32_t b0, uint32_t b1, uint32_t b2, uint32_t b3) {
     const uint32_t lo = __builtin_amdgcn_perm(b1, b0, 0x0c0c0400u); // [b0.0, b1.0, 0, 0]

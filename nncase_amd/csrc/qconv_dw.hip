@@ -71,13 +71,13 @@ __device__ __forceinline__ void dw_store4(const DwArgs &a, uint32_t o, const int
 // is replaced by the first pixel of the thread's first row, address and value, which always exists, is written
 // by this thread alone and so is merely written again.  `safe_off` / `safe_val` carry that pixel; `first` is
 // uniform.
-template <typename T>
+template <bool FF, typename T>
 __device__ __forceinline__ void dw_store_row(const DwArgs &a, uint32_t o, const T (&v)[kDwCols][4], const bool (&col_stored)[kDwCols],
                                              bool row_stored, bool first, uint32_t &safe_off, uint32_t &safe_val) {
-    if (std::is_same<T, float>::value || a.ep.out_mode == kOutU8) { // (fp32 sums are used for u8 outputs only)
+    if (FF || std::is_same<T, float>::value || a.ep.out_mode == kOutU8) { // (fp32 sums are used for u8 outputs only)
         uint32_t q[kDwCols];
 #pragma unroll
-        for (int c = 0; c < kDwCols; c++) q[c] = requant4_u8_packed(v[c], a.ep);
+        for (int c = 0; c < kDwCols; c++) q[c] = FF ? requant4_u8_packed_direct(v[c], a.ep) : requant4_u8_packed(v[c], a.ep);
         safe_off = first ? o : safe_off;
         safe_val = first ? q[0] : safe_val;
 #pragma unroll
@@ -117,7 +117,8 @@ __device__ __forceinline__ void dw_store_row(const DwArgs &a, uint32_t o, const 
 // exactly, the result is the integer form's bit for bit, and the multiply-adds run at the full rate of the
 // vector unit (v_fma_f32) instead of the integer multiplier's lower one; the accumulators need no conversion
 // before they are requantised either.
-template <int S, bool FP> __global__ __launch_bounds__(kDwThreads, (S == 2 && !FP ? 3 : 1)) void dw3x3_kernel(const DwArgs a) {
+// FF: the layer's epilogue is the one-instruction requantisation to u8 (fast and full), fixed at compile time.
+template <int S, bool FP, bool FF> __global__ __launch_bounds__(kDwThreads, (S == 2 && !FP ? 3 : 1)) void dw3x3_kernel(const DwArgs a) {
     using acc_t = typename std::conditional<FP, float, int32_t>::type;
     constexpr int NCOL = (kDwCols - 1) * S + 3;
     // Workgroups are dealt to the 8 XCDs round-robin, each XCD with an L2 of its own.  Renumber them
@@ -287,7 +288,7 @@ template <int S, bool FP> __global__ __launch_bounds__(kDwThreads, (S == 2 && !F
                             }
                         }
                 }
-                dw_store_row(a, out_off, acc, col_stored, tt < rows_here, tt == 0, safe_off, safe_val);
+                dw_store_row<FF>(a, out_off, acc, col_stored, tt < rows_here, tt == 0, safe_off, safe_val);
                 out_off += out_row;
             }
         }
@@ -452,13 +453,18 @@ int launch_qconv_depthwise(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_h
         const int grid = (int)((a.total + kDwThreads - 1) / kDwThreads);
         // Every partial sum is an integer of magnitude at most |bias - zx * sum(w')| + 9 * 255 * 255.
         const bool fp = a.ep.out_mode == kOutU8 && w->dw_const_bound + 9 * 255 * 255 <= (1 << 24);
+        const bool ff = a.ep.out_mode == kOutU8 && a.ep.fast && a.ep.full;
+        const dim3 g(grid), t(kDwThreads);
         if (c->stride_h == 1) {
-            if (fp) hipLaunchKernelGGL((dw3x3_kernel<1, true>), dim3(grid), dim3(kDwThreads), 0, ctx->stream, a);
-            else hipLaunchKernelGGL((dw3x3_kernel<1, false>), dim3(grid), dim3(kDwThreads), 0, ctx->stream, a);
+            if (fp && ff) hipLaunchKernelGGL((dw3x3_kernel<1, true, true>), g, t, 0, ctx->stream, a);
+            else if (fp) hipLaunchKernelGGL((dw3x3_kernel<1, true, false>), g, t, 0, ctx->stream, a);
+            else if (ff) hipLaunchKernelGGL((dw3x3_kernel<1, false, true>), g, t, 0, ctx->stream, a);
+            else hipLaunchKernelGGL((dw3x3_kernel<1, false, false>), g, t, 0, ctx->stream, a);
         } else {
             // (stride 2 holds nine input columns per row: as floats they leave room for two waves per SIMD only,
             // and the largest stride-2 layer of MobileNetV2 runs 15 % slower that way)
-            hipLaunchKernelGGL((dw3x3_kernel<2, false>), dim3(grid), dim3(kDwThreads), 0, ctx->stream, a);
+            if (ff) hipLaunchKernelGGL((dw3x3_kernel<2, false, true>), g, t, 0, ctx->stream, a);
+            else hipLaunchKernelGGL((dw3x3_kernel<2, false, false>), g, t, 0, ctx->stream, a);
         }
         NNHIP_LAUNCH_CHECK(ctx, "dw3x3_kernel");
         return 0;
