@@ -309,17 +309,21 @@ template <int D, int NT> __global__ __launch_bounds__(kAttnThreads, 2) void page
 }
 
 
-} // namespace nnhip
 
-using namespace nnhip;
+// Sets `count` 32-bit words to zero (counter areas are cleared with a kernel, not a memset node, so
+// the call may sit inside a captured graph).
+__global__ void attn_zero_u32_kernel(uint32_t *p, size_t count) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x) p[i] = 0u;
+}
 
-extern "C" int nncase_hip_paged_attention_decode(nncase_hip_ctx_t *ctx, const void *q_dev, const void *k_cache_dev,
-                                                 const void *v_cache_dev, const int32_t *block_table_dev,
-                                                 const int32_t *ctx_lens_dev, void *out_dev,
-                                                 const nncase_hip_paged_attn_args_t *p) {
-    NNHIP_CHECK_CTX(ctx);
-    NNHIP_REQUIRE(ctx, q_dev && k_cache_dev && v_cache_dev && block_table_dev && ctx_lens_dev && out_dev && p, -EINVAL,
-                  "paged_attention_decode: null argument");
+// Everything a launch needs except the buffers: checked geometry, split plan, sizes of the scratch areas.
+struct AttnPlan {
+    AttnArgs a;
+    int nt = 2;
+    size_t partial_bytes = 0, counter_bytes = 0;
+};
+
+static int attn_plan(nncase_hip_ctx *ctx, const nncase_hip_paged_attn_args_t *p, AttnPlan *plan) {
     NNHIP_REQUIRE(ctx, p->batch > 0 && p->num_q_heads > 0 && p->num_kv_heads > 0 && p->max_blocks_per_seq > 0 &&
                            p->num_blocks > 0,
                   -EINVAL, "paged_attention_decode: non-positive dimension");
@@ -336,14 +340,8 @@ extern "C" int nncase_hip_paged_attention_decode(nncase_hip_ctx_t *ctx, const vo
                   -NNCASE_HIP_ERR_DATATYPE_MISMATCH, "paged_attention_decode: output type 0x%x", p->out_dtype);
     NNHIP_REQUIRE(ctx, (int64_t)p->batch * p->num_kv_heads < (int64_t(1) << 31), -EINVAL, "paged_attention_decode: grid too large");
 
-    AttnArgs a;
+    AttnArgs &a = plan->a;
     memset(&a, 0, sizeof(a));
-    a.q = (const uint16_t *)q_dev;
-    a.k_cache = (const uint16_t *)k_cache_dev;
-    a.v_cache = (const uint16_t *)v_cache_dev;
-    a.block_table = block_table_dev;
-    a.ctx_lens = ctx_lens_dev;
-    a.out = out_dev;
     a.batch = p->batch;
     a.hq = p->num_q_heads;
     a.hkv = p->num_kv_heads;
@@ -362,6 +360,7 @@ extern "C" int nncase_hip_paged_attention_decode(nncase_hip_ctx_t *ctx, const vo
     while (nt < nt_max && (splits_at(nt) > kAttnMaxSplits ||
                            (int64_t)p->batch * p->num_kv_heads * splits_at(nt * 2) >= (int64_t)3 * ctx->compute_units))
         nt *= 2;
+    plan->nt = nt;
     a.split_tokens = kAttnWaves * nt * 16;
     a.splits = (int)((max_tokens + a.split_tokens - 1) / a.split_tokens);
     NNHIP_REQUIRE(ctx, a.splits <= kAttnMaxSplits, -EINVAL,
@@ -370,35 +369,26 @@ extern "C" int nncase_hip_paged_attention_decode(nncase_hip_ctx_t *ctx, const vo
     a.d_block = make_fastdiv((uint32_t)p->block_size);
     a.scale_log2e = p->scale * kLog2e;
     a.out_f16 = p->out_dtype == NNCASE_HIP_DT_F16;
+    plan->partial_bytes = (size_t)a.batch * a.hq * a.splits * (a.d + 2) * sizeof(float);
+    plan->counter_bytes = (size_t)a.batch * a.hkv * sizeof(uint32_t);
+    return 0;
+}
 
-    const size_t rows = (size_t)a.batch * a.hq * a.splits;
-    const size_t need = rows * (a.d + 2) * sizeof(float);
-    if (ctx->attn_ws_bytes < need) {
-        NNHIP_HIP(ctx, hipStreamSynchronize(ctx->stream));
-        if (ctx->attn_ws) NNHIP_HIP(ctx, hipFree(ctx->attn_ws));
-        ctx->attn_ws = nullptr;
-        ctx->attn_ws_bytes = 0;
-        NNHIP_HIP(ctx, hipMalloc(&ctx->attn_ws, need));
-        ctx->attn_ws_bytes = need;
-    }
-    const size_t counters = (size_t)a.batch * a.hkv * sizeof(uint32_t);
-    if (ctx->attn_done_bytes < counters) {
-        NNHIP_HIP(ctx, hipStreamSynchronize(ctx->stream));
-        if (ctx->attn_done) NNHIP_HIP(ctx, hipFree(ctx->attn_done));
-        ctx->attn_done = nullptr;
-        ctx->attn_done_bytes = 0;
-        const size_t cap = (counters + 4095) / 4096 * 4096;
-        NNHIP_HIP(ctx, hipMalloc(&ctx->attn_done, cap));
-        ctx->attn_done_bytes = cap;
-        // zero before the first launch; every launch leaves the counters it used at zero again
-        NNHIP_HIP(ctx, hipMemsetAsync(ctx->attn_done, 0, cap, ctx->stream));
-    }
-    a.done = reinterpret_cast<uint32_t *>(ctx->attn_done);
-    a.part_o = reinterpret_cast<float *>(ctx->attn_ws);
-    a.part_ml = a.part_o + rows * a.d;
-
+static int attn_launch(nncase_hip_ctx *ctx, AttnPlan &plan, const void *q_dev, const void *k_cache_dev, const void *v_cache_dev,
+                       const int32_t *block_table_dev, const int32_t *ctx_lens_dev, void *out_dev, void *partials, void *counters) {
+    AttnArgs &a = plan.a;
+    a.q = (const uint16_t *)q_dev;
+    a.k_cache = (const uint16_t *)k_cache_dev;
+    a.v_cache = (const uint16_t *)v_cache_dev;
+    a.block_table = block_table_dev;
+    a.ctx_lens = ctx_lens_dev;
+    a.out = out_dev;
+    a.done = reinterpret_cast<uint32_t *>(counters);
+    a.part_o = reinterpret_cast<float *>(partials);
+    a.part_ml = a.part_o + (size_t)a.batch * a.hq * a.splits * a.d;
     const dim3 grid(a.hkv * a.batch, a.splits);
     const dim3 block(kAttnThreads);
+    const int nt = plan.nt;
     if (a.d == 64) {
         if (nt == 8) hipLaunchKernelGGL((paged_attn_kernel<64, 8>), grid, block, 0, ctx->stream, a);
         else if (nt == 4) hipLaunchKernelGGL((paged_attn_kernel<64, 4>), grid, block, 0, ctx->stream, a);
@@ -409,4 +399,66 @@ extern "C" int nncase_hip_paged_attention_decode(nncase_hip_ctx_t *ctx, const vo
     }
     NNHIP_LAUNCH_CHECK(ctx, "paged_attn_kernel");
     return 0;
+}
+
+// Makes the context's split workspace and counters large enough for this geometry.  Growth frees the
+// old areas, so it is refused while a captured graph holds their addresses (-EBUSY) and while the
+// context's stream is capturing (an allocation and a synchronisation would invalidate the capture):
+// resident functions reserve when the operator is recorded, before any capture.
+int attn_reserve(nncase_hip_ctx *ctx, const nncase_hip_paged_attn_args_t *p) {
+    AttnPlan plan;
+    const int rc = attn_plan(ctx, p, &plan);
+    if (rc) return rc;
+    if (ctx->attn_ws_bytes >= plan.partial_bytes && ctx->attn_done_bytes >= plan.counter_bytes) return 0;
+    NNHIP_REQUIRE(ctx, ctx->attn_pins == 0, -EBUSY,
+                  "paged_attention_decode: the split workspace would have to grow (%zu -> %zu bytes) while %d captured "
+                  "function(s) refer to it; record the larger operator before capturing",
+                  ctx->attn_ws_bytes, plan.partial_bytes, ctx->attn_pins);
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    NNHIP_HIP(ctx, hipStreamIsCapturing(ctx->stream, &cs));
+    NNHIP_REQUIRE(ctx, cs == hipStreamCaptureStatusNone, -EBUSY,
+                  "paged_attention_decode: the split workspace cannot be allocated while the stream is capturing");
+    NNHIP_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    if (ctx->attn_ws_bytes < plan.partial_bytes) {
+        if (ctx->attn_ws) NNHIP_HIP(ctx, hipFree(ctx->attn_ws));
+        ctx->attn_ws = nullptr;
+        ctx->attn_ws_bytes = 0;
+        NNHIP_HIP(ctx, hipMalloc(&ctx->attn_ws, plan.partial_bytes));
+        ctx->attn_ws_bytes = plan.partial_bytes;
+    }
+    if (ctx->attn_done_bytes < plan.counter_bytes) {
+        if (ctx->attn_done) NNHIP_HIP(ctx, hipFree(ctx->attn_done));
+        ctx->attn_done = nullptr;
+        ctx->attn_done_bytes = 0;
+        const size_t cap = (plan.counter_bytes + 4095) / 4096 * 4096;
+        NNHIP_HIP(ctx, hipMalloc(&ctx->attn_done, cap));
+        ctx->attn_done_bytes = cap;
+        // zero before the first launch; every launch leaves the counters it used at zero again
+        hipLaunchKernelGGL(attn_zero_u32_kernel, dim3(4), dim3(256), 0, ctx->stream, (uint32_t *)ctx->attn_done, cap / 4);
+        NNHIP_LAUNCH_CHECK(ctx, "attn_zero_u32_kernel");
+        NNHIP_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    }
+    return 0;
+}
+
+} // namespace nnhip
+
+using namespace nnhip;
+
+extern "C" int nncase_hip_paged_attention_decode(nncase_hip_ctx_t *ctx, const void *q_dev, const void *k_cache_dev,
+                                                 const void *v_cache_dev, const int32_t *block_table_dev,
+                                                 const int32_t *ctx_lens_dev, void *out_dev,
+                                                 const nncase_hip_paged_attn_args_t *p) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, q_dev && k_cache_dev && v_cache_dev && block_table_dev && ctx_lens_dev && out_dev && p, -EINVAL,
+                  "paged_attention_decode: null argument");
+    AttnPlan plan;
+    int rc = attn_plan(ctx, p, &plan);
+    if (rc) return rc;
+    if (ctx->attn_ws_bytes < plan.partial_bytes || ctx->attn_done_bytes < plan.counter_bytes) {
+        rc = attn_reserve(ctx, p);
+        if (rc) return rc;
+    }
+    return attn_launch(ctx, plan, q_dev, k_cache_dev, v_cache_dev, block_table_dev, ctx_lens_dev, out_dev, ctx->attn_ws,
+                       ctx->attn_done);
 }

@@ -19,12 +19,15 @@ struct nncase_hip_ctx {
     int compute_units = 0;
     int clock_khz = 0;
     size_t hbm_bytes = 0;
-    // paged-attention partials and completion counters: grown on demand, owned by the context
-    // (calls on one context are ordered on its stream, so they can share it)
+    // paged-attention partials and completion counters, owned by the context (calls on one context
+    // are ordered on its stream, so they can share them).  Sized when an attention operator is
+    // recorded into a function or first called eagerly; never moved while a captured graph holds
+    // their addresses (attn_pins = captured functions with an attention operator).
     void *attn_ws = nullptr;
     size_t attn_ws_bytes = 0;
     void *attn_done = nullptr; // counters live apart from the partials: they must stay zero between calls
     size_t attn_done_bytes = 0;
+    int attn_pins = 0;
     char last_error[512] = {0};
 };
 
@@ -121,5 +124,9 @@ __device__ __forceinline__ uint32_t fastdiv(uint32_t n, const FastDiv &f) {
 }
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+// attn.hip: checks the geometry and sizes the context's paged-attention workspace for it
+// (-EBUSY if that needs a reallocation while a captured graph refers to it or the stream is capturing).
+int attn_reserve(nncase_hip_ctx *ctx, const nncase_hip_paged_attn_args_t *geometry);
 
 } // namespace nnhip

@@ -49,6 +49,7 @@ struct nncase_hip_function {
     int cur_lane = 0, nlanes = 1;
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
+    bool pins_attn = false; // the captured graph holds the addresses of the context's attention workspace
 };
 
 using namespace nnhip;
@@ -110,6 +111,8 @@ static void drop_graph(nncase_hip_function *fn) {
     if (fn->graph) (void)hipGraphDestroy(fn->graph);
     fn->exec = nullptr;
     fn->graph = nullptr;
+    if (fn->pins_attn) fn->ctx->attn_pins--;
+    fn->pins_attn = false;
 }
 
 static int push(nncase_hip_function *fn, const Op &op) {
@@ -335,6 +338,10 @@ extern "C" int nncase_hip_function_add_paged_attention_decode(nncase_hip_functio
     if (!fn) return -EINVAL;
     NNHIP_REQUIRE(fn->ctx, q_dev && k_cache_dev && v_cache_dev && block_table_dev && ctx_lens_dev && out_dev && args, -EINVAL,
                   "function_add_paged_attention_decode: null argument");
+    // the workspace the kernel's splits go through is sized now: capture must not allocate, and a graph
+    // keeps the addresses it was captured with
+    const int rc = attn_reserve(fn->ctx, args);
+    if (rc) return rc;
     Op op;
     op.kind = Op::kAttn;
     op.in0 = q_dev, op.in1 = k_cache_dev, op.in2 = v_cache_dev, op.in3 = block_table_dev, op.in4 = ctx_lens_dev, op.out = out_dev;
@@ -469,6 +476,10 @@ extern "C" int nncase_hip_function_capture(nncase_hip_function_t *fn) {
     if (ie != hipSuccess) {
         drop_graph(fn);
         return hip_fail(ctx, ie, "hipGraphInstantiate");
+    }
+    if (attn_lane >= 0) {
+        fn->pins_attn = true;
+        ctx->attn_pins++;
     }
     return 0;
 }

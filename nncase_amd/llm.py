@@ -133,12 +133,7 @@ class HipDecoder:
         fn.add_argmax_f32(self.logits, self.tokens if feedback else self.next_tokens, batch, c.vocab)
         fn.add_add_i32(self.ctx_lens, batch, 1)   # the step is complete: the caches hold one more token
         self.fn = fn
-        # warm-up (sizes the attention workspace before capture) on a scratch copy of the state it changes:
-        # the caches get the token appended again by the first real step, the lengths are restored
-        self.tokens.upload(np.zeros(batch, np.int32))
-        fn.invoke()
-        ctx.sync()
-        self.ctx_lens.upload(np.ascontiguousarray(ctx_lens, np.int32))
+        # nothing to warm up: recording the attention operators has already sized their workspace
         if capture_graph:
             fn.capture()
 

@@ -147,3 +147,52 @@ def test_error_paths(hip_ctx):
     with pytest.raises(rt.HipError) as e:
         K.paged_attention_decode(q, kc, K.v_cache_from_token_major(vc), bt, cl, 0.125, ctx=hip_ctx)
     assert e.value.code == -rt.ERR_SHAPE_MISMATCH
+
+
+def test_capture_without_a_warm_up_and_pinned_workspace(hip_ctx):
+    """Recording the operator sizes the context's split workspace, so a capture needs no eager call first;
+    while the captured function lives, a call that would have to move the workspace is refused (-EBUSY)
+    instead of freeing memory the graph still addresses."""
+    import errno
+    from nncase_amd import runtime as rt
+    from nncase_amd.runtime import Context, Function
+    ctx = Context(0)  # a context of its own: its workspace starts empty
+    try:
+        rng = np.random.default_rng(99)
+        q, kc, vc, bt, cl = make_case(rng, 3, 14, 2, 64, 16, 2048, [2048, 700, 33])
+        vt = K.v_cache_from_token_major(vc)
+        dq, dk, dv, dbt, dcl = (ctx.to_device(t) for t in (q, kc, vt, bt, cl))
+        dout = ctx.alloc(q.size * 4)
+        args = rt.PagedAttnArgs(3, 14, 2, 64, 16, bt.shape[1], kc.shape[0], 0.125, rt.DT_F32)
+        fn = Function(ctx)
+        fn.add_paged_attention_decode(dq, dk, dv, dbt, dcl, dout, args)
+        fn.capture()                       # no eager call came before
+        want = O.paged_attention_decode(q.view(np.uint16), kc.view(np.uint16), vt.view(np.uint16), bt, cl, 0.125)
+        first = None
+        for _ in range(3):
+            dout.fill(0)
+            fn.invoke()
+            ctx.sync()
+            got = dout.download(q.shape, np.float32)
+            assert (np.abs(got - want) <= RTOL * np.abs(want).max(axis=-1, keepdims=True) + 1e-6).all()
+            first = got if first is None else first
+            assert np.array_equal(got, first)
+        # a larger geometry on the same context would move the workspace under the graph
+        q2, kc2, vc2, bt2, cl2 = make_case(rng, 16, 14, 2, 64, 16, 4096)
+        big = rt.PagedAttnArgs(16, 14, 2, 64, 16, bt2.shape[1], kc2.shape[0], 0.125, rt.DT_F32)
+        d2 = [ctx.to_device(t) for t in (q2, kc2, K.v_cache_from_token_major(vc2), bt2, cl2)]
+        dout2 = ctx.alloc(q2.size * 4)
+        with pytest.raises(rt.HipError) as e:
+            ctx.paged_attention_decode(*d2, dout2, big)
+        assert e.value.code == -errno.EBUSY
+        fn.invoke()                        # the graph still replays on intact memory
+        ctx.sync()
+        assert np.array_equal(dout.download(q.shape, np.float32), first)
+        fn.destroy()                       # nothing refers to the workspace any more: growth is allowed again
+        ctx.paged_attention_decode(*d2, dout2, big)
+        ctx.sync()
+        want2 = O.paged_attention_decode(q2.view(np.uint16), kc2.view(np.uint16), d2 and K.v_cache_from_token_major(vc2).view(np.uint16), bt2, cl2, 0.125)
+        got2 = dout2.download(q2.shape, np.float32)
+        assert (np.abs(got2 - want2) <= RTOL * np.abs(want2).max(axis=-1, keepdims=True) + 1e-6).all()
+    finally:
+        ctx.close()
