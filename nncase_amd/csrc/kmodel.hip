@@ -113,17 +113,30 @@ extern "C" int nncase_hip_kmodel_destroy(nncase_hip_kmodel_t *m) {
     return 0;
 }
 
-// Finds section `name` among `count` section records starting at `pos`; bodies are addressed by
-// absolute position in the file.
-static bool find_section(const uint8_t *file, size_t size, size_t pos, uint32_t count, const char *name, Span *out) {
+// Finds section `name` among `count` section records starting at `pos`, as runtime::find_section does
+// (src/Native/src/runtime/section.cpp:58-91): the body starts body_start bytes behind the section
+// header (the writer stores the alignment padding there, src/Nncase.CodeGen/CodeGen/LinkedModel.cs:160),
+// or, for a section flagged SECTION_MERGED_INTO_RDATA (model.h:76), body_start bytes into the body of
+// the list's ".rdata" section.
+static bool find_section(const uint8_t *file, size_t size, size_t first, uint32_t count, const char *name, Span *out, int depth = 0) {
+    size_t pos = first;
     for (uint32_t i = 0; i < count; i++) {
         if (pos + sizeof(section_header) > size) return false;
         section_header h;
         memcpy(&h, file + pos, sizeof(h));
         if (h.size < sizeof(h) || h.size > size - pos) return false;
         if (strncmp(h.name, name, 16) == 0) {
-            if (h.body_start > size || h.body_size > size - h.body_start) return false;
-            out->p = file + h.body_start;
+            if (h.flags & 1u) { // merged into .rdata
+                Span rdata;
+                if (depth > 0 || !find_section(file, size, first, count, ".rdata", &rdata, depth + 1)) return false;
+                if (h.body_start > rdata.n || h.body_size > rdata.n - h.body_start) return false;
+                out->p = rdata.p + h.body_start;
+                out->n = (size_t)h.body_size;
+                return true;
+            }
+            const size_t body0 = pos + sizeof(section_header);
+            if (h.body_start > size - body0 || h.body_size > size - body0 - h.body_start) return false;
+            out->p = file + body0 + (size_t)h.body_start;
             out->n = (size_t)h.body_size;
             return true;
         }
@@ -148,38 +161,118 @@ extern "C" int nncase_hip_kmodel_load(nncase_hip_ctx_t *ctx, const void *data, s
     NNHIP_REQUIRE(ctx, mh.entry_module != 0xFFFFFFFFu && mh.entry_module < mh.modules, -EINVAL,
                   "kmodel_load: model has no entry function");
 
-    // ---- walk to the entry module ------------------------------------------------------------
-    size_t pos = sizeof(model_header);
-    module_header modh{};
-    for (uint32_t i = 0;; i++) {
-        NNHIP_REQUIRE(ctx, pos + sizeof(module_header) <= size, -EINVAL, "kmodel_load: truncated module header");
-        memcpy(&modh, file + pos, sizeof(modh));
-        NNHIP_REQUIRE(ctx, modh.size >= sizeof(modh) && modh.size <= size - pos, -EINVAL, "kmodel_load: bad module size");
-        if (i == mh.entry_module) break;
-        pos += (size_t)modh.size;
+    // ---- locate the hip function ------------------------------------------------------------------
+    // Modules are skipped by their size field (interpreter.cpp:55-70), functions likewise
+    // (skip_functions, runtime_module.cpp:112-117); the module sections follow the functions.
+    struct Located {
+        module_header modh{};
+        function_header fh{};
+        size_t sections_pos = 0;
+    };
+    auto locate = [&](uint32_t module_id, uint32_t function_id, Located *loc) -> int {
+        NNHIP_REQUIRE(ctx, module_id < mh.modules, -NNCASE_HIP_ERR_RUNTIME_NOT_FOUND, "kmodel_load: module %u of %u", module_id,
+                      mh.modules);
+        size_t pos = sizeof(model_header);
+        for (uint32_t i = 0;; i++) {
+            NNHIP_REQUIRE(ctx, pos + sizeof(module_header) <= size, -EINVAL, "kmodel_load: truncated module header");
+            memcpy(&loc->modh, file + pos, sizeof(module_header));
+            NNHIP_REQUIRE(ctx, loc->modh.size >= sizeof(module_header) && loc->modh.size <= size - pos, -EINVAL,
+                          "kmodel_load: bad module size");
+            if (i == module_id) break;
+            pos += (size_t)loc->modh.size;
+        }
+        NNHIP_REQUIRE(ctx, function_id < loc->modh.functions, -EINVAL, "kmodel_load: function %u of %u in module %u",
+                      function_id, loc->modh.functions, module_id);
+        const size_t module_end = pos + (size_t)loc->modh.size;
+        size_t fpos = pos + sizeof(module_header);
+        for (uint32_t i = 0; i < loc->modh.functions; i++) {
+            NNHIP_REQUIRE(ctx, fpos + sizeof(function_header) <= module_end, -EINVAL, "kmodel_load: truncated function header");
+            function_header h;
+            memcpy(&h, file + fpos, sizeof(h));
+            NNHIP_REQUIRE(ctx, h.size >= sizeof(h) && h.size <= module_end - fpos, -EINVAL, "kmodel_load: bad function size");
+            if (i == function_id) loc->fh = h;
+            fpos += (size_t)h.size;
+        }
+        loc->sections_pos = fpos;
+        return 0;
+    };
+    auto function_text = [&](const Located &loc, Span *text, Span *rdata) -> int {
+        Span text_all;
+        NNHIP_REQUIRE(ctx, find_section(file, size, loc.sections_pos, loc.modh.sections, ".text", &text_all), -EINVAL,
+                      "kmodel_load: module \"%.16s\" has no .text section", loc.modh.kind);
+        if (!find_section(file, size, loc.sections_pos, loc.modh.sections, ".rdata", rdata)) *rdata = Span{};
+        NNHIP_REQUIRE(ctx, loc.fh.entrypoint <= text_all.n && loc.fh.text_size <= text_all.n - loc.fh.entrypoint, -EINVAL,
+                      "kmodel_load: function text outside the .text section");
+        text->p = text_all.p + loc.fh.entrypoint;
+        text->n = (size_t)loc.fh.text_size;
+        return 0;
+    };
+    Located loc;
+    int lrc = locate(mh.entry_module, mh.entry_function, &loc);
+    if (lrc) return lrc;
+    Span text_span, rdata;
+    if (strncmp(loc.modh.kind, "stackvm", 16) == 0) {
+        // A compiled kmodel's entry is a stackvm function; the only one this loader runs is the call
+        // stub the compiler emits around a function of another module
+        // (modules/Nncase.Modules.StackVM/CodeGen/StackVM/CodegenVisitor.cs:281-315,470-476):
+        //   LDARG n-1 .. LDARG 0 ; LDC_I4 function id ; LDC_I4 module id ; EXTCALL args, is_prim_func ; RET
+        // with the encodings of src/Native/include/nncase/runtime/stackvm/op_reader.h:59-64,83-90,116-122,386-392
+        // (opcode byte, operands unaligned little-endian) and EXTCALL's pop order of
+        // src/Native/src/runtime/stackvm/ops/control.cpp:25-47.  Any other text needs the stackvm
+        // interpreter, which is not this library.
+        Span sv, sv_rdata;
+        lrc = function_text(loc, &sv, &sv_rdata);
+        if (lrc) return lrc;
+        size_t pc = 0;
+        auto rd = [&](void *dst, size_t n) {
+            if (pc + n > sv.n) return false;
+            memcpy(dst, sv.p + pc, n);
+            pc += n;
+            return true;
+        };
+        uint32_t n_ldarg = 0;
+        bool ok = true;
+        for (;;) { // arguments are pushed last first, so that EXTCALL pops them in declaration order
+            uint8_t opc = 0;
+            if (pc >= sv.n) { ok = false; break; }
+            opc = sv.p[pc];
+            uint16_t index = 0;
+            if (opc == 39) { // LDARG u16
+                pc++;
+                if (!rd(&index, 2)) { ok = false; break; }
+            } else if (opc >= 40 && opc <= 45) { // LDARG_0 .. LDARG_5
+                pc++;
+                index = (uint16_t)(opc - 40);
+            } else
+                break;
+            n_ldarg++;
+            if (index != loc.fh.parameters - n_ldarg) { ok = false; break; }
+        }
+        uint8_t opc = 0;
+        int32_t func_id = -1, module_id = -1;
+        uint16_t call_args = 0;
+        uint8_t is_prim = 0;
+        ok = ok && n_ldarg == loc.fh.parameters && rd(&opc, 1) && opc == 2 && rd(&func_id, 4) && rd(&opc, 1) && opc == 2 &&
+             rd(&module_id, 4) && rd(&opc, 1) && opc == 96 && rd(&call_args, 2) && rd(&is_prim, 1) && rd(&opc, 1) && opc == 93 &&
+             pc == sv.n && call_args == n_ldarg && is_prim <= 1 && func_id >= 0 && module_id >= 0;
+        NNHIP_REQUIRE(ctx, ok, -NNCASE_HIP_ERR_RUNTIME_NOT_FOUND,
+                      "kmodel_load: the stackvm entry function is not a plain call into another module (this library runs "
+                      "hip functions, not stackvm code)");
+        NNHIP_REQUIRE(ctx, (uint32_t)module_id != mh.entry_module, -NNCASE_HIP_ERR_RUNTIME_NOT_FOUND,
+                      "kmodel_load: the stackvm entry function calls its own module");
+        const uint32_t caller_args = n_ldarg;
+        lrc = locate((uint32_t)module_id, (uint32_t)func_id, &loc);
+        if (lrc) return lrc;
+        // a prim function receives its outputs as trailing parameters (control.cpp:49-68)
+        NNHIP_REQUIRE(ctx, is_prim ? loc.fh.parameters > caller_args : loc.fh.parameters == caller_args, -EINVAL,
+                      "kmodel_load: EXTCALL passes %u arguments to a function of %u parameters", caller_args, loc.fh.parameters);
     }
-    NNHIP_REQUIRE(ctx, strncmp(modh.kind, "hip", 16) == 0, -NNCASE_HIP_ERR_RUNTIME_NOT_FOUND,
-                  "kmodel_load: entry module kind \"%.16s\" is not \"hip\"", modh.kind);
-    NNHIP_REQUIRE(ctx, mh.entry_function < modh.functions, -EINVAL, "kmodel_load: entry function index out of range");
-    const size_t module_end = pos + (size_t)modh.size;
-    size_t fpos = pos + sizeof(module_header);
-    function_header fh{};
-    for (uint32_t i = 0; i < modh.functions; i++) { // skip_functions, runtime_module.cpp:112-117
-        NNHIP_REQUIRE(ctx, fpos + sizeof(function_header) <= module_end, -EINVAL, "kmodel_load: truncated function header");
-        function_header h;
-        memcpy(&h, file + fpos, sizeof(h));
-        NNHIP_REQUIRE(ctx, h.size >= sizeof(h) && h.size <= module_end - fpos, -EINVAL, "kmodel_load: bad function size");
-        if (i == mh.entry_function) fh = h;
-        fpos += (size_t)h.size;
-    }
-    Span text_all, rdata;
-    NNHIP_REQUIRE(ctx, find_section(file, size, fpos, modh.sections, ".text", &text_all), -EINVAL,
-                  "kmodel_load: hip module has no .text section");
-    if (!find_section(file, size, fpos, modh.sections, ".rdata", &rdata)) rdata = Span{};
-    NNHIP_REQUIRE(ctx, fh.entrypoint <= text_all.n && fh.text_size <= text_all.n - fh.entrypoint, -EINVAL,
-                  "kmodel_load: function text outside the .text section");
-    const uint8_t *text = text_all.p + fh.entrypoint;
-    const size_t text_size = (size_t)fh.text_size;
+    NNHIP_REQUIRE(ctx, strncmp(loc.modh.kind, "hip", 16) == 0, -NNCASE_HIP_ERR_RUNTIME_NOT_FOUND,
+                  "kmodel_load: module kind \"%.16s\" is not \"hip\"", loc.modh.kind);
+    lrc = function_text(loc, &text_span, &rdata);
+    if (lrc) return lrc;
+    const uint8_t *text = text_span.p;
+    const size_t text_size = text_span.n;
 
     // ---- function text --------------------------------------------------------------------------
     NNHIP_REQUIRE(ctx, text_size >= sizeof(hipf_header), -EINVAL, "kmodel_load: function text too short");

@@ -15,8 +15,12 @@ reader src/Native/src/runtime/interpreter.cpp:40-91, runtime_module.cpp:124-180)
       module sections
     section_header 56 B  {char name[16]; u32 flags, reserved0; u64 size, body_start, body_size, memory_size}
 
-Every `size` includes its own header and the padding to 8 bytes that follows the body; `body_start`
-is the absolute stream position of the body after aligning to the section's alignment.
+Every `size` includes its own header and the padding to 8 bytes that follows the body.  `body_start`
+is the number of padding bytes between the end of the section header and the body (the writer stores
+what AlignPosition returns, LinkedModel.cs:160 / CodeGenExtensions.cs:20-35; the reader adds it to the
+position behind the header, src/Native/src/runtime/section.cpp:35-36,77-78).  A section whose flags
+carry SECTION_MERGED_INTO_RDATA (1) has no body of its own: body_start is then an offset into the
+body of the `.rdata` section of the same section list (section.cpp:29-32,71-76).
 
 The `hip` module (kind "hip", version 1) holds one function whose `.text` is a flat operator list over
 numbered NHWC tensors (HIPF format below) and a module section `.rdata` with the constants (u8 OIHW
@@ -42,6 +46,7 @@ MODEL_IDENTIFIER = 0x4B4D444C      # 'KMDL' as a C++ multi-character constant ->
 MODEL_VERSION = 7
 MODEL_HAS_NO_ENTRY = 0xFFFFFFFF
 MIN_ALIGNMENT = 8
+SECTION_MERGED_INTO_RDATA = 1      # model.h:76
 
 MODEL_HEADER = struct.Struct("<8I")
 MODULE_HEADER = struct.Struct("<16s4IQ")
@@ -120,7 +125,8 @@ class Section:
     flags: int = 0
     alignment: int = 8
     memory_size: Optional[int] = None
-    body_start: int = 0          # filled by the reader / writer
+    body_start: int = 0          # header field, filled by the reader / writer: padding before the body
+    body_pos: int = 0            # absolute position of the body in the file, filled by the reader / writer
 
 
 @dataclass
@@ -168,9 +174,12 @@ class KModel:
             return b.ljust(16, b"\0")
 
         def write_section(s: Section):
+            if s.flags & SECTION_MERGED_INTO_RDATA:
+                raise ValueError("this writer keeps every section's body in the section itself")
             head = len(out)
             out.extend(b"\0" * SECTION_HEADER.size)
-            s.body_start = align(s.alignment)
+            s.body_pos = align(s.alignment)
+            s.body_start = s.body_pos - (head + SECTION_HEADER.size)
             out.extend(s.body)
             end = align(MIN_ALIGNMENT)
             mem = len(s.body) if s.memory_size is None else s.memory_size
@@ -210,10 +219,29 @@ class KModel:
         if version != MODEL_VERSION:
             raise ValueError(f"invalid model version {version}")  # nncase_errc::invalid_model_version
 
-        def read_section(pos: int):
-            name, flags, _r, size, body_start, body_size, memory_size = SECTION_HEADER.unpack_from(buf, pos)
-            s = Section(name.rstrip(b"\0").decode(), bytes(buf[body_start:body_start + body_size]), flags, 8, memory_size, body_start)
-            return s, pos + size
+        def read_sections(pos: int, count: int):
+            """`count` section records from `pos`: bodies located like runtime::find_section (section.cpp:58-91)."""
+            heads = []
+            for _ in range(count):
+                name, flags, _r, size, body_start, body_size, memory_size = SECTION_HEADER.unpack_from(buf, pos)
+                if size < SECTION_HEADER.size or pos + size > len(buf):
+                    raise ValueError("bad section size")
+                heads.append((name.rstrip(b"\0").decode(), flags, pos, body_start, body_size, memory_size))
+                pos += size
+            rdata_pos = next((hp + SECTION_HEADER.size + bs for n, f, hp, bs, _z, _m in heads
+                              if n == ".rdata" and not f & SECTION_MERGED_INTO_RDATA), None)
+            out = []
+            for name, flags, hp, body_start, body_size, memory_size in heads:
+                if flags & SECTION_MERGED_INTO_RDATA:
+                    if rdata_pos is None:
+                        raise ValueError(f"section {name} is merged into a .rdata section that does not exist")
+                    body_pos = rdata_pos + body_start
+                else:
+                    body_pos = hp + SECTION_HEADER.size + body_start
+                if body_pos + body_size > len(buf):
+                    raise ValueError(f"section {name} body outside the file")
+                out.append(Section(name, bytes(buf[body_pos:body_pos + body_size]), flags, 8, memory_size, body_start, body_pos))
+            return out, pos
 
         modules = []
         pos = MODEL_HEADER.size
@@ -230,14 +258,10 @@ class KModel:
                     params.append(t)
                 ret, q = decode_type(buf, q)
                 fn = Function(params, ret, entrypoint, text_size)
-                for _s in range(n_fsec):
-                    s, q = read_section(q)
-                    fn.sections.append(s)
+                fn.sections, q = read_sections(q, n_fsec)
                 m.functions.append(fn)
                 p += fsize
-            for _s in range(n_sections):
-                s, p = read_section(p)
-                m.sections.append(s)
+            m.sections, p = read_sections(p, n_sections)
             modules.append(m)
             pos += msize
         return KModel(modules, entry_module, entry_function, alignment)
@@ -323,9 +347,45 @@ def decode_hip_text(text: bytes):
     return tensors, ops, input_tensor, output_tensor
 
 
-def compile_quant_graph(qg, batch: int) -> bytes:
-    """Emits a one-module kmodel (kind "hip") for a netbuilder.QuantGraph at a fixed batch:
-    f32 NHWC input -> quantize -> the graph's u8 operators -> dequantize -> f32 output."""
+# ------------------------------------------------------------------------------------------------ stackvm entry stub
+STACKVM_MODULE_KIND = "stackvm"
+STACKVM_MODULE_VERSION = 1          # modules/Nncase.Modules.StackVM/Runtime/StackVM/StackVMRTModule.cs
+# src/Native/include/nncase/runtime/stackvm/opcode.h:26-127
+OPC_LDC_I4, OPC_LDARG, OPC_RET, OPC_EXTCALL = 2, 39, 93, 96
+
+
+def stackvm_extcall_text(n_args: int, function_id: int, module_id: int, is_prim_func: bool = False) -> bytes:
+    """The stackvm text the compiler emits for `main(args) = callee(args)` with the callee in another module
+    (modules/Nncase.Modules.StackVM/CodeGen/StackVM/CodegenVisitor.cs:281-315: arguments visited in reverse,
+    then LdFunctionId :470-476 = LDC_I4 function id, LDC_I4 module id, then EXTCALL, and RET :244).
+    Encodings (op_reader.h): opcode u8; LDARG u16 index; LDC_I4 i32; EXTCALL u16 args + u8 is_prim_func."""
+    out = bytearray()
+    for i in reversed(range(n_args)):
+        out += struct.pack("<BH", OPC_LDARG, i)
+    out += struct.pack("<Bi", OPC_LDC_I4, function_id)
+    out += struct.pack("<Bi", OPC_LDC_I4, module_id)
+    out += struct.pack("<BHB", OPC_EXTCALL, n_args, 1 if is_prim_func else 0)
+    out += struct.pack("<B", OPC_RET)
+    return bytes(out)
+
+
+def with_stackvm_main(callee: Module, function_index: int = 0) -> "KModel":
+    """A two-module kmodel as the compiler links it: module 0 = `stackvm` whose only function calls function
+    `function_index` of module 1 = `callee` through EXTCALL; the model's entry is the stackvm function.
+    `.custom_calls` holds a zero count (u32 count + count x char[16], StackVMLinkableModule.cs ctor; reader
+    src/Native/src/runtime/stackvm/runtime_module.cpp:35-54)."""
+    f = callee.functions[function_index]
+    text = stackvm_extcall_text(len(f.parameter_types), function_index, 1)
+    main = Function(list(f.parameter_types), f.return_type, 0, len(text))
+    vm = Module(STACKVM_MODULE_KIND, STACKVM_MODULE_VERSION, [main],
+                [Section(".text", text), Section(".rdata", b""), Section(".custom_calls", struct.pack("<I", 0))])
+    return KModel([vm, callee], entry_module=0, entry_function=0)
+
+
+def compile_quant_graph(qg, batch: int, stackvm_main: bool = False) -> bytes:
+    """Emits a kmodel for a netbuilder.QuantGraph at a fixed batch: f32 NHWC input -> quantize -> the graph's
+    u8 operators -> dequantize -> f32 output, as one function of a module of kind "hip".  With stackvm_main the
+    file has the shape the compiler links: its entry is a `stackvm` function that EXTCALLs the hip function."""
     rdata = RData()
     tensors: List[HipTensor] = []
     ops: List[HipOp] = []
@@ -377,4 +437,6 @@ def compile_quant_graph(qg, batch: int) -> bytes:
     fn = Function([TensorType("f32", tensors[0].dims)], ret, 0, len(text))
     mod = Module(HIP_MODULE_KIND, HIP_MODULE_VERSION, [fn],
                  [Section(".text", text), Section(".rdata", bytes(rdata.buf), alignment=64)])
+    if stackvm_main:
+        return with_stackvm_main(mod).serialize()
     return KModel([mod], entry_module=0, entry_function=0).serialize()

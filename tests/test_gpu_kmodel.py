@@ -17,8 +17,8 @@ f32 = np.float32
 GOLD = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_vectors.json")))
 
 
-def run_and_check(hip_ctx, qg, x):
-    data = km.compile_quant_graph(qg, x.shape[0])
+def run_and_check(hip_ctx, qg, x, stackvm_main=False):
+    data = km.compile_quant_graph(qg, x.shape[0], stackvm_main=stackvm_main)
     model = rt.LoadedKModel(hip_ctx, data)
     assert model.input_shape == x.shape and model.input_dtype == np.float32
     y = model.run(x)
@@ -101,3 +101,62 @@ def test_malformed_files_are_refused(hip_ctx):
     mm.modules[0].sections[0].body = km.encode_hip_text(tensors, unknown, tin, tout)
     assert code(mm.serialize()) == -rt.ERR_RUNTIME_NOT_FOUND
     rt.LoadedKModel(hip_ctx, good).destroy()                          # and the untouched file still loads
+
+
+def test_stackvm_entry_that_extcalls_the_hip_function(hip_ctx):
+    """The file form the compiler links -- module 0 `stackvm` whose main is LDARG 0; LDC_I4 function; LDC_I4 module;
+    EXTCALL; RET, module 1 `hip` -- loads and gives the oracle's bytes like the single-module form; any other
+    stackvm text is refused with runtime_not_found (there is no stackvm interpreter here)."""
+    rng = np.random.default_rng(1)
+    qg = nb.quantize_graph(nb.conv_block(seed=1), rng.random((8, 56, 56, 64), dtype=f32))
+    x = rng.random((2, 56, 56, 64), dtype=f32)
+    _, y_single, _ = run_and_check(hip_ctx, qg, x)
+    _, y_two, _ = run_and_check(hip_ctx, qg, x, stackvm_main=True)
+    assert np.array_equal(y_single.view(np.uint32), y_two.view(np.uint32))
+
+    good = km.compile_quant_graph(qg, 2, stackvm_main=True)
+
+    def code(model):
+        with pytest.raises(rt.HipError) as e:
+            rt.LoadedKModel(hip_ctx, model.serialize())
+        return e.value.code
+
+    def with_text(text):
+        m = km.KModel.parse(good)
+        m.modules[0].sections[0].body = text
+        m.modules[0].functions[0].text_size = len(text)
+        return m
+
+    stub = km.stackvm_extcall_text(1, 0, 1)
+    short_form = bytes([40]) + stub[3:]                                  # LDARG_0 instead of LDARG 0
+    rt.LoadedKModel(hip_ctx, with_text(short_form).serialize()).destroy()
+    assert code(with_text(stub[:-1])) == -rt.ERR_RUNTIME_NOT_FOUND        # no RET
+    assert code(with_text(stub + bytes([93]))) == -rt.ERR_RUNTIME_NOT_FOUND
+    assert code(with_text(bytes([1]) + stub)) == -rt.ERR_RUNTIME_NOT_FOUND   # LDNULL first: real stackvm code
+    assert code(with_text(km.stackvm_extcall_text(1, 0, 0))) == -rt.ERR_RUNTIME_NOT_FOUND   # calls itself
+    assert code(with_text(km.stackvm_extcall_text(1, 0, 7))) == -rt.ERR_RUNTIME_NOT_FOUND   # no such module
+    import errno
+    assert code(with_text(km.stackvm_extcall_text(1, 5, 1))) == -errno.EINVAL               # no such function
+    assert code(with_text(km.stackvm_extcall_text(2, 0, 1))) == -rt.ERR_RUNTIME_NOT_FOUND   # main has one parameter
+
+
+def test_sections_merged_into_rdata_are_resolved(hip_ctx):
+    """A section flagged SECTION_MERGED_INTO_RDATA keeps its bytes inside .rdata (section.cpp:29-32): a hip module
+    whose .text lives there loads to the same function."""
+    rng = np.random.default_rng(1)
+    qg = nb.quantize_graph(nb.conv_block(seed=1), rng.random((8, 56, 56, 64), dtype=f32))
+    x = rng.random((1, 56, 56, 64), dtype=f32)
+    plain = km.compile_quant_graph(qg, 1)
+    want = rt.LoadedKModel(hip_ctx, plain).run(x)
+    m = km.KModel.parse(plain)
+    text, rdata = m.modules[0].section(".text").body, m.modules[0].section(".rdata").body
+    pad = (-len(rdata)) % 64
+    m.modules[0].sections[1].body = rdata + b"\0" * pad + text         # constants keep their offsets
+    m.modules[0].sections[0].body = b""
+    data = bytearray(m.serialize())
+    pos = km.MODEL_HEADER.size + km.MODULE_HEADER.size + km.FUNCTION_HEADER.unpack_from(data, km.MODEL_HEADER.size + km.MODULE_HEADER.size)[-1]
+    name, _flags, r0, size, _bs, _bz, mem = km.SECTION_HEADER.unpack_from(data, pos)
+    assert name.rstrip(b"\0") == b".text"
+    km.SECTION_HEADER.pack_into(data, pos, name, km.SECTION_MERGED_INTO_RDATA, r0, size, len(rdata) + pad, len(text), mem)
+    got = rt.LoadedKModel(hip_ctx, bytes(data)).run(x)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))

@@ -53,7 +53,7 @@ def test_container_round_trip_and_size_fields():
     m0 = km.Module("stackvm", 1, [f0, f1], [km.Section(".text", blob(20)), km.Section(".rdata", blob(1000), alignment=128),
                                             km.Section(".custom_calls", struct.pack("<I16s", 1, b"hip"))])
     m1 = km.Module("hip", 1, [km.Function([km.TensorType("u8", (4,))], km.TensorType("u8", (4,)), 0, 9)],
-                   [km.Section(".text", blob(9)), km.Section(".rdata", blob(77), flags=1, alignment=64, memory_size=4096)])
+                   [km.Section(".text", blob(9)), km.Section(".rdata", blob(77), flags=2, alignment=64, memory_size=4096)])
     data = km.KModel([m0, m1], entry_module=0, entry_function=1).serialize()
     assert len(data) % 8 == 0
     ident, ver, flags, align, nmod, em, ef, _ = km.MODEL_HEADER.unpack_from(data, 0)
@@ -74,7 +74,8 @@ def test_container_round_trip_and_size_fields():
             assert [(s.name, s.body) for s in fa.sections] == [(s.name, s.body) for s in fb.sections]
         for sa, sb in zip(a.sections, b.sections):
             assert (sa.name, sa.body, sa.flags) == (sb.name, sb.body, sb.flags)
-            assert sa.body_start % sb.alignment == 0                # bodies start on their alignment
+            assert sa.body_pos % sb.alignment == 0                  # bodies start on their alignment
+            assert 0 <= sa.body_start < sb.alignment                # the header field holds the padding, not a position
             assert sa.memory_size == (len(sb.body) if sb.memory_size is None else sb.memory_size)
     assert back.serialize() != b"" and km.KModel.parse(back.serialize()).modules[1].section(".rdata").body == m1.sections[1].body
 
@@ -105,3 +106,60 @@ def test_hip_module_of_a_quantised_graph():
         assert (tensors[o.output].zero_point, np.float32(tensors[o.output].scale)) == (n.out_qp[0], np.float32(n.out_qp[1]))
     # a text survives its own round trip
     assert km.encode_hip_text(tensors, ops, tin, tout) == text
+
+
+def _walk_like_the_reference(data, pos, count, name):
+    """runtime::find_section over a stream (src/Native/src/runtime/section.cpp:58-91), loop for loop:
+    returns the absolute body position and size of section `name` among `count` records at `pos`."""
+    sections_pos = pos
+    for _ in range(count):
+        here = pos
+        sname, flags, _r, size, body_start, body_size, _mem = km.SECTION_HEADER.unpack_from(data, pos)
+        if sname.rstrip(b"\0") == name.encode():
+            if flags & 1:                                   # SECTION_MERGED_INTO_RDATA
+                rdata_pos, _ = _walk_like_the_reference(data, sections_pos, count, ".rdata")
+                return rdata_pos + body_start, body_size
+            return here + km.SECTION_HEADER.size + body_start, body_size
+        pos = here + size                                   # reader.skip(header.size - sizeof(header)) after the header
+    raise KeyError(name)
+
+
+def test_section_bodies_are_where_the_reference_reader_looks():
+    rng = np.random.default_rng(8)
+    text, rdata, calls = rng.bytes(21), rng.bytes(333), struct.pack("<I", 0)
+    m = km.Module("hip", 1, [], [km.Section(".text", text), km.Section(".rdata", rdata, alignment=64),
+                                 km.Section(".custom_calls", calls, alignment=16)])
+    data = km.KModel([m]).serialize()
+    first = km.MODEL_HEADER.size + km.MODULE_HEADER.size
+    for name, body in ((".text", text), (".rdata", rdata), (".custom_calls", calls)):
+        pos, n = _walk_like_the_reference(data, first, 3, name)
+        assert data[pos:pos + n] == body
+    # a file in which a section lives inside .rdata (flags & 1): body_start is an offset into .rdata's body
+    head = bytearray(data)
+    # rewrite the .custom_calls record by hand: merged, at offset 40 of .rdata, 12 bytes
+    p = first
+    for _ in range(2):
+        p += km.SECTION_HEADER.unpack_from(head, p)[3]
+    name, _flags, r0, size, _bs, _bz, mem = km.SECTION_HEADER.unpack_from(head, p)
+    km.SECTION_HEADER.pack_into(head, p, name, 1, r0, size, 40, 12, mem)
+    pos, n = _walk_like_the_reference(bytes(head), first, 3, ".custom_calls")
+    assert bytes(head[pos:pos + n]) == rdata[40:52]
+    assert km.KModel.parse(bytes(head)).modules[0].section(".custom_calls").body == rdata[40:52]
+
+
+def test_stackvm_entry_stub_bytes():
+    # opcode bytes of opcode.h:26-127 and operand widths of op_reader.h: LDARG u16; LDC_I4 i32; EXTCALL u16 + bool
+    assert km.stackvm_extcall_text(1, 0, 1) == bytes([39, 0, 0, 2, 0, 0, 0, 0, 2, 1, 0, 0, 0, 96, 1, 0, 0, 93])
+    assert km.stackvm_extcall_text(2, 3, 1, True) == bytes([39, 1, 0, 39, 0, 0, 2, 3, 0, 0, 0, 2, 1, 0, 0, 0, 96, 2, 0, 1, 93])
+    g = nb.conv_block(seed=1)
+    qg = nb.quantize_graph(g, np.random.default_rng(1).random((2, 56, 56, 64), dtype=np.float32))
+    model = km.KModel.parse(km.compile_quant_graph(qg, batch=1, stackvm_main=True))
+    assert [m.kind for m in model.modules] == ["stackvm", "hip"] and (model.entry_module, model.entry_function) == (0, 0)
+    main, callee = model.modules[0].functions[0], model.modules[1].functions[0]
+    assert main.parameter_types == callee.parameter_types and main.return_type == callee.return_type
+    assert model.modules[0].section(".text").body[main.entrypoint:main.entrypoint + main.text_size] == km.stackvm_extcall_text(1, 0, 1)
+    assert model.modules[0].section(".custom_calls").body == struct.pack("<I", 0)
+    # the hip module is byte for byte the one of the single-module file
+    single = km.KModel.parse(km.compile_quant_graph(qg, batch=1))
+    assert model.modules[1].section(".text").body == single.modules[0].section(".text").body
+    assert model.modules[1].section(".rdata").body == single.modules[0].section(".rdata").body
