@@ -392,6 +392,20 @@ NNCASE_HIP_API int nncase_hip_paged_attention_decode(nncase_hip_ctx_t *ctx, cons
                                                      const int32_t *ctx_lens_dev, void *out_dev,
                                                      const nncase_hip_paged_attn_args_t *args);
 
+/* The same operator for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  The split
+ * partials and completion counters that nncase_hip_paged_attention_decode keeps in a workspace owned by the
+ * context live here in a static device array of the library (8 MiB of partials + 64 KiB of counters per GPU,
+ * held until the process ends); the call allocates and frees nothing and issues no memset.  Geometries whose
+ * partials (batch * num_q_heads * splits * (head_dim + 2) floats, splits = context capacity / tokens per
+ * split) or counters (batch * num_kv_heads words) exceed that are refused with -E2BIG.  All calls on one GPU
+ * share the array: calls that overlap in time on one GPU (two contexts, two streams) race; calls on one
+ * context are ordered by its stream.  Results are bit-identical to nncase_hip_paged_attention_decode. */
+NNCASE_HIP_API int nncase_hip_paged_attention_decode_noalloc(nncase_hip_ctx_t *ctx, const void *q_dev, const void *k_cache_dev,
+                                                             const void *v_cache_dev, const int32_t *block_table_dev,
+                                                             const int32_t *ctx_lens_dev, void *out_dev,
+                                                             const nncase_hip_paged_attn_args_t *args);
+
 /* ---- the rest of an LLM decode step (fp16 activations, W8A16 weights) --------
  * No counterpart in this reference tree (its LLM path lives in another branch); the
  * arithmetic is defined here and checked against float64 restatements.

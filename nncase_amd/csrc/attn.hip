@@ -316,6 +316,15 @@ __global__ void attn_zero_u32_kernel(uint32_t *p, size_t count) {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x) p[i] = 0u;
 }
 
+// ---- static device scratch of the entry point that allocates nothing -------------------------
+// One copy per GPU, held until the process ends: completion counters first, split partials after.
+constexpr size_t kScratchCounterBytes = 64u << 10;  // 16384 (sequence, kv head) pairs
+constexpr size_t kScratchPartialBytes = 8u << 20;   // batch * query heads * splits * (head_dim + 2) floats
+static __device__ __align__(256) unsigned char scratch[kScratchCounterBytes + kScratchPartialBytes];
+
+constexpr int kMaxDevices = 64;
+static void *g_scratch_ptr[kMaxDevices] = {nullptr}; // device address of `scratch` on each GPU (hipGetSymbolAddress)
+
 // Everything a launch needs except the buffers: checked geometry, split plan, sizes of the scratch areas.
 struct AttnPlan {
     AttnArgs a;
@@ -461,4 +470,35 @@ extern "C" int nncase_hip_paged_attention_decode(nncase_hip_ctx_t *ctx, const vo
     }
     return attn_launch(ctx, plan, q_dev, k_cache_dev, v_cache_dev, block_table_dev, ctx_lens_dev, out_dev, ctx->attn_ws,
                        ctx->attn_done);
+}
+
+extern "C" int nncase_hip_paged_attention_decode_noalloc(nncase_hip_ctx_t *ctx, const void *q_dev, const void *k_cache_dev,
+                                                         const void *v_cache_dev, const int32_t *block_table_dev,
+                                                         const int32_t *ctx_lens_dev, void *out_dev,
+                                                         const nncase_hip_paged_attn_args_t *p) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, q_dev && k_cache_dev && v_cache_dev && block_table_dev && ctx_lens_dev && out_dev && p, -EINVAL,
+                  "paged_attention_decode_noalloc: null argument");
+    AttnPlan plan;
+    const int rc = attn_plan(ctx, p, &plan);
+    if (rc) return rc;
+    NNHIP_REQUIRE(ctx, plan.partial_bytes <= kScratchPartialBytes && plan.counter_bytes <= kScratchCounterBytes, -E2BIG,
+                  "paged_attention_decode_noalloc: needs %zu bytes of split partials and %zu of counters; the static "
+                  "scratch holds %zu and %zu (use nncase_hip_paged_attention_decode)",
+                  plan.partial_bytes, plan.counter_bytes, kScratchPartialBytes, kScratchCounterBytes);
+    NNHIP_REQUIRE(ctx, ctx->device >= 0 && ctx->device < kMaxDevices, -ENODEV, "paged_attention_decode_noalloc: device %d",
+                  ctx->device);
+    if (!g_scratch_ptr[ctx->device]) { // first call on this GPU: every GPU has its own copy at its own address
+        NNHIP_HIP(ctx, hipSetDevice(ctx->device));
+        void *ptr = nullptr;
+        NNHIP_HIP(ctx, hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        NNHIP_REQUIRE(ctx, ptr, -ENOMEM, "paged_attention_decode_noalloc: no address for the static scratch");
+        g_scratch_ptr[ctx->device] = ptr;
+    }
+    unsigned char *base = reinterpret_cast<unsigned char *>(g_scratch_ptr[ctx->device]);
+    // The array keeps the previous call's contents: the counters this launch uses must start at zero.
+    hipLaunchKernelGGL(attn_zero_u32_kernel, dim3(1), dim3(256), 0, ctx->stream, (uint32_t *)base, plan.counter_bytes / 4);
+    NNHIP_LAUNCH_CHECK(ctx, "attn_zero_u32_kernel");
+    return attn_launch(ctx, plan, q_dev, k_cache_dev, v_cache_dev, block_table_dev, ctx_lens_dev, out_dev,
+                       base + kScratchCounterBytes, base);
 }

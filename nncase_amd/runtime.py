@@ -153,6 +153,7 @@ SYMBOLS = {
     "nncase_hip_nchw_to_nhwc": (_I, [_VP, _VP, _VP, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
     "nncase_hip_nhwc_to_nchw": (_I, [_VP, _VP, _VP, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
     "nncase_hip_paged_attention_decode": (_I, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, C.POINTER(PagedAttnArgs)]),
+    "nncase_hip_paged_attention_decode_noalloc": (_I, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, C.POINTER(PagedAttnArgs)]),
     "nncase_hip_function_create": (_I, [_VP, C.POINTER(_VP)]),
     "nncase_hip_function_destroy": (_I, [_VP]),
     "nncase_hip_function_add_quantize": (_I, [_VP, _VP, _I, _VP, _I, _SZ, QuantParam]),
@@ -562,6 +563,13 @@ class Context:
                                block_table: DeviceBuffer, ctx_lens: DeviceBuffer, out: DeviceBuffer, args: PagedAttnArgs):
         self._check(self.lib.nncase_hip_paged_attention_decode(self.handle, q.ptr, k_cache.ptr, v_cache.ptr, block_table.ptr,
                                                                ctx_lens.ptr, out.ptr, C.byref(args)), "paged_attention_decode")
+
+    def paged_attention_decode_noalloc(self, q: DeviceBuffer, k_cache: DeviceBuffer, v_cache: DeviceBuffer,
+                                       block_table: DeviceBuffer, ctx_lens: DeviceBuffer, out: DeviceBuffer, args: PagedAttnArgs):
+        """The same operator on the library's static device scratch: allocates nothing (-E2BIG beyond its size)."""
+        self._check(self.lib.nncase_hip_paged_attention_decode_noalloc(self.handle, q.ptr, k_cache.ptr, v_cache.ptr,
+                                                                       block_table.ptr, ctx_lens.ptr, out.ptr, C.byref(args)),
+                    "paged_attention_decode_noalloc")
 
 
 class Function:
