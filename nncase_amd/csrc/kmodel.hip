@@ -306,8 +306,16 @@ extern "C" int nncase_hip_kmodel_load(nncase_hip_ctx_t *ctx, const void *data, s
         const hipf_tensor &x = m->tensors[t];
         NNHIP_REQUIRE(ctx, x.rank == 4 && dtype_size(x.dtype) != 0, -NNCASE_HIP_ERR_DATATYPE_MISMATCH,
                       "kmodel_load: tensor %u has rank %u / dtype 0x%x", t, x.rank, x.dtype);
-        NNHIP_REQUIRE(ctx, x.dims[0] && x.dims[1] && x.dims[2] && x.dims[3] && elems(t) < (size_t(1) << 40), -EINVAL,
-                      "kmodel_load: tensor %u has an empty or implausible shape", t);
+        // four 32-bit extents can wrap a 64-bit product: bound every extent and every partial product
+        // (2^24 * 2^40 < 2^64, so the running product cannot wrap before it is checked)
+        bool sane = true;
+        uint64_t prod = 1;
+        for (int d = 0; d < 4 && sane; d++) {
+            sane = x.dims[d] != 0 && x.dims[d] <= (1u << 24);
+            prod *= x.dims[d];
+            sane = sane && prod < (uint64_t(1) << 40);
+        }
+        NNHIP_REQUIRE(ctx, sane, -EINVAL, "kmodel_load: tensor %u has an empty or implausible shape", t);
     }
 
     // ---- which adds fold into the dense conv right before them -------------------------------

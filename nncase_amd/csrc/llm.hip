@@ -332,7 +332,7 @@ __global__ __launch_bounds__(kLlmThreads) void rope_append_kernel(const RopeArgs
     const float x0 = __half2float(src[i]), x1 = __half2float(src[i + half]);
     const int pos = a.ctx_lens[b];
     const int lb = pos / a.block_size, in_block = pos - lb * a.block_size;
-    const bool fits = lb < a.max_blocks;
+    const bool fits = pos >= 0 && lb < a.max_blocks; // a negative length appends nothing (it would index before the block)
     const int pb = fits ? min(max(a.block_table[(size_t)b * a.max_blocks + lb], 0), a.num_blocks - 1) : 0;
     if (h < a.hq + a.hkv) {
         const float inv = powf(a.theta, -2.0f * (float)i / (float)a.d);

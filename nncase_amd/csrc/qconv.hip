@@ -153,6 +153,8 @@ int nnhip::make_epilogue(nncase_hip_ctx *ctx, Epilogue *ep, float sx, float sw, 
     ep->out_mode = out_dtype == NNCASE_HIP_DT_U8 ? kOutU8 : (out_dtype == NNCASE_HIP_DT_I32 ? kOutI32 : kOutF32);
     NNHIP_REQUIRE(ctx, !(clamp_min > clamp_max), -EINVAL, "%s: fused clamp minimum above maximum", who);
     if (ep->out_mode != kOutU8) return 0;
+    NNHIP_REQUIRE(ctx, y_qp.zero_point >= 0 && y_qp.zero_point <= 255, -EINVAL, "%s: output zero point %d outside u8", who,
+                  y_qp.zero_point);
     // Range in which q0 = f * rsy and the residual f - sy * q0 stay normal for every f whose
     // requantised value is not already pinned to an end of [0, 255].
     NNHIP_REQUIRE(ctx, ep->sy >= 0x1p-64f && ep->sy <= 0x1p64f, -ERANGE, "%s: output scale %g outside [2^-64, 2^64]", who,

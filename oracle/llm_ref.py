@@ -1,6 +1,11 @@
 """float64 restatement of the decode-step operators and of the whole decode step.
 TEST INFRASTRUCTURE ONLY.  No counterpart in the reference tree (parity unpinned by the reference):
-each function is the textbook definition, checked in tests/test_oracle.py against closed forms."""
+each function is the textbook definition; tests/test_llm_ref.py pins them against closed forms and
+invariants that a swapped operand, a wrong pairing or a misplaced epsilon would break (rotary embedding:
+identity at position 0, norms kept, inner products that depend on the position difference only, the
+(i, i + d/2) pairing on one-hot vectors; RMS norm: constant rows, scale invariance, epsilon under the
+root; SwiGLU: gate / up order; the W8A16 product on small integers; one decode step of a one-layer model
+against a hand calculation)."""
 from __future__ import annotations
 
 import numpy as np

@@ -361,13 +361,23 @@ def unpack(y: np.ndarray, axes, lanes, orig_shape) -> np.ndarray:
     return np.ascontiguousarray(z[tuple(slice(0, s) for s in orig_shape)])
 
 
-def cosine(a, b) -> float:
-    """tests/compare_util.py:27-54 style cosine similarity on flattened float64 data."""
-    a = np.asarray(a, np.float64).ravel()
-    b = np.asarray(b, np.float64).ravel()
-    if np.array_equal(a, b):
+def cosine(gt, pred) -> float:
+    """Cosine similarity as the reference's test harness computes it (tests/compare_util.py:27-54):
+    NaN at the same position of both arrays is dropped, likewise Inf; any non-finite value left over on
+    either side gives -1 (so a NaN produced where the expectation is finite fails every threshold);
+    identical arrays give 1 (covers all-zero data); a NaN quotient gives -1."""
+    gt = np.asarray(gt, np.float64).ravel()
+    pred = np.asarray(pred, np.float64).ravel()
+    if np.isnan(gt).any() and np.isnan(pred).any():
+        keep = ~(np.isnan(gt) & np.isnan(pred))
+        gt, pred = gt[keep], pred[keep]
+    if np.isinf(gt).any() and np.isinf(pred).any():
+        keep = ~(np.isinf(gt) & np.isinf(pred))
+        gt, pred = gt[keep], pred[keep]
+    if not (np.isfinite(gt).all() and np.isfinite(pred).all()):
+        return -1.0
+    if np.array_equal(gt, pred):
         return 1.0
-    mask = np.isfinite(a) & np.isfinite(b)
-    a, b = a[mask], b[mask]
-    den = np.linalg.norm(a) * np.linalg.norm(b)
-    return float(a @ b / den) if den else 0.0
+    with np.errstate(invalid="ignore", divide="ignore"):
+        r = (gt @ pred) / (np.linalg.norm(gt, 2) * np.linalg.norm(pred, 2))
+    return -1.0 if np.isnan(r) else float(r)

@@ -114,7 +114,14 @@ def test_conv2d_kernel_grid(hip_ctx, case):
 # ---- shapes of the benchmark configurations ------------------------------------------------------
 # every distinct (Cin, Cout) pointwise layer of MobileNetV2 on a small image, plus stem / depthwise / FC shapes
 MBV2_PW = [(32, 16), (16, 96), (96, 24), (24, 144), (144, 24), (144, 32), (32, 192), (192, 32), (192, 64), (64, 384),
-           (384, 64), (384, 96), (96, 576), (576, 96), (576, 160), (160, 960), (960, 160), (960, 320), (320, 1280)]
+           (384, 64), (384, 96), (96, 576), (576, 96), (576, 160), (160, 960), (960, 160), (960, 320), (320, 1280),
+           (64, 144), (144, 64)]   # the last two: the conv block of BASELINE config 2
+
+
+@pytest.mark.parametrize("cin,cout", [(64, 144), (144, 64)])
+def test_conv_block_pointwise_layers_at_batch_32(hip_ctx, cin, cout):
+    # config 2's two pointwise layers at their full launch size: M = 32 * 56 * 56 = 100 352 pixels
+    run_case(hip_ctx, 32, cin, 56, 56, cout, 1, 1, (1, 1), ((0, 0), (0, 0)), (1, 1), 1, seed=cin + cout, modes=("u8",))
 
 
 @pytest.mark.parametrize("cin,cout", MBV2_PW)

@@ -96,6 +96,11 @@ def test_malformed_files_are_refused(hip_ctx):
         mm.modules[0].sections[0].body = text
         mm.modules[0].functions[0].text_size = len(text)
         assert code(mm.serialize()) == -errno.EINVAL
+    # extents whose product wraps 64 bits must not get past the size check
+    huge = [km.HipTensor(t.dtype, (1 << 20, 1 << 20, 1 << 20, 1 << 20), t.zero_point, t.scale) if i == 2 else t for i, t in enumerate(tensors)]
+    mm = km.KModel.parse(good)
+    mm.modules[0].sections[0].body = km.encode_hip_text(huge, ops, tin, tout)
+    assert code(mm.serialize()) == -errno.EINVAL
     unknown = [ops[0], km.HipOp(77, ops[1].inputs, ops[1].output)] + list(ops[2:])
     mm = km.KModel.parse(good)
     mm.modules[0].sections[0].body = km.encode_hip_text(tensors, unknown, tin, tout)

@@ -160,6 +160,28 @@ def test_rope_and_kv_append(hip_ctx):
     assert np.array_equal(q[0], qkv[0].reshape(-1, d)[:hq])                # position 0: rotation by zero
 
 
+def test_kv_append_ignores_lengths_outside_the_table(hip_ctx):
+    """A negative or over-long context length appends nothing (the query is still rotated): the caches keep every byte."""
+    rng = np.random.default_rng(10)
+    B, hq, hkv, d, blk, max_blocks = 3, 4, 2, 64, 16, 2
+    nb = B * max_blocks
+    lens = np.array([-5, max_blocks * blk, 7], np.int32)
+    bt = rng.permutation(nb).reshape(B, max_blocks).astype(np.int32)
+    qkv = rng.standard_normal((B, (hq + 2 * hkv) * d)).astype(np.float16)
+    kc = rng.standard_normal((nb, hkv, blk, d)).astype(np.float16)
+    vc = rng.standard_normal((nb, hkv, d, blk)).astype(np.float16)
+    dk, dv = hip_ctx.to_device(kc), hip_ctx.to_device(vc)
+    dq = hip_ctx.alloc(B * hq * d * 2)
+    geo = rt.PagedAttnArgs(B, hq, hkv, d, blk, max_blocks, nb, 0.125, rt.DT_F16)
+    hip_ctx.rope_kv_append(hip_ctx.to_device(qkv), dq, dk, dv, hip_ctx.to_device(bt), hip_ctx.to_device(lens), geo, 1e6)
+    k2, v2 = dk.download(kc.shape, np.float16), dv.download(vc.shape, np.float16)
+    pb = bt[2, 0]
+    want_k, want_v = kc.copy(), vc.copy()
+    want_k[pb, :, 7, :], want_v[pb, :, :, 7] = k2[pb, :, 7, :], v2[pb, :, :, 7]
+    assert np.array_equal(k2, want_k) and np.array_equal(v2, want_v)       # only sequence 2 appended
+    assert np.array_equal(v2[pb, :, :, 7], qkv[2].reshape(-1, d)[hq + hkv:])
+
+
 def test_argmax_embedding_and_counter(hip_ctx):
     rng = np.random.default_rng(4)
     x = rng.standard_normal((7, 151936)).astype(np.float32)

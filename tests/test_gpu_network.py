@@ -45,6 +45,22 @@ def test_conv_block_config2(hip_ctx):
         hip_ctx.sync()
 
 
+def test_conv_block_config2_at_batch_32(hip_ctx):
+    """BASELINE config 2 at its larger batch: every tensor of the 32-image block equals the oracle's, unfused
+    (three operators) and as HipModel fuses it, eagerly and replayed as a graph."""
+    rng = np.random.default_rng(1)
+    qg = nb.quantize_graph(nb.conv_block(seed=1), rng.random((32, 56, 56, 64), dtype=f32))
+    x = rng.random((32, 56, 56, 64), dtype=f32)
+    want, outs = netref.run_integer(qg, x, keep_all=True)
+    for capture, fuse_blocks in ((False, False), (True, "all"), (True, True)):
+        model = nb.HipModel(hip_ctx, qg, 32, capture_graph=capture, fuse_blocks=fuse_blocks)
+        y = model.run(x)
+        for i, ref in enumerate(outs):
+            if model.materialized(i):
+                assert np.array_equal(model.tensor(i), ref), f"node {i} ({qg.nodes[i].name}), capture={capture}, fuse={fuse_blocks}"
+        assert np.array_equal(y.view(np.uint32), want.view(np.uint32))
+
+
 def test_mobilenetv2_config3(hip_ctx):
     g = nb.mobilenet_v2(seed=2)
     rng = np.random.default_rng(3)
@@ -164,6 +180,35 @@ def test_yolov5s_batch_consistency_at_larger_size(hip_ctx):
                 continue
             a, b = big.tensor(i)[img:img + 1], one.tensor(i)
             assert np.array_equal(a, b), f"node {i} ({qg.nodes[i].name}), image {img}: {(a != b).sum()} bytes differ"
+
+
+def test_yolov5s_config4_at_640_batch_16(hip_ctx):
+    """BASELINE config 4 at full size: 640 x 640, batch 16.  Image 0 of the batch equals the oracle on every u8
+    tensor and on the three dequantised heads; images 0 and 15 of the batch-16 run equal their batch-1 runs
+    tensor by tensor (the property that does not need the oracle at this size)."""
+    g = nb.yolov5s(seed=4, input_hw=640)
+    rng = np.random.default_rng(7)
+    qg = nb.quantize_graph(g, rng.random((2, 640, 640, 3), dtype=f32), calib_batch=1)
+    x = rng.random((16, 640, 640, 3), dtype=f32)
+    big = nb.HipModel(hip_ctx, qg, 16, capture_graph=True)
+    big.run(x)
+    heads16 = big.all_outputs()
+    wants, outs = netref.run_integer(qg, x[:1], keep_all=True)
+    for i, ref in enumerate(outs):
+        if big.materialized(i):
+            got = big.tensor(i)[:1]
+            assert np.array_equal(got, ref), f"node {i} ({qg.nodes[i].name}, {qg.nodes[i].op}): {(got != ref).sum()} of {ref.size} bytes differ"
+    for got, want in zip(heads16, wants):
+        assert np.array_equal(got[:1].view(np.uint32), want.view(np.uint32))
+    one = nb.HipModel(hip_ctx, qg, 1, capture_graph=False)
+    for img in (0, 15):
+        one.run(x[img:img + 1])
+        for i in range(len(qg.nodes)):
+            if big.materialized(i):
+                a, b = big.tensor(i)[img:img + 1], one.tensor(i)
+                assert np.array_equal(a, b), f"node {i} ({qg.nodes[i].name}), image {img}: {(a != b).sum()} bytes differ"
+        for a, b in zip(heads16, one.all_outputs()):
+            assert np.array_equal(a[img:img + 1].view(np.uint32), b.view(np.uint32))
 
 
 def test_profile_and_kernel_names(hip_ctx):

@@ -71,3 +71,13 @@ def test_fma_form_is_found_for_typical_layers_and_is_what_it_says():
 def test_out_of_range_scales_are_refused():
     with pytest.raises(rt.HipError):
         rt.requant_plan(1.0, 1.0, qp(0, 1e-30))
+
+
+def test_output_zero_points_outside_u8_are_refused():
+    # every u8 epilogue (dense, depthwise, the three stages of the fused block) is set up through the same check
+    import errno
+    for zp in (-1, 256, 1 << 20):
+        with pytest.raises(rt.HipError) as e:
+            rt.requant_plan(0.02, 0.004, qp(zp, 0.05))
+        assert e.value.code == -errno.EINVAL
+    assert rt.requant_plan(0.02, 0.004, qp(255, 0.05))[0] in (True, False)
