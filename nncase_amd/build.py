@@ -19,7 +19,7 @@ OBJ_DIR = os.path.join(LIB_DIR, "obj")
 LIB_PATH = os.path.join(LIB_DIR, "libnncase_hip.so")
 
 SOURCES = ["ctx.hip", "quant.hip", "qconv.hip", "qconv_igemm.hip", "qconv_igemm_rows16.hip", "qconv_igemm_rows8.hip", "qconv_igemm_vec16.hip",
-           "qconv_igemm_vec8.hip", "qconv_igemm_vec4.hip", "qconv_igemm_bytes.hip", "qconv_igemm_stream.hip", "qblock.hip", "qconv_smallc.hip", "qconv_dw.hip", "layout.hip", "glue.hip", "attn.hip", "llm.hip", "function.hip", "kmodel.hip"]
+           "qconv_igemm_vec8.hip", "qconv_igemm_vec4.hip", "qconv_igemm_bytes.hip", "qconv_igemm_stream.hip", "qconv_wide_rows16.hip", "qconv_wide_vec16.hip", "qblock.hip", "qconv_smallc.hip", "qconv_dw.hip", "layout.hip", "glue.hip", "attn.hip", "llm.hip", "function.hip", "kmodel.hip"]
 
 # -ffp-contract=off / -fno-fast-math: every fp32 step of the requantisation must be a
 # single IEEE operation.  packed-fp32-ops is switched off for the device pass.
@@ -40,7 +40,8 @@ def hipcc() -> str:
 
 def _compile(src: str) -> str:
     obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
-    cmd = [hipcc(), *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    # NNCASE_HIP_EXTRA_FLAGS: additional hipcc flags (e.g. -D switches of an experiment), space separated
+    cmd = [hipcc(), *FLAGS, *os.environ.get("NNCASE_HIP_EXTRA_FLAGS", "").split(), "-c", os.path.join(CSRC, src), "-o", obj]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"hipcc failed on {src}:\n{res.stdout}\n{res.stderr}")

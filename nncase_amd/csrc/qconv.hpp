@@ -16,6 +16,8 @@ struct nncase_hip_weights {
     // igemm, reductions of at most 32: the spare half of the only k-step holds -(zw - 128) against a second copy
     // of the activations, which makes the weight zero point's share of the product part of the multiplication
     int fold = 0;
+    // igemm: packed for the wide-tile kernels (qconv_wide.hpp): long reductions over many pixels and channels
+    int wide = 0;
     long long dw_const_bound = 0; // depthwise: max over channels of |bias| + 255 |sum(w - zw)|
     int64_t pixels_hint = 0; // output pixels per call the tiling was planned for (0 = unknown)
     int32_t zw = 0;

@@ -1,6 +1,6 @@
 // Host side of the implicit-GEMM convolution: weight pre-packing into MFMA
 // operand order, the tiling plan, and the launch dispatch.
-#include "qconv_igemm.hpp"
+#include "qconv_wide.hpp"
 
 #include <algorithm>
 #include <vector>
@@ -53,6 +53,16 @@ int prepack_igemm(nncase_hip_ctx *ctx, nncase_hip_weights *w, const uint8_t *w_o
     w->ksteps = ceil_div(w->k, 64);
     const int max_tiles = (w->g_ic % 4 == 0) ? 16 : 4;
     plan_igemm(w->g_oc, w->ksteps, max_tiles, w->pixels_hint, ctx->compute_units, &w->tiles, &w->nchunks, &w->kc_steps);
+    // Long reductions over many pixels and at least 64 channels are bound by the matrix cores: they take the
+    // wide-tile kernels (a wave owns 64 pixels x 64 or 128 channels; chunks of 4 or 8 tiles).
+    w->wide = w->g_ic % 16 == 0 && w->ksteps >= kWideMinKsteps && w->g_oc >= 64 && w->pixels_hint >= kWideMinPixels;
+    if (w->wide) {
+        // 256-channel chunks (two waves side by side share the block's activations) when that still gives every
+        // compute unit a block of 256 pixels
+        w->tiles = w->g_oc <= 64 ? 4 : (w->g_oc > 128 && ceil_div((int)std::min<int64_t>(w->pixels_hint, 1 << 30), 256) * (long long)ceil_div(w->g_oc, 256) >= ctx->compute_units ? 16 : 8);
+        w->nchunks = ceil_div(w->g_oc, w->tiles * 16);
+        w->kc_steps = std::min(w->ksteps, kLdsFrags / w->tiles);
+    }
     // -(zw - 128) has to be an s8 value
     w->fold = w->ksteps == 1 && w->k <= 32 && w->zw >= 1;
     const size_t group_bytes = (size_t)w->nchunks * w->ksteps * w->tiles * 1024;
@@ -85,7 +95,7 @@ int igemm_pixel_groups(const nncase_hip_ctx *ctx, const nncase_hip_weights *w, i
 
 // Weights that do not fit the LDS budget at once are streamed through it (16-byte loaders only).
 bool igemm_streams_weights(const nncase_hip_weights *w, int mode) {
-    return w->kc_steps < w->ksteps && w->tiles <= 4 && (mode == kRows16 || mode == kVec16);
+    return !w->wide && w->kc_steps < w->ksteps && w->tiles <= 4 && (mode == kRows16 || mode == kVec16);
 }
 
 // Two pixel groups per wave halve the LDS traffic per multiply; taken when that still leaves a block per CU.
@@ -167,6 +177,11 @@ int launch_qconv_igemm(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_hip_w
         a.x_coff = g * w->g_ic;
         a.y_coff = g * w->g_oc;
         int rc;
+        if (w->wide) {
+            rc = mode == kRows16 ? launch_wide_rows16(ctx, a, w->tiles, w->nchunks) : launch_wide_vec16(ctx, a, w->tiles, w->nchunks);
+            if (rc) return rc;
+            continue;
+        }
         if (igemm_streams_weights(w, mode)) {
             const int rg = stream_pixel_groups(ctx, w, a.m);
             rc = mode == kRows16 ? launch_igemm_stream_rows16(ctx, a, w->tiles, w->nchunks, rg)

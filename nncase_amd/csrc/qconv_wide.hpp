@@ -1,0 +1,354 @@
+// u8/u8 convolution / matmul as an implicit GEMM with a wide register tile per wave, for the
+// layers that are bound by the matrix cores: long reductions over many pixels and channels.
+//
+// The kernels of qconv_igemm.hpp give a wave 16 or 32 pixels, which suits reductions of one or
+// two k-steps (most of MobileNetV2) where the epilogue is the work.  For a long reduction such a
+// tile needs a 1 KiB operand fragment per matrix instruction or two, and the operand traffic, not
+// the matrix cores, sets the pace.  Here a wave owns RG * 16 pixels x T * 16 output channels
+// (64 x 128: 128 int32 accumulator registers), so a k-step of 64 needs RG activation fragments and
+// T weight fragments for RG * T matrix instructions, and a block of WM x WN waves shares both
+// operands through LDS:
+//   * a ring of three LDS slots, each holding one k-step of the block's activations and weights;
+//     global -> registers -> LDS two k-steps ahead of the multiply, one barrier per k-step;
+//   * activations are fetched in row order (the four threads of a quad read the 64 contiguous
+//     bytes of one pixel's k-step: full-width requests to the vector L1) and re-read from LDS in
+//     matrix operand order; padding taps and the u8 -> s8 re-bias are applied on the way in;
+//   * weights are pre-packed fragments in operand order (qconv_igemm.hpp, tiles = WN * T);
+//   * a matrix instruction and an ordinary vector instruction of the same SIMD do not overlap
+//     (measured: the vector work of a k-step adds to its matrix time), so the main loop is kept
+//     almost free of vector instructions: buffer loads whose per-step offsets live in scalar
+//     registers, LDS addresses that are a per-thread constant plus the slot's scalar offset plus an
+//     immediate, tap geometry on the scalar
+//     unit when a k-step lies within one tap, and the per-pixel sum of x' (which the weight zero
+//     point multiplies) from v_dot4 on the registers being staged instead of further matrix work;
+//   * blocks are numbered so that the channel chunks of one pixel tile run back to back on one
+//     XCD: the activations are fetched from HBM once and found in that XCD's L2 by the other chunks.
+// Arithmetic, weight packing and epilogue are those of qconv_igemm.hpp: the bytes are the same
+// whichever kernel runs a layer.
+#pragma once
+
+#include "qconv_igemm.hpp"
+
+#include <type_traits>
+
+namespace nnhip {
+
+// Where the wide tiles pay: measured against the kernels of qconv_igemm.hpp layer by layer (YOLOv5s-style network at
+// batch 16, batched matmul), they win from about 65 536 output pixels and reductions of 512 on; below that a launch
+// has too few 64-pixel wave tiles to fill the device and the small tiles' larger wave count wins.
+constexpr int kWideMinKsteps = 8;
+constexpr int64_t kWideMinPixels = 65536;
+constexpr int kWideSlots = 3;
+
+// How a thread finds its 16-byte pieces of a k-step:
+//   kWideRowsFull  contiguous reduction rows (1x1 windows, matmul), reduction a multiple of 64
+//   kWideRows      contiguous reduction rows, any multiple of 16
+//   kWideTap       windows; channels per group a multiple of 64, so a k-step lies within one tap (scalar tap geometry)
+//   kWideWindow    windows; channels per group a multiple of 16
+enum WideLoad { kWideRowsFull = 0, kWideRows = 1, kWideTap = 2, kWideWindow = 3 };
+
+typedef uint32_t wide_u32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t wide_rsrc(const void *base, uint32_t bytes) {
+    // raw buffer (stride 0): offsets are range-checked against `bytes`, reads outside return 0
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
+}
+
+// T: 16-channel tiles per wave; RG: 16-pixel groups per wave; a block is WM x WN waves: WM * RG * 16 pixels by
+// WN * T * 16 channels (the block's channel chunk, packed with tiles = WN * T).
+//
+// LDS: kWideSlots slots, each [activations: pixels x 64 bytes | weights: WN * T fragments].  The four 16-byte
+// pieces of pixel p are rotated by (p >> 2) & 3, so that neither the row-order writes nor the operand-order reads
+// of 16 neighbouring lanes meet on a bank.
+template <int T, int RG, int WM, int WN, int LM>
+__global__ __launch_bounds__(WM * WN * 64, 2) void qconv_wide_kernel(const IgemmArgs a, int nchunks) {
+    constexpr int THREADS = WM * WN * 64;
+    constexpr int PIX = WM * RG * 16;                   // pixels per block
+    constexpr int TB = T * WN;                          // channel tiles per block
+    constexpr int AV = PIX * 4, WV = TB * 64;           // 16-byte vectors of activations / weights per k-step
+    constexpr int NA = AV / THREADS, NW = WV / THREADS; // ... per thread
+    static_assert(AV % THREADS == 0 && WV % THREADS == 0, "every thread moves the same number of vectors");
+    static_assert(T % 2 == 0, "channel tiles are multiplied in pairs");
+    constexpr int G = T / 2;
+    constexpr int SLOT = AV * 16 + WV * 16;             // bytes of a ring slot
+    constexpr bool kRows = LM == kWideRowsFull || LM == kWideRows;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    int32_t *cterm = reinterpret_cast<int32_t *>(smem);              // [TB * 16]
+    uint8_t *lutl = smem + TB * 16 * sizeof(int32_t);                // [256]
+    int32_t *rowsums = reinterpret_cast<int32_t *>(lutl + 256);      // [PIX]
+    uint8_t *ring = lutl + 256 + PIX * sizeof(int32_t);              // [kWideSlots][SLOT]
+
+    // channel chunks of a pixel tile are consecutive on one XCD (blocks go to the 8 XCDs round-robin)
+    const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3;
+    const int chunk = seq % nchunks;
+    const int mt = (seq / nchunks) * 8 + xcd;
+    if (mt >= a.num_mtiles) return;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wm = wave % WM, wn = wave / WM;
+    const int j = lane & 15, gq = lane >> 4; // matrix operand order: pixel j of a group, 16-byte piece gq of the k-step
+    const int ch_base = chunk * (TB * 16);
+    const int KS = a.ksteps;
+    const __amdgpu_buffer_rsrc_t wres = wide_rsrc(a.wpk + (size_t)chunk * KS * TB * 1024, (uint32_t)KS * TB * 1024);
+    const __amdgpu_buffer_rsrc_t xres = wide_rsrc(a.x, (uint32_t)a.x_bytes);
+
+    // per-channel constant of the zero-point identity and the byte table: requested now, needed by the epilogue
+    constexpr int NC = (TB * 16 + THREADS - 1) / THREADS;
+    int32_t c_bias[NC], c_wsum[NC];
+#pragma unroll
+    for (int i = 0; i < NC; i++) {
+        const int c = i * THREADS + threadIdx.x;
+        const bool real = c < TB * 16 && ch_base + c < a.n;
+        c_bias[i] = real ? a.bias[ch_base + c] : 0;
+        c_wsum[i] = real ? a.wsum[ch_base + c] : 0;
+    }
+    uint32_t lut_word = 0;
+    const bool lut_mine = a.lut && threadIdx.x < 64;
+    if (lut_mine) lut_word = a.lut[threadIdx.x];
+
+    // ---- weights: thread t moves vectors t + i * THREADS of every k-step ----
+    const uint32_t w_voff = threadIdx.x * 16;
+    auto load_w = [&](wide_u32x4 (&dst)[NW], int ks) {
+        const int ksc = min(ks, KS - 1); // a k-step past the end re-reads the last one (its data is never multiplied)
+#pragma unroll
+        for (int i = 0; i < NW; i++) dst[i] = __builtin_amdgcn_raw_buffer_load_b128(wres, w_voff, (ksc * WV + i * THREADS) * 16, 0);
+    };
+    uint8_t *const w_dst = ring + AV * 16 + threadIdx.x * 16;
+    auto store_w = [&](const wide_u32x4 (&src)[NW], int slot /* byte offset of the ring slot */) {
+#pragma unroll
+        for (int i = 0; i < NW; i++) *reinterpret_cast<wide_u32x4 *>(w_dst + slot + i * THREADS * 16) = src[i];
+    };
+
+    // ---- activations: the NA pieces this thread fetches per k-step (row order: the four threads of a quad read the
+    // 64 bytes of one pixel's k-step): piece lq of pixel lp + i * (THREADS / 4) of the block ----
+    const int lp = threadIdx.x >> 2, lq = threadIdx.x & 3;
+    int32_t p_off[NA];          // byte offset of the pixel's first piece (windows: of the window origin, may be negative)
+    int32_t p_iy0[NA], p_ix0[NA];
+#pragma unroll
+    for (int i = 0; i < NA; i++) {
+        const PixInfo pi = pix_info<kRows ? kRows16 : kVec16>(a, mt * PIX + lp + i * (THREADS / 4));
+        const bool ok = pi.base >= 0; // a pixel past the end takes pixel 0's place: any valid address, the result is not stored
+        if (kRows) {
+            p_off[i] = (ok ? pi.base : 0) * a.ldx + a.x_coff + lq * 16;
+            p_iy0[i] = p_ix0[i] = 0;
+        } else {
+            p_iy0[i] = ok ? pi.iy0 : 0;
+            p_ix0[i] = ok ? pi.ix0 : 0;
+            p_off[i] = ((ok ? pi.base : 0) + p_iy0[i] * a.in_w + p_ix0[i]) * a.ldx + a.x_coff + (LM == kWideTap ? lq * 16 : 0);
+        }
+    }
+    struct Acts {
+        wide_u32x4 raw[NA];
+        uint32_t fill;    // what a piece that is not taken holds: the zero point (padding tap) or x' = 0 (past the reduction)
+        bool take[NA];
+    };
+    auto load_acts = [&](Acts &f, int ks) {
+        const int ksc = min(ks, KS - 1); // as for the weights
+        if (LM == kWideRowsFull) {
+#pragma unroll
+            for (int i = 0; i < NA; i++) {
+                f.raw[i] = __builtin_amdgcn_raw_buffer_load_b128(xres, p_off[i], ksc * 64, 0);
+                f.take[i] = true;
+            }
+            f.fill = 0;
+        } else if (LM == kWideRows) {
+            // the last k-step may end inside the row: the piece's offset goes through the range-checked operand
+            const bool in_k = ksc * 64 + lq * 16 < a.k;
+#pragma unroll
+            for (int i = 0; i < NA; i++) {
+                f.raw[i] = __builtin_amdgcn_raw_buffer_load_b128(xres, p_off[i] + ksc * 64, 0, 0);
+                f.take[i] = in_k;
+            }
+            f.fill = 0x80808080u;
+        } else if (LM == kWideTap) {
+            // one tap per k-step: its geometry is the same for the whole block (scalar unit)
+            const uint32_t kk = (uint32_t)ksc * 64;
+            const uint32_t tap = fastdiv(kk, a.d_gic);
+            const int c0 = (int)kk - (int)tap * a.g_ic;
+            const uint32_t ky = fastdiv(tap, a.d_kw);
+            const int dy = (int)ky * a.dil_h, dx = ((int)tap - (int)ky * a.kw) * a.dil_w;
+            const int shift = (dy * a.in_w + dx) * a.ldx + c0;
+#pragma unroll
+            for (int i = 0; i < NA; i++) {
+                // no clamping: an address outside the tensor reads 0, one inside but outside the image is replaced below
+                f.raw[i] = __builtin_amdgcn_raw_buffer_load_b128(xres, p_off[i] + shift, 0, 0);
+                f.take[i] = (unsigned)(p_iy0[i] + dy) < (unsigned)a.in_h && (unsigned)(p_ix0[i] + dx) < (unsigned)a.in_w;
+            }
+            f.fill = a.zx_splat;
+        } else {
+            const int kk = ksc * 64 + lq * 16;
+            const bool in_k = kk < a.k;
+            const uint32_t tap = fastdiv((uint32_t)(in_k ? kk : 0), a.d_gic);
+            const int c = (in_k ? kk : 0) - (int)tap * a.g_ic;
+            const uint32_t ky = fastdiv(tap, a.d_kw);
+            const int dy = (int)ky * a.dil_h, dx = ((int)tap - (int)ky * a.kw) * a.dil_w;
+            const int shift = (dy * a.in_w + dx) * a.ldx + c;
+#pragma unroll
+            for (int i = 0; i < NA; i++) {
+                f.raw[i] = __builtin_amdgcn_raw_buffer_load_b128(xres, p_off[i] + shift, 0, 0);
+                f.take[i] = in_k && (unsigned)(p_iy0[i] + dy) < (unsigned)a.in_h && (unsigned)(p_ix0[i] + dx) < (unsigned)a.in_w;
+            }
+            f.fill = in_k ? a.zx_splat : 0x80808080u;
+        }
+    };
+    // (THREADS / 4 is a multiple of 16, so the rotation of a thread's pieces is the same for all its pixels)
+    uint8_t *const a_dst = ring + lp * 64 + ((lq + (lp >> 2)) & 3) * 16;
+    int32_t rsum[NA]; // sum of x' over this thread's pieces of its i-th pixel
+#pragma unroll
+    for (int i = 0; i < NA; i++) rsum[i] = 0;
+    // Padding and re-biasing happen on the way into the ring: x' = (piece taken ? x : fill) ^ 0x80; the sums of x' are
+    // taken from the same registers.  A k-step past the end of the reduction is not staged (ks < KS is uniform).
+    auto store_acts = [&](const Acts &f, int slot, int ks) {
+        if (ks >= KS) return;
+#pragma unroll
+        for (int i = 0; i < NA; i++) {
+            wide_u32x4 r;
+#pragma unroll
+            for (int d = 0; d < 4; d++) {
+                r[d] = (LM == kWideRowsFull ? f.raw[i][d] : (f.take[i] ? f.raw[i][d] : f.fill)) ^ 0x80808080u;
+                rsum[i] = __builtin_amdgcn_sdot4((int)r[d], 0x01010101, rsum[i], false);
+            }
+            *reinterpret_cast<wide_u32x4 *>(a_dst + slot + i * (THREADS / 4) * 64) = r;
+        }
+    };
+
+    v4i acc[RG][T];
+#pragma unroll
+    for (int rg = 0; rg < RG; rg++)
+#pragma unroll
+        for (int nt = 0; nt < T; nt++) acc[rg][nt] = v4i{0, 0, 0, 0};
+
+    // ---- fill the pipeline ----
+    // Loads are issued unconditionally (past the end of the reduction they re-read the last k-step): loads complete
+    // in order, and only a compile-time count of younger loads lets a wait for one k-step's operands leave the later
+    // ones in flight.
+    wide_u32x4 wreg[2][NW];
+    Acts af[2];
+    {
+        wide_u32x4 w0[NW];
+        Acts a0;
+        load_w(w0, 0);
+        load_acts(a0, 0);
+        load_w(wreg[1], 1);
+        load_acts(af[1], 1);
+        load_w(wreg[0], 2);
+        load_acts(af[0], 2);
+        store_w(w0, 0);
+        store_acts(a0, 0, 0);
+        __syncthreads(); // ring slot 0 is written
+    }
+    const uint8_t *const x_src = ring + (wm * RG * 16 + j) * 64 + ((gq + (j >> 2)) & 3) * 16; // + rg * 16 * 64
+    const uint8_t *const w_src = ring + AV * 16 + (wn * T) * 1024 + lane * 16;                 // + nt * 1024
+    // One k-step s (parity P) multiplies the ring slot at byte offset `cur`: operand reads of the next pair of channel
+    // tiles are issued before the matrix instructions of the current pair (the order is pinned by scheduling
+    // barriers).  Between the pairs data moves: the operands of k-step s + 1 (in wreg[1 - P] / af[1 - P], requested
+    // two k-steps ago) go into the next slot and those of k-step s + 3 are requested.  The slot offsets are scalars:
+    // four vector additions per k-step turn the per-thread constants into this k-step's LDS addresses, everything
+    // else is an immediate.
+    int cur = 0;
+    auto kstep = [&](int s, auto parity) __attribute__((always_inline)) {
+        constexpr int P = decltype(parity)::value;
+        const int next = cur == (kWideSlots - 1) * SLOT ? 0 : cur + SLOT;
+        const uint8_t *const xs = x_src + cur, *const ws = w_src + cur;
+        v4i xf[RG];
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) xf[rg] = *reinterpret_cast<const v4i *>(xs + rg * 16 * 64);
+        v4i wf[2][2];
+        wf[0][0] = *reinterpret_cast<const v4i *>(ws);
+        wf[0][1] = *reinterpret_cast<const v4i *>(ws + 1024);
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            __builtin_amdgcn_sched_barrier(0);
+            if (g + 1 < G) {
+                wf[(g + 1) & 1][0] = *reinterpret_cast<const v4i *>(ws + (2 * g + 2) * 1024);
+                wf[(g + 1) & 1][1] = *reinterpret_cast<const v4i *>(ws + (2 * g + 3) * 1024);
+            }
+#pragma unroll
+            for (int e = 0; e < 2; e++)
+#pragma unroll
+                for (int rg = 0; rg < RG; rg++)
+                    acc[rg][2 * g + e] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[g & 1][e], xf[rg], acc[rg][2 * g + e], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (g == 0) {
+                store_w(wreg[1 - P], next);
+                load_w(wreg[1 - P], s + 3);
+            }
+            if (g == (G > 2 ? 1 : 0)) {
+                store_acts(af[1 - P], next, s + 1);
+                load_acts(af[1 - P], s + 3);
+            }
+        }
+        cur = next;
+        __syncthreads();
+    };
+    int s = 0;
+#pragma clang loop unroll(disable)
+    for (; s + 1 < KS; s += 2) {
+        kstep(s, std::integral_constant<int, 0>());
+        kstep(s + 1, std::integral_constant<int, 1>());
+    }
+    if (s < KS) kstep(s, std::integral_constant<int, 0>()); // an odd number of k-steps
+
+    // ---- epilogue ----
+#pragma unroll
+    for (int i = 0; i < NC; i++) {
+        const int c = i * THREADS + threadIdx.x;
+        if (c < TB * 16) cterm[c] = ch_base + c < a.n ? c_bias[i] - a.zxp * c_wsum[i] + a.k * a.zxp * a.zwp : 0;
+    }
+    if (lut_mine) reinterpret_cast<uint32_t *>(lutl)[threadIdx.x] = lut_word;
+    // the sums of x' sit with the threads that loaded the pieces: add the four pieces of a pixel, pass them through LDS
+#pragma unroll
+    for (int i = 0; i < NA; i++) {
+        int32_t r = rsum[i];
+        r += __shfl_xor(r, 1);
+        r += __shfl_xor(r, 2);
+        if (lq == 0) rowsums[lp + i * (THREADS / 4)] = r;
+    }
+    __syncthreads();
+    // lane (j, gq) of wave (wm, wn) holds channels ch_base + gq * 4 TB + wn * 4 T + [0, 4 T) of its pixels
+    const int ch0 = ch_base + gq * (4 * TB) + wn * (4 * T);
+    const int32_t *ct = cterm + gq * (4 * TB) + wn * (4 * T) - gq * (4 * T); // igemm_store_tile adds gq * 4 T
+#pragma unroll
+    for (int rg = 0; rg < RG; rg++) {
+        const int pl = (wm * RG + rg) * 16 + j;
+        igemm_store_tile<T>(a, acc[rg], rowsums[pl], mt * PIX + pl, ch0, gq, ct, lutl);
+    }
+}
+
+template <int T, int RG, int WM, int WN, int LM> int launch_wide_t(nncase_hip_ctx *ctx, const IgemmArgs &a, int nchunks) {
+    IgemmArgs args = a;
+    constexpr int PIX = WM * RG * 16, TB = T * WN;
+    args.num_mtiles = ceil_div(a.m, PIX);
+    const int blocks = ceil_div(args.num_mtiles, 8) * 8 * nchunks;
+    const size_t lds = (size_t)TB * 16 * sizeof(int32_t) + 256 + PIX * sizeof(int32_t) + (size_t)kWideSlots * (PIX * 64 + TB * 1024);
+    static bool raised = false; // more than 64 KiB of dynamic LDS has to be asked for once per kernel
+    if (lds > 65536 && !raised) {
+        NNHIP_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(&qconv_wide_kernel<T, RG, WM, WN, LM>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        raised = true;
+    }
+    hipLaunchKernelGGL((qconv_wide_kernel<T, RG, WM, WN, LM>), dim3(blocks), dim3(WM * WN * 64), lds, ctx->stream, args, nchunks);
+    NNHIP_LAUNCH_CHECK(ctx, "qconv_wide_kernel");
+    return 0;
+}
+
+// Pixel tiles of 256 while that gives every compute unit a block, else 128.
+inline int wide_waves(const nncase_hip_ctx *ctx, int m, int nchunks) {
+    return (long long)ceil_div(m, 256) * nchunks >= (long long)ctx->compute_units ? 4 : 2;
+}
+
+// Block shapes: tiles = 16 -> 256 pixels x 256 channels (4 x 2 waves); tiles = 8 -> 256 or 128 pixels x 128 channels;
+// tiles = 4 -> 256 or 128 pixels x 64 channels.
+template <int LM> int launch_wide_lm(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks) {
+    if (tiles == 16) return launch_wide_t<8, 4, 4, 2, LM>(ctx, a, nchunks);
+    const int wmv = wide_waves(ctx, a.m, nchunks);
+    if (tiles == 8) return wmv == 4 ? launch_wide_t<8, 4, 4, 1, LM>(ctx, a, nchunks) : launch_wide_t<8, 4, 2, 1, LM>(ctx, a, nchunks);
+    if (tiles == 4) return wmv == 4 ? launch_wide_t<4, 4, 4, 1, LM>(ctx, a, nchunks) : launch_wide_t<4, 4, 2, 1, LM>(ctx, a, nchunks);
+    return fail(ctx, -EINVAL, "qconv2d: no wide kernel for %d channel tiles", tiles);
+}
+
+int launch_wide_rows16(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks);
+int launch_wide_vec16(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks);
+
+} // namespace nnhip

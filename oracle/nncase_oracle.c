@@ -469,6 +469,10 @@ ORACLE_API int q_conv2d_u8(const uint8_t *x, const uint8_t *wq, const int32_t *b
     const int32_t out_w = windowed_out(w, kw, stride_w, dil_w, pad_w0, pad_w1);
     const int32_t g_ic = c / groups, g_oc = oc_total / groups;
     const float m = sx * sw;
+    int err = 0;
+    /* Every output element is an exact integer sum of its own: the (image, channel) planes are computed by as
+     * many threads as the host offers, which changes no value. */
+#pragma omp parallel for collapse(2) schedule(dynamic)
     for (int32_t b = 0; b < n; b++)
         for (int32_t o = 0; o < oc_total; o++) {
             const int32_t g = o / g_oc;
@@ -490,12 +494,15 @@ ORACLE_API int q_conv2d_u8(const uint8_t *x, const uint8_t *wq, const int32_t *b
                             }
                         }
                     const size_t idx = (((size_t)b * oc_total + o) * out_h + oy) * out_w + ox;
-                    int rc = store_out(out, idx, acc, out_mode, m, act_lo, act_hi, sy,
-                                       (float)zy);
-                    if (rc) return rc;
+                    const int rc = store_out(out, idx, acc, out_mode, m, act_lo, act_hi, sy,
+                                             (float)zy);
+                    if (rc) {
+#pragma omp atomic write
+                        err = rc;
+                    }
                 }
         }
-    return 0;
+    return err;
 }
 
 /* u8/u8 matmul: A [M,K] row-major, B [K,N] row-major, optional int32 bias[N]. */

@@ -153,6 +153,91 @@ def test_depthwise_multi_row_strips_at_full_batch(hip_ctx, n, c, hw, s):
     run_case(hip_ctx, n, c, hw, hw, c, 3, 3, (s, s), pad, (1, 1), c, seed=n + c + hw + s, modes=("u8", "i32"))
 
 
+# Reductions of at least 512 over at least 65 536 pixels and 64 channels take the wide-tile kernels (a wave owns 64 pixels
+# x 64 or 128 channels): windows, strides, dilation, groups, reductions that end inside a k-step, pixel and channel counts
+# that end inside a tile, 255 channels (unaligned rows), and the matmul form with a long contiguous reduction.  Cases are
+# (n, c, h, w, oc, k, stride, pad, dilation, groups); the oracle needs about 2.5 s per 10^9 multiply-adds.
+WIDE = [
+    (1, 64, 256, 257, 72, 3, (1, 1), ((1, 1), (1, 1)), (1, 1), 1),      # K = 576 (one tap per k-step), 72 channels, ragged pixel tile
+    (1, 512, 256, 256, 64, 1, (1, 1), ((0, 0), (0, 0)), (1, 1), 1),     # 1x1 rows, K = 512, 64 channels (T = 4)
+    (2, 528, 181, 182, 66, 1, (1, 1), ((0, 0), (0, 0)), (1, 1), 1),     # 1x1 rows, K = 528: the last k-step ends inside the row
+    (1, 16, 256, 258, 64, 7, (1, 1), ((3, 3), (3, 3)), (1, 1), 1),      # 7x7 over 16 channels: K = 784, four taps per k-step
+    (1, 48, 520, 516, 80, 4, (2, 2), ((1, 1), (1, 1)), (1, 1), 1),      # K = 768, 48 channels per tap, stride 2, even window
+    (1, 128, 258, 258, 130, 3, (1, 1), ((2, 2), (2, 2)), (2, 2), 2),    # two groups of 64 -> 65 channels, dilation 2
+]
+
+
+@pytest.mark.parametrize("case", WIDE)
+def test_wide_tile_kernels(hip_ctx, case):
+    n, c, h, w, oc, k, stride, pad, dil, groups = case
+    rng = np.random.default_rng(sum(case[:6]) + 11)
+    x = rng.integers(0, 256, (n, c, h, w), dtype=np.uint8)
+    wt = rng.integers(0, 256, (oc, c // groups, k, k), dtype=np.uint8)
+    bias = rng.integers(-3000, 3000, oc).astype(np.int32)
+    zx, sx, zw, sw = 7, f32(0.0235), 131, f32(0.0041)
+    common = dict(stride=stride, padding=pad, dilation=dil, groups=groups)
+    # one oracle convolution gives the accumulators; the other output forms are the oracle's epilogue applied to them
+    acc = O.qconv2d(x, wt, bias, zx, sx, zw, sw, out_mode=O.OUT_I32, **common)
+    assert acc.shape[0] * acc.shape[2] * acc.shape[3] >= 65536
+    got = K.conv2d(x, wt, bias, stride, pad, dil, groups, FULL, qp(zx, sx), qp(zw, sw), None, np.int32, ctx=hip_ctx)
+    assert np.array_equal(got, acc), f"int32 accumulators differ in {(got != acc).sum()} of {acc.size}"
+    real = acc.astype(np.float64) * float(sx * sw)
+    sy = f32((real.max() - real.min()) * 0.7 / 255)
+    zy = int(np.clip(np.rint(-40 - real.min() / sy), 0, 255))
+    lo, hi = (float(v) for v in np.percentile(real, [10, 90]).astype(f32))
+    for clamp in ((lo, hi), FULL):
+        got = K.conv2d(x, wt, bias, stride, pad, dil, groups, clamp, qp(zx, sx), qp(zw, sw), qp(zy, sy), np.uint8, ctx=hip_ctx)
+        want = O.requant_u8(acc, sx, sw, sy, zy, clamp)
+        assert np.array_equal(got, want), f"u8 outputs differ in {(got != want).sum()} of {want.size}"
+    assert len(np.unique(want)) > 8
+    got = K.conv2d(x, wt, bias, stride, pad, dil, groups, (lo, hi), qp(zx, sx), qp(zw, sw), None, np.float32, ctx=hip_ctx)
+    want = np.clip((acc.astype(f32) * f32(sx * sw)), f32(lo), f32(hi))
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("c,hw,oc,k", [(512, 256, 136, 1), (64, 256, 192, 3)])
+def test_wide_tile_kernels_with_256_channel_blocks(hip_ctx, c, hw, oc, k):
+    """From 65 536 pixels on, layers of more than 128 channels run blocks of 256 pixels x 256 channels (two waves side by side
+    share the block's activations).  One oracle convolution gives the accumulators; the u8 expectation is the oracle's
+    requantisation of them."""
+    rng = np.random.default_rng(c + oc)
+    x = rng.integers(0, 256, (1, c, hw, hw), dtype=np.uint8)
+    w = rng.integers(0, 256, (oc, c, k, k), dtype=np.uint8)
+    bias = rng.integers(-3000, 3000, oc).astype(np.int32)
+    pad = ((k // 2, k // 2), (k // 2, k // 2))
+    zx, sx, zw, sw = 7, f32(0.0235), 131, f32(0.0041)
+    acc = O.qconv2d(x, w, bias, zx, sx, zw, sw, padding=pad, out_mode=O.OUT_I32)
+    got = K.conv2d(x, w, bias, (1, 1), pad, (1, 1), 1, FULL, qp(zx, sx), qp(zw, sw), None, np.int32, ctx=hip_ctx)
+    assert np.array_equal(got, acc)
+    real = acc.astype(np.float64) * float(sx * sw)
+    sy = f32((real.max() - real.min()) * 0.7 / 255)
+    zy = 60
+    lo, hi = (float(v) for v in np.percentile(real, [10, 90]).astype(f32))
+    got = K.conv2d(x, w, bias, (1, 1), pad, (1, 1), 1, (lo, hi), qp(zx, sx), qp(zw, sw), qp(zy, sy), np.uint8, ctx=hip_ctx)
+    want = O.requant_u8(acc, sx, sw, sy, zy, (lo, hi))
+    assert np.array_equal(got, want) and len(np.unique(want)) > 8
+
+
+def test_wide_tile_kernel_is_selected_and_zero_points_at_the_extremes(hip_ctx):
+    from nncase_amd import runtime as rt2
+    w8 = np.zeros((128, 64, 3, 3), np.uint8)
+    wts = hip_ctx.prepack_conv2d(w8, None, qp(131, 0.004), 1, expected_pixels=2 * 256 * 256)
+    args = rt2.Conv2dArgs(2, 256, 256, 1, 1, 1, 1, 1, 1, 1, 1, qp(7, 0.02), qp(0, 1.0), -rt2.FLT_MAX, rt2.FLT_MAX, rt2.DT_I32)
+    fn = rt2.Function(hip_ctx)
+    xb, yb = hip_ctx.alloc(2 * 256 * 256 * 64), hip_ctx.alloc(2 * 256 * 256 * 128 * 4)
+    fn.add_qconv2d(xb, wts, yb, args)
+    assert fn.op_kernel(0).startswith("qconv_wide<T=8")
+    fn.destroy()
+    # all-255 activations against all-0 and all-255 weights, zero points at both ends: the largest accumulators
+    rng = np.random.default_rng(3)
+    for xv, wv, zx, zw in ((255, 0, 0, 255), (255, 255, 0, 0), (0, 255, 255, 0), (255, 255, 255, 255)):
+        x = np.full((1, 64, 256, 256), xv, np.uint8)
+        w = np.full((64, 64, 3, 3), wv, np.uint8)
+        got = K.conv2d(x, w, None, (1, 1), ((1, 1), (1, 1)), (1, 1), 1, FULL, qp(zx, 1.0), qp(zw, 1.0), None, np.int32, ctx=hip_ctx)
+        want = O.qconv2d(x, w, np.zeros(64, np.int32), zx, 1.0, zw, 1.0, padding=((1, 1), (1, 1)), out_mode=O.OUT_I32)
+        assert np.array_equal(got, want)
+
+
 def test_large_reduction_stages_weights_through_lds_in_chunks(hip_ctx):
     # 3x3 over 256 channels: K = 2304 (36 k-steps) -> weights staged in several LDS chunks
     run_case(hip_ctx, 1, 256, 10, 10, 64, 3, 3, (1, 1), ((1, 1), (1, 1)), (1, 1), 1, seed=3, modes=("u8", "i32"))
@@ -399,7 +484,8 @@ def test_fused_residual_equals_conv_then_add(hip_ctx, cin, cout, hw, k):
 
 
 @pytest.mark.parametrize("cin,cout,hw,k,with_residual", [(64, 32, 12, 1, False), (32, 32, 9, 3, True), (128, 255, 5, 1, False),
-                                                         (4, 32, 20, 6, False), (256, 128, 7, 3, True)])
+                                                         (4, 32, 20, 6, False), (256, 128, 7, 3, True),
+                                                         (64, 72, 182, 3, True), (512, 255, 182, 1, True)])   # the last two: wide-tile kernels
 def test_fused_table_equals_conv_then_table(hip_ctx, cin, cout, hw, k, with_residual):
     """conv with a fused swish table (and a residual add behind it) == conv, then the table, then the add."""
     rng = np.random.default_rng(cin + cout + k)
