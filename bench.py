@@ -6,9 +6,12 @@ a resident `hip` function (one HIP-graph replay per step) with the input already
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 64]
 
 Prints ONE JSON line.  Besides the contract fields it carries
-  roofline     -- the kernel with the largest share of device time: algorithmic bytes per
-                  launch / mean launch duration (HIP events on the stream the kernels run on)
-                  against the 8 TB/s HBM peak
+  roofline     -- the kernel family (one kernel symbol, whatever its template arguments) with the
+                  largest share of device time: algorithmic bytes of its launches / their summed
+                  mean durations (HIP events on the stream the kernels run on) against the 8 TB/s
+                  HBM peak; rooflines_by_family holds the same for the five largest families
+  step_ms      -- min / avg / max of single, individually synchronised steps (the reference's
+                  benchmark protocol, benchmark/cli.cpp:41-63)
   cpu_baseline -- the same graph executed the way nncase's CPU target executes it
                   (Dequantize -> float Conv2D -> Quantize with the loop-for-loop restatement of
                   its kernels), one thread, on a bounded number of batch-1 images.
@@ -107,6 +110,20 @@ def time_calls(ctx, fn, warmup, steps):
     return (time.perf_counter() - t0) / steps * 1e3
 
 
+def step_spread(ctx, fn, steps):
+    """min / avg / max milliseconds of single steps, each synchronised on its own (the reference's benchmark
+    protocol, benchmark/cli.cpp:41-63: warm-up, then every run timed separately).  A step timed alone includes the
+    host's launch and synchronisation latency, which back-to-back steps hide; `ms_per_step` is the back-to-back figure."""
+    times = []
+    for _ in range(steps):
+        ctx.sync()
+        t0 = time.perf_counter()
+        fn()
+        ctx.sync()
+        times.append((time.perf_counter() - t0) * 1e3)
+    return {"min": round(min(times), 5), "avg": round(sum(times) / len(times), 5), "max": round(max(times), 5), "runs": len(times)}
+
+
 def side_workload(args):
     """The other BASELINE configurations' kernels at their real shapes (one JSON line each):
     --workload matmul            config 1: A[512,1024] u8 x B[1024,1024] u8 -> f32
@@ -122,20 +139,30 @@ def side_workload(args):
     base = {"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
             "vs_baseline": None, "data": "synthetic"}
     if args.workload == "matmul":
+        # config 1, and with --batched N the same product on N stacked A matrices (M = 512 N rows against the one
+        # constant B): the steady-state form, in which the matrix cores and not the launch set the time
         rng = np.random.default_rng(0)
-        a = rng.integers(0, 256, (512, 1024), dtype=np.uint8)
+        rows = 512 * max(1, args.batched)
+        a = rng.integers(0, 256, (rows, 1024), dtype=np.uint8)
         bq, zb, sb = quant.quantize_weights((rng.standard_normal((1024, 1024)) * 0.05).astype(np.float32))
-        w = ctx.prepack_matmul(bq, None, qp(zb, sb), expected_rows=512)
-        da, dy = ctx.to_device(a), ctx.alloc(512 * 1024 * 4)
-        margs = rt.MatmulArgs(512, qp(128, 0.02), qp(0, 1.0), -rt.FLT_MAX, rt.FLT_MAX, rt.DT_F32)
-        ms = time_calls(ctx, lambda: ctx.qmatmul(da, w, dy, margs), args.warmup, args.steps)
-        ops, nbytes = 2 * 512 * 1024 * 1024, 524288 + 1048576 + 2097152
-        line = dict(base, metric="int8 TOPS u8/u8 MatMul 512x1024x1024 -> f32", value=round(ops / (ms * 1e-3) / 1e12, 2), unit="TOPS",
-                    ms_per_step=round(ms, 5), dtype="u8", config={"workload": "config 1: A[512,1024] u8 x B[1024,1024] u8, f32 out"},
-                    roofline={"bound": "mfma", "achieved": round(ops / (ms * 1e-3) / 1e12, 2), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
-                              "frac": round(ops / (ms * 1e-3) / 1e12 / INT8_PEAK_TOPS, 5), "traffic": None,
-                              "hbm_GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
-                              "note": "1.07 G int8-op and 3.67 MB: both roofline floors are < 0.5 us, the launch is latency-bound"})
+        w = ctx.prepack_matmul(bq, None, qp(zb, sb), expected_rows=rows)
+        da, dy = ctx.to_device(a), ctx.alloc(rows * 1024 * 4)
+        margs = rt.MatmulArgs(rows, qp(128, 0.02), qp(0, 1.0), -rt.FLT_MAX, rt.FLT_MAX, rt.DT_F32)
+        call = lambda: ctx.qmatmul(da, w, dy, margs)
+        ms = time_calls(ctx, call, args.warmup, args.steps)
+        ops, nbytes = 2 * rows * 1024 * 1024, rows * 1024 + 1048576 + rows * 1024 * 4
+        tops = ops / (ms * 1e-3) / 1e12
+        note = ("1.07 G int8-op and 3.67 MB: both roofline floors are < 0.5 us, the launch is latency-bound" if rows == 512 else
+                f"{ops / 1e9:.1f} G int8-op, {nbytes / 1e6:.0f} MB (the f32 result is {rows * 4096 / 1e6:.0f} MB of it): floors "
+                f"{ops / INT8_PEAK_TOPS / 1e6:.1f} us on the matrix cores, {nbytes / HBM_PEAK_GBS / 1e3:.1f} us on HBM")
+        line = dict(base, metric=f"int8 TOPS u8/u8 MatMul {rows}x1024x1024 -> f32", value=round(tops, 2), unit="TOPS",
+                    ms_per_step=round(ms, 5), dtype="u8",
+                    config={"workload": "config 1: A[512,1024] u8 x B[1024,1024] u8, f32 out" +
+                                        (f", batched x{args.batched} (A stacked to [{rows},1024])" if args.batched > 1 else "")},
+                    roofline={"bound": "mfma", "achieved": round(tops, 2), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+                              "frac": round(tops / INT8_PEAK_TOPS, 5), "traffic": None,
+                              "hbm_GBps": round(nbytes / (ms * 1e-3) / 1e9, 1), "note": note},
+                    step_ms=step_spread(ctx, call, args.steps))
     elif args.workload == "conv_block":
         batch = 32
         rng = np.random.default_rng(1)
@@ -143,6 +170,7 @@ def side_workload(args):
         model = nb.HipModel(ctx, qg, batch, capture_graph=True)
         model.set_input(rng.random((batch, 56, 56, 64), dtype=np.float32))
         ms = time_calls(ctx, model.invoke, args.warmup, args.steps)
+        spread = step_spread(ctx, model.invoke, args.steps)
         op_ms = model.fn.profile(10)
         nbytes = sum(op_accounting(qg, batch, model)[0])
         line = dict(base, metric="images/sec u8/u8 conv block b32", value=round(batch / (ms * 1e-3), 1), unit="images/s",
@@ -150,6 +178,7 @@ def side_workload(args):
                     config={"workload": "config 2: f32 in -> quantize -> 1x1 64->144, dw 3x3, 1x1 144->64 (ReLU6) on 56x56 -> dequantize, batch 32"},
                     roofline={"bound": "hbm", "achieved": round(nbytes / (sum(op_ms) * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                               "frac": round(nbytes / (sum(op_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None},
+                    step_ms=spread,
                     kernels={model.fn.op_kernel(i): round(t * 1e3, 2) for i, t in enumerate(op_ms)})
     elif args.workload == "yolov5s":
         batch, hw = 16, 640
@@ -160,6 +189,7 @@ def side_workload(args):
         x = rng.random((batch, hw, hw, 3), dtype=np.float32)
         model.set_input(x)
         ms = time_calls(ctx, model.invoke, args.warmup, args.steps)
+        spread = step_spread(ctx, model.invoke, args.steps)
         # per-kernel figures on the one-chain recording (kernels of concurrent chains have no duration of their own)
         kmodel = model if args.lanes == 1 else nb.HipModel(ctx, qg, batch, capture_graph=False)
         if kmodel is not model:
@@ -189,7 +219,7 @@ def side_workload(args):
                     roofline={"bound": "mfma", "achieved": round(2 * macs / (conv_ms * 1e-3) / 1e12, 1), "peak": INT8_PEAK_TOPS,
                               "unit": "TOP/s", "frac": round(2 * macs / (conv_ms * 1e-3) / 1e12 / INT8_PEAK_TOPS, 4), "traffic": None,
                               "note": "all convolutions together: int8 op count / summed conv kernel time"},
-                    sum_of_kernel_ms=round(sum(op_ms), 4),
+                    step_ms=spread, sum_of_kernel_ms=round(sum(op_ms), 4),
                     kernel_groups_ms={k: round(v, 4) for k, v in sorted(groups.items(), key=lambda kv: -kv[1])})
     elif args.workload == "llm_decode":
         from nncase_amd import llm
@@ -242,7 +272,9 @@ def side_workload(args):
         dq, dk, dv, dbt, dcl = (ctx.to_device(t) for t in (q, kc, vc, bt, lens))
         dout = ctx.alloc(bsz * hq * d * 2)
         pargs = rt.PagedAttnArgs(bsz, hq, hkv, d, blk, max_blocks, nblocks, 0.125, rt.DT_F16)
-        ms = time_calls(ctx, lambda: ctx.paged_attention_decode(dq, dk, dv, dbt, dcl, dout, pargs), args.warmup, args.steps)
+        attn = lambda: ctx.paged_attention_decode(dq, dk, dv, dbt, dcl, dout, pargs)
+        ms = time_calls(ctx, attn, args.warmup, args.steps)
+        spread = step_spread(ctx, attn, args.steps)
         kv_bytes = int(lens.sum()) * hkv * d * 2 * 2
         line = dict(base, metric="sequence-layers/sec paged-attention decode b32", value=round(bsz / (ms * 1e-3), 1), unit="sequence-layers/s",
                     ms_per_step=round(ms, 5), dtype="f16",
@@ -250,7 +282,8 @@ def side_workload(args):
                                         f"{int(lens.sum())} cached tokens, fp16 KV"},
                     roofline={"bound": "hbm", "achieved": round(kv_bytes / (ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                               "frac": round(kv_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
-                              "algorithmic_bytes_per_launch": kv_bytes})
+                              "algorithmic_bytes_per_launch": kv_bytes},
+                    step_ms=spread)
     else:
         sys.exit(f"unknown workload {args.workload}")
     print(json.dumps(line))
@@ -263,6 +296,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--batch", type=int, default=64)
+    ap.add_argument("--batched", type=int, default=1, help="--workload matmul: number of stacked A matrices (M = 512 x this)")
     ap.add_argument("--lanes", type=int, default=2,
                     help="independent chains the batch is split into and replayed concurrently (1 = one chain of "
                          "full-batch launches); results are bit-identical for every value")
@@ -314,6 +348,7 @@ def main():
     dt = time.perf_counter() - t0
     ms_per_step = dt / args.steps * 1e3
     images_per_s = args.batch / (dt / args.steps)
+    spread = step_spread(ctx, model.invoke, args.steps)
 
     # ---- per-kernel device time (HIP events on the context's stream) --------------------------
     # Kernels of concurrently replayed chains overlap and have no duration of their own, so the per-kernel figures
@@ -340,8 +375,42 @@ def main():
         g["floor"] += fb
         g["macs"] += m
         g["launches"] += 1
-    dom_name, dom = max(groups.items(), key=lambda kv: kv[1]["ms"])
-    dom_gbs = dom["bytes"] / (dom["ms"] * 1e-3) / 1e9
+    # Kernel families (one symbol, whatever its template arguments and fused extras): the dominant one is the family
+    # with the largest share of device time.
+    def family(name):
+        return name.split("<")[0].split("+")[0]
+
+    fams = {}
+    for name, g in groups.items():
+        f = fams.setdefault(family(name), {"ms": 0.0, "bytes": 0, "floor": 0, "macs": 0, "launches": 0, "traffic": 0, "traffic_known": True})
+        for k in ("ms", "bytes", "floor", "macs", "launches"):
+            f[k] += g[k]
+        t = MEASURED_TRAFFIC_B64.get(name) if args.batch == 64 and not args.no_fuse_blocks else None
+        if t is None:
+            f["traffic_known"] = False
+        else:
+            f["traffic"] += t * g["launches"]
+
+    def roofline_of(fname, f):
+        # a fused block is held to the bytes it cannot avoid (its input, output and constants); the bytes of the
+        # operators it replaces, as the reference runs them, are reported beside it
+        own = f["floor"] if fname == "qblock" else f["bytes"]
+        gbs = own / (f["ms"] * 1e-3) / 1e9
+        r = {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+             "traffic": int(f["traffic"] / f["launches"]) if f["traffic_known"] else None,
+             "kernel": fname, "images_per_launch": args.batch, "launches_per_step": f["launches"],
+             "avg_launch_us": round(f["ms"] / f["launches"] * 1e3, 2),
+             "algorithmic_bytes_per_launch": int(own / f["launches"]),
+             "share_of_device_time": round(f["ms"] / sum(op_ms), 4),
+             "int8_TOPS": round(2 * f["macs"] / (f["ms"] * 1e-3) / 1e12, 2),
+             "mfma_frac": round(2 * f["macs"] / (f["ms"] * 1e-3) / 1e12 / INT8_PEAK_TOPS, 5)}
+        if fname == "qblock":
+            r["unfused_operator_bytes_per_launch"] = int(f["bytes"] / f["launches"])
+            r["unfused_credit_GBps"] = round(f["bytes"] / (f["ms"] * 1e-3) / 1e9, 1)
+        return r
+
+    ranked = sorted(fams.items(), key=lambda kv: -kv[1]["ms"])
+    dom_name, dom = ranked[0]
 
     def klass(name):
         if name.startswith("qblock"):
@@ -414,14 +483,9 @@ def main():
                    "batch": args.batch, "lanes": args.lanes, "ops_per_step": len(model.fn),
                    "execution": "resident hip function, " + ("eager launches" if args.no_graph else "HIP-graph replay") +
                                 (f", {args.lanes} concurrent chains of {lane_batch} images" if args.lanes > 1 and not args.no_graph else "")},
-        "roofline": {"bound": "hbm", "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(dom_gbs / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC_B64.get(dom_name) if args.batch == 64 and not args.no_fuse_blocks else None,
-                     "kernel": dom_name, "images_per_launch": args.batch,
-                     "launches_per_step": dom["launches"], "avg_launch_us": round(dom["ms"] / dom["launches"] * 1e3, 2),
-                     "algorithmic_bytes_per_launch": int(dom["bytes"] / dom["launches"]),
-                     "fused_floor_bytes_per_launch": int(dom["floor"] / dom["launches"]),
-                     "share_of_device_time": round(dom["ms"] / sum(op_ms), 4)},
+        "roofline": roofline_of(dom_name, dom),
+        "rooflines_by_family": [roofline_of(n, f) for n, f in ranked[:5]],
+        "step_ms": spread,
         "cpu_baseline": cpu,
         "int8_TOPS_whole_net": round(2 * total_macs / (ms_per_step * 1e-3) / 1e12, 2),
         "hbm_GBps_whole_net": round(sum(abytes) / (ms_per_step * 1e-3) / 1e9, 1),

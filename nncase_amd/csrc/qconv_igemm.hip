@@ -54,14 +54,19 @@ int prepack_igemm(nncase_hip_ctx *ctx, nncase_hip_weights *w, const uint8_t *w_o
     const int max_tiles = (w->g_ic % 4 == 0) ? 16 : 4;
     plan_igemm(w->g_oc, w->ksteps, max_tiles, w->pixels_hint, ctx->compute_units, &w->tiles, &w->nchunks, &w->kc_steps);
     // Long reductions over many pixels and at least 64 channels are bound by the matrix cores: they take the
-    // wide-tile kernels (a wave owns 64 pixels x 64 or 128 channels; chunks of 4 or 8 tiles).
-    w->wide = w->g_ic % 16 == 0 && w->ksteps >= kWideMinKsteps && w->g_oc >= 64 && w->pixels_hint >= kWideMinPixels;
-    if (w->wide) {
-        // 256-channel chunks (two waves side by side share the block's activations) when that still gives every
-        // compute unit a block of 256 pixels
-        w->tiles = w->g_oc <= 64 ? 4 : (w->g_oc > 128 && ceil_div((int)std::min<int64_t>(w->pixels_hint, 1 << 30), 256) * (long long)ceil_div(w->g_oc, 256) >= ctx->compute_units ? 16 : 8);
-        w->nchunks = ceil_div(w->g_oc, w->tiles * 16);
-        w->kc_steps = std::min(w->ksteps, kLdsFrags / w->tiles);
+    // wide-tile kernels (a wave owns 64 pixels x 64 or 128 channels) when the launch has a 256-pixel block for every
+    // compute unit; smaller launches keep the small tiles, whose larger wave count fills the device better.
+    {
+        const long long ptiles = ceil_div((int)std::min<int64_t>(std::max<int64_t>(w->pixels_hint, 0), 1 << 30), 256);
+        // 256-channel chunks (two waves side by side share the block's activations) where that still fills the device
+        const int wide_tiles = w->g_oc <= 64 ? 4 : (w->g_oc > 128 && ptiles * ceil_div(w->g_oc, 256) >= ctx->compute_units ? 16 : 8);
+        w->wide = w->g_ic % 16 == 0 && w->ksteps >= kWideMinKsteps && w->g_oc >= 64 &&
+                  ptiles * ceil_div(w->g_oc, wide_tiles * 16) >= ctx->compute_units;
+        if (w->wide) {
+            w->tiles = wide_tiles;
+            w->nchunks = ceil_div(w->g_oc, w->tiles * 16);
+            w->kc_steps = std::min(w->ksteps, kLdsFrags / w->tiles);
+        }
     }
     // -(zw - 128) has to be an s8 value
     w->fold = w->ksteps == 1 && w->k <= 32 && w->zw >= 1;

@@ -34,10 +34,10 @@
 namespace nnhip {
 
 // Where the wide tiles pay: measured against the kernels of qconv_igemm.hpp layer by layer (YOLOv5s-style network at
-// batch 16, batched matmul), they win from about 65 536 output pixels and reductions of 512 on; below that a launch
-// has too few 64-pixel wave tiles to fill the device and the small tiles' larger wave count wins.
+// batch 16, batched matmul), they win for reductions of 512 and more when the launch has at least one 256-pixel
+// block per compute unit; below that a launch has too few 64-pixel wave tiles to fill the device and the small tiles'
+// larger wave count wins.
 constexpr int kWideMinKsteps = 8;
-constexpr int64_t kWideMinPixels = 65536;
 constexpr int kWideSlots = 3;
 
 // How a thread finds its 16-byte pieces of a k-step:
