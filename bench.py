@@ -167,7 +167,7 @@ def side_workload(args):
         batch = 32
         rng = np.random.default_rng(1)
         qg = nb.quantize_graph(nb.conv_block(seed=1), rng.random((32, 56, 56, 64), dtype=np.float32))
-        model = nb.HipModel(ctx, qg, batch, capture_graph=True)
+        model = nb.HipModel(ctx, qg, batch, capture_graph=not args.no_graph)
         model.set_input(rng.random((batch, 56, 56, 64), dtype=np.float32))
         ms = time_calls(ctx, model.invoke, args.warmup, args.steps)
         spread = step_spread(ctx, model.invoke, args.steps)
@@ -185,7 +185,7 @@ def side_workload(args):
         rng = np.random.default_rng(7)
         g = nb.yolov5s(seed=4, input_hw=hw)
         qg = nb.quantize_graph(g, rng.random((2, hw, hw, 3), dtype=np.float32), calib_batch=1)
-        model = nb.HipModel(ctx, qg, batch, capture_graph=True, lanes=args.lanes)
+        model = nb.HipModel(ctx, qg, batch, capture_graph=not args.no_graph, lanes=args.lanes)
         x = rng.random((batch, hw, hw, 3), dtype=np.float32)
         model.set_input(x)
         ms = time_calls(ctx, model.invoke, args.warmup, args.steps)
@@ -235,7 +235,7 @@ def side_workload(args):
         kc = rng.standard_normal((nblocks, cfg.kv_heads, cfg.block_size, cfg.head_dim), dtype=np.float32).astype(np.float16)
         vc = rng.standard_normal((nblocks, cfg.kv_heads, cfg.head_dim, cfg.block_size), dtype=np.float32).astype(np.float16)
         dec = llm.HipDecoder(ctx, cfg, weights, batch, max_blocks, bt, lens, [kc] * cfg.layers, [vc] * cfg.layers,
-                             capture_graph=True, feedback=True)
+                             capture_graph=not args.no_graph, feedback=True)
         dec.set_tokens(rng.integers(0, cfg.vocab, batch).astype(np.int32))
         ms = time_calls(ctx, dec.step, args.warmup, args.steps)
         toks = dec.result()
