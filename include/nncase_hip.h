@@ -44,7 +44,10 @@ enum {
 };
 
 /* Error values beyond errno; returned negated.  The first block mirrors
- * nncase_errc (src/Native/include/nncase/runtime/error.h:21-37).            */
+ * nncase_errc (src/Native/include/nncase/runtime/error.h:21-37).  The errno
+ * values the library returns are all above it (ENOMEM 12, EFAULT 14, EBUSY 16,
+ * ENODEV 19, EINVAL 22, ENOSPC 28, ...): a status in [-7, -1] is always an
+ * nncase_errc, so a caller can map every status back without ambiguity. */
 enum {
     NNCASE_HIP_ERR_INVALID_MODEL_IDENTIFIER = 0x01,
     NNCASE_HIP_ERR_INVALID_MODEL_VERSION = 0x03,
@@ -398,7 +401,7 @@ NNCASE_HIP_API int nncase_hip_paged_attention_decode(nncase_hip_ctx_t *ctx, cons
  * context live here in a static device array of the library (8 MiB of partials + 64 KiB of counters per GPU,
  * held until the process ends); the call allocates and frees nothing and issues no memset.  Geometries whose
  * partials (batch * num_q_heads * splits * (head_dim + 2) floats, splits = context capacity / tokens per
- * split) or counters (batch * num_kv_heads words) exceed that are refused with -E2BIG.  All calls on one GPU
+ * split) or counters (batch * num_kv_heads words) exceed that are refused with -ENOSPC.  All calls on one GPU
  * share the array: calls that overlap in time on one GPU (two contexts, two streams) race; calls on one
  * context are ordered by its stream.  Results are bit-identical to nncase_hip_paged_attention_decode. */
 NNCASE_HIP_API int nncase_hip_paged_attention_decode_noalloc(nncase_hip_ctx_t *ctx, const void *q_dev, const void *k_cache_dev,
@@ -569,6 +572,14 @@ NNCASE_HIP_API int nncase_hip_function_op_kernel(nncase_hip_function_t *fn, int3
  * The file image may be released after the call. */
 typedef struct nncase_hip_kmodel nncase_hip_kmodel_t;
 NNCASE_HIP_API int nncase_hip_kmodel_load(nncase_hip_ctx_t *ctx, const void *data, size_t size, nncase_hip_kmodel_t **kmodel);
+/* The same for ONE function of a hip module, from the two byte ranges the reference's
+ * runtime gives a runtime_function: `text` is the function's slice of the module's .text
+ * section (function_header::entrypoint / text_size, model.h:60-67), `rdata` the module's
+ * .rdata section (may be empty).  This is the call a hip runtime_function's
+ * initialize_core makes (the stackvm counterpart takes the same two spans:
+ * src/Native/src/runtime/stackvm/runtime_module.cpp:27-30, runtime_function.cpp:31-36). */
+NNCASE_HIP_API int nncase_hip_kmodel_load_function(nncase_hip_ctx_t *ctx, const void *text, size_t text_size,
+                                                   const void *rdata, size_t rdata_size, nncase_hip_kmodel_t **kmodel);
 NNCASE_HIP_API int nncase_hip_kmodel_destroy(nncase_hip_kmodel_t *kmodel);
 /* The entry function (owned by the kmodel): invoke / capture / profile it with nncase_hip_function_*. */
 NNCASE_HIP_API int nncase_hip_kmodel_function(nncase_hip_kmodel_t *kmodel, nncase_hip_function_t **fn);

@@ -482,7 +482,7 @@ extern "C" int nncase_hip_paged_attention_decode_noalloc(nncase_hip_ctx_t *ctx, 
     AttnPlan plan;
     const int rc = attn_plan(ctx, p, &plan);
     if (rc) return rc;
-    NNHIP_REQUIRE(ctx, plan.partial_bytes <= kScratchPartialBytes && plan.counter_bytes <= kScratchCounterBytes, -E2BIG,
+    NNHIP_REQUIRE(ctx, plan.partial_bytes <= kScratchPartialBytes && plan.counter_bytes <= kScratchCounterBytes, -ENOSPC,
                   "paged_attention_decode_noalloc: needs %zu bytes of split partials and %zu of counters; the static "
                   "scratch holds %zu and %zu (use nncase_hip_paged_attention_decode)",
                   plan.partial_bytes, plan.counter_bytes, kScratchPartialBytes, kScratchCounterBytes);

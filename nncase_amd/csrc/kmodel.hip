@@ -145,6 +145,8 @@ static bool find_section(const uint8_t *file, size_t size, size_t first, uint32_
     return false;
 }
 
+static int build_function(nncase_hip_ctx_t *ctx, Span text_span, Span rdata, nncase_hip_kmodel_t **out);
+
 extern "C" int nncase_hip_kmodel_load(nncase_hip_ctx_t *ctx, const void *data, size_t size, nncase_hip_kmodel_t **out) {
     NNHIP_CHECK_CTX(ctx);
     NNHIP_REQUIRE(ctx, data && out, -EINVAL, "kmodel_load: null argument");
@@ -271,6 +273,23 @@ extern "C" int nncase_hip_kmodel_load(nncase_hip_ctx_t *ctx, const void *data, s
                   "kmodel_load: module kind \"%.16s\" is not \"hip\"", loc.modh.kind);
     lrc = function_text(loc, &text_span, &rdata);
     if (lrc) return lrc;
+    return build_function(ctx, text_span, rdata, out);
+}
+
+// One function of a hip module from the two byte ranges the reference's runtime hands a runtime_function:
+// its slice of the module's .text section (function_header::entrypoint, text_size) and the module's .rdata
+// section (the stackvm module reads the same pair, src/Native/src/runtime/stackvm/runtime_module.cpp:27-30,
+// runtime_function.cpp:31-36).
+extern "C" int nncase_hip_kmodel_load_function(nncase_hip_ctx_t *ctx, const void *text, size_t text_size, const void *rdata,
+                                               size_t rdata_size, nncase_hip_kmodel_t **out) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, text && out && (rdata || rdata_size == 0), -EINVAL, "kmodel_load_function: null argument");
+    *out = nullptr;
+    return build_function(ctx, Span{static_cast<const uint8_t *>(text), text_size},
+                          Span{static_cast<const uint8_t *>(rdata), rdata_size}, out);
+}
+
+static int build_function(nncase_hip_ctx_t *ctx, Span text_span, Span rdata, nncase_hip_kmodel_t **out) {
     const uint8_t *text = text_span.p;
     const size_t text_size = text_span.n;
 
@@ -492,8 +511,11 @@ extern "C" int nncase_hip_kmodel_load(nncase_hip_ctx_t *ctx, const void *data, s
         case kOpConv2d: {
             const int oc = o.p[0], gic = o.p[1], kh = o.p[2], kw = o.p[3], groups = o.p[4];
             NNHIP_REQUIRE(ctx, oc > 0 && gic > 0 && kh > 0 && kw > 0 && groups > 0, -EINVAL, "kmodel_load: op %u conv shape", k);
-            NNHIP_REQUIRE(ctx, ti.dtype == NNCASE_HIP_DT_U8 && to.dtype == NNCASE_HIP_DT_U8, -NNCASE_HIP_ERR_DATATYPE_MISMATCH,
-                          "kmodel_load: op %u conv on non-u8 tensors", k);
+            // a convolution whose Quantize consumer is absent writes float32 (the matmul of config 1 is one)
+            NNHIP_REQUIRE(ctx, ti.dtype == NNCASE_HIP_DT_U8 && (to.dtype == NNCASE_HIP_DT_U8 || to.dtype == NNCASE_HIP_DT_F32),
+                          -NNCASE_HIP_ERR_DATATYPE_MISMATCH, "kmodel_load: op %u conv needs a u8 input and a u8 or f32 output", k);
+            NNHIP_REQUIRE(ctx, to.dtype == NNCASE_HIP_DT_U8 || (fused_lut[k] < 0 && fused_add[k] < 0), -NNCASE_HIP_ERR_DATATYPE_MISMATCH,
+                          "kmodel_load: op %u writes f32, which a byte table or a residual add cannot follow", k);
             NNHIP_REQUIRE(ctx, (uint32_t)(gic * groups) == ti.dims[3] && (uint32_t)oc == to.dims[3] && ti.dims[0] == to.dims[0],
                           -NNCASE_HIP_ERR_SHAPE_MISMATCH, "kmodel_load: op %u conv channels / batch do not match its tensors", k);
             const size_t wbytes = (size_t)oc * gic * kh * kw;
@@ -518,7 +540,7 @@ extern "C" int nncase_hip_kmodel_load(nncase_hip_ctx_t *ctx, const void *data, s
             a.pad_h_before = o.p[9], a.pad_h_after = o.p[10], a.pad_w_before = o.p[11], a.pad_w_after = o.p[12];
             a.x_qp = tqp(in0), a.y_qp = tqp(dst);
             a.clamp_min = o.f[0], a.clamp_max = o.f[1];
-            a.out_dtype = NNCASE_HIP_DT_U8;
+            a.out_dtype = (int32_t)to.dtype;
             NNHIP_REQUIRE(ctx, windowed_output_size(a.in_h, kh, a.stride_h, a.dilation_h, a.pad_h_before, a.pad_h_after) == (int)to.dims[1] &&
                                    windowed_output_size(a.in_w, kw, a.stride_w, a.dilation_w, a.pad_w_before, a.pad_w_after) == (int)to.dims[2],
                           -NNCASE_HIP_ERR_SHAPE_MISMATCH, "kmodel_load: op %u conv output extent does not match its tensor", k);

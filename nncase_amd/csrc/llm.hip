@@ -443,7 +443,7 @@ extern "C" int nncase_hip_w8a16_prepack(nncase_hip_ctx_t *ctx, const int8_t *w_h
     if (hipMemcpy(w->d_packed, packed.data(), bytes, hipMemcpyHostToDevice) != hipSuccess ||
         hipMemcpy(w->d_scale, scale_host, sizeof(float) * n, hipMemcpyHostToDevice) != hipSuccess ||
         (bias_host && hipMemcpy(w->d_bias, bias_host, sizeof(float) * n, hipMemcpyHostToDevice) != hipSuccess))
-        return cleanup(fail(ctx, -EIO, "w8a16_prepack: upload failed"));
+        return cleanup(fail(ctx, -EFAULT, "w8a16_prepack: upload failed"));
     *out = w;
     return 0;
 }

@@ -145,6 +145,7 @@ SYMBOLS = {
     "nncase_hip_function_add_add_i32": (_I, [_VP, _VP, C.c_int32, C.c_int32]),
     "nncase_hip_function_set_lane": (_I, [_VP, C.c_int32]),
     "nncase_hip_kmodel_load": (_I, [_VP, _VP, _SZ, C.POINTER(_VP)]),
+    "nncase_hip_kmodel_load_function": (_I, [_VP, _VP, _SZ, _VP, _SZ, C.POINTER(_VP)]),
     "nncase_hip_kmodel_destroy": (_I, [_VP]),
     "nncase_hip_kmodel_function": (_I, [_VP, C.POINTER(_VP)]),
     "nncase_hip_kmodel_tensor": (_I, [_VP, C.c_int32, C.POINTER(_VP), _I32P, _I32P]),
@@ -566,7 +567,7 @@ class Context:
 
     def paged_attention_decode_noalloc(self, q: DeviceBuffer, k_cache: DeviceBuffer, v_cache: DeviceBuffer,
                                        block_table: DeviceBuffer, ctx_lens: DeviceBuffer, out: DeviceBuffer, args: PagedAttnArgs):
-        """The same operator on the library's static device scratch: allocates nothing (-E2BIG beyond its size)."""
+        """The same operator on the library's static device scratch: allocates nothing (-ENOSPC beyond its size)."""
         self._check(self.lib.nncase_hip_paged_attention_decode_noalloc(self.handle, q.ptr, k_cache.ptr, v_cache.ptr,
                                                                        block_table.ptr, ctx_lens.ptr, out.ptr, C.byref(args)),
                     "paged_attention_decode_noalloc")
@@ -786,11 +787,22 @@ class LoadedKModel:
     INPUT, OUTPUT = -1, -2
     _NP = {DT_F32: np.float32, DT_U8: np.uint8, DT_F16: np.float16, DT_I32: np.int32, DT_I8: np.int8, DT_I16: np.int16}
 
-    def __init__(self, ctx: Context, data: bytes):
+    def __init__(self, ctx: Context, data: bytes = None, *, text: bytes = None, rdata: bytes = b""):
+        """`data`: a whole kmodel file.  `text` / `rdata`: one function's slice of a hip module's .text
+        section and the module's .rdata section, the pair a runtime_function's initialize_core receives."""
         self.ctx = ctx
         h = C.c_void_p()
-        buf = (C.c_char * len(data)).from_buffer_copy(data)
-        ctx._check(ctx.lib.nncase_hip_kmodel_load(ctx.handle, C.cast(buf, C.c_void_p), len(data), C.byref(h)), "kmodel_load")
+        if (data is None) == (text is None):
+            raise ValueError("LoadedKModel takes either a kmodel file or a function's text (+ rdata)")
+        if data is not None:
+            buf = (C.c_char * len(data)).from_buffer_copy(data)
+            ctx._check(ctx.lib.nncase_hip_kmodel_load(ctx.handle, C.cast(buf, C.c_void_p), len(data), C.byref(h)), "kmodel_load")
+        else:
+            tbuf = (C.c_char * max(len(text), 1)).from_buffer_copy(text or b"\0")
+            rbuf = (C.c_char * max(len(rdata), 1)).from_buffer_copy(rdata or b"\0")
+            ctx._check(ctx.lib.nncase_hip_kmodel_load_function(ctx.handle, C.cast(tbuf, C.c_void_p), len(text),
+                                                               C.cast(rbuf, C.c_void_p), len(rdata), C.byref(h)),
+                       "kmodel_load_function")
         self.handle = h.value
         ctx._adopt(self)
         f = C.c_void_p()

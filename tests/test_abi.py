@@ -50,3 +50,111 @@ def test_struct_layouts_match_the_header():
     assert C.sizeof(rt.MatmulArgs) == 4 + 8 + 8 + 3 * 4
     assert C.sizeof(rt.QBlockDesc) == 3 * 4 + 3 * 8 and C.sizeof(rt.QBlockArgs) == 8 * 4 + 4 * 8 + 6 * 4 + 4 + 8 + 2 * 4
     assert C.sizeof(rt.PagedAttnArgs) == 10 * 4
+
+
+# ---- the three descriptions of every POD agree field by field: the C header, the ctypes binding, the C# binding ----
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CS_NATIVE = os.path.join(ROOT, "modules", "Nncase.Modules.Hip", "Interop", "NativeMethods.cs")
+CS_BUILDER = os.path.join(ROOT, "modules", "Nncase.Modules.Hip", "CodeGen", "Hip", "HipModuleBuilder.cs")
+KIND = {"int32_t": "i32", "int64_t": "i64", "float": "f32", "nncase_hip_quant_param_t": "qp",
+        "int": "i32", "long": "i64", "IntPtr": "ptr", "HipQuantParam": "qp"}
+SIZE_ALIGN = {"i32": (4, 4), "f32": (4, 4), "i64": (8, 8), "ptr": (8, 8), "qp": (8, 4)}
+PODS = {  # header typedef -> (C# struct, ctypes class)
+    "nncase_hip_quant_param_t": ("HipQuantParam", rt.QuantParam),
+    "nncase_hip_conv2d_desc_t": ("HipConv2DDesc", rt.Conv2dDesc),
+    "nncase_hip_conv2d_args_t": ("HipConv2DArgs", rt.Conv2dArgs),
+    "nncase_hip_qblock_desc_t": ("HipQBlockDesc", rt.QBlockDesc),
+    "nncase_hip_qblock_args_t": ("HipQBlockArgs", rt.QBlockArgs),
+    "nncase_hip_matmul_args_t": ("HipMatMulArgs", rt.MatmulArgs),
+    "nncase_hip_paged_attn_args_t": ("HipPagedAttnArgs", rt.PagedAttnArgs),
+}
+
+
+def layout(kinds):
+    """Offsets and size of a C struct with natural alignment (what LayoutKind.Sequential also produces)."""
+    off, offsets, worst = 0, [], 1
+    for k in kinds:
+        size, align = SIZE_ALIGN[k]
+        off = (off + align - 1) // align * align
+        offsets.append(off)
+        off += size
+        worst = max(worst, align)
+    return offsets, (off + worst - 1) // worst * worst
+
+
+def header_structs():
+    text = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    out = {}
+    for m in re.finditer(r"typedef struct \w+ \{(.*?)\} (\w+);", text, re.S):
+        fields = []
+        for decl in m.group(1).split(";"):
+            decl = " ".join(decl.split())
+            if not decl:
+                continue
+            if "*" in decl:
+                fields.append(("ptr", decl.split("*")[-1].strip()))
+                continue
+            ctype, names = decl.split(" ", 1)
+            fields += [(KIND[ctype], n.strip()) for n in names.split(",")]
+        out[m.group(2)] = fields
+    return out
+
+
+def csharp_structs():
+    text = open(CS_NATIVE).read()
+    out = {}
+    for m in re.finditer(r"\[StructLayout\(LayoutKind\.Sequential\)\]\s*public struct (\w+)\s*\{(.*?)\n\}", text, re.S):
+        out[m.group(1)] = [(KIND[t], n) for t, n in re.findall(r"^\s*public (\w+) (\w+);", m.group(2), re.M)]
+    return out
+
+
+def test_header_ctypes_and_csharp_pods_agree():
+    hs, cs = header_structs(), csharp_structs()
+    assert set(hs) == set(PODS), "a POD of the header has no C# / ctypes counterpart listed here"
+    for hname, (csname, ctype) in PODS.items():
+        hk = [k for k, _ in hs[hname]]
+        assert [k for k, _ in cs[csname]] == hk, f"{csname} field types / order differ from {hname}"
+        # C# PascalCase names are the header's snake_case names
+        assert [n.lower() for _, n in cs[csname]] == [n.replace("_", "") for _, n in hs[hname]], csname
+        offsets, size = layout(hk)
+        assert C.sizeof(ctype) == size, hname
+        assert [getattr(ctype, f[0]).offset for f in ctype._fields_] == offsets, hname
+        assert [f[0] for f in ctype._fields_] == [n for _, n in hs[hname]], hname
+    assert layout([k for k, _ in hs["nncase_hip_conv2d_args_t"]])[1] == 104
+
+
+def test_csharp_imports_name_exported_symbols_with_the_right_arity():
+    header = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    arity = {}
+    for m in re.finditer(r"NNCASE_HIP_API\s+[\w\s\*]+?\b(nncase_hip_\w+)\s*\((.*?)\)\s*;", header, re.S):
+        args = m.group(2).strip()
+        arity[m.group(1)] = 0 if args in ("", "void") else args.count(",") + 1
+    cs = open(CS_NATIVE).read()
+    imports = re.findall(r"public static extern \w+ (nncase_hip_\w+)\((.*?)\);", cs, re.S)
+    assert len(imports) >= 20
+    for name, args in imports:
+        assert name in arity, f"{name} is imported by the C# binding but not declared in the header"
+        assert (args.count(",") + 1 if args.strip() else 0) == arity[name], name
+
+
+def test_csharp_function_text_constants_match_the_writer():
+    from nncase_amd import kmodel as km
+    cs = open(CS_BUILDER).read()
+    const = {k: int(v) for k, v in re.findall(r"public const (?:int|uint) (\w+) = (\d+);", cs)}
+    assert const["HeaderBytes"] == km.HIPF_HEADER.size and const["TensorBytes"] == km.HIPF_TENSOR.size
+    assert const["OpBytes"] == km.HIPF_OP.size and const["TextVersion"] == km.HIPF_VERSION
+    assert const["RdataAlignment"] == 64
+    body = re.search(r"internal enum HipOpcode : uint\s*\{(.*?)\}", cs, re.S).group(1)
+    opcodes = {n.lower(): int(v) for n, v in re.findall(r"(\w+) = (\d+),", body)}
+    assert opcodes == {n.replace("_", ""): i for i, n in enumerate(km.OP_NAMES)}
+    assert '"HIPF"' in cs and km.HIPF_MAGIC == b"HIPF"
+
+
+def test_errno_statuses_stay_clear_of_the_nncase_errc_block():
+    """A status in [-7, -1] must always be an nncase_errc: the runtime-module shim maps statuses back by range."""
+    src = os.path.join(ROOT, "nncase_amd", "csrc")
+    used = set()
+    for f in os.listdir(src):
+        used |= set(re.findall(r"-(E[A-Z0-9]+)\b", open(os.path.join(src, f)).read()))
+    used -= {"ERR"}
+    assert used and all(getattr(errno, name) > 7 for name in used), sorted(used)

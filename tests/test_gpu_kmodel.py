@@ -165,3 +165,52 @@ def test_sections_merged_into_rdata_are_resolved(hip_ctx):
     km.SECTION_HEADER.pack_into(data, pos, name, km.SECTION_MERGED_INTO_RDATA, r0, size, len(rdata) + pad, len(text), mem)
     got = rt.LoadedKModel(hip_ctx, bytes(data)).run(x)
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_a_function_loads_from_its_text_and_rdata_spans(hip_ctx):
+    """The entry point a hip runtime_function's initialize_core calls: the function's slice of the module's
+    .text section plus the module's .rdata section give the same function as loading the whole file."""
+    rng = np.random.default_rng(12)
+    qg = nb.quantize_graph(nb.conv_block(seed=4), rng.random((8, 56, 56, 64), dtype=f32))
+    x = rng.random((3, 56, 56, 64), dtype=f32)
+    data = km.compile_quant_graph(qg, 3, stackvm_main=True)
+    parsed = km.KModel.parse(data)
+    hip = next(m for m in parsed.modules if m.kind == km.HIP_MODULE_KIND)
+    secs = {s.name: s.body for s in hip.sections}
+    fn = hip.functions[0]
+    text = secs[".text"][fn.entrypoint:fn.entrypoint + fn.text_size]
+    whole = rt.LoadedKModel(hip_ctx, data).run(x)
+    part = rt.LoadedKModel(hip_ctx, text=text, rdata=secs[".rdata"])
+    assert part.input_shape == x.shape
+    assert np.array_equal(part.run(x).view(np.uint32), whole.view(np.uint32))
+    with pytest.raises(rt.HipError) as e:                      # a constant that no longer fits the .rdata span
+        rt.LoadedKModel(hip_ctx, text=text, rdata=secs[".rdata"][:64])
+    assert e.value.code == -22
+    with pytest.raises(rt.HipError) as e:
+        rt.LoadedKModel(hip_ctx, text=text[:40], rdata=secs[".rdata"])
+    assert e.value.code == -22
+
+
+def test_a_matmul_function_with_f32_output_as_the_code_generator_writes_it(hip_ctx):
+    """u8 [M, K] x u8 [K, N] -> f32 recorded as a 1x1 convolution over [M, 1, 1, K] with a float32 output tensor
+    (the text the C# function builder emits for Dequantize -> MatMul without a Quantize consumer)."""
+    from oracle import oracle as O
+    rng = np.random.default_rng(21)
+    M, K, N = 96, 160, 80
+    a = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    b = rng.integers(0, 256, (K, N), dtype=np.uint8)
+    a_qp, b_qp = (7, 0.031), (131, 0.0123)
+    rdata = km.RData()
+    w_off = rdata.add(np.ascontiguousarray(b.T))            # OIHW = [N, K, 1, 1]
+    tensors = [km.HipTensor("u8", (M, 1, 1, K), *a_qp), km.HipTensor("f32", (M, 1, 1, N))]
+    inf = float(np.finfo(np.float32).max)
+    ops = [km.HipOp(km.OP_CONV2D, (0,), 1, w_off, km.NO_RDATA, (N, K, 1, 1, 1, 1, 1, 1, 1, 0, 0, 0, 0, b_qp[0]), (-inf, inf, b_qp[1]))]
+    text = km.encode_hip_text(tensors, ops, 0, 1)
+    model = rt.LoadedKModel(hip_ctx, text=text, rdata=bytes(rdata.buf))
+    assert model.input_dtype == np.uint8 and model.output_dtype == np.float32
+    got = model.run(a.reshape(M, 1, 1, K)).reshape(M, N)
+    want = O.matmul_f32(O.dequantize(a, a_qp[1], a_qp[0]), O.dequantize(b, b_qp[1], b_qp[0]))
+    # the device rounds the exact integer sum once; the float chain of the oracle rounds per term
+    exact = ((a.astype(np.int64) - a_qp[0]) @ (b.astype(np.int64) - b_qp[0])).astype(np.float64) * (np.float32(a_qp[1]).astype(np.float64) * np.float32(b_qp[1]).astype(np.float64))
+    assert np.abs(got - exact).max() <= np.abs(exact).max() * 2e-7 + 1e-6
+    assert np.abs(got - want).max() <= np.abs(want).max() * 1e-4

@@ -62,4 +62,4 @@ def test_noalloc_refuses_what_its_scratch_cannot_hold(hip_ctx):
     args = rt.PagedAttnArgs(4096, 64, 4, 64, 16, 4096, 8, 0.125, rt.DT_F32)
     with pytest.raises(rt.HipError) as e:
         hip_ctx.paged_attention_decode_noalloc(dq, dk, dv, dbt, dcl, dout, args)
-    assert e.value.code == -errno.E2BIG
+    assert e.value.code == -errno.ENOSPC
