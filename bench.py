@@ -297,9 +297,12 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--batch", type=int, default=64)
     ap.add_argument("--batched", type=int, default=1, help="--workload matmul: number of stacked A matrices (M = 512 x this)")
-    ap.add_argument("--lanes", type=int, default=2,
+    ap.add_argument("--lanes", type=int, default=1,
                     help="independent chains the batch is split into and replayed concurrently (1 = one chain of "
                          "full-batch launches); results are bit-identical for every value")
+    ap.add_argument("--in-flight", type=int, default=2,
+                    help="copies of the function (own stream and buffers each) that take the steps in turn, so that "
+                         "consecutive steps overlap on the device (1 = one step at a time)")
     ap.add_argument("--cpu-images", type=int, default=8, help="batch-1 images timed on the CPU baseline (0 = skip)")
     ap.add_argument("--profile-iters", type=int, default=10)
     ap.add_argument("--batch1-steps", type=int, default=200, help="timed batch-1 invocations (0 = skip the batch-1 figure)")
@@ -321,7 +324,8 @@ def main():
     from nncase_amd import netbuilder as nb
     from nncase_amd.runtime import Context
 
-    ctx = Context(0)  # raises if libnncase_hip.so is missing or there is no gfx950 device
+    probe_ctx = Context(0)  # raises if libnncase_hip.so is missing or there is no gfx950 device
+    ctx = probe_ctx
     if args.copy_probe:
         n = 64 << 20  # dwords
         src, dst = ctx.alloc(n * 4), ctx.alloc(n * 4)
@@ -336,19 +340,27 @@ def main():
     qg = nb.quantize_graph(graph, calib)
     x = np.random.default_rng(4).random((args.batch, 224, 224, 3), dtype=np.float32)
 
-    model = nb.HipModel(ctx, qg, args.batch, capture_graph=not args.no_graph, lanes=args.lanes, fuse_blocks=not args.no_fuse_blocks)
-    model.set_input(x)  # resident in HBM before the timed region
-    for _ in range(args.warmup):
-        model.invoke()
-    ctx.sync()
+    # --in-flight copies of the function, each with its own stream and buffers, take the steps in turn: step i + 1
+    # is enqueued while step i runs.  Every step is still one whole pass over one batch on one copy.
+    pipe = nb.HipPipeline(0, qg, args.batch, depth=args.in_flight, capture_graph=not args.no_graph, lanes=args.lanes,
+                          fuse_blocks=not args.no_fuse_blocks)
+    model = pipe.models[0]
+    ctx = pipe.contexts[0]
+    pipe.set_input(x)  # resident in HBM before the timed region
+    for _ in range(max(args.warmup, args.in_flight)):
+        pipe.submit()
+    pipe.sync()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        model.invoke()
-    ctx.sync()
+        pipe.submit()
+    pipe.sync()
     dt = time.perf_counter() - t0
     ms_per_step = dt / args.steps * 1e3
     images_per_s = args.batch / (dt / args.steps)
-    spread = step_spread(ctx, model.invoke, args.steps)
+    for m in pipe.models[1:]:
+        if not np.array_equal(m.output().view(np.uint32), model.output().view(np.uint32)):
+            sys.exit("bench.py: the copies of the function in flight disagree")
+    spread = step_spread(ctx, model.invoke, args.steps)  # one step at a time: the latency of a step on an idle device
 
     # ---- per-kernel device time (HIP events on the context's stream) --------------------------
     # Kernels of concurrently replayed chains overlap and have no duration of their own, so the per-kernel figures
@@ -480,9 +492,11 @@ def main():
         "config": {"workload": f"MobileNetV2 w1.0 224x224 u8/u8 per-tensor PTQ (32 calibration images), batch {args.batch}, "
                                "NHWC f32 input resident in HBM -> quantize -> 52 convs + 10 adds + pool + FC -> dequantize" +
                                (f"; {len(model.blocks)} expand/depthwise/project blocks fused into one kernel each" if model.blocks else ""),
-                   "batch": args.batch, "lanes": args.lanes, "ops_per_step": len(model.fn),
+                   "batch": args.batch, "lanes": args.lanes, "in_flight": args.in_flight, "ops_per_step": len(model.fn),
                    "execution": "resident hip function, " + ("eager launches" if args.no_graph else "HIP-graph replay") +
-                                (f", {args.lanes} concurrent chains of {lane_batch} images" if args.lanes > 1 and not args.no_graph else "")},
+                                (f", {args.lanes} concurrent chains of {lane_batch} images" if args.lanes > 1 and not args.no_graph else "") +
+                                (f"; {args.in_flight} copies of the function (own stream and buffers) take the steps in turn, so "
+                                 "consecutive steps overlap on the device; step_ms is one step at a time" if args.in_flight > 1 else "")},
         "roofline": roofline_of(dom_name, dom),
         "rooflines_by_family": [roofline_of(n, f) for n, f in ranked[:5]],
         "step_ms": spread,

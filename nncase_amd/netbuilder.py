@@ -620,3 +620,36 @@ class HipModel:
         self.invoke()
         self.ctx.sync()
         return self.output()
+
+
+class HipPipeline:
+    """`depth` copies of a HipModel, each on a context of its own (its stream, its activation buffers, its packed
+    constants), invoked in turn: batch i + 1 is enqueued while batch i is still running, so the small, latency-bound
+    layers at the end of one batch share the device with the bandwidth-bound layers at the start of the next.
+    Every batch is computed by one copy from start to finish, so results are the bytes a single HipModel gives.
+    This is how a server keeps a device busy with the reference too: one interpreter per request in flight
+    (an interpreter is single threaded, src/Native/src/runtime/interpreter.cpp)."""
+
+    def __init__(self, device: int, qg: QuantGraph, batch: int, depth: int = 2, **model_args):
+        if depth < 1:
+            raise ValueError("depth must be at least 1")
+        self.contexts = [Context(device) for _ in range(depth)]
+        self.models = [HipModel(c, qg, batch, **model_args) for c in self.contexts]
+        self.turn = 0
+
+    def set_input(self, x_nhwc: np.ndarray):
+        for m in self.models:
+            m.set_input(x_nhwc)
+
+    def submit(self) -> "HipModel":
+        """Enqueues one batch on the next copy and returns that copy (its output is valid after its context syncs)."""
+        m = self.models[self.turn % len(self.models)]
+        self.turn += 1
+        m.invoke()
+        return m
+
+    invoke = submit
+
+    def sync(self):
+        for c in self.contexts:
+            c.sync()

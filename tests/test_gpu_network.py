@@ -253,6 +253,27 @@ def test_lanes_split_the_batch_bit_exact(hip_ctx, lanes, capture):
         assert np.array_equal(many.run(x).view(np.uint32), y1.view(np.uint32)), f"replay {r}"
 
 
+def test_copies_in_flight_give_the_bytes_of_one_function(hip_ctx):
+    """HipPipeline: steps enqueued in turn on copies of the function (own stream, own buffers) overlap on the device;
+    every copy still holds the bytes a single function computes, whatever was in flight beside it."""
+    g = nb.mobilenet_v2(seed=2)
+    qg = nb.quantize_graph(g, np.random.default_rng(3).random((32, 224, 224, 3), dtype=f32))
+    xs = [np.random.default_rng(40 + i).random((8, 224, 224, 3), dtype=f32) for i in range(3)]
+    one = nb.HipModel(hip_ctx, qg, 8, capture_graph=False)
+    want = [one.run(x).copy() for x in xs]
+    pipe = nb.HipPipeline(0, qg, 8, depth=3, capture_graph=True)
+    for m, x in zip(pipe.models, xs):         # a different batch on every copy
+        m.set_input(x)
+    for _ in range(4):                        # 12 steps back to back, 3 in flight
+        used = [pipe.submit() for _ in range(3)]
+    assert used == pipe.models
+    pipe.sync()
+    for m, y in zip(pipe.models, want):
+        assert np.array_equal(m.output().view(np.uint32), y.view(np.uint32))
+    with pytest.raises(ValueError):
+        nb.HipPipeline(0, qg, 8, depth=0)
+
+
 def test_lanes_yolov5s_outputs(hip_ctx):
     g = nb.yolov5s(seed=5, input_hw=160)
     rng = np.random.default_rng(6)
