@@ -153,6 +153,31 @@ def test_depthwise_multi_row_strips_at_full_batch(hip_ctx, n, c, hw, s):
     run_case(hip_ctx, n, c, hw, hw, c, 3, 3, (s, s), pad, (1, 1), c, seed=n + c + hw + s, modes=("u8", "i32"))
 
 
+# 3x3 depthwise layers over patches narrower and lower than a thread's strip, images smaller than one strip, stride 2
+# with odd extents, every padding, and zero points at both ends; the second half of each case maps the accumulators
+# one to one onto the output codes, so that any error in a sum is a different byte.
+DW_SHAPES = [(2, 16, 37, 45, 1, ((1, 1), (1, 1))), (2, 48, 37, 45, 2, ((0, 1), (0, 1))), (3, 32, 7, 7, 1, ((1, 1), (1, 1))),
+             (1, 16, 1, 1, 1, ((1, 1), (1, 1))), (2, 16, 14, 14, 2, ((1, 1), (1, 1))), (1, 64, 112, 112, 1, ((1, 1), (1, 1))),
+             (1, 16, 113, 57, 2, ((1, 0), (0, 1))), (2, 32, 5, 70, 1, ((0, 0), (0, 0))), (1, 16, 40, 3, 1, ((2, 2), (2, 2)))]
+
+
+@pytest.mark.parametrize("zx,zw", [(0, 0), (255, 255), (255, 0), (0, 255), (7, 131), (3, 128), (128, 1)])
+@pytest.mark.parametrize("shape", DW_SHAPES)
+def test_depthwise_3x3_exact_sums_and_zero_points(hip_ctx, shape, zx, zw):
+    n, c, h, w, s, pad = shape
+    run_case(hip_ctx, n, c, h, w, c, 3, 3, (s, s), pad, (1, 1), c, seed=c + h * 3 + w * 5 + s + zx + zw, zx=zx, zw=zw, modes=("u8",))
+    # accumulators mapped one to one onto the codes (scales 1, zero point 128, values near the zero points):
+    # any error in a sum shows up as a different byte
+    rng = np.random.default_rng(zx * 256 + zw + h)
+    x = np.clip(zx + rng.integers(-3, 4, (n, c, h, w)), 0, 255).astype(np.uint8)
+    wt = np.clip(zw + rng.integers(-3, 4, (c, 1, 3, 3)), 0, 255).astype(np.uint8)
+    bias = rng.integers(-20, 21, c).astype(np.int32)
+    got = K.conv2d(x, wt, bias, (s, s), pad, (1, 1), c, FULL, qp(zx, 1.0), qp(zw, 1.0), qp(128, 1.0), np.uint8, ctx=hip_ctx)
+    acc = O.qconv2d(x, wt, bias, zx, 1.0, zw, 1.0, stride=(s, s), padding=pad, groups=c, out_mode=O.OUT_I32)
+    assert np.abs(acc).max() <= 127 and len(np.unique(acc)) > min(20, acc.size // 4)
+    assert np.array_equal(got, (acc + 128).astype(np.uint8))
+
+
 # Reductions of at least 512 over at least 65 536 pixels and 64 channels take the wide-tile kernels (a wave owns 64 pixels
 # x 64 or 128 channels): windows, strides, dilation, groups, reductions that end inside a k-step, pixel and channel counts
 # that end inside a tile, 255 channels (unaligned rows), and the matmul form with a long contiguous reduction.  Cases are
