@@ -155,7 +155,14 @@ def side_workload(args):
         note = ("1.07 G int8-op and 3.67 MB: both roofline floors are < 0.5 us, the launch is latency-bound" if rows == 512 else
                 f"{ops / 1e9:.1f} G int8-op, {nbytes / 1e6:.0f} MB (the f32 result is {rows * 4096 / 1e6:.0f} MB of it): floors "
                 f"{ops / INT8_PEAK_TOPS / 1e6:.1f} us on the matrix cores, {nbytes / HBM_PEAK_GBS / 1e3:.1f} us on HBM")
+        # the same product requantised to u8 (what a following quantised layer consumes): a quarter of the f32 stores
+        dy8 = ctx.alloc(rows * 1024)
+        sy = float(np.sqrt(1024.0) * 0.02 * 128 * sb * 0.6 / 128)
+        margs8 = rt.MatmulArgs(rows, qp(128, 0.02), qp(128, sy), -rt.FLT_MAX, rt.FLT_MAX, rt.DT_U8)
+        ms8 = time_calls(ctx, lambda: ctx.qmatmul(da, w, dy8, margs8), args.warmup, args.steps)
         line = dict(base, metric=f"int8 TOPS u8/u8 MatMul {rows}x1024x1024 -> f32", value=round(tops, 2), unit="TOPS",
+                    u8_out={"int8_TOPS": round(ops / (ms8 * 1e-3) / 1e12, 2), "ms_per_step": round(ms8, 5),
+                            "frac_of_int8_peak": round(ops / (ms8 * 1e-3) / 1e12 / INT8_PEAK_TOPS, 5)},
                     ms_per_step=round(ms, 5), dtype="u8",
                     config={"workload": "config 1: A[512,1024] u8 x B[1024,1024] u8, f32 out" +
                                         (f", batched x{args.batched} (A stacked to [{rows},1024])" if args.batched > 1 else "")},
@@ -185,10 +192,19 @@ def side_workload(args):
         rng = np.random.default_rng(7)
         g = nb.yolov5s(seed=4, input_hw=hw)
         qg = nb.quantize_graph(g, rng.random((2, hw, hw, 3), dtype=np.float32), calib_batch=1)
-        model = nb.HipModel(ctx, qg, batch, capture_graph=not args.no_graph, lanes=args.lanes)
+        # copies of the function in flight, as in the headline workload
+        pipe = nb.HipPipeline(0, qg, batch, depth=args.in_flight, capture_graph=not args.no_graph, lanes=args.lanes)
+        model, ctx = pipe.models[0], pipe.contexts[0]
         x = rng.random((batch, hw, hw, 3), dtype=np.float32)
-        model.set_input(x)
-        ms = time_calls(ctx, model.invoke, args.warmup, args.steps)
+        pipe.set_input(x)
+        for _ in range(max(args.warmup, args.in_flight)):
+            pipe.submit()
+        pipe.sync()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            pipe.submit()
+        pipe.sync()
+        ms = (time.perf_counter() - t0) / args.steps * 1e3
         spread = step_spread(ctx, model.invoke, args.steps)
         # per-kernel figures on the one-chain recording (kernels of concurrent chains have no duration of their own)
         kmodel = model if args.lanes == 1 else nb.HipModel(ctx, qg, batch, capture_graph=False)
@@ -214,8 +230,10 @@ def side_workload(args):
                     ms_per_step=round(ms, 4), dtype="u8",
                     config={"workload": "config 4: YOLOv5s-style backbone + neck + head, 640x640, u8/u8 per-tensor PTQ (2 calibration "
                                         "images), batch 16, SiLU as byte tables, " + str(len(kmodel.fn)) + " operators, HIP-graph replay" +
-                                        (f" as {args.lanes} concurrent chains of {batch // args.lanes} images" if args.lanes > 1 else ""),
-                            "batch_consistent": True},
+                                        (f" as {args.lanes} concurrent chains of {batch // args.lanes} images" if args.lanes > 1 else "") +
+                                        (f", {args.in_flight} copies of the function take the steps in turn (step_ms: one step at a time)"
+                                         if args.in_flight > 1 else ""),
+                            "in_flight": args.in_flight, "batch_consistent": True},
                     roofline={"bound": "mfma", "achieved": round(2 * macs / (conv_ms * 1e-3) / 1e12, 1), "peak": INT8_PEAK_TOPS,
                               "unit": "TOP/s", "frac": round(2 * macs / (conv_ms * 1e-3) / 1e12 / INT8_PEAK_TOPS, 4), "traffic": None,
                               "note": "all convolutions together: int8 op count / summed conv kernel time"},
