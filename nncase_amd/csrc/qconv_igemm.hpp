@@ -256,6 +256,66 @@ template <int MODE> __device__ __forceinline__ ActFrag load_act(const IgemmArgs 
     return f;
 }
 
+struct ActSlice { // vec16 / rows16: one 16-byte load per k-step, one fill value
+    u32x4 raw;
+    uint32_t fill;
+    uint32_t take; // 0 or ~0
+};
+
+template <int MODE> __device__ __forceinline__ ActSlice load_slice(const IgemmArgs &a, const PixInfo &pi, int kc) {
+    static_assert(MODE == kRows16 || MODE == kVec16, "one 16-byte piece per slice");
+    ActSlice f;
+    const bool pix_ok = pi.base >= 0;
+    PixInfo sp = pi;
+    if (!pix_ok) sp.base = 0, sp.iy0 = 0, sp.ix0 = 0;
+    const bool in_k = kc * 16 < a.k;
+    if (MODE == kRows16) {
+        f.raw = *reinterpret_cast<const u32x4 *>(a.x + (size_t)((uint32_t)sp.base * (uint32_t)a.ldx + a.x_coff + (in_k ? kc : 0) * 16));
+        f.fill = 0x80808080u;
+        f.take = (pix_ok && in_k) ? ~0u : 0u;
+    } else {
+        bool inside;
+        const uint32_t off = tap_offset(a, sp, in_k ? kc * 16 : 0, &inside);
+        f.raw = *reinterpret_cast<const u32x4 *>(a.x + (size_t)off);
+        f.fill = (pix_ok && in_k) ? a.zx_splat : 0x80808080u; // padding tap : outside the problem
+        f.take = (pix_ok && in_k && inside) ? ~0u : 0u;
+    }
+    return f;
+}
+
+__device__ __forceinline__ v4i finish_slice(const ActSlice &f) {
+    u32x4 r;
+#pragma unroll
+    for (int d = 0; d < 4; d++) r[d] = ((f.raw[d] & f.take) | (f.fill & ~f.take)) ^ 0x80808080u;
+    return __builtin_bit_cast(v4i, r);
+}
+
+// The activation operand in flight, by loader: the 16-byte loaders need one fill value and an all-or-nothing mask
+// (one bit operation and one xor per dword when the slice is consumed), the gathering loaders a fill and a bit per dword.
+template <int MODE> struct ActOf {
+    using type = ActFrag;
+};
+template <> struct ActOf<kRows16> {
+    using type = ActSlice;
+};
+template <> struct ActOf<kVec16> {
+    using type = ActSlice;
+};
+template <int MODE> __device__ __forceinline__ typename ActOf<MODE>::type load_operand(const IgemmArgs &a, const PixInfo &pi, int kc) {
+    if constexpr (MODE == kRows16 || MODE == kVec16) return load_slice<MODE>(a, pi, kc);
+    else return load_act<MODE>(a, pi, kc);
+}
+__device__ __forceinline__ v4i finish_operand(const ActFrag &f) { return finish_act(f); }
+__device__ __forceinline__ v4i finish_operand(const ActSlice &f) { return finish_slice(f); }
+__device__ __forceinline__ void clear_operand(ActFrag &f) {
+    f.raw = f.fill = u32x4{0, 0, 0, 0};
+    f.take = 0;
+}
+__device__ __forceinline__ void clear_operand(ActSlice &f) {
+    f.raw = u32x4{0, 0, 0, 0};
+    f.fill = 0, f.take = 0;
+}
+
 struct __attribute__((packed, aligned(1))) U32Unaligned {
     uint32_t v;
 };
@@ -416,20 +476,20 @@ __global__ void __launch_bounds__(kThreads, ((RG == 1 && T <= 12) || loads_rows(
     constexpr int pix_per_block = kWaves * RG * 16;
 
     PixInfo pcur[RG], pnxt[RG];
-    ActFrag fcur[RG], fnxt[RG];
+    using Act = typename ActOf<MODE>::type;
+    Act fcur[RG], fnxt[RG];
 #pragma unroll
     for (int rg = 0; rg < RG; rg++) {
         pnxt[rg].base = -1;
         pnxt[rg].iy0 = pnxt[rg].ix0 = 0;
-        fnxt[rg].raw = fnxt[rg].fill = u32x4{0, 0, 0, 0};
-        fnxt[rg].take = 0;
+        clear_operand(fnxt[rg]);
     }
     int mt = blockIdx.x;
     if (mt < a.num_mtiles) {
 #pragma unroll
         for (int rg = 0; rg < RG; rg++) {
             pcur[rg] = pix_info<MODE>(a, mt * pix_per_block + (wave * RG + rg) * 16 + j);
-            fcur[rg] = load_act<MODE>(a, pcur[rg], gq & a.kc_mask);
+            fcur[rg] = load_operand<MODE>(a, pcur[rg], gq & a.kc_mask);
         }
     }
     if (c_mine) cterm[threadIdx.x] = c_real ? c_bias - a.zxp * c_wsum + a.k * a.zxp * a.zwp : 0;
@@ -465,12 +525,12 @@ __global__ void __launch_bounds__(kThreads, ((RG == 1 && T <= 12) || loads_rows(
         if constexpr (kDeepBuilt) deep = nkc == 1 && a.ksteps >= 4 && a.num_mtiles <= (int)gridDim.x;
         if (deep) {
             if constexpr (kDeepBuilt) {
-                ActFrag f1 = load_act<MODE>(a, pcur[0], (4 + gq) & a.kc_mask), f2 = load_act<MODE>(a, pcur[0], (8 + gq) & a.kc_mask);
+                Act f1 = load_operand<MODE>(a, pcur[0], (4 + gq) & a.kc_mask), f2 = load_operand<MODE>(a, pcur[0], (8 + gq) & a.kc_mask);
                 int ks = 0;
-                auto step = [&](ActFrag &f) __attribute__((always_inline)) {
-                    const v4i xf = finish_act(f);
+                auto step = [&](Act &f) __attribute__((always_inline)) {
+                    const v4i xf = finish_operand(f);
                     const int nk = ks + 3 < a.ksteps ? ks + 3 : 0; // past the end: a valid slice, dropped
-                    f = load_act<MODE>(a, pcur[0], (nk * 4 + gq) & a.kc_mask);
+                    f = load_operand<MODE>(a, pcur[0], (nk * 4 + gq) & a.kc_mask);
                     rs[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, xf, rs[0], 0, 0, 0);
                     const uint8_t *wstep = wlds + (size_t)ks * T * 1024 + lane * 16;
 #pragma unroll
@@ -514,11 +574,11 @@ __global__ void __launch_bounds__(kThreads, ((RG == 1 && T <= 12) || loads_rows(
                     }
                     const int kc_next = (same_tile ? (ks + 1) * 4 + gq : gq) & a.kc_mask;
 #pragma unroll
-                    for (int rg = 0; rg < RG; rg++) fnxt[rg] = load_act<MODE>(a, select_pix(same_tile, pcur[rg], pnxt[rg]), kc_next);
+                    for (int rg = 0; rg < RG; rg++) fnxt[rg] = load_operand<MODE>(a, select_pix(same_tile, pcur[rg], pnxt[rg]), kc_next);
                 }
                 v4i xf[RG]; // the slice loaded one step ago, now needed
 #pragma unroll
-                for (int rg = 0; rg < RG; rg++) xf[rg] = finish_act(fcur[rg]);
+                for (int rg = 0; rg < RG; rg++) xf[rg] = finish_operand(fcur[rg]);
                 { // sum of x' per pixel (not needed where the weights carry the term it is for; a branch here costs more)
 #pragma unroll
                     for (int rg = 0; rg < RG; rg++)
@@ -561,40 +621,6 @@ __global__ void __launch_bounds__(kThreads, ((RG == 1 && T <= 12) || loads_rows(
 // k-steps before they are multiplied.  With one or two blocks per compute unit there are too few
 // waves to hide memory latency by switching waves, so the latency has to be covered inside the wave;
 // a one-step prefetch exposes a full memory round trip per k-step on such layers.
-struct ActSlice { // vec16 / rows16: one 16-byte load per k-step, one fill value
-    u32x4 raw;
-    uint32_t fill;
-    uint32_t take; // 0 or ~0
-};
-
-template <int MODE> __device__ __forceinline__ ActSlice load_slice(const IgemmArgs &a, const PixInfo &pi, int kc) {
-    static_assert(MODE == kRows16 || MODE == kVec16, "one 16-byte piece per slice");
-    ActSlice f;
-    const bool pix_ok = pi.base >= 0;
-    PixInfo sp = pi;
-    if (!pix_ok) sp.base = 0, sp.iy0 = 0, sp.ix0 = 0;
-    const bool in_k = kc * 16 < a.k;
-    if (MODE == kRows16) {
-        f.raw = *reinterpret_cast<const u32x4 *>(a.x + (size_t)((uint32_t)sp.base * (uint32_t)a.ldx + a.x_coff + (in_k ? kc : 0) * 16));
-        f.fill = 0x80808080u;
-        f.take = (pix_ok && in_k) ? ~0u : 0u;
-    } else {
-        bool inside;
-        const uint32_t off = tap_offset(a, sp, in_k ? kc * 16 : 0, &inside);
-        f.raw = *reinterpret_cast<const u32x4 *>(a.x + (size_t)off);
-        f.fill = (pix_ok && in_k) ? a.zx_splat : 0x80808080u; // padding tap : outside the problem
-        f.take = (pix_ok && in_k && inside) ? ~0u : 0u;
-    }
-    return f;
-}
-
-__device__ __forceinline__ v4i finish_slice(const ActSlice &f) {
-    u32x4 r;
-#pragma unroll
-    for (int d = 0; d < 4; d++) r[d] = ((f.raw[d] & f.take) | (f.fill & ~f.take)) ^ 0x80808080u;
-    return __builtin_bit_cast(v4i, r);
-}
-
 template <int T, int RG, int MODE>
 __global__ __launch_bounds__(kThreads, 2) void qconv_igemm_stream_kernel(const IgemmArgs a) {
     // three ring slots: the one being multiplied, the one being written, and one in between
