@@ -34,33 +34,57 @@ INT8_PEAK_TOPS = 5000.0    # dense int8 MFMA
 
 
 # Bytes that crossed the L2 <-> fabric boundary per launch (average over the launches of a kernel in
-# one step) at the headline workload with whole-batch launches (--lanes 1), from two rocprofv3 --pmc runs
+# one step) at the headline workload, blocks unfused (the default) and fused (--fuse-blocks), with whole-batch
+# launches one after the other (--lanes 1 --in-flight 1), from two rocprofv3 --pmc runs
 # of this script (FETCH_SIZE, then WRITE_SIZE, each scaled by what the same counter reads for the 256 MiB
 # copy that --copy-probe launches: x1.9996 and x1.0000).  Counters cannot be read from inside a timed run, so the figures
 # are recorded here and reported only for the configuration they were measured on.
 MEASURED_TRAFFIC_B64 = {
-    "dequantize": 345584,
-    "dw3x3<S=1>": 27888828,
-    "dw3x3<S=2>": 51771623,
-    "qblock+add<S=1,P=2>": 4947821,
-    "qblock+add<S=1,P=4>": 2671966,
-    "qblock+add<S=1,P=6>": 4553132,
-    "qblock<S=1,P=6>": 3246740,
-    "qblock<S=2,P=4>": 3349051,
-    "qconv_igemm+add<T=1,RG=1,rows16>": 5374109,
-    "qconv_igemm+add<T=2,RG=2,rows16>": 40883307,
-    "qconv_igemm<T=1,RG=1,rows16>": 6796878,
-    "qconv_igemm<T=1,RG=4,rows16>": 38753788,
-    "qconv_igemm<T=12,RG=1,rows16>": 9296399,
-    "qconv_igemm<T=2,RG=1,rows16>": 9024215,
-    "qconv_igemm<T=2,RG=2,rows16>": 24294005,
-    "qconv_igemm<T=5,RG=1,rows16>": 5232586,
-    "qconv_igemm<T=6,RG=1,rows16>": 8736951,
-    "qconv_igemm<T=6,RG=2,rows16>": 90273106,
-    "qconv_igemm<T=9,RG=1,rows8>": 34456035,
-    "qconv_smallc<C=3>": 38871765,
-    "qglobal_avgpool": 4237596,
-    "quantize": 48220331,
+    "unfused": {
+        "dequantize": 345584,
+        "dw3x3<S=1>": 19025622,
+        "dw3x3<S=2>": 41843409,
+        "qconv_igemm+add<T=1,RG=1,rows16>": 6194308,
+        "qconv_igemm+add<T=2,RG=1,rows16>": 11631051,
+        "qconv_igemm+add<T=2,RG=2,rows16>": 39774544,
+        "qconv_igemm<T=1,RG=1,rows16>": 5954541,
+        "qconv_igemm<T=1,RG=4,rows16>": 38749244,
+        "qconv_igemm<T=12,RG=1,rows16>": 10475918,
+        "qconv_igemm<T=2,RG=1,rows16>": 7737832,
+        "qconv_igemm<T=2,RG=2,rows16>": 24292532,
+        "qconv_igemm<T=5,RG=1,rows16>": 5242493,
+        "qconv_igemm<T=6,RG=1,rows16>": 8757427,
+        "qconv_igemm<T=6,RG=2,rows16>": 90282384,
+        "qconv_igemm<T=8,RG=1,rows16>": 6052716,
+        "qconv_igemm<T=9,RG=1,rows8>": 34453811,
+        "qconv_smallc<C=3>": 38867446,
+        "qglobal_avgpool": 4237596,
+        "quantize": 48213804,
+    },
+    "fused": {
+        "dequantize": 345584,
+        "dw3x3<S=1>": 27907587,
+        "dw3x3<S=2>": 51717610,
+        "qblock+add<S=1,P=2>": 4946701,
+        "qblock+add<S=1,P=4>": 2671624,
+        "qblock+add<S=1,P=6>": 4553259,
+        "qblock<S=1,P=6>": 3246740,
+        "qblock<S=2,P=4>": 3349274,
+        "qconv_igemm+add<T=1,RG=1,rows16>": 5371037,
+        "qconv_igemm+add<T=2,RG=2,rows16>": 39719034,
+        "qconv_igemm<T=1,RG=1,rows16>": 6795342,
+        "qconv_igemm<T=1,RG=4,rows16>": 38749372,
+        "qconv_igemm<T=12,RG=1,rows16>": 9327753,
+        "qconv_igemm<T=2,RG=1,rows16>": 9008858,
+        "qconv_igemm<T=2,RG=2,rows16>": 24292340,
+        "qconv_igemm<T=5,RG=1,rows16>": 5242695,
+        "qconv_igemm<T=6,RG=1,rows16>": 8757427,
+        "qconv_igemm<T=6,RG=2,rows16>": 90282064,
+        "qconv_igemm<T=9,RG=1,rows8>": 34453379,
+        "qconv_smallc<C=3>": 38867894,
+        "qglobal_avgpool": 4237596,
+        "quantize": 48213772,
+    },
 }
 
 
@@ -318,14 +342,16 @@ def main():
     ap.add_argument("--lanes", type=int, default=1,
                     help="independent chains the batch is split into and replayed concurrently (1 = one chain of "
                          "full-batch launches); results are bit-identical for every value")
-    ap.add_argument("--in-flight", type=int, default=2,
+    ap.add_argument("--in-flight", type=int, default=3,
                     help="copies of the function (own stream and buffers each) that take the steps in turn, so that "
                          "consecutive steps overlap on the device (1 = one step at a time)")
     ap.add_argument("--cpu-images", type=int, default=8, help="batch-1 images timed on the CPU baseline (0 = skip)")
     ap.add_argument("--profile-iters", type=int, default=10)
     ap.add_argument("--batch1-steps", type=int, default=200, help="timed batch-1 invocations (0 = skip the batch-1 figure)")
-    ap.add_argument("--no-fuse-blocks", action="store_true",
-                    help="run every expand -> depthwise -> project block as three operators")
+    ap.add_argument("--fuse-blocks", action="store_true",
+                    help="run the inverted-residual blocks on the 28x28 and 14x14 maps as one fused kernel each (38 operators "
+                         "instead of 56): shorter single steps, but more vector-ALU work in total, so fewer images per "
+                         "second once steps overlap")
     ap.add_argument("--no-graph", action="store_true",
                     help="enqueue the operators one by one instead of replaying the HIP graph (used under rocprofv3 "
                          "--kernel-trace, whose tracer crashes inside hipGraphLaunch on this image)")
@@ -361,7 +387,7 @@ def main():
     # --in-flight copies of the function, each with its own stream and buffers, take the steps in turn: step i + 1
     # is enqueued while step i runs.  Every step is still one whole pass over one batch on one copy.
     pipe = nb.HipPipeline(0, qg, args.batch, depth=args.in_flight, capture_graph=not args.no_graph, lanes=args.lanes,
-                          fuse_blocks=not args.no_fuse_blocks)
+                          fuse_blocks=args.fuse_blocks)
     model = pipe.models[0]
     ctx = pipe.contexts[0]
     pipe.set_input(x)  # resident in HBM before the timed region
@@ -384,7 +410,7 @@ def main():
     # Kernels of concurrently replayed chains overlap and have no duration of their own, so the per-kernel figures
     # are taken on the one-chain recording of the same operators (every launch then covers the whole batch).
     kmodel = model if args.lanes == 1 else nb.HipModel(ctx, qg, args.batch, capture_graph=False, lanes=1,
-                                                        fuse_blocks=not args.no_fuse_blocks)
+                                                        fuse_blocks=args.fuse_blocks)
     if kmodel is not model:
         kmodel.set_input(x)
         kmodel.invoke()
@@ -415,7 +441,7 @@ def main():
         f = fams.setdefault(family(name), {"ms": 0.0, "bytes": 0, "floor": 0, "macs": 0, "launches": 0, "traffic": 0, "traffic_known": True})
         for k in ("ms", "bytes", "floor", "macs", "launches"):
             f[k] += g[k]
-        t = MEASURED_TRAFFIC_B64.get(name) if args.batch == 64 and not args.no_fuse_blocks else None
+        t = MEASURED_TRAFFIC_B64["fused" if args.fuse_blocks else "unfused"].get(name) if args.batch == 64 else None
         if t is None:
             f["traffic_known"] = False
         else:

@@ -326,12 +326,35 @@ struct __attribute__((packed, aligned(1))) U32Unaligned {
 // OWED says what acc still lacks: kOwesAll, the channel constant (read at cterm) and -zwp * rowsum; kOwesRows, only
 // -zwp_rows * rowsum; kOwesNothing.
 enum { kOwesAll = 0, kOwesRows = 1, kOwesNothing = 2 };
-template <int T, int OWED = kOwesAll>
+// PLAIN: the launch has been checked to need none of the options -- u8 output by the one-instruction requantisation
+// (Epilogue::fast and ::full), no byte table, no residual, whole groups of 4T channels, dword-aligned rows -- so the
+// tile is converted and stored without a single test of them.
+template <int T, int OWED = kOwesAll, bool PLAIN = false>
 __device__ __forceinline__ void igemm_store_tile(const IgemmArgs &a, const v4i (&acc)[T], int32_t rowsum, int p, int ch0, int gq,
                                                  const int32_t *cterm, const uint8_t *lutl) {
     if (!(p < a.m && ch0 < a.n)) return;
     const int32_t nrsz = OWED == kOwesAll ? -a.zwp * rowsum : (OWED == kOwesRows ? -a.zwp_rows * rowsum : 0);
     const size_t obase = (size_t)p * a.ldy + a.y_coff + ch0;
+    if constexpr (PLAIN) {
+        uint32_t *yo = reinterpret_cast<uint32_t *>(reinterpret_cast<uint8_t *>(a.y) + obase);
+        uint32_t packed[T];
+#pragma unroll
+        for (int nt = 0; nt < T; nt++) {
+            v4i ct = {0, 0, 0, 0};
+            if (OWED == kOwesAll) ct = *reinterpret_cast<const v4i *>(cterm + gq * (4 * T) + nt * 4);
+            int32_t v[4];
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                v[r] = OWED == kOwesAll ? add3(acc[nt][r], ct[r], nrsz) : (OWED == kOwesRows ? acc[nt][r] + nrsz : acc[nt][r]);
+            packed[nt] = requant4_u8_packed_direct(v, a.ep);
+        }
+#pragma unroll
+        for (int nt = 0; nt + 4 <= T; nt += 4)
+            *reinterpret_cast<u32x4_a4 *>(yo + nt) = u32x4_a4{packed[nt], packed[nt + 1], packed[nt + 2], packed[nt + 3]};
+#pragma unroll
+        for (int nt = T / 4 * 4; nt < T; nt++) yo[nt] = packed[nt];
+        return;
+    }
     if (a.ep.out_mode == kOutU8) {
         uint8_t *yo = reinterpret_cast<uint8_t *>(a.y) + obase;
         uint32_t packed[T];
@@ -421,7 +444,7 @@ __device__ __forceinline__ void igemm_store_tile(const IgemmArgs &a, const v4i (
 
 // Blocks per compute unit the register allocation has to leave room for: four (at most 128 registers) for the
 // shapes that fit comfortably, so that the scheduler does not trade the occupancy away for longer live ranges.
-template <int T, int RG, int MODE>
+template <int T, int RG, int MODE, bool PLAIN = false>
 __global__ void __launch_bounds__(kThreads, ((RG == 1 && T <= 12) || loads_rows(MODE)) ? 4 : 2) qconv_igemm_kernel(const IgemmArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     int32_t *cterm = reinterpret_cast<int32_t *>(smem); // [T * 16]
@@ -603,11 +626,11 @@ __global__ void __launch_bounds__(kThreads, ((RG == 1 && T <= 12) || loads_rows(
         if (a.zwp_rows != 0) {
 #pragma unroll
             for (int rg = 0; rg < RG; rg++)
-                igemm_store_tile<T, kOwesRows>(a, acc[rg], rs[rg][0], mt * pix_per_block + (wave * RG + rg) * 16 + j, ch0, gq, cterm, lutl);
+                igemm_store_tile<T, kOwesRows, PLAIN>(a, acc[rg], rs[rg][0], mt * pix_per_block + (wave * RG + rg) * 16 + j, ch0, gq, cterm, lutl);
         } else {
 #pragma unroll
             for (int rg = 0; rg < RG; rg++)
-                igemm_store_tile<T, kOwesNothing>(a, acc[rg], 0, mt * pix_per_block + (wave * RG + rg) * 16 + j, ch0, gq, cterm, lutl);
+                igemm_store_tile<T, kOwesNothing, PLAIN>(a, acc[rg], 0, mt * pix_per_block + (wave * RG + rg) * 16 + j, ch0, gq, cterm, lutl);
         }
 #pragma unroll
         for (int rg = 0; rg < RG; rg++) pcur[rg] = pnxt[rg];
@@ -779,7 +802,15 @@ template <int T, int RG, int MODE> int launch_trg(nncase_hip_ctx *ctx, const Ige
     // one XCD and find the activations in its L2.
     if (nchunks > 1) gx = ceil_div(gx, 8) * 8;
     const size_t lds = (size_t)T * 16 * sizeof(int32_t) + 256 + (size_t)a.kc_steps * T * 1024;
-    hipLaunchKernelGGL((qconv_igemm_kernel<T, RG, MODE>), dim3(gx, nchunks, 1), dim3(kThreads), lds, ctx->stream, args);
+    // the 1x1 row loaders are also built without the epilogue's options (see igemm_store_tile)
+    bool plain = false;
+    if constexpr (loads_rows(MODE))
+        plain = a.ep.out_mode == kOutU8 && a.ep.fast && a.ep.full && !a.lut && !a.rep.res && a.n % (4 * T) == 0 && ((a.ldy | a.y_coff) & 3) == 0;
+    if (plain) {
+        if constexpr (loads_rows(MODE))
+            hipLaunchKernelGGL((qconv_igemm_kernel<T, RG, MODE, true>), dim3(gx, nchunks, 1), dim3(kThreads), lds, ctx->stream, args);
+    } else
+        hipLaunchKernelGGL((qconv_igemm_kernel<T, RG, MODE>), dim3(gx, nchunks, 1), dim3(kThreads), lds, ctx->stream, args);
     NNHIP_LAUNCH_CHECK(ctx, "qconv_igemm_kernel");
     return 0;
 }
