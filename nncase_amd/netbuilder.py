@@ -429,8 +429,7 @@ class HipModel:
                 # the epilogue's arithmetic cost, on 7x7 maps (and at small batches) a workgroup per tile leaves most
                 # of the device idle and the three latency-bound launches are quicker.
                 tiles = -(-d.out_shape[1] // 7) * -(-d.out_shape[2] // 7)        # 7x7 output tiles per image
-                largest = fuse_blocks if isinstance(fuse_blocks, int) and not isinstance(fuse_blocks, bool) else 784
-                if fuse_blocks != "all" and not (d.out_shape[1] * d.out_shape[2] >= 196 and e.out_shape[1] * e.out_shape[2] <= largest
+                if fuse_blocks != "all" and not (d.out_shape[1] * d.out_shape[2] >= 196 and e.out_shape[1] * e.out_shape[2] <= 784
                                                  and (batch // lanes) * tiles >= 64):
                     continue
                 self.blocks[i] = (i + 1, i + 2, addn)
