@@ -117,6 +117,20 @@ NNCASE_HIP_API int nncase_hip_quantize(nncase_hip_ctx_t *ctx, const void *in_dev
 NNCASE_HIP_API int nncase_hip_dequantize(nncase_hip_ctx_t *ctx, const void *in_dev, int in_dtype, void *out_dev,
                                          int out_dtype, size_t count, nncase_hip_quant_param_t qp);
 
+/* The same two operators on strided operands, as the reference's kernels take them
+ * (in_shape, in_strides, out_strides; reference/quantize.cpp:29-47, dequantize.cpp:29-44,
+ * called with the tensors' own strides from tensor_ops.cpp:268-283,681-695): element `index`
+ * is read at sum(index[d] * in_strides[d]) and written at sum(index[d] * out_strides[d]),
+ * strides in elements, rank 1..6.  Elements the output strides skip are left untouched. */
+NNCASE_HIP_API int nncase_hip_quantize_strided(nncase_hip_ctx_t *ctx, const void *in_dev, int in_dtype, void *out_dev,
+                                               int out_dtype, int32_t rank, const int64_t *shape,
+                                               const int64_t *in_strides, const int64_t *out_strides,
+                                               nncase_hip_quant_param_t qp);
+NNCASE_HIP_API int nncase_hip_dequantize_strided(nncase_hip_ctx_t *ctx, const void *in_dev, int in_dtype, void *out_dev,
+                                                 int out_dtype, int32_t rank, const int64_t *shape,
+                                                 const int64_t *in_strides, const int64_t *out_strides,
+                                                 nncase_hip_quant_param_t qp);
+
 /* ---- u8/u8 convolution and matmul --------------------------------------
  *
  * acc[p, oc] = bias[oc] + sum_{ky,kx,ic} (x - zx) * (w - zw)          (int32)

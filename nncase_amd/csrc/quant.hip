@@ -125,6 +125,54 @@ __global__ __launch_bounds__(kEwThreads) void dequantize_kernel(const TQ *__rest
     for (size_t j = nvec * kEwVec + tid; j < count; j += nthreads) out[j] = from_f32<TOut>(((float)in[j] - bias) * scale);
 }
 
+// Strided forms: element `index` of a tensor of `rank` dimensions is read at sum(index[d] * in_strides[d]) and
+// written at sum(index[d] * out_strides[d]) (strides in elements), as the reference's kernels address their
+// operands (apply(in_shape, ...) with offset(strides, index), reference/quantize.cpp:36-47, dequantize.cpp:36-44).
+// One element per thread and trip, innermost dimension fastest, so dense inner rows still coalesce.
+constexpr int kMaxStridedRank = 6;
+struct StridedArgs {
+    int rank;
+    uint32_t count;
+    FastDiv dim[kMaxStridedRank];          // innermost first
+    uint32_t in_stride[kMaxStridedRank];   // innermost first
+    uint32_t out_stride[kMaxStridedRank];
+};
+
+__device__ __forceinline__ void strided_offsets(const StridedArgs &a, uint32_t i, uint32_t *in_off, uint32_t *out_off) {
+    uint32_t io = 0, oo = 0;
+#pragma unroll
+    for (int d = 0; d < kMaxStridedRank; d++) {
+        if (d < a.rank) {
+            const uint32_t q = fastdiv(i, a.dim[d]);
+            const uint32_t r = i - q * a.dim[d].div;
+            io += r * a.in_stride[d];
+            oo += r * a.out_stride[d];
+            i = q;
+        }
+    }
+    *in_off = io, *out_off = oo;
+}
+
+template <typename TIn, typename TQ>
+__global__ __launch_bounds__(kEwThreads) void quantize_strided_kernel(const TIn *__restrict__ in, TQ *__restrict__ out, const StridedArgs a,
+                                                                      float scale, float bias) {
+    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < a.count; i += gridDim.x * blockDim.x) {
+        uint32_t io, oo;
+        strided_offsets(a, i, &io, &oo);
+        out[oo] = quantize_one<TQ>(to_f32(in[io]), scale, bias);
+    }
+}
+
+template <typename TQ, typename TOut>
+__global__ __launch_bounds__(kEwThreads) void dequantize_strided_kernel(const TQ *__restrict__ in, TOut *__restrict__ out, const StridedArgs a,
+                                                                        float scale, float bias) {
+    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < a.count; i += gridDim.x * blockDim.x) {
+        uint32_t io, oo;
+        strided_offsets(a, i, &io, &oo);
+        out[oo] = from_f32<TOut>(((float)in[io] - bias) * scale);
+    }
+}
+
 // out = Q(clamp(DQ(a) + DQ(b))) on bytes; the clamp and the u8 saturation are folded into
 // one clamp on the requantised value, the division is the exact FMA form (see qconv.hpp).
 __global__ __launch_bounds__(kEwThreads) void qadd_kernel(const uint8_t *__restrict__ a, const uint8_t *__restrict__ b,
@@ -242,6 +290,38 @@ int launch_dequantize(nncase_hip_ctx *ctx, const void *in, void *out, size_t cou
     return 0;
 }
 
+// Validates a strided operand pair and fills the kernel's arguments.  *dense is set when both sides are the
+// plain row-major layout of the shape (the caller then takes the vector kernels).
+int make_strided(nncase_hip_ctx *ctx, const char *what, int32_t rank, const int64_t *shape, const int64_t *in_strides,
+                 const int64_t *out_strides, StridedArgs *a, bool *dense) {
+    NNHIP_REQUIRE(ctx, rank >= 1 && rank <= kMaxStridedRank, -EINVAL, "%s: rank %d (1..%d are supported)", what, rank, kMaxStridedRank);
+    NNHIP_REQUIRE(ctx, shape && in_strides && out_strides, -EINVAL, "%s: null shape or strides", what);
+    memset(a, 0, sizeof(*a));
+    a->rank = rank;
+    int64_t count = 1, in_extent = 0, out_extent = 0, row_major = 1;
+    *dense = true;
+    for (int d = rank - 1; d >= 0; d--) { // innermost first
+        NNHIP_REQUIRE(ctx, shape[d] >= 0 && in_strides[d] >= 0 && out_strides[d] >= 0, -EINVAL, "%s: negative extent or stride", what);
+        NNHIP_REQUIRE(ctx, shape[d] < ((int64_t)1 << 31) && in_strides[d] < ((int64_t)1 << 31) && out_strides[d] < ((int64_t)1 << 31),
+                      -EINVAL, "%s: extent or stride of 2^31 or more", what);
+        count *= shape[d];
+        NNHIP_REQUIRE(ctx, count < ((int64_t)1 << 31), -EINVAL, "%s: 2^31 elements or more", what);
+        if (shape[d] > 0) {
+            in_extent += (shape[d] - 1) * in_strides[d];
+            out_extent += (shape[d] - 1) * out_strides[d];
+        }
+        NNHIP_REQUIRE(ctx, in_extent < ((int64_t)1 << 31) && out_extent < ((int64_t)1 << 31), -EINVAL, "%s: operand spans 2^31 elements or more", what);
+        const int k = rank - 1 - d;
+        a->dim[k] = make_fastdiv((uint32_t)std::max<int64_t>(shape[d], 1));
+        a->in_stride[k] = (uint32_t)in_strides[d];
+        a->out_stride[k] = (uint32_t)out_strides[d];
+        if (shape[d] != 1 && (in_strides[d] != row_major || out_strides[d] != row_major)) *dense = false;
+        row_major *= shape[d];
+    }
+    a->count = (uint32_t)count;
+    return 0;
+}
+
 } // namespace nnhip
 
 using namespace nnhip;
@@ -287,6 +367,69 @@ extern "C" int nncase_hip_dequantize(nncase_hip_ctx_t *ctx, const void *in_dev, 
 #undef NNHIP_DQ_CASE
     return fail(ctx, -NNCASE_HIP_ERR_DATATYPE_MISMATCH, "dequantize: unsupported types in=0x%x out=0x%x", in_dtype,
                 out_dtype);
+}
+
+extern "C" int nncase_hip_quantize_strided(nncase_hip_ctx_t *ctx, const void *in_dev, int in_dtype, void *out_dev, int out_dtype,
+                                           int32_t rank, const int64_t *shape, const int64_t *in_strides, const int64_t *out_strides,
+                                           nncase_hip_quant_param_t qp) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, qp.scale != 0.f, -EINVAL, "quantize: scale is zero");
+    StridedArgs a;
+    bool dense;
+    const int rc = make_strided(ctx, "quantize", rank, shape, in_strides, out_strides, &a, &dense);
+    if (rc) return rc;
+    if (a.count == 0) return 0;
+    NNHIP_REQUIRE(ctx, in_dev && out_dev, -EINVAL, "quantize: null buffer");
+    if (dense) return nncase_hip_quantize(ctx, in_dev, in_dtype, out_dev, out_dtype, a.count, qp);
+    const float bias = (float)qp.zero_point;
+    const int grid = ew_grid(ctx, a.count);
+#define NNHIP_QS_CASE(IN_DT, TIn, OUT_DT, TQ)                                                                          \
+    if (in_dtype == IN_DT && out_dtype == OUT_DT) {                                                                    \
+        hipLaunchKernelGGL((quantize_strided_kernel<TIn, TQ>), dim3(grid), dim3(kEwThreads), 0, ctx->stream,           \
+                           (const TIn *)in_dev, (TQ *)out_dev, a, qp.scale, bias);                                     \
+        NNHIP_LAUNCH_CHECK(ctx, "quantize_strided_kernel");                                                            \
+        return 0;                                                                                                      \
+    }
+    NNHIP_QS_CASE(NNCASE_HIP_DT_F32, float, NNCASE_HIP_DT_U8, uint8_t)
+    NNHIP_QS_CASE(NNCASE_HIP_DT_F32, float, NNCASE_HIP_DT_I8, int8_t)
+    NNHIP_QS_CASE(NNCASE_HIP_DT_F32, float, NNCASE_HIP_DT_I16, int16_t)
+    NNHIP_QS_CASE(NNCASE_HIP_DT_F16, __half, NNCASE_HIP_DT_U8, uint8_t)
+    NNHIP_QS_CASE(NNCASE_HIP_DT_F16, __half, NNCASE_HIP_DT_I8, int8_t)
+    NNHIP_QS_CASE(NNCASE_HIP_DT_F16, __half, NNCASE_HIP_DT_I16, int16_t)
+#undef NNHIP_QS_CASE
+    return fail(ctx, -NNCASE_HIP_ERR_DATATYPE_MISMATCH, "quantize: unsupported types in=0x%x out=0x%x", in_dtype, out_dtype);
+}
+
+extern "C" int nncase_hip_dequantize_strided(nncase_hip_ctx_t *ctx, const void *in_dev, int in_dtype, void *out_dev, int out_dtype,
+                                             int32_t rank, const int64_t *shape, const int64_t *in_strides, const int64_t *out_strides,
+                                             nncase_hip_quant_param_t qp) {
+    NNHIP_CHECK_CTX(ctx);
+    StridedArgs a;
+    bool dense;
+    const int rc = make_strided(ctx, "dequantize", rank, shape, in_strides, out_strides, &a, &dense);
+    if (rc) return rc;
+    if (a.count == 0) return 0;
+    NNHIP_REQUIRE(ctx, in_dev && out_dev, -EINVAL, "dequantize: null buffer");
+    if (dense) return nncase_hip_dequantize(ctx, in_dev, in_dtype, out_dev, out_dtype, a.count, qp);
+    const float bias = (float)qp.zero_point;
+    const int grid = ew_grid(ctx, a.count);
+#define NNHIP_DQS_CASE(IN_DT, TQ, OUT_DT, TOut)                                                                        \
+    if (in_dtype == IN_DT && out_dtype == OUT_DT) {                                                                    \
+        hipLaunchKernelGGL((dequantize_strided_kernel<TQ, TOut>), dim3(grid), dim3(kEwThreads), 0, ctx->stream,        \
+                           (const TQ *)in_dev, (TOut *)out_dev, a, qp.scale, bias);                                    \
+        NNHIP_LAUNCH_CHECK(ctx, "dequantize_strided_kernel");                                                          \
+        return 0;                                                                                                      \
+    }
+    NNHIP_DQS_CASE(NNCASE_HIP_DT_U8, uint8_t, NNCASE_HIP_DT_F32, float)
+    NNHIP_DQS_CASE(NNCASE_HIP_DT_I8, int8_t, NNCASE_HIP_DT_F32, float)
+    NNHIP_DQS_CASE(NNCASE_HIP_DT_I16, int16_t, NNCASE_HIP_DT_F32, float)
+    NNHIP_DQS_CASE(NNCASE_HIP_DT_I32, int32_t, NNCASE_HIP_DT_F32, float)
+    NNHIP_DQS_CASE(NNCASE_HIP_DT_U8, uint8_t, NNCASE_HIP_DT_F16, __half)
+    NNHIP_DQS_CASE(NNCASE_HIP_DT_I8, int8_t, NNCASE_HIP_DT_F16, __half)
+    NNHIP_DQS_CASE(NNCASE_HIP_DT_I16, int16_t, NNCASE_HIP_DT_F16, __half)
+    NNHIP_DQS_CASE(NNCASE_HIP_DT_I32, int32_t, NNCASE_HIP_DT_F16, __half)
+#undef NNHIP_DQS_CASE
+    return fail(ctx, -NNCASE_HIP_ERR_DATATYPE_MISMATCH, "dequantize: unsupported types in=0x%x out=0x%x", in_dtype, out_dtype);
 }
 
 extern "C" int nncase_hip_qadd(nncase_hip_ctx_t *ctx, const uint8_t *a_dev, nncase_hip_quant_param_t a_qp,

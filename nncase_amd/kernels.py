@@ -33,29 +33,66 @@ def _ctx(ctx):
     return ctx or default_context()
 
 
-def quantize(input: np.ndarray, quant_param: QuantParam, out_dtype=np.uint8, ctx: Context = None) -> np.ndarray:
-    """kernels::stackvm::quantize(out_type, input, quant_param)."""
+def _span(a: np.ndarray):
+    """(first byte, byte count, strides in elements) of the memory a strided view covers; None for views the
+    strided entry points do not take (negative or unaligned strides)."""
+    if a.size == 0:
+        return None
+    if any(st < 0 or st % a.itemsize for st in a.strides):
+        return None
+    nbytes = sum((n - 1) * st for n, st in zip(a.shape, a.strides)) + a.itemsize
+    return a.__array_interface__["data"][0], nbytes, [st // a.itemsize for st in a.strides]
+
+
+def _elementwise_strided(c: Context, call, x: np.ndarray, out: Optional[np.ndarray], out_dtype: np.dtype, qp_):
+    """Runs a strided quantize / dequantize: the operands' memory spans are mirrored on the device, so elements the
+    strides skip keep their values, as with the reference's kernels on strided tensors."""
+    import ctypes
+    xs = _span(x)
+    if out is None:
+        out = np.empty(x.shape, out_dtype)
+    os_ = _span(out)
+    if xs is None or os_ is None or out.shape != x.shape or out.dtype != out_dtype or not out.flags.writeable:
+        raise rt.HipError(-22, "strided operand", "views need non-negative element-aligned strides, equal shapes and a writable output")
+    src = c.to_device(np.frombuffer((ctypes.c_char * xs[1]).from_address(xs[0]), np.uint8))
+    host_out = np.frombuffer((ctypes.c_char * os_[1]).from_address(os_[0]), np.uint8)
+    dst = c.to_device(host_out)
+    call(src, rt.NP_TO_DT[x.dtype], dst, rt.NP_TO_DT.get(out_dtype, 0xFF), x.shape, xs[2], os_[2], qp_)
+    host_out[:] = dst.download((os_[1],), np.uint8)
+    return out
+
+
+def quantize(input: np.ndarray, quant_param: QuantParam, out_dtype=np.uint8, ctx: Context = None,
+             out: Optional[np.ndarray] = None) -> np.ndarray:
+    """kernels::stackvm::quantize(out_type, input, quant_param).  A strided view as `input`, or a strided `out` to
+    write into, goes through the strided entry point with the views' own strides, like the reference's call
+    (tensor_ops.cpp:690-693 passes input_tensor->strides() and output_tensor->strides())."""
     c = _ctx(ctx)
-    x = np.asarray(input, order="C")
+    x = np.asarray(input)
     if x.dtype not in (np.float32, np.float16):
         raise rt.HipError(-rt.ERR_DATATYPE_MISMATCH, "quantize", f"input dtype {x.dtype}")
     out_dtype = np.dtype(out_dtype)
     if x.size == 0:
-        return np.empty(x.shape, out_dtype)
+        return np.empty(x.shape, out_dtype) if out is None else out
+    if out is not None or not x.flags.c_contiguous:
+        return _elementwise_strided(c, c.quantize_strided, x, out, out_dtype, quant_param)
     src, dst = c.to_device(x), c.alloc(x.size * out_dtype.itemsize)
     c.quantize(src, rt.NP_TO_DT[x.dtype], dst, rt.NP_TO_DT.get(out_dtype, 0xFF), x.size, quant_param)
     return dst.download(x.shape, out_dtype)
 
 
-def dequantize(input: np.ndarray, quant_param: QuantParam, out_dtype=np.float32, ctx: Context = None) -> np.ndarray:
-    """kernels::stackvm::dequantize(out_type, input, quant_param)."""
+def dequantize(input: np.ndarray, quant_param: QuantParam, out_dtype=np.float32, ctx: Context = None,
+               out: Optional[np.ndarray] = None) -> np.ndarray:
+    """kernels::stackvm::dequantize(out_type, input, quant_param); strided operands as for quantize."""
     c = _ctx(ctx)
-    q = np.asarray(input, order="C")
+    q = np.asarray(input)
     out_dtype = np.dtype(out_dtype)
     if q.dtype not in rt.NP_TO_DT:
         raise rt.HipError(-rt.ERR_DATATYPE_MISMATCH, "dequantize", f"input dtype {q.dtype}")
     if q.size == 0:
-        return np.empty(q.shape, out_dtype)
+        return np.empty(q.shape, out_dtype) if out is None else out
+    if out is not None or not q.flags.c_contiguous:
+        return _elementwise_strided(c, c.dequantize_strided, q, out, out_dtype, quant_param)
     src, dst = c.to_device(q), c.alloc(q.size * out_dtype.itemsize)
     c.dequantize(src, rt.NP_TO_DT[q.dtype], dst, rt.NP_TO_DT.get(out_dtype, 0xFF), q.size, quant_param)
     return dst.download(q.shape, out_dtype)
@@ -117,24 +154,60 @@ def conv2d(input: np.ndarray, weights: np.ndarray, bias: Optional[np.ndarray], s
 def mat_mul(lhs: np.ndarray, rhs: np.ndarray, lhs_qp: QuantParam, rhs_qp: QuantParam,
             output_qp: Optional[QuantParam] = None, out_dtype=np.float32, bias: Optional[np.ndarray] = None,
             fused_clamp: Tuple[float, float] = (-rt.FLT_MAX, rt.FLT_MAX), ctx: Context = None) -> np.ndarray:
-    """kernels::stackvm::mat_mul(lhs, rhs) on u8 operands: lhs [..., M, K] (batch dims are
-    flattened into rows), rhs [K, N] constant."""
+    """kernels::stackvm::mat_mul(lhs, rhs) on u8 operands with the reference's operand forms
+    (reference/matmul.cpp:28-48): rank-1 operands are a row / a column, both operands may carry up to two batch
+    dimensions (rank <= 4) which broadcast against each other where one of them is 1.  lhs [..., M, K] against a
+    plain [K, N] matrix is one launch (the batch is stacked into rows); otherwise every distinct rhs matrix is
+    pre-packed once and serves all the lhs matrices it is paired with."""
     c = _ctx(ctx)
     a = np.ascontiguousarray(lhs, np.uint8)
     b = np.ascontiguousarray(rhs, np.uint8)
-    if b.ndim != 2 or a.ndim < 1 or a.shape[-1] != b.shape[0]:
+    if a.ndim < 1 or b.ndim < 1 or a.ndim > 4 or b.ndim > 4:
         raise rt.HipError(-rt.ERR_SHAPE_MISMATCH, "mat_mul", f"{a.shape} x {b.shape}")
-    k, n = b.shape
-    lead = a.shape[:-1]
-    m = int(np.prod(lead)) if lead else 1
+    a1, b1 = a.ndim == 1, b.ndim == 1
+    if a1:
+        a = a[None, :]
+    if b1:
+        b = b[:, None]
+    if a.shape[-1] != b.shape[-2]:
+        raise rt.HipError(-rt.ERR_SHAPE_MISMATCH, "mat_mul", f"{np.shape(lhs)} x {np.shape(rhs)}")
     out_dtype = np.dtype(out_dtype)
-    wts = c.prepack_matmul(b, bias, rhs_qp, expected_rows=m)
-    da = c.to_device(a)
-    dy = c.alloc(max(1, m * n * out_dtype.itemsize))
-    args = rt.MatmulArgs(m, lhs_qp, output_qp or qp(0, 1.0), fused_clamp[0], fused_clamp[1], _out_dt(out_dtype))
-    c.qmatmul(da, wts, dy, args)
-    out = dy.download(tuple(lead) + (n,), out_dtype)
-    wts.destroy()
+    k, n = b.shape[-2:]
+
+    def run(a2d, wts):
+        m = a2d.shape[0]
+        dy = c.alloc(max(1, m * n * out_dtype.itemsize))
+        args = rt.MatmulArgs(m, lhs_qp, output_qp or qp(0, 1.0), fused_clamp[0], fused_clamp[1], _out_dt(out_dtype))
+        c.qmatmul(c.to_device(a2d), wts, dy, args)
+        return dy.download((m, n), out_dtype)
+
+    if b.ndim == 2:                                   # one constant matrix: every lhs row in one launch
+        lead = a.shape[:-1]
+        m = int(np.prod(lead)) if lead else 1
+        wts = c.prepack_matmul(b, bias, rhs_qp, expected_rows=m)
+        out = run(a.reshape(m, k), wts).reshape(tuple(lead) + (n,))
+        wts.destroy()
+    else:
+        ab, bb = a.shape[:-2], b.shape[:-2]
+        try:
+            batch = np.broadcast_shapes(ab, bb)
+        except ValueError:
+            raise rt.HipError(-rt.ERR_SHAPE_MISMATCH, "mat_mul", f"{np.shape(lhs)} x {np.shape(rhs)}") from None
+        m = a.shape[-2]
+        ai = np.broadcast_to(np.arange(int(np.prod(ab)) if ab else 1).reshape(ab), batch).ravel()
+        bi = np.broadcast_to(np.arange(int(np.prod(bb))).reshape(bb), batch).ravel()
+        amats, bmats = a.reshape(-1, m, k), b.reshape(-1, k, n)
+        out = np.empty((len(bi), m, n), out_dtype)
+        for j in np.unique(bi):                       # one pre-pack per distinct rhs matrix
+            sel = np.nonzero(bi == j)[0]
+            wts = c.prepack_matmul(np.ascontiguousarray(bmats[j]), bias, rhs_qp, expected_rows=m * len(sel))
+            out[sel] = run(np.ascontiguousarray(amats[ai[sel]]).reshape(-1, k), wts).reshape(len(sel), m, n)
+            wts.destroy()
+        out = out.reshape(tuple(batch) + (m, n))
+    if a1:
+        out = out.squeeze(-2)
+    if b1:
+        out = out.squeeze(-1)
     return out
 
 

@@ -82,6 +82,7 @@ class PagedAttnArgs(C.Structure):
 # name -> (restype, argtypes); every symbol include/nncase_hip.h declares
 _VP, _I, _SZ = C.c_void_p, C.c_int, C.c_size_t
 _I32P = C.POINTER(C.c_int32)
+_I64P = C.POINTER(C.c_int64)
 SYMBOLS = {
     "nncase_hip_version": (_I, []),
     "nncase_hip_ctx_create": (_I, [_I, C.POINTER(_VP)]),
@@ -98,6 +99,8 @@ SYMBOLS = {
     "nncase_hip_stream_sync": (_I, [_VP]),
     "nncase_hip_quantize": (_I, [_VP, _VP, _I, _VP, _I, _SZ, QuantParam]),
     "nncase_hip_dequantize": (_I, [_VP, _VP, _I, _VP, _I, _SZ, QuantParam]),
+    "nncase_hip_quantize_strided": (_I, [_VP, _VP, _I, _VP, _I, C.c_int32, _I64P, _I64P, _I64P, QuantParam]),
+    "nncase_hip_dequantize_strided": (_I, [_VP, _VP, _I, _VP, _I, C.c_int32, _I64P, _I64P, _I64P, QuantParam]),
     "nncase_hip_qconv2d_prepack": (_I, [_VP, C.POINTER(Conv2dDesc), _VP, _VP, C.POINTER(_VP)]),
     "nncase_hip_weights_destroy": (_I, [_VP, _VP]),
     "nncase_hip_weights_set_post_lut": (_I, [_VP, _VP, _VP, QuantParam]),
@@ -427,6 +430,18 @@ class Context:
     def dequantize(self, src: DeviceBuffer, in_dtype: int, dst: DeviceBuffer, out_dtype: int, count: int, q: QuantParam):
         self._check(self.lib.nncase_hip_dequantize(self.handle, src.ptr, in_dtype, dst.ptr, out_dtype, count, q),
                     "dequantize")
+
+    def _strided(self, fn, what, src, in_dtype, dst, out_dtype, shape, in_strides, out_strides, q):
+        rank = len(shape)
+        arr = lambda v: (C.c_int64 * max(rank, 1))(*[int(e) for e in v])
+        self._check(fn(self.handle, src.ptr, in_dtype, dst.ptr, out_dtype, rank, arr(shape), arr(in_strides), arr(out_strides), q), what)
+
+    def quantize_strided(self, src, in_dtype, dst, out_dtype, shape, in_strides, out_strides, q: QuantParam):
+        """Strides in elements, as the reference's kernels take them (reference/quantize.cpp:29-47)."""
+        self._strided(self.lib.nncase_hip_quantize_strided, "quantize_strided", src, in_dtype, dst, out_dtype, shape, in_strides, out_strides, q)
+
+    def dequantize_strided(self, src, in_dtype, dst, out_dtype, shape, in_strides, out_strides, q: QuantParam):
+        self._strided(self.lib.nncase_hip_dequantize_strided, "dequantize_strided", src, in_dtype, dst, out_dtype, shape, in_strides, out_strides, q)
 
     def prepack_conv2d(self, weights_oihw: np.ndarray, bias: Optional[np.ndarray], w_qp: QuantParam, groups: int = 1,
                        expected_pixels: int = 0) -> Weights:

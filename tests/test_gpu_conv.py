@@ -416,6 +416,33 @@ def test_matmul_batched_lhs_is_flattened(hip_ctx):
     assert got.shape == (2, 3, 6, 3) and np.array_equal(got, want)
 
 
+# reference/matmul.cpp:56-87: rank-1 operands become a row / a column, both operands are extended to four
+# dimensions and the two batch dimensions broadcast where one side has extent 1 (shapes from
+# tests/kernels/test_matmul.cpp's grid and ones where the rhs carries the batch)
+@pytest.mark.parametrize("ashape,bshape", [
+    ((3, 5), (5,)), ((5,), (5, 4)), ((5,), (5,)),
+    ((2, 3, 4, 5), (2, 3, 5, 6)), ((2, 1, 4, 5), (1, 3, 5, 6)), ((4, 5), (2, 3, 5, 6)), ((3, 4, 5), (1, 1, 5, 6)),
+    ((2, 3, 7, 70), (3, 70, 20)), ((1, 3, 16, 64), (2, 1, 64, 24)),
+])
+def test_matmul_two_sided_batches_and_vectors(hip_ctx, ashape, bshape):
+    rng = np.random.default_rng(sum(ashape) * 31 + sum(bshape))
+    a = rng.integers(0, 256, ashape, dtype=np.uint8)
+    b = rng.integers(0, 256, bshape, dtype=np.uint8)
+    za, zb = 17, 201
+    want = np.matmul(a.astype(np.int64) - za, b.astype(np.int64) - zb)          # numpy broadcasts the same way
+    got = K.mat_mul(a, b, qp(za, 0.02), qp(zb, 0.003), None, np.int32, ctx=hip_ctx)
+    assert got.shape == want.shape and np.array_equal(got, want)
+    gotf = K.mat_mul(a, b, qp(za, 0.02), qp(zb, 0.003), None, np.float32, ctx=hip_ctx)
+    assert np.array_equal(gotf, want.astype(f32) * (f32(0.02) * f32(0.003)))
+    # and against the float kernel of the reference restated in the oracle (its own batching), to 1e-3 relative
+    ref = O.matmul_f32(O.dequantize(a, 0.02, za), O.dequantize(b, 0.003, zb))
+    assert ref.shape == want.shape
+    assert np.abs(gotf - ref).max() <= 1e-3 * max(1.0, np.abs(ref).max())
+    with pytest.raises(rt.HipError) as e:
+        K.mat_mul(np.zeros((2, 3, 4, 5), np.uint8), np.zeros((3, 2, 5, 6), np.uint8), qp(0, 1.0), qp(0, 1.0), None, np.int32, ctx=hip_ctx)
+    assert e.value.code == -rt.ERR_SHAPE_MISMATCH
+
+
 def test_linearity_at_full_size(hip_ctx):
     """Size-independent check at a BASELINE-sized layer (56x56x24 -> 144, batch 32): with zero
     points 0, acc(x1 + x2) == acc(x1) + acc(x2), and acc(x, w = 1) is the per-pixel channel sum."""

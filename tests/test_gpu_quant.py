@@ -153,3 +153,64 @@ def test_qglobal_avgpool(hip_ctx, shape):
     x = rng.integers(0, 256, shape, dtype=np.uint8)
     got = K.global_average_pool(x, qp(5, 0.02), qp(9, 0.015), ctx=hip_ctx)
     assert np.array_equal(got[:, :, 0, 0], O.qglobal_avgpool(x, 5, 0.02, 9, 0.015))
+
+
+# ---- strided operands: the reference's kernels address both tensors through their strides
+# (reference/quantize.cpp:36-47, dequantize.cpp:36-44); views with gaps, transposes, broadcasts (stride 0 on the
+# input), rank 1..6, and an output view whose gaps must keep what they held.
+STRIDED_VIEWS = [
+    ("rows with gaps", lambda a: a[:, ::2, 1:9]),
+    ("transposed", lambda a: a.transpose(2, 0, 1)),
+    ("inner stride 3", lambda a: a[1, :, ::3]),
+    ("single row", lambda a: a[2, 3, :]),
+    ("rank 6", lambda a: a[:4, :6, :12].reshape(2, 2, 3, 2, 3, 4)[:, :, ::2, :, 1:, ::3]),
+    ("broadcast row", lambda a: np.broadcast_to(a[0, 0, :8], (5, 8))),
+]
+
+
+@pytest.mark.parametrize("name,view", STRIDED_VIEWS)
+def test_quantize_and_dequantize_strided_views(hip_ctx, name, view):
+    rng = np.random.default_rng(len(name))
+    base = ((rng.random((6, 10, 20), dtype=f32) - 0.3) * 9).astype(f32)
+    x = view(base)
+    assert not x.flags.c_contiguous or x.ndim == 1
+    for out_np, out_code in ((np.uint8, O.U8), (np.int16, O.I16)):
+        q = K.quantize(x, qp(37, 0.043), out_np, ctx=hip_ctx)
+        want = O.quantize(np.ascontiguousarray(x), 0.043, 37, out_code)
+        assert q.shape == x.shape and np.array_equal(q, want)
+    codes = view(rng.integers(0, 256, (6, 10, 20), dtype=np.uint8))
+    y = K.dequantize(codes, qp(131, 0.0123), np.float32, ctx=hip_ctx)
+    assert np.array_equal(y.view(np.uint32), O.dequantize(np.ascontiguousarray(codes), 0.0123, 131).view(np.uint32))
+
+
+def test_strided_output_keeps_the_elements_its_strides_skip(hip_ctx):
+    rng = np.random.default_rng(3)
+    x = ((rng.random((7, 5, 12), dtype=f32) - 0.5) * 6).astype(f32)
+    store = np.full((7, 11, 40), 0xAB, np.uint8)
+    out = store[:, 1::2, 3:39:3]                      # a [7, 5, 12] window into a larger tensor
+    got = K.quantize(x[:, ::-1][:, ::-1], qp(128, 0.02), np.uint8, ctx=hip_ctx, out=out)
+    assert got is out
+    want = O.quantize(x, 0.02, 128, O.U8)
+    assert np.array_equal(out, want)
+    mask = np.ones(store.shape, bool)
+    mask[:, 1::2, 3:39:3] = False
+    assert (store[mask] == 0xAB).all()                # nothing outside the window was touched
+    fstore = np.full((7, 5, 30), -7.5, f32)
+    fout = fstore[:, :, 2:26:2]
+    K.dequantize(want, qp(128, 0.02), np.float32, ctx=hip_ctx, out=fout)
+    assert np.array_equal(fout.view(np.uint32), O.dequantize(want, 0.02, 128).view(np.uint32))
+    assert (fstore[:, :, 0:2] == -7.5).all() and (fstore[:, :, 3:26:2] == -7.5).all() and (fstore[:, :, 26:] == -7.5).all()
+
+
+def test_strided_argument_checks(hip_ctx):
+    src, dst = hip_ctx.alloc(1024), hip_ctx.alloc(1024)
+    for shape, ins, outs, code in (((4,) * 7, (1,) * 7, (1,) * 7, -22),          # rank 7
+                                   ((4, 4), (4, -1), (4, 1), -22),               # negative stride
+                                   ((1 << 20, 1 << 12), (1 << 12, 1), (1 << 12, 1), -22)):   # 2^32 elements
+        with pytest.raises(rt.HipError) as e:
+            hip_ctx.quantize_strided(src, rt.DT_F32, dst, rt.DT_U8, shape, ins, outs, qp(0, 1.0))
+        assert e.value.code == code
+    with pytest.raises(rt.HipError) as e:
+        hip_ctx.dequantize_strided(src, rt.DT_F32, dst, rt.DT_U8, (4, 2), (4, 1), (2, 2), qp(0, 1.0))
+    assert e.value.code == -rt.ERR_DATATYPE_MISMATCH
+    hip_ctx.quantize_strided(src, rt.DT_F32, dst, rt.DT_U8, (0, 4), (4, 1), (4, 1), qp(0, 1.0))   # empty: nothing to do
