@@ -10,7 +10,7 @@
 //   op     144 B : u32 opcode, n_inputs; i32 inputs[8] (tensor indices, -1 = unused); i32 output; u32 reserved;
 //                  u64 rdata0, rdata1 (byte offsets into .rdata, all ones = none); i32 p[16]; f32 f[4]
 // Opcodes: 0 quantize, 1 dequantize, 2 conv2d, 3 add, 4 global_avgpool, 5 lut, 6 concat, 7 resize_nearest,
-// 8 maxpool, 9 pad_channels.  conv2d: rdata0 = weights (OIHW u8), rdata1 = bias (int32 per output channel);
+// 8 maxpool, 9 pad_channels, 10 reshape (the output tensor is the input's buffer under other extents).  conv2d: rdata0 = weights (OIHW u8), rdata1 = bias (int32 per output channel);
 // p = {out_channels, in_channels / groups, kernel_h, kernel_w, groups, stride_h, stride_w, dilation_h,
 // dilation_w, pad_h_before, pad_h_after, pad_w_before, pad_w_after, weights zero point};
 // f = {clamp_min, clamp_max, weights scale}.  A matmul is a 1x1 conv2d over [M, 1, 1, K].
@@ -47,6 +47,7 @@ internal enum HipOpcode : uint
     ResizeNearest = 7,
     MaxPool = 8,
     PadChannels = 9,
+    Reshape = 10,
 }
 
 internal sealed class HipFunctionBuilder : FunctionBuilder

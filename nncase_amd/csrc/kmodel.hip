@@ -66,7 +66,7 @@ constexpr uint32_t kModelIdentifier = 0x4B4D444C; // 'KMDL'
 constexpr uint32_t kModelVersion = 7;
 constexpr uint64_t kNoRdata = ~uint64_t(0);
 enum { kOpQuantize, kOpDequantize, kOpConv2d, kOpAdd, kOpGlobalAvgPool, kOpLut, kOpConcat, kOpResizeNearest, kOpMaxPool,
-       kOpPadChannels };
+       kOpPadChannels, kOpReshape };
 
 struct Span {
     const uint8_t *p = nullptr;
@@ -422,6 +422,8 @@ static int build_function(nncase_hip_ctx_t *ctx, Span text_span, Span rdata, nnc
         if (fused_add[k] >= 0 && fused_lut[k] >= 0) m->owns[ops[fused_lut[k]].output] = 2;
         if (block_head[k]) m->owns[ops[k].output] = m->owns[ops[k + 1].output] = 2;
     }
+    for (uint32_t k = 0; k < th.n_ops; k++) // a reshaped tensor is its input's buffer under other extents
+        if (ops[k].opcode == kOpReshape && !skipped[k]) m->owns[ops[k].output] = 2;
     for (uint32_t t = 0; t < th.n_tensors; t++) {
         if (m->owns[t] == 2) {
             m->owns[t] = 0;
@@ -628,6 +630,12 @@ static int build_function(nncase_hip_ctx_t *ctx, Span text_span, Span rdata, nnc
                                                     static_cast<uint8_t *>(m->buffers[dst]), (int)ti.dims[0], (int)ti.dims[1],
                                                     (int)ti.dims[2], (int)ti.dims[3], o.p[0], o.p[0], o.p[1], o.p[1], o.p[2], o.p[2],
                                                     o.p[2], o.p[2], tqp(in0), tqp(dst));
+            break;
+        case kOpReshape:
+            NNHIP_REQUIRE(ctx, ti.dtype == to.dtype && elems(in0) == elems(dst) && m->buffers[in0] && !is_output((int32_t)dst),
+                          -NNCASE_HIP_ERR_SHAPE_MISMATCH, "kmodel_load: op %u reshapes %zu elements into %zu", k, elems(in0), elems(dst));
+            m->buffers[dst] = m->buffers[in0];
+            rc = 0;
             break;
         case kOpPadChannels: {
             NNHIP_REQUIRE(ctx, ti.dtype == to.dtype && ti.dims[0] == to.dims[0] && ti.dims[1] == to.dims[1] &&

@@ -277,9 +277,9 @@ HIPF_TENSOR = struct.Struct("<6Iif")
 HIPF_OP = struct.Struct("<2I8iiI2Q16i4f")
 NO_RDATA = 0xFFFFFFFFFFFFFFFF
 (OP_QUANTIZE, OP_DEQUANTIZE, OP_CONV2D, OP_ADD, OP_GLOBAL_AVGPOOL, OP_LUT, OP_CONCAT, OP_RESIZE_NEAREST, OP_MAXPOOL,
- OP_PAD_CHANNELS) = range(10)
+ OP_PAD_CHANNELS, OP_RESHAPE) = range(11)
 OP_NAMES = ["quantize", "dequantize", "conv2d", "add", "global_avgpool", "lut", "concat", "resize_nearest", "maxpool",
-            "pad_channels"]
+            "pad_channels", "reshape"]
 assert HIPF_HEADER.size == 32 and HIPF_TENSOR.size == 32 and HIPF_OP.size == 144
 
 
@@ -423,6 +423,8 @@ def compile_quant_graph(qg, batch: int, stackvm_main: bool = False) -> bytes:
             ops.append(HipOp(OP_MAXPOOL, ins, tid, p=(n.pool[0], n.pool[1], n.pool[2])))
         elif n.op == "padc":
             ops.append(HipOp(OP_PAD_CHANNELS, ins, tid))
+        elif n.op == "fold2":      # the same NHWC bytes with other extents: the tensor shares its input's buffer
+            ops.append(HipOp(OP_RESHAPE, ins, tid))
         else:
             raise ValueError(f"cannot serialise operator {n.op!r}")
     first_out = len(tensors)

@@ -334,6 +334,21 @@ def pad_small_channel_convs(qg: QuantGraph) -> QuantGraph:
             wpad = np.full((n.weights.shape[0], 4) + n.weights.shape[2:], n.w_qp[0], np.uint8)
             wpad[:, :c] = n.weights
             n.weights, n.inputs = wpad, (len(nodes) - 1,)
+            # Stride 2 along the width over an even window: two neighbouring 4-channel pixels are one 8-channel pixel
+            # of the half-width image in the same NHWC bytes ("fold2": nothing moves), and the conv becomes one of
+            # stride 1 along the width over half as many taps: out(y, x) = sum over ky, kx', (dx, c) of
+            # in[sy y + ky - ph][2 (x + kx' - pw / 2) + dx][c] w[ky][2 kx' + dx][c].  The loader then fetches 8 bytes
+            # per tap instead of 4 and computes half as many tap addresses.
+            kh, kw = n.weights.shape[2:]
+            (ph0, ph1), (pw0, pw1) = n.padding
+            if n.stride[1] == 2 and kw % 2 == 0 and w % 2 == 0 and pw0 % 2 == 0 and pw1 % 2 == 0:
+                nodes.append(QNode("fold2", (len(nodes) - 1,), n.name + ".fold2", src.out_qp, (8, h, w // 2)))
+                wf = np.empty((wpad.shape[0], 8, kh, kw // 2), np.uint8)
+                for dx in range(2):
+                    wf[:, dx * 4:dx * 4 + 4] = wpad[:, :, :, dx::2]
+                n.weights, n.inputs = wf, (len(nodes) - 1,)
+                n.stride = (n.stride[0], 1)
+                n.padding = ((ph0, ph1), (pw0 // 2, pw1 // 2))
         nodes.append(n)
         remap[i] = len(nodes) - 1
     outs = None if qg.outputs is None else [remap[j] for j in qg.outputs]
@@ -444,6 +459,9 @@ class HipModel:
             if i in fused_tail:
                 self.buffers.append(self.buffers[i - 1])  # written by the operator it is fused into
                 continue
+            if n.op == "fold2":
+                self.buffers.append(self.buffers[n.inputs[0]])  # the same bytes read as half as many, twice as deep pixels
+                continue
             if i in self.blocks or i - 1 in self.blocks:
                 self.buffers.append(ctx.alloc(16))        # the expanded tensors of a fused block live in LDS only
             else:
@@ -548,6 +566,8 @@ class HipModel:
             elif n.op == "padc":
                 src = qg.nodes[n.inputs[0]]
                 self.fn.add_pack(B(n.inputs[0]), buf, 1, [bl, hh, ww, src.out_shape[0]], [3], [cc])
+            elif n.op == "fold2":
+                continue
             elif n.op == "gap":
                 src = qg.nodes[n.inputs[0]]
                 self.fn.add_qglobal_avgpool(B(n.inputs[0]), buf, bl, src.out_shape[1], src.out_shape[2],

@@ -60,6 +60,10 @@ def run_integer(qg, x_nhwc: np.ndarray, keep_all: bool = False):
         elif n.op == "padc":
             v = outs[n.inputs[0]]
             y = np.pad(v, ((0, 0), (0, n.out_shape[0] - v.shape[1]), (0, 0), (0, 0)))
+        elif n.op == "fold2":     # pixel pairs along the width become channels: y[:, dx * C + c, :, x] = v[:, c, :, 2 x + dx]
+            v = outs[n.inputs[0]]
+            nb_, c_, h_, w_ = v.shape
+            y = np.ascontiguousarray(v.reshape(nb_, c_, h_, w_ // 2, 2).transpose(0, 4, 1, 2, 3).reshape(nb_, 2 * c_, h_, w_ // 2))
         else:
             raise ValueError(n.op)
         outs.append(y)
@@ -103,6 +107,10 @@ def run_float_chain(qg, x_nhwc: np.ndarray, keep_all: bool = False):
         elif n.op == "padc":
             v = outs[n.inputs[0]]
             y = np.pad(v, ((0, 0), (0, n.out_shape[0] - v.shape[1]), (0, 0), (0, 0)))
+        elif n.op == "fold2":     # pixel pairs along the width become channels: y[:, dx * C + c, :, x] = v[:, c, :, 2 x + dx]
+            v = outs[n.inputs[0]]
+            nb_, c_, h_, w_ = v.shape
+            y = np.ascontiguousarray(v.reshape(nb_, c_, h_, w_ // 2, 2).transpose(0, 4, 1, 2, 3).reshape(nb_, 2 * c_, h_, w_ // 2))
         else:
             raise ValueError(n.op)
         outs.append(y)
