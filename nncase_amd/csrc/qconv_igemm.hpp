@@ -637,6 +637,141 @@ __global__ void __launch_bounds__(kThreads, ((RG == 1 && T <= 12) || loads_rows(
     }
 }
 
+// ---- 1x1 convolutions over a multiple of 16 channels whose epilogue needs none of the options ----
+// The same implicit GEMM with everything that a pixel row does not need taken out of the loop: the activation
+// operand of (pixel, k-step) is 16 bytes at pixel * ldx + k-step * 64 + quad * 16, fetched by a buffer load whose
+// vector offset (the pixel's) is computed once per tile and whose scalar offset is the k-step; it is used as loaded
+// (one xor per dword makes it s8): reduction indices past K meet zero weights, and the row sum the weight zero point
+// multiplies comes from a ones operand that is zero past K, so nothing is masked; pixels past M are computed on a
+// clamped address and not stored.  The first k-step of a tile starts the sums from the channel constants (the
+// accumulator operand of the first product), so they are not copied.  One slice per pixel group is in flight ahead
+// of the products.  ROWS: the epilogue still owes -zw' * (sum of x'); false where the weights carry that term
+// (reductions of at most 32: the lanes of the upper half of the only k-step then re-read the pixel's bytes).
+template <int T, int RG, bool ROWS> __global__ void __launch_bounds__(kThreads, 4) qconv_rows_kernel(const IgemmArgs a) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    int32_t *cterm = reinterpret_cast<int32_t *>(smem); // [T * 16]
+    uint8_t *wlds = smem + T * 16 * sizeof(int32_t);    // [ksteps][T][1024]
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int j = lane & 15, gq = lane >> 4;
+    const int chunk = blockIdx.y;
+    const int ch_base = chunk * (T * 16);
+    const int KS = a.ksteps;
+    const __amdgpu_buffer_rsrc_t xres = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(a.x), 0, (int)a.x_bytes, 0x00020000);
+
+    // constants and the chunk's weights -> LDS
+    static_assert(T * 16 <= kThreads, "one constant per thread");
+    if ((int)threadIdx.x < T * 16) {
+        const int ch = ch_base + threadIdx.x;
+        cterm[threadIdx.x] = ch < a.n ? a.bias[ch] - a.zxp * a.wsum[ch] + a.k * a.zxp * a.zwp : 0;
+    }
+    {
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(a.wpk + (size_t)chunk * KS * T * 1024);
+        u32x4 *dst = reinterpret_cast<u32x4 *>(wlds);
+        const int n = KS * T * 64;
+        for (int i = threadIdx.x; i < n; i += 4 * kThreads) {
+            u32x4 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+                if (i + u * kThreads < n) v[u] = src[i + u * kThreads];
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+                if (i + u * kThreads < n) dst[i + u * kThreads] = v[u];
+        }
+    }
+
+    // this lane's 16-byte slice of a pixel row: full k-steps take (k-step * 4 + quad), the last one may end before
+    // the quad's slice (then the slice re-reads the row's first bytes and meets zero weights and a zero ones operand)
+    const int last = KS - 1;
+    const int tail_chunk = (last * 4 + gq) & a.kc_mask;
+    const bool tail_in_k = tail_chunk * 16 < a.k;
+    const uint32_t tail_off = tail_in_k ? (uint32_t)tail_chunk * 16u : 0u;
+    const uint32_t quad_off = (uint32_t)gq * 16u;
+    const int one = (ROWS && tail_in_k) ? 0x01010101 : 0;
+    const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101}, ones_tail = {one, one, one, one};
+    constexpr int pix_per_block = kWaves * RG * 16;
+
+    auto pixel_off = [&](int mt, int rg) { // byte offset of the lane's pixel of tile mt (clamped into the tensor)
+        const int p = min(mt * pix_per_block + (wave * RG + rg) * 16 + j, a.m - 1);
+        return (uint32_t)p * (uint32_t)a.ldx + (uint32_t)a.x_coff;
+    };
+    auto load = [&](uint32_t poff, int ks) { // slice of k-step ks
+        return ks == last ? __builtin_amdgcn_raw_buffer_load_b128(xres, poff + tail_off, 0, 0)
+                          : __builtin_amdgcn_raw_buffer_load_b128(xres, poff + quad_off, ks * 64, 0);
+    };
+
+    int mt = blockIdx.x;
+    uint32_t poff[RG];
+    u32x4 cur[RG];
+    if (mt < a.num_mtiles) {
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) {
+            poff[rg] = pixel_off(mt, rg);
+            cur[rg] = load(poff[rg], 0);
+        }
+    }
+    __syncthreads();
+
+    const int ch0 = ch_base + gq * (4 * T);
+#pragma clang loop unroll(disable)
+    for (; mt < a.num_mtiles; mt += gridDim.x) {
+        v4i acc[RG][T];
+        v4i rs[RG];
+        const int mt_next = mt + gridDim.x < a.num_mtiles ? mt + gridDim.x : mt; // past the end: re-read this tile, dropped
+        uint32_t poff_next[RG];
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) poff_next[rg] = pixel_off(mt_next, rg);
+#pragma clang loop unroll(disable)
+        for (int ks = 0; ks < KS; ks++) {
+            // the next slices: the next k-step of this tile, or the first of the next tile
+            u32x4 nxt[RG];
+            const bool same_tile = ks < last;
+#pragma unroll
+            for (int rg = 0; rg < RG; rg++) nxt[rg] = load(same_tile ? poff[rg] : poff_next[rg], same_tile ? ks + 1 : 0);
+            v4i xf[RG];
+#pragma unroll
+            for (int rg = 0; rg < RG; rg++) xf[rg] = __builtin_bit_cast(v4i, cur[rg] ^ 0x80808080u);
+            const uint8_t *wstep = wlds + (size_t)ks * T * 1024 + lane * 16;
+            if (ks == 0) {
+                int ct_off = gq * (4 * T);
+                asm volatile("" : "+v"(ct_off)); // (read per tile: kept in registers the constants would cost 4T of them)
+#pragma unroll
+                for (int nt = 0; nt < T; nt++) {
+                    const v4i ct = *reinterpret_cast<const v4i *>(cterm + ct_off + nt * 4);
+                    const v4i wf = *reinterpret_cast<const v4i *>(wstep + nt * 1024);
+#pragma unroll
+                    for (int rg = 0; rg < RG; rg++) acc[rg][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf, xf[rg], ct, 0, 0, 0);
+                }
+                if (ROWS) {
+                    const v4i zero = {0, 0, 0, 0};
+#pragma unroll
+                    for (int rg = 0; rg < RG; rg++) rs[rg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ks == last ? ones_tail : ones, xf[rg], zero, 0, 0, 0);
+                }
+            } else {
+#pragma unroll
+                for (int nt = 0; nt < T; nt++) {
+                    const v4i wf = *reinterpret_cast<const v4i *>(wstep + nt * 1024);
+#pragma unroll
+                    for (int rg = 0; rg < RG; rg++) acc[rg][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf, xf[rg], acc[rg][nt], 0, 0, 0);
+                }
+                if (ROWS) {
+#pragma unroll
+                    for (int rg = 0; rg < RG; rg++) rs[rg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ks == last ? ones_tail : ones, xf[rg], rs[rg], 0, 0, 0);
+                }
+            }
+#pragma unroll
+            for (int rg = 0; rg < RG; rg++) cur[rg] = nxt[rg];
+        }
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++)
+            igemm_store_tile<T, ROWS ? kOwesRows : kOwesNothing, true>(a, acc[rg], ROWS ? rs[rg][0] : 0,
+                                                                        mt * pix_per_block + (wave * RG + rg) * 16 + j, ch0, gq, cterm, nullptr);
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) poff[rg] = poff_next[rg];
+    }
+}
+
 // ---- long reductions: weights streamed through LDS -----------------------------------------------
 // When the weights of a channel chunk do not fit the LDS budget (3x3 and larger windows over many
 // channels), they are streamed: every k-step's T fragments go global -> registers -> a three-slot LDS
@@ -807,6 +942,16 @@ template <int T, int RG, int MODE> int launch_trg(nncase_hip_ctx *ctx, const Ige
     if constexpr (loads_rows(MODE))
         plain = a.ep.out_mode == kOutU8 && a.ep.fast && a.ep.full && !a.lut && !a.rep.res && a.n % (4 * T) == 0 && ((a.ldy | a.y_coff) & 3) == 0;
     if (plain) {
+        if constexpr (MODE == kRows16) {
+            // the whole chunk's weights resident, rows of at least 16 bytes: the lean kernel
+            if (a.kc_steps >= a.ksteps) {
+                const size_t lds_rows = (size_t)T * 16 * sizeof(int32_t) + (size_t)a.ksteps * T * 1024;
+                if (a.zwp_rows != 0) hipLaunchKernelGGL((qconv_rows_kernel<T, RG, true>), dim3(gx, nchunks, 1), dim3(kThreads), lds_rows, ctx->stream, args);
+                else hipLaunchKernelGGL((qconv_rows_kernel<T, RG, false>), dim3(gx, nchunks, 1), dim3(kThreads), lds_rows, ctx->stream, args);
+                NNHIP_LAUNCH_CHECK(ctx, "qconv_rows_kernel");
+                return 0;
+            }
+        }
         if constexpr (loads_rows(MODE))
             hipLaunchKernelGGL((qconv_igemm_kernel<T, RG, MODE, true>), dim3(gx, nchunks, 1), dim3(kThreads), lds, ctx->stream, args);
     } else
