@@ -191,6 +191,10 @@ typedef struct nncase_hip_conv2d_args {
     nncase_hip_quant_param_t residual_qp;
     nncase_hip_quant_param_t sum_qp;
     float sum_clamp_min, sum_clamp_max;
+    /* Output placed inside a wider NHWC tensor (the producer of one input of a channel concat writes
+     * its slice of the concat's tensor): pixel stride in channels, 0 = out_channels (dense), and the
+     * first channel written.  Dense (MFMA) kernels only; residual_dev stays a dense tensor. */
+    int32_t out_channel_stride, out_channel_offset;
 } nncase_hip_conv2d_args_t;
 
 /* Output is [batch, out_h, out_w, out_channels] with
@@ -323,7 +327,9 @@ NNCASE_HIP_API int nncase_hip_lut_u8(nncase_hip_ctx_t *ctx, const uint8_t *in_de
  * src/Native/src/kernels/stackvm/tensor_ops.cpp, on the innermost axis) with
  * every input requantised to the output's quant params, i.e. the
  * Dequantize -> Concat -> Quantize sub-graph of a u8/u8 model:
- *   out[p, off_i + c] = Q_out(DQ_i(in_i[p, c])),  off_i = channels_0 + .. + channels_{i-1}. */
+ *   out[p, off_i + c] = Q_out(DQ_i(in_i[p, c])),  off_i = channels_0 + .. + channels_{i-1}.
+ * An input whose pointer is NULL is skipped: its channels are already in place (written there by
+ * a convolution with out_channel_stride / out_channel_offset). */
 #define NNCASE_HIP_MAX_CONCAT 8
 NNCASE_HIP_API int nncase_hip_qconcat_channels(nncase_hip_ctx_t *ctx, int32_t n_inputs, const uint8_t *const *in_dev,
                                                const int32_t *channels, const nncase_hip_quant_param_t *in_qps,

@@ -60,6 +60,8 @@ public struct HipConv2DArgs
     public HipQuantParam SumQp;
     public float SumClampMin;
     public float SumClampMax;
+    public int OutChannelStride;
+    public int OutChannelOffset;
 }
 
 /// <summary>nncase_hip_qblock_desc_t.</summary>

@@ -231,13 +231,17 @@ extern "C" int nncase_hip_qconcat_channels(nncase_hip_ctx_t *ctx, int32_t n_inpu
     int64_t c_out = 0;
     bool vec = (reinterpret_cast<uintptr_t>(out_dev) & 3u) == 0;
     for (int i = 0; i < n_inputs; i++) {
-        NNHIP_REQUIRE(ctx, channels[i] > 0 && in_dev[i], -EINVAL, "qconcat_channels: input %d is empty or null", i);
-        vec = vec && channels[i] % 4 == 0 && (reinterpret_cast<uintptr_t>(in_dev[i]) & 3u) == 0;
+        NNHIP_REQUIRE(ctx, channels[i] > 0, -EINVAL, "qconcat_channels: input %d is empty", i);
+        vec = vec && channels[i] % 4 == 0 && (reinterpret_cast<uintptr_t>(in_dev[i]) & 3u) == 0; // (a skipped input is null)
         c_out += channels[i];
     }
     if (pixels == 0) return 0;
     uint32_t c_off = 0;
     for (int i = 0; i < n_inputs; i++) {
+        if (!in_dev[i]) { // already in place: written by its producer
+            c_off += (uint32_t)channels[i];
+            continue;
+        }
         uint8_t lut[256];
         const int rc = nncase_hip_make_unary_lut(NNCASE_HIP_LUT_REQUANT, in_qps[i], out_qp, lut);
         NNHIP_REQUIRE(ctx, rc == 0, rc, "qconcat_channels: cannot build the requantisation table of input %d", i);

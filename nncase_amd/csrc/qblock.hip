@@ -599,7 +599,7 @@ extern "C" int nncase_hip_qblock(nncase_hip_ctx_t *ctx, const uint8_t *x_dev, co
     a.p.m = (int)m64;
     a.p.n = blk->cout;
     a.p.k = blk->mid;
-    a.p.ldy = blk->cout;
+    a.p.ldy = a.p.ldr = blk->cout;
     a.p.zxp = g->dw_qp.zero_point - 128;
     a.p.zwp = blk->zw_p - 128;
     a.p.wsum = blk->d_wsum_p;

@@ -337,6 +337,11 @@ extern "C" int nncase_hip_qconv2d(nncase_hip_ctx_t *ctx, const uint8_t *x_dev, c
     const int out_h = windowed_output_size(a->in_h, w->kernel_h, a->stride_h, a->dilation_h, a->pad_h_before, a->pad_h_after);
     const int out_w = windowed_output_size(a->in_w, w->kernel_w, a->stride_w, a->dilation_w, a->pad_w_before, a->pad_w_after);
     NNHIP_REQUIRE(ctx, out_h > 0 && out_w > 0, -NNCASE_HIP_ERR_SHAPE_MISMATCH, "qconv2d: window larger than padded input");
+    if (a->out_channel_stride != 0 || a->out_channel_offset != 0) {
+        NNHIP_REQUIRE(ctx, w->kind == nncase_hip_weights::kIgemm, -EINVAL,
+                      "qconv2d: an output inside a wider tensor is only supported by the dense (MFMA) kernels");
+        if (!a->residual_dev && !w->d_post_lut) return launch_qconv_igemm(ctx, x_dev, w, y_dev, a, out_h, out_w);
+    }
     if (a->residual_dev || w->d_post_lut) {
         if (a->residual_dev) {
             rc = check_out_dtype(ctx, NNCASE_HIP_DT_U8, a->sum_qp, "qconv2d(residual)");

@@ -142,7 +142,13 @@ int launch_qconv_igemm(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_hip_w
     a.kc_steps = w->kc_steps;
     a.ldx = w->in_channels;
     a.x_bytes = (size_t)c->batch * c->in_h * c->in_w * w->in_channels;
-    a.ldy = w->out_channels;
+    a.ldy = c->out_channel_stride ? c->out_channel_stride : w->out_channels;
+    a.ldr = w->out_channels;
+    NNHIP_REQUIRE(ctx, c->out_channel_stride >= 0 && c->out_channel_offset >= 0 &&
+                           (c->out_channel_stride ? c->out_channel_offset + w->out_channels <= c->out_channel_stride : c->out_channel_offset == 0),
+                  -EINVAL, "qconv2d: %d output channels at offset %d do not fit a pixel stride of %d", w->out_channels, c->out_channel_offset,
+                  c->out_channel_stride);
+    NNHIP_REQUIRE(ctx, m64 * a.ldy * out_es < ((int64_t)1 << 40), -EINVAL, "qconv2d: output too large");
     a.g_ic = w->g_ic;
     a.in_h = c->in_h;
     a.in_w = c->in_w;
@@ -180,7 +186,8 @@ int launch_qconv_igemm(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_hip_w
         a.wsum = w->d_wsum + (size_t)g * w->g_oc;
         a.bias = w->d_bias + (size_t)g * w->g_oc;
         a.x_coff = g * w->g_ic;
-        a.y_coff = g * w->g_oc;
+        a.y_coff = g * w->g_oc + c->out_channel_offset;
+        a.r_coff = g * w->g_oc;
         int rc;
         if (w->wide) {
             rc = mode == kRows16 ? launch_wide_rows16(ctx, a, w->tiles, w->nchunks) : launch_wide_vec16(ctx, a, w->tiles, w->nchunks);

@@ -62,6 +62,7 @@ struct IgemmArgs {
     int ldx, x_coff;       // input pixel stride / channel offset of the group (bytes)
     size_t x_bytes;        // size of the input tensor
     int ldy, y_coff;       // output pixel stride / channel offset (elements)
+    int ldr, r_coff;       // the same for the (dense) residual tensor
     int g_ic;
     int in_h, in_w;
     int kw, stride_h, stride_w, dil_h, dil_w, pad_h, pad_w;
@@ -377,8 +378,8 @@ __device__ __forceinline__ void igemm_store_tile(const IgemmArgs &a, const v4i (
             }
         }
         if (a.rep.res) { // fused residual add on the requantised bytes
-            const uint8_t *ro = a.rep.res + obase;
-            const bool whole = ((a.ldy | a.y_coff) & 3) == 0 && ch0 + 4 * T <= a.n;
+            const uint8_t *ro = a.rep.res + ((size_t)p * a.ldr + a.r_coff + ch0);
+            const bool whole = ((a.ldr | a.r_coff) & 3) == 0 && ch0 + 4 * T <= a.n;
 #pragma unroll
             for (int nt = 0; nt < T; nt++) {
                 uint32_t rv = 0;

@@ -452,6 +452,43 @@ class HipModel:
             self.never_written |= {e, d}
             skip_nodes |= {d, pr}
         block_members = {m for e, (d, pr, _) in self.blocks.items() for m in (e, d, pr)}
+        # A dense conv (with whatever is folded into its epilogue) whose result only feeds a channel concat writes its
+        # slice of the concat's tensor itself: out[p, off + c] with the concat's pixel stride.  The concat's
+        # requantisation of that input, a byte table, is composed with the conv's own table (or becomes it); behind
+        # a folded residual add there is no table stage, so such a conv only qualifies when the requantisation is
+        # the identity.  The concat operator then skips that input, and disappears when none is left.
+        self.write_through: Dict[int, Tuple[int, int, int, Optional[np.ndarray]]] = {}   # conv -> (concat, offset, stride, table)
+        if fuse_residual:
+            owner = {**{v: k for k, v in self.fused_lut.items()}, **{v: k for k, v in self.fused_into.items()}}
+            for ci, cn in enumerate(qg.nodes):
+                if cn.op != "concat":
+                    continue
+                ctot = sum(qg.nodes[j].out_shape[0] for j in cn.inputs)
+                off = 0
+                for j in cn.inputs:
+                    ch = qg.nodes[j].out_shape[0]
+                    conv = owner.get(j, j)
+                    conv = owner.get(conv, conv)               # add -> lut -> conv
+                    cnode = qg.nodes[conv]
+                    last = self.fused_into.get(conv, self.fused_lut.get(conv, conv))
+                    ok = (cnode.op == "conv" and last == j and consumers[j] == 1 and j not in qg.output_nodes
+                          and conv not in block_members and conv not in self.write_through
+                          and not (cnode.groups > 1 and cnode.weights.shape[1] == 1) and cnode.weights.shape[1] * cnode.groups > 4
+                          and (conv == j or conv in self.fused_lut or conv in self.fused_into))
+                    if ok:
+                        table = rt.make_unary_lut(rt.LUT_REQUANT, qp(*qg.nodes[j].out_qp), qp(*cn.out_qp))
+                        identity = np.array_equal(table, np.arange(256, dtype=np.uint8))
+                        if conv in self.fused_into:
+                            ok = identity
+                            table = None
+                        elif conv in self.fused_lut:
+                            table = table[qg.nodes[self.fused_lut[conv]].lut]
+                        elif identity:
+                            table = None
+                    if ok:
+                        self.write_through[conv] = (ci, off, ctot, table)
+                        self.never_written |= {conv, j} | ({self.fused_lut[conv]} if conv in self.fused_lut else set())
+                    off += ch
         # buffers and packed weights once, shared by the lanes
         for i, n in enumerate(qg.nodes):
             cc, hh, ww = n.out_shape
@@ -462,8 +499,9 @@ class HipModel:
             if n.op == "fold2":
                 self.buffers.append(self.buffers[n.inputs[0]])  # the same bytes read as half as many, twice as deep pixels
                 continue
-            if i in self.blocks or i - 1 in self.blocks:
-                self.buffers.append(ctx.alloc(16))        # the expanded tensors of a fused block live in LDS only
+            if i in self.blocks or i - 1 in self.blocks or i in self.write_through:
+                self.buffers.append(ctx.alloc(16))        # expanded tensors of a fused block live in LDS only; a conv
+                #                                           that writes into its concat has no tensor of its own
             else:
                 self.buffers.append(ctx.alloc(lanes * self._lane_stride(bl * cc * hh * ww)))
             if i in self.blocks:
@@ -473,7 +511,10 @@ class HipModel:
             elif n.op == "conv" and i not in block_members:
                 wt = ctx.prepack_conv2d(n.weights, n.bias, qp(*n.w_qp), n.groups, expected_pixels=bl * hh * ww)
                 fused_lut = self.fused_lut.get(i)
-                if fused_lut is not None:
+                wthru = self.write_through.get(i)
+                if wthru is not None and wthru[3] is not None:
+                    wt.set_post_lut(wthru[3], qp(*qg.nodes[wthru[0]].out_qp))      # own table, then the concat's requantisation
+                elif fused_lut is not None:
                     wt.set_post_lut(qg.nodes[fused_lut].lut, qp(*qg.nodes[fused_lut].out_qp))
                 self.weights[-1] = wt
         self.outputs_f32: List[rt.DeviceBuffer] = [ctx.alloc(lanes * self._lane_stride(bl * int(np.prod(qg.nodes[j].out_shape)) * 4))
@@ -526,7 +567,7 @@ class HipModel:
                     self.op_nodes.append(addn if addn is not None else pn)
                     self.op_members.append([i, dn, pn] + ([addn] if addn is not None else []))
                 continue
-            buf = B(i)
+            buf = None if i in self.write_through else B(i)   # (a conv that writes into its concat has no tensor of its own)
             if n.op == "input":
                 self.fn.add_quantize(self.input_f32.view(lane * self._lane_stride(in_per * 4), in_per * 4), rt.DT_F32, buf, rt.DT_U8, in_per, qp(*n.out_qp))
             elif n.op == "conv":
@@ -543,6 +584,10 @@ class HipModel:
                     args.sum_qp = qp(*add.out_qp)
                     args.sum_clamp_min, args.sum_clamp_max = FULL_CLAMP
                     self.fn._keep.append(res)
+                wthru = self.write_through.get(i)
+                if wthru is not None:
+                    buf = B(wthru[0])
+                    args.out_channel_offset, args.out_channel_stride = wthru[1], wthru[2]
                 self.fn.add_qconv2d(B(n.inputs[0]), self.weights[i], buf, args)
             elif n.op == "add":
                 a, b = (qg.nodes[j] for j in n.inputs)
@@ -552,7 +597,11 @@ class HipModel:
                 self.fn.add_lut_u8(B(n.inputs[0]), buf, bl * cc * hh * ww, n.lut)
             elif n.op == "concat":
                 srcs = [qg.nodes[j] for j in n.inputs]
-                self.fn.add_qconcat_channels([B(j) for j in n.inputs], [s_.out_shape[0] for s_ in srcs],
+                in_place = {jn for conv, (ci_, _o, _s, _t) in self.write_through.items() if ci_ == i
+                            for jn in (self.fused_into.get(conv, self.fused_lut.get(conv, conv)),)}
+                if len(in_place) == len(n.inputs):
+                    continue                                   # every slice is written by its producer
+                self.fn.add_qconcat_channels([None if j in in_place else B(j) for j in n.inputs], [s_.out_shape[0] for s_ in srcs],
                                              [qp(*s_.out_qp) for s_ in srcs], buf, qp(*n.out_qp), bl * hh * ww)
             elif n.op == "resize":
                 src = qg.nodes[n.inputs[0]]

@@ -50,7 +50,8 @@ class Conv2dArgs(C.Structure):
                 ("x_qp", QuantParam), ("y_qp", QuantParam),
                 ("clamp_min", C.c_float), ("clamp_max", C.c_float), ("out_dtype", C.c_int32),
                 ("residual_dev", C.c_void_p), ("residual_qp", QuantParam), ("sum_qp", QuantParam),
-                ("sum_clamp_min", C.c_float), ("sum_clamp_max", C.c_float)]
+                ("sum_clamp_min", C.c_float), ("sum_clamp_max", C.c_float),
+                ("out_channel_stride", C.c_int32), ("out_channel_offset", C.c_int32)]
 
 
 class QBlockDesc(C.Structure):
@@ -247,7 +248,7 @@ def requant_host(acc: np.ndarray, sx, sw, y_qp: "QuantParam", clamp=(-FLT_MAX, F
 
 def _concat_args(inputs, channels, in_qps):
     n = len(inputs)
-    ptrs = (_VP * n)(*[b.ptr for b in inputs])
+    ptrs = (_VP * n)(*[None if b is None else b.ptr for b in inputs])   # None: the slice is already in place
     ch = (C.c_int32 * n)(*channels)
     qps = (QuantParam * n)(*in_qps)
     return n, ptrs, ch, qps
@@ -640,7 +641,7 @@ class Function:
                  "function_add_lut_u8")
 
     def add_qconcat_channels(self, inputs, channels, in_qps, out, out_qp, pixels):
-        self._keep += list(inputs) + [out]
+        self._keep += [b for b in inputs if b is not None] + [out]
         n, ptrs, ch, qps = _concat_args(inputs, channels, in_qps)
         self._ck(self.ctx.lib.nncase_hip_function_add_qconcat_channels(self.handle, n, ptrs, ch, qps, out.ptr, out_qp, pixels),
                  "function_add_qconcat_channels")

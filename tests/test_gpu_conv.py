@@ -244,11 +244,10 @@ def test_wide_tile_kernels_with_256_channel_blocks(hip_ctx, c, hw, oc, k):
 
 
 def test_wide_tile_kernel_is_selected_and_zero_points_at_the_extremes(hip_ctx):
-    from nncase_amd import runtime as rt2
     w8 = np.zeros((128, 64, 3, 3), np.uint8)
     wts = hip_ctx.prepack_conv2d(w8, None, qp(131, 0.004), 1, expected_pixels=2 * 256 * 256)
-    args = rt2.Conv2dArgs(2, 256, 256, 1, 1, 1, 1, 1, 1, 1, 1, qp(7, 0.02), qp(0, 1.0), -rt2.FLT_MAX, rt2.FLT_MAX, rt2.DT_I32)
-    fn = rt2.Function(hip_ctx)
+    args = rt.Conv2dArgs(2, 256, 256, 1, 1, 1, 1, 1, 1, 1, 1, qp(7, 0.02), qp(0, 1.0), -rt.FLT_MAX, rt.FLT_MAX, rt.DT_I32)
+    fn = rt.Function(hip_ctx)
     xb, yb = hip_ctx.alloc(2 * 256 * 256 * 64), hip_ctx.alloc(2 * 256 * 256 * 128 * 4)
     fn.add_qconv2d(xb, wts, yb, args)
     assert fn.op_kernel(0).startswith("qconv_wide<T=8")
@@ -441,6 +440,57 @@ def test_matmul_two_sided_batches_and_vectors(hip_ctx, ashape, bshape):
     with pytest.raises(rt.HipError) as e:
         K.mat_mul(np.zeros((2, 3, 4, 5), np.uint8), np.zeros((3, 2, 5, 6), np.uint8), qp(0, 1.0), qp(0, 1.0), None, np.int32, ctx=hip_ctx)
     assert e.value.code == -rt.ERR_SHAPE_MISMATCH
+
+
+@pytest.mark.parametrize("cin,cout,k,stride_c,offset,with_res", [
+    (16, 24, 1, 64, 8, False), (32, 64, 3, 200, 136, False), (16, 20, 1, 33, 13, False),     # unaligned stride and offset
+    (64, 32, 1, 96, 64, True), (128, 64, 3, 128, 64, False)])
+def test_conv_output_inside_a_wider_tensor(hip_ctx, cin, cout, k, stride_c, offset, with_res):
+    """out_channel_stride / out_channel_offset: the conv writes channels [offset, offset + cout) of every pixel of a
+    tensor with stride_c channels (its slice of a concat) and leaves the other channels alone; a fused residual is
+    still read as a dense tensor."""
+    rng = np.random.default_rng(cin + cout + stride_c)
+    n, h, w = 2, 19, 23
+    x = rng.integers(0, 256, (n, cin, h, w), dtype=np.uint8)
+    wt = rng.integers(0, 256, (cout, cin, k, k), dtype=np.uint8)
+    bias = rng.integers(-2000, 2000, cout).astype(np.int32)
+    pad = ((k // 2, k // 2), (k // 2, k // 2))
+    zx, sx, zw, sw, zy, sy = 7, 0.0235, 131, 0.0041, 101, 0.21
+    res = rng.integers(0, 256, (n, cout, h, w), dtype=np.uint8) if with_res else None
+    want = O.qconv2d(x, wt, bias, zx, sx, zw, sw, zy, sy, padding=pad, out_mode=O.OUT_U8)
+    if with_res:
+        want = O.qadd(want, res, zy, sy, 33, 0.11, 90, 0.3)
+    store = rng.integers(0, 256, (n, h, w, stride_c), dtype=np.uint8)
+    wts = hip_ctx.prepack_conv2d(wt, bias, qp(zw, sw), 1, expected_pixels=n * h * w)
+    xb = hip_ctx.to_device(np.ascontiguousarray(x.transpose(0, 2, 3, 1)))
+    yb = hip_ctx.to_device(store)
+    args = rt.Conv2dArgs(n, h, w, 1, 1, 1, 1, pad[0][0], pad[0][1], pad[1][0], pad[1][1], qp(zx, sx), qp(zy, sy), -rt.FLT_MAX, rt.FLT_MAX, rt.DT_U8)
+    args.out_channel_stride, args.out_channel_offset = stride_c, offset
+    if with_res:
+        rb = hip_ctx.to_device(np.ascontiguousarray(res.transpose(0, 2, 3, 1)))
+        args.residual_dev, args.residual_qp, args.sum_qp = rb.ptr, qp(33, 0.11), qp(90, 0.3)
+        args.sum_clamp_min, args.sum_clamp_max = -rt.FLT_MAX, rt.FLT_MAX
+    hip_ctx.qconv2d(xb, wts, yb, args)
+    got = yb.download(store.shape, np.uint8)
+    assert np.array_equal(got[..., offset:offset + cout], want.transpose(0, 2, 3, 1))
+    keep = np.ones(stride_c, bool)
+    keep[offset:offset + cout] = False
+    assert np.array_equal(got[..., keep], store[..., keep])
+    for bad_stride, bad_off in ((cout - 1, 0), (stride_c, stride_c - cout + 1), (0, 4)):
+        args.out_channel_stride, args.out_channel_offset = bad_stride, bad_off
+        with pytest.raises(rt.HipError) as e:
+            hip_ctx.qconv2d(xb, wts, yb, args)
+        assert e.value.code == -22
+
+
+def test_depthwise_conv_refuses_an_output_inside_a_wider_tensor(hip_ctx):
+    wts = hip_ctx.prepack_conv2d(np.zeros((32, 1, 3, 3), np.uint8), None, qp(128, 0.01), 32)
+    xb, yb = hip_ctx.alloc(8 * 8 * 32), hip_ctx.alloc(8 * 8 * 64)
+    args = rt.Conv2dArgs(1, 8, 8, 1, 1, 1, 1, 1, 1, 1, 1, qp(0, 1.0), qp(0, 1.0), -rt.FLT_MAX, rt.FLT_MAX, rt.DT_U8)
+    args.out_channel_stride = 64
+    with pytest.raises(rt.HipError) as e:
+        hip_ctx.qconv2d(xb, wts, yb, args)
+    assert e.value.code == -22
 
 
 def test_linearity_at_full_size(hip_ctx):
