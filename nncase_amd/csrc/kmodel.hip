@@ -414,6 +414,71 @@ static int build_function(nncase_hip_ctx_t *ctx, Span text_span, Span rdata, nnc
         k += 2;
     }
 
+    auto rd = [&](uint64_t off, size_t bytes) -> const uint8_t * {
+        if (off == kNoRdata || off > rdata.n || bytes > rdata.n - off) return nullptr;
+        return rdata.p + off;
+    };
+
+    // A dense conv whose result (behind its folded table / add) is read by one channel concat only writes its slice
+    // of the concat's tensor itself.  The concat's requantisation of that input is a byte table: it is composed with
+    // the conv's own table or becomes it; behind a folded add there is no table stage, so such a conv qualifies
+    // only when that requantisation is the identity.  The concat then skips the input, and disappears when none is left.
+    struct Through {
+        int concat = -1, offset = 0, stride = 0;
+        bool has_table = false;
+        uint8_t table[256];
+    };
+    std::vector<Through> through(th.n_ops);
+    {
+        std::vector<int> owner(th.n_ops, -1); // folded table / add op -> its conv
+        for (uint32_t k = 0; k < th.n_ops; k++) {
+            if (fused_lut[k] >= 0) owner[fused_lut[k]] = (int)k;
+            if (fused_add[k] >= 0) owner[fused_add[k]] = (int)k;
+        }
+        for (uint32_t ci = 0; ci < th.n_ops; ci++) {
+            const hipf_op &cn = ops[ci];
+            if (cn.opcode != kOpConcat || skipped[ci]) continue;
+            const hipf_tensor &tc = m->tensors[cn.output];
+            uint64_t total = 0;
+            for (uint32_t i = 0; i < cn.n_inputs; i++) total += m->tensors[cn.inputs[i]].dims[3];
+            if (tc.dtype != NNCASE_HIP_DT_U8 || total != tc.dims[3] || tc.scale == 0.f) continue; // (refused when it is recorded)
+            int off = 0;
+            for (uint32_t i = 0; i < cn.n_inputs; i++) {
+                const int32_t t = cn.inputs[i];
+                const hipf_tensor &tx = m->tensors[t];
+                const int at = off;
+                off += (int)tx.dims[3];
+                const int p = producer[t];
+                if (p < 0) continue;
+                const int c = owner[p] >= 0 ? owner[p] : p;
+                const hipf_op &conv = ops[c];
+                const int last = fused_add[c] >= 0 ? fused_add[c] : fused_lut[c] >= 0 ? fused_lut[c] : c;
+                if (conv.opcode != kOpConv2d || skipped[c] || block_head[c] || last != p || through[c].concat >= 0) continue;
+                if (consumers[t] != 1 || is_output(t) || tx.dtype != NNCASE_HIP_DT_U8 || !dense_conv(conv)) continue;
+                if (tx.dims[0] != tc.dims[0] || tx.dims[1] != tc.dims[1] || tx.dims[2] != tc.dims[2] || (uint32_t)conv.p[0] != tx.dims[3])
+                    continue;
+                uint8_t requant[256];
+                if (nncase_hip_make_unary_lut(NNCASE_HIP_LUT_REQUANT, tqp((uint32_t)t), tqp((uint32_t)cn.output), requant) != 0) continue;
+                bool identity = true;
+                for (int v = 0; v < 256; v++) identity = identity && requant[v] == v;
+                Through w;
+                if (fused_add[c] >= 0) {
+                    if (!identity) continue;
+                } else if (fused_lut[c] >= 0) {
+                    const uint8_t *own = rd(ops[fused_lut[c]].rdata0, 256);
+                    if (!own) continue;
+                    for (int v = 0; v < 256; v++) w.table[v] = requant[own[v]];
+                    w.has_table = true;
+                } else if (!identity) {
+                    memcpy(w.table, requant, 256);
+                    w.has_table = true;
+                }
+                w.concat = (int)ci, w.offset = at, w.stride = (int)tc.dims[3];
+                through[c] = w;
+            }
+        }
+    }
+
     // ---- device buffers ---------------------------------------------------------------------------
     m->buffers.assign(th.n_tensors, nullptr);
     m->owns.assign(th.n_tensors, 0);
@@ -421,6 +486,11 @@ static int build_function(nncase_hip_ctx_t *ctx, Span text_span, Span rdata, nnc
         if (fused_add[k] >= 0 || fused_lut[k] >= 0) m->owns[ops[k].output] = 2;
         if (fused_add[k] >= 0 && fused_lut[k] >= 0) m->owns[ops[fused_lut[k]].output] = 2;
         if (block_head[k]) m->owns[ops[k].output] = m->owns[ops[k + 1].output] = 2;
+        if (through[k].concat >= 0) { // no tensor of its own: the bytes live in the concat's tensor
+            m->owns[ops[k].output] = 2;
+            if (fused_lut[k] >= 0) m->owns[ops[fused_lut[k]].output] = 2;
+            if (fused_add[k] >= 0) m->owns[ops[fused_add[k]].output] = 2;
+        }
     }
     for (uint32_t k = 0; k < th.n_ops; k++) // a reshaped tensor is its input's buffer under other extents
         if (ops[k].opcode == kOpReshape && !skipped[k]) m->owns[ops[k].output] = 2;
@@ -435,10 +505,6 @@ static int build_function(nncase_hip_ctx_t *ctx, Span text_span, Span rdata, nnc
 
     // ---- operators ----------------------------------------------------------------------------------
     NNHIP_REQUIRE(ctx, nncase_hip_function_create(ctx, &m->fn) == 0, -ENOMEM, "kmodel_load: cannot create the function");
-    auto rd = [&](uint64_t off, size_t bytes) -> const uint8_t * {
-        if (off == kNoRdata || off > rdata.n || bytes > rdata.n - off) return nullptr;
-        return rdata.p + off;
-    };
     for (uint32_t k = 0; k < th.n_ops; k++) {
         if (skipped[k]) continue;
         const hipf_op &o = ops[k];
@@ -553,9 +619,14 @@ static int build_function(nncase_hip_ctx_t *ctx, Span text_span, Span rdata, nnc
                 NNHIP_REQUIRE(ctx, table, -EINVAL, "kmodel_load: op %d table outside .rdata", fused_lut[k]);
                 NNHIP_REQUIRE(ctx, elems((uint32_t)lut.output) == elems(dst), -NNCASE_HIP_ERR_SHAPE_MISMATCH,
                               "kmodel_load: op %d shapes differ", fused_lut[k]);
-                rc = nncase_hip_weights_set_post_lut(ctx, wt, table, tqp((uint32_t)lut.output));
+                // (a conv that writes into its concat applies its table and the concat's requantisation in one)
+                rc = through[k].has_table ? nncase_hip_weights_set_post_lut(ctx, wt, through[k].table, tqp((uint32_t)ops[through[k].concat].output))
+                                          : nncase_hip_weights_set_post_lut(ctx, wt, table, tqp((uint32_t)lut.output));
                 if (rc) return rc;
                 y = m->buffers[lut.output];
+            } else if (through[k].has_table) {
+                rc = nncase_hip_weights_set_post_lut(ctx, wt, through[k].table, tqp((uint32_t)ops[through[k].concat].output));
+                if (rc) return rc;
             }
             if (fused_add[k] >= 0) {
                 const hipf_op &add = ops[fused_add[k]];
@@ -566,6 +637,10 @@ static int build_function(nncase_hip_ctx_t *ctx, Span text_span, Span rdata, nnc
                 a.residual_qp = tqp(res), a.sum_qp = tqp(sum);
                 a.sum_clamp_min = add.f[0], a.sum_clamp_max = add.f[1];
                 y = m->buffers[sum];
+            }
+            if (through[k].concat >= 0) {
+                y = m->buffers[ops[through[k].concat].output];
+                a.out_channel_stride = through[k].stride, a.out_channel_offset = through[k].offset;
             }
             rc = nncase_hip_function_add_qconv2d(m->fn, static_cast<const uint8_t *>(m->buffers[in0]), wt, y, &a);
             break;
@@ -599,17 +674,22 @@ static int build_function(nncase_hip_ctx_t *ctx, Span text_span, Span rdata, nnc
             const uint8_t *ins[8];
             int32_t ch[8];
             nncase_hip_quant_param_t qps[8];
-            uint32_t total = 0;
+            uint32_t total = 0, to_copy = 0;
             for (uint32_t i = 0; i < o.n_inputs; i++) {
                 const hipf_tensor &x = m->tensors[o.inputs[i]];
                 NNHIP_REQUIRE(ctx, x.dims[0] == to.dims[0] && x.dims[1] == to.dims[1] && x.dims[2] == to.dims[2],
                               -NNCASE_HIP_ERR_SHAPE_MISMATCH, "kmodel_load: op %u concat input %u extent", k, i);
-                ins[i] = static_cast<const uint8_t *>(m->buffers[o.inputs[i]]);
+                ins[i] = static_cast<const uint8_t *>(m->buffers[o.inputs[i]]); // null: written in place by its conv
+                to_copy += ins[i] != nullptr;
                 ch[i] = (int32_t)x.dims[3];
                 qps[i] = tqp((uint32_t)o.inputs[i]);
                 total += x.dims[3];
             }
             NNHIP_REQUIRE(ctx, total == to.dims[3], -NNCASE_HIP_ERR_SHAPE_MISMATCH, "kmodel_load: op %u concat channels", k);
+            if (to_copy == 0) { // every slice is written by its producer
+                rc = 0;
+                break;
+            }
             rc = nncase_hip_function_add_qconcat_channels(m->fn, (int32_t)o.n_inputs, ins, ch, qps, static_cast<uint8_t *>(m->buffers[dst]),
                                                           tqp(dst), (int64_t)to.dims[0] * to.dims[1] * to.dims[2]);
             break;
