@@ -376,6 +376,15 @@ NNCASE_HIP_API int nncase_hip_pack(nncase_hip_ctx_t *ctx, const void *in_dev, vo
 NNCASE_HIP_API int nncase_hip_unpack(nncase_hip_ctx_t *ctx, const void *in_dev, void *out_dev, int32_t elem_size,
                                      int32_t rank, const int32_t *unpacked_shape, int32_t n_axes,
                                      const int32_t *axes, const int32_t *lanes);
+/* Quantize (float32 -> u8, as nncase_hip_quantize) followed by pack, in one pass over the input: what stands in
+ * front of a stem convolution over RGB.  Two layouts: <= 4 innermost channels packed by (4) (RGB -> RGBX), and an
+ * NHWC tensor with <= 4 channels and even H, W packed by (2, 2, 4) on (H, W, C), which turns every 2 x 2 block of
+ * pixels into one 16-channel pixel of the half-size image (a stride-2 convolution with an even window then reads it
+ * as a stride-1 convolution with half the window).  out_dev must be 16-byte aligned; -EINVAL for other arguments.
+ * The result equals nncase_hip_quantize then nncase_hip_pack byte for byte. */
+NNCASE_HIP_API int nncase_hip_quantize_pack(nncase_hip_ctx_t *ctx, const float *in_dev, uint8_t *out_dev, int32_t rank,
+                                            const int32_t *shape, int32_t n_axes, const int32_t *axes,
+                                            const int32_t *lanes, nncase_hip_quant_param_t qp);
 
 /* NCHW <-> NHWC relayout of a dense tensor (the Transpose nncase inserts
  * around NHWC imports, src/Nncase.Importer/TFLite/Conv2D.cs:28-29,67). */
@@ -528,6 +537,10 @@ NNCASE_HIP_API int nncase_hip_function_add_qmaxpool2d(nncase_hip_function_t *fn,
 NNCASE_HIP_API int nncase_hip_function_add_pack(nncase_hip_function_t *fn, const void *in_dev, void *out_dev,
                                                 int32_t elem_size, int32_t rank, const int32_t *shape, int32_t n_axes,
                                                 const int32_t *axes, const int32_t *lanes);
+NNCASE_HIP_API int nncase_hip_function_add_quantize_pack(nncase_hip_function_t *fn, const float *in_dev, uint8_t *out_dev,
+                                                         int32_t rank, const int32_t *shape, int32_t n_axes,
+                                                         const int32_t *axes, const int32_t *lanes,
+                                                         nncase_hip_quant_param_t qp);
 /* The decode-step operators above, recorded with the same arguments (paged attention included), so a
  * whole decode step replays as one HIP graph. */
 NNCASE_HIP_API int nncase_hip_function_add_w8a16_gemm(nncase_hip_function_t *fn, const void *a_dev, const nncase_hip_w8a16_t *weights,

@@ -125,6 +125,21 @@ __device__ __forceinline__ uint32_t fastdiv(uint32_t n, const FastDiv &f) {
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
+template <typename TQ> struct QLimits;
+template <> struct QLimits<uint8_t> { static constexpr float lo = 0.f, hi = 255.f; };
+template <> struct QLimits<int8_t> { static constexpr float lo = -128.f, hi = 127.f; };
+template <> struct QLimits<int16_t> { static constexpr float lo = -32768.f, hi = 32767.f; };
+
+// rne(v) then saturate.  The clamp is done on the float before rounding: the
+// limits are integers, so clamp and round-half-even commute, and values
+// beyond the int32 range saturate instead of wrapping.
+template <typename TQ> __device__ __forceinline__ TQ quantize_one(float x, float scale, float bias) {
+    float v = x / scale + bias;
+    v = fminf(fmaxf(v, QLimits<TQ>::lo), QLimits<TQ>::hi); // NaN -> lo
+    return (TQ)(int32_t)rintf(v);
+}
+
+
 // attn.hip: checks the geometry and sizes the context's paged-attention workspace for it
 // (-EBUSY if that needs a reallocation while a captured graph refers to it or the stream is capturing).
 int attn_reserve(nncase_hip_ctx *ctx, const nncase_hip_paged_attn_args_t *geometry);

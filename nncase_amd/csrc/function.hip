@@ -8,7 +8,7 @@
 namespace {
 
 struct Op {
-    enum Kind { kQuantize, kDequantize, kConv, kAdd, kPool, kLut, kConcat, kResize, kMaxPool, kPack,
+    enum Kind { kQuantize, kDequantize, kConv, kAdd, kPool, kLut, kConcat, kResize, kMaxPool, kPack, kQuantPack,
                 kGemm, kRmsNorm, kRope, kAttn, kArgmax, kEmbed, kAddI32, kBlock } kind;
     const void *in0 = nullptr, *in1 = nullptr;
     void *out = nullptr;
@@ -82,6 +82,8 @@ static int run_op(nncase_hip_function *fn, const Op &op) {
                                      op.pool[7], op.qp0, op.qp1);
     case Op::kPack:
         return nncase_hip_pack(ctx, op.in0, op.out, op.elem_size, op.rank, op.shape, op.n_axes, op.axes, op.lanes);
+    case Op::kQuantPack:
+        return nncase_hip_quantize_pack(ctx, (const float *)op.in0, (uint8_t *)op.out, op.rank, op.shape, op.n_axes, op.axes, op.lanes, op.qp0);
     case Op::kGemm:
         if (op.in2) return nncase_hip_rmsnorm_w8a16_gemm(ctx, op.in0, op.in2, op.eps, op.w8, op.out, op.batch, op.mode, op.in1, op.dt_out);
         return nncase_hip_w8a16_gemm(ctx, op.in0, op.w8, op.out, op.batch, op.mode, op.in1, op.dt_out);
@@ -279,6 +281,20 @@ extern "C" int nncase_hip_function_add_pack(nncase_hip_function_t *fn, const voi
     Op op;
     op.kind = Op::kPack;
     op.in0 = in_dev, op.out = out_dev, op.elem_size = elem_size, op.rank = rank, op.n_axes = n_axes;
+    for (int i = 0; i < rank; i++) op.shape[i] = shape[i];
+    for (int i = 0; i < n_axes; i++) op.axes[i] = axes[i], op.lanes[i] = lanes[i];
+    return push(fn, op);
+}
+
+extern "C" int nncase_hip_function_add_quantize_pack(nncase_hip_function_t *fn, const float *in_dev, uint8_t *out_dev, int32_t rank,
+                                                     const int32_t *shape, int32_t n_axes, const int32_t *axes, const int32_t *lanes,
+                                                     nncase_hip_quant_param_t qp) {
+    if (!fn) return -EINVAL;
+    NNHIP_REQUIRE(fn->ctx, in_dev && out_dev && shape && rank > 0 && rank <= 8 && n_axes > 0 && n_axes <= 8 && axes && lanes, -EINVAL,
+                  "function_add_quantize_pack: bad argument");
+    Op op;
+    op.kind = Op::kQuantPack;
+    op.in0 = in_dev, op.out = out_dev, op.rank = rank, op.n_axes = n_axes, op.qp0 = qp;
     for (int i = 0; i < rank; i++) op.shape[i] = shape[i];
     for (int i = 0; i < n_axes; i++) op.axes[i] = axes[i], op.lanes[i] = lanes[i];
     return push(fn, op);
@@ -501,6 +517,7 @@ extern "C" int nncase_hip_function_op_kernel(nncase_hip_function_t *fn, int32_t 
     case Op::kResize: snprintf(name, capacity, "resize_nearest"); break;
     case Op::kMaxPool: snprintf(name, capacity, "qmaxpool<%dx%d>", op.pool[0], op.pool[1]); break;
     case Op::kPack: snprintf(name, capacity, "pack"); break;
+    case Op::kQuantPack: snprintf(name, capacity, "quantize+pack"); break;
     case Op::kGemm:
         snprintf(name, capacity, "%sw8a16_gemm%s", op.in2 ? "rmsnorm+" : "",
                  op.mode == NNCASE_HIP_GEMM_SWIGLU ? "+swiglu" : (op.in1 ? "+residual" : ""));

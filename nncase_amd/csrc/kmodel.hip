@@ -479,6 +479,24 @@ static int build_function(nncase_hip_ctx_t *ctx, Span text_span, Span rdata, nnc
         }
     }
 
+    // A float32 -> u8 quantize read only by a channel padding is done by that operator (quantize and pack in one pass).
+    std::vector<int> fused_quant(th.n_ops, -1); // pad_channels op -> the quantize op in front of it
+    for (uint32_t k = 0; k < th.n_ops; k++) {
+        if (ops[k].opcode != kOpPadChannels || ops[k].n_inputs != 1) continue;
+        const int32_t t = ops[k].inputs[0];
+        const int q = producer[t];
+        if (q < 0 || ops[q].opcode != kOpQuantize || ops[q].n_inputs != 1 || consumers[t] != 1 || is_output(t)) continue;
+        if (m->tensors[ops[q].inputs[0]].dtype != NNCASE_HIP_DT_F32 || m->tensors[t].dtype != NNCASE_HIP_DT_U8 || m->tensors[t].scale == 0.f ||
+            m->tensors[t].dims[3] > 4 || elems((uint32_t)ops[q].inputs[0]) != elems((uint32_t)t))
+            continue;
+        const hipf_tensor &tp = m->tensors[ops[k].output], &tq = m->tensors[t];
+        const bool plain = tp.dims[3] == 4 && tp.dims[1] == tq.dims[1] && tp.dims[2] == tq.dims[2];
+        const bool blocks = tp.dims[3] == 16 && tq.dims[1] == 2 * tp.dims[1] && tq.dims[2] == 2 * tp.dims[2];
+        if (tp.dtype != NNCASE_HIP_DT_U8 || !(plain || blocks)) continue;
+        fused_quant[k] = q;
+        skipped[q] = 1;
+    }
+
     // ---- device buffers ---------------------------------------------------------------------------
     m->buffers.assign(th.n_tensors, nullptr);
     m->owns.assign(th.n_tensors, 0);
@@ -486,6 +504,7 @@ static int build_function(nncase_hip_ctx_t *ctx, Span text_span, Span rdata, nnc
         if (fused_add[k] >= 0 || fused_lut[k] >= 0) m->owns[ops[k].output] = 2;
         if (fused_add[k] >= 0 && fused_lut[k] >= 0) m->owns[ops[fused_lut[k]].output] = 2;
         if (block_head[k]) m->owns[ops[k].output] = m->owns[ops[k + 1].output] = 2;
+        if (fused_quant[k] >= 0) m->owns[ops[fused_quant[k]].output] = 2;
         if (through[k].concat >= 0) { // no tensor of its own: the bytes live in the concat's tensor
             m->owns[ops[k].output] = 2;
             if (fused_lut[k] >= 0) m->owns[ops[fused_lut[k]].output] = 2;
@@ -718,13 +737,22 @@ static int build_function(nncase_hip_ctx_t *ctx, Span text_span, Span rdata, nnc
             rc = 0;
             break;
         case kOpPadChannels: {
-            NNHIP_REQUIRE(ctx, ti.dtype == to.dtype && ti.dims[0] == to.dims[0] && ti.dims[1] == to.dims[1] &&
-                                   ti.dims[2] == to.dims[2] && ti.dims[3] <= to.dims[3],
+            // channels padded to 4, and with halved extents 2 x 2 blocks of such pixels as 16-channel pixels
+            const bool blocks = to.dims[3] == 16 && ti.dims[1] == 2 * to.dims[1] && ti.dims[2] == 2 * to.dims[2];
+            NNHIP_REQUIRE(ctx, ti.dtype == to.dtype && ti.dims[0] == to.dims[0] && ti.dims[3] <= to.dims[3] &&
+                                   (blocks ? ti.dims[3] <= 4 : ti.dims[1] == to.dims[1] && ti.dims[2] == to.dims[2]),
                           -NNCASE_HIP_ERR_SHAPE_MISMATCH, "kmodel_load: op %u channel padding tensors", k);
             const int32_t shape[4] = {(int32_t)ti.dims[0], (int32_t)ti.dims[1], (int32_t)ti.dims[2], (int32_t)ti.dims[3]};
-            const int32_t axis = 3, lanes = (int32_t)to.dims[3];
-            rc = nncase_hip_function_add_pack(m->fn, m->buffers[in0], m->buffers[dst], (int)dtype_size(ti.dtype), 4, shape, 1, &axis,
-                                              &lanes);
+            const int32_t axes[3] = {1, 2, 3}, lanes[3] = {2, 2, 4}, lanes_c = (int32_t)to.dims[3];
+            const int32_t n_axes = blocks ? 3 : 1;
+            const int32_t *ax = blocks ? axes : axes + 2, *ln = blocks ? lanes : &lanes_c;
+            if (fused_quant[k] >= 0) {
+                const uint32_t src = (uint32_t)ops[fused_quant[k]].inputs[0];
+                rc = nncase_hip_function_add_quantize_pack(m->fn, static_cast<const float *>(m->buffers[src]),
+                                                           static_cast<uint8_t *>(m->buffers[dst]), 4, shape, n_axes, ax, ln, tqp(in0));
+            } else {
+                rc = nncase_hip_function_add_pack(m->fn, m->buffers[in0], m->buffers[dst], (int)dtype_size(ti.dtype), 4, shape, n_axes, ax, ln);
+            }
             break;
         }
         default:

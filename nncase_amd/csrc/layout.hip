@@ -48,15 +48,80 @@ template <typename T> __global__ __launch_bounds__(kLayoutThreads) void pack_ker
     out[gid] = ok ? in[off] : (T)0;
 }
 
-// out[row] = the `c` (<= 4) bytes of row `row`, zero-extended to a dword.
-__global__ __launch_bounds__(kLayoutThreads) void pad_bytes_to_dword_kernel(const uint8_t *__restrict__ in,
-                                                                          uint32_t *__restrict__ out, uint32_t rows, int c) {
-    const uint32_t r = blockIdx.x * kLayoutThreads + threadIdx.x;
-    if (r >= rows) return;
-    const uint8_t *p = in + (size_t)r * c;
+// Pixels of c <= 4 elements -> 4-byte pixels, the missing channels zero; with FOLD = 2 the four pixels of a 2 x 2
+// block become one 16-byte pixel of the half-size image, (dy, dx) major: out[n][y][x] = {in[n][2y][2x], in[n][2y][2x+1],
+// in[n][2y+1][2x], in[n][2y+1][2x+1]}, which is what pack by lanes (2, 2, 4) on the (H, W, C) axes of an NHWC tensor
+// writes.  Float input is quantised to u8 on the way (Quantize, then Pack, in one pass).  One thread per output pixel;
+// rows counts image rows over the whole batch (H is even, so a block never straddles two images).
+template <typename TIn> __device__ __forceinline__ uint32_t pixel_to_dword(const TIn *p, int c, float scale, float bias) {
     uint32_t v = 0;
-    for (int i = 0; i < c; i++) v |= (uint32_t)p[i] << (8 * i);
-    out[r] = v;
+    for (int i = 0; i < c; i++) {
+        uint32_t b;
+        if constexpr (std::is_same<TIn, float>::value) b = quantize_one<uint8_t>(p[i], scale, bias);
+        else b = p[i];
+        v |= b << (8 * i);
+    }
+    return v;
+}
+
+template <typename TIn, int FOLD>
+__global__ __launch_bounds__(kLayoutThreads) void pack_pixels_kernel(const TIn *__restrict__ in, uint32_t *__restrict__ out, uint32_t total,
+                                                                   uint32_t w_out, FastDiv d_w, int c, float scale, float bias) {
+    const uint32_t gid = blockIdx.x * kLayoutThreads + threadIdx.x;
+    if (gid >= total) return;
+    if constexpr (FOLD == 1) {
+        out[gid] = c == 3 ? pixel_to_dword(in + (size_t)gid * 3, 3, scale, bias) : pixel_to_dword(in + (size_t)gid * c, c, scale, bias);
+    } else {
+        const uint32_t r = fastdiv(gid, d_w), x = gid - r * w_out;
+        typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+        u32x4 v;
+#pragma unroll
+        for (int dy = 0; dy < 2; dy++) {
+            const size_t pix = (size_t)(2 * r + dy) * (2 * w_out) + 2 * x;
+            if (c == 3) { // (the uniform special case lets the loads of a row's six elements be scheduled together)
+                TIn e[6];
+#pragma unroll
+                for (int i = 0; i < 6; i++) e[i] = in[pix * 3 + i];
+                v[dy * 2] = pixel_to_dword(e, 3, scale, bias);
+                v[dy * 2 + 1] = pixel_to_dword(e + 3, 3, scale, bias);
+            } else {
+                v[dy * 2] = pixel_to_dword(in + pix * c, c, scale, bias);
+                v[dy * 2 + 1] = pixel_to_dword(in + (pix + 1) * c, c, scale, bias);
+            }
+        }
+        reinterpret_cast<u32x4 *>(out)[gid] = v;
+    }
+}
+
+// The two layouts the stem convolutions read: NHWC with <= 4 channels packed by (4) on C or by (2, 2, 4) on (H, W, C).
+// Returns 1 when the arguments are neither.
+template <typename TIn>
+static int launch_pack_pixels(nncase_hip_ctx *ctx, const TIn *in, void *out, int rank, const int32_t *shape, int n_axes, const int *nax,
+                              const int32_t *lanes, float scale, float bias) {
+    if (shape[rank - 1] > 4 || (reinterpret_cast<uintptr_t>(out) & 15u) != 0) return 1;
+    uint64_t rows = 1;
+    for (int i = 0; i < rank - 1; i++) rows *= (uint64_t)shape[i];
+    const int c = shape[rank - 1];
+    if (n_axes == 1 && nax[0] == rank - 1 && lanes[0] == 4) {
+        NNHIP_REQUIRE(ctx, rows < ((uint64_t)1 << 31), -EINVAL, "pack: tensor too large");
+        if (rows == 0) return 0;
+        hipLaunchKernelGGL((pack_pixels_kernel<TIn, 1>), dim3((unsigned)((rows + kLayoutThreads - 1) / kLayoutThreads)), dim3(kLayoutThreads),
+                           0, ctx->stream, in, (uint32_t *)out, (uint32_t)rows, 1u, make_fastdiv(1), c, scale, bias);
+        NNHIP_LAUNCH_CHECK(ctx, "pack_pixels_kernel");
+        return 0;
+    }
+    if (rank == 4 && n_axes == 3 && nax[0] == 1 && nax[1] == 2 && nax[2] == 3 && lanes[0] == 2 && lanes[1] == 2 && lanes[2] == 4 &&
+        shape[1] % 2 == 0 && shape[2] % 2 == 0) {
+        const uint64_t total = rows / 4;
+        NNHIP_REQUIRE(ctx, rows < ((uint64_t)1 << 31), -EINVAL, "pack: tensor too large");
+        if (total == 0) return 0;
+        const uint32_t w_out = (uint32_t)shape[2] / 2;
+        hipLaunchKernelGGL((pack_pixels_kernel<TIn, 2>), dim3((unsigned)((total + kLayoutThreads - 1) / kLayoutThreads)), dim3(kLayoutThreads),
+                           0, ctx->stream, in, (uint32_t *)out, (uint32_t)total, w_out, make_fastdiv(w_out), c, scale, bias);
+        NNHIP_LAUNCH_CHECK(ctx, "pack_pixels_kernel");
+        return 0;
+    }
+    return 1;
 }
 
 template <typename T> __global__ __launch_bounds__(kLayoutThreads) void unpack_kernel(const T *in, T *out, const PackDesc d) {
@@ -147,19 +212,10 @@ extern "C" int nncase_hip_pack(nncase_hip_ctx_t *ctx, const void *in_dev, void *
     int nax[kMaxRank];
     int rc = build_common(ctx, rank, shape, n_axes, axes, lanes, nax);
     if (rc) return rc;
-    // Padding the innermost axis of bytes to one 4-byte lane block (RGB -> RGBX in front of a conv):
-    // one thread per pixel, a dword store.
-    if (elem_size == 1 && n_axes == 1 && nax[0] == rank - 1 && lanes[0] == 4 && shape[rank - 1] <= 4 &&
-        (reinterpret_cast<uintptr_t>(out_dev) & 3u) == 0) {
-        uint64_t rows = 1;
-        for (int i = 0; i < rank - 1; i++) rows *= (uint64_t)shape[i];
-        NNHIP_REQUIRE(ctx, rows < ((uint64_t)1 << 31), -EINVAL, "pack: tensor too large");
-        if (rows == 0) return 0;
-        hipLaunchKernelGGL(pad_bytes_to_dword_kernel, dim3((unsigned)((rows + kLayoutThreads - 1) / kLayoutThreads)),
-                           dim3(kLayoutThreads), 0, ctx->stream, (const uint8_t *)in_dev, (uint32_t *)out_dev, (uint32_t)rows,
-                           (int)shape[rank - 1]);
-        NNHIP_LAUNCH_CHECK(ctx, "pad_bytes_to_dword_kernel");
-        return 0;
+    // the stem layouts (RGB -> RGBX, and 2 x 2 blocks of RGBX pixels -> 16-channel pixels): one thread per output pixel
+    if (elem_size == 1) {
+        rc = launch_pack_pixels<uint8_t>(ctx, (const uint8_t *)in_dev, out_dev, rank, shape, n_axes, nax, lanes, 1.f, 0.f);
+        if (rc <= 0) return rc;
     }
     PackDesc d;
     memset(&d, 0, sizeof(d));
@@ -197,6 +253,21 @@ extern "C" int nncase_hip_pack(nncase_hip_ctx_t *ctx, const void *in_dev, void *
         NNHIP_LAUNCH_CHECK(ctx, "pack_kernel");
         return 0;
     });
+}
+
+extern "C" int nncase_hip_quantize_pack(nncase_hip_ctx_t *ctx, const float *in_dev, uint8_t *out_dev, int32_t rank, const int32_t *shape,
+                                        int32_t n_axes, const int32_t *axes, const int32_t *lanes, nncase_hip_quant_param_t qp) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, in_dev && out_dev, -EINVAL, "quantize_pack: null buffer");
+    NNHIP_REQUIRE(ctx, qp.scale != 0.f, -EINVAL, "quantize_pack: scale is zero");
+    int nax[kMaxRank];
+    int rc = build_common(ctx, rank, shape, n_axes, axes, lanes, nax);
+    if (rc) return rc;
+    rc = launch_pack_pixels<float>(ctx, in_dev, out_dev, rank, shape, n_axes, nax, lanes, qp.scale, (float)qp.zero_point);
+    if (rc <= 0) return rc;
+    return fail(ctx, -EINVAL,
+                "quantize_pack: only <= 4 innermost channels packed by (4), or NHWC with even H and W packed by (2, 2, 4) on (H, W, C), "
+                "into a 16-byte aligned buffer");
 }
 
 extern "C" int nncase_hip_unpack(nncase_hip_ctx_t *ctx, const void *in_dev, void *out_dev, int32_t elem_size, int32_t rank,

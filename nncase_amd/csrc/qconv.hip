@@ -35,13 +35,12 @@ void nnhip::describe_conv_kernel(const nncase_hip_ctx *ctx, const nncase_hip_wei
     const int mode = igemm_load_mode(w, a, out_h, out_w);
     const int mi = (int)std::min<long long>(m, 1 << 30);
     if (w->wide) {
-        snprintf(buf, cap, "qconv_wide%s%s<T=%d,%s>", w->d_post_lut ? "+lut" : "", a->residual_dev ? "+add" : "", w->tiles, modes[mode]);
+        snprintf(buf, cap, "qconv_wide%s%s<T=%d,%s%s>", w->d_post_lut ? "+lut" : "", a->residual_dev ? "+add" : "", w->tiles,
+                 w->wide == 2 ? "RG=2," : "", modes[mode]);
         return;
     }
-    const bool stream = igemm_streams_weights(w, mode);
-    snprintf(buf, cap, "qconv_igemm%s%s%s<T=%d,RG=%d,%s>", stream ? "_stream" : "", w->d_post_lut ? "+lut" : "",
-             a->residual_dev ? "+add" : "", w->tiles, stream ? stream_pixel_groups(ctx, w, mi) : igemm_pixel_groups(ctx, w, mi),
-             modes[mode]);
+    snprintf(buf, cap, "qconv_igemm%s%s<T=%d,RG=%d,%s>", w->d_post_lut ? "+lut" : "", a->residual_dev ? "+add" : "", w->tiles,
+             igemm_pixel_groups(ctx, w, mi), modes[mode]);
 }
 
 float nnhip::reciprocal_rn(float b) {

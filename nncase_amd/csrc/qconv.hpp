@@ -16,7 +16,9 @@ struct nncase_hip_weights {
     // igemm, reductions of at most 32: the spare half of the only k-step holds -(zw - 128) against a second copy
     // of the activations, which makes the weight zero point's share of the product part of the multiplication
     int fold = 0;
-    // igemm: packed for the wide-tile kernels (qconv_wide.hpp): long reductions over many pixels and channels
+    // igemm: packed for the wide-tile kernels (qconv_wide.hpp): 1 = long reductions over many pixels and channels
+    // (blocks of 256 or 128 pixels, waves of 64), 2 = reductions of five k-steps and more over fewer pixels (blocks of
+    // 128 pixels x 64 channels or 64 x 32, waves of 32 pixels)
     int wide = 0;
     long long dw_const_bound = 0; // depthwise: max over channels of |bias| + 255 |sum(w - zw)|
     int64_t pixels_hint = 0; // output pixels per call the tiling was planned for (0 = unknown)
@@ -98,8 +100,6 @@ int launch_qconv_depthwise(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_h
 void describe_conv_kernel(const nncase_hip_ctx *ctx, const nncase_hip_weights *w, const nncase_hip_conv2d_args_t *a, char *buf,
                           size_t cap);
 int igemm_pixel_groups(const nncase_hip_ctx *ctx, const nncase_hip_weights *w, int m);
-bool igemm_streams_weights(const nncase_hip_weights *w, int mode);
-int stream_pixel_groups(const nncase_hip_ctx *ctx, const nncase_hip_weights *w, int m);
 int igemm_load_mode(const nncase_hip_weights *w, const nncase_hip_conv2d_args_t *c, int out_h, int out_w);
 } // namespace nnhip
 // Writes the name of the kernel a fused block launches.

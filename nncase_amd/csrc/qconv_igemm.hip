@@ -68,6 +68,16 @@ int prepack_igemm(nncase_hip_ctx *ctx, nncase_hip_weights *w, const uint8_t *w_o
             w->kc_steps = std::min(w->ksteps, kLdsFrags / w->tiles);
         }
     }
+    // Reductions of kSmallWideMinKsteps k-steps and more over fewer pixels take the same kernel with 128 x 64 blocks
+    // (four waves of 32 pixels) or 64 x 32 ones: against the small tiles' per-lane loads of 16 pixels' slices, the
+    // row-order fetch through LDS needs a quarter of the requests to the vector L1, which is what such launches
+    // are bound by.
+    if (!w->wide && w->g_ic % 16 == 0 && w->ksteps >= kSmallWideMinKsteps) {
+        w->wide = 2;
+        w->tiles = w->g_oc <= 32 ? 2 : 4;
+        w->nchunks = ceil_div(w->g_oc, w->tiles * 16);
+        w->kc_steps = std::min(w->ksteps, kLdsFrags / w->tiles);
+    }
     // -(zw - 128) has to be an s8 value
     w->fold = w->ksteps == 1 && w->k <= 32 && w->zw >= 1;
     const size_t group_bytes = (size_t)w->nchunks * w->ksteps * w->tiles * 1024;
@@ -96,16 +106,6 @@ int prepack_igemm(nncase_hip_ctx *ctx, nncase_hip_weights *w, const uint8_t *w_o
 
 int igemm_pixel_groups(const nncase_hip_ctx *ctx, const nncase_hip_weights *w, int m) {
     return choose_rg(ctx, w->tiles, w->nchunks, m);
-}
-
-// Weights that do not fit the LDS budget at once are streamed through it (16-byte loaders only).
-bool igemm_streams_weights(const nncase_hip_weights *w, int mode) {
-    return !w->wide && w->kc_steps < w->ksteps && w->tiles <= 4 && (mode == kRows16 || mode == kVec16);
-}
-
-// Two pixel groups per wave halve the LDS traffic per multiply; taken when that still leaves a block per CU.
-int stream_pixel_groups(const nncase_hip_ctx *ctx, const nncase_hip_weights *w, int m) {
-    return (long long)ceil_div(m, kWaves * 2 * 16) * w->nchunks >= ctx->compute_units ? 2 : 1;
 }
 
 int igemm_load_mode(const nncase_hip_weights *w, const nncase_hip_conv2d_args_t *c, int out_h, int out_w) {
@@ -189,15 +189,13 @@ int launch_qconv_igemm(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_hip_w
         a.y_coff = g * w->g_oc + c->out_channel_offset;
         a.r_coff = g * w->g_oc;
         int rc;
-        if (w->wide) {
-            rc = mode == kRows16 ? launch_wide_rows16(ctx, a, w->tiles, w->nchunks) : launch_wide_vec16(ctx, a, w->tiles, w->nchunks);
+        if (w->wide == 2) {
+            rc = mode == kRows16 ? launch_wide_small_rows16(ctx, a, w->tiles, w->nchunks) : launch_wide_small_vec16(ctx, a, w->tiles, w->nchunks);
             if (rc) return rc;
             continue;
         }
-        if (igemm_streams_weights(w, mode)) {
-            const int rg = stream_pixel_groups(ctx, w, a.m);
-            rc = mode == kRows16 ? launch_igemm_stream_rows16(ctx, a, w->tiles, w->nchunks, rg)
-                                 : launch_igemm_stream_vec16(ctx, a, w->tiles, w->nchunks, rg);
+        if (w->wide) {
+            rc = mode == kRows16 ? launch_wide_rows16(ctx, a, w->tiles, w->nchunks) : launch_wide_vec16(ctx, a, w->tiles, w->nchunks);
             if (rc) return rc;
             continue;
         }

@@ -33,6 +33,8 @@
 //   kBytes   anything else (e.g. 3 input channels): byte gathers
 #pragma once
 
+#include <type_traits>
+
 #include "qconv.hpp"
 
 namespace nnhip {
@@ -772,146 +774,6 @@ template <int T, int RG, bool ROWS> __global__ void __launch_bounds__(kThreads, 
         for (int rg = 0; rg < RG; rg++) poff[rg] = poff_next[rg];
     }
 }
-
-// ---- long reductions: weights streamed through LDS -----------------------------------------------
-// When the weights of a channel chunk do not fit the LDS budget (3x3 and larger windows over many
-// channels), they are streamed: every k-step's T fragments go global -> registers -> a three-slot LDS
-// ring, one barrier per k-step, and both the weights and the activation slices are requested three
-// k-steps before they are multiplied.  With one or two blocks per compute unit there are too few
-// waves to hide memory latency by switching waves, so the latency has to be covered inside the wave;
-// a one-step prefetch exposes a full memory round trip per k-step on such layers.
-template <int T, int RG, int MODE>
-__global__ __launch_bounds__(kThreads, 2) void qconv_igemm_stream_kernel(const IgemmArgs a) {
-    // three ring slots: the one being multiplied, the one being written, and one in between
-    constexpr int WV = T * 64;                             // 16-byte vectors of weights per k-step
-    constexpr int NW = (WV + kThreads - 1) / kThreads;     // ... per thread
-    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    int32_t *cterm = reinterpret_cast<int32_t *>(smem);   // [T * 16]
-    uint8_t *lutl = smem + T * 16 * sizeof(int32_t);      // [256]
-    uint8_t *wring = lutl + 256;                           // [NSLOT][T][1024]
-
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const int j = lane & 15, gq = lane >> 4;
-    const int chunk = blockIdx.y;
-    const int ch_base = chunk * (T * 16);
-    const u32x4 *wsrc = reinterpret_cast<const u32x4 *>(a.wpk + (size_t)chunk * a.ksteps * T * 1024);
-    const int KS = a.ksteps;
-
-    for (int i = threadIdx.x; i < T * 16; i += kThreads) {
-        const int ch = ch_base + i;
-        cterm[i] = ch < a.n ? a.bias[ch] - a.zxp * a.wsum[ch] + a.k * a.zxp * a.zwp : 0;
-    }
-    if (a.lut && threadIdx.x < 64) reinterpret_cast<uint32_t *>(lutl)[threadIdx.x] = a.lut[threadIdx.x];
-
-    const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
-    constexpr int pix_per_block = kWaves * RG * 16;
-    auto load_w = [&](u32x4 (&dst)[NW], int ks) {
-#pragma unroll
-        for (int i = 0; i < NW; i++) {
-            const int v = threadIdx.x + i * kThreads;
-            if (v < WV) dst[i] = wsrc[(size_t)ks * WV + v];
-        }
-    };
-    auto store_w = [&](const u32x4 (&src)[NW], int slot) {
-        u32x4 *dst = reinterpret_cast<u32x4 *>(wring + (size_t)slot * T * 1024);
-#pragma unroll
-        for (int i = 0; i < NW; i++) {
-            const int v = threadIdx.x + i * kThreads;
-            if (v < WV) dst[v] = src[i];
-        }
-    };
-
-    for (int mt = blockIdx.x; mt < a.num_mtiles; mt += gridDim.x) {
-        PixInfo pix[RG];
-#pragma unroll
-        for (int rg = 0; rg < RG; rg++) pix[rg] = pix_info<MODE>(a, mt * pix_per_block + (wave * RG + rg) * 16 + j);
-        v4i acc[RG][T], rs[RG];
-#pragma unroll
-        for (int rg = 0; rg < RG; rg++) {
-            rs[rg] = v4i{0, 0, 0, 0};
-#pragma unroll
-            for (int nt = 0; nt < T; nt++) acc[rg][nt] = v4i{0, 0, 0, 0};
-        }
-        // ---- fill the pipeline: weights of k-steps 0..2, activation slices of k-steps 0..2 ----
-        u32x4 wreg[2][NW];
-        ActSlice af[3][RG];
-        {
-            u32x4 w0[NW];
-            load_w(w0, 0);
-            if (1 < KS) load_w(wreg[1], 1);
-            if (2 < KS) load_w(wreg[0], 2);
-#pragma unroll
-            for (int d = 0; d < 3; d++)
-#pragma unroll
-                for (int rg = 0; rg < RG; rg++) af[d][rg] = load_slice<MODE>(a, pix[rg], (d < KS ? d : 0) * 4 + gq);
-            __syncthreads(); // the previous pixel tile no longer reads the ring (and cterm is written)
-            store_w(w0, 0);
-            __syncthreads();
-        }
-        for (int s0 = 0; s0 < KS; s0 += 6) {
-#pragma unroll
-            for (int u = 0; u < 6; u++) {
-                const int s = s0 + u;
-                if (s < KS) { // uniform for the block
-                    v4i xf[RG];
-#pragma unroll
-                    for (int rg = 0; rg < RG; rg++) xf[rg] = finish_slice(af[u % 3][rg]);
-                    if (s + 3 < KS) {
-#pragma unroll
-                        for (int rg = 0; rg < RG; rg++) af[u % 3][rg] = load_slice<MODE>(a, pix[rg], (s + 3) * 4 + gq);
-                    }
-                    if (s + 1 < KS) store_w(wreg[(u + 1) % 2], (u + 1) % 3);
-                    if (s + 3 < KS) load_w(wreg[(u + 1) % 2], s + 3);
-#pragma unroll
-                    for (int rg = 0; rg < RG; rg++)
-                        rs[rg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, xf[rg], rs[rg], 0, 0, 0);
-                    const uint8_t *wstep = wring + (size_t)(u % 3) * T * 1024 + lane * 16;
-#pragma unroll
-                    for (int nt = 0; nt < T; nt++) {
-                        const v4i wf = *reinterpret_cast<const v4i *>(wstep + nt * 1024);
-#pragma unroll
-                        for (int rg = 0; rg < RG; rg++)
-                            acc[rg][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf, xf[rg], acc[rg][nt], 0, 0, 0);
-                    }
-                    __syncthreads();
-                }
-            }
-        }
-        const int ch0 = ch_base + gq * (4 * T);
-#pragma unroll
-        for (int rg = 0; rg < RG; rg++)
-            igemm_store_tile<T>(a, acc[rg], rs[rg][0], mt * pix_per_block + (wave * RG + rg) * 16 + j, ch0, gq, cterm, lutl);
-    }
-}
-
-template <int T, int RG, int MODE> int launch_stream_trg(nncase_hip_ctx *ctx, const IgemmArgs &a, int nchunks) {
-    IgemmArgs args = a;
-    constexpr int pix_per_block = kWaves * RG * 16;
-    args.num_mtiles = ceil_div(a.m, pix_per_block);
-    int gx = args.num_mtiles < ctx->compute_units * 4 ? args.num_mtiles : ctx->compute_units * 4;
-    if (nchunks > 1) gx = ceil_div(gx, 8) * 8; // chunks of one pixel tile on one XCD
-    const size_t lds = (size_t)T * 16 * sizeof(int32_t) + 256 + (size_t)3 * T * 1024;
-    hipLaunchKernelGGL((qconv_igemm_stream_kernel<T, RG, MODE>), dim3(gx, nchunks, 1), dim3(kThreads), lds, ctx->stream, args);
-    NNHIP_LAUNCH_CHECK(ctx, "qconv_igemm_stream_kernel");
-    return 0;
-}
-
-template <int MODE> int launch_stream_mode(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks, int rg) {
-#define NNHIP_STREAM_CASE(TT)                                                                                          \
-    case TT: return rg >= 2 ? launch_stream_trg<TT, 2, MODE>(ctx, a, nchunks) : launch_stream_trg<TT, 1, MODE>(ctx, a, nchunks);
-    switch (tiles) {
-        NNHIP_STREAM_CASE(1)
-        NNHIP_STREAM_CASE(2)
-        NNHIP_STREAM_CASE(3)
-        NNHIP_STREAM_CASE(4)
-    default: return fail(ctx, -EINVAL, "qconv2d: no streaming kernel for %d channel tiles", tiles);
-    }
-#undef NNHIP_STREAM_CASE
-}
-
-int launch_igemm_stream_rows16(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks, int rg);
-int launch_igemm_stream_vec16(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks, int rg);
 
 // Pixel groups per wave (RG) for a chunk width of T tiles.  The kernels are bound by the
 // VALU work of the epilogue, and a dependent VALU instruction issues only every ~8 cycles

@@ -38,6 +38,7 @@ namespace nnhip {
 // block per compute unit; below that a launch has too few 64-pixel wave tiles to fill the device and the small tiles'
 // larger wave count wins.
 constexpr int kWideMinKsteps = 8;
+constexpr int kSmallWideMinKsteps = 5; // (measured on MobileNetV2 at batch 64 and the YOLOv5s-style network at batch 16: flat from 4 to 8)
 constexpr int kWideSlots = 3;
 
 // How a thread finds its 16-byte pieces of a k-step:
@@ -348,6 +349,13 @@ template <int LM> int launch_wide_lm(nncase_hip_ctx *ctx, const IgemmArgs &a, in
     return fail(ctx, -EINVAL, "qconv2d: no wide kernel for %d channel tiles", tiles);
 }
 
+template <int LM> int launch_wide_small_lm(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks) {
+    if (tiles == 4) return launch_wide_t<4, 2, 4, 1, LM>(ctx, a, nchunks);
+    if (tiles == 2) return launch_wide_t<2, 2, 2, 1, LM>(ctx, a, nchunks);
+    return fail(ctx, -EINVAL, "qconv2d: no small wide kernel for %d channel tiles", tiles);
+}
+int launch_wide_small_rows16(nncase_hip_ctx *ctx, const IgemmArgs &a, int variant, int nchunks);
+int launch_wide_small_vec16(nncase_hip_ctx *ctx, const IgemmArgs &a, int variant, int nchunks);
 int launch_wide_rows16(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks);
 int launch_wide_vec16(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks);
 

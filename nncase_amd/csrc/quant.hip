@@ -41,20 +41,6 @@ template <typename T> __device__ __forceinline__ void store4(T *p, const T (&v)[
 template <typename T> __device__ __forceinline__ float to_f32(T v) { return (float)v; }
 template <> __device__ __forceinline__ float to_f32<__half>(__half v) { return __half2float(v); }
 
-template <typename TQ> struct QLimits;
-template <> struct QLimits<uint8_t> { static constexpr float lo = 0.f, hi = 255.f; };
-template <> struct QLimits<int8_t> { static constexpr float lo = -128.f, hi = 127.f; };
-template <> struct QLimits<int16_t> { static constexpr float lo = -32768.f, hi = 32767.f; };
-
-// rne(v) then saturate.  The clamp is done on the float before rounding: the
-// limits are integers, so clamp and round-half-even commute, and values
-// beyond the int32 range saturate instead of wrapping.
-template <typename TQ> __device__ __forceinline__ TQ quantize_one(float x, float scale, float bias) {
-    float v = x / scale + bias;
-    v = fminf(fmaxf(v, QLimits<TQ>::lo), QLimits<TQ>::hi); // NaN -> lo
-    return (TQ)(int32_t)rintf(v);
-}
-
 template <typename TIn, typename TQ>
 __global__ __launch_bounds__(kEwThreads) void quantize_kernel(const TIn *__restrict__ in, TQ *__restrict__ out,
                                                               size_t count, float scale, float bias, int vec_ok) {

@@ -423,6 +423,8 @@ def compile_quant_graph(qg, batch: int, stackvm_main: bool = False) -> bytes:
             ops.append(HipOp(OP_MAXPOOL, ins, tid, p=(n.pool[0], n.pool[1], n.pool[2])))
         elif n.op == "padc":
             ops.append(HipOp(OP_PAD_CHANNELS, ins, tid))
+        elif n.op == "s2d":        # channel padding to 4 and 2 x 2 pixel blocks to 16-channel pixels (extents say which)
+            ops.append(HipOp(OP_PAD_CHANNELS, ins, tid))
         elif n.op == "fold2":      # the same NHWC bytes with other extents: the tensor shares its input's buffer
             ops.append(HipOp(OP_RESHAPE, ins, tid))
         else:

@@ -334,14 +334,28 @@ def pad_small_channel_convs(qg: QuantGraph) -> QuantGraph:
             wpad = np.full((n.weights.shape[0], 4) + n.weights.shape[2:], n.w_qp[0], np.uint8)
             wpad[:, :c] = n.weights
             n.weights, n.inputs = wpad, (len(nodes) - 1,)
-            # Stride 2 along the width over an even window: two neighbouring 4-channel pixels are one 8-channel pixel
-            # of the half-width image in the same NHWC bytes ("fold2": nothing moves), and the conv becomes one of
-            # stride 1 along the width over half as many taps: out(y, x) = sum over ky, kx', (dx, c) of
-            # in[sy y + ky - ph][2 (x + kx' - pw / 2) + dx][c] w[ky][2 kx' + dx][c].  The loader then fetches 8 bytes
-            # per tap instead of 4 and computes half as many tap addresses.
             kh, kw = n.weights.shape[2:]
             (ph0, ph1), (pw0, pw1) = n.padding
-            if n.stride[1] == 2 and kw % 2 == 0 and w % 2 == 0 and pw0 % 2 == 0 and pw1 % 2 == 0:
+            if (tuple(n.stride) == (2, 2) and kh % 2 == 0 and kw % 2 == 0 and h % 2 == 0 and w % 2 == 0
+                    and all(p % 2 == 0 for p in (ph0, ph1, pw0, pw1))):
+                # Stride 2 over an even window: every 2 x 2 block of 4-channel pixels becomes one 16-channel pixel of the
+                # half-size image ("s2d": pack by lanes (2, 2, 4) on (H, W, C), channel order (dy, dx, c)), and the conv
+                # becomes one of stride 1 over half the window in both directions:
+                # out(y, x) = sum over ky', kx', (dy, dx, c) of in[2 (y + ky' - ph / 2) + dy][2 (x + kx' - pw / 2) + dx][c]
+                #             w[2 ky' + dy][2 kx' + dx][c].  The loader then fetches 16 bytes per tap and computes a quarter
+                # as many tap addresses; the padding is whole blocks, filled with the input's zero point as before.
+                nodes[-1] = QNode("s2d", nodes[-1].inputs, n.name + ".s2d", src.out_qp, (16, h // 2, w // 2))
+                wf = np.empty((wpad.shape[0], 16, kh // 2, kw // 2), np.uint8)
+                for dy in range(2):
+                    for dx in range(2):
+                        wf[:, (dy * 2 + dx) * 4:(dy * 2 + dx) * 4 + 4] = wpad[:, :, dy::2, dx::2]
+                n.weights = wf
+                n.stride = (1, 1)
+                n.padding = ((ph0 // 2, ph1 // 2), (pw0 // 2, pw1 // 2))
+            elif n.stride[1] == 2 and kw % 2 == 0 and w % 2 == 0 and pw0 % 2 == 0 and pw1 % 2 == 0:
+                # Stride 2 along the width only: two neighbouring 4-channel pixels are one 8-channel pixel of the
+                # half-width image in the same NHWC bytes ("fold2": nothing moves), and the conv becomes one of stride 1
+                # along the width over half as many taps.
                 nodes.append(QNode("fold2", (len(nodes) - 1,), n.name + ".fold2", src.out_qp, (8, h, w // 2)))
                 wf = np.empty((wpad.shape[0], 8, kh, kw // 2), np.uint8)
                 for dx in range(2):
@@ -489,6 +503,16 @@ class HipModel:
                         self.write_through[conv] = (ci, off, ctot, table)
                         self.never_written |= {conv, j} | ({self.fused_lut[conv]} if conv in self.fused_lut else set())
                     off += ch
+        # The quantisation of the float input is done by the pack operator behind it (RGB -> RGBX or 2 x 2 blocks ->
+        # 16-channel pixels in front of a stem conv) when nothing else reads the quantised RGB tensor.
+        self.fused_quant: Dict[int, int] = {}                                            # pack node -> input node
+        if fuse_residual:
+            for i, n in enumerate(qg.nodes):
+                j = n.inputs[0] if n.inputs else -1
+                if n.op in ("padc", "s2d") and qg.nodes[j].op == "input" and consumers[j] == 1 and j not in qg.output_nodes:
+                    self.fused_quant[i] = j
+                    self.never_written.add(j)
+                    skip_nodes.add(j)
         # buffers and packed weights once, shared by the lanes
         for i, n in enumerate(qg.nodes):
             cc, hh, ww = n.out_shape
@@ -499,7 +523,7 @@ class HipModel:
             if n.op == "fold2":
                 self.buffers.append(self.buffers[n.inputs[0]])  # the same bytes read as half as many, twice as deep pixels
                 continue
-            if i in self.blocks or i - 1 in self.blocks or i in self.write_through:
+            if i in self.blocks or i - 1 in self.blocks or i in self.write_through or i in self.fused_quant.values():
                 self.buffers.append(ctx.alloc(16))        # expanded tensors of a fused block live in LDS only; a conv
                 #                                           that writes into its concat has no tensor of its own
             else:
@@ -612,9 +636,15 @@ class HipModel:
                 k, st, p = n.pool
                 self.fn.add_qmaxpool2d(B(n.inputs[0]), buf, bl, src.out_shape[1], src.out_shape[2], cc, (k, k), (st, st),
                                        ((p, p), (p, p)), qp(*src.out_qp), qp(*n.out_qp))
-            elif n.op == "padc":
+            elif n.op in ("padc", "s2d"):
                 src = qg.nodes[n.inputs[0]]
-                self.fn.add_pack(B(n.inputs[0]), buf, 1, [bl, hh, ww, src.out_shape[0]], [3], [cc])
+                sc, sh_, sw_ = src.out_shape
+                axes, lns = ([3], [cc]) if n.op == "padc" else ([1, 2, 3], [2, 2, 4])
+                if i in self.fused_quant:
+                    self.fn.add_quantize_pack(self.input_f32.view(lane * self._lane_stride(in_per * 4), in_per * 4), buf,
+                                              [bl, sh_, sw_, sc], axes, lns, qp(*src.out_qp))
+                else:
+                    self.fn.add_pack(B(n.inputs[0]), buf, 1, [bl, sh_, sw_, sc], axes, lns)
             elif n.op == "fold2":
                 continue
             elif n.op == "gap":

@@ -130,6 +130,7 @@ SYMBOLS = {
     "nncase_hip_qmaxpool2d": (_I, [_VP, _VP, _VP] + [C.c_int32] * 12 + [QuantParam, QuantParam]),
     "nncase_hip_function_add_qmaxpool2d": (_I, [_VP, _VP, _VP] + [C.c_int32] * 12 + [QuantParam, QuantParam]),
     "nncase_hip_function_add_pack": (_I, [_VP, _VP, _VP, C.c_int32, C.c_int32, _I32P, C.c_int32, _I32P, _I32P]),
+    "nncase_hip_function_add_quantize_pack": (_I, [_VP, _VP, _VP, C.c_int32, _I32P, C.c_int32, _I32P, _I32P, QuantParam]),
     "nncase_hip_w8a16_prepack": (_I, [_VP, _VP, _VP, _VP, C.c_int32, C.c_int32, C.POINTER(_VP)]),
     "nncase_hip_w8a16_destroy": (_I, [_VP, _VP]),
     "nncase_hip_w8a16_gemm": (_I, [_VP, _VP, _VP, _VP, C.c_int32, C.c_int32, _VP, C.c_int32]),
@@ -155,6 +156,7 @@ SYMBOLS = {
     "nncase_hip_kmodel_tensor": (_I, [_VP, C.c_int32, C.POINTER(_VP), _I32P, _I32P]),
     "nncase_hip_pack": (_I, [_VP, _VP, _VP, C.c_int32, C.c_int32, _I32P, C.c_int32, _I32P, _I32P]),
     "nncase_hip_unpack": (_I, [_VP, _VP, _VP, C.c_int32, C.c_int32, _I32P, C.c_int32, _I32P, _I32P]),
+    "nncase_hip_quantize_pack": (_I, [_VP, _VP, _VP, C.c_int32, _I32P, C.c_int32, _I32P, _I32P, QuantParam]),
     "nncase_hip_nchw_to_nhwc": (_I, [_VP, _VP, _VP, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
     "nncase_hip_nhwc_to_nchw": (_I, [_VP, _VP, _VP, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
     "nncase_hip_paged_attention_decode": (_I, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, C.POINTER(PagedAttnArgs)]),
@@ -531,6 +533,12 @@ class Context:
         sh, ax, ln = (C.c_int32 * len(shape))(*shape), (C.c_int32 * max(1, len(axes)))(*axes), (C.c_int32 * max(1, len(lanes)))(*lanes)
         self._check(self.lib.nncase_hip_pack(self.handle, src.ptr, dst.ptr, elem_size, len(shape), sh, len(axes), ax, ln), "pack")
 
+    def quantize_pack(self, src: DeviceBuffer, dst: DeviceBuffer, shape: Sequence[int], axes: Sequence[int], lanes: Sequence[int],
+                      q: QuantParam):
+        """float32 -> u8 quantize and pack in one pass (the layouts in front of a stem convolution)."""
+        sh, ax, ln = (C.c_int32 * len(shape))(*shape), (C.c_int32 * max(1, len(axes)))(*axes), (C.c_int32 * max(1, len(lanes)))(*lanes)
+        self._check(self.lib.nncase_hip_quantize_pack(self.handle, src.ptr, dst.ptr, len(shape), sh, len(axes), ax, ln, q), "quantize_pack")
+
     def unpack(self, src: DeviceBuffer, dst: DeviceBuffer, elem_size: int, unpacked_shape: Sequence[int],
                axes: Sequence[int], lanes: Sequence[int]):
         sh = (C.c_int32 * len(unpacked_shape))(*unpacked_shape)
@@ -658,6 +666,12 @@ class Function:
         sh, ax, ln = (C.c_int32 * len(shape))(*shape), (C.c_int32 * max(1, len(axes)))(*axes), (C.c_int32 * max(1, len(lanes)))(*lanes)
         self._ck(self.ctx.lib.nncase_hip_function_add_pack(self.handle, src.ptr, dst.ptr, elem_size, len(shape), sh, len(axes), ax, ln),
                  "function_add_pack")
+
+    def add_quantize_pack(self, src, dst, shape, axes, lanes, q: QuantParam):
+        self._keep += [src, dst]
+        sh, ax, ln = (C.c_int32 * len(shape))(*shape), (C.c_int32 * max(1, len(axes)))(*axes), (C.c_int32 * max(1, len(lanes)))(*lanes)
+        self._ck(self.ctx.lib.nncase_hip_function_add_quantize_pack(self.handle, src.ptr, dst.ptr, len(shape), sh, len(axes), ax, ln, q),
+                 "function_add_quantize_pack")
 
     def add_w8a16_gemm(self, a, w, out, m, mode=GEMM_PLAIN, residual=None, out_dtype=DT_F16):
         self._keep += [a, w, out] + ([residual] if residual is not None else [])

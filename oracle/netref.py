@@ -60,6 +60,11 @@ def run_integer(qg, x_nhwc: np.ndarray, keep_all: bool = False):
         elif n.op == "padc":
             v = outs[n.inputs[0]]
             y = np.pad(v, ((0, 0), (0, n.out_shape[0] - v.shape[1]), (0, 0), (0, 0)))
+        elif n.op == "s2d":       # 2 x 2 pixel blocks of <= 4 channels -> 16 channels: y[:, (dy * 2 + dx) * 4 + c, y', x'] = v[:, c, 2 y' + dy, 2 x' + dx]
+            v = outs[n.inputs[0]]
+            nb_, c_, h_, w_ = v.shape
+            v4 = np.pad(v, ((0, 0), (0, 4 - c_), (0, 0), (0, 0)))
+            y = np.ascontiguousarray(v4.reshape(nb_, 4, h_ // 2, 2, w_ // 2, 2).transpose(0, 3, 5, 1, 2, 4).reshape(nb_, 16, h_ // 2, w_ // 2))
         elif n.op == "fold2":     # pixel pairs along the width become channels: y[:, dx * C + c, :, x] = v[:, c, :, 2 x + dx]
             v = outs[n.inputs[0]]
             nb_, c_, h_, w_ = v.shape
@@ -107,6 +112,11 @@ def run_float_chain(qg, x_nhwc: np.ndarray, keep_all: bool = False):
         elif n.op == "padc":
             v = outs[n.inputs[0]]
             y = np.pad(v, ((0, 0), (0, n.out_shape[0] - v.shape[1]), (0, 0), (0, 0)))
+        elif n.op == "s2d":       # 2 x 2 pixel blocks of <= 4 channels -> 16 channels: y[:, (dy * 2 + dx) * 4 + c, y', x'] = v[:, c, 2 y' + dy, 2 x' + dx]
+            v = outs[n.inputs[0]]
+            nb_, c_, h_, w_ = v.shape
+            v4 = np.pad(v, ((0, 0), (0, 4 - c_), (0, 0), (0, 0)))
+            y = np.ascontiguousarray(v4.reshape(nb_, 4, h_ // 2, 2, w_ // 2, 2).transpose(0, 3, 5, 1, 2, 4).reshape(nb_, 16, h_ // 2, w_ // 2))
         elif n.op == "fold2":     # pixel pairs along the width become channels: y[:, dx * C + c, :, x] = v[:, c, :, 2 x + dx]
             v = outs[n.inputs[0]]
             nb_, c_, h_, w_ = v.shape

@@ -19,6 +19,11 @@ pytestmark = pytest.mark.gpu
     ((2, 9, 11, 3), [3], [4], np.uint8),           # RGB -> RGBX: the dword fast path
     ((5, 7, 1), [2], [4], np.uint8),
     ((4, 6, 4), [-1], [4], np.uint8),              # already 4 wide
+    ((2, 6, 10, 3), [1, 2, 3], [2, 2, 4], np.uint8),   # 2 x 2 blocks of RGB -> 16-channel pixels: one thread per block
+    ((3, 4, 2, 1), [1, 2, 3], [2, 2, 4], np.uint8),
+    ((1, 8, 6, 4), [1, 2, 3], [2, 2, 4], np.uint8),
+    ((2, 5, 6, 3), [1, 2, 3], [2, 2, 4], np.uint8),    # odd height: the general kernel
+    ((2, 6, 10, 3), [2, 1, 3], [2, 2, 4], np.uint8),   # lanes in another order: the general kernel
 ])
 def test_pack_unpack(hip_ctx, shape, axes, lanes, dtype):
     rng = np.random.default_rng(len(shape) + shape[0])
@@ -36,6 +41,38 @@ def test_pack_roundtrip_full_size(hip_ctx):
     y = K.pack(x, [1], [64], ctx=hip_ctx)
     assert y.shape == (32, 3, 56, 56, 64) and (y[:, 2, :, :, 16:] == 0).all()
     assert np.array_equal(K.unpack(y, [1], [64], x.shape, ctx=hip_ctx), x)
+
+
+@pytest.mark.parametrize("shape,axes,lanes", [
+    ((2, 6, 10, 3), [1, 2, 3], [2, 2, 4]), ((1, 64, 48, 3), [1, 2, 3], [2, 2, 4]), ((3, 2, 2, 1), [1, 2, -1], [2, 2, 4]),
+    ((2, 4, 6, 4), [1, 2, 3], [2, 2, 4]), ((2, 9, 11, 3), [3], [4]), ((7, 2), [1], [4]), ((5, 4), [-1], [4])])
+def test_quantize_pack_equals_quantize_then_pack(hip_ctx, shape, axes, lanes):
+    """Quantize and Pack in one pass over a float32 tensor == the two operators one after the other (oracle: quantize,
+    then pack), for the two layouts that stand in front of a stem convolution; values beyond the u8 range, halves that
+    round to even included."""
+    from nncase_amd.runtime import qp
+    rng = np.random.default_rng(sum(shape))
+    x = ((rng.random(shape, dtype=np.float32) - 0.3) * 3).astype(np.float32)
+    flat = x.reshape(-1)
+    flat[::7] = (np.arange(flat[::7].size) - 3 + 0.5).astype(np.float32) * np.float32(0.0125)     # exact halves before rounding
+    scale, zp = np.float32(0.0125), 17
+    want = O.pack(O.quantize(x, scale, zp, O.U8), axes, lanes)
+    src, dst = hip_ctx.to_device(x), hip_ctx.alloc(want.size)
+    hip_ctx.quantize_pack(src, dst, list(shape), axes, lanes, qp(zp, scale))
+    assert np.array_equal(dst.download(want.shape, np.uint8), want)
+
+
+def test_quantize_pack_refuses_other_layouts(hip_ctx):
+    from nncase_amd import runtime as rt
+    src, dst = hip_ctx.alloc(4 * 2 * 6 * 10 * 8), hip_ctx.alloc(2 * 6 * 10 * 8)
+    for shape, axes, lanes, q in (((2, 6, 10, 8), [3], [4], rt.qp(0, 1.0)),            # more than 4 channels
+                                  ((2, 5, 10, 3), [1, 2, 3], [2, 2, 4], rt.qp(0, 1.0)),   # odd height
+                                  ((2, 6, 10, 3), [2, 1, 3], [2, 2, 4], rt.qp(0, 1.0)),   # another lane order
+                                  ((2, 6, 10, 3), [3], [8], rt.qp(0, 1.0)),
+                                  ((2, 6, 10, 3), [3], [4], rt.qp(0, 0.0))):             # zero scale
+        with pytest.raises(rt.HipError) as e:
+            hip_ctx.quantize_pack(src, dst, list(shape), axes, lanes, q)
+        assert e.value.code == -22
 
 
 @pytest.mark.parametrize("shape", [(1, 3, 224, 224), (2, 144, 7, 5), (3, 1, 1, 1), (1, 33, 65, 2)])

@@ -130,7 +130,7 @@ def test_yolov5s_config4(hip_ctx):
     qg = nb.quantize_graph(g, rng.random((4, 128, 128, 3), dtype=f32))
     ops = [n.op for n in qg.nodes]
     assert ops.count("conv") == 60 and ops.count("lut") == 57 and ops.count("concat") == 13 and ops.count("maxpool") == 3
-    assert ops.count("resize") == 2 and ops.count("add") == 7 and ops.count("padc") == 1 and ops.count("fold2") == 1
+    assert ops.count("resize") == 2 and ops.count("add") == 7 and ops.count("s2d") == 1
     assert len(qg.output_nodes) == 3
     x = rng.random((2, 128, 128, 3), dtype=f32)
     wants, outs = netref.run_integer(qg, x, keep_all=True)
@@ -138,12 +138,12 @@ def test_yolov5s_config4(hip_ctx):
         model = nb.HipModel(hip_ctx, qg, 2, capture_graph=capture, fuse_residual=fuse)
         model.run(x)
         # fused: every conv takes its swish table into the epilogue (the detect convs aside), the seven bottleneck
-        # adds go in as well; the fold of pixel pairs into channels in front of the stem is no operator
+        # adds go in as well; the input's quantisation is done by the pack of 2 x 2 pixel blocks in front of the stem
         # and 17 convs whose result only feeds a concat write their slice of the concat's tensor themselves (their
         # requantisation to the concat's quant params composed with their tables), which leaves 6 of the 13 concat
         # operators, with fewer inputs each
-        assert (len(model.fused_lut), len(model.fused_into), len(model.write_through), len(model.fn)) == \
-            ((57, 7, 17, 147 - 64 - 7) if fuse else (0, 0, 0, 147))
+        assert (len(model.fused_lut), len(model.fused_into), len(model.write_through), len(model.fused_quant), len(model.fn)) == \
+            ((57, 7, 17, 1, 147 - 64 - 7 - 1) if fuse else (0, 0, 0, 0, 147))
         for i, ref in enumerate(outs):
             if not model.materialized(i):
                 continue
@@ -151,14 +151,15 @@ def test_yolov5s_config4(hip_ctx):
             assert np.array_equal(got, ref), f"node {i} ({qg.nodes[i].name}, {qg.nodes[i].op}): {(got != ref).sum()} of {ref.size} bytes differ"
         for got, want in zip(model.all_outputs(), wants):
             assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
-    # the zero-padded 4th stem channel and the fold of pixel pairs into channels change nothing: the stem conv, a 6x3
-    # window of stride (2, 1) over 8 channels of the half-width image, equals the 6x6 stride-2 convolution over RGB
+    # the zero-padded 4th stem channel and the fold of 2 x 2 pixel blocks into channels change nothing: the stem conv, a
+    # 3x3 window of stride 1 over 16 channels of the half-size image, equals the 6x6 stride-2 convolution over RGB
     stem = next(i for i, n in enumerate(qg.nodes) if n.op == "conv")
     n, src = qg.nodes[stem], qg.nodes[0]
-    assert n.weights.shape[1:] == (8, 6, 3) and tuple(n.stride) == (2, 1) and tuple(map(tuple, n.padding)) == ((2, 2), (1, 1))
+    assert n.weights.shape[1:] == (16, 3, 3) and tuple(n.stride) == (1, 1) and tuple(map(tuple, n.padding)) == ((1, 1), (1, 1))
     w66 = np.empty((n.weights.shape[0], 3, 6, 6), np.uint8)
-    for dx in range(2):
-        w66[:, :, :, dx::2] = n.weights[:, dx * 4:dx * 4 + 3]
+    for dy in range(2):
+        for dx in range(2):
+            w66[:, :, dy::2, dx::2] = n.weights[:, (dy * 2 + dx) * 4:(dy * 2 + dx) * 4 + 3]
     plain = O.qconv2d(outs[0], w66, n.bias, src.out_qp[0], src.out_qp[1], n.w_qp[0], n.w_qp[1], n.out_qp[0], n.out_qp[1],
                       (2, 2), ((2, 2), (2, 2)), (1, 1), 1, n.clamp, O.OUT_U8)
     assert np.array_equal(plain, outs[stem])
@@ -167,7 +168,7 @@ def test_yolov5s_config4(hip_ctx):
     for want, j in zip(wants, g.outputs):
         assert O.cosine(want, fl[j]) > 0.98
     loaded = rt.LoadedKModel(hip_ctx, km.compile_quant_graph(qg, 2))
-    assert len(loaded.fn) == 147 - 64 - 7       # the native loader folds the same tables, adds and concat slices
+    assert len(loaded.fn) == 147 - 64 - 7 - 1   # the native loader folds the same tables, adds, concat slices and quantize
     ys = loaded.run(x)
     assert len(ys) == 3
     for y, want in zip(ys, wants):
