@@ -113,9 +113,8 @@ def op_accounting(qg, batch, model):
             if n.op == "input":
                 consts += 4 * size(j)            # the float32 tensor the quantize operator reads
             elif n.op == "conv":
-                oc, gic, kh, kw = n.weights.shape
                 consts += n.weights.size + 4 * n.bias.size
-                m += batch * oc * n.out_shape[1] * n.out_shape[2] * gic * kh * kw
+                m += batch * n.macs
         nbytes.append(b + consts)
         floors.append(sum(size(j) for j in external) + size(members[-1]) + consts)
         macs.append(m)

@@ -195,6 +195,13 @@ typedef struct nncase_hip_conv2d_args {
      * its slice of the concat's tensor): pixel stride in channels, 0 = out_channels (dense), and the
      * first channel written.  Dense (MFMA) kernels only; residual_dev stays a dense tensor. */
     int32_t out_channel_stride, out_channel_offset;
+    /* With out_dtype == NNCASE_HIP_DT_F32 and dequantize_output != 0 the call computes the u8 result described
+     * above (y_qp, the fused table and residual included) and stores its float32 value
+     * (q - zero_point) * scale of the last stage's quant param instead of the byte: the Dequantize that
+     * follows the last convolution of a quantised graph, bit-identical to nncase_hip_qconv2d followed by
+     * nncase_hip_dequantize without the u8 tensor in between.  Dense (MFMA) kernels only, no out_channel_stride. */
+    int32_t dequantize_output;
+    int32_t reserved;                    /* 0 */
 } nncase_hip_conv2d_args_t;
 
 /* Output is [batch, out_h, out_w, out_channels] with

@@ -62,6 +62,8 @@ public struct HipConv2DArgs
     public float SumClampMax;
     public int OutChannelStride;
     public int OutChannelOffset;
+    public int DequantizeOutput;
+    public int Reserved;
 }
 
 /// <summary>nncase_hip_qblock_desc_t.</summary>

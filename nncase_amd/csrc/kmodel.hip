@@ -479,6 +479,28 @@ static int build_function(nncase_hip_ctx_t *ctx, Span text_span, Span rdata, nnc
         }
     }
 
+    // A Dequantize that alone reads a dense conv's result (behind its folded table / add) is done by that conv: it
+    // stores the float32 value of its u8 result.
+    std::vector<int> fused_deq(th.n_ops, -1); // conv op -> the dequantize op behind it
+    for (uint32_t k = 0; k < th.n_ops; k++) {
+        const hipf_op &dq = ops[k];
+        if (dq.opcode != kOpDequantize || dq.n_inputs != 1) continue;
+        const int32_t t = dq.inputs[0];
+        const int p = producer[t];
+        if (p < 0 || consumers[t] != 1 || is_output(t)) continue;
+        int c = p;
+        for (uint32_t q = 0; q < th.n_ops; q++)
+            if (fused_lut[q] == p || fused_add[q] == p) c = (int)q;
+        const hipf_op &conv = ops[c];
+        const int last = fused_add[c] >= 0 ? fused_add[c] : fused_lut[c] >= 0 ? fused_lut[c] : c;
+        if (conv.opcode != kOpConv2d || skipped[c] || block_head[c] || last != p || through[c].concat >= 0 || !dense_conv(conv)) continue;
+        if (m->tensors[t].dtype != NNCASE_HIP_DT_U8 || m->tensors[dq.output].dtype != NNCASE_HIP_DT_F32 ||
+            elems((uint32_t)t) != elems((uint32_t)dq.output))
+            continue;
+        fused_deq[c] = (int)k;
+        skipped[k] = 1;
+    }
+
     // A float32 -> u8 quantize read only by a channel padding is done by that operator (quantize and pack in one pass).
     std::vector<int> fused_quant(th.n_ops, -1); // pad_channels op -> the quantize op in front of it
     for (uint32_t k = 0; k < th.n_ops; k++) {
@@ -505,6 +527,11 @@ static int build_function(nncase_hip_ctx_t *ctx, Span text_span, Span rdata, nnc
         if (fused_add[k] >= 0 && fused_lut[k] >= 0) m->owns[ops[fused_lut[k]].output] = 2;
         if (block_head[k]) m->owns[ops[k].output] = m->owns[ops[k + 1].output] = 2;
         if (fused_quant[k] >= 0) m->owns[ops[fused_quant[k]].output] = 2;
+        if (fused_deq[k] >= 0) { // the u8 result is never stored
+            m->owns[ops[k].output] = 2;
+            if (fused_lut[k] >= 0) m->owns[ops[fused_lut[k]].output] = 2;
+            if (fused_add[k] >= 0) m->owns[ops[fused_add[k]].output] = 2;
+        }
         if (through[k].concat >= 0) { // no tensor of its own: the bytes live in the concat's tensor
             m->owns[ops[k].output] = 2;
             if (fused_lut[k] >= 0) m->owns[ops[fused_lut[k]].output] = 2;
@@ -656,6 +683,10 @@ static int build_function(nncase_hip_ctx_t *ctx, Span text_span, Span rdata, nnc
                 a.residual_qp = tqp(res), a.sum_qp = tqp(sum);
                 a.sum_clamp_min = add.f[0], a.sum_clamp_max = add.f[1];
                 y = m->buffers[sum];
+            }
+            if (fused_deq[k] >= 0) {
+                y = m->buffers[ops[fused_deq[k]].output];
+                a.out_dtype = NNCASE_HIP_DT_F32, a.dequantize_output = 1;
             }
             if (through[k].concat >= 0) {
                 y = m->buffers[ops[through[k].concat].output];

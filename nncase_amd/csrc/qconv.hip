@@ -24,7 +24,8 @@ void nnhip::describe_conv_kernel(const nncase_hip_ctx *ctx, const nncase_hip_wei
         else snprintf(buf, cap, "dw_generic<VEC=%d>", w->out_channels % 4 == 0 ? 4 : 1);
         return;
     }
-    if (w->d_smallc && a->dilation_h == 1 && a->dilation_w == 1 && !a->residual_dev) {
+    if (w->d_smallc && a->dilation_h == 1 && a->dilation_w == 1 && !a->residual_dev && !w->d_post_lut && !a->dequantize_output &&
+        !a->out_channel_stride) {
         snprintf(buf, cap, "qconv_smallc<C=%d>", w->in_channels);
         return;
     }
@@ -35,11 +36,13 @@ void nnhip::describe_conv_kernel(const nncase_hip_ctx *ctx, const nncase_hip_wei
     const int mode = igemm_load_mode(w, a, out_h, out_w);
     const int mi = (int)std::min<long long>(m, 1 << 30);
     if (w->wide) {
-        snprintf(buf, cap, "qconv_wide%s%s<T=%d,%s%s>", w->d_post_lut ? "+lut" : "", a->residual_dev ? "+add" : "", w->tiles,
+        snprintf(buf, cap, "qconv_wide%s%s%s<T=%d,%s%s>", w->d_post_lut ? "+lut" : "", a->residual_dev ? "+add" : "",
+                 a->dequantize_output ? "+dequantize" : "", w->tiles,
                  w->wide == 2 ? "RG=2," : "", modes[mode]);
         return;
     }
-    snprintf(buf, cap, "qconv_igemm%s%s<T=%d,RG=%d,%s>", w->d_post_lut ? "+lut" : "", a->residual_dev ? "+add" : "", w->tiles,
+    snprintf(buf, cap, "qconv_igemm%s%s%s<T=%d,RG=%d,%s>", w->d_post_lut ? "+lut" : "", a->residual_dev ? "+add" : "",
+             a->dequantize_output ? "+dequantize" : "", w->tiles,
              igemm_pixel_groups(ctx, w, mi), modes[mode]);
 }
 
@@ -331,6 +334,17 @@ extern "C" int nncase_hip_qconv2d(nncase_hip_ctx_t *ctx, const uint8_t *x_dev, c
                   "qconv2d: negative padding");
     NNHIP_REQUIRE(ctx, a->x_qp.zero_point >= 0 && a->x_qp.zero_point <= 255, -EINVAL,
                   "qconv2d: input zero point %d outside u8", a->x_qp.zero_point);
+    nncase_hip_conv2d_args_t through_u8;
+    if (a->dequantize_output != 0) {
+        // the u8 result, stored as its float32 value: the kernels see a u8 call with the flag set
+        NNHIP_REQUIRE(ctx, a->out_dtype == NNCASE_HIP_DT_F32, -NNCASE_HIP_ERR_DATATYPE_MISMATCH,
+                      "qconv2d: dequantize_output needs out_dtype float32");
+        NNHIP_REQUIRE(ctx, w->kind == nncase_hip_weights::kIgemm && a->out_channel_stride == 0 && a->out_channel_offset == 0, -EINVAL,
+                      "qconv2d: dequantize_output is only supported by the dense (MFMA) kernels, with a dense output");
+        through_u8 = *a;
+        through_u8.out_dtype = NNCASE_HIP_DT_U8;
+        a = &through_u8;
+    }
     int rc = check_out_dtype(ctx, a->out_dtype, a->y_qp, "qconv2d");
     if (rc) return rc;
     const int out_h = windowed_output_size(a->in_h, w->kernel_h, a->stride_h, a->dilation_h, a->pad_h_before, a->pad_h_after);
@@ -341,6 +355,7 @@ extern "C" int nncase_hip_qconv2d(nncase_hip_ctx_t *ctx, const uint8_t *x_dev, c
                       "qconv2d: an output inside a wider tensor is only supported by the dense (MFMA) kernels");
         if (!a->residual_dev && !w->d_post_lut) return launch_qconv_igemm(ctx, x_dev, w, y_dev, a, out_h, out_w);
     }
+    if (a->dequantize_output != 0 && !a->residual_dev && !w->d_post_lut) return launch_qconv_igemm(ctx, x_dev, w, y_dev, a, out_h, out_w);
     if (a->residual_dev || w->d_post_lut) {
         if (a->residual_dev) {
             rc = check_out_dtype(ctx, NNCASE_HIP_DT_U8, a->sum_qp, "qconv2d(residual)");

@@ -122,7 +122,7 @@ int launch_qconv_igemm(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_hip_w
                        const nncase_hip_conv2d_args_t *c, int out_h, int out_w) {
     const int64_t m64 = (int64_t)c->batch * out_h * out_w;
     const int64_t in_bytes = (int64_t)c->batch * c->in_h * c->in_w * w->in_channels;
-    const int out_es = c->out_dtype == NNCASE_HIP_DT_U8 ? 1 : 4;
+    const int out_es = c->out_dtype == NNCASE_HIP_DT_U8 && !c->dequantize_output ? 1 : 4;
     NNHIP_REQUIRE(ctx, m64 > 0 && m64 < ((int64_t)1 << 30), -EINVAL, "qconv2d: %lld output pixels unsupported",
                   (long long)m64);
     NNHIP_REQUIRE(ctx, in_bytes < ((int64_t)1 << 31), -EINVAL, "qconv2d: input of %lld bytes exceeds 2 GiB",
@@ -178,6 +178,10 @@ int launch_qconv_igemm(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_hip_w
         if (rc) return rc;
     }
     a.lut = c->out_dtype == NNCASE_HIP_DT_U8 ? w->d_post_lut : nullptr;
+    if (c->dequantize_output != 0) { // (out_dtype is u8 here: the entry point has turned the call into its u8 form)
+        const nncase_hip_quant_param_t last = c->residual_dev ? c->sum_qp : (w->d_post_lut ? w->post_lut_qp : c->y_qp);
+        a.deq = 1, a.deq_zero = last.zero_point, a.deq_scale = last.scale;
+    }
     const int mode = igemm_load_mode(w, c, out_h, out_w);
 
     const size_t group_bytes = (size_t)w->nchunks * w->ksteps * w->tiles * 1024;

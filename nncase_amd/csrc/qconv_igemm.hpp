@@ -77,6 +77,9 @@ struct IgemmArgs {
     Epilogue ep;
     ResidualEpilogue rep;
     const uint32_t *lut;   // 256-entry byte table applied to the requantised byte (before the residual add), or null
+    int deq;               // the u8 result is stored as float32: (q - deq_zero) * deq_scale
+    int deq_zero;
+    float deq_scale;
 };
 
 // Packs one group's weights into MFMA operand order.
@@ -394,6 +397,24 @@ __device__ __forceinline__ void igemm_store_tile(const IgemmArgs &a, const v4i (
                 }
                 packed[nt] = residual4_packed(packed[nt], rv, a.rep);
             }
+        }
+        if (a.deq) { // the Dequantize behind the convolution: one float per channel
+            float *fo = reinterpret_cast<float *>(a.y) + obase;
+#pragma unroll
+            for (int nt = 0; nt < T; nt++) {
+                uint32_t o[4];
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    o[r] = __float_as_uint((float)((int)((packed[nt] >> (8 * r)) & 0xffu) - a.deq_zero) * a.deq_scale);
+                if (ch0 + nt * 4 + 4 <= a.n) {
+                    *reinterpret_cast<u32x4_a4 *>(fo + nt * 4) = u32x4_a4{o[0], o[1], o[2], o[3]};
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        if (ch0 + nt * 4 + r < a.n) fo[nt * 4 + r] = __uint_as_float(o[r]);
+                }
+            }
+            return;
         }
         if (((a.ldy | a.y_coff) & 3) == 0 && ch0 + 4 * T <= a.n) {
 #pragma unroll
@@ -775,6 +796,171 @@ template <int T, int RG, bool ROWS> __global__ void __launch_bounds__(kThreads, 
     }
 }
 
+// ---- windows over a multiple of 16 channels, the chunk's weights resident in LDS ---------------------------
+// The loader of qconv_igemm_kernel finds a slice's tap by two divisions per slice and clamps its coordinates; for
+// the stems that read 2 x 2 pixel blocks as 16-channel pixels (a few taps, 32 output channels, 10^6 pixels per
+// launch) that address arithmetic is most of the kernel.  Where the 16-byte slice kc of the reduction lies relative
+// to a pixel's window origin is the same for all pixels: a table in LDS, built once per block, holds per slice the
+// byte offset, the tap's row and column, and what the slice holds when the tap lies in the padding (the zero point)
+// or past the reduction (x' = 0).  A lane's slice then costs two additions and two comparisons: it is read
+// through the range-checked buffer path either from its address or, through an offset outside the buffer, as
+// zeros that the fill value is or-ed into.  The sums start from the channel constants; the row sums that the weight
+// zero point multiplies come from a ones operand.
+struct WindowSlice {
+    u32x4 raw;
+    uint32_t fill; // 0 where raw holds the data
+};
+
+template <int T, int RG, bool PLAIN> __global__ void __launch_bounds__(kThreads, 4) qconv_window_kernel(const IgemmArgs a) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    int32_t *cterm = reinterpret_cast<int32_t *>(smem);    // [T * 16]
+    uint8_t *lutl = smem + T * 16 * sizeof(int32_t);       // [256]
+    v4i *taps = reinterpret_cast<v4i *>(lutl + 256);       // [ksteps * 4]: byte offset, row, column, fill
+    const int KS = a.ksteps;
+    uint8_t *wlds = reinterpret_cast<uint8_t *>(taps + KS * 4); // [ksteps][T][1024]
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int j = lane & 15, gq = lane >> 4;
+    const int chunk = blockIdx.y;
+    const int ch_base = chunk * (T * 16);
+    const __amdgpu_buffer_rsrc_t xres = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(a.x), 0, (int)a.x_bytes, 0x00020000);
+
+    static_assert(T * 16 <= kThreads, "one constant per thread");
+    if ((int)threadIdx.x < T * 16) {
+        const int ch = ch_base + threadIdx.x;
+        cterm[threadIdx.x] = ch < a.n ? a.bias[ch] - a.zxp * a.wsum[ch] + a.k * a.zxp * a.zwp : 0;
+    }
+    if (!PLAIN && a.lut && threadIdx.x < 64) reinterpret_cast<uint32_t *>(lutl)[threadIdx.x] = a.lut[threadIdx.x];
+    for (int e = threadIdx.x; e < KS * 4; e += kThreads) {
+        const int kk = e * 16;
+        v4i t = {0, 0x40000000, 0, (int)0x80808080u}; // past the reduction: never inside the image, x' = 0
+        if (kk < a.k) {
+            const uint32_t tap = fastdiv((uint32_t)kk, a.d_gic);
+            const int c = kk - (int)tap * a.g_ic;
+            const uint32_t ky = fastdiv(tap, a.d_kw);
+            const int dy = (int)ky * a.dil_h, dx = ((int)tap - (int)ky * a.kw) * a.dil_w;
+            t = v4i{(dy * a.in_w + dx) * a.ldx + c, dy, dx, (int)a.zx_splat};
+        }
+        taps[e] = t;
+    }
+    {
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(a.wpk + (size_t)chunk * KS * T * 1024);
+        u32x4 *dst = reinterpret_cast<u32x4 *>(wlds);
+        const int n = KS * T * 64;
+        for (int i = threadIdx.x; i < n; i += 4 * kThreads) {
+            u32x4 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+                if (i + u * kThreads < n) v[u] = src[i + u * kThreads];
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+                if (i + u * kThreads < n) dst[i + u * kThreads] = v[u];
+        }
+    }
+    __syncthreads();
+
+    const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
+    constexpr int pix_per_block = kWaves * RG * 16;
+    struct Origin { // window origin of a lane's pixel: byte offset (may lie before the tensor), row, column
+        uint32_t off;
+        int iy0, ix0;
+    };
+    auto origin = [&](int mt, int rg) {
+        const PixInfo pi = pix_info<kVec16>(a, mt * pix_per_block + (wave * RG + rg) * 16 + j);
+        const bool ok = pi.base >= 0;
+        Origin o;
+        o.off = (uint32_t)(((ok ? pi.base : 0) + pi.iy0 * a.in_w + pi.ix0) * a.ldx + a.x_coff);
+        o.iy0 = ok ? pi.iy0 : 0x40000000; // (a pixel past the end reads nothing)
+        o.ix0 = pi.ix0;
+        return o;
+    };
+    const v4i *const my_taps = taps + gq;
+    auto load = [&](const Origin &o, int ks) {
+        const v4i t = my_taps[ks * 4];
+        const bool inside = (unsigned)(o.iy0 + t[1]) < (unsigned)a.in_h && (unsigned)(o.ix0 + t[2]) < (unsigned)a.in_w;
+        WindowSlice f;
+        f.raw = __builtin_amdgcn_raw_buffer_load_b128(xres, inside ? o.off + (uint32_t)t[0] : 0xffffffffu, 0, 0);
+        f.fill = inside ? 0u : (uint32_t)t[3];
+        return f;
+    };
+
+    int mt = blockIdx.x;
+    Origin org[RG];
+    WindowSlice cur[RG];
+    if (mt < a.num_mtiles) {
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) {
+            org[rg] = origin(mt, rg);
+            cur[rg] = load(org[rg], 0);
+        }
+    }
+    const int last = KS - 1;
+    const int ch0 = ch_base + gq * (4 * T);
+#pragma clang loop unroll(disable)
+    for (; mt < a.num_mtiles; mt += gridDim.x) {
+        v4i acc[RG][T];
+        v4i rs[RG];
+        const int mt_next = mt + gridDim.x < a.num_mtiles ? mt + gridDim.x : mt; // past the end: re-read this tile, dropped
+        Origin org_next[RG];
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) org_next[rg] = origin(mt_next, rg);
+#pragma clang loop unroll(disable)
+        for (int ks = 0; ks < KS; ks++) {
+            // the next slices: the next k-step of this tile, or the first of the next tile
+            WindowSlice nxt[RG];
+            const bool same_tile = ks < last;
+#pragma unroll
+            for (int rg = 0; rg < RG; rg++) {
+                Origin o;
+                o.off = same_tile ? org[rg].off : org_next[rg].off;
+                o.iy0 = same_tile ? org[rg].iy0 : org_next[rg].iy0;
+                o.ix0 = same_tile ? org[rg].ix0 : org_next[rg].ix0;
+                nxt[rg] = load(o, same_tile ? ks + 1 : 0);
+            }
+            v4i xf[RG];
+#pragma unroll
+            for (int rg = 0; rg < RG; rg++) {
+                u32x4 r;
+#pragma unroll
+                for (int d = 0; d < 4; d++) r[d] = (cur[rg].raw[d] | cur[rg].fill) ^ 0x80808080u;
+                xf[rg] = __builtin_bit_cast(v4i, r);
+            }
+            const uint8_t *wstep = wlds + (size_t)ks * T * 1024 + lane * 16;
+            if (ks == 0) {
+                int ct_off = gq * (4 * T);
+                asm volatile("" : "+v"(ct_off)); // (read per tile: kept in registers the constants would cost 4T of them)
+                const v4i zero = {0, 0, 0, 0};
+#pragma unroll
+                for (int nt = 0; nt < T; nt++) {
+                    const v4i ct = *reinterpret_cast<const v4i *>(cterm + ct_off + nt * 4);
+                    const v4i wf = *reinterpret_cast<const v4i *>(wstep + nt * 1024);
+#pragma unroll
+                    for (int rg = 0; rg < RG; rg++) acc[rg][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf, xf[rg], ct, 0, 0, 0);
+                }
+#pragma unroll
+                for (int rg = 0; rg < RG; rg++) rs[rg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, xf[rg], zero, 0, 0, 0);
+            } else {
+#pragma unroll
+                for (int nt = 0; nt < T; nt++) {
+                    const v4i wf = *reinterpret_cast<const v4i *>(wstep + nt * 1024);
+#pragma unroll
+                    for (int rg = 0; rg < RG; rg++) acc[rg][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf, xf[rg], acc[rg][nt], 0, 0, 0);
+                }
+#pragma unroll
+                for (int rg = 0; rg < RG; rg++) rs[rg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, xf[rg], rs[rg], 0, 0, 0);
+            }
+#pragma unroll
+            for (int rg = 0; rg < RG; rg++) cur[rg] = nxt[rg];
+        }
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++)
+            igemm_store_tile<T, kOwesRows, PLAIN>(a, acc[rg], rs[rg][0], mt * pix_per_block + (wave * RG + rg) * 16 + j, ch0, gq, cterm, lutl);
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) org[rg] = org_next[rg];
+    }
+}
+
 // Pixel groups per wave (RG) for a chunk width of T tiles.  The kernels are bound by the
 // VALU work of the epilogue, and a dependent VALU instruction issues only every ~8 cycles
 // from one wave, so what matters is having >= 4 waves per SIMD: RG is capped so that the
@@ -802,8 +988,19 @@ template <int T, int RG, int MODE> int launch_trg(nncase_hip_ctx *ctx, const Ige
     const size_t lds = (size_t)T * 16 * sizeof(int32_t) + 256 + (size_t)a.kc_steps * T * 1024;
     // the 1x1 row loaders are also built without the epilogue's options (see igemm_store_tile)
     bool plain = false;
-    if constexpr (loads_rows(MODE))
-        plain = a.ep.out_mode == kOutU8 && a.ep.fast && a.ep.full && !a.lut && !a.rep.res && a.n % (4 * T) == 0 && ((a.ldy | a.y_coff) & 3) == 0;
+    if constexpr (loads_rows(MODE) || MODE == kVec16)
+        plain = a.ep.out_mode == kOutU8 && !a.deq && a.ep.fast && a.ep.full && !a.lut && !a.rep.res && a.n % (4 * T) == 0 && ((a.ldy | a.y_coff) & 3) == 0;
+    if constexpr (MODE == kVec16 && T <= 6) {
+        // the whole chunk's weights resident and no folded reduction: the kernel with the tap table
+        const size_t lds_win = (size_t)T * 16 * sizeof(int32_t) + 256 + (size_t)a.ksteps * 4 * sizeof(v4i) + (size_t)a.ksteps * T * 1024;
+        if (a.kc_steps >= a.ksteps && a.kc_mask == -1 && lds_win <= 65536) {
+            if (plain) hipLaunchKernelGGL((qconv_window_kernel<T, RG, true>), dim3(gx, nchunks, 1), dim3(kThreads), lds_win, ctx->stream, args);
+            else hipLaunchKernelGGL((qconv_window_kernel<T, RG, false>), dim3(gx, nchunks, 1), dim3(kThreads), lds_win, ctx->stream, args);
+            NNHIP_LAUNCH_CHECK(ctx, "qconv_window_kernel");
+            return 0;
+        }
+        plain = false;
+    }
     if (plain) {
         if constexpr (MODE == kRows16) {
             // the whole chunk's weights resident, rows of at least 16 bytes: the lean kernel

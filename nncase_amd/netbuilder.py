@@ -255,6 +255,13 @@ class QNode:
     lut: Optional[np.ndarray] = None         # "lut": 256-entry byte table Q(f(DQ(.)))
     resize_modes: Tuple[int, int] = (rt.RESIZE_ASYMMETRIC, rt.NEAREST_FLOOR)   # "resize"
     pool: Tuple[int, int, int] = (5, 1, 2)   # "maxpool": kernel, stride, pad
+    model_k: Optional[int] = None            # "conv" whose weights were padded for the device: the model's own reduction length
+
+    @property
+    def macs(self) -> int:
+        """Multiply-accumulates of the model's conv per image (padding taps and channels added for the device not counted)."""
+        oc, gic, kh, kw = self.weights.shape
+        return oc * self.out_shape[1] * self.out_shape[2] * (self.model_k if self.model_k is not None else gic * kh * kw)
 
 
 @dataclass
@@ -274,9 +281,8 @@ class QuantGraph:
         for n in self.nodes:
             if n.op != "conv":
                 continue
-            oc, gic, kh, kw = n.weights.shape
-            m = oc * n.out_shape[1] * n.out_shape[2] * gic * kh * kw
-            if n.groups > 1 and gic == 1:
+            m = n.macs
+            if n.groups > 1 and n.weights.shape[1] == 1:
                 dw += m
             else:
                 dense += m
@@ -318,32 +324,52 @@ def quantize_graph(g: FloatGraph, calib_nhwc: np.ndarray, calib_batch: int = 8) 
     return pad_small_channel_convs(QuantGraph(qnodes, g.input_shape, g.outputs))
 
 
+def _even_window(k: int, p0: int, size: int, out: int):
+    """A stride-2 window of k taps with p0 padded positions in front, as an even window whose front padding is even
+    too: (taps to prepend, taps to append, front padding, back padding), the added taps carrying zero weights and the
+    back padding being what makes the output extent `out` again.  None when no such window exists."""
+    front = p0 % 2                      # an odd front padding: one more (zero) tap in front
+    back = (k + front) % 2              # then an odd window: one more behind
+    k2, p0 = k + front + back, p0 + front
+    p1 = 2 * (out - 1) + k2 - size - p0
+    return None if p1 < 0 or p1 % 2 else (front, back, p0, p1)
+
+
 def pad_small_channel_convs(qg: QuantGraph) -> QuantGraph:
-    """A dense conv over fewer than 4 input channels whose window is not 3x3 (YOLOv5's 6x6 RGB stem)
-    would gather single bytes.  Pad its input to 4 channels ("padc": zero-filled 4th channel) and its
-    weights with the weight zero point, which contributes (w - zw) = 0 whatever the padded byte is:
-    the integer result is unchanged and the conv reads whole dwords."""
+    """A dense conv over fewer than 4 input channels (an RGB stem) would gather single bytes.  Its input is padded to
+    4 channels ("padc": zero-filled 4th channel) and its weights with the weight zero point, which contributes
+    (w - zw) = 0 whatever the padded byte is: the integer result is unchanged and the conv reads whole dwords.  Stems
+    of stride 2 go further and read 2 x 2 pixel blocks as 16-channel pixels (below); 3x3 windows of stride 1 are left
+    to the kernel for few input channels."""
     nodes: List[QNode] = []
     remap: Dict[int, int] = {}
     for i, n in enumerate(qg.nodes):
         n = QNode(**{**n.__dict__, "inputs": tuple(remap[j] for j in n.inputs)})
-        if n.op == "conv" and n.groups == 1 and n.weights.shape[1] < 4 and n.weights.shape[2:] != (3, 3):
+        small = n.op == "conv" and n.groups == 1 and n.weights.shape[1] < 4
+        if small:
             src = nodes[n.inputs[0]]
             c, h, w = src.out_shape
+            kh, kw = n.weights.shape[2:]
+            (ph0, ph1), (pw0, pw1) = n.padding
+            ev = (_even_window(kh, ph0, h, n.out_shape[1]), _even_window(kw, pw0, w, n.out_shape[2])) \
+                if tuple(n.stride) == (2, 2) and h % 2 == 0 and w % 2 == 0 else (None, None)
+        if small and (n.weights.shape[2:] != (3, 3) or None not in ev):
             nodes.append(QNode("padc", (n.inputs[0],), n.name + ".pad4", src.out_qp, (4, h, w)))
             wpad = np.full((n.weights.shape[0], 4) + n.weights.shape[2:], n.w_qp[0], np.uint8)
             wpad[:, :c] = n.weights
+            n.model_k = int(np.prod(n.weights.shape[1:]))
             n.weights, n.inputs = wpad, (len(nodes) - 1,)
-            kh, kw = n.weights.shape[2:]
-            (ph0, ph1), (pw0, pw1) = n.padding
-            if (tuple(n.stride) == (2, 2) and kh % 2 == 0 and kw % 2 == 0 and h % 2 == 0 and w % 2 == 0
-                    and all(p % 2 == 0 for p in (ph0, ph1, pw0, pw1))):
-                # Stride 2 over an even window: every 2 x 2 block of 4-channel pixels becomes one 16-channel pixel of the
+            if None not in ev:
+                # Stride 2 (odd windows and odd front paddings first grow by taps of zero weight): every 2 x 2 block of
+                # 4-channel pixels becomes one 16-channel pixel of the
                 # half-size image ("s2d": pack by lanes (2, 2, 4) on (H, W, C), channel order (dy, dx, c)), and the conv
                 # becomes one of stride 1 over half the window in both directions:
                 # out(y, x) = sum over ky', kx', (dy, dx, c) of in[2 (y + ky' - ph / 2) + dy][2 (x + kx' - pw / 2) + dx][c]
                 #             w[2 ky' + dy][2 kx' + dx][c].  The loader then fetches 16 bytes per tap and computes a quarter
                 # as many tap addresses; the padding is whole blocks, filled with the input's zero point as before.
+                (fh, bh, ph0, ph1), (fw, bw, pw0, pw1) = ev
+                wpad = np.pad(wpad, ((0, 0), (0, 0), (fh, bh), (fw, bw)), constant_values=n.w_qp[0])
+                kh, kw = wpad.shape[2:]
                 nodes[-1] = QNode("s2d", nodes[-1].inputs, n.name + ".s2d", src.out_qp, (16, h // 2, w // 2))
                 wf = np.empty((wpad.shape[0], 16, kh // 2, kw // 2), np.uint8)
                 for dy in range(2):
@@ -513,6 +539,22 @@ class HipModel:
                     self.fused_quant[i] = j
                     self.never_written.add(j)
                     skip_nodes.add(j)
+        # The Dequantize of an output whose u8 tensor nothing else reads is done by the dense conv that produces it
+        # (behind its folded table / add): the conv stores float32 into the output buffer.
+        self.fused_dequant: Dict[int, int] = {}                                          # conv -> index into output_nodes
+        if fuse_residual:
+            owner = {**{v: k for k, v in self.fused_lut.items()}, **{v: k for k, v in self.fused_into.items()}}
+            for oi, j in enumerate(qg.output_nodes):
+                conv = owner.get(j, j)
+                conv = owner.get(conv, conv)
+                cnode = qg.nodes[conv]
+                last = self.fused_into.get(conv, self.fused_lut.get(conv, conv))
+                if (cnode.op == "conv" and last == j and consumers[j] == 0 and qg.output_nodes.count(j) == 1
+                        and conv not in block_members and conv not in self.write_through
+                        and not (cnode.groups > 1 and cnode.weights.shape[1] == 1) and cnode.weights.shape[1] * cnode.groups > 4
+                        and (conv == j or consumers[conv] == 1)):
+                    self.fused_dequant[conv] = oi
+                    self.never_written |= {conv, j} | ({self.fused_lut[conv]} if conv in self.fused_lut else set())
         # buffers and packed weights once, shared by the lanes
         for i, n in enumerate(qg.nodes):
             cc, hh, ww = n.out_shape
@@ -523,7 +565,7 @@ class HipModel:
             if n.op == "fold2":
                 self.buffers.append(self.buffers[n.inputs[0]])  # the same bytes read as half as many, twice as deep pixels
                 continue
-            if i in self.blocks or i - 1 in self.blocks or i in self.write_through or i in self.fused_quant.values():
+            if i in self.blocks or i - 1 in self.blocks or i in self.write_through or i in self.fused_quant.values() or i in self.fused_dequant:
                 self.buffers.append(ctx.alloc(16))        # expanded tensors of a fused block live in LDS only; a conv
                 #                                           that writes into its concat has no tensor of its own
             else:
@@ -591,7 +633,8 @@ class HipModel:
                     self.op_nodes.append(addn if addn is not None else pn)
                     self.op_members.append([i, dn, pn] + ([addn] if addn is not None else []))
                 continue
-            buf = None if i in self.write_through else B(i)   # (a conv that writes into its concat has no tensor of its own)
+            buf = None if i in self.write_through or i in self.fused_dequant else B(i)   # (a conv that writes into its concat or
+            #                                                                              the output has no tensor of its own)
             if n.op == "input":
                 self.fn.add_quantize(self.input_f32.view(lane * self._lane_stride(in_per * 4), in_per * 4), rt.DT_F32, buf, rt.DT_U8, in_per, qp(*n.out_qp))
             elif n.op == "conv":
@@ -612,6 +655,11 @@ class HipModel:
                 if wthru is not None:
                     buf = B(wthru[0])
                     args.out_channel_offset, args.out_channel_stride = wthru[1], wthru[2]
+                if i in self.fused_dequant:
+                    oj = qg.nodes[qg.output_nodes[self.fused_dequant[i]]]
+                    per = bl * int(np.prod(oj.out_shape)) * 4
+                    buf = self.outputs_f32[self.fused_dequant[i]].view(lane * self._lane_stride(per), per)
+                    args.out_dtype, args.dequantize_output = rt.DT_F32, 1
                 self.fn.add_qconv2d(B(n.inputs[0]), self.weights[i], buf, args)
             elif n.op == "add":
                 a, b = (qg.nodes[j] for j in n.inputs)
@@ -658,6 +706,8 @@ class HipModel:
                 self.op_nodes.append(fused_add if fused_add is not None else (fused_lut if fused_lut is not None else i))
                 self.op_members.append(members)
         for k, j in enumerate(qg.output_nodes):
+            if k in self.fused_dequant.values():
+                continue                                       # stored as float32 by the conv that produces it
             node = qg.nodes[j]
             count = bl * int(np.prod(node.out_shape))
             self.fn.add_dequantize(B(j), rt.DT_U8, self.outputs_f32[k].view(lane * self._lane_stride(count * 4), count * 4), rt.DT_F32, count, qp(*node.out_qp))

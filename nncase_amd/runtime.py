@@ -51,7 +51,8 @@ class Conv2dArgs(C.Structure):
                 ("clamp_min", C.c_float), ("clamp_max", C.c_float), ("out_dtype", C.c_int32),
                 ("residual_dev", C.c_void_p), ("residual_qp", QuantParam), ("sum_qp", QuantParam),
                 ("sum_clamp_min", C.c_float), ("sum_clamp_max", C.c_float),
-                ("out_channel_stride", C.c_int32), ("out_channel_offset", C.c_int32)]
+                ("out_channel_stride", C.c_int32), ("out_channel_offset", C.c_int32),
+                ("dequantize_output", C.c_int32), ("reserved", C.c_int32)]
 
 
 class QBlockDesc(C.Structure):

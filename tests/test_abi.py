@@ -46,7 +46,7 @@ def test_struct_layouts_match_the_header():
     # fixed-layout PODs: sizes the C side was compiled with
     assert C.sizeof(rt.QuantParam) == 8
     assert C.sizeof(rt.Conv2dDesc) == 5 * 4 + 8 + 4 + 8  # 4 bytes of padding before the int64
-    assert C.sizeof(rt.Conv2dArgs) == 11 * 4 + 8 + 8 + 3 * 4 + 8 + 8 + 8 + 2 * 4 + 2 * 4
+    assert C.sizeof(rt.Conv2dArgs) == 11 * 4 + 8 + 8 + 3 * 4 + 8 + 8 + 8 + 2 * 4 + 2 * 4 + 2 * 4
     assert C.sizeof(rt.MatmulArgs) == 4 + 8 + 8 + 3 * 4
     assert C.sizeof(rt.QBlockDesc) == 3 * 4 + 3 * 8 and C.sizeof(rt.QBlockArgs) == 8 * 4 + 4 * 8 + 6 * 4 + 4 + 8 + 2 * 4
     assert C.sizeof(rt.PagedAttnArgs) == 10 * 4
@@ -120,7 +120,7 @@ def test_header_ctypes_and_csharp_pods_agree():
         assert C.sizeof(ctype) == size, hname
         assert [getattr(ctype, f[0]).offset for f in ctype._fields_] == offsets, hname
         assert [f[0] for f in ctype._fields_] == [n for _, n in hs[hname]], hname
-    assert layout([k for k, _ in hs["nncase_hip_conv2d_args_t"]])[1] == 112
+    assert layout([k for k, _ in hs["nncase_hip_conv2d_args_t"]])[1] == 120
 
 
 def test_csharp_imports_name_exported_symbols_with_the_right_arity():

@@ -483,6 +483,56 @@ def test_conv_output_inside_a_wider_tensor(hip_ctx, cin, cout, k, stride_c, offs
         assert e.value.code == -22
 
 
+@pytest.mark.parametrize("cin,cout,k,hw,with_lut,with_res", [
+    (128, 255, 1, 20, False, False),      # a detection head: 255 channels, rows of 1020 bytes
+    (64, 64, 3, 13, True, False), (32, 48, 1, 9, True, True), (16, 24, 1, 7, False, True), (320, 1000, 1, 1, False, False),
+    (512, 255, 1, 20, False, False)])
+def test_conv_stores_the_dequantised_output(hip_ctx, cin, cout, k, hw, with_lut, with_res):
+    """dequantize_output: conv (+ table, + residual add) with float32 output == the same conv with u8 output followed by
+    Dequantize (oracle: conv, table, add, dequantize), bit for bit."""
+    rng = np.random.default_rng(cin * 3 + cout + k)
+    n = 2
+    x = rng.integers(0, 256, (n, cin, hw, hw), dtype=np.uint8)
+    wt = rng.integers(0, 256, (cout, cin, k, k), dtype=np.uint8)
+    bias = rng.integers(-2000, 2000, cout).astype(np.int32)
+    pad = ((k // 2, k // 2), (k // 2, k // 2))
+    zx, sx, zw, sw = 7, 0.0235, 131, 0.0041
+    real = O.qconv2d(x, wt, bias, zx, sx, zw, sw, padding=pad, out_mode=O.OUT_F32)
+    zy, sy = quant.get_quant_param((float(real.min()), float(real.max())))
+    zy, sy = int(zy), float(sy)
+    want = O.qconv2d(x, wt, bias, zx, sx, zw, sw, zy, sy, padding=pad, out_mode=O.OUT_U8)
+    last = (zy, sy)
+    wts = hip_ctx.prepack_conv2d(wt, bias, qp(zw, sw), 1, expected_pixels=n * hw * hw)
+    if with_lut:
+        lut = rng.integers(0, 256, 256, dtype=np.uint8)
+        last = (77, 0.043)
+        wts.set_post_lut(lut, qp(*last))
+        want = lut[want]
+    args = rt.Conv2dArgs(n, hw, hw, 1, 1, 1, 1, pad[0][0], pad[0][1], pad[1][0], pad[1][1], qp(zx, sx), qp(zy, sy), -rt.FLT_MAX, rt.FLT_MAX, rt.DT_F32)
+    args.dequantize_output = 1
+    if with_res:
+        res = rng.integers(0, 256, (n, cout, hw, hw), dtype=np.uint8)
+        want = O.qadd(want, res, last[0], last[1], 33, 0.11, 90, 0.3)
+        last = (90, 0.3)
+        rb = hip_ctx.to_device(np.ascontiguousarray(res.transpose(0, 2, 3, 1)))
+        args.residual_dev, args.residual_qp, args.sum_qp = rb.ptr, qp(33, 0.11), qp(90, 0.3)
+        args.sum_clamp_min, args.sum_clamp_max = -rt.FLT_MAX, rt.FLT_MAX
+    want_f = O.dequantize(want, last[1], last[0])
+    xb = hip_ctx.to_device(np.ascontiguousarray(x.transpose(0, 2, 3, 1)))
+    yb = hip_ctx.alloc(want_f.size * 4)
+    hip_ctx.qconv2d(xb, wts, yb, args)
+    got = yb.download((n, hw, hw, cout), np.float32)
+    assert np.array_equal(got.view(np.uint32), np.ascontiguousarray(want_f.transpose(0, 2, 3, 1)).view(np.uint32))
+    args.out_dtype = rt.DT_U8                      # the flag needs a float32 output ...
+    with pytest.raises(rt.HipError) as e:
+        hip_ctx.qconv2d(xb, wts, yb, args)
+    assert e.value.code == -rt.ERR_DATATYPE_MISMATCH
+    args.out_dtype, args.out_channel_stride = rt.DT_F32, cout + 4     # ... and a dense one
+    with pytest.raises(rt.HipError) as e:
+        hip_ctx.qconv2d(xb, wts, yb, args)
+    assert e.value.code == -22
+
+
 def test_depthwise_conv_refuses_an_output_inside_a_wider_tensor(hip_ctx):
     wts = hip_ctx.prepack_conv2d(np.zeros((32, 1, 3, 3), np.uint8), None, qp(128, 0.01), 32)
     xb, yb = hip_ctx.alloc(8 * 8 * 32), hip_ctx.alloc(8 * 8 * 64)

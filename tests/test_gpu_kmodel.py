@@ -42,7 +42,7 @@ def test_conv_block_kmodel(hip_ctx):
     qg = nb.quantize_graph(nb.conv_block(seed=1), rng.random((8, 56, 56, 64), dtype=f32))
     x = rng.random((2, 56, 56, 64), dtype=f32)
     model, y, fused = run_and_check(hip_ctx, qg, x)
-    assert fused == 0 and len(model.fn) == 5
+    assert fused == 1 and len(model.fn) == 4             # (the last conv stores the dequantised output itself)
     model.fn.capture()                                   # the loaded function replays as a HIP graph
     for _ in range(2):
         assert np.array_equal(model.run(x).view(np.uint32), y.view(np.uint32))
@@ -56,8 +56,9 @@ def test_mobilenetv2_kmodel(hip_ctx):
     qg = nb.quantize_graph(nb.mobilenet_v2(seed=2), rng.random((8, 224, 224, 3), dtype=f32))
     x = rng.random((4, 224, 224, 3), dtype=f32)
     model, y, fused = run_and_check(hip_ctx, qg, x)
-    # the loader folds the ten residual adds and, at this batch, the two 28x28 blocks (64 workgroups each) whole
-    assert fused == 14 and len(model.fn) == 52
+    # the loader folds the ten residual adds, at this batch the two 28x28 blocks (64 workgroups each) whole, the
+    # input's quantize into the pack in front of the stem and the output's dequantize into the classifier
+    assert fused == 16 and len(model.fn) == 51
     ref = nb.HipModel(hip_ctx, qg, 4, capture_graph=False)
     assert np.array_equal(ref.run(x).view(np.uint32).ravel(), y.view(np.uint32).ravel())
 

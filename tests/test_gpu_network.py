@@ -69,11 +69,12 @@ def test_mobilenetv2_config3(hip_ctx):
     assert qg.macs_per_image == {"dense": 280057856, "depthwise": 20716416}
     x = rng.random((2, 224, 224, 3), dtype=f32)
     plain, _, _ = check_model(hip_ctx, qg, x, capture=False, fuse_residual=False)   # every tensor, add as its own kernel
-    assert len(plain.fused_into) == 0 and len(plain.fn) == 66
+    assert len(plain.fused_into) == 0 and len(plain.fn) == 67     # (quantize, pack of 2 x 2 pixel blocks, 52 convs, ...)
     model, y, outs = check_model(hip_ctx, qg, x, capture=True, fuse_blocks=False)
-    assert len(model.fused_into) == 10 and len(model.fn) == 56                        # residual adds folded into the convs
+    assert len(model.fused_into) == 10 and len(model.fused_dequant) == 1 and len(model.fn) == 55   # residual adds folded into
+    #                                                                            the convs, the output's dequantize into the classifier
     model, y, outs = check_model(hip_ctx, qg, x, capture=True)
-    assert len(model.blocks) == 16 and len(model.fn) == 24                            # ... and whole blocks into one operator
+    assert len(model.blocks) == 16 and len(model.fn) == 23                            # ... and whole blocks into one operator
     # the reference's own acceptance bar for a PTQ model: cosine >= 0.98 against the float model
     fl = nb.float_forward(g, x)[-1]
     assert O.cosine(y, fl) > 0.98
@@ -142,8 +143,9 @@ def test_yolov5s_config4(hip_ctx):
         # and 17 convs whose result only feeds a concat write their slice of the concat's tensor themselves (their
         # requantisation to the concat's quant params composed with their tables), which leaves 6 of the 13 concat
         # operators, with fewer inputs each
-        assert (len(model.fused_lut), len(model.fused_into), len(model.write_through), len(model.fused_quant), len(model.fn)) == \
-            ((57, 7, 17, 1, 147 - 64 - 7 - 1) if fuse else (0, 0, 0, 0, 147))
+        # ; the three detect convs store the dequantised outputs themselves
+        assert (len(model.fused_lut), len(model.fused_into), len(model.write_through), len(model.fused_quant), len(model.fused_dequant),
+                len(model.fn)) == ((57, 7, 17, 1, 3, 147 - 64 - 7 - 1 - 3) if fuse else (0, 0, 0, 0, 0, 147))
         for i, ref in enumerate(outs):
             if not model.materialized(i):
                 continue
@@ -168,7 +170,7 @@ def test_yolov5s_config4(hip_ctx):
     for want, j in zip(wants, g.outputs):
         assert O.cosine(want, fl[j]) > 0.98
     loaded = rt.LoadedKModel(hip_ctx, km.compile_quant_graph(qg, 2))
-    assert len(loaded.fn) == 147 - 64 - 7 - 1   # the native loader folds the same tables, adds, concat slices and quantize
+    assert len(loaded.fn) == 147 - 64 - 7 - 1 - 3   # the native loader folds the same tables, adds, concat slices, quantize, dequantizes
     ys = loaded.run(x)
     assert len(ys) == 3
     for y, want in zip(ys, wants):
@@ -229,10 +231,11 @@ def test_profile_and_kernel_names(hip_ctx):
     qg = nb.quantize_graph(g, rng.random((4, 56, 56, 64), dtype=f32))
     model = nb.HipModel(hip_ctx, qg, 2, capture_graph=False)
     names = [model.fn.op_kernel(i) for i in range(len(model.fn))]
-    assert names[0] == "quantize" and names[2] == "dw3x3<S=1>" and names[4] == "dequantize"
-    assert all(n.startswith("qconv_igemm<T=") and n.endswith(",rows16>") for n in (names[1], names[3]))
+    assert names[0] == "quantize" and names[2] == "dw3x3<S=1>" and len(names) == 4
+    assert names[1].startswith("qconv_igemm<T=") and names[3].startswith("qconv_igemm+dequantize<T=")   # (the output's Dequantize
+    assert all(n.endswith(",rows16>") for n in (names[1], names[3]))                                     # is the last conv's store)
     ms = model.fn.profile(3)
-    assert len(ms) == 5 and all(0 < t < 50 for t in ms)
+    assert len(ms) == 4 and all(0 < t < 50 for t in ms)
     fused = nb.HipModel(hip_ctx, qg, 2, capture_graph=False, fuse_blocks="all")
     assert [fused.fn.op_kernel(i) for i in range(len(fused.fn))] == ["quantize", "qblock<S=1,P=4>", "dequantize"]
     assert fused.op_members == [[0], [1, 2, 3], []]
