@@ -334,14 +334,14 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--workload", default="mobilenetv2", help="mobilenetv2 (headline, default) | matmul | conv_block | yolov5s | paged_attention | llm_decode")
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--batch", type=int, default=64)
     ap.add_argument("--batched", type=int, default=1, help="--workload matmul: number of stacked A matrices (M = 512 x this)")
     ap.add_argument("--lanes", type=int, default=1,
                     help="independent chains the batch is split into and replayed concurrently (1 = one chain of "
                          "full-batch launches); results are bit-identical for every value")
-    ap.add_argument("--in-flight", type=int, default=3,
+    ap.add_argument("--in-flight", type=int, default=4,
                     help="copies of the function (own stream and buffers each) that take the steps in turn, so that "
                          "consecutive steps overlap on the device (1 = one step at a time)")
     ap.add_argument("--cpu-images", type=int, default=8, help="batch-1 images timed on the CPU baseline (0 = skip)")
