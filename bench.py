@@ -41,49 +41,48 @@ INT8_PEAK_TOPS = 5000.0    # dense int8 MFMA
 # are recorded here and reported only for the configuration they were measured on.
 MEASURED_TRAFFIC_B64 = {
     "unfused": {
-        "dequantize": 345584,
-        "dw3x3<S=1>": 19025622,
-        "dw3x3<S=2>": 41843409,
-        "qconv_igemm+add<T=1,RG=1,rows16>": 6194308,
-        "qconv_igemm+add<T=2,RG=1,rows16>": 11631051,
-        "qconv_igemm+add<T=2,RG=2,rows16>": 39774544,
-        "qconv_igemm<T=1,RG=1,rows16>": 5954541,
-        "qconv_igemm<T=1,RG=4,rows16>": 38749244,
-        "qconv_igemm<T=12,RG=1,rows16>": 10475918,
-        "qconv_igemm<T=2,RG=1,rows16>": 7737832,
-        "qconv_igemm<T=2,RG=2,rows16>": 24292532,
-        "qconv_igemm<T=5,RG=1,rows16>": 5242493,
-        "qconv_igemm<T=6,RG=1,rows16>": 8757427,
-        "qconv_igemm<T=6,RG=2,rows16>": 90282384,
-        "qconv_igemm<T=8,RG=1,rows16>": 6052716,
-        "qconv_igemm<T=9,RG=1,rows8>": 34453811,
-        "qconv_smallc<C=3>": 38867446,
-        "qglobal_avgpool": 4237596,
-        "quantize": 48213804,
+        "dw3x3<S=1>": 19033881,
+        "dw3x3<S=2>": 41826522,
+        "qconv_igemm+add<T=2,RG=1,rows16>": 13041692,
+        "qconv_igemm+add<T=2,RG=2,rows16>": 39652870,
+        "qconv_igemm<T=1,RG=1,rows16>": 3347003,
+        "qconv_igemm<T=1,RG=4,rows16>": 38602998,
+        "qconv_igemm<T=12,RG=1,rows16>": 10273335,
+        "qconv_igemm<T=2,RG=1,rows16>": 8929032,
+        "qconv_igemm<T=2,RG=2,rows16>": 24173898,
+        "qconv_igemm<T=2,RG=2,vec16>": 50437450,
+        "qconv_igemm<T=5,RG=1,rows16>": 5102379,
+        "qconv_igemm<T=6,RG=2,rows16>": 90038939,
+        "qconv_igemm<T=8,RG=1,rows16>": 5905446,
+        "qconv_igemm<T=9,RG=1,rows8>": 34302078,
+        "qconv_wide+add<T=4,RG=2,rows16>": 7622480,
+        "qconv_wide+dequantize<T=4,RG=2,rows16>": 1725050,
+        "qconv_wide<T=4,RG=2,rows16>": 6400711,
+        "qglobal_avgpool": 4238843,
+        "quantize+pack": 51434730,
     },
     "fused": {
-        "dequantize": 345584,
-        "dw3x3<S=1>": 27907587,
-        "dw3x3<S=2>": 51717610,
-        "qblock+add<S=1,P=2>": 4946701,
-        "qblock+add<S=1,P=4>": 2671624,
-        "qblock+add<S=1,P=6>": 4553259,
-        "qblock<S=1,P=6>": 3246740,
-        "qblock<S=2,P=4>": 3349274,
-        "qconv_igemm+add<T=1,RG=1,rows16>": 5371037,
-        "qconv_igemm+add<T=2,RG=2,rows16>": 39719034,
-        "qconv_igemm<T=1,RG=1,rows16>": 6795342,
-        "qconv_igemm<T=1,RG=4,rows16>": 38749372,
-        "qconv_igemm<T=12,RG=1,rows16>": 9327753,
-        "qconv_igemm<T=2,RG=1,rows16>": 9008858,
-        "qconv_igemm<T=2,RG=2,rows16>": 24292340,
-        "qconv_igemm<T=5,RG=1,rows16>": 5242695,
-        "qconv_igemm<T=6,RG=1,rows16>": 8757427,
-        "qconv_igemm<T=6,RG=2,rows16>": 90282064,
-        "qconv_igemm<T=9,RG=1,rows8>": 34453379,
-        "qconv_smallc<C=3>": 38867894,
-        "qglobal_avgpool": 4237596,
-        "quantize": 48213772,
+        "dw3x3<S=1>": 27883943,
+        "dw3x3<S=2>": 51706994,
+        "qblock+add<S=1,P=2>": 4953995,
+        "qblock+add<S=1,P=4>": 2669235,
+        "qblock+add<S=1,P=6>": 4553291,
+        "qblock<S=1,P=6>": 3245716,
+        "qblock<S=2,P=4>": 3356217,
+        "qconv_igemm+add<T=2,RG=2,rows16>": 39724185,
+        "qconv_igemm<T=1,RG=4,rows16>": 38602902,
+        "qconv_igemm<T=12,RG=1,rows16>": 9129133,
+        "qconv_igemm<T=2,RG=1,rows16>": 8929032,
+        "qconv_igemm<T=2,RG=2,rows16>": 24174314,
+        "qconv_igemm<T=2,RG=2,vec16>": 50437514,
+        "qconv_igemm<T=5,RG=1,rows16>": 5102475,
+        "qconv_igemm<T=6,RG=2,rows16>": 90038907,
+        "qconv_igemm<T=9,RG=1,rows8>": 34302542,
+        "qconv_wide+add<T=4,RG=2,rows16>": 5790802,
+        "qconv_wide+dequantize<T=4,RG=2,rows16>": 1725050,
+        "qconv_wide<T=4,RG=2,rows16>": 6303034,
+        "qglobal_avgpool": 4238907,
+        "quantize+pack": 51434922,
     },
 }
 
