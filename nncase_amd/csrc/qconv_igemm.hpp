@@ -115,6 +115,15 @@ inline void pack_group(uint8_t *dst, int32_t *wsum, int g_oc, int k, int ksteps,
             }
 }
 
+// f(std::integral_constant<int, I>) for I = first .. N - 1, as straight-line code: an index into a register array
+// stays a compile-time constant even where the optimiser would decline to unroll a loop of this size.
+template <int I, int N, typename F> __device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>());
+        static_for<I + 1, N>(f);
+    }
+}
+
 struct PixInfo {
     int base; // kRows16: pixel index; other modes: pixel index of the image origin; < 0: no such pixel
     int iy0, ix0;
@@ -335,10 +344,57 @@ enum { kOwesAll = 0, kOwesRows = 1, kOwesNothing = 2 };
 // PLAIN: the launch has been checked to need none of the options -- u8 output by the one-instruction requantisation
 // (Epilogue::fast and ::full), no byte table, no residual, whole groups of 4T channels, dword-aligned rows -- so the
 // tile is converted and stored without a single test of them.
-template <int T, int OWED = kOwesAll, bool PLAIN = false>
+// Dword outputs (float32 / int32) of a wave's 16 pixels x 16T channels.  A lane holds 4T consecutive channels of one
+// pixel, so a 16-byte store of all lanes touches 64 different places, 16 bytes each (measured on the 255-channel
+// detection heads: 1.6 TB/s).  Instead, four channel tiles at a time, every lane puts its 64 bytes into the wave's LDS
+// staging area and the wave writes them out with four lanes per 64-byte run: a store instruction then covers 16
+// whole 64-byte runs.  LDS operations of a wave execute in order, so the phases need neither a barrier nor a wait
+// beyond the one in front of the first use of the data read back.
+constexpr bool staged_store_built(int T) { return T % 4 == 0; }
+constexpr int kStagedRun = 64 + 16;                       // a lane's run and its padding against bank conflicts
+constexpr int staged_store_bytes() { return 64 * kStagedRun; } // per wave
+
+// o: the lane's values of channel tiles 4g .. 4g + 3 (channels ch0 + 16 g + [0, 16) of pixel p)
+__device__ __forceinline__ void store_dword_group(const IgemmArgs &a, const uint32_t (&o)[4][4], int g, int p, int ch0, int gq, uint8_t *stage,
+                                                  int quarter_stride) {
+    // (quarter_stride: channels between the lanes' quarters, 4T unless waves side by side share the chunk)
+    const int lane = threadIdx.x & 63;
+    const int j = lane & 15;
+    const int p_first = p - j, ch_first = ch0 - gq * quarter_stride;
+    uint32_t *yo = reinterpret_cast<uint32_t *>(a.y);
+#pragma unroll
+    for (int k = 0; k < 4; k++) *reinterpret_cast<u32x4 *>(stage + (j * 4 + gq) * kStagedRun + k * 16) = u32x4{o[k][0], o[k][1], o[k][2], o[k][3]};
+    const int u = lane & 3, qq = (lane >> 2) & 3, psub = lane >> 4;
+    const int ch = ch_first + qq * quarter_stride + g * 16 + u * 4;
+#pragma unroll
+    for (int it = 0; it < 4; it++) {
+        const int row = it * 4 + psub;
+        const u32x4 v = *reinterpret_cast<const u32x4 *>(stage + (row * 4 + qq) * kStagedRun + u * 16);
+        const int pp = p_first + row;
+        if (pp < a.m) {
+            uint32_t *dst = yo + ((size_t)pp * a.ldy + a.y_coff + ch);
+            if (ch + 4 <= a.n) {
+                *reinterpret_cast<u32x4_a4 *>(dst) = u32x4_a4{v[0], v[1], v[2], v[3]};
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    if (ch + r < a.n) dst[r] = v[r];
+            }
+        }
+    }
+}
+
+// STAGED: the kernel has a staging area per wave for the dword outputs (store_dword_group); the lane-by-lane dword
+// stores are then not built.
+template <int T, int OWED = kOwesAll, bool PLAIN = false, bool STAGED = false>
 __device__ __forceinline__ void igemm_store_tile(const IgemmArgs &a, const v4i (&acc)[T], int32_t rowsum, int p, int ch0, int gq,
-                                                 const int32_t *cterm, const uint8_t *lutl) {
-    if (!(p < a.m && ch0 < a.n)) return;
+                                                 const int32_t *cterm, const uint8_t *lutl, uint8_t *stage = nullptr,
+                                                 int quarter_stride = 4 * T) {
+    static_assert(!STAGED || (!PLAIN && staged_store_built(T)), "staged stores move four channel tiles at a time");
+    // (with a staging area every lane of the wave takes part in the stores, whatever it holds itself)
+    const bool staged = STAGED && (a.deq || a.ep.out_mode != kOutU8);
+    const bool live = p < a.m && ch0 < a.n;
+    if (!live && !staged) return;
     const int32_t nrsz = OWED == kOwesAll ? -a.zwp * rowsum : (OWED == kOwesRows ? -a.zwp_rows * rowsum : 0);
     const size_t obase = (size_t)p * a.ldy + a.y_coff + ch0;
     if constexpr (PLAIN) {
@@ -382,7 +438,7 @@ __device__ __forceinline__ void igemm_store_tile(const IgemmArgs &a, const v4i (
                              ((uint32_t)lutl[(v >> 16) & 0xffu] << 16) | ((uint32_t)lutl[v >> 24] << 24);
             }
         }
-        if (a.rep.res) { // fused residual add on the requantised bytes
+        if (a.rep.res && live) { // fused residual add on the requantised bytes
             const uint8_t *ro = a.rep.res + ((size_t)p * a.ldr + a.r_coff + ch0);
             const bool whole = ((a.ldr | a.r_coff) & 3) == 0 && ch0 + 4 * T <= a.n;
 #pragma unroll
@@ -399,19 +455,32 @@ __device__ __forceinline__ void igemm_store_tile(const IgemmArgs &a, const v4i (
             }
         }
         if (a.deq) { // the Dequantize behind the convolution: one float per channel
-            float *fo = reinterpret_cast<float *>(a.y) + obase;
+            if constexpr (STAGED) {
 #pragma unroll
-            for (int nt = 0; nt < T; nt++) {
-                uint32_t o[4];
+                for (int g = 0; g < T / 4; g++) {
+                    uint32_t o[4][4];
 #pragma unroll
-                for (int r = 0; r < 4; r++)
-                    o[r] = __float_as_uint((float)((int)((packed[nt] >> (8 * r)) & 0xffu) - a.deq_zero) * a.deq_scale);
-                if (ch0 + nt * 4 + 4 <= a.n) {
-                    *reinterpret_cast<u32x4_a4 *>(fo + nt * 4) = u32x4_a4{o[0], o[1], o[2], o[3]};
-                } else {
+                    for (int k = 0; k < 4; k++)
+#pragma unroll
+                        for (int r = 0; r < 4; r++)
+                            o[k][r] = __float_as_uint((float)((int)((packed[g * 4 + k] >> (8 * r)) & 0xffu) - a.deq_zero) * a.deq_scale);
+                    store_dword_group(a, o, g, p, ch0, gq, stage, quarter_stride);
+                }
+            } else {
+                float *fo = reinterpret_cast<float *>(a.y) + obase;
+#pragma unroll
+                for (int nt = 0; nt < T; nt++) {
+                    uint32_t o[4];
 #pragma unroll
                     for (int r = 0; r < 4; r++)
-                        if (ch0 + nt * 4 + r < a.n) fo[nt * 4 + r] = __uint_as_float(o[r]);
+                        o[r] = __float_as_uint((float)((int)((packed[nt] >> (8 * r)) & 0xffu) - a.deq_zero) * a.deq_scale);
+                    if (ch0 + nt * 4 + 4 <= a.n) {
+                        *reinterpret_cast<u32x4_a4 *>(fo + nt * 4) = u32x4_a4{o[0], o[1], o[2], o[3]};
+                    } else {
+#pragma unroll
+                        for (int r = 0; r < 4; r++)
+                            if (ch0 + nt * 4 + r < a.n) fo[nt * 4 + r] = __uint_as_float(o[r]);
+                    }
                 }
             }
             return;
@@ -442,25 +511,35 @@ __device__ __forceinline__ void igemm_store_tile(const IgemmArgs &a, const v4i (
         }
     } else {
         // int32 accumulators or clamped fp32, one dword per channel
-        uint32_t *yo = reinterpret_cast<uint32_t *>(a.y) + obase;
+        auto value = [&](int nt, int r) __attribute__((always_inline)) -> uint32_t {
+            const int32_t ct = OWED == kOwesAll ? cterm[gq * (4 * T) + nt * 4 + r] : 0;
+            const int32_t v = OWED == kOwesAll ? add3(acc[nt][r], ct, nrsz) : (OWED == kOwesRows ? acc[nt][r] + nrsz : acc[nt][r]);
+            return a.ep.out_mode == kOutI32 ? (uint32_t)v : __float_as_uint(clamp_ref((float)v * a.ep.mult, a.ep.lo, a.ep.hi));
+        };
+        if constexpr (STAGED) {
 #pragma unroll
-        for (int nt = 0; nt < T; nt++) {
-            v4i ct = {0, 0, 0, 0};
-            if (OWED == kOwesAll) ct = *reinterpret_cast<const v4i *>(cterm + gq * (4 * T) + nt * 4);
-            uint32_t o[4];
+            for (int g = 0; g < T / 4; g++) {
+                uint32_t o[4][4];
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const int32_t v =
-                    OWED == kOwesAll ? add3(acc[nt][r], ct[r], nrsz) : (OWED == kOwesRows ? acc[nt][r] + nrsz : acc[nt][r]);
-                if (a.ep.out_mode == kOutI32) o[r] = (uint32_t)v;
-                else o[r] = __float_as_uint(clamp_ref((float)v * a.ep.mult, a.ep.lo, a.ep.hi));
+                for (int k = 0; k < 4; k++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) o[k][r] = value(g * 4 + k, r);
+                store_dword_group(a, o, g, p, ch0, gq, stage, quarter_stride);
             }
-            if (ch0 + nt * 4 + 4 <= a.n) {
-                *reinterpret_cast<u32x4_a4 *>(yo + nt * 4) = u32x4_a4{o[0], o[1], o[2], o[3]};
-            } else {
+        } else {
+            uint32_t *yo = reinterpret_cast<uint32_t *>(a.y) + obase;
 #pragma unroll
-                for (int r = 0; r < 4; r++)
-                    if (ch0 + nt * 4 + r < a.n) yo[nt * 4 + r] = o[r];
+            for (int nt = 0; nt < T; nt++) {
+                uint32_t o[4];
+#pragma unroll
+                for (int r = 0; r < 4; r++) o[r] = value(nt, r);
+                if (ch0 + nt * 4 + 4 <= a.n) {
+                    *reinterpret_cast<u32x4_a4 *>(yo + nt * 4) = u32x4_a4{o[0], o[1], o[2], o[3]};
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        if (ch0 + nt * 4 + r < a.n) yo[nt * 4 + r] = o[r];
+                }
             }
         }
     }
@@ -468,7 +547,9 @@ __device__ __forceinline__ void igemm_store_tile(const IgemmArgs &a, const v4i (
 
 // Blocks per compute unit the register allocation has to leave room for: four (at most 128 registers) for the
 // shapes that fit comfortably, so that the scheduler does not trade the occupancy away for longer live ranges.
-template <int T, int RG, int MODE, bool PLAIN = false>
+// STAGED: built for dword outputs (float32 / int32 / the dequantised u8 result), which go through a staging area per
+// wave behind the weights; a kernel of its own because the staged stores raise the register count of the whole kernel.
+template <int T, int RG, int MODE, bool PLAIN = false, bool STAGED = false>
 __global__ void __launch_bounds__(kThreads, ((RG == 1 && T <= 12) || loads_rows(MODE)) ? 4 : 2) qconv_igemm_kernel(const IgemmArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     int32_t *cterm = reinterpret_cast<int32_t *>(smem); // [T * 16]
@@ -477,6 +558,9 @@ __global__ void __launch_bounds__(kThreads, ((RG == 1 && T <= 12) || loads_rows(
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
+    // dword outputs: a staging area per wave behind the weights (see store_dword_rows), when the launch asked for one
+    static_assert(!STAGED || (!PLAIN && staged_store_built(T)), "staged stores move four channel tiles at a time");
+    uint8_t *const stage = wlds + (size_t)a.kc_steps * T * 1024 + wave * staged_store_bytes(); // (reserved by the launch of a STAGED kernel)
     const int j = lane & 15;  // pixel within a group of 16
     const int gq = lane >> 4; // k-quarter on the load side, channel quarter on the store side
     const int chunk = blockIdx.y;
@@ -648,13 +732,15 @@ __global__ void __launch_bounds__(kThreads, ((RG == 1 && T <= 12) || loads_rows(
         // (written out for both cases: one epilogue behind a conditional correction would keep two copies of the sums)
         const int ch0 = ch_base + gq * (4 * T); // first of this lane's 4T channels
         if (a.zwp_rows != 0) {
-#pragma unroll
-            for (int rg = 0; rg < RG; rg++)
-                igemm_store_tile<T, kOwesRows, PLAIN>(a, acc[rg], rs[rg][0], mt * pix_per_block + (wave * RG + rg) * 16 + j, ch0, gq, cterm, lutl);
+            static_for<0, RG>([&](auto rg_c) __attribute__((always_inline)) {
+                constexpr int rg = decltype(rg_c)::value;
+                igemm_store_tile<T, kOwesRows, PLAIN, STAGED>(a, acc[rg], rs[rg][0], mt * pix_per_block + (wave * RG + rg) * 16 + j, ch0, gq, cterm, lutl, stage);
+            });
         } else {
-#pragma unroll
-            for (int rg = 0; rg < RG; rg++)
-                igemm_store_tile<T, kOwesNothing, PLAIN>(a, acc[rg], 0, mt * pix_per_block + (wave * RG + rg) * 16 + j, ch0, gq, cterm, lutl);
+            static_for<0, RG>([&](auto rg_c) __attribute__((always_inline)) {
+                constexpr int rg = decltype(rg_c)::value;
+                igemm_store_tile<T, kOwesNothing, PLAIN, STAGED>(a, acc[rg], 0, mt * pix_per_block + (wave * RG + rg) * 16 + j, ch0, gq, cterm, lutl, stage);
+            });
         }
 #pragma unroll
         for (int rg = 0; rg < RG; rg++) pcur[rg] = pnxt[rg];
@@ -985,7 +1071,10 @@ template <int T, int RG, int MODE> int launch_trg(nncase_hip_ctx *ctx, const Ige
     // columns the blocks that share a pixel tile (same x, different chunk) land on
     // one XCD and find the activations in its L2.
     if (nchunks > 1) gx = ceil_div(gx, 8) * 8;
-    const size_t lds = (size_t)T * 16 * sizeof(int32_t) + 256 + (size_t)a.kc_steps * T * 1024;
+    size_t lds = (size_t)T * 16 * sizeof(int32_t) + 256 + (size_t)a.kc_steps * T * 1024;
+    // dword outputs of chunks of 4, 8, 12 or 16 tiles go through a staging area per wave (store_dword_group)
+    const bool stage_lds = staged_store_built(T) && (loads_rows(MODE) || MODE == kVec16) && (a.deq || a.ep.out_mode != kOutU8);
+    if (stage_lds) lds += (size_t)kWaves * staged_store_bytes();
     // the 1x1 row loaders are also built without the epilogue's options (see igemm_store_tile)
     bool plain = false;
     if constexpr (loads_rows(MODE) || MODE == kVec16)
@@ -1014,6 +1103,16 @@ template <int T, int RG, int MODE> int launch_trg(nncase_hip_ctx *ctx, const Ige
         }
         if constexpr (loads_rows(MODE))
             hipLaunchKernelGGL((qconv_igemm_kernel<T, RG, MODE, true>), dim3(gx, nchunks, 1), dim3(kThreads), lds, ctx->stream, args);
+    } else if (stage_lds) {
+        if constexpr (staged_store_built(T) && (loads_rows(MODE) || MODE == kVec16)) {
+            static bool raised = false; // more than 64 KiB of dynamic LDS (full-depth weights and the staging areas) has to be asked for once
+            if (lds > 65536 && !raised) {
+                NNHIP_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(&qconv_igemm_kernel<T, RG, MODE, false, true>),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, 98304));
+                raised = true;
+            }
+            hipLaunchKernelGGL((qconv_igemm_kernel<T, RG, MODE, false, true>), dim3(gx, nchunks, 1), dim3(kThreads), lds, ctx->stream, args);
+        }
     } else
         hipLaunchKernelGGL((qconv_igemm_kernel<T, RG, MODE>), dim3(gx, nchunks, 1), dim3(kThreads), lds, ctx->stream, args);
     NNHIP_LAUNCH_CHECK(ctx, "qconv_igemm_kernel");

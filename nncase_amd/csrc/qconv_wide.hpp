@@ -307,14 +307,17 @@ __global__ __launch_bounds__(WM * WN * 64, 2) void qconv_wide_kernel(const Igemm
         if (lq == 0) rowsums[lp + i * (THREADS / 4)] = r;
     }
     __syncthreads();
+    // dword outputs are written through a staging area per wave (store_dword_rows): the ring is free now
+    static_assert(!staged_store_built(T) || WM * WN * staged_store_bytes() <= kWideSlots * SLOT, "the staging areas fit the ring");
+    uint8_t *const stage = staged_store_built(T) ? ring + wave * staged_store_bytes() : nullptr;
     // lane (j, gq) of wave (wm, wn) holds channels ch_base + gq * 4 TB + wn * 4 T + [0, 4 T) of its pixels
     const int ch0 = ch_base + gq * (4 * TB) + wn * (4 * T);
     const int32_t *ct = cterm + gq * (4 * TB) + wn * (4 * T) - gq * (4 * T); // igemm_store_tile adds gq * 4 T
-#pragma unroll
-    for (int rg = 0; rg < RG; rg++) {
+    static_for<0, RG>([&](auto rg_c) __attribute__((always_inline)) {
+        constexpr int rg = decltype(rg_c)::value;
         const int pl = (wm * RG + rg) * 16 + j;
-        igemm_store_tile<T>(a, acc[rg], rowsums[pl], mt * PIX + pl, ch0, gq, ct, lutl);
-    }
+        igemm_store_tile<T, kOwesAll, false, staged_store_built(T)>(a, acc[rg], rowsums[pl], mt * PIX + pl, ch0, gq, ct, lutl, stage, 4 * TB);
+    });
 }
 
 template <int T, int RG, int WM, int WN, int LM> int launch_wide_t(nncase_hip_ctx *ctx, const IgemmArgs &a, int nchunks) {
