@@ -550,7 +550,7 @@ __device__ __forceinline__ void igemm_store_tile(const IgemmArgs &a, const v4i (
 // STAGED: built for dword outputs (float32 / int32 / the dequantised u8 result), which go through a staging area per
 // wave behind the weights; a kernel of its own because the staged stores raise the register count of the whole kernel.
 template <int T, int RG, int MODE, bool PLAIN = false, bool STAGED = false>
-__global__ void __launch_bounds__(kThreads, ((RG == 1 && T <= 12) || loads_rows(MODE)) ? 4 : 2) qconv_igemm_kernel(const IgemmArgs a) {
+__global__ void __launch_bounds__(kThreads, (STAGED && T >= 12) ? 2 : (((RG == 1 && T <= 12) || loads_rows(MODE)) ? 4 : 2)) qconv_igemm_kernel(const IgemmArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     int32_t *cterm = reinterpret_cast<int32_t *>(smem); // [T * 16]
     uint8_t *lutl = smem + T * 16 * sizeof(int32_t);    // [256] byte table of the fused unary operator
