@@ -41,48 +41,51 @@ INT8_PEAK_TOPS = 5000.0    # dense int8 MFMA
 # are recorded here and reported only for the configuration they were measured on.
 MEASURED_TRAFFIC_B64 = {
     "unfused": {
-        "dw3x3<S=1>": 19033881,
-        "dw3x3<S=2>": 41826522,
-        "qconv_igemm+add<T=2,RG=1,rows16>": 13041692,
-        "qconv_igemm+add<T=2,RG=2,rows16>": 39652870,
+        "dw3x3<S=1>": 19062930,
+        "dw3x3<S=2>": 41864194,
+        "qconv_igemm+add<T=2,RG=1,rows16>": 13037132,
+        "qconv_igemm+add<T=2,RG=2,rows16>": 39622124,
         "qconv_igemm<T=1,RG=1,rows16>": 3347003,
-        "qconv_igemm<T=1,RG=4,rows16>": 38602998,
-        "qconv_igemm<T=12,RG=1,rows16>": 10273335,
-        "qconv_igemm<T=2,RG=1,rows16>": 8929032,
-        "qconv_igemm<T=2,RG=2,rows16>": 24173898,
-        "qconv_igemm<T=2,RG=2,vec16>": 50437450,
-        "qconv_igemm<T=5,RG=1,rows16>": 5102379,
-        "qconv_igemm<T=6,RG=2,rows16>": 90038939,
-        "qconv_igemm<T=8,RG=1,rows16>": 5905446,
-        "qconv_igemm<T=9,RG=1,rows8>": 34302078,
-        "qconv_wide+add<T=4,RG=2,rows16>": 7622480,
-        "qconv_wide+dequantize<T=4,RG=2,rows16>": 1725050,
-        "qconv_wide<T=4,RG=2,rows16>": 6400711,
-        "qglobal_avgpool": 4238843,
-        "quantize+pack": 51434730,
+        "qconv_igemm<T=1,RG=4,rows16>": 38603062,
+        "qconv_igemm<T=12,RG=1,rows16>": 10266014,
+        "qconv_igemm<T=2,RG=1,rows16>": 8914666,
+        "qconv_igemm<T=2,RG=2,rows16>": 24172938,
+        "qconv_igemm<T=2,RG=2,vec16>": 50436234,
+        "qconv_igemm<T=5,RG=1,rows16>": 5104437,
+        "qconv_igemm<T=6,RG=2,rows16>": 90039579,
+        "qconv_igemm<T=8,RG=1,rows16>": 5905454,
+        "qconv_igemm<T=9,RG=1,rows8>": 34301150,
+        "qconv_wide+add<T=2,RG=2,rows16>": 6241416,
+        "qconv_wide+add<T=4,RG=2,rows16>": 10526164,
+        "qconv_wide+dequantize<T=2,RG=2,rows16>": 1710333,
+        "qconv_wide<T=2,RG=2,rows16>": 4931864,
+        "qconv_wide<T=4,RG=2,rows16>": 7643263,
+        "qglobal_avgpool": 4238939,
+        "quantize+pack": 51434890,
     },
     "fused": {
-        "dw3x3<S=1>": 27883943,
-        "dw3x3<S=2>": 51706994,
-        "qblock+add<S=1,P=2>": 4953995,
+        "dw3x3<S=1>": 27991460,
+        "dw3x3<S=2>": 51739642,
+        "qblock+add<S=1,P=2>": 4954891,
         "qblock+add<S=1,P=4>": 2669235,
-        "qblock+add<S=1,P=6>": 4553291,
-        "qblock<S=1,P=6>": 3245716,
-        "qblock<S=2,P=4>": 3356217,
-        "qconv_igemm+add<T=2,RG=2,rows16>": 39724185,
-        "qconv_igemm<T=1,RG=4,rows16>": 38602902,
-        "qconv_igemm<T=12,RG=1,rows16>": 9129133,
-        "qconv_igemm<T=2,RG=1,rows16>": 8929032,
-        "qconv_igemm<T=2,RG=2,rows16>": 24174314,
-        "qconv_igemm<T=2,RG=2,vec16>": 50437514,
-        "qconv_igemm<T=5,RG=1,rows16>": 5102475,
-        "qconv_igemm<T=6,RG=2,rows16>": 90038907,
-        "qconv_igemm<T=9,RG=1,rows8>": 34302542,
-        "qconv_wide+add<T=4,RG=2,rows16>": 5790802,
-        "qconv_wide+dequantize<T=4,RG=2,rows16>": 1725050,
-        "qconv_wide<T=4,RG=2,rows16>": 6303034,
-        "qglobal_avgpool": 4238907,
-        "quantize+pack": 51434922,
+        "qblock+add<S=1,P=6>": 4553131,
+        "qblock<S=1,P=6>": 3246964,
+        "qblock<S=2,P=4>": 3355193,
+        "qconv_igemm+add<T=2,RG=2,rows16>": 39652422,
+        "qconv_igemm<T=1,RG=4,rows16>": 38603190,
+        "qconv_igemm<T=12,RG=1,rows16>": 9114575,
+        "qconv_igemm<T=2,RG=1,rows16>": 8914698,
+        "qconv_igemm<T=2,RG=2,rows16>": 24172522,
+        "qconv_igemm<T=2,RG=2,vec16>": 50436650,
+        "qconv_igemm<T=5,RG=1,rows16>": 5104416,
+        "qconv_igemm<T=6,RG=2,rows16>": 90039099,
+        "qconv_igemm<T=9,RG=1,rows8>": 34301902,
+        "qconv_wide+add<T=2,RG=2,rows16>": 5419156,
+        "qconv_wide+dequantize<T=2,RG=2,rows16>": 1710333,
+        "qconv_wide<T=2,RG=2,rows16>": 4932631,
+        "qconv_wide<T=4,RG=2,rows16>": 8621259,
+        "qglobal_avgpool": 4238843,
+        "quantize+pack": 51434858,
     },
 }
 
