@@ -77,6 +77,14 @@ NNCASE_HIP_API int nncase_hip_version(void);
  * nncase_interp_create (api.h:77). */
 NNCASE_HIP_API int nncase_hip_ctx_create(int device, nncase_hip_ctx_t **ctx);
 NNCASE_HIP_API int nncase_hip_ctx_destroy(nncase_hip_ctx_t *ctx);
+/* For hosts that keep several contexts busy at once (one per request in flight, as one interpreter per request
+ * with the reference): HIP multiplexes streams over at most GPU_MAX_HW_QUEUES hardware queues (4 by default) — a new
+ * stream opens a new queue until that many exist and joins the least shared one after that — and kernels of
+ * streams that share a queue run one after the other.  This call creates that many idle streams on the device, once
+ * per process, so that the streams of contexts created AFTER it land on the hardware queues in turn, one each for
+ * the first GPU_MAX_HW_QUEUES of them.  Returns the number of hardware queues (> 0) or a negative status.
+ * (No counterpart in the reference, whose interpreters are CPU threads.) */
+NNCASE_HIP_API int nncase_hip_fill_queue_pool(int device);
 
 /* The hipStream_t the context enqueues on (so a caller can record events on
  * it), and a way to make the context use a caller-owned stream instead. */

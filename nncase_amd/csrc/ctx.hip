@@ -1,6 +1,7 @@
 // Context, device memory and stream entry points of libnncase_hip.so.
 #include "common.hpp"
 
+#include <mutex>
 #include <new>
 
 using namespace nnhip;
@@ -33,6 +34,33 @@ extern "C" int nncase_hip_ctx_create(int device, nncase_hip_ctx_t **out) {
     ctx->owns_stream = true;
     *out = ctx;
     return 0;
+}
+
+// HIP multiplexes streams over at most GPU_MAX_HW_QUEUES hardware queues (4 unless the environment says otherwise): a
+// new stream opens a new queue until that many exist and joins the least shared one after that, and kernels of streams
+// that share a queue run one after the other.  Idle streams created here, once per device and kept until the process
+// ends, fill the pool, so that the streams of the contexts created afterwards are dealt out one per queue in turn.
+extern "C" int nncase_hip_fill_queue_pool(int device) {
+    constexpr int kMaxDevices = 64, kMaxQueues = 32;
+    static std::mutex lock;
+    static int filled[kMaxDevices] = {0};
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || device < 0 || device >= count || device >= kMaxDevices) return -ENODEV;
+    std::lock_guard<std::mutex> guard(lock);
+    if (filled[device]) return filled[device];
+    int queues = 4;
+    if (const char *env = getenv("GPU_MAX_HW_QUEUES")) {
+        const int v = atoi(env);
+        if (v >= 1 && v <= kMaxQueues) queues = v;
+    }
+    if (hipSetDevice(device) != hipSuccess) return -ENODEV;
+    for (int i = 0; i < queues; i++) {
+        hipStream_t idle;
+        const hipError_t e = hipStreamCreateWithFlags(&idle, hipStreamNonBlocking);
+        if (e != hipSuccess) return -(NNCASE_HIP_ERR_HIP_BASE + (int)e);
+    }
+    filled[device] = queues;
+    return queues;
 }
 
 extern "C" int nncase_hip_ctx_destroy(nncase_hip_ctx_t *ctx) {

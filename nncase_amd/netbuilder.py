@@ -17,7 +17,6 @@ reference's Evaluator during calibration and is not part of the timed path.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-import os
 from typing import Dict, List, Optional, Sequence, Tuple
 
 import numpy as np
@@ -791,8 +790,7 @@ class HipPipeline:
         # the caller's own stream give 183 k images/s on MobileNetV2 at batch 64, one per hardware queue 224 k; six or
         # eight hardware queues instead of four give 164-180 k).  So the pool is filled with idle streams first: the
         # copies' streams then land on one hardware queue each.
-        hw_queues = int(os.environ.get("GPU_MAX_HW_QUEUES", "4") or 4)
-        self._idle = [Context(device) for _ in range(hw_queues)]
+        self.hw_queues = rt.fill_queue_pool(device)
         self.contexts = [Context(device) for _ in range(depth)]
         self.models = [HipModel(c, qg, batch, **model_args) for c in self.contexts]
         self.turn = 0

@@ -155,6 +155,7 @@ SYMBOLS = {
     "nncase_hip_kmodel_destroy": (_I, [_VP]),
     "nncase_hip_kmodel_function": (_I, [_VP, C.POINTER(_VP)]),
     "nncase_hip_kmodel_tensor": (_I, [_VP, C.c_int32, C.POINTER(_VP), _I32P, _I32P]),
+    "nncase_hip_fill_queue_pool": (_I, [C.c_int]),
     "nncase_hip_pack": (_I, [_VP, _VP, _VP, C.c_int32, C.c_int32, _I32P, C.c_int32, _I32P, _I32P]),
     "nncase_hip_unpack": (_I, [_VP, _VP, _VP, C.c_int32, C.c_int32, _I32P, C.c_int32, _I32P, _I32P]),
     "nncase_hip_quantize_pack": (_I, [_VP, _VP, _VP, C.c_int32, _I32P, C.c_int32, _I32P, _I32P, QuantParam]),
@@ -205,6 +206,15 @@ class HipError(RuntimeError):
         self.code = code
         name = errno.errorcode.get(-code, "") if -code < ERR_HIP_BASE else f"hipError {-code - ERR_HIP_BASE}"
         super().__init__(f"{where}: status code {code} {name} {detail}".strip())
+
+
+def fill_queue_pool(device: int = 0) -> int:
+    """Creates the idle streams that fill HIP's pool of hardware queues (once per process), so that the contexts
+    created afterwards get a hardware queue each; returns the number of hardware queues."""
+    rc = load_library().nncase_hip_fill_queue_pool(device)
+    if rc <= 0:
+        raise HipError(rc, "fill_queue_pool")
+    return rc
 
 
 def qp(zero_point: int, scale: float) -> QuantParam:

@@ -268,6 +268,18 @@ def test_lanes_split_the_batch_bit_exact(hip_ctx, lanes, capture):
         assert np.array_equal(many.run(x).view(np.uint32), y1.view(np.uint32)), f"replay {r}"
 
 
+def test_queue_pool_is_filled_once(hip_ctx):
+    """The idle streams that spread later contexts over the hardware queues are created once per process; the call
+    reports the number of hardware queues (HIP's default of 4 unless GPU_MAX_HW_QUEUES says otherwise)."""
+    import os
+    from nncase_amd import runtime as rt
+    want = int(os.environ.get("GPU_MAX_HW_QUEUES", "4") or 4)
+    assert rt.fill_queue_pool(0) == want and rt.fill_queue_pool(0) == want
+    with pytest.raises(rt.HipError) as e:
+        rt.fill_queue_pool(999)
+    assert e.value.code == -19
+
+
 def test_copies_in_flight_give_the_bytes_of_one_function(hip_ctx):
     """HipPipeline: steps enqueued in turn on copies of the function (own stream, own buffers) overlap on the device;
     every copy still holds the bytes a single function computes, whatever was in flight beside it."""
