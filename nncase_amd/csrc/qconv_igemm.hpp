@@ -971,10 +971,20 @@ template <int T, int RG, bool PLAIN> __global__ void __launch_bounds__(kThreads,
         return f;
     };
 
-    int mt = blockIdx.x;
+    // Tiles in the order of the tensor, a contiguous eighth of them per XCD (workgroups go to the 8 XCDs round-robin, each
+    // XCD with an L2 of its own): the tiles that share input rows -- vertical neighbours -- then run on one XCD at about
+    // the same time and the shared rows are fetched from memory once (with tiles dealt round-robin the 6x6 stem over
+    // 640x640 images fetched 3.2 times its input).
+    int mt = blockIdx.x, mt_step = gridDim.x, mt_end = a.num_mtiles;
+    if (gridDim.y == 1 && (gridDim.x & 7u) == 0) {
+        const int xcd = blockIdx.x & 7, per = (a.num_mtiles + 7) >> 3;
+        mt = xcd * per + (int)(blockIdx.x >> 3);
+        mt_step = gridDim.x >> 3;
+        mt_end = min(a.num_mtiles, (xcd + 1) * per);
+    }
     Origin org[RG];
     WindowSlice cur[RG];
-    if (mt < a.num_mtiles) {
+    if (mt < mt_end) {
 #pragma unroll
         for (int rg = 0; rg < RG; rg++) {
             org[rg] = origin(mt, rg);
@@ -984,10 +994,10 @@ template <int T, int RG, bool PLAIN> __global__ void __launch_bounds__(kThreads,
     const int last = KS - 1;
     const int ch0 = ch_base + gq * (4 * T);
 #pragma clang loop unroll(disable)
-    for (; mt < a.num_mtiles; mt += gridDim.x) {
+    for (; mt < mt_end; mt += mt_step) {
         v4i acc[RG][T];
         v4i rs[RG];
-        const int mt_next = mt + gridDim.x < a.num_mtiles ? mt + gridDim.x : mt; // past the end: re-read this tile, dropped
+        const int mt_next = mt + mt_step < mt_end ? mt + mt_step : mt; // past the end: re-read this tile, dropped
         Origin org_next[RG];
 #pragma unroll
         for (int rg = 0; rg < RG; rg++) org_next[rg] = origin(mt_next, rg);

@@ -80,10 +80,13 @@ __global__ __launch_bounds__(WM * WN * 64, 2) void qconv_wide_kernel(const Igemm
     uint8_t *ring = lutl + 256 + PIX * sizeof(int32_t);              // [kWideSlots][SLOT]
 
     // channel chunks of a pixel tile are consecutive on one XCD (blocks go to the 8 XCDs round-robin)
+    // ... and every XCD takes a contiguous eighth of the pixel tiles, in the order of the tensor: the tiles that share
+    // input rows of a window (vertical neighbours) then run on one XCD at about the same time
     const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3;
     const int chunk = seq % nchunks;
-    const int mt = (seq / nchunks) * 8 + xcd;
-    if (mt >= a.num_mtiles) return;
+    const int per = (a.num_mtiles + 7) >> 3;
+    const int mt = xcd * per + seq / nchunks;
+    if (seq / nchunks >= per || mt >= a.num_mtiles) return;
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
