@@ -41,51 +41,51 @@ INT8_PEAK_TOPS = 5000.0    # dense int8 MFMA
 # are recorded here and reported only for the configuration they were measured on.
 MEASURED_TRAFFIC_B64 = {
     "unfused": {
-        "dw3x3<S=1>": 19062930,
-        "dw3x3<S=2>": 41864194,
-        "qconv_igemm+add<T=2,RG=1,rows16>": 13037132,
-        "qconv_igemm+add<T=2,RG=2,rows16>": 39622124,
-        "qconv_igemm<T=1,RG=1,rows16>": 3347003,
-        "qconv_igemm<T=1,RG=4,rows16>": 38603062,
-        "qconv_igemm<T=12,RG=1,rows16>": 10266014,
-        "qconv_igemm<T=2,RG=1,rows16>": 8914666,
-        "qconv_igemm<T=2,RG=2,rows16>": 24172938,
-        "qconv_igemm<T=2,RG=2,vec16>": 50436234,
-        "qconv_igemm<T=5,RG=1,rows16>": 5104437,
-        "qconv_igemm<T=6,RG=2,rows16>": 90039579,
-        "qconv_igemm<T=8,RG=1,rows16>": 5905454,
-        "qconv_igemm<T=9,RG=1,rows8>": 34301150,
-        "qconv_wide+add<T=2,RG=2,rows16>": 6241416,
-        "qconv_wide+add<T=4,RG=2,rows16>": 10526164,
-        "qconv_wide+dequantize<T=2,RG=2,rows16>": 1710333,
-        "qconv_wide<T=2,RG=2,rows16>": 4931864,
-        "qconv_wide<T=4,RG=2,rows16>": 7643263,
-        "qglobal_avgpool": 4238939,
+        "dw3x3<S=1>": 19028851,
+        "dw3x3<S=2>": 41847409,
+        "qconv_igemm+add<T=2,RG=1,rows16>": 13037164,
+        "qconv_igemm+add<T=2,RG=2,rows16>": 39859713,
+        "qconv_igemm<T=1,RG=1,rows16>": 3347259,
+        "qconv_igemm<T=1,RG=4,rows16>": 38602998,
+        "qconv_igemm<T=12,RG=1,rows16>": 10265961,
+        "qconv_igemm<T=2,RG=1,rows16>": 8914698,
+        "qconv_igemm<T=2,RG=2,rows16>": 24173898,
+        "qconv_igemm<T=2,RG=2,vec16>": 38614115,
+        "qconv_igemm<T=5,RG=1,rows16>": 5104416,
+        "qconv_igemm<T=6,RG=2,rows16>": 90039323,
+        "qconv_igemm<T=8,RG=1,rows16>": 5905422,
+        "qconv_igemm<T=9,RG=1,rows8>": 34301118,
+        "qconv_wide+add<T=2,RG=2,rows16>": 6175994,
+        "qconv_wide+add<T=4,RG=2,rows16>": 10527284,
+        "qconv_wide+dequantize<T=2,RG=2,rows16>": 1710205,
+        "qconv_wide<T=2,RG=2,rows16>": 4713534,
+        "qconv_wide<T=4,RG=2,rows16>": 7447634,
+        "qglobal_avgpool": 4239099,
         "quantize+pack": 51434890,
     },
     "fused": {
-        "dw3x3<S=1>": 27991460,
-        "dw3x3<S=2>": 51739642,
-        "qblock+add<S=1,P=2>": 4954891,
+        "dw3x3<S=1>": 27882249,
+        "dw3x3<S=2>": 51731083,
+        "qblock+add<S=1,P=2>": 4954955,
         "qblock+add<S=1,P=4>": 2669235,
-        "qblock+add<S=1,P=6>": 4553131,
-        "qblock<S=1,P=6>": 3246964,
-        "qblock<S=2,P=4>": 3355193,
-        "qconv_igemm+add<T=2,RG=2,rows16>": 39652422,
-        "qconv_igemm<T=1,RG=4,rows16>": 38603190,
-        "qconv_igemm<T=12,RG=1,rows16>": 9114575,
-        "qconv_igemm<T=2,RG=1,rows16>": 8914698,
-        "qconv_igemm<T=2,RG=2,rows16>": 24172522,
-        "qconv_igemm<T=2,RG=2,vec16>": 50436650,
-        "qconv_igemm<T=5,RG=1,rows16>": 5104416,
-        "qconv_igemm<T=6,RG=2,rows16>": 90039099,
-        "qconv_igemm<T=9,RG=1,rows8>": 34301902,
-        "qconv_wide+add<T=2,RG=2,rows16>": 5419156,
-        "qconv_wide+dequantize<T=2,RG=2,rows16>": 1710333,
-        "qconv_wide<T=2,RG=2,rows16>": 4932631,
-        "qconv_wide<T=4,RG=2,rows16>": 8621259,
-        "qglobal_avgpool": 4238843,
-        "quantize+pack": 51434858,
+        "qblock+add<S=1,P=6>": 4553259,
+        "qblock<S=1,P=6>": 3246740,
+        "qblock<S=2,P=4>": 3355417,
+        "qconv_igemm+add<T=2,RG=2,rows16>": 39841988,
+        "qconv_igemm<T=1,RG=4,rows16>": 38602966,
+        "qconv_igemm<T=12,RG=1,rows16>": 9114287,
+        "qconv_igemm<T=2,RG=1,rows16>": 8914666,
+        "qconv_igemm<T=2,RG=2,rows16>": 24176233,
+        "qconv_igemm<T=2,RG=2,vec16>": 38614243,
+        "qconv_igemm<T=5,RG=1,rows16>": 5104363,
+        "qconv_igemm<T=6,RG=2,rows16>": 90039131,
+        "qconv_igemm<T=9,RG=1,rows8>": 34300750,
+        "qconv_wide+add<T=2,RG=2,rows16>": 5250994,
+        "qconv_wide+dequantize<T=2,RG=2,rows16>": 1710205,
+        "qconv_wide<T=2,RG=2,rows16>": 4714430,
+        "qconv_wide<T=4,RG=2,rows16>": 8201110,
+        "qglobal_avgpool": 4238971,
+        "quantize+pack": 51434890,
     },
 }
 
