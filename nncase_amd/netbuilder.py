@@ -689,6 +689,7 @@ class HipModel:
                 sc, sh_, sw_ = src.out_shape
                 axes, lns = ([3], [cc]) if n.op == "padc" else ([1, 2, 3], [2, 2, 4])
                 if i in self.fused_quant:
+                    members = [self.fused_quant[i]] + members    # the operator also computes the input's quantisation
                     self.fn.add_quantize_pack(self.input_f32.view(lane * self._lane_stride(in_per * 4), in_per * 4), buf,
                                               [bl, sh_, sw_, sc], axes, lns, qp(*src.out_qp))
                 else:
