@@ -346,7 +346,7 @@ def main():
     ap.add_argument("--in-flight", type=int, default=4,
                     help="copies of the function (own stream and buffers each) that take the steps in turn, so that "
                          "consecutive steps overlap on the device (1 = one step at a time)")
-    ap.add_argument("--cpu-images", type=int, default=8, help="batch-1 images timed on the CPU baseline (0 = skip)")
+    ap.add_argument("--cpu-images", type=int, default=32, help="batch-1 images timed on the CPU baseline (0 = skip)")
     ap.add_argument("--profile-iters", type=int, default=10)
     ap.add_argument("--batch1-steps", type=int, default=200, help="timed batch-1 invocations (0 = skip the batch-1 figure)")
     ap.add_argument("--fuse-blocks", action="store_true",
