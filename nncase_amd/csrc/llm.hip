@@ -212,6 +212,7 @@ template <int MT, int G, bool SPLIT> __global__ __launch_bounds__(kGemmThreads) 
         if (a.ln_w) {
 #pragma unroll
             for (int u = 0; u < kGemmBatch; u++)
+                if (kb + u < ks1) // (uniform for the wave: the slices past its share are not multiplied)
 #pragma unroll
                 for (int t = 0; t < MT; t++)
 #pragma unroll
@@ -282,6 +283,98 @@ template <int MT, int G, bool SPLIT> __global__ __launch_bounds__(kGemmThreads) 
             }
         if (m >= a.m) continue;
         store_gemm_row<G>(a, v, (size_t)m * a.n_out + out_tile * 16 + kg * 4);
+    }
+}
+
+// Many output tiles and a reduction short enough for the token rows to fit in LDS (the vocabulary head): a wave owns
+// a tile and the whole reduction, as in the kernel above without SPLIT, but the block's eight waves share the token rows
+// through LDS, normalised once per block instead of once per wave, and a wave has the weights of eight k-steps in flight.
+// The arithmetic per element and the order of the multiply-adds are those of the kernel above.
+constexpr int kRowsBatch = 8;
+inline int rows_in_lds_pitch(int k) { return k * 2 + 16; } // bytes per token row: the padding spreads the rows over the banks
+
+template <int MT> __global__ __launch_bounds__(kGemmThreads) void w8a16_gemm_rows_in_lds_kernel(const GemmArgs a) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t xs[]; // [MT * 16][k halves + padding]
+    __shared__ float rstd[MT * 16];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int i16 = lane & 15, kg = lane >> 4;
+    const int pitch = a.k * 2 + 16;
+    if (a.ln_w) {
+        constexpr int R = MT * 16 / kGemmWaves; // rows per wave
+        float rs[R];
+        rms_rstd_rows<R>(reinterpret_cast<const __half *>(a.a), a.k, a.m, wave, kGemmWaves, lane, a.ln_eps, rs);
+        if (lane == 0) {
+#pragma unroll
+            for (int i = 0; i < R; i++)
+                if (wave + i * kGemmWaves < a.m) rstd[wave + i * kGemmWaves] = rs[i];
+        }
+        __syncthreads();
+    }
+    {   // token rows -> LDS, 8 halves per thread and trip (rows past m repeat row m - 1 and are never stored)
+        const int per_row = a.k >> 3, total = MT * 16 * per_row;
+        for (int u = threadIdx.x; u < total; u += kGemmThreads) {
+            const int r = u / per_row, c = u - r * per_row, src = min(r, a.m - 1);
+            lu32x4 v = *reinterpret_cast<const lu32x4 *>(a.a + (size_t)src * a.k + c * 8);
+            if (a.ln_w) {
+                const lu32x4 lw = *reinterpret_cast<const lu32x4 *>(a.ln_w + c * 8);
+                const float rr = rstd[src];
+                __half xh[8], wh[8];
+                __builtin_memcpy(xh, &v, 16);
+                __builtin_memcpy(wh, &lw, 16);
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    // the fp32 product is rounded before it is converted, as in rmsnorm_f16_kernel (see there)
+                    float pr = __half2float(xh[e]) * rr * __half2float(wh[e]);
+                    asm volatile("" : "+v"(pr));
+                    xh[e] = __float2half_rn(pr);
+                }
+                __builtin_memcpy(&v, xh, 16);
+            }
+            *reinterpret_cast<lu32x4 *>(xs + (size_t)r * pitch + c * 16) = v;
+        }
+    }
+    __syncthreads();
+    const int out_tile = (int)blockIdx.x * kGemmWaves + wave;
+    if (out_tile >= a.up_tile_offset) return; // the last block's spare waves (uniform per wave)
+    f32x4v acc[MT];
+#pragma unroll
+    for (int t = 0; t < MT; t++) acc[t] = f32x4v{0.f, 0.f, 0.f, 0.f};
+    const uint8_t *xl = xs + (size_t)i16 * pitch + kg * 32; // the lane's 16 reduction indices of a k-step
+    for (int kb = 0; kb < a.ksteps; kb += kRowsBatch) {
+        lu32x4 wv[kRowsBatch];
+#pragma unroll
+        for (int u = 0; u < kRowsBatch; u++) {
+            const int ks = min(kb + u, a.ksteps - 1); // steps past the end re-read the last one and are not multiplied
+            wv[u] = a.w[((size_t)out_tile * a.ksteps + ks) * 64 + lane];
+        }
+#pragma unroll
+        for (int u = 0; u < kRowsBatch; u++) {
+            if (kb + u < a.ksteps) { // uniform
+                const h16x8 w0 = w8_to_f16(wv[u][0], wv[u][1]), w1 = w8_to_f16(wv[u][2], wv[u][3]);
+#pragma unroll
+                for (int t = 0; t < MT; t++) {
+                    const uint8_t *xp = xl + (size_t)t * 16 * pitch + (size_t)(kb + u) * 128;
+                    const h16x8 x0 = *reinterpret_cast<const h16x8 *>(xp), x1 = *reinterpret_cast<const h16x8 *>(xp + 16);
+                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w0, x0, acc[t], 0, 0, 0);
+                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w1, x1, acc[t], 0, 0, 0);
+                }
+            }
+        }
+    }
+    // lane (i16 = token within the tile, kg): channels tile * 16 + kg * 4 + r
+#pragma unroll
+    for (int t = 0; t < MT; t++) {
+        const int m = t * 16 + i16;
+        float v[1][4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int ch = out_tile * 16 + kg * 4 + r;
+            float s = acc[t][r] * a.scale[ch];
+            if (a.bias) s += a.bias[ch];
+            v[0][r] = s;
+        }
+        if (m >= a.m) continue;
+        store_gemm_row<1>(a, v, (size_t)m * a.n_out + out_tile * 16 + kg * 4);
     }
 }
 
@@ -480,6 +573,27 @@ static int launch_w8a16_gemm(nncase_hip_ctx_t *ctx, const void *a_dev, const nnc
     const dim3 grid(split ? out_tiles : (out_tiles + kGemmWaves - 1) / kGemmWaves), block(kGemmThreads);
     const int mt = (m + 15) / 16;
     const bool glu = mode == NNCASE_HIP_GEMM_SWIGLU;
+    // a tile per wave with the token rows shared through LDS, where they fit
+    const int mt_built = mt <= 1 ? 1 : (mt == 2 ? 2 : 4);
+    const size_t rows_lds = (size_t)mt_built * 16 * rows_in_lds_pitch(w->k);
+    if (!split && !glu && rows_lds <= 128 * 1024 && w->k % 8 == 0) {
+#define NNHIP_ROWS_LAUNCH(MTV)                                                                                                 \
+    do {                                                                                                                       \
+        static int raised_on_device = -1;                                                                                      \
+        if (rows_lds > 48 * 1024 && raised_on_device != ctx->device) {                                                         \
+            NNHIP_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(&w8a16_gemm_rows_in_lds_kernel<MTV>),            \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024));                      \
+            raised_on_device = ctx->device;                                                                                    \
+        }                                                                                                                      \
+        hipLaunchKernelGGL((w8a16_gemm_rows_in_lds_kernel<MTV>), grid, block, rows_lds, ctx->stream, a);                      \
+    } while (0)
+        if (mt_built == 1) NNHIP_ROWS_LAUNCH(1);
+        else if (mt_built == 2) NNHIP_ROWS_LAUNCH(2);
+        else NNHIP_ROWS_LAUNCH(4);
+#undef NNHIP_ROWS_LAUNCH
+        NNHIP_LAUNCH_CHECK(ctx, "w8a16_gemm_rows_in_lds_kernel");
+        return 0;
+    }
 #define NNHIP_GEMM_LAUNCH(MTV)                                                                                                 \
     do {                                                                                                                       \
         if (glu && split) hipLaunchKernelGGL((w8a16_gemm_kernel<MTV, 2, true>), grid, block, 0, ctx->stream, a);              \

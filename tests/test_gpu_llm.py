@@ -18,7 +18,9 @@ def close(got, want, rtol=RTOL, atol=1e-3):
     assert (np.abs(got - want) <= tol).all(), f"max err {np.abs(got - want).max()} (max |want| {np.abs(want).max()})"
 
 
-@pytest.mark.parametrize("m,k,n", [(1, 64, 16), (32, 896, 1152), (7, 128, 48), (33, 192, 64), (64, 4864, 896), (16, 896, 2048)])
+@pytest.mark.parametrize("m,k,n", [(1, 64, 16), (32, 896, 1152), (7, 128, 48), (33, 192, 64), (64, 4864, 896), (16, 896, 2048),
+                                   # many output tiles: a tile per wave, the token rows shared through LDS (1, 2 and 4 row tiles)
+                                   (32, 896, 20480), (5, 128, 16400), (64, 256, 16384), (33, 192, 16384)])
 @pytest.mark.parametrize("out32", [False, True])
 def test_w8a16_gemm(hip_ctx, m, k, n, out32):
     rng = np.random.default_rng(m + k + n)
