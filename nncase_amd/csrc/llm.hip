@@ -123,14 +123,19 @@ __device__ __forceinline__ h16x8 w8_to_f16(uint32_t lo, uint32_t hi) {
     return v - (_Float16)1152.0f; // 1024 + (w + 128) - 1152 = w, exact in fp16
 }
 
-// Epilogue of 4 consecutive output channels of one token: SwiGLU gate, residual, conversion, store.
-template <int G> __device__ __forceinline__ void store_gemm_row(const GemmArgs &a, const float (&v)[G][4], size_t o) {
+// Epilogue of 4 consecutive output channels of one token: SwiGLU gate, residual, conversion, store.  `res`: the four
+// residual halves where the caller has loaded them already (have_res), else they are read here.
+template <int G> __device__ __forceinline__ void store_gemm_row(const GemmArgs &a, const float (&v)[G][4], size_t o, uint2 res = uint2{0u, 0u},
+                                                               bool have_res = false) {
     float y[4];
+    if (a.residual && !have_res) res = *reinterpret_cast<const uint2 *>(a.residual + o);
+    __half rh[4];
+    __builtin_memcpy(rh, &res, 8);
 #pragma unroll
     for (int r = 0; r < 4; r++) {
         if (G == 2) y[r] = v[0][r] / (1.f + __expf(-v[0][r])) * v[G - 1][r]; // silu(gate) * up
         else y[r] = v[0][r];
-        if (a.residual) y[r] += __half2float(reinterpret_cast<const __half *>(a.residual)[o + r]);
+        if (a.residual) y[r] += __half2float(rh[r]);
     }
     if (a.out_f32) {
         *reinterpret_cast<float4 *>(reinterpret_cast<float *>(a.out) + o) = float4{y[0], y[1], y[2], y[3]};
@@ -190,6 +195,20 @@ template <int MT, int G, bool SPLIT> __global__ __launch_bounds__(kGemmThreads) 
         rrow[t] = a.ln_w ? rstd[min(t * 16 + i16, a.m - 1)] : 1.f;
     }
 
+    // The epilogue's operands (SPLIT: of the token tile this wave finishes) are asked for before the products: the
+    // launch is a chain of memory round trips, and this takes the last one out of it.
+    float4 sc[G], bs[G];
+    uint2 res_pre = uint2{0u, 0u};
+    if (SPLIT) {
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            sc[g] = *reinterpret_cast<const float4 *>(a.scale + tile[g] * 16 + kg * 4);
+            bs[g] = float4{0.f, 0.f, 0.f, 0.f};
+            if (a.bias) bs[g] = *reinterpret_cast<const float4 *>(a.bias + tile[g] * 16 + kg * 4);
+        }
+        const int m_pre = min(min(wave, MT - 1) * 16 + i16, a.m - 1);
+        if (a.residual) res_pre = *reinterpret_cast<const uint2 *>(a.residual + (size_t)m_pre * a.n_out + out_tile * 16 + kg * 4);
+    }
     for (int kb = ks0; kb < ks1; kb += kGemmBatch) {
         lu32x4 wv[kGemmBatch][G];
         lu32x4 av[kGemmBatch][MT][2];
@@ -266,97 +285,142 @@ template <int MT, int G, bool SPLIT> __global__ __launch_bounds__(kGemmThreads) 
         const int m = t * 16 + i16;
         float v[G][4];
 #pragma unroll
-        for (int g = 0; g < G; g++)
+        for (int g = 0; g < G; g++) {
+            const float scv[4] = {sc[g].x, sc[g].y, sc[g].z, sc[g].w}, bsv[4] = {bs[g].x, bs[g].y, bs[g].z, bs[g].w};
 #pragma unroll
             for (int r = 0; r < 4; r++) {
                 float s = 0.f;
                 if (SPLIT) {
 #pragma unroll
                     for (int w = 0; w < kGemmWaves; w++) s += red[w][g][t][lane][r]; // fixed order: deterministic
+                    s *= scv[r];
+                    if (a.bias) s += bsv[r];
                 } else {
                     s = acc[g][tt][r];
+                    const int ch = tile[g] * 16 + kg * 4 + r;
+                    s *= a.scale[ch];
+                    if (a.bias) s += a.bias[ch];
                 }
-                const int ch = tile[g] * 16 + kg * 4 + r;
-                s *= a.scale[ch];
-                if (a.bias) s += a.bias[ch];
                 v[g][r] = s;
             }
+        }
         if (m >= a.m) continue;
-        store_gemm_row<G>(a, v, (size_t)m * a.n_out + out_tile * 16 + kg * 4);
+        store_gemm_row<G>(a, v, (size_t)m * a.n_out + out_tile * 16 + kg * 4, res_pre, SPLIT);
     }
 }
 
-// Many output tiles and a reduction short enough for the token rows to fit in LDS (the vocabulary head): a wave owns
-// a tile and the whole reduction, as in the kernel above without SPLIT, but the block's eight waves share the token rows
-// through LDS, normalised once per block instead of once per wave, and a wave has the weights of eight k-steps in flight.
-// The arithmetic per element and the order of the multiply-adds are those of the kernel above.
+// Many output tiles and a reduction short enough for the token rows to fit in LDS (the vocabulary head, the gate / up
+// projection): a wave owns a tile (G = 2: the gate tile and its up tile) and the whole reduction, as in the kernel
+// above without SPLIT, but the block's waves share the token rows through LDS.  A wave brings in whole rows (row
+// wave, wave + WAVES, ...): it adds their squares in rms_rstd_rows' order as they arrive, parks them in LDS as loaded,
+// and, knowing 1 / sqrt(mean + eps) of its own rows without asking another wave, normalises them in place -- one trip
+// to memory and one barrier in front of the products, and every element normalised once per block instead of once per
+// wave.  A wave has the weights of eight k-steps in flight.  The arithmetic per element and the order of the
+// multiply-adds are those of the kernel above.
 constexpr int kRowsBatch = 8;
+constexpr int kRowsPieces = 4;                 // 512-element pieces of a row: k <= 2048
+constexpr int kRowsMaxK = kRowsPieces * 512;
 inline int rows_in_lds_pitch(int k) { return k * 2 + 16; } // bytes per token row: the padding spreads the rows over the banks
 
-template <int MT> __global__ __launch_bounds__(kGemmThreads) void w8a16_gemm_rows_in_lds_kernel(const GemmArgs a) {
+template <int MT, int G, int WAVES> __global__ __launch_bounds__(WAVES * 64) void w8a16_gemm_rows_in_lds_kernel(const GemmArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t xs[]; // [MT * 16][k halves + padding]
-    __shared__ float rstd[MT * 16];
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int i16 = lane & 15, kg = lane >> 4;
     const int pitch = a.k * 2 + 16;
-    if (a.ln_w) {
-        constexpr int R = MT * 16 / kGemmWaves; // rows per wave
-        float rs[R];
-        rms_rstd_rows<R>(reinterpret_cast<const __half *>(a.a), a.k, a.m, wave, kGemmWaves, lane, a.ln_eps, rs);
-        if (lane == 0) {
+    {
+        constexpr int R = MT * 16 / WAVES; // rows per wave
+        lu32x4 lwp[kRowsPieces];
+        if (a.ln_w) {
 #pragma unroll
-            for (int i = 0; i < R; i++)
-                if (wave + i * kGemmWaves < a.m) rstd[wave + i * kGemmWaves] = rs[i];
-        }
-        __syncthreads();
-    }
-    {   // token rows -> LDS, 8 halves per thread and trip (rows past m repeat row m - 1 and are never stored)
-        const int per_row = a.k >> 3, total = MT * 16 * per_row;
-        for (int u = threadIdx.x; u < total; u += kGemmThreads) {
-            const int r = u / per_row, c = u - r * per_row, src = min(r, a.m - 1);
-            lu32x4 v = *reinterpret_cast<const lu32x4 *>(a.a + (size_t)src * a.k + c * 8);
-            if (a.ln_w) {
-                const lu32x4 lw = *reinterpret_cast<const lu32x4 *>(a.ln_w + c * 8);
-                const float rr = rstd[src];
-                __half xh[8], wh[8];
-                __builtin_memcpy(xh, &v, 16);
-                __builtin_memcpy(wh, &lw, 16);
-#pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    // the fp32 product is rounded before it is converted, as in rmsnorm_f16_kernel (see there)
-                    float pr = __half2float(xh[e]) * rr * __half2float(wh[e]);
-                    asm volatile("" : "+v"(pr));
-                    xh[e] = __float2half_rn(pr);
-                }
-                __builtin_memcpy(&v, xh, 16);
+            for (int p = 0; p < kRowsPieces; p++) {
+                const int e0 = lane * 8 + p * 512;
+                lwp[p] = lu32x4{0, 0, 0, 0};
+                if (e0 < a.k) lwp[p] = *reinterpret_cast<const lu32x4 *>(a.ln_w + e0);
             }
-            *reinterpret_cast<lu32x4 *>(xs + (size_t)r * pitch + c * 16) = v;
+        }
+        float ss[R];
+#pragma unroll
+        for (int i = 0; i < R; i++) ss[i] = 0.f;
+#pragma unroll
+        for (int p = 0; p < kRowsPieces; p++) {
+            const int e0 = lane * 8 + p * 512;
+            if (e0 < a.k) {
+                lu32x4 v[R];
+#pragma unroll
+                for (int i = 0; i < R; i++) {
+                    const int r = wave + i * WAVES;
+                    v[i] = lu32x4{0, 0, 0, 0}; // rows past m: zeros (their products are never stored)
+                    if (r < a.m) v[i] = *reinterpret_cast<const lu32x4 *>(a.a + (size_t)r * a.k + e0);
+                }
+#pragma unroll
+                for (int i = 0; i < R; i++) {
+                    if (a.ln_w) add_squares8(v[i], ss[i]);
+                    *reinterpret_cast<lu32x4 *>(xs + (size_t)(wave + i * WAVES) * pitch + e0 * 2) = v[i];
+                }
+            }
+        }
+        if (a.ln_w) {
+#pragma unroll
+            for (int i = 0; i < R; i++) {
+                const float rr = rstd_from_sum(ss[i], a.k, a.ln_eps);
+#pragma unroll
+                for (int p = 0; p < kRowsPieces; p++) {
+                    const int e0 = lane * 8 + p * 512;
+                    if (e0 < a.k) {
+                        lu32x4 *slot = reinterpret_cast<lu32x4 *>(xs + (size_t)(wave + i * WAVES) * pitch + e0 * 2);
+                        lu32x4 v = *slot; // (the lane's own bytes: LDS operations of a wave complete in order)
+                        __half xh[8], wh[8];
+                        __builtin_memcpy(xh, &v, 16);
+                        __builtin_memcpy(wh, &lwp[p], 16);
+#pragma unroll
+                        for (int e = 0; e < 8; e++) {
+                            // the fp32 product is rounded before it is converted, as in rmsnorm_f16_kernel (see there)
+                            float pr = __half2float(xh[e]) * rr * __half2float(wh[e]);
+                            asm volatile("" : "+v"(pr));
+                            xh[e] = __float2half_rn(pr);
+                        }
+                        __builtin_memcpy(&v, xh, 16);
+                        *slot = v;
+                    }
+                }
+            }
         }
     }
     __syncthreads();
-    const int out_tile = (int)blockIdx.x * kGemmWaves + wave;
+    const int out_tile = (int)blockIdx.x * WAVES + wave;
     if (out_tile >= a.up_tile_offset) return; // the last block's spare waves (uniform per wave)
-    f32x4v acc[MT];
+    const int tile[2] = {out_tile, out_tile + a.up_tile_offset};
+    f32x4v acc[G][MT];
 #pragma unroll
-    for (int t = 0; t < MT; t++) acc[t] = f32x4v{0.f, 0.f, 0.f, 0.f};
+    for (int g = 0; g < G; g++)
+#pragma unroll
+        for (int t = 0; t < MT; t++) acc[g][t] = f32x4v{0.f, 0.f, 0.f, 0.f};
     const uint8_t *xl = xs + (size_t)i16 * pitch + kg * 32; // the lane's 16 reduction indices of a k-step
     for (int kb = 0; kb < a.ksteps; kb += kRowsBatch) {
-        lu32x4 wv[kRowsBatch];
+        lu32x4 wv[kRowsBatch][G];
 #pragma unroll
         for (int u = 0; u < kRowsBatch; u++) {
             const int ks = min(kb + u, a.ksteps - 1); // steps past the end re-read the last one and are not multiplied
-            wv[u] = a.w[((size_t)out_tile * a.ksteps + ks) * 64 + lane];
+#pragma unroll
+            for (int g = 0; g < G; g++) wv[u][g] = a.w[((size_t)tile[g] * a.ksteps + ks) * 64 + lane];
         }
 #pragma unroll
         for (int u = 0; u < kRowsBatch; u++) {
             if (kb + u < a.ksteps) { // uniform
-                const h16x8 w0 = w8_to_f16(wv[u][0], wv[u][1]), w1 = w8_to_f16(wv[u][2], wv[u][3]);
+                h16x8 x0[MT], x1[MT];
 #pragma unroll
                 for (int t = 0; t < MT; t++) {
                     const uint8_t *xp = xl + (size_t)t * 16 * pitch + (size_t)(kb + u) * 128;
-                    const h16x8 x0 = *reinterpret_cast<const h16x8 *>(xp), x1 = *reinterpret_cast<const h16x8 *>(xp + 16);
-                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w0, x0, acc[t], 0, 0, 0);
-                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w1, x1, acc[t], 0, 0, 0);
+                    x0[t] = *reinterpret_cast<const h16x8 *>(xp), x1[t] = *reinterpret_cast<const h16x8 *>(xp + 16);
+                }
+#pragma unroll
+                for (int g = 0; g < G; g++) {
+                    const h16x8 w0 = w8_to_f16(wv[u][g][0], wv[u][g][1]), w1 = w8_to_f16(wv[u][g][2], wv[u][g][3]);
+#pragma unroll
+                    for (int t = 0; t < MT; t++) {
+                        acc[g][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w0, x0[t], acc[g][t], 0, 0, 0);
+                        acc[g][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w1, x1[t], acc[g][t], 0, 0, 0);
+                    }
                 }
             }
         }
@@ -365,16 +429,18 @@ template <int MT> __global__ __launch_bounds__(kGemmThreads) void w8a16_gemm_row
 #pragma unroll
     for (int t = 0; t < MT; t++) {
         const int m = t * 16 + i16;
-        float v[1][4];
+        float v[G][4];
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-            const int ch = out_tile * 16 + kg * 4 + r;
-            float s = acc[t][r] * a.scale[ch];
-            if (a.bias) s += a.bias[ch];
-            v[0][r] = s;
-        }
+        for (int g = 0; g < G; g++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int ch = tile[g] * 16 + kg * 4 + r;
+                float s = acc[g][t][r] * a.scale[ch];
+                if (a.bias) s += a.bias[ch];
+                v[g][r] = s;
+            }
         if (m >= a.m) continue;
-        store_gemm_row<1>(a, v, (size_t)m * a.n_out + out_tile * 16 + kg * 4);
+        store_gemm_row<G>(a, v, (size_t)m * a.n_out + out_tile * 16 + kg * 4);
     }
 }
 
@@ -555,6 +621,8 @@ static int launch_w8a16_gemm(nncase_hip_ctx_t *ctx, const void *a_dev, const nnc
                   "w8a16_gemm: SwiGLU needs gate and up halves of equal size");
     NNHIP_REQUIRE(ctx, ((reinterpret_cast<uintptr_t>(a_dev) | reinterpret_cast<uintptr_t>(out_dev)) & 15u) == 0,
                   -NNCASE_HIP_ERR_INVALID_MEMORY_LOCATION, "w8a16_gemm: buffers must be 16-byte aligned");
+    NNHIP_REQUIRE(ctx, (reinterpret_cast<uintptr_t>(residual_dev) & 7u) == 0, -NNCASE_HIP_ERR_INVALID_MEMORY_LOCATION,
+                  "w8a16_gemm: the residual must be 8-byte aligned");
     GemmArgs a;
     memset(&a, 0, sizeof(a));
     a.a = (const uint16_t *)a_dev;
@@ -573,23 +641,33 @@ static int launch_w8a16_gemm(nncase_hip_ctx_t *ctx, const void *a_dev, const nnc
     const dim3 grid(split ? out_tiles : (out_tiles + kGemmWaves - 1) / kGemmWaves), block(kGemmThreads);
     const int mt = (m + 15) / 16;
     const bool glu = mode == NNCASE_HIP_GEMM_SWIGLU;
-    // a tile per wave with the token rows shared through LDS, where they fit
+    // a tile per wave with the token rows shared through LDS: where the rows fit and the launch has a tile for every
+    // compute unit (measured on the decode step: the 72- and 56-tile products are quicker with the reduction split
+    // over a block's waves, 9.7 against 11.2 us; the 304 gate / up tile pairs take 12.5 us in 38 blocks of eight waves,
+    // 13.9 us in 76 blocks of four and 18 us split)
     const int mt_built = mt <= 1 ? 1 : (mt == 2 ? 2 : 4);
     const size_t rows_lds = (size_t)mt_built * 16 * rows_in_lds_pitch(w->k);
-    if (!split && !glu && rows_lds <= 128 * 1024 && w->k % 8 == 0) {
-#define NNHIP_ROWS_LAUNCH(MTV)                                                                                                 \
+    if (w->k <= kRowsMaxK && rows_lds <= 128 * 1024 && out_tiles >= ctx->compute_units) {
+        const dim3 rgrid((out_tiles + kGemmWaves - 1) / kGemmWaves), rblock(kGemmThreads);
+#define NNHIP_ROWS_LAUNCH(MTV, GV)                                                                                             \
     do {                                                                                                                       \
         static int raised_on_device = -1;                                                                                      \
         if (rows_lds > 48 * 1024 && raised_on_device != ctx->device) {                                                         \
-            NNHIP_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(&w8a16_gemm_rows_in_lds_kernel<MTV>),            \
+            NNHIP_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(&w8a16_gemm_rows_in_lds_kernel<MTV, GV, kGemmWaves>), \
                                                hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024));                      \
             raised_on_device = ctx->device;                                                                                    \
         }                                                                                                                      \
-        hipLaunchKernelGGL((w8a16_gemm_rows_in_lds_kernel<MTV>), grid, block, rows_lds, ctx->stream, a);                      \
+        hipLaunchKernelGGL((w8a16_gemm_rows_in_lds_kernel<MTV, GV, kGemmWaves>), rgrid, rblock, rows_lds, ctx->stream, a);    \
     } while (0)
-        if (mt_built == 1) NNHIP_ROWS_LAUNCH(1);
-        else if (mt_built == 2) NNHIP_ROWS_LAUNCH(2);
-        else NNHIP_ROWS_LAUNCH(4);
+        if (glu) {
+            if (mt_built == 1) NNHIP_ROWS_LAUNCH(1, 2);
+            else if (mt_built == 2) NNHIP_ROWS_LAUNCH(2, 2);
+            else NNHIP_ROWS_LAUNCH(4, 2);
+        } else {
+            if (mt_built == 1) NNHIP_ROWS_LAUNCH(1, 1);
+            else if (mt_built == 2) NNHIP_ROWS_LAUNCH(2, 1);
+            else NNHIP_ROWS_LAUNCH(4, 1);
+        }
 #undef NNHIP_ROWS_LAUNCH
         NNHIP_LAUNCH_CHECK(ctx, "w8a16_gemm_rows_in_lds_kernel");
         return 0;
