@@ -396,6 +396,13 @@ template <int MT, int G, int WAVES> __global__ __launch_bounds__(WAVES * 64) voi
 #pragma unroll
         for (int t = 0; t < MT; t++) acc[g][t] = f32x4v{0.f, 0.f, 0.f, 0.f};
     const uint8_t *xl = xs + (size_t)i16 * pitch + kg * 32; // the lane's 16 reduction indices of a k-step
+    float4 sc[G], bs[G]; // the epilogue's constants, asked for before the products
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+        sc[g] = *reinterpret_cast<const float4 *>(a.scale + tile[g] * 16 + kg * 4);
+        bs[g] = float4{0.f, 0.f, 0.f, 0.f};
+        if (a.bias) bs[g] = *reinterpret_cast<const float4 *>(a.bias + tile[g] * 16 + kg * 4);
+    }
     for (int kb = 0; kb < a.ksteps; kb += kRowsBatch) {
         lu32x4 wv[kRowsBatch][G];
 #pragma unroll
@@ -431,14 +438,15 @@ template <int MT, int G, int WAVES> __global__ __launch_bounds__(WAVES * 64) voi
         const int m = t * 16 + i16;
         float v[G][4];
 #pragma unroll
-        for (int g = 0; g < G; g++)
+        for (int g = 0; g < G; g++) {
+            const float scv[4] = {sc[g].x, sc[g].y, sc[g].z, sc[g].w}, bsv[4] = {bs[g].x, bs[g].y, bs[g].z, bs[g].w};
 #pragma unroll
             for (int r = 0; r < 4; r++) {
-                const int ch = tile[g] * 16 + kg * 4 + r;
-                float s = acc[g][t][r] * a.scale[ch];
-                if (a.bias) s += a.bias[ch];
+                float s = acc[g][t][r] * scv[r];
+                if (a.bias) s += bsv[r];
                 v[g][r] = s;
             }
+        }
         if (m >= a.m) continue;
         store_gemm_row<G>(a, v, (size_t)m * a.n_out + out_tile * 16 + kg * 4);
     }
