@@ -155,11 +155,11 @@ template <int G> __device__ __forceinline__ void store_gemm_row(const GemmArgs &
 // whole share of a short reduction (896 / 8 waves = 2 k-steps) is a single memory round trip.
 constexpr int kGemmWaves = 8;
 constexpr int kGemmThreads = kGemmWaves * 64;
-constexpr int kGemmBatch = 4;
+constexpr int kGemmBatch = 4; // k-steps a wave requests before it multiplies any (5 where that halves a long share's trips to memory)
 
 // SPLIT: the block's waves share one output tile and split its reduction (few tiles, long reductions);
 // otherwise every wave owns a tile of its own and the whole reduction (many tiles: the vocabulary head).
-template <int MT, int G, bool SPLIT> __global__ __launch_bounds__(kGemmThreads) void w8a16_gemm_kernel(const GemmArgs a) {
+template <int MT, int G, bool SPLIT, int B = kGemmBatch> __global__ __launch_bounds__(kGemmThreads) void w8a16_gemm_kernel(const GemmArgs a) {
     __shared__ float red[SPLIT ? kGemmWaves : 1][G][MT][64][4];
     __shared__ float rstd[MT * 16];
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -209,12 +209,12 @@ template <int MT, int G, bool SPLIT> __global__ __launch_bounds__(kGemmThreads) 
         const int m_pre = min(min(wave, MT - 1) * 16 + i16, a.m - 1);
         if (a.residual) res_pre = *reinterpret_cast<const uint2 *>(a.residual + (size_t)m_pre * a.n_out + out_tile * 16 + kg * 4);
     }
-    for (int kb = ks0; kb < ks1; kb += kGemmBatch) {
-        lu32x4 wv[kGemmBatch][G];
-        lu32x4 av[kGemmBatch][MT][2];
-        lu32x4 lw[kGemmBatch][2]; // the normalisation weights of the lane's 16 reduction indices
+    for (int kb = ks0; kb < ks1; kb += B) {
+        lu32x4 wv[B][G];
+        lu32x4 av[B][MT][2];
+        lu32x4 lw[B][2]; // the normalisation weights of the lane's 16 reduction indices
 #pragma unroll
-        for (int u = 0; u < kGemmBatch; u++) {
+        for (int u = 0; u < B; u++) {
             const int ks = min(kb + u, ks1 - 1); // steps past the share re-read the last one and are not multiplied
 #pragma unroll
             for (int g = 0; g < G; g++) wv[u][g] = a.w[((size_t)tile[g] * a.ksteps + ks) * 64 + lane];
@@ -230,7 +230,7 @@ template <int MT, int G, bool SPLIT> __global__ __launch_bounds__(kGemmThreads) 
         }
         if (a.ln_w) {
 #pragma unroll
-            for (int u = 0; u < kGemmBatch; u++)
+            for (int u = 0; u < B; u++)
                 if (kb + u < ks1) // (uniform for the wave: the slices past its share are not multiplied)
 #pragma unroll
                 for (int t = 0; t < MT; t++)
@@ -250,7 +250,7 @@ template <int MT, int G, bool SPLIT> __global__ __launch_bounds__(kGemmThreads) 
                     }
         }
 #pragma unroll
-        for (int u = 0; u < kGemmBatch; u++) {
+        for (int u = 0; u < B; u++) {
             if (kb + u < ks1) { // uniform for the wave
 #pragma unroll
                 for (int g = 0; g < G; g++) {
@@ -680,10 +680,14 @@ static int launch_w8a16_gemm(nncase_hip_ctx_t *ctx, const void *a_dev, const nnc
         NNHIP_LAUNCH_CHECK(ctx, "w8a16_gemm_rows_in_lds_kernel");
         return 0;
     }
+    // a share of 9 or 10 k-steps per wave (the 4864-deep down projection): two requests of five instead of 4 + 4 + 2
+    const int share = (w->ksteps + kGemmWaves - 1) / kGemmWaves;
+    const bool long_share = !ln_weight_dev && mt <= 2 && (share == 5 || share == 9 || share == 10);
 #define NNHIP_GEMM_LAUNCH(MTV)                                                                                                 \
     do {                                                                                                                       \
         if (glu && split) hipLaunchKernelGGL((w8a16_gemm_kernel<MTV, 2, true>), grid, block, 0, ctx->stream, a);              \
         else if (glu) hipLaunchKernelGGL((w8a16_gemm_kernel<MTV, 2, false>), grid, block, 0, ctx->stream, a);                 \
+        else if (split && long_share) hipLaunchKernelGGL((w8a16_gemm_kernel<MTV, 1, true, 5>), grid, block, 0, ctx->stream, a); \
         else if (split) hipLaunchKernelGGL((w8a16_gemm_kernel<MTV, 1, true>), grid, block, 0, ctx->stream, a);                \
         else hipLaunchKernelGGL((w8a16_gemm_kernel<MTV, 1, false>), grid, block, 0, ctx->stream, a);                          \
     } while (0)
