@@ -322,8 +322,11 @@ constexpr int kRowsPieces = 4;                 // 512-element pieces of a row: k
 constexpr int kRowsMaxK = kRowsPieces * 512;
 inline int rows_in_lds_pitch(int k) { return k * 2 + 16; } // bytes per token row: the padding spreads the rows over the banks
 
-template <int MT, int G, int WAVES> __global__ __launch_bounds__(WAVES * 64) void w8a16_gemm_rows_in_lds_kernel(const GemmArgs a) {
+// SPLIT: the block's waves share ONE output tile and split its reduction (few tiles: the q / k / v projection), combined
+// through LDS in the fixed order of the kernel above.
+template <int MT, int G, int WAVES, bool SPLIT = false> __global__ __launch_bounds__(WAVES * 64) void w8a16_gemm_rows_in_lds_kernel(const GemmArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t xs[]; // [MT * 16][k halves + padding]
+    __shared__ float red[SPLIT ? WAVES : 1][G][SPLIT ? MT : 1][64][4];
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int i16 = lane & 15, kg = lane >> 4;
     const int pitch = a.k * 2 + 16;
@@ -387,8 +390,10 @@ template <int MT, int G, int WAVES> __global__ __launch_bounds__(WAVES * 64) voi
         }
     }
     __syncthreads();
-    const int out_tile = (int)blockIdx.x * WAVES + wave;
-    if (out_tile >= a.up_tile_offset) return; // the last block's spare waves (uniform per wave)
+    const int out_tile = SPLIT ? (int)blockIdx.x : (int)blockIdx.x * WAVES + wave;
+    if (out_tile >= a.up_tile_offset) return; // SPLIT: never; otherwise the last block's spare waves (uniform per wave)
+    const int per = SPLIT ? (a.ksteps + WAVES - 1) / WAVES : a.ksteps;
+    const int ks0 = SPLIT ? wave * per : 0, ks1 = min(a.ksteps, ks0 + per);
     const int tile[2] = {out_tile, out_tile + a.up_tile_offset};
     f32x4v acc[G][MT];
 #pragma unroll
@@ -396,24 +401,27 @@ template <int MT, int G, int WAVES> __global__ __launch_bounds__(WAVES * 64) voi
 #pragma unroll
         for (int t = 0; t < MT; t++) acc[g][t] = f32x4v{0.f, 0.f, 0.f, 0.f};
     const uint8_t *xl = xs + (size_t)i16 * pitch + kg * 32; // the lane's 16 reduction indices of a k-step
-    float4 sc[G], bs[G]; // the epilogue's constants, asked for before the products
+    float4 sc[G], bs[G]; // the epilogue's operands, asked for before the products
 #pragma unroll
     for (int g = 0; g < G; g++) {
         sc[g] = *reinterpret_cast<const float4 *>(a.scale + tile[g] * 16 + kg * 4);
         bs[g] = float4{0.f, 0.f, 0.f, 0.f};
         if (a.bias) bs[g] = *reinterpret_cast<const float4 *>(a.bias + tile[g] * 16 + kg * 4);
     }
-    for (int kb = 0; kb < a.ksteps; kb += kRowsBatch) {
+    uint2 res_pre = uint2{0u, 0u};
+    if (SPLIT && a.residual) // (the token tile this wave finishes)
+        res_pre = *reinterpret_cast<const uint2 *>(a.residual + (size_t)min(min(wave, MT - 1) * 16 + i16, a.m - 1) * a.n_out + out_tile * 16 + kg * 4);
+    for (int kb = ks0; kb < ks1; kb += kRowsBatch) {
         lu32x4 wv[kRowsBatch][G];
 #pragma unroll
         for (int u = 0; u < kRowsBatch; u++) {
-            const int ks = min(kb + u, a.ksteps - 1); // steps past the end re-read the last one and are not multiplied
+            const int ks = min(kb + u, ks1 - 1); // steps past the end re-read the last one and are not multiplied
 #pragma unroll
             for (int g = 0; g < G; g++) wv[u][g] = a.w[((size_t)tile[g] * a.ksteps + ks) * 64 + lane];
         }
 #pragma unroll
         for (int u = 0; u < kRowsBatch; u++) {
-            if (kb + u < a.ksteps) { // uniform
+            if (kb + u < ks1) { // uniform
                 h16x8 x0[MT], x1[MT];
 #pragma unroll
                 for (int t = 0; t < MT; t++) {
@@ -432,9 +440,20 @@ template <int MT, int G, int WAVES> __global__ __launch_bounds__(WAVES * 64) voi
             }
         }
     }
+    if (SPLIT) {
+#pragma unroll
+        for (int g = 0; g < G; g++)
+#pragma unroll
+            for (int t = 0; t < MT; t++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) red[wave][g][t][lane][r] = acc[g][t][r];
+        __syncthreads();
+        if (wave >= MT) return; // wave w finishes token tile w
+    }
     // lane (i16 = token within the tile, kg): channels tile * 16 + kg * 4 + r
 #pragma unroll
-    for (int t = 0; t < MT; t++) {
+    for (int tt = 0; tt < (SPLIT ? 1 : MT); tt++) {
+        const int t = SPLIT ? wave : tt;
         const int m = t * 16 + i16;
         float v[G][4];
 #pragma unroll
@@ -442,13 +461,20 @@ template <int MT, int G, int WAVES> __global__ __launch_bounds__(WAVES * 64) voi
             const float scv[4] = {sc[g].x, sc[g].y, sc[g].z, sc[g].w}, bsv[4] = {bs[g].x, bs[g].y, bs[g].z, bs[g].w};
 #pragma unroll
             for (int r = 0; r < 4; r++) {
-                float s = acc[g][t][r] * scv[r];
+                float s = 0.f;
+                if (SPLIT) {
+#pragma unroll
+                    for (int w = 0; w < WAVES; w++) s += red[w][g][t][lane][r]; // fixed order: deterministic
+                } else {
+                    s = acc[g][tt][r];
+                }
+                s *= scv[r];
                 if (a.bias) s += bsv[r];
                 v[g][r] = s;
             }
         }
         if (m >= a.m) continue;
-        store_gemm_row<G>(a, v, (size_t)m * a.n_out + out_tile * 16 + kg * 4);
+        store_gemm_row<G>(a, v, (size_t)m * a.n_out + out_tile * 16 + kg * 4, res_pre, SPLIT);
     }
 }
 
@@ -655,6 +681,14 @@ static int launch_w8a16_gemm(nncase_hip_ctx_t *ctx, const void *a_dev, const nnc
     // 13.9 us in 76 blocks of four and 18 us split)
     const int mt_built = mt <= 1 ? 1 : (mt == 2 ? 2 : 4);
     const size_t rows_lds = (size_t)mt_built * 16 * rows_in_lds_pitch(w->k);
+    if (split && !glu && ln_weight_dev && w->k <= kRowsMaxK && rows_lds <= 64 * 1024 && mt_built <= 2) {
+        // few tiles and rows to normalise (the q / k / v projection): the reduction split over the block's waves, the
+        // rows parked and normalised in LDS in one trip to memory
+        if (mt_built == 1) hipLaunchKernelGGL((w8a16_gemm_rows_in_lds_kernel<1, 1, kGemmWaves, true>), grid, block, rows_lds, ctx->stream, a);
+        else hipLaunchKernelGGL((w8a16_gemm_rows_in_lds_kernel<2, 1, kGemmWaves, true>), grid, block, rows_lds, ctx->stream, a);
+        NNHIP_LAUNCH_CHECK(ctx, "w8a16_gemm_rows_in_lds_kernel");
+        return 0;
+    }
     if (w->k <= kRowsMaxK && rows_lds <= 128 * 1024 && out_tiles >= ctx->compute_units) {
         const dim3 rgrid((out_tiles + kGemmWaves - 1) / kGemmWaves), rblock(kGemmThreads);
 #define NNHIP_ROWS_LAUNCH(MTV, GV)                                                                                             \
