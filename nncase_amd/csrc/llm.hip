@@ -197,9 +197,11 @@ template <int MT, int G, bool SPLIT, int B = kGemmBatch> __global__ __launch_bou
 
     // The epilogue's operands (SPLIT: of the token tile this wave finishes) are asked for before the products: the
     // launch is a chain of memory round trips, and this takes the last one out of it.
+    // (not with four token tiles: their slices leave no registers for it)
+    constexpr bool kPre = SPLIT && MT <= 2;
     float4 sc[G], bs[G];
     uint2 res_pre = uint2{0u, 0u};
-    if (SPLIT) {
+    if (kPre) {
 #pragma unroll
         for (int g = 0; g < G; g++) {
             sc[g] = *reinterpret_cast<const float4 *>(a.scale + tile[g] * 16 + kg * 4);
@@ -231,7 +233,7 @@ template <int MT, int G, bool SPLIT, int B = kGemmBatch> __global__ __launch_bou
         if (a.ln_w) {
 #pragma unroll
             for (int u = 0; u < B; u++)
-                if (kb + u < ks1) // (uniform for the wave: the slices past its share are not multiplied)
+                if (MT > 2 || kb + u < ks1) // (uniform for the wave: the slices past its share are not multiplied; four token tiles have no registers to spare for the branch)
 #pragma unroll
                 for (int t = 0; t < MT; t++)
 #pragma unroll
@@ -293,10 +295,13 @@ template <int MT, int G, bool SPLIT, int B = kGemmBatch> __global__ __launch_bou
                 if (SPLIT) {
 #pragma unroll
                     for (int w = 0; w < kGemmWaves; w++) s += red[w][g][t][lane][r]; // fixed order: deterministic
+                } else {
+                    s = acc[g][tt][r];
+                }
+                if (kPre) {
                     s *= scv[r];
                     if (a.bias) s += bsv[r];
                 } else {
-                    s = acc[g][tt][r];
                     const int ch = tile[g] * 16 + kg * 4 + r;
                     s *= a.scale[ch];
                     if (a.bias) s += a.bias[ch];
@@ -305,7 +310,7 @@ template <int MT, int G, bool SPLIT, int B = kGemmBatch> __global__ __launch_bou
             }
         }
         if (m >= a.m) continue;
-        store_gemm_row<G>(a, v, (size_t)m * a.n_out + out_tile * 16 + kg * 4, res_pre, SPLIT);
+        store_gemm_row<G>(a, v, (size_t)m * a.n_out + out_tile * 16 + kg * 4, res_pre, kPre);
     }
 }
 
@@ -721,7 +726,7 @@ static int launch_w8a16_gemm(nncase_hip_ctx_t *ctx, const void *a_dev, const nnc
     do {                                                                                                                       \
         if (glu && split) hipLaunchKernelGGL((w8a16_gemm_kernel<MTV, 2, true>), grid, block, 0, ctx->stream, a);              \
         else if (glu) hipLaunchKernelGGL((w8a16_gemm_kernel<MTV, 2, false>), grid, block, 0, ctx->stream, a);                 \
-        else if (split && long_share) hipLaunchKernelGGL((w8a16_gemm_kernel<MTV, 1, true, 5>), grid, block, 0, ctx->stream, a); \
+        else if (split && long_share) hipLaunchKernelGGL((w8a16_gemm_kernel<(MTV <= 2 ? MTV : 2), 1, true, 5>), grid, block, 0, ctx->stream, a); \
         else if (split) hipLaunchKernelGGL((w8a16_gemm_kernel<MTV, 1, true>), grid, block, 0, ctx->stream, a);                \
         else hipLaunchKernelGGL((w8a16_gemm_kernel<MTV, 1, false>), grid, block, 0, ctx->stream, a);                          \
     } while (0)
