@@ -463,7 +463,8 @@ NNCASE_HIP_API int nncase_hip_paged_attention_decode_noalloc(nncase_hip_ctx_t *c
  *   NNCASE_HIP_GEMM_PLAIN   out is [m, n]
  *   NNCASE_HIP_GEMM_SWIGLU  the matrix holds the gate projection in rows [0, n/2) and the up
  *                           projection in rows [n/2, n): out[m, j] = silu(gate_j) * up_j, [m, n/2]
- * residual_dev (fp16, shape of out, may be NULL) is added to the result; out is fp16 or fp32. */
+ * residual_dev (fp16, shape of out, 8-byte aligned, may be NULL) is added to the result; out is fp16 or fp32
+ * (a_dev and out_dev 16-byte aligned; -invalid_memory_location otherwise). */
 #define NNCASE_HIP_GEMM_PLAIN 0
 #define NNCASE_HIP_GEMM_SWIGLU 1
 typedef struct nncase_hip_w8a16 nncase_hip_w8a16_t;
