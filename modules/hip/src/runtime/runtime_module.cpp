@@ -15,10 +15,20 @@ using namespace nncase;
 using namespace nncase::runtime;
 using namespace nncase::runtime::hip;
 
+/* Status values of libnncase_hip.so (nncase_hip.h, error block):
+ *   [-NNCASE_ERRC_LAST, -1]   an nncase_errc value with the sign flipped (the errno values the library uses are
+ *                             all above NNCASE_ERRC_LAST, so the block is unambiguous)
+ *   <= -HIP_STATUS_BASE       -(HIP_STATUS_BASE + hipError_t): a failed HIP runtime call, reported as an I/O error
+ *   everything else           -errno */
+static constexpr int NNCASE_ERRC_LAST = 0x07;
+static constexpr int HIP_STATUS_BASE = 0x1000;
+
 std::error_code nncase::runtime::hip::to_error_code(int rc) noexcept {
-    if (rc > -0x100) // -errno
-        return std::make_error_code(static_cast<std::errc>(-rc));
-    return make_error_code(static_cast<nncase_errc>(-rc)); // -nncase_errc, the values of src/Native/include/nncase/runtime/error.h
+    if (rc >= -NNCASE_ERRC_LAST)
+        return make_error_code(static_cast<nncase_errc>(-rc)); // src/Native/include/nncase/runtime/error.h:21-37
+    if (rc <= -HIP_STATUS_BASE)
+        return std::make_error_code(std::errc::io_error);
+    return std::make_error_code(static_cast<std::errc>(-rc));
 }
 
 hip_runtime_module::~hip_runtime_module() {

@@ -6,8 +6,9 @@
 
 BEGIN_NS_NNCASE_RT_MODULE(hip)
 
-/* A negative errno or nncase_errc value from libnncase_hip.so -> the error_code the runtime reports
- * (codes below -0x100 are nncase_errc values with the sign flipped, nncase_hip.h). */
+/* A status of libnncase_hip.so -> the error_code the runtime reports: [-7, -1] is an nncase_errc value with the
+ * sign flipped, -(0x1000 + hipError_t) and below a failed HIP runtime call (std::errc::io_error), anything else
+ * a negative errno (nncase_hip.h, error block). */
 std::error_code to_error_code(int rc) noexcept;
 
 #define hip_try(x)                                                                                                     \

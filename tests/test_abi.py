@@ -158,3 +158,99 @@ def test_errno_statuses_stay_clear_of_the_nncase_errc_block():
         used |= set(re.findall(r"-(E[A-Z0-9]+)\b", open(os.path.join(src, f)).read()))
     used -= {"ERR"}
     assert used and all(getattr(errno, name) > 7 for name in used), sorted(used)
+
+
+# ---- the runtime-module shim (C++ against the reference's headers, not compilable here) is checked as text ----
+SHIM_DIR = os.path.join(ROOT, "modules", "hip", "src", "runtime")
+REF_ERRC_BLOCK = {  # src/Native/include/nncase/runtime/error.h:21-37, the values a hip module can report
+    "INVALID_MODEL_IDENTIFIER": 0x01, "INVALID_MODEL_VERSION": 0x03, "RUNTIME_NOT_FOUND": 0x04,
+    "DATATYPE_MISMATCH": 0x05, "SHAPE_MISMATCH": 0x06, "INVALID_MEMORY_LOCATION": 0x07,
+}
+
+
+def shim_sources():
+    return {f: open(os.path.join(SHIM_DIR, f)).read() for f in sorted(os.listdir(SHIM_DIR))}
+
+
+def shim_status_map():
+    """to_error_code of the shim, rebuilt from its text: the two thresholds and the order of the tests."""
+    text = shim_sources()["runtime_module.cpp"]
+    last = int(re.search(r"NNCASE_ERRC_LAST\s*=\s*(0x[0-9a-fA-F]+|\d+)\s*;", text).group(1), 0)
+    base = int(re.search(r"HIP_STATUS_BASE\s*=\s*(0x[0-9a-fA-F]+|\d+)\s*;", text).group(1), 0)
+    body = text[text.index("to_error_code(int rc) noexcept {"):]
+    body = body[:body.index("\n}\n")]
+    tests_in_order = re.findall(r"if \(rc (>=|<=) -(\w+)\)\s*return ([^;]+);", body)
+    assert [(op, name) for op, name, _ in tests_in_order] == [(">=", "NNCASE_ERRC_LAST"), ("<=", "HIP_STATUS_BASE")], tests_in_order
+    assert "nncase_errc" in tests_in_order[0][2] and "io_error" in tests_in_order[1][2]
+    assert re.search(r"return std::make_error_code\(static_cast<std::errc>\(-rc\)\);\s*$", body), "the rest is -errno"
+
+    def classify(rc):
+        if rc >= -last:
+            return ("nncase_errc", -rc)
+        if rc <= -base:
+            return ("io_error", None)
+        return ("errno", -rc)
+    return classify, last, base
+
+
+def test_shim_maps_every_library_status_to_the_right_category():
+    header = open(HEADER).read()
+    enum = {n: int(v, 0) for n, v in re.findall(r"NNCASE_HIP_ERR_(\w+) = (0x[0-9a-fA-F]+)", header)}
+    hip_base = enum.pop("HIP_BASE")
+    assert enum == REF_ERRC_BLOCK, "the header's first error block is nncase_errc's"
+    classify, last, base = shim_status_map()
+    assert last == max(enum.values()) and base == hip_base
+    for name, value in enum.items():
+        assert classify(-value) == ("nncase_errc", value), name
+    # every errno the library returns keeps its meaning, whichever side of 0x100 it lies on
+    src = os.path.join(ROOT, "nncase_amd", "csrc")
+    used = set()
+    for f in os.listdir(src):
+        used |= set(re.findall(r"-(E[A-Z0-9]+)\b", open(os.path.join(src, f)).read()))
+    used -= {"ERR"}
+    for name in used:
+        assert classify(-getattr(errno, name)) == ("errno", getattr(errno, name)), name
+    # a failed HIP runtime call: -(0x1000 + hipError_t), hipError_t in [1, 1054] on this runtime
+    for hip_error in (1, 2, 98, 700, 719, 999, 1054):
+        assert classify(-(hip_base + hip_error)) == ("io_error", None)
+    # the library itself keeps the block clear (what makes the first test of the shim sound)
+    lib = rt.load_library()
+    assert lib.nncase_hip_ctx_create(0, None) == -errno.EINVAL and classify(-errno.EINVAL)[0] == "errno"
+
+
+def test_shim_calls_declared_entry_points_with_the_right_arity():
+    header = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    arity = {}
+    for m in re.finditer(r"NNCASE_HIP_API\s+[\w\s\*]+?\b(nncase_hip_\w+)\s*\((.*?)\)\s*;", header, re.S):
+        args = m.group(2).strip()
+        arity[m.group(1)] = 0 if args in ("", "void") else args.count(",") + 1
+
+    def call_args(text, start):
+        """Top-level argument count of the call whose '(' is at `start`."""
+        depth, count, i, seen = 0, 0, start, False
+        while True:
+            ch = text[i]
+            if ch in "([{":
+                depth += 1
+            elif ch in ")]}":
+                depth -= 1
+                if depth == 0:
+                    return count + 1 if seen else 0
+            elif ch == "," and depth == 1:
+                count += 1
+            elif depth >= 1 and not ch.isspace():
+                seen = True
+            i += 1
+
+    calls = 0
+    for fname, text in shim_sources().items():
+        code = re.sub(r"/\*.*?\*/", lambda m: " " * len(m.group(0)), text, flags=re.S)
+        code = re.sub(r"//[^\n]*", lambda m: " " * len(m.group(0)), code)
+        for m in re.finditer(r"\b(nncase_hip_\w+)\s*\(", code):
+            name = m.group(1)
+            if name.endswith("_t"):
+                continue
+            assert name in arity, f"{fname}: {name} is not declared in nncase_hip.h"
+            assert call_args(code, m.end() - 1) == arity[name], f"{fname}: {name}"
+            calls += 1
+    assert calls >= 8
