@@ -33,6 +33,7 @@
 //   kBytes   anything else (e.g. 3 input channels): byte gathers
 #pragma once
 
+#include <mutex>
 #include <type_traits>
 
 #include "qconv.hpp"
@@ -1115,11 +1116,13 @@ template <int T, int RG, int MODE> int launch_trg(nncase_hip_ctx *ctx, const Ige
             hipLaunchKernelGGL((qconv_igemm_kernel<T, RG, MODE, true>), dim3(gx, nchunks, 1), dim3(kThreads), lds, ctx->stream, args);
     } else if (stage_lds) {
         if constexpr (staged_store_built(T) && (loads_rows(MODE) || MODE == kVec16)) {
-            static bool raised = false; // more than 64 KiB of dynamic LDS (full-depth weights and the staging areas) has to be asked for once
-            if (lds > 65536 && !raised) {
-                NNHIP_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(&qconv_igemm_kernel<T, RG, MODE, false, true>),
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, 98304));
-                raised = true;
+            if (lds > 65536) { // more than 64 KiB of dynamic LDS (full-depth weights and the staging areas) has to be asked for once per kernel and device
+                static std::once_flag raised[16];
+                hipError_t attr = hipSuccess;
+                std::call_once(raised[ctx->device & 15], [&] {
+                    attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&qconv_igemm_kernel<T, RG, MODE, false, true>), hipFuncAttributeMaxDynamicSharedMemorySize, 98304);
+                });
+                NNHIP_HIP(ctx, attr);
             }
             hipLaunchKernelGGL((qconv_igemm_kernel<T, RG, MODE, false, true>), dim3(gx, nchunks, 1), dim3(kThreads), lds, ctx->stream, args);
         }

@@ -29,6 +29,7 @@
 
 #include "qconv_igemm.hpp"
 
+#include <mutex>
 #include <type_traits>
 
 namespace nnhip {
@@ -59,8 +60,10 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t wide_rsrc(const void *base, ui
 // WN * T * 16 channels (the block's channel chunk, packed with tiles = WN * T).
 //
 // LDS: kWideSlots slots, each [activations: pixels x 64 bytes | weights: WN * T fragments].  The four 16-byte
-// pieces of pixel p are rotated by (p >> 2) & 3, so that neither the row-order writes nor the operand-order reads
-// of 16 neighbouring lanes meet on a bank.
+// pieces of pixel p are rotated by (p >> 1) & 3: the LDS serves a 16-byte read of eight neighbouring lanes per 128 bytes of
+// banks, so pixels p and p + 2 (128 bytes apart) must not present the same piece (measured: 241 bytes per clock and
+// compute unit with this rotation, 128 with a rotation by (p >> 2) or none); the row-order writes cover whole
+// 128-byte runs whatever the rotation.
 template <int T, int RG, int WM, int WN, int LM>
 __global__ __launch_bounds__(WM * WN * 64, 2) void qconv_wide_kernel(const IgemmArgs a, int nchunks) {
     constexpr int THREADS = WM * WN * 64;
@@ -196,8 +199,8 @@ __global__ __launch_bounds__(WM * WN * 64, 2) void qconv_wide_kernel(const Igemm
             f.fill = in_k ? a.zx_splat : 0x80808080u;
         }
     };
-    // (THREADS / 4 is a multiple of 16, so the rotation of a thread's pieces is the same for all its pixels)
-    uint8_t *const a_dst = ring + lp * 64 + ((lq + (lp >> 2)) & 3) * 16;
+    // (THREADS / 4 is a multiple of 8, so the rotation of a thread's pieces is the same for all its pixels)
+    uint8_t *const a_dst = ring + lp * 64 + ((lq + (lp >> 1)) & 3) * 16;
     int32_t rsum[NA]; // sum of x' over this thread's pieces of its i-th pixel
 #pragma unroll
     for (int i = 0; i < NA; i++) rsum[i] = 0;
@@ -242,7 +245,7 @@ __global__ __launch_bounds__(WM * WN * 64, 2) void qconv_wide_kernel(const Igemm
         store_acts(a0, 0, 0);
         __syncthreads(); // ring slot 0 is written
     }
-    const uint8_t *const x_src = ring + (wm * RG * 16 + j) * 64 + ((gq + (j >> 2)) & 3) * 16; // + rg * 16 * 64
+    const uint8_t *const x_src = ring + (wm * RG * 16 + j) * 64 + ((gq + (j >> 1)) & 3) * 16; // + rg * 16 * 64
     const uint8_t *const w_src = ring + AV * 16 + (wn * T) * 1024 + lane * 16;                 // + nt * 1024
     // One k-step s (parity P) multiplies the ring slot at byte offset `cur`: operand reads of the next pair of channel
     // tiles are issued before the matrix instructions of the current pair (the order is pinned by scheduling
@@ -323,17 +326,308 @@ __global__ __launch_bounds__(WM * WN * 64, 2) void qconv_wide_kernel(const Igemm
     });
 }
 
+
+// ---- the 256-pixel x 256-channel block ------------------------------------------------------------------------
+// What a compute unit can take from its L2 bounds the matrix rate of a long reduction: a k-step of a P x C block moves
+// (P + C) * 64 bytes for P * C / 64 cycles of the four matrix units, and the vector memory path delivers 55-62 bytes
+// per cycle when a wave's load covers whole 128-byte lines (1 KiB runs of packed weights; 128 bytes per pixel) but
+// 35-40 when it takes 64 bytes out of each line (measured on an L2-resident set).  The accumulators of 256 x 256
+// outputs are half of the unit's registers, so that block is the largest there is: eight waves of 64 x 128, one block
+// per unit, 32 bytes per cycle at the full matrix rate.  It therefore
+//   * fetches activations for two k-steps at a time: eight threads read the 128 contiguous bytes of a pixel
+//     (window modes: two 64-byte halves, each at its own tap), requested two k-steps before they are staged;
+//   * keeps a ring of four k-step slots, so that a slot is free for two k-steps before its first read: the weights'
+//     DMA is requested at the top of k-step s - 3 and waited for at the end of k-step s - 2;
+// The rest (operand reads ahead of the products, rotation of a pixel's pieces, sums of x', epilogue) is the kernel above.
+template <int T, int RG, int WM, int WN, int LM>
+__global__ __launch_bounds__(WM * WN * 64, 2) void qconv_wide4_kernel(const IgemmArgs a, int nchunks) {
+    constexpr int NS = 4;
+    constexpr int THREADS = WM * WN * 64;
+    constexpr int PIX = WM * RG * 16;
+    constexpr int TB = T * WN;
+    constexpr int AV = PIX * 4, WV = TB * 64;           // 16-byte vectors of activations / weights per k-step
+    constexpr int NA2 = 2 * AV / THREADS;               // activation vectors per thread per pair of k-steps
+    constexpr int NW = WV / THREADS;                    // weight runs per wave per k-step
+    constexpr int PSTEP = THREADS / 8;                  // pixels between a thread's vectors
+    static_assert((2 * AV) % THREADS == 0 && WV % THREADS == 0 && PSTEP % 8 == 0, "every thread moves the same number of vectors");
+    static_assert(T % 4 == 0, "at least two pairs of channel tiles per k-step");
+    constexpr int G = T / 2;
+    constexpr int SLOT = AV * 16 + WV * 16;
+    constexpr bool kRows = LM == kWideRowsFull || LM == kWideRows;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    int32_t *cterm = reinterpret_cast<int32_t *>(smem);              // [TB * 16]
+    uint8_t *lutl = smem + TB * 16 * sizeof(int32_t);                // [256]
+    int32_t *rowsums = reinterpret_cast<int32_t *>(lutl + 256);      // [PIX]
+    uint8_t *ring = lutl + 256 + PIX * sizeof(int32_t);              // [NS][SLOT]
+
+    const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3;
+    const int chunk = seq % nchunks;
+    const int per = (a.num_mtiles + 7) >> 3;
+    const int mt = xcd * per + seq / nchunks;
+    if (seq / nchunks >= per || mt >= a.num_mtiles) return;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wm = wave % WM, wn = wave / WM;
+    const int j = lane & 15, gq = lane >> 4;
+    const int ch_base = chunk * (TB * 16);
+    const int KS = a.ksteps;
+    const __amdgpu_buffer_rsrc_t wres = wide_rsrc(a.wpk + (size_t)chunk * KS * TB * 1024, (uint32_t)KS * TB * 1024);
+    const __amdgpu_buffer_rsrc_t xres = wide_rsrc(a.x, (uint32_t)a.x_bytes);
+
+    constexpr int NC = (TB * 16 + THREADS - 1) / THREADS;
+    int32_t c_bias[NC], c_wsum[NC];
+#pragma unroll
+    for (int i = 0; i < NC; i++) {
+        const int c = i * THREADS + threadIdx.x;
+        const bool real = c < TB * 16 && ch_base + c < a.n;
+        c_bias[i] = real ? a.bias[ch_base + c] : 0;
+        c_wsum[i] = real ? a.wsum[ch_base + c] : 0;
+    }
+    uint32_t lut_word = 0;
+    const bool lut_mine = a.lut && threadIdx.x < 64;
+    if (lut_mine) lut_word = a.lut[threadIdx.x];
+
+    // ---- weights: DMA, wave w moves the 1 KiB runs w + i * WAVES of a k-step ----
+    const uint32_t w_voff = threadIdx.x * 16;
+    auto dma_w = [&](int slot, int ks) __attribute__((always_inline)) {
+        const int ksc = min(ks, KS - 1); // a k-step past the end re-reads the last one (its data is never multiplied)
+#pragma unroll
+        for (int i = 0; i < NW; i++) {
+            __attribute__((address_space(3))) uint8_t *dst =
+                (__attribute__((address_space(3))) uint8_t *)(ring + AV * 16 + slot + (i * THREADS + wave * 64) * 16);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(wres, dst, 16, w_voff, (ksc * WV + i * THREADS) * 16, 0, 0);
+        }
+    };
+
+    // ---- activations: thread t fetches piece lq4 of k-step 2 * pair + half of pixels lp + i * PSTEP ----
+    const int lp = threadIdx.x >> 3, half = (threadIdx.x >> 2) & 1, lq4 = threadIdx.x & 3;
+    int32_t p_off[NA2], p_iy0[NA2], p_ix0[NA2];
+#pragma unroll
+    for (int i = 0; i < NA2; i++) {
+        const PixInfo pi = pix_info<kRows ? kRows16 : kVec16>(a, mt * PIX + lp + i * PSTEP);
+        const bool ok = pi.base >= 0; // a pixel past the end takes pixel 0's place: any valid address, the result is not stored
+        if (kRows) {
+            p_off[i] = (ok ? pi.base : 0) * a.ldx + a.x_coff + lq4 * 16;
+            p_iy0[i] = p_ix0[i] = 0;
+        } else {
+            p_iy0[i] = ok ? pi.iy0 : 0;
+            p_ix0[i] = ok ? pi.ix0 : 0;
+            p_off[i] = ((ok ? pi.base : 0) + p_iy0[i] * a.in_w + p_ix0[i]) * a.ldx + a.x_coff + (LM == kWideTap ? lq4 * 16 : 0);
+        }
+    }
+    struct Acts {
+        wide_u32x4 raw[NA2];
+        uint32_t fill;
+        bool take[NA2];
+    };
+    auto load_acts = [&](Acts &f, int pair) {
+        const int ksc = min(2 * pair + half, KS - 1);
+        if (LM == kWideRowsFull) {
+#pragma unroll
+            for (int i = 0; i < NA2; i++) {
+                f.raw[i] = __builtin_amdgcn_raw_buffer_load_b128(xres, p_off[i] + ksc * 64, 0, 0);
+                f.take[i] = true;
+            }
+            f.fill = 0;
+        } else if (LM == kWideRows) {
+            const bool in_k = ksc * 64 + lq4 * 16 < a.k;
+#pragma unroll
+            for (int i = 0; i < NA2; i++) {
+                f.raw[i] = __builtin_amdgcn_raw_buffer_load_b128(xres, p_off[i] + ksc * 64, 0, 0);
+                f.take[i] = in_k;
+            }
+            f.fill = 0x80808080u;
+        } else {
+            const int kk = ksc * 64 + (LM == kWideTap ? 0 : lq4 * 16);
+            const bool in_k = LM == kWideTap || kk < a.k;
+            const uint32_t tap = fastdiv((uint32_t)(in_k ? kk : 0), a.d_gic);
+            const int c = (in_k ? kk : 0) - (int)tap * a.g_ic;
+            const uint32_t ky = fastdiv(tap, a.d_kw);
+            const int dy = (int)ky * a.dil_h, dx = ((int)tap - (int)ky * a.kw) * a.dil_w;
+            const int shift = (dy * a.in_w + dx) * a.ldx + c;
+#pragma unroll
+            for (int i = 0; i < NA2; i++) {
+                // no clamping: an address outside the tensor reads 0, one inside but outside the image is replaced below
+                f.raw[i] = __builtin_amdgcn_raw_buffer_load_b128(xres, p_off[i] + shift, 0, 0);
+                f.take[i] = in_k && (unsigned)(p_iy0[i] + dy) < (unsigned)a.in_h && (unsigned)(p_ix0[i] + dx) < (unsigned)a.in_w;
+            }
+            f.fill = in_k ? a.zx_splat : 0x80808080u;
+        }
+    };
+    uint8_t *const a_dst = ring + lp * 64 + ((lq4 + (lp >> 1)) & 3) * 16;
+    int32_t rsum[NA2];
+#pragma unroll
+    for (int i = 0; i < NA2; i++) rsum[i] = 0;
+    // slot_even / slot_odd: ring slots of the pair's two k-steps (byte offsets)
+    auto store_acts = [&](const Acts &f, int slot_even, int slot_odd, int pair) {
+        if (2 * pair + half >= KS) return; // (the second half of the last pair of an odd number of k-steps)
+        uint8_t *const dst = a_dst + (half ? slot_odd : slot_even);
+#pragma unroll
+        for (int i = 0; i < NA2; i++) {
+            wide_u32x4 r;
+#pragma unroll
+            for (int d = 0; d < 4; d++) {
+                r[d] = (LM == kWideRowsFull ? f.raw[i][d] : (f.take[i] ? f.raw[i][d] : f.fill)) ^ 0x80808080u;
+                rsum[i] = __builtin_amdgcn_sdot4((int)r[d], 0x01010101, rsum[i], false);
+            }
+            *reinterpret_cast<wide_u32x4 *>(dst + i * PSTEP * 64) = r;
+        }
+    };
+
+    v4i acc[RG][T];
+#pragma unroll
+    for (int rg = 0; rg < RG; rg++)
+#pragma unroll
+        for (int nt = 0; nt < T; nt++) acc[rg][nt] = v4i{0, 0, 0, 0};
+
+    // s_waitcnt immediates (gfx9 encoding): vmcnt in bits [3:0] and [15:14], expcnt [6:4], lgkmcnt [11:8]
+    constexpr auto waitcnt_imm = [](int vm, int lgkm) { return (vm & 15) | ((vm >> 4) << 14) | (7 << 4) | ((lgkm & 15) << 8); };
+    // ---- fill: slots 0 and 1 complete, slot 2's weights and the activations of pair 1 on their way ----
+    // (one register set for the activations in flight: with a second one, requested four k-steps ahead, the kernel
+    // no longer fits 256 registers)
+    Acts af;
+    {
+        dma_w(0, 0);
+        dma_w(SLOT, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        load_acts(af, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        dma_w(2 * SLOT, 2);
+        __builtin_amdgcn_sched_barrier(0);
+        store_acts(af, 0, SLOT, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        load_acts(af, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(NA2, 0)); // the first three k-steps' weights and the first pair's activations are in
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    const uint8_t *const x_src = ring + (wm * RG * 16 + j) * 64 + ((gq + (j >> 1)) & 3) * 16; // + rg * 16 * 64
+    const uint8_t *const w_src = ring + AV * 16 + (wn * T) * 1024 + lane * 16;                 // + nt * 1024
+    v4i xf[2][RG], wf[2][2];
+#pragma unroll
+    for (int rg = 0; rg < RG; rg++) xf[0][rg] = *reinterpret_cast<const v4i *>(x_src + rg * 16 * 64);
+    wf[0][0] = *reinterpret_cast<const v4i *>(w_src);
+    wf[0][1] = *reinterpret_cast<const v4i *>(w_src + 1024);
+    // The slot offsets are scalars (a ring of 128 KiB is beyond the 64 KiB an LDS instruction's immediate offset
+    // reaches, and as compile-time constants every slot's addresses would be held in registers of their own): a few
+    // vector additions per k-step turn the per-thread constants into this k-step's addresses.
+    int cur = 0;
+    auto kstep = [&](int s, auto parity) __attribute__((always_inline)) {
+        constexpr int P = decltype(parity)::value;
+        asm volatile("" : "+s"(cur));
+        const int nxt = (cur + SLOT) & (NS * SLOT - 1), nxt2 = (cur + 2 * SLOT) & (NS * SLOT - 1), nxt3 = (cur + 3 * SLOT) & (NS * SLOT - 1);
+        static_assert((SLOT & (SLOT - 1)) == 0, "the ring wraps by a mask");
+        const uint8_t *const ws = w_src + cur;
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            const int wb = g & 1; // (G is even)
+            __builtin_amdgcn_sched_barrier(0);
+            if (g + 1 < G) {
+                wf[1 - wb][0] = *reinterpret_cast<const v4i *>(ws + (2 * g + 2) * 1024);
+                wf[1 - wb][1] = *reinterpret_cast<const v4i *>(ws + (2 * g + 3) * 1024);
+            }
+            if (g == G - 2) {
+                const uint8_t *const xn = x_src + nxt;
+#pragma unroll
+                for (int rg = 0; rg < RG; rg++) xf[1 - P][rg] = *reinterpret_cast<const v4i *>(xn + rg * 16 * 64);
+            }
+            if (g + 1 == G) {
+                const uint8_t *const wn_ = w_src + nxt;
+                wf[1 - wb][0] = *reinterpret_cast<const v4i *>(wn_);
+                wf[1 - wb][1] = *reinterpret_cast<const v4i *>(wn_ + 1024);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int e = 0; e < 2; e++)
+#pragma unroll
+                for (int rg = 0; rg < RG; rg++)
+                    acc[rg][2 * g + e] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[wb][e], xf[P][rg], acc[rg][2 * g + e], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            // (in this order in the instruction stream: the wait below counts the requests behind a k-step's DMA)
+            if (g == 0) dma_w(nxt3, s + 3);
+            if (g == 1 && P == 0) {
+                store_acts(af, nxt2, nxt3, (s >> 1) + 1);
+                __builtin_amdgcn_sched_barrier(0);
+                load_acts(af, (s >> 1) + 2);
+            }
+        }
+        cur = nxt;
+        __builtin_amdgcn_sched_barrier(0);
+        // the DMA of k-step s + 2, requested during k-step s - 1, has landed: behind it came NW runs of this k-step's
+        // DMA and, in one of the two k-steps, NA2 register loads; this wave's LDS writes are done (LDS operations
+        // complete in order: only the two reads of the next weights may still be out)
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(NW + NA2, 2));
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    int s = 0;
+#pragma clang loop unroll(disable)
+    for (; s + 1 < KS; s += 2) {
+        kstep(s, std::integral_constant<int, 0>());
+        kstep(s + 1, std::integral_constant<int, 1>());
+    }
+    if (s < KS) kstep(s, std::integral_constant<int, 0>()); // an odd number of k-steps
+
+    // ---- epilogue ----
+#pragma unroll
+    for (int i = 0; i < NC; i++) {
+        const int c = i * THREADS + threadIdx.x;
+        if (c < TB * 16) cterm[c] = ch_base + c < a.n ? c_bias[i] - a.zxp * c_wsum[i] + a.k * a.zxp * a.zwp : 0;
+    }
+    if (lut_mine) reinterpret_cast<uint32_t *>(lutl)[threadIdx.x] = lut_word;
+    // a pixel's sum of x' is spread over the eight threads that loaded its pieces
+#pragma unroll
+    for (int i = 0; i < NA2; i++) {
+        int32_t r = rsum[i];
+        r += __shfl_xor(r, 1);
+        r += __shfl_xor(r, 2);
+        r += __shfl_xor(r, 4);
+        if ((threadIdx.x & 7) == 0) rowsums[lp + i * PSTEP] = r;
+    }
+    __syncthreads(); // (also: every wave's reads of the ring are done before the staging areas below are written, every DMA has landed)
+    static_assert(!staged_store_built(T) || WM * WN * staged_store_bytes() <= NS * SLOT, "the staging areas fit the ring");
+    uint8_t *const stage = staged_store_built(T) ? ring + wave * staged_store_bytes() : nullptr;
+    const int ch0 = ch_base + gq * (4 * TB) + wn * (4 * T);
+    const int32_t *ct = cterm + gq * (4 * TB) + wn * (4 * T) - gq * (4 * T); // igemm_store_tile adds gq * 4 T
+    static_for<0, RG>([&](auto rg_c) __attribute__((always_inline)) {
+        constexpr int rg = decltype(rg_c)::value;
+        const int pl = (wm * RG + rg) * 16 + j;
+        igemm_store_tile<T, kOwesAll, false, staged_store_built(T)>(a, acc[rg], rowsums[pl], mt * PIX + pl, ch0, gq, ct, lutl, stage, 4 * TB);
+    });
+}
+
+template <int T, int RG, int WM, int WN, int LM> int launch_wide4_t(nncase_hip_ctx *ctx, const IgemmArgs &a, int nchunks) {
+    IgemmArgs args = a;
+    constexpr int PIX = WM * RG * 16, TB = T * WN;
+    args.num_mtiles = ceil_div(a.m, PIX);
+    const int blocks = ceil_div(args.num_mtiles, 8) * 8 * nchunks;
+    const size_t lds = (size_t)TB * 16 * sizeof(int32_t) + 256 + PIX * sizeof(int32_t) + (size_t)4 * (PIX * 64 + TB * 1024);
+    static std::once_flag raised[16]; // more than 64 KiB of dynamic LDS has to be asked for once per kernel and device
+    hipError_t attr = hipSuccess;
+    std::call_once(raised[ctx->device & 15], [&] {
+        attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&qconv_wide4_kernel<T, RG, WM, WN, LM>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    });
+    NNHIP_HIP(ctx, attr);
+    hipLaunchKernelGGL((qconv_wide4_kernel<T, RG, WM, WN, LM>), dim3(blocks), dim3(WM * WN * 64), lds, ctx->stream, args, nchunks);
+    NNHIP_LAUNCH_CHECK(ctx, "qconv_wide4_kernel");
+    return 0;
+}
+
 template <int T, int RG, int WM, int WN, int LM> int launch_wide_t(nncase_hip_ctx *ctx, const IgemmArgs &a, int nchunks) {
     IgemmArgs args = a;
     constexpr int PIX = WM * RG * 16, TB = T * WN;
     args.num_mtiles = ceil_div(a.m, PIX);
     const int blocks = ceil_div(args.num_mtiles, 8) * 8 * nchunks;
     const size_t lds = (size_t)TB * 16 * sizeof(int32_t) + 256 + PIX * sizeof(int32_t) + (size_t)kWideSlots * (PIX * 64 + TB * 1024);
-    static bool raised = false; // more than 64 KiB of dynamic LDS has to be asked for once per kernel
-    if (lds > 65536 && !raised) {
-        NNHIP_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(&qconv_wide_kernel<T, RG, WM, WN, LM>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        raised = true;
+    if (lds > 65536) { // more than 64 KiB of dynamic LDS has to be asked for once per kernel and device
+        static std::once_flag raised[16];
+        hipError_t attr = hipSuccess;
+        std::call_once(raised[ctx->device & 15], [&] {
+            attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&qconv_wide_kernel<T, RG, WM, WN, LM>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        });
+        NNHIP_HIP(ctx, attr);
     }
     hipLaunchKernelGGL((qconv_wide_kernel<T, RG, WM, WN, LM>), dim3(blocks), dim3(WM * WN * 64), lds, ctx->stream, args, nchunks);
     NNHIP_LAUNCH_CHECK(ctx, "qconv_wide_kernel");
@@ -348,7 +642,7 @@ inline int wide_waves(const nncase_hip_ctx *ctx, int m, int nchunks) {
 // Block shapes: tiles = 16 -> 256 pixels x 256 channels (4 x 2 waves); tiles = 8 -> 256 or 128 pixels x 128 channels;
 // tiles = 4 -> 256 or 128 pixels x 64 channels.
 template <int LM> int launch_wide_lm(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks) {
-    if (tiles == 16) return launch_wide_t<8, 4, 4, 2, LM>(ctx, a, nchunks);
+    if (tiles == 16) return launch_wide4_t<8, 4, 4, 2, LM>(ctx, a, nchunks);
     const int wmv = wide_waves(ctx, a.m, nchunks);
     if (tiles == 8) return wmv == 4 ? launch_wide_t<8, 4, 4, 1, LM>(ctx, a, nchunks) : launch_wide_t<8, 4, 2, 1, LM>(ctx, a, nchunks);
     if (tiles == 4) return wmv == 4 ? launch_wide_t<4, 4, 4, 1, LM>(ctx, a, nchunks) : launch_wide_t<4, 4, 2, 1, LM>(ctx, a, nchunks);
