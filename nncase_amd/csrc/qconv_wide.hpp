@@ -201,11 +201,12 @@ __global__ __launch_bounds__(WM * WN * 64, 2) void qconv_wide_kernel(const Igemm
     };
     // (THREADS / 4 is a multiple of 8, so the rotation of a thread's pieces is the same for all its pixels)
     uint8_t *const a_dst = ring + lp * 64 + ((lq + (lp >> 1)) & 3) * 16;
-    int32_t rsum[NA]; // sum of x' over this thread's pieces of its i-th pixel
+    uint32_t rsum[NA]; // sum of x (the bytes as staged, before the re-bias) over this thread's pieces of its i-th pixel
 #pragma unroll
     for (int i = 0; i < NA; i++) rsum[i] = 0;
-    // Padding and re-biasing happen on the way into the ring: x' = (piece taken ? x : fill) ^ 0x80; the sums of x' are
-    // taken from the same registers.  A k-step past the end of the reduction is not staged (ks < KS is uniform).
+    // Padding and re-biasing happen on the way into the ring: x' = (piece taken ? x : fill) ^ 0x80; the sums of x are
+    // taken from the same registers (every staged k-step adds 64 bytes per pixel, positions past the reduction as 128:
+    // the sum of x' is the sum of x less 128 * 64 * k-steps).  A k-step past the end of the reduction is not staged (ks < KS is uniform).
     auto store_acts = [&](const Acts &f, int slot, int ks) {
         if (ks >= KS) return;
 #pragma unroll
@@ -213,8 +214,9 @@ __global__ __launch_bounds__(WM * WN * 64, 2) void qconv_wide_kernel(const Igemm
             wide_u32x4 r;
 #pragma unroll
             for (int d = 0; d < 4; d++) {
-                r[d] = (LM == kWideRowsFull ? f.raw[i][d] : (f.take[i] ? f.raw[i][d] : f.fill)) ^ 0x80808080u;
-                rsum[i] = __builtin_amdgcn_sdot4((int)r[d], 0x01010101, rsum[i], false);
+                const uint32_t x = LM == kWideRowsFull ? f.raw[i][d] : (f.take[i] ? f.raw[i][d] : f.fill);
+                rsum[i] = __builtin_amdgcn_sad_u8(x, 0u, rsum[i]); // (a dot product against ones costs the matrix unit seven cycles, this next to none)
+                r[d] = x ^ 0x80808080u;
             }
             *reinterpret_cast<wide_u32x4 *>(a_dst + slot + i * (THREADS / 4) * 64) = r;
         }
@@ -307,10 +309,10 @@ __global__ __launch_bounds__(WM * WN * 64, 2) void qconv_wide_kernel(const Igemm
     // the sums of x' sit with the threads that loaded the pieces: add the four pieces of a pixel, pass them through LDS
 #pragma unroll
     for (int i = 0; i < NA; i++) {
-        int32_t r = rsum[i];
+        int32_t r = (int32_t)rsum[i];
         r += __shfl_xor(r, 1);
         r += __shfl_xor(r, 2);
-        if (lq == 0) rowsums[lp + i * (THREADS / 4)] = r;
+        if (lq == 0) rowsums[lp + i * (THREADS / 4)] = r - 128 * 64 * KS;
     }
     __syncthreads();
     // dword outputs are written through a staging area per wave (store_dword_rows): the ring is free now
@@ -325,6 +327,7 @@ __global__ __launch_bounds__(WM * WN * 64, 2) void qconv_wide_kernel(const Igemm
         igemm_store_tile<T, kOwesAll, false, staged_store_built(T)>(a, acc[rg], rowsums[pl], mt * PIX + pl, ch0, gq, ct, lutl, stage, 4 * TB);
     });
 }
+
 
 
 // ---- the 256-pixel x 256-channel block ------------------------------------------------------------------------
@@ -421,58 +424,63 @@ __global__ __launch_bounds__(WM * WN * 64, 2) void qconv_wide4_kernel(const Igem
         uint32_t fill;
         bool take[NA2];
     };
-    auto load_acts = [&](Acts &f, int pair) {
+    // What the loads of a pair of k-steps have in common: where this thread's pieces lie relative to a pixel's origin.
+    struct Geom {
+        int shift;    // byte offset added to the pixel's
+        int dy, dx;   // window modes: the tap
+        bool in_k;
+        bool phantom; // a k-step past the end (the second half of the last pair of an odd number): read as zeros from outside the tensor
+    };
+    auto geometry = [&](int pair) {
         const int ksc = min(2 * pair + half, KS - 1);
-        if (LM == kWideRowsFull) {
-#pragma unroll
-            for (int i = 0; i < NA2; i++) {
-                f.raw[i] = __builtin_amdgcn_raw_buffer_load_b128(xres, p_off[i] + ksc * 64, 0, 0);
-                f.take[i] = true;
-            }
-            f.fill = 0;
-        } else if (LM == kWideRows) {
-            const bool in_k = ksc * 64 + lq4 * 16 < a.k;
-#pragma unroll
-            for (int i = 0; i < NA2; i++) {
-                f.raw[i] = __builtin_amdgcn_raw_buffer_load_b128(xres, p_off[i] + ksc * 64, 0, 0);
-                f.take[i] = in_k;
-            }
-            f.fill = 0x80808080u;
+        Geom g;
+        g.phantom = 2 * pair + half >= KS;
+        g.dy = g.dx = 0;
+        if (kRows) {
+            g.shift = ksc * 64;
+            g.in_k = LM == kWideRowsFull || ksc * 64 + lq4 * 16 < a.k;
         } else {
             const int kk = ksc * 64 + (LM == kWideTap ? 0 : lq4 * 16);
-            const bool in_k = LM == kWideTap || kk < a.k;
-            const uint32_t tap = fastdiv((uint32_t)(in_k ? kk : 0), a.d_gic);
-            const int c = (in_k ? kk : 0) - (int)tap * a.g_ic;
+            g.in_k = LM == kWideTap || kk < a.k;
+            const uint32_t tap = fastdiv((uint32_t)(g.in_k ? kk : 0), a.d_gic);
+            const int c = (g.in_k ? kk : 0) - (int)tap * a.g_ic;
             const uint32_t ky = fastdiv(tap, a.d_kw);
-            const int dy = (int)ky * a.dil_h, dx = ((int)tap - (int)ky * a.kw) * a.dil_w;
-            const int shift = (dy * a.in_w + dx) * a.ldx + c;
-#pragma unroll
-            for (int i = 0; i < NA2; i++) {
-                // no clamping: an address outside the tensor reads 0, one inside but outside the image is replaced below
-                f.raw[i] = __builtin_amdgcn_raw_buffer_load_b128(xres, p_off[i] + shift, 0, 0);
-                f.take[i] = in_k && (unsigned)(p_iy0[i] + dy) < (unsigned)a.in_h && (unsigned)(p_ix0[i] + dx) < (unsigned)a.in_w;
-            }
-            f.fill = in_k ? a.zx_splat : 0x80808080u;
+            g.dy = (int)ky * a.dil_h, g.dx = ((int)tap - (int)ky * a.kw) * a.dil_w;
+            g.shift = (g.dy * a.in_w + g.dx) * a.ldx + c;
         }
+        return g;
+    };
+    // piece i of the pair (no clamping: an address outside the tensor reads 0, one inside but outside the image is replaced when staged)
+    auto load_piece = [&](Acts &f, const Geom &g, auto i_c) __attribute__((always_inline)) {
+        constexpr int i = decltype(i_c)::value;
+        f.raw[i] = __builtin_amdgcn_raw_buffer_load_b128(xres, g.phantom ? (int)0xfffffff0u : p_off[i] + g.shift, 0, 0);
+        f.take[i] = g.phantom || (kRows ? g.in_k : (g.in_k && (unsigned)(p_iy0[i] + g.dy) < (unsigned)a.in_h && (unsigned)(p_ix0[i] + g.dx) < (unsigned)a.in_w));
+        if (i == 0) f.fill = kRows ? 0x80808080u : (g.in_k ? a.zx_splat : 0x80808080u);
+    };
+    auto load_acts = [&](Acts &f, int pair) {
+        const Geom g = geometry(pair);
+        static_for<0, NA2>([&](auto i_c) __attribute__((always_inline)) { load_piece(f, g, i_c); });
     };
     uint8_t *const a_dst = ring + lp * 64 + ((lq4 + (lp >> 1)) & 3) * 16;
-    int32_t rsum[NA2];
+    uint32_t rsum[NA2]; // sum of x (the bytes as staged, before the re-bias) over this thread's pieces of its i-th pixel
 #pragma unroll
     for (int i = 0; i < NA2; i++) rsum[i] = 0;
     // slot_even / slot_odd: ring slots of the pair's two k-steps (byte offsets)
-    auto store_acts = [&](const Acts &f, int slot_even, int slot_odd, int pair) {
-        if (2 * pair + half >= KS) return; // (the second half of the last pair of an odd number of k-steps)
+    auto store_piece = [&](const Acts &f, int slot_even, int slot_odd, int pair, auto i_c) __attribute__((always_inline)) {
+        constexpr int i = decltype(i_c)::value;
+        // (the second half of the last pair of an odd number of k-steps is staged like any other: zeros, into a slot that no product reads)
         uint8_t *const dst = a_dst + (half ? slot_odd : slot_even);
+        wide_u32x4 r;
 #pragma unroll
-        for (int i = 0; i < NA2; i++) {
-            wide_u32x4 r;
-#pragma unroll
-            for (int d = 0; d < 4; d++) {
-                r[d] = (LM == kWideRowsFull ? f.raw[i][d] : (f.take[i] ? f.raw[i][d] : f.fill)) ^ 0x80808080u;
-                rsum[i] = __builtin_amdgcn_sdot4((int)r[d], 0x01010101, rsum[i], false);
-            }
-            *reinterpret_cast<wide_u32x4 *>(dst + i * PSTEP * 64) = r;
+        for (int d = 0; d < 4; d++) {
+            const uint32_t x = LM == kWideRowsFull ? f.raw[i][d] : (f.take[i] ? f.raw[i][d] : f.fill);
+            rsum[i] = __builtin_amdgcn_sad_u8(x, 0u, rsum[i]); // (a dot product against ones costs the matrix unit seven cycles, this next to none)
+            r[d] = x ^ 0x80808080u;
         }
+        *reinterpret_cast<wide_u32x4 *>(dst + i * PSTEP * 64) = r;
+    };
+    auto store_acts = [&](const Acts &f, int slot_even, int slot_odd, int pair) {
+        static_for<0, NA2>([&](auto i_c) __attribute__((always_inline)) { store_piece(f, slot_even, slot_odd, pair, i_c); });
     };
 
     v4i acc[RG][T];
@@ -514,6 +522,8 @@ __global__ __launch_bounds__(WM * WN * 64, 2) void qconv_wide4_kernel(const Igem
     // reaches, and as compile-time constants every slot's addresses would be held in registers of their own): a few
     // vector additions per k-step turn the per-thread constants into this k-step's addresses.
     int cur = 0;
+    Geom geom = geometry(2);
+    wide_u32x4 staged_piece = {0, 0, 0, 0};
     auto kstep = [&](int s, auto parity) __attribute__((always_inline)) {
         constexpr int P = decltype(parity)::value;
         asm volatile("" : "+s"(cur));
@@ -539,19 +549,35 @@ __global__ __launch_bounds__(WM * WN * 64, 2) void qconv_wide4_kernel(const Igem
                 wf[1 - wb][1] = *reinterpret_cast<const v4i *>(wn_ + 1024);
             }
             __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int e = 0; e < 2; e++)
-#pragma unroll
-                for (int rg = 0; rg < RG; rg++)
-                    acc[rg][2 * g + e] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[wb][e], xf[P][rg], acc[rg][2 * g + e], 0, 0, 0);
-            __builtin_amdgcn_sched_barrier(0);
-            // (in this order in the instruction stream: the wait below counts the requests behind a k-step's DMA)
+            // The products of this pair of tiles, and under them this group's share of the data movement: the DMA request
+            // of the weights three k-steps on (first group), and in the even k-steps pieces of the pair of k-steps that
+            // is staged next: re-bias, sums, the LDS write, and the request for the same pieces of the pair after it
+            // into the registers just freed.  An ordinary vector instruction next to every matrix instruction costs
+            // (measured) next to nothing; a run of them stops the matrix unit, so the scheduler is told to alternate.
             if (g == 0) dma_w(nxt3, s + 3);
-            if (g == 1 && P == 0) {
-                store_acts(af, nxt2, nxt3, (s >> 1) + 1);
-                __builtin_amdgcn_sched_barrier(0);
-                load_acts(af, (s >> 1) + 2);
-            }
+            if (P == 0 && g == 0) geom = geometry((s >> 1) + 2);
+            uint8_t *const dst = a_dst + (half ? nxt3 : nxt2);
+            static_for<0, 2 * RG>([&](auto m_c) __attribute__((always_inline)) {
+                constexpr int m = decltype(m_c)::value, e = m / RG, rg = m % RG;
+                acc[rg][2 * g + e] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[wb][e], xf[P][rg], acc[rg][2 * g + e], 0, 0, 0);
+                if (P == 0) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    static_for<0, NA2>([&](auto i_c) __attribute__((always_inline)) {
+                        constexpr int i = decltype(i_c)::value;
+                        if (i % G != g) return;
+                        if (m < 4) { // dword m of the piece: padding / re-bias / sums
+                            const uint32_t x = LM == kWideRowsFull ? af.raw[i][m] : (af.take[i] ? af.raw[i][m] : af.fill);
+                            rsum[i] = __builtin_amdgcn_sad_u8(x, 0u, rsum[i]); // (a dot product against ones costs the matrix unit seven cycles, this next to none)
+                            staged_piece[m] = x ^ 0x80808080u;
+                        } else if (m == 4) {
+                            *reinterpret_cast<wide_u32x4 *>(dst + i * PSTEP * 64) = staged_piece;
+                        } else if (m == 5) {
+                            load_piece(af, geom, i_c);
+                        }
+                    });
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            });
         }
         cur = nxt;
         __builtin_amdgcn_sched_barrier(0);
@@ -580,11 +606,11 @@ __global__ __launch_bounds__(WM * WN * 64, 2) void qconv_wide4_kernel(const Igem
     // a pixel's sum of x' is spread over the eight threads that loaded its pieces
 #pragma unroll
     for (int i = 0; i < NA2; i++) {
-        int32_t r = rsum[i];
+        int32_t r = (int32_t)rsum[i];
         r += __shfl_xor(r, 1);
         r += __shfl_xor(r, 2);
         r += __shfl_xor(r, 4);
-        if ((threadIdx.x & 7) == 0) rowsums[lp + i * PSTEP] = r;
+        if ((threadIdx.x & 7) == 0) rowsums[lp + i * PSTEP] = r - 128 * 64 * KS;
     }
     __syncthreads(); // (also: every wave's reads of the ring are done before the staging areas below are written, every DMA has landed)
     static_assert(!staged_store_built(T) || WM * WN * staged_store_bytes() <= NS * SLOT, "the staging areas fit the ring");
@@ -615,6 +641,281 @@ template <int T, int RG, int WM, int WN, int LM> int launch_wide4_t(nncase_hip_c
     return 0;
 }
 
+
+
+// ---- the same block for contiguous reduction rows (1x1 windows, matmul), fed by DMA alone ------------------------
+// With nothing to substitute on the way in (no padding taps), the activations can take the DMA path as well: no
+// staging registers, no LDS writes by the waves, no wait on loaded registers inside the loop.  The re-bias to s8 and
+// the sums of x move to the consuming side: a wave reads its operand of the NEXT k-step at the top of a k-step and,
+// one instruction next to each matrix instruction of the k-step, adds the bytes of every register (v_sad_u8) and
+// xors it; a lane ends up with the sum of its own 16-byte pieces, and the four lanes of a pixel add them in the
+// epilogue (they are the lanes that need the sum).
+//   LDS = 160 KiB: weights, four k-step slots of TB KiB (requested three k-steps ahead, two to land);
+//   activations, three stages of PIX pixels x 128 bytes (a pair of k-steps; requested five k-steps ahead, four to
+//   land: the trip to HBM).  A pixel's eight 16-byte pieces sit rotated by the pixel index, so that the eight
+//   lanes an LDS read serves together -- same piece, eight consecutive pixels -- meet eight different bank groups;
+//   the lanes of a DMA request (a 1 KiB run: eight pixels) fetch the pieces in the rotated order.
+// The per-channel constants, the byte table and the staging areas of dword outputs take over the ring's memory once
+// the last k-step is done.
+template <int T, int RG, int WM, int WN, int LM>
+__global__ __launch_bounds__(WM * WN * 64, WM * WN >= 8 ? 2 : 1) void qconv_wide_dma_kernel(const IgemmArgs a, int nchunks) {
+    static_assert(LM == kWideRowsFull || LM == kWideRows, "contiguous reduction rows only");
+    constexpr int NSW = 4, NSA = 3;
+    constexpr int THREADS = WM * WN * 64, WAVES = WM * WN;
+    constexpr int PIX = WM * RG * 16;
+    constexpr int TB = T * WN;
+    constexpr int WSLOT = TB * 1024;                    // bytes of a weight slot (one k-step)
+    constexpr int ASTAGE = PIX * 128;                   // bytes of an activation stage (two k-steps)
+    constexpr int NW = TB / WAVES;                      // weight runs (1 KiB) per wave per k-step
+    constexpr int NA = PIX / 8 / WAVES;                 // activation runs per wave per pair of k-steps
+    static_assert(TB % WAVES == 0 && (PIX / 8) % WAVES == 0 && NA % 4 == 0, "every wave moves the same number of runs");
+    static_assert(T % 4 == 0, "at least two pairs of channel tiles per k-step");
+    static_assert((WSLOT & (WSLOT - 1)) == 0, "the weight ring wraps by a mask");
+    constexpr int G = T / 2;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    uint8_t *const wring = smem;                        // [NSW][WSLOT]
+    uint8_t *const aring = smem + NSW * WSLOT;          // [NSA][ASTAGE]
+    // after the main loop
+    int32_t *cterm = reinterpret_cast<int32_t *>(smem);              // [TB * 16]
+    uint8_t *lutl = smem + TB * 16 * sizeof(int32_t);                // [256]
+    uint8_t *stage_base = lutl + 256;
+
+    const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3;
+    const int chunk = seq % nchunks;
+    const int per = (a.num_mtiles + 7) >> 3;
+    const int mt = xcd * per + seq / nchunks;
+    if (seq / nchunks >= per || mt >= a.num_mtiles) return;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wm = wave % WM, wn = wave / WM;
+    const int j = lane & 15, gq = lane >> 4;
+    const int ch_base = chunk * (TB * 16);
+    const int KS = a.ksteps;
+    const __amdgpu_buffer_rsrc_t wres = wide_rsrc(a.wpk + (size_t)chunk * KS * TB * 1024, (uint32_t)KS * TB * 1024);
+    const __amdgpu_buffer_rsrc_t xres = wide_rsrc(a.x, (uint32_t)a.x_bytes);
+
+    // ---- weights: wave w moves the runs w + i * WAVES of a k-step ----
+    const uint32_t w_voff = threadIdx.x * 16;
+    auto dma_w = [&](int slot /* byte offset in the weight ring */, int ks, auto first, auto count) __attribute__((always_inline)) {
+        const int ksc = min(ks, KS - 1); // a k-step past the end re-reads the last one (its data is never multiplied)
+        static_for<decltype(first)::value, decltype(first)::value + decltype(count)::value>([&](auto i_c) __attribute__((always_inline)) {
+            constexpr int i = decltype(i_c)::value;
+            __attribute__((address_space(3))) uint8_t *dst = (__attribute__((address_space(3))) uint8_t *)(wring + slot + (i * WAVES + wave) * 1024);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(wres, dst, 16, (int)w_voff, (ksc * TB + i * WAVES) * 1024, 0, 0);
+        });
+    };
+    // ---- activations: wave w moves the runs w * NA + i of a pair; lane l of run r fetches, for pixel 8 r + (l >> 3),
+    // the piece that belongs at position l & 7 of the pixel's 128 bytes ----
+    uint32_t a_voff[NA];
+#pragma unroll
+    for (int i = 0; i < NA; i++) {
+        const int pl = (wave * NA + i) * 8 + (lane >> 3);                 // pixel of the block
+        const int p = min(mt * PIX + pl, a.m - 1);                         // (a pixel past the end repeats the last one: not stored)
+        const int piece = ((lane & 7) - pl) & 7;
+        a_voff[i] = (uint32_t)p * (uint32_t)a.ldx + (uint32_t)a.x_coff + piece * 16;
+    }
+    auto dma_a = [&](int stage /* byte offset in the activation ring */, int pair, auto first, auto count) __attribute__((always_inline)) {
+        const int pc = min(pair, (KS - 1) >> 1);
+        static_for<decltype(first)::value, decltype(first)::value + decltype(count)::value>([&](auto i_c) __attribute__((always_inline)) {
+            constexpr int i = decltype(i_c)::value;
+            __attribute__((address_space(3))) uint8_t *dst = (__attribute__((address_space(3))) uint8_t *)(aring + stage + (wave * NA + i) * 1024);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(xres, dst, 16, (int)a_voff[i], pc * 128, 0, 0);
+        });
+    };
+
+    v4i acc[RG][T];
+#pragma unroll
+    for (int rg = 0; rg < RG; rg++)
+#pragma unroll
+        for (int nt = 0; nt < T; nt++) acc[rg][nt] = v4i{0, 0, 0, 0};
+    // sums of x over this lane's pieces of its RG pixels: rs runs one k-step ahead of the products (it is taken from the
+    // operand read ahead), so what the epilogue uses is its value at the start of the last k-step
+    uint32_t rs[RG], rs_final[RG];
+#pragma unroll
+    for (int rg = 0; rg < RG; rg++) rs[rg] = rs_final[rg] = 0;
+
+    // s_waitcnt immediates (gfx9 encoding): vmcnt in bits [3:0] and [15:14], expcnt [6:4], lgkmcnt [11:8]
+    constexpr auto waitcnt_imm = [](int vm, int lgkm) { return (vm & 15) | ((vm >> 4) << 14) | (7 << 4) | ((lgkm & 15) << 8); };
+    // ---- fill (the order is what the waits count) ----
+    constexpr std::integral_constant<int, 0> c0;
+    constexpr std::integral_constant<int, NW> cNW;
+    constexpr std::integral_constant<int, NA> cNA;
+    constexpr std::integral_constant<int, NW / 2> cNWh;
+    constexpr std::integral_constant<int, NA / 2> cNAh;
+    static_assert(NW % 2 == 0 && NA % 2 == 0, "requests are issued in halves");
+    dma_w(0, 0, c0, cNW);
+    dma_w(WSLOT, 1, c0, cNW);
+    __builtin_amdgcn_sched_barrier(0);
+    dma_a(0, 0, c0, cNA);
+    __builtin_amdgcn_sched_barrier(0);
+    dma_a(ASTAGE, 1, c0, cNA);
+    __builtin_amdgcn_sched_barrier(0);
+    dma_w(2 * WSLOT, 2, c0, cNW);
+    __builtin_amdgcn_sched_barrier(0);
+    dma_a(2 * ASTAGE, 2, c0, cNA);
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(NA + NW + NA, 15)); // the first two k-steps' weights and the first pair's activations are in
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+
+    // operand addresses: pixel (wm RG + rg) * 16 + j, piece (h * 4 + gq) of the stage, rotated by the pixel index
+    const uint8_t *const x_src0 = aring + (wm * RG * 16 + j) * 128 + ((gq + j) & 7) * 16;     // first k-step of a pair, + rg * 2048
+    const uint8_t *const x_src1 = aring + (wm * RG * 16 + j) * 128 + ((4 + gq + j) & 7) * 16; // second
+    const uint8_t *const w_src = wring + (wn * T) * 1024 + lane * 16;                           // + nt * 1024
+    // the last k-step may end inside the row: pieces past K meet zero weights, and are masked out of the sums of x
+    const uint32_t tail_mask = (LM == kWideRows && (KS - 1) * 64 + gq * 16 >= a.k) ? 0u : 0xffffffffu;
+    // weight operands are read two pairs of tiles ahead of their products (an LDS read under this load takes longer
+    // than the eight matrix instructions of one pair): one register buffer per pair of a k-step
+    static_assert(G == 4, "four pairs of channel tiles per k-step");
+    v4i xf[2][RG], wf[G][2];
+#pragma unroll
+    for (int rg = 0; rg < RG; rg++) {
+        xf[0][rg] = *reinterpret_cast<const v4i *>(x_src0 + rg * 2048);
+#pragma unroll
+        for (int d = 0; d < 4; d++) {
+            const uint32_t x = (uint32_t)xf[0][rg][d] & (LM == kWideRows && KS == 1 ? tail_mask : 0xffffffffu);
+            rs[rg] = __builtin_amdgcn_sad_u8(x, 0u, rs[rg]);
+            xf[0][rg][d] = (int)((uint32_t)xf[0][rg][d] ^ 0x80808080u);
+        }
+    }
+    wf[0][0] = *reinterpret_cast<const v4i *>(w_src);
+    wf[0][1] = *reinterpret_cast<const v4i *>(w_src + 1024);
+    wf[1][0] = *reinterpret_cast<const v4i *>(w_src + 2048);
+    wf[1][1] = *reinterpret_cast<const v4i *>(w_src + 3072);
+    int wcur = 0, acur = 0; // ring offsets of k-step s: weight slot, activation stage (the latter moves every other k-step)
+    auto kstep = [&](int s, auto parity) __attribute__((always_inline)) {
+        constexpr int P = decltype(parity)::value; // s & 1: operand buffer, and which half of the stage
+        asm volatile("" : "+s"(wcur), "+s"(acur));
+        const int wnxt = (wcur + WSLOT) & (NSW * WSLOT - 1), wnxt3 = (wcur + 3 * WSLOT) & (NSW * WSLOT - 1);
+        // stage of k-step s + 1: the same for an even s, the next one for an odd s
+        const int anext = acur + ASTAGE >= NSA * ASTAGE ? 0 : acur + ASTAGE;
+        const int a_of_next = P == 0 ? acur : anext;
+        const uint8_t *const ws = w_src + wcur;
+        // the mask of the next k-step's sums (all ones but for the lanes past K of the last k-step)
+        const uint32_t mask = (LM == kWideRows && s + 1 == KS - 1) ? tail_mask : 0xffffffffu;
+        constexpr int NM = 2 * RG; // matrix instructions per group
+        {
+            const bool last = s == KS - 1;
+#pragma unroll
+            for (int rg = 0; rg < RG; rg++) rs_final[rg] = last ? rs[rg] : rs_final[rg];
+        }
+        static_for<0, G>([&](auto g_c) __attribute__((always_inline)) {
+            constexpr int g = decltype(g_c)::value;
+            constexpr int wb = g; // this pair's buffer
+            __builtin_amdgcn_sched_barrier(0);
+            {
+                // the pair two on: of this k-step, or the first two of the next (whose slot is complete since the last barrier)
+                constexpr int gn = (g + 2) % G;
+                const uint8_t *const wsrc = (g + 2 < G ? ws : w_src + wnxt) + (2 * gn) * 1024;
+                wf[gn][0] = *reinterpret_cast<const v4i *>(wsrc);
+                wf[gn][1] = *reinterpret_cast<const v4i *>(wsrc + 1024);
+            }
+            if (g == 0) {
+                // the next k-step's operand (its slot is complete since the last barrier): re-biased and summed under this k-step's products
+                const uint8_t *const xn = (P == 0 ? x_src1 : x_src0) + a_of_next;
+#pragma unroll
+                for (int rg = 0; rg < RG; rg++) xf[1 - P][rg] = *reinterpret_cast<const v4i *>(xn + rg * 2048);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            // Requests, a few per group so that the address unit's queue never fills and holds a wave at a load with its
+            // matrix instructions behind it (in this order in the instruction stream: the wait below counts what
+            // follows a k-step's weights): the weights of k-step s + 3 in halves (groups 0 and 2); activations in
+            // quarters, pair (s + 5) / 2 in the odd k-step that frees its stage -- this k-step's own pair, whose last
+            // operands were read in the first group of the previous k-step, by every wave before the barrier that
+            // ended it -- and in the even one behind it (groups 1 and 3)
+            if (g == 0) dma_w(wnxt3, s + 3, c0, cNWh);
+            if (g == 2) dma_w(wnxt3, s + 3, cNWh, cNWh);
+            if (P == 1) {
+                if (g == 1) dma_a(acur, (s + 5) >> 1, c0, std::integral_constant<int, NA / 4>());
+                if (g == 3) dma_a(acur, (s + 5) >> 1, std::integral_constant<int, NA / 4>(), std::integral_constant<int, NA / 4>());
+            } else {
+                // (an even k-step: the stage before this one's, pair (s + 4) / 2)
+                const int aprev = acur == 0 ? (NSA - 1) * ASTAGE : acur - ASTAGE;
+                if (g == 1) dma_a(aprev, (s + 4) >> 1, cNAh, std::integral_constant<int, NA / 4>());
+                if (g == 3) dma_a(aprev, (s + 4) >> 1, std::integral_constant<int, 3 * NA / 4>(), std::integral_constant<int, NA / 4>());
+            }
+            static_for<0, NM>([&](auto m_c) __attribute__((always_inline)) {
+                constexpr int m = decltype(m_c)::value, e = m / RG, rg = m % RG;
+                acc[rg][2 * g + e] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[wb][e], xf[P][rg], acc[rg][2 * g + e], 0, 0, 0);
+                // groups 1 .. G - 1 carry the 4 RG registers of the next operand, spread evenly: sum, then re-bias
+                if constexpr (g >= 1) {
+                    constexpr int slots = (G - 1) * NM;              // matrix instructions to spread over
+                    constexpr int idx = (g - 1) * NM + m;            // this one's index
+                    constexpr int lo = idx * (4 * RG) / slots, hi = (idx + 1) * (4 * RG) / slots;
+                    __builtin_amdgcn_sched_barrier(0);
+                    static_for<lo, hi>([&](auto r_c) __attribute__((always_inline)) {
+                        constexpr int r = decltype(r_c)::value, xr = r / 4, d = r % 4;
+                        const uint32_t x = (uint32_t)xf[1 - P][xr][d];
+                        rs[xr] = __builtin_amdgcn_sad_u8(LM == kWideRows ? (x & mask) : x, 0u, rs[xr]);
+                        xf[1 - P][xr][d] = (int)(x ^ 0x80808080u);
+                    });
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            });
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        wcur = wnxt;
+        acur = a_of_next;
+        __builtin_amdgcn_sched_barrier(0);
+        // the weights of k-step s + 2 (requested during k-step s - 1) and the activations requested two and three
+        // k-steps ago have landed: behind them came the last quarter of that k-step's activation runs, this k-step's
+        // NW weight runs and its NA / 2 activation runs; of this wave's operand reads only the four of the next weights
+        // may still be out
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(NA / 4 + NW + NA / 2, 4));
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    int s = 0;
+#pragma clang loop unroll(disable)
+    for (; s + 1 < KS; s += 2) {
+        kstep(s, std::integral_constant<int, 0>());
+        kstep(s + 1, std::integral_constant<int, 1>());
+    }
+    if (s < KS) kstep(s, std::integral_constant<int, 0>()); // an odd number of k-steps
+
+    // ---- epilogue ----
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0)); // every DMA of this wave has landed, every operand read is back
+    __syncthreads();                               // ... of every wave: the rings are free
+    constexpr int NC = (TB * 16 + THREADS - 1) / THREADS;
+#pragma unroll
+    for (int i = 0; i < NC; i++) {
+        const int c = i * THREADS + threadIdx.x;
+        if (c < TB * 16) cterm[c] = ch_base + c < a.n ? a.bias[ch_base + c] - a.zxp * a.wsum[ch_base + c] + a.k * a.zxp * a.zwp : 0;
+    }
+    if (a.lut && threadIdx.x < 64) reinterpret_cast<uint32_t *>(lutl)[threadIdx.x] = a.lut[threadIdx.x];
+    __syncthreads();
+    uint8_t *const stage = staged_store_built(T) ? stage_base + wave * staged_store_bytes() : nullptr;
+    const int ch0 = ch_base + gq * (4 * TB) + wn * (4 * T);
+    const int32_t *ct = cterm + gq * (4 * TB) + wn * (4 * T) - gq * (4 * T); // igemm_store_tile adds gq * 4 T
+    static_for<0, RG>([&](auto rg_c) __attribute__((always_inline)) {
+        constexpr int rg = decltype(rg_c)::value;
+        const int pl = (wm * RG + rg) * 16 + j;
+        // the pixel's sum of x, spread over the lanes of its four pieces; x' = x - 128 over the K real positions
+        int32_t sx = (int32_t)rs_final[rg];
+        sx += __shfl_xor(sx, 16);
+        sx += __shfl_xor(sx, 32);
+        igemm_store_tile<T, kOwesAll, false, staged_store_built(T)>(a, acc[rg], sx - 128 * a.k, mt * PIX + pl, ch0, gq, ct, lutl, stage, 4 * TB);
+    });
+}
+
+template <int T, int RG, int WM, int WN, int LM> int launch_wide_dma_t(nncase_hip_ctx *ctx, const IgemmArgs &a, int nchunks) {
+    IgemmArgs args = a;
+    constexpr int PIX = WM * RG * 16, TB = T * WN;
+    args.num_mtiles = ceil_div(a.m, PIX);
+    const int blocks = ceil_div(args.num_mtiles, 8) * 8 * nchunks;
+    const size_t lds = (size_t)4 * TB * 1024 + (size_t)3 * PIX * 128;
+    static std::once_flag raised[16]; // more than 64 KiB of dynamic LDS has to be asked for once per kernel and device
+    hipError_t attr = hipSuccess;
+    std::call_once(raised[ctx->device & 15], [&] {
+        attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&qconv_wide_dma_kernel<T, RG, WM, WN, LM>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    });
+    NNHIP_HIP(ctx, attr);
+    hipLaunchKernelGGL((qconv_wide_dma_kernel<T, RG, WM, WN, LM>), dim3(blocks), dim3(WM * WN * 64), lds, ctx->stream, args, nchunks);
+    NNHIP_LAUNCH_CHECK(ctx, "qconv_wide_dma_kernel");
+    return 0;
+}
+
 template <int T, int RG, int WM, int WN, int LM> int launch_wide_t(nncase_hip_ctx *ctx, const IgemmArgs &a, int nchunks) {
     IgemmArgs args = a;
     constexpr int PIX = WM * RG * 16, TB = T * WN;
@@ -642,7 +943,12 @@ inline int wide_waves(const nncase_hip_ctx *ctx, int m, int nchunks) {
 // Block shapes: tiles = 16 -> 256 pixels x 256 channels (4 x 2 waves); tiles = 8 -> 256 or 128 pixels x 128 channels;
 // tiles = 4 -> 256 or 128 pixels x 64 channels.
 template <int LM> int launch_wide_lm(nncase_hip_ctx *ctx, const IgemmArgs &a, int tiles, int nchunks) {
-    if (tiles == 16) return launch_wide4_t<8, 4, 4, 2, LM>(ctx, a, nchunks);
+    if (tiles == 16) {
+        if constexpr (LM == kWideRowsFull || LM == kWideRows) {
+            if (a.x_bytes < ((size_t)1 << 31)) return launch_wide_dma_t<8, 4, 4, 2, LM>(ctx, a, nchunks);
+        }
+        return launch_wide4_t<8, 4, 4, 2, LM>(ctx, a, nchunks);
+    }
     const int wmv = wide_waves(ctx, a.m, nchunks);
     if (tiles == 8) return wmv == 4 ? launch_wide_t<8, 4, 4, 1, LM>(ctx, a, nchunks) : launch_wide_t<8, 4, 2, 1, LM>(ctx, a, nchunks);
     if (tiles == 4) return wmv == 4 ? launch_wide_t<4, 4, 4, 1, LM>(ctx, a, nchunks) : launch_wide_t<4, 4, 2, 1, LM>(ctx, a, nchunks);

@@ -220,13 +220,16 @@ def test_wide_tile_kernels(hip_ctx, case):
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
 
 
-@pytest.mark.parametrize("c,hw,oc,k", [(512, 256, 136, 1), (64, 256, 192, 3)])
+@pytest.mark.parametrize("c,hw,oc,k", [(512, (256, 256), 136, 1), (64, (256, 256), 192, 3),
+                                       (528, (255, 259), 200, 1),    # rows that end inside the ninth k-step, a ragged last pixel tile
+                                       (256, (128, 512), 800, 1),    # four channel chunks per pixel tile, the last one an eighth full
+                                       (48, (256, 257), 160, 3)])    # windows over 48 channels: seven k-steps, taps that straddle them
 def test_wide_tile_kernels_with_256_channel_blocks(hip_ctx, c, hw, oc, k):
     """From 65 536 pixels on, layers of more than 128 channels run blocks of 256 pixels x 256 channels (two waves side by side
     share the block's activations).  One oracle convolution gives the accumulators; the u8 expectation is the oracle's
     requantisation of them."""
     rng = np.random.default_rng(c + oc)
-    x = rng.integers(0, 256, (1, c, hw, hw), dtype=np.uint8)
+    x = rng.integers(0, 256, (1, c, hw[0], hw[1]), dtype=np.uint8)
     w = rng.integers(0, 256, (oc, c, k, k), dtype=np.uint8)
     bias = rng.integers(-3000, 3000, oc).astype(np.int32)
     pad = ((k // 2, k // 2), (k // 2, k // 2))
