@@ -231,6 +231,15 @@ NNCASE_HIP_API int nncase_hip_requant_plan(float sx, float sw, nncase_hip_quant_
                                            float *c1, float *c2);
 NNCASE_HIP_API int nncase_hip_requant_host(float sx, float sw, nncase_hip_quant_param_t y_qp, float clamp_min, float clamp_max,
                                            const int32_t *acc_host, size_t count, uint8_t *out_host, int32_t *form_used);
+/* The same for the form without an int -> float conversion that the dense row / window kernels and the stride-2
+ * depthwise kernel use where it exists: the sums are started from 0x4B400000, so that their bits read as a float
+ * are 12582912 + acc, and the code is RN(fma(that float, m1, m2)).  Returns 1 and writes the codes of the
+ * accumulators (each of magnitude at most *limit, the range the search vouches for; others get 0) when the
+ * search found a pair, 0 when it did not (nothing is written then), a negative status for scales out of range.
+ * Host-only like the two above (no counterpart in the reference: its CPU kernel divides, quantize.cpp:36-43). */
+NNCASE_HIP_API int nncase_hip_requant_host_magic(float sx, float sw, nncase_hip_quant_param_t y_qp, float clamp_min, float clamp_max,
+                                                 const int32_t *acc_host, size_t count, uint8_t *out_host, float *m1, float *m2,
+                                                 int32_t *limit);
 
 /* ---- fused inverted-residual block ------------------------------------------
  * 1x1 convolution (in -> mid channels), 3x3 depthwise convolution on the mid

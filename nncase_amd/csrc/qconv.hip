@@ -77,11 +77,29 @@ inline int requant_fma(int32_t v, float c1, float c2, const nnhip::Epilogue &ep)
     return (int)std::nearbyintf(c);
 }
 
+// The magic-bias form (Epilogue::magic) on accumulator v; -1 where kMagicBias + v is no positive finite float.
+inline int requant_magic(int64_t v, float m1, float m2, const nnhip::Epilogue &ep) {
+    const int64_t bits = (int64_t)nnhip::kMagicBias + v;
+    if (bits <= 0 || bits >= 0x7f800000) return -1;
+    const uint32_t b = (uint32_t)bits;
+    float x;
+    memcpy(&x, &b, sizeof(x));
+    const float u = std::fmaf(x, m1, m2);
+    float c = std::fmin(std::fmax(u, ep.qlo), ep.qhi);
+    return (int)std::nearbyintf(c);
+}
+// Accumulators the magic-bias form is vouched for: every |acc| up to this bound (far more than a reduction of
+// 16 384 products of bytes plus a bias can reach; kMagicBias + acc stays a positive finite float up to 8.7e8).
+constexpr int32_t kMagicLimit = 800000000;
+
 // Both forms are monotone non-decreasing step functions of the accumulator, so they are equal everywhere iff
 // they agree at both ends of the int32 range and on both sides of every step of the reference form.
 void find_fast_requant(nnhip::Epilogue *ep) {
     ep->fast = 0;
     ep->c1 = ep->c2 = 0.f;
+    ep->magic = 0;
+    ep->m1 = ep->m2 = 0.f;
+    ep->magic_limit = 0;
     if (!(ep->mult > 0.f) || !(ep->sy > 0.f)) return;
     const int32_t vmin = INT32_MIN + 1, vmax = INT32_MAX;
     const int rmin = requant_ref(vmin, *ep), rmax = requant_ref(vmax, *ep);
@@ -112,6 +130,36 @@ void find_fast_requant(nnhip::Epilogue *ep) {
     };
     const float c1_0 = (float)((double)ep->mult / (double)ep->sy);
     if (!std::isfinite(c1_0) || c1_0 <= 0.f) return;
+    // The magic-bias pair: m1 near the nominal slope with its two lowest mantissa bits clear, so that 12582912 * m1
+    // (a product with 3 * 2^22) is exact in fp32 and m2 = zy - 12582912 * m1 can be too; the map is then
+    // RN(acc * m1 + zy) in one rounding.  Checked like the pair below, over the accumulator range it is used for.
+    {
+        auto magic_matches = [&](float m1, float m2) {
+            if (requant_magic(-(int64_t)kMagicLimit, m1, m2, *ep) != requant_ref(-kMagicLimit, *ep)) return false;
+            if (requant_magic(kMagicLimit, m1, m2, *ep) != requant_ref(kMagicLimit, *ep)) return false;
+            for (size_t i = 0; i < steps.size(); i++) {
+                if (requant_magic(steps[i], m1, m2, *ep) != requant_ref(steps[i], *ep)) return false;
+                if (requant_magic((int64_t)steps[i] - 1, m1, m2, *ep) != requant_ref(steps[i] - 1, *ep)) return false;
+            }
+            return true;
+        };
+        uint32_t bits;
+        memcpy(&bits, &c1_0, sizeof(bits));
+        for (int k = 0; k <= 12 && !ep->magic; k++)
+            for (int sgn = 1; sgn >= -1 && !ep->magic; sgn -= 2) {
+                if (k == 0 && sgn < 0) continue;
+                const uint32_t cb = (bits & ~3u) + (uint32_t)(sgn * 4 * k);
+                float m1;
+                memcpy(&m1, &cb, sizeof(m1));
+                if (!(m1 > 0.f) || !std::isfinite(m1)) continue;
+                const double m2d = (double)ep->zy - 12582912.0 * (double)m1;
+                const float m2 = (float)m2d;
+                if ((double)m2 != m2d) continue; // not representable: the sum would be rounded twice
+                if (magic_matches(m1, m2)) {
+                    ep->m1 = m1, ep->m2 = m2, ep->magic = 1, ep->magic_limit = kMagicLimit;
+                }
+            }
+    }
     // nominal constants first, then small perturbations of both (the reference's own rounding noise decides a
     // few steps that sit almost exactly on an integer accumulator)
     for (int ring = 0; ring <= 24; ring++)
@@ -156,6 +204,9 @@ int nnhip::make_epilogue(nncase_hip_ctx *ctx, Epilogue *ep, float sx, float sw, 
     ep->c1 = ep->c2 = 0.f;
     ep->fast = 0;
     ep->full = 1;
+    ep->m1 = ep->m2 = 0.f;
+    ep->magic = 0;
+    ep->magic_limit = 0;
     ep->out_mode = out_dtype == NNCASE_HIP_DT_U8 ? kOutU8 : (out_dtype == NNCASE_HIP_DT_I32 ? kOutI32 : kOutF32);
     NNHIP_REQUIRE(ctx, !(clamp_min > clamp_max), -EINVAL, "%s: fused clamp minimum above maximum", who);
     if (ep->out_mode != kOutU8) return 0;
@@ -183,6 +234,7 @@ int nnhip::make_epilogue(nncase_hip_ctx *ctx, Epilogue *ep, float sx, float sw, 
         for (const auto &e : g_epilogues.entries)
             if (e.first == key) {
                 ep->c1 = e.second.c1, ep->c2 = e.second.c2, ep->fast = e.second.fast;
+                ep->m1 = e.second.m1, ep->m2 = e.second.m2, ep->magic = e.second.magic, ep->magic_limit = e.second.magic_limit;
                 return 0;
             }
         find_fast_requant(ep);
@@ -244,6 +296,24 @@ extern "C" int nncase_hip_requant_host(float sx, float sw, nncase_hip_quant_para
     for (size_t i = 0; i < count; i++)
         out_host[i] = (uint8_t)(ep.fast ? requant_fma(acc_host[i], ep.c1, ep.c2, ep) : requant_ref(acc_host[i], ep));
     return 0;
+}
+
+extern "C" int nncase_hip_requant_host_magic(float sx, float sw, nncase_hip_quant_param_t y_qp, float clamp_min, float clamp_max,
+                                             const int32_t *acc_host, size_t count, uint8_t *out_host, float *m1, float *m2,
+                                             int32_t *limit) {
+    if (count && (!acc_host || !out_host)) return -EINVAL;
+    Epilogue ep;
+    const int rc = make_epilogue(nullptr, &ep, sx, sw, y_qp, clamp_min, clamp_max, NNCASE_HIP_DT_U8, "requant_host_magic");
+    if (rc) return rc;
+    if (!ep.magic) return 0;
+    if (m1) *m1 = ep.m1;
+    if (m2) *m2 = ep.m2;
+    if (limit) *limit = ep.magic_limit;
+    for (size_t i = 0; i < count; i++) {
+        const int64_t v = acc_host[i];
+        out_host[i] = (v < -(int64_t)ep.magic_limit || v > ep.magic_limit) ? 0 : (uint8_t)requant_magic(v, ep.m1, ep.m2, ep);
+    }
+    return 1;
 }
 
 extern "C" int nncase_hip_qconv2d_prepack(nncase_hip_ctx_t *ctx, const nncase_hip_conv2d_desc_t *desc,

@@ -21,6 +21,7 @@ struct nncase_hip_weights {
     // 128 pixels x 64 channels or 64 x 32, waves of 32 pixels)
     int wide = 0;
     long long dw_const_bound = 0; // depthwise: max over channels of |bias| + 255 |sum(w - zw)|
+    long long bias_absmax = 0;    // largest |bias|
     int64_t pixels_hint = 0; // output pixels per call the tiling was planned for (0 = unknown)
     int32_t zw = 0;
     float sw = 1.f;
@@ -65,7 +66,17 @@ struct Epilogue {
     float c1, c2;
     int fast;
     int full; // rne(qlo) == 0 and rne(qhi) == 255: the saturating conversion to u8 is the whole clamp
+    // The same form on an accumulator that was started from kMagicBias: while |acc| < 2^22 the bits of
+    // kMagicBias + acc, read as a float, ARE the float 12582912 + acc, so the int -> float conversion disappears:
+    //   RN(fma(as_float(kMagicBias + acc), m1, m2)),  m2 = zy - 12582912 * m1 exactly (m1 has two spare mantissa bits).
+    // Beyond 2^22 the float keeps growing with the accumulator (positive floats order like their bit patterns), which
+    // is all the proof needs: both maps are monotone, and make_epilogue checks them equal at every step of the
+    // staircase and at both ends of the accumulator range [-magic_limit, magic_limit] it vouches for.
+    float m1, m2;
+    int magic;            // 0: no such pair was found
+    int32_t magic_limit;  // largest |acc| the equality was established for
 };
+constexpr int32_t kMagicBias = 0x4B400000; // the bits of 12582912.0f = 1.5 * 2^23
 
 // Second requantisation stage of a fused residual add:
 //   s = ((float)q - zy) * sy + ((float)r - zr) * sr;   out = sat_u8(rne(clamp(s) / sum.sy + sum.zy))
@@ -190,6 +201,14 @@ template <typename T> __device__ __forceinline__ uint32_t requant4_u8_packed_dir
     uint32_t d = 0;
 #pragma unroll
     for (int r = 0; r < 4; r++) d = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_fmaf((float)v[r], ep.c1, ep.c2), r, d);
+    return d;
+}
+
+// The magic-bias form: v are accumulators that were started from kMagicBias (see Epilogue::magic).
+__device__ __forceinline__ uint32_t requant4_u8_packed_magic(const int32_t (&v)[4], const Epilogue &ep) {
+    uint32_t d = 0;
+#pragma unroll
+    for (int r = 0; r < 4; r++) d = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_fmaf(__int_as_float(v[r]), ep.m1, ep.m2), r, d);
     return d;
 }
 

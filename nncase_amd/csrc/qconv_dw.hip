@@ -71,13 +71,16 @@ __device__ __forceinline__ void dw_store4(const DwArgs &a, uint32_t o, const int
 // is replaced by the first pixel of the thread's first row, address and value, which always exists, is written
 // by this thread alone and so is merely written again.  `safe_off` / `safe_val` carry that pixel; `first` is
 // uniform.
-template <bool FF, typename T>
+template <bool FF, bool MG, typename T>
 __device__ __forceinline__ void dw_store_row(const DwArgs &a, uint32_t o, const T (&v)[kDwCols][4], const bool (&col_stored)[kDwCols],
                                              bool row_stored, bool first, uint32_t &safe_off, uint32_t &safe_val) {
     if (FF || std::is_same<T, float>::value || a.ep.out_mode == kOutU8) { // (fp32 sums are used for u8 outputs only)
         uint32_t q[kDwCols];
 #pragma unroll
-        for (int c = 0; c < kDwCols; c++) q[c] = FF ? requant4_u8_packed_direct(v[c], a.ep) : requant4_u8_packed(v[c], a.ep);
+        for (int c = 0; c < kDwCols; c++) {
+            if constexpr (MG && std::is_same<T, int32_t>::value) q[c] = requant4_u8_packed_magic(v[c], a.ep);
+            else q[c] = FF ? requant4_u8_packed_direct(v[c], a.ep) : requant4_u8_packed(v[c], a.ep);
+        }
         safe_off = first ? o : safe_off;
         safe_val = first ? q[0] : safe_val;
 #pragma unroll
@@ -118,7 +121,9 @@ __device__ __forceinline__ void dw_store_row(const DwArgs &a, uint32_t o, const 
 // vector unit (v_fma_f32) instead of the integer multiplier's lower one; the accumulators need no conversion
 // before they are requantised either.
 // FF: the layer's epilogue is the one-instruction requantisation to u8 (fast and full), fixed at compile time.
-template <int S, bool FP, bool FF> __global__ __launch_bounds__(kDwThreads, (S == 2 && !FP ? 3 : 1)) void dw3x3_kernel(const DwArgs a) {
+// MG (integer sums): they start from kMagicBias and are requantised as floats without a conversion (Epilogue::magic).
+template <int S, bool FP, bool FF, bool MG = false> __global__ __launch_bounds__(kDwThreads, (S == 2 && !FP ? 3 : 1)) void dw3x3_kernel(const DwArgs a) {
+    static_assert(!MG || (FF && !FP), "the magic-bias form replaces the conversion of integer sums in the one-instruction epilogue");
     using acc_t = typename std::conditional<FP, float, int32_t>::type;
     constexpr int NCOL = (kDwCols - 1) * S + 3;
     // Workgroups are dealt to the 8 XCDs round-robin, each XCD with an L2 of its own.  Renumber them
@@ -167,10 +172,11 @@ template <int S, bool FP, bool FF> __global__ __launch_bounds__(kDwThreads, (S =
     {
         const int4 b = *reinterpret_cast<const int4 *>(a.bias + c0);
         const int4 s = *reinterpret_cast<const int4 *>(a.wsum + c0);
-        ct[0] = (acc_t)(b.x - a.zx * s.x);
-        ct[1] = (acc_t)(b.y - a.zx * s.y);
-        ct[2] = (acc_t)(b.z - a.zx * s.z);
-        ct[3] = (acc_t)(b.w - a.zx * s.w);
+        constexpr int32_t start = MG ? kMagicBias : 0;
+        ct[0] = (acc_t)(b.x - a.zx * s.x + start);
+        ct[1] = (acc_t)(b.y - a.zx * s.y + start);
+        ct[2] = (acc_t)(b.z - a.zx * s.z + start);
+        ct[3] = (acc_t)(b.w - a.zx * s.w + start);
     }
 
     const uint32_t in_row = (uint32_t)(a.in_w * a.channels); // elements per input row
@@ -288,7 +294,7 @@ template <int S, bool FP, bool FF> __global__ __launch_bounds__(kDwThreads, (S =
                             }
                         }
                 }
-                dw_store_row<FF>(a, out_off, acc, col_stored, tt < rows_here, tt == 0, safe_off, safe_val);
+                dw_store_row<FF, MG>(a, out_off, acc, col_stored, tt < rows_here, tt == 0, safe_off, safe_val);
                 out_off += out_row;
             }
         }
@@ -463,7 +469,9 @@ int launch_qconv_depthwise(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_h
         } else {
             // (stride 2 holds nine input columns per row: as floats they leave room for two waves per SIMD only,
             // and the largest stride-2 layer of MobileNetV2 runs 15 % slower that way)
-            if (ff) hipLaunchKernelGGL((dw3x3_kernel<2, false, true>), g, t, 0, ctx->stream, a);
+            const bool mg = ff && a.ep.magic && w->dw_const_bound + 9 * 255 * 255 <= a.ep.magic_limit;
+            if (mg) hipLaunchKernelGGL((dw3x3_kernel<2, false, true, true>), g, t, 0, ctx->stream, a);
+            else if (ff) hipLaunchKernelGGL((dw3x3_kernel<2, false, true>), g, t, 0, ctx->stream, a);
             else hipLaunchKernelGGL((dw3x3_kernel<2, false, false>), g, t, 0, ctx->stream, a);
         }
         NNHIP_LAUNCH_CHECK(ctx, "dw3x3_kernel");

@@ -88,6 +88,7 @@ int prepack_igemm(nncase_hip_ctx *ctx, nncase_hip_weights *w, const uint8_t *w_o
     std::vector<uint8_t> packed(w->packed_bytes);
     std::vector<int32_t> wsum(w->out_channels), hb(w->out_channels, 0);
     if (bias) std::copy(bias, bias + w->out_channels, hb.begin());
+    for (int32_t b : hb) w->bias_absmax = std::max<long long>(w->bias_absmax, std::llabs((long long)b));
     const int g_ic = w->g_ic, kh = w->kernel_h, kw = w->kernel_w;
     for (int g = 0; g < w->groups; g++) {
         const uint8_t *wg = w_oihw + (size_t)g * w->g_oc * g_ic * kh * kw;
@@ -180,6 +181,8 @@ int launch_qconv_igemm(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_hip_w
         const int rc = make_residual_epilogue(ctx, &a.rep, c, w);
         if (rc) return rc;
     }
+    // every accumulator, the zero-point terms included, is at most |bias| + 4 K 128^2 in magnitude
+    a.magic_ok = a.ep.magic && a.ep.full && w->bias_absmax + 4ll * w->k * 16384 <= a.ep.magic_limit;
     a.lut = c->out_dtype == NNCASE_HIP_DT_U8 ? w->d_post_lut : nullptr;
     if (c->dequantize_output != 0) { // (out_dtype is u8 here: the entry point has turned the call into its u8 form)
         const nncase_hip_quant_param_t last = c->residual_dev ? c->sum_qp : (w->d_post_lut ? w->post_lut_qp : c->y_qp);

@@ -78,6 +78,7 @@ struct IgemmArgs {
     Epilogue ep;
     ResidualEpilogue rep;
     const uint32_t *lut;   // 256-entry byte table applied to the requantised byte (before the residual add), or null
+    int magic_ok;          // the epilogue's magic-bias pair exists and every accumulator of this layer stays within its range
     int deq;               // the u8 result is stored as float32: (q - deq_zero) * deq_scale
     int deq_zero;
     float deq_scale;
@@ -387,11 +388,13 @@ __device__ __forceinline__ void store_dword_group(const IgemmArgs &a, const uint
 
 // STAGED: the kernel has a staging area per wave for the dword outputs (store_dword_group); the lane-by-lane dword
 // stores are then not built.
-template <int T, int OWED = kOwesAll, bool PLAIN = false, bool STAGED = false>
+// MAGIC (with PLAIN): the accumulators were started from kMagicBias and are requantised as floats (Epilogue::magic).
+template <int T, int OWED = kOwesAll, bool PLAIN = false, bool STAGED = false, bool MAGIC = false>
 __device__ __forceinline__ void igemm_store_tile(const IgemmArgs &a, const v4i (&acc)[T], int32_t rowsum, int p, int ch0, int gq,
                                                  const int32_t *cterm, const uint8_t *lutl, uint8_t *stage = nullptr,
                                                  int quarter_stride = 4 * T) {
     static_assert(!STAGED || (!PLAIN && staged_store_built(T)), "staged stores move four channel tiles at a time");
+    static_assert(!MAGIC || PLAIN, "the magic-bias form exists for the option-free epilogue only");
     // (with a staging area every lane of the wave takes part in the stores, whatever it holds itself)
     const bool staged = STAGED && (a.deq || a.ep.out_mode != kOutU8);
     const bool live = p < a.m && ch0 < a.n;
@@ -409,7 +412,7 @@ __device__ __forceinline__ void igemm_store_tile(const IgemmArgs &a, const v4i (
 #pragma unroll
             for (int r = 0; r < 4; r++)
                 v[r] = OWED == kOwesAll ? add3(acc[nt][r], ct[r], nrsz) : (OWED == kOwesRows ? acc[nt][r] + nrsz : acc[nt][r]);
-            packed[nt] = requant4_u8_packed_direct(v, a.ep);
+            packed[nt] = MAGIC ? requant4_u8_packed_magic(v, a.ep) : requant4_u8_packed_direct(v, a.ep);
         }
 #pragma unroll
         for (int nt = 0; nt + 4 <= T; nt += 4)
@@ -758,7 +761,8 @@ __global__ void __launch_bounds__(kThreads, (STAGED && T >= 12) ? 2 : (((RG == 1
 // accumulator operand of the first product), so they are not copied.  One slice per pixel group is in flight ahead
 // of the products.  ROWS: the epilogue still owes -zw' * (sum of x'); false where the weights carry that term
 // (reductions of at most 32: the lanes of the upper half of the only k-step then re-read the pixel's bytes).
-template <int T, int RG, bool ROWS> __global__ void __launch_bounds__(kThreads, 4) qconv_rows_kernel(const IgemmArgs a) {
+// MAGIC: the sums start from kMagicBias on top of the channel constants and the epilogue reads them as floats.
+template <int T, int RG, bool ROWS, bool MAGIC> __global__ void __launch_bounds__(kThreads, 4) qconv_rows_kernel(const IgemmArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     int32_t *cterm = reinterpret_cast<int32_t *>(smem); // [T * 16]
     uint8_t *wlds = smem + T * 16 * sizeof(int32_t);    // [ksteps][T][1024]
@@ -775,7 +779,7 @@ template <int T, int RG, bool ROWS> __global__ void __launch_bounds__(kThreads, 
     static_assert(T * 16 <= kThreads, "one constant per thread");
     if ((int)threadIdx.x < T * 16) {
         const int ch = ch_base + threadIdx.x;
-        cterm[threadIdx.x] = ch < a.n ? a.bias[ch] - a.zxp * a.wsum[ch] + a.k * a.zxp * a.zwp : 0;
+        cterm[threadIdx.x] = (ch < a.n ? a.bias[ch] - a.zxp * a.wsum[ch] + a.k * a.zxp * a.zwp : 0) + (MAGIC ? kMagicBias : 0);
     }
     {
         const u32x4 *src = reinterpret_cast<const u32x4 *>(a.wpk + (size_t)chunk * KS * T * 1024);
@@ -876,7 +880,7 @@ template <int T, int RG, bool ROWS> __global__ void __launch_bounds__(kThreads, 
         }
 #pragma unroll
         for (int rg = 0; rg < RG; rg++)
-            igemm_store_tile<T, ROWS ? kOwesRows : kOwesNothing, true>(a, acc[rg], ROWS ? rs[rg][0] : 0,
+            igemm_store_tile<T, ROWS ? kOwesRows : kOwesNothing, true, false, MAGIC>(a, acc[rg], ROWS ? rs[rg][0] : 0,
                                                                         mt * pix_per_block + (wave * RG + rg) * 16 + j, ch0, gq, cterm, nullptr);
 #pragma unroll
         for (int rg = 0; rg < RG; rg++) poff[rg] = poff_next[rg];
@@ -898,7 +902,8 @@ struct WindowSlice {
     uint32_t fill; // 0 where raw holds the data
 };
 
-template <int T, int RG, bool PLAIN> __global__ void __launch_bounds__(kThreads, 4) qconv_window_kernel(const IgemmArgs a) {
+template <int T, int RG, bool PLAIN, bool MAGIC = false> __global__ void __launch_bounds__(kThreads, 4) qconv_window_kernel(const IgemmArgs a) {
+    static_assert(!MAGIC || PLAIN, "the magic-bias form exists for the option-free epilogue only");
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     int32_t *cterm = reinterpret_cast<int32_t *>(smem);    // [T * 16]
     uint8_t *lutl = smem + T * 16 * sizeof(int32_t);       // [256]
@@ -916,7 +921,7 @@ template <int T, int RG, bool PLAIN> __global__ void __launch_bounds__(kThreads,
     static_assert(T * 16 <= kThreads, "one constant per thread");
     if ((int)threadIdx.x < T * 16) {
         const int ch = ch_base + threadIdx.x;
-        cterm[threadIdx.x] = ch < a.n ? a.bias[ch] - a.zxp * a.wsum[ch] + a.k * a.zxp * a.zwp : 0;
+        cterm[threadIdx.x] = (ch < a.n ? a.bias[ch] - a.zxp * a.wsum[ch] + a.k * a.zxp * a.zwp : 0) + (MAGIC ? kMagicBias : 0);
     }
     if (!PLAIN && a.lut && threadIdx.x < 64) reinterpret_cast<uint32_t *>(lutl)[threadIdx.x] = a.lut[threadIdx.x];
     for (int e = threadIdx.x; e < KS * 4; e += kThreads) {
@@ -1052,7 +1057,7 @@ template <int T, int RG, bool PLAIN> __global__ void __launch_bounds__(kThreads,
         }
 #pragma unroll
         for (int rg = 0; rg < RG; rg++)
-            igemm_store_tile<T, kOwesRows, PLAIN>(a, acc[rg], rs[rg][0], mt * pix_per_block + (wave * RG + rg) * 16 + j, ch0, gq, cterm, lutl);
+            igemm_store_tile<T, kOwesRows, PLAIN, false, MAGIC>(a, acc[rg], rs[rg][0], mt * pix_per_block + (wave * RG + rg) * 16 + j, ch0, gq, cterm, lutl);
 #pragma unroll
         for (int rg = 0; rg < RG; rg++) org[rg] = org_next[rg];
     }
@@ -1094,7 +1099,8 @@ template <int T, int RG, int MODE> int launch_trg(nncase_hip_ctx *ctx, const Ige
         // the whole chunk's weights resident and no folded reduction: the kernel with the tap table
         const size_t lds_win = (size_t)T * 16 * sizeof(int32_t) + 256 + (size_t)a.ksteps * 4 * sizeof(v4i) + (size_t)a.ksteps * T * 1024;
         if (a.kc_steps >= a.ksteps && a.kc_mask == -1 && lds_win <= 65536) {
-            if (plain) hipLaunchKernelGGL((qconv_window_kernel<T, RG, true>), dim3(gx, nchunks, 1), dim3(kThreads), lds_win, ctx->stream, args);
+            if (plain && a.magic_ok) hipLaunchKernelGGL((qconv_window_kernel<T, RG, true, true>), dim3(gx, nchunks, 1), dim3(kThreads), lds_win, ctx->stream, args);
+            else if (plain) hipLaunchKernelGGL((qconv_window_kernel<T, RG, true>), dim3(gx, nchunks, 1), dim3(kThreads), lds_win, ctx->stream, args);
             else hipLaunchKernelGGL((qconv_window_kernel<T, RG, false>), dim3(gx, nchunks, 1), dim3(kThreads), lds_win, ctx->stream, args);
             NNHIP_LAUNCH_CHECK(ctx, "qconv_window_kernel");
             return 0;
@@ -1106,8 +1112,13 @@ template <int T, int RG, int MODE> int launch_trg(nncase_hip_ctx *ctx, const Ige
             // the whole chunk's weights resident, rows of at least 16 bytes: the lean kernel
             if (a.kc_steps >= a.ksteps) {
                 const size_t lds_rows = (size_t)T * 16 * sizeof(int32_t) + (size_t)a.ksteps * T * 1024;
-                if (a.zwp_rows != 0) hipLaunchKernelGGL((qconv_rows_kernel<T, RG, true>), dim3(gx, nchunks, 1), dim3(kThreads), lds_rows, ctx->stream, args);
-                else hipLaunchKernelGGL((qconv_rows_kernel<T, RG, false>), dim3(gx, nchunks, 1), dim3(kThreads), lds_rows, ctx->stream, args);
+                if (a.magic_ok) {
+                    if (a.zwp_rows != 0) hipLaunchKernelGGL((qconv_rows_kernel<T, RG, true, true>), dim3(gx, nchunks, 1), dim3(kThreads), lds_rows, ctx->stream, args);
+                    else hipLaunchKernelGGL((qconv_rows_kernel<T, RG, false, true>), dim3(gx, nchunks, 1), dim3(kThreads), lds_rows, ctx->stream, args);
+                } else {
+                    if (a.zwp_rows != 0) hipLaunchKernelGGL((qconv_rows_kernel<T, RG, true, false>), dim3(gx, nchunks, 1), dim3(kThreads), lds_rows, ctx->stream, args);
+                    else hipLaunchKernelGGL((qconv_rows_kernel<T, RG, false, false>), dim3(gx, nchunks, 1), dim3(kThreads), lds_rows, ctx->stream, args);
+                }
                 NNHIP_LAUNCH_CHECK(ctx, "qconv_rows_kernel");
                 return 0;
             }

@@ -109,6 +109,8 @@ SYMBOLS = {
     "nncase_hip_qconv2d": (_I, [_VP, _VP, _VP, _VP, C.POINTER(Conv2dArgs)]),
     "nncase_hip_requant_plan": (_I, [C.c_float, C.c_float, QuantParam, C.c_float, C.c_float, C.POINTER(C.c_float), C.POINTER(C.c_float)]),
     "nncase_hip_requant_host": (_I, [C.c_float, C.c_float, QuantParam, C.c_float, C.c_float, _VP, _SZ, _VP, _I32P]),
+    "nncase_hip_requant_host_magic": (_I, [C.c_float, C.c_float, QuantParam, C.c_float, C.c_float, _VP, _SZ, _VP, C.POINTER(C.c_float),
+                                           C.POINTER(C.c_float), _I32P]),
     "nncase_hip_qblock_supported": (_I, [C.POINTER(QBlockDesc)]),
     "nncase_hip_qblock_prepack": (_I, [_VP, C.POINTER(QBlockDesc), _VP, _VP, _VP, _VP, _VP, _VP, C.POINTER(_VP)]),
     "nncase_hip_qblock_destroy": (_I, [_VP, _VP]),
@@ -257,6 +259,19 @@ def requant_host(acc: np.ndarray, sx, sw, y_qp: "QuantParam", clamp=(-FLT_MAX, F
     if rc != 0:
         raise HipError(rc, "requant_host", "scales outside the supported range")
     return out, form.value
+
+
+def requant_host_magic(acc: np.ndarray, sx, sw, y_qp: "QuantParam", clamp=(-FLT_MAX, FLT_MAX)):
+    """(bytes, m1, m2, limit) by the conversion-free form RN(fma(as_float(0x4B400000 + acc), m1, m2)) that the dense row /
+    window kernels and the stride-2 depthwise kernel use where the library's search found one, or None."""
+    acc = np.ascontiguousarray(acc, np.int32)
+    out = np.empty(acc.shape, np.uint8)
+    m1, m2, limit = C.c_float(), C.c_float(), C.c_int32()
+    rc = load_library().nncase_hip_requant_host_magic(float(sx), float(sw), y_qp, clamp[0], clamp[1], acc.ctypes.data, acc.size,
+                                                      out.ctypes.data, C.byref(m1), C.byref(m2), C.byref(limit))
+    if rc < 0:
+        raise HipError(rc, "requant_host_magic", "scales outside the supported range")
+    return (out, m1.value, m2.value, limit.value) if rc else None
 
 
 def _concat_args(inputs, channels, in_qps):

@@ -11,9 +11,9 @@ from __future__ import annotations
 import numpy as np
 
 
-def w8a16_linear(a_f16, q_i8, scale_f32, bias_f32=None):
-    """out[m, n] = scale[n] * sum_k a[m, k] * q[n, k] (+ bias[n])."""
-    y = a_f16.astype(np.float64) @ q_i8.astype(np.float64).T * scale_f32.astype(np.float64)[None, :]
+def w8a16_linear(a_f16, q_i8, scale_f32, bias_f32=None, acc=np.float64):
+    """out[m, n] = scale[n] * sum_k a[m, k] * q[n, k] (+ bias[n]); `acc`: the type the sums are formed in."""
+    y = (a_f16.astype(acc) @ q_i8.astype(acc).T).astype(np.float64) * scale_f32.astype(np.float64)[None, :]
     return y if bias_f32 is None else y + bias_f32.astype(np.float64)[None, :]
 
 
@@ -42,17 +42,20 @@ def f16(x):
     return np.asarray(x, np.float64).astype(np.float16).astype(np.float64)
 
 
-def decode_step(cfg, weights, tokens, block_table, ctx_lens, k_caches, v_caches):
+def decode_step(cfg, weights, tokens, block_table, ctx_lens, k_caches, v_caches, acc=np.float64):
     """One greedy decode step in float64 with fp16 rounding wherever the device stores fp16.
     k_caches / v_caches (lists of numpy fp16 arrays in the paged layouts, K [blocks, Hkv, block, d],
-    V [blocks, Hkv, d, block]) are updated in place.  Returns (next tokens, logits float64)."""
+    V [blocks, Hkv, d, block]) are updated in place.  Returns (next tokens, logits float64).
+    acc=np.float32 forms the sums of the weight products in float32 instead (numpy's blocked order): a second valid
+    evaluation, whose distance from the float64 one shows how far fp16 storage lets two correct implementations drift
+    apart over the layers (a sum that differs in its last bits can round to the other fp16 neighbour)."""
     c = cfg
     B = len(tokens)
     G = c.q_heads // c.kv_heads
     x = weights["embedding"][np.asarray(tokens)].astype(np.float64)
     for li, lw in enumerate(weights["layers"]):
         n = f16(rmsnorm(x, lw["ln1"], c.rms_eps))
-        qkv = f16(w8a16_linear(n.astype(np.float16), lw["qkv"][0], lw["qkv"][1], lw["qkv_bias"]))
+        qkv = f16(w8a16_linear(n.astype(np.float16), lw["qkv"][0], lw["qkv"][1], lw["qkv_bias"], acc=acc))
         att = np.zeros((B, c.q_heads * c.head_dim))
         for b in range(B):
             pos = int(ctx_lens[b])
@@ -72,11 +75,11 @@ def decode_step(cfg, weights, tokens, block_table, ctx_lens, k_caches, v_caches)
                 p = np.exp(s - s.max())
                 att[b, h * c.head_dim:(h + 1) * c.head_dim] = (p / p.sum()) @ V[h // G]
         att = f16(att)
-        h_ = f16(x + w8a16_linear(att.astype(np.float16), *lw["o"]))
+        h_ = f16(x + w8a16_linear(att.astype(np.float16), *lw["o"], acc=acc))
         n2 = f16(rmsnorm(h_, lw["ln2"], c.rms_eps))
-        gu = w8a16_linear(n2.astype(np.float16), *lw["gate_up"])
+        gu = w8a16_linear(n2.astype(np.float16), *lw["gate_up"], acc=acc)
         act = f16(silu(gu[:, :c.mlp]) * gu[:, c.mlp:])
-        x = f16(h_ + w8a16_linear(act.astype(np.float16), *lw["down"]))
+        x = f16(h_ + w8a16_linear(act.astype(np.float16), *lw["down"], acc=acc))
     nf = f16(rmsnorm(x, weights["ln_f"], c.rms_eps))
-    logits = w8a16_linear(nf.astype(np.float16), *weights["lm_head"])
+    logits = w8a16_linear(nf.astype(np.float16), *weights["lm_head"], acc=acc)
     return logits.argmax(axis=-1).astype(np.int32), logits

@@ -52,6 +52,36 @@ def test_picked_form_equals_the_reference_sequence(sx, sw, sy, zy, clamp):
     assert np.all(np.diff(want.astype(np.int32)) >= 0) and len(np.unique(want)) >= 2     # a staircase, not a constant
 
 
+@pytest.mark.parametrize("sx,sw,sy,zy,clamp", CASES)
+def test_conversion_free_form_equals_the_reference_sequence(sx, sw, sy, zy, clamp):
+    """Where the search finds the form on sums started from 0x4B400000 (their bits read as a float), it gives the reference's
+    bytes on every accumulator of the range it vouches for: densely around every step, on random ones, and at the range's ends
+    (far beyond 2^22, where the float no longer equals 12582912 + acc but still grows with it)."""
+    rng = np.random.default_rng(int(zy) + 11)
+    acc = staircase_points(sx, sw, sy, zy, clamp, rng)
+    res = rt.requant_host_magic(acc, sx, sw, qp(zy, sy), clamp)
+    if res is None:
+        pytest.skip("no conversion-free pair for these quant params (the kernels use the other forms)")
+    got, m1, m2, limit = res
+    assert limit >= 2**29
+    acc = np.concatenate([acc[np.abs(acc.astype(np.int64)) <= limit], np.array([-limit, -limit + 1, -2**22 - 1, -2**22, 2**22 - 1, 2**22, limit - 1, limit], np.int32)])
+    got = rt.requant_host_magic(acc, sx, sw, qp(zy, sy), clamp)[0]
+    want = O.requant_u8(acc, sx, sw, sy, zy, clamp)
+    bad = got != want
+    assert not bad.any(), f"{bad.sum()} of {acc.size} differ, first at acc={acc[bad][0]}: {got[bad][0]} vs {want[bad][0]}"
+    # what the pair is: m1 with two spare mantissa bits, m2 = zy - 12582912 * m1 without rounding
+    assert (np.array([m1], f32).view(np.uint32)[0] & 3) == 0
+    assert float(f32(m2)) == float(zy) - 12582912.0 * float(f32(m1))
+
+
+def test_conversion_free_form_exists_for_the_layers_it_is_meant_for():
+    # a ReLU6 expansion, a linear projection and a depthwise layer of MobileNetV2 (calibrated scales)
+    found = [rt.requant_host_magic(np.zeros(1, np.int32), sx, sw, qp(zy, sy), clamp) is not None
+             for sx, sw, sy, zy, clamp in ((0.0235, 0.0041, 0.0118965, 0, (0.0, 6.0)), (0.0192766, 0.0067, 0.0180625, 135, FULL),
+                                           (0.0235294, 0.0125, 0.0235294, 0, (0.0, 6.0)), (0.02, 0.011, 0.0235, 0, (0.0, 6.0)))]
+    assert sum(found) >= 2, found
+
+
 def test_fma_form_is_found_for_typical_layers_and_is_what_it_says():
     found, c1, c2 = rt.requant_plan(0.0235, 0.0041, qp(0, 0.0118965), (0.0, 6.0))
     assert found and abs(c1 / (float(f32(0.0235) * f32(0.0041)) / 0.0118965) - 1) < 1e-5 and abs(c2) < 1e-3
