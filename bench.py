@@ -38,7 +38,11 @@ INT8_PEAK_TOPS = 5000.0    # dense int8 MFMA
 # launches one after the other (--lanes 1 --in-flight 1), from two rocprofv3 --pmc runs
 # of this script (FETCH_SIZE, then WRITE_SIZE, each scaled by what the same counter reads for the 256 MiB
 # copy that --copy-probe launches: x1.9996 and x1.0000).  Counters cannot be read from inside a timed run, so the figures
-# are recorded here and reported only for the configuration they were measured on.
+# are recorded here and reported only for the configuration they were measured on: the bench line names the profile
+# summary they come from, and reports no traffic at all when the kernels a run launches are not exactly the ones of
+# the table (a kernel selection that has changed since the profile was taken).
+MEASURED_TRAFFIC_SOURCE = {"unfused": "profiles/mobilenetv2_b64_kernels_counters.txt",
+                           "fused": "profiles/mobilenetv2_b64_fused_blocks_kernels_counters.txt"}
 MEASURED_TRAFFIC_B64 = {
     "unfused": {
         "dw3x3<S=1>": 19028851,
@@ -437,12 +441,20 @@ def main():
     def family(name):
         return name.split("<")[0].split("+")[0]
 
+    table_key = "fused" if args.fuse_blocks else "unfused"
+    table = MEASURED_TRAFFIC_B64[table_key]
+    live, recorded = set(groups), set(table)
+    traffic_source = {"profile": MEASURED_TRAFFIC_SOURCE[table_key], "kernels_in_profile": sorted(recorded),
+                      "matches_this_run": args.batch == 64 and live == recorded}
+    if live != recorded:
+        traffic_source["launched_but_not_profiled"] = sorted(live - recorded)
+        traffic_source["profiled_but_not_launched"] = sorted(recorded - live)
     fams = {}
     for name, g in groups.items():
         f = fams.setdefault(family(name), {"ms": 0.0, "bytes": 0, "floor": 0, "macs": 0, "launches": 0, "traffic": 0, "traffic_known": True})
         for k in ("ms", "bytes", "floor", "macs", "launches"):
             f[k] += g[k]
-        t = MEASURED_TRAFFIC_B64["fused" if args.fuse_blocks else "unfused"].get(name) if args.batch == 64 else None
+        t = table.get(name) if traffic_source["matches_this_run"] else None
         if t is None:
             f["traffic_known"] = False
         else:
@@ -545,7 +557,10 @@ def main():
                                  "consecutive steps overlap on the device; step_ms is one step at a time" if args.in_flight > 1 else "")},
         "roofline": roofline_of(dom_name, dom),
         "rooflines_by_family": [roofline_of(n, f) for n, f in ranked[:5]],
+        "traffic_source": traffic_source,
         "step_ms": spread,
+        # the other view of the same function: one request at a time on an idle device (value has --in-flight requests overlapping)
+        "one_request_at_a_time": {"images_per_s": round(args.batch / (spread["avg"] * 1e-3), 1), "ms_per_step": spread["avg"]},
         "cpu_baseline": cpu,
         "int8_TOPS_whole_net": round(2 * total_macs / (ms_per_step * 1e-3) / 1e12, 2),
         "hbm_GBps_whole_net": round(sum(fbytes) / (ms_per_step * 1e-3) / 1e9, 1),

@@ -85,6 +85,11 @@ NNCASE_HIP_API int nncase_hip_ctx_destroy(nncase_hip_ctx_t *ctx);
  * the first GPU_MAX_HW_QUEUES of them.  Returns the number of hardware queues (> 0) or a negative status.
  * (No counterpart in the reference, whose interpreters are CPU threads.) */
 NNCASE_HIP_API int nncase_hip_fill_queue_pool(int device);
+/* Destroys the idle streams nncase_hip_fill_queue_pool created on `device` (for a host that unloads the library or
+ * is done with overlapping requests); contexts created afterwards share hardware queues as HIP deals them out.
+ * Returns the number of streams destroyed (0: the pool was not filled), or a negative status.  No counterpart in
+ * the reference (its CPU runtime has no queues). */
+NNCASE_HIP_API int nncase_hip_release_queue_pool(int device);
 
 /* The hipStream_t the context enqueues on (so a caller can record events on
  * it), and a way to make the context use a caller-owned stream instead. */

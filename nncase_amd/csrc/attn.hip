@@ -322,8 +322,9 @@ constexpr size_t kScratchCounterBytes = 64u << 10;  // 16384 (sequence, kv head)
 constexpr size_t kScratchPartialBytes = 8u << 20;   // batch * query heads * splits * (head_dim + 2) floats
 static __device__ __align__(256) unsigned char scratch[kScratchCounterBytes + kScratchPartialBytes];
 
-constexpr int kMaxDevices = 64;
-static void *g_scratch_ptr[kMaxDevices] = {nullptr}; // device address of `scratch` on each GPU (hipGetSymbolAddress)
+// Every GPU holds its own copy of the array at its own address: a context takes the address of its device's copy when
+// it is created (ctx.hip) and the entry point uses that pointer, never the array's name.
+hipError_t attn_static_scratch_address(void **ptr) { return hipGetSymbolAddress(ptr, HIP_SYMBOL(scratch)); }
 
 // Everything a launch needs except the buffers: checked geometry, split plan, sizes of the scratch areas.
 struct AttnPlan {
@@ -487,16 +488,8 @@ extern "C" int nncase_hip_paged_attention_decode_noalloc(nncase_hip_ctx_t *ctx, 
                   "paged_attention_decode_noalloc: needs %zu bytes of split partials and %zu of counters; the static "
                   "scratch holds %zu and %zu (use nncase_hip_paged_attention_decode)",
                   plan.partial_bytes, plan.counter_bytes, kScratchPartialBytes, kScratchCounterBytes);
-    NNHIP_REQUIRE(ctx, ctx->device >= 0 && ctx->device < kMaxDevices, -ENODEV, "paged_attention_decode_noalloc: device %d",
-                  ctx->device);
-    if (!g_scratch_ptr[ctx->device]) { // first call on this GPU: every GPU has its own copy at its own address
-        NNHIP_HIP(ctx, hipSetDevice(ctx->device));
-        void *ptr = nullptr;
-        NNHIP_HIP(ctx, hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
-        NNHIP_REQUIRE(ctx, ptr, -ENOMEM, "paged_attention_decode_noalloc: no address for the static scratch");
-        g_scratch_ptr[ctx->device] = ptr;
-    }
-    unsigned char *base = reinterpret_cast<unsigned char *>(g_scratch_ptr[ctx->device]);
+    NNHIP_REQUIRE(ctx, ctx->attn_static, -ENOMEM, "paged_attention_decode_noalloc: the context has no address for the static scratch");
+    unsigned char *base = reinterpret_cast<unsigned char *>(ctx->attn_static);
     // The array keeps the previous call's contents: the counters this launch uses must start at zero.
     hipLaunchKernelGGL(attn_zero_u32_kernel, dim3(1), dim3(256), 0, ctx->stream, (uint32_t *)base, plan.counter_bytes / 4);
     NNHIP_LAUNCH_CHECK(ctx, "attn_zero_u32_kernel");

@@ -28,10 +28,17 @@ struct nncase_hip_ctx {
     void *attn_done = nullptr; // counters live apart from the partials: they must stay zero between calls
     size_t attn_done_bytes = 0;
     int attn_pins = 0;
+    // this GPU's copy of the static scratch of nncase_hip_paged_attention_decode_noalloc (its device address, taken
+    // when the context is created so that the entry point itself makes no runtime call but launches)
+    void *attn_static = nullptr;
     char last_error[512] = {0};
 };
 
 namespace nnhip {
+
+// Device address of the static scratch array of the attention entry point that allocates nothing, on `device`
+// (which must be current).  attn.hip, where the array lives.
+hipError_t attn_static_scratch_address(void **ptr);
 
 inline int fail(nncase_hip_ctx *ctx, int code, const char *fmt, ...) {
     if (ctx) {

@@ -32,34 +32,61 @@ extern "C" int nncase_hip_ctx_create(int device, nncase_hip_ctx_t **out) {
         return -(NNCASE_HIP_ERR_HIP_BASE + (int)e);
     }
     ctx->owns_stream = true;
+    e = nnhip::attn_static_scratch_address(&ctx->attn_static); // (the device is current)
+    if (e != hipSuccess || !ctx->attn_static) {
+        (void)hipStreamDestroy(ctx->stream);
+        delete ctx;
+        return e != hipSuccess ? -(NNCASE_HIP_ERR_HIP_BASE + (int)e) : -ENOMEM;
+    }
     *out = ctx;
     return 0;
 }
 
 // HIP multiplexes streams over at most GPU_MAX_HW_QUEUES hardware queues (4 unless the environment says otherwise): a
 // new stream opens a new queue until that many exist and joins the least shared one after that, and kernels of streams
-// that share a queue run one after the other.  Idle streams created here, once per device and kept until the process
-// ends, fill the pool, so that the streams of the contexts created afterwards are dealt out one per queue in turn.
+// that share a queue run one after the other.  Idle streams created here, once per device, fill the pool, so that the
+// streams of the contexts created afterwards are dealt out one per queue in turn.  They are kept until
+// nncase_hip_release_queue_pool destroys them (a host that unloads the library) or the process ends.
+namespace {
+constexpr int kPoolMaxDevices = 64, kPoolMaxQueues = 32;
+std::mutex g_pool_lock;
+int g_pool_filled[kPoolMaxDevices] = {0};
+hipStream_t g_pool_streams[kPoolMaxDevices][kPoolMaxQueues] = {};
+} // namespace
+
 extern "C" int nncase_hip_fill_queue_pool(int device) {
-    constexpr int kMaxDevices = 64, kMaxQueues = 32;
-    static std::mutex lock;
-    static int filled[kMaxDevices] = {0};
     int count = 0;
-    if (hipGetDeviceCount(&count) != hipSuccess || device < 0 || device >= count || device >= kMaxDevices) return -ENODEV;
-    std::lock_guard<std::mutex> guard(lock);
-    if (filled[device]) return filled[device];
+    if (hipGetDeviceCount(&count) != hipSuccess || device < 0 || device >= count || device >= kPoolMaxDevices) return -ENODEV;
+    std::lock_guard<std::mutex> guard(g_pool_lock);
+    if (g_pool_filled[device]) return g_pool_filled[device];
     int queues = 4;
     if (const char *env = getenv("GPU_MAX_HW_QUEUES")) {
         const int v = atoi(env);
-        if (v >= 1 && v <= kMaxQueues) queues = v;
+        if (v >= 1 && v <= kPoolMaxQueues) queues = v;
     }
     if (hipSetDevice(device) != hipSuccess) return -ENODEV;
     for (int i = 0; i < queues; i++) {
-        hipStream_t idle;
-        const hipError_t e = hipStreamCreateWithFlags(&idle, hipStreamNonBlocking);
-        if (e != hipSuccess) return -(NNCASE_HIP_ERR_HIP_BASE + (int)e);
+        const hipError_t e = hipStreamCreateWithFlags(&g_pool_streams[device][i], hipStreamNonBlocking);
+        if (e != hipSuccess) {
+            for (int j = 0; j < i; j++) (void)hipStreamDestroy(g_pool_streams[device][j]);
+            return -(NNCASE_HIP_ERR_HIP_BASE + (int)e);
+        }
     }
-    filled[device] = queues;
+    g_pool_filled[device] = queues;
+    return queues;
+}
+
+extern "C" int nncase_hip_release_queue_pool(int device) {
+    if (device < 0 || device >= kPoolMaxDevices) return -ENODEV;
+    std::lock_guard<std::mutex> guard(g_pool_lock);
+    const int queues = g_pool_filled[device];
+    if (!queues) return 0;
+    if (hipSetDevice(device) != hipSuccess) return -ENODEV;
+    for (int i = 0; i < queues; i++) {
+        (void)hipStreamDestroy(g_pool_streams[device][i]);
+        g_pool_streams[device][i] = nullptr;
+    }
+    g_pool_filled[device] = 0;
     return queues;
 }
 

@@ -16,6 +16,7 @@
 #include <hip/hip_fp16.h>
 
 #include <cmath>
+#include <mutex>
 #include <new>
 #include <vector>
 
@@ -646,6 +647,16 @@ extern "C" int nncase_hip_w8a16_prepack(nncase_hip_ctx_t *ctx, const int8_t *w_h
     return 0;
 }
 
+// A launch whose LDS (the dynamic part plus the kernel's own static arrays: `total`) passes 48 KiB asks, once per kernel
+// and device, for a dynamic limit of `limit` bytes.
+template <typename KernelT> static hipError_t raise_dynamic_lds(KernelT kernel, int device, size_t total, int limit) {
+    if (total <= 48 * 1024) return hipSuccess;
+    static std::once_flag raised[16];
+    hipError_t e = hipSuccess;
+    std::call_once(raised[device & 15], [&] { e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, limit); });
+    return e;
+}
+
 static int launch_w8a16_gemm(nncase_hip_ctx_t *ctx, const void *a_dev, const nncase_hip_w8a16_t *w, void *out_dev, int32_t m,
                              int32_t mode, const void *residual_dev, int32_t out_dtype, const void *ln_weight_dev, float ln_eps) {
     NNHIP_CHECK_CTX(ctx);
@@ -689,8 +700,14 @@ static int launch_w8a16_gemm(nncase_hip_ctx_t *ctx, const void *a_dev, const nnc
     if (split && !glu && ln_weight_dev && w->k <= kRowsMaxK && rows_lds <= 64 * 1024 && mt_built <= 2) {
         // few tiles and rows to normalise (the q / k / v projection): the reduction split over the block's waves, the
         // rows parked and normalised in LDS in one trip to memory
-        if (mt_built == 1) hipLaunchKernelGGL((w8a16_gemm_rows_in_lds_kernel<1, 1, kGemmWaves, true>), grid, block, rows_lds, ctx->stream, a);
-        else hipLaunchKernelGGL((w8a16_gemm_rows_in_lds_kernel<2, 1, kGemmWaves, true>), grid, block, rows_lds, ctx->stream, a);
+        // (the kernel's static reduction area comes on top of the rows: past 48 KiB in all, the limit is raised like below)
+        if (mt_built == 1) {
+            NNHIP_HIP(ctx, raise_dynamic_lds(w8a16_gemm_rows_in_lds_kernel<1, 1, kGemmWaves, true>, ctx->device, rows_lds + 8 * 1024, 64 * 1024));
+            hipLaunchKernelGGL((w8a16_gemm_rows_in_lds_kernel<1, 1, kGemmWaves, true>), grid, block, rows_lds, ctx->stream, a);
+        } else {
+            NNHIP_HIP(ctx, raise_dynamic_lds(w8a16_gemm_rows_in_lds_kernel<2, 1, kGemmWaves, true>, ctx->device, rows_lds + 16 * 1024, 64 * 1024));
+            hipLaunchKernelGGL((w8a16_gemm_rows_in_lds_kernel<2, 1, kGemmWaves, true>), grid, block, rows_lds, ctx->stream, a);
+        }
         NNHIP_LAUNCH_CHECK(ctx, "w8a16_gemm_rows_in_lds_kernel");
         return 0;
     }
@@ -698,12 +715,7 @@ static int launch_w8a16_gemm(nncase_hip_ctx_t *ctx, const void *a_dev, const nnc
         const dim3 rgrid((out_tiles + kGemmWaves - 1) / kGemmWaves), rblock(kGemmThreads);
 #define NNHIP_ROWS_LAUNCH(MTV, GV)                                                                                             \
     do {                                                                                                                       \
-        static int raised_on_device = -1;                                                                                      \
-        if (rows_lds > 48 * 1024 && raised_on_device != ctx->device) {                                                         \
-            NNHIP_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(&w8a16_gemm_rows_in_lds_kernel<MTV, GV, kGemmWaves>), \
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024));                      \
-            raised_on_device = ctx->device;                                                                                    \
-        }                                                                                                                      \
+        NNHIP_HIP(ctx, raise_dynamic_lds(w8a16_gemm_rows_in_lds_kernel<MTV, GV, kGemmWaves>, ctx->device, rows_lds + 1024, 128 * 1024)); \
         hipLaunchKernelGGL((w8a16_gemm_rows_in_lds_kernel<MTV, GV, kGemmWaves>), rgrid, rblock, rows_lds, ctx->stream, a);    \
     } while (0)
         if (glu) {

@@ -791,6 +791,7 @@ class HipPipeline:
         # the caller's own stream give 183 k images/s on MobileNetV2 at batch 64, one per hardware queue 224 k; six or
         # eight hardware queues instead of four give 164-180 k).  So the pool is filled with idle streams first: the
         # copies' streams then land on one hardware queue each.
+        self.device = device
         self.hw_queues = rt.fill_queue_pool(device)
         self.contexts = [Context(device) for _ in range(depth)]
         self.models = [HipModel(c, qg, batch, **model_args) for c in self.contexts]
@@ -812,3 +813,14 @@ class HipPipeline:
     def sync(self):
         for c in self.contexts:
             c.sync()
+
+    def close(self, release_queue_pool: bool = True):
+        """Waits for the copies, destroys their contexts and, unless another pipeline still wants it, the pool of idle
+        streams that spread the copies over the hardware queues."""
+        self.sync()
+        self.models = []
+        for c in self.contexts:
+            c.close()
+        self.contexts = []
+        if release_queue_pool:
+            rt.release_queue_pool(self.device)

@@ -158,6 +158,7 @@ SYMBOLS = {
     "nncase_hip_kmodel_function": (_I, [_VP, C.POINTER(_VP)]),
     "nncase_hip_kmodel_tensor": (_I, [_VP, C.c_int32, C.POINTER(_VP), _I32P, _I32P]),
     "nncase_hip_fill_queue_pool": (_I, [C.c_int]),
+    "nncase_hip_release_queue_pool": (_I, [C.c_int]),
     "nncase_hip_pack": (_I, [_VP, _VP, _VP, C.c_int32, C.c_int32, _I32P, C.c_int32, _I32P, _I32P]),
     "nncase_hip_unpack": (_I, [_VP, _VP, _VP, C.c_int32, C.c_int32, _I32P, C.c_int32, _I32P, _I32P]),
     "nncase_hip_quantize_pack": (_I, [_VP, _VP, _VP, C.c_int32, _I32P, C.c_int32, _I32P, _I32P, QuantParam]),
@@ -216,6 +217,14 @@ def fill_queue_pool(device: int = 0) -> int:
     rc = load_library().nncase_hip_fill_queue_pool(device)
     if rc <= 0:
         raise HipError(rc, "fill_queue_pool")
+    return rc
+
+
+def release_queue_pool(device: int = 0) -> int:
+    """Destroys the idle streams fill_queue_pool created on the device; returns how many there were."""
+    rc = load_library().nncase_hip_release_queue_pool(device)
+    if rc < 0:
+        raise HipError(rc, "release_queue_pool")
     return rc
 
 

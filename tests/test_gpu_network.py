@@ -6,6 +6,7 @@ import numpy as np
 import pytest
 
 from nncase_amd import netbuilder as nb
+from nncase_amd import runtime as rt
 from oracle import netref
 from oracle import oracle as O
 
@@ -299,6 +300,17 @@ def test_copies_in_flight_give_the_bytes_of_one_function(hip_ctx):
         assert np.array_equal(m.output().view(np.uint32), y.view(np.uint32))
     with pytest.raises(ValueError):
         nb.HipPipeline(0, qg, 8, depth=0)
+    # the idle streams that spread the copies over the hardware queues go with the pipeline; a later one fills the pool again
+    queues = pipe.hw_queues
+    pipe.close()
+    assert rt.release_queue_pool(0) == 0                      # already released
+    again = nb.HipPipeline(0, qg, 8, depth=2, capture_graph=False)
+    assert again.hw_queues == queues
+    again.models[0].set_input(xs[0])
+    again.submit()
+    again.sync()
+    assert np.array_equal(again.models[0].output().view(np.uint32), want[0].view(np.uint32))
+    again.close()
 
 
 def test_lanes_yolov5s_outputs(hip_ctx):

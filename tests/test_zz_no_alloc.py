@@ -63,3 +63,54 @@ def test_noalloc_refuses_what_its_scratch_cannot_hold(hip_ctx):
     with pytest.raises(rt.HipError) as e:
         hip_ctx.paged_attention_decode_noalloc(dq, dk, dv, dbt, dcl, dout, args)
     assert e.value.code == -errno.ENOSPC
+
+
+def test_noalloc_call_recorded_into_a_hip_graph_replays_correctly(hip_ctx):
+    """The entry point is meant for code under HIP graph capture: its first call on a context may be the captured one (the
+    scratch address was taken when the context was created, so the call itself only launches).  The graph is replayed
+    three times, with eager work and synchronisations of the same context in between, and every replay gives the bytes of
+    the eager call (the counters are cleared by a kernel inside the graph, not by a memset node)."""
+    import ctypes as C
+    hip = C.CDLL("libamdhip64.so")
+    ctx = rt.Context(0)                                      # a context whose first attention call is the captured one
+    rng = np.random.default_rng(77)
+    q, kc, vt, bt, cl = _case(rng, 5, 14, 2, 64, 16, 2048, [2048, 1500, 17, 600, 1025])
+    bsz, hq, d = q.shape
+    nb, hkv, blk, _ = kc.shape
+    dq, dk, dv, dbt, dcl = (ctx.to_device(t) for t in (q, kc, vt, bt, cl))
+    args = rt.PagedAttnArgs(bsz, hq, hkv, d, blk, bt.shape[1], nb, float(d ** -0.5), rt.DT_F32)
+    dout = ctx.alloc(bsz * hq * d * 4).fill(0xEE)
+    stream = C.c_void_p(ctx.stream)
+    graph, gexec = C.c_void_p(), C.c_void_p()
+    hip.hipStreamBeginCapture.argtypes = [C.c_void_p, C.c_int]
+    hip.hipStreamEndCapture.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+    hip.hipGraphInstantiate.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]
+    hip.hipGraphLaunch.argtypes = [C.c_void_p, C.c_void_p]
+    hip.hipGraphExecDestroy.argtypes = [C.c_void_p]
+    hip.hipGraphDestroy.argtypes = [C.c_void_p]
+    assert hip.hipStreamBeginCapture(stream, 2) == 0         # hipStreamCaptureModeRelaxed
+    try:
+        ctx.paged_attention_decode_noalloc(dq, dk, dv, dbt, dcl, dout, args)
+    finally:
+        rc = hip.hipStreamEndCapture(stream, C.byref(graph))
+    assert rc == 0 and graph.value
+    assert hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0) == 0
+    want_out = ctx.alloc(bsz * hq * d * 4).fill(0x11)
+    ctx.paged_attention_decode(dq, dk, dv, dbt, dcl, want_out, args)   # eager, allocating entry point
+    ctx.sync()
+    want = want_out.download((bsz, hq, d), np.float32)
+    for replay in range(3):
+        dout.fill(0xEE)
+        ctx.sync()
+        assert hip.hipGraphLaunch(gexec, stream) == 0
+        ctx.sync()
+        got = dout.download((bsz, hq, d), np.float32)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), f"replay {replay}"
+        # eager work of the same context between the replays (it uses the same static scratch)
+        other = ctx.alloc(bsz * hq * d * 4)
+        ctx.paged_attention_decode_noalloc(dq, dk, dv, dbt, dcl, other, args)
+        ctx.sync()
+        assert np.array_equal(other.download((bsz, hq, d), np.float32).view(np.uint32), want.view(np.uint32))
+    hip.hipGraphExecDestroy(gexec)
+    hip.hipGraphDestroy(graph)
+    ctx.close()
