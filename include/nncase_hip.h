@@ -556,6 +556,12 @@ NNCASE_HIP_API int nncase_hip_function_add_resize_nearest(nncase_hip_function_t 
                                                           int32_t elem_size, int32_t batch, int32_t in_h, int32_t in_w,
                                                           int32_t channels, int32_t out_h, int32_t out_w,
                                                           int32_t transformation_mode, int32_t nearest_mode);
+/* NCHW <-> NHWC relayout as a step of a function (nncase_hip_nchw_to_nhwc / nncase_hip_nhwc_to_nchw with the same
+ * extents): the IR holds activations as NCHW, a hip function works channels-last, so a compiled function converts at
+ * its two ends (the Transpose pair around NHWC imports, src/Nncase.Importer/TFLite/Conv2D.cs:28-29,67). */
+NNCASE_HIP_API int nncase_hip_function_add_layout(nncase_hip_function_t *fn, const void *in_dev, void *out_dev,
+                                                  int32_t elem_size, int32_t n, int32_t c, int32_t h, int32_t w,
+                                                  int32_t to_nchw);
 NNCASE_HIP_API int nncase_hip_function_add_qmaxpool2d(nncase_hip_function_t *fn, const uint8_t *x_dev, uint8_t *out_dev,
                                                       int32_t batch, int32_t in_h, int32_t in_w, int32_t channels,
                                                       int32_t kernel_h, int32_t kernel_w, int32_t stride_h, int32_t stride_w,

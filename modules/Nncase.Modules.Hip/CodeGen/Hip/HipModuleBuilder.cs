@@ -9,11 +9,10 @@
 //   tensor  32 B : u32 typecode, rank (= 4), dims[4] as N, H, W, C; i32 zero_point; f32 scale
 //   op     144 B : u32 opcode, n_inputs; i32 inputs[8] (tensor indices, -1 = unused); i32 output; u32 reserved;
 //                  u64 rdata0, rdata1 (byte offsets into .rdata, all ones = none); i32 p[16]; f32 f[4]
-// Opcodes: 0 quantize, 1 dequantize, 2 conv2d, 3 add, 4 global_avgpool, 5 lut, 6 concat, 7 resize_nearest,
-// 8 maxpool, 9 pad_channels, 10 reshape (the output tensor is the input's buffer under other extents).  conv2d: rdata0 = weights (OIHW u8), rdata1 = bias (int32 per output channel);
-// p = {out_channels, in_channels / groups, kernel_h, kernel_w, groups, stride_h, stride_w, dilation_h,
-// dilation_w, pad_h_before, pad_h_after, pad_w_before, pad_w_after, weights zero point};
-// f = {clamp_min, clamp_max, weights scale}.  A matmul is a 1x1 conv2d over [M, 1, 1, K].
+// What p, f and the rdata offsets of each opcode hold is the table HipOpLayouts below.  A matmul is a 1x1 conv2d
+// over [M, 1, 1, K].  The IR holds activations as NCHW and the kernels run channels-last: the function starts
+// with a layout record (NCHW -> NHWC) on its input and ends with one (NHWC -> NCHW) per output, left out where
+// the two orders are the same bytes (rank 2, one channel, or a 1 x 1 image).
 using System;
 using System.Collections.Generic;
 using System.IO;
@@ -48,6 +47,30 @@ internal enum HipOpcode : uint
     MaxPool = 8,
     PadChannels = 9,
     Reshape = 10,
+    Layout = 11,
+}
+
+/// <summary>Names of the p[] and f[] fields and the number of .rdata offsets of every opcode, in record order.</summary>
+internal static class HipOpLayouts
+{
+    public static readonly IReadOnlyDictionary<HipOpcode, (string[] P, string[] F, int Rdata)> Fields = new Dictionary<HipOpcode, (string[] P, string[] F, int Rdata)>
+    {
+        [HipOpcode.Quantize] = (new string[0], new string[0], 0),
+        [HipOpcode.Dequantize] = (new string[0], new string[0], 0),
+        [HipOpcode.Conv2D] = (
+            new[] { "out_channels", "group_in_channels", "kernel_h", "kernel_w", "groups", "stride_h", "stride_w", "dilation_h", "dilation_w", "pad_h_before", "pad_h_after", "pad_w_before", "pad_w_after", "weights_zero_point" },
+            new[] { "clamp_min", "clamp_max", "weights_scale" },
+            2),
+        [HipOpcode.Add] = (new string[0], new[] { "clamp_min", "clamp_max" }, 0),
+        [HipOpcode.GlobalAvgPool] = (new string[0], new string[0], 0),
+        [HipOpcode.Lut] = (new string[0], new string[0], 1),
+        [HipOpcode.Concat] = (new string[0], new string[0], 0),
+        [HipOpcode.ResizeNearest] = (new[] { "transformation_mode", "nearest_mode" }, new string[0], 0),
+        [HipOpcode.MaxPool] = (new[] { "kernel", "stride", "padding" }, new string[0], 0),
+        [HipOpcode.PadChannels] = (new string[0], new string[0], 0),
+        [HipOpcode.Reshape] = (new string[0], new string[0], 0),
+        [HipOpcode.Layout] = (new[] { "to_nchw" }, new string[0], 0),
+    };
 }
 
 internal sealed class HipFunctionBuilder : FunctionBuilder
@@ -58,10 +81,13 @@ internal sealed class HipFunctionBuilder : FunctionBuilder
     public const int OpBytes = 144;
     public const int RdataAlignment = 64;
     private const ulong NoRdata = ulong.MaxValue;
+    private const int HipConcatLimit = 8; // tensor indices in one operator record
 
     private readonly List<TensorRecord> _tensors = new();
     private readonly List<OpRecord> _ops = new();
+    private readonly Dictionary<uint, uint> _layoutTwin = new();
     private uint _output;
+    private uint _outputs = 1;
 
     public HipFunctionBuilder(uint id, SectionManager sectionManager)
         : base(id, sectionManager)
@@ -70,17 +96,33 @@ internal sealed class HipFunctionBuilder : FunctionBuilder
 
     protected override void Compile(BaseFunction callable)
     {
-        var fusion = (Fusion)callable;
-        if (fusion.Parameters.Length != 1)
+        // PrimFunction(in, out_0, ...) { HipStore(value_0, out_0); ... } as OutlineHipFunctionsPass builds it
+        var function = (TIR.PrimFunction)callable;
+        var parameters = function.Parameters.ToArray();
+        var stores = function.Body.Fields.ToArray().Select(f => (Call)f).ToArray();
+        if (parameters.Length != stores.Length + 1 || stores.Any(c => c.Target is not HipStore))
         {
-            throw new NotSupportedException("a hip function takes one activation");
+            throw new NotSupportedException("a hip function takes one activation and stores each of its outputs once");
         }
 
-        var values = new Dictionary<Expr, uint>(ReferenceEqualityComparer.Instance)
+        var values = new Dictionary<Expr, uint>(ReferenceEqualityComparer.Instance);
+        uint input = AddTensor((TensorType)parameters[0].CheckedType!);
+        values[parameters[0]] = ChannelsLast(input, toNchw: false);
+
+        var results = new List<uint>();
+        foreach (var store in stores)
         {
-            [fusion.Parameters[0]] = AddTensor((TensorType)fusion.Parameters[0].CheckedType!, default),
-        };
-        _output = Emit(fusion.Body, values);
+            uint value = Emit(store.Arguments[0], values);
+            uint result = ChannelsLast(value, toNchw: true);
+            if (result == input || results.Contains(result))
+            {
+                throw new NotSupportedException("an output of a hip function is a tensor of its own");
+            }
+
+            results.Add(result);
+        }
+
+        MoveOutputsLast(results);
     }
 
     protected override void WriteText()
@@ -92,7 +134,7 @@ internal sealed class HipFunctionBuilder : FunctionBuilder
         w.Write((uint)_ops.Count);
         w.Write(0u); // input tensor
         w.Write(_output);
-        w.Write(0u); // one output
+        w.Write(_outputs == 1 ? 0u : _outputs);
         w.Write(0u);
         foreach (var t in _tensors)
         {
@@ -103,8 +145,8 @@ internal sealed class HipFunctionBuilder : FunctionBuilder
                 w.Write((uint)d);
             }
 
-            w.Write(t.QuantParam.ZeroPoint);
-            w.Write(t.QuantParam.Scale);
+            w.Write(t.QuantParam?.ZeroPoint ?? 0);
+            w.Write(t.QuantParam?.Scale ?? 1f);
         }
 
         foreach (var o in _ops)
@@ -140,7 +182,7 @@ internal sealed class HipFunctionBuilder : FunctionBuilder
         : throw new NotSupportedException($"hip tensors are u8 or f32, not {type}");
 
     // IR tensors are NCHW (rank 4) or [rows, columns] (rank 2): recorded channels-last
-    private uint AddTensor(TensorType type, QuantParam qp)
+    private uint AddTensor(TensorType type, QuantParam? qp = null)
     {
         var d = type.Shape.ToValueArray();
         int[] nhwc = d.Length switch
@@ -149,8 +191,83 @@ internal sealed class HipFunctionBuilder : FunctionBuilder
             2 => new[] { d[0], 1, 1, d[1] },
             _ => throw new NotSupportedException($"hip tensors have rank 2 or 4, not {d.Length}"),
         };
-        _tensors.Add(new TensorRecord(TypeCode(type.DType), nhwc, qp.Scale == 0f ? new QuantParam(0, 1f) : qp));
+        return AddTensor(TypeCode(type.DType), nhwc, qp);
+    }
+
+    private uint AddTensor(uint typeCode, int[] nhwc, QuantParam? qp)
+    {
+        _tensors.Add(new TensorRecord(typeCode, nhwc, qp));
         return (uint)(_tensors.Count - 1);
+    }
+
+    // A tensor's QuantParam is known from the operator that writes it or from the first one that reads it; the
+    // two ends of a layout record share it.  Two operators that disagree describe a graph the rules should not
+    // have lowered.
+    private void SetQuantParam(uint tensor, QuantParam qp)
+    {
+        var known = _tensors[(int)tensor].QuantParam;
+        if (known is QuantParam k && (k.ZeroPoint != qp.ZeroPoint || k.Scale != qp.Scale))
+        {
+            throw new NotSupportedException($"tensor {tensor} is read as ({qp.ZeroPoint}, {qp.Scale}) but written as ({k.ZeroPoint}, {k.Scale})");
+        }
+
+        _tensors[(int)tensor] = _tensors[(int)tensor] with { QuantParam = qp };
+        if (_layoutTwin.TryGetValue(tensor, out var twin) && _tensors[(int)twin].QuantParam is null)
+        {
+            SetQuantParam(twin, qp);
+        }
+    }
+
+    // the same tensor in the other byte order, through a layout record; the tensor itself where both orders agree
+    private uint ChannelsLast(uint tensor, bool toNchw)
+    {
+        var t = _tensors[(int)tensor];
+        if (t.Nhwc[3] == 1 || t.Nhwc[1] * t.Nhwc[2] == 1)
+        {
+            return tensor;
+        }
+
+        uint other = AddTensor(t.TypeCode, t.Nhwc, t.QuantParam);
+        _layoutTwin[tensor] = other;
+        _layoutTwin[other] = tensor;
+        AddOp(HipOpcode.Layout, new[] { tensor }, other, p: new[] { toNchw ? 1 : 0 });
+        return other;
+    }
+
+    // outputs are the last tensors of the table, in the order of the function's output parameters
+    private void MoveOutputsLast(List<uint> results)
+    {
+        var order = Enumerable.Range(0, _tensors.Count).Select(i => (uint)i).Where(i => !results.Contains(i)).Concat(results).ToArray();
+        var renumber = new uint[order.Length];
+        for (uint position = 0; position < order.Length; position++)
+        {
+            renumber[order[position]] = position;
+        }
+
+        var tensors = order.Select(i => _tensors[(int)i]).ToArray();
+        _tensors.Clear();
+        _tensors.AddRange(tensors);
+        for (int i = 0; i < _ops.Count; i++)
+        {
+            _ops[i] = _ops[i] with { Inputs = _ops[i].Inputs.Select(t => renumber[t]).ToArray(), Output = renumber[_ops[i].Output] };
+        }
+
+        _output = (uint)(order.Length - results.Count);
+        _outputs = (uint)results.Count;
+    }
+
+    private void AddOp(HipOpcode opcode, uint[] inputs, uint output, ulong rdata0 = NoRdata, ulong rdata1 = NoRdata, int[]? p = null, float[]? f = null)
+    {
+        var (pNames, fNames, rdata) = HipOpLayouts.Fields[opcode];
+        p ??= Array.Empty<int>();
+        f ??= Array.Empty<float>();
+        int offsets = (rdata0 != NoRdata ? 1 : 0) + (rdata1 != NoRdata ? 1 : 0);
+        if (p.Length != pNames.Length || f.Length != fNames.Length || offsets > rdata || inputs.Length > HipConcatLimit)
+        {
+            throw new InvalidOperationException($"{opcode} record does not follow its layout");
+        }
+
+        _ops.Add(new OpRecord(opcode, inputs, output, rdata0, rdata1, p, f));
     }
 
     private ulong AddConstant(ReadOnlySpan<byte> bytes)
@@ -169,36 +286,20 @@ internal sealed class HipFunctionBuilder : FunctionBuilder
             return known;
         }
 
-        if (expr is not Call call)
+        if (expr is not Call { Target: IHipOp } call)
         {
             throw new NotSupportedException($"unexpected {expr.GetType().Name} in a hip function");
         }
 
-        uint input = Emit(call.Arguments[0], values);
+        var inputs = Passes.OutlineHipFunctionsPass.Activations(call).Select(a => Emit(a, values)).ToArray();
+        uint input = inputs[0];
+        var type = (TensorType)call.CheckedType!;
         uint output;
         switch (call.Target)
         {
             case HipQConv2D conv:
-                {
-                    var weights = ((TensorConst)call.Arguments[1]).Value;
-                    var bias = ((TensorConst)call.Arguments[2]).Value;
-                    _tensors[(int)input] = _tensors[(int)input] with { QuantParam = conv.InputQuantParam };
-                    output = AddTensor((TensorType)call.CheckedType!, conv.OutputQuantParam);
-                    var ws = weights.Dimensions;
-                    _ops.Add(new OpRecord(
-                        HipOpcode.Conv2D,
-                        new[] { input },
-                        output,
-                        AddConstant(weights.BytesBuffer),
-                        AddConstant(bias.BytesBuffer),
-                        new[]
-                        {
-                            ws[0], ws[1], ws[2], ws[3], conv.Groups, conv.Strides[0], conv.Strides[1], conv.Dilations[0], conv.Dilations[1],
-                            conv.Paddings[0], conv.Paddings[1], conv.Paddings[2], conv.Paddings[3], conv.WeightsQuantParam.ZeroPoint,
-                        },
-                        new[] { conv.FusedClamp.Min, conv.FusedClamp.Max, conv.WeightsQuantParam.Scale }));
-                    break;
-                }
+                output = EmitConv2D(conv, call, input);
+                break;
 
             case HipQMatMul matmul:
                 {
@@ -215,28 +316,139 @@ internal sealed class HipFunctionBuilder : FunctionBuilder
                         }
                     }
 
-                    _tensors[(int)input] = _tensors[(int)input] with { QuantParam = matmul.LhsQuantParam };
-                    output = AddTensor((TensorType)call.CheckedType!, matmul.OutputQuantParam);
-                    _ops.Add(new OpRecord(
+                    SetQuantParam(input, matmul.LhsQuantParam);
+                    output = AddTensor(type, matmul.OutputQuantParam);
+                    AddOp(
                         HipOpcode.Conv2D,
                         new[] { input },
                         output,
                         AddConstant(oihw),
                         NoRdata,
                         new[] { n, k, 1, 1, 1, 1, 1, 1, 1, 0, 0, 0, 0, matmul.RhsQuantParam.ZeroPoint },
-                        new[] { float.NegativeInfinity, float.PositiveInfinity, matmul.RhsQuantParam.Scale }));
+                        new[] { float.NegativeInfinity, float.PositiveInfinity, matmul.RhsQuantParam.Scale });
                     break;
                 }
 
+            case HipQuantize quantize:
+                output = AddTensor(type, quantize.QuantParam);
+                AddOp(HipOpcode.Quantize, new[] { input }, output);
+                break;
+
+            case HipDequantize dequantize:
+                SetQuantParam(input, dequantize.QuantParam);
+                output = AddTensor(type);
+                AddOp(HipOpcode.Dequantize, new[] { input }, output);
+                break;
+
+            case HipQAdd add:
+                SetQuantParam(inputs[0], add.LhsQuantParam);
+                SetQuantParam(inputs[1], add.RhsQuantParam);
+                output = AddTensor(type, add.OutputQuantParam);
+                AddOp(HipOpcode.Add, inputs, output, f: new[] { add.FusedClamp.Min, add.FusedClamp.Max });
+                break;
+
+            case HipQGlobalAvgPool pool:
+                SetQuantParam(input, pool.InputQuantParam);
+                output = AddTensor(type, pool.OutputQuantParam);
+                AddOp(HipOpcode.GlobalAvgPool, new[] { input }, output);
+                break;
+
+            case HipQLut lut:
+                SetQuantParam(input, lut.InputQuantParam);
+                output = AddTensor(type, lut.OutputQuantParam);
+                AddOp(HipOpcode.Lut, new[] { input }, output, AddConstant(((TensorConst)call.Arguments[1]).Value.BytesBuffer));
+                break;
+
+            case HipQConcat concat:
+                {
+                    // (0, 1) for every tensor is the byte concatenation of tensors that already share one QuantParam
+                    bool bytes = concat.OutputQuantParam.Scale == 1f && concat.OutputQuantParam.ZeroPoint == 0 && concat.InputQuantParams.All(q => q.Scale == 1f && q.ZeroPoint == 0);
+                    var shared = _tensors[(int)inputs[0]].QuantParam;
+                    for (int i = 0; i < inputs.Length; i++)
+                    {
+                        if (!bytes)
+                        {
+                            SetQuantParam(inputs[i], concat.InputQuantParams[i]);
+                        }
+                        else if (shared is null || !Nullable.Equals(_tensors[(int)inputs[i]].QuantParam, shared))
+                        {
+                            throw new NotSupportedException("a byte concatenation joins tensors of one QuantParam");
+                        }
+                    }
+
+                    output = AddTensor(type, bytes ? shared : concat.OutputQuantParam);
+                    AddOp(HipOpcode.Concat, inputs, output);
+                    break;
+                }
+
+            case HipResizeNearest resize:
+                output = AddTensor(type, _tensors[(int)input].QuantParam ?? resize.QuantParam);
+                AddOp(HipOpcode.ResizeNearest, new[] { input }, output, p: new[] { (int)resize.TransformationMode, (int)resize.NearestMode });
+                break;
+
+            case HipQMaxPool pool:
+                SetQuantParam(input, pool.InputQuantParam);
+                output = AddTensor(type, pool.OutputQuantParam);
+                AddOp(HipOpcode.MaxPool, new[] { input }, output, p: new[] { pool.Kernel, pool.Stride, pool.Padding });
+                break;
+
+            case HipReshape:
+                output = AddTensor(type, _tensors[(int)input].QuantParam);
+                AddOp(HipOpcode.Reshape, new[] { input }, output);
+                break;
+
             default:
-                throw new NotSupportedException($"{call.Target.GetType().Name} is not a hip operator");
+                throw new NotSupportedException($"{call.Target.GetType().Name} has no record in a hip function");
         }
 
         values.Add(expr, output);
         return output;
     }
 
-    private sealed record TensorRecord(uint TypeCode, int[] Nhwc, QuantParam QuantParam);
+    private uint EmitConv2D(HipQConv2D conv, Call call, uint input)
+    {
+        var weights = ((TensorConst)call.Arguments[1]).Value;
+        var bias = ((TensorConst)call.Arguments[2]).Value;
+        var ws = weights.Dimensions.ToArray();
+        var bytes = weights.BytesBuffer.ToArray();
+        SetQuantParam(input, conv.InputQuantParam);
+
+        // A dense convolution over fewer than four channels (an RGB stem) would gather single bytes: its input is
+        // padded to four channels and its weights with their zero point, whose products (w - zero point) vanish
+        // whatever the padded bytes are.  (3 x 3 windows of stride 1 are left to the kernel.)
+        bool small = conv.Groups == 1 && ws[1] < 4 && !(ws[2] == 3 && ws[3] == 3 && conv.Strides[0] == 1 && conv.Strides[1] == 1);
+        if (small)
+        {
+            var t = _tensors[(int)input];
+            uint padded = AddTensor(t.TypeCode, new[] { t.Nhwc[0], t.Nhwc[1], t.Nhwc[2], 4 }, t.QuantParam);
+            AddOp(HipOpcode.PadChannels, new[] { input }, padded);
+            int taps = ws[2] * ws[3];
+            var wide = Enumerable.Repeat((byte)conv.WeightsQuantParam.ZeroPoint, ws[0] * 4 * taps).ToArray();
+            for (int o = 0; o < ws[0]; o++)
+            {
+                Array.Copy(bytes, o * ws[1] * taps, wide, o * 4 * taps, ws[1] * taps);
+            }
+
+            (input, bytes, ws[1]) = (padded, wide, 4);
+        }
+
+        uint output = AddTensor((TensorType)call.CheckedType!, conv.OutputType == DataTypes.UInt8 ? conv.OutputQuantParam : null);
+        AddOp(
+            HipOpcode.Conv2D,
+            new[] { input },
+            output,
+            AddConstant(bytes),
+            AddConstant(bias.BytesBuffer),
+            new[]
+            {
+                ws[0], ws[1], ws[2], ws[3], conv.Groups, conv.Strides[0], conv.Strides[1], conv.Dilations[0], conv.Dilations[1],
+                conv.Paddings[0], conv.Paddings[1], conv.Paddings[2], conv.Paddings[3], conv.WeightsQuantParam.ZeroPoint,
+            },
+            new[] { conv.FusedClamp.Min, conv.FusedClamp.Max, conv.WeightsQuantParam.Scale });
+        return output;
+    }
+
+    private sealed record TensorRecord(uint TypeCode, int[] Nhwc, QuantParam? QuantParam);
 
     private sealed record OpRecord(HipOpcode Opcode, uint[] Inputs, uint Output, ulong Rdata0, ulong Rdata1, int[] P, float[] F);
 }

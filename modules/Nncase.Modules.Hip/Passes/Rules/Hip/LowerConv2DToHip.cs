@@ -27,10 +27,10 @@ public sealed partial class LowerConv2DToHip : IRewriteRule
             "conv",
             "convCall",
             c => c.PadMode == PadMode.Constant,
-            IsDequantize("dqInput", string.Empty, _ => true, IsWildcard("input") with { TypePattern = HasFixedShape() & HasDataType(DataTypes.UInt8) }, IsTensorConst("inputQp")),
-            IsDequantize("dqWeights", string.Empty, _ => true, IsTensorConst("weights", HasDataType(DataTypes.UInt8)), IsTensorConst("weightsQp")),
+            IsDequantize("dqInput", null, _ => true, IsWildcard("input") with { TypePattern = HasFixedShape() & HasDataType(DataTypes.UInt8) }, IsTensorConst("inputQp")),
+            IsDequantize("dqWeights", null, _ => true, IsTensorConst("weights", HasDataType(DataTypes.UInt8)), IsTensorConst("weightsQp")),
             IsAlt(
-                IsDequantize("dqBias", string.Empty, _ => true, IsTensorConst("bias", HasDataType(DataTypes.Int32)), IsTensorConst("biasQp")),
+                IsDequantize("dqBias", null, _ => true, IsTensorConst("bias", HasDataType(DataTypes.Int32)), IsTensorConst("biasQp")),
                 IsTensorConst("zeroBias")),
             IsTensorConst("strides"),
             IsTensorConst("paddings"),

@@ -17,8 +17,8 @@ public sealed partial class LowerMatMulToHip : IRewriteRule
         "matmul",
         "product",
         _ => true,
-        IsDequantize("dqLhs", string.Empty, _ => true, IsWildcard("lhs") with { TypePattern = HasFixedShape() & HasDataType(DataTypes.UInt8) }, IsTensorConst("lhsQp")),
-        IsDequantize("dqRhs", string.Empty, _ => true, IsTensorConst("rhs", HasRank(2) & HasDataType(DataTypes.UInt8)), IsTensorConst("rhsQp")));
+        IsDequantize("dqLhs", null, _ => true, IsWildcard("lhs") with { TypePattern = HasFixedShape() & HasDataType(DataTypes.UInt8) }, IsTensorConst("lhsQp")),
+        IsDequantize("dqRhs", null, _ => true, IsTensorConst("rhs", HasRank(2) & HasDataType(DataTypes.UInt8)), IsTensorConst("rhsQp")));
 
     public IPattern Pattern { get; } = IsAlt(
         IsQuantize("quantize", "output", q => q.TargetType == DataTypes.UInt8, Product, IsTensorConst("outputQp")),

@@ -1,7 +1,8 @@
 // ITarget of the MI355X execution target (interface: src/Nncase.Core/ITarget.cs:26-106).
-// With PTQ on, the quantised sub-graphs the importers and the quantiser leave behind
-// (Dequantize -> Conv2D / MatMul -> Quantize) become HipQConv2D / HipQMatMul calls, and chains of them are
-// outlined into functions of module kind "hip"; everything else stays in the stackvm module.
+// With PTQ on, the quantised sub-graphs the importers and the quantiser leave behind (Dequantize -> operator ->
+// Quantize, for convolutions, matrix products, residual adds, activations, pooling, concatenation and resizing)
+// become hip operators, and connected regions of them are outlined into functions of module kind "hip";
+// everything else stays in the stackvm module.
 using System;
 using System.Collections.Generic;
 using System.CommandLine;
@@ -61,6 +62,23 @@ public sealed class HipTarget : ITarget
         {
             p.Add<LowerConv2DToHip>();
             p.Add<LowerMatMulToHip>();
+            p.Add<LowerAddToHip>();
+            p.Add<LowerReduceMeanToHip>();
+            p.Add<LowerReduceWindow2DToHip>();
+            p.Add<LowerActivationToHip>();
+            p.Add<LowerConcatToHip>();
+            p.Add<LowerResizeToHip>();
+        });
+
+        // operators that only make sense next to a hip operator: they look at their neighbours, so they run once
+        // the sandwiches are gone (and the sandwich rules need the Dequantize calls these would consume)
+        passManager.AddWithName<DataflowPass>("lowering_hip_boundary").Configure(p =>
+        {
+            p.Add<LowerByteConcatToHip>();
+            p.Add<LowerResizeToHip>();
+            p.Add<LowerReshapeToHip>();
+            p.Add<LowerDequantizeToHip>();
+            p.Add<LowerQuantizeToHip>();
         });
         passManager.AddWithName<OutlineHipFunctionsPass>("outline_hip");
     }

@@ -9,7 +9,7 @@ namespace {
 
 struct Op {
     enum Kind { kQuantize, kDequantize, kConv, kAdd, kPool, kLut, kConcat, kResize, kMaxPool, kPack, kQuantPack,
-                kGemm, kRmsNorm, kRope, kAttn, kArgmax, kEmbed, kAddI32, kBlock } kind;
+                kGemm, kRmsNorm, kRope, kAttn, kArgmax, kEmbed, kAddI32, kBlock, kLayout } kind;
     const void *in0 = nullptr, *in1 = nullptr;
     void *out = nullptr;
     const nncase_hip_weights_t *weights = nullptr;
@@ -101,6 +101,9 @@ static int run_op(nncase_hip_function *fn, const Op &op) {
         return nncase_hip_embedding_f16(ctx, op.in0, (const int32_t *)op.in1, op.out, op.batch, op.channels, op.w);
     case Op::kAddI32:
         return nncase_hip_add_i32(ctx, (int32_t *)op.out, op.batch, op.delta);
+    case Op::kLayout: // mode 0: NCHW -> NHWC, 1: NHWC -> NCHW
+        return op.mode ? nncase_hip_nhwc_to_nchw(ctx, op.in0, op.out, op.elem_size, op.batch, op.channels, op.h, op.w)
+                       : nncase_hip_nchw_to_nhwc(ctx, op.in0, op.out, op.elem_size, op.batch, op.channels, op.h, op.w);
     case Op::kResize:
         return nncase_hip_resize_nearest(ctx, op.in0, op.out, op.elem_size, op.batch, op.h, op.w, op.channels, op.out_h,
                                          op.out_w, op.tmode, op.nmode);
@@ -251,6 +254,20 @@ extern "C" int nncase_hip_function_add_resize_nearest(nncase_hip_function_t *fn,
     op.kind = Op::kResize;
     op.in0 = in_dev, op.out = out_dev, op.elem_size = elem_size, op.batch = batch, op.h = in_h, op.w = in_w;
     op.channels = channels, op.out_h = out_h, op.out_w = out_w, op.tmode = transformation_mode, op.nmode = nearest_mode;
+    return push(fn, op);
+}
+
+extern "C" int nncase_hip_function_add_layout(nncase_hip_function_t *fn, const void *in_dev, void *out_dev, int32_t elem_size,
+                                              int32_t n, int32_t c, int32_t h, int32_t w, int32_t to_nchw) {
+    if (!fn) return -EINVAL;
+    NNHIP_REQUIRE(fn->ctx, in_dev && out_dev && in_dev != out_dev, -EINVAL, "function_add_layout: null or aliased buffers");
+    NNHIP_REQUIRE(fn->ctx, (elem_size == 1 || elem_size == 2 || elem_size == 4) && n > 0 && c > 0 && h > 0 && w > 0 &&
+                               (to_nchw == 0 || to_nchw == 1),
+                  -EINVAL, "function_add_layout: bad arguments");
+    Op op;
+    op.kind = Op::kLayout;
+    op.in0 = in_dev, op.out = out_dev, op.elem_size = elem_size, op.batch = n, op.channels = c, op.h = h, op.w = w;
+    op.mode = to_nchw;
     return push(fn, op);
 }
 
@@ -515,6 +532,7 @@ extern "C" int nncase_hip_function_op_kernel(nncase_hip_function_t *fn, int32_t 
     case Op::kLut: snprintf(name, capacity, "lut_u8"); break;
     case Op::kConcat: snprintf(name, capacity, "qconcat<%d>", op.n_inputs); break;
     case Op::kResize: snprintf(name, capacity, "resize_nearest"); break;
+    case Op::kLayout: snprintf(name, capacity, op.mode ? "nhwc_to_nchw" : "nchw_to_nhwc"); break;
     case Op::kMaxPool: snprintf(name, capacity, "qmaxpool<%dx%d>", op.pool[0], op.pool[1]); break;
     case Op::kPack: snprintf(name, capacity, "pack"); break;
     case Op::kQuantPack: snprintf(name, capacity, "quantize+pack"); break;

@@ -66,7 +66,7 @@ constexpr uint32_t kModelIdentifier = 0x4B4D444C; // 'KMDL'
 constexpr uint32_t kModelVersion = 7;
 constexpr uint64_t kNoRdata = ~uint64_t(0);
 enum { kOpQuantize, kOpDequantize, kOpConv2d, kOpAdd, kOpGlobalAvgPool, kOpLut, kOpConcat, kOpResizeNearest, kOpMaxPool,
-       kOpPadChannels, kOpReshape };
+       kOpPadChannels, kOpReshape, kOpLayout };
 
 struct Span {
     const uint8_t *p = nullptr;
@@ -760,6 +760,14 @@ static int build_function(nncase_hip_ctx_t *ctx, Span text_span, Span rdata, nnc
                                                     static_cast<uint8_t *>(m->buffers[dst]), (int)ti.dims[0], (int)ti.dims[1],
                                                     (int)ti.dims[2], (int)ti.dims[3], o.p[0], o.p[0], o.p[1], o.p[1], o.p[2], o.p[2],
                                                     o.p[2], o.p[2], tqp(in0), tqp(dst));
+            break;
+        case kOpLayout:
+            // p[0] = 0: the input holds N, C, H, W in that order and the output is channels-last; 1: the reverse
+            // (both tensor records give their extents as N, H, W, C)
+            NNHIP_REQUIRE(ctx, ti.dtype == to.dtype && memcmp(ti.dims, to.dims, sizeof(ti.dims)) == 0 && (o.p[0] == 0 || o.p[0] == 1),
+                          -NNCASE_HIP_ERR_SHAPE_MISMATCH, "kmodel_load: op %u layout tensors / direction", k);
+            rc = nncase_hip_function_add_layout(m->fn, m->buffers[in0], m->buffers[dst], (int)dtype_size(ti.dtype), (int)ti.dims[0],
+                                                (int)ti.dims[3], (int)ti.dims[1], (int)ti.dims[2], o.p[0]);
             break;
         case kOpReshape:
             NNHIP_REQUIRE(ctx, ti.dtype == to.dtype && elems(in0) == elems(dst) && m->buffers[in0] && !is_output((int32_t)dst),

@@ -277,9 +277,28 @@ HIPF_TENSOR = struct.Struct("<6Iif")
 HIPF_OP = struct.Struct("<2I8iiI2Q16i4f")
 NO_RDATA = 0xFFFFFFFFFFFFFFFF
 (OP_QUANTIZE, OP_DEQUANTIZE, OP_CONV2D, OP_ADD, OP_GLOBAL_AVGPOOL, OP_LUT, OP_CONCAT, OP_RESIZE_NEAREST, OP_MAXPOOL,
- OP_PAD_CHANNELS, OP_RESHAPE) = range(11)
+ OP_PAD_CHANNELS, OP_RESHAPE, OP_LAYOUT) = range(12)
 OP_NAMES = ["quantize", "dequantize", "conv2d", "add", "global_avgpool", "lut", "concat", "resize_nearest", "maxpool",
-            "pad_channels", "reshape"]
+            "pad_channels", "reshape", "layout"]
+# What each operator record holds beside its tensors: names of p[0..], names of f[0..], number of .rdata offsets.
+# (The loader, nncase_hip_kmodel_load_function, and the compiler-side writer follow this table field by field.)
+OP_FIELDS = {
+    "quantize": ((), (), 0),
+    "dequantize": ((), (), 0),
+    "conv2d": (("out_channels", "group_in_channels", "kernel_h", "kernel_w", "groups", "stride_h", "stride_w", "dilation_h",
+                "dilation_w", "pad_h_before", "pad_h_after", "pad_w_before", "pad_w_after", "weights_zero_point"),
+               ("clamp_min", "clamp_max", "weights_scale"), 2),
+    "add": ((), ("clamp_min", "clamp_max"), 0),
+    "global_avgpool": ((), (), 0),
+    "lut": ((), (), 1),
+    "concat": ((), (), 0),
+    "resize_nearest": (("transformation_mode", "nearest_mode"), (), 0),
+    "maxpool": (("kernel", "stride", "padding"), (), 0),
+    "pad_channels": ((), (), 0),
+    "reshape": ((), (), 0),
+    "layout": (("to_nchw",), (), 0),     # the tensor on the NCHW side still records its extents as N, H, W, C
+}
+assert list(OP_FIELDS) == OP_NAMES
 assert HIPF_HEADER.size == 32 and HIPF_TENSOR.size == 32 and HIPF_OP.size == 144
 
 

@@ -130,6 +130,7 @@ SYMBOLS = {
     "nncase_hip_function_add_qconcat_channels": (_I, [_VP, C.c_int32, C.POINTER(_VP), _I32P, C.POINTER(QuantParam), _VP,
                                                       QuantParam, C.c_int64]),
     "nncase_hip_function_add_resize_nearest": (_I, [_VP, _VP, _VP] + [C.c_int32] * 9),
+    "nncase_hip_function_add_layout": (_I, [_VP, _VP, _VP] + [C.c_int32] * 6),
     "nncase_hip_qmaxpool2d": (_I, [_VP, _VP, _VP] + [C.c_int32] * 12 + [QuantParam, QuantParam]),
     "nncase_hip_function_add_qmaxpool2d": (_I, [_VP, _VP, _VP] + [C.c_int32] * 12 + [QuantParam, QuantParam]),
     "nncase_hip_function_add_pack": (_I, [_VP, _VP, _VP, C.c_int32, C.c_int32, _I32P, C.c_int32, _I32P, _I32P]),
@@ -756,6 +757,12 @@ class Function:
         self._ck(self.ctx.lib.nncase_hip_function_add_resize_nearest(self.handle, src.ptr, dst.ptr, elem_size, batch, in_h,
                                                                      in_w, channels, out_h, out_w, transformation_mode,
                                                                      nearest_mode), "function_add_resize_nearest")
+
+    def add_layout(self, src, dst, elem_size, n, c, h, w, to_nchw: bool):
+        """NCHW -> NHWC (to_nchw False) or back, as a step of the function."""
+        self._keep += [src, dst]
+        self._ck(self.ctx.lib.nncase_hip_function_add_layout(self.handle, src.ptr, dst.ptr, elem_size, n, c, h, w, int(to_nchw)),
+                 "function_add_layout")
 
     def set_lane(self, lane: int):
         """Operators added from now on form independent chain `lane`; a captured function overlaps its lanes."""

@@ -150,6 +150,78 @@ def test_csharp_function_text_constants_match_the_writer():
     assert '"HIPF"' in cs and km.HIPF_MAGIC == b"HIPF"
 
 
+CS_MODULE = os.path.join(ROOT, "modules", "Nncase.Modules.Hip")
+
+
+def cs(*parts):
+    return open(os.path.join(CS_MODULE, *parts)).read()
+
+
+def csharp_op_layouts():
+    """HipOpLayouts.Fields of the function builder, as {opcode name: (p names, f names, rdata count)}."""
+    body = re.search(r"class HipOpLayouts\s*\{(.*?)\n\}", cs("CodeGen", "Hip", "HipModuleBuilder.cs"), re.S).group(1)
+    out = {}
+    for entry in body.split("[HipOpcode.")[1:]:
+        name, value = entry.split("]", 1)
+        value = value[:value.rindex("),")]
+        lists = [tuple(re.findall(r'"(\w+)"', m.group(1) or ""))
+                 for m in re.finditer(r"new string\[0\]|new\[\] \{(.*?)\}", value, re.S)]
+        assert len(lists) == 2, name
+        out[name] = (lists[0], lists[1], int(re.search(r"(\d+)\s*$", value).group(1)))
+    return out
+
+
+def test_csharp_operator_records_follow_the_writers_field_table():
+    from nncase_amd import kmodel as km
+    layouts = csharp_op_layouts()
+    assert {n.lower(): v for n, v in layouts.items()} == {n.replace("_", ""): v for n, v in km.OP_FIELDS.items()}
+
+
+def test_loader_reads_exactly_the_fields_the_table_names():
+    """Every `case kOpX:` of the loader indexes p[] and f[] of its record below the table's lengths, and uses them all."""
+    from nncase_amd import kmodel as km
+    text = open(os.path.join(ROOT, "nncase_amd", "csrc", "kmodel.hip")).read()
+    enum = re.search(r"enum \{ (kOpQuantize.*?) \};", text, re.S).group(1)
+    names = [n.strip() for n in enum.replace("\n", " ").split(",")]
+    assert [n[3:].lower() for n in names] == [n.replace("_", "") for n in km.OP_NAMES]
+    switch = text[text.index("switch (o.opcode) {"):]
+    blocks = re.split(r"\n        case (kOp\w+):", switch[:switch.index("\n        default:")])
+    seen = {}
+    for label, block in zip(blocks[1::2], blocks[2::2]):
+        seen[label] = ({int(i) for i in re.findall(r"\bo\.p\[(\d+)\]", block)}, {int(i) for i in re.findall(r"\bo\.f\[(\d+)\]", block)},
+                       len(set(re.findall(r"\bo\.rdata(\d)", block))))
+    assert set(seen) == set(names)
+    for label, name in zip(names, km.OP_NAMES):
+        p, f, r = seen[label]
+        pn, fn, rn = km.OP_FIELDS[name]
+        assert p == set(range(len(pn))) and f == set(range(len(fn))) and r == rn, (name, p, f, r)
+
+
+def test_every_opcode_and_operator_of_the_csharp_module_is_wired_through():
+    """Each opcode has an emitter; each hip operator has a lowering rule that the target registers, a case in the
+    function builder and an evaluator that the plugin registers."""
+    from nncase_amd import kmodel as km
+    builder = cs("CodeGen", "Hip", "HipModuleBuilder.cs")
+    emitted = set(re.findall(r"AddOp\(\s*HipOpcode\.(\w+)", builder))
+    assert {n.lower() for n in emitted} == {n.replace("_", "") for n in km.OP_NAMES}
+    ops = re.findall(r"public sealed partial class (Hip\w+) : Op, IHipOp", cs("IR", "Hip", "HipOps.cs"))
+    assert len(ops) == 11
+    rules = "".join(cs("Passes", "Rules", "Hip", f) for f in os.listdir(os.path.join(CS_MODULE, "Passes", "Rules", "Hip")))
+    target, plugin = cs("Targets", "HipTarget.cs"), cs("HipModule.cs")
+    evaluators = cs("Evaluator", "Hip", "HipEvaluators.cs") + cs("Evaluator", "Hip", "HipRaisedEvaluators.cs")
+    for op in ops:
+        assert re.search(r"case %s\b" % op, builder), f"{op}: no case in the function builder"
+        made_by = [r for r, body in re.findall(r"public sealed partial class (\w+) : IRewriteRule(.*?)(?=\n\[RuleGenerator\]|\ninternal static class|\Z)", rules, re.S)
+                   if re.search(r"new %s\b" % op, body) or (op == "HipQConcat" and "HipConcat.Build" in body)]
+        assert made_by and all(f"p.Add<{r}>()" in target for r in made_by), f"{op}: rules {made_by} not registered"
+        ev = re.search(r"class (\w+) : (?:HipRaisedEvaluator<%s>|IEvaluator<%s>)" % (op, op), evaluators)
+        assert ev and f"RegisterManyInterface<{ev.group(1)}>" in plugin, f"{op}: evaluator missing or not registered"
+    # the outlining pass builds what the unmodified stackvm code generator accepts: a wrapper over a prim function
+    outline = cs("Passes", "OutlineHipFunctionsPass.cs")
+    assert "new PrimFunctionWrapper(" in outline and "new PrimFunction(" in outline and "new Fusion(" not in outline
+    assert "(TIR.PrimFunction)callable" in builder
+
+
 def test_errno_statuses_stay_clear_of_the_nncase_errc_block():
     """A status in [-7, -1] must always be an nncase_errc: the runtime-module shim maps statuses back by range."""
     src = os.path.join(ROOT, "nncase_amd", "csrc")

@@ -215,3 +215,64 @@ def test_a_matmul_function_with_f32_output_as_the_code_generator_writes_it(hip_c
     exact = ((a.astype(np.int64) - a_qp[0]) @ (b.astype(np.int64) - b_qp[0])).astype(np.float64) * (np.float32(a_qp[1]).astype(np.float64) * np.float32(b_qp[1]).astype(np.float64))
     assert np.abs(got - exact).max() <= np.abs(exact).max() * 2e-7 + 1e-6
     assert np.abs(got - want).max() <= np.abs(want).max() * 1e-4
+
+
+def test_a_function_with_nchw_ends_as_the_code_generator_writes_it(hip_ctx):
+    """What the C# function builder emits for an outlined region of a quantised network whose tensors the IR holds as
+    NCHW: a layout step at the entry, every operator the lowering rules produce (conv, byte table, residual add,
+    max pool, resize, concat, global mean), two outputs, and a layout step before each 4-D output."""
+    from oracle import oracle as O
+    rng = np.random.default_rng(33)
+    N, C, H, W, OC = 2, 24, 20, 28, 24
+    x = rng.integers(0, 256, (N, C, H, W), dtype=np.uint8)
+    w = rng.integers(0, 256, (OC, C, 3, 3), dtype=np.uint8)
+    bias = rng.integers(-4000, 4000, OC, dtype=np.int32)
+    qx, qw, qc, ql, qa, qp, qcat, qm = (120, 0.02), (128, 0.004), (110, 0.05), (8, 0.03), (100, 0.06), (90, 0.07), (95, 0.065), (97, 0.05)
+    flt_max = float(np.finfo(np.float32).max)
+    table = O.unary_lut(O.LUT_SWISH, *qc, *ql)
+
+    rdata = km.RData()
+    w_off, b_off, t_off = rdata.add(w), rdata.add(bias), rdata.add(table)
+    T = km.HipTensor
+    tensors = [
+        T("u8", (N, H, W, C), *qx),             # 0 input as the caller hands it: N, C, H, W order
+        T("u8", (N, H, W, C), *qx),             # 1 channels-last
+        T("u8", (N, H, W, OC), *qc),            # 2 conv
+        T("u8", (N, H, W, OC), *ql),            # 3 swish table
+        T("u8", (N, H, W, OC), *qa),            # 4 add(3, 1)
+        T("u8", (N, H // 2, W // 2, OC), *qp),  # 5 maxpool 2x2 / 2
+        T("u8", (N, H, W, OC), *qp),            # 6 resize back to H x W
+        T("u8", (N, H, W, 2 * OC), *qcat),      # 7 concat(6, 4)
+        T("u8", (N, 1, 1, 2 * OC), *qm),        # 8 global mean: first output (H = W = 1 needs no layout step)
+        T("u8", (N, H, W, 2 * OC), *qcat),      # 9 tensor 7 in N, C, H, W order: second output
+    ]
+    ops = [
+        km.HipOp(km.OP_LAYOUT, (0,), 1, p=(0,)),
+        km.HipOp(km.OP_CONV2D, (1,), 2, w_off, b_off, (OC, C, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 1, qw[0]), (-flt_max, flt_max, qw[1])),
+        km.HipOp(km.OP_LUT, (2,), 3, t_off),
+        km.HipOp(km.OP_ADD, (3, 1), 4, f=(0.0, 6.0)),
+        km.HipOp(km.OP_MAXPOOL, (4,), 5, p=(2, 2, 0)),
+        km.HipOp(km.OP_RESIZE_NEAREST, (5,), 6, p=(rt.RESIZE_ASYMMETRIC, rt.NEAREST_FLOOR)),
+        km.HipOp(km.OP_CONCAT, (6, 4), 7),
+        km.HipOp(km.OP_GLOBAL_AVGPOOL, (7,), 8),
+        km.HipOp(km.OP_LAYOUT, (7,), 9, p=(1,)),
+    ]
+    for o in ops:  # the writer's field table describes every record used here
+        pf, ff, nr = km.OP_FIELDS[km.OP_NAMES[o.opcode]]
+        assert len(pf) == len(o.p) and len(ff) == len(o.f)
+        assert nr == (o.rdata0 != km.NO_RDATA) + (o.rdata1 != km.NO_RDATA)
+    text = km.encode_hip_text(tensors, ops, 0, 8, n_outputs=2)
+    model = rt.LoadedKModel(hip_ctx, text=text, rdata=bytes(rdata.buf))
+    assert len(model.outputs) == 2
+    # the input buffer takes the caller's NCHW bytes as they are
+    mean, cat = model.run(x.reshape(N, H, W, C))
+
+    conv = O.qconv2d(x, w, bias, qx[0], qx[1], qw[0], qw[1], qc[0], qc[1], padding=((1, 1), (1, 1)))
+    act = table[conv]
+    add = O.qadd(act, x, ql[0], ql[1], qx[0], qx[1], qa[0], qa[1], fused_clamp=(0.0, 6.0))
+    pool = O.qmaxpool(add, (2, 2), (2, 2), ((0, 0), (0, 0)), qa[0], qa[1], qp[0], qp[1])
+    up = O.resize_nearest(pool, H, W, O.ASYMMETRIC, O.FLOOR)
+    want_cat = O.qconcat([up, add], [qp, qa], qcat)
+    want_mean = O.qglobal_avgpool(want_cat, qcat[0], qcat[1], qm[0], qm[1])
+    assert np.array_equal(cat.reshape(N, 2 * OC, H, W), want_cat)
+    assert np.array_equal(mean.reshape(N, 2 * OC), want_mean)
