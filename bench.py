@@ -282,7 +282,7 @@ def side_workload(args):
         kc = rng.standard_normal((nblocks, cfg.kv_heads, cfg.block_size, cfg.head_dim), dtype=np.float32).astype(np.float16)
         vc = rng.standard_normal((nblocks, cfg.kv_heads, cfg.head_dim, cfg.block_size), dtype=np.float32).astype(np.float16)
         dec = llm.HipDecoder(ctx, cfg, weights, batch, max_blocks, bt, lens, [kc] * cfg.layers, [vc] * cfg.layers,
-                             capture_graph=not args.no_graph, feedback=True)
+                             capture_graph=not args.no_graph, feedback=True, lanes=args.decode_lanes)
         dec.set_tokens(rng.integers(0, cfg.vocab, batch).astype(np.int32))
         ms = time_calls(ctx, dec.step, args.warmup, args.steps)
         toks = dec.result()
@@ -300,7 +300,7 @@ def side_workload(args):
                     unit="tokens/s", ms_per_step=round(ms, 4), dtype="f16",
                     config={"workload": "config 5: 24 layers, hidden 896, 14 q / 2 kv heads, head_dim 64, MLP 4864, vocab 151936, W8A16 per-output-channel "
                                         "weights, fp16 paged KV (block 16), batch 32, ctx U[512,4096], greedy arg-max fed back on the device, "
-                                        f"{len(dec.fn)} operators, one HIP-graph replay per step"},
+                                        f"{len(dec.fn)} operators in {args.decode_lanes} lane(s), one HIP-graph replay per step"},
                     roofline={"bound": "hbm", "achieved": round((kv_bytes + w_bytes) / (ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                               "frac": round((kv_bytes + w_bytes) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
                               "algorithmic_bytes_per_step": kv_bytes + w_bytes, "weight_bytes": w_bytes, "kv_bytes": kv_bytes},
@@ -347,6 +347,8 @@ def main():
     ap.add_argument("--lanes", type=int, default=1,
                     help="independent chains the batch is split into and replayed concurrently (1 = one chain of "
                          "full-batch launches); results are bit-identical for every value")
+    ap.add_argument("--decode-lanes", type=int, default=2,
+                    help="--workload llm_decode: ranges the 32 sequences are split into, each recorded as a chain of its own that the graph replays beside the others")
     ap.add_argument("--in-flight", type=int, default=4,
                     help="copies of the function (own stream and buffers each) that take the steps in turn, so that "
                          "consecutive steps overlap on the device (1 = one step at a time)")

@@ -452,6 +452,26 @@ int attn_reserve(nncase_hip_ctx *ctx, const nncase_hip_paged_attn_args_t *p) {
     return 0;
 }
 
+int attn_scratch_sizes(nncase_hip_ctx *ctx, const nncase_hip_paged_attn_args_t *p, size_t *partial_bytes, size_t *counter_bytes) {
+    AttnPlan plan;
+    const int rc = attn_plan(ctx, p, &plan);
+    if (rc) return rc;
+    *partial_bytes = plan.partial_bytes, *counter_bytes = plan.counter_bytes;
+    return 0;
+}
+
+int attn_decode_on(nncase_hip_ctx *ctx, const void *q_dev, const void *k_cache_dev, const void *v_cache_dev, const int32_t *block_table_dev,
+                   const int32_t *ctx_lens_dev, void *out_dev, const nncase_hip_paged_attn_args_t *p, void *partials,
+                   size_t partial_bytes, void *counters, size_t counter_bytes) {
+    AttnPlan plan;
+    const int rc = attn_plan(ctx, p, &plan);
+    if (rc) return rc;
+    NNHIP_REQUIRE(ctx, partials && counters && plan.partial_bytes <= partial_bytes && plan.counter_bytes <= counter_bytes, -ENOSPC,
+                  "paged_attention_decode: the scratch areas brought along hold %zu and %zu bytes, the geometry needs %zu and %zu",
+                  partial_bytes, counter_bytes, plan.partial_bytes, plan.counter_bytes);
+    return attn_launch(ctx, plan, q_dev, k_cache_dev, v_cache_dev, block_table_dev, ctx_lens_dev, out_dev, partials, counters);
+}
+
 } // namespace nnhip
 
 using namespace nnhip;

@@ -150,5 +150,11 @@ template <typename TQ> __device__ __forceinline__ TQ quantize_one(float x, float
 // attn.hip: checks the geometry and sizes the context's paged-attention workspace for it
 // (-EBUSY if that needs a reallocation while a captured graph refers to it or the stream is capturing).
 int attn_reserve(nncase_hip_ctx *ctx, const nncase_hip_paged_attn_args_t *geometry);
+// Bytes of split partials and of counters paged attention needs for a geometry, and the launch on areas the caller
+// brings (the counters zero before the first launch; every launch leaves them zero again).
+int attn_scratch_sizes(nncase_hip_ctx *ctx, const nncase_hip_paged_attn_args_t *geometry, size_t *partial_bytes, size_t *counter_bytes);
+int attn_decode_on(nncase_hip_ctx *ctx, const void *q_dev, const void *k_cache_dev, const void *v_cache_dev, const int32_t *block_table_dev,
+                   const int32_t *ctx_lens_dev, void *out_dev, const nncase_hip_paged_attn_args_t *geometry, void *partials,
+                   size_t partial_bytes, void *counters, size_t counter_bytes);
 
 } // namespace nnhip

@@ -50,6 +50,10 @@ struct nncase_hip_function {
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
     bool pins_attn = false; // the captured graph holds the addresses of the context's attention workspace
+    // Paged attention on a lane other than 0 goes through split partials and counters of that lane's own (lane 0
+    // uses the context's), so that lanes may run it side by side; owned by the function.
+    void *lane_partials[NNCASE_HIP_MAX_LANES] = {nullptr}, *lane_counters[NNCASE_HIP_MAX_LANES] = {nullptr};
+    size_t lane_partial_bytes[NNCASE_HIP_MAX_LANES] = {0}, lane_counter_bytes[NNCASE_HIP_MAX_LANES] = {0};
 };
 
 using namespace nnhip;
@@ -93,6 +97,10 @@ static int run_op(nncase_hip_function *fn, const Op &op) {
         return nncase_hip_rope_kv_append(ctx, op.in0, op.out, op.out2, op.out3, (const int32_t *)op.in2, (const int32_t *)op.in3,
                                          &op.attn, op.eps);
     case Op::kAttn:
+        if (op.lane > 0)
+            return attn_decode_on(ctx, op.in0, op.in1, op.in2, (const int32_t *)op.in3, (const int32_t *)op.in4, op.out, &op.attn,
+                                  fn->lane_partials[op.lane], fn->lane_partial_bytes[op.lane], fn->lane_counters[op.lane],
+                                  fn->lane_counter_bytes[op.lane]);
         return nncase_hip_paged_attention_decode(ctx, op.in0, op.in1, op.in2, (const int32_t *)op.in3, (const int32_t *)op.in4,
                                                  op.out, &op.attn);
     case Op::kArgmax:
@@ -150,6 +158,10 @@ extern "C" int nncase_hip_function_destroy(nncase_hip_function_t *fn) {
     if (!fn) return -EINVAL;
     (void)hipStreamSynchronize(fn->ctx->stream);
     drop_graph(fn);
+    for (int l = 0; l < NNCASE_HIP_MAX_LANES; l++) {
+        if (fn->lane_partials[l]) (void)hipFree(fn->lane_partials[l]);
+        if (fn->lane_counters[l]) (void)hipFree(fn->lane_counters[l]);
+    }
     delete fn;
     return 0;
 }
@@ -373,8 +385,33 @@ extern "C" int nncase_hip_function_add_paged_attention_decode(nncase_hip_functio
                   "function_add_paged_attention_decode: null argument");
     // the workspace the kernel's splits go through is sized now: capture must not allocate, and a graph
     // keeps the addresses it was captured with
-    const int rc = attn_reserve(fn->ctx, args);
-    if (rc) return rc;
+    const int lane = fn->cur_lane;
+    if (lane == 0) {
+        const int rc = attn_reserve(fn->ctx, args);
+        if (rc) return rc;
+    } else {
+        size_t pb = 0, cb = 0;
+        const int rc = attn_scratch_sizes(fn->ctx, args, &pb, &cb);
+        if (rc) return rc;
+        if (pb > fn->lane_partial_bytes[lane] || cb > fn->lane_counter_bytes[lane]) {
+            NNHIP_REQUIRE(fn->ctx, !fn->exec, -EBUSY, "function_add_paged_attention_decode: the lane's scratch would grow under a captured graph");
+            NNHIP_HIP(fn->ctx, hipStreamSynchronize(fn->ctx->stream)); // earlier eager invocations may still use the old areas
+            if (pb > fn->lane_partial_bytes[lane]) {
+                if (fn->lane_partials[lane]) NNHIP_HIP(fn->ctx, hipFree(fn->lane_partials[lane]));
+                fn->lane_partials[lane] = nullptr, fn->lane_partial_bytes[lane] = 0;
+                NNHIP_HIP(fn->ctx, hipMalloc(&fn->lane_partials[lane], pb));
+                fn->lane_partial_bytes[lane] = pb;
+            }
+            if (cb > fn->lane_counter_bytes[lane]) {
+                if (fn->lane_counters[lane]) NNHIP_HIP(fn->ctx, hipFree(fn->lane_counters[lane]));
+                fn->lane_counters[lane] = nullptr, fn->lane_counter_bytes[lane] = 0;
+                const size_t cap = (cb + 4095) / 4096 * 4096;
+                NNHIP_HIP(fn->ctx, hipMalloc(&fn->lane_counters[lane], cap));
+                fn->lane_counter_bytes[lane] = cap;
+                NNHIP_HIP(fn->ctx, hipMemset(fn->lane_counters[lane], 0, cap)); // (not under capture: recording comes first)
+            }
+        }
+    }
     Op op;
     op.kind = Op::kAttn;
     op.in0 = q_dev, op.in1 = k_cache_dev, op.in2 = v_cache_dev, op.in3 = block_table_dev, op.in4 = ctx_lens_dev, op.out = out_dev;
@@ -442,15 +479,11 @@ extern "C" int nncase_hip_function_capture(nncase_hip_function_t *fn) {
     nncase_hip_ctx *ctx = fn->ctx;
     drop_graph(fn);
     NNHIP_HIP(ctx, hipStreamSynchronize(ctx->stream));
-    // Paged attention keeps its split partials and counters in one per-context scratch area: two lanes that
-    // both run it would overlap on that area, so all attention operators must sit on one lane.
+    // (paged attention on lane 0 goes through the context's scratch area, whose addresses the graph will hold;
+    // other lanes bring areas of their own)
     int attn_lane = -1;
-    for (const Op &op : fn->ops) {
-        if (op.kind != Op::kAttn) continue;
-        NNHIP_REQUIRE(ctx, attn_lane < 0 || attn_lane == op.lane, -EINVAL,
-                      "function_capture: paged attention on lanes %d and %d (its scratch area is per context)", attn_lane, op.lane);
-        attn_lane = op.lane;
-    }
+    for (const Op &op : fn->ops)
+        if (op.kind == Op::kAttn && op.lane == 0) attn_lane = 0;
     // Operators of different lanes are recorded on streams of their own, forked from and joined back into
     // the context's stream, so the graph holds one independent chain per lane and the device overlaps them.
     hipStream_t main_stream = ctx->stream;

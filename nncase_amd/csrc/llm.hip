@@ -321,86 +321,102 @@ template <int MT, int G, bool SPLIT, int B = kGemmBatch> __global__ __launch_bou
 // wave, wave + WAVES, ...): it adds their squares in rms_rstd_rows' order as they arrive, parks them in LDS as loaded,
 // and, knowing 1 / sqrt(mean + eps) of its own rows without asking another wave, normalises them in place -- one trip
 // to memory and one barrier in front of the products, and every element normalised once per block instead of once per
-// wave.  A wave has the weights of eight k-steps in flight.  The arithmetic per element and the order of the
+// wave.  A wave has the weights of KB k-steps in flight, the first KB from the start of the kernel.  The arithmetic per element and the order of the
 // multiply-adds are those of the kernel above.
 constexpr int kRowsBatch = 8;
+constexpr int kGluSplitWaves = 4;             // waves that split the reduction of one gate / up tile pair
+constexpr int kRowsWhole = 14;                // k-steps of a reduction that is requested in one go
 constexpr int kRowsPieces = 4;                 // 512-element pieces of a row: k <= 2048
 constexpr int kRowsMaxK = kRowsPieces * 512;
 inline int rows_in_lds_pitch(int k) { return k * 2 + 16; } // bytes per token row: the padding spreads the rows over the banks
 
 // SPLIT: the block's waves share ONE output tile and split its reduction (few tiles: the q / k / v projection), combined
 // through LDS in the fixed order of the kernel above.
-template <int MT, int G, int WAVES, bool SPLIT = false> __global__ __launch_bounds__(WAVES * 64) void w8a16_gemm_rows_in_lds_kernel(const GemmArgs a) {
+template <int MT, int G, int WAVES, bool SPLIT = false, int KB = kRowsBatch, int PIECES = kRowsPieces>
+__global__ __launch_bounds__(WAVES * 64) void w8a16_gemm_rows_in_lds_kernel(const GemmArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t xs[]; // [MT * 16][k halves + padding]
     __shared__ float red[SPLIT ? WAVES : 1][G][SPLIT ? MT : 1][64][4];
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int i16 = lane & 15, kg = lane >> 4;
     const int pitch = a.k * 2 + 16;
+    // The weights do not depend on the rows: the first KB k-steps of this wave's share are requested before anything
+    // else, so that their trip to memory runs beside the one that brings the rows in (a spare wave of the last block
+    // reads the last tile's and multiplies nothing).
+    const int out_tile = SPLIT ? (int)blockIdx.x : (int)blockIdx.x * WAVES + wave;
+    const int per = SPLIT ? (a.ksteps + WAVES - 1) / WAVES : a.ksteps;
+    const int ks0 = SPLIT ? wave * per : 0, ks1 = min(a.ksteps, ks0 + per);
+    const int tile[2] = {min(out_tile, a.up_tile_offset - 1), min(out_tile, a.up_tile_offset - 1) + a.up_tile_offset};
+    lu32x4 wv[KB][G];
+#pragma unroll
+    for (int u = 0; u < KB; u++) {
+        const int ks = max(min(ks0 + u, ks1 - 1), 0); // steps past the share re-read its last one (an empty share: step 0) and are not multiplied
+#pragma unroll
+        for (int g = 0; g < G; g++) wv[u][g] = a.w[((size_t)tile[g] * a.ksteps + ks) * 64 + lane];
+    }
     {
         constexpr int R = MT * 16 / WAVES; // rows per wave
-        lu32x4 lwp[kRowsPieces];
-        if (a.ln_w) {
+        // The wave's rows stay in registers from the load to the one LDS write: their sums of squares, the butterflies
+        // and the normalisation run for all R rows side by side (independent chains), element by element in the order
+        // rms_rstd_rows and rmsnorm_f16_kernel use.
+        lu32x4 v[R][PIECES], lwp[PIECES];
 #pragma unroll
-            for (int p = 0; p < kRowsPieces; p++) {
-                const int e0 = lane * 8 + p * 512;
-                lwp[p] = lu32x4{0, 0, 0, 0};
-                if (e0 < a.k) lwp[p] = *reinterpret_cast<const lu32x4 *>(a.ln_w + e0);
-            }
-        }
-        float ss[R];
-#pragma unroll
-        for (int i = 0; i < R; i++) ss[i] = 0.f;
-#pragma unroll
-        for (int p = 0; p < kRowsPieces; p++) {
+        for (int p = 0; p < PIECES; p++) {
             const int e0 = lane * 8 + p * 512;
-            if (e0 < a.k) {
-                lu32x4 v[R];
-#pragma unroll
-                for (int i = 0; i < R; i++) {
-                    const int r = wave + i * WAVES;
-                    v[i] = lu32x4{0, 0, 0, 0}; // rows past m: zeros (their products are never stored)
-                    if (r < a.m) v[i] = *reinterpret_cast<const lu32x4 *>(a.a + (size_t)r * a.k + e0);
-                }
-#pragma unroll
-                for (int i = 0; i < R; i++) {
-                    if (a.ln_w) add_squares8(v[i], ss[i]);
-                    *reinterpret_cast<lu32x4 *>(xs + (size_t)(wave + i * WAVES) * pitch + e0 * 2) = v[i];
-                }
-            }
-        }
-        if (a.ln_w) {
+            lwp[p] = lu32x4{0, 0, 0, 0};
+            if (a.ln_w && e0 < a.k) lwp[p] = *reinterpret_cast<const lu32x4 *>(a.ln_w + e0);
 #pragma unroll
             for (int i = 0; i < R; i++) {
-                const float rr = rstd_from_sum(ss[i], a.k, a.ln_eps);
+                const int r = wave + i * WAVES;
+                v[i][p] = lu32x4{0, 0, 0, 0}; // rows past m: zeros (their products are never stored)
+                if (r < a.m && e0 < a.k) v[i][p] = *reinterpret_cast<const lu32x4 *>(a.a + (size_t)r * a.k + e0);
+            }
+        }
+            if (a.ln_w) {
+            float ss[R];
 #pragma unroll
-                for (int p = 0; p < kRowsPieces; p++) {
-                    const int e0 = lane * 8 + p * 512;
-                    if (e0 < a.k) {
-                        lu32x4 *slot = reinterpret_cast<lu32x4 *>(xs + (size_t)(wave + i * WAVES) * pitch + e0 * 2);
-                        lu32x4 v = *slot; // (the lane's own bytes: LDS operations of a wave complete in order)
-                        __half xh[8], wh[8];
-                        __builtin_memcpy(xh, &v, 16);
-                        __builtin_memcpy(wh, &lwp[p], 16);
+            for (int i = 0; i < R; i++) ss[i] = 0.f;
 #pragma unroll
-                        for (int e = 0; e < 8; e++) {
-                            // the fp32 product is rounded before it is converted, as in rmsnorm_f16_kernel (see there)
-                            float pr = __half2float(xh[e]) * rr * __half2float(wh[e]);
-                            asm volatile("" : "+v"(pr));
-                            xh[e] = __float2half_rn(pr);
-                        }
-                        __builtin_memcpy(&v, xh, 16);
-                        *slot = v;
+            for (int p = 0; p < PIECES; p++)
+#pragma unroll
+                for (int i = 0; i < R; i++) add_squares8(v[i][p], ss[i]); // (pieces past the row are zeros: +0 leaves a sum as it is)
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1)
+#pragma unroll
+                for (int i = 0; i < R; i++) ss[i] += __shfl_xor(ss[i], o);
+            float rr[R];
+#pragma unroll
+            for (int i = 0; i < R; i++) rr[i] = 1.0f / sqrtf(ss[i] / (float)a.k + a.ln_eps); // rstd_from_sum's formula
+#pragma unroll
+            for (int p = 0; p < PIECES; p++) {
+                __half wh[8];
+                __builtin_memcpy(wh, &lwp[p], 16);
+                __half xh[R][8];
+#pragma unroll
+                for (int i = 0; i < R; i++) __builtin_memcpy(xh[i], &v[i][p], 16);
+#pragma unroll
+                for (int e = 0; e < 8; e++)
+#pragma unroll
+                    for (int i = 0; i < R; i++) {
+                        // the fp32 product is rounded before it is converted, as in rmsnorm_f16_kernel (see there)
+                        float pr = __half2float(xh[i][e]) * rr[i] * __half2float(wh[e]);
+                        asm volatile("" : "+v"(pr));
+                        xh[i][e] = __float2half_rn(pr);
                     }
-                }
+#pragma unroll
+                for (int i = 0; i < R; i++) __builtin_memcpy(&v[i][p], xh[i], 16);
+            }
+        }
+#pragma unroll
+        for (int p = 0; p < PIECES; p++) {
+            const int e0 = lane * 8 + p * 512;
+            if (e0 < a.k) {
+#pragma unroll
+                for (int i = 0; i < R; i++) *reinterpret_cast<lu32x4 *>(xs + (size_t)(wave + i * WAVES) * pitch + e0 * 2) = v[i][p];
             }
         }
     }
     __syncthreads();
-    const int out_tile = SPLIT ? (int)blockIdx.x : (int)blockIdx.x * WAVES + wave;
     if (out_tile >= a.up_tile_offset) return; // SPLIT: never; otherwise the last block's spare waves (uniform per wave)
-    const int per = SPLIT ? (a.ksteps + WAVES - 1) / WAVES : a.ksteps;
-    const int ks0 = SPLIT ? wave * per : 0, ks1 = min(a.ksteps, ks0 + per);
-    const int tile[2] = {out_tile, out_tile + a.up_tile_offset};
     f32x4v acc[G][MT];
 #pragma unroll
     for (int g = 0; g < G; g++)
@@ -417,16 +433,17 @@ template <int MT, int G, int WAVES, bool SPLIT = false> __global__ __launch_boun
     uint2 res_pre = uint2{0u, 0u};
     if (SPLIT && a.residual) // (the token tile this wave finishes)
         res_pre = *reinterpret_cast<const uint2 *>(a.residual + (size_t)min(min(wave, MT - 1) * 16 + i16, a.m - 1) * a.n_out + out_tile * 16 + kg * 4);
-    for (int kb = ks0; kb < ks1; kb += kRowsBatch) {
-        lu32x4 wv[kRowsBatch][G];
+    for (int kb = ks0; kb < ks1; kb += KB) {
+        if (kb != ks0) { // (the first batch is on its way since the start)
 #pragma unroll
-        for (int u = 0; u < kRowsBatch; u++) {
-            const int ks = min(kb + u, ks1 - 1); // steps past the end re-read the last one and are not multiplied
+            for (int u = 0; u < KB; u++) {
+                const int ks = min(kb + u, ks1 - 1); // steps past the end re-read the last one and are not multiplied
 #pragma unroll
-            for (int g = 0; g < G; g++) wv[u][g] = a.w[((size_t)tile[g] * a.ksteps + ks) * 64 + lane];
+                for (int g = 0; g < G; g++) wv[u][g] = a.w[((size_t)tile[g] * a.ksteps + ks) * 64 + lane];
+            }
         }
 #pragma unroll
-        for (int u = 0; u < kRowsBatch; u++) {
+        for (int u = 0; u < KB; u++) {
             if (kb + u < ks1) { // uniform
                 h16x8 x0[MT], x1[MT];
 #pragma unroll
@@ -693,30 +710,76 @@ static int launch_w8a16_gemm(nncase_hip_ctx_t *ctx, const void *a_dev, const nnc
     const bool glu = mode == NNCASE_HIP_GEMM_SWIGLU;
     // a tile per wave with the token rows shared through LDS: where the rows fit and the launch has a tile for every
     // compute unit (measured on the decode step: the 72- and 56-tile products are quicker with the reduction split
-    // over a block's waves, 9.7 against 11.2 us; the 304 gate / up tile pairs take 12.5 us in 38 blocks of eight waves,
-    // 13.9 us in 76 blocks of four and 18 us split)
+    // over a block's waves, 9.7 against 11.2 us; the 304 gate / up tile pairs take 11.4 us in 38 blocks of eight waves
+    // with a pair per wave, 10.7 us in 304 blocks of four waves that split a pair's reduction, 12.8 us in blocks of
+    // eight.  What the launches cost is not the weights' trip to memory but what every block repeats: the rows' trip,
+    // 1.2 us, their normalisation, 0.3 us of vector issue per row and SIMD, and, with a pair per wave, 0.24 us of
+    // conversions and matrix instructions per k-step on a SIMD that two waves share)
     const int mt_built = mt <= 1 ? 1 : (mt == 2 ? 2 : 4);
     const size_t rows_lds = (size_t)mt_built * 16 * rows_in_lds_pitch(w->k);
+    const bool short_rows = w->k <= 1024; // rows of two 512-element pieces (a lane keeps a row's pieces in registers)
+    if (split && glu && w->k <= kRowsMaxK && rows_lds <= 64 * 1024 && mt_built <= 2 && // (with or without rows to normalise: one summation order)
+        (w->ksteps + kGluSplitWaves - 1) / kGluSplitWaves <= 4) {
+        // the gate / up projection of a decode step (a few hundred tile pairs over a short reduction): a block per tile
+        // pair, its waves splitting the reduction, so that every compute unit takes part
+        constexpr int GW = kGluSplitWaves;
+        const dim3 gblock(GW * 64);
+#define NNHIP_GLU_SPLIT_LAUNCH(MTV, PV)                                                                                        \
+    do {                                                                                                                       \
+        NNHIP_HIP(ctx, raise_dynamic_lds(w8a16_gemm_rows_in_lds_kernel<MTV, 2, GW, true, 4, PV>, ctx->device,                 \
+                                         rows_lds + GW * 2 * MTV * 1024, 96 * 1024));                                          \
+        hipLaunchKernelGGL((w8a16_gemm_rows_in_lds_kernel<MTV, 2, GW, true, 4, PV>), grid, gblock, rows_lds, ctx->stream, a); \
+    } while (0)
+        if (mt_built == 1 && short_rows) NNHIP_GLU_SPLIT_LAUNCH(1, 2);
+        else if (mt_built == 1) NNHIP_GLU_SPLIT_LAUNCH(1, kRowsPieces);
+        else if (short_rows) NNHIP_GLU_SPLIT_LAUNCH(2, 2);
+        else NNHIP_GLU_SPLIT_LAUNCH(2, kRowsPieces);
+#undef NNHIP_GLU_SPLIT_LAUNCH
+        NNHIP_LAUNCH_CHECK(ctx, "w8a16_gemm_rows_in_lds_kernel");
+        return 0;
+    }
     if (split && !glu && ln_weight_dev && w->k <= kRowsMaxK && rows_lds <= 64 * 1024 && mt_built <= 2) {
         // few tiles and rows to normalise (the q / k / v projection): the reduction split over the block's waves, the
         // rows parked and normalised in LDS in one trip to memory
         // (the kernel's static reduction area comes on top of the rows: past 48 KiB in all, the limit is raised like below)
+        // (a wave's share of the reduction is requested at once where it is at most two k-steps, the decode step's case)
+        const bool short_share = (w->ksteps + kGemmWaves - 1) / kGemmWaves <= 2;
+#define NNHIP_SPLIT_ROWS_LAUNCH_P(MTV, KBV, PV)                                                                                \
+    do {                                                                                                                       \
+        NNHIP_HIP(ctx, raise_dynamic_lds(w8a16_gemm_rows_in_lds_kernel<MTV, 1, kGemmWaves, true, KBV, PV>, ctx->device,       \
+                                         rows_lds + MTV * 8 * 1024, 64 * 1024));                                               \
+        hipLaunchKernelGGL((w8a16_gemm_rows_in_lds_kernel<MTV, 1, kGemmWaves, true, KBV, PV>), grid, block, rows_lds, ctx->stream, a); \
+    } while (0)
+#define NNHIP_SPLIT_ROWS_LAUNCH(MTV, KBV)                                                                                      \
+    do {                                                                                                                       \
+        if (short_rows) NNHIP_SPLIT_ROWS_LAUNCH_P(MTV, KBV, 2);                                                                \
+        else NNHIP_SPLIT_ROWS_LAUNCH_P(MTV, KBV, kRowsPieces);                                                                 \
+    } while (0)
         if (mt_built == 1) {
-            NNHIP_HIP(ctx, raise_dynamic_lds(w8a16_gemm_rows_in_lds_kernel<1, 1, kGemmWaves, true>, ctx->device, rows_lds + 8 * 1024, 64 * 1024));
-            hipLaunchKernelGGL((w8a16_gemm_rows_in_lds_kernel<1, 1, kGemmWaves, true>), grid, block, rows_lds, ctx->stream, a);
+            if (short_share) NNHIP_SPLIT_ROWS_LAUNCH(1, 2);
+            else NNHIP_SPLIT_ROWS_LAUNCH(1, kRowsBatch);
         } else {
-            NNHIP_HIP(ctx, raise_dynamic_lds(w8a16_gemm_rows_in_lds_kernel<2, 1, kGemmWaves, true>, ctx->device, rows_lds + 16 * 1024, 64 * 1024));
-            hipLaunchKernelGGL((w8a16_gemm_rows_in_lds_kernel<2, 1, kGemmWaves, true>), grid, block, rows_lds, ctx->stream, a);
+            if (short_share) NNHIP_SPLIT_ROWS_LAUNCH(2, 2);
+            else NNHIP_SPLIT_ROWS_LAUNCH(2, kRowsBatch);
         }
+#undef NNHIP_SPLIT_ROWS_LAUNCH
+#undef NNHIP_SPLIT_ROWS_LAUNCH_P
         NNHIP_LAUNCH_CHECK(ctx, "w8a16_gemm_rows_in_lds_kernel");
         return 0;
     }
     if (w->k <= kRowsMaxK && rows_lds <= 128 * 1024 && out_tiles >= ctx->compute_units) {
         const dim3 rgrid((out_tiles + kGemmWaves - 1) / kGemmWaves), rblock(kGemmThreads);
+        // a reduction of up to 14 k-steps (hidden size 896) is requested whole: one trip to memory for all the weights
+        const bool whole = w->ksteps <= kRowsWhole;
+#define NNHIP_ROWS_LAUNCH_KB(MTV, GV, KBV, PV)                                                                                 \
+    do {                                                                                                                       \
+        NNHIP_HIP(ctx, raise_dynamic_lds(w8a16_gemm_rows_in_lds_kernel<MTV, GV, kGemmWaves, false, KBV, PV>, ctx->device, rows_lds + 1024, 128 * 1024)); \
+        hipLaunchKernelGGL((w8a16_gemm_rows_in_lds_kernel<MTV, GV, kGemmWaves, false, KBV, PV>), rgrid, rblock, rows_lds, ctx->stream, a); \
+    } while (0)
 #define NNHIP_ROWS_LAUNCH(MTV, GV)                                                                                             \
     do {                                                                                                                       \
-        NNHIP_HIP(ctx, raise_dynamic_lds(w8a16_gemm_rows_in_lds_kernel<MTV, GV, kGemmWaves>, ctx->device, rows_lds + 1024, 128 * 1024)); \
-        hipLaunchKernelGGL((w8a16_gemm_rows_in_lds_kernel<MTV, GV, kGemmWaves>), rgrid, rblock, rows_lds, ctx->stream, a);    \
+        if (whole) NNHIP_ROWS_LAUNCH_KB(MTV, GV, kRowsWhole, 2); /* (14 k-steps are 896 elements) */                           \
+        else NNHIP_ROWS_LAUNCH_KB(MTV, GV, kRowsBatch, kRowsPieces);                                                           \
     } while (0)
         if (glu) {
             if (mt_built == 1) NNHIP_ROWS_LAUNCH(1, 2);
@@ -727,18 +790,20 @@ static int launch_w8a16_gemm(nncase_hip_ctx_t *ctx, const void *a_dev, const nnc
             else if (mt_built == 2) NNHIP_ROWS_LAUNCH(2, 1);
             else NNHIP_ROWS_LAUNCH(4, 1);
         }
+#undef NNHIP_ROWS_LAUNCH_KB
 #undef NNHIP_ROWS_LAUNCH
         NNHIP_LAUNCH_CHECK(ctx, "w8a16_gemm_rows_in_lds_kernel");
         return 0;
     }
-    // a share of 9 or 10 k-steps per wave (the 4864-deep down projection): two requests of five instead of 4 + 4 + 2
+    // a share of 9 or 10 k-steps per wave (the 4864-deep down projection): one request of all ten for up to 16 token rows,
+    // two of five for up to 32 (whose slices of ten k-steps do not fit the registers), instead of 4 + 4 + 2
     const int share = (w->ksteps + kGemmWaves - 1) / kGemmWaves;
-    const bool long_share = !ln_weight_dev && mt <= 2 && (share == 5 || share == 9 || share == 10);
+    const bool long_share = !ln_weight_dev && mt <= 2 && (share == 9 || share == 10);
 #define NNHIP_GEMM_LAUNCH(MTV)                                                                                                 \
     do {                                                                                                                       \
         if (glu && split) hipLaunchKernelGGL((w8a16_gemm_kernel<MTV, 2, true>), grid, block, 0, ctx->stream, a);              \
         else if (glu) hipLaunchKernelGGL((w8a16_gemm_kernel<MTV, 2, false>), grid, block, 0, ctx->stream, a);                 \
-        else if (split && long_share) hipLaunchKernelGGL((w8a16_gemm_kernel<(MTV <= 2 ? MTV : 2), 1, true, 5>), grid, block, 0, ctx->stream, a); \
+        else if (split && long_share) hipLaunchKernelGGL((w8a16_gemm_kernel<(MTV <= 2 ? MTV : 2), 1, true, (MTV == 1 ? 10 : 5)>), grid, block, 0, ctx->stream, a); \
         else if (split) hipLaunchKernelGGL((w8a16_gemm_kernel<MTV, 1, true>), grid, block, 0, ctx->stream, a);                \
         else hipLaunchKernelGGL((w8a16_gemm_kernel<MTV, 1, false>), grid, block, 0, ctx->stream, a);                          \
     } while (0)

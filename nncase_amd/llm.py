@@ -70,7 +70,7 @@ class HipDecoder:
 
     def __init__(self, ctx: Context, cfg: DecoderConfig, weights: Dict[str, object], batch: int, max_blocks_per_seq: int,
                  block_table: np.ndarray, ctx_lens: np.ndarray, k_caches: List[np.ndarray], v_caches: List[np.ndarray],
-                 capture_graph: bool = True, feedback: bool = False, fuse_norm: bool = True):
+                 capture_graph: bool = True, feedback: bool = False, fuse_norm: bool = True, lanes: int = 1):
         self.ctx, self.cfg, self.batch = ctx, cfg, batch
         c = cfg
         qd, kvd = c.q_heads * c.head_dim, c.kv_heads * c.head_dim
@@ -95,43 +95,67 @@ class HipDecoder:
         self.attn_args = rt.PagedAttnArgs(batch, c.q_heads, c.kv_heads, c.head_dim, c.block_size, max_blocks_per_seq, num_blocks,
                                           float(c.head_dim ** -0.5), rt.DT_F16, 1)
         self.layers = []
+        assert batch % lanes == 0, "lanes split the batch evenly"
+        self.lanes = lanes
+        bl = batch // lanes
+        lane_args = rt.PagedAttnArgs(bl, c.q_heads, c.kv_heads, c.head_dim, c.block_size, max_blocks_per_seq, num_blocks,
+                                     float(c.head_dim ** -0.5), rt.DT_F16, 1)
+        lane_geometry = rt.PagedAttnArgs(bl, c.q_heads, c.kv_heads, c.head_dim, c.block_size, max_blocks_per_seq, num_blocks,
+                                         float(c.head_dim ** -0.5), rt.DT_F16)
+        for lw in weights["layers"]:
+            self.layers.append({"ln1": ctx.to_device(lw["ln1"]), "ln2": ctx.to_device(lw["ln2"]),
+                                "qkv": ctx.prepack_w8a16(lw["qkv"][0], lw["qkv"][1], lw["qkv_bias"]), "o": ctx.prepack_w8a16(*lw["o"]),
+                                "gate_up": ctx.prepack_w8a16(*lw["gate_up"]), "down": ctx.prepack_w8a16(*lw["down"])})
+        for li, L in enumerate(self.layers):
+            L["k"] = ctx.to_device(np.ascontiguousarray(k_caches[li], np.float16))
+            L["v"] = ctx.to_device(np.ascontiguousarray(v_caches[li], np.float16))
         fn = Function(ctx)
-        fn.add_embedding_f16(self.embedding, self.tokens, self.x[0], batch, c.hidden, c.vocab)
-        for li, lw in enumerate(weights["layers"]):
-            L = {"ln1": ctx.to_device(lw["ln1"]), "ln2": ctx.to_device(lw["ln2"]),
-                 "qkv": ctx.prepack_w8a16(lw["qkv"][0], lw["qkv"][1], lw["qkv_bias"]), "o": ctx.prepack_w8a16(*lw["o"]),
-                 "gate_up": ctx.prepack_w8a16(*lw["gate_up"]), "down": ctx.prepack_w8a16(*lw["down"]),
-                 "k": ctx.to_device(np.ascontiguousarray(k_caches[li], np.float16)),
-                 "v": ctx.to_device(np.ascontiguousarray(v_caches[li], np.float16))}
-            self.layers.append(L)
-            x, h = self.x[0], self.x[1]
-            # the three normalisations run inside the products that consume them (fuse_norm), or as operators of their own
-            if fuse_norm:
-                fn.add_rmsnorm_w8a16_gemm(x, L["ln1"], c.rms_eps, L["qkv"], self.qkv, batch)
-            else:
-                fn.add_rmsnorm_f16(x, L["ln1"], self.norm, batch, c.hidden, c.rms_eps)
-                fn.add_w8a16_gemm(self.norm, L["qkv"], self.qkv, batch)
-            fn.add_rope_kv_append(self.qkv, self.q, L["k"], L["v"], self.block_table, self.ctx_lens, self.geometry, c.rope_theta)
-            # the appended token takes part in its own attention (lengths + 1); the lengths themselves advance
-            # once, at the end of the step
-            fn.add_paged_attention_decode(self.q, L["k"], L["v"], self.block_table, self.ctx_lens, self.att, self.attn_args)
-            fn.add_w8a16_gemm(self.att, L["o"], h, batch, residual=x)
-            if fuse_norm:
-                fn.add_rmsnorm_w8a16_gemm(h, L["ln2"], c.rms_eps, L["gate_up"], self.act, batch, mode=rt.GEMM_SWIGLU)
-            else:
-                fn.add_rmsnorm_f16(h, L["ln2"], self.norm, batch, c.hidden, c.rms_eps)
-                fn.add_w8a16_gemm(self.norm, L["gate_up"], self.act, batch, mode=rt.GEMM_SWIGLU)
-            fn.add_w8a16_gemm(self.act, L["down"], x, batch, residual=h)
-        if fuse_norm:
-            fn.add_rmsnorm_w8a16_gemm(self.x[0], self.ln_f, c.rms_eps, self.lm_head, self.logits, batch, out_dtype=rt.DT_F32)
-        else:
-            fn.add_rmsnorm_f16(self.x[0], self.ln_f, self.norm, batch, c.hidden, c.rms_eps)
-            fn.add_w8a16_gemm(self.norm, self.lm_head, self.logits, batch, out_dtype=rt.DT_F32)
         # feedback: the arg-max lands in the token buffer the next step's embedding reads (greedy generation
         # without a host round trip); otherwise the caller feeds every step's tokens
         self.feedback = feedback
-        fn.add_argmax_f32(self.logits, self.tokens if feedback else self.next_tokens, batch, c.vocab)
-        fn.add_add_i32(self.ctx_lens, batch, 1)   # the step is complete: the caches hold one more token
+        # lanes > 1: the sequences are split into that many equal ranges and the whole step is recorded once per range,
+        # each on a lane of its own; a captured step replays the lanes side by side, so the launch and memory latency
+        # of one range's short kernels is covered by the other ranges' kernels.  Every range reads the same weights and
+        # owns its rows of every buffer, so the result is that of lanes == 1 row for row.
+        for lane in range(lanes):
+            if lanes > 1:
+                fn.set_lane(lane)
+
+            def R(buf, row_bytes):                  # this lane's rows of a [batch, ...] buffer
+                return buf if lanes == 1 else buf.view(lane * bl * row_bytes, bl * row_bytes)
+
+            tokens, next_tokens, ctx_lens = R(self.tokens, 4), R(self.next_tokens, 4), R(self.ctx_lens, 4)
+            block_table = R(self.block_table, max_blocks_per_seq * 4)
+            xs = [R(self.x[0], c.hidden * f16), R(self.x[1], c.hidden * f16)]
+            norm, qkv, q = R(self.norm, c.hidden * f16), R(self.qkv, (qd + 2 * kvd) * f16), R(self.q, qd * f16)
+            att, act, logits = R(self.att, qd * f16), R(self.act, c.mlp * f16), R(self.logits, c.vocab * 4)
+            fn.add_embedding_f16(self.embedding, tokens, xs[0], bl, c.hidden, c.vocab)
+            for L in self.layers:
+                x, h = xs[0], xs[1]
+                # the three normalisations run inside the products that consume them (fuse_norm), or as operators of their own
+                if fuse_norm:
+                    fn.add_rmsnorm_w8a16_gemm(x, L["ln1"], c.rms_eps, L["qkv"], qkv, bl)
+                else:
+                    fn.add_rmsnorm_f16(x, L["ln1"], norm, bl, c.hidden, c.rms_eps)
+                    fn.add_w8a16_gemm(norm, L["qkv"], qkv, bl)
+                fn.add_rope_kv_append(qkv, q, L["k"], L["v"], block_table, ctx_lens, lane_geometry, c.rope_theta)
+                # the appended token takes part in its own attention (lengths + 1); the lengths themselves advance
+                # once, at the end of the step
+                fn.add_paged_attention_decode(q, L["k"], L["v"], block_table, ctx_lens, att, lane_args)
+                fn.add_w8a16_gemm(att, L["o"], h, bl, residual=x)
+                if fuse_norm:
+                    fn.add_rmsnorm_w8a16_gemm(h, L["ln2"], c.rms_eps, L["gate_up"], act, bl, mode=rt.GEMM_SWIGLU)
+                else:
+                    fn.add_rmsnorm_f16(h, L["ln2"], norm, bl, c.hidden, c.rms_eps)
+                    fn.add_w8a16_gemm(norm, L["gate_up"], act, bl, mode=rt.GEMM_SWIGLU)
+                fn.add_w8a16_gemm(act, L["down"], x, bl, residual=h)
+            if fuse_norm:
+                fn.add_rmsnorm_w8a16_gemm(xs[0], self.ln_f, c.rms_eps, self.lm_head, logits, bl, out_dtype=rt.DT_F32)
+            else:
+                fn.add_rmsnorm_f16(xs[0], self.ln_f, norm, bl, c.hidden, c.rms_eps)
+                fn.add_w8a16_gemm(norm, self.lm_head, logits, bl, out_dtype=rt.DT_F32)
+            fn.add_argmax_f32(logits, tokens if feedback else next_tokens, bl, c.vocab)
+            fn.add_add_i32(ctx_lens, bl, 1)   # the step is complete: the caches hold one more token
         self.fn = fn
         # nothing to warm up: recording the attention operators has already sized their workspace
         if capture_graph:

@@ -215,17 +215,18 @@ def make_state(cfg, rng, batch, max_ctx):
     return max_blocks, lens, bt, kcs, vcs
 
 
-@pytest.mark.parametrize("capture", [False, True])
-def test_decode_steps_small_model(hip_ctx, capture):
+@pytest.mark.parametrize("capture,lanes", [(False, 1), (True, 1), (True, 2), (False, 3)])
+def test_decode_steps_small_model(hip_ctx, capture, lanes):
     """Three greedy steps of a 3-layer model (Qwen2 head geometry, reduced widths) against the float64 step:
     logits to 1e-3, the same tokens whenever the float64 top-2 margin exceeds the tolerance, and the caches
-    the steps leave behind."""
+    the steps leave behind.  lanes > 1: the six sequences recorded as that many independent chains (each with
+    its own rows of every buffer and its own attention scratch), replayed side by side when captured."""
     cfg = llm.DecoderConfig(layers=3, hidden=256, q_heads=4, kv_heads=2, head_dim=64, mlp=512, vocab=2048)
     rng = np.random.default_rng(12)
     weights = llm.random_weights(cfg, seed=3)
     batch = 6
     max_blocks, lens, bt, kcs, vcs = make_state(cfg, rng, batch, 90)
-    dec = llm.HipDecoder(hip_ctx, cfg, weights, batch, max_blocks, bt, lens, kcs, vcs, capture_graph=capture)
+    dec = llm.HipDecoder(hip_ctx, cfg, weights, batch, max_blocks, bt, lens, kcs, vcs, capture_graph=capture, lanes=lanes)
     ref_k, ref_v = [k.copy() for k in kcs], [v.copy() for v in vcs]
     ref_lens = lens.copy()
     tokens = rng.integers(0, cfg.vocab, batch).astype(np.int32)
@@ -248,7 +249,8 @@ def test_decode_steps_small_model(hip_ctx, capture):
         close(dec.layers[li]["v"].download(vcs[li].shape, np.float16).reshape(-1, cfg.block_size), ref_v[li].reshape(-1, cfg.block_size), atol=4e-3)
 
 
-def test_decode_step_at_the_benchmark_shape(hip_ctx):
+@pytest.mark.parametrize("lanes", [1, 2])
+def test_decode_step_at_the_benchmark_shape(hip_ctx, lanes):
     """One greedy step of the decode benchmark's own model and state (24 layers, hidden 896, 14 query / 2 KV heads of 64,
     MLP 4864, vocabulary 151 936, batch 32, context lengths uniform in [512, 4096], one random cache image per layer) against
     the float64 step.  Twenty-four layers of fp16 storage amplify last-bit differences of the sums (a sum that differs in
@@ -267,7 +269,7 @@ def test_decode_step_at_the_benchmark_shape(hip_ctx):
     bt = rng.permutation(nblocks).reshape(batch, max_blocks).astype(np.int32)
     kc = rng.standard_normal((nblocks, cfg.kv_heads, cfg.block_size, cfg.head_dim), dtype=np.float32).astype(np.float16)
     vc = rng.standard_normal((nblocks, cfg.kv_heads, cfg.head_dim, cfg.block_size), dtype=np.float32).astype(np.float16)
-    dec = llm.HipDecoder(hip_ctx, cfg, weights, batch, max_blocks, bt, lens, [kc] * cfg.layers, [vc] * cfg.layers, capture_graph=True)
+    dec = llm.HipDecoder(hip_ctx, cfg, weights, batch, max_blocks, bt, lens, [kc] * cfg.layers, [vc] * cfg.layers, capture_graph=True, lanes=lanes)
     tokens = rng.integers(0, cfg.vocab, batch).astype(np.int32)
     dec.set_tokens(tokens)
     dec.step()
