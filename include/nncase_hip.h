@@ -502,6 +502,17 @@ NNCASE_HIP_API int nncase_hip_rmsnorm_f16(nncase_hip_ctx_t *ctx, const void *x_d
 NNCASE_HIP_API int nncase_hip_rope_kv_append(nncase_hip_ctx_t *ctx, const void *qkv_dev, void *q_out_dev, void *k_cache_dev,
                                              void *v_cache_dev, const int32_t *block_table_dev, const int32_t *ctx_lens_dev,
                                              const nncase_hip_paged_attn_args_t *geometry, float rope_theta);
+/* The q / k / v projection of (optionally RMS-normalised, ln_weight_dev may be null) rows x, followed by
+ * nncase_hip_rope_kv_append, as one launch where the geometry allows (up to 32 rows, head_dim a multiple of 32, a
+ * reduction of up to 1024): the block that multiplies a tile of a head also multiplies the tile half a head further,
+ * so the rotate-half pairs meet in its epilogue.  The values are those of nncase_hip_rmsnorm_w8a16_gemm (or
+ * nncase_hip_w8a16_gemm) into fp16 followed by nncase_hip_rope_kv_append, bit for bit; qkv_dev [batch, (Hq + 2 Hkv) * d]
+ * is scratch that the two-launch form of other geometries writes. */
+NNCASE_HIP_API int nncase_hip_w8a16_gemm_rope_kv_append(nncase_hip_ctx_t *ctx, const void *x_dev, const void *ln_weight_dev,
+                                                        float eps, const nncase_hip_w8a16_t *weights, void *qkv_dev,
+                                                        void *q_out_dev, void *k_cache_dev, void *v_cache_dev,
+                                                        const int32_t *block_table_dev, const int32_t *ctx_lens_dev,
+                                                        const nncase_hip_paged_attn_args_t *geometry, float rope_theta);
 /* out[r] = index of the largest element of row r (the lowest index among equals). */
 NNCASE_HIP_API int nncase_hip_argmax_f32(nncase_hip_ctx_t *ctx, const float *x_dev, int32_t *out_dev, int32_t rows, int32_t cols);
 /* out[r, :] = table[ids[r], :] (fp16 rows). */
@@ -592,6 +603,13 @@ NNCASE_HIP_API int nncase_hip_function_add_rope_kv_append(nncase_hip_function_t 
                                                           void *k_cache_dev, void *v_cache_dev, const int32_t *block_table_dev,
                                                           const int32_t *ctx_lens_dev,
                                                           const nncase_hip_paged_attn_args_t *geometry, float rope_theta);
+NNCASE_HIP_API int nncase_hip_function_add_w8a16_gemm_rope_kv_append(nncase_hip_function_t *fn, const void *x_dev,
+                                                                     const void *ln_weight_dev, float eps,
+                                                                     const nncase_hip_w8a16_t *weights, void *qkv_dev,
+                                                                     void *q_out_dev, void *k_cache_dev, void *v_cache_dev,
+                                                                     const int32_t *block_table_dev, const int32_t *ctx_lens_dev,
+                                                                     const nncase_hip_paged_attn_args_t *geometry,
+                                                                     float rope_theta);
 NNCASE_HIP_API int nncase_hip_function_add_paged_attention_decode(nncase_hip_function_t *fn, const void *q_dev,
                                                                   const void *k_cache_dev, const void *v_cache_dev,
                                                                   const int32_t *block_table_dev, const int32_t *ctx_lens_dev,

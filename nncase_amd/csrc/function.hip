@@ -9,7 +9,7 @@ namespace {
 
 struct Op {
     enum Kind { kQuantize, kDequantize, kConv, kAdd, kPool, kLut, kConcat, kResize, kMaxPool, kPack, kQuantPack,
-                kGemm, kRmsNorm, kRope, kAttn, kArgmax, kEmbed, kAddI32, kBlock, kLayout } kind;
+                kGemm, kRmsNorm, kRope, kGemmRope, kAttn, kArgmax, kEmbed, kAddI32, kBlock, kLayout } kind;
     const void *in0 = nullptr, *in1 = nullptr;
     void *out = nullptr;
     const nncase_hip_weights_t *weights = nullptr;
@@ -35,7 +35,7 @@ struct Op {
     void *out2 = nullptr, *out3 = nullptr;
     nncase_hip_paged_attn_args_t attn{};
     int32_t mode = 0, delta = 0;
-    float eps = 0.f;
+    float eps = 0.f, theta = 0.f;
     const nncase_hip_qblock_t *block = nullptr;
     nncase_hip_qblock_args_t blk{};
     int lane = 0; // independent operator chain this operator belongs to
@@ -93,6 +93,9 @@ static int run_op(nncase_hip_function *fn, const Op &op) {
         return nncase_hip_w8a16_gemm(ctx, op.in0, op.w8, op.out, op.batch, op.mode, op.in1, op.dt_out);
     case Op::kRmsNorm:
         return nncase_hip_rmsnorm_f16(ctx, op.in0, op.in1, op.out, op.batch, op.channels, op.eps);
+    case Op::kGemmRope: // in0 rows, in1 normalisation weights, out the qkv scratch, out2 / out3 the caches, in2 block table, in3 lengths, in4 the query buffer
+        return nncase_hip_w8a16_gemm_rope_kv_append(ctx, op.in0, op.in1, op.eps, op.w8, op.out, const_cast<void *>(op.in4), op.out2, op.out3,
+                                                    (const int32_t *)op.in2, (const int32_t *)op.in3, &op.attn, op.theta);
     case Op::kRope:
         return nncase_hip_rope_kv_append(ctx, op.in0, op.out, op.out2, op.out3, (const int32_t *)op.in2, (const int32_t *)op.in3,
                                          &op.attn, op.eps);
@@ -376,6 +379,22 @@ extern "C" int nncase_hip_function_add_rope_kv_append(nncase_hip_function_t *fn,
     return push(fn, op);
 }
 
+extern "C" int nncase_hip_function_add_w8a16_gemm_rope_kv_append(nncase_hip_function_t *fn, const void *x_dev, const void *ln_weight_dev,
+                                                                 float eps, const nncase_hip_w8a16_t *weights, void *qkv_dev,
+                                                                 void *q_out_dev, void *k_cache_dev, void *v_cache_dev,
+                                                                 const int32_t *block_table_dev, const int32_t *ctx_lens_dev,
+                                                                 const nncase_hip_paged_attn_args_t *geometry, float rope_theta) {
+    if (!fn) return -EINVAL;
+    NNHIP_REQUIRE(fn->ctx, x_dev && weights && qkv_dev && q_out_dev && k_cache_dev && v_cache_dev && block_table_dev && ctx_lens_dev && geometry,
+                  -EINVAL, "function_add_w8a16_gemm_rope_kv_append: null argument");
+    Op op;
+    op.kind = Op::kGemmRope;
+    op.in0 = x_dev, op.in1 = ln_weight_dev, op.eps = eps, op.w8 = weights, op.out = qkv_dev, op.in4 = q_out_dev;
+    op.out2 = k_cache_dev, op.out3 = v_cache_dev, op.in2 = block_table_dev, op.in3 = ctx_lens_dev;
+    op.attn = *geometry, op.theta = rope_theta;
+    return push(fn, op);
+}
+
 extern "C" int nncase_hip_function_add_paged_attention_decode(nncase_hip_function_t *fn, const void *q_dev, const void *k_cache_dev,
                                                               const void *v_cache_dev, const int32_t *block_table_dev,
                                                               const int32_t *ctx_lens_dev, void *out_dev,
@@ -575,6 +594,7 @@ extern "C" int nncase_hip_function_op_kernel(nncase_hip_function_t *fn, int32_t 
         break;
     case Op::kRmsNorm: snprintf(name, capacity, "rmsnorm_f16"); break;
     case Op::kRope: snprintf(name, capacity, "rope_kv_append"); break;
+    case Op::kGemmRope: snprintf(name, capacity, "%sw8a16_gemm+rope_kv_append", op.in1 ? "rmsnorm+" : ""); break;
     case Op::kAttn: snprintf(name, capacity, "paged_attention_decode"); break;
     case Op::kArgmax: snprintf(name, capacity, "argmax_f32"); break;
     case Op::kEmbed: snprintf(name, capacity, "embedding_f16"); break;

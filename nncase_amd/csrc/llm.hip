@@ -44,6 +44,16 @@ struct nncase_hip_w8a16 {
 
 namespace nnhip {
 
+struct RopeArgs {
+    const __half *qkv; // [batch][(hq + 2 * hkv) * d]: q heads, then k heads, then v heads
+    __half *q_out;     // [batch][hq][d]
+    __half *k_cache;   // [blocks][hkv][block][d]
+    __half *v_cache;   // [blocks][hkv][d][block]
+    const int32_t *block_table, *ctx_lens; // the new token of sequence b goes to position ctx_lens[b]
+    int batch, hq, hkv, d, block_size, max_blocks, num_blocks;
+    float theta;
+};
+
 struct GemmArgs {
     const uint16_t *a; // [m][k] fp16
     const lu32x4 *w;
@@ -57,6 +67,9 @@ struct GemmArgs {
     // fp16(x * r * weight) as it is loaded, so the result is what the two kernels give one after the other
     const uint16_t *ln_w; // [k] fp16
     float ln_eps;
+    // ROPE kernels: the product is a q / k / v projection whose rows do not go to `out` but, rotated, to the query buffer
+    // and the paged cache (rope.qkv unused)
+    RopeArgs rope;
 };
 
 // 1 / sqrt(mean(x^2) + eps) of a row, the way every kernel here forms it.  A lane owns the 8 consecutive elements
@@ -109,6 +122,35 @@ __device__ __forceinline__ float rms_rstd_scalar(const __half *xr, int hidden, f
                 ss += f * f;
             }
     return rstd_from_sum(ss, hidden, eps);
+}
+
+// One rotate-half pair of the new token of sequence b: elements i and i + d/2 of head h (q heads, then k heads, then
+// v heads), given as the fp16 values the projection stores.  q goes rotated to the query buffer, k rotated and v as it
+// is to position ctx_lens[b] of the paged cache.  The one definition of that arithmetic: the rope kernel and the
+// projection that rotates in its own epilogue both call it.
+__device__ __forceinline__ void rope_store_pair(const RopeArgs &a, int b, int h, int i, float x0, float x1) {
+    const int half = a.d / 2;
+    const int pos = a.ctx_lens[b];
+    const int lb = pos / a.block_size, in_block = pos - lb * a.block_size;
+    const bool fits = pos >= 0 && lb < a.max_blocks; // a negative length appends nothing (it would index before the block)
+    const int pb = fits ? min(max(a.block_table[(size_t)b * a.max_blocks + lb], 0), a.num_blocks - 1) : 0;
+    if (h < a.hq + a.hkv) {
+        const float inv = powf(a.theta, -2.0f * (float)i / (float)a.d);
+        const float ang = (float)pos * inv;
+        const float c = cosf(ang), s = sinf(ang);
+        const __half y0 = __float2half_rn(x0 * c - x1 * s), y1 = __float2half_rn(x1 * c + x0 * s);
+        if (h < a.hq) {
+            __half *dst = a.q_out + ((size_t)b * a.hq + h) * a.d;
+            dst[i] = y0, dst[i + half] = y1;
+        } else if (fits) {
+            __half *dst = a.k_cache + ((((size_t)pb * a.hkv + (h - a.hq)) * a.block_size) + in_block) * a.d;
+            dst[i] = y0, dst[i + half] = y1;
+        }
+    } else if (fits) {
+        __half *dst = a.v_cache + ((size_t)pb * a.hkv + (h - a.hq - a.hkv)) * a.d * a.block_size + in_block;
+        dst[(size_t)i * a.block_size] = __float2half_rn(x0);
+        dst[(size_t)(i + half) * a.block_size] = __float2half_rn(x1);
+    }
 }
 
 // 8 int8 weights (two dwords' low / high halves handled by the caller) -> 8 fp16, exact.
@@ -332,8 +374,13 @@ inline int rows_in_lds_pitch(int k) { return k * 2 + 16; } // bytes per token ro
 
 // SPLIT: the block's waves share ONE output tile and split its reduction (few tiles: the q / k / v projection), combined
 // through LDS in the fixed order of the kernel above.
-template <int MT, int G, int WAVES, bool SPLIT = false, int KB = kRowsBatch, int PIECES = kRowsPieces>
+// ROPE (with SPLIT and G = 2): a q / k / v projection whose block owns the two tiles that hold the halves of eight
+// rotate-half pairs -- tile j of a head and tile j + up_tile_offset (= head_dim / 32) -- so that a lane ends up with
+// both elements of its four pairs; the epilogue rounds them to fp16 as the projection's output would be stored and
+// hands them to rope_store_pair.
+template <int MT, int G, int WAVES, bool SPLIT = false, int KB = kRowsBatch, int PIECES = kRowsPieces, bool ROPE = false>
 __global__ __launch_bounds__(WAVES * 64) void w8a16_gemm_rows_in_lds_kernel(const GemmArgs a) {
+    static_assert(!ROPE || (SPLIT && G == 2), "the rotating epilogue pairs two tiles of one block");
     extern __shared__ __attribute__((aligned(16))) uint8_t xs[]; // [MT * 16][k halves + padding]
     __shared__ float red[SPLIT ? WAVES : 1][G][SPLIT ? MT : 1][64][4];
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -342,10 +389,13 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_gemm_rows_in_lds_kernel(cons
     // The weights do not depend on the rows: the first KB k-steps of this wave's share are requested before anything
     // else, so that their trip to memory runs beside the one that brings the rows in (a spare wave of the last block
     // reads the last tile's and multiplies nothing).
-    const int out_tile = SPLIT ? (int)blockIdx.x : (int)blockIdx.x * WAVES + wave;
+    const int out_tile = ROPE    ? ((int)blockIdx.x / a.up_tile_offset) * (2 * a.up_tile_offset) + (int)blockIdx.x % a.up_tile_offset
+                         : SPLIT ? (int)blockIdx.x
+                                 : (int)blockIdx.x * WAVES + wave;
     const int per = SPLIT ? (a.ksteps + WAVES - 1) / WAVES : a.ksteps;
     const int ks0 = SPLIT ? wave * per : 0, ks1 = min(a.ksteps, ks0 + per);
-    const int tile[2] = {min(out_tile, a.up_tile_offset - 1), min(out_tile, a.up_tile_offset - 1) + a.up_tile_offset};
+    const int first = ROPE ? out_tile : min(out_tile, a.up_tile_offset - 1);
+    const int tile[2] = {first, first + a.up_tile_offset};
     lu32x4 wv[KB][G];
 #pragma unroll
     for (int u = 0; u < KB; u++) {
@@ -416,7 +466,7 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_gemm_rows_in_lds_kernel(cons
         }
     }
     __syncthreads();
-    if (out_tile >= a.up_tile_offset) return; // SPLIT: never; otherwise the last block's spare waves (uniform per wave)
+    if (!ROPE && out_tile >= a.up_tile_offset) return; // SPLIT: never; otherwise the last block's spare waves (uniform per wave)
     f32x4v acc[G][MT];
 #pragma unroll
     for (int g = 0; g < G; g++)
@@ -471,6 +521,32 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_gemm_rows_in_lds_kernel(cons
 #pragma unroll
                 for (int r = 0; r < 4; r++) red[wave][g][t][lane][r] = acc[g][t][r];
         __syncthreads();
+        if constexpr (ROPE) {
+            // The rotation costs a few hundred instructions per pair (the angle's power, sine and cosine), so the
+            // pairs are spread over all the waves: wave w takes channel w % 4 of each lane's four, token tile w / 4.
+            static_assert(WAVES == 8, "channel w % 4, token tile w / 4");
+            const int t = wave >> 2, r = wave & 3;
+            const int m = t * 16 + i16;
+            if (t >= MT || m >= a.m) return;
+            float v2[2];
+#pragma unroll
+            for (int g = 0; g < 2; g++) {
+                const float scv[4] = {sc[g].x, sc[g].y, sc[g].z, sc[g].w}, bsv[4] = {bs[g].x, bs[g].y, bs[g].z, bs[g].w};
+                float s = 0.f;
+#pragma unroll
+                for (int w = 0; w < WAVES; w++) s += red[w][g][t][lane][r]; // fixed order, as below
+                float sv = scv[0], bv = bsv[0];
+#pragma unroll
+                for (int q = 1; q < 4; q++) sv = r == q ? scv[q] : sv, bv = r == q ? bsv[q] : bv;
+                s *= sv;
+                if (a.bias) s += bv;
+                v2[g] = s;
+            }
+            // (rounded to fp16 as the projection's output would be stored; the partner is d / 2 channels further)
+            const int c = out_tile * 16 + kg * 4 + r;
+            rope_store_pair(a.rope, m, c / a.rope.d, c % a.rope.d, __half2float(__float2half_rn(v2[0])), __half2float(__float2half_rn(v2[1])));
+            return;
+        }
         if (wave >= MT) return; // wave w finishes token tile w
     }
     // lane (i16 = token within the tile, kg): channels tile * 16 + kg * 4 + r
@@ -525,16 +601,6 @@ __global__ __launch_bounds__(kLlmThreads) void rmsnorm_f16_kernel(const __half *
     }
 }
 
-struct RopeArgs {
-    const __half *qkv; // [batch][(hq + 2 * hkv) * d]: q heads, then k heads, then v heads
-    __half *q_out;     // [batch][hq][d]
-    __half *k_cache;   // [blocks][hkv][block][d]
-    __half *v_cache;   // [blocks][hkv][d][block]
-    const int32_t *block_table, *ctx_lens; // the new token of sequence b goes to position ctx_lens[b]
-    int batch, hq, hkv, d, block_size, max_blocks, num_blocks;
-    float theta;
-};
-
 // Rotary embedding (rotate-half pairing: element i with i + d/2, angle pos * theta^(-2i/d)) of the q
 // and k heads of the new token, and the append of the rotated k and of v at position ctx_lens[b]
 // of the paged cache.  One thread per (sequence, head, pair).
@@ -545,28 +611,7 @@ __global__ __launch_bounds__(kLlmThreads) void rope_append_kernel(const RopeArgs
     if (gid >= a.batch * heads * half) return;
     const int i = gid % half, h = (gid / half) % heads, b = gid / (half * heads);
     const __half *src = a.qkv + ((size_t)b * heads + h) * a.d;
-    const float x0 = __half2float(src[i]), x1 = __half2float(src[i + half]);
-    const int pos = a.ctx_lens[b];
-    const int lb = pos / a.block_size, in_block = pos - lb * a.block_size;
-    const bool fits = pos >= 0 && lb < a.max_blocks; // a negative length appends nothing (it would index before the block)
-    const int pb = fits ? min(max(a.block_table[(size_t)b * a.max_blocks + lb], 0), a.num_blocks - 1) : 0;
-    if (h < a.hq + a.hkv) {
-        const float inv = powf(a.theta, -2.0f * (float)i / (float)a.d);
-        const float ang = (float)pos * inv;
-        const float c = cosf(ang), s = sinf(ang);
-        const __half y0 = __float2half_rn(x0 * c - x1 * s), y1 = __float2half_rn(x1 * c + x0 * s);
-        if (h < a.hq) {
-            __half *dst = a.q_out + ((size_t)b * a.hq + h) * a.d;
-            dst[i] = y0, dst[i + half] = y1;
-        } else if (fits) {
-            __half *dst = a.k_cache + ((((size_t)pb * a.hkv + (h - a.hq)) * a.block_size) + in_block) * a.d;
-            dst[i] = y0, dst[i + half] = y1;
-        }
-    } else if (fits) {
-        __half *dst = a.v_cache + ((size_t)pb * a.hkv + (h - a.hq - a.hkv)) * a.d * a.block_size + in_block;
-        dst[(size_t)i * a.block_size] = __float2half_rn(x0);
-        dst[(size_t)(i + half) * a.block_size] = __float2half_rn(x1);
-    }
+    rope_store_pair(a, b, h, i, __half2float(src[i]), __half2float(src[i + half]));
 }
 
 // Index of the largest element of every row (the lowest index among equals); one block of 1024
@@ -674,8 +719,17 @@ template <typename KernelT> static hipError_t raise_dynamic_lds(KernelT kernel, 
     return e;
 }
 
+// Whether the q / k / v projection of this geometry can rotate and append in its own epilogue (else the caller runs
+// the projection and the rope kernel one after the other).
+static bool rope_epilogue_fits(const nncase_hip_w8a16_t *w, int m, const RopeArgs &r) {
+    const int mt_built = m <= 16 ? 1 : 2;
+    return m <= 32 && r.d % 32 == 0 && w->n == (r.hq + 2 * r.hkv) * r.d && w->k <= kRowsMaxK &&
+           (size_t)mt_built * 16 * rows_in_lds_pitch(w->k) <= 64 * 1024 && (w->ksteps + kGemmWaves - 1) / kGemmWaves <= 2;
+}
+
 static int launch_w8a16_gemm(nncase_hip_ctx_t *ctx, const void *a_dev, const nncase_hip_w8a16_t *w, void *out_dev, int32_t m,
-                             int32_t mode, const void *residual_dev, int32_t out_dtype, const void *ln_weight_dev, float ln_eps) {
+                             int32_t mode, const void *residual_dev, int32_t out_dtype, const void *ln_weight_dev, float ln_eps,
+                             const RopeArgs *rope = nullptr) {
     NNHIP_CHECK_CTX(ctx);
     NNHIP_REQUIRE(ctx, a_dev && w && out_dev, -EINVAL, "w8a16_gemm: null argument");
     NNHIP_REQUIRE(ctx, (reinterpret_cast<uintptr_t>(ln_weight_dev) & 15u) == 0, -NNCASE_HIP_ERR_INVALID_MEMORY_LOCATION,
@@ -717,6 +771,26 @@ static int launch_w8a16_gemm(nncase_hip_ctx_t *ctx, const void *a_dev, const nnc
     // conversions and matrix instructions per k-step on a SIMD that two waves share)
     const int mt_built = mt <= 1 ? 1 : (mt == 2 ? 2 : 4);
     const size_t rows_lds = (size_t)mt_built * 16 * rows_in_lds_pitch(w->k);
+    if (rope) {
+        // (the caller has checked rope_epilogue_fits) a block per pair of tiles d / 2 channels apart
+        a.rope = *rope;
+        a.up_tile_offset = rope->d / 32;
+        const dim3 pgrid(w->ntiles / 2), pblock(kGemmThreads);
+        const bool two_pieces = w->k <= 1024;
+#define NNHIP_ROPE_LAUNCH(MTV, PV)                                                                                             \
+    do {                                                                                                                       \
+        NNHIP_HIP(ctx, raise_dynamic_lds(w8a16_gemm_rows_in_lds_kernel<MTV, 2, kGemmWaves, true, 2, PV, true>, ctx->device,   \
+                                         rows_lds + MTV * 16 * 1024, 96 * 1024));                                              \
+        hipLaunchKernelGGL((w8a16_gemm_rows_in_lds_kernel<MTV, 2, kGemmWaves, true, 2, PV, true>), pgrid, pblock, rows_lds, ctx->stream, a); \
+    } while (0)
+        if (mt_built == 1 && two_pieces) NNHIP_ROPE_LAUNCH(1, 2);
+        else if (mt_built == 1) NNHIP_ROPE_LAUNCH(1, kRowsPieces);
+        else if (two_pieces) NNHIP_ROPE_LAUNCH(2, 2);
+        else NNHIP_ROPE_LAUNCH(2, kRowsPieces);
+#undef NNHIP_ROPE_LAUNCH
+        NNHIP_LAUNCH_CHECK(ctx, "w8a16_gemm_rows_in_lds_kernel");
+        return 0;
+    }
     const bool short_rows = w->k <= 1024; // rows of two 512-element pieces (a lane keeps a row's pieces in registers)
     if (split && glu && w->k <= kRowsMaxK && rows_lds <= 64 * 1024 && mt_built <= 2 && // (with or without rows to normalise: one summation order)
         (w->ksteps + kGluSplitWaves - 1) / kGluSplitWaves <= 4) {
@@ -838,25 +912,55 @@ extern "C" int nncase_hip_rmsnorm_f16(nncase_hip_ctx_t *ctx, const void *x_dev, 
     return 0;
 }
 
-extern "C" int nncase_hip_rope_kv_append(nncase_hip_ctx_t *ctx, const void *qkv_dev, void *q_out_dev, void *k_cache_dev,
-                                         void *v_cache_dev, const int32_t *block_table_dev, const int32_t *ctx_lens_dev,
-                                         const nncase_hip_paged_attn_args_t *p, float rope_theta) {
-    NNHIP_CHECK_CTX(ctx);
-    NNHIP_REQUIRE(ctx, qkv_dev && q_out_dev && k_cache_dev && v_cache_dev && block_table_dev && ctx_lens_dev && p, -EINVAL,
+static int make_rope_args(nncase_hip_ctx_t *ctx, const void *qkv_dev, void *q_out_dev, void *k_cache_dev, void *v_cache_dev,
+                          const int32_t *block_table_dev, const int32_t *ctx_lens_dev, const nncase_hip_paged_attn_args_t *p,
+                          float rope_theta, RopeArgs *out) {
+    NNHIP_REQUIRE(ctx, q_out_dev && k_cache_dev && v_cache_dev && block_table_dev && ctx_lens_dev && p, -EINVAL,
                   "rope_kv_append: null argument");
     NNHIP_REQUIRE(ctx, p->batch > 0 && p->num_q_heads > 0 && p->num_kv_heads > 0 && p->head_dim > 0 && p->head_dim % 2 == 0 &&
                            p->block_size > 0 && p->max_blocks_per_seq > 0 && p->num_blocks > 0 && rope_theta > 0.f,
                   -EINVAL, "rope_kv_append: bad geometry");
-    RopeArgs a;
+    RopeArgs &a = *out;
     a.qkv = (const __half *)qkv_dev, a.q_out = (__half *)q_out_dev, a.k_cache = (__half *)k_cache_dev, a.v_cache = (__half *)v_cache_dev;
     a.block_table = block_table_dev, a.ctx_lens = ctx_lens_dev;
     a.batch = p->batch, a.hq = p->num_q_heads, a.hkv = p->num_kv_heads, a.d = p->head_dim, a.block_size = p->block_size;
     a.max_blocks = p->max_blocks_per_seq, a.num_blocks = p->num_blocks, a.theta = rope_theta;
+    return 0;
+}
+
+extern "C" int nncase_hip_rope_kv_append(nncase_hip_ctx_t *ctx, const void *qkv_dev, void *q_out_dev, void *k_cache_dev,
+                                         void *v_cache_dev, const int32_t *block_table_dev, const int32_t *ctx_lens_dev,
+                                         const nncase_hip_paged_attn_args_t *p, float rope_theta) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, qkv_dev, -EINVAL, "rope_kv_append: null argument");
+    RopeArgs a;
+    const int rc = make_rope_args(ctx, qkv_dev, q_out_dev, k_cache_dev, v_cache_dev, block_table_dev, ctx_lens_dev, p, rope_theta, &a);
+    if (rc) return rc;
     const int64_t total = (int64_t)a.batch * (a.hq + 2 * a.hkv) * (a.d / 2);
     NNHIP_REQUIRE(ctx, total < ((int64_t)1 << 31), -EINVAL, "rope_kv_append: too large");
     hipLaunchKernelGGL(rope_append_kernel, dim3((unsigned)((total + kLlmThreads - 1) / kLlmThreads)), dim3(kLlmThreads), 0, ctx->stream, a);
     NNHIP_LAUNCH_CHECK(ctx, "rope_append_kernel");
     return 0;
+}
+
+extern "C" int nncase_hip_w8a16_gemm_rope_kv_append(nncase_hip_ctx_t *ctx, const void *x_dev, const void *ln_weight_dev, float eps,
+                                                    const nncase_hip_w8a16_t *w, void *qkv_dev, void *q_out_dev, void *k_cache_dev,
+                                                    void *v_cache_dev, const int32_t *block_table_dev, const int32_t *ctx_lens_dev,
+                                                    const nncase_hip_paged_attn_args_t *p, float rope_theta) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, x_dev && w && qkv_dev, -EINVAL, "w8a16_gemm_rope_kv_append: null argument");
+    RopeArgs r;
+    int rc = make_rope_args(ctx, qkv_dev, q_out_dev, k_cache_dev, v_cache_dev, block_table_dev, ctx_lens_dev, p, rope_theta, &r);
+    if (rc) return rc;
+    NNHIP_REQUIRE(ctx, w->n == (r.hq + 2 * r.hkv) * r.d, -NNCASE_HIP_ERR_SHAPE_MISMATCH,
+                  "w8a16_gemm_rope_kv_append: the matrix has %d output channels, the heads need %d", w->n, (r.hq + 2 * r.hkv) * r.d);
+    if (rope_epilogue_fits(w, r.batch, r))
+        return launch_w8a16_gemm(ctx, x_dev, w, qkv_dev, r.batch, NNCASE_HIP_GEMM_PLAIN, nullptr, NNCASE_HIP_DT_F16, ln_weight_dev, eps, &r);
+    // other geometries: the projection into qkv_dev, then the rope kernel (the same values: the epilogue above rounds to
+    // fp16 where this path stores fp16)
+    rc = launch_w8a16_gemm(ctx, x_dev, w, qkv_dev, r.batch, NNCASE_HIP_GEMM_PLAIN, nullptr, NNCASE_HIP_DT_F16, ln_weight_dev, eps);
+    if (rc) return rc;
+    return nncase_hip_rope_kv_append(ctx, qkv_dev, q_out_dev, k_cache_dev, v_cache_dev, block_table_dev, ctx_lens_dev, p, rope_theta);
 }
 
 extern "C" int nncase_hip_argmax_f32(nncase_hip_ctx_t *ctx, const float *x_dev, int32_t *out_dev, int32_t rows, int32_t cols) {

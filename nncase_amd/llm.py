@@ -134,11 +134,13 @@ class HipDecoder:
                 x, h = xs[0], xs[1]
                 # the three normalisations run inside the products that consume them (fuse_norm), or as operators of their own
                 if fuse_norm:
-                    fn.add_rmsnorm_w8a16_gemm(x, L["ln1"], c.rms_eps, L["qkv"], qkv, bl)
+                    # (and the rotary embedding and the cache append in the projection's epilogue)
+                    fn.add_w8a16_gemm_rope_kv_append(x, L["ln1"], c.rms_eps, L["qkv"], qkv, q, L["k"], L["v"], block_table, ctx_lens,
+                                                     lane_geometry, c.rope_theta)
                 else:
                     fn.add_rmsnorm_f16(x, L["ln1"], norm, bl, c.hidden, c.rms_eps)
                     fn.add_w8a16_gemm(norm, L["qkv"], qkv, bl)
-                fn.add_rope_kv_append(qkv, q, L["k"], L["v"], block_table, ctx_lens, lane_geometry, c.rope_theta)
+                    fn.add_rope_kv_append(qkv, q, L["k"], L["v"], block_table, ctx_lens, lane_geometry, c.rope_theta)
                 # the appended token takes part in its own attention (lengths + 1); the lengths themselves advance
                 # once, at the end of the step
                 fn.add_paged_attention_decode(q, L["k"], L["v"], block_table, ctx_lens, att, lane_args)

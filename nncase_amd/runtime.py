@@ -148,6 +148,8 @@ SYMBOLS = {
     "nncase_hip_function_add_rmsnorm_w8a16_gemm": (_I, [_VP, _VP, _VP, C.c_float, _VP, _VP, C.c_int32, C.c_int32, _VP, C.c_int32]),
     "nncase_hip_function_add_rmsnorm_f16": (_I, [_VP, _VP, _VP, _VP, C.c_int32, C.c_int32, C.c_float]),
     "nncase_hip_function_add_rope_kv_append": (_I, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, C.POINTER(PagedAttnArgs), C.c_float]),
+    "nncase_hip_function_add_w8a16_gemm_rope_kv_append": (_I, [_VP, _VP, _VP, C.c_float, _VP, _VP, _VP, _VP, _VP, _VP, _VP, C.POINTER(PagedAttnArgs), C.c_float]),
+    "nncase_hip_w8a16_gemm_rope_kv_append": (_I, [_VP, _VP, _VP, C.c_float, _VP, _VP, _VP, _VP, _VP, _VP, _VP, C.POINTER(PagedAttnArgs), C.c_float]),
     "nncase_hip_function_add_paged_attention_decode": (_I, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, C.POINTER(PagedAttnArgs)]),
     "nncase_hip_function_add_argmax_f32": (_I, [_VP, _VP, _VP, C.c_int32, C.c_int32]),
     "nncase_hip_function_add_embedding_f16": (_I, [_VP, _VP, _VP, _VP, C.c_int32, C.c_int32, C.c_int32]),
@@ -607,6 +609,11 @@ class Context:
     def rmsnorm_f16(self, x: DeviceBuffer, weight: DeviceBuffer, out: DeviceBuffer, rows: int, hidden: int, eps: float):
         self._check(self.lib.nncase_hip_rmsnorm_f16(self.handle, x.ptr, weight.ptr, out.ptr, rows, hidden, eps), "rmsnorm_f16")
 
+    def w8a16_gemm_rope_kv_append(self, x, ln_weight, eps, w, qkv, q_out, k_cache, v_cache, block_table, ctx_lens, geometry, theta):
+        self._check(self.lib.nncase_hip_w8a16_gemm_rope_kv_append(
+            self.handle, x.ptr, ln_weight.ptr if ln_weight is not None else None, eps, w.handle, qkv.ptr, q_out.ptr, k_cache.ptr,
+            v_cache.ptr, block_table.ptr, ctx_lens.ptr, C.byref(geometry), theta), "w8a16_gemm_rope_kv_append")
+
     def rope_kv_append(self, qkv, q_out, k_cache, v_cache, block_table, ctx_lens, geometry: PagedAttnArgs, theta: float):
         self._check(self.lib.nncase_hip_rope_kv_append(self.handle, qkv.ptr, q_out.ptr, k_cache.ptr, v_cache.ptr, block_table.ptr,
                                                        ctx_lens.ptr, C.byref(geometry), theta), "rope_kv_append")
@@ -731,6 +738,13 @@ class Function:
         self._ck(self.ctx.lib.nncase_hip_function_add_rope_kv_append(self.handle, qkv.ptr, q_out.ptr, k_cache.ptr, v_cache.ptr,
                                                                      block_table.ptr, ctx_lens.ptr, C.byref(geometry), theta),
                  "function_add_rope_kv_append")
+
+    def add_w8a16_gemm_rope_kv_append(self, x, ln_weight, eps, w, qkv, q_out, k_cache, v_cache, block_table, ctx_lens, geometry, theta):
+        """The q / k / v projection (of rmsnorm(x) when ln_weight is given), rotary embedding and cache append as one operator."""
+        self._keep += [x, ln_weight, w, qkv, q_out, k_cache, v_cache, block_table, ctx_lens]
+        self._ck(self.ctx.lib.nncase_hip_function_add_w8a16_gemm_rope_kv_append(
+            self.handle, x.ptr, ln_weight.ptr if ln_weight is not None else None, eps, w.handle, qkv.ptr, q_out.ptr, k_cache.ptr,
+            v_cache.ptr, block_table.ptr, ctx_lens.ptr, C.byref(geometry), theta), "function_add_w8a16_gemm_rope_kv_append")
 
     def add_paged_attention_decode(self, q, k_cache, v_cache, block_table, ctx_lens, out, args):
         self._keep += [q, k_cache, v_cache, block_table, ctx_lens, out]

@@ -96,7 +96,7 @@ def test_decoder_with_fused_normalisation_equals_separate_operators(hip_ctx):
     for fuse in (True, False):
         dec = llm.HipDecoder(hip_ctx, cfg, weights, batch, max_blocks, bt, lens.copy(), [k.copy() for k in kcs], [v.copy() for v in vcs],
                              capture_graph=True, fuse_norm=fuse)
-        assert len(dec.fn) == (3 + cfg.layers * 6 + 1 if fuse else 3 + cfg.layers * 8 + 2)
+        assert len(dec.fn) == (3 + cfg.layers * 5 + 1 if fuse else 3 + cfg.layers * 8 + 2)
         tk = tokens
         logs = []
         for _ in range(2):
@@ -160,6 +160,46 @@ def test_rope_and_kv_append(hip_ctx):
         want_v[pb, :, :, off] = v2[pb, :, :, off]
     assert np.array_equal(k2, want_k) and np.array_equal(v2, want_v)       # nothing else in the caches moved
     assert np.array_equal(q[0], qkv[0].reshape(-1, d)[:hq])                # position 0: rotation by zero
+
+
+@pytest.mark.parametrize("B,k,norm", [(32, 896, True), (16, 896, True), (5, 256, False), (32, 1024, True), (7, 1536, True), (40, 896, True)])
+def test_projection_that_rotates_and_appends_equals_the_two_operators(hip_ctx, B, k, norm):
+    """nncase_hip_w8a16_gemm_rope_kv_append against the projection into fp16 followed by nncase_hip_rope_kv_append: the same
+    bytes in the query buffer and in both caches (the last two cases take the two-launch form inside the entry point: a
+    reduction too long for the rows to be normalised in one block, more than 32 rows)."""
+    rng = np.random.default_rng(B + k)
+    hq, hkv, d, blk, max_blocks = 14, 2, 64, 16, 8
+    n = (hq + 2 * hkv) * d
+    nb = B * max_blocks + 2
+    lens = rng.integers(0, max_blocks * blk, B).astype(np.int32)
+    lens[0] = 0
+    bt = rng.permutation(nb)[:B * max_blocks].reshape(B, max_blocks).astype(np.int32)
+    x = (rng.standard_normal((B, k)) * 0.7).astype(np.float16)
+    ln = (1.0 + 0.1 * rng.standard_normal(k)).astype(np.float16)
+    wq, sc = llm.quantize_rows((rng.standard_normal((n, k)) * k ** -0.5).astype(np.float32))
+    bias = (rng.standard_normal(n) * 0.1).astype(np.float32)
+    w = hip_ctx.prepack_w8a16(wq, sc, bias)
+    kc = rng.standard_normal((nb, hkv, blk, d)).astype(np.float16)
+    vc = rng.standard_normal((nb, hkv, d, blk)).astype(np.float16)
+    geo = rt.PagedAttnArgs(B, hq, hkv, d, blk, max_blocks, nb, 0.125, rt.DT_F16)
+    dx, dln, dbt, dlens = hip_ctx.to_device(x), hip_ctx.to_device(ln), hip_ctx.to_device(bt), hip_ctx.to_device(lens)
+    got = []
+    for fused in (True, False):
+        dk, dv = hip_ctx.to_device(kc), hip_ctx.to_device(vc)
+        dq, dqkv = hip_ctx.alloc(B * hq * d * 2), hip_ctx.alloc(B * n * 2)
+        dq.fill(0)
+        if fused:
+            hip_ctx.w8a16_gemm_rope_kv_append(dx, dln if norm else None, 1e-6, w, dqkv, dq, dk, dv, dbt, dlens, geo, 1e6)
+        else:
+            if norm:
+                hip_ctx.rmsnorm_w8a16_gemm(dx, dln, 1e-6, w, dqkv, B)
+            else:
+                hip_ctx.w8a16_gemm(dx, w, dqkv, B)
+            hip_ctx.rope_kv_append(dqkv, dq, dk, dv, dbt, dlens, geo, 1e6)
+        got.append((dq.download((B, hq, d), np.uint16), dk.download(kc.shape, np.uint16), dv.download(vc.shape, np.uint16)))
+    for a, b in zip(*got):
+        assert np.array_equal(a, b)
+    assert not np.array_equal(got[0][1], kc.view(np.uint16))     # something was appended
 
 
 def test_kv_append_ignores_lengths_outside_the_table(hip_ctx):
