@@ -45,27 +45,27 @@ MEASURED_TRAFFIC_SOURCE = {"unfused": "profiles/mobilenetv2_b64_kernels_counters
                            "fused": "profiles/mobilenetv2_b64_fused_blocks_kernels_counters.txt"}
 MEASURED_TRAFFIC_B64 = {
     "unfused": {
-        "dw3x3<S=1>": 19028851,
-        "dw3x3<S=2>": 41847409,
-        "qconv_igemm+add<T=2,RG=1,rows16>": 13037164,
-        "qconv_igemm+add<T=2,RG=2,rows16>": 39859713,
-        "qconv_igemm<T=1,RG=1,rows16>": 3347259,
-        "qconv_igemm<T=1,RG=4,rows16>": 38602998,
-        "qconv_igemm<T=12,RG=1,rows16>": 10265961,
-        "qconv_igemm<T=2,RG=1,rows16>": 8914698,
-        "qconv_igemm<T=2,RG=2,rows16>": 24173898,
-        "qconv_igemm<T=2,RG=2,vec16>": 38614115,
-        "qconv_igemm<T=5,RG=1,rows16>": 5104416,
-        "qconv_igemm<T=6,RG=2,rows16>": 90039323,
-        "qconv_igemm<T=8,RG=1,rows16>": 5905422,
-        "qconv_igemm<T=9,RG=1,rows8>": 34301118,
-        "qconv_wide+add<T=2,RG=2,rows16>": 6175994,
-        "qconv_wide+add<T=4,RG=2,rows16>": 10527284,
-        "qconv_wide+dequantize<T=2,RG=2,rows16>": 1710205,
-        "qconv_wide<T=2,RG=2,rows16>": 4713534,
-        "qconv_wide<T=4,RG=2,rows16>": 7447634,
-        "qglobal_avgpool": 4239099,
-        "quantize+pack": 51434890,
+        "dw3x3<S=1>": 19011936,
+        "dw3x3<S=2>": 41883762,
+        "qconv_igemm+add<T=2,RG=1,rows16>": 13054633,
+        "qconv_igemm+add<T=2,RG=2,rows16>": 40563268,
+        "qconv_igemm<T=1,RG=1,rows16>": 3359320,
+        "qconv_igemm<T=1,RG=4,rows16>": 38602230,
+        "qconv_igemm<T=12,RG=1,rows16>": 10267976,
+        "qconv_igemm<T=2,RG=1,rows16>": 8930024,
+        "qconv_igemm<T=2,RG=2,rows16>": 24171978,
+        "qconv_igemm<T=2,RG=2,vec16>": 38626465,
+        "qconv_igemm<T=5,RG=1,rows16>": 5099510,
+        "qconv_igemm<T=6,RG=2,rows16>": 90023774,
+        "qconv_igemm<T=8,RG=1,rows16>": 5904294,
+        "qconv_igemm<T=9,RG=1,rows8>": 34301598,
+        "qconv_wide+add<T=2,RG=2,rows16>": 6175918,
+        "qconv_wide+add<T=4,RG=2,rows16>": 10530291,
+        "qconv_wide+dequantize<T=2,RG=2,rows16>": 1710972,
+        "qconv_wide<T=2,RG=2,rows16>": 4725052,
+        "qconv_wide<T=4,RG=2,rows16>": 7450706,
+        "qglobal_avgpool": 4238843,
+        "quantize+pack": 51434794,
     },
     "fused": {
         "dw3x3<S=1>": 27882249,

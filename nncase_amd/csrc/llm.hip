@@ -367,7 +367,6 @@ template <int MT, int G, bool SPLIT, int B = kGemmBatch> __global__ __launch_bou
 // multiply-adds are those of the kernel above.
 constexpr int kRowsBatch = 8;
 constexpr int kGluSplitWaves = 4;             // waves that split the reduction of one gate / up tile pair
-constexpr int kRowsWhole = 14;                // k-steps of a reduction that is requested in one go
 constexpr int kRowsPieces = 4;                 // 512-element pieces of a row: k <= 2048
 constexpr int kRowsMaxK = kRowsPieces * 512;
 inline int rows_in_lds_pitch(int k) { return k * 2 + 16; } // bytes per token row: the padding spreads the rows over the banks
@@ -843,8 +842,8 @@ static int launch_w8a16_gemm(nncase_hip_ctx_t *ctx, const void *a_dev, const nnc
     }
     if (w->k <= kRowsMaxK && rows_lds <= 128 * 1024 && out_tiles >= ctx->compute_units) {
         const dim3 rgrid((out_tiles + kGemmWaves - 1) / kGemmWaves), rblock(kGemmThreads);
-        // a reduction of up to 14 k-steps (hidden size 896) is requested whole: one trip to memory for all the weights
-        const bool whole = w->ksteps <= kRowsWhole;
+        // (eight k-steps of weights per request: asking for a whole 14-step reduction at once costs registers that the
+        // vocabulary head, 1187 blocks, needs for occupancy -- 50.7 against 43.9 us)
 #define NNHIP_ROWS_LAUNCH_KB(MTV, GV, KBV, PV)                                                                                 \
     do {                                                                                                                       \
         NNHIP_HIP(ctx, raise_dynamic_lds(w8a16_gemm_rows_in_lds_kernel<MTV, GV, kGemmWaves, false, KBV, PV>, ctx->device, rows_lds + 1024, 128 * 1024)); \
@@ -852,7 +851,7 @@ static int launch_w8a16_gemm(nncase_hip_ctx_t *ctx, const void *a_dev, const nnc
     } while (0)
 #define NNHIP_ROWS_LAUNCH(MTV, GV)                                                                                             \
     do {                                                                                                                       \
-        if (whole) NNHIP_ROWS_LAUNCH_KB(MTV, GV, kRowsWhole, 2); /* (14 k-steps are 896 elements) */                           \
+        if (short_rows) NNHIP_ROWS_LAUNCH_KB(MTV, GV, kRowsBatch, 2);                                                          \
         else NNHIP_ROWS_LAUNCH_KB(MTV, GV, kRowsBatch, kRowsPieces);                                                           \
     } while (0)
         if (glu) {
