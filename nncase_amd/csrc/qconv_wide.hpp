@@ -657,6 +657,52 @@ template <int T, int RG, int WM, int WN, int LM> int launch_wide4_t(nncase_hip_c
 //   the lanes of a DMA request (a 1 KiB run: eight pixels) fetch the pieces in the rotated order.
 // The per-channel constants, the byte table and the staging areas of dword outputs take over the ring's memory once
 // the last k-step is done.
+// Float32 (or int32) results of a wave's 16 pixels x 16 T channels, T = 8, written as whole 128-byte lines.  A lane holds
+// 4 T = 32 consecutive channels of one pixel, 128 bytes of the output row; all of them go into the wave's staging area
+// (a run per lane, padded against bank conflicts) and come back with eight lanes per run, so that a store instruction
+// covers eight complete lines -- the staged stores of four tiles at a time write half lines, and the memory side
+// pays for the other half.  LDS operations of a wave execute in order: no barrier, one wait in front of the data read back.
+constexpr int kLineRun = 128 + 16;
+constexpr int line_store_bytes() { return 64 * kLineRun; } // per wave
+template <int T>
+__device__ __forceinline__ void wide_store_lines(const IgemmArgs &a, const v4i (&acc)[T], int32_t rowsum, int p, int ch0, int gq, const int32_t *ct,
+                                                 uint8_t *stage, int quarter_stride) {
+    static_assert(T == 8, "a lane's run is one 128-byte line");
+    const int lane = threadIdx.x & 63, j = lane & 15;
+    const int32_t nrsz = -a.zwp * rowsum;
+    const bool as_int = a.ep.out_mode == kOutI32;
+#pragma unroll
+    for (int nt = 0; nt < T; nt++) {
+        const v4i c = *reinterpret_cast<const v4i *>(ct + gq * (4 * T) + nt * 4);
+        u32x4 o;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int32_t v = add3(acc[nt][r], c[r], nrsz);
+            o[r] = as_int ? (uint32_t)v : __float_as_uint(clamp_ref((float)v * a.ep.mult, a.ep.lo, a.ep.hi));
+        }
+        *reinterpret_cast<u32x4 *>(stage + (j * 4 + gq) * kLineRun + nt * 16) = o;
+    }
+    const int p_first = p - j, ch_first = ch0 - gq * quarter_stride;
+    const int u = lane & 7, sub = lane >> 3;
+    uint32_t *yo = reinterpret_cast<uint32_t *>(a.y);
+#pragma unroll
+    for (int it = 0; it < 8; it++) {
+        const int run = it * 8 + sub; // (pixel of the group, channel quarter)
+        const u32x4 v = *reinterpret_cast<const u32x4 *>(stage + run * kLineRun + u * 16);
+        const int pp = p_first + (run >> 2), ch = ch_first + (run & 3) * quarter_stride + u * 4;
+        if (pp < a.m) {
+            uint32_t *dst = yo + ((size_t)pp * a.ldy + a.y_coff + ch);
+            if (ch + 4 <= a.n) {
+                *reinterpret_cast<u32x4_a4 *>(dst) = u32x4_a4{v[0], v[1], v[2], v[3]};
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    if (ch + r < a.n) dst[r] = v[r];
+            }
+        }
+    }
+}
+
 template <int T, int RG, int WM, int WN, int LM>
 __global__ __launch_bounds__(WM * WN * 64, WM * WN >= 8 ? 2 : 1) void qconv_wide_dma_kernel(const IgemmArgs a, int nchunks) {
     static_assert(LM == kWideRowsFull || LM == kWideRows, "contiguous reduction rows only");
@@ -885,9 +931,11 @@ __global__ __launch_bounds__(WM * WN * 64, WM * WN >= 8 ? 2 : 1) void qconv_wide
     }
     if (a.lut && threadIdx.x < 64) reinterpret_cast<uint32_t *>(lutl)[threadIdx.x] = a.lut[threadIdx.x];
     __syncthreads();
-    uint8_t *const stage = staged_store_built(T) ? stage_base + wave * staged_store_bytes() : nullptr;
+    // dword results (float32, int32) of eight channel tiles leave as whole lines; everything else through the shared epilogue
+    const bool lines = T == 8 && a.ep.out_mode != kOutU8 && !a.deq;
+    uint8_t *const stage = stage_base + wave * (lines ? line_store_bytes() : staged_store_bytes());
     const int ch0 = ch_base + gq * (4 * TB) + wn * (4 * T);
-    const int32_t *ct = cterm + gq * (4 * TB) + wn * (4 * T) - gq * (4 * T); // igemm_store_tile adds gq * 4 T
+    const int32_t *ct = cterm + gq * (4 * TB) + wn * (4 * T) - gq * (4 * T); // the epilogues add gq * 4 T
     static_for<0, RG>([&](auto rg_c) __attribute__((always_inline)) {
         constexpr int rg = decltype(rg_c)::value;
         const int pl = (wm * RG + rg) * 16 + j;
@@ -895,6 +943,12 @@ __global__ __launch_bounds__(WM * WN * 64, WM * WN >= 8 ? 2 : 1) void qconv_wide
         int32_t sx = (int32_t)rs_final[rg];
         sx += __shfl_xor(sx, 16);
         sx += __shfl_xor(sx, 32);
+        if constexpr (T == 8) {
+            if (lines) {
+                wide_store_lines<T>(a, acc[rg], sx - 128 * a.k, mt * PIX + pl, ch0, gq, ct, stage, 4 * TB);
+                return;
+            }
+        }
         igemm_store_tile<T, kOwesAll, false, staged_store_built(T)>(a, acc[rg], sx - 128 * a.k, mt * PIX + pl, ch0, gq, ct, lutl, stage, 4 * TB);
     });
 }
