@@ -45,10 +45,11 @@ public sealed partial class LowerConv2DToHip : IRewriteRule
         int[] biasValues;
         if (result.GetValueOrDefault("bias") is TensorConst bias)
         {
-            // the importer gives the bias at scale xScale * wScale with zero point 0: those integers are the
-            // accumulator's own units; anything else would need a rescale and stays on the float path
+            // the importer gives the bias at scale xScale * wScale (one float product, Onnx/QLinearConv.cs:70) with zero
+            // point 0: those integers are the accumulator's own units; any other scale, however close, would need a
+            // rescale and stays on the float path
             var biasQp = ((TensorConst)result["biasQp"]).Value.ToScalar<QuantParam>();
-            if (biasQp.ZeroPoint != 0 || MathF.Abs(biasQp.Scale - (inputQp.Scale * weightsQp.Scale)) > 1e-6f * biasQp.Scale)
+            if (biasQp.ZeroPoint != 0 || biasQp.Scale != inputQp.Scale * weightsQp.Scale)
             {
                 return null;
             }
