@@ -300,6 +300,36 @@ typedef struct nncase_hip_qblock_args {
 NNCASE_HIP_API int nncase_hip_qblock(nncase_hip_ctx_t *ctx, const uint8_t *x_dev, const nncase_hip_qblock_t *block,
                                      uint8_t *y_dev, const nncase_hip_qblock_args_t *args);
 
+/* ---- pair of pointwise convolutions ------------------------------------------
+ * Two dense 1x1, stride-1, unpadded Conv2D calls of which the second reads the
+ * first's result (a bottleneck's projection and the next block's expansion,
+ * which the importer leaves as separate Conv2D calls,
+ * src/Nncase.Importer/TFLite/Conv2D.cs:17-69, each running
+ * src/Native/src/kernels/stackvm/reference/convolution.cpp:26-143) as one launch:
+ *   y1 = first(x)  [byte table of the first weights]  [+ first_args->residual_dev]
+ *   y2 = second(y1) [byte table of the second weights]
+ * Both results are stored; every byte equals what nncase_hip_qconv2d writes for
+ * the two calls with the same arguments.  Meant for small pixel counts (batch 1,
+ * late feature maps) where the two calls are bound by launch latency: each
+ * workgroup recomputes the first convolution for its 16 pixels, so on large
+ * tensors the two separate calls are faster.
+ * The pair keeps pointers to both weights handles (bias, zero points, scales,
+ * tables): they must outlive it.  The raw OIHW weights are needed again because
+ * the pair packs them in its own order.
+ * supported: in_channels a multiple of 16 up to 1024, mid_channels a multiple of
+ * 4 up to 512, out_channels a multiple of 4. */
+typedef struct nncase_hip_qpair nncase_hip_qpair_t;
+NNCASE_HIP_API int nncase_hip_qpointwise_pair_supported(int32_t in_channels, int32_t mid_channels, int32_t out_channels);
+NNCASE_HIP_API int nncase_hip_qpointwise_pair_create(nncase_hip_ctx_t *ctx, const nncase_hip_weights_t *first,
+                                                     const uint8_t *first_oihw_host, const nncase_hip_weights_t *second,
+                                                     const uint8_t *second_oihw_host, nncase_hip_qpair_t **pair);
+NNCASE_HIP_API int nncase_hip_qpointwise_pair_destroy(nncase_hip_ctx_t *ctx, nncase_hip_qpair_t *pair);
+/* first_args / second_args as for nncase_hip_qconv2d (u8 results, dense outputs; only the first may carry a residual);
+ * second_args->x_qp is the quantisation of y1 as the second convolution reads it. */
+NNCASE_HIP_API int nncase_hip_qpointwise_pair(nncase_hip_ctx_t *ctx, const uint8_t *x_dev, const nncase_hip_qpair_t *pair,
+                                              uint8_t *y1_dev, uint8_t *y2_dev, const nncase_hip_conv2d_args_t *first_args,
+                                              const nncase_hip_conv2d_args_t *second_args);
+
 /* MatMul A[M,K] (u8, device) x B[K,N] (u8, row-major, HOST, pre-packed) with
  * the same three output forms; replaces kernels::stackvm::mat_mul
  * (tensor_ops.cpp:553-565 -> reference/matmul.cpp:28-48) on the
@@ -548,6 +578,10 @@ NNCASE_HIP_API int nncase_hip_function_add_qconv2d(nncase_hip_function_t *fn, co
 NNCASE_HIP_API int nncase_hip_function_add_qblock(nncase_hip_function_t *fn, const uint8_t *x_dev,
                                                   const nncase_hip_qblock_t *block, uint8_t *y_dev,
                                                   const nncase_hip_qblock_args_t *args);
+NNCASE_HIP_API int nncase_hip_function_add_qpointwise_pair(nncase_hip_function_t *fn, const uint8_t *x_dev,
+                                                           const nncase_hip_qpair_t *pair, uint8_t *y1_dev, uint8_t *y2_dev,
+                                                           const nncase_hip_conv2d_args_t *first_args,
+                                                           const nncase_hip_conv2d_args_t *second_args);
 NNCASE_HIP_API int nncase_hip_function_add_qadd(nncase_hip_function_t *fn, const uint8_t *a_dev,
                                                 nncase_hip_quant_param_t a_qp, const uint8_t *b_dev,
                                                 nncase_hip_quant_param_t b_qp, uint8_t *out_dev,

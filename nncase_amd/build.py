@@ -19,7 +19,7 @@ OBJ_DIR = os.path.join(LIB_DIR, "obj")
 LIB_PATH = os.path.join(LIB_DIR, "libnncase_hip.so")
 
 SOURCES = ["ctx.hip", "quant.hip", "qconv.hip", "qconv_igemm.hip", "qconv_igemm_rows16.hip", "qconv_igemm_rows8.hip", "qconv_igemm_vec16.hip",
-           "qconv_igemm_vec8.hip", "qconv_igemm_vec4.hip", "qconv_igemm_bytes.hip", "qconv_wide_rows16.hip", "qconv_wide_vec16.hip", "qblock.hip", "qconv_smallc.hip", "qconv_dw.hip", "layout.hip", "glue.hip", "attn.hip", "llm.hip", "function.hip", "kmodel.hip"]
+           "qconv_igemm_vec8.hip", "qconv_igemm_vec4.hip", "qconv_igemm_bytes.hip", "qconv_wide_rows16.hip", "qconv_wide_vec16.hip", "qblock.hip", "qpair.hip", "qconv_smallc.hip", "qconv_dw.hip", "layout.hip", "glue.hip", "attn.hip", "llm.hip", "function.hip", "kmodel.hip"]
 
 # -ffp-contract=off / -fno-fast-math: every fp32 step of the requantisation must be a
 # single IEEE operation.  packed-fp32-ops is switched off for the device pass.

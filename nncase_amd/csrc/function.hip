@@ -9,7 +9,7 @@ namespace {
 
 struct Op {
     enum Kind { kQuantize, kDequantize, kConv, kAdd, kPool, kLut, kConcat, kResize, kMaxPool, kPack, kQuantPack,
-                kGemm, kRmsNorm, kRope, kGemmRope, kAttn, kArgmax, kEmbed, kAddI32, kBlock, kLayout } kind;
+                kGemm, kRmsNorm, kRope, kGemmRope, kAttn, kArgmax, kEmbed, kAddI32, kBlock, kLayout, kPair } kind;
     const void *in0 = nullptr, *in1 = nullptr;
     void *out = nullptr;
     const nncase_hip_weights_t *weights = nullptr;
@@ -38,6 +38,8 @@ struct Op {
     float eps = 0.f, theta = 0.f;
     const nncase_hip_qblock_t *block = nullptr;
     nncase_hip_qblock_args_t blk{};
+    const nncase_hip_qpair_t *pair = nullptr; // with conv (first) and conv2 (second) arguments, out / out2 the two results
+    nncase_hip_conv2d_args_t conv2{};
     int lane = 0; // independent operator chain this operator belongs to
 };
 
@@ -69,6 +71,8 @@ static int run_op(nncase_hip_function *fn, const Op &op) {
         return nncase_hip_qconv2d(ctx, (const uint8_t *)op.in0, op.weights, op.out, &op.conv);
     case Op::kBlock:
         return nncase_hip_qblock(ctx, (const uint8_t *)op.in0, op.block, (uint8_t *)op.out, &op.blk);
+    case Op::kPair:
+        return nncase_hip_qpointwise_pair(ctx, (const uint8_t *)op.in0, op.pair, (uint8_t *)op.out, (uint8_t *)op.out2, &op.conv, &op.conv2);
     case Op::kAdd:
         return nncase_hip_qadd(ctx, (const uint8_t *)op.in0, op.qp0, (const uint8_t *)op.in1, op.qp1, (uint8_t *)op.out,
                                op.qp2, op.lo, op.hi, op.count);
@@ -207,6 +211,18 @@ extern "C" int nncase_hip_function_add_qblock(nncase_hip_function_t *fn, const u
     Op op;
     op.kind = Op::kBlock;
     op.in0 = x_dev, op.out = y_dev, op.block = block, op.blk = *args;
+    return push(fn, op);
+}
+
+extern "C" int nncase_hip_function_add_qpointwise_pair(nncase_hip_function_t *fn, const uint8_t *x_dev, const nncase_hip_qpair_t *pair,
+                                                       uint8_t *y1_dev, uint8_t *y2_dev, const nncase_hip_conv2d_args_t *first_args,
+                                                       const nncase_hip_conv2d_args_t *second_args) {
+    if (!fn) return -EINVAL;
+    NNHIP_REQUIRE(fn->ctx, x_dev && pair && y1_dev && y2_dev && first_args && second_args, -EINVAL,
+                  "function_add_qpointwise_pair: null argument");
+    Op op;
+    op.kind = Op::kPair;
+    op.in0 = x_dev, op.out = y1_dev, op.out2 = y2_dev, op.pair = pair, op.conv = *first_args, op.conv2 = *second_args;
     return push(fn, op);
 }
 
@@ -579,6 +595,7 @@ extern "C" int nncase_hip_function_op_kernel(nncase_hip_function_t *fn, int32_t 
     case Op::kDequantize: snprintf(name, capacity, "dequantize"); break;
     case Op::kConv: describe_conv_kernel(fn->ctx, op.weights, &op.conv, name, capacity); break;
     case Op::kBlock: nncase_hip_qblock_describe(op.block, &op.blk, name, capacity); break;
+    case Op::kPair: snprintf(name, capacity, "qpointwise_pair_kernel"); break;
     case Op::kAdd: snprintf(name, capacity, "qadd"); break;
     case Op::kPool: snprintf(name, capacity, "qglobal_avgpool"); break;
     case Op::kLut: snprintf(name, capacity, "lut_u8"); break;

@@ -1,0 +1,369 @@
+// Two pointwise (1x1, stride 1, no padding) quantized convolutions, the second reading the first's result, as one
+// launch:  y1 = conv_a(x) [table] [+ residual],  y2 = conv_b(y1) [table].
+//
+// A linear-bottleneck network alternates a projection (many -> few channels, src/Nncase.Importer/TFLite/Conv2D.cs:17-69
+// imports each as its own Conv2D) with the next block's expansion (few -> many).  At small batches the two are
+// launch-latency-bound kernels of a few microseconds; here the few-channel tensor between them stays in LDS (it is
+// also stored: a later residual add reads it), and the second product starts as soon as the first's tile exists.
+//
+// Work split: a workgroup owns 16 pixels and a range of conv_b's channel tiles.  It computes ALL of conv_a for its
+// pixels (every workgroup of a pixel tile repeats that: the reduction is the cheap side of the pair and recomputing
+// keeps enough workgroups alive on 7x7 and 14x14 maps), requantises it exactly as nncase_hip_qconv2d does, and
+// multiplies the LDS tile with its range of conv_b.  Results are bit-identical to the two nncase_hip_qconv2d calls.
+//
+// Weights are re-packed for this kernel: [channel tile][k-step][64 lanes][16 bytes], lane (i, g) holding
+// w[16 t + i][64 ks + 16 g ..] - 128 as s8 (zero past the real extents), so that one 16-byte load per lane is an MFMA
+// operand and lane (j, g) of the result holds channels 16 t + 4 g .. + 3 of pixel j: four neighbours, one dword.
+#include "qconv.hpp"
+
+#include <new>
+#include <vector>
+
+using namespace nnhip;
+
+struct nncase_hip_qpair {
+    const nncase_hip_weights *first = nullptr, *second = nullptr;
+    int k1 = 0, n1 = 0, n2 = 0;     // x channels, y1 channels, y2 channels
+    int ks1 = 0, ks2 = 0;           // k-steps of 64 of the two reductions
+    int t1 = 0, t2 = 0;             // 16-channel tiles of the two results
+    uint8_t *d_wa = nullptr, *d_wb = nullptr;
+    int32_t *d_wsum_a = nullptr, *d_wsum_b = nullptr; // sum_k (w - 128) per output channel (padded to whole tiles)
+    int32_t *d_bias_a = nullptr, *d_bias_b = nullptr; // bias, padded to whole tiles
+};
+
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kPairMaxK1 = 1024;  // x channels
+constexpr int kPairMaxN1 = 512;   // y1 channels
+constexpr int kRowPad = 16;       // bytes between LDS rows beyond the padded reduction (spreads the 16 rows over the banks)
+
+// bytes of an LDS row: the reduction rounded up to whole chunks of `chunk` k-steps, and the pad
+__host__ __device__ constexpr int pair_row_bytes(int ksteps, int chunk) { return (ksteps + chunk - 1) / chunk * chunk * 64 + kRowPad; }
+
+struct PairArgs {
+    const uint8_t *x;
+    uint8_t *y1, *y2;
+    const uint8_t *wa, *wb;
+    const int32_t *bias_a, *wsum_a, *bias_b, *wsum_b;
+    const uint32_t *lut_a, *lut_b;
+    int m;                 // pixels
+    int k1, n1, n2;
+    int ks1, ks2, t1, t2;
+    int tiles_per_block;   // conv_b channel tiles per workgroup (blockIdx.y selects the range)
+    int zxa, zwa, zxb, zwb; // zero points - 128
+    Epilogue ep_a, ep_b;
+    ResidualEpilogue rep_a;
+};
+
+__device__ __forceinline__ uint32_t table4(const uint8_t *t, uint32_t v) {
+    return (uint32_t)t[v & 0xffu] | ((uint32_t)t[(v >> 8) & 0xffu] << 8) | ((uint32_t)t[(v >> 16) & 0xffu] << 16) |
+           ((uint32_t)t[v >> 24] << 24);
+}
+
+// What a wave fetches from global memory for one channel tile ahead of multiplying it: the first KC weight fragments,
+// and the constants of the tile's epilogue (bias, weight sums and, for the first convolution, the residual bytes).
+template <int KC> struct TileLoads {
+    v4i frag[KC];
+    v4i bias, wsum;
+    uint32_t res;
+};
+
+// Loads KC weight fragments of one tile from k-step ks0 on; past the tile's last k-step the last one is loaded again
+// (the activation tile is zero there, so what such a fragment holds does not matter, and no lane branches).
+template <int KC> __device__ __forceinline__ void load_chunk(v4i (&f)[KC], const uint8_t *w, int tile, int ks0, int ksteps, int lane) {
+    const v4i *src = reinterpret_cast<const v4i *>(w) + (size_t)tile * ksteps * 64 + lane;
+#pragma unroll
+    for (int c = 0; c < KC; c++) f[c] = src[min(ks0 + c, ksteps - 1) * 64];
+}
+
+template <int KC, bool FIRST>
+__device__ __forceinline__ void load_tile(TileLoads<KC> &l, const PairArgs &a, int tile, int ks0, int lane, int p) {
+    load_chunk<KC>(l.frag, FIRST ? a.wa : a.wb, tile, ks0, FIRST ? a.ks1 : a.ks2, lane);
+    const int ch = tile * 16 + (lane >> 4) * 4;
+    l.bias = *reinterpret_cast<const v4i *>((FIRST ? a.bias_a : a.bias_b) + ch);
+    l.wsum = *reinterpret_cast<const v4i *>((FIRST ? a.wsum_a : a.wsum_b) + ch);
+    l.res = 0;
+    if (FIRST && a.rep_a.res && p < a.m && ch < a.n1) l.res = *reinterpret_cast<const uint32_t *>(a.rep_a.res + (size_t)p * a.n1 + ch);
+}
+
+// sum over k of the LDS tile's row j (every lane of pixel j gets it)
+__device__ __forceinline__ int32_t row_sum(const uint8_t *rows, int stride, int ksteps, int lane) {
+    const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
+    const uint8_t *row = rows + (lane & 15) * stride + (lane >> 4) * 16;
+    v4i rs = {0, 0, 0, 0};
+#pragma unroll 1
+    for (int ks = 0; ks < ksteps; ks++) rs = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, *reinterpret_cast<const v4i *>(row + ks * 64), rs, 0, 0, 0);
+    return rs[0];
+}
+
+// One convolution of the pair for this wave's channel tiles first, first + step, ... below end.  `rows` is the LDS
+// activation tile ([16][stride] s8); `cur` holds the loads of the first tile already.  FIRST: results go to the LDS tile
+// `ys` as s8 (and to y1 when store_y1); else to y2.
+template <int KC, bool FIRST>
+__device__ __forceinline__ void run_stage(const PairArgs &a, const uint8_t *rows, int stride, uint8_t *ys, int sy, const uint8_t *lut, int first,
+                                          int step, int end, TileLoads<KC> &cur, int lane, int p, bool store_y1) {
+    const int j = lane & 15, g = lane >> 4;
+    const uint8_t *w = FIRST ? a.wa : a.wb;
+    const int ksteps = FIRST ? a.ks1 : a.ks2;
+    const int zx = FIRST ? a.zxa : a.zxb, zw = FIRST ? a.zwa : a.zwb;
+    const Epilogue &ep = FIRST ? a.ep_a : a.ep_b;
+    const int32_t nrs = -zw * row_sum(rows, stride, ksteps, lane);
+    const int32_t kzz = (FIRST ? a.k1 : a.n1) * zx * zw;
+    const uint8_t *row = rows + j * stride + g * 16;
+    v4i bias = cur.bias, ws = cur.wsum; // the constants of a tile arrive with its first chunk and are used after its last
+    uint32_t rv = cur.res;
+#pragma unroll 1
+    for (int t = first; t < end; t += step) {
+        v4i acc = {0, 0, 0, 0};
+#pragma unroll 1
+        for (int ks0 = 0; ks0 < ksteps; ks0 += KC) {
+            // what follows this chunk (the tile's next one, else the next tile's first) travels while this one multiplies;
+            // one wave-uniform branch around all of it: behind the last chunk nothing is requested, so nothing is waited for
+            const bool more = ks0 + KC < ksteps;
+            TileLoads<KC> nxt;
+            if (more || t + step < end) load_tile<KC, FIRST>(nxt, a, more ? t : t + step, more ? ks0 + KC : 0, lane, p);
+            if (!more) bias = cur.bias, ws = cur.wsum, rv = cur.res;
+#pragma unroll
+            for (int c = 0; c < KC; c++) {
+                const v4i xf = *reinterpret_cast<const v4i *>(row + (ks0 + c) * 64);
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(cur.frag[c], xf, acc, 0, 0, 0);
+            }
+            cur = nxt;
+        }
+        const int ch = t * 16 + g * 4;
+        int32_t v[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) v[r] = acc[r] + (bias[r] - zx * ws[r] + kzz) + nrs;
+        uint32_t q = requant4_u8_packed(v, ep);
+        if (lut) q = table4(lut, q);
+        if constexpr (FIRST) {
+            if (ch < a.n1) {
+                if (a.rep_a.res) q = residual4_packed(q, rv, a.rep_a);
+                *reinterpret_cast<uint32_t *>(ys + j * sy + ch) = q ^ 0x80808080u;
+                if (store_y1 && p < a.m) *reinterpret_cast<uint32_t *>(a.y1 + (size_t)p * a.n1 + ch) = q;
+            }
+        } else {
+            if (ch < a.n2 && p < a.m) *reinterpret_cast<uint32_t *>(a.y2 + (size_t)p * a.n2 + ch) = q;
+        }
+    }
+}
+
+// KA / KB: weight fragments a wave requests at a time for the first / second convolution (each twice in registers).
+// MAXW: most waves a workgroup is launched with; OCC: waves per SIMD the register budget is held to.
+template <int KA, int KB, int MAXW, int OCC> __global__ __launch_bounds__(MAXW * 64, OCC) void qpointwise_pair_kernel(const PairArgs a) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    // rows hold whole chunks of k-steps, zero past the real reduction
+    const int sx = pair_row_bytes(a.ks1, KA), sy = pair_row_bytes(a.ks2, KB);
+    uint8_t *xs = smem;              // [16][sx]  x - 128
+    uint8_t *ys = xs + 16 * sx;      // [16][sy]  y1 - 128
+    uint8_t *lut_a = ys + 16 * sy;   // 256 bytes each
+    uint8_t *lut_b = lut_a + 256;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, threads = blockDim.x, waves = threads >> 6;
+    const int p0 = blockIdx.x * 16, p = p0 + (lane & 15);
+    const int b_first = blockIdx.y * a.tiles_per_block;
+    const int b_end = min(a.t2, b_first + a.tiles_per_block);
+
+    // the first tiles' weights and constants travel while the pixel tile is staged
+    TileLoads<KA> la;
+    TileLoads<KB> lb;
+    if (wave < a.t1) load_tile<KA, true>(la, a, wave, 0, lane, p);
+    if (b_first + wave < b_end) load_tile<KB, false>(lb, a, b_first + wave, 0, lane, p);
+
+    // x tile as s8 (x - 128); rows past the tensor and bytes past K read as zero
+    const int pieces = (sx - kRowPad) / 16; // 16-byte pieces per row
+#pragma unroll 1
+    for (int e = tid; e < 16 * pieces; e += threads) {
+        const int r = e / pieces, c = e - r * pieces;
+        u32x4 v = {0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u};
+        if (p0 + r < a.m && c * 16 < a.k1) v = *reinterpret_cast<const u32x4 *>(a.x + (size_t)(p0 + r) * a.k1 + c * 16);
+        *reinterpret_cast<u32x4 *>(xs + r * sx + c * 16) = v ^ 0x80808080u;
+    }
+    for (int e = tid; e < 4 * sy; e += threads) reinterpret_cast<uint32_t *>(ys)[e] = 0; // channels past N1 stay zero
+    for (int e = tid; e < 128; e += threads) {
+        if (e < 64) {
+            if (a.lut_a) reinterpret_cast<uint32_t *>(lut_a)[e] = a.lut_a[e];
+        } else if (a.lut_b) {
+            reinterpret_cast<uint32_t *>(lut_b)[e - 64] = a.lut_b[e - 64];
+        }
+    }
+    __syncthreads();
+    // the first convolution over the whole of its channels, into LDS (and, from the first channel range, into y1)
+    if (wave < a.t1) run_stage<KA, true>(a, xs, sx, ys, sy, a.lut_a ? lut_a : nullptr, wave, waves, a.t1, la, lane, p, blockIdx.y == 0);
+    __syncthreads();
+    // the second: this workgroup's channel tiles from the LDS tile
+    if (b_first + wave < b_end) run_stage<KB, false>(a, ys, sy, nullptr, 0, a.lut_b ? lut_b : nullptr, b_first + wave, waves, b_end, lb, lane, p, false);
+}
+
+bool pair_is_small(int ks1, int ks2) { return ks1 <= 4 && ks2 <= 2; }
+size_t pair_lds_bytes(const nncase_hip_qpair *pr) {
+    const bool small = pair_is_small(pr->ks1, pr->ks2);
+    return 16 * (size_t)pair_row_bytes(pr->ks1, small ? 4 : 8) + 16 * (size_t)pair_row_bytes(pr->ks2, small ? 2 : 4) + 512;
+}
+
+// [tile][k-step][lane][16] s8 of w - 128, zero beyond the real channels / reduction
+void pack_pair_weights(std::vector<uint8_t> &out, std::vector<int32_t> &wsum, const uint8_t *w_oihw, int n, int k, int tiles, int ksteps) {
+    out.assign((size_t)tiles * ksteps * 1024, 0);
+    wsum.assign((size_t)tiles * 16, 0);
+    for (int ch = 0; ch < n; ch++) {
+        int32_t s = 0;
+        for (int kk = 0; kk < k; kk++) {
+            const uint8_t raw = w_oihw[(size_t)ch * k + kk];
+            s += (int32_t)raw - 128;
+            const int t = ch >> 4, i = ch & 15, ks = kk >> 6, g = (kk >> 4) & 3, b = kk & 15;
+            out[(((size_t)t * ksteps + ks) * 64 + g * 16 + i) * 16 + b] = raw ^ 0x80;
+        }
+        wsum[ch] = s;
+    }
+}
+
+void free_pair(nncase_hip_qpair *pr) {
+    if (!pr) return;
+    if (pr->d_wa) (void)hipFree(pr->d_wa);
+    if (pr->d_wb) (void)hipFree(pr->d_wb);
+    if (pr->d_wsum_a) (void)hipFree(pr->d_wsum_a);
+    if (pr->d_wsum_b) (void)hipFree(pr->d_wsum_b);
+    if (pr->d_bias_a) (void)hipFree(pr->d_bias_a);
+    if (pr->d_bias_b) (void)hipFree(pr->d_bias_b);
+    delete pr;
+}
+
+bool pair_shapes_ok(int k1, int n1, int n2) {
+    return k1 > 0 && n1 > 0 && n2 > 0 && k1 % 16 == 0 && n1 % 4 == 0 && n2 % 4 == 0 && k1 <= kPairMaxK1 && n1 <= kPairMaxN1;
+}
+
+int upload(nncase_hip_ctx *ctx, void **dst, const void *src, size_t bytes) {
+    NNHIP_HIP(ctx, hipMalloc(dst, bytes));
+    NNHIP_HIP(ctx, hipMemcpy(*dst, src, bytes, hipMemcpyHostToDevice));
+    return 0;
+}
+
+bool pointwise_weights(const nncase_hip_weights *w) {
+    return w && w->kind == nncase_hip_weights::kIgemm && w->groups == 1 && w->kernel_h == 1 && w->kernel_w == 1;
+}
+
+} // namespace
+
+extern "C" int nncase_hip_qpointwise_pair_supported(int32_t in_channels, int32_t mid_channels, int32_t out_channels) {
+    return pair_shapes_ok(in_channels, mid_channels, out_channels) ? 1 : 0;
+}
+
+extern "C" int nncase_hip_qpointwise_pair_create(nncase_hip_ctx_t *ctx, const nncase_hip_weights_t *first,
+                                                 const uint8_t *first_oihw_host, const nncase_hip_weights_t *second,
+                                                 const uint8_t *second_oihw_host, nncase_hip_qpair_t **pair) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, first && first_oihw_host && second && second_oihw_host && pair, -EINVAL, "qpointwise_pair_create: null argument");
+    *pair = nullptr;
+    NNHIP_REQUIRE(ctx, pointwise_weights(first) && pointwise_weights(second), -EINVAL,
+                  "qpointwise_pair_create: both convolutions must be dense 1x1 convolutions");
+    NNHIP_REQUIRE(ctx, first->out_channels == second->in_channels, -NNCASE_HIP_ERR_SHAPE_MISMATCH,
+                  "qpointwise_pair_create: the first convolution has %d output channels, the second reads %d", first->out_channels,
+                  second->in_channels);
+    NNHIP_REQUIRE(ctx, pair_shapes_ok(first->in_channels, first->out_channels, second->out_channels), -EINVAL,
+                  "qpointwise_pair_create: channels %d -> %d -> %d unsupported (first a multiple of 16 up to %d, second a multiple of 4 "
+                  "up to %d, third a multiple of 4)",
+                  first->in_channels, first->out_channels, second->out_channels, kPairMaxK1, kPairMaxN1);
+    nncase_hip_qpair *pr = new (std::nothrow) nncase_hip_qpair();
+    NNHIP_REQUIRE(ctx, pr, -ENOMEM, "qpointwise_pair_create: out of host memory");
+    pr->first = first, pr->second = second;
+    pr->k1 = first->in_channels, pr->n1 = first->out_channels, pr->n2 = second->out_channels;
+    pr->ks1 = (pr->k1 + 63) / 64, pr->ks2 = (pr->n1 + 63) / 64;
+    pr->t1 = (pr->n1 + 15) / 16, pr->t2 = (pr->n2 + 15) / 16;
+    NNHIP_HIP(ctx, hipSetDevice(ctx->device));
+    std::vector<uint8_t> packed;
+    std::vector<int32_t> wsum, bias;
+    int rc = 0;
+    auto side = [&](const nncase_hip_weights *w, const uint8_t *host, int n, int k, int tiles, int ksteps, uint8_t **d_w, int32_t **d_wsum,
+                    int32_t **d_bias) -> int {
+        pack_pair_weights(packed, wsum, host, n, k, tiles, ksteps);
+        bias.assign((size_t)tiles * 16, 0);
+        NNHIP_HIP(ctx, hipMemcpy(bias.data(), w->d_bias, sizeof(int32_t) * n, hipMemcpyDeviceToHost));
+        int r = upload(ctx, (void **)d_w, packed.data(), packed.size());
+        if (!r) r = upload(ctx, (void **)d_wsum, wsum.data(), wsum.size() * sizeof(int32_t));
+        if (!r) r = upload(ctx, (void **)d_bias, bias.data(), bias.size() * sizeof(int32_t));
+        return r;
+    };
+    rc = side(first, first_oihw_host, pr->n1, pr->k1, pr->t1, pr->ks1, &pr->d_wa, &pr->d_wsum_a, &pr->d_bias_a);
+    if (!rc) rc = side(second, second_oihw_host, pr->n2, pr->n1, pr->t2, pr->ks2, &pr->d_wb, &pr->d_wsum_b, &pr->d_bias_b);
+    if (rc) {
+        free_pair(pr);
+        return rc;
+    }
+    *pair = pr;
+    return 0;
+}
+
+extern "C" int nncase_hip_qpointwise_pair_destroy(nncase_hip_ctx_t *ctx, nncase_hip_qpair_t *pair) {
+    NNHIP_CHECK_CTX(ctx);
+    if (!pair) return 0;
+    NNHIP_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    free_pair(pair);
+    return 0;
+}
+
+extern "C" int nncase_hip_qpointwise_pair(nncase_hip_ctx_t *ctx, const uint8_t *x_dev, const nncase_hip_qpair_t *pr, uint8_t *y1_dev,
+                                          uint8_t *y2_dev, const nncase_hip_conv2d_args_t *fa, const nncase_hip_conv2d_args_t *sa) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, x_dev && pr && y1_dev && y2_dev && fa && sa, -EINVAL, "qpointwise_pair: null argument");
+    NNHIP_REQUIRE(ctx, fa->batch > 0 && fa->in_h > 0 && fa->in_w > 0, -EINVAL, "qpointwise_pair: non-positive input shape");
+    NNHIP_REQUIRE(ctx, sa->batch == fa->batch && sa->in_h == fa->in_h && sa->in_w == fa->in_w, -NNCASE_HIP_ERR_SHAPE_MISMATCH,
+                  "qpointwise_pair: the second convolution reads [%d,%d,%d], the first writes [%d,%d,%d]", sa->batch, sa->in_h, sa->in_w,
+                  fa->batch, fa->in_h, fa->in_w);
+    for (const nncase_hip_conv2d_args_t *c : {fa, sa}) {
+        NNHIP_REQUIRE(ctx, c->stride_h == 1 && c->stride_w == 1 && c->pad_h_before == 0 && c->pad_h_after == 0 && c->pad_w_before == 0 &&
+                               c->pad_w_after == 0,
+                      -EINVAL, "qpointwise_pair: stride 1 and no padding only");
+        NNHIP_REQUIRE(ctx, c->out_dtype == NNCASE_HIP_DT_U8 && c->dequantize_output == 0, -NNCASE_HIP_ERR_DATATYPE_MISMATCH,
+                      "qpointwise_pair: u8 results only");
+        NNHIP_REQUIRE(ctx, c->out_channel_stride == 0 && c->out_channel_offset == 0, -EINVAL, "qpointwise_pair: dense results only");
+        NNHIP_REQUIRE(ctx, c->x_qp.zero_point >= 0 && c->x_qp.zero_point <= 255, -EINVAL, "qpointwise_pair: input zero point %d outside u8",
+                      c->x_qp.zero_point);
+        NNHIP_REQUIRE(ctx, c->y_qp.scale > 0.f && std::isfinite(c->y_qp.scale) && c->y_qp.zero_point >= 0 && c->y_qp.zero_point <= 255, -EINVAL,
+                      "qpointwise_pair: output quantisation outside u8");
+    }
+    NNHIP_REQUIRE(ctx, !sa->residual_dev, -EINVAL, "qpointwise_pair: only the first convolution takes a residual");
+    if (fa->residual_dev)
+        NNHIP_REQUIRE(ctx, fa->sum_qp.scale > 0.f && std::isfinite(fa->sum_qp.scale) && fa->sum_qp.zero_point >= 0 && fa->sum_qp.zero_point <= 255,
+                      -EINVAL, "qpointwise_pair: sum quantisation outside u8");
+    const int64_t m64 = (int64_t)fa->batch * fa->in_h * fa->in_w;
+    NNHIP_REQUIRE(ctx, m64 < ((int64_t)1 << 30), -EINVAL, "qpointwise_pair: %lld pixels unsupported", (long long)m64);
+    NNHIP_REQUIRE(ctx, ((reinterpret_cast<uintptr_t>(x_dev) | reinterpret_cast<uintptr_t>(y1_dev) | reinterpret_cast<uintptr_t>(y2_dev)) & 15u) == 0,
+                  -NNCASE_HIP_ERR_INVALID_MEMORY_LOCATION, "qpointwise_pair: activation buffers must be 16-byte aligned");
+
+    PairArgs a;
+    memset(&a, 0, sizeof(a));
+    a.x = x_dev, a.y1 = y1_dev, a.y2 = y2_dev;
+    a.wa = pr->d_wa, a.wb = pr->d_wb;
+    a.bias_a = pr->d_bias_a, a.wsum_a = pr->d_wsum_a, a.bias_b = pr->d_bias_b, a.wsum_b = pr->d_wsum_b;
+    a.lut_a = pr->first->d_post_lut, a.lut_b = pr->second->d_post_lut;
+    a.m = (int)m64;
+    a.k1 = pr->k1, a.n1 = pr->n1, a.n2 = pr->n2;
+    a.ks1 = pr->ks1, a.ks2 = pr->ks2, a.t1 = pr->t1, a.t2 = pr->t2;
+    a.zxa = fa->x_qp.zero_point - 128, a.zwa = pr->first->zw - 128;
+    a.zxb = sa->x_qp.zero_point - 128, a.zwb = pr->second->zw - 128;
+    int rc = make_epilogue(ctx, &a.ep_a, fa->x_qp.scale, pr->first->sw, fa->y_qp, fa->clamp_min, fa->clamp_max, NNCASE_HIP_DT_U8, "qpointwise_pair");
+    if (!rc) rc = make_epilogue(ctx, &a.ep_b, sa->x_qp.scale, pr->second->sw, sa->y_qp, sa->clamp_min, sa->clamp_max, NNCASE_HIP_DT_U8, "qpointwise_pair");
+    if (!rc) rc = make_residual_epilogue(ctx, &a.rep_a, fa, pr->first);
+    if (rc) return rc;
+
+    // A wave per channel tile of whichever convolution has more of them in this workgroup (up to the variant's most),
+    // and enough workgroups to occupy the device: pixel tiles x ranges of the second convolution's channel tiles.
+    const bool small = pair_is_small(a.ks1, a.ks2);
+    const int max_waves = small ? 16 : 12;
+    const int ptiles = (a.m + 15) / 16;
+    int ranges = (a.t2 + max_waves - 1) / max_waves;
+    const int want = ptiles >= 512 ? 1 : 512 / ptiles;
+    if (ranges > want) ranges = want;
+    a.tiles_per_block = (a.t2 + ranges - 1) / ranges;
+    ranges = (a.t2 + a.tiles_per_block - 1) / a.tiles_per_block;
+    const int waves = std::min(max_waves, std::max(a.t1, a.tiles_per_block));
+    NNHIP_HIP(ctx, hipSetDevice(ctx->device));
+    if (small)
+        hipLaunchKernelGGL((qpointwise_pair_kernel<4, 2, 16, 5>), dim3(ptiles, ranges), dim3(waves * 64), pair_lds_bytes(pr), ctx->stream, a);
+    else
+        hipLaunchKernelGGL((qpointwise_pair_kernel<8, 4, 12, 3>), dim3(ptiles, ranges), dim3(waves * 64), pair_lds_bytes(pr), ctx->stream, a);
+    NNHIP_LAUNCH_CHECK(ctx, "qpointwise_pair_kernel");
+    return 0;
+}

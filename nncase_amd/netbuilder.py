@@ -396,6 +396,14 @@ def pad_small_channel_convs(qg: QuantGraph) -> QuantGraph:
 
 
 # --------------------------------------------------------------------------------------------- device binding
+# Where a pointwise pair replaces its two convolutions: while the weight bytes its workgroups stream between them
+# (pixel tiles x both weight tensors) stay small, and while all its workgroups (one per 16 pixels and channel range) are
+# resident at once.  Measured on MobileNetV2: every pair within these limits is quicker than its two launches at
+# batches 1 and 2 (0.215 -> 0.184 ms per image at batch 1); beyond them the separate kernels win.
+PAIR_STREAM_LIMIT = 4 << 20
+PAIR_MAX_PIXEL_TILES = 512
+
+
 class HipModel:
     """A QuantGraph resident on the device: packed weights, one HBM buffer per tensor, and the
     operator list recorded in a `hip` function.  run() = upload input, invoke, download output.
@@ -407,7 +415,7 @@ class HipModel:
     so results are bit-identical to lanes == 1."""
 
     def __init__(self, ctx: Context, qg: QuantGraph, batch: int, capture_graph: bool = True, fuse_residual: bool = True,
-                 lanes: int = 1, fuse_blocks=True):
+                 lanes: int = 1, fuse_blocks=True, fuse_pairs=True):
         if lanes < 1 or lanes > rt.MAX_LANES or batch % lanes:
             raise ValueError(f"lanes={lanes} must be in 1..{rt.MAX_LANES} and divide the batch ({batch})")
         self.ctx, self.qg, self.batch, self.lanes = ctx, qg, batch, lanes
@@ -555,6 +563,37 @@ class HipModel:
                         and (conv == j or consumers[conv] == 1)):
                     self.fused_dequant[conv] = oi
                     self.never_written |= {conv, j} | ({self.fused_lut[conv]} if conv in self.fused_lut else set())
+        # A dense 1x1 convolution (with its folded table / add) whose result a second dense 1x1 convolution reads runs
+        # with it as one launch where the two are latency-bound: a bottleneck's projection and the next block's
+        # expansion at small batches.  Every workgroup of the pair repeats the first convolution for its 16 pixels, so
+        # the weights it streams (pixel tiles x both weight tensors) bound where that still pays.
+        self.pairs: Dict[int, int] = {}                                                  # first conv -> second conv
+        if fuse_pairs and fuse_residual:
+            def pointwise1(j):
+                n = qg.nodes[j]
+                return (n.op == "conv" and n.groups == 1 and n.weights.shape[2:] == (1, 1) and tuple(n.stride) == (1, 1)
+                        and tuple(map(tuple, n.padding)) == ((0, 0), (0, 0)) and j not in block_members
+                        and j not in self.write_through and j not in self.fused_dequant)
+            taken = set()
+            for i, n in enumerate(qg.nodes):
+                if i in taken or not pointwise1(i):
+                    continue
+                tail = self.fused_into.get(i, self.fused_lut.get(i, i))
+                seconds = [j for j in range(tail + 1, len(qg.nodes)) if tuple(qg.nodes[j].inputs) == (tail,) and pointwise1(j)
+                           and j not in self.fused_into and j not in taken]
+                if not seconds:
+                    continue
+                j = seconds[0]
+                k1, n1, n2 = n.weights.shape[1], n.weights.shape[0], qg.nodes[j].weights.shape[0]
+                if not ctx.qpointwise_pair_supported(k1, n1, n2):
+                    continue
+                ptiles = -(-(bl * n.out_shape[1] * n.out_shape[2]) // 16)
+                if fuse_pairs != "all" and (ptiles > PAIR_MAX_PIXEL_TILES or ptiles * (k1 * n1 + n1 * n2) > PAIR_STREAM_LIMIT):
+                    continue
+                self.pairs[i] = j
+                taken |= {i, j}
+                skip_nodes.add(j)
+        self.pair_objects: Dict[int, rt.QPair] = {}
         # buffers and packed weights once, shared by the lanes
         for i, n in enumerate(qg.nodes):
             cc, hh, ww = n.out_shape
@@ -583,6 +622,8 @@ class HipModel:
                 elif fused_lut is not None:
                     wt.set_post_lut(qg.nodes[fused_lut].lut, qp(*qg.nodes[fused_lut].out_qp))
                 self.weights[-1] = wt
+        for a_, b_ in self.pairs.items():
+            self.pair_objects[a_] = ctx.prepack_qpointwise_pair(self.weights[a_], qg.nodes[a_].weights, self.weights[b_], qg.nodes[b_].weights)
         self.outputs_f32: List[rt.DeviceBuffer] = [ctx.alloc(lanes * self._lane_stride(bl * int(np.prod(qg.nodes[j].out_shape)) * 4))
                                                     for j in qg.output_nodes]
         for lane in range(lanes):
@@ -660,6 +701,20 @@ class HipModel:
                     per = bl * int(np.prod(oj.out_shape)) * 4
                     buf = self.outputs_f32[self.fused_dequant[i]].view(lane * self._lane_stride(per), per)
                     args.out_dtype, args.dequantize_output = rt.DT_F32, 1
+                if i in self.pairs:
+                    j = self.pairs[i]
+                    sn, sn_in = qg.nodes[j], qg.nodes[j].inputs[0]
+                    mid = qg.nodes[sn_in]
+                    second = rt.Conv2dArgs(bl, mid.out_shape[1], mid.out_shape[2], 1, 1, 1, 1, 0, 0, 0, 0, qp(*mid.out_qp), qp(*sn.out_qp),
+                                           sn.clamp[0], sn.clamp[1], rt.DT_U8)
+                    lut2 = self.fused_lut.get(j)
+                    self.fn.add_qpointwise_pair(B(n.inputs[0]), self.pair_objects[i], B(sn_in), B(lut2 if lut2 is not None else j), args, second)
+                    if lane == 0:
+                        self.op_names.append(f"pair:{n.name}" + ("+lut" if fused_lut is not None else "") + ("+add" if fused_add is not None else "")
+                                             + f">{sn.name}" + ("+lut" if lut2 is not None else ""))
+                        self.op_nodes.append(lut2 if lut2 is not None else j)
+                        self.op_members.append(members + [j] + ([lut2] if lut2 is not None else []))
+                    continue
                 self.fn.add_qconv2d(B(n.inputs[0]), self.weights[i], buf, args)
             elif n.op == "add":
                 a, b = (qg.nodes[j] for j in n.inputs)

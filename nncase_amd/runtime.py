@@ -116,6 +116,11 @@ SYMBOLS = {
     "nncase_hip_qblock_destroy": (_I, [_VP, _VP]),
     "nncase_hip_qblock": (_I, [_VP, _VP, _VP, _VP, C.POINTER(QBlockArgs)]),
     "nncase_hip_function_add_qblock": (_I, [_VP, _VP, _VP, _VP, C.POINTER(QBlockArgs)]),
+    "nncase_hip_qpointwise_pair_supported": (_I, [C.c_int32, C.c_int32, C.c_int32]),
+    "nncase_hip_qpointwise_pair_create": (_I, [_VP, _VP, _VP, _VP, _VP, C.POINTER(_VP)]),
+    "nncase_hip_qpointwise_pair_destroy": (_I, [_VP, _VP]),
+    "nncase_hip_qpointwise_pair": (_I, [_VP, _VP, _VP, _VP, _VP, C.POINTER(Conv2dArgs), C.POINTER(Conv2dArgs)]),
+    "nncase_hip_function_add_qpointwise_pair": (_I, [_VP, _VP, _VP, _VP, _VP, C.POINTER(Conv2dArgs), C.POINTER(Conv2dArgs)]),
     "nncase_hip_qmatmul_prepack": (_I, [_VP, _VP, C.c_int32, C.c_int32, QuantParam, _VP, C.c_int64, C.POINTER(_VP)]),
     "nncase_hip_qmatmul": (_I, [_VP, _VP, _VP, _VP, C.POINTER(MatmulArgs)]),
     "nncase_hip_qadd": (_I, [_VP, _VP, QuantParam, _VP, QuantParam, _VP, QuantParam, C.c_float, C.c_float, _SZ]),
@@ -381,6 +386,25 @@ class Weights:
             pass
 
 
+class QPair:
+    """Two pointwise convolutions packed to run as one launch (nncase_hip_qpair_t); keeps both Weights alive."""
+
+    def __init__(self, ctx: "Context", handle, first: "Weights", second: "Weights"):
+        self.ctx, self.handle, self.first, self.second = ctx, handle, first, second
+
+    def destroy(self):
+        if self.handle:
+            if self.ctx.handle:
+                self.ctx.lib.nncase_hip_qpointwise_pair_destroy(self.ctx.handle, self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass
+
+
 class QBlock:
     """Pre-packed constants of a fused expand -> depthwise -> project block (nncase_hip_qblock_t)."""
 
@@ -522,6 +546,23 @@ class Context:
 
     def qblock(self, x, blk: QBlock, y, args: QBlockArgs):
         self._check(self.lib.nncase_hip_qblock(self.handle, x.ptr, blk.handle, y.ptr, C.byref(args)), "qblock")
+
+    def qpointwise_pair_supported(self, cin: int, mid: int, cout: int) -> bool:
+        return bool(self.lib.nncase_hip_qpointwise_pair_supported(cin, mid, cout))
+
+    def prepack_qpointwise_pair(self, first: Weights, first_oihw: np.ndarray, second: Weights, second_oihw: np.ndarray) -> QPair:
+        """`first` / `second` are the prepack_conv2d handles of the two 1x1 convolutions (bias, quantisation, tables),
+        the arrays their OIHW u8 weights [mid, in, 1, 1] and [out, mid, 1, 1] once more."""
+        wa, wb = (np.ascontiguousarray(w, np.uint8) for w in (first_oihw, second_oihw))
+        assert wa.shape[2:] == (1, 1) and wb.shape[2:] == (1, 1)
+        h = C.c_void_p()
+        self._check(self.lib.nncase_hip_qpointwise_pair_create(self.handle, first.handle, wa.ctypes.data, second.handle, wb.ctypes.data,
+                                                               C.byref(h)), "qpointwise_pair_create")
+        return QPair(self, h.value, first, second)
+
+    def qpointwise_pair(self, x, pair: QPair, y1, y2, first_args: Conv2dArgs, second_args: Conv2dArgs):
+        self._check(self.lib.nncase_hip_qpointwise_pair(self.handle, x.ptr, pair.handle, y1.ptr, y2.ptr, C.byref(first_args),
+                                                        C.byref(second_args)), "qpointwise_pair")
 
     def prepack_matmul(self, b_kn: np.ndarray, bias: Optional[np.ndarray], b_qp: QuantParam, expected_rows: int = 0) -> Weights:
         b = np.ascontiguousarray(b_kn, np.uint8)
@@ -673,6 +714,11 @@ class Function:
         self._keep += [x, blk, y]
         self._ck(self.ctx.lib.nncase_hip_function_add_qblock(self.handle, x.ptr, blk.handle, y.ptr, C.byref(args)),
                  "function_add_qblock")
+
+    def add_qpointwise_pair(self, x, pair: QPair, y1, y2, first_args: Conv2dArgs, second_args: Conv2dArgs):
+        self._keep += [x, pair, y1, y2]
+        self._ck(self.ctx.lib.nncase_hip_function_add_qpointwise_pair(self.handle, x.ptr, pair.handle, y1.ptr, y2.ptr, C.byref(first_args),
+                                                                      C.byref(second_args)), "function_add_qpointwise_pair")
 
     def add_qadd(self, a, a_qp, b, b_qp, out, y_qp, count, clamp=(-FLT_MAX, FLT_MAX)):
         self._keep += [a, b, out]

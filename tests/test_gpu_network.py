@@ -14,8 +14,9 @@ pytestmark = pytest.mark.gpu
 f32 = np.float32
 
 
-def check_model(hip_ctx, qg, x, capture, fuse_residual=True, fuse_blocks="all"):
-    model = nb.HipModel(hip_ctx, qg, x.shape[0], capture_graph=capture, fuse_residual=fuse_residual, fuse_blocks=fuse_blocks)
+def check_model(hip_ctx, qg, x, capture, fuse_residual=True, fuse_blocks="all", fuse_pairs=True):
+    model = nb.HipModel(hip_ctx, qg, x.shape[0], capture_graph=capture, fuse_residual=fuse_residual, fuse_blocks=fuse_blocks,
+                        fuse_pairs=fuse_pairs)
     y = model.run(x)
     want, outs = netref.run_integer(qg, x, keep_all=True)
     for i, ref in enumerate(outs):
@@ -71,9 +72,13 @@ def test_mobilenetv2_config3(hip_ctx):
     x = rng.random((2, 224, 224, 3), dtype=f32)
     plain, _, _ = check_model(hip_ctx, qg, x, capture=False, fuse_residual=False)   # every tensor, add as its own kernel
     assert len(plain.fused_into) == 0 and len(plain.fn) == 67     # (quantize, pack of 2 x 2 pixel blocks, 52 convs, ...)
-    model, y, outs = check_model(hip_ctx, qg, x, capture=True, fuse_blocks=False)
+    model, y, outs = check_model(hip_ctx, qg, x, capture=True, fuse_blocks=False, fuse_pairs=False)
     assert len(model.fused_into) == 10 and len(model.fused_dequant) == 1 and len(model.fn) == 55   # residual adds folded into
     #                                                                            the convs, the output's dequantize into the classifier
+    model, y, outs = check_model(hip_ctx, qg, x, capture=True, fuse_blocks=False, fuse_pairs="all")
+    assert len(model.pairs) == 17 and len(model.fn) == 38     # every projection runs with the expansion behind it as one launch
+    model, y, outs = check_model(hip_ctx, qg, x, capture=True, fuse_blocks=False)
+    assert 0 < len(model.pairs) < 17                           # ... at this batch, where the pair streams few weights
     model, y, outs = check_model(hip_ctx, qg, x, capture=True)
     assert len(model.blocks) == 16 and len(model.fn) == 23                            # ... and whole blocks into one operator
     # the reference's own acceptance bar for a PTQ model: cosine >= 0.98 against the float model
@@ -146,7 +151,8 @@ def test_yolov5s_config4(hip_ctx):
         # operators, with fewer inputs each
         # ; the three detect convs store the dequantised outputs themselves
         assert (len(model.fused_lut), len(model.fused_into), len(model.write_through), len(model.fused_quant), len(model.fused_dequant),
-                len(model.fn)) == ((57, 7, 17, 1, 3, 147 - 64 - 7 - 1 - 3) if fuse else (0, 0, 0, 0, 0, 147))
+                len(model.fn)) == ((57, 7, 17, 1, 3, 147 - 64 - 7 - 1 - 3 - 11) if fuse else (0, 0, 0, 0, 0, 147))
+        assert len(model.pairs) == (11 if fuse else 0)     # 1x1 convolutions that read a 1x1 convolution run as one launch with it
         for i, ref in enumerate(outs):
             if not model.materialized(i):
                 continue
@@ -348,7 +354,7 @@ def test_mobilenetv2_fused_blocks_match_separate_operators(hip_ctx):
     rng = np.random.default_rng(3)
     qg = nb.quantize_graph(g, rng.random((32, 224, 224, 3), dtype=f32))
     x = np.random.default_rng(4).random((8, 224, 224, 3), dtype=f32)
-    plain = nb.HipModel(hip_ctx, qg, 8, capture_graph=False, fuse_blocks=False)
+    plain = nb.HipModel(hip_ctx, qg, 8, capture_graph=False, fuse_blocks=False, fuse_pairs=False)
     y0 = plain.run(x)
     for capture, lanes in ((False, 1), (True, 1), (True, 2)):
         fused = nb.HipModel(hip_ctx, qg, 8, capture_graph=capture, lanes=lanes, fuse_blocks="all")
