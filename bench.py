@@ -513,7 +513,7 @@ def main():
             m1.invoke()
         ctx.sync()
         b1_ms = (time.perf_counter() - t1) / args.batch1_steps * 1e3
-        b1 = {"ms_per_image": round(b1_ms, 4), "images_per_s": round(1e3 / b1_ms, 1)}
+        b1 = {"ms_per_image": round(b1_ms, 4), "images_per_s": round(1e3 / b1_ms, 1), "operators": len(m1.fn)}
         # the batched run must give image 0 the very logits it gets alone (integer arithmetic: bit-exact);
         # the batch-1 graph is the one the GPU tests follow tensor by tensor against the CPU oracle
         model.invoke()

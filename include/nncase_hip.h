@@ -330,6 +330,19 @@ NNCASE_HIP_API int nncase_hip_qpointwise_pair(nncase_hip_ctx_t *ctx, const uint8
                                               uint8_t *y1_dev, uint8_t *y2_dev, const nncase_hip_conv2d_args_t *first_args,
                                               const nncase_hip_conv2d_args_t *second_args);
 
+/* The same with the 3x3 depthwise Conv2D (stride 1 or 2, no dilation) that produces x in front, still one launch:
+ * x_dev is the DEPTHWISE convolution's input [batch, in_h, in_w, in_channels]; its result, which nothing else may
+ * need, is never stored (each workgroup computes its 16 pixels of it into LDS).  depthwise is the prepack handle of
+ * the depthwise weights (no table), depthwise_args its nncase_hip_qconv2d arguments; its y_qp must be first_args->x_qp
+ * and its output extents first_args' input extents.  y1 and y2 are bit-identical to the three nncase_hip_qconv2d
+ * calls. */
+NNCASE_HIP_API int nncase_hip_qdepthwise_pointwise_pair(nncase_hip_ctx_t *ctx, const uint8_t *x_dev,
+                                                        const nncase_hip_weights_t *depthwise,
+                                                        const nncase_hip_conv2d_args_t *depthwise_args,
+                                                        const nncase_hip_qpair_t *pair, uint8_t *y1_dev, uint8_t *y2_dev,
+                                                        const nncase_hip_conv2d_args_t *first_args,
+                                                        const nncase_hip_conv2d_args_t *second_args);
+
 /* MatMul A[M,K] (u8, device) x B[K,N] (u8, row-major, HOST, pre-packed) with
  * the same three output forms; replaces kernels::stackvm::mat_mul
  * (tensor_ops.cpp:553-565 -> reference/matmul.cpp:28-48) on the
@@ -582,6 +595,13 @@ NNCASE_HIP_API int nncase_hip_function_add_qpointwise_pair(nncase_hip_function_t
                                                            const nncase_hip_qpair_t *pair, uint8_t *y1_dev, uint8_t *y2_dev,
                                                            const nncase_hip_conv2d_args_t *first_args,
                                                            const nncase_hip_conv2d_args_t *second_args);
+NNCASE_HIP_API int nncase_hip_function_add_qdepthwise_pointwise_pair(nncase_hip_function_t *fn, const uint8_t *x_dev,
+                                                                     const nncase_hip_weights_t *depthwise,
+                                                                     const nncase_hip_conv2d_args_t *depthwise_args,
+                                                                     const nncase_hip_qpair_t *pair, uint8_t *y1_dev,
+                                                                     uint8_t *y2_dev,
+                                                                     const nncase_hip_conv2d_args_t *first_args,
+                                                                     const nncase_hip_conv2d_args_t *second_args);
 NNCASE_HIP_API int nncase_hip_function_add_qadd(nncase_hip_function_t *fn, const uint8_t *a_dev,
                                                 nncase_hip_quant_param_t a_qp, const uint8_t *b_dev,
                                                 nncase_hip_quant_param_t b_qp, uint8_t *out_dev,

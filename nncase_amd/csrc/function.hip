@@ -38,8 +38,10 @@ struct Op {
     float eps = 0.f, theta = 0.f;
     const nncase_hip_qblock_t *block = nullptr;
     nncase_hip_qblock_args_t blk{};
-    const nncase_hip_qpair_t *pair = nullptr; // with conv (first) and conv2 (second) arguments, out / out2 the two results
-    nncase_hip_conv2d_args_t conv2{};
+    // pair: conv (first) and conv2 (second) arguments, out / out2 the two results; with `weights` a depthwise
+    // convolution in front, whose arguments are conv3
+    const nncase_hip_qpair_t *pair = nullptr;
+    nncase_hip_conv2d_args_t conv2{}, conv3{};
     int lane = 0; // independent operator chain this operator belongs to
 };
 
@@ -72,6 +74,9 @@ static int run_op(nncase_hip_function *fn, const Op &op) {
     case Op::kBlock:
         return nncase_hip_qblock(ctx, (const uint8_t *)op.in0, op.block, (uint8_t *)op.out, &op.blk);
     case Op::kPair:
+        if (op.weights)
+            return nncase_hip_qdepthwise_pointwise_pair(ctx, (const uint8_t *)op.in0, op.weights, &op.conv3, op.pair, (uint8_t *)op.out,
+                                                        (uint8_t *)op.out2, &op.conv, &op.conv2);
         return nncase_hip_qpointwise_pair(ctx, (const uint8_t *)op.in0, op.pair, (uint8_t *)op.out, (uint8_t *)op.out2, &op.conv, &op.conv2);
     case Op::kAdd:
         return nncase_hip_qadd(ctx, (const uint8_t *)op.in0, op.qp0, (const uint8_t *)op.in1, op.qp1, (uint8_t *)op.out,
@@ -223,6 +228,21 @@ extern "C" int nncase_hip_function_add_qpointwise_pair(nncase_hip_function_t *fn
     Op op;
     op.kind = Op::kPair;
     op.in0 = x_dev, op.out = y1_dev, op.out2 = y2_dev, op.pair = pair, op.conv = *first_args, op.conv2 = *second_args;
+    return push(fn, op);
+}
+
+extern "C" int nncase_hip_function_add_qdepthwise_pointwise_pair(nncase_hip_function_t *fn, const uint8_t *x_dev,
+                                                                 const nncase_hip_weights_t *depthwise,
+                                                                 const nncase_hip_conv2d_args_t *depthwise_args, const nncase_hip_qpair_t *pair,
+                                                                 uint8_t *y1_dev, uint8_t *y2_dev, const nncase_hip_conv2d_args_t *first_args,
+                                                                 const nncase_hip_conv2d_args_t *second_args) {
+    if (!fn) return -EINVAL;
+    NNHIP_REQUIRE(fn->ctx, x_dev && depthwise && depthwise_args && pair && y1_dev && y2_dev && first_args && second_args, -EINVAL,
+                  "function_add_qdepthwise_pointwise_pair: null argument");
+    Op op;
+    op.kind = Op::kPair;
+    op.in0 = x_dev, op.out = y1_dev, op.out2 = y2_dev, op.pair = pair, op.conv = *first_args, op.conv2 = *second_args;
+    op.weights = depthwise, op.conv3 = *depthwise_args;
     return push(fn, op);
 }
 
@@ -595,7 +615,7 @@ extern "C" int nncase_hip_function_op_kernel(nncase_hip_function_t *fn, int32_t 
     case Op::kDequantize: snprintf(name, capacity, "dequantize"); break;
     case Op::kConv: describe_conv_kernel(fn->ctx, op.weights, &op.conv, name, capacity); break;
     case Op::kBlock: nncase_hip_qblock_describe(op.block, &op.blk, name, capacity); break;
-    case Op::kPair: snprintf(name, capacity, "qpointwise_pair_kernel"); break;
+    case Op::kPair: snprintf(name, capacity, op.weights ? "dw3x3+qpointwise_pair_kernel" : "qpointwise_pair_kernel"); break;
     case Op::kAdd: snprintf(name, capacity, "qadd"); break;
     case Op::kPool: snprintf(name, capacity, "qglobal_avgpool"); break;
     case Op::kLut: snprintf(name, capacity, "lut_u8"); break;

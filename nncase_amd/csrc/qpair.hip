@@ -56,6 +56,14 @@ struct PairArgs {
     int zxa, zwa, zxb, zwb; // zero points - 128
     Epilogue ep_a, ep_b;
     ResidualEpilogue rep_a;
+    // with a 3x3 depthwise convolution in front (the DW kernels): x is ITS input [batch, in_h, in_w, k1], and the pixel
+    // tile the first convolution multiplies is computed here instead of loaded
+    const int16_t *dw_w;             // [9][k1]  w - zw
+    const int32_t *dw_bias, *dw_wsum; // [k1]; sum over the taps of w - zw
+    int in_h, in_w, out_w, out_hw, stride, pad_h, pad_w;
+    FastDiv d_out_hw, d_out_w;
+    int dw_zx;
+    Epilogue ep_dw;
 };
 
 __device__ __forceinline__ uint32_t table4(const uint8_t *t, uint32_t v) {
@@ -151,9 +159,77 @@ __device__ __forceinline__ void run_stage(const PairArgs &a, const uint8_t *rows
     }
 }
 
+// The nine input dwords (four channels from c4) of output pixel `px`'s window; taps outside the image read as the
+// zero point, whose share the accumulator's start value takes back out (addresses are clamped into the image, so the
+// loads need no branch).
+__device__ __forceinline__ void dw_fetch(uint32_t (&buf)[9], const PairArgs &a, int px, int c4) {
+    px = min(px, a.m - 1);
+    const int n = (int)fastdiv((uint32_t)px, a.d_out_hw), rem = px - n * a.out_hw;
+    const int oy = (int)fastdiv((uint32_t)rem, a.d_out_w), ox = rem - oy * a.out_w;
+    const int iy0 = oy * a.stride - a.pad_h, ix0 = ox * a.stride - a.pad_w;
+    const uint32_t zx4 = (uint32_t)a.dw_zx * 0x01010101u;
+#pragma unroll
+    for (int ky = 0; ky < 3; ky++) {
+        const int iy = iy0 + ky, iyc = min(max(iy, 0), a.in_h - 1);
+        const uint8_t *rowp = a.x + (size_t)(n * a.in_h + iyc) * a.in_w * a.k1 + c4;
+#pragma unroll
+        for (int kx = 0; kx < 3; kx++) {
+            const int ix = ix0 + kx, ixc = min(max(ix, 0), a.in_w - 1);
+            const uint32_t v = *reinterpret_cast<const uint32_t *>(rowp + (size_t)ixc * a.k1);
+            buf[ky * 3 + kx] = (iy == iyc && ix == ixc) ? v : zx4;
+        }
+    }
+}
+
+// The depthwise convolution's 16 pixels x k1 channels, requantised, into the LDS tile as s8.  A thread keeps the
+// weights of four channels and walks the pixels pg, pg + pgs, ...: the next pixel's window is requested before this
+// one is multiplied.
+__device__ __forceinline__ void dw_stage(const PairArgs &a, uint8_t *xs, int sx, int p0, int tid, int threads) {
+    const int quads = a.k1 >> 2;
+    const bool wide = threads >= quads;            // a thread per channel quad, and pixel groups of them
+    const int pgs = wide ? threads / quads : 1, pg = wide ? tid / quads : 0;
+    if (pg >= pgs) return;
+#pragma unroll 1
+    for (int q = wide ? tid - pg * quads : tid; q < quads; q += wide ? quads : threads) {
+        const int c4 = q * 4;
+        uint32_t cur[9], w01[9], w23[9];
+        dw_fetch(cur, a, p0 + pg, c4);
+#pragma unroll
+        for (int t = 0; t < 9; t++) {
+            const uint2 wv = *reinterpret_cast<const uint2 *>(a.dw_w + (size_t)t * a.k1 + c4);
+            w01[t] = wv.x, w23[t] = wv.y;
+        }
+        const v4i bias = *reinterpret_cast<const v4i *>(a.dw_bias + c4), ws = *reinterpret_cast<const v4i *>(a.dw_wsum + c4);
+        int32_t ct[4];
+#pragma unroll
+        for (int c = 0; c < 4; c++) ct[c] = bias[c] - a.dw_zx * ws[c];
+#pragma unroll 1
+        for (int r = pg; r < 16; r += pgs) {
+            uint32_t nxt[9];
+            if (r + pgs < 16) dw_fetch(nxt, a, p0 + r + pgs, c4);
+            int32_t acc[4] = {ct[0], ct[1], ct[2], ct[3]};
+#pragma unroll
+            for (int t = 0; t < 9; t++) {
+                const uint32_t x01 = __builtin_amdgcn_perm(0, cur[t], 0x0c010c00u), x23 = __builtin_amdgcn_perm(0, cur[t], 0x0c030c02u);
+                acc[0] = mad16_lo(x01, w01[t], acc[0]);
+                acc[1] = mad16_hi(x01, w01[t], acc[1]);
+                acc[2] = mad16_lo(x23, w23[t], acc[2]);
+                acc[3] = mad16_hi(x23, w23[t], acc[3]);
+            }
+            uint32_t code = requant4_u8_packed(acc, a.ep_dw);
+            if (p0 + r >= a.m) code = 0x80808080u; // rows past the tensor read as zero
+            *reinterpret_cast<uint32_t *>(xs + r * sx + c4) = code ^ 0x80808080u;
+#pragma unroll
+            for (int t = 0; t < 9; t++) cur[t] = nxt[t];
+        }
+    }
+}
+
 // KA / KB: weight fragments a wave requests at a time for the first / second convolution (each twice in registers).
 // MAXW: most waves a workgroup is launched with; OCC: waves per SIMD the register budget is held to.
-template <int KA, int KB, int MAXW, int OCC> __global__ __launch_bounds__(MAXW * 64, OCC) void qpointwise_pair_kernel(const PairArgs a) {
+// DW: a 3x3 depthwise convolution produces the pixel tile (dw_stage).
+template <int KA, int KB, int MAXW, int OCC, bool DW>
+__global__ __launch_bounds__(MAXW * 64, OCC) void qpointwise_pair_kernel(const PairArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
     // rows hold whole chunks of k-steps, zero past the real reduction
     const int sx = pair_row_bytes(a.ks1, KA), sy = pair_row_bytes(a.ks2, KB);
@@ -174,12 +250,21 @@ template <int KA, int KB, int MAXW, int OCC> __global__ __launch_bounds__(MAXW *
 
     // x tile as s8 (x - 128); rows past the tensor and bytes past K read as zero
     const int pieces = (sx - kRowPad) / 16; // 16-byte pieces per row
+    if constexpr (DW) {
+        dw_stage(a, xs, sx, p0, tid, threads);
+        const int first = a.k1 / 16, extra = pieces - first;
+        for (int e = tid; e < 16 * extra; e += threads) {
+            const int r = e / extra, c = first + (e - r * extra);
+            *reinterpret_cast<u32x4 *>(xs + r * sx + c * 16) = u32x4{0u, 0u, 0u, 0u};
+        }
+    } else {
 #pragma unroll 1
-    for (int e = tid; e < 16 * pieces; e += threads) {
-        const int r = e / pieces, c = e - r * pieces;
-        u32x4 v = {0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u};
-        if (p0 + r < a.m && c * 16 < a.k1) v = *reinterpret_cast<const u32x4 *>(a.x + (size_t)(p0 + r) * a.k1 + c * 16);
-        *reinterpret_cast<u32x4 *>(xs + r * sx + c * 16) = v ^ 0x80808080u;
+        for (int e = tid; e < 16 * pieces; e += threads) {
+            const int r = e / pieces, c = e - r * pieces;
+            u32x4 v = {0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u};
+            if (p0 + r < a.m && c * 16 < a.k1) v = *reinterpret_cast<const u32x4 *>(a.x + (size_t)(p0 + r) * a.k1 + c * 16);
+            *reinterpret_cast<u32x4 *>(xs + r * sx + c * 16) = v ^ 0x80808080u;
+        }
     }
     for (int e = tid; e < 4 * sy; e += threads) reinterpret_cast<uint32_t *>(ys)[e] = 0; // channels past N1 stay zero
     for (int e = tid; e < 128; e += threads) {
@@ -303,34 +388,38 @@ extern "C" int nncase_hip_qpointwise_pair_destroy(nncase_hip_ctx_t *ctx, nncase_
     return 0;
 }
 
-extern "C" int nncase_hip_qpointwise_pair(nncase_hip_ctx_t *ctx, const uint8_t *x_dev, const nncase_hip_qpair_t *pr, uint8_t *y1_dev,
-                                          uint8_t *y2_dev, const nncase_hip_conv2d_args_t *fa, const nncase_hip_conv2d_args_t *sa) {
-    NNHIP_CHECK_CTX(ctx);
-    NNHIP_REQUIRE(ctx, x_dev && pr && y1_dev && y2_dev && fa && sa, -EINVAL, "qpointwise_pair: null argument");
-    NNHIP_REQUIRE(ctx, fa->batch > 0 && fa->in_h > 0 && fa->in_w > 0, -EINVAL, "qpointwise_pair: non-positive input shape");
+// dw / da: the depthwise convolution in front and its arguments, or null
+static int launch_pair(nncase_hip_ctx *ctx, const char *who, const uint8_t *x_dev, const nncase_hip_weights *dw,
+                       const nncase_hip_conv2d_args_t *da, const nncase_hip_qpair *pr, uint8_t *y1_dev, uint8_t *y2_dev,
+                       const nncase_hip_conv2d_args_t *fa, const nncase_hip_conv2d_args_t *sa) {
+    NNHIP_REQUIRE(ctx, x_dev && pr && y1_dev && y2_dev && fa && sa, -EINVAL, "%s: null argument", who);
+    NNHIP_REQUIRE(ctx, fa->batch > 0 && fa->in_h > 0 && fa->in_w > 0, -EINVAL, "%s: non-positive input shape", who);
     NNHIP_REQUIRE(ctx, sa->batch == fa->batch && sa->in_h == fa->in_h && sa->in_w == fa->in_w, -NNCASE_HIP_ERR_SHAPE_MISMATCH,
-                  "qpointwise_pair: the second convolution reads [%d,%d,%d], the first writes [%d,%d,%d]", sa->batch, sa->in_h, sa->in_w,
-                  fa->batch, fa->in_h, fa->in_w);
+                  "%s: the second convolution reads [%d,%d,%d], the first writes [%d,%d,%d]", who, sa->batch, sa->in_h, sa->in_w, fa->batch,
+                  fa->in_h, fa->in_w);
     for (const nncase_hip_conv2d_args_t *c : {fa, sa}) {
         NNHIP_REQUIRE(ctx, c->stride_h == 1 && c->stride_w == 1 && c->pad_h_before == 0 && c->pad_h_after == 0 && c->pad_w_before == 0 &&
                                c->pad_w_after == 0,
-                      -EINVAL, "qpointwise_pair: stride 1 and no padding only");
-        NNHIP_REQUIRE(ctx, c->out_dtype == NNCASE_HIP_DT_U8 && c->dequantize_output == 0, -NNCASE_HIP_ERR_DATATYPE_MISMATCH,
-                      "qpointwise_pair: u8 results only");
-        NNHIP_REQUIRE(ctx, c->out_channel_stride == 0 && c->out_channel_offset == 0, -EINVAL, "qpointwise_pair: dense results only");
-        NNHIP_REQUIRE(ctx, c->x_qp.zero_point >= 0 && c->x_qp.zero_point <= 255, -EINVAL, "qpointwise_pair: input zero point %d outside u8",
+                      -EINVAL, "%s: stride 1 and no padding only for the 1x1 convolutions", who);
+    }
+    for (const nncase_hip_conv2d_args_t *c : {fa, sa, da}) {
+        if (!c) continue;
+        NNHIP_REQUIRE(ctx, c->out_dtype == NNCASE_HIP_DT_U8 && c->dequantize_output == 0, -NNCASE_HIP_ERR_DATATYPE_MISMATCH, "%s: u8 results only",
+                      who);
+        NNHIP_REQUIRE(ctx, c->out_channel_stride == 0 && c->out_channel_offset == 0, -EINVAL, "%s: dense results only", who);
+        NNHIP_REQUIRE(ctx, c->x_qp.zero_point >= 0 && c->x_qp.zero_point <= 255, -EINVAL, "%s: input zero point %d outside u8", who,
                       c->x_qp.zero_point);
         NNHIP_REQUIRE(ctx, c->y_qp.scale > 0.f && std::isfinite(c->y_qp.scale) && c->y_qp.zero_point >= 0 && c->y_qp.zero_point <= 255, -EINVAL,
-                      "qpointwise_pair: output quantisation outside u8");
+                      "%s: output quantisation outside u8", who);
     }
-    NNHIP_REQUIRE(ctx, !sa->residual_dev, -EINVAL, "qpointwise_pair: only the first convolution takes a residual");
+    NNHIP_REQUIRE(ctx, !sa->residual_dev, -EINVAL, "%s: only the first 1x1 convolution takes a residual", who);
     if (fa->residual_dev)
         NNHIP_REQUIRE(ctx, fa->sum_qp.scale > 0.f && std::isfinite(fa->sum_qp.scale) && fa->sum_qp.zero_point >= 0 && fa->sum_qp.zero_point <= 255,
-                      -EINVAL, "qpointwise_pair: sum quantisation outside u8");
+                      -EINVAL, "%s: sum quantisation outside u8", who);
     const int64_t m64 = (int64_t)fa->batch * fa->in_h * fa->in_w;
-    NNHIP_REQUIRE(ctx, m64 < ((int64_t)1 << 30), -EINVAL, "qpointwise_pair: %lld pixels unsupported", (long long)m64);
+    NNHIP_REQUIRE(ctx, m64 < ((int64_t)1 << 30), -EINVAL, "%s: %lld pixels unsupported", who, (long long)m64);
     NNHIP_REQUIRE(ctx, ((reinterpret_cast<uintptr_t>(x_dev) | reinterpret_cast<uintptr_t>(y1_dev) | reinterpret_cast<uintptr_t>(y2_dev)) & 15u) == 0,
-                  -NNCASE_HIP_ERR_INVALID_MEMORY_LOCATION, "qpointwise_pair: activation buffers must be 16-byte aligned");
+                  -NNCASE_HIP_ERR_INVALID_MEMORY_LOCATION, "%s: activation buffers must be 16-byte aligned", who);
 
     PairArgs a;
     memset(&a, 0, sizeof(a));
@@ -343,13 +432,40 @@ extern "C" int nncase_hip_qpointwise_pair(nncase_hip_ctx_t *ctx, const uint8_t *
     a.ks1 = pr->ks1, a.ks2 = pr->ks2, a.t1 = pr->t1, a.t2 = pr->t2;
     a.zxa = fa->x_qp.zero_point - 128, a.zwa = pr->first->zw - 128;
     a.zxb = sa->x_qp.zero_point - 128, a.zwb = pr->second->zw - 128;
-    int rc = make_epilogue(ctx, &a.ep_a, fa->x_qp.scale, pr->first->sw, fa->y_qp, fa->clamp_min, fa->clamp_max, NNCASE_HIP_DT_U8, "qpointwise_pair");
-    if (!rc) rc = make_epilogue(ctx, &a.ep_b, sa->x_qp.scale, pr->second->sw, sa->y_qp, sa->clamp_min, sa->clamp_max, NNCASE_HIP_DT_U8, "qpointwise_pair");
+    int rc = make_epilogue(ctx, &a.ep_a, fa->x_qp.scale, pr->first->sw, fa->y_qp, fa->clamp_min, fa->clamp_max, NNCASE_HIP_DT_U8, who);
+    if (!rc) rc = make_epilogue(ctx, &a.ep_b, sa->x_qp.scale, pr->second->sw, sa->y_qp, sa->clamp_min, sa->clamp_max, NNCASE_HIP_DT_U8, who);
     if (!rc) rc = make_residual_epilogue(ctx, &a.rep_a, fa, pr->first);
     if (rc) return rc;
+    if (dw) {
+        NNHIP_REQUIRE(ctx, da, -EINVAL, "%s: null argument", who);
+        NNHIP_REQUIRE(ctx, dw->kind == nncase_hip_weights::kDepthwise && dw->kernel_h == 3 && dw->kernel_w == 3 && dw->out_channels == pr->k1, -EINVAL,
+                      "%s: the convolution in front must be a 3x3 depthwise convolution over the first 1x1 convolution's %d channels", who, pr->k1);
+        NNHIP_REQUIRE(ctx, !dw->d_post_lut && !da->residual_dev, -EINVAL, "%s: the depthwise convolution takes no table or residual", who);
+        NNHIP_REQUIRE(ctx, da->stride_h == da->stride_w && (da->stride_h == 1 || da->stride_h == 2) && da->dilation_h == 1 && da->dilation_w == 1,
+                      -EINVAL, "%s: depthwise stride 1 or 2, no dilation", who);
+        NNHIP_REQUIRE(ctx, da->pad_h_before >= 0 && da->pad_h_after >= 0 && da->pad_w_before >= 0 && da->pad_w_after >= 0, -EINVAL,
+                      "%s: negative padding", who);
+        NNHIP_REQUIRE(ctx, da->in_h > 0 && da->in_w > 0, -EINVAL, "%s: non-positive input shape", who);
+        const int out_h = windowed_output_size(da->in_h, 3, da->stride_h, 1, da->pad_h_before, da->pad_h_after);
+        const int out_w = windowed_output_size(da->in_w, 3, da->stride_w, 1, da->pad_w_before, da->pad_w_after);
+        NNHIP_REQUIRE(ctx, da->batch == fa->batch && out_h == fa->in_h && out_w == fa->in_w, -NNCASE_HIP_ERR_SHAPE_MISMATCH,
+                      "%s: the depthwise convolution writes [%d,%d,%d], the first 1x1 convolution reads [%d,%d,%d]", who, da->batch, out_h, out_w,
+                      fa->batch, fa->in_h, fa->in_w);
+        NNHIP_REQUIRE(ctx, da->y_qp.zero_point == fa->x_qp.zero_point && da->y_qp.scale == fa->x_qp.scale, -EINVAL,
+                      "%s: the first 1x1 convolution must read the depthwise result with the quantisation it is written with", who);
+        NNHIP_REQUIRE(ctx, (int64_t)da->batch * da->in_h * da->in_w * pr->k1 < ((int64_t)1 << 31), -EINVAL, "%s: input of 2 GiB or more", who);
+        a.dw_w = reinterpret_cast<const int16_t *>(dw->d_packed), a.dw_bias = dw->d_bias, a.dw_wsum = dw->d_wsum;
+        a.in_h = da->in_h, a.in_w = da->in_w, a.out_w = out_w, a.out_hw = out_h * out_w;
+        a.stride = da->stride_h, a.pad_h = da->pad_h_before, a.pad_w = da->pad_w_before;
+        a.d_out_hw = make_fastdiv((uint32_t)a.out_hw), a.d_out_w = make_fastdiv((uint32_t)out_w);
+        a.dw_zx = da->x_qp.zero_point;
+        rc = make_epilogue(ctx, &a.ep_dw, da->x_qp.scale, dw->sw, da->y_qp, da->clamp_min, da->clamp_max, NNCASE_HIP_DT_U8, who);
+        if (rc) return rc;
+    }
 
     // A wave per channel tile of whichever convolution has more of them in this workgroup (up to the variant's most),
-    // and enough workgroups to occupy the device: pixel tiles x ranges of the second convolution's channel tiles.
+    // and enough workgroups to occupy the device: pixel tiles x ranges of the second convolution's channel tiles.  With
+    // a depthwise stage, also enough threads that none of them walks more than four of the 16 pixels.
     const bool small = pair_is_small(a.ks1, a.ks2);
     const int max_waves = small ? 16 : 12;
     const int ptiles = (a.m + 15) / 16;
@@ -358,12 +474,35 @@ extern "C" int nncase_hip_qpointwise_pair(nncase_hip_ctx_t *ctx, const uint8_t *
     if (ranges > want) ranges = want;
     a.tiles_per_block = (a.t2 + ranges - 1) / ranges;
     ranges = (a.t2 + a.tiles_per_block - 1) / a.tiles_per_block;
-    const int waves = std::min(max_waves, std::max(a.t1, a.tiles_per_block));
+    int waves = std::min(max_waves, std::max(a.t1, a.tiles_per_block));
+    if (dw) waves = std::min(max_waves, std::max(waves, (a.k1 + 63) / 64));
     NNHIP_HIP(ctx, hipSetDevice(ctx->device));
-    if (small)
-        hipLaunchKernelGGL((qpointwise_pair_kernel<4, 2, 16, 5>), dim3(ptiles, ranges), dim3(waves * 64), pair_lds_bytes(pr), ctx->stream, a);
+    const dim3 grid(ptiles, ranges), block(waves * 64);
+    const size_t lds = pair_lds_bytes(pr);
+    if (small && dw)
+        hipLaunchKernelGGL((qpointwise_pair_kernel<4, 2, 16, 4, true>), grid, block, lds, ctx->stream, a);
+    else if (small)
+        hipLaunchKernelGGL((qpointwise_pair_kernel<4, 2, 16, 5, false>), grid, block, lds, ctx->stream, a);
+    else if (dw)
+        hipLaunchKernelGGL((qpointwise_pair_kernel<8, 4, 12, 3, true>), grid, block, lds, ctx->stream, a);
     else
-        hipLaunchKernelGGL((qpointwise_pair_kernel<8, 4, 12, 3>), dim3(ptiles, ranges), dim3(waves * 64), pair_lds_bytes(pr), ctx->stream, a);
+        hipLaunchKernelGGL((qpointwise_pair_kernel<8, 4, 12, 3, false>), grid, block, lds, ctx->stream, a);
     NNHIP_LAUNCH_CHECK(ctx, "qpointwise_pair_kernel");
     return 0;
+}
+
+extern "C" int nncase_hip_qpointwise_pair(nncase_hip_ctx_t *ctx, const uint8_t *x_dev, const nncase_hip_qpair_t *pair, uint8_t *y1_dev,
+                                          uint8_t *y2_dev, const nncase_hip_conv2d_args_t *first_args,
+                                          const nncase_hip_conv2d_args_t *second_args) {
+    NNHIP_CHECK_CTX(ctx);
+    return launch_pair(ctx, "qpointwise_pair", x_dev, nullptr, nullptr, pair, y1_dev, y2_dev, first_args, second_args);
+}
+
+extern "C" int nncase_hip_qdepthwise_pointwise_pair(nncase_hip_ctx_t *ctx, const uint8_t *x_dev, const nncase_hip_weights_t *depthwise,
+                                                    const nncase_hip_conv2d_args_t *depthwise_args, const nncase_hip_qpair_t *pair,
+                                                    uint8_t *y1_dev, uint8_t *y2_dev, const nncase_hip_conv2d_args_t *first_args,
+                                                    const nncase_hip_conv2d_args_t *second_args) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, depthwise && depthwise_args, -EINVAL, "qdepthwise_pointwise_pair: null argument");
+    return launch_pair(ctx, "qdepthwise_pointwise_pair", x_dev, depthwise, depthwise_args, pair, y1_dev, y2_dev, first_args, second_args);
 }

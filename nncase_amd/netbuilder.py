@@ -402,6 +402,9 @@ def pad_small_channel_convs(qg: QuantGraph) -> QuantGraph:
 # batches 1 and 2 (0.215 -> 0.184 ms per image at batch 1); beyond them the separate kernels win.
 PAIR_STREAM_LIMIT = 4 << 20
 PAIR_MAX_PIXEL_TILES = 512
+# A depthwise convolution in front joins the pair while it has few channels: a workgroup computes its 16 pixels of it
+# alone, about 50 ns per 16 channels, against the 3.5 us of the separate launch it saves.
+PAIR_FRONT_MAX_CHANNELS = 256
 
 
 class HipModel:
@@ -568,6 +571,7 @@ class HipModel:
         # expansion at small batches.  Every workgroup of the pair repeats the first convolution for its 16 pixels, so
         # the weights it streams (pixel tiles x both weight tensors) bound where that still pays.
         self.pairs: Dict[int, int] = {}                                                  # first conv -> second conv
+        self.pair_fronts: Dict[int, int] = {}                                            # first conv -> depthwise conv in front
         if fuse_pairs and fuse_residual:
             def pointwise1(j):
                 n = qg.nodes[j]
@@ -593,6 +597,17 @@ class HipModel:
                 self.pairs[i] = j
                 taken |= {i, j}
                 skip_nodes.add(j)
+                # ... and a 3x3 depthwise convolution that only the first of the two reads is computed by the same launch,
+                # 16 pixels per workgroup straight into LDS
+                d = n.inputs[0]
+                dn = qg.nodes[d]
+                if (fuse_pairs != "nofront" and (fuse_pairs == "all" or k1 <= PAIR_FRONT_MAX_CHANNELS)
+                        and dn.op == "conv" and dn.groups == dn.weights.shape[0] and dn.weights.shape[1:] == (1, 3, 3)
+                        and tuple(dn.stride) in ((1, 1), (2, 2)) and consumers[d] == 1 and d not in qg.output_nodes
+                        and d not in block_members and d not in self.fused_lut and d not in self.fused_into):
+                    self.pair_fronts[i] = d
+                    self.never_written.add(d)
+                    skip_nodes.add(d)
         self.pair_objects: Dict[int, rt.QPair] = {}
         # buffers and packed weights once, shared by the lanes
         for i, n in enumerate(qg.nodes):
@@ -604,7 +619,8 @@ class HipModel:
             if n.op == "fold2":
                 self.buffers.append(self.buffers[n.inputs[0]])  # the same bytes read as half as many, twice as deep pixels
                 continue
-            if i in self.blocks or i - 1 in self.blocks or i in self.write_through or i in self.fused_quant.values() or i in self.fused_dequant:
+            if (i in self.blocks or i - 1 in self.blocks or i in self.write_through or i in self.fused_quant.values() or i in self.fused_dequant
+                    or i in self.pair_fronts.values()):
                 self.buffers.append(ctx.alloc(16))        # expanded tensors of a fused block live in LDS only; a conv
                 #                                           that writes into its concat has no tensor of its own
             else:
@@ -708,10 +724,20 @@ class HipModel:
                     second = rt.Conv2dArgs(bl, mid.out_shape[1], mid.out_shape[2], 1, 1, 1, 1, 0, 0, 0, 0, qp(*mid.out_qp), qp(*sn.out_qp),
                                            sn.clamp[0], sn.clamp[1], rt.DT_U8)
                     lut2 = self.fused_lut.get(j)
-                    self.fn.add_qpointwise_pair(B(n.inputs[0]), self.pair_objects[i], B(sn_in), B(lut2 if lut2 is not None else j), args, second)
+                    d = self.pair_fronts.get(i)
+                    if d is not None:
+                        dn, dsrc = qg.nodes[d], qg.nodes[qg.nodes[d].inputs[0]]
+                        (dh0, dh1), (dw0, dw1) = dn.padding
+                        front = rt.Conv2dArgs(bl, dsrc.out_shape[1], dsrc.out_shape[2], dn.stride[0], dn.stride[1], 1, 1, dh0, dh1, dw0, dw1,
+                                              qp(*dsrc.out_qp), qp(*dn.out_qp), dn.clamp[0], dn.clamp[1], rt.DT_U8)
+                        self.fn.add_qdepthwise_pointwise_pair(B(dn.inputs[0]), self.weights[d], front, self.pair_objects[i], B(sn_in),
+                                                              B(lut2 if lut2 is not None else j), args, second)
+                        members = [d] + members
+                    else:
+                        self.fn.add_qpointwise_pair(B(n.inputs[0]), self.pair_objects[i], B(sn_in), B(lut2 if lut2 is not None else j), args, second)
                     if lane == 0:
-                        self.op_names.append(f"pair:{n.name}" + ("+lut" if fused_lut is not None else "") + ("+add" if fused_add is not None else "")
-                                             + f">{sn.name}" + ("+lut" if lut2 is not None else ""))
+                        self.op_names.append(("pair:" if d is None else f"pair:{qg.nodes[d].name}>") + n.name + ("+lut" if fused_lut is not None else "")
+                                             + ("+add" if fused_add is not None else "") + f">{sn.name}" + ("+lut" if lut2 is not None else ""))
                         self.op_nodes.append(lut2 if lut2 is not None else j)
                         self.op_members.append(members + [j] + ([lut2] if lut2 is not None else []))
                     continue

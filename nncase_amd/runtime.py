@@ -121,6 +121,9 @@ SYMBOLS = {
     "nncase_hip_qpointwise_pair_destroy": (_I, [_VP, _VP]),
     "nncase_hip_qpointwise_pair": (_I, [_VP, _VP, _VP, _VP, _VP, C.POINTER(Conv2dArgs), C.POINTER(Conv2dArgs)]),
     "nncase_hip_function_add_qpointwise_pair": (_I, [_VP, _VP, _VP, _VP, _VP, C.POINTER(Conv2dArgs), C.POINTER(Conv2dArgs)]),
+    "nncase_hip_qdepthwise_pointwise_pair": (_I, [_VP, _VP, _VP, C.POINTER(Conv2dArgs), _VP, _VP, _VP, C.POINTER(Conv2dArgs), C.POINTER(Conv2dArgs)]),
+    "nncase_hip_function_add_qdepthwise_pointwise_pair": (_I, [_VP, _VP, _VP, C.POINTER(Conv2dArgs), _VP, _VP, _VP, C.POINTER(Conv2dArgs),
+                                                           C.POINTER(Conv2dArgs)]),
     "nncase_hip_qmatmul_prepack": (_I, [_VP, _VP, C.c_int32, C.c_int32, QuantParam, _VP, C.c_int64, C.POINTER(_VP)]),
     "nncase_hip_qmatmul": (_I, [_VP, _VP, _VP, _VP, C.POINTER(MatmulArgs)]),
     "nncase_hip_qadd": (_I, [_VP, _VP, QuantParam, _VP, QuantParam, _VP, QuantParam, C.c_float, C.c_float, _SZ]),
@@ -564,6 +567,12 @@ class Context:
         self._check(self.lib.nncase_hip_qpointwise_pair(self.handle, x.ptr, pair.handle, y1.ptr, y2.ptr, C.byref(first_args),
                                                         C.byref(second_args)), "qpointwise_pair")
 
+    def qdepthwise_pointwise_pair(self, x, dw: Weights, dw_args: Conv2dArgs, pair: QPair, y1, y2, first_args: Conv2dArgs,
+                                  second_args: Conv2dArgs):
+        """x is the 3x3 depthwise convolution's input; its result only exists inside the launch."""
+        self._check(self.lib.nncase_hip_qdepthwise_pointwise_pair(self.handle, x.ptr, dw.handle, C.byref(dw_args), pair.handle, y1.ptr, y2.ptr,
+                                                                  C.byref(first_args), C.byref(second_args)), "qdepthwise_pointwise_pair")
+
     def prepack_matmul(self, b_kn: np.ndarray, bias: Optional[np.ndarray], b_qp: QuantParam, expected_rows: int = 0) -> Weights:
         b = np.ascontiguousarray(b_kn, np.uint8)
         k, n = b.shape
@@ -719,6 +728,13 @@ class Function:
         self._keep += [x, pair, y1, y2]
         self._ck(self.ctx.lib.nncase_hip_function_add_qpointwise_pair(self.handle, x.ptr, pair.handle, y1.ptr, y2.ptr, C.byref(first_args),
                                                                       C.byref(second_args)), "function_add_qpointwise_pair")
+
+    def add_qdepthwise_pointwise_pair(self, x, dw: Weights, dw_args: Conv2dArgs, pair: QPair, y1, y2, first_args: Conv2dArgs,
+                                      second_args: Conv2dArgs):
+        self._keep += [x, dw, pair, y1, y2]
+        self._ck(self.ctx.lib.nncase_hip_function_add_qdepthwise_pointwise_pair(self.handle, x.ptr, dw.handle, C.byref(dw_args), pair.handle,
+                                                                                y1.ptr, y2.ptr, C.byref(first_args), C.byref(second_args)),
+                 "function_add_qdepthwise_pointwise_pair")
 
     def add_qadd(self, a, a_qp, b, b_qp, out, y_qp, count, clamp=(-FLT_MAX, FLT_MAX)):
         self._keep += [a, b, out]

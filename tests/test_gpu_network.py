@@ -76,7 +76,10 @@ def test_mobilenetv2_config3(hip_ctx):
     assert len(model.fused_into) == 10 and len(model.fused_dequant) == 1 and len(model.fn) == 55   # residual adds folded into
     #                                                                            the convs, the output's dequantize into the classifier
     model, y, outs = check_model(hip_ctx, qg, x, capture=True, fuse_blocks=False, fuse_pairs="all")
-    assert len(model.pairs) == 17 and len(model.fn) == 38     # every projection runs with the expansion behind it as one launch
+    assert len(model.pairs) == 17 and len(model.pair_fronts) == 17 and len(model.fn) == 21   # every depthwise convolution and projection runs
+    #                                                                                          with the expansion behind them as one launch
+    model, y, outs = check_model(hip_ctx, qg, x, capture=True, fuse_blocks=False, fuse_pairs="nofront")
+    assert 0 < len(model.pairs) < 17 and not model.pair_fronts
     model, y, outs = check_model(hip_ctx, qg, x, capture=True, fuse_blocks=False)
     assert 0 < len(model.pairs) < 17                           # ... at this batch, where the pair streams few weights
     model, y, outs = check_model(hip_ctx, qg, x, capture=True)

@@ -1,6 +1,6 @@
-"""GPU parity of the pointwise pair (1x1 convolution [+ byte table] [+ residual] -> 1x1 convolution [+ byte table] as one
-launch) through the C ABI: both results must be bit-identical to the CPU oracle running the operators one after the
-other, and to nncase_hip_qconv2d called twice on the device."""
+"""GPU parity of the pointwise pair ([3x3 depthwise convolution ->] 1x1 convolution [+ byte table] [+ residual] -> 1x1
+convolution [+ byte table] as one launch) through the C ABI: both results must be bit-identical to the CPU oracle
+running the operators one after the other, and to nncase_hip_qconv2d called once per convolution on the device."""
 import numpy as np
 import pytest
 
@@ -18,14 +18,32 @@ def conv_args(n, h, w, x_qp, y_qp, clamp):
     return rt.Conv2dArgs(n, h, w, 1, 1, 1, 1, 0, 0, 0, 0, x_qp, y_qp, clamp[0], clamp[1], rt.DT_U8)
 
 
-def run_pair(ctx, n, k1, n1, n2, h, w, seed, residual=False, lut_a=False, lut_b=False, relu_b=True):
+def run_pair(ctx, n, k1, n1, n2, h, w, seed, residual=False, lut_a=False, lut_b=False, relu_b=True, dw=None):
+    """dw = (stride, padding): h x w is then the input of a 3x3 depthwise convolution in front of the pair."""
     rng = np.random.default_rng(seed)
     x = rng.integers(0, 256, (n, k1, h, w), dtype=np.uint8)
+    front = None
+    if dw is not None:
+        stride, pad = dw
+        x0, (z0, s0) = x, (11, f32(0.019))
+        wd = rng.integers(0, 256, (k1, 1, 3, 3), dtype=np.uint8)
+        bd = rng.integers(-3000, 3000, k1).astype(np.int32)
+        zwd, swd = 119, f32(0.0123)
+        dwk = dict(stride=(stride, stride), padding=pad, dilation=(1, 1), groups=k1)
+        real = O.qconv2d(x0, wd, bd, z0, s0, zwd, swd, out_mode=O.OUT_F32, **dwk)
+        cd, zd, sd = pick_quant(real)
+        x = O.qconv2d(x0, wd, bd, z0, s0, zwd, swd, zd, sd, fused_clamp=cd, out_mode=O.OUT_U8, **dwk)
+        in_h, in_w = h, w
+        h, w = x.shape[2:]
+        dww = ctx.prepack_conv2d(wd, bd, qp(zwd, swd), groups=k1)
+        (ph0, ph1), (pw0, pw1) = pad
+        da_ = rt.Conv2dArgs(n, in_h, in_w, stride, stride, 1, 1, ph0, ph1, pw0, pw1, qp(z0, s0), qp(zd, sd), cd[0], cd[1], rt.DT_U8)
+        front = (x0, dww, da_)
     wa = rng.integers(0, 256, (n1, k1, 1, 1), dtype=np.uint8)
     wb = rng.integers(0, 256, (n2, n1, 1, 1), dtype=np.uint8)
     ba = rng.integers(-3000, 3000, n1).astype(np.int32)
     bb = rng.integers(-3000, 3000, n2).astype(np.int32)
-    zx, sx = 9, f32(0.0235)
+    zx, sx = (9, f32(0.0235)) if front is None else (zd, sd)
     (zwa, swa), (zwb, swb) = (131, f32(0.0041)), (122, f32(0.0037))
     # the oracle, operator by operator
     real = O.qconv2d(x, wa, ba, zx, sx, zwa, swa, out_mode=O.OUT_F32)
@@ -65,6 +83,9 @@ def run_pair(ctx, n, k1, n1, n2, h, w, seed, residual=False, lut_a=False, lut_b=
     sa_ = conv_args(n, h, w, qp(z_mid, s_mid), qp(z2, s2), c2)
     xd = ctx.alloc(x.size).upload(np.ascontiguousarray(x.transpose(0, 2, 3, 1)))
     keep = [xd]
+    if front is not None:
+        x0d = ctx.alloc(front[0].size).upload(np.ascontiguousarray(front[0].transpose(0, 2, 3, 1)))
+        keep.append(x0d)
     if residual:
         rd = ctx.alloc(res.size).upload(np.ascontiguousarray(res.transpose(0, 2, 3, 1)))
         keep.append(rd)
@@ -74,7 +95,10 @@ def run_pair(ctx, n, k1, n1, n2, h, w, seed, residual=False, lut_a=False, lut_b=
         fa_.sum_clamp_min, fa_.sum_clamp_max = FULL
     y1d = ctx.alloc(n * h * w * n1).fill(0xA5)
     y2d = ctx.alloc(n * h * w * n2).fill(0xA5)
-    ctx.qpointwise_pair(xd, pair, y1d, y2d, fa_, sa_)
+    if front is None:
+        ctx.qpointwise_pair(xd, pair, y1d, y2d, fa_, sa_)
+    else:
+        ctx.qdepthwise_pointwise_pair(x0d, front[1], front[2], pair, y1d, y2d, fa_, sa_)
     ctx.sync()
     got1 = y1d.download((n, h, w, n1), np.uint8).transpose(0, 3, 1, 2)
     got2 = y2d.download((n, h, w, n2), np.uint8).transpose(0, 3, 1, 2)
@@ -85,12 +109,14 @@ def run_pair(ctx, n, k1, n1, n2, h, w, seed, residual=False, lut_a=False, lut_b=
     # the two stand-alone operators on the device
     u1 = ctx.alloc(n * h * w * n1).fill(0x5A)
     u2 = ctx.alloc(n * h * w * n2).fill(0x5A)
+    if front is not None:
+        ctx.qconv2d(x0d, front[1], xd.fill(0x5A), front[2])
     ctx.qconv2d(xd, first, u1, fa_)
     ctx.qconv2d(u1, second, u2, sa_)
     ctx.sync()
     assert np.array_equal(u1.download((n, h, w, n1), np.uint8), y1d.download((n, h, w, n1), np.uint8))
     assert np.array_equal(u2.download((n, h, w, n2), np.uint8), y2d.download((n, h, w, n2), np.uint8))
-    return pair, (xd, y1d, y2d, fa_, sa_, keep)
+    return pair, (xd if front is None else x0d, y1d, y2d, fa_, sa_, keep + ([front] if front is not None else []))
 
 
 MOBILENET_PAIRS = [  # (in, mid, out, h, w, residual): every projection -> expansion pair of MobileNetV2 1.0 at batch 1
@@ -116,6 +142,58 @@ RAGGED = [  # (n, in, mid, out, h, w, residual, lut_a, lut_b, relu_b): pixel cou
 @pytest.mark.parametrize("n,k1,n1,n2,h,w,residual,lut_a,lut_b,relu_b", RAGGED)
 def test_ragged_pairs(hip_ctx, n, k1, n1, n2, h, w, residual, lut_a, lut_b, relu_b):
     run_pair(hip_ctx, n, k1, n1, n2, h, w, seed=n + k1 + n1 + n2 + h * w, residual=residual, lut_a=lut_a, lut_b=lut_b, relu_b=relu_b)
+
+
+P1 = ((1, 1), (1, 1))
+MOBILENET_TRIPLES = [  # (channels, mid, out, in_h, in_w, depthwise stride, residual): MobileNetV2's depthwise -> projection -> expansion
+    (96, 24, 144, 28, 30, 2, False), (144, 24, 144, 14, 15, 1, True), (144, 32, 192, 56, 56, 2, False), (192, 32, 192, 28, 28, 1, True),
+    (192, 64, 384, 28, 28, 2, False), (384, 64, 384, 14, 14, 1, True), (384, 96, 576, 14, 14, 1, False), (576, 96, 576, 14, 14, 1, True),
+    (576, 160, 960, 14, 14, 2, False), (960, 160, 960, 7, 7, 1, True), (960, 320, 1280, 7, 7, 1, False),
+]
+
+
+@pytest.mark.parametrize("k1,n1,n2,h,w,stride,residual", MOBILENET_TRIPLES)
+def test_mobilenet_depthwise_pair_shapes(hip_ctx, k1, n1, n2, h, w, stride, residual):
+    pad = P1 if stride == 1 else ((0, 1), (0, 1))
+    run_pair(hip_ctx, 1, k1, n1, n2, h, w, seed=k1 * 3 + n1 + n2 + stride, residual=residual, dw=(stride, pad))
+
+
+RAGGED_TRIPLES = [  # (n, channels, mid, out, in_h, in_w, stride, padding, residual, lut_a): windows cut by every edge, images that end inside a pixel tile
+    (3, 16, 8, 20, 5, 5, 1, P1, True, False), (2, 48, 20, 36, 9, 7, 2, P1, False, True), (1, 32, 12, 64, 3, 3, 1, ((0, 0), (0, 0)), False, False),
+    (2, 80, 16, 48, 6, 11, 2, ((0, 1), (1, 0)), True, False), (5, 1024, 24, 32, 3, 4, 1, P1, False, False), (1, 64, 4, 4, 1, 1, 1, P1, False, False),
+]
+
+
+@pytest.mark.parametrize("n,k1,n1,n2,h,w,stride,pad,residual,lut_a", RAGGED_TRIPLES)
+def test_ragged_depthwise_pairs(hip_ctx, n, k1, n1, n2, h, w, stride, pad, residual, lut_a):
+    run_pair(hip_ctx, n, k1, n1, n2, h, w, seed=n * 5 + k1 + n1 + n2 + h * w, residual=residual, lut_a=lut_a, dw=(stride, pad))
+
+
+def test_depthwise_pair_in_a_function_repeats(hip_ctx):
+    pair, (x0d, y1d, y2d, fa_, sa_, keep) = run_pair(hip_ctx, 2, 96, 24, 144, 14, 14, seed=4, dw=(1, P1))
+    _, dww, da_ = keep[-1]
+    want1, want2 = y1d.download((y1d.nbytes,), np.uint8), y2d.download((y2d.nbytes,), np.uint8)
+    fn = rt.Function(hip_ctx)
+    fn.add_qdepthwise_pointwise_pair(x0d, dww, da_, pair, y1d, y2d, fa_, sa_)
+    assert fn.op_kernel(0) == "dw3x3+qpointwise_pair_kernel"
+    fn.capture()
+    for _ in range(2):
+        y1d.fill(0x33)
+        y2d.fill(0x33)
+        fn.invoke()
+        hip_ctx.sync()
+        assert np.array_equal(y1d.download((y1d.nbytes,), np.uint8), want1)
+        assert np.array_equal(y2d.download((y2d.nbytes,), np.uint8), want2)
+    # argument checks of the depthwise front
+    other = rt.Conv2dArgs(2, 14, 14, 1, 1, 1, 1, 0, 0, 0, 0, da_.x_qp, da_.y_qp, da_.clamp_min, da_.clamp_max, rt.DT_U8)   # 12 x 12 result
+    with pytest.raises(rt.HipError):
+        hip_ctx.qdepthwise_pointwise_pair(x0d, dww, other, pair, y1d, y2d, fa_, sa_)
+    other = rt.Conv2dArgs(2, 14, 14, 1, 1, 1, 1, 1, 1, 1, 1, da_.x_qp, qp(da_.y_qp.zero_point + 1, da_.y_qp.scale), da_.clamp_min, da_.clamp_max,
+                          rt.DT_U8)
+    with pytest.raises(rt.HipError):
+        hip_ctx.qdepthwise_pointwise_pair(x0d, dww, other, pair, y1d, y2d, fa_, sa_)
+    with pytest.raises(rt.HipError):
+        hip_ctx.qdepthwise_pointwise_pair(x0d, pair.first, da_, pair, y1d, y2d, fa_, sa_)     # not a depthwise convolution
 
 
 def test_pair_in_a_function_repeats(hip_ctx):
