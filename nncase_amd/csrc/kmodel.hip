@@ -94,6 +94,7 @@ struct nncase_hip_kmodel {
     std::vector<char> owns;           // whether buffers[i] is freed with the model
     std::vector<nncase_hip_weights_t *> weights;
     std::vector<nncase_hip_qblock_t *> blocks;
+    std::vector<nncase_hip_qpair_t *> pairs; // (point at entries of `weights`: destroyed first)
     nncase_hip_function_t *fn = nullptr;
     uint32_t input_tensor = 0, output_tensor = 0, n_outputs = 1; // outputs are consecutive tensors
 };
@@ -103,6 +104,8 @@ using namespace nnhip;
 extern "C" int nncase_hip_kmodel_destroy(nncase_hip_kmodel_t *m) {
     if (!m) return -EINVAL;
     if (m->fn) (void)nncase_hip_function_destroy(m->fn); // synchronises the stream first
+    for (auto *pr : m->pairs)
+        if (pr) (void)nncase_hip_qpointwise_pair_destroy(m->ctx, pr);
     for (auto *w : m->weights)
         if (w) (void)nncase_hip_weights_destroy(m->ctx, w);
     for (auto *b : m->blocks)
@@ -519,6 +522,45 @@ static int build_function(nncase_hip_ctx_t *ctx, Span text_span, Span rdata, nnc
         skipped[q] = 1;
     }
 
+    // A dense 1x1 convolution (behind its folded table / add) that a second dense 1x1 convolution reads runs with it as
+    // one launch where the two are latency-bound (see nncase_hip_qpointwise_pair): while the weight bytes the pair's
+    // workgroups stream between them and their number stay small.  A 3x3 depthwise convolution that only the first of
+    // them reads joins the launch while it has few channels.
+    std::vector<int> pair_second(th.n_ops, -1), pair_front(th.n_ops, -1);
+    {
+        constexpr uint64_t kStreamLimit = 4u << 20, kMaxPixelTiles = 512;
+        constexpr int kFrontMaxChannels = 256;
+        auto plain_pointwise = [&](uint32_t k) {
+            return pointwise(ops[k]) && !skipped[k] && !block_head[k] && through[k].concat < 0 && fused_deq[k] < 0 &&
+                   m->tensors[ops[k].output].dtype == NNCASE_HIP_DT_U8 && m->tensors[ops[k].inputs[0]].dtype == NNCASE_HIP_DT_U8;
+        };
+        for (uint32_t k = 0; k < th.n_ops; k++) {
+            if (!plain_pointwise(k)) continue;
+            const int tail = fused_add[k] >= 0 ? fused_add[k] : fused_lut[k] >= 0 ? fused_lut[k] : (int)k;
+            const int32_t mid = ops[tail].output;
+            int j = -1;
+            for (uint32_t q = (uint32_t)tail + 1; q < th.n_ops && j < 0; q++)
+                if (plain_pointwise(q) && ops[q].inputs[0] == mid && fused_add[q] < 0) j = (int)q;
+            if (j < 0) continue;
+            const int k1 = ops[k].p[1], n1 = ops[k].p[0], n2 = ops[j].p[0];
+            if (ops[j].p[1] != n1 || !nncase_hip_qpointwise_pair_supported(k1, n1, n2)) continue;
+            const hipf_tensor &tm = m->tensors[mid];
+            const uint64_t ptiles = ((uint64_t)tm.dims[0] * tm.dims[1] * tm.dims[2] + 15) / 16;
+            if (ptiles > kMaxPixelTiles || ptiles * ((uint64_t)k1 * n1 + (uint64_t)n1 * n2) > kStreamLimit) continue;
+            pair_second[k] = j;
+            skipped[j] = 1;
+            const int32_t x = ops[k].inputs[0];
+            const int d = producer[x];
+            if (d < 0 || skipped[d] || k1 > kFrontMaxChannels) continue;
+            const hipf_op &dc = ops[d];
+            const bool dw3 = dc.opcode == kOpConv2d && dc.n_inputs == 1 && dc.p[1] == 1 && dc.p[4] == dc.p[0] && dc.p[0] == k1 && dc.p[2] == 3 &&
+                             dc.p[3] == 3 && dc.p[5] == dc.p[6] && (dc.p[5] == 1 || dc.p[5] == 2) && dc.p[7] == 1 && dc.p[8] == 1;
+            if (!dw3 || consumers[x] != 1 || is_output(x) || m->tensors[x].dtype != NNCASE_HIP_DT_U8) continue;
+            pair_front[k] = d;
+            skipped[d] = 1;
+        }
+    }
+
     // ---- device buffers ---------------------------------------------------------------------------
     m->buffers.assign(th.n_tensors, nullptr);
     m->owns.assign(th.n_tensors, 0);
@@ -526,6 +568,7 @@ static int build_function(nncase_hip_ctx_t *ctx, Span text_span, Span rdata, nnc
         if (fused_add[k] >= 0 || fused_lut[k] >= 0) m->owns[ops[k].output] = 2;
         if (fused_add[k] >= 0 && fused_lut[k] >= 0) m->owns[ops[fused_lut[k]].output] = 2;
         if (block_head[k]) m->owns[ops[k].output] = m->owns[ops[k + 1].output] = 2;
+        if (pair_front[k] >= 0) m->owns[ops[pair_front[k]].output] = 2; // computed inside the pair's launch
         if (fused_quant[k] >= 0) m->owns[ops[fused_quant[k]].output] = 2;
         if (fused_deq[k] >= 0) { // the u8 result is never stored
             m->owns[ops[k].output] = 2;
@@ -551,6 +594,87 @@ static int build_function(nncase_hip_ctx_t *ctx, Span text_span, Span rdata, nnc
 
     // ---- operators ----------------------------------------------------------------------------------
     NNHIP_REQUIRE(ctx, nncase_hip_function_create(ctx, &m->fn) == 0, -ENOMEM, "kmodel_load: cannot create the function");
+    // Everything a convolution operator needs short of recording it: checks, packed weights (kept in m->weights), the
+    // arguments with whatever is folded into the epilogue, and where the result goes.
+    auto prepare_conv = [&](uint32_t k, nncase_hip_weights_t **wt_out, nncase_hip_conv2d_args_t *a_out, void **y_out,
+                            const uint8_t **w_host) -> int {
+        const hipf_op &o = ops[k];
+        const uint32_t in0 = (uint32_t)o.inputs[0], dst = (uint32_t)o.output;
+        const hipf_tensor &ti = m->tensors[in0], &to = m->tensors[dst];
+        int rc = -EINVAL;
+        const int oc = o.p[0], gic = o.p[1], kh = o.p[2], kw = o.p[3], groups = o.p[4];
+        NNHIP_REQUIRE(ctx, oc > 0 && gic > 0 && kh > 0 && kw > 0 && groups > 0, -EINVAL, "kmodel_load: op %u conv shape", k);
+        // a convolution whose Quantize consumer is absent writes float32 (the matmul of config 1 is one)
+        NNHIP_REQUIRE(ctx, ti.dtype == NNCASE_HIP_DT_U8 && (to.dtype == NNCASE_HIP_DT_U8 || to.dtype == NNCASE_HIP_DT_F32),
+                      -NNCASE_HIP_ERR_DATATYPE_MISMATCH, "kmodel_load: op %u conv needs a u8 input and a u8 or f32 output", k);
+        NNHIP_REQUIRE(ctx, to.dtype == NNCASE_HIP_DT_U8 || (fused_lut[k] < 0 && fused_add[k] < 0), -NNCASE_HIP_ERR_DATATYPE_MISMATCH,
+                      "kmodel_load: op %u writes f32, which a byte table or a residual add cannot follow", k);
+        NNHIP_REQUIRE(ctx, (uint32_t)(gic * groups) == ti.dims[3] && (uint32_t)oc == to.dims[3] && ti.dims[0] == to.dims[0],
+                      -NNCASE_HIP_ERR_SHAPE_MISMATCH, "kmodel_load: op %u conv channels / batch do not match its tensors", k);
+        const size_t wbytes = (size_t)oc * gic * kh * kw;
+        const uint8_t *w = rd(o.rdata0, wbytes);
+        NNHIP_REQUIRE(ctx, w, -EINVAL, "kmodel_load: op %u weights outside .rdata", k);
+        const uint8_t *b = nullptr;
+        if (o.rdata1 != kNoRdata) {
+            b = rd(o.rdata1, (size_t)oc * 4);
+            NNHIP_REQUIRE(ctx, b && (o.rdata1 & 3) == 0, -EINVAL, "kmodel_load: op %u bias outside .rdata or misaligned", k);
+        }
+        nncase_hip_conv2d_desc_t desc{};
+        desc.in_channels = gic * groups, desc.out_channels = oc, desc.kernel_h = kh, desc.kernel_w = kw, desc.groups = groups;
+        desc.w_qp = nncase_hip_quant_param_t{o.p[13], o.f[2]};
+        desc.expected_pixels = (int64_t)to.dims[0] * to.dims[1] * to.dims[2];
+        nncase_hip_weights_t *wt = nullptr;
+        rc = nncase_hip_qconv2d_prepack(ctx, &desc, w, reinterpret_cast<const int32_t *>(b), &wt);
+        if (rc) return rc;
+        m->weights.push_back(wt);
+        nncase_hip_conv2d_args_t a{};
+        a.batch = (int)ti.dims[0], a.in_h = (int)ti.dims[1], a.in_w = (int)ti.dims[2];
+        a.stride_h = o.p[5], a.stride_w = o.p[6], a.dilation_h = o.p[7], a.dilation_w = o.p[8];
+        a.pad_h_before = o.p[9], a.pad_h_after = o.p[10], a.pad_w_before = o.p[11], a.pad_w_after = o.p[12];
+        a.x_qp = tqp(in0), a.y_qp = tqp(dst);
+        a.clamp_min = o.f[0], a.clamp_max = o.f[1];
+        a.out_dtype = (int32_t)to.dtype;
+        NNHIP_REQUIRE(ctx, windowed_output_size(a.in_h, kh, a.stride_h, a.dilation_h, a.pad_h_before, a.pad_h_after) == (int)to.dims[1] &&
+                               windowed_output_size(a.in_w, kw, a.stride_w, a.dilation_w, a.pad_w_before, a.pad_w_after) == (int)to.dims[2],
+                      -NNCASE_HIP_ERR_SHAPE_MISMATCH, "kmodel_load: op %u conv output extent does not match its tensor", k);
+        void *y = m->buffers[dst];
+        if (fused_lut[k] >= 0) {
+            const hipf_op &lut = ops[fused_lut[k]];
+            const uint8_t *table = rd(lut.rdata0, 256);
+            NNHIP_REQUIRE(ctx, table, -EINVAL, "kmodel_load: op %d table outside .rdata", fused_lut[k]);
+            NNHIP_REQUIRE(ctx, elems((uint32_t)lut.output) == elems(dst), -NNCASE_HIP_ERR_SHAPE_MISMATCH,
+                          "kmodel_load: op %d shapes differ", fused_lut[k]);
+            // (a conv that writes into its concat applies its table and the concat's requantisation in one)
+            rc = through[k].has_table ? nncase_hip_weights_set_post_lut(ctx, wt, through[k].table, tqp((uint32_t)ops[through[k].concat].output))
+                                      : nncase_hip_weights_set_post_lut(ctx, wt, table, tqp((uint32_t)lut.output));
+            if (rc) return rc;
+            y = m->buffers[lut.output];
+        } else if (through[k].has_table) {
+            rc = nncase_hip_weights_set_post_lut(ctx, wt, through[k].table, tqp((uint32_t)ops[through[k].concat].output));
+            if (rc) return rc;
+        }
+        if (fused_add[k] >= 0) {
+            const hipf_op &add = ops[fused_add[k]];
+            const uint32_t res = (uint32_t)add.inputs[0], sum = (uint32_t)add.output;
+            NNHIP_REQUIRE(ctx, elems(res) == elems(dst) && elems(sum) == elems(dst), -NNCASE_HIP_ERR_SHAPE_MISMATCH,
+                          "kmodel_load: op %d add shapes differ", fused_add[k]);
+            a.residual_dev = static_cast<const uint8_t *>(m->buffers[res]);
+            a.residual_qp = tqp(res), a.sum_qp = tqp(sum);
+            a.sum_clamp_min = add.f[0], a.sum_clamp_max = add.f[1];
+            y = m->buffers[sum];
+        }
+        if (fused_deq[k] >= 0) {
+            y = m->buffers[ops[fused_deq[k]].output];
+            a.out_dtype = NNCASE_HIP_DT_F32, a.dequantize_output = 1;
+        }
+        if (through[k].concat >= 0) {
+            y = m->buffers[ops[through[k].concat].output];
+            a.out_channel_stride = through[k].stride, a.out_channel_offset = through[k].offset;
+        }
+        *wt_out = wt, *a_out = a, *y_out = y, *w_host = w;
+        return 0;
+    };
+
     for (uint32_t k = 0; k < th.n_ops; k++) {
         if (skipped[k]) continue;
         const hipf_op &o = ops[k];
@@ -623,74 +747,34 @@ static int build_function(nncase_hip_ctx_t *ctx, Span text_span, Span rdata, nnc
                                                     elems(dst), tqp(in0));
             break;
         case kOpConv2d: {
-            const int oc = o.p[0], gic = o.p[1], kh = o.p[2], kw = o.p[3], groups = o.p[4];
-            NNHIP_REQUIRE(ctx, oc > 0 && gic > 0 && kh > 0 && kw > 0 && groups > 0, -EINVAL, "kmodel_load: op %u conv shape", k);
-            // a convolution whose Quantize consumer is absent writes float32 (the matmul of config 1 is one)
-            NNHIP_REQUIRE(ctx, ti.dtype == NNCASE_HIP_DT_U8 && (to.dtype == NNCASE_HIP_DT_U8 || to.dtype == NNCASE_HIP_DT_F32),
-                          -NNCASE_HIP_ERR_DATATYPE_MISMATCH, "kmodel_load: op %u conv needs a u8 input and a u8 or f32 output", k);
-            NNHIP_REQUIRE(ctx, to.dtype == NNCASE_HIP_DT_U8 || (fused_lut[k] < 0 && fused_add[k] < 0), -NNCASE_HIP_ERR_DATATYPE_MISMATCH,
-                          "kmodel_load: op %u writes f32, which a byte table or a residual add cannot follow", k);
-            NNHIP_REQUIRE(ctx, (uint32_t)(gic * groups) == ti.dims[3] && (uint32_t)oc == to.dims[3] && ti.dims[0] == to.dims[0],
-                          -NNCASE_HIP_ERR_SHAPE_MISMATCH, "kmodel_load: op %u conv channels / batch do not match its tensors", k);
-            const size_t wbytes = (size_t)oc * gic * kh * kw;
-            const uint8_t *w = rd(o.rdata0, wbytes);
-            NNHIP_REQUIRE(ctx, w, -EINVAL, "kmodel_load: op %u weights outside .rdata", k);
-            const uint8_t *b = nullptr;
-            if (o.rdata1 != kNoRdata) {
-                b = rd(o.rdata1, (size_t)oc * 4);
-                NNHIP_REQUIRE(ctx, b && (o.rdata1 & 3) == 0, -EINVAL, "kmodel_load: op %u bias outside .rdata or misaligned", k);
-            }
-            nncase_hip_conv2d_desc_t desc{};
-            desc.in_channels = gic * groups, desc.out_channels = oc, desc.kernel_h = kh, desc.kernel_w = kw, desc.groups = groups;
-            desc.w_qp = nncase_hip_quant_param_t{o.p[13], o.f[2]};
-            desc.expected_pixels = (int64_t)to.dims[0] * to.dims[1] * to.dims[2];
             nncase_hip_weights_t *wt = nullptr;
-            rc = nncase_hip_qconv2d_prepack(ctx, &desc, w, reinterpret_cast<const int32_t *>(b), &wt);
-            if (rc) return rc;
-            m->weights.push_back(wt);
             nncase_hip_conv2d_args_t a{};
-            a.batch = (int)ti.dims[0], a.in_h = (int)ti.dims[1], a.in_w = (int)ti.dims[2];
-            a.stride_h = o.p[5], a.stride_w = o.p[6], a.dilation_h = o.p[7], a.dilation_w = o.p[8];
-            a.pad_h_before = o.p[9], a.pad_h_after = o.p[10], a.pad_w_before = o.p[11], a.pad_w_after = o.p[12];
-            a.x_qp = tqp(in0), a.y_qp = tqp(dst);
-            a.clamp_min = o.f[0], a.clamp_max = o.f[1];
-            a.out_dtype = (int32_t)to.dtype;
-            NNHIP_REQUIRE(ctx, windowed_output_size(a.in_h, kh, a.stride_h, a.dilation_h, a.pad_h_before, a.pad_h_after) == (int)to.dims[1] &&
-                                   windowed_output_size(a.in_w, kw, a.stride_w, a.dilation_w, a.pad_w_before, a.pad_w_after) == (int)to.dims[2],
-                          -NNCASE_HIP_ERR_SHAPE_MISMATCH, "kmodel_load: op %u conv output extent does not match its tensor", k);
-            void *y = m->buffers[dst];
-            if (fused_lut[k] >= 0) {
-                const hipf_op &lut = ops[fused_lut[k]];
-                const uint8_t *table = rd(lut.rdata0, 256);
-                NNHIP_REQUIRE(ctx, table, -EINVAL, "kmodel_load: op %d table outside .rdata", fused_lut[k]);
-                NNHIP_REQUIRE(ctx, elems((uint32_t)lut.output) == elems(dst), -NNCASE_HIP_ERR_SHAPE_MISMATCH,
-                              "kmodel_load: op %d shapes differ", fused_lut[k]);
-                // (a conv that writes into its concat applies its table and the concat's requantisation in one)
-                rc = through[k].has_table ? nncase_hip_weights_set_post_lut(ctx, wt, through[k].table, tqp((uint32_t)ops[through[k].concat].output))
-                                          : nncase_hip_weights_set_post_lut(ctx, wt, table, tqp((uint32_t)lut.output));
+            void *y = nullptr;
+            const uint8_t *w_host = nullptr;
+            rc = prepare_conv(k, &wt, &a, &y, &w_host);
+            if (rc) return rc;
+            if (pair_second[k] >= 0) {
+                nncase_hip_weights_t *wt2 = nullptr, *wt0 = nullptr;
+                nncase_hip_conv2d_args_t a2{}, a0{};
+                void *y2 = nullptr, *y0 = nullptr;
+                const uint8_t *w2_host = nullptr, *w0_host = nullptr;
+                rc = prepare_conv((uint32_t)pair_second[k], &wt2, &a2, &y2, &w2_host);
                 if (rc) return rc;
-                y = m->buffers[lut.output];
-            } else if (through[k].has_table) {
-                rc = nncase_hip_weights_set_post_lut(ctx, wt, through[k].table, tqp((uint32_t)ops[through[k].concat].output));
+                nncase_hip_qpair_t *pr = nullptr;
+                rc = nncase_hip_qpointwise_pair_create(ctx, wt, w_host, wt2, w2_host, &pr);
                 if (rc) return rc;
-            }
-            if (fused_add[k] >= 0) {
-                const hipf_op &add = ops[fused_add[k]];
-                const uint32_t res = (uint32_t)add.inputs[0], sum = (uint32_t)add.output;
-                NNHIP_REQUIRE(ctx, elems(res) == elems(dst) && elems(sum) == elems(dst), -NNCASE_HIP_ERR_SHAPE_MISMATCH,
-                              "kmodel_load: op %d add shapes differ", fused_add[k]);
-                a.residual_dev = static_cast<const uint8_t *>(m->buffers[res]);
-                a.residual_qp = tqp(res), a.sum_qp = tqp(sum);
-                a.sum_clamp_min = add.f[0], a.sum_clamp_max = add.f[1];
-                y = m->buffers[sum];
-            }
-            if (fused_deq[k] >= 0) {
-                y = m->buffers[ops[fused_deq[k]].output];
-                a.out_dtype = NNCASE_HIP_DT_F32, a.dequantize_output = 1;
-            }
-            if (through[k].concat >= 0) {
-                y = m->buffers[ops[through[k].concat].output];
-                a.out_channel_stride = through[k].stride, a.out_channel_offset = through[k].offset;
+                m->pairs.push_back(pr);
+                if (pair_front[k] >= 0) {
+                    rc = prepare_conv((uint32_t)pair_front[k], &wt0, &a0, &y0, &w0_host);
+                    if (rc) return rc;
+                    const void *x0 = m->buffers[ops[pair_front[k]].inputs[0]];
+                    rc = nncase_hip_function_add_qdepthwise_pointwise_pair(m->fn, static_cast<const uint8_t *>(x0), wt0, &a0, pr,
+                                                                           static_cast<uint8_t *>(y), static_cast<uint8_t *>(y2), &a, &a2);
+                } else {
+                    rc = nncase_hip_function_add_qpointwise_pair(m->fn, static_cast<const uint8_t *>(m->buffers[in0]), pr, static_cast<uint8_t *>(y),
+                                                                 static_cast<uint8_t *>(y2), &a, &a2);
+                }
+                break;
             }
             rc = nncase_hip_function_add_qconv2d(m->fn, static_cast<const uint8_t *>(m->buffers[in0]), wt, y, &a);
             break;

@@ -114,7 +114,6 @@ template <int KC, bool FIRST>
 __device__ __forceinline__ void run_stage(const PairArgs &a, const uint8_t *rows, int stride, uint8_t *ys, int sy, const uint8_t *lut, int first,
                                           int step, int end, TileLoads<KC> &cur, int lane, int p, bool store_y1) {
     const int j = lane & 15, g = lane >> 4;
-    const uint8_t *w = FIRST ? a.wa : a.wb;
     const int ksteps = FIRST ? a.ks1 : a.ks2;
     const int zx = FIRST ? a.zxa : a.zxb, zw = FIRST ? a.zwa : a.zwb;
     const Epilogue &ep = FIRST ? a.ep_a : a.ep_b;

@@ -51,16 +51,23 @@ def test_conv_block_kmodel(hip_ctx):
     assert e.value.code == -rt.ERR_SHAPE_MISMATCH
 
 
-def test_mobilenetv2_kmodel(hip_ctx):
+@pytest.mark.parametrize("batch", [4, 1])
+def test_mobilenetv2_kmodel(hip_ctx, batch):
     rng = np.random.default_rng(3)
     qg = nb.quantize_graph(nb.mobilenet_v2(seed=2), rng.random((8, 224, 224, 3), dtype=f32))
-    x = rng.random((4, 224, 224, 3), dtype=f32)
+    x = rng.random((batch, 224, 224, 3), dtype=f32)
     model, y, fused = run_and_check(hip_ctx, qg, x)
-    # the loader folds the ten residual adds, at this batch the two 28x28 blocks (64 workgroups each) whole, the
-    # input's quantize into the pack in front of the stem and the output's dequantize into the classifier
-    assert fused == 16 and len(model.fn) == 51
-    ref = nb.HipModel(hip_ctx, qg, 4, capture_graph=False)
+    ref = nb.HipModel(hip_ctx, qg, batch, capture_graph=False)
     assert np.array_equal(ref.run(x).view(np.uint32).ravel(), y.view(np.uint32).ravel())
+    # the loader folds what HipModel folds: the ten residual adds, the input's quantize into the pack in front of the stem,
+    # the output's dequantize into the classifier; at batch 4 the two 28x28 blocks (64 workgroups each) whole and the
+    # projection -> expansion pairs of the 14x14 and 7x7 maps; at batch 1 every such pair from 56x56 on, six of them with
+    # their depthwise convolution in front
+    assert len(model.fn) == len(ref.fn) == {4: 43, 1: 33}[batch]
+    assert fused == len(ref.never_written)
+    kernels = [model.fn.op_kernel(i) for i in range(len(model.fn))]
+    assert kernels == [ref.fn.op_kernel(i) for i in range(len(ref.fn))]
+    assert kernels.count("dw3x3+qpointwise_pair_kernel") == len(ref.pair_fronts) == {4: 1, 1: 6}[batch]
 
 
 def test_malformed_files_are_refused(hip_ctx):

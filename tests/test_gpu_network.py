@@ -180,7 +180,7 @@ def test_yolov5s_config4(hip_ctx):
     for want, j in zip(wants, g.outputs):
         assert O.cosine(want, fl[j]) > 0.98
     loaded = rt.LoadedKModel(hip_ctx, km.compile_quant_graph(qg, 2))
-    assert len(loaded.fn) == 147 - 64 - 7 - 1 - 3   # the native loader folds the same tables, adds, concat slices, quantize, dequantizes
+    assert len(loaded.fn) == 147 - 64 - 7 - 1 - 3 - 11   # the native loader folds the same tables, adds, concat slices, quantize, dequantizes, pairs
     ys = loaded.run(x)
     assert len(ys) == 3
     for y, want in zip(ys, wants):
