@@ -188,6 +188,9 @@ def test_loader_reads_exactly_the_fields_the_table_names():
     blocks = re.split(r"\n        case (kOp\w+):", switch[:switch.index("\n        default:")])
     seen = {}
     for label, block in zip(blocks[1::2], blocks[2::2]):
+        if label == "kOpConv2d":     # its record is read by the helper that a pair's other convolutions go through as well
+            assert "prepare_conv(k," in block
+            block = text[text.index("auto prepare_conv = "):text.index("    for (uint32_t k = 0; k < th.n_ops; k++) {", text.index("auto prepare_conv = "))]
         seen[label] = ({int(i) for i in re.findall(r"\bo\.p\[(\d+)\]", block)}, {int(i) for i in re.findall(r"\bo\.f\[(\d+)\]", block)},
                        len(set(re.findall(r"\bo\.rdata(\d)", block))))
     assert set(seen) == set(names)
