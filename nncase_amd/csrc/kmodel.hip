@@ -528,7 +528,7 @@ static int build_function(nncase_hip_ctx_t *ctx, Span text_span, Span rdata, nnc
     // them reads joins the launch while it has few channels.
     std::vector<int> pair_second(th.n_ops, -1), pair_front(th.n_ops, -1);
     {
-        constexpr uint64_t kStreamLimit = 4u << 20, kMaxPixelTiles = 512;
+        constexpr uint64_t kStreamLimit = 4u << 20, kMaxPixelTiles = 1024;
         constexpr int kFrontMaxChannels = 256;
         auto plain_pointwise = [&](uint32_t k) {
             return pointwise(ops[k]) && !skipped[k] && !block_head[k] && through[k].concat < 0 && fused_deq[k] < 0 &&

@@ -475,6 +475,13 @@ static int launch_pair(nncase_hip_ctx *ctx, const char *who, const uint8_t *x_de
     ranges = (a.t2 + a.tiles_per_block - 1) / a.tiles_per_block;
     int waves = std::min(max_waves, std::max(a.t1, a.tiles_per_block));
     if (dw) waves = std::min(max_waves, std::max(waves, (a.k1 + 63) / 64));
+    {
+        // ... but no more than lets every workgroup be resident at once (a second round of workgroups doubles the
+        // launch's latency chain; a wave that takes two channel tiles one after the other adds a fraction of it)
+        const int occupancy = small ? (dw ? 4 : 5) : 3; // waves per SIMD the variant is built for
+        const int per_cu = (ptiles * ranges + ctx->compute_units - 1) / std::max(ctx->compute_units, 1);
+        waves = std::max(1, std::min(waves, 4 * occupancy / std::max(per_cu, 1)));
+    }
     NNHIP_HIP(ctx, hipSetDevice(ctx->device));
     const dim3 grid(ptiles, ranges), block(waves * 64);
     const size_t lds = pair_lds_bytes(pr);

@@ -401,7 +401,7 @@ def pad_small_channel_convs(qg: QuantGraph) -> QuantGraph:
 # resident at once.  Measured on MobileNetV2: every pair within these limits is quicker than its two launches at
 # batches 1 and 2 (0.215 -> 0.184 ms per image at batch 1); beyond them the separate kernels win.
 PAIR_STREAM_LIMIT = 4 << 20
-PAIR_MAX_PIXEL_TILES = 512
+PAIR_MAX_PIXEL_TILES = 1024
 # A depthwise convolution in front joins the pair while it has few channels: a workgroup computes its 16 pixels of it
 # alone, about 50 ns per 16 channels, against the 3.5 us of the separate launch it saves.
 PAIR_FRONT_MAX_CHANNELS = 256
