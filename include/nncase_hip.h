@@ -300,6 +300,19 @@ typedef struct nncase_hip_qblock_args {
 NNCASE_HIP_API int nncase_hip_qblock(nncase_hip_ctx_t *ctx, const uint8_t *x_dev, const nncase_hip_qblock_t *block,
                                      uint8_t *y_dev, const nncase_hip_qblock_args_t *args);
 
+/* Global average pool (ReduceMean over H and W of a u8 tensor, src/Native/src/kernels/stackvm/reference/reduce.cpp,
+ * requantised to args->x_qp) and the dense 1x1 Conv2D that reads its [batch, 1, 1, channels] result as one launch: a
+ * classifier's pool -> fully-connected tail at small batches.  x_dev is the pool's input [batch, h, w, channels] with
+ * quantisation x_qp; args are the convolution's (in_h = in_w = 1; u8 output or dequantize_output).  Same bytes as
+ * nncase_hip_qglobal_avgpool followed by nncase_hip_qconv2d.  The weights must have been pre-packed with
+ * expected_pixels = the batch (a few rows): _supported says whether a call qualifies and pays (every workgroup pools
+ * its rows itself, so only while rows x pixels x channels is small). */
+NNCASE_HIP_API int nncase_hip_qglobal_avgpool_qconv2d_supported(const nncase_hip_weights_t *weights,
+                                                                const nncase_hip_conv2d_args_t *args, int32_t h, int32_t w);
+NNCASE_HIP_API int nncase_hip_qglobal_avgpool_qconv2d(nncase_hip_ctx_t *ctx, const uint8_t *x_dev, int32_t h, int32_t w,
+                                                      nncase_hip_quant_param_t x_qp, const nncase_hip_weights_t *weights,
+                                                      void *y_dev, const nncase_hip_conv2d_args_t *args);
+
 /* ---- pair of pointwise convolutions ------------------------------------------
  * Two dense 1x1, stride-1, unpadded Conv2D calls of which the second reads the
  * first's result (a bottleneck's projection and the next block's expansion,
@@ -602,6 +615,10 @@ NNCASE_HIP_API int nncase_hip_function_add_qdepthwise_pointwise_pair(nncase_hip_
                                                                      uint8_t *y2_dev,
                                                                      const nncase_hip_conv2d_args_t *first_args,
                                                                      const nncase_hip_conv2d_args_t *second_args);
+NNCASE_HIP_API int nncase_hip_function_add_qglobal_avgpool_qconv2d(nncase_hip_function_t *fn, const uint8_t *x_dev, int32_t h,
+                                                                   int32_t w, nncase_hip_quant_param_t x_qp,
+                                                                   const nncase_hip_weights_t *weights, void *y_dev,
+                                                                   const nncase_hip_conv2d_args_t *args);
 NNCASE_HIP_API int nncase_hip_function_add_qadd(nncase_hip_function_t *fn, const uint8_t *a_dev,
                                                 nncase_hip_quant_param_t a_qp, const uint8_t *b_dev,
                                                 nncase_hip_quant_param_t b_qp, uint8_t *out_dev,

@@ -9,7 +9,7 @@ namespace {
 
 struct Op {
     enum Kind { kQuantize, kDequantize, kConv, kAdd, kPool, kLut, kConcat, kResize, kMaxPool, kPack, kQuantPack,
-                kGemm, kRmsNorm, kRope, kGemmRope, kAttn, kArgmax, kEmbed, kAddI32, kBlock, kLayout, kPair } kind;
+                kGemm, kRmsNorm, kRope, kGemmRope, kAttn, kArgmax, kEmbed, kAddI32, kBlock, kLayout, kPair, kPoolConv } kind;
     const void *in0 = nullptr, *in1 = nullptr;
     void *out = nullptr;
     const nncase_hip_weights_t *weights = nullptr;
@@ -78,6 +78,8 @@ static int run_op(nncase_hip_function *fn, const Op &op) {
             return nncase_hip_qdepthwise_pointwise_pair(ctx, (const uint8_t *)op.in0, op.weights, &op.conv3, op.pair, (uint8_t *)op.out,
                                                         (uint8_t *)op.out2, &op.conv, &op.conv2);
         return nncase_hip_qpointwise_pair(ctx, (const uint8_t *)op.in0, op.pair, (uint8_t *)op.out, (uint8_t *)op.out2, &op.conv, &op.conv2);
+    case Op::kPoolConv: // h, w and qp0 the pool's input, conv the convolution behind it
+        return nncase_hip_qglobal_avgpool_qconv2d(ctx, (const uint8_t *)op.in0, op.h, op.w, op.qp0, op.weights, op.out, &op.conv);
     case Op::kAdd:
         return nncase_hip_qadd(ctx, (const uint8_t *)op.in0, op.qp0, (const uint8_t *)op.in1, op.qp1, (uint8_t *)op.out,
                                op.qp2, op.lo, op.hi, op.count);
@@ -243,6 +245,17 @@ extern "C" int nncase_hip_function_add_qdepthwise_pointwise_pair(nncase_hip_func
     op.kind = Op::kPair;
     op.in0 = x_dev, op.out = y1_dev, op.out2 = y2_dev, op.pair = pair, op.conv = *first_args, op.conv2 = *second_args;
     op.weights = depthwise, op.conv3 = *depthwise_args;
+    return push(fn, op);
+}
+
+extern "C" int nncase_hip_function_add_qglobal_avgpool_qconv2d(nncase_hip_function_t *fn, const uint8_t *x_dev, int32_t h, int32_t w,
+                                                               nncase_hip_quant_param_t x_qp, const nncase_hip_weights_t *weights, void *y_dev,
+                                                               const nncase_hip_conv2d_args_t *args) {
+    if (!fn) return -EINVAL;
+    NNHIP_REQUIRE(fn->ctx, x_dev && weights && y_dev && args, -EINVAL, "function_add_qglobal_avgpool_qconv2d: null argument");
+    Op op;
+    op.kind = Op::kPoolConv;
+    op.in0 = x_dev, op.out = y_dev, op.weights = weights, op.conv = *args, op.h = h, op.w = w, op.qp0 = x_qp;
     return push(fn, op);
 }
 
@@ -615,6 +628,7 @@ extern "C" int nncase_hip_function_op_kernel(nncase_hip_function_t *fn, int32_t 
     case Op::kDequantize: snprintf(name, capacity, "dequantize"); break;
     case Op::kConv: describe_conv_kernel(fn->ctx, op.weights, &op.conv, name, capacity); break;
     case Op::kBlock: nncase_hip_qblock_describe(op.block, &op.blk, name, capacity); break;
+    case Op::kPoolConv: snprintf(name, capacity, "qglobal_avgpool+qpointwise_rows%s", op.conv.dequantize_output ? "+dequantize" : ""); break;
     case Op::kPair: snprintf(name, capacity, op.weights ? "dw3x3+qpointwise_pair_kernel" : "qpointwise_pair_kernel"); break;
     case Op::kAdd: snprintf(name, capacity, "qadd"); break;
     case Op::kPool: snprintf(name, capacity, "qglobal_avgpool"); break;

@@ -11,7 +11,7 @@
 // buffer per tensor and records the operators into a resident function, which is what the
 // module's runtime_function::invoke_core would run (src/Native/include/nncase/runtime/
 // runtime_function.h:55-63).
-#include "common.hpp"
+#include "qconv.hpp"
 
 #include <memory>
 #include <new>
@@ -561,6 +561,28 @@ static int build_function(nncase_hip_ctx_t *ctx, Span text_span, Span rdata, nnc
         }
     }
 
+    // A global average pool read by one dense 1x1 convolution alone (a classifier's tail) is computed by that
+    // convolution's launch where that pays: a few rows (see nncase_hip_qglobal_avgpool_qconv2d).
+    std::vector<int> pool_reader(th.n_ops, -1), pool_of(th.n_ops, -1); // pool op -> conv op and back
+    for (uint32_t k = 0; k < th.n_ops; k++) {
+        const hipf_op &g = ops[k];
+        if (g.opcode != kOpGlobalAvgPool || g.n_inputs != 1 || skipped[k] || consumers[g.output] != 1 || is_output(g.output)) continue;
+        const hipf_tensor &tg = m->tensors[g.inputs[0]], &tp = m->tensors[g.output];
+        if (tg.dtype != NNCASE_HIP_DT_U8 || tp.dtype != NNCASE_HIP_DT_U8 || tp.dims[0] != tg.dims[0] || tp.dims[3] != tg.dims[3] || tp.dims[1] != 1 ||
+            tp.dims[2] != 1)
+            continue;
+        for (uint32_t c = k + 1; c < th.n_ops; c++) {
+            if (ops[c].n_inputs != 1 || ops[c].inputs[0] != g.output) continue;
+            // (the conditions of nncase_hip_qglobal_avgpool_qconv2d_supported, decided here because the pooled tensor gets no buffer)
+            const hipf_tensor &ty = m->tensors[ops[c].output];
+            if (pointwise(ops[c]) && !skipped[c] && !block_head[c] && through[c].concat < 0 && fused_add[c] < 0 && pair_second[c] < 0 &&
+                (ty.dtype == NNCASE_HIP_DT_U8 || fused_deq[c] >= 0) && rows_shapes_ok(ops[c].p[1], ops[c].p[0], (int64_t)tp.dims[0]) &&
+                pool_front_pays((int)tg.dims[0], (int)(tg.dims[1] * tg.dims[2]), (int)tg.dims[3]))
+                pool_reader[k] = (int)c, pool_of[c] = (int)k;
+            break;
+        }
+    }
+
     // ---- device buffers ---------------------------------------------------------------------------
     m->buffers.assign(th.n_tensors, nullptr);
     m->owns.assign(th.n_tensors, 0);
@@ -569,6 +591,7 @@ static int build_function(nncase_hip_ctx_t *ctx, Span text_span, Span rdata, nnc
         if (fused_add[k] >= 0 && fused_lut[k] >= 0) m->owns[ops[fused_lut[k]].output] = 2;
         if (block_head[k]) m->owns[ops[k].output] = m->owns[ops[k + 1].output] = 2;
         if (pair_front[k] >= 0) m->owns[ops[pair_front[k]].output] = 2; // computed inside the pair's launch
+        if (pool_reader[k] >= 0) m->owns[ops[k].output] = 2;            // ... inside the convolution's
         if (fused_quant[k] >= 0) m->owns[ops[fused_quant[k]].output] = 2;
         if (fused_deq[k] >= 0) { // the u8 result is never stored
             m->owns[ops[k].output] = 2;
@@ -753,6 +776,18 @@ static int build_function(nncase_hip_ctx_t *ctx, Span text_span, Span rdata, nnc
             const uint8_t *w_host = nullptr;
             rc = prepare_conv(k, &wt, &a, &y, &w_host);
             if (rc) return rc;
+            if (pool_of[k] >= 0) {
+                // a global average pool that only this convolution reads: one launch for both where the library says it
+                // pays (a few rows), else the pool now, in front of the convolution
+                const hipf_op &g = ops[pool_of[k]];
+                const uint32_t gin = (uint32_t)g.inputs[0];
+                const hipf_tensor &tg = m->tensors[gin];
+                NNHIP_REQUIRE(ctx, nncase_hip_qglobal_avgpool_qconv2d_supported(wt, &a, (int)tg.dims[1], (int)tg.dims[2]), -EINVAL,
+                              "kmodel_load: op %u was planned as a pooled convolution and does not qualify", k);
+                rc = nncase_hip_function_add_qglobal_avgpool_qconv2d(m->fn, static_cast<const uint8_t *>(m->buffers[gin]), (int)tg.dims[1],
+                                                                     (int)tg.dims[2], tqp(gin), wt, y, &a);
+                break;
+            }
             if (pair_second[k] >= 0) {
                 nncase_hip_weights_t *wt2 = nullptr, *wt0 = nullptr;
                 nncase_hip_conv2d_args_t a2{}, a0{};
@@ -792,6 +827,10 @@ static int build_function(nncase_hip_ctx_t *ctx, Span text_span, Span rdata, nnc
         case kOpGlobalAvgPool:
             NNHIP_REQUIRE(ctx, to.dims[0] == ti.dims[0] && to.dims[3] == ti.dims[3] && to.dims[1] == 1 && to.dims[2] == 1,
                           -NNCASE_HIP_ERR_SHAPE_MISMATCH, "kmodel_load: op %u pool shapes", k);
+            if (pool_reader[k] >= 0) { // recorded with the convolution that alone reads it
+                rc = 0;
+                break;
+            }
             rc = nncase_hip_function_add_qglobal_avgpool(m->fn, static_cast<const uint8_t *>(m->buffers[in0]),
                                                          static_cast<uint8_t *>(m->buffers[dst]), (int)ti.dims[0], (int)ti.dims[1],
                                                          (int)ti.dims[2], (int)ti.dims[3], tqp(in0), tqp(dst));

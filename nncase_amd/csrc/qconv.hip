@@ -32,6 +32,10 @@ void nnhip::describe_conv_kernel(const nncase_hip_ctx *ctx, const nncase_hip_wei
     static const char *modes[] = {"rows16", "vec16", "vec8", "vec4", "bytes", "rows8"};
     const int out_h = windowed_output_size(a->in_h, w->kernel_h, a->stride_h, a->dilation_h, a->pad_h_before, a->pad_h_after);
     const int out_w = windowed_output_size(a->in_w, w->kernel_w, a->stride_w, a->dilation_w, a->pad_w_before, a->pad_w_after);
+    if (rows_path_taken(w, a, out_h, out_w)) {
+        snprintf(buf, cap, "qpointwise_rows%s%s", w->d_post_lut ? "+lut" : "", a->dequantize_output ? "+dequantize" : "");
+        return;
+    }
     const long long m = (long long)a->batch * out_h * out_w;
     const int mode = igemm_load_mode(w, a, out_h, out_w);
     const int mi = (int)std::min<long long>(m, 1 << 30);
@@ -273,6 +277,7 @@ static void free_weights(nncase_hip_weights *w) {
     if (w->d_bias) (void)hipFree(w->d_bias);
     if (w->d_smallc) (void)hipFree(w->d_smallc);
     if (w->d_post_lut) (void)hipFree(w->d_post_lut);
+    rows_free(w);
     delete w;
 }
 
@@ -348,6 +353,7 @@ extern "C" int nncase_hip_qconv2d_prepack(nncase_hip_ctx_t *ctx, const nncase_hi
     int rc = depthwise ? prepack_depthwise(ctx, w, weights_oihw_host, bias_host)
                        : prepack_igemm(ctx, w, weights_oihw_host, bias_host);
     if (rc == 0 && !depthwise && smallc_supported(w)) rc = prepack_smallc(ctx, w, weights_oihw_host);
+    if (rc == 0 && !depthwise) rc = rows_prepack(ctx, w, weights_oihw_host);
     if (rc) {
         free_weights(w);
         return rc;
@@ -420,6 +426,7 @@ extern "C" int nncase_hip_qconv2d(nncase_hip_ctx_t *ctx, const uint8_t *x_dev, c
     const int out_h = windowed_output_size(a->in_h, w->kernel_h, a->stride_h, a->dilation_h, a->pad_h_before, a->pad_h_after);
     const int out_w = windowed_output_size(a->in_w, w->kernel_w, a->stride_w, a->dilation_w, a->pad_w_before, a->pad_w_after);
     NNHIP_REQUIRE(ctx, out_h > 0 && out_w > 0, -NNCASE_HIP_ERR_SHAPE_MISMATCH, "qconv2d: window larger than padded input");
+    if (rows_path_taken(w, a, out_h, out_w)) return launch_qconv_rows(ctx, x_dev, w, y_dev, a, nullptr);
     if (a->out_channel_stride != 0 || a->out_channel_offset != 0) {
         NNHIP_REQUIRE(ctx, w->kind == nncase_hip_weights::kIgemm, -EINVAL,
                       "qconv2d: an output inside a wider tensor is only supported by the dense (MFMA) kernels");
@@ -481,4 +488,38 @@ extern "C" int nncase_hip_qmatmul(nncase_hip_ctx_t *ctx, const uint8_t *a_dev, c
     c.clamp_max = m->clamp_max;
     c.out_dtype = m->out_dtype;
     return nncase_hip_qconv2d(ctx, a_dev, w, y_dev, &c);
+}
+
+extern "C" int nncase_hip_qglobal_avgpool_qconv2d(nncase_hip_ctx_t *ctx, const uint8_t *x_dev, int32_t h, int32_t w_,
+                                                  nncase_hip_quant_param_t x_qp, const nncase_hip_weights_t *w, void *y_dev,
+                                                  const nncase_hip_conv2d_args_t *a) {
+    NNHIP_CHECK_CTX(ctx);
+    NNHIP_REQUIRE(ctx, x_dev && w && y_dev && a, -EINVAL, "qglobal_avgpool_qconv2d: null argument");
+    NNHIP_REQUIRE(ctx, a->batch > 0 && h > 0 && w_ > 0 && a->in_h == 1 && a->in_w == 1, -EINVAL,
+                  "qglobal_avgpool_qconv2d: the convolution reads one pooled pixel per image");
+    NNHIP_REQUIRE(ctx, x_qp.zero_point >= 0 && x_qp.zero_point <= 255 && a->x_qp.zero_point >= 0 && a->x_qp.zero_point <= 255 &&
+                           a->x_qp.scale != 0.f,
+                  -EINVAL, "qglobal_avgpool_qconv2d: quantisation outside u8");
+    nncase_hip_conv2d_args_t through_u8;
+    if (a->dequantize_output != 0) {
+        NNHIP_REQUIRE(ctx, a->out_dtype == NNCASE_HIP_DT_F32, -NNCASE_HIP_ERR_DATATYPE_MISMATCH,
+                      "qglobal_avgpool_qconv2d: dequantize_output needs out_dtype float32");
+        through_u8 = *a;
+        through_u8.out_dtype = NNCASE_HIP_DT_U8;
+        a = &through_u8;
+    }
+    const int rc = check_out_dtype(ctx, a->out_dtype, a->y_qp, "qglobal_avgpool_qconv2d");
+    if (rc) return rc;
+    NNHIP_REQUIRE(ctx, rows_path_taken(w, a, 1, 1), -EINVAL,
+                  "qglobal_avgpool_qconv2d: needs a dense 1x1 convolution packed for a few pixels (expected_pixels = batch at pre-pack "
+                  "time), u8 or dequantised output, no residual");
+    const PoolFront pool{h * w_, x_qp};
+    return launch_qconv_rows(ctx, x_dev, w, y_dev, a, &pool);
+}
+
+extern "C" int nncase_hip_qglobal_avgpool_qconv2d_supported(const nncase_hip_weights_t *w, const nncase_hip_conv2d_args_t *a, int32_t h,
+                                                            int32_t w_) {
+    if (!w || !a || a->in_h != 1 || a->in_w != 1 || h <= 0 || w_ <= 0 || a->batch <= 0) return 0;
+    if (!pool_front_pays(a->batch, h * w_, w->in_channels)) return 0;
+    return rows_path_taken(w, a, 1, 1) ? 1 : 0;
 }

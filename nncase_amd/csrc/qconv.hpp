@@ -36,6 +36,9 @@ struct nncase_hip_weights {
     // few-input-channel 3x3 convolutions also carry a [oc][k] s8 layout for the per-pixel dot-product kernel
     void *d_smallc = nullptr;
     size_t smallc_bytes = 0;
+    // dense 1x1 convolutions planned for a handful of pixels (a classifier head, a batch-1 matmul) also carry the
+    // weights in the order of the kernel that keeps them in registers (qpair.hip: second convolution only)
+    struct nncase_hip_qpair *rows_pack = nullptr;
 };
 
 namespace nnhip {
@@ -106,6 +109,20 @@ bool smallc_supported(const nncase_hip_weights *w);
 int prepack_smallc(nncase_hip_ctx *ctx, nncase_hip_weights *w, const uint8_t *w_oihw);
 int launch_qconv_depthwise(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_hip_weights *w, void *y,
                            const nncase_hip_conv2d_args_t *a, int out_h, int out_w);
+
+// The few-pixel path of a dense 1x1 convolution (qpair.hip): packing at pre-pack time, whether a call takes it, the launch
+// (pool != nullptr: x is [batch, pool_hw, channels] and the convolution reads its global average, requantised to c->x_qp).
+struct PoolFront {
+    int hw;
+    nncase_hip_quant_param_t x_qp;
+};
+bool rows_shapes_ok(int in_channels, int out_channels, int64_t pixels);   // what rows_prepack packs and rows_path_taken takes
+bool pool_front_pays(int rows, int hw, int channels);
+int rows_prepack(nncase_hip_ctx *ctx, nncase_hip_weights *w, const uint8_t *w_oihw);
+void rows_free(nncase_hip_weights *w);
+bool rows_path_taken(const nncase_hip_weights *w, const nncase_hip_conv2d_args_t *c, int out_h, int out_w);
+int launch_qconv_rows(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_hip_weights *w, void *y, const nncase_hip_conv2d_args_t *c,
+                      const PoolFront *pool);
 
 // Writes the name of the kernel a conv with these weights / arguments launches.
 void describe_conv_kernel(const nncase_hip_ctx *ctx, const nncase_hip_weights *w, const nncase_hip_conv2d_args_t *a, char *buf,
@@ -230,6 +247,34 @@ __device__ __forceinline__ uint32_t residual4_packed(uint32_t q, uint32_t res, c
         d = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_amdgcn_fmed3f(u, r.sum.qlo, r.sum.qhi), e, d);
     }
     return d;
+}
+
+// Global average pool of four adjacent channels of one image (NHWC u8, p at the image's first pixel): the dequantised
+// values are added in pixel order with a float accumulator, exactly the order of the reference's reduction loop
+// (src/Native/src/kernels/stackvm/reference/reduce.cpp), then mean, requantisation and rounding; the four codes packed.
+// The loads of 64 pixels (a whole 7x7 map) are issued before their values are added: one memory round trip per 64.
+__device__ __forceinline__ uint32_t global_avgpool4(const uint8_t *p, int hw, int channels, float zx, float sx, float zy, float sy) {
+    float value[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int i0 = 0; i0 < hw; i0 += 64) {
+        uint32_t d[64];
+#pragma unroll
+        for (int k = 0; k < 64; k++) d[k] = *reinterpret_cast<const uint32_t *>(p + (size_t)min(i0 + k, hw - 1) * channels);
+#pragma unroll
+        for (int k = 0; k < 64; k++)
+            if (i0 + k < hw) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) value[e] = value[e] + ((float)((d[k] >> (8 * e)) & 0xffu) - zx) * sx;
+            }
+    }
+    uint32_t q = 0;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        const float mean = value[e] / (float)hw;
+        float t = mean / sy + zy;
+        t = fminf(fmaxf(t, 0.f), 255.f);
+        q |= (uint32_t)(int32_t)rintf(t) << (8 * e);
+    }
+    return q;
 }
 
 // a + b + c in one instruction (the compiler otherwise re-associates the zero-point

@@ -31,7 +31,7 @@ struct nncase_hip_qpair {
     int32_t *d_bias_a = nullptr, *d_bias_b = nullptr; // bias, padded to whole tiles
 };
 
-namespace {
+namespace nnhip {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -64,6 +64,12 @@ struct PairArgs {
     FastDiv d_out_hw, d_out_w;
     int dw_zx;
     Epilogue ep_dw;
+    // the second convolution alone (qpointwise_rows_kernel): x holds ITS input rows [m][n1]; its result may leave as the
+    // float32 value of the u8 code, and its rows may be the global average of x [m][pool_hw][n1]
+    int deq, deq_zero;
+    float deq_scale;
+    int pool_hw;
+    float pool_zx, pool_sx, pool_zy, pool_sy;
 };
 
 __device__ __forceinline__ uint32_t table4(const uint8_t *t, uint32_t v) {
@@ -152,8 +158,15 @@ __device__ __forceinline__ void run_stage(const PairArgs &a, const uint8_t *rows
                 *reinterpret_cast<uint32_t *>(ys + j * sy + ch) = q ^ 0x80808080u;
                 if (store_y1 && p < a.m) *reinterpret_cast<uint32_t *>(a.y1 + (size_t)p * a.n1 + ch) = q;
             }
-        } else {
-            if (ch < a.n2 && p < a.m) *reinterpret_cast<uint32_t *>(a.y2 + (size_t)p * a.n2 + ch) = q;
+        } else if (ch < a.n2 && p < a.m) {
+            if (a.deq) { // the Dequantize behind the convolution: one float per channel
+                u32x4 o;
+#pragma unroll
+                for (int r = 0; r < 4; r++) o[r] = __float_as_uint((float)((int)((q >> (8 * r)) & 0xffu) - a.deq_zero) * a.deq_scale);
+                *reinterpret_cast<u32x4 *>(reinterpret_cast<float *>(a.y2) + (size_t)p * a.n2 + ch) = o;
+            } else {
+                *reinterpret_cast<uint32_t *>(a.y2 + (size_t)p * a.n2 + ch) = q;
+            }
         }
     }
 }
@@ -281,14 +294,61 @@ __global__ __launch_bounds__(MAXW * 64, OCC) void qpointwise_pair_kernel(const P
     if (b_first + wave < b_end) run_stage<KB, false>(a, ys, sy, nullptr, 0, a.lut_b ? lut_b : nullptr, b_first + wave, waves, b_end, lb, lane, p, false);
 }
 
-bool pair_is_small(int ks1, int ks2) { return ks1 <= 4 && ks2 <= 2; }
-size_t pair_lds_bytes(const nncase_hip_qpair *pr) {
+// One dense 1x1 convolution over a few rows (pixels): the second stage of the pair kernel alone.  A workgroup stages 16
+// rows as s8 in LDS and takes a range of the channel tiles, a wave per tile, the weights straight from global memory
+// into MFMA operands with the first chunk requested before the rows are staged.  Against the tiled kernels, which
+// stream k-step by k-step through LDS with a barrier each, a launch is one memory round trip long, not one per k-step.
+// POOL: the rows are global averages over pool_hw pixels, computed here (global_avgpool4, a thread per four channels).
+constexpr int kRowsChunk = 8, kRowsWaves = 12;
+template <bool POOL> __global__ __launch_bounds__(kRowsWaves * 64, 3) void qpointwise_rows_kernel(const PairArgs a) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    const int sy = pair_row_bytes(a.ks2, kRowsChunk);
+    uint8_t *ys = smem;            // [16][sy]  rows - 128
+    uint8_t *lut_b = ys + 16 * sy; // 256 bytes
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, threads = blockDim.x, waves = threads >> 6;
+    const int p0 = blockIdx.x * 16, p = p0 + (lane & 15);
+    const int b_first = blockIdx.y * a.tiles_per_block;
+    const int b_end = min(a.t2, b_first + a.tiles_per_block);
+    TileLoads<kRowsChunk> lb;
+    if (b_first + wave < b_end) load_tile<kRowsChunk, false>(lb, a, b_first + wave, 0, lane, p);
+    if constexpr (POOL) {
+        const int quads = a.n1 >> 2;
+#pragma unroll 1
+        for (int e = tid; e < 16 * quads; e += threads) {
+            const int r = e / quads, c4 = (e - r * quads) * 4;
+            uint32_t code = 0x80808080u; // rows past the tensor read as zero
+            if (p0 + r < a.m) code = global_avgpool4(a.x + (size_t)(p0 + r) * a.pool_hw * a.n1 + c4, a.pool_hw, a.n1, a.pool_zx, a.pool_sx, a.pool_zy, a.pool_sy);
+            *reinterpret_cast<uint32_t *>(ys + r * sy + c4) = code ^ 0x80808080u;
+        }
+        const int first = a.n1 / 16, extra = (sy - kRowPad) / 16 - first; // pieces past the real reduction
+        for (int e = tid; e < 16 * extra; e += threads) {
+            const int r = e / extra, c = first + (e - r * extra);
+            *reinterpret_cast<u32x4 *>(ys + r * sy + c * 16) = u32x4{0u, 0u, 0u, 0u};
+        }
+    } else {
+        const int pieces = (sy - kRowPad) / 16;
+#pragma unroll 1
+        for (int e = tid; e < 16 * pieces; e += threads) {
+            const int r = e / pieces, c = e - r * pieces;
+            u32x4 v = {0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u};
+            if (p0 + r < a.m && c * 16 < a.n1) v = *reinterpret_cast<const u32x4 *>(a.x + (size_t)(p0 + r) * a.n1 + c * 16);
+            *reinterpret_cast<u32x4 *>(ys + r * sy + c * 16) = v ^ 0x80808080u;
+        }
+    }
+    if (a.lut_b)
+        for (int e = tid; e < 64; e += threads) reinterpret_cast<uint32_t *>(lut_b)[e] = a.lut_b[e];
+    __syncthreads();
+    if (b_first + wave < b_end) run_stage<kRowsChunk, false>(a, ys, sy, nullptr, 0, a.lut_b ? lut_b : nullptr, b_first + wave, waves, b_end, lb, lane, p, false);
+}
+
+static bool pair_is_small(int ks1, int ks2) { return ks1 <= 4 && ks2 <= 2; }
+static size_t pair_lds_bytes(const nncase_hip_qpair *pr) {
     const bool small = pair_is_small(pr->ks1, pr->ks2);
     return 16 * (size_t)pair_row_bytes(pr->ks1, small ? 4 : 8) + 16 * (size_t)pair_row_bytes(pr->ks2, small ? 2 : 4) + 512;
 }
 
 // [tile][k-step][lane][16] s8 of w - 128, zero beyond the real channels / reduction
-void pack_pair_weights(std::vector<uint8_t> &out, std::vector<int32_t> &wsum, const uint8_t *w_oihw, int n, int k, int tiles, int ksteps) {
+static void pack_pair_weights(std::vector<uint8_t> &out, std::vector<int32_t> &wsum, const uint8_t *w_oihw, int n, int k, int tiles, int ksteps) {
     out.assign((size_t)tiles * ksteps * 1024, 0);
     wsum.assign((size_t)tiles * 16, 0);
     for (int ch = 0; ch < n; ch++) {
@@ -303,7 +363,7 @@ void pack_pair_weights(std::vector<uint8_t> &out, std::vector<int32_t> &wsum, co
     }
 }
 
-void free_pair(nncase_hip_qpair *pr) {
+static void free_pair(nncase_hip_qpair *pr) {
     if (!pr) return;
     if (pr->d_wa) (void)hipFree(pr->d_wa);
     if (pr->d_wb) (void)hipFree(pr->d_wb);
@@ -314,21 +374,21 @@ void free_pair(nncase_hip_qpair *pr) {
     delete pr;
 }
 
-bool pair_shapes_ok(int k1, int n1, int n2) {
+static bool pair_shapes_ok(int k1, int n1, int n2) {
     return k1 > 0 && n1 > 0 && n2 > 0 && k1 % 16 == 0 && n1 % 4 == 0 && n2 % 4 == 0 && k1 <= kPairMaxK1 && n1 <= kPairMaxN1;
 }
 
-int upload(nncase_hip_ctx *ctx, void **dst, const void *src, size_t bytes) {
+static int upload(nncase_hip_ctx *ctx, void **dst, const void *src, size_t bytes) {
     NNHIP_HIP(ctx, hipMalloc(dst, bytes));
     NNHIP_HIP(ctx, hipMemcpy(*dst, src, bytes, hipMemcpyHostToDevice));
     return 0;
 }
 
-bool pointwise_weights(const nncase_hip_weights *w) {
+static bool pointwise_weights(const nncase_hip_weights *w) {
     return w && w->kind == nncase_hip_weights::kIgemm && w->groups == 1 && w->kernel_h == 1 && w->kernel_w == 1;
 }
 
-} // namespace
+} // namespace nnhip
 
 extern "C" int nncase_hip_qpointwise_pair_supported(int32_t in_channels, int32_t mid_channels, int32_t out_channels) {
     return pair_shapes_ok(in_channels, mid_channels, out_channels) ? 1 : 0;
@@ -386,6 +446,104 @@ extern "C" int nncase_hip_qpointwise_pair_destroy(nncase_hip_ctx_t *ctx, nncase_
     free_pair(pair);
     return 0;
 }
+
+// ---- the few-pixel path of one dense 1x1 convolution ----------------------------------------------------------------
+namespace nnhip {
+constexpr int kRowsMaxK = 2048;                 // reduction length (an LDS row: 16 of them stay below 64 KiB)
+constexpr int64_t kRowsStreamLimit = 4 << 20;   // weight bytes all pixel tiles stream between them
+constexpr int64_t kRowsMaxPixels = 32;          // beyond two pixel tiles the tiled kernels, which share the weights of a tile
+                                                // among many pixels, are the faster ones (measured on MobileNetV2's 7x7 layers)
+
+bool rows_shapes_ok(int in_channels, int out_channels, int64_t pixels) {
+    return pixels > 0 && pixels <= kRowsMaxPixels && in_channels % 16 == 0 && out_channels % 4 == 0 && in_channels <= kRowsMaxK &&
+           (pixels + 15) / 16 * (int64_t)in_channels * out_channels <= kRowsStreamLimit;
+}
+
+// Every workgroup of the pooled launch pools its (up to 16) rows itself, on one compute unit: beyond this many values
+// per workgroup the separate pool kernel, which spreads over the device, is the faster one.
+bool pool_front_pays(int rows, int hw, int channels) { return (int64_t)std::min(rows, 16) * hw * channels <= (128 << 10); }
+
+int rows_prepack(nncase_hip_ctx *ctx, nncase_hip_weights *w, const uint8_t *w_oihw) {
+    if (!(pointwise_weights(w) && rows_shapes_ok(w->in_channels, w->out_channels, w->pixels_hint))) return 0; // not a call this path is for
+    nncase_hip_qpair *pr = new (std::nothrow) nncase_hip_qpair();
+    NNHIP_REQUIRE(ctx, pr, -ENOMEM, "qconv2d_prepack: out of host memory");
+    pr->second = w;
+    pr->n1 = w->in_channels, pr->n2 = w->out_channels;
+    pr->ks2 = (pr->n1 + 63) / 64, pr->t2 = (pr->n2 + 15) / 16;
+    std::vector<uint8_t> packed;
+    std::vector<int32_t> wsum, bias((size_t)pr->t2 * 16, 0);
+    pack_pair_weights(packed, wsum, w_oihw, pr->n2, pr->n1, pr->t2, pr->ks2);
+    const hipError_t got = hipMemcpy(bias.data(), w->d_bias, sizeof(int32_t) * pr->n2, hipMemcpyDeviceToHost);
+    int rc = got == hipSuccess ? 0 : hip_fail(ctx, got, "hipMemcpy(bias)");
+    if (!rc) rc = upload(ctx, (void **)&pr->d_wb, packed.data(), packed.size());
+    if (!rc) rc = upload(ctx, (void **)&pr->d_wsum_b, wsum.data(), wsum.size() * sizeof(int32_t));
+    if (!rc) rc = upload(ctx, (void **)&pr->d_bias_b, bias.data(), bias.size() * sizeof(int32_t));
+    if (rc) { // (the failing call has left its message)
+        free_pair(pr);
+        return rc;
+    }
+    w->rows_pack = pr;
+    return 0;
+}
+
+void rows_free(nncase_hip_weights *w) {
+    if (w && w->rows_pack) free_pair(w->rows_pack);
+    if (w) w->rows_pack = nullptr;
+}
+
+bool rows_path_taken(const nncase_hip_weights *w, const nncase_hip_conv2d_args_t *c, int out_h, int out_w) {
+    if (!w->rows_pack || c->residual_dev || c->out_channel_stride || c->out_channel_offset) return false;
+    if (!(c->stride_h == 1 && c->stride_w == 1 && c->pad_h_before == 0 && c->pad_w_before == 0 && out_h == c->in_h && out_w == c->in_w)) return false;
+    // (u8 codes, or their float32 values: the entry point turns the latter into a u8 call with the flag set)
+    if (!(c->out_dtype == NNCASE_HIP_DT_U8 || (c->out_dtype == NNCASE_HIP_DT_F32 && c->dequantize_output != 0))) return false;
+    return rows_shapes_ok(w->in_channels, w->out_channels, (int64_t)c->batch * out_h * out_w);
+}
+
+int launch_qconv_rows(nncase_hip_ctx *ctx, const uint8_t *x, const nncase_hip_weights *w, void *y, const nncase_hip_conv2d_args_t *c,
+                      const PoolFront *pool) {
+    const nncase_hip_qpair *pr = w->rows_pack;
+    const int64_t m64 = (int64_t)c->batch * c->in_h * c->in_w;
+    NNHIP_REQUIRE(ctx, m64 > 0 && m64 < ((int64_t)1 << 30), -EINVAL, "qconv2d: %lld output pixels unsupported", (long long)m64);
+    NNHIP_REQUIRE(ctx, (reinterpret_cast<uintptr_t>(x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(y) & 15u) == 0,
+                  -NNCASE_HIP_ERR_INVALID_MEMORY_LOCATION, "qconv2d: activation buffers must be 16-byte aligned");
+    PairArgs a;
+    memset(&a, 0, sizeof(a));
+    a.x = x, a.y2 = reinterpret_cast<uint8_t *>(y);
+    a.wb = pr->d_wb, a.bias_b = pr->d_bias_b, a.wsum_b = pr->d_wsum_b;
+    a.lut_b = w->d_post_lut;
+    a.m = (int)m64;
+    a.n1 = pr->n1, a.n2 = pr->n2, a.ks2 = pr->ks2, a.t2 = pr->t2;
+    a.zxb = c->x_qp.zero_point - 128, a.zwb = w->zw - 128;
+    const int rc = make_epilogue(ctx, &a.ep_b, c->x_qp.scale, w->sw, c->y_qp, c->clamp_min, c->clamp_max, NNCASE_HIP_DT_U8, "qconv2d");
+    if (rc) return rc;
+    if (c->dequantize_output != 0) {
+        const nncase_hip_quant_param_t last = w->d_post_lut ? w->post_lut_qp : c->y_qp;
+        a.deq = 1, a.deq_zero = last.zero_point, a.deq_scale = last.scale;
+    }
+    if (pool) {
+        NNHIP_REQUIRE(ctx, pool->hw > 0 && (int64_t)m64 * pool->hw * pr->n1 < ((int64_t)1 << 31), -EINVAL, "qglobal_avgpool_qconv2d: input too large");
+        a.pool_hw = pool->hw;
+        a.pool_zx = (float)pool->x_qp.zero_point, a.pool_sx = pool->x_qp.scale;
+        a.pool_zy = (float)c->x_qp.zero_point, a.pool_sy = c->x_qp.scale;
+    }
+    // pixel tiles x ranges of channel tiles, a wave per tile, enough workgroups to spread the weights over the device
+    const int ptiles = (a.m + 15) / 16;
+    int ranges = (a.t2 + kRowsWaves - 1) / kRowsWaves;
+    const int want = std::max(1, 2 * ctx->compute_units / ptiles);
+    int per = std::max(1, (a.t2 + want - 1) / want); // tiles per workgroup when as many workgroups as wanted
+    if (pool) per = std::max(per, 4);                 // (every workgroup repeats the pooling)
+    ranges = (a.t2 + per - 1) / per;
+    a.tiles_per_block = per;
+    int waves = std::min(kRowsWaves, per);
+    if (pool) waves = kRowsWaves; // the pooling has a thread per four channels
+    const size_t lds = 16 * (size_t)pair_row_bytes(a.ks2, kRowsChunk) + 256;
+    NNHIP_HIP(ctx, hipSetDevice(ctx->device));
+    if (pool) hipLaunchKernelGGL(qpointwise_rows_kernel<true>, dim3(ptiles, ranges), dim3(waves * 64), lds, ctx->stream, a);
+    else hipLaunchKernelGGL(qpointwise_rows_kernel<false>, dim3(ptiles, ranges), dim3(waves * 64), lds, ctx->stream, a);
+    NNHIP_LAUNCH_CHECK(ctx, "qpointwise_rows_kernel");
+    return 0;
+}
+} // namespace nnhip
 
 // dw / da: the depthwise convolution in front and its arguments, or null
 static int launch_pair(nncase_hip_ctx *ctx, const char *who, const uint8_t *x_dev, const nncase_hip_weights *dw,

@@ -222,27 +222,7 @@ __global__ __launch_bounds__(kEwThreads) void qglobal_avgpool4_kernel(const uint
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= batch * cq) return;
     const int n = idx / cq, c = (idx - n * cq) * 4;
-    const uint8_t *p = x + (size_t)n * hw * channels + c;
-    float value[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int i0 = 0; i0 < hw; i0 += 64) {
-        uint32_t d[64];
-#pragma unroll
-        for (int k = 0; k < 64; k++) d[k] = *reinterpret_cast<const uint32_t *>(p + (size_t)min(i0 + k, hw - 1) * channels);
-#pragma unroll
-        for (int k = 0; k < 64; k++)
-            if (i0 + k < hw) {
-#pragma unroll
-                for (int e = 0; e < 4; e++) value[e] = value[e] + ((float)((d[k] >> (8 * e)) & 0xffu) - zx) * sx;
-            }
-    }
-    uint32_t q = 0;
-#pragma unroll
-    for (int e = 0; e < 4; e++) {
-        const float mean = value[e] / (float)hw;
-        float t = mean / sy + zy;
-        t = fminf(fmaxf(t, 0.f), 255.f);
-        q |= (uint32_t)(int32_t)rintf(t) << (8 * e);
-    }
+    const uint32_t q = global_avgpool4(x + (size_t)n * hw * channels + c, hw, channels, zx, sx, zy, sy);
     *reinterpret_cast<uint32_t *>(out + (size_t)n * channels + c) = q;
 }
 

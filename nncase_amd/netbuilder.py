@@ -640,6 +640,28 @@ class HipModel:
                 self.weights[-1] = wt
         for a_, b_ in self.pairs.items():
             self.pair_objects[a_] = ctx.prepack_qpointwise_pair(self.weights[a_], qg.nodes[a_].weights, self.weights[b_], qg.nodes[b_].weights)
+        # A global average pool that only a dense 1x1 convolution reads (a classifier's tail) is computed by that
+        # convolution's launch where the library says it pays: a few rows only.
+        self.pool_fronts: Dict[int, int] = {}                                            # conv -> gap node
+        if fuse_pairs and fuse_residual:
+            for i, n in enumerate(qg.nodes):
+                readers = [j for j in range(i + 1, len(qg.nodes)) if i in qg.nodes[j].inputs]
+                if n.op != "gap" or len(readers) != 1 or i in qg.output_nodes:
+                    continue
+                j = readers[0]
+                cn = qg.nodes[j]
+                if not (cn.op == "conv" and cn.groups == 1 and cn.weights.shape[2:] == (1, 1) and tuple(cn.stride) == (1, 1)
+                        and tuple(map(tuple, cn.padding)) == ((0, 0), (0, 0)) and j not in block_members and j not in self.write_through
+                        and j not in self.fused_into and j not in self.pairs and j not in self.pairs.values() and self.weights[j] is not None):
+                    continue
+                probe = rt.Conv2dArgs(bl, 1, 1, 1, 1, 1, 1, 0, 0, 0, 0, qp(*n.out_qp), qp(*cn.out_qp), cn.clamp[0], cn.clamp[1], rt.DT_U8)
+                if j in self.fused_dequant:
+                    probe.out_dtype, probe.dequantize_output = rt.DT_F32, 1
+                src = qg.nodes[n.inputs[0]]
+                if ctx.qglobal_avgpool_qconv2d_supported(self.weights[j], probe, src.out_shape[1], src.out_shape[2]):
+                    self.pool_fronts[j] = i
+                    self.never_written.add(i)
+                    skip_nodes.add(i)
         self.outputs_f32: List[rt.DeviceBuffer] = [ctx.alloc(lanes * self._lane_stride(bl * int(np.prod(qg.nodes[j].out_shape)) * 4))
                                                     for j in qg.output_nodes]
         for lane in range(lanes):
@@ -740,6 +762,16 @@ class HipModel:
                                              + ("+add" if fused_add is not None else "") + f">{sn.name}" + ("+lut" if lut2 is not None else ""))
                         self.op_nodes.append(lut2 if lut2 is not None else j)
                         self.op_members.append(members + [j] + ([lut2] if lut2 is not None else []))
+                    continue
+                if i in self.pool_fronts:
+                    g_ = self.pool_fronts[i]
+                    gsrc = qg.nodes[qg.nodes[g_].inputs[0]]
+                    self.fn.add_qglobal_avgpool_qconv2d(B(qg.nodes[g_].inputs[0]), gsrc.out_shape[1], gsrc.out_shape[2], qp(*gsrc.out_qp),
+                                                        self.weights[i], buf, args)
+                    if lane == 0:
+                        self.op_names.append(f"gap:{qg.nodes[g_].name}>conv:{n.name}" + ("+lut" if fused_lut is not None else ""))
+                        self.op_nodes.append(fused_lut if fused_lut is not None else i)
+                        self.op_members.append([g_] + members)
                     continue
                 self.fn.add_qconv2d(B(n.inputs[0]), self.weights[i], buf, args)
             elif n.op == "add":

@@ -121,6 +121,9 @@ SYMBOLS = {
     "nncase_hip_qpointwise_pair_destroy": (_I, [_VP, _VP]),
     "nncase_hip_qpointwise_pair": (_I, [_VP, _VP, _VP, _VP, _VP, C.POINTER(Conv2dArgs), C.POINTER(Conv2dArgs)]),
     "nncase_hip_function_add_qpointwise_pair": (_I, [_VP, _VP, _VP, _VP, _VP, C.POINTER(Conv2dArgs), C.POINTER(Conv2dArgs)]),
+    "nncase_hip_qglobal_avgpool_qconv2d_supported": (_I, [_VP, C.POINTER(Conv2dArgs), C.c_int32, C.c_int32]),
+    "nncase_hip_qglobal_avgpool_qconv2d": (_I, [_VP, _VP, C.c_int32, C.c_int32, QuantParam, _VP, _VP, C.POINTER(Conv2dArgs)]),
+    "nncase_hip_function_add_qglobal_avgpool_qconv2d": (_I, [_VP, _VP, C.c_int32, C.c_int32, QuantParam, _VP, _VP, C.POINTER(Conv2dArgs)]),
     "nncase_hip_qdepthwise_pointwise_pair": (_I, [_VP, _VP, _VP, C.POINTER(Conv2dArgs), _VP, _VP, _VP, C.POINTER(Conv2dArgs), C.POINTER(Conv2dArgs)]),
     "nncase_hip_function_add_qdepthwise_pointwise_pair": (_I, [_VP, _VP, _VP, C.POINTER(Conv2dArgs), _VP, _VP, _VP, C.POINTER(Conv2dArgs),
                                                            C.POINTER(Conv2dArgs)]),
@@ -567,6 +570,14 @@ class Context:
         self._check(self.lib.nncase_hip_qpointwise_pair(self.handle, x.ptr, pair.handle, y1.ptr, y2.ptr, C.byref(first_args),
                                                         C.byref(second_args)), "qpointwise_pair")
 
+    def qglobal_avgpool_qconv2d_supported(self, w: Weights, args: Conv2dArgs, h: int, w_: int) -> bool:
+        return bool(self.lib.nncase_hip_qglobal_avgpool_qconv2d_supported(w.handle, C.byref(args), h, w_))
+
+    def qglobal_avgpool_qconv2d(self, x, h: int, w_: int, x_qp: QuantParam, w: Weights, y, args: Conv2dArgs):
+        """Global average pool of x [batch, h, w, channels] and the 1x1 convolution on the pooled pixel, one launch."""
+        self._check(self.lib.nncase_hip_qglobal_avgpool_qconv2d(self.handle, x.ptr, h, w_, x_qp, w.handle, y.ptr, C.byref(args)),
+                    "qglobal_avgpool_qconv2d")
+
     def qdepthwise_pointwise_pair(self, x, dw: Weights, dw_args: Conv2dArgs, pair: QPair, y1, y2, first_args: Conv2dArgs,
                                   second_args: Conv2dArgs):
         """x is the 3x3 depthwise convolution's input; its result only exists inside the launch."""
@@ -728,6 +739,11 @@ class Function:
         self._keep += [x, pair, y1, y2]
         self._ck(self.ctx.lib.nncase_hip_function_add_qpointwise_pair(self.handle, x.ptr, pair.handle, y1.ptr, y2.ptr, C.byref(first_args),
                                                                       C.byref(second_args)), "function_add_qpointwise_pair")
+
+    def add_qglobal_avgpool_qconv2d(self, x, h: int, w_: int, x_qp: QuantParam, w: Weights, y, args: Conv2dArgs):
+        self._keep += [x, w, y]
+        self._ck(self.ctx.lib.nncase_hip_function_add_qglobal_avgpool_qconv2d(self.handle, x.ptr, h, w_, x_qp, w.handle, y.ptr, C.byref(args)),
+                 "function_add_qglobal_avgpool_qconv2d")
 
     def add_qdepthwise_pointwise_pair(self, x, dw: Weights, dw_args: Conv2dArgs, pair: QPair, y1, y2, first_args: Conv2dArgs,
                                       second_args: Conv2dArgs):

@@ -76,14 +76,14 @@ def test_mobilenetv2_config3(hip_ctx):
     assert len(model.fused_into) == 10 and len(model.fused_dequant) == 1 and len(model.fn) == 55   # residual adds folded into
     #                                                                            the convs, the output's dequantize into the classifier
     model, y, outs = check_model(hip_ctx, qg, x, capture=True, fuse_blocks=False, fuse_pairs="all")
-    assert len(model.pairs) == 17 and len(model.pair_fronts) == 17 and len(model.fn) == 21   # every depthwise convolution and projection runs
-    #                                                                                          with the expansion behind them as one launch
+    assert len(model.pairs) == 17 and len(model.pair_fronts) == 17 and len(model.pool_fronts) == 1 and len(model.fn) == 20   # every depthwise convolution and projection runs
+    #                                                                      with the expansion behind them as one launch, the classifier with its pool
     model, y, outs = check_model(hip_ctx, qg, x, capture=True, fuse_blocks=False, fuse_pairs="nofront")
     assert 0 < len(model.pairs) < 17 and not model.pair_fronts
     model, y, outs = check_model(hip_ctx, qg, x, capture=True, fuse_blocks=False)
     assert 0 < len(model.pairs) < 17                           # ... at this batch, where the pair streams few weights
     model, y, outs = check_model(hip_ctx, qg, x, capture=True)
-    assert len(model.blocks) == 16 and len(model.fn) == 23                            # ... and whole blocks into one operator
+    assert len(model.blocks) == 16 and len(model.pool_fronts) == 1 and len(model.fn) == 22   # ... and whole blocks into one operator
     # the reference's own acceptance bar for a PTQ model: cosine >= 0.98 against the float model
     fl = nb.float_forward(g, x)[-1]
     assert O.cosine(y, fl) > 0.98

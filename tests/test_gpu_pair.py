@@ -245,3 +245,108 @@ def test_pair_argument_checks(hip_ctx):
     withres.residual_qp, withres.sum_qp = qp(0, 0.02), qp(0, 0.02)
     with pytest.raises(rt.HipError):
         hip_ctx.qpointwise_pair(xd, pair, y1d, y2d, good, withres)
+
+
+# ---- the few-pixel path of one dense 1x1 convolution (weights in registers), alone and behind a global average pool ----
+ROWS = [  # (rows, in, out, table, dequantised): m of a classifier head, channel counts that fill no tile / k-step, several pixel tiles
+    (1, 1280, 1000, False, True), (2, 64, 4, False, False), (16, 16, 36, True, False), (17, 80, 200, False, False),
+    (5, 2048, 24, True, True), (32, 272, 132, False, True), (3, 1024, 1024, False, False),
+]
+
+
+@pytest.mark.parametrize("m,k,n,lut,deq", ROWS)
+def test_rows_path_of_qconv2d(hip_ctx, m, k, n, lut, deq):
+    rng = np.random.default_rng(m * 31 + k + n)
+    x = rng.integers(0, 256, (m, k, 1, 1), dtype=np.uint8)
+    w = rng.integers(0, 256, (n, k, 1, 1), dtype=np.uint8)
+    b = rng.integers(-3000, 3000, n).astype(np.int32)
+    zx, sx, zw, sw = 9, f32(0.0235), 131, f32(0.0041)
+    real = O.qconv2d(x, w, b, zx, sx, zw, sw, out_mode=O.OUT_F32)
+    c, zy, sy = pick_quant(real)
+    want = O.qconv2d(x, w, b, zx, sx, zw, sw, zy, sy, fused_clamp=c, out_mode=O.OUT_U8)
+    zl, sl = zy, sy
+    wt = hip_ctx.prepack_conv2d(w, b, qp(zw, sw), expected_pixels=m)
+    if lut:
+        table = rng.permutation(256).astype(np.uint8)
+        want = table[want]
+        zl, sl = 23, f32(sy * 1.5)
+        wt.set_post_lut(table, qp(zl, sl))
+    a = conv_args(m, 1, 1, qp(zx, sx), qp(zy, sy), c)
+    if deq:
+        a.out_dtype, a.dequantize_output = rt.DT_F32, 1
+        want = ((want.astype(np.int32) - zl).astype(f32) * sl).astype(f32)
+    fn = rt.Function(hip_ctx)
+    xd = hip_ctx.alloc(x.size).upload(np.ascontiguousarray(x.reshape(m, k)))
+    yd = hip_ctx.alloc(m * n * (4 if deq else 1)).fill(0xA5)
+    fn.add_qconv2d(xd, wt, yd, a)
+    assert fn.op_kernel(0).startswith("qpointwise_rows")          # the path under test is the one taken
+    for _ in range(2):
+        hip_ctx.qconv2d(xd, wt, yd, a)
+        hip_ctx.sync()
+        got = yd.download((m, n), f32 if deq else np.uint8)
+        assert np.array_equal(got.view(np.uint32) if deq else got, want.reshape(m, n).view(np.uint32) if deq else want.reshape(m, n))
+        yd.fill(0x5A)
+    # the same weights packed for many pixels take the tiled kernels: same bytes
+    big = hip_ctx.prepack_conv2d(w, b, qp(zw, sw), expected_pixels=1 << 20)
+    if lut:
+        big.set_post_lut(table, qp(zl, sl))
+    fn2 = rt.Function(hip_ctx)
+    fn2.add_qconv2d(xd, big, yd, a)
+    assert not fn2.op_kernel(0).startswith("qpointwise_rows")
+    hip_ctx.qconv2d(xd, big, yd, a)
+    hip_ctx.sync()
+    got = yd.download((m, n), f32 if deq else np.uint8)
+    assert np.array_equal(got.view(np.uint32) if deq else got, want.reshape(m, n).view(np.uint32) if deq else want.reshape(m, n))
+
+
+POOLED = [  # (batch, h, w, channels, out, dequantised)
+    (1, 7, 7, 1280, 1000, True), (2, 7, 7, 320, 36, False), (3, 1, 1, 64, 20, False), (1, 10, 9, 96, 132, True), (5, 3, 3, 48, 8, False),
+]
+
+
+@pytest.mark.parametrize("n,h,w,c,oc,deq", POOLED)
+def test_global_average_pool_in_front_of_a_convolution(hip_ctx, n, h, w, c, oc, deq):
+    rng = np.random.default_rng(n + h * w + c + oc)
+    x = rng.integers(0, 256, (n, c, h, w), dtype=np.uint8)
+    wt_ = rng.integers(0, 256, (oc, c, 1, 1), dtype=np.uint8)
+    b = rng.integers(-3000, 3000, oc).astype(np.int32)
+    zx, sx, zw, sw = 9, f32(0.0235), 131, f32(0.0041)
+    zp, sp = 13, f32(0.011)                                # the pooled tensor's quantisation
+    pooled = O.qglobal_avgpool(x, zx, sx, zp, sp).reshape(n, c, 1, 1)
+    assert len(np.unique(pooled)) > 4
+    real = O.qconv2d(pooled, wt_, b, zp, sp, zw, sw, out_mode=O.OUT_F32)
+    cl, zy, sy = pick_quant(real)
+    want = O.qconv2d(pooled, wt_, b, zp, sp, zw, sw, zy, sy, fused_clamp=cl, out_mode=O.OUT_U8)
+    wt = hip_ctx.prepack_conv2d(wt_, b, qp(zw, sw), expected_pixels=n)
+    a = conv_args(n, 1, 1, qp(zp, sp), qp(zy, sy), cl)
+    if deq:
+        a.out_dtype, a.dequantize_output = rt.DT_F32, 1
+        want = ((want.astype(np.int32) - zy).astype(f32) * sy).astype(f32)
+    assert hip_ctx.qglobal_avgpool_qconv2d_supported(wt, a, h, w)
+    xd = hip_ctx.alloc(x.size).upload(np.ascontiguousarray(x.transpose(0, 2, 3, 1)))
+    yd = hip_ctx.alloc(n * oc * (4 if deq else 1)).fill(0xA5)
+    fn = rt.Function(hip_ctx)
+    fn.add_qglobal_avgpool_qconv2d(xd, h, w, qp(zx, sx), wt, yd, a)
+    fn.capture()
+    for _ in range(2):
+        fn.invoke()
+        hip_ctx.sync()
+        got = yd.download((n, oc), f32 if deq else np.uint8)
+        assert np.array_equal(got.view(np.uint32) if deq else got, want.reshape(n, oc).view(np.uint32) if deq else want.reshape(n, oc))
+        yd.fill(0x5A)
+    # the two operators one after the other on the device
+    pd = hip_ctx.alloc(n * c).fill(0)
+    hip_ctx.qglobal_avgpool(xd, pd, n, h, w, c, qp(zx, sx), qp(zp, sp))
+    hip_ctx.qconv2d(pd, wt, yd, a)
+    hip_ctx.sync()
+    got = yd.download((n, oc), f32 if deq else np.uint8)
+    assert np.array_equal(got.view(np.uint32) if deq else got, want.reshape(n, oc).view(np.uint32) if deq else want.reshape(n, oc))
+    # refused: weights packed for many pixels, a convolution that is not on the pooled pixel, a pool too large for one workgroup
+    big = hip_ctx.prepack_conv2d(wt_, b, qp(zw, sw), expected_pixels=1 << 20)
+    assert not hip_ctx.qglobal_avgpool_qconv2d_supported(big, a, h, w)
+    with pytest.raises(rt.HipError):
+        hip_ctx.qglobal_avgpool_qconv2d(xd, h, w, qp(zx, sx), big, yd, a)
+    assert not hip_ctx.qglobal_avgpool_qconv2d_supported(wt, a, 512, 512)
+    bad = conv_args(n, 2, 1, qp(zp, sp), qp(zy, sy), cl)
+    with pytest.raises(rt.HipError):
+        hip_ctx.qglobal_avgpool_qconv2d(xd, h, w, qp(zx, sx), wt, yd, bad)
