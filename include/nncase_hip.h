@@ -694,8 +694,12 @@ NNCASE_HIP_API int nncase_hip_function_add_add_i32(nncase_hip_function_t *fn, in
  * lane run in the order recorded; different lanes must not touch each other's tensors.  A captured function
  * runs its lanes concurrently (e.g. the two halves of a batch, whose small layers cannot fill the device
  * alone); eager invocation runs all operators in the order recorded.  Paged attention and other operators
- * that use the context's scratch memory must stay in one lane. */
+ * that use the context's scratch memory must stay in one lane.
+ * NNCASE_HIP_LANE_JOINED: operators recorded after set_lane(fn, NNCASE_HIP_LANE_JOINED) wait for every lane and run as
+ * one chain behind them (a step that ends in one product over the whole batch, whose weights the lanes would
+ * otherwise each read); they have to be the last ones recorded. */
 #define NNCASE_HIP_MAX_LANES 8
+#define NNCASE_HIP_LANE_JOINED (-1)
 NNCASE_HIP_API int nncase_hip_function_set_lane(nncase_hip_function_t *fn, int32_t lane);
 /* Number of operators recorded so far. */
 NNCASE_HIP_API int nncase_hip_function_size(nncase_hip_function_t *fn, int32_t *count);

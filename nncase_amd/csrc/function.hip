@@ -143,6 +143,9 @@ static void drop_graph(nncase_hip_function *fn) {
 }
 
 static int push(nncase_hip_function *fn, const Op &op) {
+    // (eager invocation runs the list in order: what waits for every lane has to come last)
+    NNHIP_REQUIRE(fn->ctx, fn->cur_lane == NNCASE_HIP_LANE_JOINED || fn->ops.empty() || fn->ops.back().lane != NNCASE_HIP_LANE_JOINED, -EINVAL,
+                  "function: operators behind the join of the lanes must be recorded last");
     drop_graph(fn); // a captured graph no longer matches the list
     fn->ops.push_back(op);
     fn->ops.back().lane = fn->cur_lane;
@@ -151,8 +154,8 @@ static int push(nncase_hip_function *fn, const Op &op) {
 
 extern "C" int nncase_hip_function_set_lane(nncase_hip_function_t *fn, int32_t lane) {
     if (!fn) return -EINVAL;
-    NNHIP_REQUIRE(fn->ctx, lane >= 0 && lane < NNCASE_HIP_MAX_LANES, -EINVAL, "function_set_lane: lane %d (0..%d)", lane,
-                  NNCASE_HIP_MAX_LANES - 1);
+    NNHIP_REQUIRE(fn->ctx, lane == NNCASE_HIP_LANE_JOINED || (lane >= 0 && lane < NNCASE_HIP_MAX_LANES), -EINVAL,
+                  "function_set_lane: lane %d (0..%d, or NNCASE_HIP_LANE_JOINED)", lane, NNCASE_HIP_MAX_LANES - 1);
     fn->cur_lane = lane;
     if (lane + 1 > fn->nlanes) fn->nlanes = lane + 1;
     return 0;
@@ -454,7 +457,7 @@ extern "C" int nncase_hip_function_add_paged_attention_decode(nncase_hip_functio
     // the workspace the kernel's splits go through is sized now: capture must not allocate, and a graph
     // keeps the addresses it was captured with
     const int lane = fn->cur_lane;
-    if (lane == 0) {
+    if (lane <= 0) { // (lane 0, and behind the join, where lane 0 has finished: the context's scratch)
         const int rc = attn_reserve(fn->ctx, args);
         if (rc) return rc;
     } else {
@@ -551,7 +554,7 @@ extern "C" int nncase_hip_function_capture(nncase_hip_function_t *fn) {
     // other lanes bring areas of their own)
     int attn_lane = -1;
     for (const Op &op : fn->ops)
-        if (op.kind == Op::kAttn && op.lane == 0) attn_lane = 0;
+        if (op.kind == Op::kAttn && op.lane <= 0) attn_lane = 0;
     // Operators of different lanes are recorded on streams of their own, forked from and joined back into
     // the context's stream, so the graph holds one independent chain per lane and the device overlaps them.
     hipStream_t main_stream = ctx->stream;
@@ -586,6 +589,7 @@ extern "C" int nncase_hip_function_capture(nncase_hip_function_t *fn) {
     }
     if (se == hipSuccess) {
         for (const Op &op : fn->ops) {
+            if (op.lane == NNCASE_HIP_LANE_JOINED) continue;
             ctx->stream = op.lane == 0 ? main_stream : side[op.lane];
             rc = run_op(fn, op);
             if (rc) break;
@@ -594,6 +598,11 @@ extern "C" int nncase_hip_function_capture(nncase_hip_function_t *fn) {
         for (int l = 1; l < fn->nlanes && se == hipSuccess; l++) {
             se = hipEventRecord(join[l], side[l]);
             if (se == hipSuccess) se = hipStreamWaitEvent(main_stream, join[l], 0);
+        }
+        // what was recorded behind the join: on the context's stream, after every lane
+        for (const Op &op : fn->ops) {
+            if (rc || se != hipSuccess) break;
+            if (op.lane == NNCASE_HIP_LANE_JOINED) rc = run_op(fn, op);
         }
     }
     hipGraph_t graph = nullptr;

@@ -151,13 +151,23 @@ class HipDecoder:
                     fn.add_rmsnorm_f16(h, L["ln2"], norm, bl, c.hidden, c.rms_eps)
                     fn.add_w8a16_gemm(norm, L["gate_up"], act, bl, mode=rt.GEMM_SWIGLU)
                 fn.add_w8a16_gemm(act, L["down"], x, bl, residual=h)
-            if fuse_norm:
-                fn.add_rmsnorm_w8a16_gemm(xs[0], self.ln_f, c.rms_eps, self.lm_head, logits, bl, out_dtype=rt.DT_F32)
+            if lanes > 1 and lane + 1 < lanes:
+                continue
+            # The vocabulary head reads its 136 MB of weights once for however many rows: behind the join of the lanes it
+            # runs once over the whole batch (as do the two small operators after it), not once per lane.
+            if lanes > 1:
+                fn.set_lane(Function.LANE_JOINED)
+                tokens, next_tokens, ctx_lens, norm, logits, bl_ = self.tokens, self.next_tokens, self.ctx_lens, self.norm, self.logits, batch
+                xs = [self.x[0], self.x[1]]
             else:
-                fn.add_rmsnorm_f16(xs[0], self.ln_f, norm, bl, c.hidden, c.rms_eps)
-                fn.add_w8a16_gemm(norm, self.lm_head, logits, bl, out_dtype=rt.DT_F32)
-            fn.add_argmax_f32(logits, tokens if feedback else next_tokens, bl, c.vocab)
-            fn.add_add_i32(ctx_lens, bl, 1)   # the step is complete: the caches hold one more token
+                bl_ = bl
+            if fuse_norm:
+                fn.add_rmsnorm_w8a16_gemm(xs[0], self.ln_f, c.rms_eps, self.lm_head, logits, bl_, out_dtype=rt.DT_F32)
+            else:
+                fn.add_rmsnorm_f16(xs[0], self.ln_f, norm, bl_, c.hidden, c.rms_eps)
+                fn.add_w8a16_gemm(norm, self.lm_head, logits, bl_, out_dtype=rt.DT_F32)
+            fn.add_argmax_f32(logits, tokens if feedback else next_tokens, bl_, c.vocab)
+            fn.add_add_i32(ctx_lens, bl_, 1)   # the step is complete: the caches hold one more token
         self.fn = fn
         # nothing to warm up: recording the attention operators has already sized their workspace
         if capture_graph:

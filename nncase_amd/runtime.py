@@ -856,6 +856,8 @@ class Function:
         self._ck(self.ctx.lib.nncase_hip_function_add_layout(self.handle, src.ptr, dst.ptr, elem_size, n, c, h, w, int(to_nchw)),
                  "function_add_layout")
 
+    LANE_JOINED = -1   # set_lane(LANE_JOINED): what follows waits for every lane (recorded last)
+
     def set_lane(self, lane: int):
         """Operators added from now on form independent chain `lane`; a captured function overlaps its lanes."""
         self._ck(self.ctx.lib.nncase_hip_function_set_lane(self.handle, lane), "function_set_lane")

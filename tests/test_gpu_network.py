@@ -347,7 +347,27 @@ def test_lanes_argument_checks(hip_ctx):
     with pytest.raises(HipError):
         fn.set_lane(8)
     with pytest.raises(HipError):
-        fn.set_lane(-1)
+        fn.set_lane(-2)
+    # what is recorded behind the join of the lanes runs after all of them, and has to be recorded last
+    a, b, c = (hip_ctx.alloc(64) for _ in range(3))
+    a.upload(np.arange(64, dtype=np.uint8))
+    table = ((np.arange(256) + 3) % 256).astype(np.uint8)
+    fn.set_lane(0)
+    fn.add_lut_u8(a.view(0, 32), b.view(0, 32), 32, table)
+    fn.set_lane(1)
+    fn.add_lut_u8(a.view(32, 32), b.view(32, 32), 32, table)
+    fn.set_lane(Function.LANE_JOINED)
+    fn.add_lut_u8(b, c, 64, table)
+    fn.set_lane(1)
+    with pytest.raises(HipError):
+        fn.add_lut_u8(a, b, 64, table)
+    for capture in (False, True):
+        if capture:
+            fn.capture()
+        c.fill(0)
+        fn.invoke()
+        hip_ctx.sync()
+        assert np.array_equal(c.download((64,), np.uint8), (np.arange(64) + 6).astype(np.uint8))
 
 
 def test_mobilenetv2_fused_blocks_match_separate_operators(hip_ctx):
