@@ -14,6 +14,9 @@
 // Weights are re-packed for this kernel: [channel tile][k-step][64 lanes][16 bytes], lane (i, g) holding
 // w[16 t + i][64 ks + 16 g ..] - 128 as s8 (zero past the real extents), so that one 16-byte load per lane is an MFMA
 // operand and lane (j, g) of the result holds channels 16 t + 4 g .. + 3 of pixel j: four neighbours, one dword.
+//
+// The second stage alone is the few-pixel path of nncase_hip_qconv2d (qpointwise_rows_kernel, further down): one dense
+// 1x1 convolution over at most 32 pixels, optionally behind a global average pool computed by the same launch.
 #include "qconv.hpp"
 
 #include <new>
