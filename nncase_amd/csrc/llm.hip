@@ -621,28 +621,41 @@ __device__ __forceinline__ void argmax_take(float v, int i, float &best, int &bi
     if (v > best || (v == best && i < bi)) best = v, bi = i;
 }
 __global__ __launch_bounds__(kArgmaxThreads) void argmax_f32_kernel(const float *__restrict__ x, int32_t *__restrict__ out, int cols) {
-    __shared__ float sv[kArgmaxThreads];
-    __shared__ int si[kArgmaxThreads];
+    __shared__ float sv[kArgmaxThreads / 64];
+    __shared__ int si[kArgmaxThreads / 64];
     const float *row = x + (size_t)blockIdx.x * cols;
     float best = -INFINITY;
     int bi = 0x7fffffff;
     // rows start 16-byte aligned when cols is a multiple of 4 (x itself is aligned by the allocator)
     const int nvec = ((cols & 3) == 0 && (reinterpret_cast<uintptr_t>(x) & 15u) == 0) ? cols / 4 : 0;
-    for (int i = threadIdx.x; i < nvec; i += kArgmaxThreads) {
-        const float4 v = reinterpret_cast<const float4 *>(row)[i];
-        argmax_take(v.x, 4 * i, best, bi);
-        argmax_take(v.y, 4 * i + 1, best, bi);
-        argmax_take(v.z, 4 * i + 2, best, bi);
-        argmax_take(v.w, 4 * i + 3, best, bi);
+    // eight 16-byte loads per thread are requested before any of them is compared: a row of the vocabulary is five
+    // memory round trips, not one per load
+    constexpr int U = 8;
+    for (int i0 = threadIdx.x; i0 < nvec; i0 += U * kArgmaxThreads) {
+        float4 v[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) v[u] = reinterpret_cast<const float4 *>(row)[min(i0 + u * kArgmaxThreads, nvec - 1)];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int i = i0 + u * kArgmaxThreads;
+            if (i < nvec) {
+                argmax_take(v[u].x, 4 * i, best, bi);
+                argmax_take(v[u].y, 4 * i + 1, best, bi);
+                argmax_take(v[u].z, 4 * i + 2, best, bi);
+                argmax_take(v[u].w, 4 * i + 3, best, bi);
+            }
+        }
     }
     for (int i = nvec * 4 + threadIdx.x; i < cols; i += kArgmaxThreads) argmax_take(row[i], i, best, bi);
-    sv[threadIdx.x] = best, si[threadIdx.x] = bi;
+    // the wave's winner by exchanges between lanes, the block's through LDS
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) argmax_take(__shfl_xor(best, d), __shfl_xor(bi, d), best, bi);
+    if ((threadIdx.x & 63) == 0) sv[threadIdx.x >> 6] = best, si[threadIdx.x >> 6] = bi;
     __syncthreads();
-    for (int s = kArgmaxThreads / 2; s > 0; s >>= 1) {
-        if (threadIdx.x < s) argmax_take(sv[threadIdx.x + s], si[threadIdx.x + s], sv[threadIdx.x], si[threadIdx.x]);
-        __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < kArgmaxThreads / 64; w++) argmax_take(sv[w], si[w], best, bi);
+        out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
     }
-    if (threadIdx.x == 0) out[blockIdx.x] = si[0] == 0x7fffffff ? 0 : si[0];
 }
 
 __global__ __launch_bounds__(kLlmThreads) void embed_f16_kernel(const __half *__restrict__ table, const int32_t *__restrict__ ids,
