@@ -362,14 +362,15 @@ static int attn_plan(nncase_hip_ctx *ctx, const nncase_hip_paged_attn_args_t *p,
     a.num_blocks = p->num_blocks;
     a.len_offset = p->ctx_len_offset;
     const int64_t max_tokens = (int64_t)p->max_blocks_per_seq * p->block_size;
-    // Tiles per wave: the largest run that still leaves about two blocks per compute unit when
+    // Tiles per wave: the largest run that still leaves about one block per compute unit when
     // every sequence is at full length (the kernel cannot know the real lengths on the host).  Measured at batch 32,
-    // 2 kv heads, contexts of 512-4096 tokens: 17.6 us with two tiles per wave, 14.1 with four, 12.9 with eight.
+    // 2 kv heads, contexts of 512-4096 tokens: 17.6 us with two tiles per wave, 14.1 with four, 12.9 with eight; at
+    // batch 16 (a lane of a 24-layer decode step) eight tiles still give the quicker step, 1.150 against 1.160 ms.
     const int nt_max = 512 / p->head_dim; // 8 KiB of K per wave
     auto splits_at = [&](int tiles) { return (max_tokens + kAttnWaves * tiles * 16 - 1) / (kAttnWaves * tiles * 16); };
     int nt = 2;
     while (nt < nt_max && (splits_at(nt) > kAttnMaxSplits ||
-                           (int64_t)p->batch * p->num_kv_heads * splits_at(nt * 2) >= (int64_t)2 * ctx->compute_units))
+                           (int64_t)p->batch * p->num_kv_heads * splits_at(nt * 2) >= (int64_t)ctx->compute_units))
         nt *= 2;
     plan->nt = nt;
     a.split_tokens = kAttnWaves * nt * 16;
