@@ -350,3 +350,16 @@ def test_global_average_pool_in_front_of_a_convolution(hip_ctx, n, h, w, c, oc, 
     bad = conv_args(n, 2, 1, qp(zp, sp), qp(zy, sy), cl)
     with pytest.raises(rt.HipError):
         hip_ctx.qglobal_avgpool_qconv2d(xd, h, w, qp(zx, sx), wt, yd, bad)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_pairs(hip_ctx, seed):
+    """Seeded random shapes, options and padding: with and without the depthwise convolution in front."""
+    rng = np.random.default_rng(7000 + seed)
+    n, k1, n1, n2 = int(rng.integers(1, 4)), int(rng.integers(1, 20)) * 16, int(rng.integers(1, 24)) * 4, int(rng.integers(1, 40)) * 4
+    h, w = int(rng.integers(3, 12)), int(rng.integers(3, 12))
+    options = dict(residual=bool(rng.integers(0, 2)), lut_a=bool(rng.integers(0, 2)), lut_b=bool(rng.integers(0, 2)), relu_b=bool(rng.integers(0, 2)))
+    dw = None
+    if seed % 2:
+        dw = (int(rng.integers(1, 3)), [P1, ((0, 1), (0, 1)), ((1, 0), (1, 0)), ((0, 0), (0, 0))][int(rng.integers(0, 4))])
+    run_pair(hip_ctx, n, k1, n1, n2, h, w, seed=seed, dw=dw, **options)
