@@ -6,7 +6,7 @@
 //   grid = (sequences x kv heads, splits).  A block owns one kv head of one
 //   sequence and a contiguous range of cached tokens, and serves ALL query
 //   heads that share the kv head, so K and V cross the memory system once
-//   however many query heads there are (GQA).  Each of its four waves owns a
+//   however many query heads there are (GQA).  Each of its eight waves owns a
 //   contiguous run of 16-token tiles and issues the loads of ALL its K and V
 //   tiles before any arithmetic (8 KiB of K + 8 KiB of V in flight per wave).
 //
@@ -20,7 +20,7 @@
 //   terms (p = hi + lo), which keeps the P.V product at fp32-level accuracy.
 //
 //   Every wave keeps its own (max, sum, unnormalised output); the block merges
-//   its four waves through LDS and writes one partial per split.  The block
+//   its waves through LDS and writes one partial per split.  The block
 //   that finishes last for a (sequence, kv head) - found with one atomic
 //   counter per pair, which it resets for the next call - merges the splits
 //   and writes the output, so there is a single launch per call.
@@ -36,8 +36,6 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t au32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t au32x2 __attribute__((ext_vector_type(2)));
 
-constexpr int kAttnThreads = 256;
-constexpr int kAttnWaves = 4;
 constexpr int kAttnHeads = 16; // query heads per kv head, padded to the MFMA tile
 constexpr float kLog2e = 1.4426950408889634f;
 
@@ -63,14 +61,20 @@ __device__ __forceinline__ float coherent_load(const float *p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// NT = 16-token tiles per wave (even).
-template <int D, int NT> __global__ __launch_bounds__(kAttnThreads, 2) void paged_attn_kernel(const AttnArgs a) {
+// bytes of dynamic LDS of a block of W waves: the waves' unnormalised outputs, maxima and sums
+constexpr size_t attn_lds_bytes(int d, int waves) { return (size_t)waves * kAttnHeads * (d + 2) * sizeof(float); }
+
+// NT = 16-token tiles per wave (even); W = waves per block (a block owns W * NT * 16 tokens).
+template <int D, int NT, int W> __global__ __launch_bounds__(W * 64, W <= 8 ? 2 : 1) void paged_attn_kernel(const AttnArgs a) {
+    constexpr int kAttnWaves = W, kAttnThreads = W * 64;
     constexpr int KS = D / 32; // 32-deep steps of the logit product
     constexpr int DT = D / 16; // 16-wide column tiles of the output
     constexpr int WAVE_TOKENS = NT * 16;
     constexpr int SPLIT = kAttnWaves * WAVE_TOKENS;
-    __shared__ float red[kAttnWaves][kAttnHeads][D];
-    __shared__ float smax[kAttnWaves][kAttnHeads], ssum[kAttnWaves][kAttnHeads];
+    extern __shared__ __align__(16) float attn_smem[];
+    float(*red)[kAttnHeads][D] = reinterpret_cast<float(*)[kAttnHeads][D]>(attn_smem);                            // [W][heads][D]
+    float(*smax)[kAttnHeads] = reinterpret_cast<float(*)[kAttnHeads]>(attn_smem + (size_t)W * kAttnHeads * D);    // [W][heads]
+    float(*ssum)[kAttnHeads] = smax + W;                                                                            // [W][heads]
     __shared__ uint32_t s_last;
 
     // kv head fastest, then sequence, then split: consecutive workgroups go to different XCDs, so
@@ -210,7 +214,7 @@ template <int D, int NT> __global__ __launch_bounds__(kAttnThreads, 2) void page
         l_w += __shfl_xor(l_w, 32);
     }
 
-    // ---- merge the four waves ----------------------------------------------------------------
+    // ---- merge the waves ----------------------------------------------------------------
     if (g == 0) {
         smax[wave][j] = m_w;
         ssum[wave][j] = l_w;
@@ -329,7 +333,7 @@ hipError_t attn_static_scratch_address(void **ptr) { return hipGetSymbolAddress(
 // Everything a launch needs except the buffers: checked geometry, split plan, sizes of the scratch areas.
 struct AttnPlan {
     AttnArgs a;
-    int nt = 2;
+    int nt = 2, waves = 8;
     size_t partial_bytes = 0, counter_bytes = 0;
 };
 
@@ -362,18 +366,22 @@ static int attn_plan(nncase_hip_ctx *ctx, const nncase_hip_paged_attn_args_t *p,
     a.num_blocks = p->num_blocks;
     a.len_offset = p->ctx_len_offset;
     const int64_t max_tokens = (int64_t)p->max_blocks_per_seq * p->block_size;
-    // Tiles per wave: the largest run that still leaves about one block per compute unit when
-    // every sequence is at full length (the kernel cannot know the real lengths on the host).  Measured at batch 32,
-    // 2 kv heads, contexts of 512-4096 tokens: 17.6 us with two tiles per wave, 14.1 with four, 12.9 with eight; at
-    // batch 16 (a lane of a 24-layer decode step) eight tiles still give the quicker step, 1.150 against 1.160 ms.
+    // Eight waves per block, and tiles per wave: the largest run that still leaves about two blocks per compute unit
+    // when every sequence is at full length (the kernel cannot know the real lengths on the host).  Measured at batch
+    // 32, 2 kv heads, contexts of 512-4096 tokens, microseconds for 2 / 4 / 8 tiles per wave: four waves 17.7 / 14.2 /
+    // 13.2, eight waves 13.3 / 12.2 / 12.9, sixteen waves 13.7 / 13.6 / 22.3 -- the same tokens per block are quicker as
+    // more waves with shorter runs (more loads in flight per block, a shorter chain per wave), up to the point where a
+    // block's merge through LDS outweighs it.  The rule picks 4 tiles there and 2 for the 16 sequences of a decode lane.
     const int nt_max = 512 / p->head_dim; // 8 KiB of K per wave
-    auto splits_at = [&](int tiles) { return (max_tokens + kAttnWaves * tiles * 16 - 1) / (kAttnWaves * tiles * 16); };
+    const int waves = 8;
+    auto splits_at = [&](int tiles) { return (max_tokens + waves * tiles * 16 - 1) / (waves * tiles * 16); };
     int nt = 2;
     while (nt < nt_max && (splits_at(nt) > kAttnMaxSplits ||
-                           (int64_t)p->batch * p->num_kv_heads * splits_at(nt * 2) >= (int64_t)ctx->compute_units))
+                           (int64_t)p->batch * p->num_kv_heads * splits_at(nt * 2) >= (int64_t)2 * ctx->compute_units))
         nt *= 2;
     plan->nt = nt;
-    a.split_tokens = kAttnWaves * nt * 16;
+    plan->waves = waves;
+    a.split_tokens = waves * nt * 16;
     a.splits = (int)((max_tokens + a.split_tokens - 1) / a.split_tokens);
     NNHIP_REQUIRE(ctx, a.splits <= kAttnMaxSplits, -EINVAL,
                   "paged_attention_decode: context capacity of %lld tokens exceeds %d (head_dim %d)", (long long)max_tokens,
@@ -399,16 +407,23 @@ static int attn_launch(nncase_hip_ctx *ctx, AttnPlan &plan, const void *q_dev, c
     a.part_o = reinterpret_cast<float *>(partials);
     a.part_ml = a.part_o + (size_t)a.batch * a.hq * a.splits * a.d;
     const dim3 grid(a.hkv * a.batch, a.splits);
-    const dim3 block(kAttnThreads);
-    const int nt = plan.nt;
-    if (a.d == 64) {
-        if (nt == 8) hipLaunchKernelGGL((paged_attn_kernel<64, 8>), grid, block, 0, ctx->stream, a);
-        else if (nt == 4) hipLaunchKernelGGL((paged_attn_kernel<64, 4>), grid, block, 0, ctx->stream, a);
-        else hipLaunchKernelGGL((paged_attn_kernel<64, 2>), grid, block, 0, ctx->stream, a);
-    } else {
-        if (nt == 4) hipLaunchKernelGGL((paged_attn_kernel<128, 4>), grid, block, 0, ctx->stream, a);
-        else hipLaunchKernelGGL((paged_attn_kernel<128, 2>), grid, block, 0, ctx->stream, a);
-    }
+    const int nt = plan.nt, waves = plan.waves;
+    const dim3 block(waves * 64);
+    const size_t lds = attn_lds_bytes(a.d, waves);
+    bool launched = false;
+    auto go = [&](auto kernel) {
+        if (lds > 65536) { // more than 64 KiB of dynamic LDS has to be asked for (cheap: a field of the function's record)
+            if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return;
+        }
+        hipLaunchKernelGGL(kernel, grid, block, lds, ctx->stream, a);
+        launched = true;
+    };
+#define NNHIP_ATTN_CASE(DV, NTV, WV) \
+    if (!launched && a.d == DV && nt == NTV && waves == WV) go(paged_attn_kernel<DV, NTV, WV>);
+    NNHIP_ATTN_CASE(64, 8, 8) NNHIP_ATTN_CASE(64, 4, 8) NNHIP_ATTN_CASE(64, 2, 8)
+    NNHIP_ATTN_CASE(128, 4, 8) NNHIP_ATTN_CASE(128, 2, 8)
+#undef NNHIP_ATTN_CASE
+    NNHIP_REQUIRE(ctx, launched, -EINVAL, "paged_attention_decode: no kernel for head_dim %d, %d tiles per wave, %d waves", a.d, nt, waves);
     NNHIP_LAUNCH_CHECK(ctx, "paged_attn_kernel");
     return 0;
 }

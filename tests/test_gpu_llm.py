@@ -298,7 +298,7 @@ def test_decode_step_at_the_benchmark_shape(hip_ctx, lanes):
     evaluated a second time with float32 sums (numpy's own blocked order) already drifts from itself by some 2e-3 of a
     row's largest logit.  The device is held to that yardstick: every logit within 1e-3 of the row maximum or 1.5 times the
     drift of the float32 evaluation, whichever is larger; the same next token wherever the float64 top-2 margin exceeds
-    twice that; the appended K / V rows of the first and last layer; the advanced lengths."""
+    twice that; the appended K / V rows of the first and last layer, by the same yardstick; the advanced lengths."""
     cfg = llm.DecoderConfig()
     batch, max_ctx = 32, 4096
     rng = np.random.default_rng(5)
@@ -318,8 +318,8 @@ def test_decode_step_at_the_benchmark_shape(hip_ctx, lanes):
     logits = dec.logits.download((batch, cfg.vocab), np.float32).astype(np.float64)
     ref_k, ref_v = [kc.copy() for _ in range(cfg.layers)], [vc.copy() for _ in range(cfg.layers)]
     want_tok, want_logits = R.decode_step(cfg, weights, tokens, bt, lens.copy(), ref_k, ref_v)
-    _, drift_logits = R.decode_step(cfg, weights, tokens, bt, lens.copy(), [kc.copy() for _ in range(cfg.layers)],
-                                    [vc.copy() for _ in range(cfg.layers)], acc=np.float32)
+    drift_k, drift_v = [kc.copy() for _ in range(cfg.layers)], [vc.copy() for _ in range(cfg.layers)]
+    _, drift_logits = R.decode_step(cfg, weights, tokens, bt, lens.copy(), drift_k, drift_v, acc=np.float32)
     scale = np.abs(want_logits).max(axis=1, keepdims=True)
     err = np.abs(logits - want_logits) / scale
     drift = np.abs(drift_logits - want_logits) / scale
@@ -335,7 +335,11 @@ def test_decode_step_at_the_benchmark_shape(hip_ctx, lanes):
     for li in (0, cfg.layers - 1):
         k_dev = dec.layers[li]["k"].download(kc.shape, np.float16).astype(np.float64)
         v_dev = dec.layers[li]["v"].download(vc.shape, np.float16).astype(np.float64)
-        for name, dev, ref in (("k", k_dev, ref_k[li].astype(np.float64)), ("v", v_dev, ref_v[li].astype(np.float64))):
+        for name, dev, ref, other in (("k", k_dev, ref_k[li].astype(np.float64), drift_k[li].astype(np.float64)),
+                                      ("v", v_dev, ref_v[li].astype(np.float64), drift_v[li].astype(np.float64))):
             d = np.abs(dev - ref)
-            # fp16 storage: one unit in the last place of the stored value, on top of 1e-3 of the row's scale
-            assert d.max() <= 1e-3 * max(1.0, float(np.abs(ref).max())) + 4e-3, f"layer {li} {name} cache differs by {d.max():.3e}"
+            # fp16 storage: one unit in the last place of the stored value, on top of 1e-3 of the row's scale -- or, behind
+            # 23 layers, 1.5 times what the float32-sum evaluation's own appended rows drift by (the logits' yardstick)
+            bound = max(1e-3 * max(1.0, float(np.abs(ref).max())) + 4e-3, 1.5 * float(np.abs(other - ref).max()))
+            print(f"layer {li} {name} cache: largest difference {d.max():.2e}, float32-sum evaluation {np.abs(other - ref).max():.2e}, bound {bound:.2e}")
+            assert d.max() <= bound, f"layer {li} {name} cache differs by {d.max():.3e} (bound {bound:.3e})"
