@@ -388,20 +388,26 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_gemm_rows_in_lds_kernel(cons
     // The weights do not depend on the rows: the first KB k-steps of this wave's share are requested before anything
     // else, so that their trip to memory runs beside the one that brings the rows in (a spare wave of the last block
     // reads the last tile's and multiplies nothing).
-    const int out_tile = ROPE    ? ((int)blockIdx.x / a.up_tile_offset) * (2 * a.up_tile_offset) + (int)blockIdx.x % a.up_tile_offset
-                         : SPLIT ? (int)blockIdx.x
-                                 : (int)blockIdx.x * WAVES + wave;
+    // Without SPLIT a block walks the groups of WAVES tiles blockIdx.x, blockIdx.x + gridDim.x, ...: a launch with fewer
+    // blocks than groups (the vocabulary head) brings the rows in and normalises them once per block, not once per group.
+    int group = (int)blockIdx.x;
+    int out_tile = ROPE    ? ((int)blockIdx.x / a.up_tile_offset) * (2 * a.up_tile_offset) + (int)blockIdx.x % a.up_tile_offset
+                   : SPLIT ? (int)blockIdx.x
+                           : group * WAVES + wave;
     const int per = SPLIT ? (a.ksteps + WAVES - 1) / WAVES : a.ksteps;
     const int ks0 = SPLIT ? wave * per : 0, ks1 = min(a.ksteps, ks0 + per);
-    const int first = ROPE ? out_tile : min(out_tile, a.up_tile_offset - 1);
-    const int tile[2] = {first, first + a.up_tile_offset};
+    int first = ROPE ? out_tile : min(out_tile, a.up_tile_offset - 1);
+    int tile[2] = {first, first + a.up_tile_offset};
     lu32x4 wv[KB][G];
+    auto request_first = [&]() __attribute__((always_inline)) {
 #pragma unroll
-    for (int u = 0; u < KB; u++) {
-        const int ks = max(min(ks0 + u, ks1 - 1), 0); // steps past the share re-read its last one (an empty share: step 0) and are not multiplied
+        for (int u = 0; u < KB; u++) {
+            const int ks = max(min(ks0 + u, ks1 - 1), 0); // steps past the share re-read its last one (an empty share: step 0) and are not multiplied
 #pragma unroll
-        for (int g = 0; g < G; g++) wv[u][g] = a.w[((size_t)tile[g] * a.ksteps + ks) * 64 + lane];
-    }
+            for (int g = 0; g < G; g++) wv[u][g] = a.w[((size_t)tile[g] * a.ksteps + ks) * 64 + lane];
+        }
+    };
+    request_first();
     {
         constexpr int R = MT * 16 / WAVES; // rows per wave
         // The wave's rows stay in registers from the load to the one LDS write: their sums of squares, the butterflies
@@ -465,7 +471,9 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_gemm_rows_in_lds_kernel(cons
         }
     }
     __syncthreads();
-    if (!ROPE && out_tile >= a.up_tile_offset) return; // SPLIT: never; otherwise the last block's spare waves (uniform per wave)
+    const int groups = SPLIT ? 0 : (a.up_tile_offset + WAVES - 1) / WAVES;
+    for (;;) { // (one pass with SPLIT)
+    if (!ROPE && out_tile >= a.up_tile_offset) return; // SPLIT: never; otherwise the last group's spare waves (uniform per wave; no group follows it)
     f32x4v acc[G][MT];
 #pragma unroll
     for (int g = 0; g < G; g++)
@@ -511,6 +519,15 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_gemm_rows_in_lds_kernel(cons
                 }
             }
         }
+    }
+    // the next group's first weights are requested as soon as this one's are multiplied: they travel under the epilogue
+    group += (int)gridDim.x;
+    const bool more = !SPLIT && group < groups;
+    const int next_tile = group * WAVES + wave;
+    if (more) {
+        first = min(next_tile, a.up_tile_offset - 1);
+        tile[0] = first, tile[1] = first + a.up_tile_offset;
+        request_first();
     }
     if (SPLIT) {
 #pragma unroll
@@ -573,6 +590,9 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_gemm_rows_in_lds_kernel(cons
         }
         if (m >= a.m) continue;
         store_gemm_row<G>(a, v, (size_t)m * a.n_out + out_tile * 16 + kg * 4, res_pre, SPLIT);
+    }
+    if (!more) return;
+    out_tile = next_tile;
     }
 }
 
@@ -854,9 +874,11 @@ static int launch_w8a16_gemm(nncase_hip_ctx_t *ctx, const void *a_dev, const nnc
         return 0;
     }
     if (w->k <= kRowsMaxK && rows_lds <= 128 * 1024 && out_tiles >= ctx->compute_units) {
-        const dim3 rgrid((out_tiles + kGemmWaves - 1) / kGemmWaves), rblock(kGemmThreads);
+        // (at most two blocks per compute unit, each walking several groups of eight tiles: what a block repeats -- the
+        // rows' trip and their normalisation -- is then paid twice per compute unit, not once per group)
+        const dim3 rgrid(std::min((out_tiles + kGemmWaves - 1) / kGemmWaves, 2 * ctx->compute_units)), rblock(kGemmThreads);
         // (eight k-steps of weights per request: asking for a whole 14-step reduction at once costs registers that the
-        // vocabulary head, 1187 blocks, needs for occupancy -- 50.7 against 43.9 us)
+        // vocabulary head needs for occupancy -- 50.7 against 43.9 us when it still ran as 1187 one-group blocks)
 #define NNHIP_ROWS_LAUNCH_KB(MTV, GV, KBV, PV)                                                                                 \
     do {                                                                                                                       \
         NNHIP_HIP(ctx, raise_dynamic_lds(w8a16_gemm_rows_in_lds_kernel<MTV, GV, kGemmWaves, false, KBV, PV>, ctx->device, rows_lds + 1024, 128 * 1024)); \
