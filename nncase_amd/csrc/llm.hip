@@ -655,14 +655,24 @@ __global__ __launch_bounds__(kArgmaxThreads) void argmax_f32_kernel(const float 
         float4 v[U];
 #pragma unroll
         for (int u = 0; u < U; u++) v[u] = reinterpret_cast<const float4 *>(row)[min(i0 + u * kArgmaxThreads, nvec - 1)];
+        // the batch's maximum first (one instruction per element); only a batch that beats the running maximum -- a
+        // handful per thread -- is searched for where (its first such element: indices grow with u and i0)
+        float m = -INFINITY;
 #pragma unroll
-        for (int u = 0; u < U; u++) {
-            const int i = i0 + u * kArgmaxThreads;
-            if (i < nvec) {
-                argmax_take(v[u].x, 4 * i, best, bi);
-                argmax_take(v[u].y, 4 * i + 1, best, bi);
-                argmax_take(v[u].z, 4 * i + 2, best, bi);
-                argmax_take(v[u].w, 4 * i + 3, best, bi);
+        for (int u = 0; u < U; u++)
+            if (i0 + u * kArgmaxThreads < nvec) m = fmaxf(m, fmaxf(fmaxf(v[u].x, v[u].y), fmaxf(v[u].z, v[u].w)));
+        if (m > best) {
+            best = m;
+            bi = 0x7fffffff;
+#pragma unroll
+            for (int u = U - 1; u >= 0; u--) {
+                const int i = i0 + u * kArgmaxThreads;
+                if (i < nvec) {
+                    bi = v[u].w == m ? 4 * i + 3 : bi;
+                    bi = v[u].z == m ? 4 * i + 2 : bi;
+                    bi = v[u].y == m ? 4 * i + 1 : bi;
+                    bi = v[u].x == m ? 4 * i : bi;
+                }
             }
         }
     }

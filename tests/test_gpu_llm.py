@@ -229,11 +229,19 @@ def test_argmax_embedding_and_counter(hip_ctx):
     x = rng.standard_normal((7, 151936)).astype(np.float32)
     x[2, 777] = x[2, 5] = 50.0                                   # a tie: the lower index wins
     x[3, :] = -np.inf
+    x[4, 9] = x[4, 8] = 60.0                                     # ties inside one 16-byte load,
+    x[5, 4136] = x[5, 40] = 70.0                                 # in two loads of one thread's batch,
+    x[6, 151935] = x[6, 40 + 4 * 1024 * 8] = 80.0                # and in two batches of one thread
+    x[0, 100] = np.nan                                           # not a candidate
     out = hip_ctx.alloc(7 * 4)
     hip_ctx.argmax_f32(hip_ctx.to_device(x), out, 7, x.shape[1])
     got = out.download((7,), np.int32)
-    want = x.argmax(axis=1)
-    assert np.array_equal(got, want) and got[2] == 5 and got[3] == 0
+    want = np.where(np.isnan(x), -np.inf, x).argmax(axis=1)
+    assert np.array_equal(got, want) and got[2] == 5 and got[3] == 0 and got[4] == 8 and got[5] == 40 and got[6] == 40 + 4 * 1024 * 8
+    y = rng.standard_normal((3, 1001)).astype(np.float32)       # rows that are not whole 16-byte vectors
+    y[1, 1000] = y[1, 3] = 9.0
+    hip_ctx.argmax_f32(hip_ctx.to_device(y), out, 3, 1001)
+    assert np.array_equal(out.download((3,), np.int32), y.argmax(axis=1))
     table = rng.standard_normal((1000, 96)).astype(np.float16)
     ids = np.array([0, 999, 5, 5, 123], np.int32)
     o = hip_ctx.alloc(5 * 96 * 2)
