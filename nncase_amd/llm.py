@@ -116,7 +116,8 @@ class HipDecoder:
         # lanes > 1: the sequences are split into that many equal ranges and the whole step is recorded once per range,
         # each on a lane of its own; a captured step replays the lanes side by side, so the launch and memory latency
         # of one range's short kernels is covered by the other ranges' kernels.  Every range reads the same weights and
-        # owns its rows of every buffer, so the result is that of lanes == 1 row for row.
+        # owns its rows of every buffer, so the result is that of lanes == 1 row for row, up to the order in which a
+        # product's or an attention's partial sums are added (kernels pick their splits by the number of rows).
         for lane in range(lanes):
             if lanes > 1:
                 fn.set_lane(lane)
