@@ -5,6 +5,7 @@
 // reads are coalesced as well.
 #include "common.hpp"
 
+#include <algorithm>
 #include <type_traits>
 
 namespace nnhip {
@@ -138,6 +139,191 @@ template <typename T> __global__ __launch_bounds__(kLayoutThreads) void unpack_k
     out[gid] = in[off];
 }
 
+// ---- pack / unpack through an LDS tile ------------------------------------------------------------------------------
+// The layouts pack exists for (NCHW -> NC/32 HW 32 for a matrix operand, [K, N] -> weight tiles) put the lanes of the LAST
+// packed axis A innermost, and A is not the innermost axis of the plain tensor: every run of the packed tensor is a
+// strided column of the plain one.  One thread per output element then reads single elements a row apart.  Here a
+// block moves a tile of (one lane group of A) x (a stretch of the plain tensor's innermost axis X) through LDS: dword
+// loads along the source's contiguous axis, dword stores along the destination's, and the E x E elements of a dword
+// pair (E = 4 / element size) transposed in registers between the two, so that every LDS access is a dword as well
+// (rows padded to a dword count that is 1 mod 32: neither phase meets a bank conflict worth the name).
+// X is the trailing run of unpacked axes taken as one (NCHW: H x W), or the innermost axis when that is packed under
+// an earlier lane entry ([K, N] by (N: 16, K: 64)).  Everything else -- other axes, the lane group of A, the stretch of
+// X -- is decoded from the block index.
+struct TwoTerm { // offset(i) = (i / lanes) * hi + (i % lanes) * lo, in elements
+    uint32_t lanes;
+    uint64_t hi, lo;
+};
+__device__ __forceinline__ uint64_t two_term(const TwoTerm &t, uint32_t i) {
+    const uint32_t q = t.lanes == 1 ? i : i / t.lanes;
+    return (uint64_t)q * t.hi + (uint64_t)(i - q * t.lanes) * t.lo;
+}
+struct TileDesc {
+    int nrest;
+    uint32_t r_extent[kMaxRank], r_valid[kMaxRank]; // coordinates from r_valid on have no source: their tiles are zeros (pack)
+    TwoTerm r_plain[kMaxRank], r_packed[kMaxRank];
+    uint32_t a_groups, a_extent, la; // lane groups of A, its plain extent, its lanes
+    uint64_t a_plain_stride;          // plain elements between consecutive coordinates of A
+    uint64_t a_packed_group;          // packed elements between consecutive lane groups of A
+    uint32_t x_extent, x_padded, tx, x_tiles; // plain extent of X, its extent in the packed tensor, elements per tile
+    TwoTerm x_packed;                 // packed offset of a coordinate of X (the plain one is the coordinate itself)
+    uint32_t pitch;                   // dwords per LDS row
+    FastDiv d_cols, d_rowq;           // dwords per row of the tile; rows / E
+};
+
+template <int E> __device__ __forceinline__ void transpose_dwords(const uint32_t (&d)[E], uint32_t (&o)[E]) {
+    if constexpr (E == 1) {
+        o[0] = d[0];
+    } else if constexpr (E == 2) {
+        o[0] = __builtin_amdgcn_perm(d[1], d[0], 0x05040100u);
+        o[1] = __builtin_amdgcn_perm(d[1], d[0], 0x07060302u);
+    } else {
+        const uint32_t a_lo = __builtin_amdgcn_perm(d[1], d[0], 0x05010400u), a_hi = __builtin_amdgcn_perm(d[1], d[0], 0x07030602u);
+        const uint32_t b_lo = __builtin_amdgcn_perm(d[3], d[2], 0x05010400u), b_hi = __builtin_amdgcn_perm(d[3], d[2], 0x07030602u);
+        o[0] = __builtin_amdgcn_perm(b_lo, a_lo, 0x05040100u);
+        o[1] = __builtin_amdgcn_perm(b_lo, a_lo, 0x07060302u);
+        o[2] = __builtin_amdgcn_perm(b_hi, a_hi, 0x05040100u);
+        o[3] = __builtin_amdgcn_perm(b_hi, a_hi, 0x07060302u);
+    }
+}
+
+// E = elements per dword.  PACK: plain -> packed (LDS rows = lanes of A, columns = X); else packed -> plain (rows = X,
+// columns = lanes of A).  in / out are byte pointers, 4-byte aligned like every row the host admits.
+template <int E, bool PACK> __global__ __launch_bounds__(kLayoutThreads) void pack_tile_kernel(const uint8_t *in, uint8_t *out, const TileDesc d) {
+    extern __shared__ uint32_t tile[];
+    constexpr int ES = 4 / E;
+    // ---- which tile ----
+    uint32_t b = blockIdx.x;
+    const uint32_t xt = b % d.x_tiles;
+    b /= d.x_tiles;
+    const uint32_t ag = b % d.a_groups;
+    b /= d.a_groups;
+    uint64_t plain = (uint64_t)ag * d.la * d.a_plain_stride, packed = (uint64_t)ag * d.a_packed_group;
+    bool has_source = true;
+    for (int i = d.nrest - 1; i >= 0; i--) {
+        const uint32_t c = b % d.r_extent[i];
+        b /= d.r_extent[i];
+        has_source = has_source && c < d.r_valid[i];
+        plain += two_term(d.r_plain[i], c);
+        packed += two_term(d.r_packed[i], c);
+    }
+    const uint32_t x0 = xt * d.tx;
+    plain += x0;
+    const uint32_t vlim = min(d.la, d.a_extent - ag * d.la); // lanes of this group that exist in the plain tensor
+    const uint32_t rows = PACK ? d.la : d.tx, cols = d.d_cols.div; // (cols in dwords)
+    // ---- in ----
+    for (uint32_t idx = threadIdx.x; idx < rows * cols; idx += kLayoutThreads) {
+        const uint32_t r = fastdiv(idx, d.d_cols), c = idx - r * cols;
+        uint32_t v = 0;
+        if (PACK) { // row r = lane l, column c = E coordinates of X from x0 + c * E
+            if (has_source && r < vlim && x0 + c * E < d.x_extent)
+                v = *reinterpret_cast<const uint32_t *>(in + (plain + (uint64_t)r * d.a_plain_stride) * ES + c * 4);
+        } else { // row r = coordinate x0 + r of X, column c = E lanes
+            if (x0 + r < d.x_extent) v = *reinterpret_cast<const uint32_t *>(in + (packed + two_term(d.x_packed, x0 + r)) * ES + c * 4);
+        }
+        tile[r * d.pitch + c] = v;
+    }
+    __syncthreads();
+    // ---- out: E rows x one dword column at a time, the lanes of a wave along the destination's contiguous axis ----
+    const uint32_t rowq = d.d_rowq.div;
+    for (uint32_t idx = threadIdx.x; idx < rowq * cols; idx += kLayoutThreads) {
+        const uint32_t c = fastdiv(idx, d.d_rowq), rq = idx - c * rowq;
+        uint32_t w[E], o[E];
+#pragma unroll
+        for (int k = 0; k < E; k++) w[k] = tile[(rq * E + k) * d.pitch + c];
+        transpose_dwords<E>(w, o);
+#pragma unroll
+        for (int j = 0; j < E; j++) {
+            if (PACK) { // o[j]: lanes rq * E .. of coordinate x0 + c * E + j
+                const uint32_t x = x0 + c * E + j;
+                if (x < d.x_padded) *reinterpret_cast<uint32_t *>(out + (packed + two_term(d.x_packed, x)) * ES + rq * 4) = o[j];
+            } else { // o[j]: coordinates x0 + rq * E .. of lane c * E + j
+                const uint32_t l = c * E + j;
+                if (l < vlim && x0 + rq * E < d.x_extent)
+                    *reinterpret_cast<uint32_t *>(out + (plain + (uint64_t)l * d.a_plain_stride) * ES + rq * 4) = o[j];
+            }
+        }
+    }
+}
+
+// Fills the tile description for pack (plain -> packed) or unpack of `shape` by (axes, lanes); false when the layout is
+// not one the tile kernel moves (then the element-wise kernels do).
+static bool make_tile_desc(TileDesc &d, int es, int rank, const int32_t *shape, int n_axes, const int *nax, const int32_t *lanes, bool pack,
+                           const void *in, const void *out, uint64_t &blocks, size_t &lds) {
+    if (n_axes < 1 || (es != 1 && es != 2 && es != 4)) return false;
+    const int e = 4 / es;
+    if (((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 3u) != 0) return false;
+    uint32_t L[kMaxRank], O[kMaxRank];
+    int jpos[kMaxRank];
+    uint64_t lp_all = 1;
+    for (int i = 0; i < rank; i++) L[i] = 1, jpos[i] = -1;
+    for (int j = 0; j < n_axes; j++) L[nax[j]] = (uint32_t)lanes[j], jpos[nax[j]] = j, lp_all *= (uint64_t)lanes[j];
+    uint64_t sp[kMaxRank], sqo[kMaxRank], sql[kMaxRank];
+    uint64_t st = 1;
+    for (int i = rank - 1; i >= 0; i--) sp[i] = st, st *= (uint64_t)shape[i];
+    if (st >= ((uint64_t)1 << 40)) return false;
+    st = 1;
+    for (int j = n_axes - 1; j >= 0; j--) sql[j] = st, st *= (uint64_t)lanes[j];
+    for (int i = rank - 1; i >= 0; i--) O[i] = ((uint32_t)shape[i] + L[i] - 1) / L[i], sqo[i] = st, st *= O[i];
+    const int a = nax[n_axes - 1];
+    const uint32_t la = (uint32_t)lanes[n_axes - 1];
+    if (a == rank - 1 || la % e != 0 || la < (uint32_t)e || la > 128) return false;
+    memset(&d, 0, sizeof(d));
+    // X: the trailing unpacked axes as one, or the (packed) innermost axis
+    int xs = rank;
+    while (xs > 0 && L[xs - 1] == 1) xs--;
+    uint64_t xe = 1;
+    if (xs < rank) {
+        for (int i = xs; i < rank; i++) xe *= (uint64_t)shape[i];
+        if (xe >= ((uint64_t)1 << 31)) return false;
+        d.x_extent = d.x_padded = (uint32_t)xe;
+        d.x_packed = TwoTerm{1, lp_all, 0};
+    } else {
+        xs = rank - 1;
+        d.x_extent = (uint32_t)shape[xs];
+        d.x_padded = O[xs] * L[xs];
+        d.x_packed = TwoTerm{L[xs], sqo[xs], sql[jpos[xs]]};
+    }
+    if (a >= xs || ((uint64_t)d.x_extent * es) % 4 != 0) return false;
+    if (!pack) d.x_padded = d.x_extent;
+    // about 8 KiB per tile, rows of the plain tensor between 64 and 256 bytes of it
+    uint32_t tx = 8192 / (la * es);
+    tx = std::min<uint32_t>(std::max<uint32_t>(tx, 64 / es), 256 / es);
+    d.tx = tx / e * e;
+    d.x_tiles = (d.x_padded + d.tx - 1) / d.tx;
+    d.la = la, d.a_extent = (uint32_t)shape[a], d.a_groups = O[a];
+    d.a_plain_stride = sp[a], d.a_packed_group = sqo[a];
+    blocks = (uint64_t)d.x_tiles * d.a_groups;
+    for (int i = 0; i < xs; i++) {
+        if (i == a) continue;
+        const int k = d.nrest++;
+        d.r_extent[k] = pack ? O[i] * L[i] : (uint32_t)shape[i];
+        d.r_valid[k] = (uint32_t)shape[i];
+        d.r_plain[k] = TwoTerm{1, sp[i], 0};
+        d.r_packed[k] = L[i] == 1 ? TwoTerm{1, sqo[i], 0} : TwoTerm{L[i], sqo[i], sql[jpos[i]]};
+        blocks *= d.r_extent[k];
+    }
+    if (blocks == 0 || blocks >= ((uint64_t)1 << 31)) return false;
+    const uint32_t rows = pack ? la : d.tx, cols = (pack ? d.tx : la) / e;
+    d.pitch = (cols + 31) / 32 * 32 + 1;
+    d.d_cols = make_fastdiv(cols);
+    d.d_rowq = make_fastdiv(rows / e);
+    lds = (size_t)rows * d.pitch * 4;
+    return lds <= 64 * 1024;
+}
+
+template <bool PACK> static int launch_pack_tile(nncase_hip_ctx *ctx, const void *in, void *out, int es, const TileDesc &d, uint64_t blocks, size_t lds) {
+    const dim3 grid((unsigned)blocks), block(kLayoutThreads);
+    if (lds > 48 * 1024) return 1; // (not asked for: the tiles are sized to stay below)
+    switch (es) {
+    case 1: hipLaunchKernelGGL((pack_tile_kernel<4, PACK>), grid, block, lds, ctx->stream, (const uint8_t *)in, (uint8_t *)out, d); break;
+    case 2: hipLaunchKernelGGL((pack_tile_kernel<2, PACK>), grid, block, lds, ctx->stream, (const uint8_t *)in, (uint8_t *)out, d); break;
+    default: hipLaunchKernelGGL((pack_tile_kernel<1, PACK>), grid, block, lds, ctx->stream, (const uint8_t *)in, (uint8_t *)out, d); break;
+    }
+    NNHIP_LAUNCH_CHECK(ctx, "pack_tile_kernel");
+    return 0;
+}
+
 // [batch][rows][cols] -> [batch][cols][rows] through a 32x32 LDS tile.
 template <typename T>
 __global__ __launch_bounds__(256) void transpose_kernel(const T *__restrict__ in, T *__restrict__ out, int rows, int cols) {
@@ -217,6 +403,15 @@ extern "C" int nncase_hip_pack(nncase_hip_ctx_t *ctx, const void *in_dev, void *
         rc = launch_pack_pixels<uint8_t>(ctx, (const uint8_t *)in_dev, out_dev, rank, shape, n_axes, nax, lanes, 1.f, 0.f);
         if (rc <= 0) return rc;
     }
+    {
+        TileDesc t;
+        uint64_t blocks = 0;
+        size_t lds = 0;
+        if (make_tile_desc(t, elem_size, rank, shape, n_axes, nax, lanes, true, in_dev, out_dev, blocks, lds)) {
+            rc = launch_pack_tile<true>(ctx, in_dev, out_dev, elem_size, t, blocks, lds);
+            if (rc <= 0) return rc;
+        }
+    }
     PackDesc d;
     memset(&d, 0, sizeof(d));
     d.in_rank = rank;
@@ -277,6 +472,15 @@ extern "C" int nncase_hip_unpack(nncase_hip_ctx_t *ctx, const void *in_dev, void
     int nax[kMaxRank];
     int rc = build_common(ctx, rank, unpacked_shape, n_axes, axes, lanes, nax);
     if (rc) return rc;
+    {
+        TileDesc t;
+        uint64_t blocks = 0;
+        size_t lds = 0;
+        if (make_tile_desc(t, elem_size, rank, unpacked_shape, n_axes, nax, lanes, false, in_dev, out_dev, blocks, lds)) {
+            rc = launch_pack_tile<false>(ctx, in_dev, out_dev, elem_size, t, blocks, lds);
+            if (rc <= 0) return rc;
+        }
+    }
     PackDesc d;
     memset(&d, 0, sizeof(d));
     d.out_rank = rank;

@@ -24,6 +24,17 @@ pytestmark = pytest.mark.gpu
     ((1, 8, 6, 4), [1, 2, 3], [2, 2, 4], np.uint8),
     ((2, 5, 6, 3), [1, 2, 3], [2, 2, 4], np.uint8),    # odd height: the general kernel
     ((2, 6, 10, 3), [2, 1, 3], [2, 2, 4], np.uint8),   # lanes in another order: the general kernel
+    # the LDS-tile kernel: lanes of the last packed axis against the innermost plain axis, ragged both ways
+    ((2, 33, 300), [1], [32], np.uint8),
+    ((2, 33, 300), [1], [32], np.float32),
+    ((4, 96, 14, 14), [1], [32], np.float16),          # trailing unpacked axes taken as one (H x W)
+    ((70, 40), [1, 0], [16, 64], np.uint8),            # the innermost axis packed under an earlier lane entry
+    ((520, 272), [1, 0], [16, 64], np.uint8),
+    ((5, 3, 10, 4), [0, 2], [4, 4], np.uint8),         # another packed axis among the block coordinates, ragged
+    ((2, 2, 130, 4), [2], [128], np.uint8),
+    ((3, 20, 6), [0, 1], [2, 8], np.float16),
+    ((2, 5, 3, 7), [1], [4], np.float32),
+    ((3, 7, 6), [1], [4], np.uint8),                   # rows of 6 bytes: not dword multiples, the element-wise kernel
 ])
 def test_pack_unpack(hip_ctx, shape, axes, lanes, dtype):
     rng = np.random.default_rng(len(shape) + shape[0])
