@@ -26,19 +26,30 @@ struct PackDesc {
     int lane_dim[kMaxRank];
     int in_rank;
     uint64_t total;
+    FastDiv out_div[2 * kMaxRank]; // of out_dims (the SMALL kernels: fewer than 2^31 output elements)
 };
 
-template <typename T> __global__ __launch_bounds__(kLayoutThreads) void pack_kernel(const T *in, T *out, const PackDesc d) {
+// SMALL: fewer than 2^31 output elements, so that the coordinates come from 32-bit multiply-shift divisions.
+template <typename T, bool SMALL> __global__ __launch_bounds__(kLayoutThreads) void pack_kernel(const T *in, T *out, const PackDesc d) {
     const uint64_t gid = (uint64_t)blockIdx.x * kLayoutThreads + threadIdx.x;
     if (gid >= d.total) return;
     uint32_t coord[kMaxRank];
 #pragma unroll
     for (int i = 0; i < kMaxRank; i++) coord[i] = 0;
-    uint64_t rem = gid;
-    for (int k = d.out_rank - 1; k >= 0; k--) {
-        const uint32_t c = (uint32_t)(rem % d.out_dims[k]);
-        rem /= d.out_dims[k];
-        coord[d.axis[k]] += c * d.mul[k];
+    if constexpr (SMALL) {
+        uint32_t rem = (uint32_t)gid;
+        for (int k = d.out_rank - 1; k >= 0; k--) {
+            const uint32_t q = fastdiv(rem, d.out_div[k]);
+            coord[d.axis[k]] += (rem - q * d.out_dims[k]) * d.mul[k];
+            rem = q;
+        }
+    } else {
+        uint64_t rem = gid;
+        for (int k = d.out_rank - 1; k >= 0; k--) {
+            const uint32_t c = (uint32_t)(rem % d.out_dims[k]);
+            rem /= d.out_dims[k];
+            coord[d.axis[k]] += c * d.mul[k];
+        }
     }
     bool ok = true;
     uint64_t off = 0;
@@ -125,16 +136,27 @@ static int launch_pack_pixels(nncase_hip_ctx *ctx, const TIn *in, void *out, int
     return 1;
 }
 
-template <typename T> __global__ __launch_bounds__(kLayoutThreads) void unpack_kernel(const T *in, T *out, const PackDesc d) {
+template <typename T, bool SMALL> __global__ __launch_bounds__(kLayoutThreads) void unpack_kernel(const T *in, T *out, const PackDesc d) {
     const uint64_t gid = (uint64_t)blockIdx.x * kLayoutThreads + threadIdx.x;
     if (gid >= d.total) return;
     uint64_t rem = gid, off = 0;
     for (int k = d.out_rank - 1; k >= 0; k--) {
-        const uint32_t c = (uint32_t)(rem % d.out_dims[k]);
-        rem /= d.out_dims[k];
+        uint32_t c;
+        if constexpr (SMALL) {
+            const uint32_t q = fastdiv((uint32_t)rem, d.out_div[k]);
+            c = (uint32_t)rem - q * d.out_dims[k];
+            rem = q;
+        } else {
+            c = (uint32_t)(rem % d.out_dims[k]);
+            rem /= d.out_dims[k];
+        }
         const uint32_t l = d.lanes[k];
-        off += (uint64_t)(c / l) * d.in_strides[k];
-        if (l > 1) off += (uint64_t)(c % l) * d.in_strides[d.lane_dim[k]];
+        if (l > 1) {
+            const uint32_t g = c / l;
+            off += (uint64_t)g * d.in_strides[k] + (uint64_t)(c - g * l) * d.in_strides[d.lane_dim[k]];
+        } else {
+            off += (uint64_t)c * d.in_strides[k];
+        }
     }
     out[gid] = in[off];
 }
@@ -167,6 +189,7 @@ struct TileDesc {
     uint64_t a_packed_group;          // packed elements between consecutive lane groups of A
     uint32_t x_extent, x_padded, tx, x_tiles; // plain extent of X, its extent in the packed tensor, elements per tile
     TwoTerm x_packed;                 // packed offset of a coordinate of X (the plain one is the coordinate itself)
+    uint32_t exact;                   // 1: the destination has no padding: lanes past the plain extent of A are not stored (transposes)
     uint32_t pitch;                   // dwords per LDS row
     FastDiv d_cols, d_rowq;           // dwords per row of the tile; rows / E
 };
@@ -219,7 +242,7 @@ template <int E, bool PACK> __global__ __launch_bounds__(kLayoutThreads) void pa
             if (has_source && r < vlim && x0 + c * E < d.x_extent)
                 v = *reinterpret_cast<const uint32_t *>(in + (plain + (uint64_t)r * d.a_plain_stride) * ES + c * 4);
         } else { // row r = coordinate x0 + r of X, column c = E lanes
-            if (x0 + r < d.x_extent) v = *reinterpret_cast<const uint32_t *>(in + (packed + two_term(d.x_packed, x0 + r)) * ES + c * 4);
+            if (x0 + r < d.x_extent && c * E < vlim) v = *reinterpret_cast<const uint32_t *>(in + (packed + two_term(d.x_packed, x0 + r)) * ES + c * 4);
         }
         tile[r * d.pitch + c] = v;
     }
@@ -236,7 +259,8 @@ template <int E, bool PACK> __global__ __launch_bounds__(kLayoutThreads) void pa
         for (int j = 0; j < E; j++) {
             if (PACK) { // o[j]: lanes rq * E .. of coordinate x0 + c * E + j
                 const uint32_t x = x0 + c * E + j;
-                if (x < d.x_padded) *reinterpret_cast<uint32_t *>(out + (packed + two_term(d.x_packed, x)) * ES + rq * 4) = o[j];
+                if (x < d.x_padded && (!d.exact || rq * E < vlim))
+                    *reinterpret_cast<uint32_t *>(out + (packed + two_term(d.x_packed, x)) * ES + rq * 4) = o[j];
             } else { // o[j]: coordinates x0 + rq * E .. of lane c * E + j
                 const uint32_t l = c * E + j;
                 if (l < vlim && x0 + rq * E < d.x_extent)
@@ -245,6 +269,15 @@ template <int E, bool PACK> __global__ __launch_bounds__(kLayoutThreads) void pa
         }
     }
 }
+
+// Elements of X per tile: about 8 KiB per tile, rows of the plain tensor of 64 bytes to 2 KiB.
+static uint32_t tile_stretch(uint32_t la, int es) {
+    uint32_t tx = 8192 / (la * es);
+    tx = std::min<uint32_t>(std::max<uint32_t>(tx, 64 / es), 2048 / es);
+    return tx / (4 / es) * (4 / es);
+}
+// Dwords per LDS row: odd, so that the E rows a lane reads and the rows of neighbouring lanes spread over the banks.
+static uint32_t tile_pitch(uint32_t cols) { return cols | 1u; }
 
 // Fills the tile description for pack (plain -> packed) or unpack of `shape` by (axes, lanes); false when the layout is
 // not one the tile kernel moves (then the element-wise kernels do).
@@ -286,10 +319,7 @@ static bool make_tile_desc(TileDesc &d, int es, int rank, const int32_t *shape, 
     }
     if (a >= xs || ((uint64_t)d.x_extent * es) % 4 != 0) return false;
     if (!pack) d.x_padded = d.x_extent;
-    // about 8 KiB per tile, rows of the plain tensor between 64 and 256 bytes of it
-    uint32_t tx = 8192 / (la * es);
-    tx = std::min<uint32_t>(std::max<uint32_t>(tx, 64 / es), 256 / es);
-    d.tx = tx / e * e;
+    d.tx = tile_stretch(la, es);
     d.x_tiles = (d.x_padded + d.tx - 1) / d.tx;
     d.la = la, d.a_extent = (uint32_t)shape[a], d.a_groups = O[a];
     d.a_plain_stride = sp[a], d.a_packed_group = sqo[a];
@@ -305,11 +335,11 @@ static bool make_tile_desc(TileDesc &d, int es, int rank, const int32_t *shape, 
     }
     if (blocks == 0 || blocks >= ((uint64_t)1 << 31)) return false;
     const uint32_t rows = pack ? la : d.tx, cols = (pack ? d.tx : la) / e;
-    d.pitch = (cols + 31) / 32 * 32 + 1;
+    d.pitch = tile_pitch(cols);
     d.d_cols = make_fastdiv(cols);
     d.d_rowq = make_fastdiv(rows / e);
     lds = (size_t)rows * d.pitch * 4;
-    return lds <= 64 * 1024;
+    return lds <= 48 * 1024;
 }
 
 template <bool PACK> static int launch_pack_tile(nncase_hip_ctx *ctx, const void *in, void *out, int es, const TileDesc &d, uint64_t blocks, size_t lds) {
@@ -351,9 +381,53 @@ template <typename T> static int launch_transpose(nncase_hip_ctx *ctx, const voi
     return 0;
 }
 
+// [batch][rows][cols] -> [batch][cols][rows] as the tile kernel sees it.  Packing: the source is the plain tensor
+// (A = rows in groups of up to 128 lanes, X = cols), the destination the "packed" one, whose runs along A have no
+// padding.  Unpacking (short source rows): the destination is the plain tensor (A = cols, X = rows).
+static bool make_transpose_desc(TileDesc &d, int es, int batch, int rows, int cols, bool packing, const void *in, const void *out,
+                                uint64_t &blocks, size_t &lds) {
+    if (es != 1 && es != 2 && es != 4) return false;
+    const int e = 4 / es;
+    if (((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 3u) != 0 || rows % e != 0 || cols % e != 0) return false;
+    memset(&d, 0, sizeof(d));
+    const int na = packing ? rows : cols, nx = packing ? cols : rows; // extents of A and X
+    const uint32_t la = (uint32_t)std::min(na, 128 / e * e);
+    d.la = la, d.a_extent = (uint32_t)na, d.a_groups = ((uint32_t)na + la - 1) / la;
+    d.a_plain_stride = (uint64_t)nx, d.a_packed_group = la;
+    d.x_extent = d.x_padded = (uint32_t)nx;
+    d.x_packed = TwoTerm{1, (uint64_t)na, 0};
+    d.exact = 1;
+    d.tx = tile_stretch(la, es);
+    d.x_tiles = (d.x_padded + d.tx - 1) / d.tx;
+    d.nrest = 1;
+    d.r_extent[0] = d.r_valid[0] = (uint32_t)batch;
+    d.r_plain[0] = d.r_packed[0] = TwoTerm{1, (uint64_t)rows * cols, 0};
+    blocks = (uint64_t)d.x_tiles * d.a_groups * batch;
+    if (blocks >= ((uint64_t)1 << 31)) return false;
+    const uint32_t trows = packing ? la : d.tx, tcols = (packing ? d.tx : la) / e;
+    d.pitch = tile_pitch(tcols);
+    d.d_cols = make_fastdiv(tcols);
+    d.d_rowq = make_fastdiv(trows / e);
+    lds = (size_t)trows * d.pitch * 4;
+    return lds <= 48 * 1024;
+}
+
 static int transpose(nncase_hip_ctx *ctx, const void *in, void *out, int es, int batch, int rows, int cols) {
     NNHIP_REQUIRE(ctx, in && out, -EINVAL, "transpose: null buffer");
     NNHIP_REQUIRE(ctx, batch > 0 && rows > 0 && cols > 0, -EINVAL, "transpose: non-positive shape");
+    // The tile kernel for elements narrower than a dword (its accesses stay dwords) and for matrices with a short
+    // side (its tiles follow the long one); 4-byte elements of other shapes are the 32 x 32 tiles' case (measured:
+    // 255 x 6400 floats 34 us there, 58 us here).
+    if (es < 4 || std::min(rows, cols) < 32) {
+        TileDesc t;
+        uint64_t blocks = 0;
+        size_t lds = 0;
+        const bool packing = (size_t)cols * es >= 128; // source rows long enough to be read as rows
+        if (make_transpose_desc(t, es, batch, rows, cols, packing, in, out, blocks, lds)) {
+            const int rc = packing ? launch_pack_tile<true>(ctx, in, out, es, t, blocks, lds) : launch_pack_tile<false>(ctx, in, out, es, t, blocks, lds);
+            if (rc <= 0) return rc;
+        }
+    }
     NNHIP_REQUIRE(ctx, batch <= 65535 && ceil_div(rows, 32) <= 65535, -EINVAL, "transpose: grid too large");
     switch (es) {
     case 1: return launch_transpose<uint8_t>(ctx, in, out, batch, rows, cols);
@@ -378,11 +452,33 @@ static int build_common(nncase_hip_ctx *ctx, int rank, const int32_t *shape, int
     return 0;
 }
 
+// Where the packed tensor's innermost dimension runs along the plain tensor's innermost axis (no packed axis, or that
+// axis packed last), groups of elements of it move together: the same permutation on 16- or 4-byte elements, that many
+// times fewer of them.  Rewrites (es, shape, lanes) in place when extents, lanes and addresses allow.
+static void vector_view(int &es, int rank, int32_t *shape, int n_axes, const int *nax, int32_t *lanes, const void *in, const void *out) {
+    for (int j = 0; j < n_axes; j++)
+        if (nax[j] == rank - 1 && j != n_axes - 1) return;
+    if (n_axes > 0 && nax[n_axes - 1] != rank - 1) return; // (the innermost lanes belong to another axis)
+    for (int bytes = 16; bytes > es; bytes /= 4) {
+        if (bytes % es != 0) continue;
+        const int e = bytes / es;
+        if (((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & (uintptr_t)(bytes - 1)) != 0 || shape[rank - 1] % e != 0) continue;
+        if (n_axes > 0 && lanes[n_axes - 1] % e != 0) continue;
+        shape[rank - 1] /= e;
+        if (n_axes > 0) lanes[n_axes - 1] /= e;
+        es = bytes;
+        return;
+    }
+}
+
+typedef uint32_t layout_u32x4 __attribute__((ext_vector_type(4)));
+
 template <typename K> static int launch_by_size(nncase_hip_ctx *ctx, int es, K &&k) {
     switch (es) {
     case 1: return k((uint8_t *)nullptr);
     case 2: return k((uint16_t *)nullptr);
     case 4: return k((uint32_t *)nullptr);
+    case 16: return k((layout_u32x4 *)nullptr); // (vector_view's groups only)
     default: return fail(ctx, -NNCASE_HIP_ERR_DATATYPE_MISMATCH, "pack: element size %d", es);
     }
 }
@@ -395,6 +491,7 @@ extern "C" int nncase_hip_pack(nncase_hip_ctx_t *ctx, const void *in_dev, void *
                                const int32_t *shape, int32_t n_axes, const int32_t *axes, const int32_t *lanes) {
     NNHIP_CHECK_CTX(ctx);
     NNHIP_REQUIRE(ctx, in_dev && out_dev, -EINVAL, "pack: null buffer");
+    NNHIP_REQUIRE(ctx, elem_size == 1 || elem_size == 2 || elem_size == 4, -NNCASE_HIP_ERR_DATATYPE_MISMATCH, "pack: element size %d", elem_size);
     int nax[kMaxRank];
     int rc = build_common(ctx, rank, shape, n_axes, axes, lanes, nax);
     if (rc) return rc;
@@ -412,39 +509,47 @@ extern "C" int nncase_hip_pack(nncase_hip_ctx_t *ctx, const void *in_dev, void *
             if (rc <= 0) return rc;
         }
     }
+    int32_t shp[kMaxRank], lns[kMaxRank];
+    for (int i = 0; i < rank; i++) shp[i] = shape[i];
+    for (int j = 0; j < n_axes; j++) lns[j] = lanes[j];
+    int es = elem_size;
+    vector_view(es, rank, shp, n_axes, nax, lns, in_dev, out_dev);
     PackDesc d;
     memset(&d, 0, sizeof(d));
     d.in_rank = rank;
     d.out_rank = rank + n_axes;
     uint64_t stride = 1;
     for (int i = rank - 1; i >= 0; i--) {
-        d.in_dims[i] = (uint32_t)shape[i];
+        d.in_dims[i] = (uint32_t)shp[i];
         d.in_strides[i] = stride;
-        stride *= (uint64_t)shape[i];
+        stride *= (uint64_t)shp[i];
     }
     d.total = 1;
     for (int i = 0; i < rank; i++) {
         uint32_t l = 1;
         for (int j = 0; j < n_axes; j++)
-            if (nax[j] == i) l = (uint32_t)lanes[j];
-        d.out_dims[i] = ((uint32_t)shape[i] + l - 1) / l;
+            if (nax[j] == i) l = (uint32_t)lns[j];
+        d.out_dims[i] = ((uint32_t)shp[i] + l - 1) / l;
         d.axis[i] = i;
         d.mul[i] = l;
         d.total *= d.out_dims[i];
     }
     for (int j = 0; j < n_axes; j++) {
-        d.out_dims[rank + j] = (uint32_t)lanes[j];
+        d.out_dims[rank + j] = (uint32_t)lns[j];
         d.axis[rank + j] = nax[j];
         d.mul[rank + j] = 1;
-        d.total *= (uint64_t)lanes[j];
+        d.total *= (uint64_t)lns[j];
     }
     NNHIP_REQUIRE(ctx, d.total < ((uint64_t)1 << 40), -EINVAL, "pack: tensor too large");
+    for (int k = 0; k < d.out_rank; k++) d.out_div[k] = make_fastdiv(d.out_dims[k]);
     const uint64_t blocks = (d.total + kLayoutThreads - 1) / kLayoutThreads;
     NNHIP_REQUIRE(ctx, blocks < ((uint64_t)1 << 31), -EINVAL, "pack: tensor too large");
-    return launch_by_size(ctx, elem_size, [&](auto *tag) -> int {
+    return launch_by_size(ctx, es, [&](auto *tag) -> int {
         typedef typename std::remove_pointer<decltype(tag)>::type T;
-        hipLaunchKernelGGL(pack_kernel<T>, dim3((unsigned)blocks), dim3(kLayoutThreads), 0, ctx->stream, (const T *)in_dev,
-                           (T *)out_dev, d);
+        if (d.total < ((uint64_t)1 << 31))
+            hipLaunchKernelGGL((pack_kernel<T, true>), dim3((unsigned)blocks), dim3(kLayoutThreads), 0, ctx->stream, (const T *)in_dev, (T *)out_dev, d);
+        else
+            hipLaunchKernelGGL((pack_kernel<T, false>), dim3((unsigned)blocks), dim3(kLayoutThreads), 0, ctx->stream, (const T *)in_dev, (T *)out_dev, d);
         NNHIP_LAUNCH_CHECK(ctx, "pack_kernel");
         return 0;
     });
@@ -469,6 +574,7 @@ extern "C" int nncase_hip_unpack(nncase_hip_ctx_t *ctx, const void *in_dev, void
                                  const int32_t *unpacked_shape, int32_t n_axes, const int32_t *axes, const int32_t *lanes) {
     NNHIP_CHECK_CTX(ctx);
     NNHIP_REQUIRE(ctx, in_dev && out_dev, -EINVAL, "unpack: null buffer");
+    NNHIP_REQUIRE(ctx, elem_size == 1 || elem_size == 2 || elem_size == 4, -NNCASE_HIP_ERR_DATATYPE_MISMATCH, "unpack: element size %d", elem_size);
     int nax[kMaxRank];
     int rc = build_common(ctx, rank, unpacked_shape, n_axes, axes, lanes, nax);
     if (rc) return rc;
@@ -481,6 +587,11 @@ extern "C" int nncase_hip_unpack(nncase_hip_ctx_t *ctx, const void *in_dev, void
             if (rc <= 0) return rc;
         }
     }
+    int32_t shp[kMaxRank], lns[kMaxRank];
+    for (int i = 0; i < rank; i++) shp[i] = unpacked_shape[i];
+    for (int j = 0; j < n_axes; j++) lns[j] = lanes[j];
+    int es = elem_size;
+    vector_view(es, rank, shp, n_axes, nax, lns, in_dev, out_dev);
     PackDesc d;
     memset(&d, 0, sizeof(d));
     d.out_rank = rank;
@@ -491,14 +602,14 @@ extern "C" int nncase_hip_unpack(nncase_hip_ctx_t *ctx, const void *in_dev, void
         d.lane_dim[i] = 0;
         for (int j = 0; j < n_axes; j++)
             if (nax[j] == i) {
-                l = (uint32_t)lanes[j];
+                l = (uint32_t)lns[j];
                 d.lane_dim[i] = rank + j;
             }
         d.lanes[i] = l;
-        d.in_dims[i] = ((uint32_t)unpacked_shape[i] + l - 1) / l;
-        d.out_dims[i] = (uint32_t)unpacked_shape[i];
+        d.in_dims[i] = ((uint32_t)shp[i] + l - 1) / l;
+        d.out_dims[i] = (uint32_t)shp[i];
     }
-    for (int j = 0; j < n_axes; j++) d.in_dims[rank + j] = (uint32_t)lanes[j];
+    for (int j = 0; j < n_axes; j++) d.in_dims[rank + j] = (uint32_t)lns[j];
     uint64_t stride = 1;
     for (int i = d.in_rank - 1; i >= 0; i--) {
         d.in_strides[i] = stride;
@@ -506,12 +617,15 @@ extern "C" int nncase_hip_unpack(nncase_hip_ctx_t *ctx, const void *in_dev, void
     }
     d.total = 1;
     for (int i = 0; i < rank; i++) d.total *= d.out_dims[i];
+    for (int k = 0; k < d.out_rank; k++) d.out_div[k] = make_fastdiv(d.out_dims[k]);
     const uint64_t blocks = (d.total + kLayoutThreads - 1) / kLayoutThreads;
     NNHIP_REQUIRE(ctx, blocks < ((uint64_t)1 << 31), -EINVAL, "unpack: tensor too large");
-    return launch_by_size(ctx, elem_size, [&](auto *tag) -> int {
+    return launch_by_size(ctx, es, [&](auto *tag) -> int {
         typedef typename std::remove_pointer<decltype(tag)>::type T;
-        hipLaunchKernelGGL(unpack_kernel<T>, dim3((unsigned)blocks), dim3(kLayoutThreads), 0, ctx->stream,
-                           (const T *)in_dev, (T *)out_dev, d);
+        if (d.total < ((uint64_t)1 << 31))
+            hipLaunchKernelGGL((unpack_kernel<T, true>), dim3((unsigned)blocks), dim3(kLayoutThreads), 0, ctx->stream, (const T *)in_dev, (T *)out_dev, d);
+        else
+            hipLaunchKernelGGL((unpack_kernel<T, false>), dim3((unsigned)blocks), dim3(kLayoutThreads), 0, ctx->stream, (const T *)in_dev, (T *)out_dev, d);
         NNHIP_LAUNCH_CHECK(ctx, "unpack_kernel");
         return 0;
     });

@@ -86,7 +86,8 @@ def test_quantize_pack_refuses_other_layouts(hip_ctx):
         assert e.value.code == -22
 
 
-@pytest.mark.parametrize("shape", [(1, 3, 224, 224), (2, 144, 7, 5), (3, 1, 1, 1), (1, 33, 65, 2)])
+@pytest.mark.parametrize("shape", [(1, 3, 224, 224), (2, 144, 7, 5), (3, 1, 1, 1), (1, 33, 65, 2), (2, 256, 14, 14), (1, 64, 56, 56), (2, 132, 6, 6),
+                                   (3, 4, 2, 600)])
 @pytest.mark.parametrize("dtype", [np.uint8, np.float16, np.float32])
 def test_nchw_nhwc(hip_ctx, shape, dtype):
     rng = np.random.default_rng(shape[1])
