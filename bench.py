@@ -199,6 +199,29 @@ def side_workload(args):
                               "frac": round(tops / INT8_PEAK_TOPS, 5), "traffic": None,
                               "hbm_GBps": round(nbytes / (ms * 1e-3) / 1e9, 1), "note": note},
                     step_ms=step_spread(ctx, call, args.steps))
+    elif args.workload == "pack":
+        # pack / unpack and the NCHW <-> NHWC relayout at sizes past the 256 MiB of memory-side cache: pure byte moves
+        def moved(name, nbytes, call):
+            ms = time_calls(ctx, call, max(args.warmup, 3), min(args.steps, 30))
+            return {"case": name, "us": round(ms * 1e3, 1), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1), "frac_of_hbm": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+        n, c, hw = 512, 256, 56
+        cnt = n * c * hw * hw
+        a, b = ctx.alloc(cnt), ctx.alloc(cnt)
+        a.fill(1)
+        cases = [moved("pack u8 NCHW [512,256,56,56] -> NC/32 HW 32", 2 * cnt, lambda: ctx.pack(a, b, 1, [n, c, hw, hw], [1], [32])),
+                 moved("unpack of the same", 2 * cnt, lambda: ctx.unpack(b, a, 1, [n, c, hw, hw], [1], [32])),
+                 moved("pack u8 [16384,16384] by (N: 16, K: 64) (weight tiles)", 2 * 16384 * 16384, lambda: ctx.pack(a, b, 1, [16384, 16384], [1, 0], [16, 64])),
+                 moved("pack u8 NHWC [512,56,56,256] by 32 on C", 2 * cnt, lambda: ctx.pack(a, b, 1, [n, hw, hw, c], [3], [32])),
+                 moved("nchw -> nhwc u8 [512,256,56,56]", 2 * cnt, lambda: ctx.nchw_to_nhwc(a, b, 1, n, c, hw, hw)),
+                 moved("nhwc -> nchw u8 [512,256,56,56]", 2 * cnt, lambda: ctx.nhwc_to_nchw(b, a, 1, n, c, hw, hw)),
+                 moved("nchw -> nhwc f32 [640,3,224,224]", 2 * 4 * 640 * 3 * 224 * 224, lambda: ctx.nchw_to_nhwc(a, b, 4, 640, 3, 224, 224)),
+                 moved("nhwc -> nchw f32 [640,224,224,3]", 2 * 4 * 640 * 3 * 224 * 224, lambda: ctx.nhwc_to_nchw(b, a, 4, 640, 3, 224, 224)),
+                 moved("copy (pack without axes) u32", 2 * cnt, lambda: ctx.pack(a, b, 4, [cnt // 4], [], []))]
+        head = cases[0]
+        line = dict(base, metric="GB/s pack u8 NCHW -> NC/32 HW 32", value=head["GBps"], unit="GB/s", ms_per_step=round(head["us"] / 1e3, 5), dtype="u8",
+                    config={"workload": "pack / unpack / relayout of 411 MB tensors (read once, written once)"},
+                    roofline={"bound": "hbm", "achieved": head["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": head["frac_of_hbm"], "traffic": None},
+                    cases=cases)
     elif args.workload == "conv_block":
         batch = 32
         rng = np.random.default_rng(1)
@@ -338,7 +361,7 @@ def side_workload(args):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--workload", default="mobilenetv2", help="mobilenetv2 (headline, default) | matmul | conv_block | yolov5s | paged_attention | llm_decode")
+    ap.add_argument("--workload", default="mobilenetv2", help="mobilenetv2 (headline, default) | matmul | conv_block | yolov5s | paged_attention | llm_decode | pack")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)

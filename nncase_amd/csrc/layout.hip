@@ -234,20 +234,31 @@ template <int E, bool PACK> __global__ __launch_bounds__(kLayoutThreads) void pa
     plain += x0;
     const uint32_t vlim = min(d.la, d.a_extent - ag * d.la); // lanes of this group that exist in the plain tensor
     const uint32_t rows = PACK ? d.la : d.tx, cols = d.d_cols.div; // (cols in dwords)
-    // ---- in ----
-    for (uint32_t idx = threadIdx.x; idx < rows * cols; idx += kLayoutThreads) {
-        const uint32_t r = fastdiv(idx, d.d_cols), c = idx - r * cols;
-        uint32_t v = 0;
-        if (PACK) { // row r = lane l, column c = E coordinates of X from x0 + c * E
-            if (has_source && r < vlim && x0 + c * E < d.x_extent)
-                v = *reinterpret_cast<const uint32_t *>(in + (plain + (uint64_t)r * d.a_plain_stride) * ES + c * 4);
-        } else { // row r = coordinate x0 + r of X, column c = E lanes
-            if (x0 + r < d.x_extent && c * E < vlim) v = *reinterpret_cast<const uint32_t *>(in + (packed + two_term(d.x_packed, x0 + r)) * ES + c * 4);
+    // ---- in: four dwords per thread requested before the first is parked ----
+    constexpr int U = 4;
+    for (uint32_t base = threadIdx.x; base < rows * cols; base += U * kLayoutThreads) {
+        uint32_t v[U], at[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const uint32_t idx = min(base + u * kLayoutThreads, rows * cols - 1); // (a repeat of the last dword: the same value to the same place)
+            const uint32_t r = fastdiv(idx, d.d_cols), c = idx - r * cols;
+            at[u] = r * d.pitch + c;
+            v[u] = 0;
+            if (PACK) { // row r = lane l, column c = E coordinates of X from x0 + c * E
+                if (has_source && r < vlim && x0 + c * E < d.x_extent)
+                    v[u] = *reinterpret_cast<const uint32_t *>(in + (plain + (uint64_t)r * d.a_plain_stride) * ES + c * 4);
+            } else { // row r = coordinate x0 + r of X, column c = E lanes
+                if (x0 + r < d.x_extent && c * E < vlim)
+                    v[u] = *reinterpret_cast<const uint32_t *>(in + (packed + two_term(d.x_packed, x0 + r)) * ES + c * 4);
+            }
         }
-        tile[r * d.pitch + c] = v;
+#pragma unroll
+        for (int u = 0; u < U; u++) tile[at[u]] = v[u];
     }
     __syncthreads();
     // ---- out: E rows x one dword column at a time, the lanes of a wave along the destination's contiguous axis ----
+    // (packing, a lane's E dwords go to E different runs of the destination; parking the transposed tile in a second
+    // LDS area so that it leaves in address order was measured and is no quicker)
     const uint32_t rowq = d.d_rowq.div;
     for (uint32_t idx = threadIdx.x; idx < rowq * cols; idx += kLayoutThreads) {
         const uint32_t c = fastdiv(idx, d.d_rowq), rq = idx - c * rowq;
@@ -270,15 +281,14 @@ template <int E, bool PACK> __global__ __launch_bounds__(kLayoutThreads) void pa
     }
 }
 
-// Elements of X per tile: about 8 KiB per tile, rows of the plain tensor of 64 bytes to 2 KiB.
+// Elements of X per tile: about 16 KiB per tile, rows of the plain tensor of 64 bytes to 2 KiB.
 static uint32_t tile_stretch(uint32_t la, int es) {
-    uint32_t tx = 8192 / (la * es);
+    uint32_t tx = 16384 / (la * es);
     tx = std::min<uint32_t>(std::max<uint32_t>(tx, 64 / es), 2048 / es);
     return tx / (4 / es) * (4 / es);
 }
 // Dwords per LDS row: odd, so that the E rows a lane reads and the rows of neighbouring lanes spread over the banks.
 static uint32_t tile_pitch(uint32_t cols) { return cols | 1u; }
-
 // Fills the tile description for pack (plain -> packed) or unpack of `shape` by (axes, lanes); false when the layout is
 // not one the tile kernel moves (then the element-wise kernels do).
 static bool make_tile_desc(TileDesc &d, int es, int rank, const int32_t *shape, int n_axes, const int *nax, const int32_t *lanes, bool pack,
@@ -471,6 +481,26 @@ static void vector_view(int &es, int rank, int32_t *shape, int n_axes, const int
     }
 }
 
+// Neighbouring axes that are both unpacked are one axis to the permutation (their outer dimensions are neighbours in
+// the packed tensor too): fewer coordinates for every thread to take apart.  Rewrites (rank, shape, axes) in place.
+static void merge_unpacked_axes(int &rank, int32_t *shape, int n_axes, int *nax) {
+    bool packed[kMaxRank] = {false};
+    for (int j = 0; j < n_axes; j++) packed[nax[j]] = true;
+    int to[kMaxRank], r = 0;
+    for (int i = 0; i < rank; i++) {
+        if (i > 0 && !packed[i] && !packed[i - 1] && (int64_t)shape[r - 1] * shape[i] < ((int64_t)1 << 31)) {
+            shape[r - 1] *= shape[i];
+        } else {
+            shape[r] = shape[i];
+            packed[r] = packed[i]; // (r <= i: entries below i are no longer read)
+            r++;
+        }
+        to[i] = r - 1;
+    }
+    for (int j = 0; j < n_axes; j++) nax[j] = to[nax[j]];
+    rank = r;
+}
+
 typedef uint32_t layout_u32x4 __attribute__((ext_vector_type(4)));
 
 template <typename K> static int launch_by_size(nncase_hip_ctx *ctx, int es, K &&k) {
@@ -514,6 +544,11 @@ extern "C" int nncase_hip_pack(nncase_hip_ctx_t *ctx, const void *in_dev, void *
     for (int j = 0; j < n_axes; j++) lns[j] = lanes[j];
     int es = elem_size;
     vector_view(es, rank, shp, n_axes, nax, lns, in_dev, out_dev);
+    {
+        int merged = rank;
+        merge_unpacked_axes(merged, shp, n_axes, nax);
+        rank = merged;
+    }
     PackDesc d;
     memset(&d, 0, sizeof(d));
     d.in_rank = rank;
@@ -592,6 +627,11 @@ extern "C" int nncase_hip_unpack(nncase_hip_ctx_t *ctx, const void *in_dev, void
     for (int j = 0; j < n_axes; j++) lns[j] = lanes[j];
     int es = elem_size;
     vector_view(es, rank, shp, n_axes, nax, lns, in_dev, out_dev);
+    {
+        int merged = rank;
+        merge_unpacked_axes(merged, shp, n_axes, nax);
+        rank = merged;
+    }
     PackDesc d;
     memset(&d, 0, sizeof(d));
     d.out_rank = rank;
