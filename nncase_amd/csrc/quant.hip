@@ -12,6 +12,7 @@
 
 #include <hip/hip_fp16.h>
 
+#include <algorithm>
 #include <cmath>
 
 namespace nnhip {
@@ -47,26 +48,28 @@ __global__ __launch_bounds__(kEwThreads) void quantize_kernel(const TIn *__restr
     const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t nthreads = (size_t)gridDim.x * blockDim.x;
     const size_t nvec = vec_ok ? count / kEwVec : 0;
-    size_t i = tid;
-    for (; i + (kEwUnroll - 1) * nthreads < nvec; i += kEwUnroll * nthreads) {
+    // a block owns kEwUnroll * kEwThreads neighbouring vectors (see ew_block_grid)
+    const size_t i = (size_t)blockIdx.x * (kEwUnroll * kEwThreads) + threadIdx.x;
+    if (i + (kEwUnroll - 1) * kEwThreads < nvec) {
         TIn v[kEwUnroll][4];
 #pragma unroll
-        for (int u = 0; u < kEwUnroll; u++) load4(in + (i + u * nthreads) * kEwVec, v[u]);
+        for (int u = 0; u < kEwUnroll; u++) load4(in + (i + u * kEwThreads) * kEwVec, v[u]);
 #pragma unroll
         for (int u = 0; u < kEwUnroll; u++) {
             TQ q[4];
 #pragma unroll
             for (int e = 0; e < 4; e++) q[e] = quantize_one<TQ>(to_f32(v[u][e]), scale, bias);
-            store4(out + (i + u * nthreads) * kEwVec, q);
+            store4(out + (i + u * kEwThreads) * kEwVec, q);
         }
-    }
-    for (; i < nvec; i += nthreads) {
-        TIn v[4];
-        TQ q[4];
-        load4(in + i * kEwVec, v);
+    } else {
+        for (size_t k = i; k < nvec && k < i + kEwUnroll * kEwThreads; k += kEwThreads) {
+            TIn v[4];
+            TQ q[4];
+            load4(in + k * kEwVec, v);
 #pragma unroll
-        for (int e = 0; e < 4; e++) q[e] = quantize_one<TQ>(to_f32(v[e]), scale, bias);
-        store4(out + i * kEwVec, q);
+            for (int e = 0; e < 4; e++) q[e] = quantize_one<TQ>(to_f32(v[e]), scale, bias);
+            store4(out + k * kEwVec, q);
+        }
     }
     for (size_t j = nvec * kEwVec + tid; j < count; j += nthreads) out[j] = quantize_one<TQ>(to_f32(in[j]), scale, bias);
 }
@@ -87,26 +90,27 @@ __global__ __launch_bounds__(kEwThreads) void dequantize_kernel(const TQ *__rest
     const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t nthreads = (size_t)gridDim.x * blockDim.x;
     const size_t nvec = vec_ok ? count / kEwVec : 0;
-    size_t i = tid;
-    for (; i + (kEwUnroll - 1) * nthreads < nvec; i += kEwUnroll * nthreads) {
+    const size_t i = (size_t)blockIdx.x * (kEwUnroll * kEwThreads) + threadIdx.x;
+    if (i + (kEwUnroll - 1) * kEwThreads < nvec) {
         TQ v[kEwUnroll][4];
 #pragma unroll
-        for (int u = 0; u < kEwUnroll; u++) load4(in + (i + u * nthreads) * kEwVec, v[u]);
+        for (int u = 0; u < kEwUnroll; u++) load4(in + (i + u * kEwThreads) * kEwVec, v[u]);
 #pragma unroll
         for (int u = 0; u < kEwUnroll; u++) {
             TOut y[4];
 #pragma unroll
             for (int e = 0; e < 4; e++) y[e] = from_f32<TOut>(((float)v[u][e] - bias) * scale);
-            store4(out + (i + u * nthreads) * kEwVec, y);
+            store4(out + (i + u * kEwThreads) * kEwVec, y);
         }
-    }
-    for (; i < nvec; i += nthreads) {
-        TQ v[4];
-        TOut y[4];
-        load4(in + i * kEwVec, v);
+    } else {
+        for (size_t k = i; k < nvec && k < i + kEwUnroll * kEwThreads; k += kEwThreads) {
+            TQ v[4];
+            TOut y[4];
+            load4(in + k * kEwVec, v);
 #pragma unroll
-        for (int e = 0; e < 4; e++) y[e] = from_f32<TOut>(((float)v[e] - bias) * scale);
-        store4(out + i * kEwVec, y);
+            for (int e = 0; e < 4; e++) y[e] = from_f32<TOut>(((float)v[e] - bias) * scale);
+            store4(out + k * kEwVec, y);
+        }
     }
     for (size_t j = nvec * kEwVec + tid; j < count; j += nthreads) out[j] = from_f32<TOut>(((float)in[j] - bias) * scale);
 }
@@ -236,10 +240,20 @@ inline int ew_grid(const nncase_hip_ctx *ctx, size_t work_items) {
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// Quantize / dequantize: a block per kEwUnroll * kEwThreads neighbouring vectors, however many that makes.  Blocks that
+// run at the same time then read and write neighbouring addresses (measured on 100 M elements against a capped grid that
+// strides over the tensor: quantize f32 -> u8 114 -> 96 us, dequantize i32 -> f32 202 -> 136 us).  Without vectors (an
+// unaligned buffer) the capped grid walks the elements.
+inline int ew_block_grid(const nncase_hip_ctx *ctx, size_t count, bool vec_ok) {
+    if (!vec_ok) return ew_grid(ctx, count);
+    const size_t per_block = (size_t)kEwUnroll * kEwThreads * kEwVec;
+    return (int)std::max<size_t>(1, (count + per_block - 1) / per_block);
+}
+
 template <typename TIn, typename TQ>
 int launch_quantize(nncase_hip_ctx *ctx, const void *in, void *out, size_t count, float scale, float bias) {
     const int vec_ok = aligned16(in) && aligned16(out);
-    const int grid = ew_grid(ctx, (count + kEwVec - 1) / kEwVec);
+    const int grid = ew_block_grid(ctx, count, vec_ok);
     hipLaunchKernelGGL((quantize_kernel<TIn, TQ>), dim3(grid), dim3(kEwThreads), 0, ctx->stream, (const TIn *)in,
                        (TQ *)out, count, scale, bias, vec_ok);
     NNHIP_LAUNCH_CHECK(ctx, "quantize_kernel");
@@ -249,7 +263,7 @@ int launch_quantize(nncase_hip_ctx *ctx, const void *in, void *out, size_t count
 template <typename TQ, typename TOut>
 int launch_dequantize(nncase_hip_ctx *ctx, const void *in, void *out, size_t count, float scale, float bias) {
     const int vec_ok = aligned16(in) && aligned16(out);
-    const int grid = ew_grid(ctx, (count + kEwVec - 1) / kEwVec);
+    const int grid = ew_block_grid(ctx, count, vec_ok);
     hipLaunchKernelGGL((dequantize_kernel<TQ, TOut>), dim3(grid), dim3(kEwThreads), 0, ctx->stream, (const TQ *)in,
                        (TOut *)out, count, scale, bias, vec_ok);
     NNHIP_LAUNCH_CHECK(ctx, "dequantize_kernel");
