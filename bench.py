@@ -406,7 +406,7 @@ def main():
         src.fill(1)
         dst.fill(0)
         for _ in range(3):
-            ctx.pack(src, dst, 4, [n], [], [])  # no packed axes: pack_kernel<unsigned int> is an element-wise copy
+            ctx.pack(src, dst, 4, [n], [], [])  # no packed axes: the element-wise pack kernel is a plain copy (16 bytes per thread)
         ctx.sync()
         del src, dst
     graph = nb.mobilenet_v2(seed=2)
