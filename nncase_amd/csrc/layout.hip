@@ -192,6 +192,8 @@ struct TileDesc {
     uint32_t exact;                   // 1: the destination has no padding: lanes past the plain extent of A are not stored (transposes)
     uint32_t pitch;                   // dwords per LDS row
     FastDiv d_cols, d_rowq;           // dwords per row of the tile; rows / E
+    uint32_t wide;                    // packing: every row of the source tile is whole 16-byte pieces at 16-byte addresses
+    FastDiv d_cols4;                  // ... of which a row has this many
 };
 
 template <int E> __device__ __forceinline__ void transpose_dwords(const uint32_t (&d)[E], uint32_t (&o)[E]) {
@@ -234,8 +236,27 @@ template <int E, bool PACK> __global__ __launch_bounds__(kLayoutThreads) void pa
     plain += x0;
     const uint32_t vlim = min(d.la, d.a_extent - ag * d.la); // lanes of this group that exist in the plain tensor
     const uint32_t rows = PACK ? d.la : d.tx, cols = d.d_cols.div; // (cols in dwords)
-    // ---- in: four dwords per thread requested before the first is parked ----
+    // ---- in: four loads per thread requested before the first is parked; 16 bytes each where the plain tensor's
+    // rows allow (the bytes in flight, not the instruction count, are what this phase lives on) ----
     constexpr int U = 4;
+    if (PACK && d.wide) {
+        const uint32_t cols4 = d.d_cols4.div;
+        for (uint32_t base = threadIdx.x; base < rows * cols4; base += U * kLayoutThreads) {
+            uint4 v[U];
+            uint32_t at[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const uint32_t idx = min(base + u * kLayoutThreads, rows * cols4 - 1);
+                const uint32_t r = fastdiv(idx, d.d_cols4), c = (idx - r * cols4) * 4;
+                at[u] = r * d.pitch + c;
+                v[u] = uint4{0u, 0u, 0u, 0u};
+                if (has_source && r < vlim && x0 + c * E < d.x_extent)
+                    v[u] = *reinterpret_cast<const uint4 *>(in + (plain + (uint64_t)r * d.a_plain_stride) * ES + c * 4);
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) tile[at[u]] = v[u].x, tile[at[u] + 1] = v[u].y, tile[at[u] + 2] = v[u].z, tile[at[u] + 3] = v[u].w;
+        }
+    } else
     for (uint32_t base = threadIdx.x; base < rows * cols; base += U * kLayoutThreads) {
         uint32_t v[U], at[U];
 #pragma unroll
@@ -282,10 +303,13 @@ template <int E, bool PACK> __global__ __launch_bounds__(kLayoutThreads) void pa
 }
 
 // Elements of X per tile: about 16 KiB per tile, rows of the plain tensor of 64 bytes to 2 KiB.
-static uint32_t tile_stretch(uint32_t la, int es) {
+// The extent is then split evenly over its tiles (3136 = 7 x 448 rather than 6 x 512 + 64).
+static uint32_t tile_stretch(uint32_t la, int es, uint32_t x_extent, bool wide) {
+    const uint32_t e = (wide ? 16 : 4) / es; // tiles begin at whole dwords (16-byte pieces) of a row
     uint32_t tx = 16384 / (la * es);
-    tx = std::min<uint32_t>(std::max<uint32_t>(tx, 64 / es), 2048 / es);
-    return tx / (4 / es) * (4 / es);
+    tx = std::min<uint32_t>(std::max<uint32_t>(tx, 64 / es), 2048 / es) / e * e;
+    const uint32_t tiles = (x_extent + tx - 1) / tx;
+    return ((x_extent + tiles - 1) / tiles + e - 1) / e * e;
 }
 // Dwords per LDS row: odd, so that the E rows a lane reads and the rows of neighbouring lanes spread over the banks.
 static uint32_t tile_pitch(uint32_t cols) { return cols | 1u; }
@@ -329,7 +353,8 @@ static bool make_tile_desc(TileDesc &d, int es, int rank, const int32_t *shape, 
     }
     if (a >= xs || ((uint64_t)d.x_extent * es) % 4 != 0) return false;
     if (!pack) d.x_padded = d.x_extent;
-    d.tx = tile_stretch(la, es);
+    d.wide = pack && ((uint64_t)d.x_extent * es) % 16 == 0 && (reinterpret_cast<uintptr_t>(in) & 15u) == 0;
+    d.tx = tile_stretch(la, es, d.x_padded, d.wide);
     d.x_tiles = (d.x_padded + d.tx - 1) / d.tx;
     d.la = la, d.a_extent = (uint32_t)shape[a], d.a_groups = O[a];
     d.a_plain_stride = sp[a], d.a_packed_group = sqo[a];
@@ -348,6 +373,7 @@ static bool make_tile_desc(TileDesc &d, int es, int rank, const int32_t *shape, 
     d.pitch = tile_pitch(cols);
     d.d_cols = make_fastdiv(cols);
     d.d_rowq = make_fastdiv(rows / e);
+    d.d_cols4 = make_fastdiv(std::max<uint32_t>(cols / 4, 1));
     lds = (size_t)rows * d.pitch * 4;
     return lds <= 48 * 1024;
 }
@@ -407,7 +433,8 @@ static bool make_transpose_desc(TileDesc &d, int es, int batch, int rows, int co
     d.x_extent = d.x_padded = (uint32_t)nx;
     d.x_packed = TwoTerm{1, (uint64_t)na, 0};
     d.exact = 1;
-    d.tx = tile_stretch(la, es);
+    d.wide = packing && ((uint64_t)nx * es) % 16 == 0 && (reinterpret_cast<uintptr_t>(in) & 15u) == 0;
+    d.tx = tile_stretch(la, es, d.x_padded, d.wide);
     d.x_tiles = (d.x_padded + d.tx - 1) / d.tx;
     d.nrest = 1;
     d.r_extent[0] = d.r_valid[0] = (uint32_t)batch;
@@ -418,6 +445,7 @@ static bool make_transpose_desc(TileDesc &d, int es, int batch, int rows, int co
     d.pitch = tile_pitch(tcols);
     d.d_cols = make_fastdiv(tcols);
     d.d_rowq = make_fastdiv(trows / e);
+    d.d_cols4 = make_fastdiv(std::max<uint32_t>(tcols / 4, 1));
     lds = (size_t)trows * d.pitch * 4;
     return lds <= 48 * 1024;
 }
