@@ -42,7 +42,8 @@ __global__ __launch_bounds__(kGlueThreads) void lut_u8_kernel(const uint8_t *__r
 }
 
 // One input of a channel concat: out[p, c_off + c] = table[in[p, c]] for c < c_in.
-// VEC = bytes per thread (4 when every channel count and offset is a multiple of 4).
+// VEC = bytes per thread: 16 when every channel count (hence every offset and the output's pixel stride) is a multiple
+// of 16 and the buffers are 16-byte aligned, 4 likewise, else 1.
 template <int VEC>
 __global__ __launch_bounds__(kGlueThreads) void concat_lut_kernel(const uint8_t *__restrict__ in, uint8_t *__restrict__ out,
                                                                  uint32_t total, FastDiv d_cv, uint32_t c_in,
@@ -54,8 +55,47 @@ __global__ __launch_bounds__(kGlueThreads) void concat_lut_kernel(const uint8_t 
     const uint32_t p = fastdiv(gid, d_cv);
     const uint32_t c = (gid - p * d_cv.div) * VEC;
     const size_t src = (size_t)p * c_in + c, dst = (size_t)p * c_out + c_off + c;
-    if (VEC == 4) *reinterpret_cast<uint32_t *>(out + dst) = lut4(t, *reinterpret_cast<const uint32_t *>(in + src));
-    else out[dst] = t[in[src]];
+    if (VEC == 16) {
+        const uint4 v = *reinterpret_cast<const uint4 *>(in + src);
+        *reinterpret_cast<uint4 *>(out + dst) = uint4{lut4(t, v.x), lut4(t, v.y), lut4(t, v.z), lut4(t, v.w)};
+    } else if (VEC == 4) {
+        *reinterpret_cast<uint32_t *>(out + dst) = lut4(t, *reinterpret_cast<const uint32_t *>(in + src));
+    } else {
+        out[dst] = t[in[src]];
+    }
+}
+
+// Every input of a channel concat in one launch (vector widths of 16 or 4 bytes): a thread owns VEC channels of one output
+// pixel, finds the input they come from and applies that input's table; channels of an input that is already in place
+// (a null pointer: written there by its producer) are left alone.
+struct ConcatArgs {
+    const uint8_t *in[NNCASE_HIP_MAX_CONCAT];
+    uint32_t c_in[NNCASE_HIP_MAX_CONCAT], c_end[NNCASE_HIP_MAX_CONCAT]; // channels of input i; first output channel behind it
+    ByteTable lut[NNCASE_HIP_MAX_CONCAT];
+    uint8_t *out;
+    uint32_t total, c_out;
+    int n;
+    FastDiv d_cv; // vectors per output pixel
+};
+template <int VEC> __global__ __launch_bounds__(kGlueThreads) void concat_all_kernel(const ConcatArgs a) {
+    __shared__ __align__(16) uint8_t t[NNCASE_HIP_MAX_CONCAT][256];
+    for (int i = threadIdx.x; i < a.n * 64; i += kGlueThreads) reinterpret_cast<uint32_t *>(t[i >> 6])[i & 63] = a.lut[i >> 6].w[i & 63];
+    __syncthreads();
+    const uint32_t gid = blockIdx.x * kGlueThreads + threadIdx.x;
+    if (gid >= a.total) return;
+    const uint32_t p = fastdiv(gid, a.d_cv);
+    const uint32_t c = (gid - p * a.d_cv.div) * VEC;
+    int i = 0;
+    while (i + 1 < a.n && c >= a.c_end[i]) i++;
+    if (!a.in[i]) return;
+    const uint32_t c0 = i == 0 ? 0u : a.c_end[i - 1];
+    const size_t src = (size_t)p * a.c_in[i] + (c - c0), dst = (size_t)p * a.c_out + c;
+    if (VEC == 16) {
+        const uint4 v = *reinterpret_cast<const uint4 *>(a.in[i] + src);
+        *reinterpret_cast<uint4 *>(a.out + dst) = uint4{lut4(t[i], v.x), lut4(t[i], v.y), lut4(t[i], v.z), lut4(t[i], v.w)};
+    } else {
+        *reinterpret_cast<uint32_t *>(a.out + dst) = lut4(t[i], *reinterpret_cast<const uint32_t *>(a.in[i] + src));
+    }
 }
 
 // Coordinate of an output index in the input (get_coordinate_from_resized,
@@ -157,6 +197,19 @@ template <int VEC> __global__ __launch_bounds__(kGlueThreads) void maxpool_u8_ke
     const uint32_t n = q;
     const int y0 = max(oy * a.stride_h - a.pad_h, 0), y1 = min(oy * a.stride_h - a.pad_h + a.kh, a.in_h);
     const int x0 = max(ox * a.stride_w - a.pad_w, 0), x1 = min(ox * a.stride_w - a.pad_w + a.kw, a.in_w);
+    const bool padded = (y1 - y0) * (x1 - x0) < a.kh * a.kw;
+    if (VEC == 16) { // 16 channels per thread: a quarter of the loads for the same bytes
+        uint4 m4 = uint4{0u, 0u, 0u, 0u};
+        for (int y = y0; y < y1; y++)
+            for (int x = x0; x < x1; x++) {
+                const uint4 d = reinterpret_cast<const uint4 *>(a.in)[(((size_t)n * a.in_h + y) * a.in_w + x) * a.cvecs + v];
+                m4 = uint4{max_u8x4(m4.x, d.x), max_u8x4(m4.y, d.y), max_u8x4(m4.z, d.z), max_u8x4(m4.w, d.w)};
+            }
+        uint4 o = uint4{lut4(t, m4.x), lut4(t, m4.y), lut4(t, m4.z), lut4(t, m4.w)};
+        if (padded) o = uint4{max_u8x4(o.x, a.zero_code), max_u8x4(o.y, a.zero_code), max_u8x4(o.z, a.zero_code), max_u8x4(o.w, a.zero_code)};
+        reinterpret_cast<uint4 *>(a.out)[gid] = o;
+        return;
+    }
     uint32_t m = 0;
     for (int y = y0; y < y1; y++)
         for (int x = x0; x < x1; x++) {
@@ -164,7 +217,6 @@ template <int VEC> __global__ __launch_bounds__(kGlueThreads) void maxpool_u8_ke
             if (VEC == 4) m = max_u8x4(m, reinterpret_cast<const uint32_t *>(a.in)[src]);
             else m = max(m, (uint32_t)a.in[src]);
         }
-    const bool padded = (y1 - y0) * (x1 - x0) < a.kh * a.kw;
     if (VEC == 4) {
         uint32_t o = lut4(t, m);
         if (padded) o = max_u8x4(o, a.zero_code);
@@ -229,13 +281,43 @@ extern "C" int nncase_hip_qconcat_channels(nncase_hip_ctx_t *ctx, int32_t n_inpu
     NNHIP_REQUIRE(ctx, pixels >= 0, -EINVAL, "qconcat_channels: negative pixel count");
     NNHIP_REQUIRE(ctx, out_qp.scale != 0.f, -EINVAL, "qconcat_channels: output scale is zero");
     int64_t c_out = 0;
-    bool vec = (reinterpret_cast<uintptr_t>(out_dev) & 3u) == 0;
+    bool vec = (reinterpret_cast<uintptr_t>(out_dev) & 3u) == 0, vec16 = (reinterpret_cast<uintptr_t>(out_dev) & 15u) == 0;
     for (int i = 0; i < n_inputs; i++) {
         NNHIP_REQUIRE(ctx, channels[i] > 0, -EINVAL, "qconcat_channels: input %d is empty", i);
         vec = vec && channels[i] % 4 == 0 && (reinterpret_cast<uintptr_t>(in_dev[i]) & 3u) == 0; // (a skipped input is null)
+        vec16 = vec16 && channels[i] % 16 == 0 && (reinterpret_cast<uintptr_t>(in_dev[i]) & 15u) == 0;
         c_out += channels[i];
     }
     if (pixels == 0) return 0;
+    int live = 0;
+    for (int i = 0; i < n_inputs; i++) live += in_dev[i] != nullptr;
+    if (vec && live > 1) { // one launch for all the inputs (a single one that is not in place yet keeps the launch that covers its channels only)
+        const int v = vec16 ? 16 : 4;
+        const int64_t total = pixels * (c_out / v);
+        if (total < ((int64_t)1 << 31)) {
+            ConcatArgs a;
+            memset(&a, 0, sizeof(a));
+            uint32_t end = 0;
+            bool any = false;
+            for (int i = 0; i < n_inputs; i++) {
+                end += (uint32_t)channels[i];
+                a.in[i] = in_dev[i], a.c_in[i] = (uint32_t)channels[i], a.c_end[i] = end;
+                if (!in_dev[i]) continue;
+                any = true;
+                uint8_t lut[256];
+                const int rc = nncase_hip_make_unary_lut(NNCASE_HIP_LUT_REQUANT, in_qps[i], out_qp, lut);
+                NNHIP_REQUIRE(ctx, rc == 0, rc, "qconcat_channels: cannot build the requantisation table of input %d", i);
+                a.lut[i] = pack_table(lut);
+            }
+            if (!any) return 0;
+            a.out = out_dev, a.total = (uint32_t)total, a.c_out = (uint32_t)c_out, a.n = n_inputs, a.d_cv = make_fastdiv((uint32_t)(c_out / v));
+            const dim3 grid((unsigned)((total + kGlueThreads - 1) / kGlueThreads));
+            if (vec16) hipLaunchKernelGGL(concat_all_kernel<16>, grid, dim3(kGlueThreads), 0, ctx->stream, a);
+            else hipLaunchKernelGGL(concat_all_kernel<4>, grid, dim3(kGlueThreads), 0, ctx->stream, a);
+            NNHIP_LAUNCH_CHECK(ctx, "concat_all_kernel");
+            return 0;
+        }
+    }
     uint32_t c_off = 0;
     for (int i = 0; i < n_inputs; i++) {
         if (!in_dev[i]) { // already in place: written by its producer
@@ -245,12 +327,15 @@ extern "C" int nncase_hip_qconcat_channels(nncase_hip_ctx_t *ctx, int32_t n_inpu
         uint8_t lut[256];
         const int rc = nncase_hip_make_unary_lut(NNCASE_HIP_LUT_REQUANT, in_qps[i], out_qp, lut);
         NNHIP_REQUIRE(ctx, rc == 0, rc, "qconcat_channels: cannot build the requantisation table of input %d", i);
-        const int v = vec ? 4 : 1;
+        const int v = vec16 ? 16 : (vec ? 4 : 1);
         const int64_t total = pixels * (channels[i] / v);
         NNHIP_REQUIRE(ctx, total < ((int64_t)1 << 31), -EINVAL, "qconcat_channels: input %d too large", i);
         const FastDiv d_cv = make_fastdiv((uint32_t)(channels[i] / v));
         const dim3 grid((unsigned)((total + kGlueThreads - 1) / kGlueThreads));
-        if (vec)
+        if (vec16)
+            hipLaunchKernelGGL(concat_lut_kernel<16>, grid, dim3(kGlueThreads), 0, ctx->stream, in_dev[i], out_dev, (uint32_t)total,
+                               d_cv, (uint32_t)channels[i], (uint32_t)c_out, c_off, pack_table(lut));
+        else if (vec)
             hipLaunchKernelGGL(concat_lut_kernel<4>, grid, dim3(kGlueThreads), 0, ctx->stream, in_dev[i], out_dev, (uint32_t)total,
                                d_cv, (uint32_t)channels[i], (uint32_t)c_out, c_off, pack_table(lut));
         else
@@ -325,11 +410,12 @@ extern "C" int nncase_hip_qmaxpool2d(nncase_hip_ctx_t *ctx, const uint8_t *x_dev
     const int rc = nncase_hip_make_unary_lut(NNCASE_HIP_LUT_REQUANT, x_qp, y_qp, lut);
     NNHIP_REQUIRE(ctx, rc == 0, rc, "qmaxpool2d: cannot build the requantisation table (zero output scale?)");
     const bool vec = channels % 4 == 0 && ((reinterpret_cast<uintptr_t>(x_dev) | reinterpret_cast<uintptr_t>(out_dev)) & 3u) == 0;
+    const bool vec16 = channels % 16 == 0 && ((reinterpret_cast<uintptr_t>(x_dev) | reinterpret_cast<uintptr_t>(out_dev)) & 15u) == 0;
     PoolArgs a;
     a.in = x_dev, a.out = out_dev;
     a.in_h = in_h, a.in_w = in_w, a.out_h = out_h, a.out_w = out_w, a.kh = kernel_h, a.kw = kernel_w;
     a.stride_h = stride_h, a.stride_w = stride_w, a.pad_h = pad_h_before, a.pad_w = pad_w_before;
-    a.cvecs = (uint32_t)(vec ? channels / 4 : channels);
+    a.cvecs = (uint32_t)(vec16 ? channels / 16 : (vec ? channels / 4 : channels));
     const int64_t total = (int64_t)batch * out_h * out_w * a.cvecs;
     NNHIP_REQUIRE(ctx, total < ((int64_t)1 << 31), -EINVAL, "qmaxpool2d: too many work items");
     a.total = (uint32_t)total;
@@ -340,7 +426,8 @@ extern "C" int nncase_hip_qmaxpool2d(nncase_hip_ctx_t *ctx, const uint8_t *x_dev
         a.zero_code = (uint32_t)r * 0x01010101u;
     }
     const dim3 grid((unsigned)((total + kGlueThreads - 1) / kGlueThreads));
-    if (vec) hipLaunchKernelGGL(maxpool_u8_kernel<4>, grid, dim3(kGlueThreads), 0, ctx->stream, a, pack_table(lut));
+    if (vec16) hipLaunchKernelGGL(maxpool_u8_kernel<16>, grid, dim3(kGlueThreads), 0, ctx->stream, a, pack_table(lut));
+    else if (vec) hipLaunchKernelGGL(maxpool_u8_kernel<4>, grid, dim3(kGlueThreads), 0, ctx->stream, a, pack_table(lut));
     else hipLaunchKernelGGL(maxpool_u8_kernel<1>, grid, dim3(kGlueThreads), 0, ctx->stream, a, pack_table(lut));
     NNHIP_LAUNCH_CHECK(ctx, "maxpool_u8_kernel");
     return 0;
