@@ -236,16 +236,16 @@ template <int E, bool PACK> __global__ __launch_bounds__(kLayoutThreads) void pa
     plain += x0;
     const uint32_t vlim = min(d.la, d.a_extent - ag * d.la); // lanes of this group that exist in the plain tensor
     const uint32_t rows = PACK ? d.la : d.tx, cols = d.d_cols.div; // (cols in dwords)
-    // ---- in: four loads per thread requested before the first is parked; 16 bytes each where the plain tensor's
-    // rows allow (the bytes in flight, not the instruction count, are what this phase lives on) ----
-    constexpr int U = 4;
+    // ---- in: eight dwords per thread requested before the first is parked, or four 16-byte pieces where the plain
+    // tensor's rows allow (the bytes in flight, not the instruction count, are what this phase lives on) ----
+    constexpr int U = 8, UW = 4; // loads in flight per thread: dwords, 16-byte pieces
     if (PACK && d.wide) {
         const uint32_t cols4 = d.d_cols4.div;
-        for (uint32_t base = threadIdx.x; base < rows * cols4; base += U * kLayoutThreads) {
-            uint4 v[U];
-            uint32_t at[U];
+        for (uint32_t base = threadIdx.x; base < rows * cols4; base += UW * kLayoutThreads) {
+            uint4 v[UW];
+            uint32_t at[UW];
 #pragma unroll
-            for (int u = 0; u < U; u++) {
+            for (int u = 0; u < UW; u++) {
                 const uint32_t idx = min(base + u * kLayoutThreads, rows * cols4 - 1);
                 const uint32_t r = fastdiv(idx, d.d_cols4), c = (idx - r * cols4) * 4;
                 at[u] = r * d.pitch + c;
@@ -254,7 +254,7 @@ template <int E, bool PACK> __global__ __launch_bounds__(kLayoutThreads) void pa
                     v[u] = *reinterpret_cast<const uint4 *>(in + (plain + (uint64_t)r * d.a_plain_stride) * ES + c * 4);
             }
 #pragma unroll
-            for (int u = 0; u < U; u++) tile[at[u]] = v[u].x, tile[at[u] + 1] = v[u].y, tile[at[u] + 2] = v[u].z, tile[at[u] + 3] = v[u].w;
+            for (int u = 0; u < UW; u++) tile[at[u]] = v[u].x, tile[at[u] + 1] = v[u].y, tile[at[u] + 2] = v[u].z, tile[at[u] + 3] = v[u].w;
         }
     } else
     for (uint32_t base = threadIdx.x; base < rows * cols; base += U * kLayoutThreads) {
