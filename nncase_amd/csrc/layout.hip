@@ -1,8 +1,12 @@
 // Pure data-movement kernels: pack / unpack (lane-blocked layouts) and the
 // NCHW <-> NHWC relayout.  All are permutations with optional zero padding,
-// bound by HBM bandwidth; each thread produces one output element so writes
-// are always coalesced, and the NCHW/NHWC transposes go through an LDS tile so
-// reads are coalesced as well.
+// bound by HBM bandwidth.  Where the innermost dimension of the packed tensor
+// runs against the innermost axis of the plain one (the layouts matrix
+// operands want, and the relayout of narrow elements) a block moves a tile
+// through LDS with dword accesses on both sides (pack_tile_kernel); every
+// other permutation has a thread produce one output element -- a 16- or
+// 4-byte group of elements where the two innermost dimensions coincide -- so
+// that writes are coalesced; 4-byte transposes go through a 32 x 33 LDS tile.
 #include "common.hpp"
 
 #include <algorithm>
