@@ -37,7 +37,7 @@ pytestmark = pytest.mark.gpu
     ((3, 7, 6), [1], [4], np.uint8),                   # rows of 6 bytes: not dword multiples, the element-wise kernel
     ((2, 70, 4, 16), [1], [32], np.uint8),             # plain rows of whole 16-byte pieces: the tile kernel's wide loads, ragged lanes
     ((2, 40, 8, 8), [1], [8], np.float16),
-    ((3, 1100, 48), [1], [64], np.uint8),              # several tiles along the innermost axis? no: several lane groups, one stretch
+    ((3, 1100, 48), [1], [64], np.uint8),              # many lane groups (the last one ragged), one short stretch
     ((2, 36, 2100), [1], [4], np.uint8),               # few lanes, a long stretch split evenly over its tiles
 ])
 def test_pack_unpack(hip_ctx, shape, axes, lanes, dtype):
